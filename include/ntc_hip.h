@@ -1,0 +1,179 @@
+/*
+ * ntc_hip.h - C ABI of the MI355X (gfx950) neural-texture-set decoder.
+ *
+ * This is the seam a LibNTC maintainer binds in place of the CUDA launchers that
+ * ITextureSet::Decompress drives (reference src/TextureSet.cpp:1664-1897):
+ *
+ *   reference call (file:line)                                replaced by
+ *   --------------------------------------------------------  -------------------------
+ *   cuda::Inference(InferenceKernelParams const&)             ntc_hip_decode (one launch for
+ *     src/Regression.h:37, src/Inference.cu:159-165            every mip of every set)
+ *   cuda::UnpackLatents  src/Quantizer.h:56-62                 fused into ntc_hip_decode
+ *   cuda::ConvertNetworkFromQuantizedToFp16                    deleted: the int8 blob of
+ *     src/Quantizer.h:35-40                                    src/WeightLayout.cpp:142-268
+ *                                                              is consumed as stored
+ *   cuda::CopyImage (1:1 branch) src/ImageProcessing.h:76-80   fused output formats below
+ *   cudaMalloc / cudaMemcpy / cudaEvent* used by that path     ntc_hip_alloc / upload / ...
+ *
+ * Plain C: pointers, sizes and PODs only.  Every entry point returns 0 on success,
+ * a positive hipError_t value when a HIP call failed, or a negative NtcHipError.
+ * A message for the last failure on the calling thread is kept per thread, like
+ * the reference's thread-local error buffer (src/Errors.cpp:21-52).
+ */
+#ifndef NTC_HIP_H
+#define NTC_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NTC_HIP_MAX_MIPS      16 /* NTC_MAX_MIPS,     include/libntc/shaders/InferenceConstants.h:22 */
+#define NTC_HIP_MAX_CHANNELS  16 /* NTC_MAX_CHANNELS, include/libntc/shaders/InferenceConstants.h:23 */
+#define NTC_HIP_MLP_LAYERS    4  /* NTC_MLP_LAYERS,   include/libntc/shaders/InferenceConstants.h:28 */
+#define NTC_HIP_MAX_LAYER_WIDTH 64
+
+typedef enum NtcHipError {
+    NTC_HIP_OK                 = 0,
+    NTC_HIP_ERR_INVALID_ARG    = -1,
+    NTC_HIP_ERR_UNSUPPORTED    = -2, /* a decoder spec no compiled kernel covers */
+    NTC_HIP_ERR_NO_DEVICE      = -3,
+    NTC_HIP_ERR_NOT_INITIALIZED= -4
+} NtcHipError;
+
+/* How one latent grid feeds the network input vector. */
+typedef enum NtcHipGridMode {
+    /* 4-tap bilinear filter with wrap addressing, one input per feature
+     * (src/FeatureGridDevice.h:33-98, include/libntc/shaders/Inference.hlsli:62-87). */
+    NTC_HIP_GRID_BILINEAR  = 0,
+    /* The four unfiltered neighbours a00,a01,a10,a11 of src/FeatureGridDevice.h:67-70,
+     * concatenated: 4 x features inputs ("2x2 high-res neighbourhood"). */
+    NTC_HIP_GRID_CONCAT2X2 = 1
+} NtcHipGridMode;
+
+typedef enum NtcHipWeightType {
+    NTC_HIP_WEIGHTS_INT8 = 0, /* GenericInt8 blob, src/WeightLayout.cpp:42-49,184-247 */
+    NTC_HIP_WEIGHTS_FP8  = 1  /* e4m3 hidden layers + int8 output layer */
+} NtcHipWeightType;
+
+typedef enum NtcHipOutputFormat {
+    /* LibNTC's internal texture layout (src/ImageProcessing.h:20-33, src/RegressionKernels.h:36-45):
+     * fp16, per row groups of two channels, element index
+     *   y*W*C + (ch & ~1)*W + 2*x + (ch & 1),  C = channels rounded up to even. */
+    NTC_HIP_OUT_FP16_PLANAR_PAIRS = 0,
+    /* Pitch-linear pixels, all channels of a pixel together, fp16 (ChannelFormat::FLOAT16
+     * of src/ImageProcessing.cu:141-164). */
+    NTC_HIP_OUT_FP16_PIXELS  = 1,
+    /* Pitch-linear pixels, unorm8 (ChannelFormat::UNORM8, same function). */
+    NTC_HIP_OUT_UNORM8_PIXELS = 2
+} NtcHipOutputFormat;
+
+/* Geometry and arithmetic of one decoder.  The mounted LibNTC 0.9.2 is the preset
+ * {16,4,BILINEAR,16, 16,4,BILINEAR,16, 3, 2, 48, {64,48,32}, 16, INT8}. */
+typedef struct NtcHipDecoderSpec {
+    int32_t hrFeatures;      /* features stored per high-res cell                         */
+    int32_t hrBits;          /* bits per stored feature: 2 or 4 (16/bits features per u16) */
+    int32_t hrMode;          /* NtcHipGridMode                                             */
+    int32_t hrFeatureSlots;  /* input slots reserved per sampled cell (>= hrFeatures)      */
+    int32_t lrFeatures;
+    int32_t lrBits;
+    int32_t lrMode;
+    int32_t lrFeatureSlots;
+    int32_t posEncWaves;     /* NTC_MLP_POS_ENC_WAVES = 3 -> 12 inputs                     */
+    int32_t lodInputs;       /* 2 = the (lod, lod) pair of Inference.hlsli:117-119; 0 = none */
+    int32_t inputChannels;   /* padded input width, multiple of 16, <= 64                  */
+    int32_t hiddenChannels[NTC_HIP_MLP_LAYERS - 1];
+    int32_t outputChannels;  /* 16                                                         */
+    int32_t weightType;      /* NtcHipWeightType                                           */
+} NtcHipDecoderSpec;
+
+/* Byte offsets of the pieces of a weight blob (src/WeightLayout.h:33-50). */
+typedef struct NtcHipWeightLayout {
+    uint32_t weightOffset[NTC_HIP_MLP_LAYERS];
+    uint32_t scaleOffset[NTC_HIP_MLP_LAYERS];  /* fp32 per output channel; unused (0) for fp8 hidden layers */
+    uint32_t biasOffset[NTC_HIP_MLP_LAYERS];   /* int32 (int8 layers) or fp16 (fp8 hidden layers) */
+    uint32_t bufferSize;
+} NtcHipWeightLayout;
+
+/* One colour mip: the fields of InferenceKernelParams that vary per launch
+ * (src/RegressionCommon.h:55-80, filled at src/TextureSet.cpp:1806-1829). */
+typedef struct NtcHipMipDesc {
+    int32_t  width, height;          /* referenceWidth / referenceHeight                */
+    int32_t  hrWidth, hrHeight;      /* highResLatentWidth / Height                     */
+    int32_t  lrWidth, lrHeight;      /* lowResLatentWidth / Height                      */
+    float    positionScale;          /* src/TextureSet.cpp:460                          */
+    float    positionLod;            /* src/TextureSet.cpp:461                          */
+    uint64_t hrOffset;               /* byte offset of the grid's first u16 layer in `latents` */
+    uint64_t lrOffset;
+    uint64_t outOffset;              /* byte offset of this mip in `output`             */
+    uint64_t outRowPitch;            /* bytes between rows, pixel formats only          */
+} NtcHipMipDesc;
+
+/* One texture set to decode.  A latent grid is stored as in the NTC file:
+ * ceil(features / (16/bits)) layers of height*width little-endian u16, layer after
+ * layer (src/FeatureGridHost.h:92-93, src/Quantizer.cu:519-526); feature f of a cell
+ * sits in layer f / (16/bits) at bits [bits*(f % (16/bits)), +bits). */
+typedef struct NtcHipTextureSet {
+    NtcHipDecoderSpec spec;
+    int32_t  numMips;
+    int32_t  numChannels;            /* channels written; outputs >= numChannels are dropped (Inference.cu:131) */
+    int32_t  outputFormat;           /* NtcHipOutputFormat */
+    int32_t  outPixelStride;         /* bytes between pixels, pixel formats only */
+    const void* latents;             /* device */
+    const void* weights;             /* device, blob laid out per ntc_hip_weight_layout() */
+    void*       output;              /* device */
+    uint64_t latentsBytes;           /* sizes of the three buffers; every grid, the blob and every */
+    uint64_t weightsBytes;           /* mip's output extent are checked against them before launch */
+    uint64_t outputBytes;
+    NtcHipMipDesc mips[NTC_HIP_MAX_MIPS];
+} NtcHipTextureSet;
+
+/* ---- library / device ------------------------------------------------------------ */
+
+/* Selects the HIP device and creates the library's stream.  Replaces the reference's
+ * cudaSetDevice + cudaInitDevice in CreateContext (src/PublicFunctions.cpp:84-112). */
+int ntc_hip_init(int device);
+void ntc_hip_shutdown(void);
+/* Message of the last failed call on this thread ("" if none). GetLastErrorMessage, include/libntc/ntc.h:1331. */
+const char* ntc_hip_last_error(void);
+/* Name, compute-unit count of the initialised device. */
+int ntc_hip_device_info(char* name, size_t nameSize, int* computeUnits);
+
+/* ---- memory (DeviceArray<T> of src/CudaArray.h:104-181) --------------------------- */
+int ntc_hip_alloc(void** devPtr, size_t bytes);
+int ntc_hip_free(void* devPtr);
+int ntc_hip_upload(void* dst, const void* src, size_t bytes);     /* host -> device, synchronous */
+int ntc_hip_download(void* dst, const void* src, size_t bytes);   /* device -> host, synchronous */
+int ntc_hip_memset(void* dst, int value, size_t bytes);
+int ntc_hip_synchronize(void);
+
+/* ---- layout helpers (host only, no device needed) --------------------------------- */
+
+/* Offsets of a weight blob for `spec`: MakeQuantizedWeightLayout, src/WeightLayout.cpp:142-268. */
+int ntc_hip_weight_layout(const NtcHipDecoderSpec* spec, NtcHipWeightLayout* outLayout);
+/* Bytes one latent grid of the given shape occupies. */
+uint64_t ntc_hip_grid_bytes(int32_t width, int32_t height, int32_t features, int32_t bits);
+
+/* ---- the hot path ----------------------------------------------------------------- */
+
+/* Decodes every mip of every set in ONE launch on the library stream (asynchronous).
+ * Replaces the per-mip loop over cuda::Inference of src/TextureSet.cpp:1782-1831. */
+int ntc_hip_decode(const NtcHipTextureSet* sets, int32_t numSets);
+
+/* Same work, repeated `iterations` times between two HIP events on the library stream;
+ * returns the mean milliseconds of one repetition (the reference's own timer brackets the
+ * same region with cudaEvents, src/TextureSet.cpp:1772-1882).  Synchronous. */
+int ntc_hip_decode_timed(const NtcHipTextureSet* sets, int32_t numSets, int32_t iterations,
+                         float* outMillisecondsPerIteration);
+
+/* Self-check of the MFMA operand layout the kernels assume: multiplies a 16x64 by a
+ * 64x16 int8 matrix on the device (row-major host arrays), writes the 16x16 int32
+ * product.  No reference counterpart; used by the tests. */
+int ntc_hip_selftest_mfma(const int8_t* a16x64, const int8_t* b64x16, int32_t* d16x16);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NTC_HIP_H */

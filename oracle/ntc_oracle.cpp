@@ -1,0 +1,526 @@
+/*
+ * ntc_oracle.cpp - CPU restatement of LibNTC's int8 texture-set decode arithmetic.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file is the checker the HIP decoder is compared
+ * against; nothing in the shipped library links, loads or calls it.  Only tests, the
+ * smoke check and the CPU-baseline leg of the benchmark may use it.
+ *
+ * It is scalar, one texel at a time, and follows the reference line by line in
+ * meaning (not in code).  Each function names the reference lines it restates.
+ * All paths are relative to the LibNTC 0.9.2 tree.
+ *
+ * Arithmetic contract (what "bit-exact" means for the GPU path):
+ *   - every float operation is IEEE binary32, round-to-nearest-even, evaluated in the
+ *     order written here; a fused multiply-add happens exactly where fmaf() is written
+ *     (build with -ffp-contract=off);
+ *   - integer accumulation is exact int32;
+ *   - float -> int conversions say which rounding they use (floor / trunc / nearest-even).
+ *
+ * Pinning status of each function is listed in the table at the end of this header.
+ *
+ *   function                 pinned by (tests/test_oracle_*.py)
+ *   -----------------------  -----------------------------------------------------------
+ *   weight_layout            reference build oracle/_ref (MakeQuantizedWeightLayout) +
+ *                            committed fixture tests/golden/ref_layout.json + closed-form totals
+ *   ref_geometry             reference build oracle/_ref (FeatureGridMath) + fixture
+ *                            tests/golden/ref_geometry.json
+ *   unpack (latent fields)   Pack o Unpack = id over all 65536 words; bit positions by one-hot
+ *   bilinear / concat        integer cross-check in exact rational arithmetic for dyadic
+ *                            positions; d = 0 special case; wrap at both borders enumerated
+ *   pos-enc                  closed form, periodicity, range
+ *   hgelu_quantize           constants re-derived two ways (constexpr chain of
+ *                            src/tin/tin_activation.h:112-121 vs literals of
+ *                            Inference.hlsli:37-39); exhaustive monotone pieces and range checks
+ *   layer matmul             numpy int64 GEMM
+ *   half / unorm8 convert    numpy float16 (IEEE RNE) over all 2^16 halves and a dense fp32 sweep
+ *   e4m3 rounding            exhaustive over all half bit patterns vs an independent model
+ *   end-to-end decode        an independent numpy restatement (tests/np_decoder.py) on small sets
+ *   The exact bits of the reference's FP16-WMMA CUDA kernel (half accumulation order,
+ *   --use_fast_math) and of a hardware bilinear sampler are NOT reproduced: parity unpinned
+ *   for those two, by construction; the integer contract of Inference.hlsli is what is pinned.
+ */
+#include "../include/ntc_hip.h"
+
+#include <algorithm>
+#include <atomic>
+#include <chrono>
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <thread>
+#include <vector>
+
+namespace {
+
+// ---------------------------------------------------------------------------------------
+// Half-precision conversions (IEEE 754 binary16, round-to-nearest-even), done on the bits
+// so the result does not depend on the host's conversion instructions.
+// Reference use: __float22half2_rn stores of src/Inference.cu:121-135.
+// ---------------------------------------------------------------------------------------
+inline uint32_t f32_bits(float f) { uint32_t u; std::memcpy(&u, &f, 4); return u; }
+inline float bits_f32(uint32_t u) { float f; std::memcpy(&f, &u, 4); return f; }
+
+uint16_t float_to_half_rne(float f)
+{
+    uint32_t const x = f32_bits(f);
+    uint32_t const sign = (x >> 16) & 0x8000u;
+    uint32_t const absx = x & 0x7fffffffu;
+    if (absx >= 0x7f800000u)                       // Inf or NaN
+        return uint16_t(sign | 0x7c00u | (absx > 0x7f800000u ? 0x200u : 0u));
+    if (absx >= 0x477ff000u)                       // >= 65520 rounds to Inf
+        return uint16_t(sign | 0x7c00u);
+    if (absx < 0x33000001u)                        // <= 2^-25 rounds to zero (tie goes to even = 0)
+        return uint16_t(sign);
+    int32_t const exp = int32_t(absx >> 23) - 127;
+    uint32_t mant = (absx & 0x7fffffu) | 0x800000u; // 24-bit significand
+    int shift;                                      // bits dropped from the significand
+    uint32_t halfExpField;
+    if (exp < -14) { shift = 13 + (-14 - exp); halfExpField = 0; }   // subnormal half
+    else           { shift = 13;               halfExpField = uint32_t(exp + 15); }
+    uint32_t const kept = mant >> shift;
+    uint32_t const rem  = mant & ((1u << shift) - 1u);
+    uint32_t const halfway = 1u << (shift - 1);
+    uint32_t r = kept;
+    if (rem > halfway || (rem == halfway && (kept & 1u))) r += 1;
+    // For normals `kept` still holds the implicit bit (0x400); adding the exponent field
+    // shifted makes a mantissa carry bump the exponent correctly.
+    uint32_t out;
+    if (halfExpField == 0) out = r;                                  // may carry into exp=1: correct
+    else                   out = ((halfExpField - 1) << 10) + r;     // r includes the 0x400 bit
+    return uint16_t(sign | out);
+}
+
+float half_to_float(uint16_t h)
+{
+    uint32_t const sign = uint32_t(h & 0x8000u) << 16;
+    uint32_t const exp = (h >> 10) & 0x1fu;
+    uint32_t const mant = h & 0x3ffu;
+    if (exp == 0) {
+        if (mant == 0) return bits_f32(sign);
+        float const v = float(mant) * 0x1p-24f;   // exact
+        return (sign ? -v : v);
+    }
+    if (exp == 31) return bits_f32(sign | 0x7f800000u | (mant << 13));
+    return bits_f32(sign | ((exp + 112u) << 23) | (mant << 13));
+}
+
+// IsHalfSpecial, src/CudaUtils.h:30-35: exponent field all ones.
+inline bool half_is_special(uint16_t h) { return (h & 0x7c00u) == 0x7c00u; }
+
+// The value Inference.cu stores for one output: network output as fp16, Inf/NaN replaced
+// by zero (src/Inference.cu:123-126).  Channel scale/bias are identity on the decode
+// path (src/TextureSet.cpp:1726-1729).
+inline uint16_t output_to_half(float o)
+{
+    uint16_t h = float_to_half_rne(o);
+    if (half_is_special(h)) h = 0;
+    return h;
+}
+
+// WriteImageChannel, UNORM8 case, no dithering, linear colour space
+// (src/ImageProcessing.cu:146-149): roundf = round half away from zero, then clamp.
+// The source of that copy is the fp16 image Decompress wrote, so the value is rounded
+// to half first.
+inline uint8_t half_to_unorm8(uint16_t h)
+{
+    float const v = half_to_float(h) * 255.f;     // exact: 11-bit x 8-bit significands
+    float r = std::trunc(v);
+    float const frac = v - r;                     // exact
+    if (frac >= 0.5f) r += 1.f; else if (frac <= -0.5f) r -= 1.f;
+    r = std::max(0.f, std::min(255.f, r));
+    return uint8_t(r);
+}
+
+// ---------------------------------------------------------------------------------------
+// Weight blob layout: MakeQuantizedWeightLayout for GenericInt8 and GenericFP8
+// (src/WeightLayout.cpp:142-268; prose :42-71).
+// ---------------------------------------------------------------------------------------
+int layer_inputs(NtcHipDecoderSpec const& s, int layer)
+{
+    return layer == 0 ? s.inputChannels : s.hiddenChannels[layer - 1];   // src/MlpDesc.h:57-75
+}
+int layer_outputs(NtcHipDecoderSpec const& s, int layer)
+{
+    return layer == NTC_HIP_MLP_LAYERS - 1 ? s.outputChannels : s.hiddenChannels[layer]; // src/MlpDesc.h:78-99
+}
+
+bool weight_layout(NtcHipDecoderSpec const& s, NtcHipWeightLayout& L)
+{
+    std::memset(&L, 0, sizeof(L));
+    uint32_t off = 0;
+    for (int l = 0; l < NTC_HIP_MLP_LAYERS; ++l) {           // all matrices, 1 byte per weight, back to back
+        L.weightOffset[l] = off;
+        off += uint32_t(layer_inputs(s, l) * layer_outputs(s, l));
+    }
+    if (s.weightType == NTC_HIP_WEIGHTS_INT8) {
+        for (int l = 0; l < NTC_HIP_MLP_LAYERS; ++l) {       // all fp32 scale vectors ...
+            L.scaleOffset[l] = off;
+            off += 4u * uint32_t(layer_outputs(s, l));
+        }
+        for (int l = 0; l < NTC_HIP_MLP_LAYERS; ++l) {       // ... then all int32 bias vectors
+            L.biasOffset[l] = off;
+            off += 4u * uint32_t(layer_outputs(s, l));
+        }
+    } else if (s.weightType == NTC_HIP_WEIGHTS_FP8) {
+        for (int l = 0; l < NTC_HIP_MLP_LAYERS - 1; ++l) {   // fp16 bias of the fp8 layers, no scale
+            L.biasOffset[l] = off;
+            off += 2u * uint32_t(layer_outputs(s, l));
+        }
+        int const last = NTC_HIP_MLP_LAYERS - 1;             // int8 output layer: fp32 scale, int32 bias
+        L.scaleOffset[last] = off; off += 4u * uint32_t(layer_outputs(s, last));
+        L.biasOffset[last]  = off; off += 4u * uint32_t(layer_outputs(s, last));
+    } else {
+        return false;
+    }
+    L.bufferSize = off;
+    return true;
+}
+
+// ---------------------------------------------------------------------------------------
+// Latent fields.  PackLatentsKernel stores feature i of a layer at bits [4i, 4i+4) of a
+// u16 (src/Quantizer.cu:519-523); UnquantizeValue(q, bits) = q / (2^bits - 1)
+// (src/Quantizer.cu:490-495) takes the width as a parameter, so a 2-bit grid holds 8
+// features per u16, feature i at bits [2i, 2i+2).
+// ---------------------------------------------------------------------------------------
+inline int unpack_field(uint16_t word, int index, int bits)
+{
+    return (word >> (index * bits)) & ((1 << bits) - 1);
+}
+
+struct Grid {
+    uint16_t const* base; int width, height, features, bits;
+    int fetch(int x, int y, int f) const
+    {
+        int const perWord = 16 / bits;
+        size_t const layer = size_t(f / perWord);
+        uint16_t const w = base[(layer * size_t(height) + size_t(y)) * size_t(width) + size_t(x)];
+        return unpack_field(w, f % perWord, bits);
+    }
+};
+
+struct Footprint { int x0, y0, x1, y1; float w00, w10, w01, w11; };
+
+// FeatureGrid::SetupBilinearFilter, src/FeatureGridDevice.h:33-58 (weights kept in fp32:
+// the int8 contract samples in float, Inference.hlsli:62-87).
+Footprint bilinear_footprint(float u, float v, int gw, int gh)
+{
+    float const x = u * float(gw) - 0.5f;
+    float const y = v * float(gh) - 0.5f;
+    float const fx = std::floor(x), fy = std::floor(y);
+    float const dx = x - fx, dy = y - fy;
+    float const dxn = 1.f - dx, dyn = 1.f - dy;
+    Footprint fp;
+    fp.w00 = dxn * dyn; fp.w10 = dx * dyn; fp.w01 = dxn * dy; fp.w11 = dx * dy;
+    int xb = int(fx), yb = int(fy);
+    if (xb < 0) xb += gw;                      // wrap addressing
+    if (yb < 0) yb += gh;
+    fp.x0 = xb % gw;       fp.y0 = yb % gh;
+    fp.x1 = (xb + 1) % gw; fp.y1 = (yb + 1) % gh;
+    return fp;
+}
+
+// One grid's contribution to the int8 input vector.
+//  bilinear: Inference.hlsli:72-82 - the sampler returns s = t/(2^bits-1) with t the
+//    filtered code; the shader takes floor(s*255 - 128).  With t kept un-normalised that
+//    is floor(t * 255/(2^bits-1)) - 128 (255/15 = 17, 255/3 = 85, both exact).
+//  concat 2x2: the four taps a00,a01,a10,a11 of FeatureGridDevice.h:67-70, unfiltered,
+//    each code mapped by the same affine map (a tap with weight one).
+// Slots beyond `features` stay zero (mask of Inference.hlsli:76-80).
+void sample_grid(Grid const& g, int mode, int slots, float u, float v, int8_t* out)
+{
+    Footprint const fp = bilinear_footprint(u, v, g.width, g.height);
+    float const codeScale = 255.f / float((1 << g.bits) - 1);
+    if (mode == NTC_HIP_GRID_BILINEAR) {
+        for (int f = 0; f < g.features; ++f) {
+            float const q00 = float(g.fetch(fp.x0, fp.y0, f));
+            float const q10 = float(g.fetch(fp.x1, fp.y0, f));
+            float const q01 = float(g.fetch(fp.x0, fp.y1, f));
+            float const q11 = float(g.fetch(fp.x1, fp.y1, f));
+            float t = fp.w00 * q00;
+            t = std::fmaf(fp.w10, q10, t);
+            t = std::fmaf(fp.w01, q01, t);
+            t = std::fmaf(fp.w11, q11, t);
+            out[f] = int8_t(int(std::floor(t * codeScale)) - 128);
+        }
+    } else {
+        int const xs[4] = { fp.x0, fp.x1, fp.x0, fp.x1 };
+        int const ys[4] = { fp.y0, fp.y0, fp.y1, fp.y1 };
+        for (int tap = 0; tap < 4; ++tap)
+            for (int f = 0; f < g.features; ++f)
+                out[tap * slots + f] = int8_t(g.fetch(xs[tap], ys[tap], f) * int(codeScale) - 128);
+    }
+}
+
+// NtcEvaluatePositionalEncoding + NtcEncodeSamplePosition, Inference.hlsli:89-120
+// (CUDA twin: src/RegressionKernels.h:59-85).  int(float) truncates toward zero.
+inline float frac_hlsl(float x) { return x - std::floor(x); }
+
+void encode_position(float px, float py, float lod, int waves, int lodInputs, int8_t* out)
+{
+    int idx = 0;
+    for (int w = 0; w < waves; ++w) {
+        float const e[4] = {
+            frac_hlsl(px) * 2.f - 1.f, frac_hlsl(py) * 2.f - 1.f,
+            frac_hlsl(px + 0.25f) * 2.f - 1.f, frac_hlsl(py + 0.25f) * 2.f - 1.f };
+        for (int i = 0; i < 4; ++i) out[idx++] = int8_t(int(e[i] * 127.5f));
+        px *= 2.f; py *= 2.f;
+    }
+    for (int i = 0; i < lodInputs; ++i) out[idx++] = int8_t(int(lod * 127.5f));
+}
+
+// NtcHGELUClamp_ForwardFloat + _QuantizeFloat, Inference.hlsli:36-39,123-131:
+//   y = min(x,3) * saturate(mad(x, 0.333333, 0.5));  q = int(round(y*80) + (-113)).
+// HLSL round() is round-half-to-even; mad is taken as fused.
+inline int hgelu_quantize(float x)
+{
+    float t = std::fmaf(x, 0.333333f, 0.5f);
+    t = std::min(std::max(t, 0.f), 1.f);
+    float const y = std::min(x, 3.f) * t;
+    float const r = std::nearbyintf(y * 80.f);   // default rounding mode = nearest-even
+    return int(r + -113.f);
+}
+
+// NtcEvaluateLayerINT8, Inference.hlsli:133-182: acc starts at the int32 bias, adds
+// dot4add_i8packed products, then float(acc) * scale.  W is [out][in] row-major
+// (Inference.hlsli:153, src/Quantizer.cu:144).
+void layer_int8(int8_t const* W, float const* scale, int32_t const* bias,
+                int in, int out, int8_t const* x, float* r)
+{
+    for (int c = 0; c < out; ++c) {
+        int32_t acc = bias[c];
+        for (int k = 0; k < in; ++k) acc += int32_t(x[k]) * int32_t(W[c * in + k]);
+        r[c] = float(acc) * scale[c];
+    }
+}
+
+struct SetView {
+    NtcHipTextureSet const* set;
+    NtcHipWeightLayout layout;
+};
+
+void prepare_inputs(NtcHipTextureSet const& set, NtcHipMipDesc const& mip, int x, int y, int8_t* in)
+{
+    NtcHipDecoderSpec const& s = set.spec;
+    std::memset(in, 0, size_t(s.inputChannels));               // Inference.hlsli:221-224
+    // src/Inference.cu:52-53
+    float const u = (float(x) + 0.5f) / float(mip.width);
+    float const v = (float(y) + 0.5f) / float(mip.height);
+    uint8_t const* lat = static_cast<uint8_t const*>(set.latents);
+    Grid const hr{ reinterpret_cast<uint16_t const*>(lat + mip.hrOffset), mip.hrWidth, mip.hrHeight, s.hrFeatures, s.hrBits };
+    Grid const lr{ reinterpret_cast<uint16_t const*>(lat + mip.lrOffset), mip.lrWidth, mip.lrHeight, s.lrFeatures, s.lrBits };
+    int const hrInputs = (s.hrMode == NTC_HIP_GRID_CONCAT2X2 ? 4 : 1) * s.hrFeatureSlots;
+    int const lrInputs = (s.lrMode == NTC_HIP_GRID_CONCAT2X2 ? 4 : 1) * s.lrFeatureSlots;
+    sample_grid(hr, s.hrMode, s.hrFeatureSlots, u, v, in);               // Inference.hlsli:229-230
+    sample_grid(lr, s.lrMode, s.lrFeatureSlots, u, v, in + hrInputs);    // Inference.hlsli:232-234
+    encode_position(float(x) * mip.positionScale, float(y) * mip.positionScale, mip.positionLod,
+                    s.posEncWaves, s.lodInputs, in + hrInputs + lrInputs);   // Inference.hlsli:237-238
+}
+
+// One texel through the int8 network: NtcSampleTextureSet, Inference.hlsli:282-357.
+void decode_texel_int8(SetView const& sv, NtcHipMipDesc const& mip, int x, int y, float* outputs, int8_t* inputsOut)
+{
+    NtcHipTextureSet const& set = *sv.set;
+    NtcHipDecoderSpec const& s = set.spec;
+    uint8_t const* blob = static_cast<uint8_t const*>(set.weights);
+    int8_t act[NTC_HIP_MAX_LAYER_WIDTH];
+    prepare_inputs(set, mip, x, y, act);
+    if (inputsOut) std::memcpy(inputsOut, act, size_t(s.inputChannels));
+    float r[NTC_HIP_MAX_LAYER_WIDTH];
+    for (int l = 0; l < NTC_HIP_MLP_LAYERS; ++l) {
+        int const in = layer_inputs(s, l), out = layer_outputs(s, l);
+        layer_int8(reinterpret_cast<int8_t const*>(blob + sv.layout.weightOffset[l]),
+                   reinterpret_cast<float const*>(blob + sv.layout.scaleOffset[l]),
+                   reinterpret_cast<int32_t const*>(blob + sv.layout.biasOffset[l]),
+                   in, out, act, r);
+        if (l == NTC_HIP_MLP_LAYERS - 1) break;
+        for (int c = 0; c < out; ++c) act[c] = int8_t(hgelu_quantize(r[c]));   // NtcPackInt8x4: & 0xff
+    }
+    for (int c = 0; c < s.outputChannels; ++c) outputs[c] = r[c];
+}
+
+// Output addressing.  Planar pairs: GetPixelBaseAddress/GetChannelAddress,
+// src/RegressionKernels.h:36-45; channel count rounded up to even, src/TextureSet.cpp:86.
+void store_texel(NtcHipTextureSet const& set, NtcHipMipDesc const& mip, int x, int y, float const* o)
+{
+    uint8_t* out = static_cast<uint8_t*>(set.output) + mip.outOffset;
+    if (set.outputFormat == NTC_HIP_OUT_FP16_PLANAR_PAIRS) {
+        int const C = (set.numChannels + 1) & ~1;
+        uint16_t* img = reinterpret_cast<uint16_t*>(out);
+        for (int ch = 0; ch < set.numChannels; ++ch) {
+            size_t const a = size_t(y) * size_t(mip.width) * size_t(C) + size_t(x) * 2
+                           + size_t(ch & ~1) * size_t(mip.width) + size_t(ch & 1);
+            img[a] = output_to_half(o[ch]);
+        }
+        // An odd channel count still stores whole half2 pairs (Inference.cu:131-134).
+        if (set.numChannels & 1) {
+            int const ch = set.numChannels;
+            size_t const a = size_t(y) * size_t(mip.width) * size_t(C) + size_t(x) * 2
+                           + size_t(ch & ~1) * size_t(mip.width) + size_t(ch & 1);
+            img[a] = output_to_half(o[ch]);
+        }
+    } else {
+        uint8_t* px = out + size_t(y) * mip.outRowPitch + size_t(x) * size_t(set.outPixelStride);
+        for (int ch = 0; ch < set.numChannels; ++ch) {
+            uint16_t const h = output_to_half(o[ch]);
+            if (set.outputFormat == NTC_HIP_OUT_FP16_PIXELS) std::memcpy(px + 2 * ch, &h, 2);
+            else px[ch] = half_to_unorm8(h);
+        }
+    }
+}
+
+} // namespace
+
+// =========================================================================================
+// C entry points (loaded by the tests through ctypes)
+// =========================================================================================
+extern "C" {
+
+int ntc_oracle_weight_layout(const NtcHipDecoderSpec* spec, NtcHipWeightLayout* out)
+{
+    return weight_layout(*spec, *out) ? 0 : -1;
+}
+
+uint16_t ntc_oracle_float_to_half(float f) { return float_to_half_rne(f); }
+float    ntc_oracle_half_to_float(uint16_t h) { return half_to_float(h); }
+uint16_t ntc_oracle_output_to_half(float f) { return output_to_half(f); }
+uint8_t  ntc_oracle_half_to_unorm8(uint16_t h) { return half_to_unorm8(h); }
+int      ntc_oracle_hgelu_quantize(float x) { return hgelu_quantize(x); }
+int      ntc_oracle_unpack_field(uint16_t w, int index, int bits) { return unpack_field(w, index, bits); }
+
+// PackLatentsKernel's QuantizeValue, src/Quantizer.cu:482-488 (encoder side; here only so
+// the tests can check Pack o Unpack = id).
+uint32_t ntc_oracle_quantize_value(float value, int bits)
+{
+    float const step = 1.f / float((1 << bits) - 1);
+    value = std::max(0.f, std::min(1.f, value));
+    return uint32_t(std::round(value / step));
+}
+
+void ntc_oracle_encode_position(float px, float py, float lod, int waves, int lodInputs, int8_t* out)
+{
+    encode_position(px, py, lod, waves, lodInputs, out);
+}
+
+void ntc_oracle_bilinear_footprint(float u, float v, int gw, int gh, int* xy, float* w)
+{
+    Footprint const fp = bilinear_footprint(u, v, gw, gh);
+    xy[0] = fp.x0; xy[1] = fp.y0; xy[2] = fp.x1; xy[3] = fp.y1;
+    w[0] = fp.w00; w[1] = fp.w10; w[2] = fp.w01; w[3] = fp.w11;
+}
+
+// Inputs (int8, spec.inputChannels of them) and raw fp32 outputs of one texel.
+int ntc_oracle_decode_texel(const NtcHipTextureSet* set, int mip, int x, int y, float* outputs, int8_t* inputs)
+{
+    SetView sv{ set, {} };
+    if (set->spec.weightType != NTC_HIP_WEIGHTS_INT8 || !weight_layout(set->spec, sv.layout)) return -1;
+    decode_texel_int8(sv, set->mips[mip], x, y, outputs, inputs);
+    return 0;
+}
+
+// Neural-LOD geometry of the reference, for a texture set of the given size:
+//  LodToNeuralLod / GetGridDimension / CalculateNumNeuralMipLevels, src/FeatureGridMath.cpp:47-77;
+//  colour-mip constants, src/TextureSet.cpp:441-463; low-res dims, src/TextureSet.cpp:1816-1817;
+//  grids stored neural LOD after neural LOD, layers inside (src/FeatureGridHost.cpp:140-161).
+// Fills width/height/grid dims/positionScale/positionLod/hrOffset/lrOffset of mips[0..numMips).
+// Returns the number of neural LODs, or -1.
+int ntc_oracle_ref_geometry(int width, int height, int numMips, int gridSizeScale, int numFeatures,
+                            NtcHipMipDesc* mips, uint64_t* outLatentBytes)
+{
+    static int const sharedMipsForGridScale[] = { 2, 3, 3, 3, 4, 4 };
+    if (gridSizeScale < 1 || gridSizeScale > 6 || numMips < 1 || numMips > NTC_HIP_MAX_MIPS) return -1;
+    int const minGrid = int(float(std::min(width, height)) / float(gridSizeScale));
+    int numNeural = std::max(2, int(1.f + std::floor(std::log2(float(minGrid))))) & ~1;
+    auto lodToNeural = [&](int lod, int neuralLods) {
+        int n = (lod - sharedMipsForGridScale[gridSizeScale - 1] + 2) & ~1;
+        return std::max(0, std::min(n, neuralLods - 2));
+    };
+    // Clamp as CalculateQuantizedLatentsSize does (src/FeatureGridMath.cpp:27-33); the host
+    // grid applies the same clamp when it is sized (src/FeatureGridHost.cpp:27-79).
+    int const lastNeural = lodToNeural(numMips - 1, 8 /* NTC_MAX_NEURAL_MIPS */) + 1;
+    numNeural = std::min(numNeural, lastNeural + 1);
+    auto gridDim = [&](int dim, int nlod) { return std::max((dim / gridSizeScale) >> nlod, 1); };
+    int const layers = (numFeatures + 3) / 4;
+    std::vector<uint64_t> offs(size_t(numNeural) + 1, 0);
+    for (int n = 0; n < numNeural; ++n)
+        offs[size_t(n) + 1] = offs[size_t(n)] + uint64_t(gridDim(width, n)) * uint64_t(gridDim(height, n)) * 2u * uint64_t(layers);
+    if (outLatentBytes) *outLatentBytes = offs[size_t(numNeural)];
+    for (int m = 0; m < numMips; ++m) {
+        NtcHipMipDesc& d = mips[m];
+        int const nlod = lodToNeural(m, numNeural);
+        d.width = std::max(1, width >> m);
+        d.height = std::max(1, height >> m);
+        d.hrWidth = gridDim(width, nlod);  d.hrHeight = gridDim(height, nlod);
+        d.lrWidth = std::max(d.hrWidth >> 1, 1); d.lrHeight = std::max(d.hrHeight >> 1, 1);
+        float const ws = float(d.hrWidth) / float(d.width), hs = float(d.hrHeight) / float(d.height);
+        d.positionScale = 0.5f * std::max(ws, hs);
+        d.positionLod = std::max(-1.f, std::min(1.f, 0.25f * std::log2(d.positionScale)));
+        d.hrOffset = offs[size_t(nlod)];
+        d.lrOffset = offs[size_t(nlod) + 1];
+    }
+    return numNeural;
+}
+
+// Decodes every mip of one set into set->output (host memory).  Rows of each mip are handed
+// out in bands to `threads` workers.  Returns seconds spent decoding (steady clock), < 0 on error.
+double ntc_oracle_decode(const NtcHipTextureSet* set, int threads)
+{
+    SetView sv{ set, {} };
+    if (set->spec.weightType != NTC_HIP_WEIGHTS_INT8 || !weight_layout(set->spec, sv.layout)) return -1.0;
+    if (threads < 1) threads = 1;
+    auto const t0 = std::chrono::steady_clock::now();
+    for (int m = 0; m < set->numMips; ++m) {
+        NtcHipMipDesc const& mip = set->mips[m];
+        std::atomic<int> nextRow{0};
+        int const band = 4;
+        auto work = [&]() {
+            float o[NTC_HIP_MAX_LAYER_WIDTH];
+            for (;;) {
+                int const y0 = nextRow.fetch_add(band);
+                if (y0 >= mip.height) break;
+                int const y1 = std::min(mip.height, y0 + band);
+                for (int y = y0; y < y1; ++y)
+                    for (int x = 0; x < mip.width; ++x) {
+                        decode_texel_int8(sv, mip, x, y, o, nullptr);
+                        store_texel(*set, mip, x, y, o);
+                    }
+            }
+        };
+        int const n = std::min(threads, std::max(1, (mip.height + band - 1) / band));
+        if (n == 1) work();
+        else {
+            std::vector<std::thread> pool;
+            for (int i = 0; i < n; ++i) pool.emplace_back(work);
+            for (auto& t : pool) t.join();
+        }
+    }
+    return std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+}
+
+// Decodes only rows [y0, y1) of mip `mipIndex` (bounded CPU-baseline samples).
+double ntc_oracle_decode_rows(const NtcHipTextureSet* set, int mipIndex, int y0, int y1, int threads)
+{
+    SetView sv{ set, {} };
+    if (set->spec.weightType != NTC_HIP_WEIGHTS_INT8 || !weight_layout(set->spec, sv.layout)) return -1.0;
+    NtcHipMipDesc const& mip = set->mips[mipIndex];
+    y0 = std::max(0, y0); y1 = std::min(mip.height, y1);
+    if (threads < 1) threads = 1;
+    auto const t0 = std::chrono::steady_clock::now();
+    std::atomic<int> nextRow{y0};
+    auto work = [&]() {
+        float o[NTC_HIP_MAX_LAYER_WIDTH];
+        for (;;) {
+            int const y = nextRow.fetch_add(1);
+            if (y >= y1) break;
+            for (int x = 0; x < mip.width; ++x) {
+                decode_texel_int8(sv, mip, x, y, o, nullptr);
+                store_texel(*set, mip, x, y, o);
+            }
+        }
+    };
+    std::vector<std::thread> pool;
+    for (int i = 0; i < threads; ++i) pool.emplace_back(work);
+    for (auto& t : pool) t.join();
+    return std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+}
+
+} // extern "C"

@@ -1,0 +1,119 @@
+"""ctypes view of include/ntc_hip.h: the structs, the loader and the error type.
+
+The shared library is built in-tree (csrc/libntc_hip.so) by __graft_entry__.build();
+loading fails loudly when it is missing - there is no CPU decode path in this package.
+"""
+import ctypes as C
+import os
+
+MAX_MIPS = 16
+MAX_CHANNELS = 16
+MLP_LAYERS = 4
+
+GRID_BILINEAR, GRID_CONCAT2X2 = 0, 1
+WEIGHTS_INT8, WEIGHTS_FP8 = 0, 1
+OUT_FP16_PLANAR_PAIRS, OUT_FP16_PIXELS, OUT_UNORM8_PIXELS = 0, 1, 2
+
+ERR_INVALID_ARG, ERR_UNSUPPORTED, ERR_NO_DEVICE, ERR_NOT_INITIALIZED = -1, -2, -3, -4
+
+
+class DecoderSpec(C.Structure):
+    _fields_ = [
+        ("hrFeatures", C.c_int32), ("hrBits", C.c_int32), ("hrMode", C.c_int32), ("hrFeatureSlots", C.c_int32),
+        ("lrFeatures", C.c_int32), ("lrBits", C.c_int32), ("lrMode", C.c_int32), ("lrFeatureSlots", C.c_int32),
+        ("posEncWaves", C.c_int32), ("lodInputs", C.c_int32), ("inputChannels", C.c_int32),
+        ("hiddenChannels", C.c_int32 * (MLP_LAYERS - 1)), ("outputChannels", C.c_int32), ("weightType", C.c_int32),
+    ]
+
+    def layer_inputs(self, layer):
+        return self.inputChannels if layer == 0 else self.hiddenChannels[layer - 1]
+
+    def layer_outputs(self, layer):
+        return self.outputChannels if layer == MLP_LAYERS - 1 else self.hiddenChannels[layer]
+
+    def hr_inputs(self):
+        return (4 if self.hrMode == GRID_CONCAT2X2 else 1) * self.hrFeatureSlots
+
+    def lr_inputs(self):
+        return (4 if self.lrMode == GRID_CONCAT2X2 else 1) * self.lrFeatureSlots
+
+    def copy(self):
+        out = DecoderSpec()
+        C.memmove(C.byref(out), C.byref(self), C.sizeof(DecoderSpec))
+        return out
+
+
+class WeightLayout(C.Structure):
+    _fields_ = [
+        ("weightOffset", C.c_uint32 * MLP_LAYERS), ("scaleOffset", C.c_uint32 * MLP_LAYERS),
+        ("biasOffset", C.c_uint32 * MLP_LAYERS), ("bufferSize", C.c_uint32),
+    ]
+
+
+class MipDesc(C.Structure):
+    _fields_ = [
+        ("width", C.c_int32), ("height", C.c_int32), ("hrWidth", C.c_int32), ("hrHeight", C.c_int32),
+        ("lrWidth", C.c_int32), ("lrHeight", C.c_int32), ("positionScale", C.c_float), ("positionLod", C.c_float),
+        ("hrOffset", C.c_uint64), ("lrOffset", C.c_uint64), ("outOffset", C.c_uint64), ("outRowPitch", C.c_uint64),
+    ]
+
+
+class TextureSet(C.Structure):
+    _fields_ = [
+        ("spec", DecoderSpec), ("numMips", C.c_int32), ("numChannels", C.c_int32),
+        ("outputFormat", C.c_int32), ("outPixelStride", C.c_int32),
+        ("latents", C.c_void_p), ("weights", C.c_void_p), ("output", C.c_void_p),
+        ("latentsBytes", C.c_uint64), ("weightsBytes", C.c_uint64), ("outputBytes", C.c_uint64),
+        ("mips", MipDesc * MAX_MIPS),
+    ]
+
+
+class NtcHipError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__(f"ntc_hip error {code}: {message}")
+        self.code = code
+        self.message = message
+
+
+# Every symbol include/ntc_hip.h declares: (name, restype, argtypes)
+EXPORTS = [
+    ("ntc_hip_init", C.c_int, [C.c_int]),
+    ("ntc_hip_shutdown", None, []),
+    ("ntc_hip_last_error", C.c_char_p, []),
+    ("ntc_hip_device_info", C.c_int, [C.c_char_p, C.c_size_t, C.POINTER(C.c_int)]),
+    ("ntc_hip_alloc", C.c_int, [C.POINTER(C.c_void_p), C.c_size_t]),
+    ("ntc_hip_free", C.c_int, [C.c_void_p]),
+    ("ntc_hip_upload", C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    ("ntc_hip_download", C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    ("ntc_hip_memset", C.c_int, [C.c_void_p, C.c_int, C.c_size_t]),
+    ("ntc_hip_synchronize", C.c_int, []),
+    ("ntc_hip_weight_layout", C.c_int, [C.POINTER(DecoderSpec), C.POINTER(WeightLayout)]),
+    ("ntc_hip_grid_bytes", C.c_uint64, [C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
+    ("ntc_hip_decode", C.c_int, [C.POINTER(TextureSet), C.c_int32]),
+    ("ntc_hip_decode_timed", C.c_int, [C.POINTER(TextureSet), C.c_int32, C.c_int32, C.POINTER(C.c_float)]),
+    ("ntc_hip_selftest_mfma", C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
+]
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libntc_hip.so")
+_lib = None
+
+
+def load_library():
+    """Loads csrc/libntc_hip.so and types every export.  Raises if the library is not built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(f"{LIB_PATH} is not built; run __graft_entry__.build() (make -C rtxntc-library_amd/csrc)")
+        lib = C.CDLL(LIB_PATH)
+        for name, restype, argtypes in EXPORTS:
+            fn = getattr(lib, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = lib
+    return _lib
+
+
+def check(code):
+    if code != 0:
+        raise NtcHipError(code, load_library().ntc_hip_last_error().decode("utf-8", "replace"))

@@ -1,0 +1,45 @@
+// ntc_decode_kernel.h - what the host side of the library knows about the device code.
+#pragma once
+#include <hip/hip_runtime_api.h>
+#include <stdint.h>
+
+namespace ntc_hip_dev {
+
+enum {
+    NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS = 0,
+    NTC_HIP_DEV_OUT_FP16_PIXELS = 1,
+    NTC_HIP_DEV_OUT_UNORM8_PIXELS = 2
+};
+
+// Compiled decoder variants (geometry is a template parameter of the kernel).
+enum {
+    NTC_HIP_VARIANT_NONE = -1,
+    NTC_HIP_VARIANT_CFG01 = 0,  // HR 2x2 concat of 8 x 2-bit, LR bilinear 16 x 4-bit, IN 64, 64-48-32
+    NTC_HIP_VARIANT_CFG2,       // HR 2x2 concat of 8 x 2-bit, LR bilinear 12 x 4-bit, IN 64, 48-48-32
+    NTC_HIP_VARIANT_REF16,      // LibNTC 0.9.2: both grids bilinear 4-bit, (lod,lod), IN 48, 64-48-32
+    NTC_HIP_VARIANT_REF12,
+    NTC_HIP_VARIANT_REF8,
+    NTC_HIP_VARIANT_REF4
+};
+
+// One colour mip of one texture set, as the kernel sees it.  Entries are sorted by
+// tileStart; a workgroup tile covers 64 x 4 texels.
+struct DevMip {
+    uint16_t const* hr;        // first u16 layer of the high-res grid
+    uint16_t const* lr;
+    uint8_t*        out;       // start of this mip in the output
+    uint8_t const*  weights;   // weight blob of the set this mip belongs to
+    uint64_t outRowPitch;
+    int32_t width, height;
+    int32_t hrWidth, hrHeight, lrWidth, lrHeight;
+    float   positionScale, positionLod;
+    int32_t outPixelStride, numChannels, outFormat;
+    int32_t tileStart, tilesX, tilesY;
+};
+
+constexpr int kTileWidth = 64, kTileHeight = 4;
+
+hipError_t launch_decode(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream);
+hipError_t launch_selftest_mfma(int8_t const* a, int8_t const* b, int32_t* d, hipStream_t stream);
+
+} // namespace ntc_hip_dev

@@ -1,0 +1,427 @@
+// ntc_hip_api.cpp - the C ABI of include/ntc_hip.h: argument checks, the per-launch mip
+// table, device memory and timing.  No CPU decode path exists here: without a HIP device
+// every compute entry point fails with NTC_HIP_ERR_NO_DEVICE / NOT_INITIALIZED.
+#include "../../include/ntc_hip.h"
+#include "ntc_decode_kernel.h"
+
+#include <hip/hip_runtime_api.h>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <vector>
+
+using namespace ntc_hip_dev;
+
+namespace {
+
+thread_local char t_error[1024] = "";
+
+void set_error(char const* fmt, ...)
+{
+    va_list args;
+    va_start(args, fmt);
+    vsnprintf(t_error, sizeof(t_error), fmt, args);
+    va_end(args);
+}
+void clear_error() { t_error[0] = 0; }
+
+// Message shape of SetCudaErrorMessage (reference src/Errors.cpp:43-46).
+int hip_fail(char const* call, hipError_t err)
+{
+    set_error("Call to %s failed, error code = %s.", call, hipGetErrorName(err));
+    return int(err);
+}
+#define HIP_TRY(expr) do { hipError_t e_ = (expr); if (e_ != hipSuccess) return hip_fail(#expr, e_); } while (0)
+
+struct Library {
+    bool initialized = false;
+    int device = -1;
+    int computeUnits = 0;
+    char name[256] = "";
+    hipStream_t stream = nullptr;
+    hipEvent_t evStart = nullptr, evStop = nullptr;
+    DevMip* tableDev = nullptr;        // device copy of the mip table
+    DevMip* tableHost = nullptr;       // pinned staging
+    size_t tableCapacity = 0;          // entries
+    std::vector<DevMip> lastTable;     // what tableDev currently holds
+};
+Library g_lib;
+
+int require_init()
+{
+    if (!g_lib.initialized) {
+        set_error("ntc_hip_init has not been called (or found no HIP device).");
+        return NTC_HIP_ERR_NOT_INITIALIZED;
+    }
+    return 0;
+}
+
+bool spec_equal(NtcHipDecoderSpec const& a, NtcHipDecoderSpec const& b) { return std::memcmp(&a, &b, sizeof(a)) == 0; }
+
+int layer_in(NtcHipDecoderSpec const& s, int l) { return l == 0 ? s.inputChannels : s.hiddenChannels[l - 1]; }
+int layer_out(NtcHipDecoderSpec const& s, int l) { return l == NTC_HIP_MLP_LAYERS - 1 ? s.outputChannels : s.hiddenChannels[l]; }
+
+bool spec_sane(NtcHipDecoderSpec const& s)
+{
+    auto widthOk = [](int w) { return w >= 16 && w <= NTC_HIP_MAX_LAYER_WIDTH && (w % 16) == 0; };
+    if (!widthOk(s.inputChannels) || s.outputChannels != 16) return false;
+    for (int l = 0; l < NTC_HIP_MLP_LAYERS - 1; ++l) if (!widthOk(s.hiddenChannels[l])) return false;
+    if ((s.hrBits != 2 && s.hrBits != 4) || (s.lrBits != 2 && s.lrBits != 4)) return false;
+    if (s.hrFeatures < 1 || s.lrFeatures < 1 || s.hrFeatures > s.hrFeatureSlots || s.lrFeatures > s.lrFeatureSlots) return false;
+    if (s.weightType != NTC_HIP_WEIGHTS_INT8 && s.weightType != NTC_HIP_WEIGHTS_FP8) return false;
+    return true;
+}
+
+// Which compiled kernel covers this spec.
+int pick_variant(NtcHipDecoderSpec const& s)
+{
+    if (s.weightType != NTC_HIP_WEIGHTS_INT8 || s.posEncWaves != 3 || s.outputChannels != 16) return NTC_HIP_VARIANT_NONE;
+    if (s.lrMode != NTC_HIP_GRID_BILINEAR || s.lrBits != 4) return NTC_HIP_VARIANT_NONE;
+    bool const concat8x2 = s.hrMode == NTC_HIP_GRID_CONCAT2X2 && s.hrFeatures == 8 && s.hrBits == 2 && s.hrFeatureSlots == 8;
+    if (concat8x2 && s.lodInputs == 0 && s.inputChannels == 64 && s.hiddenChannels[2] == 32) {
+        if (s.lrFeatures == 16 && s.lrFeatureSlots == 16 && s.hiddenChannels[0] == 64 && s.hiddenChannels[1] == 48)
+            return NTC_HIP_VARIANT_CFG01;
+        if (s.lrFeatures == 12 && s.lrFeatureSlots == 12 && s.hiddenChannels[0] == 48 && s.hiddenChannels[1] == 48)
+            return NTC_HIP_VARIANT_CFG2;
+    }
+    bool const ref = s.hrMode == NTC_HIP_GRID_BILINEAR && s.hrBits == 4 && s.hrFeatureSlots == 16 && s.lrFeatureSlots == 16
+        && s.hrFeatures == s.lrFeatures && s.lodInputs == 2 && s.inputChannels == 48
+        && s.hiddenChannels[0] == 64 && s.hiddenChannels[1] == 48 && s.hiddenChannels[2] == 32;
+    if (ref) {
+        switch (s.hrFeatures) {
+        case 16: return NTC_HIP_VARIANT_REF16;
+        case 12: return NTC_HIP_VARIANT_REF12;
+        case 8:  return NTC_HIP_VARIANT_REF8;
+        case 4:  return NTC_HIP_VARIANT_REF4;
+        default: break;
+        }
+    }
+    return NTC_HIP_VARIANT_NONE;
+}
+
+uint64_t grid_bytes(int32_t w, int32_t h, int32_t features, int32_t bits)
+{
+    if (w <= 0 || h <= 0 || features <= 0 || (bits != 2 && bits != 4)) return 0;
+    int const perWord = 16 / bits;
+    return uint64_t(w) * uint64_t(h) * 2u * uint64_t((features + perWord - 1) / perWord);
+}
+
+// Validates the sets, builds the mip table (sorted by tileStart) and picks the kernel.
+int build_table(NtcHipTextureSet const* sets, int32_t numSets, std::vector<DevMip>& table, int& variant, int& totalTiles)
+{
+    if (!sets || numSets < 1) { set_error("ntc_hip_decode: no texture sets given."); return NTC_HIP_ERR_INVALID_ARG; }
+    table.clear();
+    totalTiles = 0;
+    for (int s = 0; s < numSets; ++s) {
+        NtcHipTextureSet const& set = sets[s];
+        if (!spec_sane(set.spec)) { set_error("ntc_hip_decode: set %d has a malformed decoder spec.", s); return NTC_HIP_ERR_INVALID_ARG; }
+        if (!spec_equal(set.spec, sets[0].spec)) {
+            set_error("ntc_hip_decode: all sets of one call must share one decoder spec (set %d differs).", s);
+            return NTC_HIP_ERR_INVALID_ARG;
+        }
+        if (set.numMips < 1 || set.numMips > NTC_HIP_MAX_MIPS) { set_error("ntc_hip_decode: set %d: numMips %d out of range 1..%d.", s, set.numMips, NTC_HIP_MAX_MIPS); return NTC_HIP_ERR_INVALID_ARG; }
+        if (set.numChannels < 1 || set.numChannels > NTC_HIP_MAX_CHANNELS) { set_error("ntc_hip_decode: set %d: numChannels %d out of range 1..%d.", s, set.numChannels, NTC_HIP_MAX_CHANNELS); return NTC_HIP_ERR_INVALID_ARG; }
+        if (!set.latents || !set.weights || !set.output) { set_error("ntc_hip_decode: set %d: null latents / weights / output pointer.", s); return NTC_HIP_ERR_INVALID_ARG; }
+        if (set.outputFormat < NTC_HIP_OUT_FP16_PLANAR_PAIRS || set.outputFormat > NTC_HIP_OUT_UNORM8_PIXELS) { set_error("ntc_hip_decode: set %d: unknown output format %d.", s, set.outputFormat); return NTC_HIP_ERR_INVALID_ARG; }
+        if ((reinterpret_cast<uintptr_t>(set.weights) & 3u) || (reinterpret_cast<uintptr_t>(set.latents) & 1u)) { set_error("ntc_hip_decode: set %d: weights must be 4-byte and latents 2-byte aligned.", s); return NTC_HIP_ERR_INVALID_ARG; }
+        NtcHipWeightLayout layout;
+        if (ntc_hip_weight_layout(&set.spec, &layout) != 0) return NTC_HIP_ERR_INVALID_ARG;
+        if (set.weightsBytes < layout.bufferSize) {
+            set_error("ntc_hip_decode: set %d: weight blob holds %llu bytes, the spec needs %u.", s,
+                      (unsigned long long)set.weightsBytes, layout.bufferSize);
+            return NTC_HIP_ERR_INVALID_ARG;
+        }
+        int const bytesPerChannel = set.outputFormat == NTC_HIP_OUT_UNORM8_PIXELS ? 1 : 2;
+        if (set.outputFormat != NTC_HIP_OUT_FP16_PLANAR_PAIRS && set.outPixelStride < set.numChannels * bytesPerChannel) {
+            set_error("ntc_hip_decode: set %d: pixel stride %d is smaller than %d channels.", s, set.outPixelStride, set.numChannels);
+            return NTC_HIP_ERR_INVALID_ARG;
+        }
+        for (int m = 0; m < set.numMips; ++m) {
+            NtcHipMipDesc const& d = set.mips[m];
+            if (d.width < 1 || d.height < 1 || d.hrWidth < 1 || d.hrHeight < 1 || d.lrWidth < 1 || d.lrHeight < 1
+                || d.width > 65536 || d.height > 65536) {
+                set_error("ntc_hip_decode: set %d mip %d: bad dimensions.", s, m);
+                return NTC_HIP_ERR_INVALID_ARG;
+            }
+            if ((d.hrOffset & 1u) || (d.lrOffset & 1u)) { set_error("ntc_hip_decode: set %d mip %d: latent offsets must be even.", s, m); return NTC_HIP_ERR_INVALID_ARG; }
+            if (set.outputFormat == NTC_HIP_OUT_FP16_PLANAR_PAIRS) {
+                if (d.outOffset & 3u) { set_error("ntc_hip_decode: set %d mip %d: planar output offset must be 4-byte aligned.", s, m); return NTC_HIP_ERR_INVALID_ARG; }
+            } else if (d.outRowPitch < uint64_t(d.width) * uint64_t(set.outPixelStride)) {
+                set_error("ntc_hip_decode: set %d mip %d: row pitch smaller than a row.", s, m);
+                return NTC_HIP_ERR_INVALID_ARG;
+            }
+            uint64_t const hrBytes = grid_bytes(d.hrWidth, d.hrHeight, set.spec.hrFeatures, set.spec.hrBits);
+            uint64_t const lrBytes = grid_bytes(d.lrWidth, d.lrHeight, set.spec.lrFeatures, set.spec.lrBits);
+            if (d.hrOffset + hrBytes > set.latentsBytes || d.lrOffset + lrBytes > set.latentsBytes) {
+                set_error("ntc_hip_decode: set %d mip %d: a latent grid reaches past the %llu-byte latent buffer.", s, m,
+                          (unsigned long long)set.latentsBytes);
+                return NTC_HIP_ERR_INVALID_ARG;
+            }
+            uint64_t outBytes;
+            if (set.outputFormat == NTC_HIP_OUT_FP16_PLANAR_PAIRS)
+                outBytes = uint64_t(d.width) * uint64_t(d.height) * uint64_t((set.numChannels + 1) & ~1) * 2u;
+            else
+                outBytes = uint64_t(d.height - 1) * d.outRowPitch + uint64_t(d.width - 1) * uint64_t(set.outPixelStride)
+                         + uint64_t(set.numChannels * bytesPerChannel);
+            if (d.outOffset + outBytes > set.outputBytes) {
+                set_error("ntc_hip_decode: set %d mip %d: output reaches past the %llu-byte output buffer.", s, m,
+                          (unsigned long long)set.outputBytes);
+                return NTC_HIP_ERR_INVALID_ARG;
+            }
+            DevMip e{};
+            e.hr = reinterpret_cast<uint16_t const*>(static_cast<uint8_t const*>(set.latents) + d.hrOffset);
+            e.lr = reinterpret_cast<uint16_t const*>(static_cast<uint8_t const*>(set.latents) + d.lrOffset);
+            e.out = static_cast<uint8_t*>(set.output) + d.outOffset;
+            e.weights = static_cast<uint8_t const*>(set.weights);
+            e.outRowPitch = d.outRowPitch;
+            e.width = d.width; e.height = d.height;
+            e.hrWidth = d.hrWidth; e.hrHeight = d.hrHeight; e.lrWidth = d.lrWidth; e.lrHeight = d.lrHeight;
+            e.positionScale = d.positionScale; e.positionLod = d.positionLod;
+            e.outPixelStride = set.outPixelStride; e.numChannels = set.numChannels; e.outFormat = set.outputFormat;
+            e.tilesX = (d.width + kTileWidth - 1) / kTileWidth;
+            e.tilesY = (d.height + kTileHeight - 1) / kTileHeight;
+            e.tileStart = totalTiles;
+            long long const next = (long long)totalTiles + (long long)e.tilesX * e.tilesY;
+            if (next > 0x7fffffffLL) { set_error("ntc_hip_decode: too many tiles in one call."); return NTC_HIP_ERR_INVALID_ARG; }
+            totalTiles = int(next);
+            table.push_back(e);
+        }
+    }
+    variant = pick_variant(sets[0].spec);
+    if (variant == NTC_HIP_VARIANT_NONE) {
+        set_error("ntc_hip_decode: no compiled kernel covers this decoder spec "
+                  "(weights %d, HR %dx%d-bit mode %d, LR %dx%d-bit mode %d, lod %d, MLP %d-%d-%d-%d-%d).",
+                  sets[0].spec.weightType, sets[0].spec.hrFeatures, sets[0].spec.hrBits, sets[0].spec.hrMode,
+                  sets[0].spec.lrFeatures, sets[0].spec.lrBits, sets[0].spec.lrMode, sets[0].spec.lodInputs,
+                  sets[0].spec.inputChannels, sets[0].spec.hiddenChannels[0], sets[0].spec.hiddenChannels[1],
+                  sets[0].spec.hiddenChannels[2], sets[0].spec.outputChannels);
+        return NTC_HIP_ERR_UNSUPPORTED;
+    }
+    return 0;
+}
+
+// Makes the device table hold `table` (re-uploads only when it changed).
+int upload_table(std::vector<DevMip> const& table)
+{
+    Library& L = g_lib;
+    if (table.size() > L.tableCapacity) {
+        size_t const cap = table.size() * 2 + 16;
+        if (L.tableDev)  { HIP_TRY(hipStreamSynchronize(L.stream)); HIP_TRY(hipFree(L.tableDev)); L.tableDev = nullptr; }
+        if (L.tableHost) { HIP_TRY(hipHostFree(L.tableHost)); L.tableHost = nullptr; }
+        L.tableCapacity = 0; L.lastTable.clear();
+        HIP_TRY(hipMalloc(reinterpret_cast<void**>(&L.tableDev), cap * sizeof(DevMip)));
+        HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&L.tableHost), cap * sizeof(DevMip), hipHostMallocDefault));
+        L.tableCapacity = cap;
+    }
+    bool const same = L.lastTable.size() == table.size()
+        && std::memcmp(L.lastTable.data(), table.data(), table.size() * sizeof(DevMip)) == 0;
+    if (!same) {
+        // The pinned staging copy may still be in flight for an earlier launch.
+        HIP_TRY(hipStreamSynchronize(L.stream));
+        std::memcpy(L.tableHost, table.data(), table.size() * sizeof(DevMip));
+        HIP_TRY(hipMemcpyAsync(L.tableDev, L.tableHost, table.size() * sizeof(DevMip), hipMemcpyHostToDevice, L.stream));
+        L.lastTable = table;
+    }
+    return 0;
+}
+
+int grid_size_for(int totalTiles)
+{
+    // Persistent workgroups: two per compute unit (launch bounds keep 2 x 4 waves resident).
+    int const resident = g_lib.computeUnits * 2;
+    return totalTiles < resident ? totalTiles : resident;
+}
+
+} // namespace
+
+extern "C" {
+
+int ntc_hip_init(int device)
+{
+    clear_error();
+    int count = 0;
+    hipError_t err = hipGetDeviceCount(&count);
+    if (err != hipSuccess || count == 0) {
+        set_error("No HIP device is available (hipGetDeviceCount: %s).", hipGetErrorName(err));
+        return NTC_HIP_ERR_NO_DEVICE;
+    }
+    if (device < 0 || device >= count) { set_error("ntc_hip_init: device %d out of range 0..%d.", device, count - 1); return NTC_HIP_ERR_INVALID_ARG; }
+    if (g_lib.initialized) {
+        if (g_lib.device == device) return 0;
+        ntc_hip_shutdown();
+    }
+    HIP_TRY(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, device));
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        set_error("ntc_hip_init: device %d is %s; this library holds gfx950 code only.", device, prop.gcnArchName);
+        return NTC_HIP_ERR_UNSUPPORTED;
+    }
+    g_lib.device = device;
+    g_lib.computeUnits = prop.multiProcessorCount;
+    std::snprintf(g_lib.name, sizeof(g_lib.name), "%s (%s)", prop.name, prop.gcnArchName);
+    HIP_TRY(hipStreamCreate(&g_lib.stream));
+    HIP_TRY(hipEventCreate(&g_lib.evStart));
+    HIP_TRY(hipEventCreate(&g_lib.evStop));
+    g_lib.initialized = true;
+    return 0;
+}
+
+void ntc_hip_shutdown(void)
+{
+    if (!g_lib.initialized) return;
+    (void)hipStreamSynchronize(g_lib.stream);
+    if (g_lib.tableDev) (void)hipFree(g_lib.tableDev);
+    if (g_lib.tableHost) (void)hipHostFree(g_lib.tableHost);
+    (void)hipEventDestroy(g_lib.evStart);
+    (void)hipEventDestroy(g_lib.evStop);
+    (void)hipStreamDestroy(g_lib.stream);
+    g_lib = Library();
+}
+
+const char* ntc_hip_last_error(void) { return t_error; }
+
+int ntc_hip_device_info(char* name, size_t nameSize, int* computeUnits)
+{
+    if (int r = require_init()) return r;
+    if (name && nameSize) { std::snprintf(name, nameSize, "%s", g_lib.name); }
+    if (computeUnits) *computeUnits = g_lib.computeUnits;
+    return 0;
+}
+
+int ntc_hip_alloc(void** devPtr, size_t bytes)
+{
+    if (int r = require_init()) return r;
+    if (!devPtr) { set_error("ntc_hip_alloc: null out-pointer."); return NTC_HIP_ERR_INVALID_ARG; }
+    *devPtr = nullptr;
+    HIP_TRY(hipMalloc(devPtr, bytes ? bytes : 1));
+    return 0;
+}
+
+int ntc_hip_free(void* devPtr)
+{
+    if (int r = require_init()) return r;
+    if (!devPtr) return 0;
+    HIP_TRY(hipStreamSynchronize(g_lib.stream));
+    HIP_TRY(hipFree(devPtr));
+    return 0;
+}
+
+int ntc_hip_upload(void* dst, const void* src, size_t bytes)
+{
+    if (int r = require_init()) return r;
+    if (bytes == 0) return 0;
+    if (!dst || !src) { set_error("ntc_hip_upload: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
+    HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g_lib.stream));
+    HIP_TRY(hipStreamSynchronize(g_lib.stream));
+    return 0;
+}
+
+int ntc_hip_download(void* dst, const void* src, size_t bytes)
+{
+    if (int r = require_init()) return r;
+    if (bytes == 0) return 0;
+    if (!dst || !src) { set_error("ntc_hip_download: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
+    HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g_lib.stream));
+    HIP_TRY(hipStreamSynchronize(g_lib.stream));
+    return 0;
+}
+
+int ntc_hip_memset(void* dst, int value, size_t bytes)
+{
+    if (int r = require_init()) return r;
+    if (bytes == 0) return 0;
+    if (!dst) { set_error("ntc_hip_memset: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
+    HIP_TRY(hipMemsetAsync(dst, value, bytes, g_lib.stream));
+    return 0;
+}
+
+int ntc_hip_synchronize(void)
+{
+    if (int r = require_init()) return r;
+    HIP_TRY(hipStreamSynchronize(g_lib.stream));
+    return 0;
+}
+
+int ntc_hip_weight_layout(const NtcHipDecoderSpec* spec, NtcHipWeightLayout* out)
+{
+    if (!spec || !out) { set_error("ntc_hip_weight_layout: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
+    if (!spec_sane(*spec)) { set_error("ntc_hip_weight_layout: malformed decoder spec."); return NTC_HIP_ERR_INVALID_ARG; }
+    std::memset(out, 0, sizeof(*out));
+    uint32_t cursor = 0;
+    // Matrices first, one byte per weight, layer after layer (src/WeightLayout.cpp:157-176).
+    for (int l = 0; l < NTC_HIP_MLP_LAYERS; ++l) {
+        out->weightOffset[l] = cursor;
+        cursor += uint32_t(layer_in(*spec, l)) * uint32_t(layer_out(*spec, l));
+    }
+    if (spec->weightType == NTC_HIP_WEIGHTS_INT8) {
+        // then every scale vector, then every bias vector (src/WeightLayout.cpp:229-247)
+        for (int l = 0; l < NTC_HIP_MLP_LAYERS; ++l) { out->scaleOffset[l] = cursor; cursor += 4u * uint32_t(layer_out(*spec, l)); }
+        for (int l = 0; l < NTC_HIP_MLP_LAYERS; ++l) { out->biasOffset[l] = cursor; cursor += 4u * uint32_t(layer_out(*spec, l)); }
+    } else {
+        // fp16 bias of the e4m3 layers, then scale and bias of the int8 output layer (src/WeightLayout.cpp:249-262)
+        int const last = NTC_HIP_MLP_LAYERS - 1;
+        for (int l = 0; l < last; ++l) { out->biasOffset[l] = cursor; cursor += 2u * uint32_t(layer_out(*spec, l)); }
+        out->scaleOffset[last] = cursor; cursor += 4u * uint32_t(layer_out(*spec, last));
+        out->biasOffset[last] = cursor;  cursor += 4u * uint32_t(layer_out(*spec, last));
+    }
+    out->bufferSize = cursor;
+    return 0;
+}
+
+uint64_t ntc_hip_grid_bytes(int32_t width, int32_t height, int32_t features, int32_t bits)
+{
+    return grid_bytes(width, height, features, bits);
+}
+
+int ntc_hip_decode(const NtcHipTextureSet* sets, int32_t numSets)
+{
+    if (int r = require_init()) return r;
+    std::vector<DevMip> table;
+    int variant = NTC_HIP_VARIANT_NONE, totalTiles = 0;
+    if (int r = build_table(sets, numSets, table, variant, totalTiles)) return r;
+    if (int r = upload_table(table)) return r;
+    HIP_TRY(launch_decode(variant, g_lib.tableDev, int(table.size()), totalTiles, grid_size_for(totalTiles), g_lib.stream));
+    clear_error();
+    return 0;
+}
+
+int ntc_hip_decode_timed(const NtcHipTextureSet* sets, int32_t numSets, int32_t iterations, float* outMs)
+{
+    if (int r = require_init()) return r;
+    if (iterations < 1 || !outMs) { set_error("ntc_hip_decode_timed: iterations must be >= 1 and the result pointer non-null."); return NTC_HIP_ERR_INVALID_ARG; }
+    std::vector<DevMip> table;
+    int variant = NTC_HIP_VARIANT_NONE, totalTiles = 0;
+    if (int r = build_table(sets, numSets, table, variant, totalTiles)) return r;
+    if (int r = upload_table(table)) return r;
+    int const grid = grid_size_for(totalTiles);
+    HIP_TRY(hipEventRecord(g_lib.evStart, g_lib.stream));
+    for (int i = 0; i < iterations; ++i)
+        HIP_TRY(launch_decode(variant, g_lib.tableDev, int(table.size()), totalTiles, grid, g_lib.stream));
+    HIP_TRY(hipEventRecord(g_lib.evStop, g_lib.stream));
+    HIP_TRY(hipEventSynchronize(g_lib.evStop));
+    float ms = 0.f;
+    HIP_TRY(hipEventElapsedTime(&ms, g_lib.evStart, g_lib.evStop));
+    *outMs = ms / float(iterations);
+    clear_error();
+    return 0;
+}
+
+int ntc_hip_selftest_mfma(const int8_t* a16x64, const int8_t* b64x16, int32_t* d16x16)
+{
+    if (int r = require_init()) return r;
+    if (!a16x64 || !b64x16 || !d16x16) { set_error("ntc_hip_selftest_mfma: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
+    int8_t *a = nullptr, *b = nullptr; int32_t* d = nullptr;
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&a), 1024));
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&b), 1024));
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&d), 1024));
+    HIP_TRY(hipMemcpy(a, a16x64, 1024, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(b, b64x16, 1024, hipMemcpyHostToDevice));
+    HIP_TRY(launch_selftest_mfma(a, b, d, g_lib.stream));
+    HIP_TRY(hipStreamSynchronize(g_lib.stream));
+    HIP_TRY(hipMemcpy(d16x16, d, 1024, hipMemcpyDeviceToHost));
+    (void)hipFree(a); (void)hipFree(b); (void)hipFree(d);
+    return 0;
+}
+
+} // extern "C"

@@ -1,0 +1,85 @@
+"""Device-side plumbing over the C ABI: buffers, texture-set assembly, decode calls."""
+import ctypes as C
+
+import numpy as np
+
+from . import abi, presets
+
+
+class Device:
+    """ntc_hip_init on construction; raises NtcHipError when there is no gfx950 device."""
+
+    def __init__(self, index=0):
+        self.lib = abi.load_library()
+        abi.check(self.lib.ntc_hip_init(index))
+        name = C.create_string_buffer(256)
+        cus = C.c_int(0)
+        abi.check(self.lib.ntc_hip_device_info(name, 256, C.byref(cus)))
+        self.name = name.value.decode()
+        self.compute_units = cus.value
+
+    def alloc(self, nbytes):
+        return DeviceBuffer(self, nbytes)
+
+    def upload(self, array):
+        array = np.ascontiguousarray(array)
+        buf = DeviceBuffer(self, array.nbytes)
+        abi.check(self.lib.ntc_hip_upload(buf.ptr, array.ctypes.data, array.nbytes))
+        return buf
+
+    def synchronize(self):
+        abi.check(self.lib.ntc_hip_synchronize())
+
+    def decode(self, sets):
+        arr = (abi.TextureSet * len(sets))(*sets)
+        abi.check(self.lib.ntc_hip_decode(arr, len(sets)))
+
+    def decode_timed(self, sets, iterations):
+        arr = (abi.TextureSet * len(sets))(*sets)
+        ms = C.c_float(0)
+        abi.check(self.lib.ntc_hip_decode_timed(arr, len(sets), iterations, C.byref(ms)))
+        return ms.value
+
+
+class DeviceBuffer:
+    def __init__(self, device, nbytes):
+        self.device = device
+        self.nbytes = int(nbytes)
+        p = C.c_void_p()
+        abi.check(device.lib.ntc_hip_alloc(C.byref(p), self.nbytes))
+        self.ptr = p.value
+
+    def download(self, dtype=np.uint8):
+        out = np.empty(self.nbytes, dtype=np.uint8)
+        abi.check(self.device.lib.ntc_hip_download(out.ctypes.data, self.ptr, self.nbytes))
+        return out.view(dtype)
+
+    def fill(self, value):
+        abi.check(self.device.lib.ntc_hip_memset(self.ptr, value, self.nbytes))
+
+    def free(self):
+        if self.ptr:
+            abi.check(self.device.lib.ntc_hip_free(self.ptr))
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def make_texture_set(spec, mips, num_channels, output_format, latents_ptr, latents_bytes,
+                     weights_ptr, weights_bytes, output_ptr, output_bytes, pixel_stride=0):
+    """Fills an abi.TextureSet from already-placed buffers (device or host addresses)."""
+    ts = abi.TextureSet()
+    ts.spec = spec.copy()
+    ts.numMips = len(mips)
+    ts.numChannels = num_channels
+    ts.outputFormat = output_format
+    ts.outPixelStride = pixel_stride
+    ts.latents, ts.weights, ts.output = latents_ptr, weights_ptr, output_ptr
+    ts.latentsBytes, ts.weightsBytes, ts.outputBytes = latents_bytes, weights_bytes, output_bytes
+    for i, d in enumerate(mips):
+        C.memmove(C.byref(ts.mips[i]), C.byref(d), C.sizeof(abi.MipDesc))
+    return ts

@@ -1,0 +1,42 @@
+"""Seeded synthetic latents and weight blobs (there are no .ntc sample files to decode).
+
+Distributions follow the benchmark description: latent codes uniform over the code range;
+int8 weights uniform in [-127, 127]; per-channel fp32 scale log-uniform in [2^-10, 2^-4];
+fp32 bias ~ N(0, 0.1), stored the way the reference's quantiser stores a float bias:
+bias_i32 = roundf(bias / scale) (src/Quantizer.cu:202).
+"""
+import numpy as np
+
+from . import abi
+
+
+def make_latents(total_bytes, seed):
+    rng = np.random.default_rng(seed)
+    return rng.integers(0, 65536, size=total_bytes // 2, dtype=np.uint16)
+
+
+def weight_layout(spec):
+    """Offsets of the blob pieces, from the library's own host-side layout helper."""
+    lib = abi.load_library()
+    layout = abi.WeightLayout()
+    abi.check(lib.ntc_hip_weight_layout(spec, layout))
+    return layout
+
+
+def make_weights(spec, seed, scale_log2_range=(-10.0, -4.0), bias_sigma=0.1, layout=None):
+    """Returns the int8 weight blob (uint8 array) for `spec`."""
+    assert spec.weightType == abi.WEIGHTS_INT8
+    layout = layout or weight_layout(spec)
+    rng = np.random.default_rng(seed)
+    blob = np.zeros(layout.bufferSize, dtype=np.uint8)
+    for layer in range(abi.MLP_LAYERS):
+        n_in, n_out = spec.layer_inputs(layer), spec.layer_outputs(layer)
+        w = rng.integers(-127, 128, size=(n_out, n_in), dtype=np.int8)
+        scale = np.exp2(rng.uniform(scale_log2_range[0], scale_log2_range[1], size=n_out)).astype(np.float32)
+        bias = rng.normal(0.0, bias_sigma, size=n_out).astype(np.float32)
+        q = (bias / scale).astype(np.float32).astype(np.float64)
+        bias_i32 = np.trunc(q + np.copysign(0.5, q)).astype(np.int32)      # roundf
+        blob[layout.weightOffset[layer]:layout.weightOffset[layer] + n_in * n_out] = w.reshape(-1).view(np.uint8)
+        blob[layout.scaleOffset[layer]:layout.scaleOffset[layer] + 4 * n_out] = scale.view(np.uint8)
+        blob[layout.biasOffset[layer]:layout.biasOffset[layer] + 4 * n_out] = bias_i32.view(np.uint8)
+    return blob

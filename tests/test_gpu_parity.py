@@ -1,0 +1,136 @@
+"""GPU parity: the HIP decoder, called through the C ABI, against the CPU checker on the
+same seeded inputs.  Integer/byte work: every output byte must be equal."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from cases import cfg_case, ref_case, first_mismatch
+
+pytestmark = pytest.mark.gpu
+
+# scale range that keeps layer outputs inside the active part of HGELU (|x| of a few units)
+# instead of saturating it, so rounding in the requantiser is exercised
+ACTIVE = (-17.0, -12.0)
+
+
+def run_both(device, case):
+    host = case.host_set()
+    host.decode(threads=8)
+    dset = case.device_set(device)
+    device.decode([dset])
+    device.synchronize()
+    got = case.d_output.download()
+    return host.output, got
+
+
+def assert_equal_bytes(expected, got, what):
+    mm = first_mismatch(expected, got)
+    assert mm is None, f"{what}: {mm[1]} of {expected.size} bytes differ, first at {mm[0]}: oracle {mm[2]} gpu {mm[3]}"
+
+
+def test_mfma_operand_layout(device):
+    rng = np.random.default_rng(5)
+    a = rng.integers(-128, 128, size=(16, 64), dtype=np.int8)
+    b = rng.integers(-128, 128, size=(64, 16), dtype=np.int8)
+    d = np.zeros((16, 16), dtype=np.int32)
+    from importlib import import_module
+    abi = import_module("rtxntc-library_amd").abi
+    abi.check(device.lib.ntc_hip_selftest_mfma(a.ctypes.data, b.ctypes.data, d.ctypes.data))
+    assert np.array_equal(d, a.astype(np.int64) @ b.astype(np.int64))
+
+
+@pytest.mark.parametrize("scale_range", [(-10.0, -4.0), ACTIVE])
+def test_cfg0_plumbing_512_fp16(ntc, device, scale_range):
+    """BASELINE config 0: 512x512, one mip, 8 channels, 64-48-32 int8, fp16 planar output."""
+    case = cfg_case(ntc, ntc.presets.spec_cfg01(), 512, 512, 1, 8, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=0,
+                    scale_log2_range=scale_range)
+    expected, got = run_both(device, case)
+    assert_equal_bytes(expected, got, "cfg0")
+
+
+@pytest.mark.parametrize("fmt", ["planar", "fp16px", "unorm8"])
+def test_cfg1_shape_small_full_mip_chain(ntc, device, fmt):
+    """Config 1's shape at 256x256: full mip chain down to 1x1, 16 channels, all output formats."""
+    f = {"planar": ntc.abi.OUT_FP16_PLANAR_PAIRS, "fp16px": ntc.abi.OUT_FP16_PIXELS, "unorm8": ntc.abi.OUT_UNORM8_PIXELS}[fmt]
+    case = cfg_case(ntc, ntc.presets.spec_cfg01(), 256, 256, 9, 16, f, seed=11, scale_log2_range=ACTIVE)
+    expected, got = run_both(device, case)
+    assert_equal_bytes(expected, got, f"cfg1-small {fmt}")
+
+
+@pytest.mark.parametrize("w,h,ch", [(100, 36, 7), (67, 5, 16), (1, 1, 3), (130, 130, 10), (16, 300, 1)])
+def test_ragged_sizes_and_channel_counts(ntc, device, w, h, ch):
+    """Non-power-of-two sizes (the general fp32 sampling path), tile tails, odd channel counts."""
+    for f in (ntc.abi.OUT_FP16_PLANAR_PAIRS, ntc.abi.OUT_FP16_PIXELS, ntc.abi.OUT_UNORM8_PIXELS):
+        case = cfg_case(ntc, ntc.presets.spec_cfg01(), w, h, ntc.presets.full_mip_count(w, h), ch, f, seed=w * 31 + h,
+                        scale_log2_range=ACTIVE)
+        expected, got = run_both(device, case)
+        # bytes the decoder must not touch keep the fill pattern on the GPU and zero on the host
+        touched = expected != 0
+        assert_equal_bytes(expected[touched], got[touched], f"ragged {w}x{h}x{ch} fmt {f}")
+
+
+@pytest.mark.parametrize("features,grid_scale", [(16, 2), (8, 4), (12, 3), (4, 1)])
+def test_ref092_geometry(ntc, device, features, grid_scale):
+    """The mounted LibNTC 0.9.2 decoder: both grids bilinear 4-bit, shared neural LODs, (lod, lod) inputs."""
+    spec = ntc.presets.spec_ref092(features)
+    case = ref_case(ntc, spec, 192, 128, 8, grid_scale, 10, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=features,
+                    scale_log2_range=ACTIVE)
+    expected, got = run_both(device, case)
+    assert_equal_bytes(expected, got, f"ref092 f{features} gs{grid_scale}")
+
+
+def test_cfg2_batch_of_sets(ntc, device):
+    """Config 2's shape, small: several sets with their own weights and latents in one launch."""
+    spec = ntc.presets.spec_cfg2()
+    cases = [cfg_case(ntc, spec, 128, 128, 8, 12, ntc.abi.OUT_UNORM8_PIXELS, seed=100 + i, scale_log2_range=ACTIVE)
+             for i in range(5)]
+    hosts = [c.host_set() for c in cases]
+    for hset in hosts:
+        hset.decode(threads=8)
+    dsets = [c.device_set(device) for c in cases]
+    device.decode(dsets)
+    device.synchronize()
+    for i, (c, hset) in enumerate(zip(cases, hosts)):
+        assert_equal_bytes(hset.output, c.d_output.download(), f"cfg2 set {i}")
+
+
+def test_extreme_weights_saturate_cleanly(ntc, device):
+    """All-(-127)/127 weights with the largest scale and huge biases: accumulators near their
+    extremes, activations pinned at both ends of the quantiser."""
+    spec = ntc.presets.spec_cfg01()
+    layout = ntc.synth.weight_layout(spec)
+    blob = ntc.synth.make_weights(spec, 3, scale_log2_range=(-4.0, -4.0))
+    w = blob[:layout.scaleOffset[0]].view(np.int8)
+    w[:] = np.where(np.arange(w.size) % 3 == 0, -127, 127)
+    bias = blob[layout.biasOffset[0]:layout.bufferSize].view(np.int32)
+    bias[::2] = 2 ** 30
+    bias[1::2] = -(2 ** 30)
+    case = cfg_case(ntc, spec, 64, 64, 1, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=9, weights=blob)
+    expected, got = run_both(device, case)
+    assert_equal_bytes(expected, got, "extreme weights")
+
+
+def test_decode_is_idempotent_and_timed_variant_matches(ntc, device):
+    case = cfg_case(ntc, ntc.presets.spec_cfg01(), 320, 200, 4, 16, ntc.abi.OUT_UNORM8_PIXELS, seed=21, scale_log2_range=ACTIVE)
+    dset = case.device_set(device)
+    device.decode([dset])
+    device.synchronize()
+    first = case.d_output.download().copy()
+    ms = device.decode_timed([dset], 3)
+    assert ms > 0
+    assert np.array_equal(first, case.d_output.download())
+
+
+def test_argument_errors_are_reported(ntc, device):
+    case = cfg_case(ntc, ntc.presets.spec_cfg01(), 64, 64, 1, 8, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=1)
+    dset = case.device_set(device)
+    dset.latentsBytes = 16
+    with pytest.raises(ntc.NtcHipError) as e:
+        device.decode([dset])
+    assert e.value.code == ntc.abi.ERR_INVALID_ARG and "latent" in e.value.message
+    dset = case.device_set(device)
+    dset.spec.hiddenChannels[0] = 32
+    with pytest.raises(ntc.NtcHipError) as e:
+        device.decode([dset])
+    assert e.value.code in (ntc.abi.ERR_UNSUPPORTED, ntc.abi.ERR_INVALID_ARG)
