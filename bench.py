@@ -75,7 +75,7 @@ def main():
         host = case.host_set()
         from oracle_lib import load_oracle
         orc = load_oracle()
-        rows = 16
+        rows = 256
         t = orc.ntc_oracle_decode_rows(host.desc, 0, 0, rows, cores)          # calibrate
         rate = rows * size / t
         rows = int(max(rows, min(size, args.cpu_seconds * rate / size)))

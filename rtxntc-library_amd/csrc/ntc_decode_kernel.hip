@@ -118,6 +118,10 @@ __device__ __forceinline__ uint32_t activate4(v4i acc, v4f scale)
 
 __device__ __forceinline__ uint32_t to_half_bits(float o)
 {
+    // The network output is an fp32 product that is THEN rounded to half.  Without this
+    // barrier the compiler folds multiply + convert into v_fma_mixlo_f16, which rounds the
+    // exact product once, straight to half, and differs in rare double-rounding cases.
+    asm volatile("" : "+v"(o));
     _Float16 const h = (_Float16)o;                          // v_cvt_f16_f32, round-nearest-even
     uint32_t bits = uint32_t(__builtin_bit_cast(uint16_t, h));
     if ((bits & 0x7c00u) == 0x7c00u) bits = 0;               // IsHalfSpecial -> 0 (Inference.cu:125-126)

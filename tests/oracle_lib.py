@@ -74,10 +74,12 @@ def load_ref():
 class HostSet:
     """A texture set whose latents / weights / output live in numpy arrays (for the oracle)."""
 
+    FILL = 0xCD   # bytes the decoder must leave alone keep this pattern (same fill as the device buffer)
+
     def __init__(self, ntc, spec, mips, num_channels, output_format, latents, weights, output_bytes, pixel_stride=0):
         self.latents = np.ascontiguousarray(latents)
         self.weights = np.ascontiguousarray(weights)
-        self.output = np.zeros(output_bytes, dtype=np.uint8)
+        self.output = np.full(output_bytes, self.FILL, dtype=np.uint8)
         self.desc = ntc.make_texture_set(
             spec, mips, num_channels, output_format,
             self.latents.ctypes.data, self.latents.nbytes, self.weights.ctypes.data, self.weights.nbytes,

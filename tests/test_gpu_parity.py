@@ -65,9 +65,8 @@ def test_ragged_sizes_and_channel_counts(ntc, device, w, h, ch):
         case = cfg_case(ntc, ntc.presets.spec_cfg01(), w, h, ntc.presets.full_mip_count(w, h), ch, f, seed=w * 31 + h,
                         scale_log2_range=ACTIVE)
         expected, got = run_both(device, case)
-        # bytes the decoder must not touch keep the fill pattern on the GPU and zero on the host
-        touched = expected != 0
-        assert_equal_bytes(expected[touched], got[touched], f"ragged {w}x{h}x{ch} fmt {f}")
+        # includes padding and dropped channels: both sides start from the same fill pattern
+        assert_equal_bytes(expected, got, f"ragged {w}x{h}x{ch} fmt {f}")
 
 
 @pytest.mark.parametrize("features,grid_scale", [(16, 2), (8, 4), (12, 3), (4, 1)])
