@@ -26,7 +26,7 @@ INT8_PEAK_TOPS = 5000.0        # MI355X dense int8 MFMA
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--size", type=int, default=4096)
     ap.add_argument("--format", choices=["fp16", "unorm8"], default="fp16")
@@ -54,34 +54,42 @@ def main():
     bytes_per_texel = out_bytes_per_texel + (16 / 4 + 64 / 16) / 8.0
     ops_per_texel = 2 * (64 * 64 + 64 * 48 + 48 * 32 + 32 * 16)
 
+    sets = dev.pack_sets([dset])
     for _ in range(args.warmup):
-        dev.decode([dset])
+        dev.decode(sets)
     dev.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        dev.decode([dset])
+        dev.decode(sets)
     dev.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall / args.steps * 1e3
 
-    kernel_ms = dev.decode_timed([dset], args.steps)      # HIP events on the launch stream
+    kernel_ms = dev.decode_timed(sets, args.steps)      # HIP events on the launch stream
     gtexels = texels / (ms_per_step * 1e-3) / 1e9
     achieved_gbs = texels * bytes_per_texel / (kernel_ms * 1e-3) / 1e9
     achieved_tops = texels * ops_per_texel / (kernel_ms * 1e-3) / 1e12
 
     cpu = None
     if not args.no_cpu:
+        # The CPU checker (scalar C++ restatement, oracle/ntc_oracle.cpp) on this machine's host
+        # cores, over the WHOLE set when that fits the time budget, else over leading rows of mip 0.
         cores = min(16, os.cpu_count() or 1)
         host = case.host_set()
         from oracle_lib import load_oracle
         orc = load_oracle()
-        rows = 256
+        rows = min(256, size)
         t = orc.ntc_oracle_decode_rows(host.desc, 0, 0, rows, cores)          # calibrate
-        rate = rows * size / t
-        rows = int(max(rows, min(size, args.cpu_seconds * rate / size)))
-        t = orc.ntc_oracle_decode_rows(host.desc, 0, 0, rows, cores)
-        cpu = {"value": rows * size / t / 1e9, "unit": "Gtexels/s", "cores": cores, "kind": "port",
-               "sample": f"rows 0..{rows} of mip 0 ({rows * size} texels) of the same set, {t:.1f} s"}
+        est_full = t * texels / (rows * size)
+        if est_full <= args.cpu_seconds:
+            best = min(orc.ntc_oracle_decode(host.desc, cores) for _ in range(2))
+            cpu = {"value": texels / best / 1e9, "unit": "Gtexels/s", "cores": cores, "kind": "port",
+                   "sample": f"the whole set ({texels} texels), best of 2, {best:.2f} s"}
+        else:
+            rows = int(max(rows, min(size, args.cpu_seconds * rows / t)))
+            t = orc.ntc_oracle_decode_rows(host.desc, 0, 0, rows, cores)
+            cpu = {"value": rows * size / t / 1e9, "unit": "Gtexels/s", "cores": cores, "kind": "port",
+                   "sample": f"rows 0..{rows} of mip 0 ({rows * size} texels) of the same set, {t:.1f} s"}
 
     line = {
         "metric": "decoded Gtexels/s, 4096^2 16-ch set, 64-48-32 int8; % of int8-MFMA/HBM roof",

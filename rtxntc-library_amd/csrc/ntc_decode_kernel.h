@@ -35,11 +35,18 @@ struct DevMip {
     float   positionScale, positionLod;
     int32_t outPixelStride, numChannels, outFormat;
     int32_t tileStart, tilesX, tilesY;
+    // All-integer input stage, valid when `fast` is set (every size a power of two, positionScale
+    // a power of two).  An axis word packs, for p = u*grid - 1/2 = N / 2^n with
+    // N = ((2x+1) << shl) - (1 << sublog):  shl | n << 8 | sublog << 16 | log2(grid size) << 24.
+    uint32_t fast;
+    uint32_t hrAxisX, hrAxisY, lrAxisX, lrAxisY;
+    uint32_t posMask;          // (texels per period of the positional encoding) - 1
 };
 
 constexpr int kTileWidth = 64, kTileHeight = 4;
 
 hipError_t launch_decode(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream);
+int resident_workgroups_per_cu(int variant);
 hipError_t launch_selftest_mfma(int8_t const* a, int8_t const* b, int32_t* d, hipStream_t stream);
 
 } // namespace ntc_hip_dev

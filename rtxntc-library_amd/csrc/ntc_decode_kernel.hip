@@ -29,6 +29,24 @@
 namespace ntc_hip_dev {
 
 typedef int   v4i __attribute__((ext_vector_type(4)));
+// Latent grids live in global memory; saying so lets loads use "scalar base + 32-bit lane offset"
+// addressing instead of 64-bit flat addresses built per lane.
+typedef __attribute__((address_space(1))) uint16_t const* GlobalU16Ptr;
+typedef __attribute__((address_space(1))) uint8_t const*  GlobalU8Ptr;
+
+// One u16 at a uniform base plus a 32-bit byte offset per lane (global_load_ushort v, v_off, s[base]).
+__device__ __forceinline__ uint32_t load_u16(GlobalU8Ptr base, uint32_t byteOffset)
+{
+    return *reinterpret_cast<GlobalU16Ptr>(base + byteOffset);
+}
+
+// 24-bit multiply, full rate (the compiler otherwise picks the quarter-rate 32-bit multiply).
+__device__ __forceinline__ uint32_t mul24(uint32_t a, uint32_t b)
+{
+    uint32_t r;
+    asm("v_mul_u32_u24 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kWaves       = 4;     // waves per workgroup
@@ -99,44 +117,146 @@ __device__ __forceinline__ uint32_t bilinear4(Taps const& tp, uint32_t s00, uint
 }
 
 // HGELU-clamp + requantise of four D values of one lane (Inference.hlsli:36-39,123-131,164-179).
-// round-half-even of y*80 is taken from the low mantissa bits of y*80 + 1.5*2^23.
-__device__ __forceinline__ uint32_t activate4(v4i acc, v4f scale)
+// round-half-even of y*80 is taken from the low mantissa bits of y*80 + 1.5*2^23; the "-113"
+// (= +143 mod 256) and the byte packing are one SDWA integer add per value.
+__device__ __forceinline__ uint32_t activate4(v4i acc, v4f scale, uint32_t c143)
 {
-    uint32_t packed = 0;
+    float z[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         float const x = float(acc[r]) * scale[r];
         float t = __builtin_fmaf(x, 0.333333f, 0.5f);
         t = fminf(fmaxf(t, 0.f), 1.f);
         float const y = fminf(x, 3.f) * t;
-        float const z = y * 80.f;
-        uint32_t const q = __float_as_uint(z + 12582912.f);  // low byte = rne(z) mod 256
-        packed |= ((q + 143u) & 0xffu) << (8 * r);           // -113 mod 256
+        z[r] = y * 80.f + 12582912.f;                        // low byte = rne(y*80) mod 256
     }
+    uint32_t packed;
+    asm("v_add_u32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:BYTE_0 src1_sel:DWORD"
+        : "=v"(packed) : "v"(z[0]), "v"(c143));
+    asm("v_add_u32_sdwa %0, %1, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_0 src1_sel:DWORD"
+        : "+v"(packed) : "v"(z[1]), "v"(c143));
+    asm("v_add_u32_sdwa %0, %1, %2 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_0 src1_sel:DWORD"
+        : "+v"(packed) : "v"(z[2]), "v"(c143));
+    asm("v_add_u32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_0 src1_sel:DWORD"
+        : "+v"(packed) : "v"(z[3]), "v"(c143));
     return packed;
 }
 
-__device__ __forceinline__ uint32_t to_half_bits(float o)
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+typedef float    v2f __attribute__((ext_vector_type(2)));
+
+// Two network outputs -> two fp16 in one dword.  The output is an fp32 product that is THEN
+// rounded to half (round-nearest-even); a half that would be Inf/NaN is stored as zero
+// (IsHalfSpecial, Inference.cu:125-126).  |o| >= 65520 is exactly the set that rounds to
+// Inf.  The empty asm keeps the compiler from folding multiply + convert into
+// v_fma_mixlo_f16, which rounds the exact product once, straight to half.
+__device__ __forceinline__ uint32_t to_half2_bits(float a, float b)
 {
-    // The network output is an fp32 product that is THEN rounded to half.  Without this
-    // barrier the compiler folds multiply + convert into v_fma_mixlo_f16, which rounds the
-    // exact product once, straight to half, and differs in rare double-rounding cases.
-    asm volatile("" : "+v"(o));
-    _Float16 const h = (_Float16)o;                          // v_cvt_f16_f32, round-nearest-even
-    uint32_t bits = uint32_t(__builtin_bit_cast(uint16_t, h));
-    if ((bits & 0x7c00u) == 0x7c00u) bits = 0;               // IsHalfSpecial -> 0 (Inference.cu:125-126)
-    return bits;
+    asm("" : "+v"(a));
+    asm("" : "+v"(b));
+    a = (__builtin_fabsf(a) < 65520.f) ? a : 0.f;
+    b = (__builtin_fabsf(b) < 65520.f) ? b : 0.f;
+    v2h const h = __builtin_convertvector(v2f{a, b}, v2h);
+    return __builtin_bit_cast(uint32_t, h);
 }
 
-// WriteImageChannel UNORM8 (src/ImageProcessing.cu:146-149): roundf, clamp.
-__device__ __forceinline__ uint32_t half_bits_to_unorm8(uint32_t hbits)
+// WriteImageChannel UNORM8 (src/ImageProcessing.cu:146-149): u8(clamp(roundf(v * 255), 0, 255)) of
+// the stored half.  v*255 is exact (11-bit x 8-bit significands); for such values
+// floor(v*255 + 1/2) equals roundf(v*255) exactly, and the float->uint conversion truncates and
+// sends negatives to 0.
+__device__ __forceinline__ uint32_t half_to_unorm8(_Float16 h)
 {
-    float const v = float(__builtin_bit_cast(_Float16, uint16_t(hbits))) * 255.f;
-    float r = truncf(v);
-    float const fr = v - r;
-    if (fr >= 0.5f) r += 1.f; else if (fr <= -0.5f) r -= 1.f;
-    r = fminf(fmaxf(r, 0.f), 255.f);
-    return uint32_t(r);
+    float const v = float(h) * 255.f;
+    uint32_t const u = uint32_t(v + 0.5f);                   // v_cvt_u32_f32: truncates, saturates below at 0
+    return u < 255u ? u : 255u;
+}
+
+typedef __attribute__((address_space(1))) uint8_t* GlobalOutPtr;
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// Stores of one 16-texel block row.  `row` is uniform (start of image row y in the output),
+// `laneOff` the lane's byte offset inside the row, h01/h23 the lane's four channels as halves.
+template <int FORMAT>
+__device__ __forceinline__ void store_channels(GlobalOutPtr row, uint32_t laneOff, uint32_t planarPairStride,
+                                               uint32_t h01, uint32_t h23, int nch)
+{
+    GlobalOutPtr const dst = row + laneOff;
+    if constexpr (FORMAT == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS) {
+        // src/RegressionKernels.h:36-45; whole half2 pairs (Inference.cu:131-134)
+        *reinterpret_cast<__attribute__((address_space(1))) uint32_t*>(dst) = h01;
+        if (nch > 2) *reinterpret_cast<__attribute__((address_space(1))) uint32_t*>(dst + planarPairStride) = h23;
+    } else if constexpr (FORMAT == NTC_HIP_DEV_OUT_FP16_PIXELS) {
+        if (nch == 4 && ((reinterpret_cast<uintptr_t>(dst) & 7u) == 0)) {
+            *reinterpret_cast<__attribute__((address_space(1))) u32x2*>(dst) = u32x2{ h01, h23 };
+        } else {
+            uint32_t const h[4] = { h01 & 0xffffu, h01 >> 16, h23 & 0xffffu, h23 >> 16 };
+            for (int r = 0; r < nch; ++r) reinterpret_cast<__attribute__((address_space(1))) uint16_t*>(dst)[r] = uint16_t(h[r]);
+        }
+    } else {
+        v2h const a = __builtin_bit_cast(v2h, h01), b = __builtin_bit_cast(v2h, h23);
+        uint32_t const u8[4] = { half_to_unorm8(a[0]), half_to_unorm8(a[1]), half_to_unorm8(b[0]), half_to_unorm8(b[1]) };
+        if (nch == 4 && ((reinterpret_cast<uintptr_t>(dst) & 3u) == 0)) {
+            *reinterpret_cast<__attribute__((address_space(1))) uint32_t*>(dst) = u8[0] | (u8[1] << 8) | (u8[2] << 16) | (u8[3] << 24);
+        } else {
+            for (int r = 0; r < nch; ++r) dst[r] = uint8_t(u8[r]);
+        }
+    }
+}
+
+template <int FORMAT>
+__device__ __forceinline__ void store_tile(DevMip const& m, v4i const (&D)[4], v4f S, int x, int y0, int chBase)
+{
+    int const nch = min(4, m.numChannels - chBase);
+    if (x >= m.width || nch <= 0) return;
+    uint32_t const C2 = uint32_t((m.numChannels + 1) & ~1);
+    uint32_t const laneOff = (FORMAT == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)
+        ? (uint32_t(chBase) * uint32_t(m.width) + uint32_t(x) * 2u) * 2u
+        : uint32_t(x) * uint32_t(m.outPixelStride) + uint32_t(chBase) * (FORMAT == NTC_HIP_DEV_OUT_FP16_PIXELS ? 2u : 1u);
+    size_t const rowBytes = (FORMAT == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS) ? size_t(m.width) * C2 * 2 : size_t(m.outRowPitch);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        int const y = y0 + b;
+        if (y >= m.height) break;                            // uniform
+        uint32_t const h01 = to_half2_bits(float(D[b][0]) * S[0], float(D[b][1]) * S[1]);
+        uint32_t const h23 = to_half2_bits(float(D[b][2]) * S[2], float(D[b][3]) * S[3]);
+        store_channels<FORMAT>((GlobalOutPtr)m.out + size_t(y) * rowBytes, laneOff, uint32_t(m.width) * 4u, h01, h23, nch);
+    }
+}
+
+// ---- all-integer input stage (power-of-two mip and grid sizes) --------------------------
+//
+// With W and the grid size powers of two, u*Wg - 1/2 = ((2x+1)*2^e - 1)/2 with e = log2(Wg/W):
+// floor and fraction are shifts and masks, the bilinear weights are small integers, and
+// every float operation of the general path is exact, so both paths give the same bytes.
+
+struct AxisFoot { uint32_t c0, c1, f; };
+
+__device__ __forceinline__ AxisFoot axis_fast(int x, uint32_t packedAxis, int gridSize)
+{
+    int const shl = int(packedAxis & 0xffu), n = int((packedAxis >> 8) & 0xffu), sublog = int((packedAxis >> 16) & 0xffu);
+    int const N = ((2 * x + 1) << shl) - (1 << sublog);
+    int const b = N >> n;                                    // arithmetic shift = floor
+    AxisFoot a;
+    a.f = uint32_t(N) & ((1u << n) - 1u);
+    a.c0 = uint32_t(b) & uint32_t(gridSize - 1);             // wrap addressing
+    a.c1 = uint32_t(b + 1) & uint32_t(gridSize - 1);
+    return a;
+}
+
+// Four 4-bit features of the four taps, filtered: ((17 * sum w*q) >> n) - 128 per byte.
+// Nibbles are spread into 16-bit lanes, two dwords per tap ((f0,f2) and (f1,f3)); weights
+// are pre-multiplied by 17; no lane can overflow because 17*15*2^n < 65536 (n <= 8).
+__device__ __forceinline__ uint32_t bilinear4_int(uint32_t c00, uint32_t c10, uint32_t c01, uint32_t c11,
+                                                  uint32_t w00, uint32_t w10, uint32_t w01, uint32_t w11, uint32_t n)
+{
+    uint32_t const m = 0x000f000fu;
+    uint32_t const d00 = c00 | (c00 << 8), d10 = c10 | (c10 << 8), d01 = c01 | (c01 << 8), d11 = c11 | (c11 << 8);
+    uint32_t const te = __umul24(w00, d00 & m) + __umul24(w10, d10 & m) + __umul24(w01, d01 & m) + __umul24(w11, d11 & m);
+    uint32_t const to = __umul24(w00, (d00 >> 4) & m) + __umul24(w10, (d10 >> 4) & m)
+                      + __umul24(w01, (d01 >> 4) & m) + __umul24(w11, (d11 >> 4) & m);
+    uint32_t const ve = (te >> n) & 0x00ff00ffu;             // features 0 and 2 in bytes 0 and 2
+    uint32_t const vo = (to >> n) & 0x00ff00ffu;             // features 1 and 3
+    return (ve | (vo << 8)) ^ 0x80808080u;
 }
 
 // ---- decoder variants -----------------------------------------------------------------
@@ -166,6 +286,9 @@ struct alignas(16) Lds {
     float    scale[10][4][4];         // [M-tile][k-group g][r]  -> channel 16t+4g+r
     int32_t  bias[10][4][4];
     uint32_t in[kWaves][kWaveTexels][kInStride];
+    uint32_t lut2[256];               // byte of four 2-bit codes -> four input bytes 85*q - 128
+    uint32_t xtab[64][4];             // positional encoding by x phase: dword w = enc(px*2^w) | enc(px*2^w+1/4) << 16
+    uint32_t ytab[64][4];             // same for y, one byte up
 };
 
 // Copies the int8 blob (src/WeightLayout.cpp:42-49: matrices, then fp32 scales, then int32
@@ -204,7 +327,7 @@ __device__ void stage_weights(Lds& lds, uint8_t const* __restrict__ blob)
 
 // Input vector of one texel as 16 dwords (int8 x 64, zero padded).
 template <class V>
-__device__ __forceinline__ void prepare_inputs(DevMip const& m, int x, int y, uint32_t (&in)[16])
+__device__ __forceinline__ void prepare_inputs_general(DevMip const& m, int x, int y, uint32_t (&in)[16])
 {
 #pragma unroll
     for (int i = 0; i < 16; ++i) in[i] = 0;
@@ -300,6 +423,106 @@ __device__ __forceinline__ void prepare_inputs(DevMip const& m, int x, int y, ui
     }
 }
 
+// Input vector of one texel from integer arithmetic only (see axis_fast above).
+template <class V>
+__device__ __forceinline__ void prepare_inputs_fast(DevMip const& m, Lds const& lds, int x, int y, uint32_t (&in)[16])
+{
+#pragma unroll
+    for (int i = 0; i < 16; ++i) in[i] = 0;
+
+    // ---- high-res grid
+    {
+        AxisFoot const ax = axis_fast(x, m.hrAxisX, m.hrWidth), ay = axis_fast(y, m.hrAxisY, m.hrHeight);
+        GlobalU8Ptr const g = (GlobalU8Ptr)m.hr;
+        uint32_t const lgw = ((m.hrAxisX >> 24) & 0xffu) + 1u;   // log2(bytes per grid row)
+        uint32_t const layerStride = uint32_t(m.hrWidth) * uint32_t(m.hrHeight) * 2u;   // bytes
+        uint32_t const r0 = ay.c0 << lgw, r1 = ay.c1 << lgw, c0 = ax.c0 << 1, c1 = ax.c1 << 1;
+        uint32_t const a00 = r0 + c0, a10 = r0 + c1, a01 = r1 + c0, a11 = r1 + c1;   // byte offsets
+        if constexpr (V::HR_MODE == 1) {
+            static_assert(V::HR_MODE != 1 || (V::HR_BITS == 2 && V::HR_F == 8 && V::HR_SLOTS == 8), "concat grids: 8 x 2-bit");
+            uint32_t const addr[4] = { a00, a10, a01, a11 };
+#pragma unroll
+            for (int tap = 0; tap < 4; ++tap) {
+                uint32_t const w = load_u16(g, addr[tap]);
+                in[2 * tap]     = lds.lut2[w & 0xffu];
+                in[2 * tap + 1] = lds.lut2[w >> 8];
+            }
+        } else {
+            uint32_t const nx = (m.hrAxisX >> 8) & 0xffu, ny = (m.hrAxisY >> 8) & 0xffu;
+            uint32_t const wx1 = ax.f, wx0 = (1u << nx) - ax.f, wy1 = ay.f * 17u, wy0 = ((1u << ny) - ay.f) * 17u;
+            uint32_t const w00 = mul24(wx0, wy0), w10 = mul24(wx1, wy0), w01 = mul24(wx0, wy1), w11 = mul24(wx1, wy1);
+            constexpr int layers = (V::HR_F + 3) / 4;
+#pragma unroll
+            for (int L = 0; L < layers; ++L) {
+                GlobalU8Ptr const gl = g + size_t(L) * layerStride;
+                uint32_t b = bilinear4_int(load_u16(gl, a00), load_u16(gl, a10), load_u16(gl, a01), load_u16(gl, a11),
+                                           w00, w10, w01, w11, nx + ny);
+                if (4 * L + 4 > V::HR_F) b &= (1u << (8 * (V::HR_F - 4 * L))) - 1u;
+                in[L] = b;
+            }
+        }
+    }
+    // ---- low-res grid: bilinear, 4-bit
+    {
+        AxisFoot const ax = axis_fast(x, m.lrAxisX, m.lrWidth), ay = axis_fast(y, m.lrAxisY, m.lrHeight);
+        GlobalU8Ptr const g = (GlobalU8Ptr)m.lr;
+        uint32_t const lgw = ((m.lrAxisX >> 24) & 0xffu) + 1u;
+        uint32_t const layerStride = uint32_t(m.lrWidth) * uint32_t(m.lrHeight) * 2u;
+        uint32_t const r0 = ay.c0 << lgw, r1 = ay.c1 << lgw, c0 = ax.c0 << 1, c1 = ax.c1 << 1;
+        uint32_t const a00 = r0 + c0, a10 = r0 + c1, a01 = r1 + c0, a11 = r1 + c1;
+        uint32_t const nx = (m.lrAxisX >> 8) & 0xffu, ny = (m.lrAxisY >> 8) & 0xffu;
+        uint32_t const wx1 = ax.f, wx0 = (1u << nx) - ax.f, wy1 = ay.f * 17u, wy0 = ((1u << ny) - ay.f) * 17u;
+        uint32_t const w00 = mul24(wx0, wy0), w10 = mul24(wx1, wy0), w01 = mul24(wx0, wy1), w11 = mul24(wx1, wy1);
+        constexpr int layers = (V::LR_F + 3) / 4;
+#pragma unroll
+        for (int L = 0; L < layers; ++L) {
+            GlobalU8Ptr const gl = g + size_t(L) * layerStride;
+            uint32_t b = bilinear4_int(load_u16(gl, a00), load_u16(gl, a10), load_u16(gl, a01), load_u16(gl, a11),
+                                       w00, w10, w01, w11, nx + ny);
+            if (4 * L + 4 > V::LR_F) b &= (1u << (8 * (V::LR_F - 4 * L))) - 1u;
+            in[V::HR_INPUTS / 4 + L] = b;
+        }
+    }
+    // ---- positional encoding from the per-mip phase tables
+    {
+        uint4 const ex = *reinterpret_cast<uint4 const*>(&lds.xtab[uint32_t(x) & m.posMask][0]);
+        uint4 const ey = *reinterpret_cast<uint4 const*>(&lds.ytab[uint32_t(y) & m.posMask][0]);
+        in[V::POS_BASE / 4 + 0] = ex.x | ey.x;
+        in[V::POS_BASE / 4 + 1] = ex.y | ey.y;
+        in[V::POS_BASE / 4 + 2] = ex.z | ey.z;
+        if constexpr (V::LOD == 2) {
+            uint32_t const l = uint32_t(int(m.positionLod * 127.5f)) & 0xffu;
+            in[V::POS_BASE / 4 + 3] = l | (l << 8);
+        }
+    }
+}
+
+// One byte of the positional encoding (Inference.hlsli:89-113): int(enc * 127.5), truncating.
+__device__ __forceinline__ uint32_t posenc_byte(float p)
+{
+    float const e = (p - floorf(p)) * 2.f - 1.f;
+    return uint32_t(int(e * 127.5f)) & 0xffu;
+}
+
+// Fills the phase tables for a mip whose positionScale is a power of two: the encoding of
+// texel x depends only on x mod (1/positionScale), and all arithmetic involved is exact.
+__device__ void build_posenc_tables(Lds& lds, float positionScale)
+{
+    int const t = threadIdx.x;
+    if (t < 128) {
+        int const phase = t & 63;
+        float p = float(phase) * positionScale;
+        uint32_t e[3];
+#pragma unroll
+        for (int w = 0; w < 3; ++w) {
+            e[w] = posenc_byte(p) | (posenc_byte(p + 0.25f) << 16);
+            p *= 2.f;
+        }
+        if (t < 64) { lds.xtab[phase][0] = e[0];      lds.xtab[phase][1] = e[1];      lds.xtab[phase][2] = e[2];      lds.xtab[phase][3] = 0; }
+        else        { lds.ytab[phase][0] = e[0] << 8; lds.ytab[phase][1] = e[1] << 8; lds.ytab[phase][2] = e[2] << 8; lds.ytab[phase][3] = 0; }
+    }
+}
+
 template <class V>
 __global__ void __launch_bounds__(256, 2)
 decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
@@ -314,17 +537,30 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     int const tileBegin = blockIdx.x * per;
     int const tileEnd = min(totalTiles, tileBegin + per);
 
+    {   // 2-bit code bytes -> input bytes: code q maps to 85*q - 128 (255/3 = 85)
+        uint32_t x = threadIdx.x & 0xffu;
+        x = (x | (x << 12)) & 0x000f000fu;
+        x = (x | (x << 6))  & 0x03030303u;
+        lds.lut2[threadIdx.x & 0xffu] = (x * 85u) ^ 0x80808080u;
+    }
+
+    uint32_t c143 = 143u;
+    asm volatile("" : "+v"(c143));                           // stays in a VGPR: SDWA operands cannot be literals
+
     uint8_t const* stagedBlob = nullptr;
+    int stagedEntry = -1;
     int entry = 0;
 
     for (int tile = tileBegin; tile < tileEnd; ++tile) {
         while (entry + 1 < numMips && mips[entry + 1].tileStart <= tile) ++entry;
         DevMip const& m = mips[entry];
 
-        if (m.weights != stagedBlob) {                       // uniform across the workgroup
+        if (m.weights != stagedBlob || entry != stagedEntry) {   // uniform across the workgroup
             __syncthreads();
-            stage_weights<V>(lds, m.weights);
+            if (m.weights != stagedBlob) stage_weights<V>(lds, m.weights);
+            if (m.fast) build_posenc_tables(lds, m.positionScale);
             stagedBlob = m.weights;
+            stagedEntry = entry;
             __syncthreads();
         }
 
@@ -338,7 +574,8 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
         {
             int const x = min(x0 + j, m.width - 1), y = min(y0 + g, m.height - 1);
             uint32_t in[16];
-            prepare_inputs<V>(m, x, y, in);
+            if (m.fast) prepare_inputs_fast<V>(m, lds, x, y, in);
+            else        prepare_inputs_general<V>(m, x, y, in);
             uint4* dst = reinterpret_cast<uint4*>(&lds.in[wave][lane][0]);
             dst[0] = make_uint4(in[0], in[1], in[2], in[3]);
             dst[1] = make_uint4(in[4], in[5], in[6], in[7]);
@@ -378,7 +615,7 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
 #pragma unroll
                 for (int b = 0; b < 4; ++b) {
                     v4i const D = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
-                    Y[b][t] = activate4(D, S);
+                    Y[b][t] = activate4(D, S, c143);
                 }
             }
 #pragma unroll
@@ -392,44 +629,12 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
             v4i const A = v4i{ int(wa.x), int(wa.y), int(wa.z), int(wa.w) };
             v4i const C = *reinterpret_cast<v4i const*>(&lds.bias[tb][g][0]);
             v4f const S = *reinterpret_cast<v4f const*>(&lds.scale[tb][g][0]);
-            int const x = x0 + j;
-            int const chBase = 4 * g;
+            v4i D[4];
 #pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                v4i const D = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
-                int const y = y0 + b;
-                if (x >= m.width || y >= m.height || chBase >= m.numChannels) continue;
-                uint32_t h[4];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) h[r] = to_half_bits(float(D[r]) * S[r]);
-                int const nch = min(4, m.numChannels - chBase);
-                if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS) {
-                    // src/RegressionKernels.h:36-45; whole half2 pairs (Inference.cu:131-134)
-                    size_t const C2 = size_t((m.numChannels + 1) & ~1);
-                    uint16_t* img = reinterpret_cast<uint16_t*>(m.out);
-                    size_t const a = size_t(y) * size_t(m.width) * C2 + size_t(chBase) * size_t(m.width) + size_t(x) * 2;
-                    *reinterpret_cast<uint32_t*>(img + a) = h[0] | (h[1] << 16);
-                    if (nch > 2)
-                        *reinterpret_cast<uint32_t*>(img + a + 2 * size_t(m.width)) = h[2] | (h[3] << 16);
-                } else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS) {
-                    uint8_t* px = m.out + size_t(y) * m.outRowPitch + size_t(x) * size_t(m.outPixelStride) + 2 * chBase;
-                    if (nch == 4 && ((reinterpret_cast<uintptr_t>(px) & 7u) == 0)) {
-                        *reinterpret_cast<uint2*>(px) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
-                    } else {
-                        for (int r = 0; r < nch; ++r) reinterpret_cast<uint16_t*>(px)[r] = uint16_t(h[r]);
-                    }
-                } else {
-                    uint8_t* px = m.out + size_t(y) * m.outRowPitch + size_t(x) * size_t(m.outPixelStride) + chBase;
-                    uint32_t u8[4];
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) u8[r] = half_bits_to_unorm8(h[r]);
-                    if (nch == 4 && ((reinterpret_cast<uintptr_t>(px) & 3u) == 0)) {
-                        *reinterpret_cast<uint32_t*>(px) = u8[0] | (u8[1] << 8) | (u8[2] << 16) | (u8[3] << 24);
-                    } else {
-                        for (int r = 0; r < nch; ++r) px[r] = uint8_t(u8[r]);
-                    }
-                }
-            }
+            for (int b = 0; b < 4; ++b) D[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
+            if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)      store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, x0 + j, y0, 4 * g);
+            else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)       store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
+            else                                                       store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
         }
     }
 }
@@ -482,6 +687,28 @@ hipError_t launch_decode(int variant, DevMip const* mips, int numMips, int total
     case NTC_HIP_VARIANT_REF8:  return launch_variant<VRef8>(mips, numMips, totalTiles, gridSize, stream);
     case NTC_HIP_VARIANT_REF4:  return launch_variant<VRef4>(mips, numMips, totalTiles, gridSize, stream);
     default: return hipErrorInvalidValue;
+    }
+}
+
+template <class V>
+static int occupancy_variant()
+{
+    int blocks = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, decode_kernel<V>, 256, 0) != hipSuccess || blocks < 1) blocks = 2;
+    return blocks;
+}
+
+// Workgroups of the variant's kernel that fit on one compute unit (registers and LDS).
+int resident_workgroups_per_cu(int variant)
+{
+    switch (variant) {
+    case NTC_HIP_VARIANT_CFG01: return occupancy_variant<VCfg01>();
+    case NTC_HIP_VARIANT_CFG2:  return occupancy_variant<VCfg2>();
+    case NTC_HIP_VARIANT_REF16: return occupancy_variant<VRef16>();
+    case NTC_HIP_VARIANT_REF12: return occupancy_variant<VRef12>();
+    case NTC_HIP_VARIANT_REF8:  return occupancy_variant<VRef8>();
+    case NTC_HIP_VARIANT_REF4:  return occupancy_variant<VRef4>();
+    default: return 2;
     }
 }
 

@@ -5,8 +5,10 @@
 #include "ntc_decode_kernel.h"
 
 #include <hip/hip_runtime_api.h>
+#include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 
@@ -99,6 +101,47 @@ int pick_variant(NtcHipDecoderSpec const& s)
     return NTC_HIP_VARIANT_NONE;
 }
 
+uint64_t grid_bytes(int32_t w, int32_t h, int32_t features, int32_t bits);
+
+bool is_pow2(int32_t v) { return v > 0 && (v & (v - 1)) == 0; }
+int log2i(int32_t v) { int l = 0; while ((1 << l) < v) ++l; return l; }
+
+// Integer form of p = u*grid - 1/2 for power-of-two sizes: p = N / 2^n with
+// N = ((2x+1) << shl) - (1 << sublog).  Returns false when the axis is not a power of two.
+bool axis_params(int32_t size, int32_t grid, uint32_t& packed, int& n)
+{
+    if (!is_pow2(size) || !is_pow2(grid)) return false;
+    int const e = log2i(grid) - log2i(size);
+    int const shl = e > 0 ? e : 0, sublog = e < 0 ? -e : 0;
+    n = 1 - e > 1 ? 1 - e : 1;
+    if (shl > 12 || n > 16) return false;
+    packed = uint32_t(shl) | (uint32_t(n) << 8) | (uint32_t(sublog) << 16) | (uint32_t(log2i(grid)) << 24);
+    return true;
+}
+
+// Decides whether a mip may take the kernel's all-integer input stage and fills its parameters.
+// Conditions: every size a power of two (then every float operation of the general stage is
+// exact and the integer form gives the same bytes); bilinear weights of at most 8 fractional
+// bits in total (16-bit lanes of the packed filter cannot overflow); positionScale a power of
+// two, at least 2^-6 (the encoding has a period of at most 64 texels).
+void fill_fast_path(NtcHipDecoderSpec const& spec, DevMip& e)
+{
+    e.fast = 0;
+    int hx, hy, lx, ly;
+    if (!axis_params(e.width, e.hrWidth, e.hrAxisX, hx) || !axis_params(e.height, e.hrHeight, e.hrAxisY, hy)) return;
+    if (!axis_params(e.width, e.lrWidth, e.lrAxisX, lx) || !axis_params(e.height, e.lrHeight, e.lrAxisY, ly)) return;
+    if (lx + ly > 8) return;
+    if (spec.hrMode == NTC_HIP_GRID_BILINEAR && hx + hy > 8) return;
+    if (grid_bytes(e.hrWidth, e.hrHeight, spec.hrFeatures, spec.hrBits) >= (1ull << 31)) return;
+    if (grid_bytes(e.lrWidth, e.lrHeight, spec.lrFeatures, spec.lrBits) >= (1ull << 31)) return;
+    int exp2 = 0;
+    float const mant = std::frexp(e.positionScale, &exp2);      // scale = mant * 2^exp2, mant in [0.5, 1)
+    if (!(mant == 0.5f) || exp2 - 1 < -6 || exp2 - 1 > 20) return;
+    int const k = -(exp2 - 1);                                  // scale = 2^-k
+    e.posMask = k > 0 ? (1u << k) - 1u : 0u;
+    e.fast = 1;
+}
+
 uint64_t grid_bytes(int32_t w, int32_t h, int32_t features, int32_t bits)
 {
     if (w <= 0 || h <= 0 || features <= 0 || (bits != 2 && bits != 4)) return 0;
@@ -178,6 +221,7 @@ int build_table(NtcHipTextureSet const* sets, int32_t numSets, std::vector<DevMi
             e.hrWidth = d.hrWidth; e.hrHeight = d.hrHeight; e.lrWidth = d.lrWidth; e.lrHeight = d.lrHeight;
             e.positionScale = d.positionScale; e.positionLod = d.positionLod;
             e.outPixelStride = set.outPixelStride; e.numChannels = set.numChannels; e.outFormat = set.outputFormat;
+            fill_fast_path(set.spec, e);
             e.tilesX = (d.width + kTileWidth - 1) / kTileWidth;
             e.tilesY = (d.height + kTileHeight - 1) / kTileHeight;
             e.tileStart = totalTiles;
@@ -225,10 +269,15 @@ int upload_table(std::vector<DevMip> const& table)
     return 0;
 }
 
-int grid_size_for(int totalTiles)
+int grid_size_for(int variant, int totalTiles)
 {
-    // Persistent workgroups: two per compute unit (launch bounds keep 2 x 4 waves resident).
-    int const resident = g_lib.computeUnits * 2;
+    // Persistent workgroups: as many as stay resident at once, each walking a contiguous share of tiles.
+    static int perCu[16] = { 0 };
+    if (perCu[variant] == 0) {
+        perCu[variant] = resident_workgroups_per_cu(variant);
+        if (char const* env = std::getenv("NTC_HIP_WG_PER_CU")) { int v = std::atoi(env); if (v >= 1 && v <= 8) perCu[variant] = v; }
+    }
+    int const resident = g_lib.computeUnits * perCu[variant];
     return totalTiles < resident ? totalTiles : resident;
 }
 
@@ -381,7 +430,7 @@ int ntc_hip_decode(const NtcHipTextureSet* sets, int32_t numSets)
     int variant = NTC_HIP_VARIANT_NONE, totalTiles = 0;
     if (int r = build_table(sets, numSets, table, variant, totalTiles)) return r;
     if (int r = upload_table(table)) return r;
-    HIP_TRY(launch_decode(variant, g_lib.tableDev, int(table.size()), totalTiles, grid_size_for(totalTiles), g_lib.stream));
+    HIP_TRY(launch_decode(variant, g_lib.tableDev, int(table.size()), totalTiles, grid_size_for(variant, totalTiles), g_lib.stream));
     clear_error();
     return 0;
 }
@@ -394,7 +443,7 @@ int ntc_hip_decode_timed(const NtcHipTextureSet* sets, int32_t numSets, int32_t 
     int variant = NTC_HIP_VARIANT_NONE, totalTiles = 0;
     if (int r = build_table(sets, numSets, table, variant, totalTiles)) return r;
     if (int r = upload_table(table)) return r;
-    int const grid = grid_size_for(totalTiles);
+    int const grid = grid_size_for(variant, totalTiles);
     HIP_TRY(hipEventRecord(g_lib.evStart, g_lib.stream));
     for (int i = 0; i < iterations; ++i)
         HIP_TRY(launch_decode(variant, g_lib.tableDev, int(table.size()), totalTiles, grid, g_lib.stream));

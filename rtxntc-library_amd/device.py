@@ -30,14 +30,19 @@ class Device:
     def synchronize(self):
         abi.check(self.lib.ntc_hip_synchronize())
 
+    @staticmethod
+    def pack_sets(sets):
+        """A C array of texture sets, reusable across decode calls."""
+        return sets if isinstance(sets, C.Array) else (abi.TextureSet * len(sets))(*sets)
+
     def decode(self, sets):
-        arr = (abi.TextureSet * len(sets))(*sets)
-        abi.check(self.lib.ntc_hip_decode(arr, len(sets)))
+        arr = self.pack_sets(sets)
+        abi.check(self.lib.ntc_hip_decode(arr, len(arr)))
 
     def decode_timed(self, sets, iterations):
-        arr = (abi.TextureSet * len(sets))(*sets)
+        arr = self.pack_sets(sets)
         ms = C.c_float(0)
-        abi.check(self.lib.ntc_hip_decode_timed(arr, len(sets), iterations, C.byref(ms)))
+        abi.check(self.lib.ntc_hip_decode_timed(arr, len(arr), iterations, C.byref(ms)))
         return ms.value
 
 
