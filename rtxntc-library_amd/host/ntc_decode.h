@@ -1,0 +1,177 @@
+// ntc_decode.h - C++ host interface of the MI355X texture-set decoder.
+//
+// It mirrors the part of LibNTC's public interface that the decompression path uses
+// (reference include/libntc/ntc.h): the same names in namespace ntc, the same argument meaning,
+// the same status codes and error-message convention, so code written against LibNTC's
+//   CreateContext -> IContext::CreateTextureSet -> ITextureSet::SetLatentShape ->
+//   (load) -> ITextureSet::Decompress -> ITextureSet::ReadChannels
+// sequence reads the same here.  Compression, file I/O and graphics-API interop are not part
+// of this library; the interface below simply does not declare them.
+//
+// Everything device-side goes through the C ABI of include/ntc_hip.h; this layer never
+// includes a HIP header.
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+
+namespace ntc
+{
+
+// Same value as the reference's InterfaceVersion (include/libntc/ntc.h:40): applications pass
+// it in ContextParameters and CreateContext rejects a mismatch (src/PublicFunctions.cpp:66-71).
+constexpr uint32_t InterfaceVersion = 0x25121500;
+
+// Numeric values follow include/libntc/ntc.h:53-74.
+enum class Status
+{
+    Ok = 0, InterfaceMismatch = 1, CudaError = 2, CudaUnavailable = 3, FileUnavailable = 4,
+    FileUnrecognized = 5, FileIncompatible = 6, Incomplete = 7, Unsupported = 8, InternalError = 9,
+    InvalidArgument = 10, InvalidData = 11, InvalidState = 12, IOError = 13, NotImplemented = 14,
+    OutOfMemory = 15, OutOfRange = 16, ShaderUnavailable = 17, UnknownError = 18
+};
+
+// include/libntc/ntc.h:227-236
+enum class ChannelFormat { UNKNOWN = 0, UNORM8 = 1, UNORM16 = 2, FLOAT16 = 3, FLOAT32 = 4, UINT32 = 5 };
+// include/libntc/ntc.h:272-276
+enum class AddressSpace { Host, Device };
+enum class TextureDataPage { Reference, Output };
+
+constexpr int DisableCudaDevice = -1;          // ContextParameters::cudaDevice: do not touch the GPU
+
+// include/libntc/ntc.h:131-156
+struct LatentShape
+{
+    int gridSizeScale = 4;
+    int numFeatures = 16;
+    bool operator==(LatentShape const& o) const { return gridSizeScale == o.gridSizeScale && numFeatures == o.numFeatures; }
+    bool operator!=(LatentShape const& o) const { return !(*this == o); }
+    static constexpr LatentShape Empty() { return LatentShape{ 0, 0 }; }
+    bool IsEmpty() const { return *this == Empty(); }
+};
+
+// include/libntc/ntc.h:158-177
+struct TextureSetDesc
+{
+    int width = 0;
+    int height = 0;
+    int channels = 0;
+    int mips = 1;
+};
+
+// include/libntc/ntc.h:179-199 (the fields the decode path reads)
+struct TextureSetFeatures
+{
+    int stagingBytesPerPixel = 4;   // staging buffer for ReadChannels into host memory; 0 = none
+    int stagingWidth = 0;           // 0 = texture-set width
+    int stagingHeight = 0;
+    bool enableCompression = false; // accepted for source compatibility; compression is not available
+    bool separateRefOutData = false;
+};
+
+// include/libntc/ntc.h:689-730
+struct ReadChannelsParameters
+{
+    TextureDataPage page = TextureDataPage::Output;
+    int mipLevel = 0;
+    int firstChannel = 0;
+    int numChannels = 0;
+    unsigned char* pOutData = nullptr;
+    AddressSpace addressSpace = AddressSpace::Host;
+    int width = 0;
+    int height = 0;
+    size_t pixelStride = 0;
+    size_t rowPitch = 0;
+    ChannelFormat channelFormat = ChannelFormat::UNKNOWN;
+    void const* dstColorSpaces = nullptr;   // must be null: only linear storage is supported
+    bool useDithering = false;              // must be false
+};
+
+// include/libntc/ntc.h:810-816.  Losses stay zero: with no reference image registered the
+// reference takes the same branch (src/Inference.cu:119-136, src/TextureSet.cpp:1833).
+struct DecompressionStats
+{
+    float perChannelLoss[16];
+    float perMipLoss[16];
+    float overallLoss = 0;
+    float gpuTimeMilliseconds = 0;
+};
+
+// include/libntc/ntc.h:1278-1305 (graphics-API fields left out)
+struct ContextParameters
+{
+    uint32_t interfaceVersion = InterfaceVersion;
+    int cudaDevice = 0;             // index of the HIP device; the name is kept for source compatibility
+};
+
+// Decoder families beyond the one compiled into LibNTC 0.9.2, selected with
+// ITextureSet::SetDecoderPreset (an addition; the reference changes decoders by editing
+// InferenceConstants.h, README.md:32-36).
+enum class DecoderPreset
+{
+    LibNTC092 = 0,      // both grids bilinear 4-bit, shared neural LODs, (lod, lod) inputs, MLP 48-64-48-32-16
+    Concat2x2_64 = 1,   // per-mip grids: HR (W/2) 2x2-concat of 8 x 2-bit, LR (W/4) bilinear 16 x 4-bit, MLP 64-64-48-32-16
+    Concat2x2_48 = 2    // same grids with 12 LR features, MLP 64-48-48-32-16
+};
+
+class ITextureSet
+{
+public:
+    virtual TextureSetDesc const& GetDesc() const = 0;
+    virtual LatentShape const& GetLatentShape() const = 0;
+
+    // Changes the latent shape; all compressed data is lost (include/libntc/ntc.h:858-861).
+    // Range rules follow src/TextureSetMetadata.cpp:1137-1159.
+    virtual Status SetLatentShape(LatentShape const& newShape) = 0;
+
+    // --- additions: the reference can only receive latents and weights from an NTC file ---
+    virtual Status SetDecoderPreset(DecoderPreset preset) = 0;
+    // Size in bytes of the latent buffer / weight blob the current shape expects.
+    virtual uint64_t GetLatentDataSize() const = 0;
+    virtual uint64_t GetWeightDataSize() const = 0;
+    // Latent grids exactly as stored in an NTC file (u16 layers, neural LOD after neural LOD)
+    // and the GenericInt8 weight blob of src/WeightLayout.cpp:42-49.  Host memory.
+    virtual Status SetLatentData(void const* data, size_t size) = 0;
+    virtual Status SetWeightData(void const* data, size_t size) = 0;
+
+    // Decompresses into the internal representation; ReadChannels extracts it
+    // (include/libntc/ntc.h:929-933, src/TextureSet.cpp:1664-1897).  useInt8Weights is accepted
+    // and ignored: the int8 weights are the only weights.
+    virtual Status Decompress(DecompressionStats* pOutStats, bool useInt8Weights = false) = 0;
+
+    // include/libntc/ntc.h:902, src/TextureSet.cpp:915-985.
+    virtual Status ReadChannels(ReadChannelsParameters const& params) = 0;
+
+    // Always 0: no reference images can be registered (include/libntc/ntc.h:638-640).
+    virtual uint32_t GetValidChannelMask() const = 0;
+
+    virtual ~ITextureSet() = default;
+};
+
+class IContext
+{
+public:
+    // include/libntc/ntc.h:1149, src/Context.cpp:235-261
+    virtual Status CreateTextureSet(TextureSetDesc const& desc, TextureSetFeatures const& features,
+        ITextureSet** pOutTextureSet) const = 0;
+    // include/libntc/ntc.h:1153
+    virtual void DestroyTextureSet(ITextureSet* textureSet) const = 0;
+    // True when a gfx950 device was initialised (reference: IsCudaAvailable).
+    virtual bool IsCudaAvailable() const = 0;
+    virtual ~IContext() = default;
+};
+
+extern "C" {
+// include/libntc/ntc.h:1307-1331.  CreateContext returns CudaUnavailable together with a usable
+// context when no device can be used (src/PublicFunctions.cpp:161).
+uint32_t GetInterfaceVersion();
+Status CreateContext(IContext** pOutContext, ContextParameters const& params);
+void DestroyContext(IContext* context);
+char const* GetLastErrorMessage();
+char const* StatusToString(Status status);
+char const* ChannelFormatToString(ChannelFormat format);
+size_t GetBytesPerPixelComponent(ChannelFormat format);
+float LossToPSNR(float loss);
+}
+
+} // namespace ntc
