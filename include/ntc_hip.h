@@ -168,6 +168,25 @@ int ntc_hip_decode(const NtcHipTextureSet* sets, int32_t numSets);
 int ntc_hip_decode_timed(const NtcHipTextureSet* sets, int32_t numSets, int32_t iterations,
                          float* outMillisecondsPerIteration);
 
+/* Extracts channels of one decoded mip from the internal fp16 layout into a user image:
+ * what ITextureSet::ReadChannels does through cuda::CopyImage (src/TextureSet.cpp:915-985,
+ * src/ImageProcessing.cu:141-164,220-277).  Same-size copies only (the reference's 1:1
+ * branch), no dithering, linear colour spaces.  Destination channels beyond numChannels get
+ * the reference's defaults (alpha 1, others 0).  Asynchronous on the library stream. */
+typedef struct NtcHipReadChannels {
+    const void* planarPairs;    /* device: start of the mip, NTC_HIP_OUT_FP16_PLANAR_PAIRS layout */
+    uint64_t    planarBytes;    /* bytes available from planarPairs */
+    int32_t     width, height;  /* of the mip */
+    int32_t     setChannels;    /* channel count of the set, even */
+    int32_t     firstChannel, numChannels;
+    void*       dst;            /* device */
+    uint64_t    dstBytes;
+    int32_t     format;         /* ChannelFormat of include/libntc/ntc.h:227-236: 1 UNORM8, 2 UNORM16, 3 FLOAT16, 4 FLOAT32, 5 UINT32 */
+    int32_t     reserved;
+    uint64_t    pixelStride, rowPitch;
+} NtcHipReadChannels;
+int ntc_hip_read_channels(const NtcHipReadChannels* params);
+
 /* Self-check of the MFMA operand layout the kernels assume: multiplies a 16x64 by a
  * 64x16 int8 matrix on the device (row-major host arrays), writes the 16x16 int32
  * product.  No reference counterpart; used by the tests. */

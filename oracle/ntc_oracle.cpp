@@ -460,6 +460,50 @@ int ntc_oracle_ref_geometry(int width, int height, int numMips, int gridSizeScal
     return numNeural;
 }
 
+// ITextureSet::ReadChannels' copy, 1:1 branch, no dithering, linear colour spaces:
+// CopyImageKernel + ReadImageChannel (FLOAT16 source) + WriteImageChannel
+// (src/ImageProcessing.cu:107-164,220-265) reading the internal planar-pair layout
+// (GetTextureDataSlice, src/TextureSet.cpp:1958-1983).  Destination channels beyond
+// numChannels get GetDefaultChannelValue (src/ImageProcessing.cu:166-170).
+// format: 1 UNORM8, 2 UNORM16, 3 FLOAT16, 4 FLOAT32, 5 UINT32 (include/libntc/ntc.h:227-236).
+int ntc_oracle_read_channels(const uint16_t* planarPairs, int width, int height, int setChannels,
+                             int firstChannel, int numChannels, uint8_t* dst, int format,
+                             uint64_t pixelStride, uint64_t rowPitch)
+{
+    int const bpc = (format == 1) ? 1 : (format == 2 || format == 3) ? 2 : (format == 4 || format == 5) ? 4 : 0;
+    if (!bpc) return -1;
+    int const dstChannels = int(pixelStride / uint64_t(bpc));
+    auto roundHalfAway = [](float v) {                       // roundf
+        float r = std::trunc(v);
+        float const fr = v - r;
+        if (fr >= 0.5f) r += 1.f; else if (fr <= -0.5f) r -= 1.f;
+        return r;
+    };
+    for (int y = 0; y < height; ++y)
+        for (int x = 0; x < width; ++x) {
+            uint8_t* px = dst + size_t(y) * rowPitch + size_t(x) * pixelStride;
+            for (int ch = 0; ch < dstChannels; ++ch) {
+                float value;
+                if (ch < numChannels) {
+                    int const c = firstChannel + ch;
+                    size_t const a = size_t(y) * size_t(width) * size_t(setChannels) + size_t(x) * 2
+                                   + size_t(c & ~1) * size_t(width) + size_t(c & 1);
+                    value = half_to_float(planarPairs[a]);
+                } else {
+                    value = (ch == 3) ? 1.f : 0.f;
+                }
+                switch (format) {
+                case 1: px[ch] = uint8_t(std::max(0.f, std::min(255.f, roundHalfAway(value * 255.f)))); break;
+                case 2: { uint16_t v = uint16_t(std::max(0.f, std::min(65535.f, roundHalfAway(value * 65535.f)))); std::memcpy(px + 2 * ch, &v, 2); break; }
+                case 3: { uint16_t v = float_to_half_rne(std::max(-65504.f, std::min(65504.f, value))); std::memcpy(px + 2 * ch, &v, 2); break; }
+                case 4: std::memcpy(px + 4 * ch, &value, 4); break;
+                case 5: { uint32_t v = uint32_t(std::max(value, 0.f)); std::memcpy(px + 4 * ch, &v, 4); break; }
+                }
+            }
+        }
+    return 0;
+}
+
 // Decodes every mip of one set into set->output (host memory).  Rows of each mip are handed
 // out in bands to `threads` workers.  Returns seconds spent decoding (steady clock), < 0 on error.
 double ntc_oracle_decode(const NtcHipTextureSet* set, int threads)

@@ -68,6 +68,18 @@ class TextureSet(C.Structure):
     ]
 
 
+class ReadChannels(C.Structure):
+    _fields_ = [
+        ("planarPairs", C.c_void_p), ("planarBytes", C.c_uint64), ("width", C.c_int32), ("height", C.c_int32),
+        ("setChannels", C.c_int32), ("firstChannel", C.c_int32), ("numChannels", C.c_int32),
+        ("dst", C.c_void_p), ("dstBytes", C.c_uint64), ("format", C.c_int32), ("reserved", C.c_int32),
+        ("pixelStride", C.c_uint64), ("rowPitch", C.c_uint64),
+    ]
+
+
+FORMAT_UNORM8, FORMAT_UNORM16, FORMAT_FLOAT16, FORMAT_FLOAT32, FORMAT_UINT32 = 1, 2, 3, 4, 5
+
+
 class NtcHipError(RuntimeError):
     def __init__(self, code, message):
         super().__init__(f"ntc_hip error {code}: {message}")
@@ -91,6 +103,7 @@ EXPORTS = [
     ("ntc_hip_grid_bytes", C.c_uint64, [C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     ("ntc_hip_decode", C.c_int, [C.POINTER(TextureSet), C.c_int32]),
     ("ntc_hip_decode_timed", C.c_int, [C.POINTER(TextureSet), C.c_int32, C.c_int32, C.POINTER(C.c_float)]),
+    ("ntc_hip_read_channels", C.c_int, [C.POINTER(ReadChannels)]),
     ("ntc_hip_selftest_mfma", C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
 ]
 

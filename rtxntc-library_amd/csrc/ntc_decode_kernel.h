@@ -45,6 +45,20 @@ struct DevMip {
 
 constexpr int kTileWidth = 64, kTileHeight = 4;
 
+// ChannelFormat values of the reference (include/libntc/ntc.h:227-236)
+enum {
+    NTC_HIP_DEV_FORMAT_UNORM8 = 1, NTC_HIP_DEV_FORMAT_UNORM16 = 2, NTC_HIP_DEV_FORMAT_FLOAT16 = 3,
+    NTC_HIP_DEV_FORMAT_FLOAT32 = 4, NTC_HIP_DEV_FORMAT_UINT32 = 5
+};
+
+struct ReadChannelsArgs {
+    uint16_t const* planarPairs;   // start of the mip in the internal fp16 layout
+    uint8_t* dst;
+    uint64_t pixelStride, rowPitch;
+    int32_t width, height, setChannels, firstChannel, numChannels, dstChannels, format;
+};
+hipError_t launch_read_channels(ReadChannelsArgs const& args, hipStream_t stream);
+
 hipError_t launch_decode(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream);
 int resident_workgroups_per_cu(int variant);
 hipError_t launch_selftest_mfma(int8_t const* a, int8_t const* b, int32_t* d, hipStream_t stream);

@@ -456,6 +456,47 @@ int ntc_hip_decode_timed(const NtcHipTextureSet* sets, int32_t numSets, int32_t 
     return 0;
 }
 
+int ntc_hip_read_channels(const NtcHipReadChannels* p)
+{
+    if (int r = require_init()) return r;
+    if (!p || !p->planarPairs || !p->dst) { set_error("ntc_hip_read_channels: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
+    int bpc = 0;
+    switch (p->format) {
+    case NTC_HIP_DEV_FORMAT_UNORM8: bpc = 1; break;
+    case NTC_HIP_DEV_FORMAT_UNORM16: case NTC_HIP_DEV_FORMAT_FLOAT16: bpc = 2; break;
+    case NTC_HIP_DEV_FORMAT_FLOAT32: case NTC_HIP_DEV_FORMAT_UINT32: bpc = 4; break;
+    default: set_error("ntc_hip_read_channels: unknown channel format %d.", p->format); return NTC_HIP_ERR_INVALID_ARG;
+    }
+    if (p->width < 1 || p->height < 1 || p->setChannels < 2 || (p->setChannels & 1) || p->setChannels > NTC_HIP_MAX_CHANNELS
+        || p->firstChannel < 0 || p->numChannels < 1 || p->firstChannel + p->numChannels > p->setChannels) {
+        set_error("ntc_hip_read_channels: bad image or channel range.");
+        return NTC_HIP_ERR_INVALID_ARG;
+    }
+    if (p->pixelStride < uint64_t(bpc) || p->rowPitch < p->pixelStride * uint64_t(p->width)
+        || (p->pixelStride % uint64_t(bpc)) || (p->rowPitch % uint64_t(bpc)) || (reinterpret_cast<uintptr_t>(p->dst) % uintptr_t(bpc))) {
+        set_error("ntc_hip_read_channels: pixel stride / row pitch do not fit the format.");
+        return NTC_HIP_ERR_INVALID_ARG;
+    }
+    uint64_t const dstChannels = p->pixelStride / uint64_t(bpc);
+    if (dstChannels > 64) { set_error("ntc_hip_read_channels: pixel stride too large."); return NTC_HIP_ERR_INVALID_ARG; }
+    uint64_t const need = uint64_t(p->height - 1) * p->rowPitch + uint64_t(p->width) * p->pixelStride;
+    uint64_t const srcNeed = uint64_t(p->width) * uint64_t(p->height) * uint64_t(p->setChannels) * 2u;
+    if (need > p->dstBytes || srcNeed > p->planarBytes) {
+        set_error("ntc_hip_read_channels: image reaches past the given buffer sizes.");
+        return NTC_HIP_ERR_INVALID_ARG;
+    }
+    ReadChannelsArgs a{};
+    a.planarPairs = static_cast<uint16_t const*>(p->planarPairs);
+    a.dst = static_cast<uint8_t*>(p->dst);
+    a.pixelStride = p->pixelStride; a.rowPitch = p->rowPitch;
+    a.width = p->width; a.height = p->height; a.setChannels = p->setChannels;
+    a.firstChannel = p->firstChannel; a.numChannels = p->numChannels;
+    a.dstChannels = int32_t(dstChannels); a.format = p->format;
+    HIP_TRY(launch_read_channels(a, g_lib.stream));
+    clear_error();
+    return 0;
+}
+
 int ntc_hip_selftest_mfma(const int8_t* a16x64, const int8_t* b64x16, int32_t* d16x16)
 {
     if (int r = require_init()) return r;

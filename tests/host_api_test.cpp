@@ -1,0 +1,194 @@
+// host_api_test.cpp - drives the C++ host layer (rtxntc-library_amd/host/ntc_decode.h) the way an
+// application drives LibNTC.  Built by tests/Makefile, run by tests/test_host_api.py.
+//   host_api_test cpu
+//       host-only checks (no GPU): status codes, messages, state machine, sizes
+//   host_api_test decode <preset> <w> <h> <mips> <channels> <gridScale> <features> <latents> <weights> <outPrefix>
+//       loads raw latents/weights, decompresses, reads every mip back as UNORM8 (host address
+//       space) and FLOAT16 (device address space is exercised through a second read), writes files
+#include "../rtxntc-library_amd/host/ntc_decode.h"
+#include "../include/ntc_hip.h"
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+using namespace ntc;
+
+#define CHECK(cond) do { if (!(cond)) { std::fprintf(stderr, "FAILED %s:%d: %s\n  last error: %s\n", __FILE__, __LINE__, #cond, GetLastErrorMessage()); return 1; } } while (0)
+
+static std::vector<unsigned char> readFile(char const* path)
+{
+    std::vector<unsigned char> data;
+    if (FILE* f = std::fopen(path, "rb")) {
+        std::fseek(f, 0, SEEK_END); long n = std::ftell(f); std::fseek(f, 0, SEEK_SET);
+        data.resize(size_t(n));
+        if (std::fread(data.data(), 1, size_t(n), f) != size_t(n)) data.clear();
+        std::fclose(f);
+    }
+    return data;
+}
+static bool writeFile(std::string const& path, void const* p, size_t n)
+{
+    FILE* f = std::fopen(path.c_str(), "wb");
+    if (!f) return false;
+    bool ok = std::fwrite(p, 1, n, f) == n;
+    std::fclose(f);
+    return ok;
+}
+
+static int cpuChecks()
+{
+    IContext* ctx = nullptr;
+    ContextParameters params;
+    params.interfaceVersion = 0x12345678;
+    CHECK(CreateContext(&ctx, params) == Status::InterfaceMismatch);
+    CHECK(std::strstr(GetLastErrorMessage(), "Invalid interface version") != nullptr);
+    params = ContextParameters();
+    CHECK(CreateContext(nullptr, params) == Status::InvalidArgument);
+    params.cudaDevice = DisableCudaDevice;
+    CHECK(CreateContext(&ctx, params) == Status::CudaUnavailable);     // ... and still a usable context
+    CHECK(ctx != nullptr && !ctx->IsCudaAvailable());
+    CHECK(GetInterfaceVersion() == InterfaceVersion);
+    CHECK(std::strcmp(StatusToString(Status::OutOfRange), "OutOfRange") == 0);
+    CHECK(std::strcmp(StatusToString(Status::CudaUnavailable), "CudaUnavailable") == 0);
+    CHECK(GetBytesPerPixelComponent(ChannelFormat::FLOAT16) == 2 && GetBytesPerPixelComponent(ChannelFormat::UNKNOWN) == 0);
+    CHECK(LossToPSNR(0.01f) == 20.f);
+
+    ITextureSet* set = nullptr;
+    TextureSetDesc desc;                       // all zero
+    TextureSetFeatures features;
+    CHECK(ctx->CreateTextureSet(desc, features, &set) == Status::OutOfRange && set == nullptr);
+    desc.width = 4096; desc.height = 4096; desc.channels = 17; desc.mips = 13;
+    CHECK(ctx->CreateTextureSet(desc, features, &set) == Status::OutOfRange);
+    CHECK(std::strstr(GetLastErrorMessage(), "too many channels") != nullptr);
+    desc.channels = 15;
+    CHECK(ctx->CreateTextureSet(desc, features, nullptr) == Status::InvalidArgument);
+    CHECK(ctx->CreateTextureSet(desc, features, &set) == Status::Ok && set != nullptr);
+    CHECK(set->GetDesc().channels == 16);       // rounded up to even (src/TextureSet.cpp:86)
+    CHECK(set->GetLatentShape().IsEmpty() && set->GetValidChannelMask() == 0);
+    CHECK(set->GetLatentDataSize() == 0);
+
+    // Decompress on an empty set: InvalidState (src/TextureSet.cpp:1666-1673)
+    CHECK(set->Decompress(nullptr) == Status::InvalidState);
+    CHECK(std::strstr(GetLastErrorMessage(), "Invalid network state for Decompress") != nullptr);
+
+    LatentShape shape; shape.gridSizeScale = 7; shape.numFeatures = 16;
+    CHECK(set->SetLatentShape(shape) == Status::OutOfRange);
+    CHECK(std::strstr(GetLastErrorMessage(), "gridSizeScale (7) must be between 1 and 6") != nullptr);
+    shape.gridSizeScale = 2; shape.numFeatures = 10;
+    CHECK(set->SetLatentShape(shape) == Status::OutOfRange);
+    shape.numFeatures = 16;
+    CHECK(set->SetLatentShape(shape) == Status::Ok);
+    CHECK(set->GetWeightDataSize() == 9472);                 // src/WeightLayout.cpp, 48-64-48-32-16
+    CHECK(set->GetLatentDataSize() == 44738560ull);          // 4096^2, grid scale 2, 16 features, 13 mips
+    CHECK(set->Decompress(nullptr) == Status::InvalidState); // shape set, no data yet
+    std::vector<unsigned char> blob(9472);
+    CHECK(set->SetWeightData(blob.data(), 100) == Status::InvalidArgument);
+    CHECK(set->SetWeightData(nullptr, 9472) == Status::InvalidArgument);
+    CHECK(set->SetWeightData(blob.data(), blob.size()) == Status::CudaUnavailable);
+    CHECK(set->SetDecoderPreset(DecoderPreset::Concat2x2_64) == Status::Ok);
+    CHECK(set->GetWeightDataSize() == 10496 && set->GetLatentDataSize() == 22369636ull);
+    CHECK(set->SetDecoderPreset(DecoderPreset::Concat2x2_48) == Status::Ok);
+    CHECK(set->GetWeightDataSize() == 8576);
+
+    // ReadChannels argument checks (src/TextureSet.cpp:1914-1956)
+    std::vector<unsigned char> pixels(16);
+    ReadChannelsParameters rp;
+    CHECK(set->ReadChannels(rp) == Status::InvalidArgument);                 // pOutData NULL
+    rp.pOutData = pixels.data(); rp.mipLevel = 13;
+    CHECK(set->ReadChannels(rp) == Status::OutOfRange);
+    rp.mipLevel = 12; rp.firstChannel = 16;
+    CHECK(set->ReadChannels(rp) == Status::OutOfRange);
+    rp.firstChannel = 14; rp.numChannels = 3;
+    CHECK(set->ReadChannels(rp) == Status::OutOfRange);
+    rp.numChannels = 2;
+    CHECK(set->ReadChannels(rp) == Status::OutOfRange);                      // width/height 0
+    rp.width = 1; rp.height = 1; rp.pixelStride = 4; rp.rowPitch = 2;
+    CHECK(set->ReadChannels(rp) == Status::InvalidArgument);
+    rp.rowPitch = 4; rp.channelFormat = ChannelFormat::UNORM8;
+    CHECK(set->ReadChannels(rp) == Status::CudaUnavailable);                 // arguments fine, no device
+
+    ctx->DestroyTextureSet(set);
+    DestroyContext(ctx);
+    std::printf("host cpu checks OK\n");
+    return 0;
+}
+
+static int decode(int argc, char** argv)
+{
+    if (argc < 12) { std::fprintf(stderr, "usage: decode <preset> <w> <h> <mips> <channels> <gridScale> <features> <latents> <weights> <outPrefix>\n"); return 2; }
+    int const preset = std::atoi(argv[2]), w = std::atoi(argv[3]), h = std::atoi(argv[4]), mips = std::atoi(argv[5]);
+    int const channels = std::atoi(argv[6]), gridScale = std::atoi(argv[7]), features = std::atoi(argv[8]);
+    std::vector<unsigned char> latents = readFile(argv[9]), weights = readFile(argv[10]);
+    std::string const prefix = argv[11];
+
+    IContext* ctx = nullptr;
+    ContextParameters params;
+    CHECK(CreateContext(&ctx, params) == Status::Ok);
+    CHECK(ctx->IsCudaAvailable());
+    TextureSetDesc desc; desc.width = w; desc.height = h; desc.channels = channels; desc.mips = mips;
+    TextureSetFeatures features_;
+    features_.stagingBytesPerPixel = 16 * 4;
+    ITextureSet* set = nullptr;
+    CHECK(ctx->CreateTextureSet(desc, features_, &set) == Status::Ok);
+    if (preset == 0) { LatentShape shape; shape.gridSizeScale = gridScale; shape.numFeatures = features; CHECK(set->SetLatentShape(shape) == Status::Ok); }
+    else CHECK(set->SetDecoderPreset(DecoderPreset(preset)) == Status::Ok);
+    CHECK(set->GetLatentDataSize() == latents.size());
+    CHECK(set->GetWeightDataSize() == weights.size());
+    CHECK(set->SetLatentData(latents.data(), latents.size()) == Status::Ok);
+    CHECK(set->Decompress(nullptr) == Status::InvalidState);                // weights still missing
+    CHECK(set->SetWeightData(weights.data(), weights.size()) == Status::Ok);
+    DecompressionStats stats;
+    CHECK(set->Decompress(&stats) == Status::Ok);
+    CHECK(stats.gpuTimeMilliseconds > 0.f && stats.overallLoss == 0.f);
+    CHECK(set->Decompress(nullptr) == Status::Ok);                           // asynchronous form, idempotent
+    int const C = set->GetDesc().channels;
+    for (int mip = 0; mip < mips; ++mip) {
+        int const mw = std::max(w >> mip, 1), mh = std::max(h >> mip, 1);
+        // UNORM8, all channels, host memory, padded rows
+        ReadChannelsParameters rp;
+        rp.mipLevel = mip; rp.firstChannel = 0; rp.numChannels = C;
+        rp.width = mw; rp.height = mh; rp.pixelStride = size_t(C); rp.rowPitch = size_t(C) * size_t(mw) + 8;
+        rp.channelFormat = ChannelFormat::UNORM8;
+        std::vector<unsigned char> u8(rp.rowPitch * size_t(mh), 0xEE);
+        rp.pOutData = u8.data();
+        CHECK(set->ReadChannels(rp) == Status::Ok);
+        CHECK(writeFile(prefix + "_mip" + std::to_string(mip) + "_unorm8.bin", u8.data(), u8.size()));
+        // FLOAT16, channels 1..3 into an RGBA pixel (4th channel takes the default), device memory
+        if (C >= 4) {
+            void* dev = nullptr;
+            size_t const bytes = size_t(mw) * size_t(mh) * 8;
+            CHECK(ntc_hip_alloc(&dev, bytes) == 0);
+            ReadChannelsParameters rd;
+            rd.mipLevel = mip; rd.firstChannel = 1; rd.numChannels = 3;
+            rd.width = mw; rd.height = mh; rd.pixelStride = 8; rd.rowPitch = size_t(mw) * 8;
+            rd.channelFormat = ChannelFormat::FLOAT16; rd.addressSpace = AddressSpace::Device;
+            rd.pOutData = static_cast<unsigned char*>(dev);
+            CHECK(set->ReadChannels(rd) == Status::Ok);
+            std::vector<unsigned char> f16(bytes);
+            CHECK(ntc_hip_download(f16.data(), dev, bytes) == 0);
+            CHECK(ntc_hip_free(dev) == 0);
+            CHECK(writeFile(prefix + "_mip" + std::to_string(mip) + "_rgba16f.bin", f16.data(), f16.size()));
+        }
+    }
+    // a resizing read is refused, not silently approximated
+    ReadChannelsParameters bad;
+    std::vector<unsigned char> tmp(64);
+    bad.pOutData = tmp.data(); bad.numChannels = 1; bad.width = 2; bad.height = 2; bad.pixelStride = 1; bad.rowPitch = 2;
+    bad.channelFormat = ChannelFormat::UNORM8;
+    if (w != 2 || h != 2) CHECK(set->ReadChannels(bad) == Status::Unsupported);
+    ctx->DestroyTextureSet(set);
+    DestroyContext(ctx);
+    std::printf("host decode OK, gpu %.3f ms\n", stats.gpuTimeMilliseconds);
+    return 0;
+}
+
+int main(int argc, char** argv)
+{
+    if (argc >= 2 && std::strcmp(argv[1], "cpu") == 0) return cpuChecks();
+    if (argc >= 2 && std::strcmp(argv[1], "decode") == 0) return decode(argc, argv);
+    std::fprintf(stderr, "usage: host_api_test cpu | decode ...\n");
+    return 2;
+}
