@@ -168,6 +168,20 @@ int ntc_hip_decode(const NtcHipTextureSet* sets, int32_t numSets);
 int ntc_hip_decode_timed(const NtcHipTextureSet* sets, int32_t numSets, int32_t iterations,
                          float* outMillisecondsPerIteration);
 
+/* Random-access decode: "inference on sample", NtcSampleTextureSet of
+ * include/libntc/shaders/Inference.hlsli:282-357, for a list of sample points instead of a
+ * shader invocation.  Query i decodes texel (floor(u*W), floor(v*H)) of colour mip `mip`
+ * (clamped to the image, as the reference clamps out-of-bounds texels) and writes its 16
+ * network outputs as fp16 at out + 32*i.  A mip index outside the set writes zeros (the
+ * reference returns false and leaves the outputs alone).  The set's output fields are not
+ * used.  Queries and out are device memory.  Asynchronous / timed like ntc_hip_decode. */
+typedef struct NtcHipQuery { float u, v; int32_t mip; } NtcHipQuery;
+int ntc_hip_decode_queries(const NtcHipTextureSet* set, const NtcHipQuery* queries, uint64_t numQueries,
+                           void* out, uint64_t outBytes);
+int ntc_hip_decode_queries_timed(const NtcHipTextureSet* set, const NtcHipQuery* queries, uint64_t numQueries,
+                                 void* out, uint64_t outBytes, int32_t iterations,
+                                 float* outMillisecondsPerIteration);
+
 /* Extracts channels of one decoded mip from the internal fp16 layout into a user image:
  * what ITextureSet::ReadChannels does through cuda::CopyImage (src/TextureSet.cpp:915-985,
  * src/ImageProcessing.cu:141-164,220-277).  Same-size copies only (the reference's 1:1

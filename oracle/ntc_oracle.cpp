@@ -504,6 +504,40 @@ int ntc_oracle_read_channels(const uint16_t* planarPairs, int width, int height,
     return 0;
 }
 
+// Random-access decode of a list of (u, v, mip) sample points: NtcSampleTextureSet
+// (Inference.hlsli:282-357) evaluated at texel (floor(u*W), floor(v*H)) clamped to the mip,
+// 16 outputs per query as fp16 (Inf/NaN -> 0 as in the raster path).  Mips outside the set give zeros.
+int ntc_oracle_decode_queries(const NtcHipTextureSet* set, const float* uvmip /* 3 words per query: u, v, int32 mip */,
+                              uint64_t numQueries, uint16_t* out, int threads)
+{
+    SetView sv{ set, {} };
+    if (set->spec.weightType != NTC_HIP_WEIGHTS_INT8 || !weight_layout(set->spec, sv.layout)) return -1;
+    if (threads < 1) threads = 1;
+    std::atomic<uint64_t> next{0};
+    auto work = [&]() {
+        float o[NTC_HIP_MAX_LAYER_WIDTH];
+        for (;;) {
+            uint64_t const q0 = next.fetch_add(1024);
+            if (q0 >= numQueries) break;
+            for (uint64_t q = q0; q < std::min(numQueries, q0 + 1024); ++q) {
+                float const u = uvmip[3 * q], v = uvmip[3 * q + 1];
+                int32_t mipIndex; std::memcpy(&mipIndex, &uvmip[3 * q + 2], 4);
+                if (mipIndex < 0 || mipIndex >= set->numMips) { std::memset(out + 16 * q, 0, 32); continue; }
+                NtcHipMipDesc const& mip = set->mips[mipIndex];
+                int x = int(std::floor(u * float(mip.width))), y = int(std::floor(v * float(mip.height)));
+                x = std::max(0, std::min(x, mip.width - 1));
+                y = std::max(0, std::min(y, mip.height - 1));
+                decode_texel_int8(sv, mip, x, y, o, nullptr);
+                for (int c = 0; c < 16; ++c) out[16 * q + uint64_t(c)] = output_to_half(o[c]);
+            }
+        }
+    };
+    std::vector<std::thread> pool;
+    for (int i = 0; i < threads; ++i) pool.emplace_back(work);
+    for (auto& t : pool) t.join();
+    return 0;
+}
+
 // Decodes every mip of one set into set->output (host memory).  Rows of each mip are handed
 // out in bands to `threads` workers.  Returns seconds spent decoding (steady clock), < 0 on error.
 double ntc_oracle_decode(const NtcHipTextureSet* set, int threads)

@@ -77,6 +77,10 @@ class ReadChannels(C.Structure):
     ]
 
 
+class Query(C.Structure):
+    _fields_ = [("u", C.c_float), ("v", C.c_float), ("mip", C.c_int32)]
+
+
 FORMAT_UNORM8, FORMAT_UNORM16, FORMAT_FLOAT16, FORMAT_FLOAT32, FORMAT_UINT32 = 1, 2, 3, 4, 5
 
 
@@ -103,6 +107,9 @@ EXPORTS = [
     ("ntc_hip_grid_bytes", C.c_uint64, [C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     ("ntc_hip_decode", C.c_int, [C.POINTER(TextureSet), C.c_int32]),
     ("ntc_hip_decode_timed", C.c_int, [C.POINTER(TextureSet), C.c_int32, C.c_int32, C.POINTER(C.c_float)]),
+    ("ntc_hip_decode_queries", C.c_int, [C.POINTER(TextureSet), C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint64]),
+    ("ntc_hip_decode_queries_timed", C.c_int, [C.POINTER(TextureSet), C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint64,
+                                               C.c_int32, C.POINTER(C.c_float)]),
     ("ntc_hip_read_channels", C.c_int, [C.POINTER(ReadChannels)]),
     ("ntc_hip_selftest_mfma", C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
 ]

@@ -43,6 +43,9 @@ struct DevMip {
     uint32_t posMask;          // (texels per period of the positional encoding) - 1
 };
 
+// One random-access query (same layout as NtcHipQuery of the C ABI).
+struct DevQuery { float u, v; int32_t mip; };
+
 constexpr int kTileWidth = 64, kTileHeight = 4;
 
 // ChannelFormat values of the reference (include/libntc/ntc.h:227-236)
@@ -60,6 +63,8 @@ struct ReadChannelsArgs {
 hipError_t launch_read_channels(ReadChannelsArgs const& args, hipStream_t stream);
 
 hipError_t launch_decode(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream);
+hipError_t launch_queries(int variant, DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries,
+                          uint16_t* out, int gridSize, hipStream_t stream);
 int resident_workgroups_per_cu(int variant);
 hipError_t launch_selftest_mfma(int8_t const* a, int8_t const* b, int32_t* d, hipStream_t stream);
 

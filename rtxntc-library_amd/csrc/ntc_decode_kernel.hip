@@ -523,6 +523,71 @@ __device__ void build_posenc_tables(Lds& lds, float positionScale)
     }
 }
 
+// The network for the 64 texels of one wave.  `in` is the lane's own texel (lane = 16*b + j).
+// On return D[b] holds, for lane (j = lane%16, g = lane/16), the int32 accumulators of output
+// channels 4g..4g+3 of texel 16*b + j, and S their scales.
+template <class V>
+__device__ __forceinline__ void mlp_forward(Lds& lds, int wave, int lane, uint32_t const (&in)[16], uint32_t c143,
+                                            v4i (&D)[4], v4f& S)
+{
+    int const j = lane & 15, g = lane >> 4;
+    {
+        uint4* dst = reinterpret_cast<uint4*>(&lds.in[wave][lane][0]);
+        dst[0] = make_uint4(in[0], in[1], in[2], in[3]);
+        dst[1] = make_uint4(in[4], in[5], in[6], in[7]);
+        dst[2] = make_uint4(in[8], in[9], in[10], in[11]);
+        dst[3] = make_uint4(in[12], in[13], in[14], in[15]);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    // B operands of layer 0: block b = texels 16b..16b+15, column j, k-group g
+    v4i X[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        uint4 const t = *reinterpret_cast<uint4 const*>(&lds.in[wave][b * 16 + j][4 * g]);
+        X[b] = v4i{ int(t.x), int(t.y), int(t.z), int(t.w) };
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    // hidden layers
+    constexpr int tiles[3] = { V::T0, V::T1, V::T2 };
+    int tb = 0;
+#pragma unroll
+    for (int l = 0; l < 3; ++l) {
+        uint32_t Y[4][4];
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+#pragma unroll
+            for (int d = 0; d < 4; ++d) Y[b][d] = 0;
+#pragma unroll
+        for (int t = 0; t < tiles[l]; ++t) {
+            uint4 const wa = *reinterpret_cast<uint4 const*>(&lds.w[tb + t][lane][0]);
+            v4i const A = v4i{ int(wa.x), int(wa.y), int(wa.z), int(wa.w) };
+            v4i const C = *reinterpret_cast<v4i const*>(&lds.bias[tb + t][g][0]);
+            v4f const Sc = *reinterpret_cast<v4f const*>(&lds.scale[tb + t][g][0]);
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                v4i const Dh = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
+                Y[b][t] = activate4(Dh, Sc, c143);
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < 4; ++b) X[b] = v4i{ int(Y[b][0]), int(Y[b][1]), int(Y[b][2]), int(Y[b][3]) };
+        tb += tiles[l];
+    }
+
+    // output layer
+    uint4 const wa = *reinterpret_cast<uint4 const*>(&lds.w[tb][lane][0]);
+    v4i const A = v4i{ int(wa.x), int(wa.y), int(wa.z), int(wa.w) };
+    v4i const C = *reinterpret_cast<v4i const*>(&lds.bias[tb][g][0]);
+    S = *reinterpret_cast<v4f const*>(&lds.scale[tb][g][0]);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) D[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
+}
+
 template <class V>
 __global__ void __launch_bounds__(256, 2)
 decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
@@ -571,70 +636,74 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
         if (x0 >= m.width) continue;                         // whole wave tile outside the image
 
         // ---- 1. input stage: lane = texel (tx = lane%16, ty = lane/16)
+        uint32_t in[16];
         {
             int const x = min(x0 + j, m.width - 1), y = min(y0 + g, m.height - 1);
-            uint32_t in[16];
             if (m.fast) prepare_inputs_fast<V>(m, lds, x, y, in);
             else        prepare_inputs_general<V>(m, x, y, in);
-            uint4* dst = reinterpret_cast<uint4*>(&lds.in[wave][lane][0]);
-            dst[0] = make_uint4(in[0], in[1], in[2], in[3]);
-            dst[1] = make_uint4(in[4], in[5], in[6], in[7]);
-            dst[2] = make_uint4(in[8], in[9], in[10], in[11]);
-            dst[3] = make_uint4(in[12], in[13], in[14], in[15]);
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-
-        // ---- 2. B operands of layer 0: block b = tile row b, column j, k-group g
-        v4i X[4];
-#pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            uint4 const t = *reinterpret_cast<uint4 const*>(&lds.in[wave][b * 16 + j][4 * g]);
-            X[b] = v4i{ int(t.x), int(t.y), int(t.z), int(t.w) };
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-
-        // ---- 3. hidden layers
-        constexpr int tiles[3] = { V::T0, V::T1, V::T2 };
-        int tb = 0;
-#pragma unroll
-        for (int l = 0; l < 3; ++l) {
-            uint32_t Y[4][4];
-#pragma unroll
-            for (int b = 0; b < 4; ++b)
-#pragma unroll
-                for (int d = 0; d < 4; ++d) Y[b][d] = 0;
-#pragma unroll
-            for (int t = 0; t < tiles[l]; ++t) {
-                uint4 const wa = *reinterpret_cast<uint4 const*>(&lds.w[tb + t][lane][0]);
-                v4i const A = v4i{ int(wa.x), int(wa.y), int(wa.z), int(wa.w) };
-                v4i const C = *reinterpret_cast<v4i const*>(&lds.bias[tb + t][g][0]);
-                v4f const S = *reinterpret_cast<v4f const*>(&lds.scale[tb + t][g][0]);
-#pragma unroll
-                for (int b = 0; b < 4; ++b) {
-                    v4i const D = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
-                    Y[b][t] = activate4(D, S, c143);
-                }
-            }
-#pragma unroll
-            for (int b = 0; b < 4; ++b) X[b] = v4i{ int(Y[b][0]), int(Y[b][1]), int(Y[b][2]), int(Y[b][3]) };
-            tb += tiles[l];
-        }
-
-        // ---- 4. output layer + stores: lane (j, g) holds channels 4g..4g+3 of texel (x0+j, y0+b)
+        // ---- 2.-4. transpose, hidden layers, output layer
         {
-            uint4 const wa = *reinterpret_cast<uint4 const*>(&lds.w[tb][lane][0]);
-            v4i const A = v4i{ int(wa.x), int(wa.y), int(wa.z), int(wa.w) };
-            v4i const C = *reinterpret_cast<v4i const*>(&lds.bias[tb][g][0]);
-            v4f const S = *reinterpret_cast<v4f const*>(&lds.scale[tb][g][0]);
             v4i D[4];
-#pragma unroll
-            for (int b = 0; b < 4; ++b) D[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
+            v4f S;
+            mlp_forward<V>(lds, wave, lane, in, c143, D, S);
             if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)      store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, x0 + j, y0, 4 * g);
             else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)       store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
             else                                                       store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
+        }
+    }
+}
+
+// Random-access decode ("inference on sample", NtcSampleTextureSet of Inference.hlsli:282-357):
+// one query = (u, v, mip) -> the 16 outputs of texel (floor(u*W), floor(v*H)) of that mip, clamped to
+// the image, as 16 fp16.  Lane = query in the input stage (each lane carries its own mip, so the
+// general per-lane stage is used); the network is the same 64-column tile as in raster decode.
+// A query whose mip is out of range writes zeros.
+template <class V>
+__global__ void __launch_bounds__(256, 2)
+query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __restrict__ queries, uint64_t numQueries,
+             uint16_t* __restrict__ out)
+{
+    __shared__ Lds lds;
+    int const lane = threadIdx.x & 63;
+    int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int const j = lane & 15, g = lane >> 4;
+
+    uint32_t c143 = 143u;
+    asm volatile("" : "+v"(c143));
+
+    stage_weights<V>(lds, mips[0].weights);
+    __syncthreads();
+
+    uint64_t const numBlocks = (numQueries + 255) / 256;
+    for (uint64_t block = blockIdx.x; block < numBlocks; block += gridDim.x) {
+        uint64_t const q0 = block * 256 + uint64_t(wave) * 64;
+        if (q0 >= numQueries) continue;
+        uint64_t const qi = min(q0 + uint64_t(lane), numQueries - 1);
+        DevQuery const query = queries[qi];
+        bool const validMip = query.mip >= 0 && query.mip < numMips;
+        DevMip const& m = mips[validMip ? query.mip : 0];
+        int x = int(floorf(query.u * float(m.width)));
+        int y = int(floorf(query.v * float(m.height)));
+        x = max(0, min(x, m.width - 1));
+        y = max(0, min(y, m.height - 1));
+        uint32_t in[16];
+        prepare_inputs_general<V>(m, x, y, in);
+
+        v4i D[4];
+        v4f S;
+        mlp_forward<V>(lds, wave, lane, in, c143, D, S);
+
+        // lane (j, g) holds channels 4g..4g+3 of query q0 + 16b + j; validity travels by shuffle
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            uint64_t const q = q0 + uint64_t(16 * b + j);
+            int const ok = __shfl(validMip ? 1 : 0, 16 * b + j, 64);
+            if (q >= numQueries) continue;
+            uint32_t h01 = to_half2_bits(float(D[b][0]) * S[0], float(D[b][1]) * S[1]);
+            uint32_t h23 = to_half2_bits(float(D[b][2]) * S[2], float(D[b][3]) * S[3]);
+            if (!ok) { h01 = 0; h23 = 0; }
+            *reinterpret_cast<u32x2*>(out + q * 16 + 4 * g) = u32x2{ h01, h23 };
         }
     }
 }
@@ -686,6 +755,28 @@ hipError_t launch_decode(int variant, DevMip const* mips, int numMips, int total
     case NTC_HIP_VARIANT_REF12: return launch_variant<VRef12>(mips, numMips, totalTiles, gridSize, stream);
     case NTC_HIP_VARIANT_REF8:  return launch_variant<VRef8>(mips, numMips, totalTiles, gridSize, stream);
     case NTC_HIP_VARIANT_REF4:  return launch_variant<VRef4>(mips, numMips, totalTiles, gridSize, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+template <class V>
+static hipError_t launch_query_variant(DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries,
+                                       uint16_t* out, int gridSize, hipStream_t stream)
+{
+    hipLaunchKernelGGL(query_kernel<V>, dim3(gridSize), dim3(256), 0, stream, mips, numMips, queries, numQueries, out);
+    return hipGetLastError();
+}
+
+hipError_t launch_queries(int variant, DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries,
+                          uint16_t* out, int gridSize, hipStream_t stream)
+{
+    switch (variant) {
+    case NTC_HIP_VARIANT_CFG01: return launch_query_variant<VCfg01>(mips, numMips, queries, numQueries, out, gridSize, stream);
+    case NTC_HIP_VARIANT_CFG2:  return launch_query_variant<VCfg2>(mips, numMips, queries, numQueries, out, gridSize, stream);
+    case NTC_HIP_VARIANT_REF16: return launch_query_variant<VRef16>(mips, numMips, queries, numQueries, out, gridSize, stream);
+    case NTC_HIP_VARIANT_REF12: return launch_query_variant<VRef12>(mips, numMips, queries, numQueries, out, gridSize, stream);
+    case NTC_HIP_VARIANT_REF8:  return launch_query_variant<VRef8>(mips, numMips, queries, numQueries, out, gridSize, stream);
+    case NTC_HIP_VARIANT_REF4:  return launch_query_variant<VRef4>(mips, numMips, queries, numQueries, out, gridSize, stream);
     default: return hipErrorInvalidValue;
     }
 }

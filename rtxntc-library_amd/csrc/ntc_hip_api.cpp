@@ -150,7 +150,8 @@ uint64_t grid_bytes(int32_t w, int32_t h, int32_t features, int32_t bits)
 }
 
 // Validates the sets, builds the mip table (sorted by tileStart) and picks the kernel.
-int build_table(NtcHipTextureSet const* sets, int32_t numSets, std::vector<DevMip>& table, int& variant, int& totalTiles)
+int build_table(NtcHipTextureSet const* sets, int32_t numSets, std::vector<DevMip>& table, int& variant, int& totalTiles,
+                bool forQueries = false)
 {
     if (!sets || numSets < 1) { set_error("ntc_hip_decode: no texture sets given."); return NTC_HIP_ERR_INVALID_ARG; }
     table.clear();
@@ -164,8 +165,8 @@ int build_table(NtcHipTextureSet const* sets, int32_t numSets, std::vector<DevMi
         }
         if (set.numMips < 1 || set.numMips > NTC_HIP_MAX_MIPS) { set_error("ntc_hip_decode: set %d: numMips %d out of range 1..%d.", s, set.numMips, NTC_HIP_MAX_MIPS); return NTC_HIP_ERR_INVALID_ARG; }
         if (set.numChannels < 1 || set.numChannels > NTC_HIP_MAX_CHANNELS) { set_error("ntc_hip_decode: set %d: numChannels %d out of range 1..%d.", s, set.numChannels, NTC_HIP_MAX_CHANNELS); return NTC_HIP_ERR_INVALID_ARG; }
-        if (!set.latents || !set.weights || !set.output) { set_error("ntc_hip_decode: set %d: null latents / weights / output pointer.", s); return NTC_HIP_ERR_INVALID_ARG; }
-        if (set.outputFormat < NTC_HIP_OUT_FP16_PLANAR_PAIRS || set.outputFormat > NTC_HIP_OUT_UNORM8_PIXELS) { set_error("ntc_hip_decode: set %d: unknown output format %d.", s, set.outputFormat); return NTC_HIP_ERR_INVALID_ARG; }
+        if (!set.latents || !set.weights || (!set.output && !forQueries)) { set_error("ntc_hip_decode: set %d: null latents / weights / output pointer.", s); return NTC_HIP_ERR_INVALID_ARG; }
+        if (!forQueries && (set.outputFormat < NTC_HIP_OUT_FP16_PLANAR_PAIRS || set.outputFormat > NTC_HIP_OUT_UNORM8_PIXELS)) { set_error("ntc_hip_decode: set %d: unknown output format %d.", s, set.outputFormat); return NTC_HIP_ERR_INVALID_ARG; }
         if ((reinterpret_cast<uintptr_t>(set.weights) & 3u) || (reinterpret_cast<uintptr_t>(set.latents) & 1u)) { set_error("ntc_hip_decode: set %d: weights must be 4-byte and latents 2-byte aligned.", s); return NTC_HIP_ERR_INVALID_ARG; }
         NtcHipWeightLayout layout;
         if (ntc_hip_weight_layout(&set.spec, &layout) != 0) return NTC_HIP_ERR_INVALID_ARG;
@@ -175,7 +176,7 @@ int build_table(NtcHipTextureSet const* sets, int32_t numSets, std::vector<DevMi
             return NTC_HIP_ERR_INVALID_ARG;
         }
         int const bytesPerChannel = set.outputFormat == NTC_HIP_OUT_UNORM8_PIXELS ? 1 : 2;
-        if (set.outputFormat != NTC_HIP_OUT_FP16_PLANAR_PAIRS && set.outPixelStride < set.numChannels * bytesPerChannel) {
+        if (!forQueries && set.outputFormat != NTC_HIP_OUT_FP16_PLANAR_PAIRS && set.outPixelStride < set.numChannels * bytesPerChannel) {
             set_error("ntc_hip_decode: set %d: pixel stride %d is smaller than %d channels.", s, set.outPixelStride, set.numChannels);
             return NTC_HIP_ERR_INVALID_ARG;
         }
@@ -187,7 +188,9 @@ int build_table(NtcHipTextureSet const* sets, int32_t numSets, std::vector<DevMi
                 return NTC_HIP_ERR_INVALID_ARG;
             }
             if ((d.hrOffset & 1u) || (d.lrOffset & 1u)) { set_error("ntc_hip_decode: set %d mip %d: latent offsets must be even.", s, m); return NTC_HIP_ERR_INVALID_ARG; }
-            if (set.outputFormat == NTC_HIP_OUT_FP16_PLANAR_PAIRS) {
+            if (forQueries) {
+                // no per-mip output
+            } else if (set.outputFormat == NTC_HIP_OUT_FP16_PLANAR_PAIRS) {
                 if (d.outOffset & 3u) { set_error("ntc_hip_decode: set %d mip %d: planar output offset must be 4-byte aligned.", s, m); return NTC_HIP_ERR_INVALID_ARG; }
             } else if (d.outRowPitch < uint64_t(d.width) * uint64_t(set.outPixelStride)) {
                 set_error("ntc_hip_decode: set %d mip %d: row pitch smaller than a row.", s, m);
@@ -206,7 +209,7 @@ int build_table(NtcHipTextureSet const* sets, int32_t numSets, std::vector<DevMi
             else
                 outBytes = uint64_t(d.height - 1) * d.outRowPitch + uint64_t(d.width - 1) * uint64_t(set.outPixelStride)
                          + uint64_t(set.numChannels * bytesPerChannel);
-            if (d.outOffset + outBytes > set.outputBytes) {
+            if (!forQueries && d.outOffset + outBytes > set.outputBytes) {
                 set_error("ntc_hip_decode: set %d mip %d: output reaches past the %llu-byte output buffer.", s, m,
                           (unsigned long long)set.outputBytes);
                 return NTC_HIP_ERR_INVALID_ARG;
@@ -454,6 +457,48 @@ int ntc_hip_decode_timed(const NtcHipTextureSet* sets, int32_t numSets, int32_t 
     *outMs = ms / float(iterations);
     clear_error();
     return 0;
+}
+
+static int run_queries(const NtcHipTextureSet* set, const NtcHipQuery* queries, uint64_t numQueries, void* out, uint64_t outBytes,
+                       int iterations, float* outMs)
+{
+    if (int r = require_init()) return r;
+    if (!set || !queries || !out) { set_error("ntc_hip_decode_queries: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
+    if (numQueries == 0) { if (outMs) *outMs = 0.f; return 0; }
+    if (outBytes < numQueries * 32u) { set_error("ntc_hip_decode_queries: the output buffer holds %llu bytes, %llu queries need %llu.", (unsigned long long)outBytes, (unsigned long long)numQueries, (unsigned long long)(numQueries * 32u)); return NTC_HIP_ERR_INVALID_ARG; }
+    if ((reinterpret_cast<uintptr_t>(out) & 7u) || (reinterpret_cast<uintptr_t>(queries) & 3u)) { set_error("ntc_hip_decode_queries: output must be 8-byte and queries 4-byte aligned."); return NTC_HIP_ERR_INVALID_ARG; }
+    std::vector<DevMip> table;
+    int variant = NTC_HIP_VARIANT_NONE, totalTiles = 0;
+    if (int r = build_table(set, 1, table, variant, totalTiles, true)) return r;
+    if (int r = upload_table(table)) return r;
+    uint64_t const blocks = (numQueries + 255) / 256;
+    uint64_t const resident = uint64_t(g_lib.computeUnits) * uint64_t(grid_size_for(variant, 0x7fffffff) / g_lib.computeUnits);
+    int const grid = int(blocks < resident ? blocks : resident);
+    if (outMs) HIP_TRY(hipEventRecord(g_lib.evStart, g_lib.stream));
+    for (int i = 0; i < iterations; ++i)
+        HIP_TRY(launch_queries(variant, g_lib.tableDev, int(table.size()), reinterpret_cast<DevQuery const*>(queries), numQueries,
+                               static_cast<uint16_t*>(out), grid, g_lib.stream));
+    if (outMs) {
+        HIP_TRY(hipEventRecord(g_lib.evStop, g_lib.stream));
+        HIP_TRY(hipEventSynchronize(g_lib.evStop));
+        float ms = 0.f;
+        HIP_TRY(hipEventElapsedTime(&ms, g_lib.evStart, g_lib.evStop));
+        *outMs = ms / float(iterations);
+    }
+    clear_error();
+    return 0;
+}
+
+int ntc_hip_decode_queries(const NtcHipTextureSet* set, const NtcHipQuery* queries, uint64_t numQueries, void* out, uint64_t outBytes)
+{
+    return run_queries(set, queries, numQueries, out, outBytes, 1, nullptr);
+}
+
+int ntc_hip_decode_queries_timed(const NtcHipTextureSet* set, const NtcHipQuery* queries, uint64_t numQueries, void* out, uint64_t outBytes,
+                                 int32_t iterations, float* outMillisecondsPerIteration)
+{
+    if (iterations < 1 || !outMillisecondsPerIteration) { set_error("ntc_hip_decode_queries_timed: iterations must be >= 1 and the result pointer non-null."); return NTC_HIP_ERR_INVALID_ARG; }
+    return run_queries(set, queries, numQueries, out, outBytes, iterations, outMillisecondsPerIteration);
 }
 
 int ntc_hip_read_channels(const NtcHipReadChannels* p)

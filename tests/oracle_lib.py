@@ -49,6 +49,8 @@ def load_oracle():
         lib.ntc_oracle_decode.argtypes = [C.POINTER(_abi.TextureSet), C.c_int]
         lib.ntc_oracle_decode_rows.restype = C.c_double
         lib.ntc_oracle_decode_rows.argtypes = [C.POINTER(_abi.TextureSet), C.c_int, C.c_int, C.c_int, C.c_int]
+        lib.ntc_oracle_decode_queries.restype = C.c_int
+        lib.ntc_oracle_decode_queries.argtypes = [C.POINTER(_abi.TextureSet), C.c_void_p, C.c_uint64, C.c_void_p, C.c_int]
         lib.ntc_oracle_read_channels.restype = C.c_int
         lib.ntc_oracle_read_channels.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p,
                                                  C.c_int, C.c_uint64, C.c_uint64]
