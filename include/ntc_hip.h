@@ -55,7 +55,16 @@ typedef enum NtcHipGridMode {
 
 typedef enum NtcHipWeightType {
     NTC_HIP_WEIGHTS_INT8 = 0, /* GenericInt8 blob, src/WeightLayout.cpp:42-49,184-247 */
-    NTC_HIP_WEIGHTS_FP8  = 1  /* e4m3 hidden layers + int8 output layer */
+    /* The reference's GenericFP8 blob (src/WeightLayout.cpp:51-71,249-262): e4m3 matrices and fp16
+     * biases for the hidden layers, int8 + fp32 scale + int32 bias for the output layer.  Only the
+     * layout helper knows it; no decode kernel consumes it. */
+    NTC_HIP_WEIGHTS_FP8  = 1,
+    /* Laid out exactly like NTC_HIP_WEIGHTS_INT8, but the bytes of the three hidden-layer matrices
+     * are OCP e4m3 values w.  A hidden layer computes acc = bias_i32 + sum(512*w * in) exactly in
+     * int32 (the result of an fp32-accumulating dot product without its rounding noise), then
+     * r = float(acc) * scale as in the int8 path, so `scale` is per unit of w/512.  Inputs and
+     * activations stay int8.  NaN encodings decode as 0. */
+    NTC_HIP_WEIGHTS_FP8_SCALED = 2
 } NtcHipWeightType;
 
 typedef enum NtcHipOutputFormat {

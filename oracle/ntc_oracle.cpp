@@ -152,7 +152,7 @@ bool weight_layout(NtcHipDecoderSpec const& s, NtcHipWeightLayout& L)
         L.weightOffset[l] = off;
         off += uint32_t(layer_inputs(s, l) * layer_outputs(s, l));
     }
-    if (s.weightType == NTC_HIP_WEIGHTS_INT8) {
+    if (s.weightType == NTC_HIP_WEIGHTS_INT8 || s.weightType == NTC_HIP_WEIGHTS_FP8_SCALED) {
         for (int l = 0; l < NTC_HIP_MLP_LAYERS; ++l) {       // all fp32 scale vectors ...
             L.scaleOffset[l] = off;
             off += 4u * uint32_t(layer_outputs(s, l));
@@ -293,6 +293,31 @@ void layer_int8(int8_t const* W, float const* scale, int32_t const* bias,
     }
 }
 
+// OCP FP8 e4m3 (sign, 4 exponent bits with bias 7, 3 mantissa bits; no infinities, the all-ones
+// pattern is NaN): the weight format of the reference's FP8 layers (src/Quantizer.cu:210-252 stores
+// __nv_fp8_e4m3 bytes; src/tin/tin_activation.h:44-81 describes the same grid, max 448).
+// Returned as the exact integer 512*value (smallest subnormal 2^-9 -> 1, largest 448 -> 229376).
+int32_t e4m3_times_512(uint8_t byte)
+{
+    int const e = (byte >> 3) & 15, m = byte & 7;
+    if ((byte & 0x7f) == 0x7f) return 0;                       // NaN encodings decode as zero
+    int32_t const mag = (e == 0) ? m : ((8 + m) << (e - 1));
+    return (byte & 0x80) ? -mag : mag;
+}
+
+// A hidden layer with e4m3 weights: the dot product of an fp32-accumulating implementation,
+// taken without accumulation noise - the exact sum of (512 w)*x in int32 (wrapping like the
+// device's accumulators), converted to float once, times the per-channel scale.
+void layer_fp8_weights(uint8_t const* W, float const* scale, int32_t const* bias,
+                       int in, int out, int8_t const* x, float* r)
+{
+    for (int c = 0; c < out; ++c) {
+        int64_t acc = bias[c];
+        for (int k = 0; k < in; ++k) acc += int64_t(x[k]) * int64_t(e4m3_times_512(W[c * in + k]));
+        r[c] = float(int32_t(uint32_t(uint64_t(acc)))) * scale[c];
+    }
+}
+
 struct SetView {
     NtcHipTextureSet const* set;
     NtcHipWeightLayout layout;
@@ -316,6 +341,11 @@ void prepare_inputs(NtcHipTextureSet const& set, NtcHipMipDesc const& mip, int x
                     s.posEncWaves, s.lodInputs, in + hrInputs + lrInputs);   // Inference.hlsli:237-238
 }
 
+inline bool decodable(NtcHipDecoderSpec const& s)
+{
+    return s.weightType == NTC_HIP_WEIGHTS_INT8 || s.weightType == NTC_HIP_WEIGHTS_FP8_SCALED;
+}
+
 // One texel through the int8 network: NtcSampleTextureSet, Inference.hlsli:282-357.
 void decode_texel_int8(SetView const& sv, NtcHipMipDesc const& mip, int x, int y, float* outputs, int8_t* inputsOut)
 {
@@ -328,10 +358,16 @@ void decode_texel_int8(SetView const& sv, NtcHipMipDesc const& mip, int x, int y
     float r[NTC_HIP_MAX_LAYER_WIDTH];
     for (int l = 0; l < NTC_HIP_MLP_LAYERS; ++l) {
         int const in = layer_inputs(s, l), out = layer_outputs(s, l);
-        layer_int8(reinterpret_cast<int8_t const*>(blob + sv.layout.weightOffset[l]),
-                   reinterpret_cast<float const*>(blob + sv.layout.scaleOffset[l]),
-                   reinterpret_cast<int32_t const*>(blob + sv.layout.biasOffset[l]),
-                   in, out, act, r);
+        if (s.weightType == NTC_HIP_WEIGHTS_FP8_SCALED && l < NTC_HIP_MLP_LAYERS - 1)
+            layer_fp8_weights(blob + sv.layout.weightOffset[l],
+                              reinterpret_cast<float const*>(blob + sv.layout.scaleOffset[l]),
+                              reinterpret_cast<int32_t const*>(blob + sv.layout.biasOffset[l]),
+                              in, out, act, r);
+        else
+            layer_int8(reinterpret_cast<int8_t const*>(blob + sv.layout.weightOffset[l]),
+                       reinterpret_cast<float const*>(blob + sv.layout.scaleOffset[l]),
+                       reinterpret_cast<int32_t const*>(blob + sv.layout.biasOffset[l]),
+                       in, out, act, r);
         if (l == NTC_HIP_MLP_LAYERS - 1) break;
         for (int c = 0; c < out; ++c) act[c] = int8_t(hgelu_quantize(r[c]));   // NtcPackInt8x4: & 0xff
     }
@@ -386,6 +422,7 @@ uint16_t ntc_oracle_output_to_half(float f) { return output_to_half(f); }
 uint8_t  ntc_oracle_half_to_unorm8(uint16_t h) { return half_to_unorm8(h); }
 int      ntc_oracle_hgelu_quantize(float x) { return hgelu_quantize(x); }
 int      ntc_oracle_unpack_field(uint16_t w, int index, int bits) { return unpack_field(w, index, bits); }
+int32_t  ntc_oracle_e4m3_times_512(uint8_t byte) { return e4m3_times_512(byte); }
 
 // PackLatentsKernel's QuantizeValue, src/Quantizer.cu:482-488 (encoder side; here only so
 // the tests can check Pack o Unpack = id).
@@ -412,7 +449,7 @@ void ntc_oracle_bilinear_footprint(float u, float v, int gw, int gh, int* xy, fl
 int ntc_oracle_decode_texel(const NtcHipTextureSet* set, int mip, int x, int y, float* outputs, int8_t* inputs)
 {
     SetView sv{ set, {} };
-    if (set->spec.weightType != NTC_HIP_WEIGHTS_INT8 || !weight_layout(set->spec, sv.layout)) return -1;
+    if (!decodable(set->spec) || !weight_layout(set->spec, sv.layout)) return -1;
     decode_texel_int8(sv, set->mips[mip], x, y, outputs, inputs);
     return 0;
 }
@@ -511,7 +548,7 @@ int ntc_oracle_decode_queries(const NtcHipTextureSet* set, const float* uvmip /*
                               uint64_t numQueries, uint16_t* out, int threads)
 {
     SetView sv{ set, {} };
-    if (set->spec.weightType != NTC_HIP_WEIGHTS_INT8 || !weight_layout(set->spec, sv.layout)) return -1;
+    if (!decodable(set->spec) || !weight_layout(set->spec, sv.layout)) return -1;
     if (threads < 1) threads = 1;
     std::atomic<uint64_t> next{0};
     auto work = [&]() {
@@ -543,7 +580,7 @@ int ntc_oracle_decode_queries(const NtcHipTextureSet* set, const float* uvmip /*
 double ntc_oracle_decode(const NtcHipTextureSet* set, int threads)
 {
     SetView sv{ set, {} };
-    if (set->spec.weightType != NTC_HIP_WEIGHTS_INT8 || !weight_layout(set->spec, sv.layout)) return -1.0;
+    if (!decodable(set->spec) || !weight_layout(set->spec, sv.layout)) return -1.0;
     if (threads < 1) threads = 1;
     auto const t0 = std::chrono::steady_clock::now();
     for (int m = 0; m < set->numMips; ++m) {
@@ -578,7 +615,7 @@ double ntc_oracle_decode(const NtcHipTextureSet* set, int threads)
 double ntc_oracle_decode_rows(const NtcHipTextureSet* set, int mipIndex, int y0, int y1, int threads)
 {
     SetView sv{ set, {} };
-    if (set->spec.weightType != NTC_HIP_WEIGHTS_INT8 || !weight_layout(set->spec, sv.layout)) return -1.0;
+    if (!decodable(set->spec) || !weight_layout(set->spec, sv.layout)) return -1.0;
     NtcHipMipDesc const& mip = set->mips[mipIndex];
     y0 = std::max(0, y0); y1 = std::min(mip.height, y1);
     if (threads < 1) threads = 1;

@@ -11,7 +11,7 @@ MAX_CHANNELS = 16
 MLP_LAYERS = 4
 
 GRID_BILINEAR, GRID_CONCAT2X2 = 0, 1
-WEIGHTS_INT8, WEIGHTS_FP8 = 0, 1
+WEIGHTS_INT8, WEIGHTS_FP8, WEIGHTS_FP8_SCALED = 0, 1, 2
 OUT_FP16_PLANAR_PAIRS, OUT_FP16_PIXELS, OUT_UNORM8_PIXELS = 0, 1, 2
 
 ERR_INVALID_ARG, ERR_UNSUPPORTED, ERR_NO_DEVICE, ERR_NOT_INITIALIZED = -1, -2, -3, -4

@@ -19,7 +19,8 @@ enum {
     NTC_HIP_VARIANT_REF16,      // LibNTC 0.9.2: both grids bilinear 4-bit, (lod,lod), IN 48, 64-48-32
     NTC_HIP_VARIANT_REF12,
     NTC_HIP_VARIANT_REF8,
-    NTC_HIP_VARIANT_REF4
+    NTC_HIP_VARIANT_REF4,
+    NTC_HIP_VARIANT_CFG3_FP8    // both grids bilinear 16 x 4-bit, (lod,lod), IN 48, 64-64-64, e4m3 hidden-layer weights
 };
 
 // One colour mip of one texture set, as the kernel sees it.  Entries are sorted by

@@ -262,8 +262,13 @@ __device__ __forceinline__ uint32_t bilinear4_int(uint32_t c00, uint32_t c10, ui
 // ---- decoder variants -----------------------------------------------------------------
 
 template <int HR_MODE_, int HR_F_, int HR_BITS_, int HR_SLOTS_, int LR_F_, int LR_SLOTS_, int LOD_,
-          int IN_, int H0_, int H1_, int H2_>
+          int IN_, int H0_, int H1_, int H2_, bool FP8_WEIGHTS_ = false>
 struct Variant {
+    // e4m3 weights in the three hidden layers: each weight w is the integer 512*w (at most 18 bits
+    // plus sign) split into three 6-bit planes, 512*w = 4096*c2 + 64*c1 + c0, and the layer runs
+    // as three int8 MFMA passes whose int32 results are recombined exactly.
+    static constexpr bool FP8_WEIGHTS = FP8_WEIGHTS_;
+    static constexpr int PLANES = FP8_WEIGHTS_ ? 3 : 1;
     static constexpr int HR_MODE = HR_MODE_, HR_F = HR_F_, HR_BITS = HR_BITS_, HR_SLOTS = HR_SLOTS_;
     static constexpr int LR_F = LR_F_, LR_SLOTS = LR_SLOTS_, LOD = LOD_;
     static constexpr int IN = IN_, H0 = H0_, H1 = H1_, H2 = H2_, OUT = 16;
@@ -281,20 +286,31 @@ struct Variant {
     static_assert(HR_INPUTS % 4 == 0 && LR_INPUTS % 4 == 0, "grid blocks are dword aligned");
 };
 
-struct alignas(16) Lds {
-    uint32_t w[10][64][4];            // A operands: [M-tile][lane][4 dwords]; 10 = max tiles (64+48+32+16)/16
-    float    scale[10][4][4];         // [M-tile][k-group g][r]  -> channel 16t+4g+r
-    int32_t  bias[10][4][4];
+template <class V>
+struct alignas(16) LdsT {
+    uint32_t w[V::PLANES][V::NTILES][64][4];   // A operands: [plane][M-tile][lane][4 dwords]
+    float    scale[V::NTILES][4][4];           // [M-tile][k-group g][r]  -> channel 16t+4g+r
+    int32_t  bias[V::NTILES][4][4];
     uint32_t in[kWaves][kWaveTexels][kInStride];
     uint32_t lut2[256];               // byte of four 2-bit codes -> four input bytes 85*q - 128
     uint32_t xtab[64][4];             // positional encoding by x phase: dword w = enc(px*2^w) | enc(px*2^w+1/4) << 16
     uint32_t ytab[64][4];             // same for y, one byte up
 };
 
+// OCP e4m3 (1-4-3, bias 7, no infinities) byte -> the integer 512*value: subnormals m * 2^-9,
+// normals (8+m) * 2^(e-10).  The two NaN encodings decode as 0.
+__device__ __forceinline__ int32_t e4m3_times_512(uint32_t byte)
+{
+    uint32_t const e = (byte >> 3) & 15u, m = byte & 7u;
+    int32_t mag = (e == 0) ? int32_t(m) : int32_t((8u + m) << (e - 1u));
+    if ((byte & 0x7fu) == 0x7fu) mag = 0;
+    return (byte & 0x80u) ? -mag : mag;
+}
+
 // Copies the int8 blob (src/WeightLayout.cpp:42-49: matrices, then fp32 scales, then int32
 // biases; W[c*IN + k]) into LDS in MFMA operand order.
 template <class V>
-__device__ void stage_weights(Lds& lds, uint8_t const* __restrict__ blob)
+__device__ void stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
 {
     constexpr int ins[4]   = { V::IN, V::H0, V::H1, V::H2 };
     constexpr int tiles[4] = { V::T0, V::T1, V::T2, V::T3 };
@@ -312,7 +328,21 @@ __device__ void stage_weights(Lds& lds, uint8_t const* __restrict__ blob)
             int const k = (l == 0) ? (16 * g + 4 * d) : (16 * d + 4 * g);
             uint32_t v = 0;
             if (k < in) v = blob32[(woff[l] + row * in + k) >> 2];
-            lds.w[tileBase + t][lane][d] = v;
+            if (V::FP8_WEIGHTS && l < 3) {
+                uint32_t p0 = 0, p1 = 0, p2 = 0;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    int32_t const W = e4m3_times_512((v >> (8 * r)) & 0xffu);
+                    p0 |= uint32_t(W & 63) << (8 * r);
+                    p1 |= uint32_t((W >> 6) & 63) << (8 * r);
+                    p2 |= (uint32_t(W >> 12) & 0xffu) << (8 * r);      // signed top plane
+                }
+                lds.w[0][tileBase + t][lane][d] = p0;
+                lds.w[V::PLANES > 1 ? 1 : 0][tileBase + t][lane][d] = p1;
+                lds.w[V::PLANES > 2 ? 2 : 0][tileBase + t][lane][d] = p2;
+            } else {
+                lds.w[0][tileBase + t][lane][d] = v;
+            }
         }
         for (int e = threadIdx.x; e < tiles[l] * 16; e += blockDim.x) {
             int const r = e & 3, g = (e >> 2) & 3, t = e >> 4;
@@ -425,7 +455,7 @@ __device__ __forceinline__ void prepare_inputs_general(DevMip const& m, int x, i
 
 // Input vector of one texel from integer arithmetic only (see axis_fast above).
 template <class V>
-__device__ __forceinline__ void prepare_inputs_fast(DevMip const& m, Lds const& lds, int x, int y, uint32_t (&in)[16])
+__device__ __forceinline__ void prepare_inputs_fast(DevMip const& m, LdsT<V> const& lds, int x, int y, uint32_t (&in)[16])
 {
 #pragma unroll
     for (int i = 0; i < 16; ++i) in[i] = 0;
@@ -506,7 +536,8 @@ __device__ __forceinline__ uint32_t posenc_byte(float p)
 
 // Fills the phase tables for a mip whose positionScale is a power of two: the encoding of
 // texel x depends only on x mod (1/positionScale), and all arithmetic involved is exact.
-__device__ void build_posenc_tables(Lds& lds, float positionScale)
+template <class V>
+__device__ void build_posenc_tables(LdsT<V>& lds, float positionScale)
 {
     int const t = threadIdx.x;
     if (t < 128) {
@@ -527,7 +558,7 @@ __device__ void build_posenc_tables(Lds& lds, float positionScale)
 // On return D[b] holds, for lane (j = lane%16, g = lane/16), the int32 accumulators of output
 // channels 4g..4g+3 of texel 16*b + j, and S their scales.
 template <class V>
-__device__ __forceinline__ void mlp_forward(Lds& lds, int wave, int lane, uint32_t const (&in)[16], uint32_t c143,
+__device__ __forceinline__ void mlp_forward(LdsT<V>& lds, int wave, int lane, uint32_t const (&in)[16], uint32_t c143,
                                             v4i (&D)[4], v4f& S)
 {
     int const j = lane & 15, g = lane >> 4;
@@ -564,14 +595,33 @@ __device__ __forceinline__ void mlp_forward(Lds& lds, int wave, int lane, uint32
             for (int d = 0; d < 4; ++d) Y[b][d] = 0;
 #pragma unroll
         for (int t = 0; t < tiles[l]; ++t) {
-            uint4 const wa = *reinterpret_cast<uint4 const*>(&lds.w[tb + t][lane][0]);
+            uint4 const wa = *reinterpret_cast<uint4 const*>(&lds.w[0][tb + t][lane][0]);
             v4i const A = v4i{ int(wa.x), int(wa.y), int(wa.z), int(wa.w) };
             v4i const C = *reinterpret_cast<v4i const*>(&lds.bias[tb + t][g][0]);
             v4f const Sc = *reinterpret_cast<v4f const*>(&lds.scale[tb + t][g][0]);
+            if constexpr (V::FP8_WEIGHTS) {
+                uint4 const wb = *reinterpret_cast<uint4 const*>(&lds.w[V::PLANES > 1 ? 1 : 0][tb + t][lane][0]);
+                uint4 const wc = *reinterpret_cast<uint4 const*>(&lds.w[V::PLANES > 2 ? 2 : 0][tb + t][lane][0]);
+                v4i const A1 = v4i{ int(wb.x), int(wb.y), int(wb.z), int(wb.w) };
+                v4i const A2 = v4i{ int(wc.x), int(wc.y), int(wc.z), int(wc.w) };
+                v4i const Z = v4i{ 0, 0, 0, 0 };
 #pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                v4i const Dh = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
-                Y[b][t] = activate4(Dh, Sc, c143);
+                for (int b = 0; b < 4; ++b) {
+                    v4i const D0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
+                    v4i const D1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A1, X[b], Z, 0, 0, 0);
+                    v4i const D2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A2, X[b], Z, 0, 0, 0);
+                    v4i Dh;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)                    // 4096*D2 + 64*D1 + D0, wrapping like int32
+                        Dh[r] = int((((uint32_t(D2[r]) << 6) + uint32_t(D1[r])) << 6) + uint32_t(D0[r]));
+                    Y[b][t] = activate4(Dh, Sc, c143);
+                }
+            } else {
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    v4i const Dh = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
+                    Y[b][t] = activate4(Dh, Sc, c143);
+                }
             }
         }
 #pragma unroll
@@ -580,7 +630,7 @@ __device__ __forceinline__ void mlp_forward(Lds& lds, int wave, int lane, uint32
     }
 
     // output layer
-    uint4 const wa = *reinterpret_cast<uint4 const*>(&lds.w[tb][lane][0]);
+    uint4 const wa = *reinterpret_cast<uint4 const*>(&lds.w[0][tb][lane][0]);
     v4i const A = v4i{ int(wa.x), int(wa.y), int(wa.z), int(wa.w) };
     v4i const C = *reinterpret_cast<v4i const*>(&lds.bias[tb][g][0]);
     S = *reinterpret_cast<v4f const*>(&lds.scale[tb][g][0]);
@@ -592,7 +642,7 @@ template <class V>
 __global__ void __launch_bounds__(256, 2)
 decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
 {
-    __shared__ Lds lds;
+    __shared__ LdsT<V> lds;
     int const lane = threadIdx.x & 63;
     int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int const j = lane & 15, g = lane >> 4;
@@ -623,7 +673,7 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
         if (m.weights != stagedBlob || entry != stagedEntry) {   // uniform across the workgroup
             __syncthreads();
             if (m.weights != stagedBlob) stage_weights<V>(lds, m.weights);
-            if (m.fast) build_posenc_tables(lds, m.positionScale);
+            if (m.fast) build_posenc_tables<V>(lds, m.positionScale);
             stagedBlob = m.weights;
             stagedEntry = entry;
             __syncthreads();
@@ -664,7 +714,7 @@ __global__ void __launch_bounds__(256, 2)
 query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __restrict__ queries, uint64_t numQueries,
              uint16_t* __restrict__ out)
 {
-    __shared__ Lds lds;
+    __shared__ LdsT<V> lds;
     int const lane = threadIdx.x & 63;
     int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int const j = lane & 15, g = lane >> 4;
@@ -738,6 +788,7 @@ using VRef16  = Variant<0, 16, 4, 16, 16, 16, 2, 48, 64, 48, 32>; // LibNTC 0.9.
 using VRef12  = Variant<0, 12, 4, 16, 12, 16, 2, 48, 64, 48, 32>;
 using VRef8   = Variant<0, 8, 4, 16, 8, 16, 2, 48, 64, 48, 32>;
 using VRef4   = Variant<0, 4, 4, 16, 4, 16, 2, 48, 64, 48, 32>;
+using VCfg3   = Variant<0, 16, 4, 16, 16, 16, 2, 48, 64, 64, 64, true>;   // wide decoder, e4m3 hidden-layer weights
 
 template <class V>
 static hipError_t launch_variant(DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream)
@@ -755,6 +806,7 @@ hipError_t launch_decode(int variant, DevMip const* mips, int numMips, int total
     case NTC_HIP_VARIANT_REF12: return launch_variant<VRef12>(mips, numMips, totalTiles, gridSize, stream);
     case NTC_HIP_VARIANT_REF8:  return launch_variant<VRef8>(mips, numMips, totalTiles, gridSize, stream);
     case NTC_HIP_VARIANT_REF4:  return launch_variant<VRef4>(mips, numMips, totalTiles, gridSize, stream);
+    case NTC_HIP_VARIANT_CFG3_FP8: return launch_variant<VCfg3>(mips, numMips, totalTiles, gridSize, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -777,6 +829,7 @@ hipError_t launch_queries(int variant, DevMip const* mips, int numMips, DevQuery
     case NTC_HIP_VARIANT_REF12: return launch_query_variant<VRef12>(mips, numMips, queries, numQueries, out, gridSize, stream);
     case NTC_HIP_VARIANT_REF8:  return launch_query_variant<VRef8>(mips, numMips, queries, numQueries, out, gridSize, stream);
     case NTC_HIP_VARIANT_REF4:  return launch_query_variant<VRef4>(mips, numMips, queries, numQueries, out, gridSize, stream);
+    case NTC_HIP_VARIANT_CFG3_FP8: return launch_query_variant<VCfg3>(mips, numMips, queries, numQueries, out, gridSize, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -799,6 +852,7 @@ int resident_workgroups_per_cu(int variant)
     case NTC_HIP_VARIANT_REF12: return occupancy_variant<VRef12>();
     case NTC_HIP_VARIANT_REF8:  return occupancy_variant<VRef8>();
     case NTC_HIP_VARIANT_REF4:  return occupancy_variant<VRef4>();
+    case NTC_HIP_VARIANT_CFG3_FP8: return occupancy_variant<VCfg3>();
     default: return 2;
     }
 }

@@ -70,15 +70,22 @@ bool spec_sane(NtcHipDecoderSpec const& s)
     for (int l = 0; l < NTC_HIP_MLP_LAYERS - 1; ++l) if (!widthOk(s.hiddenChannels[l])) return false;
     if ((s.hrBits != 2 && s.hrBits != 4) || (s.lrBits != 2 && s.lrBits != 4)) return false;
     if (s.hrFeatures < 1 || s.lrFeatures < 1 || s.hrFeatures > s.hrFeatureSlots || s.lrFeatures > s.lrFeatureSlots) return false;
-    if (s.weightType != NTC_HIP_WEIGHTS_INT8 && s.weightType != NTC_HIP_WEIGHTS_FP8) return false;
+    if (s.weightType < NTC_HIP_WEIGHTS_INT8 || s.weightType > NTC_HIP_WEIGHTS_FP8_SCALED) return false;
     return true;
 }
 
 // Which compiled kernel covers this spec.
 int pick_variant(NtcHipDecoderSpec const& s)
 {
-    if (s.weightType != NTC_HIP_WEIGHTS_INT8 || s.posEncWaves != 3 || s.outputChannels != 16) return NTC_HIP_VARIANT_NONE;
+    if (s.posEncWaves != 3 || s.outputChannels != 16) return NTC_HIP_VARIANT_NONE;
     if (s.lrMode != NTC_HIP_GRID_BILINEAR || s.lrBits != 4) return NTC_HIP_VARIANT_NONE;
+    if (s.weightType == NTC_HIP_WEIGHTS_FP8_SCALED) {
+        bool const wide = s.hrMode == NTC_HIP_GRID_BILINEAR && s.hrBits == 4 && s.hrFeatures == 16 && s.hrFeatureSlots == 16
+            && s.lrFeatures == 16 && s.lrFeatureSlots == 16 && s.lodInputs == 2 && s.inputChannels == 48
+            && s.hiddenChannels[0] == 64 && s.hiddenChannels[1] == 64 && s.hiddenChannels[2] == 64;
+        return wide ? NTC_HIP_VARIANT_CFG3_FP8 : NTC_HIP_VARIANT_NONE;
+    }
+    if (s.weightType != NTC_HIP_WEIGHTS_INT8) return NTC_HIP_VARIANT_NONE;
     bool const concat8x2 = s.hrMode == NTC_HIP_GRID_CONCAT2X2 && s.hrFeatures == 8 && s.hrBits == 2 && s.hrFeatureSlots == 8;
     if (concat8x2 && s.lodInputs == 0 && s.inputChannels == 64 && s.hiddenChannels[2] == 32) {
         if (s.lrFeatures == 16 && s.lrFeatureSlots == 16 && s.hiddenChannels[0] == 64 && s.hiddenChannels[1] == 48)
@@ -406,7 +413,7 @@ int ntc_hip_weight_layout(const NtcHipDecoderSpec* spec, NtcHipWeightLayout* out
         out->weightOffset[l] = cursor;
         cursor += uint32_t(layer_in(*spec, l)) * uint32_t(layer_out(*spec, l));
     }
-    if (spec->weightType == NTC_HIP_WEIGHTS_INT8) {
+    if (spec->weightType == NTC_HIP_WEIGHTS_INT8 || spec->weightType == NTC_HIP_WEIGHTS_FP8_SCALED) {
         // then every scale vector, then every bias vector (src/WeightLayout.cpp:229-247)
         for (int l = 0; l < NTC_HIP_MLP_LAYERS; ++l) { out->scaleOffset[l] = cursor; cursor += 4u * uint32_t(layer_out(*spec, l)); }
         for (int l = 0; l < NTC_HIP_MLP_LAYERS; ++l) { out->biasOffset[l] = cursor; cursor += 4u * uint32_t(layer_out(*spec, l)); }

@@ -5,6 +5,7 @@ ref092  : the geometry compiled into the mounted LibNTC 0.9.2
 cfg01   : 2x2-concat high-res grid of 8 x 2-bit features + bilinear low-res grid of
           16 x 4-bit features + 12 positional inputs = 60 -> 64, MLP 64-48-32, 16 outputs.
 cfg2    : same high-res grid, 12 low-res features (56 -> 64 inputs), MLP 48-48-32.
+cfg3    : both grids bilinear 16 x 4-bit, MLP 64-64-64, hidden-layer weights stored as FP8 e4m3.
 """
 import math
 
@@ -37,6 +38,12 @@ def spec_cfg01():
 
 def spec_cfg2():
     return make_spec((8, 2, abi.GRID_CONCAT2X2, 8), (12, 4, abi.GRID_BILINEAR, 12), 0, 64, (48, 48, 32))
+
+
+def spec_cfg3():
+    """Wide decoder with e4m3 hidden-layer weights: both grids bilinear 16 x 4-bit, (lod, lod), 48 -> 64-64-64 -> 16."""
+    return make_spec((16, 4, abi.GRID_BILINEAR, 16), (16, 4, abi.GRID_BILINEAR, 16), 2, 48, (64, 64, 64),
+                     abi.WEIGHTS_FP8_SCALED)
 
 
 def grid_bytes(width, height, features, bits):

@@ -25,14 +25,22 @@ def weight_layout(spec):
 
 def make_weights(spec, seed, scale_log2_range=(-10.0, -4.0), bias_sigma=0.1, layout=None):
     """Returns the int8 weight blob (uint8 array) for `spec`."""
-    assert spec.weightType == abi.WEIGHTS_INT8
+    assert spec.weightType in (abi.WEIGHTS_INT8, abi.WEIGHTS_FP8_SCALED)
+    fp8 = spec.weightType == abi.WEIGHTS_FP8_SCALED
     layout = layout or weight_layout(spec)
     rng = np.random.default_rng(seed)
     blob = np.zeros(layout.bufferSize, dtype=np.uint8)
     for layer in range(abi.MLP_LAYERS):
         n_in, n_out = spec.layer_inputs(layer), spec.layer_outputs(layer)
-        w = rng.integers(-127, 128, size=(n_out, n_in), dtype=np.int8)
-        scale = np.exp2(rng.uniform(scale_log2_range[0], scale_log2_range[1], size=n_out)).astype(np.float32)
+        if fp8 and layer < abi.MLP_LAYERS - 1:
+            # uniform over the 254 finite e4m3 bit patterns; the blob's scale is per unit of w/512
+            w = rng.integers(0, 254, size=(n_out, n_in)).astype(np.uint8)
+            w = (w + (w >= 127)).astype(np.uint8).view(np.int8)       # skip 0x7f; 0xff is never reached
+            unit = np.float32(1.0 / 512.0)
+        else:
+            w = rng.integers(-127, 128, size=(n_out, n_in), dtype=np.int8)
+            unit = np.float32(1.0)
+        scale = np.exp2(rng.uniform(scale_log2_range[0], scale_log2_range[1], size=n_out)).astype(np.float32) * unit
         bias = rng.normal(0.0, bias_sigma, size=n_out).astype(np.float32)
         q = (bias / scale).astype(np.float32).astype(np.float64)
         bias_i32 = np.trunc(q + np.copysign(0.5, q)).astype(np.int32)      # roundf

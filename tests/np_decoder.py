@@ -122,6 +122,18 @@ def hgelu_quantize(x):
     return (r.astype(np.int32) - 113).astype(np.int8)
 
 
+def e4m3_times_512(byte_array):
+    """OCP e4m3 bytes -> the exact integers 512*value, from the format definition:
+    (-1)^s * 2^(e-7) * (1 + m/8) for e > 0, (-1)^s * 2^-6 * (m/8) for e = 0; NaN patterns -> 0."""
+    b = np.asarray(byte_array).view(np.uint8).astype(np.int64)
+    sgn, e, m = b >> 7, (b >> 3) & 15, b & 7
+    val = np.where(e > 0, np.ldexp(1.0 + m / 8.0, e - 7), np.ldexp(m / 8.0, -6)) * 512.0
+    out = np.where(sgn == 1, -val, val)
+    out = np.where((b & 0x7F) == 0x7F, 0.0, out)
+    assert np.array_equal(out, np.rint(out))
+    return out.astype(np.int64)
+
+
 def decode_mip(spec, layout, blob, latents_u16, mip):
     """Returns (inputs int8 [H,W,IN], outputs float32 [H,W,16]) for one colour mip."""
     W, H = mip.width, mip.height
@@ -142,6 +154,8 @@ def decode_mip(spec, layout, blob, latents_u16, mip):
     for layer in range(4):
         n_in, n_out = spec.layer_inputs(layer), spec.layer_outputs(layer)
         w = blob[layout.weightOffset[layer]: layout.weightOffset[layer] + n_in * n_out].view(np.int8).reshape(n_out, n_in)
+        if spec.weightType == 2 and layer < 3:
+            w = e4m3_times_512(w)
         scale = blob[layout.scaleOffset[layer]: layout.scaleOffset[layer] + 4 * n_out].view(np.float32)
         bias = blob[layout.biasOffset[layer]: layout.biasOffset[layer] + 4 * n_out].view(np.int32)
         acc = act @ w.astype(np.int64).T + bias.astype(np.int64)             # Inference.hlsli:148-162

@@ -35,6 +35,8 @@ def load_oracle():
         lib.ntc_oracle_hgelu_quantize.argtypes = [C.c_float]
         lib.ntc_oracle_unpack_field.restype = C.c_int
         lib.ntc_oracle_unpack_field.argtypes = [C.c_uint16, C.c_int, C.c_int]
+        lib.ntc_oracle_e4m3_times_512.restype = C.c_int32
+        lib.ntc_oracle_e4m3_times_512.argtypes = [C.c_uint8]
         lib.ntc_oracle_quantize_value.restype = C.c_uint32
         lib.ntc_oracle_quantize_value.argtypes = [C.c_float, C.c_int]
         lib.ntc_oracle_encode_position.restype = None

@@ -94,6 +94,35 @@ def test_cfg2_batch_of_sets(ntc, device):
         assert_equal_bytes(hset.output, c.d_output.download(), f"cfg2 set {i}")
 
 
+@pytest.mark.parametrize("w,h,mips,fmt", [(256, 256, 1, "planar"), (128, 64, 8, "unorm8"), (90, 70, 4, "fp16px")])
+def test_cfg3_fp8_weights(ntc, device, w, h, mips, fmt):
+    """Config 3's shape: wide 64-64-64 decoder whose hidden-layer weights are FP8 e4m3 with a per-channel
+    fp32 scale.  The device evaluates the e4m3 dot products exactly (three 6-bit integer planes on the
+    int8 MFMA), so the comparison is byte equality - inside the 1e-3 / 1 LSB bound with room to spare."""
+    f = {"planar": ntc.abi.OUT_FP16_PLANAR_PAIRS, "fp16px": ntc.abi.OUT_FP16_PIXELS, "unorm8": ntc.abi.OUT_UNORM8_PIXELS}[fmt]
+    for scales in ((-17.0, -13.0), (-10.0, -4.0)):
+        case = cfg_case(ntc, ntc.presets.spec_cfg3(), w, h, mips, 16, f, seed=w + mips, scale_log2_range=scales)
+        expected, got = run_both(device, case)
+        assert_equal_bytes(expected, got, f"cfg3 fp8 {w}x{h} {fmt} {scales}")
+        if fmt == "planar":
+            a, b = expected.view(np.float16).astype(np.float32), got.view(np.float16).astype(np.float32)
+            assert np.max(np.abs(a - b)) <= 1e-3              # the bound the FP8 variant is specified to
+
+
+def test_cfg3_fp8_extreme_weights(ntc, device):
+    """Every hidden weight at +-448 (the largest e4m3) and the e4m3 subnormals, inputs saturating: int32
+    accumulators near their limits on both sides must match the checker's wrapped arithmetic."""
+    spec = ntc.presets.spec_cfg3()
+    layout = ntc.synth.weight_layout(spec)
+    blob = ntc.synth.make_weights(spec, 3, scale_log2_range=(-20.0, -18.0))
+    w = blob[:layout.weightOffset[3]]
+    pattern = np.array([0x7E, 0xFE, 0x01, 0x81, 0x7E, 0x7E, 0x08, 0xF7], dtype=np.uint8)
+    w[:] = np.resize(pattern, w.size)
+    case = cfg_case(ntc, spec, 64, 64, 1, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=19, weights=blob)
+    expected, got = run_both(device, case)
+    assert_equal_bytes(expected, got, "cfg3 fp8 extreme")
+
+
 def test_extreme_weights_saturate_cleanly(ntc, device):
     """All-(-127)/127 weights with the largest scale and huge biases: accumulators near their
     extremes, activations pinned at both ends of the quantiser."""

@@ -344,11 +344,28 @@ def _np_decode_case(ntc, case):
     return inputs, out
 
 
-@pytest.mark.parametrize("name", ["cfg01_planar", "cfg01_fp16px", "cfg01_unorm8", "cfg2_unorm8", "ref16_gs2", "ref8_gs4",
+def test_e4m3_decode_exhaustive(oracle):
+    all_bytes = np.arange(256, dtype=np.uint8)
+    got = np.array([oracle.ntc_oracle_e4m3_times_512(int(b)) for b in all_bytes], dtype=np.int64)
+    assert np.array_equal(got, np_decoder.e4m3_times_512(all_bytes))
+    # known values of the OCP e4m3 grid: 1.0, largest finite 448, smallest subnormal 2^-9, smallest normal 2^-6
+    assert got[0x38] == 512 and got[0x7E] == 448 * 512 and got[0x01] == 1 and got[0x08] == 8
+    assert got[0xB8] == -512 and got[0x7F] == 0 and got[0xFF] == 0 and got[0x00] == 0 and got[0x80] == 0
+    finite = np.delete(got, [0x7F, 0xFF])
+    assert np.unique(finite).size == 253                      # 254 finite patterns, +0 and -0 coincide
+    assert np.all(np.diff(got[:0x7F]) > 0)                    # positive half is strictly increasing
+    # three 6-bit planes reassemble every weight exactly (what the device stages into LDS)
+    c0, c1, c2 = got & 63, (got >> 6) & 63, got >> 12
+    assert np.array_equal(4096 * c2 + 64 * c1 + c0, got) and c2.min() >= -64 and c2.max() <= 63
+
+
+@pytest.mark.parametrize("name", ["cfg3_fp8_planar", "cfg3_fp8_ragged_unorm8", "cfg01_planar", "cfg01_fp16px", "cfg01_unorm8", "cfg2_unorm8", "ref16_gs2", "ref8_gs4",
                                   "ref12_gs3_ragged", "cfg01_ragged", "cfg01_default_scales"])
 def test_oracle_against_numpy_decoder(ntc, oracle, name):
     A = ntc.abi
     make = {
+        "cfg3_fp8_planar": lambda: cfg_case(ntc, ntc.presets.spec_cfg3(), 64, 64, 7, 16, A.OUT_FP16_PLANAR_PAIRS, 9, scale_log2_range=(-17.0, -13.0)),
+        "cfg3_fp8_ragged_unorm8": lambda: cfg_case(ntc, ntc.presets.spec_cfg3(), 50, 30, 3, 11, A.OUT_UNORM8_PIXELS, 10, scale_log2_range=(-17.0, -13.0)),
         "cfg01_planar": lambda: cfg_case(ntc, ntc.presets.spec_cfg01(), 64, 64, 7, 16, A.OUT_FP16_PLANAR_PAIRS, 1, scale_log2_range=ACTIVE),
         "cfg01_fp16px": lambda: cfg_case(ntc, ntc.presets.spec_cfg01(), 64, 32, 7, 9, A.OUT_FP16_PIXELS, 2, scale_log2_range=ACTIVE),
         "cfg01_unorm8": lambda: cfg_case(ntc, ntc.presets.spec_cfg01(), 32, 64, 7, 16, A.OUT_UNORM8_PIXELS, 3, scale_log2_range=ACTIVE),

@@ -50,11 +50,13 @@ def test_checker_queries_against_numpy_decoder(ntc, oracle):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("kind,n", [("cfg01", 5000), ("cfg01", 1), ("cfg01", 256), ("ref8", 3001), ("cfg2", 777)])
+@pytest.mark.parametrize("kind,n", [("cfg01", 5000), ("cfg01", 1), ("cfg01", 256), ("ref8", 3001), ("cfg2", 777), ("cfg3", 2049)])
 def test_gpu_queries_match_checker(ntc, device, oracle, kind, n):
     A = ntc.abi
     if kind == "cfg01":
         case = cfg_case(ntc, ntc.presets.spec_cfg01(), 512, 256, 10, 16, A.OUT_FP16_PLANAR_PAIRS, 41, scale_log2_range=ACTIVE)
+    elif kind == "cfg3":
+        case = cfg_case(ntc, ntc.presets.spec_cfg3(), 256, 256, 9, 16, A.OUT_FP16_PLANAR_PAIRS, 44, scale_log2_range=(-17.0, -13.0))
     elif kind == "cfg2":
         case = cfg_case(ntc, ntc.presets.spec_cfg2(), 200, 120, 8, 12, A.OUT_FP16_PLANAR_PAIRS, 42, scale_log2_range=ACTIVE)
     else:
