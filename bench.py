@@ -1,14 +1,18 @@
 #!/usr/bin/env python3
-"""Headline benchmark: decode a 4096x4096, 16-channel texture set with its full 13-level mip
-chain (22 369 621 texels; 2x2-concat 8x2-bit high-res grid + bilinear 16x4-bit low-res grid,
-MLP 64-48-32 int8, fp16 output) on one MI355X, bit-exact arithmetic, one launch per step.
+"""Benchmark of the texture-set decode path on one MI355X.
 
-Prints ONE JSON line.  A step = one full decode of the set; inputs (latents, weights) are
-resident in HBM before the timed region.  `roofline` is for the decode kernel (the only
-kernel of the path), timed with HIP events on the library's own stream; `cpu_baseline` is the
-CPU checker on a bounded sample of the same workload, on this machine's host cores.
+Default (the headline, BASELINE config 1): decode a 4096x4096, 16-channel texture set with its
+full 13-level mip chain (22 369 621 texels; 2x2-concat 8x2-bit high-res grid + bilinear 16x4-bit
+low-res grid, MLP 64-48-32 int8, fp16 output), bit-exact arithmetic, ONE launch per step.
+
+Prints ONE JSON line.  A step = one full decode of the workload; inputs (latents, weights,
+queries) are resident in HBM before the timed region.  `roofline` is for the decode kernel (the
+only kernel of the path), timed with HIP events on the library's own launch stream;
+`cpu_baseline` is the CPU checker on the same workload (or a bounded sample of it) on this
+machine's host cores.  Other --workload values measure the other BASELINE configurations.
 """
 import argparse
+import ctypes as C
 import importlib
 import json
 import os
@@ -23,14 +27,19 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0        # MI355X dense int8 MFMA
 
 
+def macs(widths):
+    return sum(a * b for a, b in zip(widths[:-1], widths[1:]))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--size", type=int, default=4096)
-    ap.add_argument("--format", choices=["fp16", "unorm8"], default="fp16")
-    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU-baseline sample time")
+    ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4", "ref092"])
+    ap.add_argument("--size", type=int, default=0, help="override the texture size of the workload")
+    ap.add_argument("--format", choices=["fp16", "unorm8"], default=None)
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="time budget of the CPU-baseline sample")
     ap.add_argument("--no-cpu", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -39,33 +48,87 @@ def main():
         sys.exit(2)
 
     ntc = importlib.import_module("rtxntc-library_amd")
-    from cases import cfg_case
+    from cases import cfg_case, ref_case
+    A, P = ntc.abi, ntc.presets
 
     dev = ntc.Device(0)
-    size = args.size
-    spec = ntc.presets.spec_cfg01()
-    num_mips = ntc.presets.full_mip_count(size, size)
-    fmt = ntc.abi.OUT_FP16_PLANAR_PAIRS if args.format == "fp16" else ntc.abi.OUT_UNORM8_PIXELS
-    case = cfg_case(ntc, spec, size, size, num_mips, 16, fmt, seed=0)
-    dset = case.device_set(dev)
-    texels = case.texels
-    out_bytes_per_texel = 32 if args.format == "fp16" else 16
-    # algorithmic HBM bytes per texel: output + latent bits amortised (HR 16 b per 4 texels, LR 64 b per 16)
-    bytes_per_texel = out_bytes_per_texel + (16 / 4 + 64 / 16) / 8.0
-    ops_per_texel = 2 * (64 * 64 + 64 * 48 + 48 * 32 + 32 * 16)
+    wl = args.workload
+    fmt_name = args.format or {"cfg2": "unorm8"}.get(wl, "fp16")
+    fmt = A.OUT_FP16_PLANAR_PAIRS if fmt_name == "fp16" else A.OUT_UNORM8_PIXELS
+    queries = None
+    if wl == "cfg0":
+        size = args.size or 512
+        cases = [cfg_case(ntc, P.spec_cfg01(), size, size, 1, 8, fmt, seed=0)]
+        widths, channels, latent_b = (64, 64, 48, 32, 16), 8, 1.0
+        what = f"cfg0 plumbing: {size}x{size}, 1 mip, 8 channels, MLP 64-64-48-32-16 int8"
+    elif wl == "cfg1":
+        size = args.size or 4096
+        cases = [cfg_case(ntc, P.spec_cfg01(), size, size, P.full_mip_count(size, size), 16, fmt, seed=0)]
+        widths, channels, latent_b = (64, 64, 48, 32, 16), 16, 1.0
+        what = (f"cfg1 headline: {size}x{size} set, {P.full_mip_count(size, size)} mips, 16 channels, "
+                "MLP 64-64-48-32-16 int8, HR 2x2x8 f@2b + LR 16 f@4b")
+    elif wl == "cfg2":
+        size = args.size or 2048
+        cases = [cfg_case(ntc, P.spec_cfg2(), size, size, P.full_mip_count(size, size), 12, fmt, seed=100 + i) for i in range(8)]
+        widths, channels, latent_b = (56, 48, 48, 32, 16), 12, 0.875
+        what = f"cfg2 batch: 8 sets of {size}x{size}, full mip chains, 12 channels, MLP 64(56)-48-48-32-16 int8, one launch"
+    elif wl == "cfg3":
+        size = args.size or 4096
+        cases = [cfg_case(ntc, P.spec_cfg3(), size, size, 1, 16, fmt, seed=3)]
+        widths, channels, latent_b = (46, 64, 64, 64, 16), 16, 2.5
+        what = f"cfg3 wide: {size}x{size}, 1 mip, 16 channels, MLP 48(46)-64-64-64-16, e4m3 hidden-layer weights, both grids bilinear 16 f@4b"
+    elif wl == "ref092":
+        size = args.size or 4096
+        cases = [ref_case(ntc, P.spec_ref092(16), size, size, P.full_mip_count(size, size), 2, 16, fmt, seed=5)]
+        widths, channels, latent_b = (46, 64, 48, 32, 16), 16, 44738560 / 22369621.0
+        what = f"LibNTC 0.9.2 geometry: {size}x{size}, full mip chain, grid scale 2, 16 features, MLP 48(46)-64-48-32-16 int8"
+    else:
+        size = args.size or 8192
+        cases = [cfg_case(ntc, P.spec_cfg01(), size, size, P.full_mip_count(size, size), 16, fmt, seed=4)]
+        widths, channels, latent_b = (64, 64, 48, 32, 16), 16, 0.0
+        import numpy as np
+        n = 1 << 24
+        rng = np.random.default_rng(4)
+        queries = np.zeros(n, dtype=[("u", np.float32), ("v", np.float32), ("mip", np.int32)])
+        queries["u"], queries["v"] = rng.random(n, dtype=np.float32), rng.random(n, dtype=np.float32)
+        queries["mip"] = rng.integers(0, len(cases[0].mips), n)
+        what = f"cfg4 random access: {size}x{size} set, {len(cases[0].mips)} mips, 2^24 (u,v,mip) queries, 16 x fp16 per query"
+        fmt_name = "fp16"
 
-    sets = dev.pack_sets([dset])
+    dsets = [c.device_set(dev) for c in cases]
+    sets = dev.pack_sets(dsets)
+    if queries is None:
+        texels = sum(c.texels for c in cases)
+        out_b = channels * (2 if fmt_name == "fp16" else 1)
+        bytes_per_texel = out_b + latent_b            # algorithmic HBM bytes: output + latent bits amortised
+        run = lambda: dev.decode(sets)
+        run_timed = lambda k: dev.decode_timed(sets, k)
+    else:
+        texels = queries.size
+        bytes_per_texel = 32 + 12 + 40                # output + the query + 4 HR cells x 2 B + 4 LR cells x 8 B
+        d_q = dev.upload(queries.view("u1"))
+        d_out = dev.alloc(queries.size * 32)
+
+        def run():
+            A.check(dev.lib.ntc_hip_decode_queries(sets, d_q.ptr, queries.size, d_out.ptr, d_out.nbytes))
+
+        def run_timed(k):
+            ms = C.c_float()
+            A.check(dev.lib.ntc_hip_decode_queries_timed(sets, d_q.ptr, queries.size, d_out.ptr, d_out.nbytes, k, C.byref(ms)))
+            return ms.value
+    ops_per_texel = 2 * macs(widths)
+
     for _ in range(args.warmup):
-        dev.decode(sets)
+        run()
     dev.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        dev.decode(sets)
+        run()
     dev.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall / args.steps * 1e3
 
-    kernel_ms = dev.decode_timed(sets, args.steps)      # HIP events on the launch stream
+    kernel_ms = run_timed(args.steps)                 # HIP events on the launch stream
     gtexels = texels / (ms_per_step * 1e-3) / 1e9
     achieved_gbs = texels * bytes_per_texel / (kernel_ms * 1e-3) / 1e9
     achieved_tops = texels * ops_per_texel / (kernel_ms * 1e-3) / 1e12
@@ -73,34 +136,50 @@ def main():
     cpu = None
     if not args.no_cpu:
         # The CPU checker (scalar C++ restatement, oracle/ntc_oracle.cpp) on this machine's host
-        # cores, over the WHOLE set when that fits the time budget, else over leading rows of mip 0.
+        # cores, over the whole workload when that fits the time budget, else over a leading part.
         cores = min(16, os.cpu_count() or 1)
-        host = case.host_set()
         from oracle_lib import load_oracle
         orc = load_oracle()
-        rows = min(256, size)
-        t = orc.ntc_oracle_decode_rows(host.desc, 0, 0, rows, cores)          # calibrate
-        est_full = t * texels / (rows * size)
-        if est_full <= args.cpu_seconds:
-            best = min(orc.ntc_oracle_decode(host.desc, cores) for _ in range(2))
-            cpu = {"value": texels / best / 1e9, "unit": "Gtexels/s", "cores": cores, "kind": "port",
-                   "sample": f"the whole set ({texels} texels), best of 2, {best:.2f} s"}
+        host = cases[0].host_set()
+        if queries is None:
+            mip0 = cases[0].mips[0]
+            rows = min(256, mip0.height)
+            t = orc.ntc_oracle_decode_rows(host.desc, 0, 0, rows, cores)          # calibrate
+            per_texel = t / (rows * mip0.width)
+            if per_texel * texels <= args.cpu_seconds:
+                hosts = [host] + [c.host_set() for c in cases[1:]]
+                best = None
+                for _ in range(2):
+                    total = sum(orc.ntc_oracle_decode(h.desc, cores) for h in hosts)
+                    best = total if best is None else min(best, total)
+                cpu = {"value": texels / best / 1e9, "unit": "Gtexels/s", "cores": cores, "kind": "port",
+                       "sample": f"the whole workload ({texels} texels), best of 2, {best:.2f} s"}
+            else:
+                rows = int(max(rows, min(mip0.height, args.cpu_seconds / (per_texel * mip0.width))))
+                t = orc.ntc_oracle_decode_rows(host.desc, 0, 0, rows, cores)
+                cpu = {"value": rows * mip0.width / t / 1e9, "unit": "Gtexels/s", "cores": cores, "kind": "port",
+                       "sample": f"rows 0..{rows} of mip 0 of the first set ({rows * mip0.width} texels), {t:.1f} s"}
         else:
-            rows = int(max(rows, min(size, args.cpu_seconds * rows / t)))
-            t = orc.ntc_oracle_decode_rows(host.desc, 0, 0, rows, cores)
-            cpu = {"value": rows * size / t / 1e9, "unit": "Gtexels/s", "cores": cores, "kind": "port",
-                   "sample": f"rows 0..{rows} of mip 0 ({rows * size} texels) of the same set, {t:.1f} s"}
+            import numpy as np
+            n = min(queries.size, 1 << 21)
+            out = np.zeros((n, 16), dtype=np.uint16)
+            t0 = time.perf_counter()
+            orc.ntc_oracle_decode_queries(host.desc, queries.ctypes.data, n, out.ctypes.data, cores)
+            t = time.perf_counter() - t0
+            cpu = {"value": n / t / 1e9, "unit": "Gtexels/s", "cores": cores, "kind": "port",
+                   "sample": f"the first {n} queries of the same list, {t:.1f} s"}
 
     line = {
         "metric": "decoded Gtexels/s, 4096^2 16-ch set, 64-48-32 int8; % of int8-MFMA/HBM roof",
         "value": gtexels, "unit": "Gtexels/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8", "data": "synthetic",
-        "config": {"workload": f"cfg1 headline: {size}x{size} set, {num_mips} mips, 16 channels, MLP 64-64-48-32-16 int8, "
-                               f"HR 2x2x8 f@2b + LR 16 f@4b, {args.format} output, {texels} texels per step",
+        "config": {"workload": f"{what}, {fmt_name} output, {texels} texels per step",
                    "device": dev.name, "compute_units": dev.compute_units},
         "roofline": {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved_gbs / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved_gbs / HBM_PEAK_GBS,
+                     # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE (profiles/), headline workload only
+                     "traffic": 764.4e6 if (wl == "cfg1" and fmt_name == "fp16" and not args.size) else None,
                      "kernel_ms": kernel_ms, "bytes_per_texel": bytes_per_texel,
                      "mfma_achieved_tops": achieved_tops, "mfma_frac": achieved_tops / INT8_PEAK_TOPS},
         "cpu_baseline": cpu,

@@ -308,12 +308,12 @@ int32_t e4m3_times_512(uint8_t byte)
 // A hidden layer with e4m3 weights: the dot product of an fp32-accumulating implementation,
 // taken without accumulation noise - the exact sum of (512 w)*x in int32 (wrapping like the
 // device's accumulators), converted to float once, times the per-channel scale.
-void layer_fp8_weights(uint8_t const* W, float const* scale, int32_t const* bias,
+void layer_fp8_weights(int32_t const* W512 /* 512*w, decoded once per set */, float const* scale, int32_t const* bias,
                        int in, int out, int8_t const* x, float* r)
 {
     for (int c = 0; c < out; ++c) {
         int64_t acc = bias[c];
-        for (int k = 0; k < in; ++k) acc += int64_t(x[k]) * int64_t(e4m3_times_512(W[c * in + k]));
+        for (int k = 0; k < in; ++k) acc += int64_t(x[k]) * int64_t(W512[c * in + k]);
         r[c] = float(int32_t(uint32_t(uint64_t(acc)))) * scale[c];
     }
 }
@@ -321,6 +321,14 @@ void layer_fp8_weights(uint8_t const* W, float const* scale, int32_t const* bias
 struct SetView {
     NtcHipTextureSet const* set;
     NtcHipWeightLayout layout;
+    std::vector<int32_t> fp8Weights;       // 512*w of every e4m3 weight, blob order (hidden layers)
+    void prepare()
+    {
+        if (set->spec.weightType != NTC_HIP_WEIGHTS_FP8_SCALED) return;
+        uint8_t const* blob = static_cast<uint8_t const*>(set->weights);
+        fp8Weights.resize(layout.weightOffset[NTC_HIP_MLP_LAYERS - 1]);
+        for (size_t i = 0; i < fp8Weights.size(); ++i) fp8Weights[i] = e4m3_times_512(blob[i]);
+    }
 };
 
 void prepare_inputs(NtcHipTextureSet const& set, NtcHipMipDesc const& mip, int x, int y, int8_t* in)
@@ -359,7 +367,7 @@ void decode_texel_int8(SetView const& sv, NtcHipMipDesc const& mip, int x, int y
     for (int l = 0; l < NTC_HIP_MLP_LAYERS; ++l) {
         int const in = layer_inputs(s, l), out = layer_outputs(s, l);
         if (s.weightType == NTC_HIP_WEIGHTS_FP8_SCALED && l < NTC_HIP_MLP_LAYERS - 1)
-            layer_fp8_weights(blob + sv.layout.weightOffset[l],
+            layer_fp8_weights(sv.fp8Weights.data() + sv.layout.weightOffset[l],
                               reinterpret_cast<float const*>(blob + sv.layout.scaleOffset[l]),
                               reinterpret_cast<int32_t const*>(blob + sv.layout.biasOffset[l]),
                               in, out, act, r);
@@ -448,8 +456,9 @@ void ntc_oracle_bilinear_footprint(float u, float v, int gw, int gh, int* xy, fl
 // Inputs (int8, spec.inputChannels of them) and raw fp32 outputs of one texel.
 int ntc_oracle_decode_texel(const NtcHipTextureSet* set, int mip, int x, int y, float* outputs, int8_t* inputs)
 {
-    SetView sv{ set, {} };
+    SetView sv{ set, {}, {} };
     if (!decodable(set->spec) || !weight_layout(set->spec, sv.layout)) return -1;
+    sv.prepare();
     decode_texel_int8(sv, set->mips[mip], x, y, outputs, inputs);
     return 0;
 }
@@ -547,8 +556,9 @@ int ntc_oracle_read_channels(const uint16_t* planarPairs, int width, int height,
 int ntc_oracle_decode_queries(const NtcHipTextureSet* set, const float* uvmip /* 3 words per query: u, v, int32 mip */,
                               uint64_t numQueries, uint16_t* out, int threads)
 {
-    SetView sv{ set, {} };
+    SetView sv{ set, {}, {} };
     if (!decodable(set->spec) || !weight_layout(set->spec, sv.layout)) return -1;
+    sv.prepare();
     if (threads < 1) threads = 1;
     std::atomic<uint64_t> next{0};
     auto work = [&]() {
@@ -579,8 +589,9 @@ int ntc_oracle_decode_queries(const NtcHipTextureSet* set, const float* uvmip /*
 // out in bands to `threads` workers.  Returns seconds spent decoding (steady clock), < 0 on error.
 double ntc_oracle_decode(const NtcHipTextureSet* set, int threads)
 {
-    SetView sv{ set, {} };
+    SetView sv{ set, {}, {} };
     if (!decodable(set->spec) || !weight_layout(set->spec, sv.layout)) return -1.0;
+    sv.prepare();
     if (threads < 1) threads = 1;
     auto const t0 = std::chrono::steady_clock::now();
     for (int m = 0; m < set->numMips; ++m) {
@@ -614,8 +625,9 @@ double ntc_oracle_decode(const NtcHipTextureSet* set, int threads)
 // Decodes only rows [y0, y1) of mip `mipIndex` (bounded CPU-baseline samples).
 double ntc_oracle_decode_rows(const NtcHipTextureSet* set, int mipIndex, int y0, int y1, int threads)
 {
-    SetView sv{ set, {} };
+    SetView sv{ set, {}, {} };
     if (!decodable(set->spec) || !weight_layout(set->spec, sv.layout)) return -1.0;
+    sv.prepare();
     NtcHipMipDesc const& mip = set->mips[mipIndex];
     y0 = std::max(0, y0); y1 = std::min(mip.height, y1);
     if (threads < 1) threads = 1;

@@ -1,0 +1,113 @@
+"""BASELINE.json's full-size configurations on the GPU: complete comparison with the CPU checker
+where that takes seconds, and size-independent properties (periodicity under periodic latents,
+batch = individual, queries = raster) where the checker would be too slow to cover everything."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from cases import Case, cfg_case, first_mismatch
+
+pytestmark = pytest.mark.gpu
+
+
+def test_headline_4096_full_mip_chain_equals_checker(ntc, device):
+    """Config 1 at full size, fp16 planar output: all 22 369 621 texels, every byte."""
+    case = cfg_case(ntc, ntc.presets.spec_cfg01(), 4096, 4096, 13, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=0)
+    assert case.texels == 22369621
+    host = case.host_set()
+    host.decode(threads=16)
+    dset = case.device_set(device)
+    device.decode([dset])
+    device.synchronize()
+    mm = first_mismatch(host.output, case.d_output.download())
+    assert mm is None, f"{mm[1]} bytes differ, first at {mm[0]}"
+
+
+def test_headline_4096_periodic_latents_give_periodic_output(ntc, device):
+    """Wrap addressing + periodic positional encoding: latents that repeat every P cells must decode
+    to an image that repeats every 2P (HR) = 4P' (LR) texels.  No checker involved; unorm8 output."""
+    spec = ntc.presets.spec_cfg01()
+    mips, latent_bytes = ntc.presets.mips_private_grids(spec, 4096, 4096, 1)
+    m = mips[0]
+    rng = np.random.default_rng(77)
+    period = 64                                                 # texels; HR cells repeat every 32, LR every 16
+    hr_tile = rng.integers(0, 65536, size=(period // 2, period // 2), dtype=np.uint16)
+    lr_tile = rng.integers(0, 65536, size=(4, period // 4, period // 4), dtype=np.uint16)
+    hr = np.tile(hr_tile, (m.hrHeight // (period // 2), m.hrWidth // (period // 2)))
+    lr = np.tile(lr_tile, (1, m.lrHeight // (period // 4), m.lrWidth // (period // 4)))
+    latents = np.concatenate([hr.reshape(-1), lr.reshape(-1)])
+    assert latents.nbytes == latent_bytes
+    case = Case(ntc, spec, mips, latent_bytes, 16, ntc.abi.OUT_UNORM8_PIXELS, seed=5, latents=latents,
+                scale_log2_range=(-17.0, -12.0))
+    dset = case.device_set(device)
+    device.decode([dset])
+    device.synchronize()
+    img = case.d_output.download().reshape(4096, 4096, 16)
+    ref = img[:period, :period]
+    assert ref.std() > 10                                       # a real image, not a constant
+    blocks = img.reshape(4096 // period, period, 4096 // period, period, 16)
+    assert np.array_equal(blocks, np.broadcast_to(ref[None, :, None, :, :], blocks.shape))
+
+
+def test_batch_of_eight_2048_sets_equals_individual_decodes(ntc, device, oracle):
+    """Config 2 at full size (8 x 2048^2, 12 channels, full mip chains, unorm8): one launch over the
+    batch gives the same bytes as eight separate launches; mips >= 2 of two sets also go to the checker."""
+    spec = ntc.presets.spec_cfg2()
+    cases = [cfg_case(ntc, spec, 2048, 2048, 12, 12, ntc.abi.OUT_UNORM8_PIXELS, seed=200 + i) for i in range(8)]
+    dsets = [c.device_set(device) for c in cases]
+    device.decode(dsets)
+    device.synchronize()
+    together = [c.d_output.download().copy() for c in cases]
+    for c, dset, want in zip(cases, dsets, together):
+        c.d_output.fill(0xCD)
+        device.decode([dset])
+        device.synchronize()
+        assert np.array_equal(c.d_output.download(), want)
+    for i in (0, 7):
+        host = cases[i].host_set()
+        for m in range(2, 12):                                  # 512^2 and smaller: quick on the CPU
+            assert oracle.ntc_oracle_decode_rows(host.desc, m, 0, cases[i].mips[m].height, 16) >= 0
+        start = cases[i].mips[2].outOffset
+        assert np.array_equal(host.output[start:], together[i][start:])
+
+
+def test_wide_fp8_4096_rows_equal_checker(ntc, device, oracle):
+    """Config 3 at full size (4096^2, one mip): bands of rows at the top, middle and bottom."""
+    case = cfg_case(ntc, ntc.presets.spec_cfg3(), 4096, 4096, 1, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=3)
+    dset = case.device_set(device)
+    device.decode([dset])
+    device.synchronize()
+    got = case.d_output.download()
+    host = case.host_set()
+    row_bytes = 4096 * 16 * 2
+    for y0 in (0, 2040, 4096 - 24):
+        oracle.ntc_oracle_decode_rows(host.desc, 0, y0, y0 + 24, 16)
+        assert np.array_equal(host.output[y0 * row_bytes:(y0 + 24) * row_bytes], got[y0 * row_bytes:(y0 + 24) * row_bytes]), y0
+
+
+def test_random_access_8192_queries(ntc, device, oracle):
+    """Config 4 at full size: 2^24 queries into an 8192^2, 14-mip set.  A 2^20 sample goes to the
+    checker; repeated queries must repeat their answers; mip 13 (1x1) answers are all one texel."""
+    case = cfg_case(ntc, ntc.presets.spec_cfg01(), 8192, 8192, 14, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=4)
+    n = 1 << 24
+    rng = np.random.default_rng(4)
+    q = np.zeros(n, dtype=[("u", np.float32), ("v", np.float32), ("mip", np.int32)])
+    q["u"], q["v"] = rng.random(n, dtype=np.float32), rng.random(n, dtype=np.float32)
+    q["mip"] = rng.integers(0, 14, n)
+    q[n // 2:] = q[: n // 2]                                    # second half repeats the first
+    d_lat, d_w = device.upload(case.latents), device.upload(case.weights)
+    dset = ntc.make_texture_set(case.spec, case.mips, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, d_lat.ptr, d_lat.nbytes,
+                                d_w.ptr, d_w.nbytes, None, 0)
+    d_q, d_out = device.upload(q.view(np.uint8)), device.alloc(n * 32)
+    ntc.abi.check(device.lib.ntc_hip_decode_queries(dset, d_q.ptr, n, d_out.ptr, d_out.nbytes))
+    device.synchronize()
+    got = d_out.download(np.uint16).reshape(n, 16)
+    assert np.array_equal(got[: n // 2], got[n // 2:])
+    last = got[q["mip"] == 13]
+    assert np.array_equal(last, np.broadcast_to(last[0], last.shape))
+    host = case.host_set()
+    sample = 1 << 20
+    want = np.zeros((sample, 16), dtype=np.uint16)
+    assert oracle.ntc_oracle_decode_queries(host.desc, q.ctypes.data, sample, want.ctypes.data, 16) == 0
+    assert np.array_equal(got[:sample], want)
