@@ -293,8 +293,10 @@ struct alignas(16) LdsT {
     int32_t  bias[V::NTILES][4][4];
     uint32_t in[kWaves][kWaveTexels][kInStride];
     uint32_t lut2[256];               // byte of four 2-bit codes -> four input bytes 85*q - 128
-    uint32_t xtab[64][4];             // positional encoding by x phase: dword w = enc(px*2^w) | enc(px*2^w+1/4) << 16
-    uint32_t ytab[64][4];             // same for y, one byte up
+    // Positional encoding for every power-of-two positionScale 2^-k, k = 0..6: the entry for phase p of
+    // scale 2^-k sits at index (2^k - 1) + p; dword w = enc(px*2^w) | enc(px*2^w + 1/4) << 16, px = p*2^-k.
+    uint32_t xtab[128][4];
+    uint32_t ytab[128][4];            // same for y, one byte up
 };
 
 // OCP e4m3 (1-4-3, bias 7, no infinities) byte -> the integer 512*value: subnormals m * 2^-9,
@@ -515,8 +517,8 @@ __device__ __forceinline__ void prepare_inputs_fast(DevMip const& m, LdsT<V> con
     }
     // ---- positional encoding from the per-mip phase tables
     {
-        uint4 const ex = *reinterpret_cast<uint4 const*>(&lds.xtab[uint32_t(x) & m.posMask][0]);
-        uint4 const ey = *reinterpret_cast<uint4 const*>(&lds.ytab[uint32_t(y) & m.posMask][0]);
+        uint4 const ex = *reinterpret_cast<uint4 const*>(&lds.xtab[m.posMask + (uint32_t(x) & m.posMask)][0]);
+        uint4 const ey = *reinterpret_cast<uint4 const*>(&lds.ytab[m.posMask + (uint32_t(y) & m.posMask)][0]);
         in[V::POS_BASE / 4 + 0] = ex.x | ey.x;
         in[V::POS_BASE / 4 + 1] = ex.y | ey.y;
         in[V::POS_BASE / 4 + 2] = ex.z | ey.z;
@@ -534,23 +536,25 @@ __device__ __forceinline__ uint32_t posenc_byte(float p)
     return uint32_t(int(e * 127.5f)) & 0xffu;
 }
 
-// Fills the phase tables for a mip whose positionScale is a power of two: the encoding of
-// texel x depends only on x mod (1/positionScale), and all arithmetic involved is exact.
+// Fills the phase tables.  For positionScale = 2^-k the encoding of texel x depends only on
+// x mod 2^k, and all arithmetic involved is exact, so table and per-lane evaluation agree; scales of
+// 1 and above have period 1 (k = 0).  One entry per thread, threads 0..126 fill both tables.
 template <class V>
-__device__ void build_posenc_tables(LdsT<V>& lds, float positionScale)
+__device__ void build_posenc_tables(LdsT<V>& lds)
 {
     int const t = threadIdx.x;
-    if (t < 128) {
-        int const phase = t & 63;
-        float p = float(phase) * positionScale;
+    if (t < 127) {
+        int const k = 31 - __builtin_clz(uint32_t(t + 1));   // floor(log2(t + 1))
+        int const phase = t + 1 - (1 << k);
+        float p = float(phase) * __builtin_ldexpf(1.f, -k);
         uint32_t e[3];
 #pragma unroll
         for (int w = 0; w < 3; ++w) {
             e[w] = posenc_byte(p) | (posenc_byte(p + 0.25f) << 16);
             p *= 2.f;
         }
-        if (t < 64) { lds.xtab[phase][0] = e[0];      lds.xtab[phase][1] = e[1];      lds.xtab[phase][2] = e[2];      lds.xtab[phase][3] = 0; }
-        else        { lds.ytab[phase][0] = e[0] << 8; lds.ytab[phase][1] = e[1] << 8; lds.ytab[phase][2] = e[2] << 8; lds.ytab[phase][3] = 0; }
+        lds.xtab[t][0] = e[0];      lds.xtab[t][1] = e[1];      lds.xtab[t][2] = e[2];      lds.xtab[t][3] = 0;
+        lds.ytab[t][0] = e[0] << 8; lds.ytab[t][1] = e[1] << 8; lds.ytab[t][2] = e[2] << 8; lds.ytab[t][3] = 0;
     }
 }
 
@@ -662,21 +666,20 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     uint32_t c143 = 143u;
     asm volatile("" : "+v"(c143));                           // stays in a VGPR: SDWA operands cannot be literals
 
+    build_posenc_tables<V>(lds);
+
     uint8_t const* stagedBlob = nullptr;
-    int stagedEntry = -1;
     int entry = 0;
 
     for (int tile = tileBegin; tile < tileEnd; ++tile) {
         while (entry + 1 < numMips && mips[entry + 1].tileStart <= tile) ++entry;
         DevMip const& m = mips[entry];
 
-        if (m.weights != stagedBlob || entry != stagedEntry) {   // uniform across the workgroup
+        if (m.weights != stagedBlob) {                       // uniform across the workgroup
             __syncthreads();
-            if (m.weights != stagedBlob) stage_weights<V>(lds, m.weights);
-            if (m.fast) build_posenc_tables<V>(lds, m.positionScale);
+            stage_weights<V>(lds, m.weights);
             stagedBlob = m.weights;
-            stagedEntry = entry;
-            __syncthreads();
+            __syncthreads();                                 // also publishes the tables built above
         }
 
         int const local = tile - m.tileStart;
@@ -707,7 +710,7 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
 // Random-access decode ("inference on sample", NtcSampleTextureSet of Inference.hlsli:282-357):
 // one query = (u, v, mip) -> the 16 outputs of texel (floor(u*W), floor(v*H)) of that mip, clamped to
 // the image, as 16 fp16.  Lane = query in the input stage (each lane carries its own mip, so the
-// general per-lane stage is used); the network is the same 64-column tile as in raster decode.
+// per-lane form of either input stage is used); the network is the same 64-column tile as in raster decode.
 // A query whose mip is out of range writes zeros.
 template <class V>
 __global__ void __launch_bounds__(256, 2)
@@ -722,6 +725,13 @@ query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __res
     uint32_t c143 = 143u;
     asm volatile("" : "+v"(c143));
 
+    {   // 2-bit code bytes -> input bytes (see decode_kernel)
+        uint32_t x = threadIdx.x & 0xffu;
+        x = (x | (x << 12)) & 0x000f000fu;
+        x = (x | (x << 6))  & 0x03030303u;
+        lds.lut2[threadIdx.x & 0xffu] = (x * 85u) ^ 0x80808080u;
+    }
+    build_posenc_tables<V>(lds);
     stage_weights<V>(lds, mips[0].weights);
     __syncthreads();
 
@@ -738,7 +748,8 @@ query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __res
         x = max(0, min(x, m.width - 1));
         y = max(0, min(y, m.height - 1));
         uint32_t in[16];
-        prepare_inputs_general<V>(m, x, y, in);
+        if (__all(m.fast != 0)) prepare_inputs_fast<V>(m, lds, x, y, in);     // every lane's mip is power-of-two sized
+        else                    prepare_inputs_general<V>(m, x, y, in);
 
         v4i D[4];
         v4f S;

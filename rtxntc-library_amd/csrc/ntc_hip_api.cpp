@@ -8,7 +8,6 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
-#include <cstdlib>
 #include <cstring>
 #include <vector>
 
@@ -43,9 +42,12 @@ struct Library {
     hipStream_t stream = nullptr;
     hipEvent_t evStart = nullptr, evStop = nullptr;
     DevMip* tableDev = nullptr;        // device copy of the mip table
-    DevMip* tableHost = nullptr;       // pinned staging
     size_t tableCapacity = 0;          // entries
-    std::vector<DevMip> lastTable;     // what tableDev currently holds
+    std::vector<DevMip> lastTable;     // what tableDev currently holds (or will, in stream order)
+    static constexpr int kSlots = 4;
+    struct Slot { DevMip* host = nullptr; size_t capacity = 0; hipEvent_t done = nullptr; bool inFlight = false; };
+    Slot slots[kSlots];                // pinned staging for asynchronous table uploads
+    int nextSlot = 0;
 };
 Library g_lib;
 
@@ -254,28 +256,38 @@ int build_table(NtcHipTextureSet const* sets, int32_t numSets, std::vector<DevMi
     return 0;
 }
 
-// Makes the device table hold `table` (re-uploads only when it changed).
+// Makes the device table hold `table` (re-uploads only when it changed).  The copy is asynchronous
+// from one of a few pinned staging slots; a slot is reused only after the copy that last read it
+// has completed (its event), so back-to-back launches with different tables never wait on the GPU.
 int upload_table(std::vector<DevMip> const& table)
 {
     Library& L = g_lib;
-    if (table.size() > L.tableCapacity) {
-        size_t const cap = table.size() * 2 + 16;
-        if (L.tableDev)  { HIP_TRY(hipStreamSynchronize(L.stream)); HIP_TRY(hipFree(L.tableDev)); L.tableDev = nullptr; }
-        if (L.tableHost) { HIP_TRY(hipHostFree(L.tableHost)); L.tableHost = nullptr; }
-        L.tableCapacity = 0; L.lastTable.clear();
-        HIP_TRY(hipMalloc(reinterpret_cast<void**>(&L.tableDev), cap * sizeof(DevMip)));
-        HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&L.tableHost), cap * sizeof(DevMip), hipHostMallocDefault));
-        L.tableCapacity = cap;
-    }
     bool const same = L.lastTable.size() == table.size()
         && std::memcmp(L.lastTable.data(), table.data(), table.size() * sizeof(DevMip)) == 0;
-    if (!same) {
-        // The pinned staging copy may still be in flight for an earlier launch.
+    if (same) return 0;
+    if (table.size() > L.tableCapacity) {
+        // The device table is read by kernels already queued on the stream: wait before replacing it.
+        size_t const cap = table.size() * 2 + 16;
         HIP_TRY(hipStreamSynchronize(L.stream));
-        std::memcpy(L.tableHost, table.data(), table.size() * sizeof(DevMip));
-        HIP_TRY(hipMemcpyAsync(L.tableDev, L.tableHost, table.size() * sizeof(DevMip), hipMemcpyHostToDevice, L.stream));
-        L.lastTable = table;
+        if (L.tableDev) { HIP_TRY(hipFree(L.tableDev)); L.tableDev = nullptr; }
+        L.tableCapacity = 0; L.lastTable.clear();
+        HIP_TRY(hipMalloc(reinterpret_cast<void**>(&L.tableDev), cap * sizeof(DevMip)));
+        L.tableCapacity = cap;
     }
+    Library::Slot& slot = L.slots[L.nextSlot];
+    L.nextSlot = (L.nextSlot + 1) % Library::kSlots;
+    if (slot.inFlight) { HIP_TRY(hipEventSynchronize(slot.done)); slot.inFlight = false; }
+    if (table.size() > slot.capacity) {
+        if (slot.host) { HIP_TRY(hipHostFree(slot.host)); slot.host = nullptr; slot.capacity = 0; }
+        HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&slot.host), L.tableCapacity * sizeof(DevMip), hipHostMallocDefault));
+        slot.capacity = L.tableCapacity;
+    }
+    if (!slot.done) HIP_TRY(hipEventCreateWithFlags(&slot.done, hipEventDisableTiming));
+    std::memcpy(slot.host, table.data(), table.size() * sizeof(DevMip));
+    HIP_TRY(hipMemcpyAsync(L.tableDev, slot.host, table.size() * sizeof(DevMip), hipMemcpyHostToDevice, L.stream));
+    HIP_TRY(hipEventRecord(slot.done, L.stream));
+    slot.inFlight = true;
+    L.lastTable = table;
     return 0;
 }
 
@@ -285,7 +297,6 @@ int grid_size_for(int variant, int totalTiles)
     static int perCu[16] = { 0 };
     if (perCu[variant] == 0) {
         perCu[variant] = resident_workgroups_per_cu(variant);
-        if (char const* env = std::getenv("NTC_HIP_WG_PER_CU")) { int v = std::atoi(env); if (v >= 1 && v <= 8) perCu[variant] = v; }
     }
     int const resident = g_lib.computeUnits * perCu[variant];
     return totalTiles < resident ? totalTiles : resident;
@@ -331,7 +342,10 @@ void ntc_hip_shutdown(void)
     if (!g_lib.initialized) return;
     (void)hipStreamSynchronize(g_lib.stream);
     if (g_lib.tableDev) (void)hipFree(g_lib.tableDev);
-    if (g_lib.tableHost) (void)hipHostFree(g_lib.tableHost);
+    for (Library::Slot& slot : g_lib.slots) {
+        if (slot.host) (void)hipHostFree(slot.host);
+        if (slot.done) (void)hipEventDestroy(slot.done);
+    }
     (void)hipEventDestroy(g_lib.evStart);
     (void)hipEventDestroy(g_lib.evStop);
     (void)hipStreamDestroy(g_lib.stream);
