@@ -210,6 +210,28 @@ typedef struct NtcHipReadChannels {
 } NtcHipReadChannels;
 int ntc_hip_read_channels(const NtcHipReadChannels* params);
 
+/* Stores a user image into the internal fp16 layout of one mip: what ITextureSet::WriteChannels
+ * does through cuda::CopyImage (src/TextureSet.cpp:829-913, src/ImageProcessing.cu:107-164,220-277).
+ * Same-size copies, linear colour spaces.  Asynchronous on the library stream. */
+typedef struct NtcHipWriteChannels {
+    const void* src;            /* device: pitch-linear user image */
+    uint64_t    srcBytes;
+    int32_t     format;         /* ChannelFormat, as in NtcHipReadChannels */
+    int32_t     verticalFlip;
+    uint64_t    pixelStride, rowPitch;
+    void*       planarPairs;    /* device: start of the mip in the internal layout */
+    uint64_t    planarBytes;
+    int32_t     width, height, setChannels, firstChannel, numChannels, reserved;
+} NtcHipWriteChannels;
+int ntc_hip_write_channels(const NtcHipWriteChannels* params);
+
+/* Mean squared error per channel between two images in the internal layout (a decoded mip and its
+ * reference): the loss branch of InferenceKernel + ReduceLoss (src/Inference.cu:77-118,142-156,
+ * src/Optimizer.cu:335-390) as a pass of its own, without the alpha-mask options.  Channels whose bit
+ * is clear in validChannelMask report 0.  outMse receives 16 floats.  Synchronous. */
+int ntc_hip_image_loss(const void* decodedPlanarPairs, const void* referencePlanarPairs, uint64_t planarBytes,
+                       int32_t width, int32_t height, int32_t setChannels, uint32_t validChannelMask, float* outMse);
+
 /* Self-check of the MFMA operand layout the kernels assume: multiplies a 16x64 by a
  * 64x16 int8 matrix on the device (row-major host arrays), writes the 16x16 int32
  * product.  No reference counterpart; used by the tests. */

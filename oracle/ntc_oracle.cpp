@@ -431,6 +431,8 @@ uint8_t  ntc_oracle_half_to_unorm8(uint16_t h) { return half_to_unorm8(h); }
 int      ntc_oracle_hgelu_quantize(float x) { return hgelu_quantize(x); }
 int      ntc_oracle_unpack_field(uint16_t w, int index, int bits) { return unpack_field(w, index, bits); }
 int32_t  ntc_oracle_e4m3_times_512(uint8_t byte) { return e4m3_times_512(byte); }
+void     ntc_oracle_layer_int8(const int8_t* W, const float* scale, const int32_t* bias, int in, int out,
+                               const int8_t* x, float* r) { layer_int8(W, scale, bias, in, out, x, r); }
 
 // PackLatentsKernel's QuantizeValue, src/Quantizer.cu:482-488 (encoder side; here only so
 // the tests can check Pack o Unpack = id).
@@ -548,6 +550,56 @@ int ntc_oracle_read_channels(const uint16_t* planarPairs, int width, int height,
             }
         }
     return 0;
+}
+
+// ITextureSet::WriteChannels' copy (1:1, linear colour spaces): ReadImageChannel in the user's format,
+// WriteImageChannel FLOAT16 into the internal planar-pair layout (src/ImageProcessing.cu:107-164,220-265),
+// with the optional vertical flip of SetupBilinearFilter (src/ImageProcessing.cu:36-37).
+int ntc_oracle_write_channels(const uint8_t* src, int format, int verticalFlip, uint64_t pixelStride, uint64_t rowPitch,
+                              uint16_t* planarPairs, int width, int height, int setChannels, int firstChannel, int numChannels)
+{
+    for (int y = 0; y < height; ++y)
+        for (int x = 0; x < width; ++x) {
+            int const srcY = verticalFlip ? height - 1 - y : y;
+            uint8_t const* px = src + size_t(srcY) * rowPitch + size_t(x) * pixelStride;
+            for (int ch = 0; ch < numChannels; ++ch) {
+                float v;
+                switch (format) {
+                case 1: v = float(px[ch]) / 255.f; break;
+                case 2: { uint16_t t; std::memcpy(&t, px + 2 * ch, 2); v = float(t) / 65535.f; break; }
+                case 3: { uint16_t t; std::memcpy(&t, px + 2 * ch, 2); v = half_to_float(t); break; }
+                case 4: std::memcpy(&v, px + 4 * ch, 4); break;
+                case 5: { uint32_t t; std::memcpy(&t, px + 4 * ch, 4); v = float(t); break; }
+                default: return -1;
+                }
+                v = std::max(-65504.f, std::min(65504.f, v));
+                int const c = firstChannel + ch;
+                planarPairs[size_t(y) * size_t(width) * size_t(setChannels) + size_t(x) * 2
+                            + size_t(c & ~1) * size_t(width) + size_t(c & 1)] = float_to_half_rne(v);
+            }
+        }
+    return 0;
+}
+
+// Per-channel mean squared error between a decoded mip and its reference, both in the internal
+// layout: what InferenceKernel's loss branch and ReduceLoss add up (src/Inference.cu:96-115,142-156,
+// src/Optimizer.cu:335-390), here in double.
+void ntc_oracle_image_loss(const uint16_t* a, const uint16_t* b, int width, int height, int setChannels,
+                           uint32_t validChannelMask, double* outMse /* 16 */)
+{
+    for (int c = 0; c < 16; ++c) outMse[c] = 0.0;
+    for (int y = 0; y < height; ++y)
+        for (int c = 0; c < setChannels; ++c) {
+            if (!((validChannelMask >> c) & 1u)) continue;
+            size_t const base = size_t(y) * size_t(width) * size_t(setChannels) + size_t(c & ~1) * size_t(width) + size_t(c & 1);
+            double acc = 0.0;
+            for (int x = 0; x < width; ++x) {
+                double const d = double(half_to_float(a[base + size_t(x) * 2])) - double(half_to_float(b[base + size_t(x) * 2]));
+                acc += d * d;
+            }
+            outMse[c] += acc;
+        }
+    for (int c = 0; c < 16; ++c) outMse[c] /= double(width) * double(height);
 }
 
 // Random-access decode of a list of (u, v, mip) sample points: NtcSampleTextureSet

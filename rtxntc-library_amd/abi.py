@@ -77,6 +77,15 @@ class ReadChannels(C.Structure):
     ]
 
 
+class WriteChannels(C.Structure):
+    _fields_ = [
+        ("src", C.c_void_p), ("srcBytes", C.c_uint64), ("format", C.c_int32), ("verticalFlip", C.c_int32),
+        ("pixelStride", C.c_uint64), ("rowPitch", C.c_uint64), ("planarPairs", C.c_void_p), ("planarBytes", C.c_uint64),
+        ("width", C.c_int32), ("height", C.c_int32), ("setChannels", C.c_int32), ("firstChannel", C.c_int32),
+        ("numChannels", C.c_int32), ("reserved", C.c_int32),
+    ]
+
+
 class Query(C.Structure):
     _fields_ = [("u", C.c_float), ("v", C.c_float), ("mip", C.c_int32)]
 
@@ -111,6 +120,9 @@ EXPORTS = [
     ("ntc_hip_decode_queries_timed", C.c_int, [C.POINTER(TextureSet), C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint64,
                                                C.c_int32, C.POINTER(C.c_float)]),
     ("ntc_hip_read_channels", C.c_int, [C.POINTER(ReadChannels)]),
+    ("ntc_hip_write_channels", C.c_int, [C.POINTER(WriteChannels)]),
+    ("ntc_hip_image_loss", C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64, C.c_int32, C.c_int32, C.c_int32, C.c_uint32,
+                                     C.POINTER(C.c_float)]),
     ("ntc_hip_selftest_mfma", C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
 ]
 

@@ -63,6 +63,21 @@ struct ReadChannelsArgs {
 };
 hipError_t launch_read_channels(ReadChannelsArgs const& args, hipStream_t stream);
 
+constexpr int NTC_HIP_DEV_MAX_CHANNELS = 16;
+
+struct WriteChannelsArgs {
+    uint8_t const* src;
+    uint16_t* planarPairs;
+    uint64_t pixelStride, rowPitch;
+    int32_t width, height, setChannels, firstChannel, numChannels, format, verticalFlip;
+};
+hipError_t launch_write_channels(WriteChannelsArgs const& args, hipStream_t stream);
+
+// Workgroups (= partial-sum rows of 16 doubles) the loss kernel uses for an image.
+inline size_t image_loss_blocks(int width, int height) { return size_t((width + 63) / 64) * size_t((height + 15) / 16); }
+hipError_t launch_image_loss(uint16_t const* a, uint16_t const* b, int width, int height, int setChannels,
+                             uint32_t validChannelMask, double* partials, hipStream_t stream);
+
 hipError_t launch_decode(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream);
 hipError_t launch_queries(int variant, DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries,
                           uint16_t* out, int gridSize, hipStream_t stream);

@@ -44,6 +44,9 @@ struct Library {
     DevMip* tableDev = nullptr;        // device copy of the mip table
     size_t tableCapacity = 0;          // entries
     std::vector<DevMip> lastTable;     // what tableDev currently holds (or will, in stream order)
+    double* lossDev = nullptr;         // per-workgroup partial sums of the loss pass
+    double* lossHost = nullptr;        // pinned copy of them
+    size_t lossBytes = 0;
     static constexpr int kSlots = 4;
     struct Slot { DevMip* host = nullptr; size_t capacity = 0; hipEvent_t done = nullptr; bool inFlight = false; };
     Slot slots[kSlots];                // pinned staging for asynchronous table uploads
@@ -342,6 +345,8 @@ void ntc_hip_shutdown(void)
     if (!g_lib.initialized) return;
     (void)hipStreamSynchronize(g_lib.stream);
     if (g_lib.tableDev) (void)hipFree(g_lib.tableDev);
+    if (g_lib.lossDev) (void)hipFree(g_lib.lossDev);
+    if (g_lib.lossHost) (void)hipHostFree(g_lib.lossHost);
     for (Library::Slot& slot : g_lib.slots) {
         if (slot.host) (void)hipHostFree(slot.host);
         if (slot.done) (void)hipEventDestroy(slot.done);
@@ -559,6 +564,82 @@ int ntc_hip_read_channels(const NtcHipReadChannels* p)
     a.firstChannel = p->firstChannel; a.numChannels = p->numChannels;
     a.dstChannels = int32_t(dstChannels); a.format = p->format;
     HIP_TRY(launch_read_channels(a, g_lib.stream));
+    clear_error();
+    return 0;
+}
+
+static int bytes_per_component(int format)
+{
+    switch (format) {
+    case NTC_HIP_DEV_FORMAT_UNORM8: return 1;
+    case NTC_HIP_DEV_FORMAT_UNORM16: case NTC_HIP_DEV_FORMAT_FLOAT16: return 2;
+    case NTC_HIP_DEV_FORMAT_FLOAT32: case NTC_HIP_DEV_FORMAT_UINT32: return 4;
+    default: return 0;
+    }
+}
+
+int ntc_hip_write_channels(const NtcHipWriteChannels* p)
+{
+    if (int r = require_init()) return r;
+    if (!p || !p->src || !p->planarPairs) { set_error("ntc_hip_write_channels: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
+    int const bpc = bytes_per_component(p->format);
+    if (!bpc) { set_error("ntc_hip_write_channels: unknown channel format %d.", p->format); return NTC_HIP_ERR_INVALID_ARG; }
+    if (p->width < 1 || p->height < 1 || p->setChannels < 2 || (p->setChannels & 1) || p->setChannels > NTC_HIP_MAX_CHANNELS
+        || p->firstChannel < 0 || p->numChannels < 1 || p->firstChannel + p->numChannels > p->setChannels) {
+        set_error("ntc_hip_write_channels: bad image or channel range.");
+        return NTC_HIP_ERR_INVALID_ARG;
+    }
+    if (p->pixelStride < uint64_t(bpc) * uint64_t(p->numChannels) || p->rowPitch < p->pixelStride * uint64_t(p->width)
+        || (p->pixelStride % uint64_t(bpc)) || (p->rowPitch % uint64_t(bpc)) || (reinterpret_cast<uintptr_t>(p->src) % uintptr_t(bpc))) {
+        set_error("ntc_hip_write_channels: pixel stride / row pitch do not fit the format and channel count.");
+        return NTC_HIP_ERR_INVALID_ARG;
+    }
+    uint64_t const srcNeed = uint64_t(p->height - 1) * p->rowPitch + uint64_t(p->width - 1) * p->pixelStride + uint64_t(bpc) * uint64_t(p->numChannels);
+    uint64_t const dstNeed = uint64_t(p->width) * uint64_t(p->height) * uint64_t(p->setChannels) * 2u;
+    if (srcNeed > p->srcBytes || dstNeed > p->planarBytes) { set_error("ntc_hip_write_channels: image reaches past the given buffer sizes."); return NTC_HIP_ERR_INVALID_ARG; }
+    WriteChannelsArgs a{};
+    a.src = static_cast<uint8_t const*>(p->src);
+    a.planarPairs = static_cast<uint16_t*>(p->planarPairs);
+    a.pixelStride = p->pixelStride; a.rowPitch = p->rowPitch;
+    a.width = p->width; a.height = p->height; a.setChannels = p->setChannels;
+    a.firstChannel = p->firstChannel; a.numChannels = p->numChannels; a.format = p->format; a.verticalFlip = p->verticalFlip ? 1 : 0;
+    HIP_TRY(launch_write_channels(a, g_lib.stream));
+    clear_error();
+    return 0;
+}
+
+int ntc_hip_image_loss(const void* decoded, const void* reference, uint64_t planarBytes, int32_t width, int32_t height,
+                       int32_t setChannels, uint32_t validChannelMask, float* outMse)
+{
+    if (int r = require_init()) return r;
+    if (!decoded || !reference || !outMse) { set_error("ntc_hip_image_loss: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
+    if (width < 1 || height < 1 || setChannels < 2 || (setChannels & 1) || setChannels > NTC_HIP_MAX_CHANNELS
+        || uint64_t(width) * uint64_t(height) * uint64_t(setChannels) * 2u > planarBytes) {
+        set_error("ntc_hip_image_loss: bad image shape or buffer size.");
+        return NTC_HIP_ERR_INVALID_ARG;
+    }
+    size_t const blocks = image_loss_blocks(width, height);
+    size_t const bytes = blocks * NTC_HIP_DEV_MAX_CHANNELS * sizeof(double);
+    Library& L = g_lib;
+    if (bytes > L.lossBytes) {
+        HIP_TRY(hipStreamSynchronize(L.stream));
+        if (L.lossDev) { HIP_TRY(hipFree(L.lossDev)); L.lossDev = nullptr; }
+        if (L.lossHost) { HIP_TRY(hipHostFree(L.lossHost)); L.lossHost = nullptr; }
+        L.lossBytes = 0;
+        HIP_TRY(hipMalloc(reinterpret_cast<void**>(&L.lossDev), bytes));
+        HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&L.lossHost), bytes, hipHostMallocDefault));
+        L.lossBytes = bytes;
+    }
+    HIP_TRY(launch_image_loss(static_cast<uint16_t const*>(decoded), static_cast<uint16_t const*>(reference), width, height,
+                              setChannels, validChannelMask, L.lossDev, L.stream));
+    HIP_TRY(hipMemcpyAsync(L.lossHost, L.lossDev, bytes, hipMemcpyDeviceToHost, L.stream));
+    HIP_TRY(hipStreamSynchronize(L.stream));
+    double const norm = 1.0 / (double(width) * double(height));
+    for (int c = 0; c < NTC_HIP_DEV_MAX_CHANNELS; ++c) {
+        double acc = 0.0;
+        for (size_t b = 0; b < blocks; ++b) acc += L.lossHost[b * NTC_HIP_DEV_MAX_CHANNELS + size_t(c)];
+        outMse[c] = float(acc * norm);
+    }
     clear_error();
     return 0;
 }

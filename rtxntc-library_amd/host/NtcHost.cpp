@@ -13,6 +13,7 @@
 #include <cstring>
 #include <limits>
 #include <new>
+#include <string>
 #include <vector>
 
 namespace ntc
@@ -95,6 +96,34 @@ void PositionConstants(NtcHipMipDesc& d)
 
 class Context;
 
+// src/TextureMetadata.cpp:30-75 (name and channel range only)
+class TextureMetadata final : public ITextureMetadata
+{
+public:
+    explicit TextureMetadata(TextureSetDesc const& setDesc) : m_setDesc(setDesc) {}
+    void SetName(char const* name) override { m_name = name ? name : ""; }
+    char const* GetName() const override { return m_name.c_str(); }
+    Status SetChannels(int firstChannel, int numChannels) override
+    {
+        if (firstChannel < 0 || firstChannel >= m_setDesc.channels) {
+            SetErrorMessage("firstChannel (%d) must be between 0 and %d.", firstChannel, m_setDesc.channels - 1);
+            return Status::OutOfRange;
+        }
+        if (numChannels < 1 || numChannels + firstChannel > m_setDesc.channels) {
+            SetErrorMessage("For the provided firstChannel (%d), numChannels (%d) must be between 1 and %d.",
+                firstChannel, numChannels, m_setDesc.channels - firstChannel);
+            return Status::OutOfRange;
+        }
+        m_firstChannel = firstChannel; m_numChannels = numChannels;
+        return Status::Ok;
+    }
+    void GetChannels(int& outFirstChannel, int& outNumChannels) const override { outFirstChannel = m_firstChannel; outNumChannels = m_numChannels; }
+private:
+    TextureSetDesc const& m_setDesc;
+    std::string m_name;
+    int m_firstChannel = 0, m_numChannels = 0;
+};
+
 class TextureSet final : public ITextureSet
 {
 public:
@@ -103,7 +132,9 @@ public:
 
     ~TextureSet() override
     {
+        ClearTextureMetadata();
         ReleaseDevice(m_textureData);
+        ReleaseDevice(m_textureDataOut);
         ReleaseDevice(m_staging);
         ReleaseDevice(m_latents);
         ReleaseDevice(m_weights);
@@ -129,6 +160,9 @@ public:
         m_stagingBytes = uint64_t(stagingWidth) * uint64_t(stagingHeight) * uint64_t(std::max(0, m_features.stagingBytesPerPixel));
         if (m_deviceAvailable) {
             if (int r = ntc_hip_alloc(&m_textureData, m_textureBytes)) return AllocationFailure(r, "texture data", m_textureBytes);
+            // A second page keeps the reference image apart from the decoded one (src/TextureSet.cpp:103-124).
+            if (m_features.separateRefOutData)
+                if (int r = ntc_hip_alloc(&m_textureDataOut, m_textureBytes)) return AllocationFailure(r, "texture data (output)", m_textureBytes);
             if (m_stagingBytes)
                 if (int r = ntc_hip_alloc(&m_staging, m_stagingBytes)) return AllocationFailure(r, "staging", m_stagingBytes);
         }
@@ -137,7 +171,35 @@ public:
 
     TextureSetDesc const& GetDesc() const override { return m_desc; }
     LatentShape const& GetLatentShape() const override { return m_latentShape; }
-    uint32_t GetValidChannelMask() const override { return 0; }
+    ITextureMetadata* AddTexture() override
+    {
+        TextureMetadata* t = new (std::nothrow) TextureMetadata(m_desc);
+        if (t) m_textures.push_back(t);
+        return t;
+    }
+    Status RemoveTexture(ITextureMetadata* texture) override
+    {
+        auto it = std::find(m_textures.begin(), m_textures.end(), texture);
+        if (it == m_textures.end()) { SetErrorMessage("The texture does not belong to this texture set."); return Status::OutOfRange; }
+        delete *it;
+        m_textures.erase(it);
+        return Status::Ok;
+    }
+    void ClearTextureMetadata() override { for (TextureMetadata* t : m_textures) delete t; m_textures.clear(); }
+    int GetTextureCount() const override { return int(m_textures.size()); }
+    ITextureMetadata* GetTexture(int index) override { return (index >= 0 && index < int(m_textures.size())) ? m_textures[size_t(index)] : nullptr; }
+
+    // src/TextureSetMetadata.cpp:807-832 (no output shuffling here)
+    uint32_t GetValidChannelMask() const override
+    {
+        uint32_t mask = 0;
+        for (TextureMetadata const* t : m_textures) {
+            int first, count;
+            t->GetChannels(first, count);
+            mask |= ((1u << count) - 1u) << first;
+        }
+        return mask;
+    }
 
     Status SetDecoderPreset(DecoderPreset preset) override
     {
@@ -187,6 +249,13 @@ public:
         if (pOutStats) { *pOutStats = DecompressionStats(); std::fill_n(pOutStats->perChannelLoss, 16, 0.f); std::fill_n(pOutStats->perMipLoss, 16, 0.f); }
         if (!m_deviceAvailable) { SetErrorMessage("No HIP device is available to this context."); return Status::CudaUnavailable; }
 
+        // Losses need the reference image to survive the decode: decode into a second page.
+        uint32_t const validMask = GetValidChannelMask();
+        bool const lazyOutPage = validMask != 0 && !m_textureDataOut;
+        if (lazyOutPage)
+            if (int r = ntc_hip_alloc(&m_textureDataOut, m_textureBytes)) return AllocationFailure(r, "texture data (output)", m_textureBytes);
+        void* const outPage = m_textureDataOut ? m_textureDataOut : m_textureData;   // src/TextureSet.cpp:1799-1802
+
         NtcHipTextureSet set{};
         set.spec = m_spec;
         set.numMips = m_desc.mips;
@@ -194,7 +263,7 @@ public:
         set.outputFormat = NTC_HIP_OUT_FP16_PLANAR_PAIRS;
         set.latents = m_latents; set.latentsBytes = m_latentBytes;
         set.weights = m_weights; set.weightsBytes = m_weightLayout.bufferSize;
-        set.output = m_textureData; set.outputBytes = m_textureBytes;
+        set.output = outPage; set.outputBytes = m_textureBytes;
         for (int mip = 0; mip < m_desc.mips; ++mip) {
             set.mips[mip] = m_mips[mip];
             set.mips[mip].outOffset = m_mipOffsets[mip] * uint64_t(m_desc.channels) * 2u;   // src/TextureSet.cpp:1804
@@ -208,7 +277,73 @@ public:
         } else if (int r = ntc_hip_decode(&set, 1)) {
             return DeviceFailure(r);
         }
+
+        // Per-channel / per-mip / overall mean squared error, weighted by pixel count exactly as
+        // src/TextureSet.cpp:1833-1863,1884-1892 combine them.
+        if (validMask != 0 && pOutStats) {
+            int validChannels = 0;
+            for (int ch = 0; ch < m_desc.channels; ++ch) if (validMask & (1u << ch)) ++validChannels;
+            double perChannel[16] = {};
+            double overall = 0.0, pixels = 0.0;
+            for (int mip = 0; mip < m_desc.mips; ++mip) {
+                uint64_t const offset = m_mipOffsets[mip] * uint64_t(m_desc.channels) * 2u;
+                float mse[16];
+                if (int r = ntc_hip_image_loss(static_cast<uint8_t const*>(outPage) + offset, static_cast<uint8_t const*>(m_textureData) + offset,
+                                               m_textureBytes - offset, m_mips[mip].width, m_mips[mip].height, m_desc.channels, validMask, mse))
+                    return DeviceFailure(r);
+                double const mipPixels = double(m_mips[mip].width) * double(m_mips[mip].height);
+                double mean = 0.0;
+                for (int ch = 0; ch < m_desc.channels; ++ch) {
+                    if (!(validMask & (1u << ch))) continue;
+                    mean += mse[ch];
+                    perChannel[ch] += mipPixels * mse[ch];
+                }
+                mean /= double(validChannels);
+                pOutStats->perMipLoss[mip] = float(mean);
+                overall += mipPixels * mean;
+                pixels += mipPixels;
+            }
+            pOutStats->overallLoss = float(overall / pixels);
+            for (int ch = 0; ch < 16; ++ch) pOutStats->perChannelLoss[ch] = float(perChannel[ch] / pixels);
+        }
+        // Without separateRefOutData both pages are one memory in the reference and the decode
+        // overwrites the reference image; keep that: the decoded page becomes the only page.
+        if (lazyOutPage) {
+            if (int r = ntc_hip_synchronize()) return DeviceFailure(r);
+            std::swap(m_textureData, m_textureDataOut);
+            ReleaseDevice(m_textureDataOut);
+        }
         m_decompressed = true;
+        ClearErrorMessage();
+        return Status::Ok;
+    }
+
+    // src/TextureSet.cpp:829-913
+    Status WriteChannels(WriteChannelsParameters const& params) override
+    {
+        if (!params.pData) { SetErrorMessage("pData is NULL."); return Status::InvalidArgument; }
+        size_t const sizeToCopy = size_t(params.height) * params.rowPitch;
+        bool const fromHost = params.addressSpace == AddressSpace::Host;
+        if (Status st = ValidateReadWriteChannelsArgs(params.mipLevel, params.firstChannel, params.numChannels, params.width, params.height,
+                params.pixelStride, params.rowPitch, fromHost ? sizeToCopy : 0, params.channelFormat, "writes"); st != Status::Ok)
+            return st;
+        if (params.srcColorSpaces || params.dstColorSpaces) { SetErrorMessage("Non-linear colour spaces are not supported."); return Status::Unsupported; }
+        if (!m_deviceAvailable) { SetErrorMessage("No HIP device is available to this context."); return Status::CudaUnavailable; }
+        if (fromHost)
+            if (int r = ntc_hip_upload(m_staging, params.pData, sizeToCopy)) return DeviceFailure(r);
+        int const mipWidth = std::max(m_desc.width >> params.mipLevel, 1), mipHeight = std::max(m_desc.height >> params.mipLevel, 1);
+        NtcHipWriteChannels wc{};
+        wc.src = fromHost ? m_staging : static_cast<void const*>(params.pData);
+        wc.srcBytes = sizeToCopy;
+        wc.format = int(params.channelFormat);
+        wc.verticalFlip = params.verticalFlip ? 1 : 0;
+        wc.pixelStride = params.pixelStride; wc.rowPitch = params.rowPitch;
+        uint64_t const offset = m_mipOffsets[params.mipLevel] * uint64_t(m_desc.channels) * 2u;
+        wc.planarPairs = static_cast<uint8_t*>(m_textureData) + offset;               // the reference page
+        wc.planarBytes = m_textureBytes - offset;
+        wc.width = mipWidth; wc.height = mipHeight; wc.setChannels = m_desc.channels;
+        wc.firstChannel = params.firstChannel; wc.numChannels = params.numChannels;
+        if (int r = ntc_hip_write_channels(&wc)) return DeviceFailure(r);
         ClearErrorMessage();
         return Status::Ok;
     }
@@ -218,40 +353,11 @@ public:
     {
         if (!params.pOutData) { SetErrorMessage("pOutData is NULL."); return Status::InvalidArgument; }
         size_t const sizeToCopy = size_t(params.height) * params.rowPitch;
-        if (params.mipLevel < 0 || params.mipLevel >= m_desc.mips) {
-            SetErrorMessage("mipLevel (%d) must be between 0 and %d.", params.mipLevel, m_desc.mips - 1);
-            return Status::OutOfRange;
-        }
-        if (params.firstChannel < 0 || params.firstChannel >= m_desc.channels) {
-            SetErrorMessage("firstChannel (%d) must be between 0 and %d.", params.firstChannel, m_desc.channels - 1);
-            return Status::OutOfRange;
-        }
-        if (params.numChannels < 1 || params.numChannels + params.firstChannel > m_desc.channels) {
-            SetErrorMessage("For the provided firstChannel (%d), numChannels (%d) must be between 1 and %d.",
-                params.firstChannel, params.numChannels, m_desc.channels - params.firstChannel);
-            return Status::OutOfRange;
-        }
-        if (params.width <= 0 || params.height <= 0) {
-            SetErrorMessage("width (%d) and height (%d) must be positive.", params.width, params.height);
-            return Status::OutOfRange;
-        }
-        if (params.pixelStride < 1 || params.rowPitch < params.pixelStride) {
-            SetErrorMessage("pixelStride (%zu) must be between 1 and rowPitch (%zu).", params.pixelStride, params.rowPitch);
-            return Status::InvalidArgument;
-        }
         bool const toHost = params.addressSpace == AddressSpace::Host;
-        if (toHost && sizeToCopy > m_stagingBytes) {
-            SetErrorMessage("The operation requires copying too much data (%zu bytes), must fit into "
-                "the staging buffer (%zu bytes).", sizeToCopy, size_t(m_stagingBytes));
-            return Status::OutOfRange;
-        }
-        size_t const bpc = GetBytesPerPixelComponent(params.channelFormat);
-        if (bpc == 0) { SetErrorMessage("Unknown channel format %d.", int(params.channelFormat)); return Status::InvalidArgument; }
+        if (Status st = ValidateReadWriteChannelsArgs(params.mipLevel, params.firstChannel, params.numChannels, params.width, params.height,
+                params.pixelStride, params.rowPitch, toHost ? sizeToCopy : 0, params.channelFormat, "reads"); st != Status::Ok)
+            return st;
         int const mipWidth = std::max(m_desc.width >> params.mipLevel, 1), mipHeight = std::max(m_desc.height >> params.mipLevel, 1);
-        if (params.width != mipWidth || params.height != mipHeight) {
-            SetErrorMessage("Resizing reads are not supported: the image must be %dx%d for mip %d.", mipWidth, mipHeight, params.mipLevel);
-            return Status::Unsupported;
-        }
         if (params.useDithering || params.dstColorSpaces) {
             SetErrorMessage("Dithering and non-linear destination colour spaces are not supported.");
             return Status::Unsupported;
@@ -263,7 +369,9 @@ public:
             if (int r = ntc_hip_memset(m_staging, 0, sizeToCopy)) return DeviceFailure(r);
 
         NtcHipReadChannels rc{};
-        rc.planarPairs = static_cast<uint8_t const*>(m_textureData) + m_mipOffsets[params.mipLevel] * uint64_t(m_desc.channels) * 2u;
+        // GetTextureDataSlice: the output page when it exists and is asked for (src/TextureSet.cpp:1961-1964)
+        void const* const page = (params.page == TextureDataPage::Output && m_textureDataOut) ? m_textureDataOut : m_textureData;
+        rc.planarPairs = static_cast<uint8_t const*>(page) + m_mipOffsets[params.mipLevel] * uint64_t(m_desc.channels) * 2u;
         rc.planarBytes = uint64_t(mipWidth) * uint64_t(mipHeight) * uint64_t(m_desc.channels) * 2u;
         rc.width = mipWidth; rc.height = mipHeight;
         rc.setChannels = m_desc.channels;
@@ -280,6 +388,45 @@ public:
     }
 
 private:
+    // src/TextureSet.cpp:1914-1956, plus what this library cannot do (resizing copies)
+    Status ValidateReadWriteChannelsArgs(int mipLevel, int firstChannel, int numChannels, int width, int height,
+        size_t pixelStride, size_t rowPitch, size_t stagedBytes, ChannelFormat format, char const* what)
+    {
+        if (mipLevel < 0 || mipLevel >= m_desc.mips) {
+            SetErrorMessage("mipLevel (%d) must be between 0 and %d.", mipLevel, m_desc.mips - 1);
+            return Status::OutOfRange;
+        }
+        if (firstChannel < 0 || firstChannel >= m_desc.channels) {
+            SetErrorMessage("firstChannel (%d) must be between 0 and %d.", firstChannel, m_desc.channels - 1);
+            return Status::OutOfRange;
+        }
+        if (numChannels < 1 || numChannels + firstChannel > m_desc.channels) {
+            SetErrorMessage("For the provided firstChannel (%d), numChannels (%d) must be between 1 and %d.",
+                firstChannel, numChannels, m_desc.channels - firstChannel);
+            return Status::OutOfRange;
+        }
+        if (width <= 0 || height <= 0) {
+            SetErrorMessage("width (%d) and height (%d) must be positive.", width, height);
+            return Status::OutOfRange;
+        }
+        if (pixelStride < 1 || rowPitch < pixelStride) {
+            SetErrorMessage("pixelStride (%zu) must be between 1 and rowPitch (%zu).", pixelStride, rowPitch);
+            return Status::InvalidArgument;
+        }
+        if (stagedBytes > m_stagingBytes) {
+            SetErrorMessage("The operation requires copying too much data (%zu bytes), must fit into "
+                "the staging buffer (%zu bytes).", stagedBytes, size_t(m_stagingBytes));
+            return Status::OutOfRange;
+        }
+        if (GetBytesPerPixelComponent(format) == 0) { SetErrorMessage("Unknown channel format %d.", int(format)); return Status::InvalidArgument; }
+        int const mipWidth = std::max(m_desc.width >> mipLevel, 1), mipHeight = std::max(m_desc.height >> mipLevel, 1);
+        if (width != mipWidth || height != mipHeight) {
+            SetErrorMessage("Resizing %s are not supported: the image must be %dx%d for mip %d.", what, mipWidth, mipHeight, mipLevel);
+            return Status::Unsupported;
+        }
+        return Status::Ok;
+    }
+
     Status AllocationFailure(int code, char const* what, uint64_t bytes)
     {
         if (code > 0) { SetErrorMessage("Failed to allocate %llu bytes of device memory for the %s buffer.", (unsigned long long)bytes, what); return Status::OutOfMemory; }
@@ -389,7 +536,9 @@ private:
     NtcHipMipDesc m_mips[NTC_HIP_MAX_MIPS]{};
     uint64_t m_mipOffsets[NTC_HIP_MAX_MIPS + 1]{};
     uint64_t m_textureBytes = 0, m_stagingBytes = 0, m_latentBytes = 0;
-    void* m_textureData = nullptr;
+    std::vector<TextureMetadata*> m_textures;
+    void* m_textureData = nullptr;      // reference page (and the only page without separateRefOutData)
+    void* m_textureDataOut = nullptr;   // output page
     void* m_staging = nullptr;
     void* m_latents = nullptr;
     void* m_weights = nullptr;

@@ -69,6 +69,24 @@ struct TextureSetFeatures
     bool separateRefOutData = false;
 };
 
+// include/libntc/ntc.h:645-687
+struct WriteChannelsParameters
+{
+    int mipLevel = 0;
+    int firstChannel = 0;
+    int numChannels = 0;
+    unsigned char const* pData = nullptr;
+    AddressSpace addressSpace = AddressSpace::Host;
+    int width = 0;
+    int height = 0;
+    size_t pixelStride = 0;
+    size_t rowPitch = 0;
+    ChannelFormat channelFormat = ChannelFormat::UNKNOWN;
+    void const* srcColorSpaces = nullptr;   // must be null: only linear storage is supported
+    void const* dstColorSpaces = nullptr;
+    bool verticalFlip = false;
+};
+
 // include/libntc/ntc.h:689-730
 struct ReadChannelsParameters
 {
@@ -87,8 +105,9 @@ struct ReadChannelsParameters
     bool useDithering = false;              // must be false
 };
 
-// include/libntc/ntc.h:810-816.  Losses stay zero: with no reference image registered the
-// reference takes the same branch (src/Inference.cu:119-136, src/TextureSet.cpp:1833).
+// include/libntc/ntc.h:810-816.  Losses are mean squared errors against the image written with
+// WriteChannels, over the channels that textures claim (GetValidChannelMask); with no texture
+// registered they stay zero, as in the reference (src/Inference.cu:119-136, src/TextureSet.cpp:1833).
 struct DecompressionStats
 {
     float perChannelLoss[16];
@@ -114,11 +133,31 @@ enum class DecoderPreset
     Concat2x2_48 = 2    // same grids with 12 LR features, MLP 64-48-48-32-16
 };
 
+// The slice of include/libntc/ntc.h:385-455 that decides which channels hold image data.
+class ITextureMetadata
+{
+public:
+    virtual void SetName(char const* name) = 0;
+    virtual char const* GetName() const = 0;
+    // Assigns the texture's channels inside the set; OutOfRange unless the range lies inside the
+    // set's channels (src/TextureMetadata.cpp:48-69).
+    virtual Status SetChannels(int firstChannel, int numChannels) = 0;
+    virtual void GetChannels(int& outFirstChannel, int& outNumChannels) const = 0;
+    virtual ~ITextureMetadata() = default;
+};
+
 class ITextureSet
 {
 public:
     virtual TextureSetDesc const& GetDesc() const = 0;
     virtual LatentShape const& GetLatentShape() const = 0;
+
+    // include/libntc/ntc.h:551-568
+    virtual ITextureMetadata* AddTexture() = 0;
+    virtual Status RemoveTexture(ITextureMetadata* texture) = 0;
+    virtual void ClearTextureMetadata() = 0;
+    virtual int GetTextureCount() const = 0;
+    virtual ITextureMetadata* GetTexture(int textureIndex) = 0;
 
     // Changes the latent shape; all compressed data is lost (include/libntc/ntc.h:858-861).
     // Range rules follow src/TextureSetMetadata.cpp:1137-1159.
@@ -139,10 +178,15 @@ public:
     // and ignored: the int8 weights are the only weights.
     virtual Status Decompress(DecompressionStats* pOutStats, bool useInt8Weights = false) = 0;
 
+    // Stores a reference image (include/libntc/ntc.h:899, src/TextureSet.cpp:829-913): the data
+    // Decompress measures its loss against.
+    virtual Status WriteChannels(WriteChannelsParameters const& params) = 0;
+
     // include/libntc/ntc.h:902, src/TextureSet.cpp:915-985.
     virtual Status ReadChannels(ReadChannelsParameters const& params) = 0;
 
-    // Always 0: no reference images can be registered (include/libntc/ntc.h:638-640).
+    // Union of the channel ranges of the registered textures (include/libntc/ntc.h:638-640,
+    // src/TextureSetMetadata.cpp:807-832).
     virtual uint32_t GetValidChannelMask() const = 0;
 
     virtual ~ITextureSet() = default;

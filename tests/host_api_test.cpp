@@ -5,6 +5,9 @@
 //   host_api_test decode <preset> <w> <h> <mips> <channels> <gridScale> <features> <latents> <weights> <outPrefix>
 //       loads raw latents/weights, decompresses, reads every mip back as UNORM8 (host address
 //       space) and FLOAT16 (device address space is exercised through a second read), writes files
+//   host_api_test loss <preset> <w> <h> <mips> <channels> <gridScale> <features> <latents> <weights> <refPrefix> <separate 0|1>
+//       registers two textures (channels 0..2 and 4..5), writes <refPrefix>_mip<N>.bin (FLOAT32 pixels,
+//       all channels) as the reference image, decompresses twice and prints the loss statistics
 #include "../rtxntc-library_amd/host/ntc_decode.h"
 #include "../include/ntc_hip.h"
 
@@ -92,6 +95,37 @@ static int cpuChecks()
     CHECK(set->GetWeightDataSize() == 10496 && set->GetLatentDataSize() == 22369636ull);
     CHECK(set->SetDecoderPreset(DecoderPreset::Concat2x2_48) == Status::Ok);
     CHECK(set->GetWeightDataSize() == 8576);
+
+    // texture metadata decides which channels count (src/TextureMetadata.cpp:48-69)
+    ITextureMetadata* albedo = set->AddTexture();
+    CHECK(albedo != nullptr && set->GetTextureCount() == 1 && set->GetTexture(0) == albedo && set->GetTexture(1) == nullptr);
+    albedo->SetName("albedo");
+    CHECK(std::strcmp(albedo->GetName(), "albedo") == 0);
+    CHECK(albedo->SetChannels(-1, 3) == Status::OutOfRange && albedo->SetChannels(16, 1) == Status::OutOfRange);
+    CHECK(albedo->SetChannels(14, 3) == Status::OutOfRange && albedo->SetChannels(0, 0) == Status::OutOfRange);
+    CHECK(albedo->SetChannels(1, 3) == Status::Ok && set->GetValidChannelMask() == 0xEu);
+    ITextureMetadata* height = set->AddTexture();
+    CHECK(height->SetChannels(8, 1) == Status::Ok && set->GetValidChannelMask() == 0x10Eu);
+    int first = -1, count = -1;
+    height->GetChannels(first, count);
+    CHECK(first == 8 && count == 1);
+    CHECK(set->RemoveTexture(albedo) == Status::Ok && set->RemoveTexture(albedo) == Status::OutOfRange);
+    CHECK(set->GetTextureCount() == 1 && set->GetValidChannelMask() == 0x100u);
+    set->ClearTextureMetadata();
+    CHECK(set->GetTextureCount() == 0 && set->GetValidChannelMask() == 0);
+
+    // WriteChannels shares the argument checks of ReadChannels (src/TextureSet.cpp:829-850,1914-1956)
+    WriteChannelsParameters wp;
+    CHECK(set->WriteChannels(wp) == Status::InvalidArgument);                // pData NULL
+    std::vector<unsigned char> source(64);
+    wp.pData = source.data(); wp.mipLevel = -1;
+    CHECK(set->WriteChannels(wp) == Status::OutOfRange);
+    wp.mipLevel = 12; wp.firstChannel = 15; wp.numChannels = 2;
+    CHECK(set->WriteChannels(wp) == Status::OutOfRange);
+    wp.numChannels = 1; wp.width = 1; wp.height = 1; wp.pixelStride = 0; wp.rowPitch = 4;
+    CHECK(set->WriteChannels(wp) == Status::InvalidArgument);
+    wp.pixelStride = 4; wp.channelFormat = ChannelFormat::FLOAT32;
+    CHECK(set->WriteChannels(wp) == Status::CudaUnavailable);
 
     // ReadChannels argument checks (src/TextureSet.cpp:1914-1956)
     std::vector<unsigned char> pixels(16);
@@ -185,8 +219,76 @@ static int decode(int argc, char** argv)
     return 0;
 }
 
+static int loss(int argc, char** argv)
+{
+    if (argc < 13) { std::fprintf(stderr, "usage: loss <preset> <w> <h> <mips> <channels> <gridScale> <features> <latents> <weights> <refPrefix> <separate>\n"); return 2; }
+    int const preset = std::atoi(argv[2]), w = std::atoi(argv[3]), h = std::atoi(argv[4]), mips = std::atoi(argv[5]);
+    int const channels = std::atoi(argv[6]), gridScale = std::atoi(argv[7]), features = std::atoi(argv[8]);
+    std::vector<unsigned char> latents = readFile(argv[9]), weights = readFile(argv[10]);
+    std::string const prefix = argv[11];
+    bool const separate = std::atoi(argv[12]) != 0;
+
+    IContext* ctx = nullptr;
+    ContextParameters params;
+    CHECK(CreateContext(&ctx, params) == Status::Ok);
+    TextureSetDesc desc; desc.width = w; desc.height = h; desc.channels = channels; desc.mips = mips;
+    TextureSetFeatures features_;
+    features_.stagingBytesPerPixel = 16 * 4;
+    features_.separateRefOutData = separate;
+    ITextureSet* set = nullptr;
+    CHECK(ctx->CreateTextureSet(desc, features_, &set) == Status::Ok);
+    if (preset == 0) { LatentShape shape; shape.gridSizeScale = gridScale; shape.numFeatures = features; CHECK(set->SetLatentShape(shape) == Status::Ok); }
+    else CHECK(set->SetDecoderPreset(DecoderPreset(preset)) == Status::Ok);
+    CHECK(set->SetLatentData(latents.data(), latents.size()) == Status::Ok);
+    CHECK(set->SetWeightData(weights.data(), weights.size()) == Status::Ok);
+    ITextureMetadata* a = set->AddTexture(); CHECK(a->SetChannels(0, 3) == Status::Ok);
+    ITextureMetadata* b = set->AddTexture(); CHECK(b->SetChannels(4, 2) == Status::Ok);
+    CHECK(set->GetValidChannelMask() == 0x37u);
+    int const C = set->GetDesc().channels;
+    for (int mip = 0; mip < mips; ++mip) {
+        int const mw = std::max(w >> mip, 1), mh = std::max(h >> mip, 1);
+        std::vector<unsigned char> ref = readFile((prefix + "_mip" + std::to_string(mip) + ".bin").c_str());
+        CHECK(ref.size() == size_t(mw) * size_t(mh) * size_t(C) * 4);
+        WriteChannelsParameters wp;
+        wp.mipLevel = mip; wp.firstChannel = 0; wp.numChannels = C; wp.pData = ref.data();
+        wp.width = mw; wp.height = mh; wp.pixelStride = size_t(C) * 4; wp.rowPitch = wp.pixelStride * size_t(mw);
+        wp.channelFormat = ChannelFormat::FLOAT32;
+        CHECK(set->WriteChannels(wp) == Status::Ok);
+    }
+    auto printStats = [&](char const* tag, DecompressionStats const& st) {
+        std::printf("%s overall %.9g\n%s mips", tag, st.overallLoss, tag);
+        for (int m = 0; m < mips; ++m) std::printf(" %.9g", st.perMipLoss[m]);
+        std::printf("\n%s channels", tag);
+        for (int c = 0; c < 16; ++c) std::printf(" %.9g", st.perChannelLoss[c]);
+        std::printf("\n");
+    };
+    DecompressionStats first, second;
+    CHECK(set->Decompress(&first) == Status::Ok);
+    printStats("first", first);
+    CHECK(set->Decompress(&second) == Status::Ok);
+    printStats("second", second);
+    // Reference page after the decode: the written image when the pages are separate, the
+    // decoded image when they share memory (src/TextureSet.cpp:103-124).
+    ReadChannelsParameters rp;
+    rp.mipLevel = 0; rp.firstChannel = 0; rp.numChannels = C; rp.width = w; rp.height = h;
+    rp.pixelStride = size_t(C) * 2; rp.rowPitch = rp.pixelStride * size_t(w); rp.channelFormat = ChannelFormat::FLOAT16;
+    std::vector<unsigned char> page(rp.rowPitch * size_t(h));
+    rp.pOutData = page.data();
+    rp.page = TextureDataPage::Reference;
+    CHECK(set->ReadChannels(rp) == Status::Ok);
+    CHECK(writeFile(prefix + "_page_reference.bin", page.data(), page.size()));
+    rp.page = TextureDataPage::Output;
+    CHECK(set->ReadChannels(rp) == Status::Ok);
+    CHECK(writeFile(prefix + "_page_output.bin", page.data(), page.size()));
+    ctx->DestroyTextureSet(set);
+    DestroyContext(ctx);
+    std::printf("host loss OK\n");
+    return 0;
+}
+
 int main(int argc, char** argv)
 {
+    if (argc >= 2 && std::strcmp(argv[1], "loss") == 0) return loss(argc, argv);
     if (argc >= 2 && std::strcmp(argv[1], "cpu") == 0) return cpuChecks();
     if (argc >= 2 && std::strcmp(argv[1], "decode") == 0) return decode(argc, argv);
     std::fprintf(stderr, "usage: host_api_test cpu | decode ...\n");

@@ -37,6 +37,8 @@ def load_oracle():
         lib.ntc_oracle_unpack_field.argtypes = [C.c_uint16, C.c_int, C.c_int]
         lib.ntc_oracle_e4m3_times_512.restype = C.c_int32
         lib.ntc_oracle_e4m3_times_512.argtypes = [C.c_uint8]
+        lib.ntc_oracle_layer_int8.restype = None
+        lib.ntc_oracle_layer_int8.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
         lib.ntc_oracle_quantize_value.restype = C.c_uint32
         lib.ntc_oracle_quantize_value.argtypes = [C.c_float, C.c_int]
         lib.ntc_oracle_encode_position.restype = None
@@ -53,6 +55,11 @@ def load_oracle():
         lib.ntc_oracle_decode_rows.argtypes = [C.POINTER(_abi.TextureSet), C.c_int, C.c_int, C.c_int, C.c_int]
         lib.ntc_oracle_decode_queries.restype = C.c_int
         lib.ntc_oracle_decode_queries.argtypes = [C.POINTER(_abi.TextureSet), C.c_void_p, C.c_uint64, C.c_void_p, C.c_int]
+        lib.ntc_oracle_write_channels.restype = C.c_int
+        lib.ntc_oracle_write_channels.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_uint64, C.c_uint64, C.c_void_p,
+                                                  C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
+        lib.ntc_oracle_image_loss.restype = None
+        lib.ntc_oracle_image_loss.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_uint32, C.c_void_p]
         lib.ntc_oracle_read_channels.restype = C.c_int
         lib.ntc_oracle_read_channels.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p,
                                                  C.c_int, C.c_uint64, C.c_uint64]

@@ -136,3 +136,177 @@ def test_host_layer_decode_and_read_back(ntc, oracle, tmp_path, preset):
         oracle.ntc_oracle_read_channels(planar.ctypes.data, mip.width, mip.height, channels, 1, 3, want16.ctypes.data, 3, 8, mip.width * 8)
         got16 = np.fromfile(f"{prefix}_mip{m}_rgba16f.bin", dtype=np.uint8)
         assert np.array_equal(got16, want16), f"preset {preset} mip {m} rgba16f"
+
+
+# ---- WriteChannels and the loss statistics of Decompress ------------------------------------------
+
+BPC = {1: 1, 2: 2, 3: 2, 4: 4, 5: 4}
+
+
+def random_user_image(rng, fmt, width, height, channels, pad):
+    """Pitch-linear user image in channel format fmt; returns (bytes, float32 values [h, w, c])."""
+    if fmt == 1:
+        raw = rng.integers(0, 256, (height, width, channels)).astype(np.uint8)
+        vals = (raw.astype(np.float32) / np.float32(255.0)).astype(np.float32)
+    elif fmt == 2:
+        raw = rng.integers(0, 65536, (height, width, channels)).astype(np.uint16)
+        vals = (raw.astype(np.float32) / np.float32(65535.0)).astype(np.float32)
+    elif fmt == 3:
+        raw = (rng.standard_normal((height, width, channels)) * 50).astype(np.float16)
+        vals = raw.astype(np.float32)
+    elif fmt == 4:
+        raw = (rng.standard_normal((height, width, channels)) * 3).astype(np.float32)
+        raw.reshape(-1)[:4] = [1e9, -1e9, 65519.9, 1e-9]                      # saturate, not overflow to Inf
+        vals = raw
+    else:
+        raw = rng.integers(0, 70000, (height, width, channels)).astype(np.uint32)
+        vals = raw.astype(np.float32)
+    stride = channels * BPC[fmt]
+    pitch = width * stride + pad
+    img = np.full(height * pitch, 0x5A, dtype=np.uint8)
+    for y in range(height):
+        img[y * pitch: y * pitch + width * stride] = np.ascontiguousarray(raw[y]).view(np.uint8).reshape(-1)
+    return img, vals, stride, pitch
+
+
+def np_write_channels(planar, vals, set_channels, first, flip):
+    """numpy model: clamp to the finite half range, round to half (nearest even), planar pairs."""
+    h, w, n = vals.shape
+    img = planar.reshape(h, set_channels // 2, w, 2)
+    src = vals[::-1] if flip else vals
+    halves = np.clip(src, -65504.0, 65504.0).astype(np.float32).astype(np.float16).view(np.uint16)
+    for ch in range(n):
+        c = first + ch
+        img[:, c // 2, :, c % 2] = halves[:, :, ch]
+
+
+@pytest.mark.parametrize("fmt", [1, 2, 3, 4, 5])
+def test_checker_write_channels_against_numpy(oracle, fmt):
+    rng = np.random.default_rng(40 + fmt)
+    w, h, C_ = 29, 7, 8
+    for first, count, flip in ((0, 8, 0), (3, 4, 1), (7, 1, 0)):
+        img, vals, stride, pitch = random_user_image(rng, fmt, w, h, count, 6 * BPC[fmt])
+        got = np.full(w * h * C_, 0x1234, dtype=np.uint16)
+        want = got.copy()
+        assert oracle.ntc_oracle_write_channels(img.ctypes.data, fmt, flip, stride, pitch, got.ctypes.data, w, h, C_, first, count) == 0
+        np_write_channels(want, vals, C_, first, flip)
+        assert np.array_equal(got, want), (fmt, first, count, flip)
+
+
+def np_image_loss(a, b, width, height, set_channels, mask):
+    fa = a.view(np.float16).astype(np.float64).reshape(height, set_channels // 2, width, 2)
+    fb = b.view(np.float16).astype(np.float64).reshape(height, set_channels // 2, width, 2)
+    out = np.zeros(16)
+    for c in range(set_channels):
+        if mask >> c & 1:
+            out[c] = np.mean((fa[:, c // 2, :, c % 2] - fb[:, c // 2, :, c % 2]) ** 2)
+    return out
+
+
+def test_checker_image_loss_against_numpy(oracle):
+    rng = np.random.default_rng(50)
+    w, h, C_ = 61, 13, 10
+    a = (rng.random(w * h * C_)).astype(np.float16).view(np.uint16)
+    b = (rng.random(w * h * C_)).astype(np.float16).view(np.uint16)
+    for mask in (0x3FF, 0x155, 0x200, 0):
+        got = np.zeros(16, dtype=np.float64)
+        oracle.ntc_oracle_image_loss(a.ctypes.data, b.ctypes.data, w, h, C_, mask, got.ctypes.data)
+        assert np.allclose(got, np_image_loss(a, b, w, h, C_, mask), rtol=1e-12, atol=0)
+        assert all(got[c] == 0 for c in range(16) if not mask >> c & 1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fmt", [1, 2, 3, 4, 5])
+def test_gpu_write_channels_all_formats(ntc, device, oracle, fmt):
+    rng = np.random.default_rng(60 + fmt)
+    w, h, C_ = 203, 31, 16
+    for first, count, flip in ((0, 16, 0), (5, 3, 1), (15, 1, 0), (2, 7, 1)):
+        img, _, stride, pitch = random_user_image(rng, fmt, w, h, count, 4 * BPC[fmt])
+        start = np.full(w * h * C_, 0x1234, dtype=np.uint16)
+        d_src, d_dst = device.upload(img), device.upload(start)
+        wc = ntc.abi.WriteChannels()
+        wc.src, wc.srcBytes, wc.format, wc.verticalFlip, wc.pixelStride, wc.rowPitch = d_src.ptr, d_src.nbytes, fmt, flip, stride, pitch
+        wc.planarPairs, wc.planarBytes = d_dst.ptr, d_dst.nbytes
+        wc.width, wc.height, wc.setChannels, wc.firstChannel, wc.numChannels = w, h, C_, first, count
+        ntc.abi.check(device.lib.ntc_hip_write_channels(wc))
+        device.synchronize()
+        want = start.copy()
+        assert oracle.ntc_oracle_write_channels(img.ctypes.data, fmt, flip, stride, pitch, want.ctypes.data, w, h, C_, first, count) == 0
+        assert np.array_equal(d_dst.download().view(np.uint16), want), (fmt, first, count, flip)
+    # a source image shorter than height * rowPitch is refused before any launch
+    wc.srcBytes = h * pitch - pitch
+    assert device.lib.ntc_hip_write_channels(wc) == ntc.abi.ERR_INVALID_ARG
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(1, 1, 2), (67, 5, 6), (512, 300, 16), (2048, 2048, 12)])
+def test_gpu_image_loss_against_checker(ntc, device, oracle, shape):
+    w, h, C_ = shape
+    rng = np.random.default_rng(w)
+    a = rng.random(w * h * C_).astype(np.float16).view(np.uint16)
+    b = (a.view(np.float16).astype(np.float32) + rng.standard_normal(w * h * C_).astype(np.float32) * 0.05).astype(np.float16).view(np.uint16)
+    d_a, d_b = device.upload(a), device.upload(b)
+    for mask in ((1 << C_) - 1, 0x5 & ((1 << C_) - 1), 0):
+        got = (C.c_float * 16)()
+        ntc.abi.check(device.lib.ntc_hip_image_loss(d_a.ptr, d_b.ptr, d_a.nbytes, w, h, C_, mask, got))
+        want = np.zeros(16, dtype=np.float64)
+        oracle.ntc_oracle_image_loss(a.ctypes.data, b.ctypes.data, w, h, C_, mask, want.ctypes.data)
+        # double accumulation on both sides; the result is rounded to float once
+        assert np.allclose(np.array(got[:], dtype=np.float64), want, rtol=2e-7, atol=0), (shape, mask)
+    assert device.lib.ntc_hip_image_loss(d_a.ptr, d_b.ptr, d_a.nbytes - 2, w, h, C_, 1, got) == ntc.abi.ERR_INVALID_ARG
+
+
+def parse_stats(text, tag, mips):
+    lines = {ln.split()[1]: [float(v) for v in ln.split()[2:]] for ln in text.splitlines() if ln.startswith(tag + " ")}
+    return lines["overall"][0], np.array(lines["mips"][:mips]), np.array(lines["channels"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("separate", [0, 1])
+def test_host_layer_loss_statistics(ntc, oracle, tmp_path, separate):
+    """Decompress(&stats) after WriteChannels: per-channel / per-mip / overall MSE combined as
+    src/TextureSet.cpp:1833-1892 does, over the channels the registered textures claim."""
+    w, h, channels = 128, 64, 8
+    mips = ntc.presets.full_mip_count(w, h)
+    case = cfg_case(ntc, ntc.presets.spec_cfg01(), w, h, mips, channels, ntc.abi.OUT_FP16_PLANAR_PAIRS, 91, scale_log2_range=(-17.0, -12.0))
+    lat, wts = tmp_path / "latents.bin", tmp_path / "weights.bin"
+    case.latents.tofile(lat)
+    case.weights.tofile(wts)
+    host = case.host_set()
+    host.decode(threads=8)
+    rng = np.random.default_rng(92)
+    prefix = str(tmp_path / "ref")
+    mask = 0x37                                     # textures on channels 0..2 and 4..5
+    valid = [c for c in range(channels) if mask >> c & 1]
+    mse = np.zeros((mips, 16))
+    pixels = np.array([m.width * m.height for m in case.mips], dtype=np.float64)
+    planes = []
+    for m, mip in enumerate(case.mips):
+        decoded = np.ascontiguousarray(host.output[mip.outOffset: mip.outOffset + mip.width * mip.height * channels * 2].view(np.uint16))
+        ref = rng.random((mip.height, mip.width, channels)).astype(np.float32)
+        ref.tofile(f"{prefix}_mip{m}.bin")
+        ref_planar = np.zeros(mip.width * mip.height * channels, dtype=np.uint16)
+        np_write_channels(ref_planar, ref, channels, 0, False)
+        mse[m] = np_image_loss(decoded, ref_planar, mip.width, mip.height, channels, mask)
+        planes.append((decoded, ref_planar))
+    out = run_exe("loss", 1, w, h, mips, channels, 0, 0, lat, wts, prefix, separate)
+    assert "host loss OK" in out
+    overall, per_mip, per_channel = parse_stats(out, "first", mips)
+    want_mip = mse[:, valid].mean(axis=1)
+    assert np.allclose(per_mip, want_mip, rtol=1e-6)
+    assert np.allclose(per_channel, (mse * pixels[:, None]).sum(axis=0) / pixels.sum(), rtol=1e-6)
+    assert np.isclose(overall, (want_mip * pixels).sum() / pixels.sum(), rtol=1e-6)
+    assert all(per_channel[c] == 0 for c in range(16) if c not in valid)
+    overall2, per_mip2, _ = parse_stats(out, "second", mips)
+    if separate:    # the reference image survives the decode: same numbers again
+        assert overall2 == overall and np.array_equal(per_mip2, per_mip)
+    else:           # shared page: the first decode overwrote the reference image (as in the reference library)
+        assert overall2 == 0 and not per_mip2.any()
+
+    def pixels_of(planar):
+        return planar.reshape(h, channels // 2, w, 2).transpose(0, 2, 1, 3).reshape(-1)
+    decoded0, ref0 = planes[0]
+    page_ref = np.fromfile(prefix + "_page_reference.bin", dtype=np.uint16)
+    page_out = np.fromfile(prefix + "_page_output.bin", dtype=np.uint16)
+    assert np.array_equal(page_out, pixels_of(decoded0))
+    assert np.array_equal(page_ref, pixels_of(ref0 if separate else decoded0))
