@@ -1,0 +1,518 @@
+// NtcFile.cpp - JSON chunk parser of the NTC container.  See NtcFile.h.
+//
+// Two stages: a small strict JSON reader builds a value tree (texts are a few kB), then typed
+// extraction walks the tree member by member with the presence and type rules of the
+// reference's schema tables (src/JsonFileFormat.cpp:25-186): plain scalars are required,
+// optionals and arrays are not, unknown members are ignored, integers must fit their field.
+#include "NtcFile.h"
+
+#include <cinttypes>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <utility>
+
+namespace ntc::file
+{
+namespace
+{
+
+struct Value
+{
+    enum Kind { Null, Bool, Integer, Real, String, Array, Object };
+    Kind kind = Null;
+    bool boolean = false;
+    bool negative = false;          // Integer: sign, magnitude below
+    uint64_t magnitude = 0;
+    double real = 0.0;
+    std::string text;
+    std::vector<Value> items;
+    std::vector<std::pair<std::string, Value>> members;
+
+    Value const* Find(char const* name) const
+    {
+        Value const* found = nullptr;       // the last of duplicate keys wins, as with a streaming reader
+        for (auto const& m : members) if (m.first == name) found = &m.second;
+        return found;
+    }
+};
+
+char const* KindName(Value::Kind k)
+{
+    switch (k) {
+    case Value::Null: return "null";
+    case Value::Bool: return "bool";
+    case Value::Integer: return "integer";
+    case Value::Real: return "double";
+    case Value::String: return "string";
+    case Value::Array: return "array";
+    default: return "object";
+    }
+}
+
+class Reader
+{
+public:
+    Reader(char const* text, size_t length, std::string& error) : m_p(text), m_end(text + length), m_begin(text), m_error(error) {}
+
+    bool ParseRoot(Value& out)
+    {
+        SkipSpace();
+        if (m_p == m_end) return Fail("The document is empty.");
+        if (!ParseValue(out, 0)) return false;
+        SkipSpace();
+        if (m_p != m_end && *m_p != 0) return Fail("The document root must not be followed by other values.");
+        return true;
+    }
+
+private:
+    static constexpr int kMaxDepth = 32;
+
+    bool Fail(char const* what)
+    {
+        char snippet[32];
+        size_t const left = size_t(m_end - m_p);
+        size_t const n = left < 28 ? left : 28;
+        std::memcpy(snippet, m_p, n);
+        snippet[n] = 0;
+        char buf[256];
+        std::snprintf(buf, sizeof buf, "Error at character %zu (%s%s): %s", size_t(m_p - m_begin), snippet, left > n ? "..." : "", what);
+        m_error = buf;
+        return false;
+    }
+    void SkipSpace() { while (m_p != m_end && (*m_p == ' ' || *m_p == '\t' || *m_p == '\n' || *m_p == '\r')) ++m_p; }
+    bool Literal(char const* word)
+    {
+        size_t const n = std::strlen(word);
+        if (size_t(m_end - m_p) < n || std::memcmp(m_p, word, n) != 0) return Fail("Invalid value.");
+        m_p += n;
+        return true;
+    }
+
+    bool ParseValue(Value& out, int depth)
+    {
+        if (depth > kMaxDepth) return Fail("The document is nested too deeply.");
+        if (m_p == m_end) return Fail("Invalid value.");
+        switch (*m_p) {
+        case '{': return ParseObject(out, depth);
+        case '[': return ParseArray(out, depth);
+        case '"': out.kind = Value::String; return ParseString(out.text);
+        case 't': out.kind = Value::Bool; out.boolean = true; return Literal("true");
+        case 'f': out.kind = Value::Bool; out.boolean = false; return Literal("false");
+        case 'n': out.kind = Value::Null; return Literal("null");
+        default: return ParseNumber(out);
+        }
+    }
+
+    bool ParseObject(Value& out, int depth)
+    {
+        out.kind = Value::Object;
+        ++m_p;
+        SkipSpace();
+        if (m_p != m_end && *m_p == '}') { ++m_p; return true; }
+        for (;;) {
+            SkipSpace();
+            if (m_p == m_end || *m_p != '"') return Fail("Missing a name for object member.");
+            std::string key;
+            if (!ParseString(key)) return false;
+            SkipSpace();
+            if (m_p == m_end || *m_p != ':') return Fail("Missing a colon after a name of object member.");
+            ++m_p;
+            SkipSpace();
+            out.members.emplace_back(std::move(key), Value());
+            if (!ParseValue(out.members.back().second, depth + 1)) return false;
+            SkipSpace();
+            if (m_p != m_end && *m_p == ',') { ++m_p; continue; }
+            if (m_p != m_end && *m_p == '}') { ++m_p; return true; }
+            return Fail("Missing a comma or '}' after an object member.");
+        }
+    }
+
+    bool ParseArray(Value& out, int depth)
+    {
+        out.kind = Value::Array;
+        ++m_p;
+        SkipSpace();
+        if (m_p != m_end && *m_p == ']') { ++m_p; return true; }
+        for (;;) {
+            SkipSpace();
+            out.items.emplace_back();
+            if (!ParseValue(out.items.back(), depth + 1)) return false;
+            SkipSpace();
+            if (m_p != m_end && *m_p == ',') { ++m_p; continue; }
+            if (m_p != m_end && *m_p == ']') { ++m_p; return true; }
+            return Fail("Missing a comma or ']' after an array element.");
+        }
+    }
+
+    static void AppendUtf8(std::string& s, uint32_t cp)
+    {
+        if (cp < 0x80) s += char(cp);
+        else if (cp < 0x800) { s += char(0xC0 | (cp >> 6)); s += char(0x80 | (cp & 0x3F)); }
+        else if (cp < 0x10000) { s += char(0xE0 | (cp >> 12)); s += char(0x80 | ((cp >> 6) & 0x3F)); s += char(0x80 | (cp & 0x3F)); }
+        else { s += char(0xF0 | (cp >> 18)); s += char(0x80 | ((cp >> 12) & 0x3F)); s += char(0x80 | ((cp >> 6) & 0x3F)); s += char(0x80 | (cp & 0x3F)); }
+    }
+    bool Hex4(uint32_t& out)
+    {
+        if (m_end - m_p < 4) return Fail("Incorrect hex digit after \\u escape in string.");
+        out = 0;
+        for (int i = 0; i < 4; ++i) {
+            char const c = *m_p++;
+            out <<= 4;
+            if (c >= '0' && c <= '9') out |= uint32_t(c - '0');
+            else if (c >= 'a' && c <= 'f') out |= uint32_t(c - 'a' + 10);
+            else if (c >= 'A' && c <= 'F') out |= uint32_t(c - 'A' + 10);
+            else { --m_p; return Fail("Incorrect hex digit after \\u escape in string."); }
+        }
+        return true;
+    }
+
+    bool ParseString(std::string& out)
+    {
+        ++m_p;      // opening quote
+        for (;;) {
+            if (m_p == m_end) return Fail("Missing a closing quotation mark in string.");
+            unsigned char const c = static_cast<unsigned char>(*m_p);
+            if (c == '"') { ++m_p; return true; }
+            if (c < 0x20) return Fail("Invalid encoding in string.");
+            if (c != '\\') { out += char(c); ++m_p; continue; }
+            ++m_p;
+            if (m_p == m_end) return Fail("Invalid escape character in string.");
+            char const e = *m_p++;
+            switch (e) {
+            case '"': out += '"'; break;
+            case '\\': out += '\\'; break;
+            case '/': out += '/'; break;
+            case 'b': out += '\b'; break;
+            case 'f': out += '\f'; break;
+            case 'n': out += '\n'; break;
+            case 'r': out += '\r'; break;
+            case 't': out += '\t'; break;
+            case 'u': {
+                uint32_t cp = 0;
+                if (!Hex4(cp)) return false;
+                if (cp >= 0xD800 && cp <= 0xDBFF) {
+                    uint32_t low = 0;
+                    if (m_end - m_p < 2 || m_p[0] != '\\' || m_p[1] != 'u') return Fail("The surrogate pair in string is invalid.");
+                    m_p += 2;
+                    if (!Hex4(low)) return false;
+                    if (low < 0xDC00 || low > 0xDFFF) return Fail("The surrogate pair in string is invalid.");
+                    cp = 0x10000 + ((cp - 0xD800) << 10) + (low - 0xDC00);
+                } else if (cp >= 0xDC00 && cp <= 0xDFFF) {
+                    return Fail("The surrogate pair in string is invalid.");
+                }
+                AppendUtf8(out, cp);
+                break;
+            }
+            default: --m_p; return Fail("Invalid escape character in string.");
+            }
+        }
+    }
+
+    bool ParseNumber(Value& out)
+    {
+        char const* const start = m_p;
+        bool negative = false;
+        if (m_p != m_end && *m_p == '-') { negative = true; ++m_p; }
+        if (m_p == m_end || *m_p < '0' || *m_p > '9') { m_p = start; return Fail("Invalid value."); }
+        uint64_t magnitude = 0;
+        bool overflow = false;
+        if (*m_p == '0') ++m_p;
+        else while (m_p != m_end && *m_p >= '0' && *m_p <= '9') {
+            uint64_t const digit = uint64_t(*m_p - '0');
+            if (magnitude > (UINT64_MAX - digit) / 10) overflow = true;
+            else magnitude = magnitude * 10 + digit;
+            ++m_p;
+        }
+        bool real = false;
+        if (m_p != m_end && *m_p == '.') {
+            real = true;
+            ++m_p;
+            if (m_p == m_end || *m_p < '0' || *m_p > '9') return Fail("Miss fraction part in number.");
+            while (m_p != m_end && *m_p >= '0' && *m_p <= '9') ++m_p;
+        }
+        if (m_p != m_end && (*m_p == 'e' || *m_p == 'E')) {
+            real = true;
+            ++m_p;
+            if (m_p != m_end && (*m_p == '+' || *m_p == '-')) ++m_p;
+            if (m_p == m_end || *m_p < '0' || *m_p > '9') return Fail("Miss exponent in number.");
+            while (m_p != m_end && *m_p >= '0' && *m_p <= '9') ++m_p;
+        }
+        if (real || overflow || (negative && magnitude > uint64_t(INT64_MAX) + 1)) {
+            std::string const token(start, size_t(m_p - start));
+            out.kind = Value::Real;
+            out.real = std::strtod(token.c_str(), nullptr);
+            if (!std::isfinite(out.real)) { m_p = start; return Fail("Number too big to be stored in double."); }
+            return true;
+        }
+        out.kind = Value::Integer;
+        out.negative = negative && magnitude != 0;
+        out.magnitude = magnitude;
+        return true;
+    }
+
+    char const* m_p;
+    char const* m_end;
+    char const* m_begin;
+    std::string& m_error;
+};
+
+// Typed access to the members of one JSON object of schema type `typeName`.
+class Members
+{
+public:
+    Members(Value const& object, char const* typeName, std::string& error) : m_object(object), m_type(typeName), m_error(error) {}
+
+    bool UInt(char const* name, uint32_t& out) { return Required(name) && AsUnsigned(name, *m_found, UINT32_MAX, "uint", [&](uint64_t v) { out = uint32_t(v); }); }
+    bool UInt64(char const* name, uint64_t& out) { return Required(name) && AsUnsigned(name, *m_found, uint64_t(INT64_MAX), "uint64", [&](uint64_t v) { out = v; }); }
+    bool OptionalUInt(char const* name, std::optional<uint32_t>& out)
+    {
+        if (!Optional(name)) return true;
+        return AsUnsigned(name, *m_found, UINT32_MAX, "uint", [&](uint64_t v) { out = uint32_t(v); });
+    }
+    bool OptionalUInt64(char const* name, std::optional<uint64_t>& out)
+    {
+        if (!Optional(name)) return true;
+        return AsUnsigned(name, *m_found, uint64_t(INT64_MAX), "uint64", [&](uint64_t v) { out = v; });
+    }
+    bool OptionalFloat(char const* name, std::optional<float>& out)
+    {
+        if (!Optional(name)) return true;
+        Value const& v = *m_found;
+        if (v.kind == Value::Real) { out = float(v.real); return true; }
+        if (v.kind == Value::Integer) { out = v.negative ? -float(v.magnitude) : float(v.magnitude); return true; }
+        return WrongType(name, "float", v);
+    }
+    bool String(char const* name, std::string& out)
+    {
+        if (!Required(name)) return false;
+        if (m_found->kind != Value::String) return WrongType(name, "string", *m_found);
+        out = m_found->text;
+        return true;
+    }
+    // names[i] is the spelling of enum value i
+    template <typename E> bool Enum(char const* name, E& out, std::initializer_list<char const*> names)
+    {
+        if (!Required(name)) return false;
+        int index;
+        if (!AsEnum(name, *m_found, names, index)) return false;
+        out = E(index);
+        return true;
+    }
+    template <typename E> bool OptionalEnum(char const* name, std::optional<E>& out, std::initializer_list<char const*> names)
+    {
+        if (!Optional(name)) return true;
+        int index;
+        if (!AsEnum(name, *m_found, names, index)) return false;
+        out = E(index);
+        return true;
+    }
+    // Arrays are never required (src/JsonSerialization.h:262-282); returns null when absent.
+    bool Array(char const* name, char const* expected, Value const*& out)
+    {
+        out = nullptr;
+        if (!Optional(name)) return true;
+        if (m_found->kind != Value::Array) return WrongType(name, expected, *m_found);
+        out = m_found;
+        return true;
+    }
+    bool OptionalObject(char const* name, Value const*& out)
+    {
+        out = nullptr;
+        if (!Optional(name)) return true;
+        if (m_found->kind != Value::Object) return WrongType(name, "object", *m_found);
+        out = m_found;
+        return true;
+    }
+    bool ArrayOfUInt(char const* name, std::vector<uint32_t>& out)
+    {
+        Value const* array;
+        if (!Array(name, "uint", array)) return false;
+        if (array) for (Value const& item : array->items)
+            if (!AsUnsigned(name, item, UINT32_MAX, "uint", [&](uint64_t v) { out.push_back(uint32_t(v)); })) return false;
+        return true;
+    }
+    bool ElementMustBeObject(char const* name, Value const& item) { return item.kind == Value::Object ? true : WrongType(name, "array", item); }
+
+private:
+    bool Optional(char const* name) { m_found = m_object.Find(name); return m_found != nullptr; }
+    bool Required(char const* name)
+    {
+        if (Optional(name)) return true;
+        Format("Missing value for required field '%s.%s'", m_type, name);
+        return false;
+    }
+    bool WrongType(char const* name, char const* expected, Value const& v)
+    {
+        Format("Expected %s for '%s.%s', got %s", expected, m_type, name, KindName(v.kind));
+        return false;
+    }
+    template <typename Store> bool AsUnsigned(char const* name, Value const& v, uint64_t limit, char const* expected, Store store)
+    {
+        if (v.kind != Value::Integer) return WrongType(name, expected, v);
+        if (v.negative || v.magnitude > limit) {
+            char buf[256];
+            std::snprintf(buf, sizeof buf, "Value %s%" PRIu64 " is out of range for %s field '%s.%s'", v.negative ? "-" : "", v.magnitude, expected, m_type, name);
+            m_error = buf;
+            return false;
+        }
+        store(v.magnitude);
+        return true;
+    }
+    bool AsEnum(char const* name, Value const& v, std::initializer_list<char const*> names, int& index)
+    {
+        if (v.kind != Value::String) return WrongType(name, "enum", v);
+        index = 0;
+        for (char const* candidate : names) {
+            if (v.text == candidate) return true;
+            ++index;
+        }
+        Format("Unknown value '%s' specified for '%s.%s'", v.text.c_str(), m_type, name);
+        return false;
+    }
+    void Format(char const* fmt, char const* a, char const* b, char const* c = nullptr, char const* d = nullptr)
+    {
+        char buf[320];
+        std::snprintf(buf, sizeof buf, fmt, a, b, c, d);
+        m_error = buf;
+    }
+
+    Value const& m_object;
+    char const* m_type;
+    std::string& m_error;
+    Value const* m_found = nullptr;
+};
+
+// spellings in the order of the enums (src/JsonFileFormat.cpp:25-113)
+#define NTC_FILE_MLP_TYPES { "Int8", "Int32", "FloatE4M3", "FloatE5M2", "Float16", "Float32" }
+#define NTC_FILE_CHANNEL_FORMATS { "UNKNOWN", "UNORM8", "UNORM16", "FLOAT16", "FLOAT32", "UINT32" }
+#define NTC_FILE_COLOR_SPACES { "Linear", "sRGB", "HLG" }
+#define NTC_FILE_BC_FORMATS { "None", "BC1", "BC2", "BC3", "BC4", "BC5", "BC6", "BC7" }
+
+bool ReadView(Value const& v, BufferView& out, std::string& error)
+{
+    Members m(v, "BufferView", error);
+    return m.UInt64("offset", out.offset) && m.UInt64("storedSize", out.storedSize)
+        && m.OptionalEnum("compression", out.compression, { "None", "GDeflate" })
+        && m.OptionalUInt64("uncompressedSize", out.uncompressedSize) && m.OptionalUInt("crc32", out.crc32);
+}
+
+bool ReadLayer(Value const& v, MlpLayer& out, std::string& error)
+{
+    Members m(v, "MLPLayer", error);
+    return m.UInt("inputChannels", out.inputChannels) && m.UInt("outputChannels", out.outputChannels)
+        && m.UInt("weightView", out.weightView) && m.OptionalUInt("scaleView", out.scaleView) && m.UInt("biasView", out.biasView)
+        && m.Enum("weightType", out.weightType, NTC_FILE_MLP_TYPES)
+        && m.OptionalEnum("scaleType", out.scaleType, NTC_FILE_MLP_TYPES)
+        && m.Enum("biasType", out.biasType, NTC_FILE_MLP_TYPES);
+}
+
+bool ReadMlp(Value const& v, Mlp& out, std::string& error)
+{
+    Members m(v, "MLP", error);
+    Value const* layers;
+    if (!m.Array("layers", "array", layers)) return false;
+    if (layers) for (Value const& item : layers->items) {
+        if (!m.ElementMustBeObject("layers", item)) return false;
+        out.layers.emplace_back();
+        if (!ReadLayer(item, out.layers.back(), error)) return false;
+    }
+    std::optional<int> activation;
+    return m.OptionalEnum("activation", activation, { "HGELUClamp" })
+        && m.OptionalEnum("weightLayout", out.weightLayout, { "RowMajor", "ColumnMajor" });
+}
+
+bool ReadTexture(Value const& v, Texture& out, std::string& error)
+{
+    Members m(v, "Texture", error);
+    Value const* modeBuffers;
+    if (!(m.String("name", out.name) && m.UInt("firstChannel", out.firstChannel) && m.UInt("numChannels", out.numChannels)
+        && m.OptionalEnum("channelFormat", out.channelFormat, NTC_FILE_CHANNEL_FORMATS)
+        && m.OptionalEnum("rgbColorSpace", out.rgbColorSpace, NTC_FILE_COLOR_SPACES)
+        && m.OptionalEnum("alphaColorSpace", out.alphaColorSpace, NTC_FILE_COLOR_SPACES)
+        && m.OptionalEnum("bcFormat", out.bcFormat, NTC_FILE_BC_FORMATS)
+        && m.Array("bcModeBuffers", "array", modeBuffers)))
+        return false;
+    // BC7 mode buffers belong to the block-compression step after decoding; their entries are
+    // checked for shape and otherwise left alone.
+    if (modeBuffers) for (Value const& item : modeBuffers->items) {
+        if (!m.ElementMustBeObject("bcModeBuffers", item)) return false;
+        Members b(item, "BCModeBuffer", error);
+        uint32_t mipLevel, view;
+        if (!(b.UInt("mipLevel", mipLevel) && b.UInt("view", view))) return false;
+    }
+    return true;
+}
+
+bool ReadColorMip(Value const& v, ColorMip& out, std::string& error)
+{
+    Members m(v, "ColorMip", error);
+    return m.OptionalUInt("width", out.width) && m.OptionalUInt("height", out.height) && m.OptionalUInt("latentMip", out.latentMip)
+        && m.OptionalFloat("positionLod", out.positionLod) && m.OptionalFloat("positionScale", out.positionScale);
+}
+
+template <typename T, typename ReadOne>
+bool ReadObjectArray(Members& parent, char const* name, std::vector<T>& out, ReadOne readOne)
+{
+    Value const* array;
+    if (!parent.Array(name, "array", array)) return false;
+    if (array) for (Value const& item : array->items) {
+        if (!parent.ElementMustBeObject(name, item)) return false;
+        out.emplace_back();
+        if (!readOne(item, out.back())) return false;
+    }
+    return true;
+}
+
+} // namespace
+
+bool ParseDocument(char const* json, size_t length, Document& out, std::string& error)
+{
+    Value root;
+    Reader reader(json, length, error);
+    if (!reader.ParseRoot(root)) return false;
+    if (root.kind != Value::Object) { error = std::string("Expected object, got ") + KindName(root.kind); return false; }
+
+    Members m(root, "Document", error);
+    if (!m.UInt("schemaVersion", out.schemaVersion)) return false;
+    if (out.schemaVersion != kSchemaVersion) {      // src/JsonFileFormat.cpp:194-210
+        char buf[128];
+        std::snprintf(buf, sizeof buf, "Incompatible file schema version %u, expected %u", out.schemaVersion, kSchemaVersion);
+        error = buf;
+        return false;
+    }
+    if (!(m.UInt("width", out.width) && m.UInt("height", out.height) && m.UInt("numChannels", out.numChannels)
+        && m.OptionalUInt("numColorMips", out.numColorMips)))
+        return false;
+    Value const* latentShape;
+    if (!m.OptionalObject("latentShape", latentShape)) return false;
+    if (latentShape) {
+        Members s(*latentShape, "LatentShape", error);
+        uint32_t features;
+        if (!s.UInt("numFeatures", features)) return false;
+        out.latentFeatures = features;
+    }
+    return ReadObjectArray(m, "mlpVersions", out.mlpVersions, [&](Value const& v, Mlp& o) { return ReadMlp(v, o, error); })
+        && ReadObjectArray(m, "textures", out.textures, [&](Value const& v, Texture& o) { return ReadTexture(v, o, error); })
+        && ReadObjectArray(m, "channels", out.channelColorSpaces, [&](Value const& v, std::optional<int>& o) {
+               Members c(v, "Channel", error);
+               return c.OptionalEnum("colorSpace", o, NTC_FILE_COLOR_SPACES); })
+        && ReadObjectArray(m, "latents", out.latents, [&](Value const& v, LatentImage& o) {
+               Members l(v, "LatentImage", error);
+               return l.UInt("width", o.width) && l.UInt("height", o.height) && l.ArrayOfUInt("layerViews", o.layerViews); })
+        && ReadObjectArray(m, "colorMips", out.colorMips, [&](Value const& v, ColorMip& o) { return ReadColorMip(v, o, error); })
+        && ReadObjectArray(m, "views", out.views, [&](Value const& v, BufferView& o) { return ReadView(v, o, error); });
+}
+
+Header DecodeHeader(unsigned char const* b)
+{
+    auto u32 = [&](int at) { return uint32_t(b[at]) | uint32_t(b[at + 1]) << 8 | uint32_t(b[at + 2]) << 16 | uint32_t(b[at + 3]) << 24; };
+    auto u64 = [&](int at) { return uint64_t(u32(at)) | uint64_t(u32(at + 4)) << 32; };
+    Header h;
+    h.signature = u32(0); h.version = u32(4);
+    h.jsonChunkOffset = u64(8); h.jsonChunkSize = u64(16); h.binaryChunkOffset = u64(24); h.binaryChunkSize = u64(32);
+    return h;
+}
+
+} // namespace ntc::file

@@ -2,11 +2,14 @@
 //
 // Counterpart of the parts of reference src/Context.cpp, src/TextureSet.cpp,
 // src/FeatureGridHost.cpp, src/FeatureGridMath.cpp and src/Errors.cpp that the decompression
-// path goes through.  All device work is done by libntc_hip.so through include/ntc_hip.h.
+// path goes through, src/TextureSetMetadata.cpp for loading NTC files and src/Stream.cpp.  All device work is done by libntc_hip.so through include/ntc_hip.h.
 #include "ntc_decode.h"
+#include "NtcFile.h"
 #include "../../include/ntc_hip.h"
 
 #include <algorithm>
+#include <cerrno>
+#include <cinttypes>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -84,6 +87,66 @@ NtcHipDecoderSpec MakeSpec(DecoderPreset preset, int numFeatures)
     return s;
 }
 
+// Neural-LOD geometry, src/FeatureGridMath.cpp:47-77.
+int SharedMipCount(int gridSizeScale) { static int const table[] = { 2, 3, 3, 3, 4, 4 }; return table[gridSizeScale - 1]; }
+int LodToNeuralLod(int lod, int gridSizeScale, int neuralLods) { return std::max(0, std::min((lod - SharedMipCount(gridSizeScale) + 2) & ~1, neuralLods - 2)); }
+int GridDimension(int imageDimension, int neuralLod, int gridSizeScale) { return std::max((imageDimension / gridSizeScale) >> neuralLod, 1); }
+int NeuralLodCount(int width, int height, int mips, int gridSizeScale)      // with src/FeatureGridHost.cpp:27-58
+{
+    int const minGrid = int(float(std::min(width, height)) / float(gridSizeScale));
+    int const byGridSize = std::max(2, int(1.f + std::floor(std::log2(float(minGrid))))) & ~1;
+    return std::min(byGridSize, LodToNeuralLod(mips - 1, gridSizeScale, 8) + 2);
+}
+
+// src/Stream.cpp:27-121
+class FileStream final : public IStream
+{
+public:
+    explicit FileStream(FILE* file) : m_file(file) {}
+    ~FileStream() override { if (m_file) std::fclose(m_file); }
+    bool Read(void* dst, size_t size) override { return size == 0 || std::fread(dst, size, 1, m_file) == 1; }
+    bool Write(const void* src, size_t size) override { return size == 0 || std::fwrite(src, size, 1, m_file) == 1; }
+    bool Seek(uint64_t offset) override { return fseeko(m_file, off_t(offset), SEEK_SET) == 0; }
+    uint64_t Tell() override { return uint64_t(ftello(m_file)); }
+    uint64_t Size() override
+    {
+        off_t const current = ftello(m_file);
+        fseeko(m_file, 0, SEEK_END);
+        off_t const size = ftello(m_file);
+        fseeko(m_file, current, SEEK_SET);
+        return uint64_t(size);
+    }
+private:
+    FILE* m_file;
+};
+
+class MemoryStream final : public IStream
+{
+public:
+    MemoryStream(uint8_t* data, size_t size, bool readonly) : m_data(data), m_size(size), m_readonly(readonly) {}
+    bool Read(void* dst, size_t size) override
+    {
+        if (size > m_size - m_at) return false;
+        std::memcpy(dst, m_data + m_at, size);
+        m_at += size;
+        return true;
+    }
+    bool Write(const void* src, size_t size) override
+    {
+        if (m_readonly || size > m_size - m_at) return false;
+        std::memcpy(m_data + m_at, src, size);
+        m_at += size;
+        return true;
+    }
+    bool Seek(uint64_t offset) override { if (offset >= m_size) return false; m_at = size_t(offset); return true; }
+    uint64_t Tell() override { return m_at; }
+    uint64_t Size() override { return m_size; }
+private:
+    uint8_t* m_data;
+    size_t m_size, m_at = 0;
+    bool m_readonly;
+};
+
 // positionScale / positionLod of a colour mip, src/TextureSet.cpp:456-461
 void PositionConstants(NtcHipMipDesc& d)
 {
@@ -118,11 +181,112 @@ public:
         return Status::Ok;
     }
     void GetChannels(int& outFirstChannel, int& outNumChannels) const override { outFirstChannel = m_firstChannel; outNumChannels = m_numChannels; }
+    int GetFirstChannel() const override { return m_firstChannel; }
+    int GetNumChannels() const override { return m_numChannels; }
+    void SetChannelFormat(ChannelFormat format) override { m_channelFormat = format; }
+    ChannelFormat GetChannelFormat() const override { return m_channelFormat; }
+    void SetBlockCompressedFormat(BlockCompressedFormat format) override { m_bcFormat = format; }
+    BlockCompressedFormat GetBlockCompressedFormat() const override { return m_bcFormat; }
+    void SetRgbColorSpace(ColorSpace colorSpace) override { m_rgbColorSpace = colorSpace; }
+    ColorSpace GetRgbColorSpace() const override { return m_rgbColorSpace; }
+    void SetAlphaColorSpace(ColorSpace colorSpace) override { m_alphaColorSpace = colorSpace; }
+    ColorSpace GetAlphaColorSpace() const override { return m_alphaColorSpace; }
 private:
     TextureSetDesc const& m_setDesc;
     std::string m_name;
     int m_firstChannel = 0, m_numChannels = 0;
+    ChannelFormat m_channelFormat = ChannelFormat::UNORM8;
+    BlockCompressedFormat m_bcFormat = BlockCompressedFormat::None;
+    ColorSpace m_rgbColorSpace = ColorSpace::Linear, m_alphaColorSpace = ColorSpace::Linear;
 };
+
+// Header + JSON chunk of an NTC file (src/TextureSetMetadata.cpp:1210-1264).
+Status LoadFileHeadersFromStream(IStream* stream, file::Document& document, uint64_t& binaryChunkOffset, uint64_t& binaryChunkSize)
+{
+    unsigned char raw[40];
+    if (!stream->Read(raw, sizeof raw)) {
+        SetErrorMessage("Failed to read the file header - file smaller than %zu bytes?", sizeof raw);
+        return Status::IOError;
+    }
+    file::Header const header = file::DecodeHeader(raw);
+    if (header.signature != file::kSignature) { SetErrorMessage("Unrecognized file format."); return Status::FileUnrecognized; }
+    if (header.version != file::kContainerVersion) {
+        SetErrorMessage("Incompatible file format version: expected %d, got %d.", int(file::kContainerVersion), int(header.version));
+        return Status::FileUnrecognized;
+    }
+    uint64_t const streamSize = stream->Size();
+    uint64_t const expected = std::max(header.jsonChunkOffset + header.jsonChunkSize, header.binaryChunkOffset + header.binaryChunkSize);
+    bool const wraps = header.jsonChunkOffset + header.jsonChunkSize < header.jsonChunkOffset
+                    || header.binaryChunkOffset + header.binaryChunkSize < header.binaryChunkOffset;
+    if (wraps || streamSize < expected) {
+        SetErrorMessage("File incomplete: expected at least %" PRIu64 " bytes, actual size %" PRIu64 " bytes.", expected, streamSize);
+        return Status::FileUnrecognized;
+    }
+    if (!stream->Seek(header.jsonChunkOffset)) return Status::IOError;
+    std::vector<char> json(size_t(header.jsonChunkSize) + 1, 0);
+    if (!stream->Read(json.data(), size_t(header.jsonChunkSize))) return Status::IOError;
+    std::string error;
+    if (!file::ParseDocument(json.data(), std::strlen(json.data()), document, error)) {
+        SetErrorMessage("%s", error.c_str());
+        return Status::FileUnrecognized;
+    }
+    binaryChunkOffset = header.binaryChunkOffset;
+    binaryChunkSize = header.binaryChunkSize;
+    return Status::Ok;
+}
+
+Status ValidateLatentShape(LatentShape const& shape)        // src/TextureSetMetadata.cpp:1137-1159
+{
+    if (shape.IsEmpty()) return Status::Ok;
+    if (shape.numFeatures <= 0 || shape.numFeatures > 16 || (shape.numFeatures % 4) != 0) {
+        SetErrorMessage("Invalid LatentShape: numFeatures (%d) must be a positive multiple of %d up to %d.", shape.numFeatures, 4, 16);
+        return Status::OutOfRange;
+    }
+    if (shape.gridSizeScale < 1 || shape.gridSizeScale > 6) {
+        SetErrorMessage("Invalid LatentShape: gridSizeScale (%d) must be between 1 and 6.", shape.gridSizeScale);
+        return Status::OutOfRange;
+    }
+    return Status::Ok;
+}
+
+Status ValidateTextureSetDesc(TextureSetDesc const& desc)   // src/TextureSetMetadata.cpp:1161-1178
+{
+    if (desc.width <= 0 || desc.height <= 0 || desc.channels <= 0 || desc.mips <= 0) {
+        SetErrorMessage("Invalid TextureSetDesc: width (%d), height (%d), channels (%d) and mips (%d) "
+            "must be positive numbers.", desc.width, desc.height, desc.channels, desc.mips);
+        return Status::OutOfRange;
+    }
+    if (desc.channels > NTC_HIP_MAX_CHANNELS) {
+        SetErrorMessage("Invalid TextureSetDesc: too many channels (%d). Only up to %d channels are supported.", desc.channels, NTC_HIP_MAX_CHANNELS);
+        return Status::OutOfRange;
+    }
+    if (desc.mips > NTC_HIP_MAX_MIPS) {
+        SetErrorMessage("Invalid TextureSetDesc: too many mips (%d). Only up to %d mips are supported.", desc.mips, NTC_HIP_MAX_MIPS);
+        return Status::OutOfRange;
+    }
+    return Status::Ok;
+}
+
+// src/TextureSetMetadata.cpp:1180-1208: the grid size scale is not stored, it follows from the
+// size of the first latent image.
+Status DeserializeTextureSetDesc(file::Document const& document, TextureSetDesc& desc, LatentShape& shape)
+{
+    desc.width = int(document.width);
+    desc.height = int(document.height);
+    desc.channels = int(document.numChannels);
+    desc.mips = int(document.numColorMips.value_or(1));
+    if (document.latentFeatures.has_value() && !document.latents.empty()) {
+        shape.numFeatures = int(*document.latentFeatures);
+        file::LatentImage const& first = document.latents[0];
+        float const widthRatio = float(desc.width) / float(std::max(first.width, 1u));
+        float const heightRatio = float(desc.height) / float(std::max(first.height, 1u));
+        shape.gridSizeScale = int(roundf(std::min(widthRatio, heightRatio)));
+    } else {
+        shape = LatentShape::Empty();
+    }
+    if (Status st = ValidateTextureSetDesc(desc); st != Status::Ok) return st;
+    return ValidateLatentShape(shape);
+}
 
 class TextureSet final : public ITextureSet
 {
@@ -201,6 +365,187 @@ public:
         return mask;
     }
 
+    // src/TextureSet.cpp:718-745
+    Status LoadFromStream(IStream* stream) override
+    {
+        if (!stream) { SetErrorMessage("inputStream is NULL."); return Status::InvalidArgument; }
+        file::Document document;
+        uint64_t binaryChunkOffset = 0, binaryChunkSize = 0;
+        if (Status st = LoadFileHeadersFromStream(stream, document, binaryChunkOffset, binaryChunkSize); st != Status::Ok) return st;
+        TextureSetDesc desc;
+        LatentShape shape;
+        if (Status st = DeserializeTextureSetDesc(document, desc, shape); st != Status::Ok) return st;
+        if (desc.width != m_desc.width || desc.height != m_desc.height || desc.channels != m_desc.channels || desc.mips != m_desc.mips) {
+            SetErrorMessage("Incompatible texture set in the file - dimensions do not match.");
+            return Status::FileIncompatible;
+        }
+        return LoadFromStreamPostHeader(document, binaryChunkOffset, binaryChunkSize, stream, shape);
+    }
+    Status LoadFromMemory(void const* pData, size_t size) override
+    {
+        if (!pData) { SetErrorMessage("pData is NULL."); return Status::InvalidArgument; }
+        if (size == 0) { SetErrorMessage("size is 0."); return Status::InvalidArgument; }
+        MemoryStream stream(const_cast<uint8_t*>(static_cast<uint8_t const*>(pData)), size, true);
+        return LoadFromStream(&stream);
+    }
+    Status LoadFromFile(char const* fileName) override
+    {
+        if (!fileName) { SetErrorMessage("fileName is NULL."); return Status::InvalidArgument; }
+        FILE* f = std::fopen(fileName, "rb");
+        if (!f) { SetErrorMessage("Cannot open file '%s': %s.", fileName, std::strerror(errno)); return Status::FileUnavailable; }
+        FileStream stream(f);
+        return LoadFromStream(&stream);
+    }
+    ColorSpace GetChannelStorageColorSpace(int channel) const override
+    {
+        return (channel >= 0 && channel < NTC_HIP_MAX_CHANNELS) ? m_channelColorSpaces[channel] : ColorSpace::Linear;
+    }
+
+    // LoadMetadataFromStream + LoadFromStreamPostHeader + LoadWeightsFromStream
+    // (src/TextureSetMetadata.cpp:434-581,676-784, src/TextureSet.cpp:154-294).  Everything is
+    // validated and assembled in host memory first; the device is touched last.
+    Status LoadFromStreamPostHeader(file::Document const& document, uint64_t binaryChunkOffset, uint64_t binaryChunkSize,
+        IStream* stream, LatentShape const& shape)
+    {
+        ClearTextureMetadata();
+        if (shape.IsEmpty()) { SetErrorMessage("The file does not describe a latent shape."); return Status::FileUnrecognized; }
+
+        // MLP versions
+        if (document.mlpVersions.empty()) { SetErrorMessage("File doesn't contain MLP information"); return Status::FileUnrecognized; }
+        NtcHipDecoderSpec const spec = MakeSpec(DecoderPreset::LibNTC092, shape.numFeatures);
+        for (file::Mlp const& mlp : document.mlpVersions)
+            if (!ValidateMLP(document, mlp, spec, binaryChunkSize)) return Status::FileUnrecognized;
+
+        // Texture headers
+        for (file::Texture const& t : document.textures) {
+            ITextureMetadata* texture = AddTexture();
+            if (!texture) { SetErrorMessage("Failed to allocate a texture metadata object."); return Status::OutOfMemory; }
+            texture->SetName(t.name.c_str());
+            (void)texture->SetChannels(int(t.firstChannel), int(t.numChannels));
+            texture->SetChannelFormat(ChannelFormat(t.channelFormat.value_or(int(ChannelFormat::UNORM8))));
+            texture->SetBlockCompressedFormat(BlockCompressedFormat(t.bcFormat.value_or(0)));
+            texture->SetRgbColorSpace(ColorSpace(t.rgbColorSpace.value_or(0)));
+            texture->SetAlphaColorSpace(ColorSpace(t.alphaColorSpace.value_or(0)));
+        }
+
+        // Channel headers
+        std::fill_n(m_channelColorSpaces, NTC_HIP_MAX_CHANNELS, ColorSpace::Linear);
+        if (!document.channelColorSpaces.empty()) {
+            if (int(document.channelColorSpaces.size()) != m_desc.channels) {
+                SetErrorMessage("The file describes %d texture channels while %d are expected", int(document.numChannels), m_desc.channels);
+                return Status::FileUnrecognized;
+            }
+            for (size_t i = 0; i < document.channelColorSpaces.size(); ++i)
+                m_channelColorSpaces[i] = ColorSpace(document.channelColorSpaces[i].value_or(0));
+        }
+
+        // Latent image headers
+        int const numLayers = (shape.numFeatures + 3) / 4;
+        for (size_t neuralLod = 0; neuralLod < document.latents.size(); ++neuralLod) {
+            file::LatentImage const& image = document.latents[neuralLod];
+            uint64_t const layerSize = uint64_t(image.width) * uint64_t(image.height) * 2u;
+            if (int(image.layerViews.size()) != numLayers) {
+                SetErrorMessage("Expected %d layers, got %d for the latent image in MIP %d", numLayers, int(image.layerViews.size()), int(neuralLod));
+                return Status::FileUnrecognized;
+            }
+            for (uint32_t view : image.layerViews)
+                if (!ValidateBufferView(view, layerSize, document, binaryChunkSize)) return Status::FileUnrecognized;
+        }
+
+        // Colour mips
+        if (int(document.colorMips.size()) > m_desc.mips) {
+            SetErrorMessage("The file describes %d color MIP levels while %d are expected", int(document.colorMips.size()), m_desc.mips);
+            return Status::FileUnrecognized;
+        }
+        int fileNeuralLod[NTC_HIP_MAX_MIPS] = {};
+        for (size_t mipLevel = 0; mipLevel < document.colorMips.size(); ++mipLevel) {
+            file::ColorMip const& colorMip = document.colorMips[mipLevel];
+            if (!colorMip.latentMip.has_value()) {
+                SetErrorMessage("Color MIP %d doesn't have a mapping to a latent image, which is currently unsupported.", int(mipLevel));
+                return Status::FileUnrecognized;
+            }
+            fileNeuralLod[mipLevel] = int(*colorMip.latentMip);
+            if (!colorMip.positionLod.has_value() || !colorMip.positionScale.has_value()) {
+                SetErrorMessage("Color MIP %d doesn't have the positionLod and positionScale parameters.", int(mipLevel));
+                return Status::FileUnrecognized;
+            }
+            if (colorMip.width.has_value() && colorMip.height.has_value()) {
+                int const mipWidth = std::max(m_desc.width >> mipLevel, 1), mipHeight = std::max(m_desc.height >> mipLevel, 1);
+                if (int(*colorMip.width) != mipWidth || int(*colorMip.height) != mipHeight) {
+                    SetErrorMessage("Color MIP %d specifies dimensions of %dx%d, but it is expected to be %dx%d.", int(mipLevel),
+                        int(*colorMip.width), int(*colorMip.height), mipWidth, mipHeight);
+                    return Status::FileUnrecognized;
+                }
+            }
+        }
+
+        // The decoder relies on one specific geometry (src/TextureSet.cpp:161-196).
+        for (size_t neuralLod = 0; neuralLod < document.latents.size(); ++neuralLod) {
+            file::LatentImage const& image = document.latents[neuralLod];
+            int const width = GridDimension(m_desc.width, int(neuralLod), shape.gridSizeScale);
+            int const height = GridDimension(m_desc.height, int(neuralLod), shape.gridSizeScale);
+            if (int(image.width) != width || int(image.height) != height) {
+                SetErrorMessage("Neural MIP %d dimensions (%dx%d) don't match the expected dimensions (%dx%d)", int(neuralLod),
+                    int(image.width), int(image.height), width, height);
+                return Status::FileUnrecognized;
+            }
+        }
+        for (int mipLevel = 0; mipLevel < m_desc.mips; ++mipLevel) {
+            int const expected = LodToNeuralLod(mipLevel, shape.gridSizeScale, int(document.latents.size()));
+            if (fileNeuralLod[mipLevel] != expected) {
+                SetErrorMessage("Color MIP %d specifies latent image index %d, but it is expected to be %d.", mipLevel, fileNeuralLod[mipLevel], expected);
+                return Status::FileUnrecognized;
+            }
+        }
+        int const neuralLods = NeuralLodCount(m_desc.width, m_desc.height, m_desc.mips, shape.gridSizeScale);
+        if (int(document.latents.size()) < neuralLods) {
+            SetErrorMessage("The file holds %d latent images while %d are expected", int(document.latents.size()), neuralLods);
+            return Status::FileUnrecognized;
+        }
+
+        // MLP data: the Int8 version, expanded to the layer sizes the decoder is built for.
+        NtcHipWeightLayout layout{};
+        if (ntc_hip_weight_layout(&spec, &layout) != 0) { SetErrorMessage("%s", ntc_hip_last_error()); return Status::InternalError; }
+        std::vector<uint8_t> blob(layout.bufferSize, 0);
+        bool haveInt8 = false;
+        for (file::Mlp const& mlp : document.mlpVersions) {
+            if (mlp.layers.empty() || mlp.layers[0].weightType != file::MlpDataType::Int8) continue;
+            if (Status st = ReadMlpData(document, mlp, spec, layout, binaryChunkOffset, stream, blob); st != Status::Ok) return st;
+            haveInt8 = true;
+        }
+        if (!haveInt8) { SetErrorMessage("The file holds no Int8 version of the MLP; FP8 weights are not decoded by this library."); return Status::Unsupported; }
+
+        // Latents: u16 layers, neural LOD after neural LOD (src/FeatureGridHost.cpp:140-161).
+        std::vector<uint8_t> latents;
+        for (int neuralLod = 0; neuralLod < neuralLods; ++neuralLod) {
+            file::LatentImage const& image = document.latents[size_t(neuralLod)];
+            size_t const layerSize = size_t(image.width) * size_t(image.height) * 2u;
+            for (uint32_t viewIndex : image.layerViews) {
+                file::BufferView const& view = document.views[viewIndex];
+                file::Compression const compression = view.compression.value_or(file::Compression::None);
+                if (compression != file::Compression::None) {
+                    SetErrorMessage("Latent image view %d is stored with GDeflate compression, which this library does not decode.", int(viewIndex));
+                    return Status::Unsupported;
+                }
+                size_t const at = latents.size();
+                latents.resize(at + layerSize);
+                if (!(stream->Seek(binaryChunkOffset + view.offset) && stream->Read(latents.data() + at, layerSize))) {
+                    SetErrorMessage("Failed to read latent image view %d.", int(viewIndex));
+                    return Status::IOError;
+                }
+            }
+        }
+
+        // Same order as the reference: the shape is (re)applied, then the data goes in.
+        m_latentShape = LatentShape::Empty();
+        if (Status st = SetLatentShape(shape); st != Status::Ok) return st;
+        if (latents.size() != m_latentBytes || blob.size() != m_weightLayout.bufferSize) { SetErrorMessage("Inconsistent sizes for MLP or latent data"); return Status::InternalError; }
+        if (Status st = SetWeightData(blob.data(), blob.size()); st != Status::Ok) return st;
+        if (Status st = SetLatentData(latents.data(), latents.size()); st != Status::Ok) return st;
+        ClearErrorMessage();
+        return Status::Ok;
+    }
+
     Status SetDecoderPreset(DecoderPreset preset) override
     {
         if (int(preset) < 0 || int(preset) > int(DecoderPreset::Concat2x2_48)) {
@@ -217,17 +562,7 @@ public:
     // src/TextureSetMetadata.cpp:1137-1159
     Status SetLatentShape(LatentShape const& newShape) override
     {
-        if (!newShape.IsEmpty()) {
-            if (newShape.numFeatures <= 0 || newShape.numFeatures > 16 || (newShape.numFeatures % 4) != 0) {
-                SetErrorMessage("Invalid LatentShape: numFeatures (%d) must be a positive multiple of %d up to %d.",
-                    newShape.numFeatures, 4, 16);
-                return Status::OutOfRange;
-            }
-            if (newShape.gridSizeScale < 1 || newShape.gridSizeScale > 6) {
-                SetErrorMessage("Invalid LatentShape: gridSizeScale (%d) must be between 1 and 6.", newShape.gridSizeScale);
-                return Status::OutOfRange;
-            }
-        }
+        if (Status st = ValidateLatentShape(newShape); st != Status::Ok) return st;
         m_latentShape = newShape;
         if (newShape.IsEmpty()) return ResetShape();
         m_preset = DecoderPreset::LibNTC092;
@@ -251,7 +586,7 @@ public:
 
         // Losses need the reference image to survive the decode: decode into a second page.
         uint32_t const validMask = GetValidChannelMask();
-        bool const lazyOutPage = validMask != 0 && !m_textureDataOut;
+        bool const lazyOutPage = validMask != 0 && pOutStats && !m_textureDataOut;
         if (lazyOutPage)
             if (int r = ntc_hip_alloc(&m_textureDataOut, m_textureBytes)) return AllocationFailure(r, "texture data (output)", m_textureBytes);
         void* const outPage = m_textureDataOut ? m_textureDataOut : m_textureData;   // src/TextureSet.cpp:1799-1802
@@ -427,6 +762,112 @@ private:
         return Status::Ok;
     }
 
+    // src/TextureSetMetadata.cpp:978-1016
+    bool ValidateBufferView(uint32_t view, uint64_t minSize, file::Document const& document, uint64_t binaryChunkSize)
+    {
+        if (view >= document.views.size()) { SetErrorMessage("Invalid view index %u", view); return false; }
+        file::BufferView const& desc = document.views[view];
+        if ((desc.offset & 3) != 0) { SetErrorMessage("View %u offset %" PRIu64 " is not 4-byte aligned", view, desc.offset); return false; }
+        uint64_t const uncompressedSize = desc.compression.value_or(file::Compression::None) != file::Compression::None
+            ? desc.uncompressedSize.value_or(0) : desc.storedSize;
+        if (uncompressedSize < minSize) {
+            SetErrorMessage("View %u size %" PRIu64 " is less than minimum expected size %" PRIu64 ".", view, desc.storedSize, minSize);
+            return false;
+        }
+        if (desc.offset + desc.storedSize < desc.offset || desc.offset + desc.storedSize > binaryChunkSize) {
+            SetErrorMessage("View %u ends at byte offset %" PRIu64 " from the binary chunk start, "
+                "which is outside of the chunk size %" PRIu64 ".", view, desc.offset + desc.storedSize, binaryChunkSize);
+            return false;
+        }
+        return true;
+    }
+
+    static size_t MlpDataTypeSize(file::MlpDataType type)      // src/TextureSetMetadata.cpp:1018-1029
+    {
+        switch (type) {
+        case file::MlpDataType::Int8: case file::MlpDataType::FloatE4M3: case file::MlpDataType::FloatE5M2: return 1;
+        case file::MlpDataType::Float16: return 2;
+        case file::MlpDataType::Float32: return 4;
+        default: return 0;
+        }
+    }
+
+    // src/TextureSetMetadata.cpp:1031-1135: four layers, row-major, one of the two known type
+    // patterns, hidden layers no wider than the decoder's, views large enough.
+    bool ValidateMLP(file::Document const& document, file::Mlp const& mlp, NtcHipDecoderSpec const& spec, uint64_t binaryChunkSize)
+    {
+        using T = file::MlpDataType;
+        if (mlp.layers.size() != 4) {
+            SetErrorMessage("File describes an MLP with %d layers, while only %d layers are supported", int(mlp.layers.size()), 4);
+            return false;
+        }
+        if (mlp.weightLayout != file::MatrixLayout::RowMajor) { SetErrorMessage("Only row-major MLP weight layout is supported at this time."); return false; }
+        bool int8Pattern = true, fp8Pattern = true;
+        for (int l = 0; l < 4; ++l) {
+            file::MlpLayer const& layer = mlp.layers[size_t(l)];
+            bool const last = l == 3;
+            int8Pattern = int8Pattern && layer.weightType == T::Int8 && layer.scaleType == T::Float32 && layer.biasType == T::Int32;
+            fp8Pattern = fp8Pattern && (last ? (layer.weightType == T::Int8 && layer.scaleType == T::Float32 && layer.biasType == T::Int32)
+                                             : (layer.weightType == T::FloatE4M3 && !layer.scaleType.has_value() && layer.biasType == T::Float16));
+        }
+        if (!int8Pattern && !fp8Pattern) {
+            SetErrorMessage("Only Int8 weights + Float32 scale + Int32 bias or FloatE4M3 + Float16 bias MLP configurations are supported at this time.");
+            return false;
+        }
+        for (int l = 0; l < 4; ++l) {
+            file::MlpLayer const& layer = mlp.layers[size_t(l)];
+            bool const smallerInputsAllowed = l > 0, smallerOutputsAllowed = l < 3;
+            uint32_t const expectedInputs = uint32_t(LayerInputs(spec, l)), expectedOutputs = uint32_t(LayerOutputs(spec, l));
+            bool const inputsFine = smallerInputsAllowed ? layer.inputChannels <= expectedInputs : layer.inputChannels == expectedInputs;
+            bool const outputsFine = smallerOutputsAllowed ? layer.outputChannels <= expectedOutputs : layer.outputChannels == expectedOutputs;
+            if (!inputsFine || !outputsFine) {
+                SetErrorMessage("File describes MLP layer %d with %d inputs and %d outputs, but that layer should have %s%d inputs and %s%d outputs.",
+                    l, int(layer.inputChannels), int(layer.outputChannels), smallerInputsAllowed ? "at most " : "", int(expectedInputs),
+                    smallerOutputsAllowed ? "at most " : "", int(expectedOutputs));
+                return false;
+            }
+            if (!ValidateBufferView(layer.weightView, uint64_t(layer.inputChannels) * layer.outputChannels * MlpDataTypeSize(layer.weightType), document, binaryChunkSize)) return false;
+            if (layer.scaleType.has_value() && layer.scaleView.has_value())
+                if (!ValidateBufferView(*layer.scaleView, uint64_t(layer.outputChannels) * MlpDataTypeSize(*layer.scaleType), document, binaryChunkSize)) return false;
+            if (!ValidateBufferView(layer.biasView, uint64_t(layer.outputChannels) * MlpDataTypeSize(layer.biasType), document, binaryChunkSize)) return false;
+        }
+        return true;
+    }
+
+    static int LayerInputs(NtcHipDecoderSpec const& spec, int layer) { return layer == 0 ? spec.inputChannels : spec.hiddenChannels[layer - 1]; }
+    static int LayerOutputs(NtcHipDecoderSpec const& spec, int layer) { return layer == 3 ? spec.outputChannels : spec.hiddenChannels[layer]; }
+
+    // src/TextureSetMetadata.cpp:661-761: a narrower hidden layer lands in the top-left corner of
+    // the zero-filled matrix, missing scales become 1, missing biases stay 0.
+    Status ReadMlpData(file::Document const& document, file::Mlp const& mlp, NtcHipDecoderSpec const& spec, NtcHipWeightLayout const& layout,
+        uint64_t binaryChunkOffset, IStream* stream, std::vector<uint8_t>& blob)
+    {
+        auto readView = [&](uint32_t view, void* dst, size_t size) {
+            return size == 0 || (stream->Seek(binaryChunkOffset + document.views[view].offset) && stream->Read(dst, size));
+        };
+        std::vector<uint8_t> narrow;
+        for (int l = 0; l < 4; ++l) {
+            file::MlpLayer const& layer = mlp.layers[size_t(l)];
+            size_t const expectedInputs = size_t(LayerInputs(spec, l)), expectedOutputs = size_t(LayerOutputs(spec, l));
+            uint8_t* const weights = blob.data() + layout.weightOffset[l];
+            if (layer.inputChannels < expectedInputs || layer.outputChannels < expectedOutputs) {
+                narrow.resize(size_t(layer.inputChannels) * layer.outputChannels);
+                if (!readView(layer.weightView, narrow.data(), narrow.size())) return ReadFailure("weights", l);
+                for (size_t row = 0; row < layer.outputChannels; ++row)
+                    std::memcpy(weights + row * expectedInputs, narrow.data() + row * layer.inputChannels, layer.inputChannels);
+            } else if (!readView(layer.weightView, weights, expectedInputs * expectedOutputs)) {
+                return ReadFailure("weights", l);
+            }
+            float* const scales = reinterpret_cast<float*>(blob.data() + layout.scaleOffset[l]);
+            size_t const providedScales = layer.scaleView.has_value() ? layer.outputChannels : 0;
+            if (providedScales && !readView(*layer.scaleView, scales, providedScales * sizeof(float))) return ReadFailure("scales", l);
+            for (size_t i = providedScales; i < expectedOutputs; ++i) scales[i] = 1.0f;
+            if (!readView(layer.biasView, blob.data() + layout.biasOffset[l], size_t(layer.outputChannels) * sizeof(int32_t))) return ReadFailure("biases", l);
+        }
+        return Status::Ok;
+    }
+    Status ReadFailure(char const* what, int layer) { SetErrorMessage("Failed to read the %s of MLP layer %d.", what, layer); return Status::IOError; }
+
     Status AllocationFailure(int code, char const* what, uint64_t bytes)
     {
         if (code > 0) { SetErrorMessage("Failed to allocate %llu bytes of device memory for the %s buffer.", (unsigned long long)bytes, what); return Status::OutOfMemory; }
@@ -471,13 +912,10 @@ private:
     // colour-mip constants (src/TextureSet.cpp:441-463), low-res dimensions (src/TextureSet.cpp:1816-1817).
     void BuildSharedNeuralLods()
     {
-        static int const sharedMips[] = { 2, 3, 3, 3, 4, 4 };
         int const gs = m_latentShape.gridSizeScale;
-        auto neuralOf = [&](int lod, int count) { return std::max(0, std::min((lod - sharedMips[gs - 1] + 2) & ~1, count - 2)); };
-        auto gridDim = [&](int dim, int nlod) { return std::max((dim / gs) >> nlod, 1); };
-        int const minGrid = int(float(std::min(m_desc.width, m_desc.height)) / float(gs));
-        int neuralLods = std::max(2, int(1.f + std::floor(std::log2(float(minGrid))))) & ~1;
-        neuralLods = std::min(neuralLods, neuralOf(m_desc.mips - 1, 8) + 2);
+        auto neuralOf = [&](int lod, int count) { return LodToNeuralLod(lod, gs, count); };
+        auto gridDim = [&](int dim, int nlod) { return GridDimension(dim, nlod, gs); };
+        int const neuralLods = NeuralLodCount(m_desc.width, m_desc.height, m_desc.mips, gs);
         uint64_t const layers = uint64_t((m_latentShape.numFeatures + 3) / 4);
         std::vector<uint64_t> offset(size_t(neuralLods) + 1, 0);
         for (int n = 0; n < neuralLods; ++n)
@@ -537,6 +975,7 @@ private:
     uint64_t m_mipOffsets[NTC_HIP_MAX_MIPS + 1]{};
     uint64_t m_textureBytes = 0, m_stagingBytes = 0, m_latentBytes = 0;
     std::vector<TextureMetadata*> m_textures;
+    ColorSpace m_channelColorSpaces[NTC_HIP_MAX_CHANNELS] = {};
     void* m_textureData = nullptr;      // reference page (and the only page without separateRefOutData)
     void* m_textureDataOut = nullptr;   // output page
     void* m_staging = nullptr;
@@ -555,19 +994,7 @@ public:
     {
         if (!pOutTextureSet) { SetErrorMessage("pOutTextureSet is NULL."); return Status::InvalidArgument; }
         *pOutTextureSet = nullptr;
-        if (desc.width <= 0 || desc.height <= 0 || desc.channels <= 0 || desc.mips <= 0) {
-            SetErrorMessage("Invalid TextureSetDesc: width (%d), height (%d), channels (%d) and mips (%d) "
-                "must be positive numbers.", desc.width, desc.height, desc.channels, desc.mips);
-            return Status::OutOfRange;
-        }
-        if (desc.channels > NTC_HIP_MAX_CHANNELS) {
-            SetErrorMessage("Invalid TextureSetDesc: too many channels (%d). Only up to %d channels are supported.", desc.channels, NTC_HIP_MAX_CHANNELS);
-            return Status::OutOfRange;
-        }
-        if (desc.mips > NTC_HIP_MAX_MIPS) {
-            SetErrorMessage("Invalid TextureSetDesc: too many mips (%d). Only up to %d mips are supported.", desc.mips, NTC_HIP_MAX_MIPS);
-            return Status::OutOfRange;
-        }
+        if (Status st = ValidateTextureSetDesc(desc); st != Status::Ok) return st;
         TextureSet* set = new (std::nothrow) TextureSet(this, desc, features);
         if (!set) { SetErrorMessage("Failed to allocate the texture set object."); return Status::OutOfMemory; }
         Status const status = set->Initialize(m_deviceAvailable);
@@ -580,7 +1007,73 @@ public:
     void DestroyTextureSet(ITextureSet* textureSet) const override { delete textureSet; }
     bool IsCudaAvailable() const override { return m_deviceAvailable; }
 
+    // src/Context.cpp:80-176
+    Status OpenFile(char const* fileName, bool write, IStream** pOutStream) const override
+    {
+        if (!fileName) { SetErrorMessage("fileName is NULL."); return Status::InvalidArgument; }
+        if (!pOutStream) { SetErrorMessage("pOutStream is NULL."); return Status::InvalidArgument; }
+        FILE* file = std::fopen(fileName, write ? "wb" : "rb");
+        if (!file) { SetErrorMessage("Cannot open file '%s': %s.", fileName, std::strerror(errno)); return Status::FileUnavailable; }
+        *pOutStream = new (std::nothrow) FileStream(file);
+        if (!*pOutStream) { std::fclose(file); SetErrorMessage("Failed to allocate the stream object."); return Status::OutOfMemory; }
+        return Status::Ok;
+    }
+    void CloseFile(IStream* stream) const override { delete stream; }
+    Status OpenMemory(void* pData, size_t size, IStream** pOutStream) const override { return OpenMemoryStream(pData, size, false, pOutStream); }
+    Status OpenReadOnlyMemory(void const* pData, size_t size, IStream** pOutStream) const override
+    {
+        return OpenMemoryStream(const_cast<void*>(pData), size, true, pOutStream);
+    }
+    void CloseMemory(IStream* stream) const override { delete stream; }
+
+    // src/Context.cpp:296-352
+    Status CreateCompressedTextureSetFromStream(IStream* inputStream, TextureSetFeatures const& features, ITextureSet** pOutTextureSet) const override
+    {
+        if (!pOutTextureSet) { SetErrorMessage("pOutTextureSet is NULL."); return Status::InvalidArgument; }
+        *pOutTextureSet = nullptr;
+        if (!inputStream) { SetErrorMessage("inputStream is NULL."); return Status::InvalidArgument; }
+        file::Document document;
+        uint64_t binaryChunkOffset = 0, binaryChunkSize = 0;
+        if (Status st = LoadFileHeadersFromStream(inputStream, document, binaryChunkOffset, binaryChunkSize); st != Status::Ok) return st;
+        TextureSetDesc desc;
+        LatentShape shape;
+        if (Status st = DeserializeTextureSetDesc(document, desc, shape); st != Status::Ok) return st;
+        ITextureSet* created = nullptr;
+        if (Status st = CreateTextureSet(desc, features, &created); st != Status::Ok) return st;
+        Status const status = static_cast<TextureSet*>(created)->LoadFromStreamPostHeader(document, binaryChunkOffset, binaryChunkSize, inputStream, shape);
+        if (status != Status::Ok) { DestroyTextureSet(created); return status; }
+        *pOutTextureSet = created;
+        ClearErrorMessage();
+        return Status::Ok;
+    }
+    Status CreateCompressedTextureSetFromMemory(void const* pData, size_t size, TextureSetFeatures const& features, ITextureSet** pOutTextureSet) const override
+    {
+        IStream* stream = nullptr;
+        if (Status st = OpenReadOnlyMemory(pData, size, &stream); st != Status::Ok) return st;
+        Status const status = CreateCompressedTextureSetFromStream(stream, features, pOutTextureSet);
+        CloseMemory(stream);
+        return status;
+    }
+    Status CreateCompressedTextureSetFromFile(char const* fileName, TextureSetFeatures const& features, ITextureSet** pOutTextureSet) const override
+    {
+        IStream* stream = nullptr;
+        if (Status st = OpenFile(fileName, false, &stream); st != Status::Ok) return st;
+        Status const status = CreateCompressedTextureSetFromStream(stream, features, pOutTextureSet);
+        CloseFile(stream);
+        return status;
+    }
+
 private:
+    Status OpenMemoryStream(void* pData, size_t size, bool readonly, IStream** pOutStream) const
+    {
+        if (!pData) { SetErrorMessage("pData is NULL."); return Status::InvalidArgument; }
+        if (size == 0) { SetErrorMessage("size is 0."); return Status::InvalidArgument; }
+        if (!pOutStream) { SetErrorMessage("pOutStream is NULL."); return Status::InvalidArgument; }
+        *pOutStream = new (std::nothrow) MemoryStream(static_cast<uint8_t*>(pData), size, readonly);
+        if (!*pOutStream) { SetErrorMessage("Failed to allocate the stream object."); return Status::OutOfMemory; }
+        return Status::Ok;
+    }
+
     bool m_deviceAvailable;
 };
 

@@ -3,9 +3,9 @@
 // It mirrors the part of LibNTC's public interface that the decompression path uses
 // (reference include/libntc/ntc.h): the same names in namespace ntc, the same argument meaning,
 // the same status codes and error-message convention, so code written against LibNTC's
-//   CreateContext -> IContext::CreateTextureSet -> ITextureSet::SetLatentShape ->
-//   (load) -> ITextureSet::Decompress -> ITextureSet::ReadChannels
-// sequence reads the same here.  Compression, file I/O and graphics-API interop are not part
+//   CreateContext -> IContext::CreateCompressedTextureSetFromFile (or CreateTextureSet +
+//   ITextureSet::LoadFromFile) -> ITextureSet::Decompress -> ITextureSet::ReadChannels
+// sequence reads the same here.  Compression, saving files and graphics-API interop are not part
 // of this library; the interface below simply does not declare them.
 //
 // Everything device-side goes through the C ABI of include/ntc_hip.h; this layer never
@@ -36,6 +36,21 @@ enum class ChannelFormat { UNKNOWN = 0, UNORM8 = 1, UNORM16 = 2, FLOAT16 = 3, FL
 // include/libntc/ntc.h:272-276
 enum class AddressSpace { Host, Device };
 enum class TextureDataPage { Reference, Output };
+// include/libntc/ntc.h:238-256
+enum class BlockCompressedFormat { None = 0, BC1 = 1, BC2 = 2, BC3 = 3, BC4 = 4, BC5 = 5, BC6 = 6, BC7 = 7 };
+enum class ColorSpace { Linear = 0, sRGB = 1, HLG = 2 };
+
+// Application-provided or library-provided byte streams (include/libntc/ntc.h:91-114).
+class IStream
+{
+public:
+    virtual bool Read(void* dst, size_t size) = 0;          // false on error or a short read
+    virtual bool Write(const void* src, size_t size) = 0;
+    virtual bool Seek(uint64_t offset) = 0;                 // from the beginning of the stream
+    virtual uint64_t Tell() = 0;
+    virtual uint64_t Size() = 0;
+    virtual ~IStream() = default;
+};
 
 constexpr int DisableCudaDevice = -1;          // ContextParameters::cudaDevice: do not touch the GPU
 
@@ -143,6 +158,17 @@ public:
     // set's channels (src/TextureMetadata.cpp:48-69).
     virtual Status SetChannels(int firstChannel, int numChannels) = 0;
     virtual void GetChannels(int& outFirstChannel, int& outNumChannels) const = 0;
+    virtual int GetFirstChannel() const = 0;
+    virtual int GetNumChannels() const = 0;
+    // Stored with the texture and read back from NTC files; the decoder itself does not use them.
+    virtual void SetChannelFormat(ChannelFormat format) = 0;
+    virtual ChannelFormat GetChannelFormat() const = 0;
+    virtual void SetBlockCompressedFormat(BlockCompressedFormat format) = 0;
+    virtual BlockCompressedFormat GetBlockCompressedFormat() const = 0;
+    virtual void SetRgbColorSpace(ColorSpace colorSpace) = 0;
+    virtual ColorSpace GetRgbColorSpace() const = 0;
+    virtual void SetAlphaColorSpace(ColorSpace colorSpace) = 0;
+    virtual ColorSpace GetAlphaColorSpace() const = 0;
     virtual ~ITextureMetadata() = default;
 };
 
@@ -163,7 +189,16 @@ public:
     // Range rules follow src/TextureSetMetadata.cpp:1137-1159.
     virtual Status SetLatentShape(LatentShape const& newShape) = 0;
 
-    // --- additions: the reference can only receive latents and weights from an NTC file ---
+    // Loads latents, the Int8 MLP and texture metadata from an NTC file whose dimensions match
+    // this set (include/libntc/ntc.h:871-889, src/TextureSet.cpp:154-294,718-800).  Views stored
+    // with GDeflate compression are refused with Status::Unsupported.
+    virtual Status LoadFromStream(IStream* stream) = 0;
+    virtual Status LoadFromMemory(void const* pData, size_t size) = 0;
+    virtual Status LoadFromFile(char const* fileName) = 0;
+    // Storage colour space of a channel as recorded in the file (include/libntc/ntc.h:592-595).
+    virtual ColorSpace GetChannelStorageColorSpace(int channel) const = 0;
+
+    // --- additions: raw latents and weights without a file ---
     virtual Status SetDecoderPreset(DecoderPreset preset) = 0;
     // Size in bytes of the latent buffer / weight blob the current shape expects.
     virtual uint64_t GetLatentDataSize() const = 0;
@@ -200,6 +235,20 @@ public:
         ITextureSet** pOutTextureSet) const = 0;
     // include/libntc/ntc.h:1153
     virtual void DestroyTextureSet(ITextureSet* textureSet) const = 0;
+    // Streams over files and memory (include/libntc/ntc.h:1127-1145, src/Context.cpp:80-176).
+    virtual Status OpenFile(char const* fileName, bool write, IStream** pOutStream) const = 0;
+    virtual void CloseFile(IStream* stream) const = 0;
+    virtual Status OpenMemory(void* pData, size_t size, IStream** pOutStream) const = 0;
+    virtual Status OpenReadOnlyMemory(void const* pData, size_t size, IStream** pOutStream) const = 0;
+    virtual void CloseMemory(IStream* stream) const = 0;
+    // Creates a texture set with the dimensions found in an NTC file and loads it
+    // (include/libntc/ntc.h:1166-1177, src/Context.cpp:296-376).
+    virtual Status CreateCompressedTextureSetFromStream(IStream* inputStream, TextureSetFeatures const& features,
+        ITextureSet** pOutTextureSet) const = 0;
+    virtual Status CreateCompressedTextureSetFromMemory(void const* pData, size_t size, TextureSetFeatures const& features,
+        ITextureSet** pOutTextureSet) const = 0;
+    virtual Status CreateCompressedTextureSetFromFile(char const* fileName, TextureSetFeatures const& features,
+        ITextureSet** pOutTextureSet) const = 0;
     // True when a gfx950 device was initialised (reference: IsCudaAvailable).
     virtual bool IsCudaAvailable() const = 0;
     virtual ~IContext() = default;

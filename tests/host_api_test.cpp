@@ -8,6 +8,11 @@
 //   host_api_test loss <preset> <w> <h> <mips> <channels> <gridScale> <features> <latents> <weights> <refPrefix> <separate 0|1>
 //       registers two textures (channels 0..2 and 4..5), writes <refPrefix>_mip<N>.bin (FLOAT32 pixels,
 //       all channels) as the reference image, decompresses twice and prints the loss statistics
+//   host_api_test load <file> <device 0|1> [<w> <h> <channels> <mips>]
+//       loads an NTC file: with dimensions through CreateTextureSet + LoadFromFile, without through
+//       CreateCompressedTextureSetFromFile; prints the status, the message and what the set holds
+//   host_api_test decodefile <file> <outPrefix>
+//       CreateCompressedTextureSetFromMemory -> Decompress -> every mip as FLOAT16 pixels to files
 #include "../rtxntc-library_amd/host/ntc_decode.h"
 #include "../include/ntc_hip.h"
 
@@ -286,8 +291,88 @@ static int loss(int argc, char** argv)
     return 0;
 }
 
+static void describe(ITextureSet* set)
+{
+    TextureSetDesc const& d = set->GetDesc();
+    std::printf("desc %d %d %d %d\n", d.width, d.height, d.channels, d.mips);
+    std::printf("shape %d %d\n", set->GetLatentShape().gridSizeScale, set->GetLatentShape().numFeatures);
+    std::printf("sizes %llu %llu\n", (unsigned long long)set->GetLatentDataSize(), (unsigned long long)set->GetWeightDataSize());
+    for (int i = 0; i < set->GetTextureCount(); ++i) {
+        ITextureMetadata* t = set->GetTexture(i);
+        std::printf("texture %s|%d|%d|%s|%d|%d|%d\n", t->GetName(), t->GetFirstChannel(), t->GetNumChannels(),
+            ChannelFormatToString(t->GetChannelFormat()), int(t->GetBlockCompressedFormat()), int(t->GetRgbColorSpace()), int(t->GetAlphaColorSpace()));
+    }
+    std::printf("colorspaces");
+    for (int c = 0; c < d.channels; ++c) std::printf(" %d", int(set->GetChannelStorageColorSpace(c)));
+    std::printf("\nmask 0x%x\n", set->GetValidChannelMask());
+}
+
+static int load(int argc, char** argv)
+{
+    if (argc < 4) { std::fprintf(stderr, "usage: load <file> <device 0|1> [<w> <h> <channels> <mips>]\n"); return 2; }
+    IContext* ctx = nullptr;
+    ContextParameters params;
+    if (std::atoi(argv[3]) == 0) params.cudaDevice = DisableCudaDevice;
+    Status const created = CreateContext(&ctx, params);
+    CHECK(ctx != nullptr && (created == Status::Ok || created == Status::CudaUnavailable));
+    ITextureSet* set = nullptr;
+    Status status;
+    if (argc >= 8) {
+        TextureSetDesc desc; desc.width = std::atoi(argv[4]); desc.height = std::atoi(argv[5]); desc.channels = std::atoi(argv[6]); desc.mips = std::atoi(argv[7]);
+        CHECK(ctx->CreateTextureSet(desc, TextureSetFeatures(), &set) == Status::Ok);
+        status = set->LoadFromFile(argv[2]);
+    } else {
+        status = ctx->CreateCompressedTextureSetFromFile(argv[2], TextureSetFeatures(), &set);
+        CHECK((status == Status::Ok) == (set != nullptr));
+    }
+    std::printf("status %d %s\nmessage %s\n", int(status), StatusToString(status), GetLastErrorMessage());
+    if (set) { describe(set); ctx->DestroyTextureSet(set); }
+    DestroyContext(ctx);
+    return 0;
+}
+
+static int decodeFile(int argc, char** argv)
+{
+    if (argc < 4) { std::fprintf(stderr, "usage: decodefile <file> <outPrefix>\n"); return 2; }
+    std::vector<unsigned char> image = readFile(argv[2]);
+    std::string const prefix = argv[3];
+    IContext* ctx = nullptr;
+    ContextParameters params;
+    CHECK(CreateContext(&ctx, params) == Status::Ok);
+    TextureSetFeatures features;
+    features.stagingBytesPerPixel = 16 * 2;
+    ITextureSet* set = nullptr;
+    CHECK(ctx->CreateCompressedTextureSetFromMemory(image.data(), image.size(), features, &set) == Status::Ok);
+    describe(set);
+    CHECK(set->Decompress(nullptr) == Status::Ok);
+    TextureSetDesc const desc = set->GetDesc();
+    for (int mip = 0; mip < desc.mips; ++mip) {
+        ReadChannelsParameters rp;
+        rp.mipLevel = mip; rp.firstChannel = 0; rp.numChannels = desc.channels;
+        rp.width = std::max(desc.width >> mip, 1); rp.height = std::max(desc.height >> mip, 1);
+        rp.pixelStride = size_t(desc.channels) * 2; rp.rowPitch = rp.pixelStride * size_t(rp.width);
+        rp.channelFormat = ChannelFormat::FLOAT16;
+        std::vector<unsigned char> pixels(rp.rowPitch * size_t(rp.height));
+        rp.pOutData = pixels.data();
+        CHECK(set->ReadChannels(rp) == Status::Ok);
+        CHECK(writeFile(prefix + "_mip" + std::to_string(mip) + ".bin", pixels.data(), pixels.size()));
+    }
+    // loading the same file again into the existing set, through a stream this time
+    IStream* stream = nullptr;
+    CHECK(ctx->OpenFile(argv[2], false, &stream) == Status::Ok);
+    CHECK(set->LoadFromStream(stream) == Status::Ok);
+    ctx->CloseFile(stream);
+    CHECK(set->Decompress(nullptr) == Status::Ok);
+    ctx->DestroyTextureSet(set);
+    DestroyContext(ctx);
+    std::printf("host decodefile OK\n");
+    return 0;
+}
+
 int main(int argc, char** argv)
 {
+    if (argc >= 2 && std::strcmp(argv[1], "load") == 0) return load(argc, argv);
+    if (argc >= 2 && std::strcmp(argv[1], "decodefile") == 0) return decodeFile(argc, argv);
     if (argc >= 2 && std::strcmp(argv[1], "loss") == 0) return loss(argc, argv);
     if (argc >= 2 && std::strcmp(argv[1], "cpu") == 0) return cpuChecks();
     if (argc >= 2 && std::strcmp(argv[1], "decode") == 0) return decode(argc, argv);
