@@ -18,7 +18,7 @@
  *
  * Pinning status of each function is listed in the table at the end of this header.
  *
- *   function                 pinned by (tests/test_oracle_*.py)
+ *   function                 pinned by (tests/test_oracle_pins.py unless another file is named)
  *   -----------------------  -----------------------------------------------------------
  *   weight_layout            reference build oracle/_ref (MakeQuantizedWeightLayout) +
  *                            committed fixture tests/golden/ref_layout.json + closed-form totals
@@ -33,8 +33,16 @@
  *                            Inference.hlsli:37-39); exhaustive monotone pieces and range checks
  *   layer matmul             numpy int64 GEMM
  *   half / unorm8 convert    numpy float16 (IEEE RNE) over all 2^16 halves and a dense fp32 sweep
- *   e4m3 rounding            exhaustive over all half bit patterns vs an independent model
+ *   e4m3_times_512           the OCP e4m3 definition evaluated in numpy over all 256 bytes
+ *   layer_fp8_weights        numpy int64 GEMM on the decoded weights (tests/np_decoder.py)
+ *   scale/bias semantics     a numpy restatement of QuantizeColumnInt8 (src/Quantizer.cu:88-208)
+ *   (layer_int8)             must be reproduced by layer_int8 to quantisation error
+ *                            (tests/test_quantizer_semantics.py)
  *   end-to-end decode        an independent numpy restatement (tests/np_decoder.py) on small sets
+ *   decode_queries           the raster decode of the texels the queries hit (tests/test_queries.py)
+ *   read_channels,           numpy models of the 1:1 branch of cuda::CopyImage, five channel
+ *   write_channels           formats, padded rows, vertical flip (tests/test_host_api.py)
+ *   image_loss               numpy float64 mean squared error (tests/test_host_api.py)
  *   The exact bits of the reference's FP16-WMMA CUDA kernel (half accumulation order,
  *   --use_fast_math) and of a hardware bilinear sampler are NOT reproduced: parity unpinned
  *   for those two, by construction; the integer contract of Inference.hlsli is what is pinned.
