@@ -237,6 +237,12 @@ int ntc_hip_image_loss(const void* decodedPlanarPairs, const void* referencePlan
  * product.  No reference counterpart; used by the tests. */
 int ntc_hip_selftest_mfma(const int8_t* a16x64, const int8_t* b64x16, int32_t* d16x16);
 
+/* Same for the fp16 MFMA the hidden layers use when every partial sum of a layer stays an integer
+ * below 2^24: D = A*B + C, A 16 x depth and B depth x 16 as row-major IEEE halves, C and D 16x16
+ * floats, depth 16 or 32.  With integer-valued operands of that size the result must be the
+ * exact integer, whatever order the hardware adds in.  No reference counterpart; used by the tests. */
+int ntc_hip_selftest_mfma_f16(const uint16_t* aHalves, const uint16_t* bHalves, const float* c16x16, float* d16x16, int32_t depth);
+
 #ifdef __cplusplus
 }
 #endif

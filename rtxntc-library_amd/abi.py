@@ -124,6 +124,7 @@ EXPORTS = [
     ("ntc_hip_image_loss", C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64, C.c_int32, C.c_int32, C.c_int32, C.c_uint32,
                                      C.POINTER(C.c_float)]),
     ("ntc_hip_selftest_mfma", C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
+    ("ntc_hip_selftest_mfma_f16", C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32]),
 ]
 
 _HERE = os.path.dirname(os.path.abspath(__file__))

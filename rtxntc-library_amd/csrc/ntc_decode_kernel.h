@@ -83,5 +83,6 @@ hipError_t launch_queries(int variant, DevMip const* mips, int numMips, DevQuery
                           uint16_t* out, int gridSize, hipStream_t stream);
 int resident_workgroups_per_cu(int variant);
 hipError_t launch_selftest_mfma(int8_t const* a, int8_t const* b, int32_t* d, hipStream_t stream);
+hipError_t launch_selftest_mfma_f16(uint16_t const* a, uint16_t const* b, float const* c, float* d, int depth, hipStream_t stream);
 
 } // namespace ntc_hip_dev

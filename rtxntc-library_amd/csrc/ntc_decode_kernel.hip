@@ -143,6 +143,8 @@ __device__ __forceinline__ uint32_t activate4(v4i acc, v4f scale, uint32_t c143)
 }
 
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef float    v2f __attribute__((ext_vector_type(2)));
 
 // Two network outputs -> two fp16 in one dword.  The output is an fp32 product that is THEN
@@ -203,8 +205,8 @@ __device__ __forceinline__ void store_channels(GlobalOutPtr row, uint32_t laneOf
     }
 }
 
-template <int FORMAT>
-__device__ __forceinline__ void store_tile(DevMip const& m, v4i const (&D)[4], v4f S, int x, int y0, int chBase)
+template <int FORMAT, class Acc>
+__device__ __forceinline__ void store_tile(DevMip const& m, Acc const (&D)[4], v4f S, int x, int y0, int chBase)
 {
     int const nch = min(4, m.numChannels - chBase);
     if (x >= m.width || nch <= 0) return;
@@ -281,6 +283,21 @@ struct Variant {
     static constexpr int WEIGHT_BYTES = W3_OFF + H2 * OUT;
     static constexpr int TOTAL_OUT = H0 + H1 + H2 + OUT;
     static constexpr int SCALE_OFF = WEIGHT_BYTES, BIAS_OFF = WEIGHT_BYTES + 4 * TOTAL_OUT;
+    // Layers 1..3 can also run on the fp16 matrix instruction (see mlp_forward_f16).  Their A operands
+    // then take, per output tile, one 1024-byte block for every pair of input tiles (K = 32) and one
+    // 512-byte block for an odd last input tile (K = 16); sizes below are in 16-byte units.
+    static constexpr bool F16_LAYERS = !FP8_WEIGHTS_;
+    static constexpr int f16_units(int inTiles) { return (inTiles / 2) * 64 + (inTiles % 2) * 32; }
+    static constexpr int F16_L1 = 0;
+    static constexpr int F16_L2 = F16_L1 + T1 * f16_units(T0);
+    static constexpr int F16_L3 = F16_L2 + T2 * f16_units(T1);
+    static constexpr int F16_END = F16_L3 + T3 * f16_units(T2);
+    static constexpr int LATE_INT8_UNITS = (T1 + T2 + T3) * 64;
+    static constexpr int LATE_UNITS = F16_LAYERS ? (F16_END > LATE_INT8_UNITS ? F16_END : LATE_INT8_UNITS) : 1;
+    // A operands kept in `w`: every layer for the e4m3 variants, layer 0 only otherwise (the later
+    // layers then live in `late`, as int8 or as fp16).
+    static constexpr int W_TILES = F16_LAYERS ? T0 : NTILES;
+    static constexpr int LATE_CHANNELS = H1 + H2 + OUT;
     static_assert(POS_BASE + 12 + LOD <= IN, "input vector does not fit");
     static_assert(IN % 16 == 0 && IN <= 64 && H0 <= 64 && H1 <= 64 && H2 <= 64, "layer widths");
     static_assert(HR_INPUTS % 4 == 0 && LR_INPUTS % 4 == 0, "grid blocks are dword aligned");
@@ -288,15 +305,16 @@ struct Variant {
 
 template <class V>
 struct alignas(16) LdsT {
-    uint32_t w[V::PLANES][V::NTILES][64][4];   // A operands: [plane][M-tile][lane][4 dwords]
+    uint32_t w[V::PLANES][V::W_TILES][64][4];  // int8 A operands: [plane][M-tile][lane][4 dwords]
+    uint4    late[V::LATE_UNITS];              // A operands of layers 1..3 when V::F16_LAYERS: int8 tiles or fp16 blocks
     float    scale[V::NTILES][4][4];           // [M-tile][k-group g][r]  -> channel 16t+4g+r
     int32_t  bias[V::NTILES][4][4];
     uint32_t in[kWaves][kWaveTexels][kInStride];
     uint32_t lut2[256];               // byte of four 2-bit codes -> four input bytes 85*q - 128
-    // Positional encoding for every power-of-two positionScale 2^-k, k = 0..6: the entry for phase p of
+    // Positional encoding for every power-of-two positionScale 2^-k, k = 0..5: the entry for phase p of
     // scale 2^-k sits at index (2^k - 1) + p; dword w = enc(px*2^w) | enc(px*2^w + 1/4) << 16, px = p*2^-k.
-    uint32_t xtab[128][4];
-    uint32_t ytab[128][4];            // same for y, one byte up
+    uint32_t xtab[64][4];
+    uint32_t ytab[64][4];             // same for y, one byte up
 };
 
 // OCP e4m3 (1-4-3, bias 7, no infinities) byte -> the integer 512*value: subnormals m * 2^-9,
@@ -309,51 +327,150 @@ __device__ __forceinline__ int32_t e4m3_times_512(uint32_t byte)
     return (byte & 0x80u) ? -mag : mag;
 }
 
+// A operand dword of an int8 layer: four consecutive weights of one row (0 beyond the layer's inputs).
+__device__ __forceinline__ uint32_t weight_dword(uint32_t const* blob32, int woff, int row, int in, int k)
+{
+    return (k < in) ? blob32[(woff + row * in + k) >> 2] : 0u;
+}
+
+__device__ __forceinline__ uint32_t halves_of_bytes(uint32_t v, int firstByte)     // two int8 -> two fp16 (exact)
+{
+    v2h const h = { _Float16(int(int8_t(v >> (8 * firstByte)))), _Float16(int(int8_t(v >> (8 * firstByte + 8)))) };
+    return __builtin_bit_cast(uint32_t, h);
+}
+
 // Copies the int8 blob (src/WeightLayout.cpp:42-49: matrices, then fp32 scales, then int32
-// biases; W[c*IN + k]) into LDS in MFMA operand order.
+// biases; W[c*IN + k]) into LDS in MFMA operand order.  Returns true when layers 1..3 were staged
+// for the fp16 matrix instruction (see mlp_forward_f16): that needs, for every channel of those
+// layers, |bias - 113*sum(W)| + 240*sum|W| < 2^24.  Otherwise they are staged as int8 tiles.
 template <class V>
-__device__ void stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
+__device__ bool stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
 {
     constexpr int ins[4]   = { V::IN, V::H0, V::H1, V::H2 };
     constexpr int tiles[4] = { V::T0, V::T1, V::T2, V::T3 };
     constexpr int woff[4]  = { 0, V::W1_OFF, V::W2_OFF, V::W3_OFF };
     uint32_t const* blob32 = reinterpret_cast<uint32_t const*>(blob);
-    int tileBase = 0, chanBase = 0;
+
+    // scales and biases of every layer, in D-register order
+    {
+        int tileBase = 0, chanBase = 0;
 #pragma unroll
-    for (int l = 0; l < 4; ++l) {
-        int const in = ins[l];
-        for (int e = threadIdx.x; e < tiles[l] * 64 * 4; e += blockDim.x) {
-            int const d = e & 3, lane = (e >> 2) & 63, t = e >> 8;
-            int const i = lane & 15, g = lane >> 4;
-            int const row = 16 * t + i;
-            // layer 0: k-slot (g, 4d+r) = input 16g+4d+r.  layers >= 1: = channel 16d+4g+r.
-            int const k = (l == 0) ? (16 * g + 4 * d) : (16 * d + 4 * g);
-            uint32_t v = 0;
-            if (k < in) v = blob32[(woff[l] + row * in + k) >> 2];
-            if (V::FP8_WEIGHTS && l < 3) {
-                uint32_t p0 = 0, p1 = 0, p2 = 0;
+        for (int l = 0; l < 4; ++l) {
+            for (int e = threadIdx.x; e < tiles[l] * 16; e += blockDim.x) {
+                int const r = e & 3, g = (e >> 2) & 3, t = e >> 4;
+                int const c = chanBase + 16 * t + 4 * g + r;
+                lds.scale[tileBase + t][g][r] = reinterpret_cast<float const*>(blob + V::SCALE_OFF)[c];
+                lds.bias[tileBase + t][g][r]  = reinterpret_cast<int32_t const*>(blob + V::BIAS_OFF)[c];
+            }
+            tileBase += tiles[l];
+            chanBase += tiles[l] * 16;
+        }
+    }
+
+    // int8 tiles: all layers for the e4m3 variants, layer 0 otherwise
+    {
+        int tileBase = 0;
+#pragma unroll
+        for (int l = 0; l < (V::F16_LAYERS ? 1 : 4); ++l) {
+            int const in = ins[l];
+            for (int e = threadIdx.x; e < tiles[l] * 64 * 4; e += blockDim.x) {
+                int const d = e & 3, lane = (e >> 2) & 63, t = e >> 8;
+                int const i = lane & 15, g = lane >> 4;
+                // layer 0: k-slot (g, 4d+r) = input 16g+4d+r.  layers >= 1: = channel 16d+4g+r.
+                int const k = (l == 0) ? (16 * g + 4 * d) : (16 * d + 4 * g);
+                uint32_t const v = weight_dword(blob32, woff[l], 16 * t + i, in, k);
+                if (V::FP8_WEIGHTS && l < 3) {
+                    uint32_t p0 = 0, p1 = 0, p2 = 0;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        int32_t const W = e4m3_times_512((v >> (8 * r)) & 0xffu);
+                        p0 |= uint32_t(W & 63) << (8 * r);
+                        p1 |= uint32_t((W >> 6) & 63) << (8 * r);
+                        p2 |= (uint32_t(W >> 12) & 0xffu) << (8 * r);      // signed top plane
+                    }
+                    lds.w[0][tileBase + t][lane][d] = p0;
+                    lds.w[V::PLANES > 1 ? 1 : 0][tileBase + t][lane][d] = p1;
+                    lds.w[V::PLANES > 2 ? 2 : 0][tileBase + t][lane][d] = p2;
+                } else {
+                    lds.w[0][tileBase + t][lane][d] = v;
+                }
+            }
+            tileBase += tiles[l];
+        }
+    }
+    if constexpr (!V::F16_LAYERS) {
+        return false;
+    } else {
+        // One thread per channel of layers 1..3: row sums decide whether the fp16 path is exact.
+        bool fits = true;
+        int64_t shifted = 0;
+        int slotTile = 0, slotG = 0, slotR = 0;
+        if (threadIdx.x < V::LATE_CHANNELS) {
+            int const c = threadIdx.x;
+            int const l = c < V::H1 ? 1 : (c < V::H1 + V::H2 ? 2 : 3);
+            int const row = c - (l == 1 ? 0 : (l == 2 ? V::H1 : V::H1 + V::H2));
+            int const in = l == 1 ? V::H0 : (l == 2 ? V::H1 : V::H2);
+            int const off = l == 1 ? V::W1_OFF : (l == 2 ? V::W2_OFF : V::W3_OFF);
+            int32_t sum = 0, sumAbs = 0;
+            for (int k = 0; k < in; k += 4) {
+                uint32_t const v = blob32[(off + row * in + k) >> 2];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    int32_t const W = e4m3_times_512((v >> (8 * r)) & 0xffu);
-                    p0 |= uint32_t(W & 63) << (8 * r);
-                    p1 |= uint32_t((W >> 6) & 63) << (8 * r);
-                    p2 |= (uint32_t(W >> 12) & 0xffu) << (8 * r);      // signed top plane
+                    int const w = int(int8_t(v >> (8 * r)));
+                    sum += w;
+                    sumAbs += w < 0 ? -w : w;
                 }
-                lds.w[0][tileBase + t][lane][d] = p0;
-                lds.w[V::PLANES > 1 ? 1 : 0][tileBase + t][lane][d] = p1;
-                lds.w[V::PLANES > 2 ? 2 : 0][tileBase + t][lane][d] = p2;
-            } else {
-                lds.w[0][tileBase + t][lane][d] = v;
+            }
+            int32_t const bias = reinterpret_cast<int32_t const*>(blob + V::BIAS_OFF)[V::H0 + c];
+            shifted = int64_t(bias) - 113 * int64_t(sum);     // activations enter as q + 113 in [-15, 240]
+            int64_t const bound = (shifted < 0 ? -shifted : shifted) + 240 * int64_t(sumAbs);
+            fits = bound < (int64_t(1) << 24);
+            slotTile = V::T0 + (l == 1 ? 0 : (l == 2 ? V::T1 : V::T1 + V::T2)) + row / 16;
+            slotG = (row >> 2) & 3;
+            slotR = row & 3;
+        }
+        bool const useF16 = __syncthreads_and(fits ? 1 : 0) != 0;     // also orders the bias writes above
+        if (useF16) {
+            if (threadIdx.x < V::LATE_CHANNELS)
+                lds.bias[slotTile][slotG][slotR] = __builtin_bit_cast(int32_t, float(shifted));
+            // fp16 blocks.  Lane (i, kg) of the block of output tile t and input-tile pair p holds
+            // W[16t + i][16*(2p + e/4) + 4*kg + e%4], e = 0..7: the channels lane (j, kg) of the
+            // previous layer's D registers owns, in register order.
+            constexpr int base[4] = { 0, V::F16_L1, V::F16_L2, V::F16_L3 };
+            uint32_t* const late32 = reinterpret_cast<uint32_t*>(lds.late);
+#pragma unroll
+            for (int l = 1; l < 4; ++l) {
+                int const in = ins[l];
+                int const inTiles = tiles[l - 1], pairs = inTiles / 2, per = V::f16_units(inTiles);
+                // one work item = one (output tile, input tile, lane): 4 weights -> 2 dwords
+                for (int e = threadIdx.x; e < tiles[l] * inTiles * 64; e += blockDim.x) {
+                    int const lane = e & 63, rest = e >> 6;
+                    int const ti = rest % inTiles, t = rest / inTiles;
+                    int const i = lane & 15, kg = lane >> 4;
+                    uint32_t const v = blob32[(woff[l] + (16 * t + i) * in + 16 * ti + 4 * kg) >> 2];
+                    int const p = ti >> 1;
+                    // dword index inside `late`: paired blocks hold 4 dwords per lane, the tail block 2
+                    int const at = (p < pairs) ? ((base[l] + t * per + p * 64 + lane) * 4 + (ti & 1) * 2)
+                                               : ((base[l] + t * per + pairs * 64) * 4 + lane * 2);
+                    late32[at]     = halves_of_bytes(v, 0);
+                    late32[at + 1] = halves_of_bytes(v, 2);
+                }
+            }
+        } else {
+            int tileBase = 0;
+#pragma unroll
+            for (int l = 1; l < 4; ++l) {
+                int const in = ins[l];
+                for (int e = threadIdx.x; e < tiles[l] * 64 * 4; e += blockDim.x) {
+                    int const d = e & 3, lane = (e >> 2) & 63, t = e >> 8;
+                    int const i = lane & 15, g = lane >> 4;
+                    reinterpret_cast<uint32_t*>(lds.late)[((tileBase + t) * 64 + lane) * 4 + d] =
+                        weight_dword(blob32, woff[l], 16 * t + i, in, 16 * d + 4 * g);
+                }
+                tileBase += tiles[l];
             }
         }
-        for (int e = threadIdx.x; e < tiles[l] * 16; e += blockDim.x) {
-            int const r = e & 3, g = (e >> 2) & 3, t = e >> 4;
-            int const c = chanBase + 16 * t + 4 * g + r;
-            lds.scale[tileBase + t][g][r] = reinterpret_cast<float const*>(blob + V::SCALE_OFF)[c];
-            lds.bias[tileBase + t][g][r]  = reinterpret_cast<int32_t const*>(blob + V::BIAS_OFF)[c];
-        }
-        tileBase += tiles[l];
-        chanBase += tiles[l] * 16;
+        return useF16;
     }
 }
 
@@ -538,12 +655,12 @@ __device__ __forceinline__ uint32_t posenc_byte(float p)
 
 // Fills the phase tables.  For positionScale = 2^-k the encoding of texel x depends only on
 // x mod 2^k, and all arithmetic involved is exact, so table and per-lane evaluation agree; scales of
-// 1 and above have period 1 (k = 0).  One entry per thread, threads 0..126 fill both tables.
+// 1 and above have period 1 (k = 0).  One entry per thread, threads 0..62 fill both tables.
 template <class V>
 __device__ void build_posenc_tables(LdsT<V>& lds)
 {
     int const t = threadIdx.x;
-    if (t < 127) {
+    if (t < 63) {
         int const k = 31 - __builtin_clz(uint32_t(t + 1));   // floor(log2(t + 1))
         int const phase = t + 1 - (1 << k);
         float p = float(phase) * __builtin_ldexpf(1.f, -k);
@@ -599,7 +716,8 @@ __device__ __forceinline__ void mlp_forward(LdsT<V>& lds, int wave, int lane, ui
             for (int d = 0; d < 4; ++d) Y[b][d] = 0;
 #pragma unroll
         for (int t = 0; t < tiles[l]; ++t) {
-            uint4 const wa = *reinterpret_cast<uint4 const*>(&lds.w[0][tb + t][lane][0]);
+            uint4 const wa = (V::F16_LAYERS && l > 0) ? lds.late[(tb - V::T0 + t) * 64 + lane]
+                                                      : *reinterpret_cast<uint4 const*>(&lds.w[0][V::F16_LAYERS ? t : tb + t][lane][0]);
             v4i const A = v4i{ int(wa.x), int(wa.y), int(wa.z), int(wa.w) };
             v4i const C = *reinterpret_cast<v4i const*>(&lds.bias[tb + t][g][0]);
             v4f const Sc = *reinterpret_cast<v4f const*>(&lds.scale[tb + t][g][0]);
@@ -634,12 +752,135 @@ __device__ __forceinline__ void mlp_forward(LdsT<V>& lds, int wave, int lane, ui
     }
 
     // output layer
-    uint4 const wa = *reinterpret_cast<uint4 const*>(&lds.w[0][tb][lane][0]);
+    uint4 const wa = V::F16_LAYERS ? lds.late[(tb - V::T0) * 64 + lane] : *reinterpret_cast<uint4 const*>(&lds.w[0][V::F16_LAYERS ? 0 : tb][lane][0]);
     v4i const A = v4i{ int(wa.x), int(wa.y), int(wa.z), int(wa.w) };
     v4i const C = *reinterpret_cast<v4i const*>(&lds.bias[tb][g][0]);
     S = *reinterpret_cast<v4f const*>(&lds.scale[tb][g][0]);
 #pragma unroll
     for (int b = 0; b < 4; ++b) D[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
+}
+
+// ---- layers 1..3 on the fp16 matrix instruction --------------------------------------------
+//
+// Same integers, fewer vector operations.  The int8 matrix instruction returns int32, which costs a
+// conversion per activation, and its operands are signed bytes, which forces the "- 113" and the
+// clamp of min(x, 3) into fp32.  Here the previous layer's activations enter as the fp16 numbers
+// u = q + 113 in [-15, 240] and the weights as fp16 integers; products and every partial sum are
+// integers below 2^24 (stage_weights checked that), so the fp32 accumulator of
+// v_mfma_f32_16x16x32_f16 holds exactly acc = bias + sum W*(u - 113) once the accumulator starts at
+// bias - 113*sum(W).  The epilogue is then 6 operations per activation:
+//   v_mul (scale), v_fma clamp, v_mul (x*t), v_mul (80), v_rndne, and half each of
+//   v_cvt_pkrtz_f16_f32 and v_pk_min_f16 (the cap at 240 = the min(x, 3) of the definition: below 3
+//   both agree term by term, from 3 on t = 1 and x*80 >= 240).
+
+// HGELU-clamp + requantise of four accumulators to the fp16 values q + 113, two dwords.
+template <class Acc>
+__device__ __forceinline__ void activate4_h(Acc acc, v4f scale, uint32_t (&out)[2])
+{
+    float v[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        float const x = float(acc[r]) * scale[r];
+        float t = __builtin_fmaf(x, 0.333333f, 0.5f);
+        t = fminf(fmaxf(t, 0.f), 1.f);
+        float const y = x * t;
+        v[r] = __builtin_rintf(y * 80.f);
+    }
+    v2h const cap = { _Float16(240.f), _Float16(240.f) };
+    v2h const lo = __builtin_bit_cast(v2h, __builtin_amdgcn_cvt_pkrtz(v[0], v[1]));
+    v2h const hi = __builtin_bit_cast(v2h, __builtin_amdgcn_cvt_pkrtz(v[2], v[3]));
+    out[0] = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(lo, cap));
+    out[1] = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(hi, cap));
+}
+
+// acc[b] += W(tile t of the layer at `base`) * H[b], for the four 16-texel blocks of the wave.
+template <class V, int IN_TILES>
+__device__ __forceinline__ void f16_tile(LdsT<V> const& lds, int base, int t, int lane, uint32_t const (&H)[4][4][2], v4f (&acc)[4])
+{
+    constexpr int PAIRS = IN_TILES / 2, PER = V::f16_units(IN_TILES);
+    uint4 const* const block = lds.late + base + t * PER;
+#pragma unroll
+    for (int p = 0; p < PAIRS; ++p) {
+        v8h const A = __builtin_bit_cast(v8h, block[p * 64 + lane]);
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            uint4 const h = make_uint4(H[b][2 * p][0], H[b][2 * p][1], H[b][2 * p + 1][0], H[b][2 * p + 1][1]);
+            acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, __builtin_bit_cast(v8h, h), acc[b], 0, 0, 0);
+        }
+    }
+    if constexpr (IN_TILES % 2 == 1) {
+        v4h const A = __builtin_bit_cast(v4h, reinterpret_cast<uint2 const*>(block + PAIRS * 64)[lane]);
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            uint2 const h = make_uint2(H[b][IN_TILES - 1][0], H[b][IN_TILES - 1][1]);
+            acc[b] = __builtin_amdgcn_mfma_f32_16x16x16f16(A, __builtin_bit_cast(v4h, h), acc[b], 0, 0, 0);
+        }
+    }
+}
+
+template <class V, int IN_TILES, int OUT_TILES>
+__device__ __forceinline__ void f16_hidden_layer(LdsT<V> const& lds, int base, int tileBase, int lane,
+                                                 uint32_t const (&Hin)[4][4][2], uint32_t (&Hout)[4][4][2])
+{
+    int const g = lane >> 4;
+#pragma unroll
+    for (int t = 0; t < OUT_TILES; ++t) {
+        v4f const C = *reinterpret_cast<v4f const*>(&lds.bias[tileBase + t][g][0]);       // float(bias - 113*sum W)
+        v4f const Sc = *reinterpret_cast<v4f const*>(&lds.scale[tileBase + t][g][0]);
+        v4f acc[4] = { C, C, C, C };
+        f16_tile<V, IN_TILES>(lds, base, t, lane, Hin, acc);
+#pragma unroll
+        for (int b = 0; b < 4; ++b) activate4_h(acc[b], Sc, Hout[b][t]);
+    }
+}
+
+// The network for the 64 texels of one wave with layers 1..3 on the fp16 matrix instruction.
+// Same interface as mlp_forward, except that D holds the output layer's accumulators as floats
+// (exact integers).
+template <class V>
+__device__ __forceinline__ void mlp_forward_f16(LdsT<V>& lds, int wave, int lane, uint32_t const (&in)[16], v4f (&D)[4], v4f& S)
+{
+    int const j = lane & 15, g = lane >> 4;
+    {
+        uint4* dst = reinterpret_cast<uint4*>(&lds.in[wave][lane][0]);
+        dst[0] = make_uint4(in[0], in[1], in[2], in[3]);
+        dst[1] = make_uint4(in[4], in[5], in[6], in[7]);
+        dst[2] = make_uint4(in[8], in[9], in[10], in[11]);
+        dst[3] = make_uint4(in[12], in[13], in[14], in[15]);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    v4i X[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        uint4 const t = *reinterpret_cast<uint4 const*>(&lds.in[wave][b * 16 + j][4 * g]);
+        X[b] = v4i{ int(t.x), int(t.y), int(t.z), int(t.w) };
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    // layer 0: int8 inputs, int32 accumulators
+    uint32_t Ha[4][4][2], Hb[4][4][2];
+#pragma unroll
+    for (int t = 0; t < V::T0; ++t) {
+        uint4 const wa = *reinterpret_cast<uint4 const*>(&lds.w[0][t][lane][0]);
+        v4i const A = v4i{ int(wa.x), int(wa.y), int(wa.z), int(wa.w) };
+        v4i const C = *reinterpret_cast<v4i const*>(&lds.bias[t][g][0]);
+        v4f const Sc = *reinterpret_cast<v4f const*>(&lds.scale[t][g][0]);
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+            activate4_h(__builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0), Sc, Ha[b][t]);
+    }
+    f16_hidden_layer<V, V::T0, V::T1>(lds, V::F16_L1, V::T0, lane, Ha, Hb);
+    f16_hidden_layer<V, V::T1, V::T2>(lds, V::F16_L2, V::T0 + V::T1, lane, Hb, Ha);
+
+    constexpr int outTile = V::T0 + V::T1 + V::T2;
+    v4f const C = *reinterpret_cast<v4f const*>(&lds.bias[outTile][g][0]);
+    S = *reinterpret_cast<v4f const*>(&lds.scale[outTile][g][0]);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) D[b] = C;
+    f16_tile<V, V::T2>(lds, V::F16_L3, 0, lane, Ha, D);
 }
 
 template <class V>
@@ -669,6 +910,7 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     build_posenc_tables<V>(lds);
 
     uint8_t const* stagedBlob = nullptr;
+    bool useF16 = false;                                     // uniform: how layers 1..3 of the staged set run
     int entry = 0;
 
     for (int tile = tileBegin; tile < tileEnd; ++tile) {
@@ -677,7 +919,7 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
 
         if (m.weights != stagedBlob) {                       // uniform across the workgroup
             __syncthreads();
-            stage_weights<V>(lds, m.weights);
+            useF16 = stage_weights<V>(lds, m.weights);
             stagedBlob = m.weights;
             __syncthreads();                                 // also publishes the tables built above
         }
@@ -696,7 +938,14 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
             else        prepare_inputs_general<V>(m, x, y, in);
         }
         // ---- 2.-4. transpose, hidden layers, output layer
-        {
+        if (V::F16_LAYERS && useF16) {
+            v4f D[4];
+            v4f S;
+            mlp_forward_f16<V>(lds, wave, lane, in, D, S);
+            if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)      store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, x0 + j, y0, 4 * g);
+            else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)       store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
+            else                                                       store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
+        } else {
             v4i D[4];
             v4f S;
             mlp_forward<V>(lds, wave, lane, in, c143, D, S);
@@ -732,7 +981,7 @@ query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __res
         lds.lut2[threadIdx.x & 0xffu] = (x * 85u) ^ 0x80808080u;
     }
     build_posenc_tables<V>(lds);
-    stage_weights<V>(lds, mips[0].weights);
+    bool const useF16 = stage_weights<V>(lds, mips[0].weights);
     __syncthreads();
 
     uint64_t const numBlocks = (numQueries + 255) / 256;
@@ -751,9 +1000,18 @@ query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __res
         if (__all(m.fast != 0)) prepare_inputs_fast<V>(m, lds, x, y, in);     // every lane's mip is power-of-two sized
         else                    prepare_inputs_general<V>(m, x, y, in);
 
-        v4i D[4];
+        // output-layer accumulators as floats: exact either way (|acc| < 2^24 on the fp16 path; the
+        // int32 -> float conversion is the definition's on the int8 path)
+        v4f F[4];
         v4f S;
-        mlp_forward<V>(lds, wave, lane, in, c143, D, S);
+        if (V::F16_LAYERS && useF16) {
+            mlp_forward_f16<V>(lds, wave, lane, in, F, S);
+        } else {
+            v4i D[4];
+            mlp_forward<V>(lds, wave, lane, in, c143, D, S);
+#pragma unroll
+            for (int b = 0; b < 4; ++b) F[b] = v4f{ float(D[b][0]), float(D[b][1]), float(D[b][2]), float(D[b][3]) };
+        }
 
         // lane (j, g) holds channels 4g..4g+3 of query q0 + 16b + j; validity travels by shuffle
 #pragma unroll
@@ -761,8 +1019,8 @@ query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __res
             uint64_t const q = q0 + uint64_t(16 * b + j);
             int const ok = __shfl(validMip ? 1 : 0, 16 * b + j, 64);
             if (q >= numQueries) continue;
-            uint32_t h01 = to_half2_bits(float(D[b][0]) * S[0], float(D[b][1]) * S[1]);
-            uint32_t h23 = to_half2_bits(float(D[b][2]) * S[2], float(D[b][3]) * S[3]);
+            uint32_t h01 = to_half2_bits(F[b][0] * S[0], F[b][1] * S[1]);
+            uint32_t h23 = to_half2_bits(F[b][2] * S[2], F[b][3] * S[3]);
             if (!ok) { h01 = 0; h23 = 0; }
             *reinterpret_cast<u32x2*>(out + q * 16 + 4 * g) = u32x2{ h01, h23 };
         }
@@ -789,6 +1047,33 @@ __global__ void selftest_mfma_kernel(int8_t const* __restrict__ a, int8_t const*
     v4i const D = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, B, v4i{0, 0, 0, 0}, 0, 0, 0);
 #pragma unroll
     for (int r = 0; r < 4; ++r) d[(4 * g + r) * 16 + ij] = D[r];      // D[i = 4g+r][j]
+}
+
+// D = A * B + C with the fp16 MFMA and the operand layouts the decode kernel assumes: for K = 32,
+// A[i][k] sits in lane i + 16*(k/8), element k%8 (B alike with column j), for K = 16 in lane
+// i + 16*(k/4), element k%4; D[i][j] in lane j + 16*(i/4), element i%4.
+__global__ void selftest_mfma_f16_kernel(_Float16 const* __restrict__ a, _Float16 const* __restrict__ b,
+                                         float const* __restrict__ c, float* __restrict__ d, int depth)
+{
+    int const lane = threadIdx.x & 63;
+    int const ij = lane & 15, g = lane >> 4;
+    v4f C;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) C[r] = c[(4 * g + r) * 16 + ij];
+    v4f D;
+    if (depth == 32) {
+        v8h A, B;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { A[e] = a[ij * 32 + 8 * g + e]; B[e] = b[(8 * g + e) * 16 + ij]; }
+        D = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B, C, 0, 0, 0);
+    } else {
+        v4h A, B;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { A[e] = a[ij * 16 + 4 * g + e]; B[e] = b[(4 * g + e) * 16 + ij]; }
+        D = __builtin_amdgcn_mfma_f32_16x16x16f16(A, B, C, 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) d[(4 * g + r) * 16 + ij] = D[r];
 }
 
 // ---- host-callable launchers ------------------------------------------------------------
@@ -871,6 +1156,13 @@ int resident_workgroups_per_cu(int variant)
 hipError_t launch_selftest_mfma(int8_t const* a, int8_t const* b, int32_t* d, hipStream_t stream)
 {
     hipLaunchKernelGGL(selftest_mfma_kernel, dim3(1), dim3(64), 0, stream, a, b, d);
+    return hipGetLastError();
+}
+
+hipError_t launch_selftest_mfma_f16(uint16_t const* a, uint16_t const* b, float const* c, float* d, int depth, hipStream_t stream)
+{
+    hipLaunchKernelGGL(selftest_mfma_f16_kernel, dim3(1), dim3(64), 0, stream,
+                       reinterpret_cast<_Float16 const*>(a), reinterpret_cast<_Float16 const*>(b), c, d, depth);
     return hipGetLastError();
 }
 

@@ -135,7 +135,7 @@ bool axis_params(int32_t size, int32_t grid, uint32_t& packed, int& n)
 // Conditions: every size a power of two (then every float operation of the general stage is
 // exact and the integer form gives the same bytes); bilinear weights of at most 8 fractional
 // bits in total (16-bit lanes of the packed filter cannot overflow); positionScale a power of
-// two, at least 2^-6 (the encoding has a period of at most 64 texels).
+// two, at least 2^-5 (the encoding has a period of at most 32 texels).
 void fill_fast_path(NtcHipDecoderSpec const& spec, DevMip& e)
 {
     e.fast = 0;
@@ -148,7 +148,7 @@ void fill_fast_path(NtcHipDecoderSpec const& spec, DevMip& e)
     if (grid_bytes(e.lrWidth, e.lrHeight, spec.lrFeatures, spec.lrBits) >= (1ull << 31)) return;
     int exp2 = 0;
     float const mant = std::frexp(e.positionScale, &exp2);      // scale = mant * 2^exp2, mant in [0.5, 1)
-    if (!(mant == 0.5f) || exp2 - 1 < -6 || exp2 - 1 > 20) return;
+    if (!(mant == 0.5f) || exp2 - 1 < -5 || exp2 - 1 > 20) return;
     int const k = -(exp2 - 1);                                  // scale = 2^-k
     e.posMask = k > 0 ? (1u << k) - 1u : 0u;
     e.fast = 1;
@@ -658,6 +658,29 @@ int ntc_hip_selftest_mfma(const int8_t* a16x64, const int8_t* b64x16, int32_t* d
     HIP_TRY(hipStreamSynchronize(g_lib.stream));
     HIP_TRY(hipMemcpy(d16x16, d, 1024, hipMemcpyDeviceToHost));
     (void)hipFree(a); (void)hipFree(b); (void)hipFree(d);
+    return 0;
+}
+
+int ntc_hip_selftest_mfma_f16(const uint16_t* aHalves, const uint16_t* bHalves, const float* c16x16, float* d16x16, int32_t depth)
+{
+    if (int r = require_init()) return r;
+    if (!aHalves || !bHalves || !c16x16 || !d16x16) { set_error("ntc_hip_selftest_mfma_f16: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
+    if (depth != 16 && depth != 32) { set_error("ntc_hip_selftest_mfma_f16: depth must be 16 or 32."); return NTC_HIP_ERR_INVALID_ARG; }
+    size_t const operandBytes = size_t(16) * size_t(depth) * 2;
+    uint8_t* dev = nullptr;
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&dev), 4096));
+    uint16_t* a = reinterpret_cast<uint16_t*>(dev);
+    uint16_t* b = reinterpret_cast<uint16_t*>(dev + 1024);
+    float* c = reinterpret_cast<float*>(dev + 2048);
+    float* d = reinterpret_cast<float*>(dev + 3072);
+    hipError_t e = hipMemcpy(a, aHalves, operandBytes, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(b, bHalves, operandBytes, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(c, c16x16, 1024, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = launch_selftest_mfma_f16(a, b, c, d, depth, g_lib.stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(g_lib.stream);
+    if (e == hipSuccess) e = hipMemcpy(d16x16, d, 1024, hipMemcpyDeviceToHost);
+    (void)hipFree(dev);
+    HIP_TRY(e);
     return 0;
 }
 

@@ -40,6 +40,36 @@ def test_mfma_operand_layout(device):
     assert np.array_equal(d, a.astype(np.int64) @ b.astype(np.int64))
 
 
+@pytest.mark.parametrize("depth", [16, 32])
+def test_mfma_f16_integer_sums_are_exact(device, depth):
+    """The fp16 matrix instruction with integer-valued operands: layout, and exactness of the fp32
+    accumulation while every partial sum stays below 2^24 -- including accumulator inputs that
+    leave only a few units of headroom, positive and negative."""
+    from importlib import import_module
+    abi = import_module("rtxntc-library_amd").abi
+    rng = np.random.default_rng(6 + depth)
+    for trial in range(8):
+        a = rng.integers(-127, 128, size=(16, depth))
+        b = rng.integers(-15, 241, size=(depth, 16))
+        if trial == 1:                                   # worst case magnitudes, all one sign
+            a[:], b[:] = 127, 240
+        if trial == 2:
+            a[:], b[:] = -127, 240
+        room = (1 << 24) - 1 - np.abs(a).sum(axis=1, keepdims=True) * 240
+        c = rng.integers(-room, room + 1, size=(16, 16))
+        if trial in (1, 3):
+            c = np.broadcast_to(room, (16, 16)).copy()      # the sum ends exactly at 2^24 - 1 ...
+        if trial in (2, 4):
+            c = -np.broadcast_to(room, (16, 16)).copy()     # ... or at -(2^24 - 1) for all-negative rows
+        exact = a @ b + c
+        assert np.abs(exact).max() < (1 << 24)
+        ah, bh = a.astype(np.float16), b.astype(np.float16)
+        cf, d = c.astype(np.float32), np.zeros((16, 16), dtype=np.float32)
+        assert np.array_equal(ah.astype(np.int64), a) and np.array_equal(cf.astype(np.int64), c)
+        abi.check(device.lib.ntc_hip_selftest_mfma_f16(ah.ctypes.data, bh.ctypes.data, cf.ctypes.data, d.ctypes.data, depth))
+        assert np.array_equal(d.astype(np.int64), exact), (depth, trial)
+
+
 @pytest.mark.parametrize("scale_range", [(-10.0, -4.0), ACTIVE])
 def test_cfg0_plumbing_512_fp16(ntc, device, scale_range):
     """BASELINE config 0: 512x512, one mip, 8 channels, 64-48-32 int8, fp16 planar output."""
@@ -137,6 +167,27 @@ def test_extreme_weights_saturate_cleanly(ntc, device):
     case = cfg_case(ntc, spec, 64, 64, 1, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=9, weights=blob)
     expected, got = run_both(device, case)
     assert_equal_bytes(expected, got, "extreme weights")
+
+
+@pytest.mark.parametrize("slack", [-1, 0, 1, 4096])
+def test_fp16_layer_path_boundary(ntc, device, slack):
+    """Layers 1..3 run on the fp16 matrix instruction only while |bias - 113*sum(W)| + 240*sum|W| stays
+    below 2^24 for every channel; one channel is put exactly at (slack = -1: just inside), on and just
+    past that limit, with both signs, so both code paths and the switch between them face the checker."""
+    spec = ntc.presets.spec_cfg01()
+    layout = ntc.synth.weight_layout(spec)
+    for sign in (1, -1):
+        blob = ntc.synth.make_weights(spec, 40 + slack % 7, scale_log2_range=(-22.0, -21.0))
+        ins, outs = [64, 64, 48, 32], [64, 48, 32, 16]
+        bias = blob[layout.biasOffset[0]:layout.bufferSize].view(np.int32)
+        for layer, row in ((1, 5), (2, 17), (3, 9)):
+            w = blob[layout.weightOffset[layer]: layout.weightOffset[layer] + ins[layer] * outs[layer]].view(np.int8).reshape(outs[layer], ins[layer])
+            total, total_abs = int(w[row].astype(np.int64).sum()), int(np.abs(w[row].astype(np.int64)).sum())
+            shifted = sign * ((1 << 24) + slack - 240 * total_abs)        # |shifted| + 240*sum|W| = 2^24 + slack
+            bias[sum(outs[:layer]) + row] = shifted + 113 * total
+        case = cfg_case(ntc, spec, 128, 64, 3, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=50, weights=blob)
+        expected, got = run_both(device, case)
+        assert_equal_bytes(expected, got, f"fp16 path boundary, slack {slack}, sign {sign}")
 
 
 def test_decode_is_idempotent_and_timed_variant_matches(ntc, device):
