@@ -179,7 +179,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved_gbs / HBM_PEAK_GBS,
                      # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE (profiles/), headline workload only
-                     "traffic": 764.4e6 if (wl == "cfg1" and fmt_name == "fp16" and not args.size) else None,
+                     "traffic": 766.4e6 if (wl == "cfg1" and fmt_name == "fp16" and not args.size) else None,
                      "kernel_ms": kernel_ms, "bytes_per_texel": bytes_per_texel,
                      "mfma_achieved_tops": achieved_tops, "mfma_frac": achieved_tops / INT8_PEAK_TOPS},
         "cpu_baseline": cpu,
