@@ -157,6 +157,15 @@ void PositionConstants(NtcHipMipDesc& d)
 }
 } // namespace
 
+// For the other translation units of this library.
+void SetQuantizeError(char const* fmt, ...)
+{
+    va_list args;
+    va_start(args, fmt);
+    vsnprintf(t_message, sizeof t_message, fmt, args);
+    va_end(args);
+}
+
 class Context;
 
 // src/TextureMetadata.cpp:30-75 (name and channel range only)

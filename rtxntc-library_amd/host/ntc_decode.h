@@ -254,7 +254,26 @@ public:
     virtual ~IContext() = default;
 };
 
+// One layer of a float MLP: weights[out][in] row-major, bias[out].
+struct FloatLayerDesc
+{
+    int inputChannels = 0;
+    int outputChannels = 0;
+    float const* weights = nullptr;
+    float const* bias = nullptr;
+};
+// Maps an output channel from the network's range to linear values: v * scale + bias
+// (optimalToLinearScale / Bias of src/ChannelInfo.h, folded into the output layer by the quantiser).
+struct OutputChannelTransform { float scale = 1.f; float bias = 0.f; };
+
 extern "C" {
+// An addition: quantises a four-layer float MLP into the GenericInt8 weight blob
+// (src/WeightLayout.cpp:42-49) as the reference's encoder does (cuda::QuantizeNetwork,
+// src/Quantizer.cu:88-208,266-283), on the host.  pOutSize (optional) receives the blob size;
+// outputTransforms (optional) holds one entry per output channel.
+Status QuantizeNetworkInt8(FloatLayerDesc const* layers, int numLayers, OutputChannelTransform const* outputTransforms,
+    void* pOutBlob, size_t blobSize, size_t* pOutSize);
+
 // include/libntc/ntc.h:1307-1331.  CreateContext returns CudaUnavailable together with a usable
 // context when no device can be used (src/PublicFunctions.cpp:161).
 uint32_t GetInterfaceVersion();

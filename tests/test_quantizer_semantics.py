@@ -25,12 +25,16 @@ def quantize_layer_int8(w, b, input_layer):
     for c in range(n_out):
         col = w[:, c].astype(np.float32)
         limit = np.float32(max(abs(col.max()), abs(col.min())))                # Quantizer.cu:99-111
-        q = np.float32(127.5) * col / limit
-        q = np.where(q >= 0, np.floor(q + 0.5), np.ceil(q - 0.5))              # round(): half away from zero
+        # even input indices: (w * 127.5) * (1 / limit); odd ones: w * (127.5 / limit)   (Quantizer.cu:125-133)
+        q = np.empty(n_in, dtype=np.float32)
+        q[0::2] = (col[0::2] * np.float32(127.5)).astype(np.float32) * (np.float32(1) / limit)
+        q[1::2] = col[1::2] * (np.float32(127.5) / limit)
+        q = np.where(q >= 0, np.floor(q + np.float32(0.5)), np.ceil(q - np.float32(0.5)))   # round(): half away from zero
         q = np.clip(q, -127, 127)                                              # Quantizer.cu:116-131
         wq[c] = q.astype(np.int8)
-        w_deq[:, c] = (q * limit / np.float32(127.5)).astype(np.float32)
-        layer_scale = limit / np.float32(127.5)
+        iscale = np.float32(1) / np.float32(127.5)                             # `1 / scale`, a float constant (:117)
+        w_deq[:, c] = ((q.astype(np.float32) * limit).astype(np.float32) * iscale).astype(np.float32)
+        layer_scale = limit * iscale
         layer_bias = np.float32(b[c])
         if input_layer:
             layer_scale = layer_scale / np.float32(127.5)                      # tin::InputQuant::scale, :157-160
@@ -38,8 +42,8 @@ def quantize_layer_int8(w, b, input_layer):
             layer_scale = layer_scale * np.float32(3.1875 / 255)               # ActHGELUClamp::step = 1/80
             layer_bias = layer_bias - np.float32(int(q.sum()) * -113) * layer_scale      # :163-164
         scale[c] = layer_scale
-        t = np.float64(layer_bias) / np.float64(layer_scale)
-        bias_i[c] = int(np.floor(t + 0.5) if t >= 0 else np.ceil(t - 0.5))     # roundf, :202
+        t = np.float64(np.float32(layer_bias) / np.float32(layer_scale))       # float division, then roundf (:202)
+        bias_i[c] = int(np.floor(t + 0.5) if t >= 0 else np.ceil(t - 0.5))
     return wq, scale, bias_i, w_deq
 
 
@@ -64,3 +68,157 @@ def test_integer_layer_equals_dequantised_float_layer(oracle, n_in, n_out, input
         want = b.astype(np.float64) + a_real @ w_deq.astype(np.float64)
         tol = 0.5 * scale.astype(np.float64) * 1.001 + 2e-6 * (1 + np.abs(want))
         assert np.all(np.abs(r.astype(np.float64) - want) <= tol), (trial, np.abs(r - want).max(), tol.min())
+
+
+# ---- the host library's quantiser (rtxntc-library_amd/host/NtcQuantize.cpp) ------------------------
+
+import ctypes as C
+import os
+
+HOST_LIB = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "rtxntc-library_amd", "host", "libntc_amd.so")
+
+
+class FloatLayerDesc(C.Structure):
+    _fields_ = [("inputChannels", C.c_int), ("outputChannels", C.c_int), ("weights", C.c_void_p), ("bias", C.c_void_p)]
+
+
+class OutputChannelTransform(C.Structure):
+    _fields_ = [("scale", C.c_float), ("bias", C.c_float)]
+
+
+def host_lib():
+    lib = C.CDLL(HOST_LIB)
+    lib.QuantizeNetworkInt8.restype = C.c_int
+    lib.QuantizeNetworkInt8.argtypes = [C.POINTER(FloatLayerDesc), C.c_int, C.POINTER(OutputChannelTransform), C.c_void_p, C.c_size_t, C.POINTER(C.c_size_t)]
+    lib.GetLastErrorMessage.restype = C.c_char_p
+    return lib
+
+
+def float_network(rng, widths):
+    """Random float MLP with fp16-representable values: [(w [in][out], b [out])]."""
+    layers = []
+    for n_in, n_out in zip(widths[:-1], widths[1:]):
+        w = (rng.standard_normal((n_in, n_out)) * (1.5 / np.sqrt(n_in))).astype(np.float16).astype(np.float32)
+        b = (rng.standard_normal(n_out) * 0.2).astype(np.float16).astype(np.float32)
+        layers.append((w, b))
+    return layers
+
+
+def quantize_with_host_library(lib, layers, transforms=None):
+    descs = (FloatLayerDesc * len(layers))()
+    keep = []
+    for d, (w, b) in zip(descs, layers):
+        rows = np.ascontiguousarray(w.T)                  # the library takes weights[out][in]
+        bias = np.ascontiguousarray(b)
+        keep += [rows, bias]
+        d.inputChannels, d.outputChannels, d.weights, d.bias = w.shape[0], w.shape[1], rows.ctypes.data, bias.ctypes.data
+    size = C.c_size_t(0)
+    t = None
+    if transforms is not None:
+        t = (OutputChannelTransform * len(transforms))(*[OutputChannelTransform(s, o) for s, o in transforms])
+    assert lib.QuantizeNetworkInt8(descs, len(layers), t, None, 0, C.byref(size)) == 10      # InvalidArgument, size reported
+    blob = np.zeros(size.value, dtype=np.uint8)
+    assert lib.QuantizeNetworkInt8(descs, len(layers), t, blob.ctypes.data, blob.size, None) == 0, lib.GetLastErrorMessage()
+    return blob
+
+
+@pytest.mark.parametrize("widths", [(64, 64, 48, 32, 16), (48, 64, 48, 32, 16), (64, 48, 48, 32, 16)])
+def test_host_quantiser_equals_the_numpy_restatement(widths):
+    """Bit equality: both follow src/Quantizer.cu:88-208 operation by operation in IEEE binary32."""
+    lib = host_lib()
+    rng = np.random.default_rng(sum(widths))
+    layers = float_network(rng, widths)
+    blob = quantize_with_host_library(lib, layers)
+    weight_bytes = sum(a * b for a, b in zip(widths[:-1], widths[1:]))
+    channels = sum(widths[1:])
+    assert blob.size == weight_bytes + 8 * channels
+    w_at, c_at = 0, 0
+    for index, (w, b) in enumerate(layers):
+        wq, scale, bias_i, _ = quantize_layer_int8(w, b, index == 0)
+        n_in, n_out = w.shape
+        assert np.array_equal(blob[w_at: w_at + n_in * n_out].view(np.int8).reshape(n_out, n_in), wq), index
+        assert np.array_equal(blob[weight_bytes + 4 * c_at: weight_bytes + 4 * (c_at + n_out)].view(np.float32), scale), index
+        assert np.array_equal(blob[weight_bytes + 4 * channels + 4 * c_at: weight_bytes + 4 * channels + 4 * (c_at + n_out)].view(np.int32), bias_i), index
+        w_at += n_in * n_out
+        c_at += n_out
+
+
+def test_host_quantiser_special_cases_and_errors():
+    lib = host_lib()
+    rng = np.random.default_rng(3)
+    widths = (64, 64, 48, 32, 16)
+    layers = float_network(rng, widths)
+    layers[3][0][:, 5] = 0.0                                     # a constant output channel: zero scale
+    layers[3][1][5] = 0.25
+    transforms = [(1.0, 0.0)] * 16
+    transforms[2] = (0.5, 0.125)                                 # optimal-to-linear mapping of channel 2
+    transforms[7] = (0.0, 0.75)                                  # a constant image channel maps with scale 0
+    blob = quantize_with_host_library(lib, layers, transforms)
+    plain = quantize_with_host_library(lib, layers)
+    weight_bytes, channels = 9216, 160
+    scale = blob[weight_bytes: weight_bytes + 4 * channels].view(np.float32)
+    bias = blob[weight_bytes + 4 * channels:].view(np.int32)
+    w3 = blob[64 * 64 + 64 * 48 + 48 * 32: weight_bytes].view(np.int8).reshape(16, 32)
+    assert scale[144 + 5] == np.float32(1 / 65536) and bias[144 + 5] == 16384 and not w3[5].any()     # Quantizer.cu:181-198
+    assert scale[144 + 7] == np.float32(1 / 65536) and bias[144 + 7] == 49152 and not w3[7].any()
+    plain_scale = plain[weight_bytes: weight_bytes + 4 * channels].view(np.float32)
+    assert scale[144 + 2] == np.float32(plain_scale[144 + 2] * np.float32(0.5))
+    # (x + bias_i) * scale of the transformed channel = 0.5 * (plain value) + 0.125 at x = 0, to half a step
+    plain_bias = plain[weight_bytes + 4 * channels:].view(np.int32)
+    assert abs(bias[144 + 2] * float(scale[144 + 2]) - (0.5 * plain_bias[144 + 2] * float(plain_scale[144 + 2]) + 0.125)) <= float(scale[144 + 2])
+    # argument errors
+    descs = (FloatLayerDesc * 4)()
+    assert lib.QuantizeNetworkInt8(descs, 3, None, None, 0, None) == 16 and b"numLayers" in lib.GetLastErrorMessage()
+    assert lib.QuantizeNetworkInt8(None, 4, None, None, 0, None) == 10
+    assert lib.QuantizeNetworkInt8(descs, 4, None, None, 0, None) == 10 and b"NULL" in lib.GetLastErrorMessage()
+
+
+def test_quantised_network_tracks_the_float_network(ntc, oracle):
+    """End to end on the checker: quantise a float MLP with the host library, decode a small texture
+    set with the blob, and compare with the float MLP evaluated on the same (de-quantised) inputs.
+    Quantisation noise only: a few steps of 1/80 through three hidden layers."""
+    lib = host_lib()
+    rng = np.random.default_rng(11)
+    widths = (64, 64, 48, 32, 16)
+    layers = float_network(rng, widths)
+    blob = quantize_with_host_library(lib, layers)
+    from cases import cfg_case
+    spec = ntc.presets.spec_cfg01()
+    case = cfg_case(ntc, spec, 32, 32, 1, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=12, weights=blob)
+    host = case.host_set()
+    host.decode(threads=4)
+    got = host.output.view(np.float16).astype(np.float64).reshape(32, 8, 32, 2).transpose(0, 2, 1, 3).reshape(32, 32, 16)
+    # float network on the same int8 inputs
+    import np_decoder
+    layout = ntc.synth.weight_layout(spec)
+    inputs, _ = np_decoder.decode_mip(spec, layout, blob, case.latents.view(np.uint16), case.mips[0])
+    x = inputs.reshape(-1, 64).astype(np.float64) / 127.5
+    for index, (w, b) in enumerate(layers):
+        x = x @ w.astype(np.float64) + b.astype(np.float64)
+        if index < 3:
+            x = np.minimum(x, 3.0) * np.clip(x / 3.0 + 0.5, 0.0, 1.0)
+    want = x.reshape(32, 32, 16)
+    err = np.abs(got - want)
+    assert err.max() < 0.15 and err.mean() < 0.02, (err.max(), err.mean())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("preset", ["cfg01", "ref092"])
+def test_gpu_decode_with_a_quantised_float_network(ntc, device, preset):
+    """A blob produced by the host quantiser (realistic scales and biases, unlike the synthetic
+    blobs of the other tests) decodes bit-exactly."""
+    from cases import cfg_case, ref_case, first_mismatch
+    lib = host_lib()
+    rng = np.random.default_rng(21)
+    if preset == "cfg01":
+        blob = quantize_with_host_library(lib, float_network(rng, (64, 64, 48, 32, 16)))
+        case = cfg_case(ntc, ntc.presets.spec_cfg01(), 512, 256, 6, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=22, weights=blob)
+    else:
+        blob = quantize_with_host_library(lib, float_network(rng, (48, 64, 48, 32, 16)))
+        case = ref_case(ntc, ntc.presets.spec_ref092(16), 512, 256, 6, 2, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=23, weights=blob)
+    host = case.host_set()
+    host.decode(threads=8)
+    dset = case.device_set(device)
+    device.decode([dset])
+    device.synchronize()
+    assert first_mismatch(host.output, case.d_output.download()) is None
