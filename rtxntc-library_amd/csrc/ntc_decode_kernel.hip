@@ -163,14 +163,14 @@ __device__ __forceinline__ uint32_t to_half2_bits(float a, float b)
 }
 
 // WriteImageChannel UNORM8 (src/ImageProcessing.cu:146-149): u8(clamp(roundf(v * 255), 0, 255)) of
-// the stored half.  v*255 is exact (11-bit x 8-bit significands); for such values
-// floor(v*255 + 1/2) equals roundf(v*255) exactly, and the float->uint conversion truncates and
-// sends negatives to 0.
-__device__ __forceinline__ uint32_t half_to_unorm8(_Float16 h)
+// the stored half.  v*255 is exact (11-bit x 8-bit significands) and so is v*255 + 1/2 wherever the
+// result matters (below 256), so floor(fma(v, 255, 1/2)) equals roundf(v*255) for v >= 0; negatives
+// end at or below 0.  v_cvt_pk_u8_f32 then converts the integer-valued float with saturation to
+// [0, 255] and drops it into byte `slot` of `packed`.
+__device__ __forceinline__ uint32_t pack_unorm8(_Float16 h, uint32_t slot, uint32_t packed)
 {
-    float const v = float(h) * 255.f;
-    uint32_t const u = uint32_t(v + 0.5f);                   // v_cvt_u32_f32: truncates, saturates below at 0
-    return u < 255u ? u : 255u;
+    float const v = floorf(__builtin_fmaf(float(h), 255.f, 0.5f));
+    return __builtin_amdgcn_cvt_pk_u8_f32(v, slot, packed);
 }
 
 typedef __attribute__((address_space(1))) uint8_t* GlobalOutPtr;
@@ -196,11 +196,11 @@ __device__ __forceinline__ void store_channels(GlobalOutPtr row, uint32_t laneOf
         }
     } else {
         v2h const a = __builtin_bit_cast(v2h, h01), b = __builtin_bit_cast(v2h, h23);
-        uint32_t const u8[4] = { half_to_unorm8(a[0]), half_to_unorm8(a[1]), half_to_unorm8(b[0]), half_to_unorm8(b[1]) };
+        uint32_t const u8 = pack_unorm8(b[1], 3, pack_unorm8(b[0], 2, pack_unorm8(a[1], 1, pack_unorm8(a[0], 0, 0u))));
         if (nch == 4 && ((reinterpret_cast<uintptr_t>(dst) & 3u) == 0)) {
-            *reinterpret_cast<__attribute__((address_space(1))) uint32_t*>(dst) = u8[0] | (u8[1] << 8) | (u8[2] << 16) | (u8[3] << 24);
+            *reinterpret_cast<__attribute__((address_space(1))) uint32_t*>(dst) = u8;
         } else {
-            for (int r = 0; r < nch; ++r) dst[r] = uint8_t(u8[r]);
+            for (int r = 0; r < nch; ++r) dst[r] = uint8_t(u8 >> (8 * r));
         }
     }
 }
