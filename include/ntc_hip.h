@@ -193,9 +193,12 @@ int ntc_hip_decode_queries_timed(const NtcHipTextureSet* set, const NtcHipQuery*
 
 /* Extracts channels of one decoded mip from the internal fp16 layout into a user image:
  * what ITextureSet::ReadChannels does through cuda::CopyImage (src/TextureSet.cpp:915-985,
- * src/ImageProcessing.cu:141-164,220-277).  Same-size copies only (the reference's 1:1
- * branch), no dithering, linear colour spaces.  Destination channels beyond numChannels get
- * the reference's defaults (alpha 1, others 0).  Asynchronous on the library stream. */
+ * src/ImageProcessing.cu:86-164,220-277).  Same-size copies only (the reference's 1:1
+ * branch).  Each copied channel is decoded from its storage colour space and encoded into the
+ * destination's (0 linear, 1 sRGB, 2 HLG; src/CudaUtils.h:61-114); with useDithering every
+ * destination channel of UNORM formats gets the reference's hash-based noise of +-1/2 step
+ * (src/CudaUtils.h:117-184).  Destination channels beyond numChannels get the reference's
+ * defaults (alpha 1, others 0).  Asynchronous on the library stream. */
 typedef struct NtcHipReadChannels {
     const void* planarPairs;    /* device: start of the mip, NTC_HIP_OUT_FP16_PLANAR_PAIRS layout */
     uint64_t    planarBytes;    /* bytes available from planarPairs */
@@ -205,14 +208,16 @@ typedef struct NtcHipReadChannels {
     void*       dst;            /* device */
     uint64_t    dstBytes;
     int32_t     format;         /* ChannelFormat of include/libntc/ntc.h:227-236: 1 UNORM8, 2 UNORM16, 3 FLOAT16, 4 FLOAT32, 5 UINT32 */
-    int32_t     reserved;
+    int32_t     useDithering;
     uint64_t    pixelStride, rowPitch;
+    uint8_t     srcColorSpaces[16];   /* storage colour space of set channel firstChannel + i */
+    uint8_t     dstColorSpaces[16];   /* colour space wanted for copied channel i */
 } NtcHipReadChannels;
 int ntc_hip_read_channels(const NtcHipReadChannels* params);
 
 /* Stores a user image into the internal fp16 layout of one mip: what ITextureSet::WriteChannels
  * does through cuda::CopyImage (src/TextureSet.cpp:829-913, src/ImageProcessing.cu:107-164,220-277).
- * Same-size copies, linear colour spaces.  Asynchronous on the library stream. */
+ * Same-size copies; colour spaces as in NtcHipReadChannels.  Asynchronous on the library stream. */
 typedef struct NtcHipWriteChannels {
     const void* src;            /* device: pitch-linear user image */
     uint64_t    srcBytes;
@@ -222,6 +227,8 @@ typedef struct NtcHipWriteChannels {
     void*       planarPairs;    /* device: start of the mip in the internal layout */
     uint64_t    planarBytes;
     int32_t     width, height, setChannels, firstChannel, numChannels, reserved;
+    uint8_t     srcColorSpaces[16];   /* colour space of channel i of the user image */
+    uint8_t     dstColorSpaces[16];   /* storage colour space of set channel firstChannel + i */
 } NtcHipWriteChannels;
 int ntc_hip_write_channels(const NtcHipWriteChannels* params);
 

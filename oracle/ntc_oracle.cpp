@@ -516,15 +516,81 @@ int ntc_oracle_ref_geometry(int width, int height, int numMips, int gridSizeScal
     return numNeural;
 }
 
-// ITextureSet::ReadChannels' copy, 1:1 branch, no dithering, linear colour spaces:
-// CopyImageKernel + ReadImageChannel (FLOAT16 source) + WriteImageChannel
-// (src/ImageProcessing.cu:107-164,220-265) reading the internal planar-pair layout
-// (GetTextureDataSlice, src/TextureSet.cpp:1958-1983).  Destination channels beyond
-// numChannels get GetDefaultChannelValue (src/ImageProcessing.cu:166-170).
+// Transfer functions of the colour spaces (src/CudaUtils.h:61-114): sRGB and Hybrid Log-Gamma,
+// with the host math library's powf / expf / logf / sqrtf -- results agree with the device's to a few
+// units in the last place, not bit for bit, and the tests that use them say so.
+static float decode_color_space(int cs, float v)
+{
+    if (cs == 1) return (v <= 0.04045f) ? v / 12.92f : std::pow((v + 0.055f) / 1.055f, 2.4f);
+    if (cs == 2) {
+        float const sign = (v < 0.f) ? -1.f : 1.f;
+        float const h = std::fabs(v);
+        return (h < 0.5f) ? 4.f * h * h * sign : (std::exp((h - 0.55991073f) / 0.17883277f) + 0.28466892f) * sign;
+    }
+    return v;
+}
+static float encode_color_space(int cs, float v)
+{
+    if (cs == 1) return (v <= 0.0031308f) ? v * 12.92f : 1.055f * std::pow(v, 1.0f / 2.4f) - 0.055f;
+    if (cs == 2) {
+        float const sign = (v < 0.f) ? -1.f : 1.f;
+        float const e = std::fabs(v);
+        return (e < 1.f) ? 0.5f * std::sqrt(e) * sign : (0.17883277f * std::log(e - 0.28466892f) + 0.55991073f) * sign;
+    }
+    return v;
+}
+
+// HashBasedRNG (src/CudaUtils.h:117-184): the seed is a Jenkins hash of the pixel's linear index,
+// every draw is one Murmur3 round over a running counter that starts at 1; the float takes the low
+// 23 bits as a mantissa in [1, 2) and subtracts 1.
+struct HashRng {
+    uint32_t seed, index = 1;
+    explicit HashRng(uint32_t linearIndex)
+    {
+        uint32_t a = linearIndex;
+        a = (a + 0x7ed55d16u) + (a << 12);
+        a = (a ^ 0xc761c23cu) ^ (a >> 19);
+        a = (a + 0x165667b1u) + (a << 5);
+        a = (a + 0xd3a2646cu) ^ (a << 9);
+        a = (a + 0xfd7046c5u) + (a << 3);
+        a = (a ^ 0xb55a4f09u) ^ (a >> 16);
+        seed = a;
+    }
+    static uint32_t rotl(uint32_t x, int n) { return (x << n) | (x >> (32 - n)); }
+    uint32_t next_uint()
+    {
+        uint32_t k = index * 0xcc9e2d51u;
+        k = rotl(k, 15) * 0x1b873593u;
+        uint32_t h = rotl(seed ^ k, 13) * 5u + 0xe6546b64u;
+        h ^= 4u;
+        h ^= h >> 16; h *= 0x85ebca6bu;
+        h ^= h >> 13; h *= 0xc2b2ae35u;
+        h ^= h >> 16;
+        ++index;
+        return h;
+    }
+    float next_float() { return bits_f32((next_uint() & 0x7fffffu) | 0x3f800000u) - 1.f; }
+};
+
+// Draw number `draw` (0-based) of the dithering generator of pixel `linearIndex`, in [0, 1).
+float ntc_oracle_dither_float(uint32_t linearIndex, int draw)
+{
+    HashRng rng(linearIndex);
+    float v = 0.f;
+    for (int i = 0; i <= draw; ++i) v = rng.next_float();
+    return v;
+}
+
+// ITextureSet::ReadChannels' copy, 1:1 branch: CopyImageKernel + ReadImageChannel (FLOAT16 source)
+// + WriteImageChannel (src/ImageProcessing.cu:86-164,220-265) reading the internal planar-pair
+// layout (GetTextureDataSlice, src/TextureSet.cpp:1958-1983).  Destination channels beyond
+// numChannels get GetDefaultChannelValue (src/ImageProcessing.cu:166-170); with useDithering every
+// destination channel draws one number, in channel order.
 // format: 1 UNORM8, 2 UNORM16, 3 FLOAT16, 4 FLOAT32, 5 UINT32 (include/libntc/ntc.h:227-236).
-int ntc_oracle_read_channels(const uint16_t* planarPairs, int width, int height, int setChannels,
-                             int firstChannel, int numChannels, uint8_t* dst, int format,
-                             uint64_t pixelStride, uint64_t rowPitch)
+int ntc_oracle_read_channels_ex(const uint16_t* planarPairs, int width, int height, int setChannels,
+                                int firstChannel, int numChannels, uint8_t* dst, int format,
+                                uint64_t pixelStride, uint64_t rowPitch, int useDithering,
+                                const uint8_t* srcColorSpaces /* 16 or null */, const uint8_t* dstColorSpaces /* 16 or null */)
 {
     int const bpc = (format == 1) ? 1 : (format == 2 || format == 3) ? 2 : (format == 4 || format == 5) ? 4 : 0;
     if (!bpc) return -1;
@@ -538,19 +604,22 @@ int ntc_oracle_read_channels(const uint16_t* planarPairs, int width, int height,
     for (int y = 0; y < height; ++y)
         for (int x = 0; x < width; ++x) {
             uint8_t* px = dst + size_t(y) * rowPitch + size_t(x) * pixelStride;
+            HashRng rng(uint32_t(x) + uint32_t(y) * uint32_t(width));
             for (int ch = 0; ch < dstChannels; ++ch) {
                 float value;
                 if (ch < numChannels) {
                     int const c = firstChannel + ch;
                     size_t const a = size_t(y) * size_t(width) * size_t(setChannels) + size_t(x) * 2
                                    + size_t(c & ~1) * size_t(width) + size_t(c & 1);
-                    value = half_to_float(planarPairs[a]);
+                    value = decode_color_space(srcColorSpaces ? srcColorSpaces[ch] : 0, half_to_float(planarPairs[a]));
                 } else {
                     value = (ch == 3) ? 1.f : 0.f;
                 }
+                float const dither = useDithering ? rng.next_float() - 0.5f : 0.f;
+                value = encode_color_space((dstColorSpaces && ch < 16) ? dstColorSpaces[ch] : 0, value);
                 switch (format) {
-                case 1: px[ch] = uint8_t(std::max(0.f, std::min(255.f, roundHalfAway(value * 255.f)))); break;
-                case 2: { uint16_t v = uint16_t(std::max(0.f, std::min(65535.f, roundHalfAway(value * 65535.f)))); std::memcpy(px + 2 * ch, &v, 2); break; }
+                case 1: value += dither / 255.f; px[ch] = uint8_t(std::max(0.f, std::min(255.f, roundHalfAway(value * 255.f)))); break;
+                case 2: { value += dither / 65535.f; uint16_t v = uint16_t(std::max(0.f, std::min(65535.f, roundHalfAway(value * 65535.f)))); std::memcpy(px + 2 * ch, &v, 2); break; }
                 case 3: { uint16_t v = float_to_half_rne(std::max(-65504.f, std::min(65504.f, value))); std::memcpy(px + 2 * ch, &v, 2); break; }
                 case 4: std::memcpy(px + 4 * ch, &value, 4); break;
                 case 5: { uint32_t v = uint32_t(std::max(value, 0.f)); std::memcpy(px + 4 * ch, &v, 4); break; }
@@ -560,11 +629,21 @@ int ntc_oracle_read_channels(const uint16_t* planarPairs, int width, int height,
     return 0;
 }
 
-// ITextureSet::WriteChannels' copy (1:1, linear colour spaces): ReadImageChannel in the user's format,
-// WriteImageChannel FLOAT16 into the internal planar-pair layout (src/ImageProcessing.cu:107-164,220-265),
-// with the optional vertical flip of SetupBilinearFilter (src/ImageProcessing.cu:36-37).
-int ntc_oracle_write_channels(const uint8_t* src, int format, int verticalFlip, uint64_t pixelStride, uint64_t rowPitch,
-                              uint16_t* planarPairs, int width, int height, int setChannels, int firstChannel, int numChannels)
+int ntc_oracle_read_channels(const uint16_t* planarPairs, int width, int height, int setChannels,
+                             int firstChannel, int numChannels, uint8_t* dst, int format,
+                             uint64_t pixelStride, uint64_t rowPitch)
+{
+    return ntc_oracle_read_channels_ex(planarPairs, width, height, setChannels, firstChannel, numChannels, dst, format,
+                                       pixelStride, rowPitch, 0, nullptr, nullptr);
+}
+
+// ITextureSet::WriteChannels' copy (1:1): ReadImageChannel in the user's format and colour space,
+// WriteImageChannel FLOAT16 in the storage colour space into the internal planar-pair layout
+// (src/ImageProcessing.cu:86-164,220-265), with the optional vertical flip of SetupBilinearFilter
+// (src/ImageProcessing.cu:36-37).
+int ntc_oracle_write_channels_ex(const uint8_t* src, int format, int verticalFlip, uint64_t pixelStride, uint64_t rowPitch,
+                                 uint16_t* planarPairs, int width, int height, int setChannels, int firstChannel, int numChannels,
+                                 const uint8_t* srcColorSpaces, const uint8_t* dstColorSpaces)
 {
     for (int y = 0; y < height; ++y)
         for (int x = 0; x < width; ++x) {
@@ -580,6 +659,8 @@ int ntc_oracle_write_channels(const uint8_t* src, int format, int verticalFlip, 
                 case 5: { uint32_t t; std::memcpy(&t, px + 4 * ch, 4); v = float(t); break; }
                 default: return -1;
                 }
+                v = decode_color_space(srcColorSpaces ? srcColorSpaces[ch] : 0, v);
+                v = encode_color_space(dstColorSpaces ? dstColorSpaces[ch] : 0, v);
                 v = std::max(-65504.f, std::min(65504.f, v));
                 int const c = firstChannel + ch;
                 planarPairs[size_t(y) * size_t(width) * size_t(setChannels) + size_t(x) * 2
@@ -587,6 +668,13 @@ int ntc_oracle_write_channels(const uint8_t* src, int format, int verticalFlip, 
             }
         }
     return 0;
+}
+
+int ntc_oracle_write_channels(const uint8_t* src, int format, int verticalFlip, uint64_t pixelStride, uint64_t rowPitch,
+                              uint16_t* planarPairs, int width, int height, int setChannels, int firstChannel, int numChannels)
+{
+    return ntc_oracle_write_channels_ex(src, format, verticalFlip, pixelStride, rowPitch, planarPairs, width, height, setChannels,
+                                        firstChannel, numChannels, nullptr, nullptr);
 }
 
 // Per-channel mean squared error between a decoded mip and its reference, both in the internal

@@ -72,8 +72,9 @@ class ReadChannels(C.Structure):
     _fields_ = [
         ("planarPairs", C.c_void_p), ("planarBytes", C.c_uint64), ("width", C.c_int32), ("height", C.c_int32),
         ("setChannels", C.c_int32), ("firstChannel", C.c_int32), ("numChannels", C.c_int32),
-        ("dst", C.c_void_p), ("dstBytes", C.c_uint64), ("format", C.c_int32), ("reserved", C.c_int32),
+        ("dst", C.c_void_p), ("dstBytes", C.c_uint64), ("format", C.c_int32), ("useDithering", C.c_int32),
         ("pixelStride", C.c_uint64), ("rowPitch", C.c_uint64),
+        ("srcColorSpaces", C.c_uint8 * 16), ("dstColorSpaces", C.c_uint8 * 16),
     ]
 
 
@@ -83,6 +84,7 @@ class WriteChannels(C.Structure):
         ("pixelStride", C.c_uint64), ("rowPitch", C.c_uint64), ("planarPairs", C.c_void_p), ("planarBytes", C.c_uint64),
         ("width", C.c_int32), ("height", C.c_int32), ("setChannels", C.c_int32), ("firstChannel", C.c_int32),
         ("numChannels", C.c_int32), ("reserved", C.c_int32),
+        ("srcColorSpaces", C.c_uint8 * 16), ("dstColorSpaces", C.c_uint8 * 16),
     ]
 
 

@@ -1,8 +1,8 @@
-// ntc_copy_kernel.hip - internal fp16 texture layout -> user pitch-linear image (gfx950).
+// ntc_copy_kernel.hip - internal fp16 texture layout <-> user pitch-linear image, image loss (gfx950).
 //
-// The 1:1 branch of the reference's CopyImageKernel as ITextureSet::ReadChannels uses it
-// (src/ImageProcessing.cu:141-164,220-265, src/TextureSet.cpp:948-967): no resize, no
-// dithering, linear colour spaces.  One lane per pixel; source reads are the half2 pairs of
+// The 1:1 branch of the reference's CopyImageKernel as ITextureSet::ReadChannels / WriteChannels
+// use it (src/ImageProcessing.cu:86-164,220-265, src/TextureSet.cpp:835-985): no resize; colour
+// space decode/encode and dithering as the reference defines them.  One lane per pixel; source reads are the half2 pairs of
 // the planar-pair layout (coalesced across x), destination writes are the pixel's bytes.
 // HBM-bound: 2 bytes read and 1-4 bytes written per channel.
 #include <hip/hip_runtime.h>
@@ -21,13 +21,69 @@ __device__ __forceinline__ float round_half_away(float v)
     return r;
 }
 
-__device__ __forceinline__ void write_channel(uint8_t* px, uint32_t ch, int format, float value)
+// Transfer functions, src/CudaUtils.h:61-114 (sRGB, Hybrid Log-Gamma) and src/ImageProcessing.cu:86-111.
+// The transcendental parts are the device math library's, so results agree with a CPU
+// evaluation to a few units in the last place, not bit for bit.
+__device__ __forceinline__ float decode_color_space(int colorSpace, float v)
 {
+    if (colorSpace == 1) return (v <= 0.04045f) ? v / 12.92f : powf((v + 0.055f) / 1.055f, 2.4f);
+    if (colorSpace == 2) {
+        float const sign = (v < 0.f) ? -1.f : 1.f;
+        float const h = fabsf(v);
+        return (h < 0.5f) ? 4.f * h * h * sign : (expf((h - 0.55991073f) / 0.17883277f) + 0.28466892f) * sign;
+    }
+    return v;
+}
+__device__ __forceinline__ float encode_color_space(int colorSpace, float v)
+{
+    if (colorSpace == 1) return (v <= 0.0031308f) ? v * 12.92f : 1.055f * powf(v, 1.0f / 2.4f) - 0.055f;
+    if (colorSpace == 2) {
+        float const sign = (v < 0.f) ? -1.f : 1.f;
+        float const e = fabsf(v);
+        return (e < 1.f) ? 0.5f * sqrtf(e) * sign : (0.17883277f * logf(e - 0.28466892f) + 0.55991073f) * sign;
+    }
+    return v;
+}
+
+// HashBasedRNG, src/CudaUtils.h:117-184: Jenkins hash of the pixel index seeds a Murmur3 round per draw.
+struct DitherRng {
+    uint32_t seed, index;
+    __device__ explicit DitherRng(uint32_t linearIndex) : index(1)
+    {
+        uint32_t a = linearIndex;
+        a = (a + 0x7ed55d16u) + (a << 12);
+        a = (a ^ 0xc761c23cu) ^ (a >> 19);
+        a = (a + 0x165667b1u) + (a << 5);
+        a = (a + 0xd3a2646cu) ^ (a << 9);
+        a = (a + 0xfd7046c5u) + (a << 3);
+        a = (a ^ 0xb55a4f09u) ^ (a >> 16);
+        seed = a;
+    }
+    __device__ float next_float()                            // [0, 1)
+    {
+        uint32_t k = index++ * 0xcc9e2d51u;
+        k = (k << 15) | (k >> 17);
+        k *= 0x1b873593u;
+        uint32_t h = seed ^ k;
+        h = ((h << 13) | (h >> 19)) * 5u + 0xe6546b64u;
+        h ^= 4u;
+        h ^= h >> 16; h *= 0x85ebca6bu;
+        h ^= h >> 13; h *= 0xc2b2ae35u;
+        h ^= h >> 16;
+        return __builtin_bit_cast(float, (h & 0x7fffffu) | 0x3f800000u) - 1.f;
+    }
+};
+
+__device__ __forceinline__ void write_channel(uint8_t* px, uint32_t ch, int format, int colorSpace, float value, float dither)
+{
+    value = encode_color_space(colorSpace, value);
     switch (format) {
     case NTC_HIP_DEV_FORMAT_UNORM8:
+        value += dither / 255.f;
         px[ch] = uint8_t(fmaxf(0.f, fminf(255.f, round_half_away(value * 255.f))));
         break;
     case NTC_HIP_DEV_FORMAT_UNORM16:
+        value += dither / 65535.f;
         reinterpret_cast<uint16_t*>(px)[ch] = uint16_t(fmaxf(0.f, fminf(65535.f, round_half_away(value * 65535.f))));
         break;
     case NTC_HIP_DEV_FORMAT_FLOAT16: {
@@ -56,16 +112,18 @@ read_channels_kernel(ReadChannelsArgs a)
     // GetPixelBaseAddress / GetChannelAddress, src/RegressionKernels.h:36-45
     uint16_t const* src = a.planarPairs + size_t(y) * size_t(a.width) * size_t(a.setChannels) + size_t(x) * 2;
     uint8_t* px = a.dst + size_t(y) * a.rowPitch + size_t(x) * a.pixelStride;
+    DitherRng rng(uint32_t(x) + uint32_t(y) * uint32_t(a.width));
     for (int ch = 0; ch < a.dstChannels; ++ch) {
         float value;
         if (ch < a.numChannels) {
             int const c = a.firstChannel + ch;
             uint16_t const bits = src[size_t(c & ~1) * size_t(a.width) + size_t(c & 1)];
-            value = float(__builtin_bit_cast(_Float16, bits));
+            value = decode_color_space(a.srcColorSpaces[ch], float(__builtin_bit_cast(_Float16, bits)));
         } else {
             value = (ch == 3) ? 1.f : 0.f;                   // GetDefaultChannelValue, src/ImageProcessing.cu:166-170
         }
-        write_channel(px, uint32_t(ch), a.format, value);
+        float const dither = a.useDithering ? rng.next_float() - 0.5f : 0.f;      // one draw per destination channel
+        write_channel(px, uint32_t(ch), a.format, ch < 16 ? a.dstColorSpaces[ch] : 0, value, dither);
     }
 }
 
@@ -94,7 +152,8 @@ write_channels_kernel(WriteChannelsArgs a)
     uint8_t const* px = a.src + size_t(srcY) * a.rowPitch + size_t(x) * a.pixelStride;
     uint16_t* dst = a.planarPairs + size_t(y) * size_t(a.width) * size_t(a.setChannels) + size_t(x) * 2;
     for (int ch = 0; ch < a.numChannels; ++ch) {
-        float v = read_channel(px, uint32_t(ch), a.format);
+        float v = decode_color_space(a.srcColorSpaces[ch], read_channel(px, uint32_t(ch), a.format));
+        v = encode_color_space(a.dstColorSpaces[ch], v);
         v = fmaxf(-65504.f, fminf(65504.f, v));                      // WriteImageChannel FLOAT16, src/ImageProcessing.cu:154-156
         asm volatile("" : "+v"(v));
         int const c = a.firstChannel + ch;

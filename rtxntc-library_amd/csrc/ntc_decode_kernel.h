@@ -60,6 +60,8 @@ struct ReadChannelsArgs {
     uint8_t* dst;
     uint64_t pixelStride, rowPitch;
     int32_t width, height, setChannels, firstChannel, numChannels, dstChannels, format;
+    int32_t useDithering;
+    uint8_t srcColorSpaces[16], dstColorSpaces[16];   // per copied channel: 0 linear, 1 sRGB, 2 HLG
 };
 hipError_t launch_read_channels(ReadChannelsArgs const& args, hipStream_t stream);
 
@@ -70,6 +72,7 @@ struct WriteChannelsArgs {
     uint16_t* planarPairs;
     uint64_t pixelStride, rowPitch;
     int32_t width, height, setChannels, firstChannel, numChannels, format, verticalFlip;
+    uint8_t srcColorSpaces[16], dstColorSpaces[16];
 };
 hipError_t launch_write_channels(WriteChannelsArgs const& args, hipStream_t stream);
 

@@ -563,6 +563,12 @@ int ntc_hip_read_channels(const NtcHipReadChannels* p)
     a.width = p->width; a.height = p->height; a.setChannels = p->setChannels;
     a.firstChannel = p->firstChannel; a.numChannels = p->numChannels;
     a.dstChannels = int32_t(dstChannels); a.format = p->format;
+    a.useDithering = p->useDithering ? 1 : 0;
+    for (int i = 0; i < 16; ++i) {
+        if (p->srcColorSpaces[i] > 2 || p->dstColorSpaces[i] > 2) { set_error("ntc_hip_read_channels: unknown colour space for channel %d.", i); return NTC_HIP_ERR_INVALID_ARG; }
+        a.srcColorSpaces[i] = p->srcColorSpaces[i];
+        a.dstColorSpaces[i] = p->dstColorSpaces[i];
+    }
     HIP_TRY(launch_read_channels(a, g_lib.stream));
     clear_error();
     return 0;
@@ -603,6 +609,11 @@ int ntc_hip_write_channels(const NtcHipWriteChannels* p)
     a.pixelStride = p->pixelStride; a.rowPitch = p->rowPitch;
     a.width = p->width; a.height = p->height; a.setChannels = p->setChannels;
     a.firstChannel = p->firstChannel; a.numChannels = p->numChannels; a.format = p->format; a.verticalFlip = p->verticalFlip ? 1 : 0;
+    for (int i = 0; i < 16; ++i) {
+        if (p->srcColorSpaces[i] > 2 || p->dstColorSpaces[i] > 2) { set_error("ntc_hip_write_channels: unknown colour space for channel %d.", i); return NTC_HIP_ERR_INVALID_ARG; }
+        a.srcColorSpaces[i] = p->srcColorSpaces[i];
+        a.dstColorSpaces[i] = p->dstColorSpaces[i];
+    }
     HIP_TRY(launch_write_channels(a, g_lib.stream));
     clear_error();
     return 0;

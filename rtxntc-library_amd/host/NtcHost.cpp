@@ -671,7 +671,6 @@ public:
         if (Status st = ValidateReadWriteChannelsArgs(params.mipLevel, params.firstChannel, params.numChannels, params.width, params.height,
                 params.pixelStride, params.rowPitch, fromHost ? sizeToCopy : 0, params.channelFormat, "writes"); st != Status::Ok)
             return st;
-        if (params.srcColorSpaces || params.dstColorSpaces) { SetErrorMessage("Non-linear colour spaces are not supported."); return Status::Unsupported; }
         if (!m_deviceAvailable) { SetErrorMessage("No HIP device is available to this context."); return Status::CudaUnavailable; }
         if (fromHost)
             if (int r = ntc_hip_upload(m_staging, params.pData, sizeToCopy)) return DeviceFailure(r);
@@ -687,6 +686,14 @@ public:
         wc.planarBytes = m_textureBytes - offset;
         wc.width = mipWidth; wc.height = mipHeight; wc.setChannels = m_desc.channels;
         wc.firstChannel = params.firstChannel; wc.numChannels = params.numChannels;
+        for (int channel = 0; channel < params.numChannels; ++channel) {
+            ColorSpace const source = params.srcColorSpaces ? params.srcColorSpaces[channel] : ColorSpace::Linear;
+            ColorSpace const storage = params.dstColorSpaces ? params.dstColorSpaces[channel] : ColorSpace::Linear;
+            if (unsigned(source) > 2u || unsigned(storage) > 2u) { SetErrorMessage("Unknown colour space for channel %d.", channel); return Status::InvalidArgument; }
+            wc.srcColorSpaces[channel] = uint8_t(source);
+            wc.dstColorSpaces[channel] = uint8_t(storage);
+            m_channelColorSpaces[channel + params.firstChannel] = storage;       // src/TextureSet.cpp:899-902
+        }
         if (int r = ntc_hip_write_channels(&wc)) return DeviceFailure(r);
         ClearErrorMessage();
         return Status::Ok;
@@ -702,10 +709,6 @@ public:
                 params.pixelStride, params.rowPitch, toHost ? sizeToCopy : 0, params.channelFormat, "reads"); st != Status::Ok)
             return st;
         int const mipWidth = std::max(m_desc.width >> params.mipLevel, 1), mipHeight = std::max(m_desc.height >> params.mipLevel, 1);
-        if (params.useDithering || params.dstColorSpaces) {
-            SetErrorMessage("Dithering and non-linear destination colour spaces are not supported.");
-            return Status::Unsupported;
-        }
         if (!m_deviceAvailable) { SetErrorMessage("No HIP device is available to this context."); return Status::CudaUnavailable; }
 
         // Rows the copy does not fully overwrite must not carry garbage to the client (src/TextureSet.cpp:936-946).
@@ -724,6 +727,13 @@ public:
         rc.dstBytes = toHost ? m_stagingBytes : sizeToCopy;
         rc.format = int(params.channelFormat);
         rc.pixelStride = params.pixelStride; rc.rowPitch = params.rowPitch;
+        rc.useDithering = params.useDithering ? 1 : 0;
+        for (int channel = 0; channel < params.numChannels; ++channel) {
+            ColorSpace const wanted = params.dstColorSpaces ? params.dstColorSpaces[channel] : ColorSpace::Linear;
+            if (unsigned(wanted) > 2u) { SetErrorMessage("Unknown colour space for channel %d.", channel); return Status::InvalidArgument; }
+            rc.srcColorSpaces[channel] = uint8_t(m_channelColorSpaces[channel + params.firstChannel]);
+            rc.dstColorSpaces[channel] = uint8_t(wanted);
+        }
         if (int r = ntc_hip_read_channels(&rc)) return DeviceFailure(r);
         if (toHost)
             if (int r = ntc_hip_download(params.pOutData, m_staging, sizeToCopy)) return DeviceFailure(r);

@@ -33,13 +33,13 @@ enum class Status
 
 // include/libntc/ntc.h:227-236
 enum class ChannelFormat { UNKNOWN = 0, UNORM8 = 1, UNORM16 = 2, FLOAT16 = 3, FLOAT32 = 4, UINT32 = 5 };
-// include/libntc/ntc.h:272-276
-enum class AddressSpace { Host, Device };
-enum class TextureDataPage { Reference, Output };
 // include/libntc/ntc.h:238-256
 enum class BlockCompressedFormat { None = 0, BC1 = 1, BC2 = 2, BC3 = 3, BC4 = 4, BC5 = 5, BC6 = 6, BC7 = 7 };
 enum class ColorSpace { Linear = 0, sRGB = 1, HLG = 2 };
 
+// include/libntc/ntc.h:272-276
+enum class AddressSpace { Host, Device };
+enum class TextureDataPage { Reference, Output };
 // Application-provided or library-provided byte streams (include/libntc/ntc.h:91-114).
 class IStream
 {
@@ -97,8 +97,8 @@ struct WriteChannelsParameters
     size_t pixelStride = 0;
     size_t rowPitch = 0;
     ChannelFormat channelFormat = ChannelFormat::UNKNOWN;
-    void const* srcColorSpaces = nullptr;   // must be null: only linear storage is supported
-    void const* dstColorSpaces = nullptr;
+    ColorSpace const* srcColorSpaces = nullptr;   // per written channel; null = all linear
+    ColorSpace const* dstColorSpaces = nullptr;   // storage colour spaces, recorded with the set; null = all linear
     bool verticalFlip = false;
 };
 
@@ -116,8 +116,8 @@ struct ReadChannelsParameters
     size_t pixelStride = 0;
     size_t rowPitch = 0;
     ChannelFormat channelFormat = ChannelFormat::UNKNOWN;
-    void const* dstColorSpaces = nullptr;   // must be null: only linear storage is supported
-    bool useDithering = false;              // must be false
+    ColorSpace const* dstColorSpaces = nullptr;   // per read channel; null = all linear
+    bool useDithering = false;                    // +-1/2 step of hash noise on UNORM outputs
 };
 
 // include/libntc/ntc.h:810-816.  Losses are mean squared errors against the image written with

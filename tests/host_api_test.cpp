@@ -212,6 +212,19 @@ static int decode(int argc, char** argv)
             CHECK(writeFile(prefix + "_mip" + std::to_string(mip) + "_rgba16f.bin", f16.data(), f16.size()));
         }
     }
+    // dithered read of mip 0 into sRGB for the first three channels
+    {
+        ColorSpace wanted[16];
+        for (int c = 0; c < 16; ++c) wanted[c] = c < 3 ? ColorSpace::sRGB : ColorSpace::Linear;
+        ReadChannelsParameters rp;
+        rp.mipLevel = 0; rp.firstChannel = 0; rp.numChannels = C; rp.width = w; rp.height = h;
+        rp.pixelStride = size_t(C); rp.rowPitch = size_t(C) * size_t(w);
+        rp.channelFormat = ChannelFormat::UNORM8; rp.dstColorSpaces = wanted; rp.useDithering = true;
+        std::vector<unsigned char> u8(rp.rowPitch * size_t(h));
+        rp.pOutData = u8.data();
+        CHECK(set->ReadChannels(rp) == Status::Ok);
+        CHECK(writeFile(prefix + "_srgb_dither.bin", u8.data(), u8.size()));
+    }
     // a resizing read is refused, not silently approximated
     ReadChannelsParameters bad;
     std::vector<unsigned char> tmp(64);
@@ -285,6 +298,27 @@ static int loss(int argc, char** argv)
     rp.page = TextureDataPage::Output;
     CHECK(set->ReadChannels(rp) == Status::Ok);
     CHECK(writeFile(prefix + "_page_output.bin", page.data(), page.size()));
+    // storage colour spaces given to WriteChannels are recorded with the set (src/TextureSet.cpp:899-902)
+    {
+        CHECK(set->GetChannelStorageColorSpace(1) == ColorSpace::Linear);
+        std::vector<unsigned char> one(size_t(w) * size_t(h), 128);
+        ColorSpace const source = ColorSpace::Linear, storage = ColorSpace::sRGB;
+        WriteChannelsParameters wp;
+        wp.mipLevel = 0; wp.firstChannel = 1; wp.numChannels = 1; wp.pData = one.data();
+        wp.width = w; wp.height = h; wp.pixelStride = 1; wp.rowPitch = size_t(w);
+        wp.channelFormat = ChannelFormat::UNORM8; wp.srcColorSpaces = &source; wp.dstColorSpaces = &storage;
+        CHECK(set->WriteChannels(wp) == Status::Ok);
+        CHECK(set->GetChannelStorageColorSpace(1) == ColorSpace::sRGB && set->GetChannelStorageColorSpace(0) == ColorSpace::Linear);
+        // reading it back as linear UNORM8 returns the written codes (sRGB there and back), to one code
+        ReadChannelsParameters rb;
+        rb.page = TextureDataPage::Reference;
+        rb.mipLevel = 0; rb.firstChannel = 1; rb.numChannels = 1; rb.width = w; rb.height = h; rb.pixelStride = 1; rb.rowPitch = size_t(w);
+        rb.channelFormat = ChannelFormat::UNORM8;
+        std::vector<unsigned char> back(one.size());
+        rb.pOutData = back.data();
+        CHECK(set->ReadChannels(rb) == Status::Ok);
+        for (unsigned char v : back) CHECK(v >= 127 && v <= 129);
+    }
     ctx->DestroyTextureSet(set);
     DestroyContext(ctx);
     std::printf("host loss OK\n");

@@ -136,6 +136,17 @@ def test_host_layer_decode_and_read_back(ntc, oracle, tmp_path, preset):
         oracle.ntc_oracle_read_channels(planar.ctypes.data, mip.width, mip.height, channels, 1, 3, want16.ctypes.data, 3, 8, mip.width * 8)
         got16 = np.fromfile(f"{prefix}_mip{m}_rgba16f.bin", dtype=np.uint8)
         assert np.array_equal(got16, want16), f"preset {preset} mip {m} rgba16f"
+    # mip 0 again, dithered, channels 0..2 encoded as sRGB: one code of slack for the transfer function
+    mip = case.mips[0]
+    planar = np.ascontiguousarray(host.output[mip.outOffset: mip.outOffset + w * h * channels * 2].view(np.uint16))
+    want = np.zeros(h * w * channels, dtype=np.uint8)
+    src_cs = np.zeros(16, dtype=np.uint8)
+    dst_cs = np.array([1, 1, 1] + [0] * 13, dtype=np.uint8)
+    oracle.ntc_oracle_read_channels_ex(planar.ctypes.data, w, h, channels, 0, channels, want.ctypes.data, 1, channels, channels * w, 1,
+                                       src_cs.ctypes.data, dst_cs.ctypes.data)
+    got = np.fromfile(f"{prefix}_srgb_dither.bin", dtype=np.uint8)
+    assert np.abs(got.astype(int) - want.astype(int)).max() <= 1
+    assert np.array_equal(got.reshape(h, w, channels)[:, :, 3:], want.reshape(h, w, channels)[:, :, 3:])     # linear channels: exact
 
 
 # ---- WriteChannels and the loss statistics of Decompress ------------------------------------------
@@ -310,3 +321,177 @@ def test_host_layer_loss_statistics(ntc, oracle, tmp_path, separate):
     page_out = np.fromfile(prefix + "_page_output.bin", dtype=np.uint16)
     assert np.array_equal(page_out, pixels_of(decoded0))
     assert np.array_equal(page_ref, pixels_of(ref0 if separate else decoded0))
+
+
+# ---- colour spaces and dithering in ReadChannels / WriteChannels -----------------------------------
+
+def jenkins(a):
+    """Robert Jenkins' 32-bit integer hash as HashBasedRNG seeds with it (src/CudaUtils.h:147-157)."""
+    m = 0xFFFFFFFF
+    a = ((a + 0x7ed55d16) + (a << 12)) & m
+    a = ((a ^ 0xc761c23c) ^ (a >> 19)) & m
+    a = ((a + 0x165667b1) + (a << 5)) & m
+    a = ((a + 0xd3a2646c) ^ (a << 9)) & m
+    a = ((a + 0xfd7046c5) + (a << 3)) & m
+    a = ((a ^ 0xb55a4f09) ^ (a >> 16)) & m
+    return a
+
+
+def dither_model(linear_index, draw):
+    """Draw `draw` of HashBasedRNG: its Murmur3Hash() is MurmurHash3_x86_32 of the 4-byte counter
+    (starting at 1) with the Jenkins-hashed pixel index as seed -- computed here with scikit-learn's
+    implementation of that hash."""
+    from sklearn.utils import murmurhash3_32
+    h = murmurhash3_32((draw + 1).to_bytes(4, "little"), seed=jenkins(linear_index), positive=True)
+    return np.uint32((h & 0x7FFFFF) | 0x3F800000).view(np.float32) - np.float32(1.0)
+
+
+def test_checker_dither_generator_is_murmur3_of_the_counter(oracle):
+    for index in (0, 1, 2, 77, 4095, 123456789, 0xFFFFFFFF):
+        for draw in range(5):
+            assert oracle.ntc_oracle_dither_float(index, draw) == dither_model(index, draw), (index, draw)
+
+
+def srgb_encode(v):
+    v = np.asarray(v, dtype=np.float64)
+    return np.where(v <= 0.0031308, v * 12.92, 1.055 * np.power(np.maximum(v, 1e-30), 1 / 2.4) - 0.055)
+
+
+def srgb_decode(v):
+    v = np.asarray(v, dtype=np.float64)
+    return np.where(v <= 0.04045, v / 12.92, np.power((np.maximum(v, 0) + 0.055) / 1.055, 2.4))
+
+
+def hlg_encode(v):
+    v = np.asarray(v, dtype=np.float64)
+    e = np.abs(v)
+    return np.sign(v) * np.where(e < 1, 0.5 * np.sqrt(e), 0.17883277 * np.log(np.maximum(e - 0.28466892, 1e-30)) + 0.55991073)
+
+
+def hlg_decode(v):
+    v = np.asarray(v, dtype=np.float64)
+    h = np.abs(v)
+    return np.sign(v) * np.where(h < 0.5, 4 * h * h, np.exp((h - 0.55991073) / 0.17883277) + 0.28466892)
+
+
+ENCODE = {0: lambda v: np.asarray(v, dtype=np.float64), 1: srgb_encode, 2: hlg_encode}
+DECODE = {0: lambda v: np.asarray(v, dtype=np.float64), 1: srgb_decode, 2: hlg_decode}
+
+
+def unit_planar(rng, width, height, channels):
+    return rng.uniform(0.0, 1.0, width * height * channels).astype(np.float16).view(np.uint16)
+
+
+def test_checker_color_spaces_and_dithering_against_float64_models(oracle):
+    """UNORM8 reads: storage colour space -> linear -> requested colour space, plus dithering; the
+    float64 model must agree to one code (the transfer functions are float32 in the checker)."""
+    rng = np.random.default_rng(70)
+    w, h, C_ = 33, 6, 4
+    planar = unit_planar(rng, w, h, C_)
+    values = planar.view(np.float16).astype(np.float64).reshape(h, C_ // 2, w, 2).transpose(0, 2, 1, 3).reshape(h, w, C_)
+    for src_cs, dst_cs, dither in ((0, 1, 0), (1, 0, 0), (2, 0, 0), (0, 2, 0), (1, 2, 1), (0, 0, 1)):
+        got = np.zeros(h * w * C_, dtype=np.uint8)
+        src = np.full(16, src_cs, dtype=np.uint8)
+        dst = np.full(16, dst_cs, dtype=np.uint8)
+        assert oracle.ntc_oracle_read_channels_ex(planar.ctypes.data, w, h, C_, 0, C_, got.ctypes.data, 1, C_, w * C_, dither,
+                                                  src.ctypes.data, dst.ctypes.data) == 0
+        want = ENCODE[dst_cs](DECODE[src_cs](values))
+        if dither:
+            noise = np.array([[[float(dither_model(x + y * w, ch)) - 0.5 for ch in range(C_)] for x in range(w)] for y in range(h)])
+            want = want + noise / 255.0
+        want = np.clip(np.floor(want * 255.0 + 0.5), 0, 255)
+        assert np.abs(got.reshape(h, w, C_).astype(np.float64) - want).max() <= 1, (src_cs, dst_cs, dither)
+        if src_cs == 0 and dst_cs == 0:       # no transcendental involved: the model is exact up to float32 rounding at ties
+            assert (got.reshape(h, w, C_) != want).mean() < 0.01
+
+
+def gpu_read_ex(ntc, device, planar, w, h, C_, first, count, fmt, stride, pitch, dither, src_cs, dst_cs):
+    d_src = device.upload(planar)
+    d_dst = device.alloc(h * pitch)
+    d_dst.fill(0xEE)
+    rc = ntc.abi.ReadChannels()
+    rc.planarPairs, rc.planarBytes = d_src.ptr, d_src.nbytes
+    rc.width, rc.height, rc.setChannels, rc.firstChannel, rc.numChannels = w, h, C_, first, count
+    rc.dst, rc.dstBytes, rc.format, rc.pixelStride, rc.rowPitch = d_dst.ptr, d_dst.nbytes, fmt, stride, pitch
+    rc.useDithering = dither
+    for i in range(16):
+        rc.srcColorSpaces[i], rc.dstColorSpaces[i] = src_cs[i], dst_cs[i]
+    ntc.abi.check(device.lib.ntc_hip_read_channels(rc))
+    device.synchronize()
+    return d_dst.download()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fmt", [1, 2, 3, 4])
+def test_gpu_read_channels_dithering_is_bit_exact(ntc, device, oracle, fmt):
+    """Linear colour spaces: the noise generator is integer arithmetic and the rest IEEE float32."""
+    rng = np.random.default_rng(80 + fmt)
+    w, h, C_ = 301, 17, 8
+    planar = unit_planar(rng, w, h, C_)
+    zeros = np.zeros(16, dtype=np.uint8)
+    for first, count, dst_channels in ((0, 8, 8), (2, 3, 4)):
+        stride = dst_channels * BPC[fmt]
+        pitch = w * stride + 8
+        got = gpu_read_ex(ntc, device, planar, w, h, C_, first, count, fmt, stride, pitch, 1, zeros, zeros)
+        want = np.full(h * pitch, 0xEE, dtype=np.uint8)
+        assert oracle.ntc_oracle_read_channels_ex(planar.ctypes.data, w, h, C_, first, count, want.ctypes.data, fmt, stride, pitch, 1,
+                                                  zeros.ctypes.data, zeros.ctypes.data) == 0
+        assert np.array_equal(got, want), (fmt, first)
+    if fmt == 1:      # the noise does something: about a quarter of the codes move against the undithered read
+        plain = gpu_read_ex(ntc, device, planar, w, h, C_, 0, 8, 1, 8, w * 8, 0, zeros, zeros)
+        noisy = gpu_read_ex(ntc, device, planar, w, h, C_, 0, 8, 1, 8, w * 8, 1, zeros, zeros)
+        moved = (plain != noisy).mean()
+        assert 0.15 < moved < 0.35 and np.abs(plain.astype(int) - noisy.astype(int)).max() == 1
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fmt", [1, 2, 3, 4])
+def test_gpu_read_channels_color_spaces_within_one_code(ntc, device, oracle, fmt):
+    """sRGB / HLG: powf, expf, logf, sqrtf come from different math libraries on the two sides, so
+    the comparison allows 1 code of UNORM8, 3 of UNORM16, 1 ulp of fp16, 4e-6 relative in fp32."""
+    rng = np.random.default_rng(90 + fmt)
+    w, h, C_ = 257, 9, 6
+    planar = unit_planar(rng, w, h, C_)
+    src_cs = np.array([0, 1, 2, 0, 1, 2] + [0] * 10, dtype=np.uint8)
+    dst_cs = np.array([1, 0, 0, 2, 2, 1] + [0] * 10, dtype=np.uint8)
+    stride = C_ * BPC[fmt]
+    pitch = w * stride
+    got = gpu_read_ex(ntc, device, planar, w, h, C_, 0, C_, fmt, stride, pitch, 0, src_cs, dst_cs)
+    want = np.zeros(h * pitch, dtype=np.uint8)
+    assert oracle.ntc_oracle_read_channels_ex(planar.ctypes.data, w, h, C_, 0, C_, want.ctypes.data, fmt, stride, pitch, 0,
+                                              src_cs.ctypes.data, dst_cs.ctypes.data) == 0
+    if fmt == 1:
+        assert np.abs(got.astype(int) - want.astype(int)).max() <= 1 and (got != want).mean() < 0.01
+    elif fmt == 2:
+        assert np.abs(got.view(np.uint16).astype(int) - want.view(np.uint16).astype(int)).max() <= 3
+    elif fmt == 3:
+        assert np.abs(got.view(np.int16).astype(int) - want.view(np.int16).astype(int)).max() <= 1
+    else:
+        a, b = got.view(np.float32).astype(np.float64), want.view(np.float32).astype(np.float64)
+        assert np.all(np.abs(a - b) <= 4e-6 * np.abs(b) + 1e-9)
+
+
+@pytest.mark.gpu
+def test_gpu_write_channels_color_spaces_within_one_ulp(ntc, device, oracle):
+    rng = np.random.default_rng(95)
+    w, h, C_ = 130, 11, 6
+    img, _, stride, pitch = random_user_image(rng, 1, w, h, C_, 4)
+    src_cs = np.array([1, 1, 2, 0, 0, 2] + [0] * 10, dtype=np.uint8)
+    dst_cs = np.array([0, 2, 0, 1, 2, 2] + [0] * 10, dtype=np.uint8)
+    start = np.zeros(w * h * C_, dtype=np.uint16)
+    d_src, d_dst = device.upload(img), device.upload(start)
+    wc = ntc.abi.WriteChannels()
+    wc.src, wc.srcBytes, wc.format, wc.verticalFlip, wc.pixelStride, wc.rowPitch = d_src.ptr, d_src.nbytes, 1, 0, stride, pitch
+    wc.planarPairs, wc.planarBytes = d_dst.ptr, d_dst.nbytes
+    wc.width, wc.height, wc.setChannels, wc.firstChannel, wc.numChannels = w, h, C_, 0, C_
+    for i in range(16):
+        wc.srcColorSpaces[i], wc.dstColorSpaces[i] = src_cs[i], dst_cs[i]
+    ntc.abi.check(device.lib.ntc_hip_write_channels(wc))
+    device.synchronize()
+    want = start.copy()
+    assert oracle.ntc_oracle_write_channels_ex(img.ctypes.data, 1, 0, stride, pitch, want.ctypes.data, w, h, C_, 0, C_,
+                                               src_cs.ctypes.data, dst_cs.ctypes.data) == 0
+    got = d_dst.download().view(np.int16).astype(int)
+    assert np.abs(got - want.view(np.int16).astype(int)).max() <= 1
+    wc.dstColorSpaces[3] = 9
+    assert device.lib.ntc_hip_write_channels(wc) == ntc.abi.ERR_INVALID_ARG
