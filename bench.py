@@ -31,12 +31,65 @@ def macs(widths):
     return sum(a * b for a, b in zip(widths[:-1], widths[1:]))
 
 
+def bench_copy_kernels(args, ntc, dev):
+    """The streaming kernels around the decoder on one 4096x4096, 16-channel mip in the internal fp16
+    layout: read = ReadChannels to UNORM8 pixels, write = WriteChannels from UNORM8 pixels, loss =
+    per-channel squared error of two images.  Wall-clock per call, synchronised at both ends."""
+    import numpy as np
+    A = ntc.abi
+    size = args.size or 4096
+    w = h = size
+    channels = 16
+    rng = np.random.default_rng(0)
+    planar = rng.integers(0, 0x3C00, w * h * channels, dtype=np.uint16)          # halves in [0, 1)
+    d_planar = dev.upload(planar)
+    wl = args.workload
+    if wl == "read":
+        d_pixels = dev.alloc(w * h * channels)
+        rc = A.ReadChannels()
+        rc.planarPairs, rc.planarBytes = d_planar.ptr, d_planar.nbytes
+        rc.width, rc.height, rc.setChannels, rc.firstChannel, rc.numChannels = w, h, channels, 0, channels
+        rc.dst, rc.dstBytes, rc.format, rc.pixelStride, rc.rowPitch = d_pixels.ptr, d_pixels.nbytes, 1, channels, w * channels
+        run = lambda: A.check(dev.lib.ntc_hip_read_channels(rc))
+        bytes_per_texel, what = 2 * channels + channels, "ReadChannels, internal fp16 -> UNORM8 pixels"
+    elif wl == "write":
+        d_pixels = dev.upload(rng.integers(0, 256, w * h * channels, dtype=np.uint8))
+        wc = A.WriteChannels()
+        wc.src, wc.srcBytes, wc.format, wc.pixelStride, wc.rowPitch = d_pixels.ptr, d_pixels.nbytes, 1, channels, w * channels
+        wc.planarPairs, wc.planarBytes = d_planar.ptr, d_planar.nbytes
+        wc.width, wc.height, wc.setChannels, wc.firstChannel, wc.numChannels = w, h, channels, 0, channels
+        run = lambda: A.check(dev.lib.ntc_hip_write_channels(wc))
+        bytes_per_texel, what = channels + 2 * channels, "WriteChannels, UNORM8 pixels -> internal fp16"
+    else:
+        d_other = dev.upload(rng.integers(0, 0x3C00, w * h * channels, dtype=np.uint16))
+        mse = (C.c_float * 16)()
+        run = lambda: A.check(dev.lib.ntc_hip_image_loss(d_planar.ptr, d_other.ptr, d_planar.nbytes, w, h, channels, 0xFFFF, mse))
+        bytes_per_texel, what = 4 * channels, "per-channel squared error of two images in the internal fp16 layout"
+    for _ in range(args.warmup):
+        run()
+    dev.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run()
+    dev.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    gbs = w * h * bytes_per_texel / (ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "Gtexels/s of a streaming kernel around the decoder", "value": w * h / (ms * 1e-3) / 1e9, "unit": "Gtexels/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"{what}, {w}x{h}, {channels} channels", "device": dev.name, "compute_units": dev.compute_units},
+        "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+                     "bytes_per_texel": bytes_per_texel},
+        "cpu_baseline": None}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=30)   # the GPU clock takes ~30 launches to settle
-    ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4", "ref092"])
+    ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4", "ref092", "read", "write", "loss"])
     ap.add_argument("--size", type=int, default=0, help="override the texture size of the workload")
     ap.add_argument("--format", choices=["fp16", "unorm8"], default=None)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="time budget of the CPU-baseline sample")
@@ -53,6 +106,8 @@ def main():
 
     dev = ntc.Device(0)
     wl = args.workload
+    if wl in ("read", "write", "loss"):
+        return bench_copy_kernels(args, ntc, dev)
     fmt_name = args.format or {"cfg2": "unorm8"}.get(wl, "fp16")
     fmt = A.OUT_FP16_PLANAR_PAIRS if fmt_name == "fp16" else A.OUT_UNORM8_PIXELS
     queries = None

@@ -11,14 +11,13 @@
 
 namespace ntc_hip_dev {
 
-// WriteImageChannel, src/ImageProcessing.cu:141-164.  roundf = round half away from zero,
-// written as trunc + exact fraction test so that host and device agree on every input.
-__device__ __forceinline__ float round_half_away(float v)
+// u(clamp(roundf(p), 0, top)) of WriteImageChannel (src/ImageProcessing.cu:141-152) for the UNORM formats.
+// roundf rounds halves away from zero; for |p| < 2^23 it equals trunc(p + copysign(c, p)) with c the
+// largest float below 1/2 (the sum rounds up to the next integer exactly when the fraction is at
+// least 1/2), and negative p end at 0 either way, so: max with 0, add c, cap, truncating conversion.
+__device__ __forceinline__ uint32_t unorm_code(float p, float top)
 {
-    float r = truncf(v);
-    float const fr = v - r;                                  // exact
-    if (fr >= 0.5f) r += 1.f; else if (fr <= -0.5f) r -= 1.f;
-    return r;
+    return uint32_t(fminf(fmaxf(p, 0.f) + 0.49999997f, top));
 }
 
 // Transfer functions, src/CudaUtils.h:61-114 (sRGB, Hybrid Log-Gamma) and src/ImageProcessing.cu:86-111.
@@ -74,104 +73,185 @@ struct DitherRng {
     }
 };
 
-__device__ __forceinline__ void write_channel(uint8_t* px, uint32_t ch, int format, int colorSpace, float value, float dither)
+constexpr int kRowsPerGroup = 4;       // image rows one workgroup of the copy kernels covers (more rows per workgroup measured slower)
+
+constexpr int bytes_per_channel(int format)
+{
+    return format == NTC_HIP_DEV_FORMAT_UNORM8 ? 1 : (format == NTC_HIP_DEV_FORMAT_UNORM16 || format == NTC_HIP_DEV_FORMAT_FLOAT16) ? 2 : 4;
+}
+
+// WriteImageChannel (src/ImageProcessing.cu:141-164): the channel's bits in the destination format.
+template <int FORMAT>
+__device__ __forceinline__ uint32_t encode_channel(int colorSpace, float value, bool dithering, float dither)
 {
     value = encode_color_space(colorSpace, value);
-    switch (format) {
-    case NTC_HIP_DEV_FORMAT_UNORM8:
-        value += dither / 255.f;
-        px[ch] = uint8_t(fmaxf(0.f, fminf(255.f, round_half_away(value * 255.f))));
-        break;
-    case NTC_HIP_DEV_FORMAT_UNORM16:
-        value += dither / 65535.f;
-        reinterpret_cast<uint16_t*>(px)[ch] = uint16_t(fmaxf(0.f, fminf(65535.f, round_half_away(value * 65535.f))));
-        break;
-    case NTC_HIP_DEV_FORMAT_FLOAT16: {
+    if constexpr (FORMAT == NTC_HIP_DEV_FORMAT_UNORM8) {
+        if (dithering) value += dither / 255.f;
+        return unorm_code(value * 255.f, 255.f);
+    } else if constexpr (FORMAT == NTC_HIP_DEV_FORMAT_UNORM16) {
+        if (dithering) value += dither / 65535.f;
+        return unorm_code(value * 65535.f, 65535.f);
+    } else if constexpr (FORMAT == NTC_HIP_DEV_FORMAT_FLOAT16) {
         float v = fmaxf(-65504.f, fminf(65504.f, value));
-        asm volatile("" : "+v"(v));
-        reinterpret_cast<_Float16*>(px)[ch] = (_Float16)v;
-        break;
-    }
-    case NTC_HIP_DEV_FORMAT_FLOAT32:
-        reinterpret_cast<float*>(px)[ch] = value;
-        break;
-    case NTC_HIP_DEV_FORMAT_UINT32:
-        reinterpret_cast<uint32_t*>(px)[ch] = uint32_t(fmaxf(value, 0.f));
-        break;
-    default:
-        break;
+        asm volatile("" : "+v"(v));                          // round the clamped value, not a fused expression
+        return uint32_t(__builtin_bit_cast(uint16_t, (_Float16)v));
+    } else if constexpr (FORMAT == NTC_HIP_DEV_FORMAT_FLOAT32) {
+        return __builtin_bit_cast(uint32_t, value);
+    } else {
+        return uint32_t(fmaxf(value, 0.f));
     }
 }
 
+// One lane per pixel.  The pixel is produced 16 bytes at a time (16 / 8 / 4 channels for 1 / 2 / 4-byte
+// formats) and stored with the widest access the image's alignment allows (a.vectorBytes, decided
+// on the host from base, pitch and stride); source halves come in as the dword pairs of the
+// planar-pair layout, coalesced across the lanes of a row.
+template <int FORMAT>
 __global__ void __launch_bounds__(256)
 read_channels_kernel(ReadChannelsArgs a)
 {
+    constexpr int BPC = bytes_per_channel(FORMAT), PER = 16 / BPC;
     int const x = blockIdx.x * 64 + (threadIdx.x & 63);
-    int const y = blockIdx.y * 4 + (threadIdx.x >> 6);
-    if (x >= a.width || y >= a.height) return;
+    if (x >= a.width) return;
+    for (int y = blockIdx.y * kRowsPerGroup + (threadIdx.x >> 6); y < min(a.height, int(blockIdx.y + 1) * kRowsPerGroup); y += 4) {
     // GetPixelBaseAddress / GetChannelAddress, src/RegressionKernels.h:36-45
     uint16_t const* src = a.planarPairs + size_t(y) * size_t(a.width) * size_t(a.setChannels) + size_t(x) * 2;
     uint8_t* px = a.dst + size_t(y) * a.rowPitch + size_t(x) * a.pixelStride;
     DitherRng rng(uint32_t(x) + uint32_t(y) * uint32_t(a.width));
-    for (int ch = 0; ch < a.dstChannels; ++ch) {
-        float value;
-        if (ch < a.numChannels) {
-            int const c = a.firstChannel + ch;
-            uint16_t const bits = src[size_t(c & ~1) * size_t(a.width) + size_t(c & 1)];
-            value = decode_color_space(a.srcColorSpaces[ch], float(__builtin_bit_cast(_Float16, bits)));
-        } else {
-            value = (ch == 3) ? 1.f : 0.f;                   // GetDefaultChannelValue, src/ImageProcessing.cu:166-170
+    int loadedPair = -1;
+    uint32_t pairBits = 0;
+    for (int base = 0; base < a.dstChannels; base += PER) {
+        uint32_t words[4] = { 0u, 0u, 0u, 0u };
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+            int const ch = base + k;
+            if (ch >= a.dstChannels) continue;               // uniform
+            float value;
+            if (ch < a.numChannels) {
+                int const c = a.firstChannel + ch;
+                if ((c >> 1) != loadedPair) {
+                    loadedPair = c >> 1;
+                    pairBits = *reinterpret_cast<uint32_t const*>(src + size_t(c & ~1) * size_t(a.width));
+                }
+                uint16_t const bits = uint16_t((c & 1) ? pairBits >> 16 : pairBits);
+                value = decode_color_space(a.srcColorSpaces[ch], float(__builtin_bit_cast(_Float16, bits)));
+            } else {
+                value = (ch == 3) ? 1.f : 0.f;               // GetDefaultChannelValue, src/ImageProcessing.cu:166-170
+            }
+            float const dither = a.useDithering ? rng.next_float() - 0.5f : 0.f;      // one draw per destination channel
+            uint32_t const bits = encode_channel<FORMAT>(ch < 16 ? a.dstColorSpaces[ch] : 0, value, a.useDithering != 0, dither);
+            words[(k * BPC) >> 2] |= bits << (8 * ((k * BPC) & 3));
         }
-        float const dither = a.useDithering ? rng.next_float() - 0.5f : 0.f;      // one draw per destination channel
-        write_channel(px, uint32_t(ch), a.format, ch < 16 ? a.dstColorSpaces[ch] : 0, value, dither);
+        int const bytes = min(PER, a.dstChannels - base) * BPC;
+        uint8_t* const out = px + base * BPC;
+        if (bytes == 16 && a.vectorBytes >= 16) {
+            *reinterpret_cast<uint4*>(out) = make_uint4(words[0], words[1], words[2], words[3]);
+        } else if ((bytes & 7) == 0 && a.vectorBytes >= 8) {
+            for (int q = 0; q < bytes / 8; ++q) reinterpret_cast<uint2*>(out)[q] = make_uint2(words[2 * q], words[2 * q + 1]);
+        } else if ((bytes & 3) == 0 && a.vectorBytes >= 4) {
+            for (int q = 0; q < bytes / 4; ++q) reinterpret_cast<uint32_t*>(out)[q] = words[q];
+        } else if constexpr (BPC == 1) {
+            for (int q = 0; q < bytes; ++q) out[q] = uint8_t(words[q >> 2] >> (8 * (q & 3)));
+        } else if constexpr (BPC == 2) {
+            for (int q = 0; q < bytes / 2; ++q) reinterpret_cast<uint16_t*>(out)[q] = uint16_t(words[q >> 1] >> (16 * (q & 1)));
+        } else {
+            for (int q = 0; q < bytes / 4; ++q) reinterpret_cast<uint32_t*>(out)[q] = words[q];
+        }
+    }
     }
 }
 
-// ReadImageChannel, src/ImageProcessing.cu:107-139 (linear colour space).
-__device__ __forceinline__ float read_channel(uint8_t const* px, uint32_t ch, int format)
+// ReadImageChannel, src/ImageProcessing.cu:113-139: channel k of a 16-byte piece of the pixel.
+template <int FORMAT>
+__device__ __forceinline__ float decode_channel(uint32_t const (&words)[4], int k, float const* unorm8Table)
 {
-    switch (format) {
-    case NTC_HIP_DEV_FORMAT_UNORM8:  return float(px[ch]) / 255.f;
-    case NTC_HIP_DEV_FORMAT_UNORM16: return float(reinterpret_cast<uint16_t const*>(px)[ch]) / 65535.f;
-    case NTC_HIP_DEV_FORMAT_FLOAT16: return float(reinterpret_cast<_Float16 const*>(px)[ch]);
-    case NTC_HIP_DEV_FORMAT_FLOAT32: return reinterpret_cast<float const*>(px)[ch];
-    case NTC_HIP_DEV_FORMAT_UINT32:  return float(reinterpret_cast<uint32_t const*>(px)[ch]);
-    default: return 0.f;
-    }
+    constexpr int BPC = bytes_per_channel(FORMAT);
+    uint32_t const w = words[(k * BPC) >> 2] >> (8 * ((k * BPC) & 3));
+    if constexpr (FORMAT == NTC_HIP_DEV_FORMAT_UNORM8)       return unorm8Table[w & 0xffu];          // = float(code) / 255.f
+    else if constexpr (FORMAT == NTC_HIP_DEV_FORMAT_UNORM16) return float(w & 0xffffu) / 65535.f;
+    else if constexpr (FORMAT == NTC_HIP_DEV_FORMAT_FLOAT16) return float(__builtin_bit_cast(_Float16, uint16_t(w)));
+    else if constexpr (FORMAT == NTC_HIP_DEV_FORMAT_FLOAT32) return __builtin_bit_cast(float, w);
+    else                                                     return float(w);
 }
 
 // User image -> internal fp16 planar pairs: ITextureSet::WriteChannels through CopyImageKernel's 1:1
-// branch (src/TextureSet.cpp:829-913, src/ImageProcessing.cu:220-265), optional vertical flip.
+// branch (src/TextureSet.cpp:835-913, src/ImageProcessing.cu:220-265), optional vertical flip.
+// The pixel is read 16 bytes at a time with the widest loads its alignment allows; channel pairs
+// that fall on a half2 of the internal layout are written as one dword.
+template <int FORMAT>
 __global__ void __launch_bounds__(256)
 write_channels_kernel(WriteChannelsArgs a)
 {
+    constexpr int BPC = bytes_per_channel(FORMAT), PER = 16 / BPC;
+    __shared__ float unorm8Table[FORMAT == NTC_HIP_DEV_FORMAT_UNORM8 ? 256 : 1];
+    if constexpr (FORMAT == NTC_HIP_DEV_FORMAT_UNORM8) {     // one correctly rounded division per code instead of per channel
+        unorm8Table[threadIdx.x & 255] = float(threadIdx.x & 255) / 255.f;
+        __syncthreads();
+    }
     int const x = blockIdx.x * 64 + (threadIdx.x & 63);
-    int const y = blockIdx.y * 4 + (threadIdx.x >> 6);
-    if (x >= a.width || y >= a.height) return;
+    if (x >= a.width) return;
+    for (int y = blockIdx.y * kRowsPerGroup + (threadIdx.x >> 6); y < min(a.height, int(blockIdx.y + 1) * kRowsPerGroup); y += 4) {
     int const srcY = a.verticalFlip ? a.height - 1 - y : y;          // SetupBilinearFilter flips the read position
     uint8_t const* px = a.src + size_t(srcY) * a.rowPitch + size_t(x) * a.pixelStride;
     uint16_t* dst = a.planarPairs + size_t(y) * size_t(a.width) * size_t(a.setChannels) + size_t(x) * 2;
-    for (int ch = 0; ch < a.numChannels; ++ch) {
-        float v = decode_color_space(a.srcColorSpaces[ch], read_channel(px, uint32_t(ch), a.format));
-        v = encode_color_space(a.dstColorSpaces[ch], v);
-        v = fmaxf(-65504.f, fminf(65504.f, v));                      // WriteImageChannel FLOAT16, src/ImageProcessing.cu:154-156
-        asm volatile("" : "+v"(v));
-        int const c = a.firstChannel + ch;
-        dst[size_t(c & ~1) * size_t(a.width) + size_t(c & 1)] = __builtin_bit_cast(uint16_t, (_Float16)v);
+    uint32_t pending = 0;                                            // low half of a pair waiting for its partner
+    for (int base = 0; base < a.numChannels; base += PER) {
+        int const bytes = min(PER, a.numChannels - base) * BPC;
+        uint8_t const* const in = px + base * BPC;
+        uint32_t words[4] = { 0u, 0u, 0u, 0u };
+        if (bytes == 16 && a.vectorBytes >= 16) {
+            uint4 const v = *reinterpret_cast<uint4 const*>(in);
+            words[0] = v.x; words[1] = v.y; words[2] = v.z; words[3] = v.w;
+        } else if ((bytes & 3) == 0 && a.vectorBytes >= 4) {
+            for (int q = 0; q < bytes / 4; ++q) words[q] = reinterpret_cast<uint32_t const*>(in)[q];
+        } else if constexpr (BPC == 1) {
+            for (int q = 0; q < bytes; ++q) words[q >> 2] |= uint32_t(in[q]) << (8 * (q & 3));
+        } else if constexpr (BPC == 2) {
+            for (int q = 0; q < bytes / 2; ++q) words[q >> 1] |= uint32_t(reinterpret_cast<uint16_t const*>(in)[q]) << (16 * (q & 1));
+        } else {
+            for (int q = 0; q < bytes / 4; ++q) words[q] = reinterpret_cast<uint32_t const*>(in)[q];
+        }
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+            int const ch = base + k;
+            if (ch >= a.numChannels) continue;                       // uniform
+            float v = decode_color_space(a.srcColorSpaces[ch], decode_channel<FORMAT>(words, k, unorm8Table));
+            v = encode_color_space(a.dstColorSpaces[ch], v);
+            v = fmaxf(-65504.f, fminf(65504.f, v));                  // WriteImageChannel FLOAT16, src/ImageProcessing.cu:154-156
+            asm volatile("" : "+v"(v));
+            uint32_t const half = __builtin_bit_cast(uint16_t, (_Float16)v);
+            int const c = a.firstChannel + ch;
+            uint16_t* const at = dst + size_t(c & ~1) * size_t(a.width);
+            if ((c & 1) == 0) {
+                if (ch + 1 < a.numChannels) pending = half;          // partner follows: store both together
+                else at[0] = uint16_t(half);
+            } else {
+                if (ch > 0) *reinterpret_cast<uint32_t*>(at) = pending | (half << 16);
+                else at[1] = uint16_t(half);
+            }
+        }
+    }
     }
 }
 
 hipError_t launch_write_channels(WriteChannelsArgs const& a, hipStream_t stream)
 {
-    dim3 const grid((a.width + 63) / 64, (a.height + 3) / 4);
-    hipLaunchKernelGGL(write_channels_kernel, grid, dim3(256), 0, stream, a);
+    dim3 const grid((a.width + 63) / 64, (a.height + kRowsPerGroup - 1) / kRowsPerGroup);
+    switch (a.format) {
+    case NTC_HIP_DEV_FORMAT_UNORM8:  hipLaunchKernelGGL(write_channels_kernel<NTC_HIP_DEV_FORMAT_UNORM8>, grid, dim3(256), 0, stream, a); break;
+    case NTC_HIP_DEV_FORMAT_UNORM16: hipLaunchKernelGGL(write_channels_kernel<NTC_HIP_DEV_FORMAT_UNORM16>, grid, dim3(256), 0, stream, a); break;
+    case NTC_HIP_DEV_FORMAT_FLOAT16: hipLaunchKernelGGL(write_channels_kernel<NTC_HIP_DEV_FORMAT_FLOAT16>, grid, dim3(256), 0, stream, a); break;
+    case NTC_HIP_DEV_FORMAT_FLOAT32: hipLaunchKernelGGL(write_channels_kernel<NTC_HIP_DEV_FORMAT_FLOAT32>, grid, dim3(256), 0, stream, a); break;
+    case NTC_HIP_DEV_FORMAT_UINT32:  hipLaunchKernelGGL(write_channels_kernel<NTC_HIP_DEV_FORMAT_UINT32>, grid, dim3(256), 0, stream, a); break;
+    default: return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 
 // Per-channel sum of squared differences between a decoded mip and its reference image, both in the
 // internal layout: the loss branch of InferenceKernel (src/Inference.cu:77-118) without its masking
-// options.  Each workgroup covers 64 x 16 texels and writes 16 double partial sums; the host adds the
-// partials (as ReduceLoss finishes its reduction on the host in double, src/Optimizer.cu:382-387).
+// options.  Each workgroup covers 64 x 16 texels and writes 16 double partial sums (channel-major, so
+// that the second stage reads them coalesced); ReduceLoss likewise finishes in double (src/Optimizer.cu:382-387).
 __global__ void __launch_bounds__(256)
 image_loss_kernel(uint16_t const* __restrict__ a, uint16_t const* __restrict__ b, int width, int height, int setChannels,
                   uint32_t validChannelMask, double* __restrict__ partials)
@@ -209,8 +289,27 @@ image_loss_kernel(uint16_t const* __restrict__ a, uint16_t const* __restrict__ b
     __syncthreads();
     if (threadIdx.x < NTC_HIP_DEV_MAX_CHANNELS) {
         int const c = threadIdx.x;
-        size_t const block = size_t(blockIdx.y) * gridDim.x + blockIdx.x;
-        partials[block * NTC_HIP_DEV_MAX_CHANNELS + c] = sums[0][c] + sums[1][c] + sums[2][c] + sums[3][c];
+        size_t const block = size_t(blockIdx.y) * gridDim.x + blockIdx.x, blocks = size_t(gridDim.x) * gridDim.y;
+        partials[size_t(c) * blocks + block] = sums[0][c] + sums[1][c] + sums[2][c] + sums[3][c];
+    }
+}
+
+// Second stage: workgroup c adds the partial sums of channel c, in double and in a fixed order
+// (thread t takes entries t, t + 256, ...; then one thread adds the 256 sub-totals), and writes the
+// total behind the partials.
+__global__ void __launch_bounds__(256)
+image_loss_reduce_kernel(double const* __restrict__ partials, size_t blocks, double* __restrict__ totals)
+{
+    __shared__ double sums[256];
+    int const c = blockIdx.x;
+    double acc = 0.0;
+    for (size_t b = threadIdx.x; b < blocks; b += 256) acc += partials[size_t(c) * blocks + b];
+    sums[threadIdx.x] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double total = 0.0;
+        for (int t = 0; t < 256; ++t) total += sums[t];
+        totals[c] = total;
     }
 }
 
@@ -218,14 +317,23 @@ hipError_t launch_image_loss(uint16_t const* a, uint16_t const* b, int width, in
                              uint32_t validChannelMask, double* partials, hipStream_t stream)
 {
     dim3 const grid((width + 63) / 64, (height + 15) / 16);
+    size_t const blocks = size_t(grid.x) * size_t(grid.y);
     hipLaunchKernelGGL(image_loss_kernel, grid, dim3(256), 0, stream, a, b, width, height, setChannels, validChannelMask, partials);
+    hipLaunchKernelGGL(image_loss_reduce_kernel, dim3(NTC_HIP_DEV_MAX_CHANNELS), dim3(256), 0, stream, partials, blocks, partials + blocks * NTC_HIP_DEV_MAX_CHANNELS);
     return hipGetLastError();
 }
 
 hipError_t launch_read_channels(ReadChannelsArgs const& a, hipStream_t stream)
 {
-    dim3 const grid((a.width + 63) / 64, (a.height + 3) / 4);
-    hipLaunchKernelGGL(read_channels_kernel, grid, dim3(256), 0, stream, a);
+    dim3 const grid((a.width + 63) / 64, (a.height + kRowsPerGroup - 1) / kRowsPerGroup);
+    switch (a.format) {
+    case NTC_HIP_DEV_FORMAT_UNORM8:  hipLaunchKernelGGL(read_channels_kernel<NTC_HIP_DEV_FORMAT_UNORM8>, grid, dim3(256), 0, stream, a); break;
+    case NTC_HIP_DEV_FORMAT_UNORM16: hipLaunchKernelGGL(read_channels_kernel<NTC_HIP_DEV_FORMAT_UNORM16>, grid, dim3(256), 0, stream, a); break;
+    case NTC_HIP_DEV_FORMAT_FLOAT16: hipLaunchKernelGGL(read_channels_kernel<NTC_HIP_DEV_FORMAT_FLOAT16>, grid, dim3(256), 0, stream, a); break;
+    case NTC_HIP_DEV_FORMAT_FLOAT32: hipLaunchKernelGGL(read_channels_kernel<NTC_HIP_DEV_FORMAT_FLOAT32>, grid, dim3(256), 0, stream, a); break;
+    case NTC_HIP_DEV_FORMAT_UINT32:  hipLaunchKernelGGL(read_channels_kernel<NTC_HIP_DEV_FORMAT_UINT32>, grid, dim3(256), 0, stream, a); break;
+    default: return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 

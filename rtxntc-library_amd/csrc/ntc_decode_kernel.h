@@ -61,6 +61,7 @@ struct ReadChannelsArgs {
     uint64_t pixelStride, rowPitch;
     int32_t width, height, setChannels, firstChannel, numChannels, dstChannels, format;
     int32_t useDithering;
+    int32_t vectorBytes;           // widest store every pixel start is aligned to: 16, 8, 4, 2 or 1
     uint8_t srcColorSpaces[16], dstColorSpaces[16];   // per copied channel: 0 linear, 1 sRGB, 2 HLG
 };
 hipError_t launch_read_channels(ReadChannelsArgs const& args, hipStream_t stream);
@@ -72,6 +73,7 @@ struct WriteChannelsArgs {
     uint16_t* planarPairs;
     uint64_t pixelStride, rowPitch;
     int32_t width, height, setChannels, firstChannel, numChannels, format, verticalFlip;
+    int32_t vectorBytes;           // widest load every pixel start is aligned to
     uint8_t srcColorSpaces[16], dstColorSpaces[16];
 };
 hipError_t launch_write_channels(WriteChannelsArgs const& args, hipStream_t stream);

@@ -527,6 +527,14 @@ int ntc_hip_decode_queries_timed(const NtcHipTextureSet* set, const NtcHipQuery*
     return run_queries(set, queries, numQueries, out, outBytes, iterations, outMillisecondsPerIteration);
 }
 
+// Largest power of two up to 16 that divides the base address, the row pitch and the pixel stride:
+// every pixel of the image starts on such a boundary.
+static int32_t common_alignment(uintptr_t base, uint64_t rowPitch, uint64_t pixelStride)
+{
+    uint64_t const bits = uint64_t(base) | rowPitch | pixelStride | 16u;
+    return int32_t(bits & (~bits + 1));
+}
+
 int ntc_hip_read_channels(const NtcHipReadChannels* p)
 {
     if (int r = require_init()) return r;
@@ -564,6 +572,7 @@ int ntc_hip_read_channels(const NtcHipReadChannels* p)
     a.firstChannel = p->firstChannel; a.numChannels = p->numChannels;
     a.dstChannels = int32_t(dstChannels); a.format = p->format;
     a.useDithering = p->useDithering ? 1 : 0;
+    a.vectorBytes = common_alignment(reinterpret_cast<uintptr_t>(p->dst), p->rowPitch, p->pixelStride);
     for (int i = 0; i < 16; ++i) {
         if (p->srcColorSpaces[i] > 2 || p->dstColorSpaces[i] > 2) { set_error("ntc_hip_read_channels: unknown colour space for channel %d.", i); return NTC_HIP_ERR_INVALID_ARG; }
         a.srcColorSpaces[i] = p->srcColorSpaces[i];
@@ -609,6 +618,7 @@ int ntc_hip_write_channels(const NtcHipWriteChannels* p)
     a.pixelStride = p->pixelStride; a.rowPitch = p->rowPitch;
     a.width = p->width; a.height = p->height; a.setChannels = p->setChannels;
     a.firstChannel = p->firstChannel; a.numChannels = p->numChannels; a.format = p->format; a.verticalFlip = p->verticalFlip ? 1 : 0;
+    a.vectorBytes = common_alignment(reinterpret_cast<uintptr_t>(p->src), p->rowPitch, p->pixelStride);
     for (int i = 0; i < 16; ++i) {
         if (p->srcColorSpaces[i] > 2 || p->dstColorSpaces[i] > 2) { set_error("ntc_hip_write_channels: unknown colour space for channel %d.", i); return NTC_HIP_ERR_INVALID_ARG; }
         a.srcColorSpaces[i] = p->srcColorSpaces[i];
@@ -630,27 +640,23 @@ int ntc_hip_image_loss(const void* decoded, const void* reference, uint64_t plan
         return NTC_HIP_ERR_INVALID_ARG;
     }
     size_t const blocks = image_loss_blocks(width, height);
-    size_t const bytes = blocks * NTC_HIP_DEV_MAX_CHANNELS * sizeof(double);
+    size_t const bytes = (blocks + 1) * NTC_HIP_DEV_MAX_CHANNELS * sizeof(double);    // partial sums, then the 16 totals
     Library& L = g_lib;
     if (bytes > L.lossBytes) {
         HIP_TRY(hipStreamSynchronize(L.stream));
         if (L.lossDev) { HIP_TRY(hipFree(L.lossDev)); L.lossDev = nullptr; }
-        if (L.lossHost) { HIP_TRY(hipHostFree(L.lossHost)); L.lossHost = nullptr; }
         L.lossBytes = 0;
         HIP_TRY(hipMalloc(reinterpret_cast<void**>(&L.lossDev), bytes));
-        HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&L.lossHost), bytes, hipHostMallocDefault));
+        if (!L.lossHost) HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&L.lossHost), NTC_HIP_DEV_MAX_CHANNELS * sizeof(double), hipHostMallocDefault));
         L.lossBytes = bytes;
     }
     HIP_TRY(launch_image_loss(static_cast<uint16_t const*>(decoded), static_cast<uint16_t const*>(reference), width, height,
                               setChannels, validChannelMask, L.lossDev, L.stream));
-    HIP_TRY(hipMemcpyAsync(L.lossHost, L.lossDev, bytes, hipMemcpyDeviceToHost, L.stream));
+    HIP_TRY(hipMemcpyAsync(L.lossHost, L.lossDev + blocks * NTC_HIP_DEV_MAX_CHANNELS, NTC_HIP_DEV_MAX_CHANNELS * sizeof(double),
+                           hipMemcpyDeviceToHost, L.stream));
     HIP_TRY(hipStreamSynchronize(L.stream));
     double const norm = 1.0 / (double(width) * double(height));
-    for (int c = 0; c < NTC_HIP_DEV_MAX_CHANNELS; ++c) {
-        double acc = 0.0;
-        for (size_t b = 0; b < blocks; ++b) acc += L.lossHost[b * NTC_HIP_DEV_MAX_CHANNELS + size_t(c)];
-        outMse[c] = float(acc * norm);
-    }
+    for (int c = 0; c < NTC_HIP_DEV_MAX_CHANNELS; ++c) outMse[c] = float(L.lossHost[c] * norm);
     clear_error();
     return 0;
 }
