@@ -573,8 +573,24 @@ __device__ __forceinline__ void prepare_inputs_general(DevMip const& m, int x, i
 }
 
 // Input vector of one texel from integer arithmetic only (see axis_fast above).
-template <class V>
-__device__ __forceinline__ void prepare_inputs_fast(DevMip const& m, LdsT<V> const& lds, int x, int y, uint32_t (&in)[16])
+// The two horizontally adjacent cells (x0, y) and (x0 + 1, y) as one dword: low half = left cell.
+// Cells are 2 bytes, so the dword may sit on a 2-byte boundary; global memory takes such loads.
+// A footprint that wraps around the grid edge (x1 = 0) cannot be fetched this way -- the dword
+// would run past the row -- and takes two 16-bit loads instead.
+typedef uint32_t __attribute__((aligned(2))) u32_align2;
+__device__ __forceinline__ uint32_t load_cell_pair(GlobalU8Ptr base, uint32_t off0, uint32_t off1)
+{
+    if (off1 == off0 + 2u)
+        return *reinterpret_cast<__attribute__((address_space(1))) u32_align2 const*>(base + off0);
+    return load_u16(base, off0) | (load_u16(base, off1) << 16);
+}
+
+// PAIR_LOADS: fetch horizontally adjacent taps with one load (load_cell_pair).  Halves the number
+// of memory instructions, at a few extra vector operations per tap: pays where the loads are
+// scattered (random-access queries), not in the raster decode, which is bound by vector issue.
+// `Mip` is DevMip or any struct with the same members for the fields used here (QueryMip).
+template <class V, bool PAIR_LOADS = false, class Mip = DevMip>
+__device__ __forceinline__ void prepare_inputs_fast(Mip const& m, LdsT<V> const& lds, int x, int y, uint32_t (&in)[16])
 {
 #pragma unroll
     for (int i = 0; i < 16; ++i) in[i] = 0;
@@ -589,12 +605,23 @@ __device__ __forceinline__ void prepare_inputs_fast(DevMip const& m, LdsT<V> con
         uint32_t const a00 = r0 + c0, a10 = r0 + c1, a01 = r1 + c0, a11 = r1 + c1;   // byte offsets
         if constexpr (V::HR_MODE == 1) {
             static_assert(V::HR_MODE != 1 || (V::HR_BITS == 2 && V::HR_F == 8 && V::HR_SLOTS == 8), "concat grids: 8 x 2-bit");
-            uint32_t const addr[4] = { a00, a10, a01, a11 };
+            if constexpr (PAIR_LOADS) {
+                uint32_t const row[2] = { load_cell_pair(g, a00, a10), load_cell_pair(g, a01, a11) };
 #pragma unroll
-            for (int tap = 0; tap < 4; ++tap) {
-                uint32_t const w = load_u16(g, addr[tap]);
-                in[2 * tap]     = lds.lut2[w & 0xffu];
-                in[2 * tap + 1] = lds.lut2[w >> 8];
+                for (int r = 0; r < 2; ++r) {
+                    in[4 * r]     = lds.lut2[row[r] & 0xffu];
+                    in[4 * r + 1] = lds.lut2[(row[r] >> 8) & 0xffu];
+                    in[4 * r + 2] = lds.lut2[(row[r] >> 16) & 0xffu];
+                    in[4 * r + 3] = lds.lut2[row[r] >> 24];
+                }
+            } else {
+                uint32_t const addr[4] = { a00, a10, a01, a11 };
+#pragma unroll
+                for (int tap = 0; tap < 4; ++tap) {
+                    uint32_t const w = load_u16(g, addr[tap]);
+                    in[2 * tap]     = lds.lut2[w & 0xffu];
+                    in[2 * tap + 1] = lds.lut2[w >> 8];
+                }
             }
         } else {
             uint32_t const nx = (m.hrAxisX >> 8) & 0xffu, ny = (m.hrAxisY >> 8) & 0xffu;
@@ -604,8 +631,14 @@ __device__ __forceinline__ void prepare_inputs_fast(DevMip const& m, LdsT<V> con
 #pragma unroll
             for (int L = 0; L < layers; ++L) {
                 GlobalU8Ptr const gl = g + size_t(L) * layerStride;
-                uint32_t b = bilinear4_int(load_u16(gl, a00), load_u16(gl, a10), load_u16(gl, a01), load_u16(gl, a11),
-                                           w00, w10, w01, w11, nx + ny);
+                uint32_t b;
+                if constexpr (PAIR_LOADS) {
+                    uint32_t const p0 = load_cell_pair(gl, a00, a10), p1 = load_cell_pair(gl, a01, a11);
+                    b = bilinear4_int(p0 & 0xffffu, p0 >> 16, p1 & 0xffffu, p1 >> 16, w00, w10, w01, w11, nx + ny);
+                } else {
+                    b = bilinear4_int(load_u16(gl, a00), load_u16(gl, a10), load_u16(gl, a01), load_u16(gl, a11),
+                                      w00, w10, w01, w11, nx + ny);
+                }
                 if (4 * L + 4 > V::HR_F) b &= (1u << (8 * (V::HR_F - 4 * L))) - 1u;
                 in[L] = b;
             }
@@ -626,8 +659,14 @@ __device__ __forceinline__ void prepare_inputs_fast(DevMip const& m, LdsT<V> con
 #pragma unroll
         for (int L = 0; L < layers; ++L) {
             GlobalU8Ptr const gl = g + size_t(L) * layerStride;
-            uint32_t b = bilinear4_int(load_u16(gl, a00), load_u16(gl, a10), load_u16(gl, a01), load_u16(gl, a11),
-                                       w00, w10, w01, w11, nx + ny);
+            uint32_t b;
+            if constexpr (PAIR_LOADS) {
+                uint32_t const p0 = load_cell_pair(gl, a00, a10), p1 = load_cell_pair(gl, a01, a11);
+                b = bilinear4_int(p0 & 0xffffu, p0 >> 16, p1 & 0xffffu, p1 >> 16, w00, w10, w01, w11, nx + ny);
+            } else {
+                b = bilinear4_int(load_u16(gl, a00), load_u16(gl, a10), load_u16(gl, a01), load_u16(gl, a11),
+                                  w00, w10, w01, w11, nx + ny);
+            }
             if (4 * L + 4 > V::LR_F) b &= (1u << (8 * (V::LR_F - 4 * L))) - 1u;
             in[V::HR_INPUTS / 4 + L] = b;
         }
@@ -961,12 +1000,37 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
 // the image, as 16 fp16.  Lane = query in the input stage (each lane carries its own mip, so the
 // per-lane form of either input stage is used); the network is the same 64-column tile as in raster decode.
 // A query whose mip is out of range writes zeros.
+// What a query needs of its mip, kept in LDS: every lane of a wave may address another mip, and
+// fetching these fields per lane from the table in global memory put a long dependent load in
+// front of the latent gathers.
+struct QueryMip {
+    uint16_t const* hr;
+    uint16_t const* lr;
+    uint32_t hrAxisX, hrAxisY, lrAxisX, lrAxisY;
+    int32_t hrWidth, hrHeight, lrWidth, lrHeight;
+    int32_t width, height;
+    uint32_t posMask, fast;
+    float positionLod;
+    uint32_t pad[3];
+};
+static_assert(sizeof(QueryMip) == 80, "QueryMip layout");
+
 template <class V>
 __global__ void __launch_bounds__(256, 2)
 query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __restrict__ queries, uint64_t numQueries,
              uint16_t* __restrict__ out)
 {
     __shared__ LdsT<V> lds;
+    __shared__ QueryMip qmips[16];
+    if (threadIdx.x < 16) {
+        DevMip const& d = mips[min(int(threadIdx.x), numMips - 1)];
+        QueryMip& q = qmips[threadIdx.x];
+        q.hr = d.hr; q.lr = d.lr;
+        q.hrAxisX = d.hrAxisX; q.hrAxisY = d.hrAxisY; q.lrAxisX = d.lrAxisX; q.lrAxisY = d.lrAxisY;
+        q.hrWidth = d.hrWidth; q.hrHeight = d.hrHeight; q.lrWidth = d.lrWidth; q.lrHeight = d.lrHeight;
+        q.width = d.width; q.height = d.height;
+        q.posMask = d.posMask; q.fast = d.fast; q.positionLod = d.positionLod;
+    }
     int const lane = threadIdx.x & 63;
     int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int const j = lane & 15, g = lane >> 4;
@@ -991,14 +1055,14 @@ query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __res
         uint64_t const qi = min(q0 + uint64_t(lane), numQueries - 1);
         DevQuery const query = queries[qi];
         bool const validMip = query.mip >= 0 && query.mip < numMips;
-        DevMip const& m = mips[validMip ? query.mip : 0];
+        QueryMip const& m = qmips[validMip ? query.mip : 0];
         int x = int(floorf(query.u * float(m.width)));
         int y = int(floorf(query.v * float(m.height)));
         x = max(0, min(x, m.width - 1));
         y = max(0, min(y, m.height - 1));
         uint32_t in[16];
-        if (__all(m.fast != 0)) prepare_inputs_fast<V>(m, lds, x, y, in);     // every lane's mip is power-of-two sized
-        else                    prepare_inputs_general<V>(m, x, y, in);
+        if (__all(m.fast != 0)) prepare_inputs_fast<V, true>(m, lds, x, y, in);   // every lane's mip is power-of-two sized
+        else                    prepare_inputs_general<V>(mips[validMip ? query.mip : 0], x, y, in);
 
         // output-layer accumulators as floats: exact either way (|acc| < 2^24 on the fp16 path; the
         // int32 -> float conversion is the definition's on the int8 path)
