@@ -152,12 +152,16 @@ typedef float    v2f __attribute__((ext_vector_type(2)));
 // (IsHalfSpecial, Inference.cu:125-126).  |o| >= 65520 is exactly the set that rounds to
 // Inf.  The empty asm keeps the compiler from folding multiply + convert into
 // v_fma_mixlo_f16, which rounds the exact product once, straight to half.
+// CHECKED = false is for callers that know |a|, |b| stay far below 65520.
+template <bool CHECKED = true>
 __device__ __forceinline__ uint32_t to_half2_bits(float a, float b)
 {
     asm("" : "+v"(a));
     asm("" : "+v"(b));
-    a = (__builtin_fabsf(a) < 65520.f) ? a : 0.f;
-    b = (__builtin_fabsf(b) < 65520.f) ? b : 0.f;
+    if constexpr (CHECKED) {
+        a = (__builtin_fabsf(a) < 65520.f) ? a : 0.f;
+        b = (__builtin_fabsf(b) < 65520.f) ? b : 0.f;
+    }
     v2h const h = __builtin_convertvector(v2f{a, b}, v2h);
     return __builtin_bit_cast(uint32_t, h);
 }
@@ -205,7 +209,7 @@ __device__ __forceinline__ void store_channels(GlobalOutPtr row, uint32_t laneOf
     }
 }
 
-template <int FORMAT, class Acc>
+template <int FORMAT, bool CHECKED = true, class Acc>
 __device__ __forceinline__ void store_tile(DevMip const& m, Acc const (&D)[4], v4f S, int x, int y0, int chBase)
 {
     int const nch = min(4, m.numChannels - chBase);
@@ -219,8 +223,8 @@ __device__ __forceinline__ void store_tile(DevMip const& m, Acc const (&D)[4], v
     for (int b = 0; b < 4; ++b) {
         int const y = y0 + b;
         if (y >= m.height) break;                            // uniform
-        uint32_t const h01 = to_half2_bits(float(D[b][0]) * S[0], float(D[b][1]) * S[1]);
-        uint32_t const h23 = to_half2_bits(float(D[b][2]) * S[2], float(D[b][3]) * S[3]);
+        uint32_t const h01 = to_half2_bits<CHECKED>(float(D[b][0]) * S[0], float(D[b][1]) * S[1]);
+        uint32_t const h23 = to_half2_bits<CHECKED>(float(D[b][2]) * S[2], float(D[b][3]) * S[3]);
         store_channels<FORMAT>((GlobalOutPtr)m.out + size_t(y) * rowBytes, laneOff, uint32_t(m.width) * 4u, h01, h23, nch);
     }
 }
@@ -340,11 +344,14 @@ __device__ __forceinline__ uint32_t halves_of_bytes(uint32_t v, int firstByte)  
 }
 
 // Copies the int8 blob (src/WeightLayout.cpp:42-49: matrices, then fp32 scales, then int32
-// biases; W[c*IN + k]) into LDS in MFMA operand order.  Returns true when layers 1..3 were staged
-// for the fp16 matrix instruction (see mlp_forward_f16): that needs, for every channel of those
-// layers, |bias - 113*sum(W)| + 240*sum|W| < 2^24.  Otherwise they are staged as int8 tiles.
+// biases; W[c*IN + k]) into LDS in MFMA operand order.  Returns kStagedF16 when layers 1..3 were
+// staged for the fp16 matrix instruction (see mlp_forward_f16): that needs, for every channel of
+// those layers, |bias - 113*sum(W)| + 240*sum|W| < 2^24; otherwise they are staged as int8 tiles.
+// With kStagedF16, kOutputsBounded says that no output can come near the fp16 overflow threshold
+// (the same bound times the channel's scale stays below 60000), so stores may skip that check.
+constexpr int kStagedF16 = 1, kOutputsBounded = 2;
 template <class V>
-__device__ bool stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
+__device__ int stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
 {
     constexpr int ins[4]   = { V::IN, V::H0, V::H1, V::H2 };
     constexpr int tiles[4] = { V::T0, V::T1, V::T2, V::T3 };
@@ -399,10 +406,10 @@ __device__ bool stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
         }
     }
     if constexpr (!V::F16_LAYERS) {
-        return false;
+        return 0;
     } else {
         // One thread per channel of layers 1..3: row sums decide whether the fp16 path is exact.
-        bool fits = true;
+        bool fits = true, bounded = true;
         int64_t shifted = 0;
         int slotTile = 0, slotG = 0, slotR = 0;
         if (threadIdx.x < V::LATE_CHANNELS) {
@@ -425,11 +432,13 @@ __device__ bool stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
             shifted = int64_t(bias) - 113 * int64_t(sum);     // activations enter as q + 113 in [-15, 240]
             int64_t const bound = (shifted < 0 ? -shifted : shifted) + 240 * int64_t(sumAbs);
             fits = bound < (int64_t(1) << 24);
+            if (l == 3) bounded = float(bound) * fabsf(reinterpret_cast<float const*>(blob + V::SCALE_OFF)[V::H0 + c]) < 60000.f;
             slotTile = V::T0 + (l == 1 ? 0 : (l == 2 ? V::T1 : V::T1 + V::T2)) + row / 16;
             slotG = (row >> 2) & 3;
             slotR = row & 3;
         }
         bool const useF16 = __syncthreads_and(fits ? 1 : 0) != 0;     // also orders the bias writes above
+        bool const outputsBounded = __syncthreads_and(bounded ? 1 : 0) != 0;
         if (useF16) {
             if (threadIdx.x < V::LATE_CHANNELS)
                 lds.bias[slotTile][slotG][slotR] = __builtin_bit_cast(int32_t, float(shifted));
@@ -470,7 +479,7 @@ __device__ bool stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
                 tileBase += tiles[l];
             }
         }
-        return useF16;
+        return useF16 ? (kStagedF16 | (outputsBounded ? kOutputsBounded : 0)) : 0;
     }
 }
 
@@ -922,8 +931,10 @@ __device__ __forceinline__ void mlp_forward_f16(LdsT<V>& lds, int wave, int lane
     f16_tile<V, V::T2>(lds, V::F16_L3, 0, lane, Ha, D);
 }
 
+// Four workgroups per CU (16 waves, 128 VGPRs each) is what the LDS footprint allows and what hides
+// the latency of the input stage; the e4m3 variants hold three weight planes in LDS and fit two.
 template <class V>
-__global__ void __launch_bounds__(256, 2)
+__global__ void __launch_bounds__(256, V::FP8_WEIGHTS ? 2 : 4)
 decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
 {
     __shared__ LdsT<V> lds;
@@ -949,7 +960,7 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     build_posenc_tables<V>(lds);
 
     uint8_t const* stagedBlob = nullptr;
-    bool useF16 = false;                                     // uniform: how layers 1..3 of the staged set run
+    int staged = 0;                                          // uniform: how layers 1..3 of the staged set run (kStagedF16, ...)
     int entry = 0;
 
     for (int tile = tileBegin; tile < tileEnd; ++tile) {
@@ -958,7 +969,7 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
 
         if (m.weights != stagedBlob) {                       // uniform across the workgroup
             __syncthreads();
-            useF16 = stage_weights<V>(lds, m.weights);
+            staged = stage_weights<V>(lds, m.weights);
             stagedBlob = m.weights;
             __syncthreads();                                 // also publishes the tables built above
         }
@@ -977,13 +988,19 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
             else        prepare_inputs_general<V>(m, x, y, in);
         }
         // ---- 2.-4. transpose, hidden layers, output layer
-        if (V::F16_LAYERS && useF16) {
+        if (V::F16_LAYERS && (staged & kStagedF16)) {
             v4f D[4];
             v4f S;
             mlp_forward_f16<V>(lds, wave, lane, in, D, S);
-            if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)      store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, x0 + j, y0, 4 * g);
-            else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)       store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
-            else                                                       store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
+            if (staged & kOutputsBounded) {
+                if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)  store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS, false>(m, D, S, x0 + j, y0, 4 * g);
+                else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)   store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS, false>(m, D, S, x0 + j, y0, 4 * g);
+                else                                                   store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS, false>(m, D, S, x0 + j, y0, 4 * g);
+            } else {
+                if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)  store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, x0 + j, y0, 4 * g);
+                else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)   store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
+                else                                                   store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
+            }
         } else {
             v4i D[4];
             v4f S;
@@ -1016,7 +1033,7 @@ struct QueryMip {
 static_assert(sizeof(QueryMip) == 80, "QueryMip layout");
 
 template <class V>
-__global__ void __launch_bounds__(256, 2)
+__global__ void __launch_bounds__(256, V::FP8_WEIGHTS ? 2 : 4)
 query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __restrict__ queries, uint64_t numQueries,
              uint16_t* __restrict__ out)
 {
@@ -1045,7 +1062,7 @@ query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __res
         lds.lut2[threadIdx.x & 0xffu] = (x * 85u) ^ 0x80808080u;
     }
     build_posenc_tables<V>(lds);
-    bool const useF16 = stage_weights<V>(lds, mips[0].weights);
+    bool const useF16 = (stage_weights<V>(lds, mips[0].weights) & kStagedF16) != 0;
     __syncthreads();
 
     uint64_t const numBlocks = (numQueries + 255) / 256;

@@ -190,6 +190,19 @@ def test_fp16_layer_path_boundary(ntc, device, slack):
         assert_equal_bytes(expected, got, f"fp16 path boundary, slack {slack}, sign {sign}")
 
 
+def test_outputs_beyond_the_fp16_range_become_zero(ntc, device):
+    """Large output scales: network outputs pass 65520 in magnitude, which the contract stores as 0
+    (Inference.cu:125-126).  The weights still qualify for the fp16 form of layers 1..3, but not for
+    its unchecked stores; the checker must agree byte for byte and zeros must actually occur."""
+    spec = ntc.presets.spec_cfg01()
+    blob = ntc.synth.make_weights(spec, 77, scale_log2_range=(-2.0, 1.0))
+    case = cfg_case(ntc, spec, 256, 128, 4, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=78, weights=blob)
+    expected, got = run_both(device, case)
+    assert_equal_bytes(expected, got, "overflowing outputs")
+    halves = np.asarray(expected).view(np.uint16)
+    assert (halves == 0).mean() > 0.01 and (np.abs(halves.view(np.float16).astype(np.float32)) > 30000).mean() > 0.01
+
+
 def test_decode_is_idempotent_and_timed_variant_matches(ntc, device):
     case = cfg_case(ntc, ntc.presets.spec_cfg01(), 320, 200, 4, 16, ntc.abi.OUT_UNORM8_PIXELS, seed=21, scale_log2_range=ACTIVE)
     dset = case.device_set(device)
