@@ -63,7 +63,7 @@ def bench_copy_kernels(args, ntc, dev):
     else:
         d_other = dev.upload(rng.integers(0, 0x3C00, w * h * channels, dtype=np.uint16))
         mse = (C.c_float * 16)()
-        run = lambda: A.check(dev.lib.ntc_hip_image_loss(d_planar.ptr, d_other.ptr, d_planar.nbytes, w, h, channels, 0xFFFF, mse))
+        run = lambda: A.check(dev.lib.ntc_hip_image_loss(d_planar.ptr, d_other.ptr, d_planar.nbytes, w, h, channels, 0xFFFF, -1, 0, mse))
         bytes_per_texel, what = 4 * channels, "per-channel squared error of two images in the internal fp16 layout"
     for _ in range(args.warmup):
         run()

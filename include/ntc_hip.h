@@ -234,10 +234,16 @@ int ntc_hip_write_channels(const NtcHipWriteChannels* params);
 
 /* Mean squared error per channel between two images in the internal layout (a decoded mip and its
  * reference): the loss branch of InferenceKernel + ReduceLoss (src/Inference.cu:77-118,142-156,
- * src/Optimizer.cu:335-390) as a pass of its own, without the alpha-mask options.  Channels whose bit
- * is clear in validChannelMask report 0.  outMse receives 16 floats.  Synchronous. */
-int ntc_hip_image_loss(const void* decodedPlanarPairs, const void* referencePlanarPairs, uint64_t planarBytes,
-                       int32_t width, int32_t height, int32_t setChannels, uint32_t validChannelMask, float* outMse);
+ * src/Optimizer.cu:335-390) as a pass of its own.  Channels whose bit is clear in validChannelMask
+ * report 0.  maskChannelIndex / discardMaskedOutPixels are the alpha-mask options of
+ * ITextureSet::SetMaskChannelIndex (include/libntc/ntc.h:936-940): with an index >= 0 the DECODED mask
+ * channel is clamped to [0, 1] in place before it is compared (Inference.cu:96-97), and with the
+ * discard flag texels whose reference mask value is zero count on the mask channel only
+ * (Inference.cu:80-84,107-108).  A negative index means no mask channel; the decoded image is then only
+ * read.  outMse receives 16 floats.  Synchronous. */
+int ntc_hip_image_loss(void* decodedPlanarPairs, const void* referencePlanarPairs, uint64_t planarBytes,
+                       int32_t width, int32_t height, int32_t setChannels, uint32_t validChannelMask,
+                       int32_t maskChannelIndex, int32_t discardMaskedOutPixels, float* outMse);
 
 /* Self-check of the MFMA operand layout the kernels assume: multiplies a 16x64 by a
  * 64x16 int8 matrix on the device (row-major host arrays), writes the 16x16 int32

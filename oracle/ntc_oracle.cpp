@@ -42,7 +42,10 @@
  *   decode_queries           the raster decode of the texels the queries hit (tests/test_queries.py)
  *   read_channels,           numpy models of the 1:1 branch of cuda::CopyImage, five channel
  *   write_channels           formats, padded rows, vertical flip (tests/test_host_api.py)
- *   image_loss               numpy float64 mean squared error (tests/test_host_api.py)
+ *   image_loss,              numpy float64 mean squared error, with the mask options restated from
+ *   image_loss_masked        src/Inference.cu:80-112 in numpy and three special cases: no zero in the
+ *                            mask = no mask, all masked = mask channel only, clamp idempotent
+ *                            (tests/test_host_api.py)
  *   The exact bits of the reference's FP16-WMMA CUDA kernel (half accumulation order,
  *   --use_fast_math) and of a hardware bilinear sampler are NOT reproduced: parity unpinned
  *   for those two, by construction; the integer contract of Inference.hlsli is what is pinned.
@@ -694,6 +697,35 @@ void ntc_oracle_image_loss(const uint16_t* a, const uint16_t* b, int width, int 
                 acc += d * d;
             }
             outMse[c] += acc;
+        }
+    for (int c = 0; c < 16; ++c) outMse[c] /= double(width) * double(height);
+}
+
+// The same with the alpha-mask options of the loss branch (src/Inference.cu:80-84,96-97,107-108,112):
+// the decoded mask channel is clamped to [0, 1] IN PLACE (a negative zero becomes +0: the device
+// max(0.f, x) of the reference returns +0 for x = -0), and with discardMaskedOut a texel whose
+// reference mask value is +-0 counts on the mask channel only.
+void ntc_oracle_image_loss_masked(uint16_t* a, const uint16_t* b, int width, int height, int setChannels,
+                                  uint32_t validChannelMask, int maskChannel, int discardMaskedOut, double* outMse /* 16 */)
+{
+    for (int c = 0; c < 16; ++c) outMse[c] = 0.0;
+    auto at = [&](int x, int y, int c) {
+        return size_t(y) * size_t(width) * size_t(setChannels) + size_t(c & ~1) * size_t(width) + size_t(x) * 2 + size_t(c & 1);
+    };
+    for (int y = 0; y < height; ++y)
+        for (int x = 0; x < width; ++x) {
+            bool maskedOut = false;
+            if (maskChannel >= 0 && maskChannel < setChannels) {
+                uint16_t& m = a[at(x, y, maskChannel)];
+                float const v = half_to_float(m);
+                m = float_to_half_rne(v > 0.f ? std::min(v, 1.f) : 0.f);
+                maskedOut = discardMaskedOut && half_to_float(b[at(x, y, maskChannel)]) == 0.f;
+            }
+            for (int c = 0; c < setChannels; ++c) {
+                if (!((validChannelMask >> c) & 1u) || (maskedOut && c != maskChannel)) continue;
+                double const d = double(half_to_float(a[at(x, y, c)])) - double(half_to_float(b[at(x, y, c)]));
+                outMse[c] += d * d;
+            }
         }
     for (int c = 0; c < 16; ++c) outMse[c] /= double(width) * double(height);
 }

@@ -123,7 +123,7 @@ EXPORTS = [
                                                C.c_int32, C.POINTER(C.c_float)]),
     ("ntc_hip_read_channels", C.c_int, [C.POINTER(ReadChannels)]),
     ("ntc_hip_write_channels", C.c_int, [C.POINTER(WriteChannels)]),
-    ("ntc_hip_image_loss", C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64, C.c_int32, C.c_int32, C.c_int32, C.c_uint32,
+    ("ntc_hip_image_loss", C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64, C.c_int32, C.c_int32, C.c_int32, C.c_uint32, C.c_int32, C.c_int32,
                                      C.POINTER(C.c_float)]),
     ("ntc_hip_selftest_mfma", C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
     ("ntc_hip_selftest_mfma_f16", C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32]),

@@ -249,12 +249,16 @@ hipError_t launch_write_channels(WriteChannelsArgs const& a, hipStream_t stream)
 }
 
 // Per-channel sum of squared differences between a decoded mip and its reference image, both in the
-// internal layout: the loss branch of InferenceKernel (src/Inference.cu:77-118) without its masking
-// options.  Each workgroup covers 64 x 16 texels and writes 16 double partial sums (channel-major, so
-// that the second stage reads them coalesced); ReduceLoss likewise finishes in double (src/Optimizer.cu:382-387).
+// internal layout: the loss branch of InferenceKernel (src/Inference.cu:77-118) as a pass of its own.
+// With maskChannel >= 0 the decoded mask channel is first clamped to [0, 1] and stored back clamped
+// (Inference.cu:96-97,112; a negative zero becomes +0 as the device max() of the reference returns),
+// and with discardMaskedOut set a texel whose REFERENCE mask value is zero counts on the mask channel
+// only (Inference.cu:80-84,107-108).  Each workgroup covers 64 x 16 texels and writes 16 double partial
+// sums (channel-major, so that the second stage reads them coalesced); ReduceLoss likewise finishes in
+// double (src/Optimizer.cu:382-387).
 __global__ void __launch_bounds__(256)
-image_loss_kernel(uint16_t const* __restrict__ a, uint16_t const* __restrict__ b, int width, int height, int setChannels,
-                  uint32_t validChannelMask, double* __restrict__ partials)
+image_loss_kernel(uint16_t* __restrict__ a, uint16_t const* __restrict__ b, int width, int height, int setChannels,
+                  uint32_t validChannelMask, int maskChannel, int discardMaskedOut, double* __restrict__ partials)
 {
     __shared__ double sums[4][NTC_HIP_DEV_MAX_CHANNELS];
     int const lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -266,13 +270,30 @@ image_loss_kernel(uint16_t const* __restrict__ a, uint16_t const* __restrict__ b
         int const y = blockIdx.y * 16 + wave * 4 + r;
         if (x < width && y < height) {
             size_t const base = size_t(y) * size_t(width) * size_t(setChannels) + size_t(x) * 2;
+            bool maskedOut = false;
+            if (maskChannel >= 0 && discardMaskedOut) {
+                uint16_t const m = b[base + size_t(maskChannel & ~1) * size_t(width) + size_t(maskChannel & 1)];
+                maskedOut = (m & 0x7FFFu) == 0;
+            }
 #pragma unroll
             for (int p = 0; p < NTC_HIP_DEV_MAX_CHANNELS / 2; ++p) {
                 if (2 * p < setChannels) {
-                    uint32_t const va = *reinterpret_cast<uint32_t const*>(a + base + size_t(2 * p) * size_t(width));
+                    uint32_t* const pa = reinterpret_cast<uint32_t*>(a + base + size_t(2 * p) * size_t(width));
+                    uint32_t const va = *pa;
                     uint32_t const vb = *reinterpret_cast<uint32_t const*>(b + base + size_t(2 * p) * size_t(width));
-                    float const d0 = float(__builtin_bit_cast(_Float16, uint16_t(va))) - float(__builtin_bit_cast(_Float16, uint16_t(vb)));
-                    float const d1 = float(__builtin_bit_cast(_Float16, uint16_t(va >> 16))) - float(__builtin_bit_cast(_Float16, uint16_t(vb >> 16)));
+                    float a0 = float(__builtin_bit_cast(_Float16, uint16_t(va)));
+                    float a1 = float(__builtin_bit_cast(_Float16, uint16_t(va >> 16)));
+                    if ((maskChannel >> 1) == p) {      // never true for a negative maskChannel
+                        if (maskChannel & 1) a1 = a1 > 0.f ? fminf(a1, 1.f) : 0.f;
+                        else                 a0 = a0 > 0.f ? fminf(a0, 1.f) : 0.f;
+                        uint32_t const clamped = uint32_t(__builtin_bit_cast(uint16_t, _Float16(a0)))
+                                               | uint32_t(__builtin_bit_cast(uint16_t, _Float16(a1))) << 16;
+                        if (clamped != va) *pa = clamped;
+                    }
+                    float d0 = a0 - float(__builtin_bit_cast(_Float16, uint16_t(vb)));
+                    float d1 = a1 - float(__builtin_bit_cast(_Float16, uint16_t(vb >> 16)));
+                    if (maskedOut && maskChannel != 2 * p) d0 = 0.f;
+                    if (maskedOut && maskChannel != 2 * p + 1) d1 = 0.f;
                     acc[2 * p] += d0 * d0;
                     acc[2 * p + 1] += d1 * d1;
                 }
@@ -313,12 +334,13 @@ image_loss_reduce_kernel(double const* __restrict__ partials, size_t blocks, dou
     }
 }
 
-hipError_t launch_image_loss(uint16_t const* a, uint16_t const* b, int width, int height, int setChannels,
-                             uint32_t validChannelMask, double* partials, hipStream_t stream)
+hipError_t launch_image_loss(uint16_t* a, uint16_t const* b, int width, int height, int setChannels,
+                             uint32_t validChannelMask, int maskChannel, int discardMaskedOut, double* partials, hipStream_t stream)
 {
     dim3 const grid((width + 63) / 64, (height + 15) / 16);
     size_t const blocks = size_t(grid.x) * size_t(grid.y);
-    hipLaunchKernelGGL(image_loss_kernel, grid, dim3(256), 0, stream, a, b, width, height, setChannels, validChannelMask, partials);
+    hipLaunchKernelGGL(image_loss_kernel, grid, dim3(256), 0, stream, a, b, width, height, setChannels, validChannelMask,
+                       maskChannel, discardMaskedOut, partials);
     hipLaunchKernelGGL(image_loss_reduce_kernel, dim3(NTC_HIP_DEV_MAX_CHANNELS), dim3(256), 0, stream, partials, blocks, partials + blocks * NTC_HIP_DEV_MAX_CHANNELS);
     return hipGetLastError();
 }

@@ -80,8 +80,8 @@ hipError_t launch_write_channels(WriteChannelsArgs const& args, hipStream_t stre
 
 // Workgroups (= partial-sum rows of 16 doubles) the loss kernel uses for an image.
 inline size_t image_loss_blocks(int width, int height) { return size_t((width + 63) / 64) * size_t((height + 15) / 16); }
-hipError_t launch_image_loss(uint16_t const* a, uint16_t const* b, int width, int height, int setChannels,
-                             uint32_t validChannelMask, double* partials, hipStream_t stream);
+hipError_t launch_image_loss(uint16_t* a, uint16_t const* b, int width, int height, int setChannels,
+                             uint32_t validChannelMask, int maskChannel, int discardMaskedOut, double* partials, hipStream_t stream);
 
 hipError_t launch_decode(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream);
 hipError_t launch_queries(int variant, DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries,

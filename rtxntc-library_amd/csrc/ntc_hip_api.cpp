@@ -629,8 +629,9 @@ int ntc_hip_write_channels(const NtcHipWriteChannels* p)
     return 0;
 }
 
-int ntc_hip_image_loss(const void* decoded, const void* reference, uint64_t planarBytes, int32_t width, int32_t height,
-                       int32_t setChannels, uint32_t validChannelMask, float* outMse)
+int ntc_hip_image_loss(void* decoded, const void* reference, uint64_t planarBytes, int32_t width, int32_t height,
+                       int32_t setChannels, uint32_t validChannelMask, int32_t maskChannelIndex, int32_t discardMaskedOutPixels,
+                       float* outMse)
 {
     if (int r = require_init()) return r;
     if (!decoded || !reference || !outMse) { set_error("ntc_hip_image_loss: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
@@ -638,6 +639,18 @@ int ntc_hip_image_loss(const void* decoded, const void* reference, uint64_t plan
         || uint64_t(width) * uint64_t(height) * uint64_t(setChannels) * 2u > planarBytes) {
         set_error("ntc_hip_image_loss: bad image shape or buffer size.");
         return NTC_HIP_ERR_INVALID_ARG;
+    }
+    if (maskChannelIndex >= setChannels) {      // src/TextureSet.cpp:1899-1902; negative = no mask channel
+        set_error("ntc_hip_image_loss: maskChannelIndex (%d) must be below the channel count (%d).", maskChannelIndex, setChannels);
+        return NTC_HIP_ERR_INVALID_ARG;
+    }
+    if (maskChannelIndex >= 0) {                // the decoded image is then written while the reference is read
+        uintptr_t const d = reinterpret_cast<uintptr_t>(decoded), r = reinterpret_cast<uintptr_t>(reference);
+        uint64_t const imageBytes = uint64_t(width) * uint64_t(height) * uint64_t(setChannels) * 2u;
+        if (d < r + imageBytes && r < d + imageBytes) {
+            set_error("ntc_hip_image_loss: with a mask channel the decoded and the reference image must not overlap.");
+            return NTC_HIP_ERR_INVALID_ARG;
+        }
     }
     size_t const blocks = image_loss_blocks(width, height);
     size_t const bytes = (blocks + 1) * NTC_HIP_DEV_MAX_CHANNELS * sizeof(double);    // partial sums, then the 16 totals
@@ -650,8 +663,9 @@ int ntc_hip_image_loss(const void* decoded, const void* reference, uint64_t plan
         if (!L.lossHost) HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&L.lossHost), NTC_HIP_DEV_MAX_CHANNELS * sizeof(double), hipHostMallocDefault));
         L.lossBytes = bytes;
     }
-    HIP_TRY(launch_image_loss(static_cast<uint16_t const*>(decoded), static_cast<uint16_t const*>(reference), width, height,
-                              setChannels, validChannelMask, L.lossDev, L.stream));
+    HIP_TRY(launch_image_loss(static_cast<uint16_t*>(decoded), static_cast<uint16_t const*>(reference), width, height,
+                              setChannels, validChannelMask, maskChannelIndex < 0 ? -1 : maskChannelIndex,
+                              discardMaskedOutPixels ? 1 : 0, L.lossDev, L.stream));
     HIP_TRY(hipMemcpyAsync(L.lossHost, L.lossDev + blocks * NTC_HIP_DEV_MAX_CHANNELS, NTC_HIP_DEV_MAX_CHANNELS * sizeof(double),
                            hipMemcpyDeviceToHost, L.stream));
     HIP_TRY(hipStreamSynchronize(L.stream));

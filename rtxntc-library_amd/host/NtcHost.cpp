@@ -363,6 +363,16 @@ public:
     ITextureMetadata* GetTexture(int index) override { return (index >= 0 && index < int(m_textures.size())) ? m_textures[size_t(index)] : nullptr; }
 
     // src/TextureSetMetadata.cpp:807-832 (no output shuffling here)
+    // src/TextureSet.cpp:1899-1907
+    Status SetMaskChannelIndex(int index, bool discardMaskedOutPixels) override
+    {
+        if (index >= m_desc.channels) { SetErrorMessage("Mask channel index (%d) must be below the channel count (%d).", index, m_desc.channels); return Status::OutOfRange; }
+        m_maskChannelIndex = index;
+        m_discardMaskedOutPixels = discardMaskedOutPixels;
+        ClearErrorMessage();
+        return Status::Ok;
+    }
+
     uint32_t GetValidChannelMask() const override
     {
         uint32_t mask = 0;
@@ -595,7 +605,10 @@ public:
 
         // Losses need the reference image to survive the decode: decode into a second page.
         uint32_t const validMask = GetValidChannelMask();
-        bool const lazyOutPage = validMask != 0 && pOutStats && !m_textureDataOut;
+        // The loss branch runs whenever the valid mask is non-zero (src/Inference.cu:77); here it is a pass
+        // of its own, needed for the statistics or for the clamp of the mask channel.
+        bool const lossPass = validMask != 0 && (pOutStats || m_maskChannelIndex >= 0);
+        bool const lazyOutPage = lossPass && !m_textureDataOut;
         if (lazyOutPage)
             if (int r = ntc_hip_alloc(&m_textureDataOut, m_textureBytes)) return AllocationFailure(r, "texture data (output)", m_textureBytes);
         void* const outPage = m_textureDataOut ? m_textureDataOut : m_textureData;   // src/TextureSet.cpp:1799-1802
@@ -624,7 +637,7 @@ public:
 
         // Per-channel / per-mip / overall mean squared error, weighted by pixel count exactly as
         // src/TextureSet.cpp:1833-1863,1884-1892 combine them.
-        if (validMask != 0 && pOutStats) {
+        if (lossPass) {
             int validChannels = 0;
             for (int ch = 0; ch < m_desc.channels; ++ch) if (validMask & (1u << ch)) ++validChannels;
             double perChannel[16] = {};
@@ -632,9 +645,11 @@ public:
             for (int mip = 0; mip < m_desc.mips; ++mip) {
                 uint64_t const offset = m_mipOffsets[mip] * uint64_t(m_desc.channels) * 2u;
                 float mse[16];
-                if (int r = ntc_hip_image_loss(static_cast<uint8_t const*>(outPage) + offset, static_cast<uint8_t const*>(m_textureData) + offset,
-                                               m_textureBytes - offset, m_mips[mip].width, m_mips[mip].height, m_desc.channels, validMask, mse))
+                if (int r = ntc_hip_image_loss(static_cast<uint8_t*>(outPage) + offset, static_cast<uint8_t const*>(m_textureData) + offset,
+                                               m_textureBytes - offset, m_mips[mip].width, m_mips[mip].height, m_desc.channels, validMask,
+                                               m_maskChannelIndex < 0 ? -1 : m_maskChannelIndex, m_discardMaskedOutPixels ? 1 : 0, mse))
                     return DeviceFailure(r);
+                if (!pOutStats) continue;
                 double const mipPixels = double(m_mips[mip].width) * double(m_mips[mip].height);
                 double mean = 0.0;
                 for (int ch = 0; ch < m_desc.channels; ++ch) {
@@ -647,8 +662,10 @@ public:
                 overall += mipPixels * mean;
                 pixels += mipPixels;
             }
-            pOutStats->overallLoss = float(overall / pixels);
-            for (int ch = 0; ch < 16; ++ch) pOutStats->perChannelLoss[ch] = float(perChannel[ch] / pixels);
+            if (pOutStats) {
+                pOutStats->overallLoss = float(overall / pixels);
+                for (int ch = 0; ch < 16; ++ch) pOutStats->perChannelLoss[ch] = float(perChannel[ch] / pixels);
+            }
         }
         // Without separateRefOutData both pages are one memory in the reference and the decode
         // overwrites the reference image; keep that: the decoded page becomes the only page.
@@ -1000,6 +1017,8 @@ private:
     void* m_staging = nullptr;
     void* m_latents = nullptr;
     void* m_weights = nullptr;
+    int m_maskChannelIndex = -1;
+    bool m_discardMaskedOutPixels = false;
     bool m_deviceAvailable = false, m_haveLatents = false, m_haveWeights = false, m_decompressed = false;
 };
 

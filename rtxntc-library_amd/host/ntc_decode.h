@@ -220,6 +220,13 @@ public:
     // include/libntc/ntc.h:902, src/TextureSet.cpp:915-985.
     virtual Status ReadChannels(ReadChannelsParameters const& params) = 0;
 
+    // Index of the channel that holds an alpha mask; negative = none (include/libntc/ntc.h:936-940,
+    // src/TextureSet.cpp:1899-1907).  Decompress then clamps the decoded mask channel to [0, 1] when
+    // it compares against a reference (valid channel mask != 0), and with discardMaskedOutPixels texels
+    // whose reference mask is zero count in the loss of the mask channel only.  OutOfRange for an
+    // index at or beyond the channel count.
+    virtual Status SetMaskChannelIndex(int index, bool discardMaskedOutPixels) = 0;
+
     // Union of the channel ranges of the registered textures (include/libntc/ntc.h:638-640,
     // src/TextureSetMetadata.cpp:807-832).
     virtual uint32_t GetValidChannelMask() const = 0;

@@ -6,6 +6,7 @@
 //       loads raw latents/weights, decompresses, reads every mip back as UNORM8 (host address
 //       space) and FLOAT16 (device address space is exercised through a second read), writes files
 //   host_api_test loss <preset> <w> <h> <mips> <channels> <gridScale> <features> <latents> <weights> <refPrefix> <separate 0|1>
+//                      [<maskChannel> <discardMaskedOut 0|1> <withStats 0|1>]
 //       registers two textures (channels 0..2 and 4..5), writes <refPrefix>_mip<N>.bin (FLOAT32 pixels,
 //       all channels) as the reference image, decompresses twice and prints the loss statistics
 //   host_api_test load <file> <device 0|1> [<w> <h> <channels> <mips>]
@@ -245,6 +246,9 @@ static int loss(int argc, char** argv)
     std::vector<unsigned char> latents = readFile(argv[9]), weights = readFile(argv[10]);
     std::string const prefix = argv[11];
     bool const separate = std::atoi(argv[12]) != 0;
+    int const maskChannel = argc >= 16 ? std::atoi(argv[13]) : -1;
+    bool const discard = argc >= 16 && std::atoi(argv[14]) != 0;
+    bool const withStats = argc < 16 || std::atoi(argv[15]) != 0;
 
     IContext* ctx = nullptr;
     ContextParameters params;
@@ -262,6 +266,8 @@ static int loss(int argc, char** argv)
     ITextureMetadata* a = set->AddTexture(); CHECK(a->SetChannels(0, 3) == Status::Ok);
     ITextureMetadata* b = set->AddTexture(); CHECK(b->SetChannels(4, 2) == Status::Ok);
     CHECK(set->GetValidChannelMask() == 0x37u);
+    CHECK(set->SetMaskChannelIndex(set->GetDesc().channels, false) == Status::OutOfRange);
+    CHECK(set->SetMaskChannelIndex(maskChannel, discard) == Status::Ok);
     int const C = set->GetDesc().channels;
     for (int mip = 0; mip < mips; ++mip) {
         int const mw = std::max(w >> mip, 1), mh = std::max(h >> mip, 1);
@@ -280,10 +286,10 @@ static int loss(int argc, char** argv)
         for (int c = 0; c < 16; ++c) std::printf(" %.9g", st.perChannelLoss[c]);
         std::printf("\n");
     };
-    DecompressionStats first, second;
-    CHECK(set->Decompress(&first) == Status::Ok);
+    DecompressionStats first{}, second{};
+    CHECK(set->Decompress(withStats ? &first : nullptr) == Status::Ok);
     printStats("first", first);
-    CHECK(set->Decompress(&second) == Status::Ok);
+    CHECK(set->Decompress(withStats ? &second : nullptr) == Status::Ok);
     printStats("second", second);
     // Reference page after the decode: the written image when the pages are separate, the
     // decoded image when they share memory (src/TextureSet.cpp:103-124).

@@ -226,6 +226,81 @@ def test_checker_image_loss_against_numpy(oracle):
         assert all(got[c] == 0 for c in range(16) if not mask >> c & 1)
 
 
+def np_image_loss_masked(a, b, width, height, set_channels, mask, mask_channel, discard):
+    """numpy statement of the loss branch with its mask options (src/Inference.cu:80-84,96-97,107-112).
+    Returns (mse[16], the decoded image with its mask channel clamped)."""
+    fa = a.view(np.float16).astype(np.float64).reshape(height, set_channels // 2, width, 2).copy()
+    fb = b.view(np.float16).astype(np.float64).reshape(height, set_channels // 2, width, 2)
+    masked_out = np.zeros((height, width), dtype=bool)
+    if mask_channel >= 0:
+        plane = fa[:, mask_channel // 2, :, mask_channel % 2]
+        fa[:, mask_channel // 2, :, mask_channel % 2] = np.clip(plane, 0.0, 1.0) + 0.0    # + 0.0: -0 -> +0
+        if discard:
+            masked_out = fb[:, mask_channel // 2, :, mask_channel % 2] == 0
+    out = np.zeros(16)
+    for c in range(set_channels):
+        if mask >> c & 1:
+            d = fa[:, c // 2, :, c % 2] - fb[:, c // 2, :, c % 2]
+            if c != mask_channel:
+                d = np.where(masked_out, 0.0, d)
+            out[c] = np.mean(d ** 2)
+    return out, fa.astype(np.float16).view(np.uint16).reshape(-1)
+
+
+def masked_loss_images(rng, w, h, C_, mask_channel):
+    """A decoded image whose mask channel leaves [0, 1] (and holds -0), and a reference whose mask
+    channel is zero (+0 or -0) on about a third of the texels."""
+    a = (rng.random(w * h * C_) * 1.5 - 0.25).astype(np.float16).view(np.uint16).copy()
+    b = rng.random(w * h * C_).astype(np.float16).view(np.uint16).copy()
+    av = a.reshape(h, C_ // 2, w, 2)
+    bv = b.reshape(h, C_ // 2, w, 2)
+    pick = rng.random((h, w))
+    bv[:, mask_channel // 2, :, mask_channel % 2][pick < 0.2] = 0x0000
+    bv[:, mask_channel // 2, :, mask_channel % 2][(pick >= 0.2) & (pick < 0.33)] = 0x8000
+    av[:, mask_channel // 2, :, mask_channel % 2][rng.random((h, w)) < 0.1] = 0x8000
+    return a, b
+
+
+def test_checker_masked_image_loss(oracle):
+    rng = np.random.default_rng(51)
+    w, h, C_ = 45, 17, 8
+    for mask_channel in (3, 6):
+        a, b = masked_loss_images(rng, w, h, C_, mask_channel)
+        for discard in (0, 1):
+            for mask in (0xFF, 0x0F, 1 << mask_channel):
+                got, work = np.zeros(16), a.copy()
+                oracle.ntc_oracle_image_loss_masked(work.ctypes.data, b.ctypes.data, w, h, C_, mask, mask_channel, discard, got.ctypes.data)
+                want, clamped = np_image_loss_masked(a, b, w, h, C_, mask, mask_channel, discard)
+                assert np.allclose(got, want, rtol=1e-12, atol=0)
+                assert np.array_equal(work, clamped)
+                assert not np.array_equal(work, a)
+                # clamping is idempotent and changes the mask channel only
+                again, work2 = np.zeros(16), work.copy()
+                oracle.ntc_oracle_image_loss_masked(work2.ctypes.data, b.ctypes.data, w, h, C_, mask, mask_channel, discard, again.ctypes.data)
+                assert np.array_equal(work2, work) and np.array_equal(again, got)
+                other = np.ones(C_, dtype=bool); other[mask_channel] = False
+                assert np.array_equal(work.reshape(h, C_ // 2, w, 2).transpose(0, 2, 1, 3).reshape(h, w, C_)[:, :, other],
+                                      a.reshape(h, C_ // 2, w, 2).transpose(0, 2, 1, 3).reshape(h, w, C_)[:, :, other])
+    # special cases: no mask channel = the plain loss; a reference mask without zeros = discard has no
+    # effect; a reference mask of zeros = only the mask channel counts
+    a, b = masked_loss_images(rng, w, h, C_, 2)
+    plain, got = np.zeros(16), np.zeros(16)
+    oracle.ntc_oracle_image_loss(a.ctypes.data, b.ctypes.data, w, h, C_, 0xFF, plain.ctypes.data)
+    work = a.copy()
+    oracle.ntc_oracle_image_loss_masked(work.ctypes.data, b.ctypes.data, w, h, C_, 0xFF, -1, 1, got.ctypes.data)
+    assert np.array_equal(got, plain) and np.array_equal(work, a)
+    bv = b.reshape(h, C_ // 2, w, 2)
+    bv[:, 1, :, 0] = np.float16(0.5).view(np.uint16)
+    keep, drop = np.zeros(16), np.zeros(16)
+    work = a.copy()
+    oracle.ntc_oracle_image_loss_masked(work.ctypes.data, b.ctypes.data, w, h, C_, 0xFF, 2, 0, keep.ctypes.data)
+    oracle.ntc_oracle_image_loss_masked(work.ctypes.data, b.ctypes.data, w, h, C_, 0xFF, 2, 1, drop.ctypes.data)
+    assert np.array_equal(keep, drop)
+    bv[:, 1, :, 0] = 0
+    oracle.ntc_oracle_image_loss_masked(work.ctypes.data, b.ctypes.data, w, h, C_, 0xFF, 2, 1, drop.ctypes.data)
+    assert drop[2] > 0 and not np.delete(drop, 2).any()
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("fmt", [1, 2, 3, 4, 5])
 def test_gpu_write_channels_all_formats(ntc, device, oracle, fmt):
@@ -259,12 +334,35 @@ def test_gpu_image_loss_against_checker(ntc, device, oracle, shape):
     d_a, d_b = device.upload(a), device.upload(b)
     for mask in ((1 << C_) - 1, 0x5 & ((1 << C_) - 1), 0):
         got = (C.c_float * 16)()
-        ntc.abi.check(device.lib.ntc_hip_image_loss(d_a.ptr, d_b.ptr, d_a.nbytes, w, h, C_, mask, got))
+        ntc.abi.check(device.lib.ntc_hip_image_loss(d_a.ptr, d_b.ptr, d_a.nbytes, w, h, C_, mask, -1, 0, got))
         want = np.zeros(16, dtype=np.float64)
         oracle.ntc_oracle_image_loss(a.ctypes.data, b.ctypes.data, w, h, C_, mask, want.ctypes.data)
         # double accumulation on both sides; the result is rounded to float once
         assert np.allclose(np.array(got[:], dtype=np.float64), want, rtol=2e-7, atol=0), (shape, mask)
-    assert device.lib.ntc_hip_image_loss(d_a.ptr, d_b.ptr, d_a.nbytes - 2, w, h, C_, 1, got) == ntc.abi.ERR_INVALID_ARG
+    assert np.array_equal(d_a.download().view(np.uint16), a)        # without a mask channel the decoded image is only read
+    assert device.lib.ntc_hip_image_loss(d_a.ptr, d_b.ptr, d_a.nbytes - 2, w, h, C_, 1, -1, 0, got) == ntc.abi.ERR_INVALID_ARG
+    assert device.lib.ntc_hip_image_loss(d_a.ptr, d_b.ptr, d_a.nbytes, w, h, C_, 1, C_, 0, got) == ntc.abi.ERR_INVALID_ARG
+    assert device.lib.ntc_hip_image_loss(d_a.ptr, d_a.ptr, d_a.nbytes, w, h, C_, 1, 0, 0, got) == ntc.abi.ERR_INVALID_ARG   # overlap
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(1, 1, 2), (67, 5, 6), (515, 300, 16)])
+def test_gpu_masked_image_loss_against_checker(ntc, device, oracle, shape):
+    """Alpha-mask options of the loss branch: the decoded mask channel is clamped in place (bit-exact
+    against the checker), masked-out texels count on the mask channel only."""
+    w, h, C_ = shape
+    rng = np.random.default_rng(w + 1)
+    for mask_channel in sorted({0, C_ - 1, C_ // 2}):
+        a, b = masked_loss_images(rng, w, h, C_, mask_channel)
+        for discard in (0, 1):
+            mask = (1 << C_) - 1
+            d_a, d_b = device.upload(a), device.upload(b)
+            got = (C.c_float * 16)()
+            ntc.abi.check(device.lib.ntc_hip_image_loss(d_a.ptr, d_b.ptr, d_a.nbytes, w, h, C_, mask, mask_channel, discard, got))
+            want, work = np.zeros(16), a.copy()
+            oracle.ntc_oracle_image_loss_masked(work.ctypes.data, b.ctypes.data, w, h, C_, mask, mask_channel, discard, want.ctypes.data)
+            assert np.array_equal(d_a.download().view(np.uint16), work), (shape, mask_channel, discard)
+            assert np.allclose(np.array(got[:], dtype=np.float64), want, rtol=2e-7, atol=0), (shape, mask_channel, discard)
 
 
 def parse_stats(text, tag, mips):
@@ -321,6 +419,50 @@ def test_host_layer_loss_statistics(ntc, oracle, tmp_path, separate):
     page_out = np.fromfile(prefix + "_page_output.bin", dtype=np.uint16)
     assert np.array_equal(page_out, pixels_of(decoded0))
     assert np.array_equal(page_ref, pixels_of(ref0 if separate else decoded0))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("with_stats", [1, 0])
+def test_host_layer_mask_channel(ntc, oracle, tmp_path, with_stats):
+    """SetMaskChannelIndex (include/libntc/ntc.h:936-940): Decompress clamps the decoded mask channel to
+    [0, 1] whenever textures are registered, and with discardMaskedOutPixels the loss of the other
+    channels skips texels whose reference mask is zero (src/Inference.cu:80-112)."""
+    w, h, channels, mask_channel = 96, 40, 8, 5
+    mips = ntc.presets.full_mip_count(w, h)
+    case = cfg_case(ntc, ntc.presets.spec_cfg01(), w, h, mips, channels, ntc.abi.OUT_FP16_PLANAR_PAIRS, 93, scale_log2_range=(-17.0, -12.0))
+    lat, wts = tmp_path / "latents.bin", tmp_path / "weights.bin"
+    case.latents.tofile(lat)
+    case.weights.tofile(wts)
+    host = case.host_set()
+    host.decode(threads=8)
+    rng = np.random.default_rng(94)
+    prefix = str(tmp_path / "ref")
+    mask = 0x37
+    valid = [c for c in range(channels) if mask >> c & 1]
+    mse = np.zeros((mips, 16))
+    pixels = np.array([m.width * m.height for m in case.mips], dtype=np.float64)
+    clamped0 = decoded0 = None
+    for m, mip in enumerate(case.mips):
+        decoded = np.ascontiguousarray(host.output[mip.outOffset: mip.outOffset + mip.width * mip.height * channels * 2].view(np.uint16))
+        ref = rng.random((mip.height, mip.width, channels)).astype(np.float32)
+        ref[:, :, mask_channel][rng.random((mip.height, mip.width)) < 0.3] = 0.0
+        ref.tofile(f"{prefix}_mip{m}.bin")
+        ref_planar = np.zeros(mip.width * mip.height * channels, dtype=np.uint16)
+        np_write_channels(ref_planar, ref, channels, 0, False)
+        mse[m], clamped = np_image_loss_masked(decoded, ref_planar, mip.width, mip.height, channels, mask, mask_channel, True)
+        if m == 0:
+            decoded0, clamped0 = decoded, clamped
+    assert not np.array_equal(decoded0, clamped0)       # the decoded mask channel does leave [0, 1]
+    out = run_exe("loss", 1, w, h, mips, channels, 0, 0, lat, wts, prefix, 1, mask_channel, 1, with_stats)
+    assert "host loss OK" in out
+    page_out = np.fromfile(prefix + "_page_output.bin", dtype=np.uint16)
+    assert np.array_equal(page_out, clamped0.reshape(h, channels // 2, w, 2).transpose(0, 2, 1, 3).reshape(-1))
+    if with_stats:
+        overall, per_mip, per_channel = parse_stats(out, "first", mips)
+        want_mip = mse[:, valid].mean(axis=1)
+        assert np.allclose(per_mip, want_mip, rtol=1e-6)
+        assert np.allclose(per_channel, (mse * pixels[:, None]).sum(axis=0) / pixels.sum(), rtol=1e-6)
+        assert np.isclose(overall, (want_mip * pixels).sum() / pixels.sum(), rtol=1e-6)
 
 
 # ---- colour spaces and dithering in ReadChannels / WriteChannels -----------------------------------
