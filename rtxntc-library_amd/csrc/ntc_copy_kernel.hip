@@ -73,11 +73,24 @@ struct DitherRng {
     }
 };
 
-constexpr int kRowsPerGroup = 4;       // image rows one workgroup of the copy kernels covers (more rows per workgroup measured slower)
-
 constexpr int bytes_per_channel(int format)
 {
     return format == NTC_HIP_DEV_FORMAT_UNORM8 ? 1 : (format == NTC_HIP_DEV_FORMAT_UNORM16 || format == NTC_HIP_DEV_FORMAT_FLOAT16) ? 2 : 4;
+}
+
+// Lane -> pixel of the copy kernels: a workgroup covers 256 pixels of one row, or 64 pixels of four
+// rows for images narrower than 256 (xShift = 8 or 6, chosen on the host).
+struct CopyGrid {
+    int x, y;
+    __device__ explicit CopyGrid(int xShift)
+        : x((int(blockIdx.x) << xShift) + (int(threadIdx.x) & ((1 << xShift) - 1))),
+          y(int(blockIdx.y) * (256 >> xShift) + (int(threadIdx.x) >> xShift)) {}
+};
+inline dim3 copy_grid(int width, int height, int& xShift, bool wide = true)
+{
+    xShift = (wide && width >= 256) ? 8 : 6;
+    int const rows = 256 >> xShift;
+    return dim3((width + (1 << xShift) - 1) >> xShift, (height + rows - 1) / rows);
 }
 
 // WriteImageChannel (src/ImageProcessing.cu:141-164): the channel's bits in the destination format.
@@ -102,25 +115,40 @@ __device__ __forceinline__ uint32_t encode_channel(int colorSpace, float value, 
     }
 }
 
-// One lane per pixel.  The pixel is produced 16 bytes at a time (16 / 8 / 4 channels for 1 / 2 / 4-byte
-// formats) and stored with the widest access the image's alignment allows (a.vectorBytes, decided
-// on the host from base, pitch and stride); source halves come in as the dword pairs of the
-// planar-pair layout, coalesced across the lanes of a row.
-template <int FORMAT>
+// One lane per pixel.  All the half2 pairs the pixel needs are loaded before any arithmetic (the
+// loads of a lane overlap; issued one by one behind their uses the kernel ran at half the rate),
+// coalesced across the lanes of a row.  The pixel is produced 16 bytes at a time (16 / 8 / 4
+// channels for 1 / 2 / 4-byte formats) and stored with the widest access the image's alignment allows
+// (a.vectorBytes, decided on the host from base, pitch and stride).  PLAIN = every colour space
+// linear and no dithering: the transfer functions and the generator are compiled out.
+template <int FORMAT, bool PLAIN>
 __global__ void __launch_bounds__(256)
 read_channels_kernel(ReadChannelsArgs a)
 {
     constexpr int BPC = bytes_per_channel(FORMAT), PER = 16 / BPC;
-    int const x = blockIdx.x * 64 + (threadIdx.x & 63);
-    if (x >= a.width) return;
-    for (int y = blockIdx.y * kRowsPerGroup + (threadIdx.x >> 6); y < min(a.height, int(blockIdx.y + 1) * kRowsPerGroup); y += 4) {
+    CopyGrid const at(a.xShift);
+    int const x = at.x, y = at.y;
+    if (x >= a.width || y >= a.height) return;
     // GetPixelBaseAddress / GetChannelAddress, src/RegressionKernels.h:36-45
     uint16_t const* src = a.planarPairs + size_t(y) * size_t(a.width) * size_t(a.setChannels) + size_t(x) * 2;
     uint8_t* px = a.dst + size_t(y) * a.rowPitch + size_t(x) * a.pixelStride;
-    DitherRng rng(uint32_t(x) + uint32_t(y) * uint32_t(a.width));
-    int loadedPair = -1;
-    uint32_t pairBits = 0;
-    for (int base = 0; base < a.dstChannels; base += PER) {
+    int const firstPair = a.firstChannel >> 1;
+    bool const odd = (a.firstChannel & 1) != 0;
+    int const pairs = ((a.firstChannel + a.numChannels + 1) >> 1) - firstPair;     // at most 8
+    uint32_t pr[NTC_HIP_DEV_MAX_CHANNELS / 2];
+#pragma unroll
+    for (int p = 0; p < NTC_HIP_DEV_MAX_CHANNELS / 2; ++p) {
+        pr[p] = 0u;
+        if (p < pairs) pr[p] = *reinterpret_cast<uint32_t const*>(src + size_t(2 * (firstPair + p)) * size_t(a.width));     // uniform
+    }
+    auto half_of = [&](int k) -> uint32_t {                  // half k of the loaded pairs, k a compile-time constant after unrolling
+        return k < NTC_HIP_DEV_MAX_CHANNELS ? ((k & 1) ? pr[(k >> 1) & 7] >> 16 : pr[(k >> 1) & 7] & 0xffffu) : 0u;
+    };
+    [[maybe_unused]] DitherRng rng(uint32_t(x) + uint32_t(y) * uint32_t(a.width));
+#pragma unroll
+    for (int piece = 0; piece < NTC_HIP_DEV_MAX_CHANNELS / PER; ++piece) {
+        int const base = piece * PER;
+        if (base >= a.dstChannels) break;                    // uniform
         uint32_t words[4] = { 0u, 0u, 0u, 0u };
 #pragma unroll
         for (int k = 0; k < PER; ++k) {
@@ -128,18 +156,19 @@ read_channels_kernel(ReadChannelsArgs a)
             if (ch >= a.dstChannels) continue;               // uniform
             float value;
             if (ch < a.numChannels) {
-                int const c = a.firstChannel + ch;
-                if ((c >> 1) != loadedPair) {
-                    loadedPair = c >> 1;
-                    pairBits = *reinterpret_cast<uint32_t const*>(src + size_t(c & ~1) * size_t(a.width));
-                }
-                uint16_t const bits = uint16_t((c & 1) ? pairBits >> 16 : pairBits);
-                value = decode_color_space(a.srcColorSpaces[ch], float(__builtin_bit_cast(_Float16, bits)));
+                uint32_t const bits = odd ? half_of(ch + 1) : half_of(ch);
+                value = float(__builtin_bit_cast(_Float16, uint16_t(bits)));
+                if constexpr (!PLAIN) value = decode_color_space(a.srcColorSpaces[ch], value);
             } else {
                 value = (ch == 3) ? 1.f : 0.f;               // GetDefaultChannelValue, src/ImageProcessing.cu:166-170
             }
-            float const dither = a.useDithering ? rng.next_float() - 0.5f : 0.f;      // one draw per destination channel
-            uint32_t const bits = encode_channel<FORMAT>(ch < 16 ? a.dstColorSpaces[ch] : 0, value, a.useDithering != 0, dither);
+            uint32_t bits;
+            if constexpr (PLAIN) {
+                bits = encode_channel<FORMAT>(0, value, false, 0.f);
+            } else {
+                float const dither = a.useDithering ? rng.next_float() - 0.5f : 0.f;  // one draw per destination channel
+                bits = encode_channel<FORMAT>(a.dstColorSpaces[ch], value, a.useDithering != 0, dither);
+            }
             words[(k * BPC) >> 2] |= bits << (8 * ((k * BPC) & 3));
         }
         int const bytes = min(PER, a.dstChannels - base) * BPC;
@@ -157,7 +186,6 @@ read_channels_kernel(ReadChannelsArgs a)
         } else {
             for (int q = 0; q < bytes / 4; ++q) reinterpret_cast<uint32_t*>(out)[q] = words[q];
         }
-    }
     }
 }
 
@@ -177,8 +205,8 @@ __device__ __forceinline__ float decode_channel(uint32_t const (&words)[4], int 
 // User image -> internal fp16 planar pairs: ITextureSet::WriteChannels through CopyImageKernel's 1:1
 // branch (src/TextureSet.cpp:835-913, src/ImageProcessing.cu:220-265), optional vertical flip.
 // The pixel is read 16 bytes at a time with the widest loads its alignment allows; channel pairs
-// that fall on a half2 of the internal layout are written as one dword.
-template <int FORMAT>
+// that fall on a half2 of the internal layout are written as one dword.  PLAIN as above.
+template <int FORMAT, bool PLAIN>
 __global__ void __launch_bounds__(256)
 write_channels_kernel(WriteChannelsArgs a)
 {
@@ -188,14 +216,17 @@ write_channels_kernel(WriteChannelsArgs a)
         unorm8Table[threadIdx.x & 255] = float(threadIdx.x & 255) / 255.f;
         __syncthreads();
     }
-    int const x = blockIdx.x * 64 + (threadIdx.x & 63);
-    if (x >= a.width) return;
-    for (int y = blockIdx.y * kRowsPerGroup + (threadIdx.x >> 6); y < min(a.height, int(blockIdx.y + 1) * kRowsPerGroup); y += 4) {
+    CopyGrid const at(a.xShift);
+    int const x = at.x, y = at.y;
+    if (x >= a.width || y >= a.height) return;
     int const srcY = a.verticalFlip ? a.height - 1 - y : y;          // SetupBilinearFilter flips the read position
     uint8_t const* px = a.src + size_t(srcY) * a.rowPitch + size_t(x) * a.pixelStride;
     uint16_t* dst = a.planarPairs + size_t(y) * size_t(a.width) * size_t(a.setChannels) + size_t(x) * 2;
     uint32_t pending = 0;                                            // low half of a pair waiting for its partner
-    for (int base = 0; base < a.numChannels; base += PER) {
+#pragma unroll
+    for (int piece = 0; piece < NTC_HIP_DEV_MAX_CHANNELS / PER; ++piece) {
+        int const base = piece * PER;
+        if (base >= a.numChannels) break;                            // uniform
         int const bytes = min(PER, a.numChannels - base) * BPC;
         uint8_t const* const in = px + base * BPC;
         uint32_t words[4] = { 0u, 0u, 0u, 0u };
@@ -215,34 +246,49 @@ write_channels_kernel(WriteChannelsArgs a)
         for (int k = 0; k < PER; ++k) {
             int const ch = base + k;
             if (ch >= a.numChannels) continue;                       // uniform
-            float v = decode_color_space(a.srcColorSpaces[ch], decode_channel<FORMAT>(words, k, unorm8Table));
-            v = encode_color_space(a.dstColorSpaces[ch], v);
+            float v = decode_channel<FORMAT>(words, k, unorm8Table);
+            if constexpr (!PLAIN) v = encode_color_space(a.dstColorSpaces[ch], decode_color_space(a.srcColorSpaces[ch], v));
             v = fmaxf(-65504.f, fminf(65504.f, v));                  // WriteImageChannel FLOAT16, src/ImageProcessing.cu:154-156
             asm volatile("" : "+v"(v));
             uint32_t const half = __builtin_bit_cast(uint16_t, (_Float16)v);
             int const c = a.firstChannel + ch;
-            uint16_t* const at = dst + size_t(c & ~1) * size_t(a.width);
+            uint16_t* const to = dst + size_t(c & ~1) * size_t(a.width);
             if ((c & 1) == 0) {
                 if (ch + 1 < a.numChannels) pending = half;          // partner follows: store both together
-                else at[0] = uint16_t(half);
+                else to[0] = uint16_t(half);
             } else {
-                if (ch > 0) *reinterpret_cast<uint32_t*>(at) = pending | (half << 16);
-                else at[1] = uint16_t(half);
+                if (ch > 0) *reinterpret_cast<uint32_t*>(to) = pending | (half << 16);
+                else to[1] = uint16_t(half);
             }
         }
     }
-    }
 }
 
-hipError_t launch_write_channels(WriteChannelsArgs const& a, hipStream_t stream)
+static bool plain_copy(uint8_t const* srcSpaces, uint8_t const* dstSpaces, int useDithering)
 {
-    dim3 const grid((a.width + 63) / 64, (a.height + kRowsPerGroup - 1) / kRowsPerGroup);
+    bool plain = useDithering == 0;
+    for (int i = 0; i < 16; ++i) plain = plain && srcSpaces[i] == 0 && dstSpaces[i] == 0;
+    return plain;
+}
+
+template <int FORMAT>
+static void launch_write_format(WriteChannelsArgs const& a, dim3 grid, bool plain, hipStream_t stream)
+{
+    if (plain) hipLaunchKernelGGL((write_channels_kernel<FORMAT, true>), grid, dim3(256), 0, stream, a);
+    else       hipLaunchKernelGGL((write_channels_kernel<FORMAT, false>), grid, dim3(256), 0, stream, a);
+}
+
+hipError_t launch_write_channels(WriteChannelsArgs const& args, hipStream_t stream)
+{
+    WriteChannelsArgs a = args;
+    dim3 const grid = copy_grid(a.width, a.height, a.xShift, false);
+    bool const plain = plain_copy(a.srcColorSpaces, a.dstColorSpaces, 0);
     switch (a.format) {
-    case NTC_HIP_DEV_FORMAT_UNORM8:  hipLaunchKernelGGL(write_channels_kernel<NTC_HIP_DEV_FORMAT_UNORM8>, grid, dim3(256), 0, stream, a); break;
-    case NTC_HIP_DEV_FORMAT_UNORM16: hipLaunchKernelGGL(write_channels_kernel<NTC_HIP_DEV_FORMAT_UNORM16>, grid, dim3(256), 0, stream, a); break;
-    case NTC_HIP_DEV_FORMAT_FLOAT16: hipLaunchKernelGGL(write_channels_kernel<NTC_HIP_DEV_FORMAT_FLOAT16>, grid, dim3(256), 0, stream, a); break;
-    case NTC_HIP_DEV_FORMAT_FLOAT32: hipLaunchKernelGGL(write_channels_kernel<NTC_HIP_DEV_FORMAT_FLOAT32>, grid, dim3(256), 0, stream, a); break;
-    case NTC_HIP_DEV_FORMAT_UINT32:  hipLaunchKernelGGL(write_channels_kernel<NTC_HIP_DEV_FORMAT_UINT32>, grid, dim3(256), 0, stream, a); break;
+    case NTC_HIP_DEV_FORMAT_UNORM8:  launch_write_format<NTC_HIP_DEV_FORMAT_UNORM8>(a, grid, plain, stream); break;
+    case NTC_HIP_DEV_FORMAT_UNORM16: launch_write_format<NTC_HIP_DEV_FORMAT_UNORM16>(a, grid, plain, stream); break;
+    case NTC_HIP_DEV_FORMAT_FLOAT16: launch_write_format<NTC_HIP_DEV_FORMAT_FLOAT16>(a, grid, plain, stream); break;
+    case NTC_HIP_DEV_FORMAT_FLOAT32: launch_write_format<NTC_HIP_DEV_FORMAT_FLOAT32>(a, grid, plain, stream); break;
+    case NTC_HIP_DEV_FORMAT_UINT32:  launch_write_format<NTC_HIP_DEV_FORMAT_UINT32>(a, grid, plain, stream); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
@@ -250,59 +296,90 @@ hipError_t launch_write_channels(WriteChannelsArgs const& a, hipStream_t stream)
 
 // Per-channel sum of squared differences between a decoded mip and its reference image, both in the
 // internal layout: the loss branch of InferenceKernel (src/Inference.cu:77-118) as a pass of its own.
-// With maskChannel >= 0 the decoded mask channel is first clamped to [0, 1] and stored back clamped
-// (Inference.cu:96-97,112; a negative zero becomes +0 as the device max() of the reference returns),
-// and with discardMaskedOut set a texel whose REFERENCE mask value is zero counts on the mask channel
-// only (Inference.cu:80-84,107-108).  Each workgroup covers 64 x 16 texels and writes 16 double partial
-// sums (channel-major, so that the second stage reads them coalesced); ReduceLoss likewise finishes in
+// MASKED (maskChannel >= 0): the decoded mask channel is first clamped to [0, 1] and stored back
+// clamped (Inference.cu:96-97,112; a negative zero becomes +0 as the device max() of the reference
+// returns), and with discardMaskedOut a texel whose REFERENCE mask value is zero counts on the mask
+// channel only (Inference.cu:80-84,107-108).
+// A lane takes PX adjacent texels (2 when the width is even: 8-byte loads) of kLossRowsPerWave rows; all
+// loads of a row are issued before its arithmetic.  Squares are fp32 as in the reference; their sum over the
+// lane's texels of a row goes into a double accumulator, and the workgroup writes 16 double partial sums
+// (channel-major, so that the second stage reads them coalesced); ReduceLoss likewise finishes in
 // double (src/Optimizer.cu:382-387).
+template <int PX, bool MASKED>
 __global__ void __launch_bounds__(256)
 image_loss_kernel(uint16_t* __restrict__ a, uint16_t const* __restrict__ b, int width, int height, int setChannels,
                   uint32_t validChannelMask, int maskChannel, int discardMaskedOut, double* __restrict__ partials)
 {
+    constexpr int PAIRS = NTC_HIP_DEV_MAX_CHANNELS / 2;
     __shared__ double sums[4][NTC_HIP_DEV_MAX_CHANNELS];
     int const lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    int const x = blockIdx.x * 64 + lane;
-    float acc[NTC_HIP_DEV_MAX_CHANNELS];
+    int const x = (blockIdx.x * 64 + lane) * PX;
+    int const pairs = setChannels >> 1;
+    double acc[NTC_HIP_DEV_MAX_CHANNELS];
 #pragma unroll
-    for (int c = 0; c < NTC_HIP_DEV_MAX_CHANNELS; ++c) acc[c] = 0.f;
-    for (int r = 0; r < 4; ++r) {
-        int const y = blockIdx.y * 16 + wave * 4 + r;
-        if (x < width && y < height) {
-            size_t const base = size_t(y) * size_t(width) * size_t(setChannels) + size_t(x) * 2;
-            bool maskedOut = false;
-            if (maskChannel >= 0 && discardMaskedOut) {
-                uint16_t const m = b[base + size_t(maskChannel & ~1) * size_t(width) + size_t(maskChannel & 1)];
-                maskedOut = (m & 0x7FFFu) == 0;
+    for (int c = 0; c < NTC_HIP_DEV_MAX_CHANNELS; ++c) acc[c] = 0.0;
+    for (int r = 0; r < kLossRowsPerWave; ++r) {
+        int const y = (blockIdx.y * 4 + wave) * kLossRowsPerWave + r;
+        if (x >= width || y >= height) continue;             // width is a multiple of PX
+        size_t const base = size_t(y) * size_t(width) * size_t(setChannels) + size_t(x) * 2;
+        uint32_t va[PAIRS][PX], vb[PAIRS][PX];
+#pragma unroll
+        for (int p = 0; p < PAIRS; ++p) {
+            // no branch around a load (the loads of a row must all be in flight together): pairs the
+            // set does not have re-read its last pair, and their sums are dropped at the end
+            size_t const at = base + size_t(2 * min(p, pairs - 1)) * size_t(width);
+            if constexpr (PX == 2) {
+                uint2 const u = *reinterpret_cast<uint2 const*>(a + at), v = *reinterpret_cast<uint2 const*>(b + at);
+                va[p][0] = u.x; va[p][1] = u.y; vb[p][0] = v.x; vb[p][1] = v.y;
+            } else {
+                va[p][0] = *reinterpret_cast<uint32_t const*>(a + at);
+                vb[p][0] = *reinterpret_cast<uint32_t const*>(b + at);
             }
+        }
+        __builtin_amdgcn_sched_barrier(0);                   // keep the loads ahead of the arithmetic
+        [[maybe_unused]] bool maskedOut[PX];
+        if constexpr (MASKED) {
 #pragma unroll
-            for (int p = 0; p < NTC_HIP_DEV_MAX_CHANNELS / 2; ++p) {
-                if (2 * p < setChannels) {
-                    uint32_t* const pa = reinterpret_cast<uint32_t*>(a + base + size_t(2 * p) * size_t(width));
-                    uint32_t const va = *pa;
-                    uint32_t const vb = *reinterpret_cast<uint32_t const*>(b + base + size_t(2 * p) * size_t(width));
-                    float a0 = float(__builtin_bit_cast(_Float16, uint16_t(va)));
-                    float a1 = float(__builtin_bit_cast(_Float16, uint16_t(va >> 16)));
-                    if ((maskChannel >> 1) == p) {      // never true for a negative maskChannel
+            for (int k = 0; k < PX; ++k) maskedOut[k] = false;
+#pragma unroll
+            for (int p = 0; p < PAIRS; ++p) {
+                if ((maskChannel >> 1) != p || !discardMaskedOut) continue;          // uniform
+#pragma unroll
+                for (int k = 0; k < PX; ++k) maskedOut[k] = (((maskChannel & 1) ? vb[p][k] >> 16 : vb[p][k]) & 0x7FFFu) == 0;
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < PAIRS; ++p) {
+            float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+            for (int k = 0; k < PX; ++k) {
+                float a0 = float(__builtin_bit_cast(_Float16, uint16_t(va[p][k])));
+                float a1 = float(__builtin_bit_cast(_Float16, uint16_t(va[p][k] >> 16)));
+                if constexpr (MASKED) {
+                    if ((maskChannel >> 1) == p) {              // uniform; the mask channel is below setChannels
                         if (maskChannel & 1) a1 = a1 > 0.f ? fminf(a1, 1.f) : 0.f;
                         else                 a0 = a0 > 0.f ? fminf(a0, 1.f) : 0.f;
                         uint32_t const clamped = uint32_t(__builtin_bit_cast(uint16_t, _Float16(a0)))
                                                | uint32_t(__builtin_bit_cast(uint16_t, _Float16(a1))) << 16;
-                        if (clamped != va) *pa = clamped;
+                        if (clamped != va[p][k]) *reinterpret_cast<uint32_t*>(a + base + size_t(2 * p) * size_t(width) + size_t(2 * k)) = clamped;
                     }
-                    float d0 = a0 - float(__builtin_bit_cast(_Float16, uint16_t(vb)));
-                    float d1 = a1 - float(__builtin_bit_cast(_Float16, uint16_t(vb >> 16)));
-                    if (maskedOut && maskChannel != 2 * p) d0 = 0.f;
-                    if (maskedOut && maskChannel != 2 * p + 1) d1 = 0.f;
-                    acc[2 * p] += d0 * d0;
-                    acc[2 * p + 1] += d1 * d1;
                 }
+                float d0 = a0 - float(__builtin_bit_cast(_Float16, uint16_t(vb[p][k])));
+                float d1 = a1 - float(__builtin_bit_cast(_Float16, uint16_t(vb[p][k] >> 16)));
+                if constexpr (MASKED) {
+                    if (maskedOut[k] && maskChannel != 2 * p) d0 = 0.f;
+                    if (maskedOut[k] && maskChannel != 2 * p + 1) d1 = 0.f;
+                }
+                s0 += d0 * d0;
+                s1 += d1 * d1;
             }
+            acc[2 * p] += double(s0);
+            acc[2 * p + 1] += double(s1);
         }
     }
 #pragma unroll
     for (int c = 0; c < NTC_HIP_DEV_MAX_CHANNELS; ++c) {
-        double v = ((validChannelMask >> c) & 1u) ? double(acc[c]) : 0.0;
+        double v = (c < setChannels && ((validChannelMask >> c) & 1u)) ? acc[c] : 0.0;
 #pragma unroll
         for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
         if (lane == 0) sums[wave][c] = v;
@@ -316,44 +393,65 @@ image_loss_kernel(uint16_t* __restrict__ a, uint16_t const* __restrict__ b, int 
 }
 
 // Second stage: workgroup c adds the partial sums of channel c, in double and in a fixed order
-// (thread t takes entries t, t + 256, ...; then one thread adds the 256 sub-totals), and writes the
-// total behind the partials.
+// (thread t takes entries t, t + 256, ... into four interleaved sub-totals; then one thread adds the
+// 256 thread totals), and writes the total behind the partials.
 __global__ void __launch_bounds__(256)
 image_loss_reduce_kernel(double const* __restrict__ partials, size_t blocks, double* __restrict__ totals)
 {
     __shared__ double sums[256];
-    int const c = blockIdx.x;
-    double acc = 0.0;
-    for (size_t b = threadIdx.x; b < blocks; b += 256) acc += partials[size_t(c) * blocks + b];
-    sums[threadIdx.x] = acc;
+    double const* const mine = partials + size_t(blockIdx.x) * blocks;
+    double acc[4] = { 0.0, 0.0, 0.0, 0.0 };
+    size_t b = threadIdx.x;
+    for (; b + 768 < blocks; b += 1024) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) acc[k] += mine[b + size_t(k) * 256];
+    }
+#pragma unroll
+    for (int k = 0; k < 3; ++k)
+        if (b + size_t(k) * 256 < blocks) acc[k] += mine[b + size_t(k) * 256];
+    sums[threadIdx.x] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
     __syncthreads();
     if (threadIdx.x == 0) {
         double total = 0.0;
         for (int t = 0; t < 256; ++t) total += sums[t];
-        totals[c] = total;
+        totals[blockIdx.x] = total;
     }
 }
 
 hipError_t launch_image_loss(uint16_t* a, uint16_t const* b, int width, int height, int setChannels,
                              uint32_t validChannelMask, int maskChannel, int discardMaskedOut, double* partials, hipStream_t stream)
 {
-    dim3 const grid((width + 63) / 64, (height + 15) / 16);
+    dim3 const grid = image_loss_grid(width, height);
     size_t const blocks = size_t(grid.x) * size_t(grid.y);
-    hipLaunchKernelGGL(image_loss_kernel, grid, dim3(256), 0, stream, a, b, width, height, setChannels, validChannelMask,
-                       maskChannel, discardMaskedOut, partials);
+    bool const two = (width & 1) == 0, masked = maskChannel >= 0;
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, a, b, width, height, setChannels, validChannelMask,
+                           maskChannel, discardMaskedOut, partials);
+    };
+    if (two) { if (masked) launch(image_loss_kernel<2, true>); else launch(image_loss_kernel<2, false>); }
+    else     { if (masked) launch(image_loss_kernel<1, true>); else launch(image_loss_kernel<1, false>); }
     hipLaunchKernelGGL(image_loss_reduce_kernel, dim3(NTC_HIP_DEV_MAX_CHANNELS), dim3(256), 0, stream, partials, blocks, partials + blocks * NTC_HIP_DEV_MAX_CHANNELS);
     return hipGetLastError();
 }
 
-hipError_t launch_read_channels(ReadChannelsArgs const& a, hipStream_t stream)
+template <int FORMAT>
+static void launch_read_format(ReadChannelsArgs const& a, dim3 grid, bool plain, hipStream_t stream)
 {
-    dim3 const grid((a.width + 63) / 64, (a.height + kRowsPerGroup - 1) / kRowsPerGroup);
+    if (plain) hipLaunchKernelGGL((read_channels_kernel<FORMAT, true>), grid, dim3(256), 0, stream, a);
+    else       hipLaunchKernelGGL((read_channels_kernel<FORMAT, false>), grid, dim3(256), 0, stream, a);
+}
+
+hipError_t launch_read_channels(ReadChannelsArgs const& args, hipStream_t stream)
+{
+    ReadChannelsArgs a = args;
+    dim3 const grid = copy_grid(a.width, a.height, a.xShift);
+    bool const plain = plain_copy(a.srcColorSpaces, a.dstColorSpaces, a.useDithering);
     switch (a.format) {
-    case NTC_HIP_DEV_FORMAT_UNORM8:  hipLaunchKernelGGL(read_channels_kernel<NTC_HIP_DEV_FORMAT_UNORM8>, grid, dim3(256), 0, stream, a); break;
-    case NTC_HIP_DEV_FORMAT_UNORM16: hipLaunchKernelGGL(read_channels_kernel<NTC_HIP_DEV_FORMAT_UNORM16>, grid, dim3(256), 0, stream, a); break;
-    case NTC_HIP_DEV_FORMAT_FLOAT16: hipLaunchKernelGGL(read_channels_kernel<NTC_HIP_DEV_FORMAT_FLOAT16>, grid, dim3(256), 0, stream, a); break;
-    case NTC_HIP_DEV_FORMAT_FLOAT32: hipLaunchKernelGGL(read_channels_kernel<NTC_HIP_DEV_FORMAT_FLOAT32>, grid, dim3(256), 0, stream, a); break;
-    case NTC_HIP_DEV_FORMAT_UINT32:  hipLaunchKernelGGL(read_channels_kernel<NTC_HIP_DEV_FORMAT_UINT32>, grid, dim3(256), 0, stream, a); break;
+    case NTC_HIP_DEV_FORMAT_UNORM8:  launch_read_format<NTC_HIP_DEV_FORMAT_UNORM8>(a, grid, plain, stream); break;
+    case NTC_HIP_DEV_FORMAT_UNORM16: launch_read_format<NTC_HIP_DEV_FORMAT_UNORM16>(a, grid, plain, stream); break;
+    case NTC_HIP_DEV_FORMAT_FLOAT16: launch_read_format<NTC_HIP_DEV_FORMAT_FLOAT16>(a, grid, plain, stream); break;
+    case NTC_HIP_DEV_FORMAT_FLOAT32: launch_read_format<NTC_HIP_DEV_FORMAT_FLOAT32>(a, grid, plain, stream); break;
+    case NTC_HIP_DEV_FORMAT_UINT32:  launch_read_format<NTC_HIP_DEV_FORMAT_UINT32>(a, grid, plain, stream); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

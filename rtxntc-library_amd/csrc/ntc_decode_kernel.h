@@ -62,6 +62,7 @@ struct ReadChannelsArgs {
     int32_t width, height, setChannels, firstChannel, numChannels, dstChannels, format;
     int32_t useDithering;
     int32_t vectorBytes;           // widest store every pixel start is aligned to: 16, 8, 4, 2 or 1
+    int32_t xShift;                // set by the launcher: log2 of the pixels of a row one workgroup covers
     uint8_t srcColorSpaces[16], dstColorSpaces[16];   // per copied channel: 0 linear, 1 sRGB, 2 HLG
 };
 hipError_t launch_read_channels(ReadChannelsArgs const& args, hipStream_t stream);
@@ -74,12 +75,24 @@ struct WriteChannelsArgs {
     uint64_t pixelStride, rowPitch;
     int32_t width, height, setChannels, firstChannel, numChannels, format, verticalFlip;
     int32_t vectorBytes;           // widest load every pixel start is aligned to
+    int32_t xShift;                // set by the launcher
     uint8_t srcColorSpaces[16], dstColorSpaces[16];
 };
 hipError_t launch_write_channels(WriteChannelsArgs const& args, hipStream_t stream);
 
-// Workgroups (= partial-sum rows of 16 doubles) the loss kernel uses for an image.
-inline size_t image_loss_blocks(int width, int height) { return size_t((width + 63) / 64) * size_t((height + 15) / 16); }
+// Grid of the loss kernel: a workgroup (= one row of 16 double partial sums) covers 64 lanes x 1 or 2
+// texels (2 when the width is even) by 4 waves x kLossRowsPerWave rows.
+constexpr int kLossRowsPerWave = 8;
+inline dim3 image_loss_grid(int width, int height)
+{
+    int const perLane = (width & 1) ? 1 : 2;
+    return dim3((width + 64 * perLane - 1) / (64 * perLane), (height + 4 * kLossRowsPerWave - 1) / (4 * kLossRowsPerWave));
+}
+inline size_t image_loss_blocks(int width, int height)
+{
+    dim3 const grid = image_loss_grid(width, height);
+    return size_t(grid.x) * size_t(grid.y);
+}
 hipError_t launch_image_loss(uint16_t* a, uint16_t const* b, int width, int height, int setChannels,
                              uint32_t validChannelMask, int maskChannel, int discardMaskedOut, double* partials, hipStream_t stream);
 
