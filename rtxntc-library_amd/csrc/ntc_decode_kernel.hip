@@ -582,23 +582,7 @@ __device__ __forceinline__ void prepare_inputs_general(DevMip const& m, int x, i
 }
 
 // Input vector of one texel from integer arithmetic only (see axis_fast above).
-// The two horizontally adjacent cells (x0, y) and (x0 + 1, y) as one dword: low half = left cell.
-// Cells are 2 bytes, so the dword may sit on a 2-byte boundary; global memory takes such loads.
-// A footprint that wraps around the grid edge (x1 = 0) cannot be fetched this way -- the dword
-// would run past the row -- and takes two 16-bit loads instead.
-typedef uint32_t __attribute__((aligned(2))) u32_align2;
-__device__ __forceinline__ uint32_t load_cell_pair(GlobalU8Ptr base, uint32_t off0, uint32_t off1)
-{
-    if (off1 == off0 + 2u)
-        return *reinterpret_cast<__attribute__((address_space(1))) u32_align2 const*>(base + off0);
-    return load_u16(base, off0) | (load_u16(base, off1) << 16);
-}
-
-// PAIR_LOADS: fetch horizontally adjacent taps with one load (load_cell_pair).  Halves the number
-// of memory instructions, at a few extra vector operations per tap: pays where the loads are
-// scattered (random-access queries), not in the raster decode, which is bound by vector issue.
-// `Mip` is DevMip or any struct with the same members for the fields used here (QueryMip).
-template <class V, bool PAIR_LOADS = false, class Mip = DevMip>
+template <class V, class Mip = DevMip>
 __device__ __forceinline__ void prepare_inputs_fast(Mip const& m, LdsT<V> const& lds, int x, int y, uint32_t (&in)[16])
 {
 #pragma unroll
@@ -614,23 +598,12 @@ __device__ __forceinline__ void prepare_inputs_fast(Mip const& m, LdsT<V> const&
         uint32_t const a00 = r0 + c0, a10 = r0 + c1, a01 = r1 + c0, a11 = r1 + c1;   // byte offsets
         if constexpr (V::HR_MODE == 1) {
             static_assert(V::HR_MODE != 1 || (V::HR_BITS == 2 && V::HR_F == 8 && V::HR_SLOTS == 8), "concat grids: 8 x 2-bit");
-            if constexpr (PAIR_LOADS) {
-                uint32_t const row[2] = { load_cell_pair(g, a00, a10), load_cell_pair(g, a01, a11) };
+            uint32_t const addr[4] = { a00, a10, a01, a11 };
 #pragma unroll
-                for (int r = 0; r < 2; ++r) {
-                    in[4 * r]     = lds.lut2[row[r] & 0xffu];
-                    in[4 * r + 1] = lds.lut2[(row[r] >> 8) & 0xffu];
-                    in[4 * r + 2] = lds.lut2[(row[r] >> 16) & 0xffu];
-                    in[4 * r + 3] = lds.lut2[row[r] >> 24];
-                }
-            } else {
-                uint32_t const addr[4] = { a00, a10, a01, a11 };
-#pragma unroll
-                for (int tap = 0; tap < 4; ++tap) {
-                    uint32_t const w = load_u16(g, addr[tap]);
-                    in[2 * tap]     = lds.lut2[w & 0xffu];
-                    in[2 * tap + 1] = lds.lut2[w >> 8];
-                }
+            for (int tap = 0; tap < 4; ++tap) {
+                uint32_t const w = load_u16(g, addr[tap]);
+                in[2 * tap]     = lds.lut2[w & 0xffu];
+                in[2 * tap + 1] = lds.lut2[w >> 8];
             }
         } else {
             uint32_t const nx = (m.hrAxisX >> 8) & 0xffu, ny = (m.hrAxisY >> 8) & 0xffu;
@@ -640,14 +613,8 @@ __device__ __forceinline__ void prepare_inputs_fast(Mip const& m, LdsT<V> const&
 #pragma unroll
             for (int L = 0; L < layers; ++L) {
                 GlobalU8Ptr const gl = g + size_t(L) * layerStride;
-                uint32_t b;
-                if constexpr (PAIR_LOADS) {
-                    uint32_t const p0 = load_cell_pair(gl, a00, a10), p1 = load_cell_pair(gl, a01, a11);
-                    b = bilinear4_int(p0 & 0xffffu, p0 >> 16, p1 & 0xffffu, p1 >> 16, w00, w10, w01, w11, nx + ny);
-                } else {
-                    b = bilinear4_int(load_u16(gl, a00), load_u16(gl, a10), load_u16(gl, a01), load_u16(gl, a11),
-                                      w00, w10, w01, w11, nx + ny);
-                }
+                uint32_t b = bilinear4_int(load_u16(gl, a00), load_u16(gl, a10), load_u16(gl, a01), load_u16(gl, a11),
+                                           w00, w10, w01, w11, nx + ny);
                 if (4 * L + 4 > V::HR_F) b &= (1u << (8 * (V::HR_F - 4 * L))) - 1u;
                 in[L] = b;
             }
@@ -668,19 +635,119 @@ __device__ __forceinline__ void prepare_inputs_fast(Mip const& m, LdsT<V> const&
 #pragma unroll
         for (int L = 0; L < layers; ++L) {
             GlobalU8Ptr const gl = g + size_t(L) * layerStride;
-            uint32_t b;
-            if constexpr (PAIR_LOADS) {
-                uint32_t const p0 = load_cell_pair(gl, a00, a10), p1 = load_cell_pair(gl, a01, a11);
-                b = bilinear4_int(p0 & 0xffffu, p0 >> 16, p1 & 0xffffu, p1 >> 16, w00, w10, w01, w11, nx + ny);
-            } else {
-                b = bilinear4_int(load_u16(gl, a00), load_u16(gl, a10), load_u16(gl, a01), load_u16(gl, a11),
-                                  w00, w10, w01, w11, nx + ny);
-            }
+            uint32_t b = bilinear4_int(load_u16(gl, a00), load_u16(gl, a10), load_u16(gl, a01), load_u16(gl, a11),
+                                       w00, w10, w01, w11, nx + ny);
             if (4 * L + 4 > V::LR_F) b &= (1u << (8 * (V::LR_F - 4 * L))) - 1u;
             in[V::HR_INPUTS / 4 + L] = b;
         }
     }
     // ---- positional encoding from the per-mip phase tables
+    {
+        uint4 const ex = *reinterpret_cast<uint4 const*>(&lds.xtab[m.posMask + (uint32_t(x) & m.posMask)][0]);
+        uint4 const ey = *reinterpret_cast<uint4 const*>(&lds.ytab[m.posMask + (uint32_t(y) & m.posMask)][0]);
+        in[V::POS_BASE / 4 + 0] = ex.x | ey.x;
+        in[V::POS_BASE / 4 + 1] = ex.y | ey.y;
+        in[V::POS_BASE / 4 + 2] = ex.z | ey.z;
+        if constexpr (V::LOD == 2) {
+            uint32_t const l = uint32_t(int(m.positionLod * 127.5f)) & 0xffu;
+            in[V::POS_BASE / 4 + 3] = l | (l << 8);
+        }
+    }
+}
+
+// The same input vector for scattered sample points (random-access queries), where what costs is
+// the memory round trip of each gather, not vector issue.  Three steps:
+//   1. one dword load per pair of horizontally adjacent taps (cells are 2 bytes, so the dword may sit
+//      on a 2-byte boundary; global memory takes such loads) for every row and layer of both grids,
+//      all issued back to back.  A footprint that wraps around the grid edge, or a grid one cell wide,
+//      has no such dword: those lanes load from `safe` (any readable 4 bytes) instead, so that the
+//      step has no branch and every lane's loads are in flight together;
+//   2. the lanes without adjacent taps (few, except on the smallest mips) fetch their two cells with
+//      16-bit loads in one divergent region;
+//   3. arithmetic.
+// Issued behind their uses, with a branch per pair, the gathers of a lane ran one after the other:
+// about ten round trips per query instead of one.
+typedef uint32_t __attribute__((aligned(2))) u32_align2;
+typedef __attribute__((address_space(1))) u32_align2 const* GlobalU32A2Ptr;
+
+template <class V, class Mip>
+__device__ __forceinline__ void prepare_inputs_scattered(Mip const& m, LdsT<V> const& lds, int x, int y, GlobalU8Ptr safe,
+                                                         uint32_t (&in)[16])
+{
+    constexpr int HL = V::HR_MODE == 1 ? 1 : (V::HR_F + 3) / 4, LL = (V::LR_F + 3) / 4;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) in[i] = 0;
+
+    AxisFoot const hx = axis_fast(x, m.hrAxisX, m.hrWidth), hy = axis_fast(y, m.hrAxisY, m.hrHeight);
+    AxisFoot const lx = axis_fast(x, m.lrAxisX, m.lrWidth), ly = axis_fast(y, m.lrAxisY, m.lrHeight);
+    GlobalU8Ptr const gh = (GlobalU8Ptr)m.hr, gl = (GlobalU8Ptr)m.lr;
+    uint32_t const hlgw = ((m.hrAxisX >> 24) & 0xffu) + 1u, llgw = ((m.lrAxisX >> 24) & 0xffu) + 1u;
+    uint32_t const hStride = uint32_t(m.hrWidth) * uint32_t(m.hrHeight) * 2u, lStride = uint32_t(m.lrWidth) * uint32_t(m.lrHeight) * 2u;
+    uint32_t const hc0 = hx.c0 << 1, hc1 = hx.c1 << 1, lc0 = lx.c0 << 1, lc1 = lx.c1 << 1;
+    uint32_t const hrow[2] = { hy.c0 << hlgw, hy.c1 << hlgw }, lrow[2] = { ly.c0 << llgw, ly.c1 << llgw };
+    bool const hAdj = hc1 == hc0 + 2u, lAdj = lc1 == lc0 + 2u;
+
+    uint32_t hp[HL][2], lp[LL][2];                           // [layer][row]: left cell in the low half
+#pragma unroll
+    for (int L = 0; L < HL; ++L)
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+            hp[L][r] = *reinterpret_cast<GlobalU32A2Ptr>(hAdj ? gh + size_t(L) * hStride + (hrow[r] + hc0) : safe);
+#pragma unroll
+    for (int L = 0; L < LL; ++L)
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+            lp[L][r] = *reinterpret_cast<GlobalU32A2Ptr>(lAdj ? gl + size_t(L) * lStride + (lrow[r] + lc0) : safe);
+    __builtin_amdgcn_sched_barrier(0);
+    if (!(hAdj && lAdj)) {
+        if (!hAdj) {
+#pragma unroll
+            for (int L = 0; L < HL; ++L)
+#pragma unroll
+                for (int r = 0; r < 2; ++r)
+                    hp[L][r] = load_u16(gh + size_t(L) * hStride, hrow[r] + hc0) | (load_u16(gh + size_t(L) * hStride, hrow[r] + hc1) << 16);
+        }
+        if (!lAdj) {
+#pragma unroll
+            for (int L = 0; L < LL; ++L)
+#pragma unroll
+                for (int r = 0; r < 2; ++r)
+                    lp[L][r] = load_u16(gl + size_t(L) * lStride, lrow[r] + lc0) | (load_u16(gl + size_t(L) * lStride, lrow[r] + lc1) << 16);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    if constexpr (V::HR_MODE == 1) {
+        static_assert(V::HR_MODE != 1 || (V::HR_BITS == 2 && V::HR_F == 8 && V::HR_SLOTS == 8), "concat grids: 8 x 2-bit");
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            in[4 * r]     = lds.lut2[hp[0][r] & 0xffu];
+            in[4 * r + 1] = lds.lut2[(hp[0][r] >> 8) & 0xffu];
+            in[4 * r + 2] = lds.lut2[(hp[0][r] >> 16) & 0xffu];
+            in[4 * r + 3] = lds.lut2[hp[0][r] >> 24];
+        }
+    } else {
+        uint32_t const nx = (m.hrAxisX >> 8) & 0xffu, ny = (m.hrAxisY >> 8) & 0xffu;
+        uint32_t const wx1 = hx.f, wx0 = (1u << nx) - hx.f, wy1 = hy.f * 17u, wy0 = ((1u << ny) - hy.f) * 17u;
+        uint32_t const w00 = mul24(wx0, wy0), w10 = mul24(wx1, wy0), w01 = mul24(wx0, wy1), w11 = mul24(wx1, wy1);
+#pragma unroll
+        for (int L = 0; L < HL; ++L) {
+            uint32_t b = bilinear4_int(hp[L][0] & 0xffffu, hp[L][0] >> 16, hp[L][1] & 0xffffu, hp[L][1] >> 16, w00, w10, w01, w11, nx + ny);
+            if (4 * L + 4 > V::HR_F) b &= (1u << (8 * (V::HR_F - 4 * L))) - 1u;
+            in[L] = b;
+        }
+    }
+    {
+        uint32_t const nx = (m.lrAxisX >> 8) & 0xffu, ny = (m.lrAxisY >> 8) & 0xffu;
+        uint32_t const wx1 = lx.f, wx0 = (1u << nx) - lx.f, wy1 = ly.f * 17u, wy0 = ((1u << ny) - ly.f) * 17u;
+        uint32_t const w00 = mul24(wx0, wy0), w10 = mul24(wx1, wy0), w01 = mul24(wx0, wy1), w11 = mul24(wx1, wy1);
+#pragma unroll
+        for (int L = 0; L < LL; ++L) {
+            uint32_t b = bilinear4_int(lp[L][0] & 0xffffu, lp[L][0] >> 16, lp[L][1] & 0xffffu, lp[L][1] >> 16, w00, w10, w01, w11, nx + ny);
+            if (4 * L + 4 > V::LR_F) b &= (1u << (8 * (V::LR_F - 4 * L))) - 1u;
+            in[V::HR_INPUTS / 4 + L] = b;
+        }
+    }
     {
         uint4 const ex = *reinterpret_cast<uint4 const*>(&lds.xtab[m.posMask + (uint32_t(x) & m.posMask)][0]);
         uint4 const ey = *reinterpret_cast<uint4 const*>(&lds.ytab[m.posMask + (uint32_t(y) & m.posMask)][0]);
@@ -1078,7 +1145,7 @@ query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __res
         x = max(0, min(x, m.width - 1));
         y = max(0, min(y, m.height - 1));
         uint32_t in[16];
-        if (__all(m.fast != 0)) prepare_inputs_fast<V, true>(m, lds, x, y, in);   // every lane's mip is power-of-two sized
+        if (__all(m.fast != 0)) prepare_inputs_scattered<V>(m, lds, x, y, (GlobalU8Ptr)mips, in);   // every lane's mip is power-of-two sized
         else                    prepare_inputs_general<V>(mips[validMip ? query.mip : 0], x, y, in);
 
         // output-layer accumulators as floats: exact either way (|acc| < 2^24 on the fp16 path; the
