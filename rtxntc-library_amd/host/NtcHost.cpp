@@ -301,7 +301,7 @@ class TextureSet final : public ITextureSet
 {
 public:
     TextureSet(Context const* context, TextureSetDesc const& desc, TextureSetFeatures const& features)
-        : m_context(context), m_desc(desc), m_features(features) {}
+        : m_context(context), m_desc(desc), m_features(features) { ResetShuffle(); }
 
     ~TextureSet() override
     {
@@ -381,7 +381,90 @@ public:
             t->GetChannels(first, count);
             mask |= ((1u << count) - 1u) << first;
         }
-        return mask;
+        // textures name un-shuffled channels: carry the mask through the mapping
+        uint32_t shuffled = 0;
+        for (int ch = 0; ch < NTC_HIP_MAX_CHANNELS; ++ch) {
+            ShuffleSource const& src = m_shuffle[ch];
+            if ((src.type == ShuffleSourceType::Channel && (mask & (1u << src.channelIndex))) || src.type == ShuffleSourceType::Constant)
+                shuffled |= 1u << ch;
+        }
+        return shuffled;
+    }
+
+    InferenceWeightType GetBestSupportedWeightType() const override
+    {
+        return m_hostWeights.empty() ? InferenceWeightType::Unknown : InferenceWeightType::GenericInt8;
+    }
+
+    // src/TextureSetMetadata.cpp:245-286
+    Status GetInferenceWeights(InferenceWeightType weightType, void const** pOutData, size_t* pOutSize, size_t* pOutConvertedSize) override
+    {
+        if (weightType != InferenceWeightType::GenericInt8 || m_hostWeights.empty()) {
+            SetErrorMessage("No weights available for weightType = %s.", InferenceWeightTypeToString(weightType));
+            return Status::Unsupported;
+        }
+        if (pOutData) *pOutData = m_hostWeights.data();
+        if (pOutSize) *pOutSize = m_hostWeights.size();
+        if (pOutConvertedSize) *pOutConvertedSize = 0;
+        ClearErrorMessage();
+        return Status::Ok;
+    }
+
+    // src/TextureSetMetadata.cpp:305-432
+    Status ShuffleInferenceOutputs(ShuffleSource mapping[16]) override
+    {
+        if (!mapping) { SetErrorMessage("mapping is NULL"); return Status::InvalidArgument; }
+        for (int ch = 0; ch < NTC_HIP_MAX_CHANNELS; ++ch) {
+            int const type = int(mapping[ch].type);
+            if (type < int(ShuffleSourceType::Undefined) || type > int(ShuffleSourceType::Constant)) {
+                SetErrorMessage("mapping[%d] has invalid type %d", ch, type);
+                return Status::InvalidArgument;
+            }
+            if (mapping[ch].type == ShuffleSourceType::Channel && (mapping[ch].channelIndex < 0 || mapping[ch].channelIndex >= NTC_HIP_MAX_CHANNELS)) {
+                SetErrorMessage("mapping[%d] is using invalid channel %d, must be between 0 and %d", ch, mapping[ch].channelIndex, NTC_HIP_MAX_CHANNELS - 1);
+                return Status::OutOfRange;
+            }
+        }
+        if (!m_hostWeights.empty()) {
+            constexpr int last = NTC_HIP_MLP_LAYERS - 1, outputs = NTC_HIP_MAX_CHANNELS;
+            constexpr float constantUnit = 65536.f;          // constants are stored as bias = round(c * 2^16), scale = 2^-16
+            int const inputs = m_spec.hiddenChannels[last - 1];
+            uint8_t* const weights = m_hostWeights.data() + m_weightLayout.weightOffset[last];
+            uint8_t* const scales = m_hostWeights.data() + m_weightLayout.scaleOffset[last];
+            uint8_t* const biases = m_hostWeights.data() + m_weightLayout.biasOffset[last];
+            std::vector<uint8_t> newWeights(size_t(inputs) * outputs, 0);
+            float newScales[outputs];
+            int32_t newBiases[outputs];
+            for (int row = 0; row < outputs; ++row) {
+                ShuffleSource const& src = mapping[row];
+                if (src.type == ShuffleSourceType::Channel) {
+                    std::memcpy(newWeights.data() + size_t(row) * inputs, weights + size_t(src.channelIndex) * inputs, size_t(inputs));
+                    std::memcpy(&newScales[row], scales + 4 * src.channelIndex, 4);
+                    std::memcpy(&newBiases[row], biases + 4 * src.channelIndex, 4);
+                } else {
+                    newScales[row] = 1.f / constantUnit;
+                    newBiases[row] = src.type == ShuffleSourceType::Constant ? int32_t(roundf(src.constantValue * constantUnit)) : 0;
+                }
+            }
+            std::memcpy(weights, newWeights.data(), newWeights.size());
+            std::memcpy(scales, newScales, sizeof newScales);
+            std::memcpy(biases, newBiases, sizeof newBiases);
+        }
+        ColorSpace newSpaces[NTC_HIP_MAX_CHANNELS];
+        ShuffleSource newShuffle[NTC_HIP_MAX_CHANNELS];
+        for (int ch = 0; ch < NTC_HIP_MAX_CHANNELS; ++ch) {
+            if (mapping[ch].type == ShuffleSourceType::Channel) {
+                newSpaces[ch] = m_channelColorSpaces[mapping[ch].channelIndex];
+                newShuffle[ch] = m_shuffle[mapping[ch].channelIndex];
+            } else {
+                newSpaces[ch] = ColorSpace::Linear;
+                newShuffle[ch] = mapping[ch];
+            }
+        }
+        std::copy(newSpaces, newSpaces + NTC_HIP_MAX_CHANNELS, m_channelColorSpaces);
+        std::copy(newShuffle, newShuffle + NTC_HIP_MAX_CHANNELS, m_shuffle);
+        ClearErrorMessage();
+        return Status::Ok;
     }
 
     // src/TextureSet.cpp:718-745
@@ -592,7 +675,15 @@ public:
     uint64_t GetWeightDataSize() const override { return m_state == NetworkState::Empty ? 0 : m_weightLayout.bufferSize; }
 
     Status SetLatentData(void const* data, size_t size) override { return Upload(data, size, m_latentBytes, m_latents, "latent", m_haveLatents); }
-    Status SetWeightData(void const* data, size_t size) override { return Upload(data, size, m_weightLayout.bufferSize, m_weights, "weight", m_haveWeights); }
+    Status SetWeightData(void const* data, size_t size) override
+    {
+        Status const st = Upload(data, size, m_weightLayout.bufferSize, m_weights, "weight", m_haveWeights);
+        if (st == Status::Ok) {                              // the copy GetInferenceWeights hands out; a new blob starts un-shuffled
+            m_hostWeights.assign(static_cast<uint8_t const*>(data), static_cast<uint8_t const*>(data) + size);
+            ResetShuffle();
+        }
+        return st;
+    }
 
     Status Decompress(DecompressionStats* pOutStats, bool /*useInt8Weights*/) override
     {
@@ -915,6 +1006,7 @@ private:
     Status ResetShape()
     {
         ReleaseDevice(m_latents); ReleaseDevice(m_weights);
+        m_hostWeights.clear();
         m_latentBytes = 0; m_haveLatents = m_haveWeights = false;
         m_state = NetworkState::Empty;
         ClearErrorMessage();
@@ -933,6 +1025,7 @@ private:
         }
         if (ntc_hip_weight_layout(&m_spec, &m_weightLayout) != 0) { SetErrorMessage("%s", ntc_hip_last_error()); return Status::InternalError; }
         ReleaseDevice(m_latents); ReleaseDevice(m_weights);
+        m_hostWeights.clear();
         m_haveLatents = m_haveWeights = false;
         if (m_deviceAvailable) {
             if (int r = ntc_hip_alloc(&m_latents, m_latentBytes)) return AllocationFailure(r, "latent", m_latentBytes);
@@ -1017,6 +1110,9 @@ private:
     void* m_staging = nullptr;
     void* m_latents = nullptr;
     void* m_weights = nullptr;
+    std::vector<uint8_t> m_hostWeights;
+    ShuffleSource m_shuffle[NTC_HIP_MAX_CHANNELS];
+    void ResetShuffle() { for (int ch = 0; ch < NTC_HIP_MAX_CHANNELS; ++ch) m_shuffle[ch] = ShuffleSource::Channel(ch); }
     int m_maskChannelIndex = -1;
     bool m_discardMaskedOutPixels = false;
     bool m_deviceAvailable = false, m_haveLatents = false, m_haveWeights = false, m_decompressed = false;
@@ -1143,26 +1239,56 @@ void DestroyContext(IContext* context) { delete context; }
 
 char const* GetLastErrorMessage() { return t_message; }
 
+// Enum names as include/libntc/ntc.h spells them; a value outside the enum is printed as its number
+// into a static buffer, as the reference does (src/PublicFunctions.cpp:177-327).
+namespace
+{
+char const* NameOrNumber(char const* const* names, int count, int value)
+{
+    static char number[16];
+    if (value >= 0 && value < count) return names[value];
+    snprintf(number, sizeof number, "%d", value);
+    return number;
+}
+}
+
 char const* StatusToString(Status status)
 {
     static char const* const names[] = {
         "Ok", "InterfaceMismatch", "CudaError", "CudaUnavailable", "FileUnavailable", "FileUnrecognized",
         "FileIncompatible", "Incomplete", "Unsupported", "InternalError", "InvalidArgument", "InvalidData",
         "InvalidState", "IOError", "NotImplemented", "OutOfMemory", "OutOfRange", "ShaderUnavailable", "UnknownError" };
-    int const i = int(status);
-    return (i >= 0 && i < int(sizeof names / sizeof names[0])) ? names[i] : "Invalid";
+    return NameOrNumber(names, int(sizeof names / sizeof names[0]), int(status));
 }
 
 char const* ChannelFormatToString(ChannelFormat format)
 {
-    switch (format) {
-    case ChannelFormat::UNORM8: return "UNORM8";
-    case ChannelFormat::UNORM16: return "UNORM16";
-    case ChannelFormat::FLOAT16: return "FLOAT16";
-    case ChannelFormat::FLOAT32: return "FLOAT32";
-    case ChannelFormat::UINT32: return "UINT32";
-    default: return "UNKNOWN";
-    }
+    static char const* const names[] = { "UNKNOWN", "UNORM8", "UNORM16", "FLOAT16", "FLOAT32", "UINT32" };
+    return NameOrNumber(names, 6, int(format));
+}
+
+char const* BlockCompressedFormatToString(BlockCompressedFormat format)
+{
+    static char const* const names[] = { "None", "BC1", "BC2", "BC3", "BC4", "BC5", "BC6", "BC7" };
+    return NameOrNumber(names, 8, int(format));
+}
+
+char const* ColorSpaceToString(ColorSpace colorSpace)
+{
+    static char const* const names[] = { "Linear", "sRGB", "HLG" };
+    return NameOrNumber(names, 3, int(colorSpace));
+}
+
+char const* InferenceWeightTypeToString(InferenceWeightType weightType)
+{
+    static char const* const names[] = { "Unknown", "GenericInt8", "GenericFP8", "CoopVecFP8" };
+    return NameOrNumber(names, 4, int(weightType));
+}
+
+char const* CompressionTypeToString(CompressionType type)
+{
+    static char const* const names[] = { "None", "GDeflate" };
+    return NameOrNumber(names, 2, int(type));
 }
 
 // src/PublicFunctions.cpp:329-344
@@ -1181,6 +1307,152 @@ float LossToPSNR(float loss)
 {
     return (loss == 0.f) ? std::numeric_limits<float>::infinity() : -10.f * log10f(loss);
 }
+
+// src/PublicFunctions.cpp:36-45.  The version of the interface this library follows; branch and
+// commit describe this implementation.
+VersionInfo GetLibraryVersion()
+{
+    VersionInfo info;
+    info.major = 0; info.minor = 9; info.point = 2;
+    info.branch = "mi355x";
+    info.commitHash = "";
+    return info;
+}
+
+// src/PublicFunctions.cpp:354-380: latent grids of every neural LOD plus the Int8 network of the
+// 48-64-48-32-16 decoder (one byte per weight, fp32 scale and bias per output).
+Status EstimateCompressedTextureSetSize(TextureSetDesc const& textureSetDesc, LatentShape const& latentShape, size_t& outSize)
+{
+    if (Status st = ValidateTextureSetDesc(textureSetDesc); st != Status::Ok) return st;
+    if (Status st = ValidateLatentShape(latentShape); st != Status::Ok) return st;
+    if (latentShape.IsEmpty()) { SetErrorMessage("latentShape is empty."); return Status::OutOfRange; }
+    int const gs = latentShape.gridSizeScale;
+    int const neuralLods = NeuralLodCount(textureSetDesc.width, textureSetDesc.height, textureSetDesc.mips, gs);
+    size_t cells = 0;
+    for (int lod = 0; lod < neuralLods; ++lod)
+        cells += size_t(GridDimension(textureSetDesc.width, lod, gs)) * size_t(GridDimension(textureSetDesc.height, lod, gs));
+    size_t const layers = size_t((latentShape.numFeatures + 3) / 4);
+    size_t const weights = 48 * 64 + 64 * 48 + 48 * 32 + 32 * 16, outputs = 64 + 48 + 32 + 16;
+    outSize = cells * 2 * layers + weights + outputs * 2 * sizeof(float);
+    ClearErrorMessage();
+    return Status::Ok;
+}
+
+// The latent shapes the reference recommends per bit rate (src/PublicFunctions.cpp:382-393), sorted by rate.
+namespace
+{
+struct KnownLatentShape { float bitsPerPixel; LatentShape shape; };
+KnownLatentShape const kKnownLatentShapes[] = {
+    { 1.11f, { 6, 8 } }, { 1.67f, { 6, 12 } }, { 2.50f, { 4, 8 } }, { 3.75f, { 4, 12 } }, { 5.00f, { 4, 16 } },
+    { 6.67f, { 3, 12 } }, { 10.0f, { 2, 8 } }, { 15.0f, { 2, 12 } }, { 20.0f, { 2, 16 } } };
+constexpr int kKnownLatentShapeCount = int(sizeof kKnownLatentShapes / sizeof kKnownLatentShapes[0]);
+}
+
+int GetKnownLatentShapeCount() { return kKnownLatentShapeCount; }
+
+Status EnumerateKnownLatentShapes(int index, float& outBitsPerPixel, LatentShape& outShape)
+{
+    if (index < 0 || index >= kKnownLatentShapeCount) {
+        SetErrorMessage("Invalid index (%d), must be 0-%d.", index, kKnownLatentShapeCount - 1);
+        return Status::OutOfRange;
+    }
+    outBitsPerPixel = kKnownLatentShapes[index].bitsPerPixel;
+    outShape = kKnownLatentShapes[index].shape;
+    ClearErrorMessage();
+    return Status::Ok;
+}
+
+// The known shape nearest to the requested rate, if it lies within 25 % of the request
+// (src/PublicFunctions.cpp:415-452).
+Status PickLatentShape(float requestedBitsPerPixel, float& outBitsPerPixel, LatentShape& outShape)
+{
+    if (!(requestedBitsPerPixel > 0.f)) {
+        SetErrorMessage("requestedBitsPerPixel (%f) must be positive.", requestedBitsPerPixel);
+        return Status::OutOfRange;
+    }
+    int best = -1;
+    float bestDiff = std::numeric_limits<float>::max();
+    for (int i = 0; i < kKnownLatentShapeCount; ++i) {
+        float const diff = fabsf(kKnownLatentShapes[i].bitsPerPixel - requestedBitsPerPixel);
+        if (diff < requestedBitsPerPixel * 0.25f && diff < bestDiff) { best = i; bestDiff = diff; }
+    }
+    if (best < 0) {
+        SetErrorMessage("The provided requestedBitsPerPixel (%f) is out of the supported range.", requestedBitsPerPixel);
+        return Status::OutOfRange;
+    }
+    outBitsPerPixel = kKnownLatentShapes[best].bitsPerPixel;
+    outShape = kKnownLatentShapes[best].shape;
+    ClearErrorMessage();
+    return Status::Ok;
+}
+
+// src/PublicFunctions.cpp:454-461: two adjacent neural LODs are read together, so a latent cell of
+// `layers` x 2 bytes costs 16 bits x 1.25 per layer, spread over gridSizeScale^2 texels.
+float GetLatentShapeBitsPerPixel(LatentShape const& shape)
+{
+    int const layers = (shape.numFeatures + 3) / 4;
+    return float(layers) / float(shape.gridSizeScale * shape.gridSizeScale) * 2.f * 10.f;
+}
+
+// 16.48 fixed point -> double (src/PublicFunctions.cpp:463-467).
+double DecodeImageDifferenceResult(uint64_t value) { return double(value) * 0x1p-48; }
+
+// BC7 mode bitmap: 9 bits per block (3 bits mode, 6 bits partition), rounded up to whole dwords
+// (src/PublicFunctions.cpp:469-473, include/libntc/shaders/BlockCompressConstants.h:24-27).
+namespace { constexpr size_t kBc7ModeBits = 9; constexpr uint32_t kBc7Mode0Partition0 = 0x1BF; }
+
+size_t GetBC7ModeBufferSize(int widthInBlocks, int heightInBlocks)
+{
+    size_t const blocks = size_t(widthInBlocks) * size_t(heightInBlocks);
+    return ((blocks * kBc7ModeBits + 31) >> 5) << 2;
+}
+
+// src/PublicFunctions.cpp:475-557.  The mode of a BC7 block is the position of the lowest set bit of
+// its first byte (8 and above: the reserved mode, treated as 7); the partition index follows the mode
+// bit with 4, 6, 6, 6, 3 (rotation + index selector), 2, 0, 6 bits.  Entries are OR-ed into the
+// buffer, which the caller provides zeroed.
+Status MakeBC7ModeBuffer(int widthInBlocks, int heightInBlocks, void const* blockData, size_t blockDataSize,
+    size_t rowPitch, void* modeBuffer, size_t modeBufferSize)
+{
+    if (!blockData) { SetErrorMessage("blockData is NULL."); return Status::InvalidArgument; }
+    if (!modeBuffer) { SetErrorMessage("modeBuffer is NULL."); return Status::InvalidArgument; }
+    size_t const bytesPerBlock = 16, minPitch = size_t(widthInBlocks) * bytesPerBlock;
+    if (rowPitch < minPitch || rowPitch % bytesPerBlock != 0) {
+        SetErrorMessage("Invalid rowPitch (%zu), must be at least %zu and a multiple of %zu.", rowPitch, minPitch, bytesPerBlock);
+        return Status::InvalidArgument;
+    }
+    if (blockDataSize < size_t(heightInBlocks) * rowPitch) {
+        SetErrorMessage("Size of BC7 block data (%zu bytes) does not match the expected size (%zu bytes).",
+            blockDataSize, size_t(heightInBlocks) * rowPitch);
+        return Status::InvalidArgument;
+    }
+    size_t const needed = GetBC7ModeBufferSize(widthInBlocks, heightInBlocks);
+    if (modeBufferSize < needed) {
+        SetErrorMessage("Size of BC7 mode buffer (%zu bytes) is smaller than the expected size (%zu bytes).", modeBufferSize, needed);
+        return Status::InvalidArgument;
+    }
+    static uint32_t const partitionMask[8] = { 15, 63, 63, 63, 7, 3, 0, 63 };
+    uint8_t const* const blocks = static_cast<uint8_t const*>(blockData);
+    uint8_t* const bits = static_cast<uint8_t*>(modeBuffer);
+    for (int row = 0; row < heightInBlocks; ++row)
+        for (int col = 0; col < widthInBlocks; ++col) {
+            uint32_t first;
+            std::memcpy(&first, blocks + size_t(row) * rowPitch + size_t(col) * bytesPerBlock, 4);
+            uint32_t const mode = first ? std::min(7u, uint32_t(__builtin_ctz(first))) : 7u;
+            uint32_t const partition = (first >> (mode + 1)) & partitionMask[mode];
+            uint32_t entry = (mode << 6) | partition;
+            if (entry == 0) entry = kBc7Mode0Partition0;       // zero stays free to mean "not written"
+            size_t const bit = (size_t(row) * size_t(widthInBlocks) + size_t(col)) * kBc7ModeBits;
+            bits[bit / 8] |= uint8_t(entry << (bit & 7));
+            bits[bit / 8 + 1] |= uint8_t(entry >> (8 - (bit & 7)));
+        }
+    ClearErrorMessage();
+    return Status::Ok;
+}
+
+// GDeflate streams are not supported by this library (the reference's codec is an external
+// dependency that its tree does not contain): no header.
+size_t GetGDeflateHeaderSize(size_t /*uncompressedSize*/) { return 0; }
 
 } // extern "C"
 

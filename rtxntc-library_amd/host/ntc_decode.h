@@ -37,6 +37,38 @@ enum class ChannelFormat { UNKNOWN = 0, UNORM8 = 1, UNORM16 = 2, FLOAT16 = 3, FL
 enum class BlockCompressedFormat { None = 0, BC1 = 1, BC2 = 2, BC3 = 3, BC4 = 4, BC5 = 5, BC6 = 6, BC7 = 7 };
 enum class ColorSpace { Linear = 0, sRGB = 1, HLG = 2 };
 
+// include/libntc/ntc.h:285-293, 367-371
+enum class InferenceWeightType { Unknown = 0, GenericInt8 = 1, GenericFP8 = 2, CoopVecFP8 = 3, Count };
+enum class CompressionType { None = 0, GDeflate = 1 };
+
+// include/libntc/ntc.h:43-51
+struct VersionInfo
+{
+    int major;
+    int minor;
+    int point;
+    char const* branch;
+    char const* commitHash;
+};
+
+// Source of one output channel in ITextureSet::ShuffleInferenceOutputs (include/libntc/ntc.h:459-517).
+enum class ShuffleSourceType
+{
+    Undefined,   // the channel outputs zero and is not counted as valid
+    Channel,     // the channel outputs what channel `channelIndex` used to output
+    Constant     // the channel outputs `constantValue` and counts as valid
+};
+struct ShuffleSource
+{
+    ShuffleSourceType type = ShuffleSourceType::Undefined;
+    union { int channelIndex; float constantValue; };
+    ShuffleSource() : channelIndex(0) {}
+    int GetChannelIndex() const { return type == ShuffleSourceType::Channel ? channelIndex : -1; }
+    static ShuffleSource Undefined() { return ShuffleSource(); }
+    static ShuffleSource Channel(int index) { ShuffleSource s; s.type = ShuffleSourceType::Channel; s.channelIndex = index; return s; }
+    static ShuffleSource Constant(float value) { ShuffleSource s; s.type = ShuffleSourceType::Constant; s.constantValue = value; return s; }
+};
+
 // include/libntc/ntc.h:272-276
 enum class AddressSpace { Host, Device };
 enum class TextureDataPage { Reference, Output };
@@ -227,8 +259,23 @@ public:
     // index at or beyond the channel count.
     virtual Status SetMaskChannelIndex(int index, bool discardMaskedOutPixels) = 0;
 
-    // Union of the channel ranges of the registered textures (include/libntc/ntc.h:638-640,
-    // src/TextureSetMetadata.cpp:807-832).
+    // The weight blob an application uploads for inference in its own shaders (include/libntc/ntc.h:596-605,
+    // src/TextureSetMetadata.cpp:245-286): host memory owned by the set, valid until the weights
+    // change.  Only InferenceWeightType::GenericInt8 exists here (others: Status::Unsupported);
+    // *pOutConvertedSize is 0.
+    virtual InferenceWeightType GetBestSupportedWeightType() const = 0;
+    virtual Status GetInferenceWeights(InferenceWeightType weightType, void const** pOutData, size_t* pOutSize,
+        size_t* pOutConvertedSize) = 0;
+
+    // Rearranges the rows of the output layer in the weights GetInferenceWeights returns
+    // (include/libntc/ntc.h:620-636, src/TextureSetMetadata.cpp:305-432): afterwards output `ch` is what
+    // output mapping[ch].channelIndex used to be, a constant (zero weights, scale 2^-16, bias
+    // round(c * 2^16)), or zero.  Storage colour spaces and the valid channel mask follow the mapping.
+    // As in the reference, Decompress keeps using the weights as loaded; `mapping` has 16 entries.
+    virtual Status ShuffleInferenceOutputs(ShuffleSource mapping[16]) = 0;
+
+    // Union of the channel ranges of the registered textures, carried through the shuffle mapping;
+    // constant outputs count as valid (include/libntc/ntc.h:638-640, src/TextureSetMetadata.cpp:807-832).
     virtual uint32_t GetValidChannelMask() const = 0;
 
     virtual ~ITextureSet() = default;
@@ -289,8 +336,29 @@ void DestroyContext(IContext* context);
 char const* GetLastErrorMessage();
 char const* StatusToString(Status status);
 char const* ChannelFormatToString(ChannelFormat format);
+char const* BlockCompressedFormatToString(BlockCompressedFormat format);
+char const* ColorSpaceToString(ColorSpace colorSpace);
+char const* InferenceWeightTypeToString(InferenceWeightType weightType);
+char const* CompressionTypeToString(CompressionType type);
 size_t GetBytesPerPixelComponent(ChannelFormat format);
 float LossToPSNR(float loss);
+
+// include/libntc/ntc.h:1312-1313, 1352-1391 (src/PublicFunctions.cpp:36-45,354-557).
+VersionInfo GetLibraryVersion();
+// Size of the compressed data of a set: latent grids plus the Int8 network, without file headers.
+Status EstimateCompressedTextureSetSize(TextureSetDesc const& textureSetDesc, LatentShape const& latentShape, size_t& outSize);
+int GetKnownLatentShapeCount();
+Status EnumerateKnownLatentShapes(int index, float& outBitsPerPixel, LatentShape& outShape);
+// The known shape nearest to the requested bit rate within 25 %, else OutOfRange.
+Status PickLatentShape(float requestedBitsPerPixel, float& outBitsPerPixel, LatentShape& outShape);
+float GetLatentShapeBitsPerPixel(LatentShape const& shape);
+// 16.48 fixed-point result of an image-difference pass -> mean squared error.
+double DecodeImageDifferenceResult(uint64_t value);
+size_t GetBC7ModeBufferSize(int widthInBlocks, int heightInBlocks);
+Status MakeBC7ModeBuffer(int widthInBlocks, int heightInBlocks, void const* blockData, size_t blockDataSize,
+    size_t rowPitch, void* modeBuffer, size_t modeBufferSize);
+// Always 0: GDeflate-compressed views are not supported.
+size_t GetGDeflateHeaderSize(size_t uncompressedSize);
 }
 
 } // namespace ntc

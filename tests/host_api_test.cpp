@@ -9,6 +9,9 @@
 //                      [<maskChannel> <discardMaskedOut 0|1> <withStats 0|1>]
 //       registers two textures (channels 0..2 and 4..5), writes <refPrefix>_mip<N>.bin (FLOAT32 pixels,
 //       all channels) as the reference image, decompresses twice and prints the loss statistics
+//   host_api_test shuffle <preset> <w> <h> <channels> <gridScale> <features> <latents> <weights>
+//       ShuffleInferenceOutputs / GetInferenceWeights: decodes with the loaded weights, shuffles, decodes
+//       again with the weights GetInferenceWeights returns and compares the channels
 //   host_api_test load <file> <device 0|1> [<w> <h> <channels> <mips>]
 //       loads an NTC file: with dimensions through CreateTextureSet + LoadFromFile, without through
 //       CreateCompressedTextureSetFromFile; prints the status, the message and what the set holds
@@ -17,6 +20,7 @@
 #include "../rtxntc-library_amd/host/ntc_decode.h"
 #include "../include/ntc_hip.h"
 
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -238,6 +242,121 @@ static int decode(int argc, char** argv)
     return 0;
 }
 
+// IEEE binary16 bits of a float in the normal half range, round to nearest even (expected constants)
+static uint16_t halfBits(float v)
+{
+    uint32_t f;
+    std::memcpy(&f, &v, 4);
+    uint32_t const sign = (f >> 16) & 0x8000u, exponent = (f >> 23) & 0xffu, mantissa = f & 0x7fffffu;
+    if (exponent == 0) return uint16_t(sign);
+    uint32_t half = ((exponent - 112u) << 10) | (mantissa >> 13);      // exponent rebias 127 -> 15
+    uint32_t const rest = mantissa & 0x1fffu;
+    if (rest > 0x1000u || (rest == 0x1000u && (half & 1u))) ++half;     // a carry into the exponent is the right result
+    return uint16_t(sign | half);
+}
+
+static int shuffle(int argc, char** argv)
+{
+    if (argc < 10) { std::fprintf(stderr, "usage: shuffle <preset> <w> <h> <channels> <gridScale> <features> <latents> <weights>\n"); return 2; }
+    int const preset = std::atoi(argv[2]), w = std::atoi(argv[3]), h = std::atoi(argv[4]), channels = std::atoi(argv[5]);
+    int const gridScale = std::atoi(argv[6]), features = std::atoi(argv[7]);
+    std::vector<unsigned char> latents = readFile(argv[8]), weights = readFile(argv[9]);
+    IContext* ctx = nullptr;
+    ContextParameters params;
+    CHECK(CreateContext(&ctx, params) == Status::Ok);
+    TextureSetDesc desc; desc.width = w; desc.height = h; desc.channels = channels; desc.mips = 1;
+    TextureSetFeatures features_;
+    features_.stagingBytesPerPixel = 16 * 2;
+    ITextureSet* set = nullptr;
+    CHECK(ctx->CreateTextureSet(desc, features_, &set) == Status::Ok);
+    void const* blob = nullptr; size_t blobSize = 0, converted = 1;
+    CHECK(set->GetInferenceWeights(InferenceWeightType::GenericInt8, &blob, &blobSize, &converted) == Status::Unsupported);   // nothing loaded yet
+    CHECK(set->GetBestSupportedWeightType() == InferenceWeightType::Unknown);
+    if (preset == 0) { LatentShape shape; shape.gridSizeScale = gridScale; shape.numFeatures = features; CHECK(set->SetLatentShape(shape) == Status::Ok); }
+    else CHECK(set->SetDecoderPreset(DecoderPreset(preset)) == Status::Ok);
+    CHECK(set->SetLatentData(latents.data(), latents.size()) == Status::Ok);
+    CHECK(set->SetWeightData(weights.data(), weights.size()) == Status::Ok);
+    CHECK(set->GetBestSupportedWeightType() == InferenceWeightType::GenericInt8);
+    CHECK(set->GetInferenceWeights(InferenceWeightType::GenericFP8, &blob, &blobSize, &converted) == Status::Unsupported);
+    CHECK(std::strstr(GetLastErrorMessage(), "GenericFP8") != nullptr);
+    CHECK(set->GetInferenceWeights(InferenceWeightType::GenericInt8, &blob, &blobSize, &converted) == Status::Ok);
+    CHECK(blobSize == weights.size() && converted == 0 && std::memcmp(blob, weights.data(), blobSize) == 0);
+    ITextureMetadata* tex = set->AddTexture(); CHECK(tex->SetChannels(0, 4) == Status::Ok);
+    CHECK(set->GetValidChannelMask() == 0xFu);
+
+    auto decodeAll = [&](std::vector<uint16_t>& out) -> int {
+        CHECK(set->Decompress(nullptr) == Status::Ok);
+        ReadChannelsParameters rp;
+        rp.mipLevel = 0; rp.firstChannel = 0; rp.numChannels = channels; rp.width = w; rp.height = h;
+        rp.pixelStride = size_t(channels) * 2; rp.rowPitch = rp.pixelStride * size_t(w); rp.channelFormat = ChannelFormat::FLOAT16;
+        out.assign(size_t(w) * size_t(h) * size_t(channels), 0);
+        rp.pOutData = reinterpret_cast<unsigned char*>(out.data());
+        CHECK(set->ReadChannels(rp) == Status::Ok);
+        return 0;
+    };
+    std::vector<uint16_t> before, unchanged, after;
+    if (decodeAll(before)) return 1;
+
+    ShuffleSource mapping[16];
+    for (int ch = 0; ch < 16; ++ch) mapping[ch] = ShuffleSource::Channel((ch * 7 + 3) % 16);
+    mapping[0] = ShuffleSource::Channel(5);
+    mapping[1] = ShuffleSource::Constant(0.625f);      // exactly representable
+    mapping[2] = ShuffleSource::Undefined();
+    mapping[3] = ShuffleSource::Channel(3);
+    mapping[4] = ShuffleSource::Constant(0.1f);        // stored as round(0.1 * 2^16) / 2^16
+    mapping[5] = ShuffleSource::Constant(-2.5f);
+    ShuffleSource bad[16];
+    for (int ch = 0; ch < 16; ++ch) bad[ch] = ShuffleSource::Channel(ch);
+    bad[7] = ShuffleSource::Channel(16);
+    CHECK(set->ShuffleInferenceOutputs(nullptr) == Status::InvalidArgument);
+    CHECK(set->ShuffleInferenceOutputs(bad) == Status::OutOfRange);
+    bad[7].type = ShuffleSourceType(9);
+    CHECK(set->ShuffleInferenceOutputs(bad) == Status::InvalidArgument);
+    CHECK(set->ShuffleInferenceOutputs(mapping) == Status::Ok);
+    // valid mask: channels whose source lies in the texture's channels 0..3, and constants
+    uint32_t wantMask = 0;
+    for (int ch = 0; ch < 16; ++ch)
+        if (mapping[ch].type == ShuffleSourceType::Constant || (mapping[ch].type == ShuffleSourceType::Channel && mapping[ch].channelIndex < 4)) wantMask |= 1u << ch;
+    CHECK(set->GetValidChannelMask() == wantMask);
+    // Decompress keeps the weights as loaded
+    if (decodeAll(unchanged)) return 1;
+    CHECK(unchanged == before);
+    // the shuffled weights, used as the set's weights, give the shuffled channels
+    CHECK(set->GetInferenceWeights(InferenceWeightType::GenericInt8, &blob, &blobSize, nullptr) == Status::Ok);
+    std::vector<unsigned char> shuffled(static_cast<unsigned char const*>(blob), static_cast<unsigned char const*>(blob) + blobSize);
+    CHECK(shuffled != weights);
+    CHECK(set->SetWeightData(shuffled.data(), shuffled.size()) == Status::Ok);
+    CHECK(set->GetValidChannelMask() == 0xFu);         // a new blob starts un-shuffled
+    if (decodeAll(after)) return 1;
+    size_t mismatches = 0;
+    for (size_t px = 0; px < size_t(w) * size_t(h); ++px)
+        for (int ch = 0; ch < channels; ++ch) {
+            uint16_t want = 0;
+            if (mapping[ch].type == ShuffleSourceType::Channel) {
+                int const src = mapping[ch].channelIndex;
+                if (src >= channels) continue;             // the source was never stored by the first decode
+                want = before[px * size_t(channels) + size_t(src)];
+            } else if (mapping[ch].type == ShuffleSourceType::Constant) {
+                want = halfBits(float(int32_t(roundf(mapping[ch].constantValue * 65536.f))) * (1.f / 65536.f));
+            }
+            if (after[px * size_t(channels) + size_t(ch)] != want) ++mismatches;
+        }
+    CHECK(mismatches == 0);
+    // shuffling twice composes: the inverse permutation of a bijective mapping restores the blob
+    ShuffleSource perm[16], inverse[16];
+    for (int ch = 0; ch < 16; ++ch) { perm[ch] = ShuffleSource::Channel((ch * 5 + 2) % 16); inverse[(ch * 5 + 2) % 16] = ShuffleSource::Channel(ch); }
+    CHECK(set->SetWeightData(weights.data(), weights.size()) == Status::Ok);
+    CHECK(set->ShuffleInferenceOutputs(perm) == Status::Ok);
+    CHECK(set->ShuffleInferenceOutputs(inverse) == Status::Ok);
+    CHECK(set->GetInferenceWeights(InferenceWeightType::GenericInt8, &blob, &blobSize, nullptr) == Status::Ok);
+    CHECK(std::memcmp(blob, weights.data(), blobSize) == 0);
+    CHECK(set->GetValidChannelMask() == 0xFu);
+    ctx->DestroyTextureSet(set);
+    DestroyContext(ctx);
+    std::printf("host shuffle OK\n");
+    return 0;
+}
+
 static int loss(int argc, char** argv)
 {
     if (argc < 13) { std::fprintf(stderr, "usage: loss <preset> <w> <h> <mips> <channels> <gridScale> <features> <latents> <weights> <refPrefix> <separate>\n"); return 2; }
@@ -414,6 +533,7 @@ int main(int argc, char** argv)
     if (argc >= 2 && std::strcmp(argv[1], "load") == 0) return load(argc, argv);
     if (argc >= 2 && std::strcmp(argv[1], "decodefile") == 0) return decodeFile(argc, argv);
     if (argc >= 2 && std::strcmp(argv[1], "loss") == 0) return loss(argc, argv);
+    if (argc >= 2 && std::strcmp(argv[1], "shuffle") == 0) return shuffle(argc, argv);
     if (argc >= 2 && std::strcmp(argv[1], "cpu") == 0) return cpuChecks();
     if (argc >= 2 && std::strcmp(argv[1], "decode") == 0) return decode(argc, argv);
     std::fprintf(stderr, "usage: host_api_test cpu | decode ...\n");

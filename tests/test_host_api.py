@@ -422,6 +422,25 @@ def test_host_layer_loss_statistics(ntc, oracle, tmp_path, separate):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("preset", [0, 1])
+def test_host_layer_shuffle_inference_outputs(ntc, tmp_path, preset):
+    """ShuffleInferenceOutputs permutes the rows of the output layer in the weights that
+    GetInferenceWeights returns (src/TextureSetMetadata.cpp:305-432).  Checked through the decoder:
+    with the shuffled blob as the set's weights, channel ch decodes to what channel
+    mapping[ch].channelIndex decoded to before, bit for bit; constants come out as
+    round(c * 2^16) / 2^16; undefined channels as zero; a permutation and its inverse restore the blob."""
+    w, h, channels = 96, 64, 16
+    if preset == 0:
+        case = ref_case(ntc, ntc.presets.spec_ref092(16), w, h, 1, 2, channels, ntc.abi.OUT_FP16_PLANAR_PAIRS, 95, scale_log2_range=(-17.0, -12.0))
+    else:
+        case = cfg_case(ntc, ntc.presets.spec_cfg01(), w, h, 1, channels, ntc.abi.OUT_FP16_PLANAR_PAIRS, 96, scale_log2_range=(-17.0, -12.0))
+    lat, wts = tmp_path / "latents.bin", tmp_path / "weights.bin"
+    case.latents.tofile(lat)
+    case.weights.tofile(wts)
+    assert "host shuffle OK" in run_exe("shuffle", preset, w, h, channels, 2, 16, lat, wts)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("with_stats", [1, 0])
 def test_host_layer_mask_channel(ntc, oracle, tmp_path, with_stats):
     """SetMaskChannelIndex (include/libntc/ntc.h:936-940): Decompress clamps the decoded mask channel to
