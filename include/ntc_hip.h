@@ -245,6 +245,39 @@ int ntc_hip_image_loss(void* decodedPlanarPairs, const void* referencePlanarPair
                        int32_t width, int32_t height, int32_t setChannels, uint32_t validChannelMask,
                        int32_t maskChannelIndex, int32_t discardMaskedOutPixels, float* outMse);
 
+/* One image of an image-difference pass: pitch-linear pixels of 1..4 channels (R, G, B, A) in one
+ * of the ChannelFormat encodings; channels a pixel does not store read as 0, 0, 0, 1. */
+typedef struct NtcHipImage {
+    const void* data;           /* device */
+    uint64_t    bytes;
+    uint64_t    pixelStride, rowPitch;
+    int32_t     width, height;  /* size of the whole image (the compared extent must lie inside) */
+    int32_t     format;         /* ChannelFormat, as in NtcHipReadChannels */
+    int32_t     numChannels;
+} NtcHipImage;
+
+/* Per-channel mean squared error (or mean squared log error) between the same rectangle of two
+ * images: the compute pass IContext::MakeImageDifferenceComputePass describes
+ * (include/libntc/ntc.h:1103-1121,1227-1239, src/shaders/ImageDifference.hlsl, constants
+ * include/libntc/shaders/ImageDifferenceConstants.h).  Every workgroup covers 64 x 64 pixels, divides
+ * its four sums by width * height and ADDS them, as 16.48 fixed point, to the four uint64 at
+ * output + outputOffset, which the caller clears beforehand; ntc::DecodeImageDifferenceResult turns
+ * them into doubles.  With useAlphaThreshold, pixels whose alpha is below the threshold in both
+ * images contribute to the alpha channel only; with useMSLE the compared values are log(|v| + 1).
+ * The order in which a workgroup adds its pixels is not defined by the reference (wave intrinsics);
+ * here it is fixed, so results are reproducible.  Asynchronous on the library stream. */
+typedef struct NtcHipImageDifference {
+    NtcHipImage a, b;
+    int32_t     left, top, width, height;     /* extent compared in both images */
+    float       alphaThreshold;
+    int32_t     useAlphaThreshold;
+    int32_t     useMSLE;
+    uint32_t    outputOffset;                 /* bytes, multiple of 8 */
+    void*       output;                       /* device */
+    uint64_t    outputBytes;
+} NtcHipImageDifference;
+int ntc_hip_image_difference(const NtcHipImageDifference* params);
+
 /* Self-check of the MFMA operand layout the kernels assume: multiplies a 16x64 by a
  * 64x16 int8 matrix on the device (row-major host arrays), writes the 16x16 int32
  * product.  No reference counterpart; used by the tests. */

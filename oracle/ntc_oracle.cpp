@@ -46,6 +46,11 @@
  *   image_loss_masked        src/Inference.cu:80-112 in numpy and three special cases: no zero in the
  *                            mask = no mask, all masked = mask channel only, clamp idempotent
  *                            (tests/test_host_api.py)
+ *   image_difference         numpy float64 mean squared error / mean squared log error over the
+ *                            extent, to the fp32 accumulation error; the fixed-point split on
+ *                            values with an exact binary expansion (tests/test_image_difference.py).
+ *                            The reference does not define the order of a workgroup's additions,
+ *                            so its exact low bits are parity unpinned by construction.
  *   The exact bits of the reference's FP16-WMMA CUDA kernel (half accumulation order,
  *   --use_fast_math) and of a hardware bilinear sampler are NOT reproduced: parity unpinned
  *   for those two, by construction; the integer contract of Inference.hlsli is what is pinned.
@@ -728,6 +733,74 @@ void ntc_oracle_image_loss_masked(uint16_t* a, const uint16_t* b, int width, int
             }
         }
     for (int c = 0; c < 16; ++c) outMse[c] /= double(width) * double(height);
+}
+
+// Image-difference pass (src/shaders/ImageDifference.hlsl): per-channel squared differences of two
+// RGBA images over an extent, summed per 64 x 64 workgroup in fp32, normalised, converted to 16.48
+// fixed point and accumulated as integers (hlsl:103-127).  The reference leaves the order of a
+// workgroup's additions to the wave intrinsics; the order restated here is the one the HIP kernel
+// documents: lane = column, wave w takes rows 16w..16w+15 in order, lanes are combined by an xor
+// butterfly with offsets 32..1, the four waves are added in order.  `images` hold host pointers.
+// MSLE uses the host logf; the device's differs in the last places.
+static float diff_channel(NtcHipImage const& im, uint8_t const* px, int c)
+{
+    if (c >= im.numChannels) return c == 3 ? 1.f : 0.f;
+    switch (im.format) {
+    case 1: return float(px[c]) / 255.f;
+    case 2: { uint16_t v; std::memcpy(&v, px + 2 * c, 2); return float(v) / 65535.f; }
+    case 3: { uint16_t v; std::memcpy(&v, px + 2 * c, 2); return half_to_float(v); }
+    case 4: { float v; std::memcpy(&v, px + 4 * c, 4); return v; }
+    default: { uint32_t v; std::memcpy(&v, px + 4 * c, 4); return float(v); }
+    }
+}
+
+static uint32_t saturating_u32(float v)
+{
+    if (!(v > 0.f)) return 0u;                               // negatives and NaN
+    return v >= 4294967296.f ? 0xffffffffu : uint32_t(v);
+}
+
+void ntc_oracle_image_difference(const NtcHipImageDifference* p, uint64_t* out /* 4, added to */)
+{
+    for (int by = 0; by < (p->height + 63) / 64; ++by)
+        for (int bx = 0; bx < (p->width + 63) / 64; ++bx) {
+            float waveSum[4][4];
+            for (int wave = 0; wave < 4; ++wave) {
+                float lanes[64][4];
+                for (int lane = 0; lane < 64; ++lane) {
+                    float mse[4] = { 0.f, 0.f, 0.f, 0.f };
+                    int const x = bx * 64 + lane;
+                    for (int r = 0; r < 16; ++r) {
+                        int const y = by * 64 + wave * 16 + r;
+                        if (x >= p->width || y >= p->height) continue;
+                        uint8_t const* pa = static_cast<uint8_t const*>(p->a.data) + size_t(y + p->top) * p->a.rowPitch + size_t(x + p->left) * p->a.pixelStride;
+                        uint8_t const* pb = static_cast<uint8_t const*>(p->b.data) + size_t(y + p->top) * p->b.rowPitch + size_t(x + p->left) * p->b.pixelStride;
+                        float t1[4], t2[4], diff[4];
+                        for (int c = 0; c < 4; ++c) { t1[c] = diff_channel(p->a, pa, c); t2[c] = diff_channel(p->b, pb, c); }
+                        for (int c = 0; c < 4; ++c)
+                            diff[c] = p->useMSLE ? logf(fabsf(t1[c]) + 1.f) - logf(fabsf(t2[c]) + 1.f) : t1[c] - t2[c];
+                        if (p->useAlphaThreshold && t1[3] < p->alphaThreshold && t2[3] < p->alphaThreshold) diff[0] = diff[1] = diff[2] = 0.f;
+                        for (int c = 0; c < 4; ++c) { float const sq = diff[c] * diff[c]; mse[c] = mse[c] + sq; }
+                    }
+                    for (int c = 0; c < 4; ++c) lanes[lane][c] = mse[c];
+                }
+                for (int off = 32; off >= 1; off >>= 1) {
+                    float next[64][4];
+                    for (int lane = 0; lane < 64; ++lane)
+                        for (int c = 0; c < 4; ++c) next[lane][c] = lanes[lane][c] + lanes[lane ^ off][c];
+                    std::memcpy(lanes, next, sizeof lanes);
+                }
+                for (int c = 0; c < 4; ++c) waveSum[wave][c] = lanes[0][c];
+            }
+            for (int c = 0; c < 4; ++c) {
+                float total = ((waveSum[0][c] + waveSum[1][c]) + waveSum[2][c]) + waveSum[3][c];
+                total = total / float(p->width * p->height);
+                total = total * 65536.f;
+                float const whole = floorf(total);
+                uint64_t const high = saturating_u32(whole), low = saturating_u32(floorf((total - whole) * 4294967296.f));
+                out[c] += (high << 32) | low;
+            }
+        }
 }
 
 // Random-access decode of a list of (u, v, mip) sample points: NtcSampleTextureSet

@@ -88,6 +88,22 @@ class WriteChannels(C.Structure):
     ]
 
 
+class Image(C.Structure):
+    _fields_ = [
+        ("data", C.c_void_p), ("bytes", C.c_uint64), ("pixelStride", C.c_uint64), ("rowPitch", C.c_uint64),
+        ("width", C.c_int32), ("height", C.c_int32), ("format", C.c_int32), ("numChannels", C.c_int32),
+    ]
+
+
+class ImageDifference(C.Structure):
+    _fields_ = [
+        ("a", Image), ("b", Image),
+        ("left", C.c_int32), ("top", C.c_int32), ("width", C.c_int32), ("height", C.c_int32),
+        ("alphaThreshold", C.c_float), ("useAlphaThreshold", C.c_int32), ("useMSLE", C.c_int32), ("outputOffset", C.c_uint32),
+        ("output", C.c_void_p), ("outputBytes", C.c_uint64),
+    ]
+
+
 class Query(C.Structure):
     _fields_ = [("u", C.c_float), ("v", C.c_float), ("mip", C.c_int32)]
 
@@ -125,6 +141,7 @@ EXPORTS = [
     ("ntc_hip_write_channels", C.c_int, [C.POINTER(WriteChannels)]),
     ("ntc_hip_image_loss", C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64, C.c_int32, C.c_int32, C.c_int32, C.c_uint32, C.c_int32, C.c_int32,
                                      C.POINTER(C.c_float)]),
+    ("ntc_hip_image_difference", C.c_int, [C.POINTER(ImageDifference)]),
     ("ntc_hip_selftest_mfma", C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
     ("ntc_hip_selftest_mfma_f16", C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32]),
 ]

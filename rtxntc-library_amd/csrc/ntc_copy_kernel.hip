@@ -434,6 +434,78 @@ hipError_t launch_image_loss(uint16_t* a, uint16_t const* b, int width, int heig
     return hipGetLastError();
 }
 
+// ---- image difference (src/shaders/ImageDifference.hlsl) -------------------------------------------
+//
+// A workgroup covers 64 x 64 pixels of the extent, as the reference's does (16 x 16 threads of 4 x 4
+// pixels); here lane = column and each wave walks 16 rows, so that the loads of a wave are one
+// contiguous row piece.  Every thread adds its 16 squared differences in row order, the 64 lanes
+// of a wave are combined by an xor butterfly (offsets 32 ... 1), the four waves in order.  Squares
+// and sums are separate fp32 operations (no fused multiply-add).  The workgroup's sums are divided
+// by width * height, scaled by 2^16, split into floor and fraction * 2^32 and added to the 64-bit
+// accumulators (ImageDifference.hlsl:103-127; the integer atomics make the total independent of
+// the order in which workgroups finish).
+__device__ __forceinline__ float diff_channel(DiffImageArgs const& im, uint8_t const* px, int c)
+{
+    if (c >= im.numChannels) return c == 3 ? 1.f : 0.f;
+    switch (im.format) {
+    case NTC_HIP_DEV_FORMAT_UNORM8:  return float(px[c]) / 255.f;
+    case NTC_HIP_DEV_FORMAT_UNORM16: return float(reinterpret_cast<uint16_t const*>(px)[c]) / 65535.f;
+    case NTC_HIP_DEV_FORMAT_FLOAT16: return float(reinterpret_cast<_Float16 const*>(px)[c]);
+    case NTC_HIP_DEV_FORMAT_FLOAT32: return reinterpret_cast<float const*>(px)[c];
+    default:                         return float(reinterpret_cast<uint32_t const*>(px)[c]);
+    }
+}
+
+__global__ void __launch_bounds__(256)
+image_difference_kernel(ImageDifferenceArgs a)
+{
+    __shared__ float sums[4][4];
+    int const lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int const x = blockIdx.x * 64 + lane;
+    float mse[4] = { 0.f, 0.f, 0.f, 0.f };
+    for (int r = 0; r < 16; ++r) {
+        int const y = blockIdx.y * 64 + wave * 16 + r;
+        if (x >= a.width || y >= a.height) continue;
+        uint8_t const* const pa = a.a.data + size_t(y + a.top) * a.a.rowPitch + size_t(x + a.left) * a.a.pixelStride;
+        uint8_t const* const pb = a.b.data + size_t(y + a.top) * a.b.rowPitch + size_t(x + a.left) * a.b.pixelStride;
+        float t1[4], t2[4], diff[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) { t1[c] = diff_channel(a.a, pa, c); t2[c] = diff_channel(a.b, pb, c); }
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            diff[c] = a.useMSLE ? __fsub_rn(logf(fabsf(t1[c]) + 1.f), logf(fabsf(t2[c]) + 1.f)) : __fsub_rn(t1[c], t2[c]);
+        if (a.useAlphaThreshold && t1[3] < a.alphaThreshold && t2[3] < a.alphaThreshold) { diff[0] = 0.f; diff[1] = 0.f; diff[2] = 0.f; }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) mse[c] = __fadd_rn(mse[c], __fmul_rn(diff[c], diff[c]));
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        float v = mse[c];
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) v = __fadd_rn(v, __shfl_xor(v, off, 64));
+        if (lane == 0) sums[wave][c] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x < 4) {
+        int const c = threadIdx.x;
+        float total = __fadd_rn(__fadd_rn(__fadd_rn(sums[0][c], sums[1][c]), sums[2][c]), sums[3][c]);
+        total = __fdiv_rn(total, float(a.width * a.height));
+        total = __fmul_rn(total, 65536.f);
+        float const whole = floorf(total);
+        // float -> uint32 conversions saturate; a NaN (from NaN pixels) adds nothing
+        unsigned long long const high = uint32_t(whole), low = uint32_t(floorf(__fmul_rn(__fsub_rn(total, whole), 4294967296.f)));
+        unsigned long long const fixed = (high << 32) | low;
+        if (fixed) atomicAdd(a.output + c, fixed);
+    }
+}
+
+hipError_t launch_image_difference(ImageDifferenceArgs const& a, hipStream_t stream)
+{
+    dim3 const grid((a.width + 63) / 64, (a.height + 63) / 64);
+    hipLaunchKernelGGL(image_difference_kernel, grid, dim3(256), 0, stream, a);
+    return hipGetLastError();
+}
+
 template <int FORMAT>
 static void launch_read_format(ReadChannelsArgs const& a, dim3 grid, bool plain, hipStream_t stream)
 {

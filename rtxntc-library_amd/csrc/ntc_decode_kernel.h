@@ -96,6 +96,20 @@ inline size_t image_loss_blocks(int width, int height)
 hipError_t launch_image_loss(uint16_t* a, uint16_t const* b, int width, int height, int setChannels,
                              uint32_t validChannelMask, int maskChannel, int discardMaskedOut, double* partials, hipStream_t stream);
 
+struct DiffImageArgs {
+    uint8_t const* data;
+    uint64_t pixelStride, rowPitch;
+    int32_t format, numChannels;
+};
+struct ImageDifferenceArgs {
+    DiffImageArgs a, b;
+    int32_t left, top, width, height;
+    float alphaThreshold;
+    int32_t useAlphaThreshold, useMSLE;
+    unsigned long long* output;    // four 16.48 fixed-point accumulators
+};
+hipError_t launch_image_difference(ImageDifferenceArgs const& args, hipStream_t stream);
+
 hipError_t launch_decode(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream);
 hipError_t launch_queries(int variant, DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries,
                           uint16_t* out, int gridSize, hipStream_t stream);

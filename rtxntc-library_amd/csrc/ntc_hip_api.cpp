@@ -675,6 +675,54 @@ int ntc_hip_image_loss(void* decoded, const void* reference, uint64_t planarByte
     return 0;
 }
 
+static int check_diff_image(NtcHipImage const& im, char const* which, int left, int top, int width, int height, DiffImageArgs& out)
+{
+    int const bpc = bytes_per_component(im.format);
+    if (!im.data || !bpc) { set_error("ntc_hip_image_difference: image %s has no data or an unknown channel format (%d).", which, im.format); return NTC_HIP_ERR_INVALID_ARG; }
+    if (im.numChannels < 1 || im.numChannels > 4 || im.width < 1 || im.height < 1) { set_error("ntc_hip_image_difference: image %s: 1..4 channels and a positive size are required.", which); return NTC_HIP_ERR_INVALID_ARG; }
+    if (im.pixelStride < uint64_t(bpc) * uint64_t(im.numChannels) || im.rowPitch < im.pixelStride * uint64_t(im.width)
+        || (im.pixelStride % uint64_t(bpc)) || (im.rowPitch % uint64_t(bpc)) || (reinterpret_cast<uintptr_t>(im.data) % uintptr_t(bpc))) {
+        set_error("ntc_hip_image_difference: image %s: pixel stride / row pitch do not fit the format and channel count.", which);
+        return NTC_HIP_ERR_INVALID_ARG;
+    }
+    if (uint64_t(im.height - 1) * im.rowPitch + uint64_t(im.width - 1) * im.pixelStride + uint64_t(bpc) * uint64_t(im.numChannels) > im.bytes) {
+        set_error("ntc_hip_image_difference: image %s reaches past its buffer.", which);
+        return NTC_HIP_ERR_INVALID_ARG;
+    }
+    if (int64_t(left) + width > im.width || int64_t(top) + height > im.height) {
+        set_error("ntc_hip_image_difference: the extent (%d, %d, %d x %d) does not lie inside image %s (%d x %d).", left, top, width, height, which, im.width, im.height);
+        return NTC_HIP_ERR_INVALID_ARG;
+    }
+    out.data = static_cast<uint8_t const*>(im.data);
+    out.pixelStride = im.pixelStride; out.rowPitch = im.rowPitch; out.format = im.format; out.numChannels = im.numChannels;
+    return 0;
+}
+
+int ntc_hip_image_difference(const NtcHipImageDifference* p)
+{
+    if (int r = require_init()) return r;
+    if (!p || !p->output) { set_error("ntc_hip_image_difference: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
+    // src/Context.cpp:796-812
+    if (p->left < 0 || p->top < 0) { set_error("ntc_hip_image_difference: left (%d) and top (%d) must be non-negative.", p->left, p->top); return NTC_HIP_ERR_INVALID_ARG; }
+    if (p->width <= 0 || p->height <= 0 || int64_t(p->width) * int64_t(p->height) > INT32_MAX) {
+        set_error("ntc_hip_image_difference: width (%d) and height (%d) must be positive (and their product below 2^31).", p->width, p->height);
+        return NTC_HIP_ERR_INVALID_ARG;
+    }
+    if ((p->outputOffset & 7u) || (reinterpret_cast<uintptr_t>(p->output) & 7u) || uint64_t(p->outputOffset) + 32u > p->outputBytes) {
+        set_error("ntc_hip_image_difference: the four 64-bit results at outputOffset (%u) must be 8-byte aligned and inside the output buffer.", p->outputOffset);
+        return NTC_HIP_ERR_INVALID_ARG;
+    }
+    ImageDifferenceArgs a{};
+    if (int r = check_diff_image(p->a, "A", p->left, p->top, p->width, p->height, a.a)) return r;
+    if (int r = check_diff_image(p->b, "B", p->left, p->top, p->width, p->height, a.b)) return r;
+    a.left = p->left; a.top = p->top; a.width = p->width; a.height = p->height;
+    a.alphaThreshold = p->alphaThreshold; a.useAlphaThreshold = p->useAlphaThreshold ? 1 : 0; a.useMSLE = p->useMSLE ? 1 : 0;
+    a.output = reinterpret_cast<unsigned long long*>(static_cast<uint8_t*>(p->output) + p->outputOffset);
+    HIP_TRY(launch_image_difference(a, g_lib.stream));
+    clear_error();
+    return 0;
+}
+
 int ntc_hip_selftest_mfma(const int8_t* a16x64, const int8_t* b64x16, int32_t* d16x16)
 {
     if (int r = require_init()) return r;

@@ -1141,6 +1141,42 @@ public:
     void DestroyTextureSet(ITextureSet* textureSet) const override { delete textureSet; }
     bool IsCudaAvailable() const override { return m_deviceAvailable; }
 
+    // Argument rules and messages of src/Context.cpp:796-812; the pass itself is ntc_hip_image_difference.
+    Status ComputeImageDifference(ImageDifferenceParameters const& params) const override
+    {
+        if (!params.pOutputBuffer) { SetErrorMessage("pOutputBuffer is NULL"); return Status::InvalidArgument; }
+        if (!params.imageA.pData || !params.imageB.pData) { SetErrorMessage("Image data is NULL"); return Status::InvalidArgument; }
+        if (params.extent.left < 0 || params.extent.top < 0) {
+            SetErrorMessage("Left (%d) and top (%d) must be non-negative", params.extent.left, params.extent.top);
+            return Status::OutOfRange;
+        }
+        if (params.extent.width <= 0 || params.extent.height <= 0) {
+            SetErrorMessage("Width (%d) and height (%d) must be positive", params.extent.width, params.extent.height);
+            return Status::OutOfRange;
+        }
+        if ((params.outputOffset & 7u) != 0) {
+            SetErrorMessage("outputOffset (%d) must be aligned to 8 bytes", int(params.outputOffset));
+            return Status::OutOfRange;
+        }
+        if (!m_deviceAvailable) { SetErrorMessage("No HIP device is available to this context."); return Status::CudaUnavailable; }
+        NtcHipImageDifference p{};
+        auto fill = [](NtcHipImage& dst, ImageDesc const& src) {
+            dst.data = src.pData; dst.bytes = src.dataSize; dst.pixelStride = src.pixelStride; dst.rowPitch = src.rowPitch;
+            dst.width = src.width; dst.height = src.height; dst.format = int32_t(src.channelFormat); dst.numChannels = src.numChannels;
+        };
+        fill(p.a, params.imageA);
+        fill(p.b, params.imageB);
+        p.left = params.extent.left; p.top = params.extent.top; p.width = params.extent.width; p.height = params.extent.height;
+        p.alphaThreshold = params.alphaThreshold;
+        p.useAlphaThreshold = params.useAlphaThreshold ? 1 : 0;
+        p.useMSLE = params.useMSLE ? 1 : 0;
+        p.outputOffset = params.outputOffset;
+        p.output = params.pOutputBuffer; p.outputBytes = params.outputBufferSize;
+        if (int r = ntc_hip_image_difference(&p)) return DeviceFailure(r);
+        ClearErrorMessage();
+        return Status::Ok;
+    }
+
     // src/Context.cpp:80-176
     Status OpenFile(char const* fileName, bool write, IStream** pOutStream) const override
     {

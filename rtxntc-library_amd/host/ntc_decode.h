@@ -170,6 +170,37 @@ struct ContextParameters
     int cudaDevice = 0;             // index of the HIP device; the name is kept for source compatibility
 };
 
+// include/libntc/ntc.h (Rect): a rectangle of pixels.
+struct Rect { int left = 0; int top = 0; int width = 0; int height = 0; };
+
+// One image of IContext::ComputeImageDifference: pitch-linear pixels of 1..4 channels (R, G, B, A) in
+// device memory; channels a pixel does not store read as 0, 0, 0, 1.
+struct ImageDesc
+{
+    unsigned char const* pData = nullptr;
+    size_t dataSize = 0;
+    int width = 0;
+    int height = 0;
+    size_t pixelStride = 0;
+    size_t rowPitch = 0;
+    ChannelFormat channelFormat = ChannelFormat::UNKNOWN;
+    int numChannels = 4;
+};
+
+// The fields of MakeImageDifferenceComputePassParameters (include/libntc/ntc.h:1103-1121) plus what a
+// graphics application binds to that pass: the two images and the output buffer.
+struct ImageDifferenceParameters
+{
+    ImageDesc imageA, imageB;
+    Rect extent;                        // compared in both images
+    bool useAlphaThreshold = false;     // ignore colour differences where both alphas are below the threshold
+    float alphaThreshold = 1.f / 255.f;
+    bool useMSLE = false;               // mean squared log error of |values| instead of mean squared error
+    void* pOutputBuffer = nullptr;      // device memory, cleared by the caller: four uint64 in 16.48 fixed point are ADDED
+    size_t outputBufferSize = 0;
+    uint32_t outputOffset = 0;          // bytes, multiple of 8
+};
+
 // Decoder families beyond the one compiled into LibNTC 0.9.2, selected with
 // ITextureSet::SetDecoderPreset (an addition; the reference changes decoders by editing
 // InferenceConstants.h, README.md:32-36).
@@ -303,6 +334,10 @@ public:
         ITextureSet** pOutTextureSet) const = 0;
     virtual Status CreateCompressedTextureSetFromFile(char const* fileName, TextureSetFeatures const& features,
         ITextureSet** pOutTextureSet) const = 0;
+    // Runs the image-difference pass that IContext::MakeImageDifferenceComputePass describes for a
+    // graphics API (include/libntc/ntc.h:1227-1239, src/Context.cpp:781-860, src/shaders/ImageDifference.hlsl)
+    // on the device, asynchronously; DecodeImageDifferenceResult converts the four results.
+    virtual Status ComputeImageDifference(ImageDifferenceParameters const& params) const = 0;
     // True when a gfx950 device was initialised (reference: IsCudaAvailable).
     virtual bool IsCudaAvailable() const = 0;
     virtual ~IContext() = default;

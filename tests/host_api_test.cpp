@@ -12,6 +12,8 @@
 //   host_api_test shuffle <preset> <w> <h> <channels> <gridScale> <features> <latents> <weights>
 //       ShuffleInferenceOutputs / GetInferenceWeights: decodes with the loaded weights, shuffles, decodes
 //       again with the weights GetInferenceWeights returns and compares the channels
+//   host_api_test imagediff
+//       IContext::ComputeImageDifference on images with exactly known differences
 //   host_api_test load <file> <device 0|1> [<w> <h> <channels> <mips>]
 //       loads an NTC file: with dimensions through CreateTextureSet + LoadFromFile, without through
 //       CreateCompressedTextureSetFromFile; prints the status, the message and what the set holds
@@ -153,6 +155,27 @@ static int cpuChecks()
     CHECK(set->ReadChannels(rp) == Status::InvalidArgument);
     rp.rowPitch = 4; rp.channelFormat = ChannelFormat::UNORM8;
     CHECK(set->ReadChannels(rp) == Status::CudaUnavailable);                 // arguments fine, no device
+
+    // image-difference pass: argument rules come first, then the missing device
+    {
+        unsigned char pixels[64] = {};
+        uint64_t result[4] = {};
+        ImageDifferenceParameters dp;
+        dp.imageA.pData = pixels; dp.imageA.dataSize = sizeof pixels; dp.imageA.width = 4; dp.imageA.height = 4;
+        dp.imageA.pixelStride = 4; dp.imageA.rowPitch = 16; dp.imageA.channelFormat = ChannelFormat::UNORM8;
+        dp.imageB = dp.imageA;
+        dp.extent.width = 4; dp.extent.height = 4;
+        CHECK(ctx->ComputeImageDifference(dp) == Status::InvalidArgument);       // no output buffer
+        dp.pOutputBuffer = result; dp.outputBufferSize = sizeof result;
+        dp.extent.left = -1;
+        CHECK(ctx->ComputeImageDifference(dp) == Status::OutOfRange);
+        dp.extent.left = 0; dp.extent.height = 0;
+        CHECK(ctx->ComputeImageDifference(dp) == Status::OutOfRange);
+        dp.extent.height = 4; dp.outputOffset = 4;
+        CHECK(ctx->ComputeImageDifference(dp) == Status::OutOfRange);
+        dp.outputOffset = 0;
+        CHECK(ctx->ComputeImageDifference(dp) == Status::CudaUnavailable);
+    }
 
     ctx->DestroyTextureSet(set);
     DestroyContext(ctx);
@@ -357,6 +380,48 @@ static int shuffle(int argc, char** argv)
     return 0;
 }
 
+// IContext::ComputeImageDifference on two small images in device memory: every byte differs by 255
+// in one image pair (mean squared error exactly 1 in all four channels), the alpha threshold removes
+// the colour channels, and a sub-rectangle of identical pixels gives zero.
+static int imageDifference()
+{
+    IContext* ctx = nullptr;
+    ContextParameters params;
+    CHECK(CreateContext(&ctx, params) == Status::Ok);
+    int const w = 192, h = 80;
+    std::vector<unsigned char> a(size_t(w) * h * 4, 0), b(size_t(w) * h * 4, 255);
+    for (int y = 0; y < 16; ++y) for (int x = 0; x < 32; ++x) std::memcpy(&b[(size_t(y) * w + x) * 4], &a[(size_t(y) * w + x) * 4], 4);   // identical corner
+    void *dA = nullptr, *dB = nullptr, *dOut = nullptr;
+    CHECK(ntc_hip_alloc(&dA, a.size()) == 0 && ntc_hip_alloc(&dB, b.size()) == 0 && ntc_hip_alloc(&dOut, 64) == 0);
+    CHECK(ntc_hip_upload(dA, a.data(), a.size()) == 0 && ntc_hip_upload(dB, b.data(), b.size()) == 0);
+    uint64_t zeros[8] = {}, result[8] = {};
+    CHECK(ntc_hip_upload(dOut, zeros, sizeof zeros) == 0);
+    ImageDifferenceParameters dp;
+    dp.imageA.pData = static_cast<unsigned char const*>(dA); dp.imageA.dataSize = a.size(); dp.imageA.width = w; dp.imageA.height = h;
+    dp.imageA.pixelStride = 4; dp.imageA.rowPitch = size_t(w) * 4; dp.imageA.channelFormat = ChannelFormat::UNORM8;
+    dp.imageB = dp.imageA; dp.imageB.pData = static_cast<unsigned char const*>(dB);
+    dp.pOutputBuffer = dOut; dp.outputBufferSize = 64;
+    dp.extent.left = 64; dp.extent.top = 16; dp.extent.width = 128; dp.extent.height = 64;     // all pixels differ
+    CHECK(ctx->ComputeImageDifference(dp) == Status::Ok);
+    dp.outputOffset = 32; dp.extent = Rect{ 0, 0, 32, 16 };                                     // identical pixels
+    CHECK(ctx->ComputeImageDifference(dp) == Status::Ok);
+    CHECK(ntc_hip_download(result, dOut, sizeof result) == 0);
+    for (int c = 0; c < 4; ++c) CHECK(DecodeImageDifferenceResult(result[c]) == 1.0 && result[4 + c] == 0);
+    // both alphas (0 and 1) below a threshold of 2: colour ignored, alpha still compared
+    CHECK(ntc_hip_upload(dOut, zeros, sizeof zeros) == 0);
+    dp.outputOffset = 0; dp.extent = Rect{ 64, 16, 128, 64 }; dp.useAlphaThreshold = true; dp.alphaThreshold = 2.f;
+    CHECK(ctx->ComputeImageDifference(dp) == Status::Ok);
+    CHECK(ntc_hip_download(result, dOut, sizeof result) == 0);
+    CHECK(result[0] == 0 && result[1] == 0 && result[2] == 0 && DecodeImageDifferenceResult(result[3]) == 1.0);
+    dp.extent.width = 200;                                                                      // leaves the image
+    CHECK(ctx->ComputeImageDifference(dp) == Status::InvalidArgument);
+    CHECK(std::strstr(GetLastErrorMessage(), "does not lie inside") != nullptr);
+    CHECK(ntc_hip_free(dA) == 0 && ntc_hip_free(dB) == 0 && ntc_hip_free(dOut) == 0);
+    DestroyContext(ctx);
+    std::printf("host image difference OK\n");
+    return 0;
+}
+
 static int loss(int argc, char** argv)
 {
     if (argc < 13) { std::fprintf(stderr, "usage: loss <preset> <w> <h> <mips> <channels> <gridScale> <features> <latents> <weights> <refPrefix> <separate>\n"); return 2; }
@@ -534,6 +599,7 @@ int main(int argc, char** argv)
     if (argc >= 2 && std::strcmp(argv[1], "decodefile") == 0) return decodeFile(argc, argv);
     if (argc >= 2 && std::strcmp(argv[1], "loss") == 0) return loss(argc, argv);
     if (argc >= 2 && std::strcmp(argv[1], "shuffle") == 0) return shuffle(argc, argv);
+    if (argc >= 2 && std::strcmp(argv[1], "imagediff") == 0) return imageDifference();
     if (argc >= 2 && std::strcmp(argv[1], "cpu") == 0) return cpuChecks();
     if (argc >= 2 && std::strcmp(argv[1], "decode") == 0) return decode(argc, argv);
     std::fprintf(stderr, "usage: host_api_test cpu | decode ...\n");

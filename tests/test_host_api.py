@@ -441,6 +441,11 @@ def test_host_layer_shuffle_inference_outputs(ntc, tmp_path, preset):
 
 
 @pytest.mark.gpu
+def test_host_layer_image_difference():
+    assert "host image difference OK" in run_exe("imagediff")
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("with_stats", [1, 0])
 def test_host_layer_mask_channel(ntc, oracle, tmp_path, with_stats):
     """SetMaskChannelIndex (include/libntc/ntc.h:936-940): Decompress clamps the decoded mask channel to
