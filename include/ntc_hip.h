@@ -193,8 +193,9 @@ int ntc_hip_decode_queries_timed(const NtcHipTextureSet* set, const NtcHipQuery*
 
 /* Extracts channels of one decoded mip from the internal fp16 layout into a user image:
  * what ITextureSet::ReadChannels does through cuda::CopyImage (src/TextureSet.cpp:915-985,
- * src/ImageProcessing.cu:86-164,220-277).  Same-size copies only (the reference's 1:1
- * branch).  Each copied channel is decoded from its storage colour space and encoded into the
+ * src/ImageProcessing.cu:24-72,86-164,220-277).  When dstWidth x dstHeight differs from the mip's size the
+ * image is resampled with the reference's bilinear filter (edge texels clamped, taps of zero weight
+ * not read; a 2x reduction is a 2x2 box filter).  Each copied channel is decoded from its storage colour space and encoded into the
  * destination's (0 linear, 1 sRGB, 2 HLG; src/CudaUtils.h:61-114); with useDithering every
  * destination channel of UNORM formats gets the reference's hash-based noise of +-1/2 step
  * (src/CudaUtils.h:117-184).  Destination channels beyond numChannels get the reference's
@@ -212,12 +213,14 @@ typedef struct NtcHipReadChannels {
     uint64_t    pixelStride, rowPitch;
     uint8_t     srcColorSpaces[16];   /* storage colour space of set channel firstChannel + i */
     uint8_t     dstColorSpaces[16];   /* colour space wanted for copied channel i */
+    int32_t     dstWidth, dstHeight;  /* size of the user image; 0, 0 = the mip's size */
 } NtcHipReadChannels;
 int ntc_hip_read_channels(const NtcHipReadChannels* params);
 
 /* Stores a user image into the internal fp16 layout of one mip: what ITextureSet::WriteChannels
  * does through cuda::CopyImage (src/TextureSet.cpp:829-913, src/ImageProcessing.cu:107-164,220-277).
- * Same-size copies; colour spaces as in NtcHipReadChannels.  Asynchronous on the library stream. */
+ * A source image of another size (srcWidth x srcHeight) is resampled as in NtcHipReadChannels; colour
+ * spaces as there.  Asynchronous on the library stream. */
 typedef struct NtcHipWriteChannels {
     const void* src;            /* device: pitch-linear user image */
     uint64_t    srcBytes;
@@ -229,8 +232,17 @@ typedef struct NtcHipWriteChannels {
     int32_t     width, height, setChannels, firstChannel, numChannels, reserved;
     uint8_t     srcColorSpaces[16];   /* colour space of channel i of the user image */
     uint8_t     dstColorSpaces[16];   /* storage colour space of set channel firstChannel + i */
+    int32_t     srcWidth, srcHeight;  /* size of the user image; 0, 0 = the mip's size */
 } NtcHipWriteChannels;
 int ntc_hip_write_channels(const NtcHipWriteChannels* params);
+
+/* Resamples one image of the internal layout into another (all channels), decoding each channel from
+ * its storage colour space, filtering, and encoding it again: cuda::ResizeMultichannelImage as
+ * ITextureSet::GenerateMips uses it from one mip to the next (src/ImageProcessing.cu:178-218,
+ * src/TextureSet.cpp:1121-1142).  The images must not overlap.  Asynchronous on the library stream. */
+int ntc_hip_resize_planar(const void* srcPlanarPairs, uint64_t srcBytes, int32_t srcWidth, int32_t srcHeight,
+                          void* dstPlanarPairs, uint64_t dstBytes, int32_t dstWidth, int32_t dstHeight,
+                          int32_t setChannels, const uint8_t* channelColorSpaces /* 16 */);
 
 /* Mean squared error per channel between two images in the internal layout (a decoded mip and its
  * reference): the loss branch of InferenceKernel + ReduceLoss (src/Inference.cu:77-118,142-156,

@@ -42,6 +42,10 @@
  *   decode_queries           the raster decode of the texels the queries hit (tests/test_queries.py)
  *   read_channels,           numpy models of the 1:1 branch of cuda::CopyImage, five channel
  *   write_channels           formats, padded rows, vertical flip (tests/test_host_api.py)
+ *   resampling copies        numpy float64 bilinear resampling with clamped edges (to fp32 rounding);
+ *   (read/write_channels_    exact cases: a 2x reduction is the mean of each 2x2 block added in
+ *   resized, resize_planar)  tap order, same-size calls equal the 1:1 functions, a constant image
+ *                            stays constant (tests/test_resampling.py)
  *   image_loss,              numpy float64 mean squared error, with the mask options restated from
  *   image_loss_masked        src/Inference.cu:80-112 in numpy and three special cases: no zero in the
  *                            mask = no mask, all masked = mask channel only, clamp idempotent
@@ -683,6 +687,138 @@ int ntc_oracle_write_channels(const uint8_t* src, int format, int verticalFlip, 
 {
     return ntc_oracle_write_channels_ex(src, format, verticalFlip, pixelStride, rowPitch, planarPairs, width, height, setChannels,
                                         firstChannel, numChannels, nullptr, nullptr);
+}
+
+// ---- resampling copies: SetupBilinearFilter (src/ImageProcessing.cu:24-72) ---------------------------
+// Destination pixel (x, y) looks at ((x + 1/2) / dstW) * srcW - 1/2 in the source, clamped to the image;
+// four taps, bilinear weights, taps of zero weight not read (:232-237).  The blend
+// a*w0 + b*w1 + c*w2 + d*w3 is evaluated as one multiply and three fused multiply-adds (the
+// contraction a CUDA compiler applies to that expression); the reference's fast-math division in
+// the position is an IEEE division here, so its last bits are parity unpinned.
+struct ResampleTaps { int x0, y0, x1, y1; float w[4]; };
+
+static ResampleTaps resample_taps(int srcW, int srcH, int dstW, int dstH, int x, int y)
+{
+    if (srcW == dstW && srcH == dstH) return ResampleTaps{ x, y, x, y, { 1.f, 0.f, 0.f, 0.f } };    // the 1:1 shortcut, :39-45
+    float const u = (float(x) + 0.5f) / float(dstW), v = (float(y) + 0.5f) / float(dstH);
+    float const px = std::max(0.f, std::min(float(srcW) - 1.f, u * float(srcW) - 0.5f));
+    float const py = std::max(0.f, std::min(float(srcH) - 1.f, v * float(srcH) - 0.5f));
+    float const fx = px - std::floor(px), fy = py - std::floor(py);
+    ResampleTaps t;
+    t.x0 = int(std::floor(px)); t.y0 = int(std::floor(py));
+    t.x1 = std::min(t.x0 + 1, srcW - 1); t.y1 = std::min(t.y0 + 1, srcH - 1);
+    t.w[0] = (1.f - fx) * (1.f - fy); t.w[1] = fx * (1.f - fy); t.w[2] = (1.f - fx) * fy; t.w[3] = fx * fy;
+    return t;
+}
+
+static float resample_blend(ResampleTaps const& t, float a, float b, float c, float d)
+{
+    a = t.w[0] > 0.f ? a : 0.f; b = t.w[1] > 0.f ? b : 0.f; c = t.w[2] > 0.f ? c : 0.f; d = t.w[3] > 0.f ? d : 0.f;
+    return std::fmaf(d, t.w[3], std::fmaf(c, t.w[2], std::fmaf(b, t.w[1], a * t.w[0])));
+}
+
+static float planar_value(const uint16_t* image, int width, int setChannels, int x, int y, int c)
+{
+    return half_to_float(image[size_t(y) * size_t(width) * size_t(setChannels) + size_t(c & ~1) * size_t(width) + size_t(x) * 2 + size_t(c & 1)]);
+}
+
+static float user_value(const uint8_t* px, int format, int ch)
+{
+    switch (format) {
+    case 1: return float(px[ch]) / 255.f;
+    case 2: { uint16_t t; std::memcpy(&t, px + 2 * ch, 2); return float(t) / 65535.f; }
+    case 3: { uint16_t t; std::memcpy(&t, px + 2 * ch, 2); return half_to_float(t); }
+    case 4: { float t; std::memcpy(&t, px + 4 * ch, 4); return t; }
+    default: { uint32_t t; std::memcpy(&t, px + 4 * ch, 4); return float(t); }
+    }
+}
+
+// ReadChannels into an image of another size (CopyImageKernel, src/ImageProcessing.cu:220-265).
+int ntc_oracle_read_channels_resized(const uint16_t* planarPairs, int width, int height, int setChannels,
+                                     int firstChannel, int numChannels, uint8_t* dst, int format,
+                                     uint64_t pixelStride, uint64_t rowPitch, int dstWidth, int dstHeight, int useDithering,
+                                     const uint8_t* srcColorSpaces, const uint8_t* dstColorSpaces)
+{
+    int const bpc = (format == 1) ? 1 : (format == 2 || format == 3) ? 2 : (format == 4 || format == 5) ? 4 : 0;
+    if (!bpc) return -1;
+    int const dstChannels = int(pixelStride / uint64_t(bpc));
+    auto roundHalfAway = [](float v) {
+        float r = std::trunc(v);
+        float const fr = v - r;
+        if (fr >= 0.5f) r += 1.f; else if (fr <= -0.5f) r -= 1.f;
+        return r;
+    };
+    for (int y = 0; y < dstHeight; ++y)
+        for (int x = 0; x < dstWidth; ++x) {
+            ResampleTaps const t = resample_taps(width, height, dstWidth, dstHeight, x, y);
+            uint8_t* px = dst + size_t(y) * rowPitch + size_t(x) * pixelStride;
+            HashRng rng(uint32_t(x) + uint32_t(y) * uint32_t(dstWidth));
+            for (int ch = 0; ch < dstChannels; ++ch) {
+                float value;
+                if (ch < numChannels) {
+                    int const c = firstChannel + ch, space = srcColorSpaces ? srcColorSpaces[ch] : 0;
+                    value = resample_blend(t, decode_color_space(space, planar_value(planarPairs, width, setChannels, t.x0, t.y0, c)),
+                                              decode_color_space(space, planar_value(planarPairs, width, setChannels, t.x1, t.y0, c)),
+                                              decode_color_space(space, planar_value(planarPairs, width, setChannels, t.x0, t.y1, c)),
+                                              decode_color_space(space, planar_value(planarPairs, width, setChannels, t.x1, t.y1, c)));
+                } else {
+                    value = (ch == 3) ? 1.f : 0.f;
+                }
+                float const dither = useDithering ? rng.next_float() - 0.5f : 0.f;
+                value = encode_color_space((dstColorSpaces && ch < 16) ? dstColorSpaces[ch] : 0, value);
+                switch (format) {
+                case 1: value += dither / 255.f; px[ch] = uint8_t(std::max(0.f, std::min(255.f, roundHalfAway(value * 255.f)))); break;
+                case 2: { value += dither / 65535.f; uint16_t v = uint16_t(std::max(0.f, std::min(65535.f, roundHalfAway(value * 65535.f)))); std::memcpy(px + 2 * ch, &v, 2); break; }
+                case 3: { uint16_t v = float_to_half_rne(std::max(-65504.f, std::min(65504.f, value))); std::memcpy(px + 2 * ch, &v, 2); break; }
+                case 4: std::memcpy(px + 4 * ch, &value, 4); break;
+                case 5: { uint32_t v = uint32_t(std::max(value, 0.f)); std::memcpy(px + 4 * ch, &v, 4); break; }
+                }
+            }
+        }
+    return 0;
+}
+
+// WriteChannels from an image of another size.  With verticalFlip the destination row is mirrored
+// before the source position is computed (src/ImageProcessing.cu:36-37).
+int ntc_oracle_write_channels_resized(const uint8_t* src, int format, int verticalFlip, uint64_t pixelStride, uint64_t rowPitch,
+                                      int srcWidth, int srcHeight, uint16_t* planarPairs, int width, int height, int setChannels,
+                                      int firstChannel, int numChannels, const uint8_t* srcColorSpaces, const uint8_t* dstColorSpaces)
+{
+    if (format < 1 || format > 5) return -1;
+    for (int y = 0; y < height; ++y)
+        for (int x = 0; x < width; ++x) {
+            ResampleTaps const t = resample_taps(srcWidth, srcHeight, width, height, x, verticalFlip ? height - 1 - y : y);
+            auto at = [&](int sx, int sy) { return src + size_t(sy) * rowPitch + size_t(sx) * pixelStride; };
+            for (int ch = 0; ch < numChannels; ++ch) {
+                int const space = srcColorSpaces ? srcColorSpaces[ch] : 0;
+                float v = resample_blend(t, decode_color_space(space, user_value(at(t.x0, t.y0), format, ch)), decode_color_space(space, user_value(at(t.x1, t.y0), format, ch)),
+                                            decode_color_space(space, user_value(at(t.x0, t.y1), format, ch)), decode_color_space(space, user_value(at(t.x1, t.y1), format, ch)));
+                v = encode_color_space(dstColorSpaces ? dstColorSpaces[ch] : 0, v);
+                v = std::max(-65504.f, std::min(65504.f, v));
+                int const c = firstChannel + ch;
+                planarPairs[size_t(y) * size_t(width) * size_t(setChannels) + size_t(x) * 2 + size_t(c & ~1) * size_t(width) + size_t(c & 1)] = float_to_half_rne(v);
+            }
+        }
+    return 0;
+}
+
+// ResizeMultichannelImage (src/ImageProcessing.cu:178-218): what GenerateMips runs from mip to mip.
+void ntc_oracle_resize_planar(const uint16_t* src, int srcWidth, int srcHeight, uint16_t* dst, int dstWidth, int dstHeight,
+                              int setChannels, const uint8_t* colorSpaces /* 16 or null */)
+{
+    for (int y = 0; y < dstHeight; ++y)
+        for (int x = 0; x < dstWidth; ++x) {
+            ResampleTaps const t = resample_taps(srcWidth, srcHeight, dstWidth, dstHeight, x, y);
+            for (int c = 0; c < setChannels; ++c) {
+                int const space = colorSpaces ? colorSpaces[c] : 0;
+                float v = resample_blend(t, decode_color_space(space, planar_value(src, srcWidth, setChannels, t.x0, t.y0, c)),
+                                            decode_color_space(space, planar_value(src, srcWidth, setChannels, t.x1, t.y0, c)),
+                                            decode_color_space(space, planar_value(src, srcWidth, setChannels, t.x0, t.y1, c)),
+                                            decode_color_space(space, planar_value(src, srcWidth, setChannels, t.x1, t.y1, c)));
+                v = std::max(-65504.f, std::min(65504.f, encode_color_space(space, v)));
+                dst[size_t(y) * size_t(dstWidth) * size_t(setChannels) + size_t(c & ~1) * size_t(dstWidth) + size_t(x) * 2 + size_t(c & 1)] = float_to_half_rne(v);
+            }
+        }
 }
 
 // Per-channel mean squared error between a decoded mip and its reference, both in the internal

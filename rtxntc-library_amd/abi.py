@@ -75,6 +75,7 @@ class ReadChannels(C.Structure):
         ("dst", C.c_void_p), ("dstBytes", C.c_uint64), ("format", C.c_int32), ("useDithering", C.c_int32),
         ("pixelStride", C.c_uint64), ("rowPitch", C.c_uint64),
         ("srcColorSpaces", C.c_uint8 * 16), ("dstColorSpaces", C.c_uint8 * 16),
+        ("dstWidth", C.c_int32), ("dstHeight", C.c_int32),
     ]
 
 
@@ -85,6 +86,7 @@ class WriteChannels(C.Structure):
         ("width", C.c_int32), ("height", C.c_int32), ("setChannels", C.c_int32), ("firstChannel", C.c_int32),
         ("numChannels", C.c_int32), ("reserved", C.c_int32),
         ("srcColorSpaces", C.c_uint8 * 16), ("dstColorSpaces", C.c_uint8 * 16),
+        ("srcWidth", C.c_int32), ("srcHeight", C.c_int32),
     ]
 
 
@@ -142,6 +144,8 @@ EXPORTS = [
     ("ntc_hip_image_loss", C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64, C.c_int32, C.c_int32, C.c_int32, C.c_uint32, C.c_int32, C.c_int32,
                                      C.POINTER(C.c_float)]),
     ("ntc_hip_image_difference", C.c_int, [C.POINTER(ImageDifference)]),
+    ("ntc_hip_resize_planar", C.c_int, [C.c_void_p, C.c_uint64, C.c_int32, C.c_int32, C.c_void_p, C.c_uint64, C.c_int32, C.c_int32,
+                                        C.c_int32, C.c_void_p]),
     ("ntc_hip_selftest_mfma", C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
     ("ntc_hip_selftest_mfma_f16", C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32]),
 ]

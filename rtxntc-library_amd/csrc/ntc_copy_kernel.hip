@@ -264,6 +264,156 @@ write_channels_kernel(WriteChannelsArgs a)
     }
 }
 
+// ---- resampling copies (src/ImageProcessing.cu:24-72: SetupBilinearFilter) -------------------------
+//
+// The position of destination pixel (x, y) in the source is ((x + 1/2) / dstW) * srcW - 1/2, clamped
+// to the source image; the four taps around it are weighted bilinearly, and a tap whose weight is
+// zero is not used (at the right and bottom edges it would lie outside the image; here its index is
+// clamped and its value dropped).  The blend is a * w0 + b * w1 + c * w2 + d * w3 evaluated as one
+// multiply and three fused multiply-adds, which is what the reference's compiler makes of that
+// expression.  These kernels are general rather than fast: one lane per destination pixel, one
+// channel at a time.
+struct BilinearTaps { int x0, y0, x1, y1; float w[4]; };
+
+__device__ __forceinline__ BilinearTaps setup_bilinear(int srcW, int srcH, int dstW, int dstH, int x, int y)
+{
+    if (srcW == dstW && srcH == dstH) return BilinearTaps{ x, y, x, y, { 1.f, 0.f, 0.f, 0.f } };   // the reference's 1:1 shortcut
+    float const u = (float(x) + 0.5f) / float(dstW), v = (float(y) + 0.5f) / float(dstH);
+    float const px = fmaxf(0.f, fminf(float(srcW) - 1.f, u * float(srcW) - 0.5f));
+    float const py = fmaxf(0.f, fminf(float(srcH) - 1.f, v * float(srcH) - 0.5f));
+    float const fx = px - floorf(px), fy = py - floorf(py);
+    BilinearTaps t;
+    t.x0 = int(floorf(px)); t.y0 = int(floorf(py));
+    t.x1 = min(t.x0 + 1, srcW - 1); t.y1 = min(t.y0 + 1, srcH - 1);
+    t.w[0] = (1.f - fx) * (1.f - fy); t.w[1] = fx * (1.f - fy); t.w[2] = (1.f - fx) * fy; t.w[3] = fx * fy;
+    return t;
+}
+
+__device__ __forceinline__ float blend_taps(BilinearTaps const& t, float a, float b, float c, float d)
+{
+    a = t.w[0] > 0.f ? a : 0.f; b = t.w[1] > 0.f ? b : 0.f; c = t.w[2] > 0.f ? c : 0.f; d = t.w[3] > 0.f ? d : 0.f;
+    return __builtin_fmaf(d, t.w[3], __builtin_fmaf(c, t.w[2], __builtin_fmaf(b, t.w[1], a * t.w[0])));
+}
+
+__device__ __forceinline__ float planar_half(uint16_t const* image, int width, int setChannels, int x, int y, int c)
+{
+    uint16_t const bits = image[size_t(y) * size_t(width) * size_t(setChannels) + size_t(c & ~1) * size_t(width) + size_t(x) * 2 + size_t(c & 1)];
+    return float(__builtin_bit_cast(_Float16, bits));
+}
+
+// Channel `k` of a pixel of the user image, any format and alignment the format allows.
+__device__ __forceinline__ float user_channel(uint8_t const* px, int format, int k)
+{
+    switch (format) {
+    case NTC_HIP_DEV_FORMAT_UNORM8:  return float(px[k]) / 255.f;
+    case NTC_HIP_DEV_FORMAT_UNORM16: return float(reinterpret_cast<uint16_t const*>(px)[k]) / 65535.f;
+    case NTC_HIP_DEV_FORMAT_FLOAT16: return float(reinterpret_cast<_Float16 const*>(px)[k]);
+    case NTC_HIP_DEV_FORMAT_FLOAT32: return reinterpret_cast<float const*>(px)[k];
+    default:                         return float(reinterpret_cast<uint32_t const*>(px)[k]);
+    }
+}
+
+__device__ __forceinline__ uint16_t stored_half(float v)     // WriteImageChannel FLOAT16, src/ImageProcessing.cu:154-156
+{
+    v = fmaxf(-65504.f, fminf(65504.f, v));
+    asm volatile("" : "+v"(v));
+    return __builtin_bit_cast(uint16_t, (_Float16)v);
+}
+
+template <int FORMAT>
+__global__ void __launch_bounds__(256)
+read_channels_resize_kernel(ReadChannelsArgs a)
+{
+    constexpr int BPC = bytes_per_channel(FORMAT);
+    int const x = blockIdx.x * 64 + (threadIdx.x & 63), y = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (x >= a.dstWidth || y >= a.dstHeight) return;
+    BilinearTaps const t = setup_bilinear(a.width, a.height, a.dstWidth, a.dstHeight, x, y);
+    uint8_t* const px = a.dst + size_t(y) * a.rowPitch + size_t(x) * a.pixelStride;
+    DitherRng rng(uint32_t(x) + uint32_t(y) * uint32_t(a.dstWidth));
+    for (int ch = 0; ch < a.dstChannels; ++ch) {
+        float value;
+        if (ch < a.numChannels) {
+            int const c = a.firstChannel + ch, space = a.srcColorSpaces[ch];
+            value = blend_taps(t, decode_color_space(space, planar_half(a.planarPairs, a.width, a.setChannels, t.x0, t.y0, c)),
+                                  decode_color_space(space, planar_half(a.planarPairs, a.width, a.setChannels, t.x1, t.y0, c)),
+                                  decode_color_space(space, planar_half(a.planarPairs, a.width, a.setChannels, t.x0, t.y1, c)),
+                                  decode_color_space(space, planar_half(a.planarPairs, a.width, a.setChannels, t.x1, t.y1, c)));
+        } else {
+            value = (ch == 3) ? 1.f : 0.f;
+        }
+        float const dither = a.useDithering ? rng.next_float() - 0.5f : 0.f;
+        uint32_t const bits = encode_channel<FORMAT>(ch < 16 ? a.dstColorSpaces[ch] : 0, value, a.useDithering != 0, dither);
+        if constexpr (BPC == 1) px[ch] = uint8_t(bits);
+        else if constexpr (BPC == 2) reinterpret_cast<uint16_t*>(px)[ch] = uint16_t(bits);
+        else reinterpret_cast<uint32_t*>(px)[ch] = bits;
+    }
+}
+
+__global__ void __launch_bounds__(256)
+write_channels_resize_kernel(WriteChannelsArgs a)
+{
+    int const x = blockIdx.x * 64 + (threadIdx.x & 63), y = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (x >= a.width || y >= a.height) return;
+    BilinearTaps const t = setup_bilinear(a.srcWidth, a.srcHeight, a.width, a.height, x, a.verticalFlip ? a.height - 1 - y : y);
+    uint8_t const* const p00 = a.src + size_t(t.y0) * a.rowPitch + size_t(t.x0) * a.pixelStride;
+    uint8_t const* const p10 = a.src + size_t(t.y0) * a.rowPitch + size_t(t.x1) * a.pixelStride;
+    uint8_t const* const p01 = a.src + size_t(t.y1) * a.rowPitch + size_t(t.x0) * a.pixelStride;
+    uint8_t const* const p11 = a.src + size_t(t.y1) * a.rowPitch + size_t(t.x1) * a.pixelStride;
+    uint16_t* const dst = a.planarPairs + size_t(y) * size_t(a.width) * size_t(a.setChannels) + size_t(x) * 2;
+    for (int ch = 0; ch < a.numChannels; ++ch) {
+        int const space = a.srcColorSpaces[ch];
+        float const value = blend_taps(t, decode_color_space(space, user_channel(p00, a.format, ch)), decode_color_space(space, user_channel(p10, a.format, ch)),
+                                          decode_color_space(space, user_channel(p01, a.format, ch)), decode_color_space(space, user_channel(p11, a.format, ch)));
+        int const c = a.firstChannel + ch;
+        dst[size_t(c & ~1) * size_t(a.width) + size_t(c & 1)] = stored_half(encode_color_space(a.dstColorSpaces[ch], value));
+    }
+}
+
+// ResizeMultichannelImageKernel (src/ImageProcessing.cu:178-207): every channel of one image of the
+// internal layout resampled into another; a channel pair is read as dwords and written as one.
+struct ResizePlanarArgs {
+    uint16_t const* src; uint16_t* dst;
+    int32_t srcWidth, srcHeight, dstWidth, dstHeight, setChannels;
+    uint8_t colorSpaces[16];
+};
+
+__global__ void __launch_bounds__(256)
+resize_planar_kernel(ResizePlanarArgs a)
+{
+    int const x = blockIdx.x * 64 + (threadIdx.x & 63), y = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (x >= a.dstWidth || y >= a.dstHeight) return;
+    BilinearTaps const t = setup_bilinear(a.srcWidth, a.srcHeight, a.dstWidth, a.dstHeight, x, y);
+    size_t const srcRow = size_t(a.srcWidth) * size_t(a.setChannels), pairStride = size_t(a.srcWidth) * 2;
+    uint16_t const* const r0 = a.src + size_t(t.y0) * srcRow;
+    uint16_t const* const r1 = a.src + size_t(t.y1) * srcRow;
+    uint32_t* const out = reinterpret_cast<uint32_t*>(a.dst + size_t(y) * size_t(a.dstWidth) * size_t(a.setChannels) + size_t(x) * 2);
+    for (int p = 0; p < a.setChannels / 2; ++p) {
+        uint32_t const v00 = *reinterpret_cast<uint32_t const*>(r0 + p * pairStride + size_t(t.x0) * 2);
+        uint32_t const v10 = *reinterpret_cast<uint32_t const*>(r0 + p * pairStride + size_t(t.x1) * 2);
+        uint32_t const v01 = *reinterpret_cast<uint32_t const*>(r1 + p * pairStride + size_t(t.x0) * 2);
+        uint32_t const v11 = *reinterpret_cast<uint32_t const*>(r1 + p * pairStride + size_t(t.x1) * 2);
+        uint32_t packed = 0;
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            int const space = a.colorSpaces[2 * p + k];
+            auto half_of = [&](uint32_t v) { return decode_color_space(space, float(__builtin_bit_cast(_Float16, uint16_t(v >> (16 * k))))); };
+            float const value = blend_taps(t, half_of(v00), half_of(v10), half_of(v01), half_of(v11));
+            packed |= uint32_t(stored_half(encode_color_space(space, value))) << (16 * k);
+        }
+        out[size_t(p) * size_t(a.dstWidth)] = packed;
+    }
+}
+
+hipError_t launch_resize_planar(uint16_t const* src, int srcWidth, int srcHeight, uint16_t* dst, int dstWidth, int dstHeight,
+                                int setChannels, uint8_t const* colorSpaces, hipStream_t stream)
+{
+    ResizePlanarArgs a{};
+    a.src = src; a.dst = dst; a.srcWidth = srcWidth; a.srcHeight = srcHeight; a.dstWidth = dstWidth; a.dstHeight = dstHeight; a.setChannels = setChannels;
+    for (int i = 0; i < 16; ++i) a.colorSpaces[i] = colorSpaces ? colorSpaces[i] : 0;
+    hipLaunchKernelGGL(resize_planar_kernel, dim3((dstWidth + 63) / 64, (dstHeight + 3) / 4), dim3(256), 0, stream, a);
+    return hipGetLastError();
+}
+
 static bool plain_copy(uint8_t const* srcSpaces, uint8_t const* dstSpaces, int useDithering)
 {
     bool plain = useDithering == 0;
@@ -281,6 +431,10 @@ static void launch_write_format(WriteChannelsArgs const& a, dim3 grid, bool plai
 hipError_t launch_write_channels(WriteChannelsArgs const& args, hipStream_t stream)
 {
     WriteChannelsArgs a = args;
+    if (a.srcWidth > 0) {                                    // resampling copy
+        hipLaunchKernelGGL(write_channels_resize_kernel, dim3((a.width + 63) / 64, (a.height + 3) / 4), dim3(256), 0, stream, a);
+        return hipGetLastError();
+    }
     dim3 const grid = copy_grid(a.width, a.height, a.xShift, false);
     bool const plain = plain_copy(a.srcColorSpaces, a.dstColorSpaces, 0);
     switch (a.format) {
@@ -516,6 +670,18 @@ static void launch_read_format(ReadChannelsArgs const& a, dim3 grid, bool plain,
 hipError_t launch_read_channels(ReadChannelsArgs const& args, hipStream_t stream)
 {
     ReadChannelsArgs a = args;
+    if (a.dstWidth > 0) {                                    // resampling copy
+        dim3 const grid((a.dstWidth + 63) / 64, (a.dstHeight + 3) / 4);
+        switch (a.format) {
+        case NTC_HIP_DEV_FORMAT_UNORM8:  hipLaunchKernelGGL(read_channels_resize_kernel<NTC_HIP_DEV_FORMAT_UNORM8>, grid, dim3(256), 0, stream, a); break;
+        case NTC_HIP_DEV_FORMAT_UNORM16: hipLaunchKernelGGL(read_channels_resize_kernel<NTC_HIP_DEV_FORMAT_UNORM16>, grid, dim3(256), 0, stream, a); break;
+        case NTC_HIP_DEV_FORMAT_FLOAT16: hipLaunchKernelGGL(read_channels_resize_kernel<NTC_HIP_DEV_FORMAT_FLOAT16>, grid, dim3(256), 0, stream, a); break;
+        case NTC_HIP_DEV_FORMAT_FLOAT32: hipLaunchKernelGGL(read_channels_resize_kernel<NTC_HIP_DEV_FORMAT_FLOAT32>, grid, dim3(256), 0, stream, a); break;
+        case NTC_HIP_DEV_FORMAT_UINT32:  hipLaunchKernelGGL(read_channels_resize_kernel<NTC_HIP_DEV_FORMAT_UINT32>, grid, dim3(256), 0, stream, a); break;
+        default: return hipErrorInvalidValue;
+        }
+        return hipGetLastError();
+    }
     dim3 const grid = copy_grid(a.width, a.height, a.xShift);
     bool const plain = plain_copy(a.srcColorSpaces, a.dstColorSpaces, a.useDithering);
     switch (a.format) {

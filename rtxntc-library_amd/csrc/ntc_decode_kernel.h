@@ -63,6 +63,7 @@ struct ReadChannelsArgs {
     int32_t useDithering;
     int32_t vectorBytes;           // widest store every pixel start is aligned to: 16, 8, 4, 2 or 1
     int32_t xShift;                // set by the launcher: log2 of the pixels of a row one workgroup covers
+    int32_t dstWidth, dstHeight;   // size of the user image when it differs from the mip's (resampling copy), else 0
     uint8_t srcColorSpaces[16], dstColorSpaces[16];   // per copied channel: 0 linear, 1 sRGB, 2 HLG
 };
 hipError_t launch_read_channels(ReadChannelsArgs const& args, hipStream_t stream);
@@ -76,6 +77,7 @@ struct WriteChannelsArgs {
     int32_t width, height, setChannels, firstChannel, numChannels, format, verticalFlip;
     int32_t vectorBytes;           // widest load every pixel start is aligned to
     int32_t xShift;                // set by the launcher
+    int32_t srcWidth, srcHeight;   // size of the user image when it differs from the mip's (resampling copy), else 0
     uint8_t srcColorSpaces[16], dstColorSpaces[16];
 };
 hipError_t launch_write_channels(WriteChannelsArgs const& args, hipStream_t stream);
@@ -95,6 +97,9 @@ inline size_t image_loss_blocks(int width, int height)
 }
 hipError_t launch_image_loss(uint16_t* a, uint16_t const* b, int width, int height, int setChannels,
                              uint32_t validChannelMask, int maskChannel, int discardMaskedOut, double* partials, hipStream_t stream);
+
+hipError_t launch_resize_planar(uint16_t const* src, int srcWidth, int srcHeight, uint16_t* dst, int dstWidth, int dstHeight,
+                                int setChannels, uint8_t const* colorSpaces, hipStream_t stream);
 
 struct DiffImageArgs {
     uint8_t const* data;

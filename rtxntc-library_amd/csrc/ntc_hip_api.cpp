@@ -551,14 +551,20 @@ int ntc_hip_read_channels(const NtcHipReadChannels* p)
         set_error("ntc_hip_read_channels: bad image or channel range.");
         return NTC_HIP_ERR_INVALID_ARG;
     }
-    if (p->pixelStride < uint64_t(bpc) || p->rowPitch < p->pixelStride * uint64_t(p->width)
+    if ((p->dstWidth == 0) != (p->dstHeight == 0) || p->dstWidth < 0 || p->dstHeight < 0) {
+        set_error("ntc_hip_read_channels: dstWidth and dstHeight must both be positive, or both 0 for the mip's size.");
+        return NTC_HIP_ERR_INVALID_ARG;
+    }
+    bool const resample = p->dstWidth > 0 && (p->dstWidth != p->width || p->dstHeight != p->height);
+    int const imageWidth = resample ? p->dstWidth : p->width, imageHeight = resample ? p->dstHeight : p->height;
+    if (p->pixelStride < uint64_t(bpc) || p->rowPitch < p->pixelStride * uint64_t(imageWidth)
         || (p->pixelStride % uint64_t(bpc)) || (p->rowPitch % uint64_t(bpc)) || (reinterpret_cast<uintptr_t>(p->dst) % uintptr_t(bpc))) {
         set_error("ntc_hip_read_channels: pixel stride / row pitch do not fit the format.");
         return NTC_HIP_ERR_INVALID_ARG;
     }
     uint64_t const dstChannels = p->pixelStride / uint64_t(bpc);
     if (dstChannels > 64) { set_error("ntc_hip_read_channels: pixel stride too large."); return NTC_HIP_ERR_INVALID_ARG; }
-    uint64_t const need = uint64_t(p->height - 1) * p->rowPitch + uint64_t(p->width) * p->pixelStride;
+    uint64_t const need = uint64_t(imageHeight - 1) * p->rowPitch + uint64_t(imageWidth) * p->pixelStride;
     uint64_t const srcNeed = uint64_t(p->width) * uint64_t(p->height) * uint64_t(p->setChannels) * 2u;
     if (need > p->dstBytes || srcNeed > p->planarBytes) {
         set_error("ntc_hip_read_channels: image reaches past the given buffer sizes.");
@@ -573,6 +579,7 @@ int ntc_hip_read_channels(const NtcHipReadChannels* p)
     a.dstChannels = int32_t(dstChannels); a.format = p->format;
     a.useDithering = p->useDithering ? 1 : 0;
     a.vectorBytes = common_alignment(reinterpret_cast<uintptr_t>(p->dst), p->rowPitch, p->pixelStride);
+    a.dstWidth = resample ? p->dstWidth : 0; a.dstHeight = resample ? p->dstHeight : 0;
     for (int i = 0; i < 16; ++i) {
         if (p->srcColorSpaces[i] > 2 || p->dstColorSpaces[i] > 2) { set_error("ntc_hip_read_channels: unknown colour space for channel %d.", i); return NTC_HIP_ERR_INVALID_ARG; }
         a.srcColorSpaces[i] = p->srcColorSpaces[i];
@@ -604,12 +611,18 @@ int ntc_hip_write_channels(const NtcHipWriteChannels* p)
         set_error("ntc_hip_write_channels: bad image or channel range.");
         return NTC_HIP_ERR_INVALID_ARG;
     }
-    if (p->pixelStride < uint64_t(bpc) * uint64_t(p->numChannels) || p->rowPitch < p->pixelStride * uint64_t(p->width)
+    if ((p->srcWidth == 0) != (p->srcHeight == 0) || p->srcWidth < 0 || p->srcHeight < 0) {
+        set_error("ntc_hip_write_channels: srcWidth and srcHeight must both be positive, or both 0 for the mip's size.");
+        return NTC_HIP_ERR_INVALID_ARG;
+    }
+    bool const resample = p->srcWidth > 0 && (p->srcWidth != p->width || p->srcHeight != p->height);
+    int const imageWidth = resample ? p->srcWidth : p->width, imageHeight = resample ? p->srcHeight : p->height;
+    if (p->pixelStride < uint64_t(bpc) * uint64_t(p->numChannels) || p->rowPitch < p->pixelStride * uint64_t(imageWidth)
         || (p->pixelStride % uint64_t(bpc)) || (p->rowPitch % uint64_t(bpc)) || (reinterpret_cast<uintptr_t>(p->src) % uintptr_t(bpc))) {
         set_error("ntc_hip_write_channels: pixel stride / row pitch do not fit the format and channel count.");
         return NTC_HIP_ERR_INVALID_ARG;
     }
-    uint64_t const srcNeed = uint64_t(p->height - 1) * p->rowPitch + uint64_t(p->width - 1) * p->pixelStride + uint64_t(bpc) * uint64_t(p->numChannels);
+    uint64_t const srcNeed = uint64_t(imageHeight - 1) * p->rowPitch + uint64_t(imageWidth - 1) * p->pixelStride + uint64_t(bpc) * uint64_t(p->numChannels);
     uint64_t const dstNeed = uint64_t(p->width) * uint64_t(p->height) * uint64_t(p->setChannels) * 2u;
     if (srcNeed > p->srcBytes || dstNeed > p->planarBytes) { set_error("ntc_hip_write_channels: image reaches past the given buffer sizes."); return NTC_HIP_ERR_INVALID_ARG; }
     WriteChannelsArgs a{};
@@ -619,6 +632,7 @@ int ntc_hip_write_channels(const NtcHipWriteChannels* p)
     a.width = p->width; a.height = p->height; a.setChannels = p->setChannels;
     a.firstChannel = p->firstChannel; a.numChannels = p->numChannels; a.format = p->format; a.verticalFlip = p->verticalFlip ? 1 : 0;
     a.vectorBytes = common_alignment(reinterpret_cast<uintptr_t>(p->src), p->rowPitch, p->pixelStride);
+    a.srcWidth = resample ? p->srcWidth : 0; a.srcHeight = resample ? p->srcHeight : 0;
     for (int i = 0; i < 16; ++i) {
         if (p->srcColorSpaces[i] > 2 || p->dstColorSpaces[i] > 2) { set_error("ntc_hip_write_channels: unknown colour space for channel %d.", i); return NTC_HIP_ERR_INVALID_ARG; }
         a.srcColorSpaces[i] = p->srcColorSpaces[i];
@@ -671,6 +685,31 @@ int ntc_hip_image_loss(void* decoded, const void* reference, uint64_t planarByte
     HIP_TRY(hipStreamSynchronize(L.stream));
     double const norm = 1.0 / (double(width) * double(height));
     for (int c = 0; c < NTC_HIP_DEV_MAX_CHANNELS; ++c) outMse[c] = float(L.lossHost[c] * norm);
+    clear_error();
+    return 0;
+}
+
+int ntc_hip_resize_planar(const void* src, uint64_t srcBytes, int32_t srcWidth, int32_t srcHeight,
+                          void* dst, uint64_t dstBytes, int32_t dstWidth, int32_t dstHeight,
+                          int32_t setChannels, const uint8_t* channelColorSpaces)
+{
+    if (int r = require_init()) return r;
+    if (!src || !dst) { set_error("ntc_hip_resize_planar: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
+    if (srcWidth < 1 || srcHeight < 1 || dstWidth < 1 || dstHeight < 1 || setChannels < 2 || (setChannels & 1) || setChannels > NTC_HIP_MAX_CHANNELS) {
+        set_error("ntc_hip_resize_planar: bad image shape.");
+        return NTC_HIP_ERR_INVALID_ARG;
+    }
+    uint64_t const srcNeed = uint64_t(srcWidth) * uint64_t(srcHeight) * uint64_t(setChannels) * 2u;
+    uint64_t const dstNeed = uint64_t(dstWidth) * uint64_t(dstHeight) * uint64_t(setChannels) * 2u;
+    if (srcNeed > srcBytes || dstNeed > dstBytes) { set_error("ntc_hip_resize_planar: image reaches past the given buffer sizes."); return NTC_HIP_ERR_INVALID_ARG; }
+    uintptr_t const s = reinterpret_cast<uintptr_t>(src), d = reinterpret_cast<uintptr_t>(dst);
+    if (s < d + dstNeed && d < s + srcNeed) { set_error("ntc_hip_resize_planar: source and destination overlap."); return NTC_HIP_ERR_INVALID_ARG; }
+    if ((s | d) & 3u) { set_error("ntc_hip_resize_planar: images must be 4-byte aligned."); return NTC_HIP_ERR_INVALID_ARG; }
+    if (channelColorSpaces)
+        for (int i = 0; i < 16; ++i)
+            if (channelColorSpaces[i] > 2) { set_error("ntc_hip_resize_planar: unknown colour space for channel %d.", i); return NTC_HIP_ERR_INVALID_ARG; }
+    HIP_TRY(launch_resize_planar(static_cast<uint16_t const*>(src), srcWidth, srcHeight, static_cast<uint16_t*>(dst), dstWidth, dstHeight,
+                                 setChannels, channelColorSpaces, g_lib.stream));
     clear_error();
     return 0;
 }

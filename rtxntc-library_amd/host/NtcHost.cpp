@@ -793,6 +793,7 @@ public:
         wc.planarPairs = static_cast<uint8_t*>(m_textureData) + offset;               // the reference page
         wc.planarBytes = m_textureBytes - offset;
         wc.width = mipWidth; wc.height = mipHeight; wc.setChannels = m_desc.channels;
+        wc.srcWidth = params.width; wc.srcHeight = params.height;               // another size: resampled (src/ImageProcessing.cu:24-72)
         wc.firstChannel = params.firstChannel; wc.numChannels = params.numChannels;
         for (int channel = 0; channel < params.numChannels; ++channel) {
             ColorSpace const source = params.srcColorSpaces ? params.srcColorSpaces[channel] : ColorSpace::Linear;
@@ -829,6 +830,7 @@ public:
         rc.planarPairs = static_cast<uint8_t const*>(page) + m_mipOffsets[params.mipLevel] * uint64_t(m_desc.channels) * 2u;
         rc.planarBytes = uint64_t(mipWidth) * uint64_t(mipHeight) * uint64_t(m_desc.channels) * 2u;
         rc.width = mipWidth; rc.height = mipHeight;
+        rc.dstWidth = params.width; rc.dstHeight = params.height;               // another size: resampled
         rc.setChannels = m_desc.channels;
         rc.firstChannel = params.firstChannel; rc.numChannels = params.numChannels;
         rc.dst = toHost ? m_staging : params.pOutData;
@@ -849,8 +851,28 @@ public:
         return Status::Ok;
     }
 
+    // src/TextureSet.cpp:1121-1142: every mip of the reference page from the one above it, through the
+    // storage colour spaces of the channels; a 2x reduction is a 2x2 box filter.
+    Status GenerateMips() override
+    {
+        if (m_desc.mips <= 1) { ClearErrorMessage(); return Status::Ok; }
+        if (!m_deviceAvailable) { SetErrorMessage("No HIP device is available to this context."); return Status::CudaUnavailable; }
+        uint8_t spaces[NTC_HIP_MAX_CHANNELS];
+        for (int ch = 0; ch < NTC_HIP_MAX_CHANNELS; ++ch) spaces[ch] = uint8_t(m_channelColorSpaces[ch]);
+        for (int mip = 1; mip < m_desc.mips; ++mip) {
+            uint64_t const srcOffset = m_mipOffsets[mip - 1] * uint64_t(m_desc.channels) * 2u, dstOffset = m_mipOffsets[mip] * uint64_t(m_desc.channels) * 2u;
+            if (int r = ntc_hip_resize_planar(static_cast<uint8_t const*>(m_textureData) + srcOffset, dstOffset - srcOffset,
+                                              std::max(m_desc.width >> (mip - 1), 1), std::max(m_desc.height >> (mip - 1), 1),
+                                              static_cast<uint8_t*>(m_textureData) + dstOffset, m_textureBytes - dstOffset,
+                                              std::max(m_desc.width >> mip, 1), std::max(m_desc.height >> mip, 1), m_desc.channels, spaces))
+                return DeviceFailure(r);
+        }
+        ClearErrorMessage();
+        return Status::Ok;
+    }
+
 private:
-    // src/TextureSet.cpp:1914-1956, plus what this library cannot do (resizing copies)
+    // src/TextureSet.cpp:1914-1956
     Status ValidateReadWriteChannelsArgs(int mipLevel, int firstChannel, int numChannels, int width, int height,
         size_t pixelStride, size_t rowPitch, size_t stagedBytes, ChannelFormat format, char const* what)
     {
@@ -880,12 +902,7 @@ private:
                 "the staging buffer (%zu bytes).", stagedBytes, size_t(m_stagingBytes));
             return Status::OutOfRange;
         }
-        if (GetBytesPerPixelComponent(format) == 0) { SetErrorMessage("Unknown channel format %d.", int(format)); return Status::InvalidArgument; }
-        int const mipWidth = std::max(m_desc.width >> mipLevel, 1), mipHeight = std::max(m_desc.height >> mipLevel, 1);
-        if (width != mipWidth || height != mipHeight) {
-            SetErrorMessage("Resizing %s are not supported: the image must be %dx%d for mip %d.", what, mipWidth, mipHeight, mipLevel);
-            return Status::Unsupported;
-        }
+        if (GetBytesPerPixelComponent(format) == 0) { SetErrorMessage("Unknown channel format %d for %s.", int(format), what); return Status::InvalidArgument; }
         return Status::Ok;
     }
 

@@ -280,8 +280,13 @@ public:
     // Decompress measures its loss against.
     virtual Status WriteChannels(WriteChannelsParameters const& params) = 0;
 
-    // include/libntc/ntc.h:902, src/TextureSet.cpp:915-985.
+    // include/libntc/ntc.h:902, src/TextureSet.cpp:915-985.  As in WriteChannels, an image whose size
+    // differs from the mip's is resampled bilinearly (src/ImageProcessing.cu:24-72).
     virtual Status ReadChannels(ReadChannelsParameters const& params) = 0;
+
+    // Fills mips 1.. of the reference page from mip 0 with a 2x2 box filter (include/libntc/ntc.h:910-912,
+    // src/TextureSet.cpp:1121-1142).
+    virtual Status GenerateMips() = 0;
 
     // Index of the channel that holds an alpha mask; negative = none (include/libntc/ntc.h:936-940,
     // src/TextureSet.cpp:1899-1907).  Decompress then clamps the decoded mask channel to [0, 1] when

@@ -12,6 +12,8 @@
 //   host_api_test shuffle <preset> <w> <h> <channels> <gridScale> <features> <latents> <weights>
 //       ShuffleInferenceOutputs / GetInferenceWeights: decodes with the loaded weights, shuffles, decodes
 //       again with the weights GetInferenceWeights returns and compares the channels
+//   host_api_test genmips <w> <h> <channels> <mips> <image> <outPrefix>
+//       WriteChannels from an image of twice the size, GenerateMips, reference page of every mip to files
 //   host_api_test imagediff
 //       IContext::ComputeImageDifference on images with exactly known differences
 //   host_api_test load <file> <device 0|1> [<w> <h> <channels> <mips>]
@@ -253,12 +255,15 @@ static int decode(int argc, char** argv)
         CHECK(set->ReadChannels(rp) == Status::Ok);
         CHECK(writeFile(prefix + "_srgb_dither.bin", u8.data(), u8.size()));
     }
-    // a resizing read is refused, not silently approximated
-    ReadChannelsParameters bad;
-    std::vector<unsigned char> tmp(64);
-    bad.pOutData = tmp.data(); bad.numChannels = 1; bad.width = 2; bad.height = 2; bad.pixelStride = 1; bad.rowPitch = 2;
-    bad.channelFormat = ChannelFormat::UNORM8;
-    if (w != 2 || h != 2) CHECK(set->ReadChannels(bad) == Status::Unsupported);
+    // a read at another size resamples mip 0 (here: down to 2 x 2, channel 0)
+    {
+        ReadChannelsParameters small;
+        std::vector<unsigned char> tmp(64, 0xEE);
+        small.pOutData = tmp.data(); small.numChannels = 1; small.width = 2; small.height = 2; small.pixelStride = 1; small.rowPitch = 2;
+        small.channelFormat = ChannelFormat::UNORM8;
+        CHECK(set->ReadChannels(small) == Status::Ok);
+        CHECK(writeFile(prefix + "_2x2.bin", tmp.data(), 4));
+    }
     ctx->DestroyTextureSet(set);
     DestroyContext(ctx);
     std::printf("host decode OK, gpu %.3f ms\n", stats.gpuTimeMilliseconds);
@@ -419,6 +424,50 @@ static int imageDifference()
     CHECK(ntc_hip_free(dA) == 0 && ntc_hip_free(dB) == 0 && ntc_hip_free(dOut) == 0);
     DestroyContext(ctx);
     std::printf("host image difference OK\n");
+    return 0;
+}
+
+// WriteChannels at twice the size of mip 0 (resampled down), GenerateMips, then every mip of the
+// reference page read back as FLOAT16 pixels into <prefix>_mip<N>.bin for the test to compare.
+static int generateMips(int argc, char** argv)
+{
+    if (argc < 8) { std::fprintf(stderr, "usage: genmips <w> <h> <channels> <mips> <image(FLOAT32 pixels, 2w x 2h)> <outPrefix>\n"); return 2; }
+    int const w = std::atoi(argv[2]), h = std::atoi(argv[3]), channels = std::atoi(argv[4]), mips = std::atoi(argv[5]);
+    std::vector<unsigned char> image = readFile(argv[6]);
+    std::string const prefix = argv[7];
+    IContext* ctx = nullptr;
+    ContextParameters params;
+    CHECK(CreateContext(&ctx, params) == Status::Ok);
+    TextureSetDesc desc; desc.width = w; desc.height = h; desc.channels = channels; desc.mips = mips;
+    TextureSetFeatures features_;
+    features_.stagingBytesPerPixel = 16 * 4; features_.stagingWidth = 2 * w; features_.stagingHeight = 2 * h;
+    ITextureSet* set = nullptr;
+    CHECK(ctx->CreateTextureSet(desc, features_, &set) == Status::Ok);
+    int const C = set->GetDesc().channels;
+    CHECK(image.size() == size_t(2 * w) * size_t(2 * h) * size_t(C) * 4);
+    ColorSpace source[16], storage[16];
+    for (int c = 0; c < 16; ++c) { source[c] = ColorSpace::Linear; storage[c] = c == 1 ? ColorSpace::sRGB : ColorSpace::Linear; }
+    WriteChannelsParameters wp;
+    wp.mipLevel = 0; wp.firstChannel = 0; wp.numChannels = C; wp.pData = image.data();
+    wp.width = 2 * w; wp.height = 2 * h; wp.pixelStride = size_t(C) * 4; wp.rowPitch = wp.pixelStride * size_t(2 * w);
+    wp.channelFormat = ChannelFormat::FLOAT32; wp.srcColorSpaces = source; wp.dstColorSpaces = storage;
+    CHECK(set->WriteChannels(wp) == Status::Ok);
+    CHECK(set->GenerateMips() == Status::Ok);
+    for (int mip = 0; mip < mips; ++mip) {
+        int const mw = std::max(w >> mip, 1), mh = std::max(h >> mip, 1);
+        ReadChannelsParameters rp;
+        rp.page = TextureDataPage::Reference;
+        rp.mipLevel = mip; rp.firstChannel = 0; rp.numChannels = C; rp.width = mw; rp.height = mh;
+        rp.pixelStride = size_t(C) * 2; rp.rowPitch = rp.pixelStride * size_t(mw); rp.channelFormat = ChannelFormat::FLOAT16;
+        rp.dstColorSpaces = storage;                         // read the stored values as they are
+        std::vector<unsigned char> out(rp.rowPitch * size_t(mh));
+        rp.pOutData = out.data();
+        CHECK(set->ReadChannels(rp) == Status::Ok);
+        CHECK(writeFile(prefix + "_mip" + std::to_string(mip) + ".bin", out.data(), out.size()));
+    }
+    ctx->DestroyTextureSet(set);
+    DestroyContext(ctx);
+    std::printf("host genmips OK\n");
     return 0;
 }
 
@@ -600,6 +649,7 @@ int main(int argc, char** argv)
     if (argc >= 2 && std::strcmp(argv[1], "loss") == 0) return loss(argc, argv);
     if (argc >= 2 && std::strcmp(argv[1], "shuffle") == 0) return shuffle(argc, argv);
     if (argc >= 2 && std::strcmp(argv[1], "imagediff") == 0) return imageDifference();
+    if (argc >= 2 && std::strcmp(argv[1], "genmips") == 0) return generateMips(argc, argv);
     if (argc >= 2 && std::strcmp(argv[1], "cpu") == 0) return cpuChecks();
     if (argc >= 2 && std::strcmp(argv[1], "decode") == 0) return decode(argc, argv);
     std::fprintf(stderr, "usage: host_api_test cpu | decode ...\n");

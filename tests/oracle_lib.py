@@ -68,6 +68,14 @@ def load_oracle():
         lib.ntc_oracle_dither_float.argtypes = [C.c_uint32, C.c_int]
         lib.ntc_oracle_image_loss.restype = None
         lib.ntc_oracle_image_loss.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_uint32, C.c_void_p]
+        lib.ntc_oracle_read_channels_resized.restype = C.c_int
+        lib.ntc_oracle_read_channels_resized.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int,
+                                                         C.c_uint64, C.c_uint64, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+        lib.ntc_oracle_write_channels_resized.restype = C.c_int
+        lib.ntc_oracle_write_channels_resized.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_uint64, C.c_uint64, C.c_int, C.c_int, C.c_void_p,
+                                                          C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+        lib.ntc_oracle_resize_planar.restype = None
+        lib.ntc_oracle_resize_planar.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]
         lib.ntc_oracle_image_difference.restype = None
         lib.ntc_oracle_image_difference.argtypes = [C.c_void_p, C.c_void_p]
         lib.ntc_oracle_image_loss_masked.restype = None
