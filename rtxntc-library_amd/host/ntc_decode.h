@@ -367,6 +367,13 @@ extern "C" {
 // outputTransforms (optional) holds one entry per output channel.
 Status QuantizeNetworkInt8(FloatLayerDesc const* layers, int numLayers, OutputChannelTransform const* outputTransforms,
     void* pOutBlob, size_t blobSize, size_t* pOutSize);
+// The same network as the GenericFP8 blob (src/WeightLayout.cpp:51-71): e4m3 weights and fp16 biases
+// for the hidden layers (src/Quantizer.cu:210-252), the Int8 output layer.  The decoder of this
+// library does not consume that blob; it is what LibNTC stores as the second MLP version of a file.
+Status QuantizeNetworkFP8(FloatLayerDesc const* layers, int numLayers, OutputChannelTransform const* outputTransforms,
+    void* pOutBlob, size_t blobSize, size_t* pOutSize);
+// IEEE half bits -> OCP e4m3 byte: round to nearest even, saturating at +-448, NaN -> 0x7F | sign.
+uint8_t HalfToE4M3(uint16_t halfBits);
 
 // include/libntc/ntc.h:1307-1331.  CreateContext returns CudaUnavailable together with a usable
 // context when no device can be used (src/PublicFunctions.cpp:161).

@@ -222,3 +222,84 @@ def test_gpu_decode_with_a_quantised_float_network(ntc, device, preset):
     device.decode([dset])
     device.synchronize()
     assert first_mismatch(host.output, case.d_output.download()) is None
+
+
+def test_half_to_e4m3_is_round_to_nearest_even_saturating(oracle):
+    """Every half against the textbook statement: the nearest of the 253 distinct finite e4m3 values
+    (decoded by the checker's table, itself pinned against the OCP definition), ties to the even
+    code, magnitudes from 448 up and infinities to +-448, NaN to the NaN code."""
+    lib = host_lib()
+    lib.HalfToE4M3.restype = C.c_uint8
+    lib.HalfToE4M3.argtypes = [C.c_uint16]
+    codes = np.arange(0x7F, dtype=np.int64)                                  # 0x00 .. 0x7E: non-negative finite codes, ascending
+    values = np.array([oracle.ntc_oracle_e4m3_times_512(int(c)) for c in codes], dtype=np.float64) / 512.0
+    assert np.all(np.diff(values) > 0) and values[-1] == 448.0
+    halves = np.arange(0x7C01, dtype=np.uint16)                              # 0 .. +inf
+    x = halves.view(np.float16).astype(np.float64)
+    hi = np.clip(np.searchsorted(values, x, side="left"), 0, len(values) - 1)   # first code with value >= x
+    lo = np.clip(hi - 1, 0, len(values) - 1)
+    d_lo, d_hi = np.abs(x - values[lo]), np.abs(values[hi] - x)
+    want = np.where(d_lo < d_hi, lo, np.where(d_hi < d_lo, hi, np.where(lo % 2 == 0, lo, hi)))
+    want = np.where(x >= 448.0, 0x7E, want)
+    got = np.array([lib.HalfToE4M3(int(h)) for h in halves], dtype=np.int64)
+    assert np.array_equal(got, want), np.flatnonzero(got != want)[:10]
+    # sign symmetry, NaN
+    for h in (0x0001, 0x1400, 0x3C00, 0x5EFF, 0x5F00, 0x7BFF, 0x7C00):
+        assert lib.HalfToE4M3(h | 0x8000) == (lib.HalfToE4M3(h) | 0x80)
+    assert lib.HalfToE4M3(0x7E00) == 0x7F and lib.HalfToE4M3(0xFE00) == 0xFF
+
+
+@pytest.mark.parametrize("widths", [(48, 64, 48, 32, 16), (64, 64, 48, 32, 16)])
+def test_host_fp8_quantiser_blob(widths, oracle):
+    """GenericFP8 blob: e4m3 weights + fp16 biases for the hidden layers, the Int8 blob's output layer;
+    layout sizes against the reference's own WeightLayout (oracle/_ref) for the 48-64-48-32-16 network."""
+    import oracle_lib
+    lib = host_lib()
+    lib.QuantizeNetworkFP8.restype = C.c_int
+    lib.QuantizeNetworkFP8.argtypes = lib.QuantizeNetworkInt8.argtypes
+    lib.HalfToE4M3.restype = C.c_uint8
+    lib.HalfToE4M3.argtypes = [C.c_uint16]
+    rng = np.random.default_rng(sum(widths) + 1)
+    layers = float_network(rng, widths)
+    layers[1][0][0, :4] = [500.0, -1000.0, 447.9, 2.0 ** -11]               # saturation and underflow
+    int8_blob = quantize_with_host_library(lib, layers)
+    descs = (FloatLayerDesc * 4)()
+    keep = []
+    for d, (w, b) in zip(descs, layers):
+        wt = np.ascontiguousarray(w.T, dtype=np.float32)
+        bb = np.ascontiguousarray(b, dtype=np.float32)
+        keep += [wt, bb]
+        d.inputChannels, d.outputChannels, d.weights, d.bias = w.shape[0], w.shape[1], wt.ctypes.data, bb.ctypes.data
+    size = C.c_size_t()
+    assert lib.QuantizeNetworkFP8(descs, 4, None, None, 0, size) == 10       # InvalidArgument: no blob, but the size is reported
+    weight_bytes = sum(a * b for a, b in zip(widths[:-1], widths[1:]))
+    hidden = sum(widths[1:-1])
+    assert size.value == weight_bytes + 2 * hidden + 8 * widths[-1]
+    ref = oracle_lib.load_ref()
+    if ref is not None and widths[0] == 48:
+        out = (C.c_uint64 * 16)()
+        assert ref.ntc_ref_weight_layout(2, out) == 0                        # InferenceWeightType::GenericFP8
+        assert size.value == out[12] == 8608
+    blob = np.zeros(size.value, dtype=np.uint8)
+    assert lib.QuantizeNetworkFP8(descs, 4, None, blob.ctypes.data, blob.size, None) == 0, lib.GetLastErrorMessage()
+    w_at, b_at = 0, weight_bytes
+    for index, (w, b) in enumerate(layers[:-1]):
+        n_in, n_out = w.shape
+        halves = np.ascontiguousarray(w.T).astype(np.float16).view(np.uint16).reshape(-1)
+        want = np.array([lib.HalfToE4M3(int(h)) for h in halves], dtype=np.uint8)
+        assert np.array_equal(blob[w_at: w_at + n_in * n_out], want), index
+        # and what the bytes mean: within half an e4m3 step of the weight (relative 1/16 for normal values)
+        decoded = np.array([oracle.ntc_oracle_e4m3_times_512(int(c)) for c in want], dtype=np.float64) / 512.0
+        exact = np.clip(np.ascontiguousarray(w.T).reshape(-1).astype(np.float64), -448, 448)
+        assert np.all(np.abs(decoded - exact) <= np.maximum(np.abs(exact) / 16, 2.0 ** -10) + 1e-12), index
+        assert np.array_equal(blob[b_at: b_at + 2 * n_out].view(np.float16), b.astype(np.float16)), index
+        w_at += n_in * n_out
+        b_at += 2 * n_out
+    # output layer: the Int8 blob's weights, scales and biases
+    n_in, n_out = layers[-1][0].shape
+    channels = sum(widths[1:])
+    assert np.array_equal(blob[w_at: w_at + n_in * n_out], int8_blob[w_at: w_at + n_in * n_out])
+    int8_scales = int8_blob[weight_bytes + 4 * (channels - n_out): weight_bytes + 4 * channels]
+    int8_biases = int8_blob[weight_bytes + 4 * channels + 4 * (channels - n_out):]
+    assert np.array_equal(blob[b_at: b_at + 4 * n_out], int8_scales)
+    assert np.array_equal(blob[b_at + 4 * n_out:], int8_biases)
