@@ -277,7 +277,7 @@ def test_host_fp8_quantiser_blob(widths, oracle):
     assert size.value == weight_bytes + 2 * hidden + 8 * widths[-1]
     ref = oracle_lib.load_ref()
     if ref is not None and widths[0] == 48:
-        out = (C.c_uint64 * 16)()
+        out = (C.c_uint64 * 25)()
         assert ref.ntc_ref_weight_layout(2, out) == 0                        # InferenceWeightType::GenericFP8
         assert size.value == out[12] == 8608
     blob = np.zeros(size.value, dtype=np.uint8)
