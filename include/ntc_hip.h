@@ -137,6 +137,8 @@ typedef struct NtcHipTextureSet {
     uint64_t weightsBytes;           /* mip's output extent are checked against them before launch */
     uint64_t outputBytes;
     NtcHipMipDesc mips[NTC_HIP_MAX_MIPS];
+    const void* queryLatents;        /* device, optional: the grids once more in query order, see      */
+    uint64_t queryLatentsBytes;      /* ntc_hip_build_query_latents; used by ntc_hip_decode_queries only */
 } NtcHipTextureSet;
 
 /* ---- library / device ------------------------------------------------------------ */
@@ -190,6 +192,19 @@ int ntc_hip_decode_queries(const NtcHipTextureSet* set, const NtcHipQuery* queri
 int ntc_hip_decode_queries_timed(const NtcHipTextureSet* set, const NtcHipQuery* queries, uint64_t numQueries,
                                  void* out, uint64_t outBytes, int32_t iterations,
                                  float* outMillisecondsPerIteration);
+
+/* A second copy of a set's latent grids laid out for scattered sample points.  In the file layout a
+ * grid is ceil(features/4) separate layers, so the 2 x 2 cells a sample point needs lie in 8 different
+ * cache lines per grid; here a grid is cut into bricks of 4 x 4 cells (8 x 8 for one-layer grids) that
+ * hold all layers of their cells together, [cell row][cell column][layer], one 128-byte line per brick
+ * for four layers, and a sample point touches 1.6 lines per grid on average.  No reference counterpart
+ * (the reference samples a hardware texture there, Inference.hlsli:62-87).
+ * ntc_hip_query_latents_bytes: size of that copy for the set's geometry (0 on a malformed set).
+ * ntc_hip_build_query_latents: fills dst (device, 128-byte aligned) from set->latents; asynchronous on
+ * the library stream.  Put dst into set->queryLatents / queryLatentsBytes for ntc_hip_decode_queries;
+ * results are the same bits with or without it. */
+uint64_t ntc_hip_query_latents_bytes(const NtcHipTextureSet* set);
+int ntc_hip_build_query_latents(const NtcHipTextureSet* set, void* dst, uint64_t dstBytes);
 
 /* Extracts channels of one decoded mip from the internal fp16 layout into a user image:
  * what ITextureSet::ReadChannels does through cuda::CopyImage (src/TextureSet.cpp:915-985,

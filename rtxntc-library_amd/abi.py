@@ -65,6 +65,7 @@ class TextureSet(C.Structure):
         ("latents", C.c_void_p), ("weights", C.c_void_p), ("output", C.c_void_p),
         ("latentsBytes", C.c_uint64), ("weightsBytes", C.c_uint64), ("outputBytes", C.c_uint64),
         ("mips", MipDesc * MAX_MIPS),
+        ("queryLatents", C.c_void_p), ("queryLatentsBytes", C.c_uint64),
     ]
 
 
@@ -139,6 +140,8 @@ EXPORTS = [
     ("ntc_hip_decode_queries", C.c_int, [C.POINTER(TextureSet), C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint64]),
     ("ntc_hip_decode_queries_timed", C.c_int, [C.POINTER(TextureSet), C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint64,
                                                C.c_int32, C.POINTER(C.c_float)]),
+    ("ntc_hip_query_latents_bytes", C.c_uint64, [C.POINTER(TextureSet)]),
+    ("ntc_hip_build_query_latents", C.c_int, [C.POINTER(TextureSet), C.c_void_p, C.c_uint64]),
     ("ntc_hip_read_channels", C.c_int, [C.POINTER(ReadChannels)]),
     ("ntc_hip_write_channels", C.c_int, [C.POINTER(WriteChannels)]),
     ("ntc_hip_image_loss", C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64, C.c_int32, C.c_int32, C.c_int32, C.c_uint32, C.c_int32, C.c_int32,

@@ -42,7 +42,16 @@ struct DevMip {
     uint32_t fast;
     uint32_t hrAxisX, hrAxisY, lrAxisX, lrAxisY;
     uint32_t posMask;          // (texels per period of the positional encoding) - 1
+    // The two grids once more in query order (bricks of 4 x 4 or 8 x 8 cells, all layers of a cell
+    // together), or null; read by the query kernel only.
+    uint8_t const* hrBricks;
+    uint8_t const* lrBricks;
 };
+
+// Brick geometry of a grid with `layers` u16 layers: log2 of the brick's side in cells.
+constexpr int brick_side_log2(int layers) { return layers == 1 ? 3 : 2; }
+constexpr int brick_bytes(int layers) { return (1 << (2 * brick_side_log2(layers))) * layers * 2; }
+hipError_t launch_build_bricks(uint16_t const* src, uint8_t* dst, int width, int height, int layers, hipStream_t stream);
 
 // One random-access query (same layout as NtcHipQuery of the C ABI).
 struct DevQuery { float u, v; int32_t mip; };

@@ -761,6 +761,108 @@ __device__ __forceinline__ void prepare_inputs_scattered(Mip const& m, LdsT<V> c
     }
 }
 
+// The same input vector from the query-ordered copy of the grids: bricks of T x T cells (T = 4, or 8
+// for a one-layer grid), [brick row][brick column][cell row][cell column][layer], so that all layers
+// of a cell are one load of 2, 4, 6 or 8 bytes and the 2 x 2 footprint usually lies in one or two
+// cache lines.  Every tap is addressed on its own (wrap included), so there is no branch at all:
+// eight loads per sample point for the 8 x 2-bit + 16 x 4-bit geometry, all in flight together.
+typedef __attribute__((address_space(1))) u32x2 const* GlobalU32x2Ptr;
+
+template <int LAYERS>
+__device__ __forceinline__ uint32_t brick_offset(uint32_t cx, uint32_t cy, uint32_t log2GridWidth)
+{
+    constexpr uint32_t T = brick_side_log2(LAYERS), MASK = (1u << T) - 1u;
+    uint32_t const lgBricksX = log2GridWidth > T ? log2GridWidth - T : 0u;
+    uint32_t const brick = ((cy >> T) << lgBricksX) + (cx >> T);
+    uint32_t const cell = ((cy & MASK) << T) + (cx & MASK);
+    return brick * uint32_t(brick_bytes(LAYERS)) + cell * uint32_t(2 * LAYERS);     // below 2^32: a grid holds less than 2^31 bytes
+}
+
+// All layers of one cell: layer L in the low or high half of out[L / 2].
+template <int LAYERS>
+__device__ __forceinline__ void load_brick_cell(GlobalU8Ptr base, uint32_t off, uint32_t (&out)[2])
+{
+    out[0] = 0; out[1] = 0;
+    if constexpr (LAYERS == 1) {
+        out[0] = load_u16(base, off);
+    } else if constexpr (LAYERS == 2) {
+        out[0] = *reinterpret_cast<GlobalU32A2Ptr>(base + off);
+    } else if constexpr (LAYERS == 3) {
+        out[0] = *reinterpret_cast<GlobalU32A2Ptr>(base + off);
+        out[1] = load_u16(base, off + 4u);
+    } else {
+        u32x2 const v = *reinterpret_cast<GlobalU32x2Ptr>(base + off);
+        out[0] = v[0]; out[1] = v[1];
+    }
+}
+
+template <class V, class Mip>
+__device__ __forceinline__ void prepare_inputs_bricked(Mip const& m, LdsT<V> const& lds, int x, int y, uint32_t (&in)[16])
+{
+    constexpr int HL = V::HR_MODE == 1 ? 1 : (V::HR_F + 3) / 4, LL = (V::LR_F + 3) / 4;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) in[i] = 0;
+
+    AxisFoot const hx = axis_fast(x, m.hrAxisX, m.hrWidth), hy = axis_fast(y, m.hrAxisY, m.hrHeight);
+    AxisFoot const lx = axis_fast(x, m.lrAxisX, m.lrWidth), ly = axis_fast(y, m.lrAxisY, m.lrHeight);
+    GlobalU8Ptr const gh = (GlobalU8Ptr)m.hrBricks, gl = (GlobalU8Ptr)m.lrBricks;
+    uint32_t const hlg = (m.hrAxisX >> 24) & 0xffu, llg = (m.lrAxisX >> 24) & 0xffu;     // log2(grid width)
+
+    // taps in the order a00 (x0, y0), a10 (x1, y0), a01 (x0, y1), a11 (x1, y1)
+    uint32_t hc[4][2], lc[4][2];
+    load_brick_cell<HL>(gh, brick_offset<HL>(hx.c0, hy.c0, hlg), hc[0]);
+    load_brick_cell<HL>(gh, brick_offset<HL>(hx.c1, hy.c0, hlg), hc[1]);
+    load_brick_cell<HL>(gh, brick_offset<HL>(hx.c0, hy.c1, hlg), hc[2]);
+    load_brick_cell<HL>(gh, brick_offset<HL>(hx.c1, hy.c1, hlg), hc[3]);
+    load_brick_cell<LL>(gl, brick_offset<LL>(lx.c0, ly.c0, llg), lc[0]);
+    load_brick_cell<LL>(gl, brick_offset<LL>(lx.c1, ly.c0, llg), lc[1]);
+    load_brick_cell<LL>(gl, brick_offset<LL>(lx.c0, ly.c1, llg), lc[2]);
+    load_brick_cell<LL>(gl, brick_offset<LL>(lx.c1, ly.c1, llg), lc[3]);
+    __builtin_amdgcn_sched_barrier(0);                       // all loads before any arithmetic
+
+    auto layer_of = [](uint32_t const (&cell)[2], int L) -> uint32_t { return (L & 1) ? cell[L >> 1] >> 16 : cell[L >> 1] & 0xffffu; };
+    if constexpr (V::HR_MODE == 1) {
+        static_assert(V::HR_MODE != 1 || (V::HR_BITS == 2 && V::HR_F == 8 && V::HR_SLOTS == 8), "concat grids: 8 x 2-bit");
+#pragma unroll
+        for (int tap = 0; tap < 4; ++tap) {
+            in[2 * tap]     = lds.lut2[hc[tap][0] & 0xffu];
+            in[2 * tap + 1] = lds.lut2[(hc[tap][0] >> 8) & 0xffu];
+        }
+    } else {
+        uint32_t const nx = (m.hrAxisX >> 8) & 0xffu, ny = (m.hrAxisY >> 8) & 0xffu;
+        uint32_t const wx1 = hx.f, wx0 = (1u << nx) - hx.f, wy1 = hy.f * 17u, wy0 = ((1u << ny) - hy.f) * 17u;
+        uint32_t const w00 = mul24(wx0, wy0), w10 = mul24(wx1, wy0), w01 = mul24(wx0, wy1), w11 = mul24(wx1, wy1);
+#pragma unroll
+        for (int L = 0; L < HL; ++L) {
+            uint32_t b = bilinear4_int(layer_of(hc[0], L), layer_of(hc[1], L), layer_of(hc[2], L), layer_of(hc[3], L), w00, w10, w01, w11, nx + ny);
+            if (4 * L + 4 > V::HR_F) b &= (1u << (8 * (V::HR_F - 4 * L))) - 1u;
+            in[L] = b;
+        }
+    }
+    {
+        uint32_t const nx = (m.lrAxisX >> 8) & 0xffu, ny = (m.lrAxisY >> 8) & 0xffu;
+        uint32_t const wx1 = lx.f, wx0 = (1u << nx) - lx.f, wy1 = ly.f * 17u, wy0 = ((1u << ny) - ly.f) * 17u;
+        uint32_t const w00 = mul24(wx0, wy0), w10 = mul24(wx1, wy0), w01 = mul24(wx0, wy1), w11 = mul24(wx1, wy1);
+#pragma unroll
+        for (int L = 0; L < LL; ++L) {
+            uint32_t b = bilinear4_int(layer_of(lc[0], L), layer_of(lc[1], L), layer_of(lc[2], L), layer_of(lc[3], L), w00, w10, w01, w11, nx + ny);
+            if (4 * L + 4 > V::LR_F) b &= (1u << (8 * (V::LR_F - 4 * L))) - 1u;
+            in[V::HR_INPUTS / 4 + L] = b;
+        }
+    }
+    {
+        uint4 const ex = *reinterpret_cast<uint4 const*>(&lds.xtab[m.posMask + (uint32_t(x) & m.posMask)][0]);
+        uint4 const ey = *reinterpret_cast<uint4 const*>(&lds.ytab[m.posMask + (uint32_t(y) & m.posMask)][0]);
+        in[V::POS_BASE / 4 + 0] = ex.x | ey.x;
+        in[V::POS_BASE / 4 + 1] = ex.y | ey.y;
+        in[V::POS_BASE / 4 + 2] = ex.z | ey.z;
+        if constexpr (V::LOD == 2) {
+            uint32_t const l = uint32_t(int(m.positionLod * 127.5f)) & 0xffu;
+            in[V::POS_BASE / 4 + 3] = l | (l << 8);
+        }
+    }
+}
+
 // One byte of the positional encoding (Inference.hlsli:89-113): int(enc * 127.5), truncating.
 __device__ __forceinline__ uint32_t posenc_byte(float p)
 {
@@ -1096,8 +1198,10 @@ struct QueryMip {
     uint32_t posMask, fast;
     float positionLod;
     uint32_t pad[3];
+    uint8_t const* hrBricks;
+    uint8_t const* lrBricks;
 };
-static_assert(sizeof(QueryMip) == 80, "QueryMip layout");
+static_assert(sizeof(QueryMip) == 96, "QueryMip layout");
 
 template <class V>
 __global__ void __launch_bounds__(256, V::FP8_WEIGHTS ? 2 : 4)
@@ -1114,7 +1218,9 @@ query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __res
         q.hrWidth = d.hrWidth; q.hrHeight = d.hrHeight; q.lrWidth = d.lrWidth; q.lrHeight = d.lrHeight;
         q.width = d.width; q.height = d.height;
         q.posMask = d.posMask; q.fast = d.fast; q.positionLod = d.positionLod;
+        q.hrBricks = d.hrBricks; q.lrBricks = d.lrBricks;
     }
+    bool const bricked = mips[0].hrBricks != nullptr;          // a set has the query-ordered copy for all of its mips or for none
     int const lane = threadIdx.x & 63;
     int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int const j = lane & 15, g = lane >> 4;
@@ -1145,7 +1251,10 @@ query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __res
         x = max(0, min(x, m.width - 1));
         y = max(0, min(y, m.height - 1));
         uint32_t in[16];
-        if (__all(m.fast != 0)) prepare_inputs_scattered<V>(m, lds, x, y, (GlobalU8Ptr)mips, in);   // every lane's mip is power-of-two sized
+        if (__all(m.fast != 0)) {                                // every lane's mip is power-of-two sized
+            if (bricked) prepare_inputs_bricked<V>(m, lds, x, y, in);
+            else         prepare_inputs_scattered<V>(m, lds, x, y, (GlobalU8Ptr)mips, in);
+        }
         else                    prepare_inputs_general<V>(mips[validMip ? query.mip : 0], x, y, in);
 
         // output-layer accumulators as floats: exact either way (|acc| < 2^24 on the fp16 path; the
@@ -1260,6 +1369,30 @@ static hipError_t launch_query_variant(DevMip const* mips, int numMips, DevQuery
                                        uint16_t* out, int gridSize, hipStream_t stream)
 {
     hipLaunchKernelGGL(query_kernel<V>, dim3(gridSize), dim3(256), 0, stream, mips, numMips, queries, numQueries, out);
+    return hipGetLastError();
+}
+
+// Plain grid ([layer][row][column] u16) -> bricks; one thread per stored u16, reads coalesced.
+__global__ void __launch_bounds__(256)
+build_bricks_kernel(uint16_t const* __restrict__ src, uint16_t* __restrict__ dst, int width, int height, int layers, int sideLog2)
+{
+    size_t const cells = size_t(width) * size_t(height);
+    size_t const i = size_t(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= cells * size_t(layers)) return;
+    int const layer = int(i / cells);
+    size_t const cell = i - size_t(layer) * cells;
+    uint32_t const cy = uint32_t(cell / size_t(width)), cx = uint32_t(cell - size_t(cy) * size_t(width));
+    uint32_t const side = 1u << sideLog2, bricksX = (uint32_t(width) + side - 1u) >> sideLog2;
+    size_t const brick = size_t(cy >> sideLog2) * bricksX + (cx >> sideLog2);
+    size_t const inBrick = ((cy & (side - 1u)) << sideLog2) + (cx & (side - 1u));
+    dst[(brick * (size_t(1) << (2 * sideLog2)) + inBrick) * size_t(layers) + size_t(layer)] = src[i];
+}
+
+hipError_t launch_build_bricks(uint16_t const* src, uint8_t* dst, int width, int height, int layers, hipStream_t stream)
+{
+    size_t const count = size_t(width) * size_t(height) * size_t(layers);
+    hipLaunchKernelGGL(build_bricks_kernel, dim3(unsigned((count + 255) / 256)), dim3(256), 0, stream,
+                       src, reinterpret_cast<uint16_t*>(dst), width, height, layers, brick_side_log2(layers));
     return hipGetLastError();
 }
 

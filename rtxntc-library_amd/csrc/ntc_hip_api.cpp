@@ -161,6 +161,49 @@ uint64_t grid_bytes(int32_t w, int32_t h, int32_t features, int32_t bits)
     return uint64_t(w) * uint64_t(h) * 2u * uint64_t((features + perWord - 1) / perWord);
 }
 
+// Where each grid of a set lives in the query-ordered copy (ntc_hip_build_query_latents).  Grids
+// that several mips share (same offset and size in `latents`) are stored once; every grid starts
+// on a 128-byte boundary.
+struct BrickGrid { uint64_t srcOffset, dstOffset; int32_t width, height, layers; };
+struct BrickPlan {
+    std::vector<BrickGrid> grids;
+    uint64_t hr[NTC_HIP_MAX_MIPS], lr[NTC_HIP_MAX_MIPS];
+    uint64_t totalBytes = 0;
+};
+
+int grid_layers(int32_t features, int32_t bits) { return (features + 16 / bits - 1) / (16 / bits); }
+
+uint64_t bricked_bytes(int32_t width, int32_t height, int layers)
+{
+    uint64_t const side = uint64_t(1) << brick_side_log2(layers);
+    uint64_t const bytes = ((uint64_t(width) + side - 1) / side) * ((uint64_t(height) + side - 1) / side) * uint64_t(brick_bytes(layers));
+    return (bytes + 127u) & ~uint64_t(127);
+}
+
+bool plan_bricks(NtcHipTextureSet const& set, BrickPlan& plan)
+{
+    if (!spec_sane(set.spec) || set.numMips < 1 || set.numMips > NTC_HIP_MAX_MIPS) return false;
+    plan.grids.clear();
+    plan.totalBytes = 0;
+    auto place = [&](uint64_t srcOffset, int32_t w, int32_t h, int layers) -> uint64_t {
+        for (BrickGrid const& g : plan.grids)
+            if (g.srcOffset == srcOffset && g.width == w && g.height == h && g.layers == layers) return g.dstOffset;
+        BrickGrid const g{ srcOffset, plan.totalBytes, w, h, layers };
+        plan.grids.push_back(g);
+        plan.totalBytes += bricked_bytes(w, h, layers);
+        return g.dstOffset;
+    };
+    int const hrLayers = grid_layers(set.spec.hrFeatures, set.spec.hrBits), lrLayers = grid_layers(set.spec.lrFeatures, set.spec.lrBits);
+    if (hrLayers < 1 || hrLayers > 4 || lrLayers < 1 || lrLayers > 4) return false;
+    for (int m = 0; m < set.numMips; ++m) {
+        NtcHipMipDesc const& d = set.mips[m];
+        if (d.hrWidth < 1 || d.hrHeight < 1 || d.lrWidth < 1 || d.lrHeight < 1) return false;
+        plan.hr[m] = place(d.hrOffset, d.hrWidth, d.hrHeight, hrLayers);
+        plan.lr[m] = place(d.lrOffset, d.lrWidth, d.lrHeight, lrLayers);
+    }
+    return true;
+}
+
 // Validates the sets, builds the mip table (sorted by tileStart) and picks the kernel.
 int build_table(NtcHipTextureSet const* sets, int32_t numSets, std::vector<DevMip>& table, int& variant, int& totalTiles,
                 bool forQueries = false)
@@ -180,6 +223,15 @@ int build_table(NtcHipTextureSet const* sets, int32_t numSets, std::vector<DevMi
         if (!set.latents || !set.weights || (!set.output && !forQueries)) { set_error("ntc_hip_decode: set %d: null latents / weights / output pointer.", s); return NTC_HIP_ERR_INVALID_ARG; }
         if (!forQueries && (set.outputFormat < NTC_HIP_OUT_FP16_PLANAR_PAIRS || set.outputFormat > NTC_HIP_OUT_UNORM8_PIXELS)) { set_error("ntc_hip_decode: set %d: unknown output format %d.", s, set.outputFormat); return NTC_HIP_ERR_INVALID_ARG; }
         if ((reinterpret_cast<uintptr_t>(set.weights) & 3u) || (reinterpret_cast<uintptr_t>(set.latents) & 1u)) { set_error("ntc_hip_decode: set %d: weights must be 4-byte and latents 2-byte aligned.", s); return NTC_HIP_ERR_INVALID_ARG; }
+        BrickPlan bricks;
+        bool const bricked = forQueries && set.queryLatents != nullptr;
+        if (bricked) {
+            if (!plan_bricks(set, bricks) || set.queryLatentsBytes < bricks.totalBytes || (reinterpret_cast<uintptr_t>(set.queryLatents) & 127u)) {
+                set_error("ntc_hip_decode_queries: set %d: queryLatents must be 128-byte aligned and hold %llu bytes (ntc_hip_query_latents_bytes).",
+                          s, (unsigned long long)bricks.totalBytes);
+                return NTC_HIP_ERR_INVALID_ARG;
+            }
+        }
         NtcHipWeightLayout layout;
         if (ntc_hip_weight_layout(&set.spec, &layout) != 0) return NTC_HIP_ERR_INVALID_ARG;
         if (set.weightsBytes < layout.bufferSize) {
@@ -237,6 +289,10 @@ int build_table(NtcHipTextureSet const* sets, int32_t numSets, std::vector<DevMi
             e.positionScale = d.positionScale; e.positionLod = d.positionLod;
             e.outPixelStride = set.outPixelStride; e.numChannels = set.numChannels; e.outFormat = set.outputFormat;
             fill_fast_path(set.spec, e);
+            if (bricked) {
+                e.hrBricks = static_cast<uint8_t const*>(set.queryLatents) + bricks.hr[m];
+                e.lrBricks = static_cast<uint8_t const*>(set.queryLatents) + bricks.lr[m];
+            }
             e.tilesX = (d.width + kTileWidth - 1) / kTileWidth;
             e.tilesY = (d.height + kTileHeight - 1) / kTileHeight;
             e.tileStart = totalTiles;
@@ -511,6 +567,38 @@ static int run_queries(const NtcHipTextureSet* set, const NtcHipQuery* queries, 
         HIP_TRY(hipEventElapsedTime(&ms, g_lib.evStart, g_lib.evStop));
         *outMs = ms / float(iterations);
     }
+    clear_error();
+    return 0;
+}
+
+uint64_t ntc_hip_query_latents_bytes(const NtcHipTextureSet* set)
+{
+    BrickPlan plan;
+    if (!set || !plan_bricks(*set, plan)) { set_error("ntc_hip_query_latents_bytes: malformed texture set."); return 0; }
+    return plan.totalBytes;
+}
+
+int ntc_hip_build_query_latents(const NtcHipTextureSet* set, void* dst, uint64_t dstBytes)
+{
+    if (int r = require_init()) return r;
+    if (!set || !dst || !set->latents) { set_error("ntc_hip_build_query_latents: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
+    BrickPlan plan;
+    if (!plan_bricks(*set, plan)) { set_error("ntc_hip_build_query_latents: malformed texture set."); return NTC_HIP_ERR_INVALID_ARG; }
+    if (dstBytes < plan.totalBytes || (reinterpret_cast<uintptr_t>(dst) & 127u) || (reinterpret_cast<uintptr_t>(set->latents) & 1u)) {
+        set_error("ntc_hip_build_query_latents: the destination must be 128-byte aligned and hold %llu bytes.", (unsigned long long)plan.totalBytes);
+        return NTC_HIP_ERR_INVALID_ARG;
+    }
+    for (BrickGrid const& g : plan.grids) {
+        uint64_t const srcBytes = uint64_t(g.width) * uint64_t(g.height) * 2u * uint64_t(g.layers);
+        if ((g.srcOffset & 1u) || g.srcOffset + srcBytes > set->latentsBytes || srcBytes >= (1ull << 32)) {
+            set_error("ntc_hip_build_query_latents: a latent grid reaches past the %llu-byte latent buffer.", (unsigned long long)set->latentsBytes);
+            return NTC_HIP_ERR_INVALID_ARG;
+        }
+    }
+    // (bricks of grids narrower than a brick keep cells that nothing writes and no query reads)
+    for (BrickGrid const& g : plan.grids)
+        HIP_TRY(launch_build_bricks(reinterpret_cast<uint16_t const*>(static_cast<uint8_t const*>(set->latents) + g.srcOffset),
+                                    static_cast<uint8_t*>(dst) + g.dstOffset, g.width, g.height, g.layers, g_lib.stream));
     clear_error();
     return 0;
 }
