@@ -305,6 +305,27 @@ typedef struct NtcHipImageDifference {
 } NtcHipImageDifference;
 int ntc_hip_image_difference(const NtcHipImageDifference* params);
 
+/* BC4 / BC5 compression of an image: the block-compression compute pass of
+ * IContext::MakeBlockCompressionComputePass for those two formats (include/libntc/ntc.h:1050-1100,
+ * src/shaders/CompressBC4.hlsl, CompressBC5.hlsl, BC4_* of src/shaders/BlockCompressCommon.hlsli).
+ * widthInBlocks x heightInBlocks blocks of 4 x 4 pixels starting at (srcLeft, srcTop) are encoded from
+ * channel R (BC4, 8 bytes per block) or R and G (BC5, 16 bytes) and stored row-major with dstRowPitch
+ * bytes per row of blocks, the first at block (dstOffsetX, dstOffsetY).  Pixels outside the image read as
+ * 0, like a texture load there.  dstFormat is a BlockCompressedFormat: 4 or 5; the other formats return
+ * NTC_HIP_ERR_UNSUPPORTED.  Asynchronous on the library stream. */
+typedef struct NtcHipBlockCompress {
+    NtcHipImage src;
+    int32_t     srcLeft, srcTop;
+    int32_t     widthInBlocks, heightInBlocks;
+    int32_t     dstFormat;
+    int32_t     dstOffsetX, dstOffsetY;       /* in blocks */
+    int32_t     reserved;
+    void*       dst;                          /* device, 8-byte aligned */
+    uint64_t    dstBytes;
+    uint64_t    dstRowPitch;                  /* bytes per row of blocks, multiple of 8 */
+} NtcHipBlockCompress;
+int ntc_hip_block_compress(const NtcHipBlockCompress* params);
+
 /* Self-check of the MFMA operand layout the kernels assume: multiplies a 16x64 by a
  * 64x16 int8 matrix on the device (row-major host arrays), writes the 16x16 int32
  * product.  No reference counterpart; used by the tests. */

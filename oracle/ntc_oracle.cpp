@@ -55,6 +55,13 @@
  *                            values with an exact binary expansion (tests/test_image_difference.py).
  *                            The reference does not define the order of a workgroup's additions,
  *                            so its exact low bits are parity unpinned by construction.
+ *   block_compress (BC4/5)   the format's standard decoder in numpy: blocks of at most two distinct
+ *                            values and exact ramps decode exactly, the decoded error of random
+ *                            blocks never exceeds that of the start endpoints and stays within
+ *                            half a palette step + 1 (tests/test_block_compress.py).  The choices
+ *                            of the reference's shader compiler (fused multiply-adds in the
+ *                            least-squares fit) are not known: parity with its exact blocks is
+ *                            unpinned; blocks are valid BC4 by construction.
  *   The exact bits of the reference's FP16-WMMA CUDA kernel (half accumulation order,
  *   --use_fast_math) and of a hardware bilinear sampler are NOT reproduced: parity unpinned
  *   for those two, by construction; the integer contract of Inference.hlsli is what is pinned.
@@ -937,6 +944,157 @@ void ntc_oracle_image_difference(const NtcHipImageDifference* p, uint64_t* out /
                 out[c] += (high << 32) | low;
             }
         }
+}
+
+// ---- BC4 / BC5 encoder (BC4_* of src/shaders/BlockCompressCommon.hlsli:510-796, CompressBC4.hlsl,
+// CompressBC5.hlsl) --------------------------------------------------------------------------------------
+// Both palettes of the format are tried: from start endpoints (the block's extremes moved inwards by
+// range / 34; for the six-value palette the extremes that are not 0 / 255) texels are assigned to their
+// nearest palette entry, then at most eight rounds of least-squares endpoints + re-assignment, ending
+// when the error stops falling or the assignment repeats (hlsli:710-795).  HLSL round() is taken as
+// round-half-even, clamp() as min(max()) (a NaN becomes the lower bound).
+namespace bc4 {
+
+void palette(uint32_t e0, uint32_t e1, uint32_t p[8])       // hlsli:563-603
+{
+    p[0] = e0; p[1] = e1;
+    if (e0 > e1) {
+        p[2] = (6 * e0 + 1 * e1 + 3) / 7; p[3] = (5 * e0 + 2 * e1 + 3) / 7; p[4] = (4 * e0 + 3 * e1 + 3) / 7;
+        p[5] = (3 * e0 + 4 * e1 + 3) / 7; p[6] = (2 * e0 + 5 * e1 + 3) / 7; p[7] = (1 * e0 + 6 * e1 + 3) / 7;
+    } else {
+        p[2] = (4 * e0 + 1 * e1 + 2) / 5; p[3] = (3 * e0 + 2 * e1 + 2) / 5; p[4] = (2 * e0 + 3 * e1 + 2) / 5; p[5] = (1 * e0 + 4 * e1 + 2) / 5;
+        p[6] = 0; p[7] = 255;
+    }
+}
+
+struct Block {
+    uint32_t e0 = 0, e1 = 0;
+    uint32_t index[16] = {};
+    bool same_indices(Block const& o) const { return std::memcmp(index, o.index, sizeof index) == 0; }
+    uint64_t bits() const
+    {
+        uint64_t v = uint64_t(e0 & 0xffu) | (uint64_t(e1 & 0xffu) << 8);
+        for (int t = 0; t < 16; ++t) v |= uint64_t(index[t] & 7u) << (16 + 3 * t);
+        return v;
+    }
+};
+
+float assign(const uint32_t values[16], Block& b)           // hlsli:605-632
+{
+    uint32_t pal[8];
+    palette(b.e0 & 0xffu, b.e1 & 0xffu, pal);
+    float total = 0.f;
+    for (int t = 0; t < 16; ++t) {
+        int best = 0x7fffffff;
+        uint32_t pick = 8;
+        for (uint32_t k = 0; k < 8; ++k) {
+            int d = int(values[t]) - int(pal[k]);
+            d *= d;
+            if (d < best) { best = d; pick = k; }
+        }
+        total += float(best);
+        b.index[t] = pick;
+    }
+    return total;
+}
+
+uint32_t endpoint(float v) { return uint32_t(std::nearbyint(std::fmin(std::fmax(v, 0.f), 255.f))); }
+
+void refit8(const uint32_t values[16], Block& b, bool zeroE1, bool oneE0)     // hlsli:634-670
+{
+    float aa = 0, bb = 0, ab = 0, ax = 0, bx = 0;
+    for (int t = 0; t < 16; ++t) {
+        uint32_t const k = b.index[t];
+        float const alpha = k < 2 ? 1.f - float(k) : (8.f - float(k)) / 7.f;
+        float const beta = 1.f - alpha;
+        aa += alpha * alpha; bb += beta * beta; ab += alpha * beta;
+        ax += alpha * float(values[t]); bx += beta * float(values[t]);
+    }
+    float const factor = 1.f / (aa * bb - ab * ab);
+    float const a = (ax * bb - bx * ab) * factor, c = (bx * aa - ax * ab) * factor;
+    uint32_t e0 = oneE0 ? 255u : endpoint(a), e1 = zeroE1 ? 0u : endpoint(c);
+    if (e0 < e1) std::swap(e0, e1);
+    b.e0 = e0; b.e1 = e1;
+}
+
+void refit6(const uint32_t values[16], Block& b)            // hlsli:672-708
+{
+    float aa = 0, bb = 0, ab = 0, ax = 0, bx = 0;
+    for (int t = 0; t < 16; ++t) {
+        uint32_t const k = b.index[t];
+        float alpha;
+        if (k < 2) alpha = 1.f - float(k);
+        else if (k < 6) alpha = (6.f - float(k)) / 5.f;
+        else continue;
+        float const beta = 1.f - alpha;
+        aa += alpha * alpha; bb += beta * beta; ab += alpha * beta;
+        ax += alpha * float(values[t]); bx += beta * float(values[t]);
+    }
+    float const factor = aa * bb - ab * ab;
+    if (factor == 0.f) return;
+    b.e0 = endpoint((ax * bb - bx * ab) / factor);
+    b.e1 = endpoint((bx * aa - ax * ab) / factor);
+}
+
+uint64_t encode(const float texels[16])                     // hlsli:710-795
+{
+    uint32_t values[16], mina = 255, maxa = 0, minaInner = 255, maxaInner = 0;
+    for (int t = 0; t < 16; ++t) {
+        float const s = std::fmin(std::fmax(texels[t], 0.f), 1.f);
+        values[t] = uint32_t(std::nearbyint(s * 255.f));
+        mina = std::min(mina, values[t]); maxa = std::max(maxa, values[t]);
+        if (values[t] != 0) minaInner = std::min(minaInner, values[t]);
+        if (values[t] != 255) maxaInner = std::max(maxaInner, values[t]);
+    }
+    bool const zeroE1 = mina == 0, oneE0 = maxa == 255;
+
+    Block block;
+    block.e0 = oneE0 ? 255u : maxa - (maxa - mina) / 34u;
+    block.e1 = zeroE1 ? 0u : mina + (maxa - mina) / 34u;
+    float bestError = assign(values, block);
+    Block best = block;
+    for (int i = 0; i < 8; ++i) {
+        refit8(values, block, zeroE1, oneE0);
+        float const error = assign(values, block);
+        if (error >= bestError) break;
+        if (block.same_indices(best)) { best = block; break; }
+        best = block; bestError = error;
+    }
+
+    block.e0 = (minaInner + (maxaInner - minaInner) / 34u) & 0xffu;     // uint32 arithmetic, wraps when there are no inner values
+    block.e1 = (maxaInner - (maxaInner - minaInner) / 34u) & 0xffu;
+    float bestError2 = assign(values, block);
+    Block best2 = block;
+    for (int i = 0; i < 8; ++i) {
+        refit6(values, block);
+        float const error = assign(values, block);
+        if (error >= bestError2) break;
+        if (block.same_indices(best2)) { best2 = block; break; }
+        best2 = block; bestError2 = error;
+    }
+    return (bestError2 < bestError ? best2 : best).bits();
+}
+
+} // namespace bc4
+
+// dstFormat 4 (BC4: channel R) or 5 (BC5: R then G); host pointers in `p`.  Returns -1 for other formats.
+int ntc_oracle_block_compress(const NtcHipBlockCompress* p)
+{
+    if (p->dstFormat != 4 && p->dstFormat != 5) return -1;
+    int const channels = p->dstFormat == 4 ? 1 : 2;
+    auto fetch = [&](int x, int y, int c) -> float {
+        if (x < 0 || y < 0 || x >= p->src.width || y >= p->src.height) return 0.f;
+        return diff_channel(p->src, static_cast<uint8_t const*>(p->src.data) + size_t(y) * p->src.rowPitch + size_t(x) * p->src.pixelStride, c);
+    };
+    for (int by = 0; by < p->heightInBlocks; ++by)
+        for (int bx = 0; bx < p->widthInBlocks; ++bx)
+            for (int c = 0; c < channels; ++c) {
+                float texels[16];
+                for (int t = 0; t < 16; ++t) texels[t] = fetch(p->srcLeft + bx * 4 + (t & 3), p->srcTop + by * 4 + (t >> 2), c);
+                uint64_t const bits = bc4::encode(texels);
+                std::memcpy(static_cast<uint8_t*>(p->dst) + size_t(by + p->dstOffsetY) * p->dstRowPitch + (size_t(bx + p->dstOffsetX) * channels + c) * 8, &bits, 8);
+            }
+    return 0;
 }
 
 // Random-access decode of a list of (u, v, mip) sample points: NtcSampleTextureSet

@@ -107,6 +107,14 @@ class ImageDifference(C.Structure):
     ]
 
 
+class BlockCompress(C.Structure):
+    _fields_ = [
+        ("src", Image), ("srcLeft", C.c_int32), ("srcTop", C.c_int32), ("widthInBlocks", C.c_int32), ("heightInBlocks", C.c_int32),
+        ("dstFormat", C.c_int32), ("dstOffsetX", C.c_int32), ("dstOffsetY", C.c_int32), ("reserved", C.c_int32),
+        ("dst", C.c_void_p), ("dstBytes", C.c_uint64), ("dstRowPitch", C.c_uint64),
+    ]
+
+
 class Query(C.Structure):
     _fields_ = [("u", C.c_float), ("v", C.c_float), ("mip", C.c_int32)]
 
@@ -147,6 +155,7 @@ EXPORTS = [
     ("ntc_hip_image_loss", C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64, C.c_int32, C.c_int32, C.c_int32, C.c_uint32, C.c_int32, C.c_int32,
                                      C.POINTER(C.c_float)]),
     ("ntc_hip_image_difference", C.c_int, [C.POINTER(ImageDifference)]),
+    ("ntc_hip_block_compress", C.c_int, [C.POINTER(BlockCompress)]),
     ("ntc_hip_resize_planar", C.c_int, [C.c_void_p, C.c_uint64, C.c_int32, C.c_int32, C.c_void_p, C.c_uint64, C.c_int32, C.c_int32,
                                         C.c_int32, C.c_void_p]),
     ("ntc_hip_selftest_mfma", C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),

@@ -124,6 +124,15 @@ struct ImageDifferenceArgs {
 };
 hipError_t launch_image_difference(ImageDifferenceArgs const& args, hipStream_t stream);
 
+struct BlockCompressArgs {
+    uint8_t const* src;
+    uint8_t* dst;
+    uint64_t pixelStride, rowPitch, dstRowPitch;
+    int32_t srcWidth, srcHeight, format, numChannels;
+    int32_t srcLeft, srcTop, widthInBlocks, heightInBlocks, dstOffsetX, dstOffsetY;
+};
+hipError_t launch_block_compress(BlockCompressArgs const& args, int channels, hipStream_t stream);
+
 hipError_t launch_decode(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream);
 hipError_t launch_queries(int variant, DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries,
                           uint16_t* out, int gridSize, hipStream_t stream);

@@ -850,6 +850,40 @@ int ntc_hip_image_difference(const NtcHipImageDifference* p)
     return 0;
 }
 
+int ntc_hip_block_compress(const NtcHipBlockCompress* p)
+{
+    if (int r = require_init()) return r;
+    if (!p || !p->dst) { set_error("ntc_hip_block_compress: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
+    if (p->dstFormat < 1 || p->dstFormat > 7) { set_error("ntc_hip_block_compress: dstFormat (%d) is not a block-compressed format.", p->dstFormat); return NTC_HIP_ERR_INVALID_ARG; }
+    if (p->dstFormat != 4 && p->dstFormat != 5) {
+        set_error("ntc_hip_block_compress: only BC4 and BC5 are implemented (dstFormat %d).", p->dstFormat);
+        return NTC_HIP_ERR_UNSUPPORTED;
+    }
+    if (p->srcLeft < 0 || p->srcTop < 0 || p->widthInBlocks < 1 || p->heightInBlocks < 1 || p->dstOffsetX < 0 || p->dstOffsetY < 0
+        || p->widthInBlocks > (1 << 20) || p->heightInBlocks > (1 << 20) || p->dstOffsetX > (1 << 20) || p->dstOffsetY > (1 << 20)) {
+        set_error("ntc_hip_block_compress: bad extent or destination offset.");
+        return NTC_HIP_ERR_INVALID_ARG;
+    }
+    BlockCompressArgs a{};
+    DiffImageArgs image{};
+    if (int r = check_diff_image(p->src, "src", 0, 0, 1, 1, image)) return r;     // the extent may reach past the image: such pixels read as 0
+    uint64_t const blockBytes = p->dstFormat == 4 ? 8u : 16u;
+    uint64_t const rowNeed = uint64_t(p->dstOffsetX + p->widthInBlocks) * blockBytes;
+    if ((p->dstRowPitch & 7u) || p->dstRowPitch < rowNeed || (reinterpret_cast<uintptr_t>(p->dst) & 7u)
+        || uint64_t(p->dstOffsetY + p->heightInBlocks - 1) * p->dstRowPitch + rowNeed > p->dstBytes) {
+        set_error("ntc_hip_block_compress: the destination (8-byte aligned, row pitch a multiple of 8) does not hold the blocks.");
+        return NTC_HIP_ERR_INVALID_ARG;
+    }
+    a.src = image.data; a.pixelStride = image.pixelStride; a.rowPitch = image.rowPitch; a.format = image.format; a.numChannels = image.numChannels;
+    a.srcWidth = p->src.width; a.srcHeight = p->src.height;
+    a.dst = static_cast<uint8_t*>(p->dst); a.dstRowPitch = p->dstRowPitch;
+    a.srcLeft = p->srcLeft; a.srcTop = p->srcTop; a.widthInBlocks = p->widthInBlocks; a.heightInBlocks = p->heightInBlocks;
+    a.dstOffsetX = p->dstOffsetX; a.dstOffsetY = p->dstOffsetY;
+    HIP_TRY(launch_block_compress(a, p->dstFormat == 4 ? 1 : 2, g_lib.stream));
+    clear_error();
+    return 0;
+}
+
 int ntc_hip_selftest_mfma(const int8_t* a16x64, const int8_t* b64x16, int32_t* d16x16)
 {
     if (int r = require_init()) return r;

@@ -1158,6 +1158,40 @@ public:
     void DestroyTextureSet(ITextureSet* textureSet) const override { delete textureSet; }
     bool IsCudaAvailable() const override { return m_deviceAvailable; }
 
+    Status CompressBlocks(BlockCompressionParameters const& params) const override
+    {
+        if (!params.pDstData || !params.srcImage.pData) { SetErrorMessage("Source or destination data is NULL"); return Status::InvalidArgument; }
+        if (params.srcRect.left < 0 || params.srcRect.top < 0) {
+            SetErrorMessage("Left (%d) and top (%d) must be non-negative", params.srcRect.left, params.srcRect.top);
+            return Status::OutOfRange;
+        }
+        if (params.srcRect.width <= 0 || params.srcRect.height <= 0) {
+            SetErrorMessage("Width (%d) and height (%d) must be positive", params.srcRect.width, params.srcRect.height);
+            return Status::OutOfRange;
+        }
+        if (params.dstOffsetInBlocks.x < 0 || params.dstOffsetInBlocks.y < 0) {
+            SetErrorMessage("dstOffsetInBlocks (%d, %d) must be non-negative", params.dstOffsetInBlocks.x, params.dstOffsetInBlocks.y);
+            return Status::OutOfRange;
+        }
+        if (int(params.dstFormat) < int(BlockCompressedFormat::BC1) || int(params.dstFormat) > int(BlockCompressedFormat::BC7)) {
+            SetErrorMessage("Invalid dstFormat (%s)", BlockCompressedFormatToString(params.dstFormat));
+            return Status::OutOfRange;
+        }
+        if (!m_deviceAvailable) { SetErrorMessage("No HIP device is available to this context."); return Status::CudaUnavailable; }
+        NtcHipBlockCompress p{};
+        ImageDesc const& src = params.srcImage;
+        p.src.data = src.pData; p.src.bytes = src.dataSize; p.src.pixelStride = src.pixelStride; p.src.rowPitch = src.rowPitch;
+        p.src.width = src.width; p.src.height = src.height; p.src.format = int32_t(src.channelFormat); p.src.numChannels = src.numChannels;
+        p.srcLeft = params.srcRect.left; p.srcTop = params.srcRect.top;
+        p.widthInBlocks = (params.srcRect.width + 3) / 4; p.heightInBlocks = (params.srcRect.height + 3) / 4;
+        p.dstFormat = int32_t(params.dstFormat);
+        p.dstOffsetX = params.dstOffsetInBlocks.x; p.dstOffsetY = params.dstOffsetInBlocks.y;
+        p.dst = params.pDstData; p.dstBytes = params.dstDataSize; p.dstRowPitch = params.dstRowPitch;
+        if (int r = ntc_hip_block_compress(&p)) return DeviceFailure(r);
+        ClearErrorMessage();
+        return Status::Ok;
+    }
+
     // Argument rules and messages of src/Context.cpp:796-812; the pass itself is ntc_hip_image_difference.
     Status ComputeImageDifference(ImageDifferenceParameters const& params) const override
     {

@@ -201,6 +201,21 @@ struct ImageDifferenceParameters
     uint32_t outputOffset = 0;          // bytes, multiple of 8
 };
 
+// The fields of MakeBlockCompressionComputePassParameters (include/libntc/ntc.h:1050-1100) that BC4 and
+// BC5 use, plus what a graphics application binds to that pass: the source image and the destination.
+struct Point { int x = 0; int y = 0; };
+struct BlockCompressionParameters
+{
+    ImageDesc srcImage;                 // device memory
+    Rect srcRect;                       // pixels to compress; width and height are rounded up to whole blocks
+    Point dstOffsetInBlocks;
+    BlockCompressedFormat dstFormat = BlockCompressedFormat::None;      // BC4 or BC5
+    float alphaThreshold = 1.f / 255.f; // BC1 only in the reference; unused here
+    void* pDstData = nullptr;           // device memory: rows of 8-byte (BC4) or 16-byte (BC5) blocks
+    size_t dstDataSize = 0;
+    size_t dstRowPitch = 0;             // bytes per row of blocks
+};
+
 // Decoder families beyond the one compiled into LibNTC 0.9.2, selected with
 // ITextureSet::SetDecoderPreset (an addition; the reference changes decoders by editing
 // InferenceConstants.h, README.md:32-36).
@@ -343,6 +358,11 @@ public:
     // graphics API (include/libntc/ntc.h:1227-1239, src/Context.cpp:781-860, src/shaders/ImageDifference.hlsl)
     // on the device, asynchronously; DecodeImageDifferenceResult converts the four results.
     virtual Status ComputeImageDifference(ImageDifferenceParameters const& params) const = 0;
+    // Runs the block-compression pass that IContext::MakeBlockCompressionComputePass describes for a
+    // graphics API (include/libntc/ntc.h:1213-1225, src/Context.cpp, src/shaders/CompressBC4.hlsl and
+    // CompressBC5.hlsl) on the device, asynchronously.  BC4 and BC5 only: the other formats return
+    // Status::Unsupported.
+    virtual Status CompressBlocks(BlockCompressionParameters const& params) const = 0;
     // True when a gfx950 device was initialised (reference: IsCudaAvailable).
     virtual bool IsCudaAvailable() const = 0;
     virtual ~IContext() = default;

@@ -421,6 +421,33 @@ static int imageDifference()
     dp.extent.width = 200;                                                                      // leaves the image
     CHECK(ctx->ComputeImageDifference(dp) == Status::InvalidArgument);
     CHECK(std::strstr(GetLastErrorMessage(), "does not lie inside") != nullptr);
+    // block compression of image B: constant 255 everywhere except the zero corner -> BC4 blocks 0xFF, 0xFF / 0, 0 with all indices 0
+    {
+        size_t const blocksX = size_t(w) / 4, blocksY = size_t(h) / 4;
+        void* dBlocks = nullptr;
+        CHECK(ntc_hip_alloc(&dBlocks, blocksX * blocksY * 16) == 0);
+        BlockCompressionParameters bp;
+        bp.srcImage = dp.imageB;
+        bp.srcRect = Rect{ 0, 0, w, h };
+        bp.dstFormat = BlockCompressedFormat::BC5;
+        bp.pDstData = dBlocks; bp.dstDataSize = blocksX * blocksY * 16; bp.dstRowPitch = blocksX * 16;
+        CHECK(ctx->CompressBlocks(bp) == Status::Ok);
+        std::vector<uint64_t> blocks(blocksX * blocksY * 2);
+        CHECK(ntc_hip_download(blocks.data(), dBlocks, blocks.size() * 8) == 0);
+        for (size_t by = 0; by < blocksY; ++by)
+            for (size_t bx = 0; bx < blocksX; ++bx) {
+                bool const corner = bx < 8 && by < 4;
+                uint64_t const want = corner ? 0ull : 0xFFFFull;
+                CHECK(blocks[(by * blocksX + bx) * 2] == want && blocks[(by * blocksX + bx) * 2 + 1] == want);
+            }
+        bp.dstFormat = BlockCompressedFormat::BC7;
+        CHECK(ctx->CompressBlocks(bp) == Status::Unsupported);
+        bp.dstFormat = BlockCompressedFormat::None;
+        CHECK(ctx->CompressBlocks(bp) == Status::OutOfRange);
+        bp.dstFormat = BlockCompressedFormat::BC4; bp.dstDataSize = 8;
+        CHECK(ctx->CompressBlocks(bp) == Status::InvalidArgument);
+        CHECK(ntc_hip_free(dBlocks) == 0);
+    }
     CHECK(ntc_hip_free(dA) == 0 && ntc_hip_free(dB) == 0 && ntc_hip_free(dOut) == 0);
     DestroyContext(ctx);
     std::printf("host image difference OK\n");
