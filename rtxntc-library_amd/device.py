@@ -59,6 +59,12 @@ class DeviceBuffer:
         abi.check(self.device.lib.ntc_hip_download(out.ctypes.data, self.ptr, self.nbytes))
         return out.view(dtype)
 
+    def download_range(self, offset, nbytes, dtype=np.uint8):
+        assert 0 <= offset and offset + nbytes <= self.nbytes
+        out = np.empty(int(nbytes), dtype=np.uint8)
+        abi.check(self.device.lib.ntc_hip_download(out.ctypes.data, self.ptr + int(offset), int(nbytes)))
+        return out.view(dtype)
+
     def fill(self, value):
         abi.check(self.device.lib.ntc_hip_memset(self.ptr, value, self.nbytes))
 
