@@ -391,6 +391,60 @@ public:
         return shuffled;
     }
 
+    // src/TextureSetMetadata.cpp:109-228.  m_neuralLodOfMip is filled for the shared-LOD geometry only.
+    LatentTextureDesc GetLatentTextureDesc() const override
+    {
+        LatentTextureDesc desc;
+        if (m_numNeuralLods == 0) return desc;
+        desc.width = GridDimension(m_desc.width, 0, m_latentShape.gridSizeScale);
+        desc.height = GridDimension(m_desc.height, 0, m_latentShape.gridSizeScale);
+        desc.arraySize = (m_latentShape.numFeatures + 3) / 4;
+        desc.mipLevels = m_numNeuralLods;
+        return desc;
+    }
+    int GetNumLatentImages() const override { return m_numNeuralLods; }
+
+    Status GetFusedMipLevels(int mipLevel, int* pOutFirstFusedMip, int* pOutLastFusedMip) const override
+    {
+        if (m_numNeuralLods == 0) { SetErrorMessage("This decoder geometry has no shared latent images."); return Status::Unsupported; }
+        if (mipLevel < 0 || mipLevel >= m_desc.mips) {
+            SetErrorMessage("mipLevel (%d) must be between 0 and %d", mipLevel, m_desc.mips - 1);
+            return Status::OutOfRange;
+        }
+        int first = mipLevel, last = mipLevel;
+        while (first > 0 && m_neuralLodOfMip[first - 1] == m_neuralLodOfMip[mipLevel]) --first;
+        while (last + 1 < m_desc.mips && m_neuralLodOfMip[last + 1] == m_neuralLodOfMip[mipLevel]) ++last;
+        if (pOutFirstFusedMip) *pOutFirstFusedMip = first;
+        if (pOutLastFusedMip) *pOutLastFusedMip = last;
+        ClearErrorMessage();
+        return Status::Ok;
+    }
+
+    Status GetMipLevelsForLatentImage(int latentImageIndex, int* pOutFirstColorMip, int* pOutLastColorMip) const override
+    {
+        if (latentImageIndex < 0 || latentImageIndex >= m_numNeuralLods) {
+            SetErrorMessage("Invalid latentImageIndex (%d), it must be between 0 and %d", latentImageIndex, m_numNeuralLods);
+            return m_numNeuralLods == 0 ? Status::Unsupported : Status::OutOfRange;
+        }
+        int first = -1, last = -1;
+        for (int mip = 0; mip < m_desc.mips; ++mip)
+            if (m_neuralLodOfMip[mip] == latentImageIndex) { if (first < 0) first = mip; last = mip; }
+        if (first < 0) {                                     // the odd LODs are only ever the low-resolution partner
+            SetErrorMessage("No color MIPs found that are represented by latent image %d", latentImageIndex);
+            return Status::OutOfRange;
+        }
+        if (pOutFirstColorMip) *pOutFirstColorMip = first;
+        if (pOutLastColorMip) *pOutLastColorMip = last;
+        ClearErrorMessage();
+        return Status::Ok;
+    }
+
+    bool IsInferenceWeightTypeSupported(InferenceWeightType weightType) const override
+    {
+        return weightType == InferenceWeightType::GenericInt8 && !m_hostWeights.empty();
+    }
+    void SetExperimentalKnob(float) override {}
+
     InferenceWeightType GetBestSupportedWeightType() const override
     {
         return m_hostWeights.empty() ? InferenceWeightType::Unknown : InferenceWeightType::GenericInt8;
@@ -1025,6 +1079,7 @@ private:
         ReleaseDevice(m_latents); ReleaseDevice(m_weights);
         m_hostWeights.clear();
         m_latentBytes = 0; m_haveLatents = m_haveWeights = false;
+        m_numNeuralLods = 0;
         m_state = NetworkState::Empty;
         ClearErrorMessage();
         return Status::Ok;
@@ -1067,10 +1122,12 @@ private:
         for (int n = 0; n < neuralLods; ++n)
             offset[size_t(n) + 1] = offset[size_t(n)] + uint64_t(gridDim(m_desc.width, n)) * uint64_t(gridDim(m_desc.height, n)) * 2u * layers;
         m_latentBytes = offset[size_t(neuralLods)];
+        m_numNeuralLods = neuralLods;
         for (int mip = 0; mip < m_desc.mips; ++mip) {
             NtcHipMipDesc& d = m_mips[mip];
             d = NtcHipMipDesc{};
             int const nlod = neuralOf(mip, neuralLods);
+            m_neuralLodOfMip[mip] = nlod;
             d.width = std::max(1, m_desc.width >> mip); d.height = std::max(1, m_desc.height >> mip);
             d.hrWidth = gridDim(m_desc.width, nlod); d.hrHeight = gridDim(m_desc.height, nlod);
             d.lrWidth = std::max(d.hrWidth >> 1, 1); d.lrHeight = std::max(d.hrHeight >> 1, 1);
@@ -1082,6 +1139,7 @@ private:
     // Every colour mip owns a high-res grid of half and a low-res grid of a quarter of its size.
     void BuildPerMipGrids()
     {
+        m_numNeuralLods = 0;
         uint64_t cursor = 0;
         for (int mip = 0; mip < m_desc.mips; ++mip) {
             NtcHipMipDesc& d = m_mips[mip];
@@ -1127,6 +1185,8 @@ private:
     void* m_staging = nullptr;
     void* m_latents = nullptr;
     void* m_weights = nullptr;
+    int m_numNeuralLods = 0;                       // shared-LOD geometry only
+    int m_neuralLodOfMip[NTC_HIP_MAX_MIPS] = {};
     std::vector<uint8_t> m_hostWeights;
     ShuffleSource m_shuffle[NTC_HIP_MAX_CHANNELS];
     void ResetShuffle() { for (int ch = 0; ch < NTC_HIP_MAX_CHANNELS; ++ch) m_shuffle[ch] = ShuffleSource::Channel(ch); }

@@ -173,6 +173,10 @@ struct ContextParameters
 // include/libntc/ntc.h (Rect): a rectangle of pixels.
 struct Rect { int left = 0; int top = 0; int width = 0; int height = 0; };
 
+// The latent grids seen as one texture: width x height of the finest grid, one array layer per four
+// features, one mip level per neural LOD (include/libntc/ntc.h:519-528).
+struct LatentTextureDesc { int width = 0; int height = 0; int arraySize = 0; int mipLevels = 0; };
+
 // One image of IContext::ComputeImageDifference: pitch-linear pixels of 1..4 channels (R, G, B, A) in
 // device memory; channels a pixel does not store read as 0, 0, 0, 1.
 struct ImageDesc
@@ -275,6 +279,19 @@ public:
     virtual Status LoadFromFile(char const* fileName) = 0;
     // Storage colour space of a channel as recorded in the file (include/libntc/ntc.h:592-595).
     virtual ColorSpace GetChannelStorageColorSpace(int channel) const = 0;
+
+    // Which colour mips share latent grids (include/libntc/ntc.h:572-591, src/TextureSetMetadata.cpp:109-228).
+    // Meaningful for the LibNTC 0.9.2 geometry, where a neural LOD serves several colour mips; with the
+    // other decoder presets every colour mip owns its grids and these return zeros / Status::Unsupported.
+    virtual LatentTextureDesc GetLatentTextureDesc() const = 0;
+    virtual int GetNumLatentImages() const = 0;
+    // The range of colour mips decoded from the same latent image as mipLevel.
+    virtual Status GetFusedMipLevels(int mipLevel, int* pOutFirstFusedMip, int* pOutLastFusedMip) const = 0;
+    // The range of colour mips whose high-resolution grid is latent image latentImageIndex.
+    virtual Status GetMipLevelsForLatentImage(int latentImageIndex, int* pOutFirstColorMip, int* pOutLastColorMip) const = 0;
+    virtual bool IsInferenceWeightTypeSupported(InferenceWeightType weightType) const = 0;
+    // Accepted for source compatibility; has no effect (include/libntc/ntc.h:942-944).
+    virtual void SetExperimentalKnob(float value) = 0;
 
     // --- additions: raw latents and weights without a file ---
     virtual Status SetDecoderPreset(DecoderPreset preset) = 0;

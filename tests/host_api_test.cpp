@@ -101,12 +101,33 @@ static int cpuChecks()
     CHECK(set->GetWeightDataSize() == 9472);                 // src/WeightLayout.cpp, 48-64-48-32-16
     CHECK(set->GetLatentDataSize() == 44738560ull);          // 4096^2, grid scale 2, 16 features, 13 mips
     CHECK(set->Decompress(nullptr) == Status::InvalidState); // shape set, no data yet
+    // which colour mips share latent images (4096^2, grid scale 2: mips 0-2 -> LOD 0, 3-4 -> 2, 5-6 -> 4, 7-12 -> 6;
+    // eight neural LODs, the odd ones serve as the low-resolution partner only)
+    {
+        CHECK(set->GetNumLatentImages() == 8);
+        LatentTextureDesc const lt = set->GetLatentTextureDesc();
+        CHECK(lt.width == 2048 && lt.height == 2048 && lt.arraySize == 4 && lt.mipLevels == 8);
+        int first = -1, last = -1;
+        CHECK(set->GetFusedMipLevels(0, &first, &last) == Status::Ok && first == 0 && last == 2);
+        CHECK(set->GetFusedMipLevels(4, &first, &last) == Status::Ok && first == 3 && last == 4);
+        CHECK(set->GetFusedMipLevels(9, &first, nullptr) == Status::Ok && first == 7);
+        CHECK(set->GetFusedMipLevels(12, nullptr, &last) == Status::Ok && last == 12);
+        CHECK(set->GetFusedMipLevels(13, &first, &last) == Status::OutOfRange);
+        CHECK(set->GetMipLevelsForLatentImage(0, &first, &last) == Status::Ok && first == 0 && last == 2);
+        CHECK(set->GetMipLevelsForLatentImage(2, &first, &last) == Status::Ok && first == 3 && last == 4);
+        CHECK(set->GetMipLevelsForLatentImage(6, &first, &last) == Status::Ok && first == 7 && last == 12);
+        CHECK(set->GetMipLevelsForLatentImage(1, &first, &last) == Status::OutOfRange);
+        CHECK(set->GetMipLevelsForLatentImage(8, &first, &last) == Status::OutOfRange);
+        CHECK(!set->IsInferenceWeightTypeSupported(InferenceWeightType::GenericInt8));       // no weights yet
+        set->SetExperimentalKnob(1.f);
+    }
     std::vector<unsigned char> blob(9472);
     CHECK(set->SetWeightData(blob.data(), 100) == Status::InvalidArgument);
     CHECK(set->SetWeightData(nullptr, 9472) == Status::InvalidArgument);
     CHECK(set->SetWeightData(blob.data(), blob.size()) == Status::CudaUnavailable);
     CHECK(set->SetDecoderPreset(DecoderPreset::Concat2x2_64) == Status::Ok);
     CHECK(set->GetWeightDataSize() == 10496 && set->GetLatentDataSize() == 22369636ull);
+    CHECK(set->GetNumLatentImages() == 0 && set->GetFusedMipLevels(0, nullptr, nullptr) == Status::Unsupported);   // per-mip grids
     CHECK(set->SetDecoderPreset(DecoderPreset::Concat2x2_48) == Status::Ok);
     CHECK(set->GetWeightDataSize() == 8576);
 
