@@ -305,21 +305,26 @@ typedef struct NtcHipImageDifference {
 } NtcHipImageDifference;
 int ntc_hip_image_difference(const NtcHipImageDifference* params);
 
-/* BC4 / BC5 compression of an image: the block-compression compute pass of
- * IContext::MakeBlockCompressionComputePass for those two formats (include/libntc/ntc.h:1050-1100,
- * src/shaders/CompressBC4.hlsl, CompressBC5.hlsl, BC4_* of src/shaders/BlockCompressCommon.hlsli).
- * widthInBlocks x heightInBlocks blocks of 4 x 4 pixels starting at (srcLeft, srcTop) are encoded from
- * channel R (BC4, 8 bytes per block) or R and G (BC5, 16 bytes) and stored row-major with dstRowPitch
- * bytes per row of blocks, the first at block (dstOffsetX, dstOffsetY).  Pixels outside the image read as
- * 0, like a texture load there.  dstFormat is a BlockCompressedFormat: 4 or 5; the other formats return
- * NTC_HIP_ERR_UNSUPPORTED.  Asynchronous on the library stream. */
+/* BC1 .. BC5 compression of an image: the block-compression compute pass of
+ * IContext::MakeBlockCompressionComputePass for those formats (include/libntc/ntc.h:1050-1100,
+ * src/shaders/CompressBC1.hlsl .. CompressBC5.hlsl, src/shaders/BlockCompressCommon.hlsli).
+ * widthInBlocks x heightInBlocks blocks of 4 x 4 pixels starting at (srcLeft, srcTop) are encoded and
+ * stored row-major with dstRowPitch bytes per row of blocks, the first at block (dstOffsetX, dstOffsetY).
+ * dstFormat is a BlockCompressedFormat:
+ *   1  BC1, 8 bytes per block, from R, G, B and A (pixels with A <= alphaThreshold may become transparent);
+ *   2  BC2, 16 bytes: 4-bit alpha, then a BC1 colour block;
+ *   3  BC3, 16 bytes: a BC4 block of A, then a BC1 colour block;
+ *   4  BC4, 8 bytes, from R;      5  BC5, 16 bytes, from R then G;
+ *   6, 7 (BC6H, BC7) return NTC_HIP_ERR_UNSUPPORTED.
+ * Channels the image does not have read as 0 (alpha as 1); pixels outside the image read as 0 in every
+ * channel, like a texture load there.  Asynchronous on the library stream. */
 typedef struct NtcHipBlockCompress {
     NtcHipImage src;
     int32_t     srcLeft, srcTop;
     int32_t     widthInBlocks, heightInBlocks;
     int32_t     dstFormat;
     int32_t     dstOffsetX, dstOffsetY;       /* in blocks */
-    int32_t     reserved;
+    float       alphaThreshold;               /* BC1 only; the reference's default is 1 / 255 */
     void*       dst;                          /* device, 8-byte aligned */
     uint64_t    dstBytes;
     uint64_t    dstRowPitch;                  /* bytes per row of blocks, multiple of 8 */

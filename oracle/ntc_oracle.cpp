@@ -62,6 +62,15 @@
  *                            of the reference's shader compiler (fused multiply-adds in the
  *                            least-squares fit) are not known: parity with its exact blocks is
  *                            unpinned; blocks are valid BC4 by construction.
+ *   block_compress (BC1/2/3) the single-colour endpoint tables, regenerated from their rule, equal
+ *                            the reference's literal tables entry by entry; the BC1 decoder in
+ *                            numpy: constant blocks within 2.6/255, blocks of two 5:6:5 colours
+ *                            exact, transparent texels decode transparent, smaller error than a
+ *                            plain bounding-box encoder; BC2 alpha against its closed form, BC3
+ *                            alpha against the BC4 encoder (tests/test_block_compress_color.py).
+ *                            HLSL leaves dot / lerp / fusion to the shader compiler: the float
+ *                            operation order here is a choice, parity with the reference's exact
+ *                            blocks is unpinned.
  *   The exact bits of the reference's FP16-WMMA CUDA kernel (half accumulation order,
  *   --use_fast_math) and of a hardware bilinear sampler are NOT reproduced: parity unpinned
  *   for those two, by construction; the integer contract of Inference.hlsli is what is pinned.
@@ -1077,23 +1086,301 @@ uint64_t encode(const float texels[16])                     // hlsli:710-795
 
 } // namespace bc4
 
-// dstFormat 4 (BC4: channel R) or 5 (BC5: R then G); host pointers in `p`.  Returns -1 for other formats.
+// BC1 colour blocks: CompressBC1.hlsl, BC1_* of BlockCompressCommon.hlsli:36-493.  HLSL leaves the
+// evaluation of dot / lerp / fused operations to the shader compiler; here every operation is a
+// separate IEEE binary32 one, dot products add left to right, lerp(a, b, t) = a + (b - a) * t,
+// round() is to nearest even.
+namespace bc1 {
+namespace {         // internal linkage: this file's functions sit in an extern "C" block
+
+// hlsli:36-78: the two tables are the single-colour tables of NVTT.  Their rule, as published with
+// stb_dxt / NVTT: for every 8-bit value, over endpoint pairs (first, second) with `second` in the outer
+// loop, minimise 100 * |(2 * expand(first) + expand(second)) / 3 - value| + 3 * |first - second|
+// (integer division), keeping the first minimum.  tests/ compares the result with the reference's
+// literal tables.
+struct MatchTables {
+    uint16_t five[256], six[256];
+    MatchTables()
+    {
+        for (int bits = 5; bits <= 6; ++bits)
+            for (int value = 0; value < 256; ++value) {
+                int best = INT32_MAX, pick = 0;
+                for (int second = 0; second < (1 << bits); ++second)
+                    for (int first = 0; first < (1 << bits); ++first) {
+                        int const a = bits == 5 ? (first << 3) | (first >> 2) : (first << 2) | (first >> 4);
+                        int const b = bits == 5 ? (second << 3) | (second >> 2) : (second << 2) | (second >> 4);
+                        int const cost = 100 * std::abs((2 * a + b) / 3 - value) + 3 * std::abs(first - second);
+                        if (cost < best) { best = cost; pick = first | (second << 8); }
+                    }
+                (bits == 5 ? five : six)[value] = uint16_t(pick);
+            }
+    }
+};
+MatchTables const& match_tables() { static MatchTables const t; return t; }
+
+float sat(float v) { return std::fmin(std::fmax(v, 0.f), 1.f); }
+float dist2(const float a[3], const float b[3])
+{
+    float const d0 = a[0] - b[0], d1 = a[1] - b[1], d2 = a[2] - b[2];
+    return d0 * d0 + d1 * d1 + d2 * d2;
+}
+void lerp3(const float a[3], const float b[3], float t, float out[3]) { for (int c = 0; c < 3; ++c) out[c] = a[c] + (b[c] - a[c]) * t; }
+void expand565(uint32_t w, float out[3])                                 // hlsli:181-188
+{
+    out[0] = float((w >> 11) & 0x1f) / 31.f; out[1] = float((w >> 5) & 0x3f) / 63.f; out[2] = float(w & 0x1f) / 31.f;
+}
+uint32_t round565(float v[3])                                            // hlsli:190-203, v becomes the rounded colour
+{
+    uint32_t const x = uint32_t(std::nearbyint(sat(v[0]) * 31.f)), y = uint32_t(std::nearbyint(sat(v[1]) * 63.f)), z = uint32_t(std::nearbyint(sat(v[2]) * 31.f));
+    v[0] = float(x) / 31.f; v[1] = float(y) / 63.f; v[2] = float(z) / 31.f;
+    return (x << 11) | (y << 5) | z;
+}
+uint32_t select_index(const float d[4], float& error)                    // hlsli:116-144
+{
+    uint32_t k;
+    if (std::fmin(d[0], d[1]) < std::fmin(d[2], d[3])) k = d[0] < d[1] ? 0 : 1;
+    else k = d[2] < d[3] ? 2 : 3;
+    error = d[k];
+    return k;
+}
+uint32_t index4(const float px[4], const float hi[3], const float lo[3], float& error)      // hlsli:146-159
+{
+    float c2[3], c3[3], d[4];
+    lerp3(hi, lo, 1.f / 3.f, c2); lerp3(hi, lo, 2.f / 3.f, c3);
+    float const alphaDistance = (1.f - px[3]) * (1.f - px[3]);
+    d[0] = dist2(hi, px) + alphaDistance; d[1] = dist2(lo, px) + alphaDistance;
+    d[2] = dist2(c2, px) + alphaDistance; d[3] = dist2(c3, px) + alphaDistance;
+    return select_index(d, error);
+}
+uint32_t index3(const float px[4], const float hi[3], const float lo[3], float threshold, float& error)     // hlsli:161-179
+{
+    if (px[3] <= threshold) { error = 0.f; return 3; }
+    float c2[3], d[4];
+    lerp3(hi, lo, 0.5f, c2);
+    float const alphaDistance = (1.f - px[3]) * (1.f - px[3]);
+    d[0] = dist2(hi, px) + alphaDistance; d[1] = dist2(lo, px) + alphaDistance; d[2] = dist2(c2, px) + alphaDistance;
+    d[3] = px[0] * px[0] + px[1] * px[1] + px[2] * px[2] + px[3] * px[3];
+    return select_index(d, error);
+}
+
+struct Result { uint32_t x, y; float error; };
+
+Result transparent_block(const float px[16][4], float threshold)        // hlsli:99-109
+{
+    Result r{ 0u, 0xffffffffu, 0.f };
+    for (int t = 0; t < 16; ++t)
+        if (!(px[t][3] <= threshold)) r.error += px[t][0] * px[t][0] + px[t][1] * px[t][1] + px[t][2] * px[t][2] + px[t][3] * px[t][3];
+    return r;
+}
+
+Result single_color(const float px[16][4])                               // hlsli:205-247
+{
+    float avg[3] = { 0.f, 0.f, 0.f };
+    for (int t = 0; t < 16; ++t) for (int c = 0; c < 3; ++c) avg[c] += px[t][c];
+    uint32_t m[3];
+    for (int c = 0; c < 3; ++c) {
+        // the reference indexes its table with the rounded mean unchecked; outside [0, 255] (inputs outside
+        // [0, 1]) that read is undefined there and clamped here
+        float const i = std::fmin(std::fmax(std::nearbyint(avg[c] / 16.f * 255.f), 0.f), 255.f);
+        m[c] = (c == 1 ? match_tables().six : match_tables().five)[int(i)];
+    }
+    uint32_t const color0 = ((m[0] & 0x1f) << 11) | ((m[1] & 0x3f) << 5) | (m[2] & 0x1f);
+    uint32_t const color1 = (((m[0] >> 8) & 0x1f) << 11) | (((m[1] >> 8) & 0x3f) << 5) | ((m[2] >> 8) & 0x1f);
+    Result r;
+    if (color0 < color1) { r.x = (color0 << 16) | color1; r.y = 0xffffffffu; }
+    else                 { r.x = (color1 << 16) | color0; r.y = 0xaaaaaaaau; }
+    float e0[3], e1[3], enc[3];
+    expand565(color0, e0); expand565(color1, e1); lerp3(e0, e1, 1.f / 3.f, enc);
+    r.error = 0.f;
+    for (int t = 0; t < 16; ++t) {
+        float const d0 = px[t][0] - enc[0], d1 = px[t][1] - enc[1], d2 = px[t][2] - enc[2], d3 = px[t][3] - 1.f;
+        r.error += d0 * d0 + d1 * d1 + d2 * d2 + d3 * d3;
+    }
+    return r;
+}
+
+// Shared start of both fitted modes (hlsli:251-290, 380-424): bounding box of the texels in `use`,
+// component ends swapped by covariance sign, inset by extent / divisor.
+void start_box(const float px[16][4], const bool use[16], float divisor, int count, float lo[3], float hi[3])
+{
+    float sums[3] = { 0, 0, 0 };
+    for (int c = 0; c < 3; ++c) { lo[c] = 1.f; hi[c] = 0.f; }
+    for (int t = 0; t < 16; ++t) if (use[t])
+        for (int c = 0; c < 3; ++c) { sums[c] += px[t][c]; lo[c] = std::fmin(lo[c], px[t][c]); hi[c] = std::fmax(hi[c], px[t][c]); }
+    float center[3] = { 0, 0, 0 };
+    if (count > 0) for (int c = 0; c < 3; ++c) center[c] = sums[c] / float(count);
+    float rg = 0, rb = 0, gb = 0;
+    for (int t = 0; t < 16; ++t) if (use[t]) {
+        float const r = px[t][0] - center[0], g = px[t][1] - center[1], b = px[t][2] - center[2];
+        rg += r * g; rb += r * b; gb += g * b;
+    }
+    if (lo[0] != hi[0]) {
+        if (rg < 0) std::swap(lo[1], hi[1]);
+        if (rb < 0) std::swap(lo[2], hi[2]);
+    } else if (lo[1] != hi[1]) {
+        if (gb < 0) std::swap(lo[2], hi[2]);
+    }
+    for (int c = 0; c < 3; ++c) {
+        float const inset = (hi[c] - lo[c]) / divisor;
+        hi[c] = sat(hi[c] - inset);
+        lo[c] = sat(lo[c] + inset);
+    }
+}
+
+struct Sums { float a2 = 0, b2 = 0, ab = 0, ax[3] = { 0, 0, 0 }, bx[3] = { 0, 0, 0 }; };
+void accumulate(Sums& s, float beta, const float px[4])
+{
+    float const alpha = 1.f - beta;
+    s.a2 += alpha * alpha; s.b2 += beta * beta; s.ab += alpha * beta;
+    for (int c = 0; c < 3; ++c) { s.ax[c] += alpha * px[c]; s.bx[c] += beta * px[c]; }
+}
+bool solve(Sums const& s, float a[3], float b[3])
+{
+    float const denom = s.a2 * s.b2 - s.ab * s.ab;
+    if (!(std::fabs(denom) > 0.0001f)) return false;
+    float const factor = 1.f / denom;
+    for (int c = 0; c < 3; ++c) {
+        a[c] = (s.ax[c] * s.b2 - s.bx[c] * s.ab) * factor;
+        b[c] = (s.bx[c] * s.a2 - s.ax[c] * s.ab) * factor;
+    }
+    return true;
+}
+void keep_extremes(float cur[3], const float fitted[3])                 // "preserve 0 and 1 cases"
+{
+    for (int c = 0; c < 3; ++c) if (!(cur[c] == 0.f || cur[c] == 1.f)) cur[c] = sat(fitted[c]);
+}
+
+Result compress_fast(const float px[16][4])                              // hlsli:249-376
+{
+    bool all[16]; for (bool& u : all) u = true;
+    float lo[3], hi[3];
+    start_box(px, all, 16.f, 16, lo, hi);
+    uint32_t color0 = 0, color1 = 0;
+    for (int pass = 0; pass < 4; ++pass) {
+        Sums s;
+        for (int t = 0; t < 16; ++t) {
+            float e;
+            uint32_t const index = index4(px[t], hi, lo, e);
+            float beta = float(index & 1);
+            if (index & 2) beta = (1 + beta) / 3.0f;
+            accumulate(s, beta, px[t]);
+        }
+        float a[3], b[3];
+        if (solve(s, a, b)) { keep_extremes(lo, b); keep_extremes(hi, a); }
+        uint32_t const new0 = round565(hi), new1 = round565(lo);
+        if (new0 == color0 && new1 == color1) break;
+        color0 = new0; color1 = new1;
+    }
+    if (color0 == color1) {
+        if (color0 == 0) { color0 = 1; expand565(color0, hi); }
+        else { color1 = color0 - 1; expand565(color1, lo); }
+    } else if (color0 < color1) {
+        for (int c = 0; c < 3; ++c) std::swap(hi[c], lo[c]);
+        std::swap(color0, color1);
+    }
+    Result r{ (color1 << 16) | color0, 0u, 0.f };
+    for (int t = 0; t < 16; ++t) {
+        float e;
+        r.y |= index4(px[t], hi, lo, e) << (2 * t);
+        r.error += e;
+    }
+    return r;
+}
+
+Result compress_fast_alpha(const float px[16][4], float threshold)       // hlsli:378-493
+{
+    bool opaque[16]; int count = 0;
+    for (int t = 0; t < 16; ++t) { opaque[t] = !(px[t][3] <= threshold); count += opaque[t]; }
+    float lo[3], hi[3];
+    start_box(px, opaque, float(count), count, lo, hi);
+    Sums s;
+    for (int t = 0; t < 16; ++t) {
+        float e;
+        uint32_t const index = index3(px[t], hi, lo, threshold, e);
+        if (index != 3) accumulate(s, (index & 2) ? 0.5f : float(index & 1), px[t]);
+    }
+    float a[3], b[3];
+    if (solve(s, a, b)) { keep_extremes(lo, a); keep_extremes(hi, b); }     // a -> min, b -> max: as written at hlsli:453-455
+    uint32_t color0 = round565(hi), color1 = round565(lo);
+    if (color0 > color1) {
+        for (int c = 0; c < 3; ++c) std::swap(hi[c], lo[c]);
+        std::swap(color0, color1);
+    }
+    Result r{ (color1 << 16) | color0, 0u, 0.f };
+    for (int t = 0; t < 16; ++t) {
+        float e;
+        uint32_t const index = index3(px[t], hi, lo, threshold, e);
+        r.y |= index << (2 * t);
+        if (index != 3 || opaque[t]) r.error += e;
+    }
+    return r;
+}
+
+// CompressBC1.hlsl:31-63 (withAlpha) / CompressBC2.hlsl, CompressBC3.hlsl:32-43 (alpha forced to 1 by the caller)
+uint64_t encode_color(const float px[16][4], bool withAlpha, float threshold)
+{
+    Result best;
+    if (withAlpha) {
+        best = transparent_block(px, threshold);
+        Result const one = single_color(px);
+        if (one.error < best.error) best = one;
+    } else best = single_color(px);
+    Result const four = compress_fast(px);
+    if (four.error < best.error) best = four;
+    if (withAlpha) {
+        Result const three = compress_fast_alpha(px, threshold);
+        if (three.error < best.error) best = three;
+    }
+    return uint64_t(best.x) | (uint64_t(best.y) << 32);
+}
+
+uint64_t bc2_alpha(const float alpha[16])                                // hlsli:495-508
+{
+    uint64_t v = 0;
+    for (int t = 0; t < 16; ++t) v |= uint64_t(uint32_t(std::nearbyint(sat(alpha[t]) * 15.f))) << (4 * t);
+    return v;
+}
+
+} // namespace
+} // namespace bc1
+
+// For tests: the single-colour tables (256 entries each, first endpoint | second << 8).
+void ntc_oracle_bc1_match_tables(uint16_t* five, uint16_t* six)
+{
+    std::memcpy(five, bc1::match_tables().five, 512);
+    std::memcpy(six, bc1::match_tables().six, 512);
+}
+
+// dstFormat 1..5 (BC1, BC2, BC3, BC4: channel R, BC5: R then G); host pointers in `p`.  Returns -1 for other formats.
 int ntc_oracle_block_compress(const NtcHipBlockCompress* p)
 {
-    if (p->dstFormat != 4 && p->dstFormat != 5) return -1;
-    int const channels = p->dstFormat == 4 ? 1 : 2;
+    if (p->dstFormat < 1 || p->dstFormat > 5) return -1;
     auto fetch = [&](int x, int y, int c) -> float {
         if (x < 0 || y < 0 || x >= p->src.width || y >= p->src.height) return 0.f;
         return diff_channel(p->src, static_cast<uint8_t const*>(p->src.data) + size_t(y) * p->src.rowPitch + size_t(x) * p->src.pixelStride, c);
     };
+    size_t const blockBytes = (p->dstFormat == 1 || p->dstFormat == 4) ? 8 : 16;
     for (int by = 0; by < p->heightInBlocks; ++by)
-        for (int bx = 0; bx < p->widthInBlocks; ++bx)
-            for (int c = 0; c < channels; ++c) {
-                float texels[16];
-                for (int t = 0; t < 16; ++t) texels[t] = fetch(p->srcLeft + bx * 4 + (t & 3), p->srcTop + by * 4 + (t >> 2), c);
-                uint64_t const bits = bc4::encode(texels);
-                std::memcpy(static_cast<uint8_t*>(p->dst) + size_t(by + p->dstOffsetY) * p->dstRowPitch + (size_t(bx + p->dstOffsetX) * channels + c) * 8, &bits, 8);
+        for (int bx = 0; bx < p->widthInBlocks; ++bx) {
+            uint64_t words[2] = { 0, 0 };
+            if (p->dstFormat >= 4) {
+                for (int c = 0; c < p->dstFormat - 3; ++c) {
+                    float texels[16];
+                    for (int t = 0; t < 16; ++t) texels[t] = fetch(p->srcLeft + bx * 4 + (t & 3), p->srcTop + by * 4 + (t >> 2), c);
+                    words[c] = bc4::encode(texels);
+                }
+            } else {
+                float px[16][4], alpha[16];
+                for (int t = 0; t < 16; ++t) {
+                    for (int c = 0; c < 4; ++c) px[t][c] = fetch(p->srcLeft + bx * 4 + (t & 3), p->srcTop + by * 4 + (t >> 2), c);
+                    if (p->dstFormat != 1) { alpha[t] = px[t][3]; px[t][3] = 1.f; }
+                }
+                uint64_t const color = bc1::encode_color(px, p->dstFormat == 1, p->alphaThreshold);
+                if (p->dstFormat == 1) words[0] = color;
+                else { words[0] = p->dstFormat == 2 ? bc1::bc2_alpha(alpha) : bc4::encode(alpha); words[1] = color; }
             }
+            std::memcpy(static_cast<uint8_t*>(p->dst) + size_t(by + p->dstOffsetY) * p->dstRowPitch + size_t(bx + p->dstOffsetX) * blockBytes, words, blockBytes);
+        }
     return 0;
 }
 

@@ -110,7 +110,7 @@ class ImageDifference(C.Structure):
 class BlockCompress(C.Structure):
     _fields_ = [
         ("src", Image), ("srcLeft", C.c_int32), ("srcTop", C.c_int32), ("widthInBlocks", C.c_int32), ("heightInBlocks", C.c_int32),
-        ("dstFormat", C.c_int32), ("dstOffsetX", C.c_int32), ("dstOffsetY", C.c_int32), ("reserved", C.c_int32),
+        ("dstFormat", C.c_int32), ("dstOffsetX", C.c_int32), ("dstOffsetY", C.c_int32), ("alphaThreshold", C.c_float),
         ("dst", C.c_void_p), ("dstBytes", C.c_uint64), ("dstRowPitch", C.c_uint64),
     ]
 

@@ -130,8 +130,9 @@ struct BlockCompressArgs {
     uint64_t pixelStride, rowPitch, dstRowPitch;
     int32_t srcWidth, srcHeight, format, numChannels;
     int32_t srcLeft, srcTop, widthInBlocks, heightInBlocks, dstOffsetX, dstOffsetY;
+    float alphaThreshold;       // BC1: texels with alpha <= threshold are transparent
 };
-hipError_t launch_block_compress(BlockCompressArgs const& args, int channels, hipStream_t stream);
+hipError_t launch_block_compress(BlockCompressArgs const& args, int dstFormat /* 1..5 */, hipStream_t stream);
 
 hipError_t launch_decode(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream);
 hipError_t launch_queries(int variant, DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries,

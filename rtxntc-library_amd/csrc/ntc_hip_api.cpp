@@ -855,8 +855,8 @@ int ntc_hip_block_compress(const NtcHipBlockCompress* p)
     if (int r = require_init()) return r;
     if (!p || !p->dst) { set_error("ntc_hip_block_compress: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
     if (p->dstFormat < 1 || p->dstFormat > 7) { set_error("ntc_hip_block_compress: dstFormat (%d) is not a block-compressed format.", p->dstFormat); return NTC_HIP_ERR_INVALID_ARG; }
-    if (p->dstFormat != 4 && p->dstFormat != 5) {
-        set_error("ntc_hip_block_compress: only BC4 and BC5 are implemented (dstFormat %d).", p->dstFormat);
+    if (p->dstFormat > 5) {
+        set_error("ntc_hip_block_compress: BC6H and BC7 are not implemented (dstFormat %d).", p->dstFormat);
         return NTC_HIP_ERR_UNSUPPORTED;
     }
     if (p->srcLeft < 0 || p->srcTop < 0 || p->widthInBlocks < 1 || p->heightInBlocks < 1 || p->dstOffsetX < 0 || p->dstOffsetY < 0
@@ -867,7 +867,7 @@ int ntc_hip_block_compress(const NtcHipBlockCompress* p)
     BlockCompressArgs a{};
     DiffImageArgs image{};
     if (int r = check_diff_image(p->src, "src", 0, 0, 1, 1, image)) return r;     // the extent may reach past the image: such pixels read as 0
-    uint64_t const blockBytes = p->dstFormat == 4 ? 8u : 16u;
+    uint64_t const blockBytes = (p->dstFormat == 1 || p->dstFormat == 4) ? 8u : 16u;
     uint64_t const rowNeed = uint64_t(p->dstOffsetX + p->widthInBlocks) * blockBytes;
     if ((p->dstRowPitch & 7u) || p->dstRowPitch < rowNeed || (reinterpret_cast<uintptr_t>(p->dst) & 7u)
         || uint64_t(p->dstOffsetY + p->heightInBlocks - 1) * p->dstRowPitch + rowNeed > p->dstBytes) {
@@ -879,7 +879,8 @@ int ntc_hip_block_compress(const NtcHipBlockCompress* p)
     a.dst = static_cast<uint8_t*>(p->dst); a.dstRowPitch = p->dstRowPitch;
     a.srcLeft = p->srcLeft; a.srcTop = p->srcTop; a.widthInBlocks = p->widthInBlocks; a.heightInBlocks = p->heightInBlocks;
     a.dstOffsetX = p->dstOffsetX; a.dstOffsetY = p->dstOffsetY;
-    HIP_TRY(launch_block_compress(a, p->dstFormat == 4 ? 1 : 2, g_lib.stream));
+    a.alphaThreshold = p->alphaThreshold;
+    HIP_TRY(launch_block_compress(a, p->dstFormat, g_lib.stream));
     clear_error();
     return 0;
 }

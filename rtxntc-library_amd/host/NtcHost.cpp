@@ -1245,6 +1245,7 @@ public:
         p.srcLeft = params.srcRect.left; p.srcTop = params.srcRect.top;
         p.widthInBlocks = (params.srcRect.width + 3) / 4; p.heightInBlocks = (params.srcRect.height + 3) / 4;
         p.dstFormat = int32_t(params.dstFormat);
+        p.alphaThreshold = params.alphaThreshold;
         p.dstOffsetX = params.dstOffsetInBlocks.x; p.dstOffsetY = params.dstOffsetInBlocks.y;
         p.dst = params.pDstData; p.dstBytes = params.dstDataSize; p.dstRowPitch = params.dstRowPitch;
         if (int r = ntc_hip_block_compress(&p)) return DeviceFailure(r);

@@ -205,7 +205,7 @@ struct ImageDifferenceParameters
     uint32_t outputOffset = 0;          // bytes, multiple of 8
 };
 
-// The fields of MakeBlockCompressionComputePassParameters (include/libntc/ntc.h:1050-1100) that BC4 and
+// The fields of MakeBlockCompressionComputePassParameters (include/libntc/ntc.h:1050-1100) that BC1 ..
 // BC5 use, plus what a graphics application binds to that pass: the source image and the destination.
 struct Point { int x = 0; int y = 0; };
 struct BlockCompressionParameters
@@ -213,9 +213,9 @@ struct BlockCompressionParameters
     ImageDesc srcImage;                 // device memory
     Rect srcRect;                       // pixels to compress; width and height are rounded up to whole blocks
     Point dstOffsetInBlocks;
-    BlockCompressedFormat dstFormat = BlockCompressedFormat::None;      // BC4 or BC5
-    float alphaThreshold = 1.f / 255.f; // BC1 only in the reference; unused here
-    void* pDstData = nullptr;           // device memory: rows of 8-byte (BC4) or 16-byte (BC5) blocks
+    BlockCompressedFormat dstFormat = BlockCompressedFormat::None;      // BC1 .. BC5
+    float alphaThreshold = 1.f / 255.f; // BC1: pixels with alpha at or below it may become transparent
+    void* pDstData = nullptr;           // device memory: rows of 8-byte (BC1, BC4) or 16-byte (BC2, BC3, BC5) blocks
     size_t dstDataSize = 0;
     size_t dstRowPitch = 0;             // bytes per row of blocks
 };
@@ -376,9 +376,8 @@ public:
     // on the device, asynchronously; DecodeImageDifferenceResult converts the four results.
     virtual Status ComputeImageDifference(ImageDifferenceParameters const& params) const = 0;
     // Runs the block-compression pass that IContext::MakeBlockCompressionComputePass describes for a
-    // graphics API (include/libntc/ntc.h:1213-1225, src/Context.cpp, src/shaders/CompressBC4.hlsl and
-    // CompressBC5.hlsl) on the device, asynchronously.  BC4 and BC5 only: the other formats return
-    // Status::Unsupported.
+    // graphics API (include/libntc/ntc.h:1213-1225, src/Context.cpp:630-779, src/shaders/CompressBC1.hlsl ..
+    // CompressBC5.hlsl) on the device, asynchronously.  BC1 .. BC5; BC6 and BC7 return Status::Unsupported.
     virtual Status CompressBlocks(BlockCompressionParameters const& params) const = 0;
     // True when a gfx950 device was initialised (reference: IsCudaAvailable).
     virtual bool IsCudaAvailable() const = 0;

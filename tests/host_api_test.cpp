@@ -461,6 +461,15 @@ static int imageDifference()
                 uint64_t const want = corner ? 0ull : 0xFFFFull;
                 CHECK(blocks[(by * blocksX + bx) * 2] == want && blocks[(by * blocksX + bx) * 2 + 1] == want);
             }
+        // BC1 of the same image: opaque white is the single-colour block of 0xFFFF twice with every index 2,
+        // the zero corner (alpha 0) the all-transparent block
+        bp.dstFormat = BlockCompressedFormat::BC1; bp.dstRowPitch = blocksX * 8;
+        CHECK(ctx->CompressBlocks(bp) == Status::Ok);
+        CHECK(ntc_hip_download(blocks.data(), dBlocks, blocksX * blocksY * 8) == 0);
+        for (size_t by = 0; by < blocksY; ++by)
+            for (size_t bx = 0; bx < blocksX; ++bx)
+                CHECK(blocks[by * blocksX + bx] == ((bx < 8 && by < 4) ? 0xFFFFFFFF00000000ull : 0xAAAAAAAAFFFFFFFFull));
+        bp.dstRowPitch = blocksX * 16;
         bp.dstFormat = BlockCompressedFormat::BC7;
         CHECK(ctx->CompressBlocks(bp) == Status::Unsupported);
         bp.dstFormat = BlockCompressedFormat::None;

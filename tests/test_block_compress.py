@@ -217,7 +217,7 @@ def test_gpu_block_compress_matches_checker(ntc, device, oracle, fmt, dst_format
         bad = np.argwhere(got != want)
         assert bad.size == 0, (fmt, dst_format, len(bad), bad[:3], [hex(int(got[tuple(b)])) for b in bad[:3]], [hex(int(want[tuple(b)])) for b in bad[:3]])
     # argument checks
-    p.dstFormat = 1
+    p.dstFormat = 6
     assert device.lib.ntc_hip_block_compress(p) == ntc.abi.ERR_UNSUPPORTED
     p.dstFormat = 9
     assert device.lib.ntc_hip_block_compress(p) == ntc.abi.ERR_INVALID_ARG
