@@ -695,4 +695,29 @@ hipError_t launch_read_channels(ReadChannelsArgs const& args, hipStream_t stream
     return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------------------------
+// Byte fill (what a memset does, as a kernel: the library clears memory only this way).  The
+// 16-byte-aligned middle goes out as uint4 stores, the unaligned ends byte by byte.
+__global__ void __launch_bounds__(256)
+fill_kernel(uint8_t* dst, uint32_t pattern, uint64_t headBytes, uint64_t vectors, uint64_t tailBytes)
+{
+    uint64_t const stride = uint64_t(gridDim.x) * blockDim.x, first = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    uint4* const body = reinterpret_cast<uint4*>(dst + headBytes);
+    for (uint64_t i = first; i < vectors; i += stride) body[i] = make_uint4(pattern, pattern, pattern, pattern);
+    if (first < headBytes) dst[first] = uint8_t(pattern);
+    if (first < tailBytes) dst[headBytes + vectors * 16u + first] = uint8_t(pattern);
+}
+
+hipError_t launch_fill(uint8_t* dst, uint8_t value, uint64_t bytes, hipStream_t stream)
+{
+    if (bytes == 0) return hipSuccess;
+    uint64_t const misaligned = reinterpret_cast<uintptr_t>(dst) & 15u;
+    uint64_t const headBytes = misaligned ? (16u - misaligned < bytes ? 16u - misaligned : bytes) : 0u;
+    uint64_t const vectors = (bytes - headBytes) / 16u, tailBytes = bytes - headBytes - vectors * 16u;
+    uint64_t const groups = (vectors + 255u) / 256u;
+    uint32_t const grid = uint32_t(groups < 1u ? 1u : (groups > 16384u ? 16384u : groups));
+    hipLaunchKernelGGL(fill_kernel, dim3(grid), dim3(256), 0, stream, dst, uint32_t(value) * 0x01010101u, headBytes, vectors, tailBytes);
+    return hipGetLastError();
+}
+
 } // namespace ntc_hip_dev

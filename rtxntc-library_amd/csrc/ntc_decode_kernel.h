@@ -132,6 +132,8 @@ struct BlockCompressArgs {
     int32_t srcLeft, srcTop, widthInBlocks, heightInBlocks, dstOffsetX, dstOffsetY;
     float alphaThreshold;       // BC1: texels with alpha <= threshold are transparent
 };
+// Sets `bytes` bytes at dst to `value` (any alignment).
+hipError_t launch_fill(uint8_t* dst, uint8_t value, uint64_t bytes, hipStream_t stream);
 hipError_t launch_block_compress(BlockCompressArgs const& args, int dstFormat /* 1..5 */, hipStream_t stream);
 
 hipError_t launch_decode(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream);

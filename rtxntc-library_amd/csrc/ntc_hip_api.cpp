@@ -63,6 +63,10 @@ int require_init()
     return 0;
 }
 
+// Caller-given strides and offsets enter 64-bit size products: bounded so that none can wrap.
+constexpr uint64_t kMaxRowPitch = uint64_t(1) << 40, kMaxPixelStride = uint64_t(1) << 20;
+bool reaches_past(uint64_t offset, uint64_t bytes, uint64_t bufferBytes) { return bytes > bufferBytes || offset > bufferBytes - bytes; }
+
 bool spec_equal(NtcHipDecoderSpec const& a, NtcHipDecoderSpec const& b) { return std::memcmp(&a, &b, sizeof(a)) == 0; }
 
 int layer_in(NtcHipDecoderSpec const& s, int l) { return l == 0 ? s.inputChannels : s.hiddenChannels[l - 1]; }
@@ -240,7 +244,8 @@ int build_table(NtcHipTextureSet const* sets, int32_t numSets, std::vector<DevMi
             return NTC_HIP_ERR_INVALID_ARG;
         }
         int const bytesPerChannel = set.outputFormat == NTC_HIP_OUT_UNORM8_PIXELS ? 1 : 2;
-        if (!forQueries && set.outputFormat != NTC_HIP_OUT_FP16_PLANAR_PAIRS && set.outPixelStride < set.numChannels * bytesPerChannel) {
+        if (!forQueries && set.outputFormat != NTC_HIP_OUT_FP16_PLANAR_PAIRS
+            && (set.outPixelStride < set.numChannels * bytesPerChannel || uint64_t(set.outPixelStride) > kMaxPixelStride)) {
             set_error("ntc_hip_decode: set %d: pixel stride %d is smaller than %d channels.", s, set.outPixelStride, set.numChannels);
             return NTC_HIP_ERR_INVALID_ARG;
         }
@@ -256,13 +261,13 @@ int build_table(NtcHipTextureSet const* sets, int32_t numSets, std::vector<DevMi
                 // no per-mip output
             } else if (set.outputFormat == NTC_HIP_OUT_FP16_PLANAR_PAIRS) {
                 if (d.outOffset & 3u) { set_error("ntc_hip_decode: set %d mip %d: planar output offset must be 4-byte aligned.", s, m); return NTC_HIP_ERR_INVALID_ARG; }
-            } else if (d.outRowPitch < uint64_t(d.width) * uint64_t(set.outPixelStride)) {
+            } else if (d.outRowPitch < uint64_t(d.width) * uint64_t(set.outPixelStride) || d.outRowPitch > kMaxRowPitch) {
                 set_error("ntc_hip_decode: set %d mip %d: row pitch smaller than a row.", s, m);
                 return NTC_HIP_ERR_INVALID_ARG;
             }
             uint64_t const hrBytes = grid_bytes(d.hrWidth, d.hrHeight, set.spec.hrFeatures, set.spec.hrBits);
             uint64_t const lrBytes = grid_bytes(d.lrWidth, d.lrHeight, set.spec.lrFeatures, set.spec.lrBits);
-            if (d.hrOffset + hrBytes > set.latentsBytes || d.lrOffset + lrBytes > set.latentsBytes) {
+            if (reaches_past(d.hrOffset, hrBytes, set.latentsBytes) || reaches_past(d.lrOffset, lrBytes, set.latentsBytes)) {
                 set_error("ntc_hip_decode: set %d mip %d: a latent grid reaches past the %llu-byte latent buffer.", s, m,
                           (unsigned long long)set.latentsBytes);
                 return NTC_HIP_ERR_INVALID_ARG;
@@ -273,7 +278,7 @@ int build_table(NtcHipTextureSet const* sets, int32_t numSets, std::vector<DevMi
             else
                 outBytes = uint64_t(d.height - 1) * d.outRowPitch + uint64_t(d.width - 1) * uint64_t(set.outPixelStride)
                          + uint64_t(set.numChannels * bytesPerChannel);
-            if (!forQueries && d.outOffset + outBytes > set.outputBytes) {
+            if (!forQueries && reaches_past(d.outOffset, outBytes, set.outputBytes)) {
                 set_error("ntc_hip_decode: set %d mip %d: output reaches past the %llu-byte output buffer.", s, m,
                           (unsigned long long)set.outputBytes);
                 return NTC_HIP_ERR_INVALID_ARG;
@@ -466,7 +471,7 @@ int ntc_hip_memset(void* dst, int value, size_t bytes)
     if (int r = require_init()) return r;
     if (bytes == 0) return 0;
     if (!dst) { set_error("ntc_hip_memset: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
-    HIP_TRY(hipMemsetAsync(dst, value, bytes, g_lib.stream));
+    HIP_TRY(launch_fill(static_cast<uint8_t*>(dst), uint8_t(value), bytes, g_lib.stream));    // a kernel, not hipMemsetAsync
     return 0;
 }
 
@@ -547,6 +552,7 @@ static int run_queries(const NtcHipTextureSet* set, const NtcHipQuery* queries, 
     if (int r = require_init()) return r;
     if (!set || !queries || !out) { set_error("ntc_hip_decode_queries: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
     if (numQueries == 0) { if (outMs) *outMs = 0.f; return 0; }
+    if (numQueries > (uint64_t(1) << 40)) { set_error("ntc_hip_decode_queries: too many queries in one call."); return NTC_HIP_ERR_INVALID_ARG; }
     if (outBytes < numQueries * 32u) { set_error("ntc_hip_decode_queries: the output buffer holds %llu bytes, %llu queries need %llu.", (unsigned long long)outBytes, (unsigned long long)numQueries, (unsigned long long)(numQueries * 32u)); return NTC_HIP_ERR_INVALID_ARG; }
     if ((reinterpret_cast<uintptr_t>(out) & 7u) || (reinterpret_cast<uintptr_t>(queries) & 3u)) { set_error("ntc_hip_decode_queries: output must be 8-byte and queries 4-byte aligned."); return NTC_HIP_ERR_INVALID_ARG; }
     std::vector<DevMip> table;
@@ -590,7 +596,7 @@ int ntc_hip_build_query_latents(const NtcHipTextureSet* set, void* dst, uint64_t
     }
     for (BrickGrid const& g : plan.grids) {
         uint64_t const srcBytes = uint64_t(g.width) * uint64_t(g.height) * 2u * uint64_t(g.layers);
-        if ((g.srcOffset & 1u) || g.srcOffset + srcBytes > set->latentsBytes || srcBytes >= (1ull << 32)) {
+        if ((g.srcOffset & 1u) || reaches_past(g.srcOffset, srcBytes, set->latentsBytes) || srcBytes >= (1ull << 32)) {
             set_error("ntc_hip_build_query_latents: a latent grid reaches past the %llu-byte latent buffer.", (unsigned long long)set->latentsBytes);
             return NTC_HIP_ERR_INVALID_ARG;
         }
@@ -645,7 +651,7 @@ int ntc_hip_read_channels(const NtcHipReadChannels* p)
     }
     bool const resample = p->dstWidth > 0 && (p->dstWidth != p->width || p->dstHeight != p->height);
     int const imageWidth = resample ? p->dstWidth : p->width, imageHeight = resample ? p->dstHeight : p->height;
-    if (p->pixelStride < uint64_t(bpc) || p->rowPitch < p->pixelStride * uint64_t(imageWidth)
+    if (p->pixelStride < uint64_t(bpc) || p->pixelStride > kMaxPixelStride || p->rowPitch > kMaxRowPitch || p->rowPitch < p->pixelStride * uint64_t(imageWidth)
         || (p->pixelStride % uint64_t(bpc)) || (p->rowPitch % uint64_t(bpc)) || (reinterpret_cast<uintptr_t>(p->dst) % uintptr_t(bpc))) {
         set_error("ntc_hip_read_channels: pixel stride / row pitch do not fit the format.");
         return NTC_HIP_ERR_INVALID_ARG;
@@ -705,8 +711,8 @@ int ntc_hip_write_channels(const NtcHipWriteChannels* p)
     }
     bool const resample = p->srcWidth > 0 && (p->srcWidth != p->width || p->srcHeight != p->height);
     int const imageWidth = resample ? p->srcWidth : p->width, imageHeight = resample ? p->srcHeight : p->height;
-    if (p->pixelStride < uint64_t(bpc) * uint64_t(p->numChannels) || p->rowPitch < p->pixelStride * uint64_t(imageWidth)
-        || (p->pixelStride % uint64_t(bpc)) || (p->rowPitch % uint64_t(bpc)) || (reinterpret_cast<uintptr_t>(p->src) % uintptr_t(bpc))) {
+    if (p->pixelStride < uint64_t(bpc) * uint64_t(p->numChannels) || p->pixelStride > kMaxPixelStride || p->rowPitch > kMaxRowPitch
+        || p->rowPitch < p->pixelStride * uint64_t(imageWidth) || (p->pixelStride % uint64_t(bpc)) || (p->rowPitch % uint64_t(bpc)) || (reinterpret_cast<uintptr_t>(p->src) % uintptr_t(bpc))) {
         set_error("ntc_hip_write_channels: pixel stride / row pitch do not fit the format and channel count.");
         return NTC_HIP_ERR_INVALID_ARG;
     }
@@ -807,8 +813,8 @@ static int check_diff_image(NtcHipImage const& im, char const* which, int left, 
     int const bpc = bytes_per_component(im.format);
     if (!im.data || !bpc) { set_error("ntc_hip_image_difference: image %s has no data or an unknown channel format (%d).", which, im.format); return NTC_HIP_ERR_INVALID_ARG; }
     if (im.numChannels < 1 || im.numChannels > 4 || im.width < 1 || im.height < 1) { set_error("ntc_hip_image_difference: image %s: 1..4 channels and a positive size are required.", which); return NTC_HIP_ERR_INVALID_ARG; }
-    if (im.pixelStride < uint64_t(bpc) * uint64_t(im.numChannels) || im.rowPitch < im.pixelStride * uint64_t(im.width)
-        || (im.pixelStride % uint64_t(bpc)) || (im.rowPitch % uint64_t(bpc)) || (reinterpret_cast<uintptr_t>(im.data) % uintptr_t(bpc))) {
+    if (im.pixelStride < uint64_t(bpc) * uint64_t(im.numChannels) || im.pixelStride > kMaxPixelStride || im.rowPitch > kMaxRowPitch
+        || im.rowPitch < im.pixelStride * uint64_t(im.width) || (im.pixelStride % uint64_t(bpc)) || (im.rowPitch % uint64_t(bpc)) || (reinterpret_cast<uintptr_t>(im.data) % uintptr_t(bpc))) {
         set_error("ntc_hip_image_difference: image %s: pixel stride / row pitch do not fit the format and channel count.", which);
         return NTC_HIP_ERR_INVALID_ARG;
     }
@@ -869,7 +875,7 @@ int ntc_hip_block_compress(const NtcHipBlockCompress* p)
     if (int r = check_diff_image(p->src, "src", 0, 0, 1, 1, image)) return r;     // the extent may reach past the image: such pixels read as 0
     uint64_t const blockBytes = (p->dstFormat == 1 || p->dstFormat == 4) ? 8u : 16u;
     uint64_t const rowNeed = uint64_t(p->dstOffsetX + p->widthInBlocks) * blockBytes;
-    if ((p->dstRowPitch & 7u) || p->dstRowPitch < rowNeed || (reinterpret_cast<uintptr_t>(p->dst) & 7u)
+    if ((p->dstRowPitch & 7u) || p->dstRowPitch < rowNeed || p->dstRowPitch > kMaxRowPitch || (reinterpret_cast<uintptr_t>(p->dst) & 7u)
         || uint64_t(p->dstOffsetY + p->heightInBlocks - 1) * p->dstRowPitch + rowNeed > p->dstBytes) {
         set_error("ntc_hip_block_compress: the destination (8-byte aligned, row pitch a multiple of 8) does not hold the blocks.");
         return NTC_HIP_ERR_INVALID_ARG;

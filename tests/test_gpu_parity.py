@@ -226,3 +226,33 @@ def test_argument_errors_are_reported(ntc, device):
     with pytest.raises(ntc.NtcHipError) as e:
         device.decode([dset])
     assert e.value.code in (ntc.abi.ERR_UNSUPPORTED, ntc.abi.ERR_INVALID_ARG)
+
+
+def test_offsets_that_would_wrap_are_rejected(ntc, device):
+    """Offsets and pitches near 2^64 must not slip through a wrapped sum."""
+    case = cfg_case(ntc, ntc.presets.spec_cfg01(), 64, 64, 1, 8, ntc.abi.OUT_UNORM8_PIXELS, seed=1)
+    for field, value in (("hrOffset", (1 << 64) - 2), ("lrOffset", (1 << 64) - 2), ("outOffset", (1 << 64) - 4), ("outRowPitch", 1 << 62)):
+        dset = case.device_set(device)
+        setattr(dset.mips[0], field, value)
+        with pytest.raises(ntc.NtcHipError) as e:
+            device.decode([dset])
+        assert e.value.code == ntc.abi.ERR_INVALID_ARG, field
+
+
+def test_fill_any_alignment(ntc, device):
+    """ntc_hip_memset is a kernel: every alignment of start and end, bytes outside untouched."""
+    rng = np.random.default_rng(5)
+    base = rng.integers(0, 256, 4096, dtype=np.uint8)
+    for start, count, value in ((0, 4096, 0), (1, 1, 7), (3, 13, 255), (5, 27, 1), (16, 16, 9), (15, 17, 3), (31, 1000, 0xAB), (8, 4080, 0x55), (2, 3, 4)):
+        buf = device.upload(base)
+        ntc.abi.check(device.lib.ntc_hip_memset(buf.ptr + start, value, count))
+        device.synchronize()
+        want = base.copy()
+        want[start:start + count] = value
+        assert np.array_equal(buf.download(), want), (start, count)
+    big = device.alloc((1 << 26) + 5)
+    big.fill(0x11)
+    ntc.abi.check(device.lib.ntc_hip_memset(big.ptr + 3, 0xEE, (1 << 26) - 1))
+    device.synchronize()
+    got = big.download()
+    assert np.all(got[:3] == 0x11) and np.all(got[3:(1 << 26) + 2] == 0xEE) and np.all(got[(1 << 26) + 2:] == 0x11)
