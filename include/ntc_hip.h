@@ -19,6 +19,11 @@
  * a positive hipError_t value when a HIP call failed, or a negative NtcHipError.
  * A message for the last failure on the calling thread is kept per thread, like
  * the reference's thread-local error buffer (src/Errors.cpp:21-52).
+ *
+ * Threading: the library holds one device, one stream, one mip table and one set of loss partials per
+ * process and takes no locks (nor does the reference: its texture sets share __constant__ state,
+ * src/Regression.cu:40-51).  Calls from several threads must be serialised by the caller.  Work is
+ * queued on the library's stream in call order; ntc_hip_synchronize waits for it.
  */
 #ifndef NTC_HIP_H
 #define NTC_HIP_H
