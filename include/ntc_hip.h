@@ -310,9 +310,9 @@ typedef struct NtcHipImageDifference {
 } NtcHipImageDifference;
 int ntc_hip_image_difference(const NtcHipImageDifference* params);
 
-/* BC1 .. BC5 compression of an image: the block-compression compute pass of
+/* BC1 .. BC5 and BC7 compression of an image: the block-compression compute pass of
  * IContext::MakeBlockCompressionComputePass for those formats (include/libntc/ntc.h:1050-1100,
- * src/shaders/CompressBC1.hlsl .. CompressBC5.hlsl, src/shaders/BlockCompressCommon.hlsli).
+ * src/shaders/CompressBC1.hlsl .. CompressBC5.hlsl, CompressBC7.hlsl, src/shaders/BlockCompressCommon.hlsli).
  * widthInBlocks x heightInBlocks blocks of 4 x 4 pixels starting at (srcLeft, srcTop) are encoded and
  * stored row-major with dstRowPitch bytes per row of blocks, the first at block (dstOffsetX, dstOffsetY).
  * dstFormat is a BlockCompressedFormat:
@@ -320,7 +320,10 @@ int ntc_hip_image_difference(const NtcHipImageDifference* params);
  *   2  BC2, 16 bytes: 4-bit alpha, then a BC1 colour block;
  *   3  BC3, 16 bytes: a BC4 block of A, then a BC1 colour block;
  *   4  BC4, 8 bytes, from R;      5  BC5, 16 bytes, from R then G;
- *   6, 7 (BC6H, BC7) return NTC_HIP_ERR_UNSUPPORTED.
+ *   7  BC7, 16 bytes, from R, G, B and A (src/shaders/CompressBC7.hlsl); see modeBuffer below.  The
+ *      reference's BC7 shader ignores dstOffsetInBlocks (CompressBC7.hlsl:1590); here it is honoured as for
+ *      the other formats;
+ *   6  (BC6H) returns NTC_HIP_ERR_UNSUPPORTED.
  * Channels the image does not have read as 0 (alpha as 1); pixels outside the image read as 0 in every
  * channel, like a texture load there.  Asynchronous on the library stream. */
 typedef struct NtcHipBlockCompress {
@@ -333,6 +336,16 @@ typedef struct NtcHipBlockCompress {
     void*       dst;                          /* device, 8-byte aligned */
     uint64_t    dstBytes;
     uint64_t    dstRowPitch;                  /* bytes per row of blocks, multiple of 8 */
+    /* BC7 only: the mode buffer of MakeBC7ModeBuffer (include/libntc/ntc.h:1381-1391), 9 bits per block of a
+     * modeMapWidthInBlocks x modeMapHeightInBlocks map; the block (x, y) of this call uses the entry at
+     * (x + modeMapOffsetX, y + modeMapOffsetY).  Then only that mode and partition are encoded (several times
+     * faster); a block with no entry becomes the reference's marker block of four coloured squares.  NULL:
+     * every mode is tried. */
+    const void* modeBuffer;                   /* device, 4-byte aligned */
+    uint64_t    modeBufferBytes;
+    uint64_t    modeBufferByteOffset;         /* multiple of 4 */
+    int32_t     modeMapWidthInBlocks, modeMapHeightInBlocks;
+    int32_t     modeMapOffsetX, modeMapOffsetY;
 } NtcHipBlockCompress;
 int ntc_hip_block_compress(const NtcHipBlockCompress* params);
 

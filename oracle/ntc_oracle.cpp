@@ -80,6 +80,7 @@
 #include <algorithm>
 #include <atomic>
 #include <chrono>
+#include <cfloat>
 #include <cmath>
 #include <cstdint>
 #include <cstring>
@@ -1344,6 +1345,439 @@ uint64_t bc2_alpha(const float alpha[16])                                // hlsl
 } // namespace
 } // namespace bc1
 
+// ---- BC7 encoder (src/shaders/CompressBC7.hlsl) --------------------------------------------------------
+// The reference tries, per block: for opaque blocks the three-subset modes 0 / 2 and the two-subset
+// modes 1 / 3 (partition chosen by an estimated error over all 64 partitions), then for every block
+// modes 4 and 5 in all four channel rotations, mode 6 and mode 7; a candidate replaces the current
+// block when its error is not larger.  With a mode buffer (one 9-bit mode + partition entry per
+// block, MakeBC7ModeBuffer) only that mode and partition are encoded and no error is computed.
+// Same float conventions as for BC1: separate IEEE binary32 operations, dot products left to right,
+// round() to nearest even.
+extern "C++" {      // templates: not inside this file's extern "C" block
+namespace bc7 {
+namespace {
+
+// Table.P2 and Table.P3 of the BPTC format specification (ARB_texture_compression_bptc): the subset of
+// each of the 16 texels, texel 0 first; anchor tables A2, A3a, A3b of the same specification.
+const char* const kTwoSubsets[64] = {
+    "0011001100110011", "0001000100010001", "0111011101110111", "0001001100110111",
+    "0000000100010011", "0011011101111111", "0001001101111111", "0000000100110111",
+    "0000000000010011", "0011011111111111", "0000000101111111", "0000000000010111",
+    "0001011111111111", "0000000011111111", "0000111111111111", "0000000000001111",
+    "0000100011101111", "0111000100000000", "0000000010001110", "0111001100010000",
+    "0011000100000000", "0000100011001110", "0000000010001100", "0111001100110001",
+    "0011000100010000", "0000100010001100", "0110011001100110", "0011011001101100",
+    "0001011111101000", "0000111111110000", "0111000110001110", "0011100110011100",
+    "0101010101010101", "0000111100001111", "0101101001011010", "0011001111001100",
+    "0011110000111100", "0101010110101010", "0110100101101001", "0101101010100101",
+    "0111001111001110", "0001001111001000", "0011001001001100", "0011101111011100",
+    "0110100110010110", "0011110011000011", "0110011010011001", "0000011001100000",
+    "0100111001000000", "0010011100100000", "0000001001110010", "0000010011100100",
+    "0110110010010011", "0011011011001001", "0110001110011100", "0011100111000110",
+    "0110110011001001", "0110001100111001", "0111111010000001", "0001100011100111",
+    "0000111100110011", "0011001111110000", "0010001011101110", "0100010001110111",
+};
+const char* const kThreeSubsets[64] = {
+    "0011001102212222", "0001001122112221", "0000200122112211", "0222002200110111",
+    "0000000011221122", "0011001100220022", "0022002211111111", "0011001122112211",
+    "0000000011112222", "0000111111112222", "0000111122222222", "0012001200120012",
+    "0112011201120112", "0122012201220122", "0011011211221222", "0011200122002220",
+    "0001001101121122", "0111001120012200", "0000112211221122", "0022002200221111",
+    "0111011102220222", "0001000122212221", "0000001101220122", "0000110022102210",
+    "0122012200110000", "0012001211222222", "0110122112210110", "0000011012211221",
+    "0022110211020022", "0110011020022222", "0011012201220011", "0000200022112221",
+    "0000000211221222", "0222002200120011", "0011001200220222", "0120012001200120",
+    "0000111122220000", "0120120120120120", "0120201212010120", "0011220011220011",
+    "0011112222000011", "0101010122222222", "0000000021212121", "0022112200221122",
+    "0022001100220011", "0220122102201221", "0101222222220101", "0000212121212121",
+    "0101010101012222", "0222011102220111", "0002111200021112", "0000211221122112",
+    "0222011101110222", "0002111211120002", "0110011001102222", "0000000021122112",
+    "0110011022222222", "0022001100110022", "0022112211220022", "0000000000002112",
+    "0002000100020001", "0222122202221222", "0101222222222222", "0111201122012220",
+};
+const uint8_t kAnchorSecondOfTwo[64] = {
+    15, 15, 15, 15, 15, 15, 15, 15, 15, 15, 15, 15, 15, 15, 15, 15,
+    15,  2,  8,  2,  2,  8,  8, 15,  2,  8,  2,  2,  8,  8,  2,  2,
+    15, 15,  6,  8,  2,  8, 15, 15,  2,  8,  2,  2,  2, 15, 15,  6,
+     6,  2,  6,  8, 15, 15,  2,  2, 15, 15, 15, 15, 15,  2,  2, 15,
+};
+const uint8_t kAnchorSecondOfThree[64] = {
+     3,  3, 15, 15,  8,  3, 15, 15,  8,  8,  6,  6,  6,  5,  3,  3,
+     3,  3,  8, 15,  3,  3,  6, 10,  5,  8,  8,  6,  8,  5, 15, 15,
+     8, 15,  3,  5,  6, 10,  8, 15, 15,  3, 15,  5, 15, 15, 15, 15,
+     3, 15,  5,  5,  5,  8,  5, 10,  5, 10,  8, 13, 15, 12,  3,  3,
+};
+const uint8_t kAnchorThirdOfThree[64] = {
+    15,  8,  8,  3, 15, 15,  3,  8, 15, 15, 15, 15, 15, 15, 15,  8,
+    15,  8, 15,  3, 15,  8, 15,  8,  3, 15,  6, 10, 15, 15, 10,  8,
+    15,  3, 15, 10, 10,  8,  9, 10,  6, 15,  8, 15,  3,  6,  6,  8,
+    15,  3, 15, 15, 15, 15, 15, 15, 15, 15, 15, 15,  3, 15, 15,  8,
+};
+struct Masks {
+    uint32_t two[64][2], three[64][3];
+    Masks()
+    {
+        for (int p = 0; p < 64; ++p) {
+            two[p][0] = two[p][1] = three[p][0] = three[p][1] = three[p][2] = 0;
+            for (int t = 0; t < 16; ++t) {
+                two[p][kTwoSubsets[p][t] - '0'] |= 1u << t;
+                three[p][kThreeSubsets[p][t] - '0'] |= 1u << t;
+            }
+        }
+    }
+};
+Masks const& masks() { static Masks const m; return m; }
+
+uint32_t subset_mask(int subsets, int partition, int s) { return subsets == 1 ? 0xffffu : subsets == 2 ? masks().two[partition][s] : masks().three[partition][s]; }
+int subset_anchor(int subsets, int partition, int s)
+{
+    if (s == 0) return 0;
+    if (subsets == 2) return kAnchorSecondOfTwo[partition];
+    return s == 1 ? kAnchorSecondOfThree[partition] : kAnchorThirdOfThree[partition];
+}
+
+template <int C> struct Color { float c[C]; };
+float sat(float v) { return std::fmin(std::fmax(v, 0.f), 1.f); }
+template <int C> float dot(Color<C> const& a, Color<C> const& b) { float s = a.c[0] * b.c[0]; for (int k = 1; k < C; ++k) s += a.c[k] * b.c[k]; return s; }
+template <int C> Color<C> sub(Color<C> const& a, Color<C> const& b) { Color<C> r; for (int k = 0; k < C; ++k) r.c[k] = a.c[k] - b.c[k]; return r; }
+int popcount16(uint32_t m) { int n = 0; for (int t = 0; t < 16; ++t) n += (m >> t) & 1; return n; }
+
+template <int C> void min_max(const Color<C> px[16], uint32_t mask, Color<C>& lo, Color<C>& hi)          // hlsl:175-189
+{
+    for (int k = 0; k < C; ++k) { lo.c[k] = FLT_MAX; hi.c[k] = -FLT_MAX; }
+    for (int t = 0; t < 16; ++t) if (mask & (1u << t))
+        for (int k = 0; k < C; ++k) { lo.c[k] = std::fmin(lo.c[k], px[t].c[k]); hi.c[k] = std::fmax(hi.c[k], px[t].c[k]); }
+}
+
+// hlsl:243-343: with the first component whose ends differ as the axis, later components' ends are swapped
+// where their covariance with the axis is negative.
+template <int C> void orient(const Color<C> px[16], uint32_t mask, Color<C>& e0, Color<C>& e1)
+{
+    Color<C> center;
+    for (int k = 0; k < C; ++k) center.c[k] = 0.f;
+    for (int t = 0; t < 16; ++t) if (mask & (1u << t)) for (int k = 0; k < C; ++k) center.c[k] += px[t].c[k];
+    float const count = float(popcount16(mask));
+    for (int k = 0; k < C; ++k) center.c[k] /= count;
+    float cov[C][C] = {};
+    for (int t = 0; t < 16; ++t) if (mask & (1u << t)) {
+        Color<C> const d = sub(px[t], center);
+        for (int a = 0; a < C; ++a) for (int b = a + 1; b < C; ++b) cov[a][b] += d.c[a] * d.c[b];
+    }
+    for (int a = 0; a + 1 < C; ++a)
+        if (e0.c[a] != e1.c[a]) {
+            for (int b = a + 1; b < C; ++b) if (cov[a][b] < 0.f) std::swap(e0.c[b], e1.c[b]);
+            break;
+        }
+}
+
+template <int C> void refine(const Color<C> px[16], uint32_t mask, Color<C>& e0, Color<C>& e1, int indexBits)     // hlsl:191-241
+{
+    for (int iter = 0; iter < 2; ++iter) {
+        Color<C> const axis = sub(e1, e0);
+        float mul = dot(axis, axis);
+        if (mul > 0.f) mul = 1.f / mul;
+        float const scale = float((1u << indexBits) - 1), iscale = 1.f / scale;
+        float a2 = 0, b2 = 0, ab = 0;
+        Color<C> ax, bx;
+        for (int k = 0; k < C; ++k) ax.c[k] = bx.c[k] = 0.f;
+        for (int t = 0; t < 16; ++t) if (mask & (1u << t)) {
+            float const f = sat(dot(sub(px[t], e0), axis) * mul);
+            float const beta = std::nearbyint(f * scale) * iscale, alpha = 1.f - beta;
+            a2 += alpha * alpha; b2 += beta * beta; ab += alpha * beta;
+            for (int k = 0; k < C; ++k) { ax.c[k] += alpha * px[t].c[k]; bx.c[k] += beta * px[t].c[k]; }
+        }
+        float const denom = a2 * b2 - ab * ab;
+        if (!(std::fabs(denom) > 0.0001f)) break;
+        float const factor = 1.f / denom;
+        for (int k = 0; k < C; ++k) {
+            float const a = sat((ax.c[k] * b2 - bx.c[k] * ab) * factor), b = sat((bx.c[k] * a2 - ax.c[k] * ab) * factor);
+            if (!(e0.c[k] == 0.f || e0.c[k] == 1.f)) e0.c[k] = a;
+            if (!(e1.c[k] == 0.f || e1.c[k] == 1.f)) e1.c[k] = b;
+        }
+    }
+}
+
+template <int C> float estimate(const Color<C> px[16], uint32_t mask, Color<C> const& e0, Color<C> const& e1, int indexBits)     // hlsl:345-373
+{
+    Color<C> const axis = sub(e1, e0);
+    float mul = dot(axis, axis);
+    if (mul > 0.f) mul = 1.f / mul;
+    float const maxIndex = float((1u << indexBits) - 1), indexScale = 1.f / maxIndex;
+    float error = 0.f;
+    for (int t = 0; t < 16; ++t) if (mask & (1u << t)) {
+        Color<C> const p = sub(px[t], e0);
+        float f = dot(p, axis) * mul;
+        f = std::nearbyint(f * maxIndex) * indexScale;
+        Color<C> diff;
+        for (int k = 0; k < C; ++k) diff.c[k] = f * axis.c[k] - p.c[k];
+        error += dot(diff, diff);
+    }
+    return error;
+}
+
+int quantize(float v, int bits) { return int(std::nearbyint(sat(v) * float((1u << bits) - 1))); }         // hlsl:131-135
+int expand8(int q, int bits) { return (q << (8 - bits)) | (q >> (2 * bits - 8)); }                       // hlsl:154-157
+
+template <int C> struct Quantized { int c[C]; };
+
+template <int C> float decoded_error(const Color<C> px[16], const int index[16], uint32_t mask, Quantized<C> q0, Quantized<C> q1,
+                                     int indexBits, int endpointBits)                                    // hlsl:375-405
+{
+    for (int k = 0; k < C; ++k) { q0.c[k] = expand8(q0.c[k], endpointBits); q1.c[k] = expand8(q1.c[k], endpointBits); }
+    float const indexScale = 64.f / float((1u << indexBits) - 1);
+    float error = 0.f;
+    for (int t = 0; t < 16; ++t) if (mask & (1u << t)) {
+        int const w = int(std::nearbyint(float(index[t]) * indexScale));
+        Color<C> diff;
+        for (int k = 0; k < C; ++k) diff.c[k] = float((q0.c[k] * (64 - w) + q1.c[k] * w + 32) >> 6) / 255.f - px[t].c[k];
+        error += dot(diff, diff);
+    }
+    return error;
+}
+
+// Indices of a subset's texels along the dequantised endpoints; when the anchor texel's index has its
+// top bit set all of the subset's indices are complemented and true is returned (the caller then
+// swaps the endpoints).  hlsl:445-527
+template <int C> bool assign(const Color<C> px[16], uint32_t mask, int anchor, int indexBits, int endpointBits,
+                             Quantized<C> const& q0, Quantized<C> const& q1, int index[16])
+{
+    Color<C> e0, e1;
+    for (int k = 0; k < C; ++k) { e0.c[k] = float(expand8(q0.c[k], endpointBits)) / 255.f; e1.c[k] = float(expand8(q1.c[k], endpointBits)) / 255.f; }
+    Color<C> const axis = sub(e1, e0);
+    float mul = dot(axis, axis);
+    if (mul > 0.f) mul = 1.f / mul;
+    for (int t = 0; t < 16; ++t) if (mask & (1u << t)) index[t] = quantize(dot(sub(px[t], e0), axis) * mul, indexBits);
+    bool const flip = (index[anchor] >> (indexBits - 1)) & 1;
+    if (flip) for (int t = 0; t < 16; ++t) if (mask & (1u << t)) index[t] ^= (1 << indexBits) - 1;
+    return flip;
+}
+
+struct Bits {
+    uint64_t lo = 0, hi = 0;
+    int at = 0;
+    void put(int length, uint32_t value)
+    {
+        uint64_t const v = value & ((1u << length) - 1u);
+        if (at < 64) { lo |= v << at; if (at + length > 64) hi |= v >> (64 - at); }
+        else hi |= v << (at - 64);
+        at += length;
+    }
+};
+
+struct Best { float error = FLT_MAX; uint64_t lo = 0, hi = 0; bool fixedMode = false; };
+
+enum PBit { kNoPBit, kPBitPerEndpoint, kPBitPerSubset };
+struct Mode { int id, subsets, partitionBits, endpointBits /* with the p-bit */, indexBits; PBit pbit; };
+const Mode kMode0{ 0, 3, 4, 5, 3, kPBitPerEndpoint }, kMode1{ 1, 2, 6, 7, 3, kPBitPerSubset }, kMode2{ 2, 3, 6, 5, 2, kNoPBit },
+           kMode3{ 3, 2, 6, 8, 2, kPBitPerEndpoint }, kMode6{ 6, 1, 0, 8, 4, kPBitPerEndpoint }, kMode7{ 7, 2, 6, 6, 2, kPBitPerEndpoint };
+
+// hlsl:407-443: endpoint quantisation with the mode's p-bit rule.
+template <int C> void quantize_endpoints(Mode const& m, const Color<C> e[6], Quantized<C> q[6])
+{
+    int const n = 2 * m.subsets;
+    for (int i = 0; i < n; ++i) for (int k = 0; k < C; ++k) q[i].c[k] = quantize(e[i].c[k], m.endpointBits);
+    if (m.pbit == kPBitPerEndpoint) {
+        for (int i = 0; i < n; ++i) {
+            int odd = 0;
+            for (int k = 0; k < C; ++k) odd += q[i].c[k] & 1;
+            int lsb = odd >= 2 ? 1 : 0;
+            if (C == 4) lsb = ((odd >= 2 && q[i].c[3] != 0) || e[i].c[3] == 1.f) ? 1 : 0;      // keeps alpha 0 and alpha 1 exact
+            for (int k = 0; k < C; ++k) q[i].c[k] = (q[i].c[k] & 0xFE) | lsb;
+        }
+    } else if (m.pbit == kPBitPerSubset) {
+        for (int i = 0; i < n; i += 2) {
+            int odd = 0;
+            for (int k = 0; k < C; ++k) odd += (q[i].c[k] & 1) + (q[i + 1].c[k] & 1);
+            int const lsb = odd >= 4 ? 1 : 0;
+            for (int k = 0; k < C; ++k) { q[i].c[k] = (q[i].c[k] & 0xFE) | lsb; q[i + 1].c[k] = (q[i + 1].c[k] & 0xFE) | lsb; }
+        }
+    }
+}
+
+// Refines the start endpoints of every subset, quantises, assigns indices and, if the result is not
+// worse than the best so far, encodes the block (hlsl:570-726, 787-928, 1247-1407).
+template <int C> void finish(Mode const& m, const Color<C> px[16], int partition, const Color<C> start[6], Best& best)
+{
+    Color<C> e[6];
+    Quantized<C> q[6];
+    for (int i = 0; i < 2 * m.subsets; ++i) e[i] = start[i];
+    for (int s = 0; s < m.subsets; ++s) refine(px, subset_mask(m.subsets, partition, s), e[2 * s], e[2 * s + 1], m.indexBits);
+    quantize_endpoints(m, e, q);
+    int index[16] = {};
+    float error = 0.f;
+    for (int s = 0; s < m.subsets; ++s) {
+        uint32_t const mask = subset_mask(m.subsets, partition, s);
+        if (assign(px, mask, subset_anchor(m.subsets, partition, s), m.indexBits, m.endpointBits, q[2 * s], q[2 * s + 1], index))
+            std::swap(q[2 * s], q[2 * s + 1]);
+        if (!best.fixedMode) {
+            float const e2 = decoded_error(px, index, mask, q[2 * s], q[2 * s + 1], m.indexBits, m.endpointBits);
+            error = s == 0 ? e2 : error + e2;
+        }
+    }
+    if (error > best.error) return;
+    Bits b;
+    b.put(m.id + 1, 1u << m.id);
+    b.put(m.partitionBits, uint32_t(partition));
+    int const drop = m.pbit == kNoPBit ? 0 : 1;
+    for (int k = 0; k < C; ++k) for (int i = 0; i < 2 * m.subsets; ++i) b.put(m.endpointBits - drop, uint32_t(q[i].c[k]) >> drop);
+    if (m.pbit == kPBitPerEndpoint) for (int i = 0; i < 2 * m.subsets; ++i) b.put(1, uint32_t(q[i].c[0]));
+    if (m.pbit == kPBitPerSubset) for (int s = 0; s < m.subsets; ++s) b.put(1, uint32_t(q[2 * s].c[0]));
+    for (int t = 0; t < 16; ++t) {
+        bool anchor = t == 0;
+        for (int s = 1; s < m.subsets; ++s) anchor = anchor || t == subset_anchor(m.subsets, partition, s);
+        b.put(anchor ? m.indexBits - 1 : m.indexBits, uint32_t(index[t]));
+    }
+    best.error = error; best.lo = b.lo; best.hi = b.hi;
+}
+
+// Start endpoints (bounding box per subset, oriented) for one partition, and their estimated error.
+template <int C> float start_endpoints(const Color<C> px[16], int subsets, int partition, bool orientEnds, int searchIndexBits, bool wantError, Color<C> e[6])
+{
+    float error = 0.f;
+    for (int s = 0; s < subsets; ++s) min_max(px, subset_mask(subsets, partition, s), e[2 * s], e[2 * s + 1]);
+    if (orientEnds) for (int s = 0; s < subsets; ++s) orient(px, subset_mask(subsets, partition, s), e[2 * s], e[2 * s + 1]);
+    if (wantError)
+        for (int s = 0; s < subsets; ++s) {
+            float const e2 = estimate(px, subset_mask(subsets, partition, s), e[2 * s], e[2 * s + 1], searchIndexBits);
+            error = s == 0 ? e2 : error + e2;
+        }
+    return error;
+}
+
+// The partition with the smallest estimated error (the first of equals) and its start endpoints; with a
+// fixed partition just that one's endpoints (hlsl:728-785, 930-983, 1296-1345).
+template <int C> int pick_partition(const Color<C> px[16], int subsets, bool orientEnds, int searchIndexBits, int fixedPartition, Color<C> bestEnds[6])
+{
+    if (fixedPartition >= 0) { start_endpoints(px, subsets, fixedPartition, orientEnds, searchIndexBits, false, bestEnds); return fixedPartition; }
+    int bestPartition = 0;
+    float bestError = FLT_MAX;
+    // a NaN texel makes every estimate NaN and no partition "best": the reference then goes on with
+    // uninitialised endpoints, here they are zero (and the partition 0)
+    for (int i = 0; i < 2 * subsets; ++i) for (int k = 0; k < C; ++k) bestEnds[i].c[k] = 0.f;
+    for (int p = 0; p < 64; ++p) {
+        Color<C> e[6];
+        float const error = start_endpoints(px, subsets, p, orientEnds, searchIndexBits, true, e);
+        if (error < bestError) { bestPartition = p; bestError = error; for (int i = 0; i < 2 * subsets; ++i) bestEnds[i] = e[i]; }
+    }
+    return bestPartition;
+}
+
+// Modes 4 and 5: a colour plane of three channels and a scalar plane, each with its own endpoints and
+// indices; `px` is already rotated so that the scalar channel is the fourth (hlsl:985-1148).
+void dual_plane(int mode, bool wideColorIndex, const Color<4> px[16], uint32_t rotation, Best& best)
+{
+    int const colorIndexBits = mode == 5 ? 2 : (wideColorIndex ? 3 : 2), alphaIndexBits = mode == 5 ? 2 : (wideColorIndex ? 2 : 3);
+    int const colorBits = mode == 5 ? 7 : 5, alphaBits = mode == 5 ? 8 : 6;
+    Color<3> rgb[16];
+    Color<1> a[16];
+    for (int t = 0; t < 16; ++t) { rgb[t] = Color<3>{ { px[t].c[0], px[t].c[1], px[t].c[2] } }; a[t] = Color<1>{ { px[t].c[3] } }; }
+    Color<1> a0, a1;
+    min_max(a, 0xffffu, a0, a1);
+    refine(a, 0xffffu, a0, a1, alphaIndexBits);
+    Color<3> e0, e1;
+    min_max(rgb, 0xffffu, e0, e1);
+    orient(rgb, 0xffffu, e0, e1);
+    refine(rgb, 0xffffu, e0, e1, colorIndexBits);
+    Quantized<3> q0, q1;
+    for (int k = 0; k < 3; ++k) { q0.c[k] = quantize(e0.c[k], colorBits); q1.c[k] = quantize(e1.c[k], colorBits); }
+    Quantized<1> qa0{ { quantize(a0.c[0], alphaBits) } }, qa1{ { quantize(a1.c[0], alphaBits) } };
+    int colorIndex[16], alphaIndex[16];
+    float error = 0.f;
+    if (assign(rgb, 0xffffu, 0, colorIndexBits, colorBits, q0, q1, colorIndex)) std::swap(q0, q1);
+    if (!best.fixedMode) error = decoded_error(rgb, colorIndex, 0xffffu, q0, q1, colorIndexBits, colorBits);
+    if (assign(a, 0xffffu, 0, alphaIndexBits, alphaBits, qa0, qa1, alphaIndex)) std::swap(qa0, qa1);
+    if (!best.fixedMode) error += decoded_error(a, alphaIndex, 0xffffu, qa0, qa1, alphaIndexBits, alphaBits);
+    if (error > best.error) return;
+    Bits b;
+    b.put(mode + 1, 1u << mode);
+    b.put(2, rotation);
+    if (mode == 4) b.put(1, wideColorIndex ? 1u : 0u);
+    for (int k = 0; k < 3; ++k) { b.put(colorBits, uint32_t(q0.c[k])); b.put(colorBits, uint32_t(q1.c[k])); }
+    b.put(alphaBits, uint32_t(qa0.c[0])); b.put(alphaBits, uint32_t(qa1.c[0]));
+    // mode 4 stores its 2-bit indices first, then the 3-bit ones; mode 5 colour first, then the scalar
+    bool const alphaFirst = mode == 4 && wideColorIndex;
+    const int* first = alphaFirst ? alphaIndex : colorIndex;
+    const int* second = alphaFirst ? colorIndex : alphaIndex;
+    int const firstBits = alphaFirst ? alphaIndexBits : colorIndexBits, secondBits = alphaFirst ? colorIndexBits : alphaIndexBits;
+    for (int t = 0; t < 16; ++t) b.put(t == 0 ? firstBits - 1 : firstBits, uint32_t(first[t]));
+    for (int t = 0; t < 16; ++t) b.put(t == 0 ? secondBits - 1 : secondBits, uint32_t(second[t]));
+    best.error = error; best.lo = b.lo; best.hi = b.hi;
+}
+
+// Channel order for rotation r: the scalar plane takes channel {A, R, G, B}[r], alpha takes its place.
+void rotate(const Color<4> px[16], uint32_t rotation, Color<4> out[16])
+{
+    for (int t = 0; t < 16; ++t) {
+        out[t] = px[t];
+        if (rotation) std::swap(out[t].c[rotation - 1], out[t].c[3]);
+    }
+}
+
+// One block.  fixedMode < 0: every mode is tried (CompressBC7.hlsl:1575-1587); otherwise only that
+// mode with that partition (for modes 4 / 5: rotation in bits 0-1, "wide colour index" in bit 2).
+void encode(const Color<4> px[16], int fixedMode, int fixedPartition, uint64_t out[2])
+{
+    Best best;
+    best.fixedMode = fixedMode >= 0;
+    Color<3> rgb[16];
+    bool opaque = true;
+    for (int t = 0; t < 16; ++t) { rgb[t] = Color<3>{ { px[t].c[0], px[t].c[1], px[t].c[2] } }; if (px[t].c[3] < 1.f) opaque = false; }
+    auto three_subsets = [&](bool mode0, bool mode2, int partition) {
+        Color<3> ends[6];
+        int const p = pick_partition(rgb, 3, true, 3, partition, ends);
+        if (mode0 && (partition >= 0 || p < 16)) finish(kMode0, rgb, p, ends, best);
+        if (mode2) finish(kMode2, rgb, p, ends, best);
+    };
+    auto two_subsets = [&](bool mode1, bool mode3, int partition) {
+        Color<3> ends[6];
+        int const p = pick_partition(rgb, 2, true, 3, partition, ends);
+        if (mode1) finish(kMode1, rgb, p, ends, best);
+        if (mode3) finish(kMode3, rgb, p, ends, best);
+    };
+    auto mode6 = [&]() {
+        Color<4> ends[6];
+        start_endpoints(px, 1, 0, true, 4, false, ends);
+        finish(kMode6, px, 0, ends, best);
+    };
+    auto mode7 = [&](int partition) {
+        Color<4> ends[6];
+        int const p = pick_partition(px, 2, false, 2, partition, ends);
+        finish(kMode7, px, p, ends, best);
+    };
+    if (fixedMode < 0) {
+        if (opaque) { three_subsets(true, true, -1); two_subsets(true, true, -1); }
+        for (uint32_t rotation = 0; rotation < 4; ++rotation) {
+            Color<4> r[16];
+            rotate(px, rotation, r);
+            dual_plane(4, false, r, rotation, best);
+            dual_plane(4, true, r, rotation, best);
+            dual_plane(5, false, r, rotation, best);
+        }
+        mode6();
+        mode7(-1);
+    } else {
+        switch (fixedMode) {
+        case 0: three_subsets(true, false, fixedPartition); break;
+        case 2: three_subsets(false, true, fixedPartition); break;
+        case 1: two_subsets(true, false, fixedPartition); break;
+        case 3: two_subsets(false, true, fixedPartition); break;
+        case 4: case 5: {
+            Color<4> r[16];
+            rotate(px, uint32_t(fixedPartition) & 3u, r);
+            dual_plane(fixedMode, fixedMode == 4 && (fixedPartition & 4), r, uint32_t(fixedPartition) & 3u, best);
+            break;
+        }
+        case 6: mode6(); break;
+        default: mode7(fixedPartition); break;
+        }
+    }
+    out[0] = best.lo; out[1] = best.hi;
+}
+
+} // namespace
+} // namespace bc7
+} // extern "C++"
+
 // For tests: the single-colour tables (256 entries each, first endpoint | second << 8).
 void ntc_oracle_bc1_match_tables(uint16_t* five, uint16_t* six)
 {
@@ -1351,10 +1785,22 @@ void ntc_oracle_bc1_match_tables(uint16_t* five, uint16_t* six)
     std::memcpy(six, bc1::match_tables().six, 512);
 }
 
-// dstFormat 1..5 (BC1, BC2, BC3, BC4: channel R, BC5: R then G); host pointers in `p`.  Returns -1 for other formats.
+// For tests: the subset masks the BC7 encoder derives from the specification's tables (two-subset:
+// 64 x 2, three-subset: 64 x 3) and the three anchor tables.
+void ntc_oracle_bc7_tables(uint32_t* two, uint32_t* three, uint8_t* anchors)
+{
+    for (int p = 0; p < 64; ++p) {
+        for (int s = 0; s < 2; ++s) two[2 * p + s] = bc7::masks().two[p][s];
+        for (int s = 0; s < 3; ++s) three[3 * p + s] = bc7::masks().three[p][s];
+        anchors[p] = bc7::kAnchorSecondOfTwo[p]; anchors[64 + p] = bc7::kAnchorSecondOfThree[p]; anchors[128 + p] = bc7::kAnchorThirdOfThree[p];
+    }
+}
+
+// dstFormat 1..5 and 7 (BC1, BC2, BC3, BC4: channel R, BC5: R then G, BC7); host pointers in `p`.
+// Returns -1 for other formats.
 int ntc_oracle_block_compress(const NtcHipBlockCompress* p)
 {
-    if (p->dstFormat < 1 || p->dstFormat > 5) return -1;
+    if (p->dstFormat < 1 || p->dstFormat > 7 || p->dstFormat == 6) return -1;
     auto fetch = [&](int x, int y, int c) -> float {
         if (x < 0 || y < 0 || x >= p->src.width || y >= p->src.height) return 0.f;
         return diff_channel(p->src, static_cast<uint8_t const*>(p->src.data) + size_t(y) * p->src.rowPitch + size_t(x) * p->src.pixelStride, c);
@@ -1363,12 +1809,34 @@ int ntc_oracle_block_compress(const NtcHipBlockCompress* p)
     for (int by = 0; by < p->heightInBlocks; ++by)
         for (int bx = 0; bx < p->widthInBlocks; ++bx) {
             uint64_t words[2] = { 0, 0 };
-            if (p->dstFormat >= 4) {
+            if (p->dstFormat == 4 || p->dstFormat == 5) {
                 for (int c = 0; c < p->dstFormat - 3; ++c) {
                     float texels[16];
                     for (int t = 0; t < 16; ++t) texels[t] = fetch(p->srcLeft + bx * 4 + (t & 3), p->srcTop + by * 4 + (t >> 2), c);
                     words[c] = bc4::encode(texels);
                 }
+            } else if (p->dstFormat == 7) {
+                bc7::Color<4> px[16];
+                for (int t = 0; t < 16; ++t)
+                    for (int c = 0; c < 4; ++c) px[t].c[c] = fetch(p->srcLeft + bx * 4 + (t & 3), p->srcTop + by * 4 + (t >> 2), c);
+                int mode = -1, partition = -1;
+                bool valid = true;
+                if (p->modeBuffer) {
+                    // CompressBC7.hlsl:1409-1443: 9 bits per block of the mode map, 0 = no entry, 0x1BF = mode 0 partition 0
+                    int64_t const mx = int64_t(bx) + p->modeMapOffsetX, my = int64_t(by) + p->modeMapOffsetY;
+                    valid = mx >= 0 && my >= 0 && mx < p->modeMapWidthInBlocks && my < p->modeMapHeightInBlocks;
+                    if (valid) {
+                        uint64_t const bit = (uint64_t(my) * uint64_t(p->modeMapWidthInBlocks) + uint64_t(mx)) * 9u;
+                        uint8_t const* bytes = static_cast<uint8_t const*>(p->modeBuffer) + p->modeBufferByteOffset;
+                        uint32_t entry = 0;
+                        for (uint64_t b = 0; b < 9; ++b) entry |= uint32_t((bytes[(bit + b) >> 3] >> ((bit + b) & 7)) & 1u) << b;
+                        valid = entry != 0;
+                        if (entry == 0x1BF) entry = 0;
+                        mode = int((entry >> 6) & 7u); partition = int(entry & 63u);
+                    }
+                }
+                if (valid) bc7::encode(px, mode, partition, words);
+                else { words[0] = 0x0001f00000f80004ull; words[1] = 0x1f9e00003ff0001full; }      // hlsl:1541-1548: four coloured squares
             } else {
                 float px[16][4], alpha[16];
                 for (int t = 0; t < 16; ++t) {

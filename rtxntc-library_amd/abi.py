@@ -112,6 +112,8 @@ class BlockCompress(C.Structure):
         ("src", Image), ("srcLeft", C.c_int32), ("srcTop", C.c_int32), ("widthInBlocks", C.c_int32), ("heightInBlocks", C.c_int32),
         ("dstFormat", C.c_int32), ("dstOffsetX", C.c_int32), ("dstOffsetY", C.c_int32), ("alphaThreshold", C.c_float),
         ("dst", C.c_void_p), ("dstBytes", C.c_uint64), ("dstRowPitch", C.c_uint64),
+        ("modeBuffer", C.c_void_p), ("modeBufferBytes", C.c_uint64), ("modeBufferByteOffset", C.c_uint64),
+        ("modeMapWidthInBlocks", C.c_int32), ("modeMapHeightInBlocks", C.c_int32), ("modeMapOffsetX", C.c_int32), ("modeMapOffsetY", C.c_int32),
     ]
 
 

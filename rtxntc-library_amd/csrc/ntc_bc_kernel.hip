@@ -30,6 +30,7 @@
 #include <stdint.h>
 #include <atomic>
 #include "ntc_decode_kernel.h"
+#include "ntc_bc_source.h"
 
 namespace ntc_hip_dev {
 
@@ -148,22 +149,6 @@ __device__ uint64_t bc4_encode(float const (&texels)[16])
     uint32_t const inset = (hiInner - loInner) / 34u;
     uint64_t const block6 = bc4_refine(values, bc4_with_endpoints(0, loInner + inset, hiInner - inset), false, false, false, error6);
     return error6 < error8 ? block6 : block8;
-}
-
-// Channel c of the pixel at (x, y) of the source image; outside the image everything reads as 0,
-// like a texture load there.
-__device__ __forceinline__ float source_channel(BlockCompressArgs const& a, int x, int y, int c)
-{
-    if (x < 0 || y < 0 || x >= a.srcWidth || y >= a.srcHeight) return 0.f;
-    if (c >= a.numChannels) return c == 3 ? 1.f : 0.f;
-    uint8_t const* px = a.src + size_t(y) * a.rowPitch + size_t(x) * a.pixelStride;
-    switch (a.format) {
-    case NTC_HIP_DEV_FORMAT_UNORM8:  return float(px[c]) / 255.f;
-    case NTC_HIP_DEV_FORMAT_UNORM16: return float(reinterpret_cast<uint16_t const*>(px)[c]) / 65535.f;
-    case NTC_HIP_DEV_FORMAT_FLOAT16: return float(reinterpret_cast<_Float16 const*>(px)[c]);
-    case NTC_HIP_DEV_FORMAT_FLOAT32: return reinterpret_cast<float const*>(px)[c];
-    default:                         return float(reinterpret_cast<uint32_t const*>(px)[c]);
-    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -542,6 +527,7 @@ hipError_t launch_block_compress(BlockCompressArgs const& a, int dstFormat, hipS
     case 3: hipLaunchKernelGGL(bc1_compress_kernel<3>, grid, dim3(128), 0, stream, a); break;
     case 4: hipLaunchKernelGGL(bc4_compress_kernel<1>, grid, dim3(128), 0, stream, a); break;
     case 5: hipLaunchKernelGGL(bc4_compress_kernel<2>, grid, dim3(128), 0, stream, a); break;
+    case 7: return launch_bc7_compress(a, stream);
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

@@ -131,10 +131,14 @@ struct BlockCompressArgs {
     int32_t srcWidth, srcHeight, format, numChannels;
     int32_t srcLeft, srcTop, widthInBlocks, heightInBlocks, dstOffsetX, dstOffsetY;
     float alphaThreshold;       // BC1: texels with alpha <= threshold are transparent
+    // BC7: 9-bit (mode, partition) entries of a modeMapWidthInBlocks x modeMapHeightInBlocks map, or null
+    uint32_t const* modeBuffer;
+    int32_t modeMapWidthInBlocks, modeMapHeightInBlocks, modeMapOffsetX, modeMapOffsetY;
 };
 // Sets `bytes` bytes at dst to `value` (any alignment).
 hipError_t launch_fill(uint8_t* dst, uint8_t value, uint64_t bytes, hipStream_t stream);
-hipError_t launch_block_compress(BlockCompressArgs const& args, int dstFormat /* 1..5 */, hipStream_t stream);
+hipError_t launch_block_compress(BlockCompressArgs const& args, int dstFormat /* 1..5, 7 */, hipStream_t stream);
+hipError_t launch_bc7_compress(BlockCompressArgs const& args, hipStream_t stream);
 
 hipError_t launch_decode(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream);
 hipError_t launch_queries(int variant, DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries,

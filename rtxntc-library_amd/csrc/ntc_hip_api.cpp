@@ -861,8 +861,8 @@ int ntc_hip_block_compress(const NtcHipBlockCompress* p)
     if (int r = require_init()) return r;
     if (!p || !p->dst) { set_error("ntc_hip_block_compress: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
     if (p->dstFormat < 1 || p->dstFormat > 7) { set_error("ntc_hip_block_compress: dstFormat (%d) is not a block-compressed format.", p->dstFormat); return NTC_HIP_ERR_INVALID_ARG; }
-    if (p->dstFormat > 5) {
-        set_error("ntc_hip_block_compress: BC6H and BC7 are not implemented (dstFormat %d).", p->dstFormat);
+    if (p->dstFormat == 6) {
+        set_error("ntc_hip_block_compress: BC6H is not implemented (dstFormat %d).", p->dstFormat);
         return NTC_HIP_ERR_UNSUPPORTED;
     }
     if (p->srcLeft < 0 || p->srcTop < 0 || p->widthInBlocks < 1 || p->heightInBlocks < 1 || p->dstOffsetX < 0 || p->dstOffsetY < 0
@@ -886,6 +886,23 @@ int ntc_hip_block_compress(const NtcHipBlockCompress* p)
     a.srcLeft = p->srcLeft; a.srcTop = p->srcTop; a.widthInBlocks = p->widthInBlocks; a.heightInBlocks = p->heightInBlocks;
     a.dstOffsetX = p->dstOffsetX; a.dstOffsetY = p->dstOffsetY;
     a.alphaThreshold = p->alphaThreshold;
+    if (p->dstFormat == 7 && p->modeBuffer) {
+        if (p->modeMapWidthInBlocks < 1 || p->modeMapHeightInBlocks < 1 || p->modeMapWidthInBlocks > (1 << 20) || p->modeMapHeightInBlocks > (1 << 20)
+            || p->modeMapOffsetX < -(1 << 20) || p->modeMapOffsetX > (1 << 20) || p->modeMapOffsetY < -(1 << 20) || p->modeMapOffsetY > (1 << 20)) {
+            set_error("ntc_hip_block_compress: bad mode map size or offset.");
+            return NTC_HIP_ERR_INVALID_ARG;
+        }
+        // size of MakeBC7ModeBuffer's output for the map: 9 bits per block, rounded up to whole 32-bit words
+        uint64_t const mapBytes = ((uint64_t(p->modeMapWidthInBlocks) * uint64_t(p->modeMapHeightInBlocks) * 9u + 31u) >> 5) << 2;
+        if ((p->modeBufferByteOffset & 3u) || (reinterpret_cast<uintptr_t>(p->modeBuffer) & 3u) || reaches_past(p->modeBufferByteOffset, mapBytes, p->modeBufferBytes)) {
+            set_error("ntc_hip_block_compress: the mode buffer (4-byte aligned, offset a multiple of 4) does not hold the %llu bytes of a %d x %d mode map.",
+                      (unsigned long long)mapBytes, p->modeMapWidthInBlocks, p->modeMapHeightInBlocks);
+            return NTC_HIP_ERR_INVALID_ARG;
+        }
+        a.modeBuffer = reinterpret_cast<uint32_t const*>(static_cast<uint8_t const*>(p->modeBuffer) + p->modeBufferByteOffset);
+        a.modeMapWidthInBlocks = p->modeMapWidthInBlocks; a.modeMapHeightInBlocks = p->modeMapHeightInBlocks;
+        a.modeMapOffsetX = p->modeMapOffsetX; a.modeMapOffsetY = p->modeMapOffsetY;
+    }
     HIP_TRY(launch_block_compress(a, p->dstFormat, g_lib.stream));
     clear_error();
     return 0;

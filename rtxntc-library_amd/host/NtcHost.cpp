@@ -1237,6 +1237,10 @@ public:
             SetErrorMessage("Invalid dstFormat (%s)", BlockCompressedFormatToString(params.dstFormat));
             return Status::OutOfRange;
         }
+        if (params.pModeBuffer && params.dstFormat != BlockCompressedFormat::BC7) {     // src/Context.cpp:666-671
+            SetErrorMessage("Mode buffer can only be used with BC7 compression");
+            return Status::InvalidArgument;
+        }
         if (!m_deviceAvailable) { SetErrorMessage("No HIP device is available to this context."); return Status::CudaUnavailable; }
         NtcHipBlockCompress p{};
         ImageDesc const& src = params.srcImage;
@@ -1248,6 +1252,9 @@ public:
         p.alphaThreshold = params.alphaThreshold;
         p.dstOffsetX = params.dstOffsetInBlocks.x; p.dstOffsetY = params.dstOffsetInBlocks.y;
         p.dst = params.pDstData; p.dstBytes = params.dstDataSize; p.dstRowPitch = params.dstRowPitch;
+        p.modeBuffer = params.pModeBuffer; p.modeBufferBytes = params.modeBufferSize; p.modeBufferByteOffset = params.modeBufferByteOffset;
+        p.modeMapWidthInBlocks = params.modeMapWidthInBlocks; p.modeMapHeightInBlocks = params.modeMapHeightInBlocks;
+        p.modeMapOffsetX = params.modeMapOffsetInBlocks.x; p.modeMapOffsetY = params.modeMapOffsetInBlocks.y;
         if (int r = ntc_hip_block_compress(&p)) return DeviceFailure(r);
         ClearErrorMessage();
         return Status::Ok;

@@ -206,18 +206,28 @@ struct ImageDifferenceParameters
 };
 
 // The fields of MakeBlockCompressionComputePassParameters (include/libntc/ntc.h:1050-1100) that BC1 ..
-// BC5 use, plus what a graphics application binds to that pass: the source image and the destination.
+// BC5 and BC7 use, plus what a graphics application binds to that pass: the source image and the destination.
 struct Point { int x = 0; int y = 0; };
 struct BlockCompressionParameters
 {
     ImageDesc srcImage;                 // device memory
     Rect srcRect;                       // pixels to compress; width and height are rounded up to whole blocks
     Point dstOffsetInBlocks;
-    BlockCompressedFormat dstFormat = BlockCompressedFormat::None;      // BC1 .. BC5
+    BlockCompressedFormat dstFormat = BlockCompressedFormat::None;      // BC1 .. BC5, BC7
     float alphaThreshold = 1.f / 255.f; // BC1: pixels with alpha at or below it may become transparent
     void* pDstData = nullptr;           // device memory: rows of 8-byte (BC1, BC4) or 16-byte (BC2, BC3, BC5) blocks
     size_t dstDataSize = 0;
     size_t dstRowPitch = 0;             // bytes per row of blocks
+    // BC7 with a mode buffer (the reference's modeBufferSource == Custom): device memory holding
+    // MakeBC7ModeBuffer's output for a map of modeMapWidthInBlocks x modeMapHeightInBlocks blocks; the block
+    // (x, y) of srcRect uses the map entry (x + modeMapOffsetInBlocks.x, y + modeMapOffsetInBlocks.y).
+    // Only the recorded mode and partition of each block are encoded then.  Null: every mode is tried.
+    void const* pModeBuffer = nullptr;
+    size_t modeBufferSize = 0;
+    uint64_t modeBufferByteOffset = 0;  // multiple of 4
+    Point modeMapOffsetInBlocks;
+    int modeMapWidthInBlocks = 0;
+    int modeMapHeightInBlocks = 0;
 };
 
 // Decoder families beyond the one compiled into LibNTC 0.9.2, selected with
@@ -377,7 +387,8 @@ public:
     virtual Status ComputeImageDifference(ImageDifferenceParameters const& params) const = 0;
     // Runs the block-compression pass that IContext::MakeBlockCompressionComputePass describes for a
     // graphics API (include/libntc/ntc.h:1213-1225, src/Context.cpp:630-779, src/shaders/CompressBC1.hlsl ..
-    // CompressBC5.hlsl) on the device, asynchronously.  BC1 .. BC5; BC6 and BC7 return Status::Unsupported.
+    // CompressBC5.hlsl, CompressBC7.hlsl) on the device, asynchronously.  BC1 .. BC5 and BC7; BC6 returns
+    // Status::Unsupported.
     virtual Status CompressBlocks(BlockCompressionParameters const& params) const = 0;
     // True when a gfx950 device was initialised (reference: IsCudaAvailable).
     virtual bool IsCudaAvailable() const = 0;

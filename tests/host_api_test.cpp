@@ -470,7 +470,29 @@ static int imageDifference()
             for (size_t bx = 0; bx < blocksX; ++bx)
                 CHECK(blocks[by * blocksX + bx] == ((bx < 8 && by < 4) ? 0xFFFFFFFF00000000ull : 0xAAAAAAAAFFFFFFFFull));
         bp.dstRowPitch = blocksX * 16;
+        // BC7 of the same image, then once more through the mode buffer made from those blocks: the same blocks.
+        // Opaque white is exact in BC7; the zero corner has alpha 0.
         bp.dstFormat = BlockCompressedFormat::BC7;
+        CHECK(ctx->CompressBlocks(bp) == Status::Ok);
+        CHECK(ntc_hip_download(blocks.data(), dBlocks, blocks.size() * 8) == 0);
+        {
+            std::vector<uint8_t> modes(GetBC7ModeBufferSize(int(blocksX), int(blocksY)), 0);
+            CHECK(MakeBC7ModeBuffer(int(blocksX), int(blocksY), blocks.data(), blocks.size() * 8, blocksX * 16, modes.data(), modes.size()) == Status::Ok);
+            void* dModes = nullptr;
+            CHECK(ntc_hip_alloc(&dModes, modes.size()) == 0 && ntc_hip_upload(dModes, modes.data(), modes.size()) == 0);
+            CHECK(ntc_hip_memset(dBlocks, 0, blocksX * blocksY * 16) == 0);
+            bp.pModeBuffer = dModes; bp.modeBufferSize = modes.size();
+            bp.modeMapWidthInBlocks = int(blocksX); bp.modeMapHeightInBlocks = int(blocksY);
+            CHECK(ctx->CompressBlocks(bp) == Status::Ok);
+            std::vector<uint64_t> again(blocks.size());
+            CHECK(ntc_hip_download(again.data(), dBlocks, again.size() * 8) == 0);
+            CHECK(again == blocks);
+            bp.dstFormat = BlockCompressedFormat::BC3;
+            CHECK(ctx->CompressBlocks(bp) == Status::InvalidArgument);
+            bp.pModeBuffer = nullptr;
+            CHECK(ntc_hip_free(dModes) == 0);
+        }
+        bp.dstFormat = BlockCompressedFormat::BC6;
         CHECK(ctx->CompressBlocks(bp) == Status::Unsupported);
         bp.dstFormat = BlockCompressedFormat::None;
         CHECK(ctx->CompressBlocks(bp) == Status::OutOfRange);

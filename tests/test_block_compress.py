@@ -180,7 +180,7 @@ def test_checker_block_geometry_and_inputs(ntc, oracle):
     part = oracle_bc(ntc, oracle, image, 4, 3, 4, 2, 2, left=8, top=4)
     assert np.array_equal(part, full[1:3, 2:4])
     p = ntc.abi.BlockCompress()
-    p.dstFormat = 7
+    p.dstFormat = 6
     assert oracle.ntc_oracle_block_compress(C.byref(p)) == -1
 
 
