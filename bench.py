@@ -60,7 +60,7 @@ def bench_copy_kernels(args, ntc, dev):
         wc.width, wc.height, wc.setChannels, wc.firstChannel, wc.numChannels = w, h, channels, 0, channels
         run = lambda: A.check(dev.lib.ntc_hip_write_channels(wc))
         bytes_per_texel, what = channels + 2 * channels, "WriteChannels, UNORM8 pixels -> internal fp16"
-    elif wl in ("bc1", "bc3", "bc5", "bc7"):
+    elif wl in ("bc1", "bc3", "bc5", "bc7", "bc7m"):
         # RGBA8 image (smooth + noise, a tenth of the pixels transparent) -> blocks
         xs, ys = np.meshgrid(np.arange(w, dtype=np.float32), np.arange(h, dtype=np.float32))
         img = np.stack([127 + 100 * np.sin(xs / (9 + 4 * c) + ys / (17 - 3 * c)) + rng.normal(0, 4, (h, w)) for c in range(4)], axis=2)
@@ -75,10 +75,25 @@ def bench_copy_kernels(args, ntc, dev):
         bc.widthInBlocks, bc.heightInBlocks, bc.dstFormat, bc.alphaThreshold = w // 4, h // 4, int(wl[2]), 1.0 / 255.0
         bc.dst, bc.dstBytes, bc.dstRowPitch = d_blocks.ptr, d_blocks.nbytes, (w // 4) * block_bytes
         run = lambda: A.check(dev.lib.ntc_hip_block_compress(bc))
-        if wl == "bc7":
+        if wl in ("bc7", "bc7m"):
             img[:, : w // 2, 3] = 255                            # left half opaque: every mode takes part there
             d_pixels = dev.upload(np.clip(np.rint(img), 0, 255).astype(np.uint8).reshape(-1))
             bc.src.data = d_pixels.ptr
+        if wl == "bc7m":
+            # the full search once; its modes and partitions, packed as MakeBC7ModeBuffer packs them (9 bits per
+            # block), then drive the timed single-mode encodes
+            run()
+            dev.synchronize()
+            first = d_blocks.download().view(np.uint32).reshape(-1, 4)[:, 0].astype(np.int64)
+            mode = np.minimum(7, np.log2(first & -first).astype(np.int64))
+            partition = (first >> (mode + 1)) & np.array([15, 63, 63, 63, 7, 3, 0, 63])[mode]
+            entry = (mode << 6) | partition
+            entry[entry == 0] = 0x1BF
+            bits = ((entry[:, None] >> np.arange(9)) & 1).astype(np.uint8).reshape(-1)
+            packed = np.packbits(bits, bitorder="little")
+            packed = np.concatenate([packed, np.zeros((-len(packed)) % 4 + 4, dtype=np.uint8)])
+            d_modes = dev.upload(packed)
+            bc.modeBuffer, bc.modeBufferBytes, bc.modeMapWidthInBlocks, bc.modeMapHeightInBlocks = d_modes.ptr, d_modes.nbytes, w // 4, h // 4
         if wl == "bc5":
             channels = 2
             bytes_per_texel, what = 2 + 1, "BC5 compression of the R and G channels of an RGBA8 image (2 B read, 1 B written per texel)"
@@ -86,6 +101,8 @@ def bench_copy_kernels(args, ntc, dev):
             channels = 4
             bytes_per_texel = 4 + block_bytes / 16
             what = f"{wl.upper()} compression of an RGBA8 image (4 B read, {block_bytes / 16:g} B written per texel)"
+            if wl == "bc7m":
+                what = "BC7 compression of an RGBA8 image with a mode buffer (each block's mode and partition given)"
     else:
         d_other = dev.upload(rng.integers(0, 0x3C00, w * h * channels, dtype=np.uint16))
         mse = (C.c_float * 16)()
@@ -115,7 +132,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=30)   # the GPU clock takes ~30 launches to settle
-    ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4", "ref092", "read", "write", "loss", "bc1", "bc3", "bc5", "bc7"])
+    ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4", "ref092", "read", "write", "loss", "bc1", "bc3", "bc5", "bc7", "bc7m"])
     ap.add_argument("--size", type=int, default=0, help="override the texture size of the workload")
     ap.add_argument("--format", choices=["fp16", "unorm8"], default=None)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="time budget of the CPU-baseline sample")
@@ -134,7 +151,7 @@ def main():
 
     dev = ntc.Device(0)
     wl = args.workload
-    if wl in ("read", "write", "loss", "bc1", "bc3", "bc5", "bc7"):
+    if wl in ("read", "write", "loss", "bc1", "bc3", "bc5", "bc7", "bc7m"):
         return bench_copy_kernels(args, ntc, dev)
     fmt_name = args.format or {"cfg2": "unorm8"}.get(wl, "fp16")
     fmt = A.OUT_FP16_PLANAR_PAIRS if fmt_name == "fp16" else A.OUT_UNORM8_PIXELS

@@ -71,6 +71,14 @@
  *                            HLSL leaves dot / lerp / fusion to the shader compiler: the float
  *                            operation order here is a choice, parity with the reference's exact
  *                            blocks is unpinned.
+ *   block_compress (BC7)     partition and anchor tables, typed from the BPTC specification, equal
+ *                            the reference's; a BC7 decoder written from the specification in
+ *                            numpy: every emitted block is valid and decodes close to its source
+ *                            (constant colours, alpha 0 / 1, one- / two- / three-region blocks,
+ *                            against BC1), each mode decodable when forced, and the single-mode
+ *                            path reproduces the full search's blocks
+ *                            (tests/test_block_compress_bc7.py).  Float operation order as for
+ *                            BC1: parity with the reference's exact blocks is unpinned.
  *   The exact bits of the reference's FP16-WMMA CUDA kernel (half accumulation order,
  *   --use_fast_math) and of a hardware bilinear sampler are NOT reproduced: parity unpinned
  *   for those two, by construction; the integer contract of Inference.hlsli is what is pinned.

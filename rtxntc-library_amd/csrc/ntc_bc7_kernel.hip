@@ -478,12 +478,15 @@ BC7_INLINE void dual_plane(int mode, bool wideColorIndex, Color<4> const (&rgba)
     best.error = error; best.lo = b.lo; best.hi = b.hi;
 }
 
-// One block.  fixedMode < 0: every mode is tried; otherwise only that mode with that partition (for
-// modes 4 / 5: rotation in bits 0-1 of the partition, "wide colour index" in bit 2).  Both cases run
-// through the same code, the fixed one with every range narrowed to one candidate.
-__device__ void bc7_encode(Color<4> const (&px)[16], int fixedMode, int fixedPartition, uint64_t& lo, uint64_t& hi)
+// One block.  FIXED false: every mode is tried; true: only fixedMode with fixedPartition (for modes 4 / 5:
+// rotation in bits 0-1 of the partition, "wide colour index" in bit 2).  Both cases run through the same
+// code, the fixed one with every range narrowed to one candidate.  (Two instantiations because in the
+// full search every lane of a wave walks the same partitions, so the subset masks are uniform and the
+// texel loops branch on scalar bits instead of being predicated per lane.)
+template <bool FIXED>
+BC7_INLINE void bc7_encode(Color<4> const (&px)[16], int fixedMode, int fixedPartition, uint64_t& lo, uint64_t& hi)
 {
-    bool const fixed = fixedMode >= 0;
+    constexpr bool fixed = FIXED;
     Best best{ FLT_MAX, 0, 0 };
     bool opaque = true;
 #pragma unroll
@@ -532,6 +535,7 @@ __device__ void bc7_encode(Color<4> const (&px)[16], int fixedMode, int fixedPar
 } // namespace
 
 // 8 x 8 blocks per 64-thread group: one wave, so that the register file of a SIMD is the only limit.
+template <bool FIXED>
 __global__ void __launch_bounds__(64)
 bc7_compress_kernel(BlockCompressArgs a)
 {
@@ -540,7 +544,7 @@ bc7_compress_kernel(BlockCompressArgs a)
     uint64_t lo, hi;
     int mode = -1, partition = 0;
     bool valid = true;
-    if (a.modeBuffer) {
+    if constexpr (FIXED) {
         // 9 bits per block of the mode map; 0 = no entry, 0x1BF stands for mode 0 partition 0
         int64_t const mx = int64_t(bx) + a.modeMapOffsetX, my = int64_t(by) + a.modeMapOffsetY;
         valid = mx >= 0 && my >= 0 && mx < a.modeMapWidthInBlocks && my < a.modeMapHeightInBlocks;
@@ -564,7 +568,7 @@ bc7_compress_kernel(BlockCompressArgs a)
 #pragma unroll
             for (int c = 0; c < 4; ++c) px[t].c[c] = source_channel(a, x, y, c);
         }
-        bc7_encode(px, mode, partition, lo, hi);
+        bc7_encode<FIXED>(px, mode, partition, lo, hi);
     } else {
         lo = 0x0001f00000f80004ull; hi = 0x1f9e00003ff0001full;       // the reference's marker: black, red, green and blue squares
     }
@@ -575,7 +579,8 @@ bc7_compress_kernel(BlockCompressArgs a)
 hipError_t launch_bc7_compress(BlockCompressArgs const& a, hipStream_t stream)
 {
     dim3 const grid((a.widthInBlocks + 7) / 8, (a.heightInBlocks + 7) / 8);
-    hipLaunchKernelGGL(bc7_compress_kernel, grid, dim3(64), 0, stream, a);
+    if (a.modeBuffer) hipLaunchKernelGGL(bc7_compress_kernel<true>, grid, dim3(64), 0, stream, a);
+    else              hipLaunchKernelGGL(bc7_compress_kernel<false>, grid, dim3(64), 0, stream, a);
     return hipGetLastError();
 }
 
