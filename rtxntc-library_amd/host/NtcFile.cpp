@@ -434,13 +434,13 @@ bool ReadTexture(Value const& v, Texture& out, std::string& error)
         && m.OptionalEnum("bcFormat", out.bcFormat, NTC_FILE_BC_FORMATS)
         && m.Array("bcModeBuffers", "array", modeBuffers)))
         return false;
-    // BC7 mode buffers belong to the block-compression step after decoding; their entries are
-    // checked for shape and otherwise left alone.
+    // BC7 mode buffers: which view holds the (mode, partition) map of which colour mip
     if (modeBuffers) for (Value const& item : modeBuffers->items) {
         if (!m.ElementMustBeObject("bcModeBuffers", item)) return false;
         Members b(item, "BCModeBuffer", error);
-        uint32_t mipLevel, view;
-        if (!(b.UInt("mipLevel", mipLevel) && b.UInt("view", view))) return false;
+        Texture::ModeBuffer ref;
+        if (!(b.UInt("mipLevel", ref.mipLevel) && b.UInt("view", ref.view))) return false;
+        out.bcModeBuffers.push_back(ref);
     }
     return true;
 }

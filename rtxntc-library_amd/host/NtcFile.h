@@ -57,6 +57,8 @@ struct Texture
     std::string name;
     uint32_t firstChannel = 0, numChannels = 0;
     std::optional<int> channelFormat, rgbColorSpace, alphaColorSpace, bcFormat;   // values of the public enums
+    struct ModeBuffer { uint32_t mipLevel = 0, view = 0; };
+    std::vector<ModeBuffer> bcModeBuffers;              // BC7 acceleration data, one view per colour mip
 };
 
 struct LatentImage

@@ -200,7 +200,52 @@ public:
     ColorSpace GetRgbColorSpace() const override { return m_rgbColorSpace; }
     void SetAlphaColorSpace(ColorSpace colorSpace) override { m_alphaColorSpace = colorSpace; }
     ColorSpace GetAlphaColorSpace() const override { return m_alphaColorSpace; }
+
+    // src/TextureMetadata.cpp:96-135
+    Status MakeAndStoreBC7ModeBuffer(int mipLevel, int widthInBlocks, int heightInBlocks,
+        void const* blockData, size_t blockDataSize, size_t rowPitch) override
+    {
+        if (mipLevel < 0 || mipLevel >= m_setDesc.mips) {
+            SetErrorMessage("mipLevel (%d) must be between 0 and %d.", mipLevel, m_setDesc.mips - 1);
+            return Status::OutOfRange;
+        }
+        int const mipWidthInBlocks = (std::max(1, m_setDesc.width >> mipLevel) + 3) / 4;
+        int const mipHeightInBlocks = (std::max(1, m_setDesc.height >> mipLevel) + 3) / 4;
+        if (widthInBlocks != mipWidthInBlocks || heightInBlocks != mipHeightInBlocks) {
+            SetErrorMessage("Provided widthInBlocks (%d) and heightInBlocks (%d) do not match the expected "
+                "dimensions (%d x %d) for mip level %d.", widthInBlocks, heightInBlocks, mipWidthInBlocks, mipHeightInBlocks, mipLevel);
+            return Status::InvalidArgument;
+        }
+        ModeBuffer& buffer = m_modeBuffers[size_t(mipLevel)];
+        buffer = ModeBuffer();
+        buffer.data.assign(GetBC7ModeBufferSize(mipWidthInBlocks, mipHeightInBlocks), 0);
+        Status const status = MakeBC7ModeBuffer(widthInBlocks, heightInBlocks, blockData, blockDataSize, rowPitch, buffer.data.data(), buffer.data.size());
+        if (status != Status::Ok) { buffer.data.clear(); return status; }
+        ClearErrorMessage();
+        return Status::Ok;
+    }
+    void GetBC7ModeBuffer(int mipLevel, void const** outData, size_t* outSize) const override
+    {
+        if (outData) *outData = nullptr;
+        if (outSize) *outSize = 0;
+        if (mipLevel < 0 || mipLevel >= NTC_HIP_MAX_MIPS || m_modeBuffers[size_t(mipLevel)].data.empty()) return;
+        if (outData) *outData = m_modeBuffers[size_t(mipLevel)].data.data();
+        if (outSize) *outSize = m_modeBuffers[size_t(mipLevel)].data.size();
+    }
+    BufferFootprint GetBC7ModeBufferFootprint(int mipLevel) const override
+    {
+        return (mipLevel < 0 || mipLevel >= NTC_HIP_MAX_MIPS) ? BufferFootprint() : m_modeBuffers[size_t(mipLevel)].footprint;
+    }
+    // Used by the file loader: where the file keeps the map of a mip, and the map itself once read.
+    void SetBC7ModeBufferFromFile(int mipLevel, BufferFootprint const& footprint, std::vector<uint8_t>&& data)
+    {
+        if (mipLevel < 0 || mipLevel >= NTC_HIP_MAX_MIPS) return;
+        m_modeBuffers[size_t(mipLevel)].footprint = footprint;
+        m_modeBuffers[size_t(mipLevel)].data = std::move(data);
+    }
 private:
+    struct ModeBuffer { std::vector<uint8_t> data; BufferFootprint footprint; };
+    ModeBuffer m_modeBuffers[NTC_HIP_MAX_MIPS];
     TextureSetDesc const& m_setDesc;
     std::string m_name;
     int m_firstChannel = 0, m_numChannels = 0;
@@ -582,6 +627,27 @@ public:
             texture->SetBlockCompressedFormat(BlockCompressedFormat(t.bcFormat.value_or(0)));
             texture->SetRgbColorSpace(ColorSpace(t.rgbColorSpace.value_or(0)));
             texture->SetAlphaColorSpace(ColorSpace(t.alphaColorSpace.value_or(0)));
+            // BC7 mode maps (src/TextureSetMetadata.cpp:470-476, src/TextureMetadata.cpp:151-213); a map stored with
+            // GDeflate is described by its footprint but not loaded
+            for (file::Texture::ModeBuffer const& ref : t.bcModeBuffers) {
+                if (!ValidateBufferView(ref.view, 0, document, binaryChunkSize)) return Status::FileUnrecognized;
+                file::BufferView const& view = document.views[ref.view];
+                BufferFootprint footprint;
+                footprint.rangeInStream = StreamRange{ view.offset + binaryChunkOffset, view.storedSize };
+                footprint.compressionType = CompressionType(int(view.compression.value_or(file::Compression::None)));
+                footprint.uncompressedSize = view.uncompressedSize.value_or(view.storedSize);
+                footprint.uncompressedCrc32 = view.crc32.value_or(0);
+                std::vector<uint8_t> data;
+                if (footprint.compressionType == CompressionType::None && view.storedSize != 0) {
+                    data.resize(size_t(view.storedSize));
+                    if (!stream->Seek(footprint.rangeInStream.offset) || !stream->Read(data.data(), data.size())) {
+                        SetErrorMessage("Failed to read BC7 mode buffer data of size %llu for mip level %u.",
+                            (unsigned long long)view.storedSize, ref.mipLevel);
+                        return Status::IOError;
+                    }
+                }
+                static_cast<TextureMetadata*>(texture)->SetBC7ModeBufferFromFile(int(ref.mipLevel), footprint, std::move(data));
+            }
         }
 
         // Channel headers

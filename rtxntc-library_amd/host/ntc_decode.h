@@ -40,6 +40,15 @@ enum class ColorSpace { Linear = 0, sRGB = 1, HLG = 2 };
 // include/libntc/ntc.h:285-293, 367-371
 enum class InferenceWeightType { Unknown = 0, GenericInt8 = 1, GenericFP8 = 2, CoopVecFP8 = 3, Count };
 enum class CompressionType { None = 0, GDeflate = 1 };
+// Where a buffer lies in a stream such as an NTC file and how it is stored (include/libntc/ntc.h:116-122,373-387).
+struct StreamRange { uint64_t offset = 0; uint64_t size = 0; };
+struct BufferFootprint
+{
+    StreamRange rangeInStream;
+    CompressionType compressionType = CompressionType::None;
+    uint64_t uncompressedSize = 0;      // equals rangeInStream.size when not compressed
+    uint32_t uncompressedCrc32 = 0;     // 0 = none recorded
+};
 
 // include/libntc/ntc.h:43-51
 struct VersionInfo
@@ -261,6 +270,17 @@ public:
     virtual ColorSpace GetRgbColorSpace() const = 0;
     virtual void SetAlphaColorSpace(ColorSpace colorSpace) = 0;
     virtual ColorSpace GetAlphaColorSpace() const = 0;
+    // BC7 acceleration data of one colour mip (include/libntc/ntc.h:437-453, src/TextureMetadata.cpp:96-223):
+    // MakeAndStoreBC7ModeBuffer extracts mode and partition of every block of a BC7-compressed mip (host
+    // memory; the block grid must be the mip's) and keeps them with the texture; GetBC7ModeBuffer returns the
+    // stored map (host memory, null / 0 when there is none) - upload it and pass it to
+    // IContext::CompressBlocks as pModeBuffer.  Maps stored uncompressed in an NTC file are loaded with the
+    // file; GetBC7ModeBufferFootprint says where a mip's map lies in the file and how it is stored (a
+    // GDeflate-compressed one is not loaded: GetBC7ModeBuffer then returns nothing).
+    virtual Status MakeAndStoreBC7ModeBuffer(int mipLevel, int widthInBlocks, int heightInBlocks,
+        void const* blockData, size_t blockDataSize, size_t rowPitch) = 0;
+    virtual void GetBC7ModeBuffer(int mipLevel, void const** outData, size_t* outSize) const = 0;
+    virtual BufferFootprint GetBC7ModeBufferFootprint(int mipLevel) const = 0;
     virtual ~ITextureMetadata() = default;
 };
 

@@ -57,6 +57,39 @@ static bool writeFile(std::string const& path, void const* p, size_t n)
 
 static int cpuChecks()
 {
+    {   // BC7 mode maps kept with a texture (include/libntc/ntc.h:437-453)
+        IContext* c = nullptr; ContextParameters cp; cp.cudaDevice = DisableCudaDevice;
+        (void)CreateContext(&c, cp);
+        CHECK(c != nullptr);
+        ITextureSet* set = nullptr;
+        TextureSetDesc desc; desc.width = 64; desc.height = 40; desc.channels = 4; desc.mips = 3;
+        CHECK(c->CreateTextureSet(desc, TextureSetFeatures(), &set) == Status::Ok);
+        ITextureMetadata* t = set->AddTexture();
+        CHECK(t != nullptr);
+        void const* data = reinterpret_cast<void const*>(1); size_t size = 1;
+        t->GetBC7ModeBuffer(1, &data, &size);
+        CHECK(data == nullptr && size == 0 && t->GetBC7ModeBufferFootprint(1).rangeInStream.size == 0);
+        // mip 1 is 32 x 20 pixels = 8 x 5 blocks; block n gets mode n % 8 and a partition from n
+        std::vector<uint32_t> blocks(8 * 5 * 4 + 4, 0);
+        for (uint32_t n = 0; n < 40; ++n) blocks[n * 4] = (1u << (n % 8)) | ((n * 7u % 64u) << (n % 8 + 1));
+        CHECK(t->MakeAndStoreBC7ModeBuffer(1, 8, 5, blocks.data(), 40 * 16, 8 * 16) == Status::Ok);
+        t->GetBC7ModeBuffer(1, &data, &size);
+        std::vector<uint8_t> direct(GetBC7ModeBufferSize(8, 5), 0);
+        CHECK(MakeBC7ModeBuffer(8, 5, blocks.data(), 40 * 16, 8 * 16, direct.data(), direct.size()) == Status::Ok);
+        CHECK(data != nullptr && size == direct.size() && std::memcmp(data, direct.data(), size) == 0);
+        CHECK(size == ((40 * 9 + 31) / 32) * 4);
+        t->GetBC7ModeBuffer(0, &data, &size);
+        CHECK(data == nullptr && size == 0);
+        CHECK(t->MakeAndStoreBC7ModeBuffer(1, 8, 4, blocks.data(), 40 * 16, 8 * 16) == Status::InvalidArgument);
+        CHECK(std::strstr(GetLastErrorMessage(), "do not match the expected dimensions (8 x 5)") != nullptr);
+        CHECK(t->MakeAndStoreBC7ModeBuffer(3, 2, 2, blocks.data(), 40 * 16, 8 * 16) == Status::OutOfRange);
+        CHECK(t->MakeAndStoreBC7ModeBuffer(1, 8, 5, blocks.data(), 39 * 16, 8 * 16) == Status::InvalidArgument);   // too little block data
+        t->GetBC7ModeBuffer(1, &data, &size);
+        CHECK(data == nullptr && size == 0);                                                                       // the failed call discarded the old map
+        c->DestroyTextureSet(set);
+        DestroyContext(c);
+    }
+
     IContext* ctx = nullptr;
     ContextParameters params;
     params.interfaceVersion = 0x12345678;
@@ -653,6 +686,16 @@ static void describe(ITextureSet* set)
         ITextureMetadata* t = set->GetTexture(i);
         std::printf("texture %s|%d|%d|%s|%d|%d|%d\n", t->GetName(), t->GetFirstChannel(), t->GetNumChannels(),
             ChannelFormatToString(t->GetChannelFormat()), int(t->GetBlockCompressedFormat()), int(t->GetRgbColorSpace()), int(t->GetAlphaColorSpace()));
+        for (int mip = 0; mip < d.mips; ++mip) {
+            BufferFootprint const fp = t->GetBC7ModeBufferFootprint(mip);
+            if (fp.rangeInStream.size == 0) continue;
+            void const* data = nullptr; size_t size = 0;
+            t->GetBC7ModeBuffer(mip, &data, &size);
+            unsigned long long sum = 0;
+            for (size_t b = 0; b < size; ++b) sum = sum * 131 + static_cast<unsigned char const*>(data)[b];
+            std::printf("modes %d %d %llu %llu %d %llu %zu %llu\n", i, mip, (unsigned long long)fp.rangeInStream.offset, (unsigned long long)fp.rangeInStream.size,
+                int(fp.compressionType), (unsigned long long)fp.uncompressedSize, size, sum);
+        }
     }
     std::printf("colorspaces");
     for (int c = 0; c < d.channels; ++c) std::printf(" %d", int(set->GetChannelStorageColorSpace(c)));

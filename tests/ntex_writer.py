@@ -71,7 +71,7 @@ def split_int8_blob(blob, widths=LAYER_WIDTHS_092):
 
 def write_ntex(width, height, channels, mips, grid_scale, features, latents, int8_blob, textures=(),
                fp8_version=True, layer_widths=None, layer_data=None, channel_color_spaces=None,
-               extra_document_fields=None, mutate=None, json_indent=None):
+               extra_document_fields=None, mutate=None, json_indent=None, mode_buffers=()):
     """Returns the bytes of an NTC file.
 
     latents: the quantised latent buffer, u16 layers neural LOD after neural LOD.
@@ -79,6 +79,7 @@ def write_ntex(width, height, channels, mips, grid_scale, features, latents, int
     layer_widths / layer_data: store narrower hidden layers: widths [(in, out)] x 4 and
         data [(weights int8 [out, in], scales f32 [out], biases i32 [out])] x 4.
     mutate(document): last-minute edits of the JSON document (for malformed-file tests).
+    mode_buffers: BC7 mode maps to store: (texture index, mip level, bytes, extra view fields or None).
     """
     latents = np.ascontiguousarray(latents).view(np.uint8)
     table = ViewTable()
@@ -131,6 +132,10 @@ def write_ntex(width, height, channels, mips, grid_scale, features, latents, int
                                       np.float32(grid_dim(height, nlod, grid_scale)) / np.float32(mh))
         lod = max(-1.0, min(1.0, 0.25 * math.log2(float(scale))))
         color_mips.append({"width": mw, "height": mh, "latentMip": nlod, "positionLod": lod, "positionScale": float(scale)})
+
+    textures = [dict(t) for t in textures]
+    for texture_index, mip_level, data, extra in mode_buffers:
+        textures[texture_index].setdefault("bcModeBuffers", []).append({"mipLevel": mip_level, "view": table.add(data, extra)})
 
     document = {
         "schemaVersion": SCHEMA_VERSION, "width": width, "height": height, "numChannels": channels, "numColorMips": mips,

@@ -209,6 +209,46 @@ def test_unknown_members_whitespace_and_escapes_are_tolerated(ntc, tmp_path):
     assert info["textures"] == ["tab\there|0|4|UNORM8|0|0|0"]
 
 
+def test_bc7_mode_maps_stored_in_a_file(ntc, tmp_path):
+    """bcModeBuffers of a texture (src/TextureSetMetadata.cpp:470-476, src/TextureMetadata.cpp:151-213): maps
+    stored as they are come back from GetBC7ModeBuffer, one stored with GDeflate is described by its
+    footprint only; the reference's front end accepts the same file."""
+    case = make_case(ntc)                                           # 64 x 32: mip 0 is 16 x 8 blocks, mip 1 8 x 4
+    rng = np.random.default_rng(11)
+    map0 = rng.integers(0, 256, ((16 * 8 * 9 + 31) // 32) * 4, dtype=np.uint8)
+    map1 = rng.integers(0, 256, ((8 * 4 * 9 + 31) // 32) * 4, dtype=np.uint8)
+    packed = rng.integers(0, 256, 20, dtype=np.uint8)
+    buffers = [(0, 0, map0.tobytes(), None), (0, 1, map1.tobytes(), None),
+               (0, 2, packed.tobytes(), {"compression": "GDeflate", "uncompressedSize": 12, "crc32": 1234})]
+    data = file_of(case, 64, 32, 2, 8, 8, textures=TEXTURES, mode_buffers=buffers)
+    lib = ref_file_lib()
+    if lib is not None:
+        assert ref_parse(lib, data)[0] == 0
+    path = tmp_path / "modes.ntc"
+    path.write_bytes(data)
+    out = run_exe("load", path, 0, 64, 32, 8, len(case.mips))
+    rows = [ln.split()[1:] for ln in out.splitlines() if ln.startswith("modes ")]
+    text, binary = nw.split_container(data)
+    doc = json.loads(text)
+    chunk_offset = len(data) - len(binary)
+    views = [doc["views"][b["view"]] for b in doc["textures"][0]["bcModeBuffers"]]
+
+    def digest(a):
+        total = 0
+        for byte in a.tolist():
+            total = (total * 131 + byte) % (1 << 64)
+        return total
+    assert rows == [
+        ["0", "0", str(views[0]["offset"] + chunk_offset), str(map0.size), "0", str(map0.size), str(map0.size), str(digest(map0))],
+        ["0", "1", str(views[1]["offset"] + chunk_offset), str(map1.size), "0", str(map1.size), str(map1.size), str(digest(map1))],
+        ["0", "2", str(views[2]["offset"] + chunk_offset), "20", "1", "12", "0", "0"]], rows
+    # a view index that does not exist is a malformed file
+    broken = file_of(case, 64, 32, 2, 8, 8, textures=TEXTURES, mode_buffers=buffers[:1],
+                     mutate=lambda d: d["textures"][0]["bcModeBuffers"][0].update(view=999))
+    status, message, _ = host_load(tmp_path, broken, dims=(64, 32, 8, len(case.mips)))
+    assert status == STATUS["FileUnrecognized"] and "Invalid view index" in message
+
+
 GOLDEN_JSON = os.path.join(HERE, "golden", "ntex_reference_json.json")
 
 
