@@ -60,7 +60,7 @@ def bench_copy_kernels(args, ntc, dev):
         wc.width, wc.height, wc.setChannels, wc.firstChannel, wc.numChannels = w, h, channels, 0, channels
         run = lambda: A.check(dev.lib.ntc_hip_write_channels(wc))
         bytes_per_texel, what = channels + 2 * channels, "WriteChannels, UNORM8 pixels -> internal fp16"
-    elif wl in ("bc1", "bc3", "bc5", "bc7", "bc7m"):
+    elif wl in ("bc1", "bc3", "bc5", "bc6", "bc7", "bc7m"):
         # RGBA8 image (smooth + noise, a tenth of the pixels transparent) -> blocks
         xs, ys = np.meshgrid(np.arange(w, dtype=np.float32), np.arange(h, dtype=np.float32))
         img = np.stack([127 + 100 * np.sin(xs / (9 + 4 * c) + ys / (17 - 3 * c)) + rng.normal(0, 4, (h, w)) for c in range(4)], axis=2)
@@ -132,7 +132,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=30)   # the GPU clock takes ~30 launches to settle
-    ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4", "ref092", "read", "write", "loss", "bc1", "bc3", "bc5", "bc7", "bc7m"])
+    ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4", "ref092", "read", "write", "loss", "bc1", "bc3", "bc5", "bc6", "bc7", "bc7m"])
     ap.add_argument("--size", type=int, default=0, help="override the texture size of the workload")
     ap.add_argument("--format", choices=["fp16", "unorm8"], default=None)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="time budget of the CPU-baseline sample")
@@ -151,7 +151,7 @@ def main():
 
     dev = ntc.Device(0)
     wl = args.workload
-    if wl in ("read", "write", "loss", "bc1", "bc3", "bc5", "bc7", "bc7m"):
+    if wl in ("read", "write", "loss", "bc1", "bc3", "bc5", "bc6", "bc7", "bc7m"):
         return bench_copy_kernels(args, ntc, dev)
     fmt_name = args.format or {"cfg2": "unorm8"}.get(wl, "fp16")
     fmt = A.OUT_FP16_PLANAR_PAIRS if fmt_name == "fp16" else A.OUT_UNORM8_PIXELS

@@ -310,9 +310,9 @@ typedef struct NtcHipImageDifference {
 } NtcHipImageDifference;
 int ntc_hip_image_difference(const NtcHipImageDifference* params);
 
-/* BC1 .. BC5 and BC7 compression of an image: the block-compression compute pass of
+/* BC1 .. BC7 compression of an image: the block-compression compute pass of
  * IContext::MakeBlockCompressionComputePass for those formats (include/libntc/ntc.h:1050-1100,
- * src/shaders/CompressBC1.hlsl .. CompressBC5.hlsl, CompressBC7.hlsl, src/shaders/BlockCompressCommon.hlsli).
+ * src/shaders/CompressBC1.hlsl .. CompressBC7.hlsl, src/shaders/BlockCompressCommon.hlsli).
  * widthInBlocks x heightInBlocks blocks of 4 x 4 pixels starting at (srcLeft, srcTop) are encoded and
  * stored row-major with dstRowPitch bytes per row of blocks, the first at block (dstOffsetX, dstOffsetY).
  * dstFormat is a BlockCompressedFormat:
@@ -323,7 +323,7 @@ int ntc_hip_image_difference(const NtcHipImageDifference* params);
  *   7  BC7, 16 bytes, from R, G, B and A (src/shaders/CompressBC7.hlsl); see modeBuffer below.  The
  *      reference's BC7 shader ignores dstOffsetInBlocks (CompressBC7.hlsl:1590); here it is honoured as for
  *      the other formats;
- *   6  (BC6H) returns NTC_HIP_ERR_UNSUPPORTED.
+ *   6  BC6H, unsigned half floats, 16 bytes, from R, G and B clamped to [0, 65504] (src/shaders/CompressBC6.hlsl);
  * Channels the image does not have read as 0 (alpha as 1); pixels outside the image read as 0 in every
  * channel, like a texture load there.  Asynchronous on the library stream. */
 typedef struct NtcHipBlockCompress {

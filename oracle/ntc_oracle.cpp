@@ -71,6 +71,13 @@
  *                            HLSL leaves dot / lerp / fusion to the shader compiler: the float
  *                            operation order here is a choice, parity with the reference's exact
  *                            blocks is unpinned.
+ *   block_compress (BC6H)    its deterministic log2 / exp2 against numpy's (2.5e-7 relative); a BC6H
+ *                            decoder written from the specification for the three modes emitted:
+ *                            constant blocks within one 10-bit endpoint step, 4-bit ramps to 2 %,
+ *                            two-region blocks in the two-subset modes, out-of-range texels clamped
+ *                            (tests/test_block_compress_bc6.py).  The shader's transcendental
+ *                            functions are hardware approximations: parity with its exact blocks is
+ *                            unpinned.
  *   block_compress (BC7)     partition and anchor tables, typed from the BPTC specification, equal
  *                            the reference's; a BC7 decoder written from the specification in
  *                            numpy: every emitted block is valid and decodes close to its source
@@ -1786,6 +1793,305 @@ void encode(const Color<4> px[16], int fixedMode, int fixedPartition, uint64_t o
 } // namespace bc7
 } // extern "C++"
 
+// ---- BC6H encoder, unsigned half floats (src/shaders/CompressBC6.hlsl) ----------------------------------
+// Two candidates per block, the smaller mean squared logarithmic error (luminance-weighted) wins:
+//   * one subset, 10-bit endpoints, 4-bit indices (mode 11): bounding box, inset in log2 space by at most 1/32
+//     of its extent towards the second-smallest / second-largest values, one least-squares refit;
+//   * two subsets, 3-bit indices, on the partition (of the format's first 32) whose texels lie closest to the
+//     two bounding-box diagonals: endpoints as 7-bit base + 6-bit deltas (mode 2) or 9-bit base + 5-bit deltas
+//     (mode 6), whichever decodes with the smaller error.
+// The shader's log2 / exp2 / rcp / normalize are hardware approximations there; here they are the
+// deterministic functions below (plain binary32 operations, so that checker and kernel agree bit for bit),
+// correct to a few units in the last place.  f32tof16 rounds to nearest even.  Texels are clamped to
+// [0, 65504] first (a NaN becomes 0): the shader feeds other values into conversions that are undefined.
+extern "C++" {
+namespace bc6 {
+namespace {
+
+float bits_to_float(uint32_t b) { float f; std::memcpy(&f, &b, 4); return f; }
+uint32_t float_to_bits(float f) { uint32_t b; std::memcpy(&b, &f, 4); return b; }
+
+// log2 for x >= 0 (0 -> -inf), NaN for negative or NaN input.
+float det_log2(float x)
+{
+    if (!(x >= 0.f)) return bits_to_float(0x7fc00000u);
+    if (x == 0.f) return bits_to_float(0xff800000u);
+    uint32_t b = float_to_bits(x);
+    if (b >= 0x7f800000u) return x;                                      // +inf
+    int e = 0;
+    if (b < 0x00800000u) { x *= 8388608.f; b = float_to_bits(x); e = -23; }      // subnormal
+    e += int(b >> 23) - 127;
+    float m = bits_to_float((b & 0x007fffffu) | 0x3f800000u);            // [1, 2)
+    if (m > 1.41421354f) { m *= 0.5f; e += 1; }
+    float const t = (m - 1.f) / (m + 1.f), t2 = t * t;
+    float p = t2 * (1.f / 9.f) + (1.f / 7.f);
+    p = p * t2 + 0.2f;
+    p = p * t2 + (1.f / 3.f);
+    p = p * t2 + 1.f;
+    return float(e) + p * t * 2.88539004f;                               // 2 / ln 2
+}
+
+// 2^x; overflows to +inf from 128, underflows to 0 below -150.
+float det_exp2(float x)
+{
+    if (x != x) return x;
+    if (x >= 128.f) return bits_to_float(0x7f800000u);
+    if (x < -150.f) return 0.f;
+    float const n = std::nearbyint(x), g = (x - n) * 0.693147182f;
+    float p = g * (1.f / 5040.f) + (1.f / 720.f);
+    p = p * g + (1.f / 120.f);
+    p = p * g + (1.f / 24.f);
+    p = p * g + (1.f / 6.f);
+    p = p * g + 0.5f;
+    p = p * g + 1.f;
+    p = p * g + 1.f;
+    int k = int(n);
+    if (k > 127) { p *= 2.f; k -= 1; }
+    if (k < -126) { p *= 5.96046448e-08f; k += 24; }                     // 2^-24
+    return p * bits_to_float(uint32_t(k + 127) << 23);
+}
+
+struct V3 { float x, y, z; };
+V3 operator+(V3 a, V3 b) { return { a.x + b.x, a.y + b.y, a.z + b.z }; }
+V3 operator-(V3 a, V3 b) { return { a.x - b.x, a.y - b.y, a.z - b.z }; }
+V3 operator*(V3 a, float s) { return { a.x * s, a.y * s, a.z * s }; }
+V3 operator*(V3 a, V3 b) { return { a.x * b.x, a.y * b.y, a.z * b.z }; }
+float dot(V3 a, V3 b) { return a.x * b.x + a.y * b.y + a.z * b.z; }
+V3 vmin(V3 a, V3 b) { return { std::fmin(a.x, b.x), std::fmin(a.y, b.y), std::fmin(a.z, b.z) }; }
+V3 vmax(V3 a, V3 b) { return { std::fmax(a.x, b.x), std::fmax(a.y, b.y), std::fmax(a.z, b.z) }; }
+template <class F> V3 map(V3 a, F f) { return { f(a.x), f(a.y), f(a.z) }; }
+float clampf(float v, float lo, float hi) { return std::fmin(std::fmax(v, lo), hi); }
+float to_half_bits(float v) { return v != v ? 32256.f : float(float_to_half_rne(v)); }     // f32tof16 as a number; any NaN -> 0x7e00
+float from_half_bits(float v) { return half_to_float(uint16_t(uint32_t(v))); }
+
+constexpr float kHalfMax = 65504.f;
+
+float msle(V3 a, V3 b)                                                   // hlsl:62-73
+{
+    V3 const d = map(V3{ (b.x + 1.f) / (a.x + 1.f), (b.y + 1.f) / (a.y + 1.f), (b.z + 1.f) / (a.z + 1.f) }, det_log2);
+    V3 const sq = d * d * V3{ 0.299f, 0.587f, 0.114f };
+    return sq.x + sq.y + sq.z;
+}
+
+// Partitions: the format's first 32 two-subset partitions (the same table as BC7) and their anchors.
+uint32_t subset_of(int pattern, int t) { return (bc7::masks().two[pattern][1] >> t) & 1u; }
+int fixup_of(int pattern) { return bc7::kAnchorSecondOfTwo[pattern]; }
+
+V3 quantize(V3 v, float levels) { return map(v, [&](float c) { return (to_half_bits(c) * levels) / 31744.f; }); }      // hlsl:111-124 (0x7bff + 1)
+V3 unquantize(V3 v, float levels) { return map(v, [&](float c) { return (c * 65536.f + 32768.f) / levels; }); }        // hlsl:126-139
+V3 interpolate(V3 e0, V3 e1, float weight)                              // hlsl:141-145
+{
+    return map((e0 * (64.f - weight) + e1 * weight + V3{ 32.f, 32.f, 32.f }) * (31.f / 4096.f), from_half_bits);
+}
+uint32_t index_of(float pos, float e0, float e1, float scale, float bias, float top)           // hlsl:161-171
+{
+    float const r = (pos - e0) / (e1 - e0);
+    return uint32_t(clampf(r * scale + bias + 0.5f, 0.f, top));
+}
+uint32_t index3(float pos, float e0, float e1) { return index_of(pos, e0, e1, 6.98182f, 0.00909f, 7.f); }
+uint32_t index4(float pos, float e0, float e1) { return index_of(pos, e0, e1, 14.93333f, 0.03333f, 15.f); }
+V3 direction(V3 lo, V3 hi) { V3 const d = hi - lo; float const s = d.x + d.y + d.z; return { d.x / s, d.y / s, d.z / s }; }
+
+void inset_box(const V3 px[16], V3& lo, V3& hi)                         // hlsl:183-207
+{
+    V3 innerLo = hi, innerHi = lo;
+    for (int t = 0; t < 16; ++t) {
+        V3 const p = px[t];
+        innerLo = vmin(innerLo, V3{ p.x == lo.x ? innerLo.x : p.x, p.y == lo.y ? innerLo.y : p.y, p.z == lo.z ? innerLo.z : p.z });
+        innerHi = vmax(innerHi, V3{ p.x == hi.x ? innerHi.x : p.x, p.y == hi.y ? innerHi.y : p.y, p.z == hi.z ? innerHi.z : p.z });
+    }
+    auto lg = [](float c) { return det_log2(c + 1.f); };
+    V3 const logInnerHi = map(innerHi, lg), logInnerLo = map(innerLo, lg);
+    V3 logHi = map(hi, lg), logLo = map(lo, lg);
+    V3 const ext = (logHi - logLo) * (1.f / 32.f);
+    logLo = logLo + vmin(logInnerLo - logLo, ext);
+    logHi = logHi - vmin(logHi - logInnerHi, ext);
+    lo = map(logLo, [](float c) { return det_exp2(c) - 1.f; });
+    hi = map(logHi, [](float c) { return det_exp2(c) - 1.f; });
+}
+
+// Least-squares endpoints (in half-bit space) for the indices the current endpoints give; `member` selects
+// the subset.  Returns false when the system is singular.  hlsl:239-326
+template <class Member> bool refit(const V3 px[16], Member member, bool fourBit, V3 lo, V3 hi, V3& outLo, V3& outHi)
+{
+    V3 const dir = direction(lo, hi);
+    float const e0 = to_half_bits(dot(lo, dir)), e1 = to_half_bits(dot(hi, dir));
+    V3 alphaSum{ 0, 0, 0 }, betaSum{ 0, 0, 0 };
+    float ab = 0, aa = 0, bb = 0;
+    for (int t = 0; t < 16; ++t) if (member(t)) {
+        float const pos = to_half_bits(dot(px[t], dir));
+        uint32_t const index = fourBit ? index4(pos, e0, e1) : index3(pos, e0, e1);
+        float const beta = clampf(float(index) / (fourBit ? 15.f : 7.f), 0.f, 1.f), alpha = 1.f - beta;
+        V3 const h = map(px[t], to_half_bits);
+        alphaSum = alphaSum + h * alpha; betaSum = betaSum + h * beta;
+        ab += alpha * beta; aa += alpha * alpha; bb += beta * beta;
+    }
+    float const det = aa * bb - ab * ab;
+    if (!(std::fabs(det) > 0.00001f)) return false;
+    float const rcp = 1.f / det;
+    // (the shader clamps these codes to 65504, which lets the codes of infinities and NaNs through; here to 0x7bff)
+    auto finish = [&](V3 v) { return map(v * rcp, [](float c) { return from_half_bits(clampf(c, 0.f, 31743.f)); }); };
+    outLo = finish(alphaSum * bb - betaSum * ab);
+    outHi = finish(betaSum * aa - alphaSum * ab);
+    return true;
+}
+
+struct Block { uint32_t w[4] = { 0, 0, 0, 0 }; float error = 0.f; };
+
+void encode_one_subset(const V3 px[16], Block& out)                     // hlsl:328-419
+{
+    V3 lo = px[0], hi = px[0];
+    for (int t = 1; t < 16; ++t) { lo = vmin(lo, px[t]); hi = vmax(hi, px[t]); }
+    V3 const boxLo = lo, boxHi = hi;
+    inset_box(px, lo, hi);
+    V3 fitLo, fitHi;
+    if (refit(px, [](int) { return true; }, true, lo, hi, fitLo, fitHi)) {
+        lo = vmin(vmax(fitLo, boxLo), boxHi);
+        hi = vmin(vmax(fitHi, boxLo), boxHi);
+    }
+    V3 const dir = direction(lo, hi);
+    V3 q0 = quantize(lo, 1024.f), q1 = quantize(hi, 1024.f);
+    float e0 = to_half_bits(dot(lo, dir)), e1 = to_half_bits(dot(hi, dir));
+    if (index4(to_half_bits(dot(px[0], dir)), e0, e1) > 7) { std::swap(e0, e1); std::swap(q0, q1); }
+    uint32_t index[16];
+    for (int t = 0; t < 16; ++t) index[t] = index4(to_half_bits(dot(px[t], dir)), e0, e1);
+    V3 const u0 = unquantize(q0, 1024.f), u1 = unquantize(q1, 1024.f);
+    float error = 0.f;
+    for (int t = 0; t < 16; ++t) error += msle(px[t], interpolate(u0, u1, std::floor((float(index[t]) * 64.f) / 15.f + 0.5f)));
+    out = Block();
+    out.error = error;
+    uint32_t const e[6] = { uint32_t(q0.x), uint32_t(q0.y), uint32_t(q0.z), uint32_t(q1.x), uint32_t(q1.y), uint32_t(q1.z) };
+    // mode 11: six 10-bit endpoint components from bit 5, then 4-bit indices (the first with 3 bits) from bit 65
+    unsigned __int128 bits = 0x03;
+    for (int i = 0; i < 6; ++i) bits |= (unsigned __int128)(e[i] & 0x3ffu) << (5 + 10 * i);
+    int at = 65;
+    for (int t = 0; t < 16; ++t) { int const n = t == 0 ? 3 : 4; bits |= (unsigned __int128)(index[t] & ((1u << n) - 1u)) << at; at += n; }
+    out.w[0] = uint32_t(bits); out.w[1] = uint32_t(bits >> 32); out.w[2] = uint32_t(bits >> 64); out.w[3] = uint32_t(bits >> 96);
+}
+
+float distance_to_line2(V3 origin, V3 dir, V3 p)                        // hlsl:421-426
+{
+    V3 const w = p - origin, x = w - dir * dot(w, dir);
+    return dot(x, x);
+}
+V3 normalized(V3 v) { float const len = std::sqrt(dot(v, v)); return { v.x / len, v.y / len, v.z / len }; }
+
+void subset_boxes(const V3 px[16], int pattern, V3 lo[2], V3 hi[2])
+{
+    for (int s = 0; s < 2; ++s) { lo[s] = V3{ kHalfMax, kHalfMax, kHalfMax }; hi[s] = V3{ 0, 0, 0 }; }
+    for (int t = 0; t < 16; ++t) { uint32_t const s = subset_of(pattern, t); lo[s] = vmin(lo[s], px[t]); hi[s] = vmax(hi[s], px[t]); }
+}
+
+float pattern_score(const V3 px[16], int pattern)                       // hlsl:428-470
+{
+    V3 lo[2], hi[2];
+    subset_boxes(px, pattern, lo, hi);
+    V3 const dir[2] = { normalized(hi[0] - lo[0]), normalized(hi[1] - lo[1]) };
+    float total = 0.f;
+    for (int t = 0; t < 16; ++t) { uint32_t const s = subset_of(pattern, t); total += distance_to_line2(lo[s], dir[s], px[t]); }
+    return total;
+}
+
+int as_int(float v) { return int(v); }
+// Two's complement field of `bits` bits of a small signed integer held in a float (hlsl:173-181).
+uint32_t field(float v, int bits) { return uint32_t(as_int(v)) & ((1u << bits) - 1u); }
+
+void encode_two_subsets(const V3 px[16], int pattern, Block& best)      // hlsl:472-733
+{
+    V3 lo[2], hi[2];
+    subset_boxes(px, pattern, lo, hi);
+    for (uint32_t s = 0; s < 2; ++s) {
+        V3 fitLo, fitHi;
+        if (refit(px, [&](int t) { return subset_of(pattern, t) == s; }, false, lo[s], hi[s], fitLo, fitHi)) { lo[s] = fitLo; hi[s] = fitHi; }
+    }
+    V3 const dir[2] = { direction(lo[0], hi[0]), direction(lo[1], hi[1]) };
+    float e0[2], e1[2];
+    for (int s = 0; s < 2; ++s) { e0[s] = to_half_bits(dot(lo[s], dir[s])); e1[s] = to_half_bits(dot(hi[s], dir[s])); }
+    int const anchor[2] = { 0, fixup_of(pattern) };
+    for (int s = 0; s < 2; ++s)
+        if (index3(to_half_bits(dot(px[anchor[s]], dir[s])), e0[s], e1[s]) > 3) { std::swap(e0[s], e1[s]); std::swap(lo[s], hi[s]); }
+    uint32_t index[16];
+    for (int t = 0; t < 16; ++t) {
+        uint32_t const s = subset_of(pattern, t);
+        index[t] = index3(to_half_bits(dot(px[t], dir[s])), e0[s], e1[s]);
+    }
+    // endpoints: base + three signed deltas, as 7 + 6 bits and as 9 + 5 bits
+    V3 const ends[4] = { lo[0], hi[0], lo[1], hi[1] };
+    V3 q7[4], q9[4], u7[4], u9[4];
+    auto fl = [](float c) { return std::floor(c); };
+    for (int i = 0; i < 4; ++i) { q7[i] = map(quantize(ends[i], 128.f), fl); q9[i] = map(quantize(ends[i], 512.f), fl); }
+    for (int i = 1; i < 4; ++i) {
+        q7[i] = map(q7[i] - q7[0], [](float c) { return clampf(c, -31.f, 31.f); });
+        q9[i] = map(q9[i] - q9[0], [](float c) { return clampf(c, -15.f, 15.f); });
+    }
+    u7[0] = unquantize(q7[0], 128.f); u9[0] = unquantize(q9[0], 512.f);
+    for (int i = 1; i < 4; ++i) { u7[i] = unquantize(q7[0] + q7[i], 128.f); u9[i] = unquantize(q9[0] + q9[i], 512.f); }
+    float error7 = 0.f, error9 = 0.f;
+    for (int t = 0; t < 16; ++t) {
+        uint32_t const s = subset_of(pattern, t);
+        float const weight = std::floor((float(index[t]) * 64.f) / 7.f + 0.5f);
+        error7 += msle(px[t], interpolate(u7[2 * s], u7[2 * s + 1], weight));
+        error9 += msle(px[t], interpolate(u9[2 * s], u9[2 * s + 1], weight));
+    }
+    float const error = std::fmin(error7, error9);
+    if (!(error < best.error)) return;
+    bool const sevenSix = error == error7;
+    V3 const* q = sevenSix ? q7 : q9;
+    int const baseBits = sevenSix ? 7 : 9, deltaBits = sevenSix ? 6 : 5;
+    // w = base, x / y / z = deltas of the first subset's second end and of the second subset's ends
+    uint32_t const rw = field(q[0].x, baseBits), gw = field(q[0].y, baseBits), bw = field(q[0].z, baseBits);
+    uint32_t const rx = field(q[1].x, deltaBits), gx = field(q[1].y, deltaBits), bx = field(q[1].z, deltaBits);
+    uint32_t const ry = field(q[2].x, deltaBits), gy = field(q[2].y, deltaBits), by = field(q[2].z, deltaBits);
+    uint32_t const rz = field(q[3].x, deltaBits), gz = field(q[3].y, deltaBits), bz = field(q[3].z, deltaBits);
+    unsigned __int128 bits = 0;
+    auto put = [&](int at, uint32_t value, int n) { bits |= (unsigned __int128)(value & ((1u << n) - 1u)) << at; };
+    auto bit = [](uint32_t v, int i) { return (v >> i) & 1u; };
+    if (sevenSix) {         // mode 2 of the format: 7.666
+        put(0, 0x01, 5);
+        put(2, bit(gy, 5), 1); put(3, bit(gz, 4), 1); put(4, bit(gz, 5), 1);
+        put(5, rw, 7); put(12, bit(bz, 0), 1); put(13, bit(bz, 1), 1); put(14, bit(by, 4), 1);
+        put(15, gw, 7); put(22, bit(by, 5), 1); put(23, bit(bz, 2), 1); put(24, bit(gy, 4), 1);
+        put(25, bw, 7); put(32, bit(bz, 3), 1); put(33, bit(bz, 5), 1); put(34, bit(bz, 4), 1);
+        put(35, rx, 6); put(41, gy, 4); put(45, gx, 6); put(51, gz, 4); put(55, bx, 6); put(61, by, 4);
+        put(65, ry, 6); put(71, rz, 6);
+    } else {                // mode 6 of the format: 9.555
+        put(0, 0x0E, 5);
+        put(5, rw, 9); put(14, bit(by, 4), 1); put(15, gw, 9); put(24, bit(gy, 4), 1); put(25, bw, 9); put(34, bit(bz, 4), 1);
+        put(35, rx, 5); put(40, bit(gz, 4), 1); put(41, gy, 4); put(45, gx, 5); put(50, bit(bz, 0), 1); put(51, gz, 4);
+        put(55, bx, 5); put(60, bit(bz, 1), 1); put(61, by, 4); put(65, ry, 5); put(70, bit(bz, 2), 1); put(71, rz, 5); put(76, bit(bz, 3), 1);
+    }
+    put(77, uint32_t(pattern), 5);
+    int at = 82;
+    for (int t = 0; t < 16; ++t) { int const n = (t == 0 || t == anchor[1]) ? 2 : 3; put(at, index[t], n); at += n; }
+    best.error = error;
+    best.w[0] = uint32_t(bits); best.w[1] = uint32_t(bits >> 32); best.w[2] = uint32_t(bits >> 64); best.w[3] = uint32_t(bits >> 96);
+}
+
+void encode(const float rgb[16][3], uint64_t out[2])                    // hlsl:735-778
+{
+    V3 px[16];
+    for (int t = 0; t < 16; ++t) px[t] = V3{ clampf(rgb[t][0], 0.f, kHalfMax), clampf(rgb[t][1], 0.f, kHalfMax), clampf(rgb[t][2], 0.f, kHalfMax) };
+    Block best;
+    encode_one_subset(px, best);
+    float bestScore = pattern_score(px, 0);
+    int bestPattern = 0;
+    for (int p = 1; p < 32; ++p) {
+        float const score = pattern_score(px, p);
+        if (score < bestScore) { bestPattern = p; bestScore = score; }
+    }
+    encode_two_subsets(px, bestPattern, best);
+    out[0] = uint64_t(best.w[0]) | (uint64_t(best.w[1]) << 32);
+    out[1] = uint64_t(best.w[2]) | (uint64_t(best.w[3]) << 32);
+}
+
+} // namespace
+} // namespace bc6
+} // extern "C++"
+
+// For tests: the deterministic log2 / exp2 of the BC6H encoder.
+float ntc_oracle_bc6_log2(float x) { return bc6::det_log2(x); }
+float ntc_oracle_bc6_exp2(float x) { return bc6::det_exp2(x); }
+
 // For tests: the single-colour tables (256 entries each, first endpoint | second << 8).
 void ntc_oracle_bc1_match_tables(uint16_t* five, uint16_t* six)
 {
@@ -1804,11 +2110,11 @@ void ntc_oracle_bc7_tables(uint32_t* two, uint32_t* three, uint8_t* anchors)
     }
 }
 
-// dstFormat 1..5 and 7 (BC1, BC2, BC3, BC4: channel R, BC5: R then G, BC7); host pointers in `p`.
-// Returns -1 for other formats.
+// dstFormat 1..7 (BC1, BC2, BC3, BC4: channel R, BC5: R then G, BC6H unsigned, BC7); host pointers in `p`.
+// Returns -1 for other values.
 int ntc_oracle_block_compress(const NtcHipBlockCompress* p)
 {
-    if (p->dstFormat < 1 || p->dstFormat > 7 || p->dstFormat == 6) return -1;
+    if (p->dstFormat < 1 || p->dstFormat > 7) return -1;
     auto fetch = [&](int x, int y, int c) -> float {
         if (x < 0 || y < 0 || x >= p->src.width || y >= p->src.height) return 0.f;
         return diff_channel(p->src, static_cast<uint8_t const*>(p->src.data) + size_t(y) * p->src.rowPitch + size_t(x) * p->src.pixelStride, c);
@@ -1823,6 +2129,11 @@ int ntc_oracle_block_compress(const NtcHipBlockCompress* p)
                     for (int t = 0; t < 16; ++t) texels[t] = fetch(p->srcLeft + bx * 4 + (t & 3), p->srcTop + by * 4 + (t >> 2), c);
                     words[c] = bc4::encode(texels);
                 }
+            } else if (p->dstFormat == 6) {
+                float rgb[16][3];
+                for (int t = 0; t < 16; ++t)
+                    for (int c = 0; c < 3; ++c) rgb[t][c] = fetch(p->srcLeft + bx * 4 + (t & 3), p->srcTop + by * 4 + (t >> 2), c);
+                bc6::encode(rgb, words);
             } else if (p->dstFormat == 7) {
                 bc7::Color<4> px[16];
                 for (int t = 0; t < 16; ++t)

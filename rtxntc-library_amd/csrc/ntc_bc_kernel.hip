@@ -527,6 +527,7 @@ hipError_t launch_block_compress(BlockCompressArgs const& a, int dstFormat, hipS
     case 3: hipLaunchKernelGGL(bc1_compress_kernel<3>, grid, dim3(128), 0, stream, a); break;
     case 4: hipLaunchKernelGGL(bc4_compress_kernel<1>, grid, dim3(128), 0, stream, a); break;
     case 5: hipLaunchKernelGGL(bc4_compress_kernel<2>, grid, dim3(128), 0, stream, a); break;
+    case 6: return launch_bc6_compress(a, stream);
     case 7: return launch_bc7_compress(a, stream);
     default: return hipErrorInvalidValue;
     }

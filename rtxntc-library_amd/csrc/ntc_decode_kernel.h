@@ -137,7 +137,8 @@ struct BlockCompressArgs {
 };
 // Sets `bytes` bytes at dst to `value` (any alignment).
 hipError_t launch_fill(uint8_t* dst, uint8_t value, uint64_t bytes, hipStream_t stream);
-hipError_t launch_block_compress(BlockCompressArgs const& args, int dstFormat /* 1..5, 7 */, hipStream_t stream);
+hipError_t launch_block_compress(BlockCompressArgs const& args, int dstFormat /* 1..7 */, hipStream_t stream);
+hipError_t launch_bc6_compress(BlockCompressArgs const& args, hipStream_t stream);
 hipError_t launch_bc7_compress(BlockCompressArgs const& args, hipStream_t stream);
 
 hipError_t launch_decode(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream);

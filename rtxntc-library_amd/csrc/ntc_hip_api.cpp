@@ -861,10 +861,6 @@ int ntc_hip_block_compress(const NtcHipBlockCompress* p)
     if (int r = require_init()) return r;
     if (!p || !p->dst) { set_error("ntc_hip_block_compress: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
     if (p->dstFormat < 1 || p->dstFormat > 7) { set_error("ntc_hip_block_compress: dstFormat (%d) is not a block-compressed format.", p->dstFormat); return NTC_HIP_ERR_INVALID_ARG; }
-    if (p->dstFormat == 6) {
-        set_error("ntc_hip_block_compress: BC6H is not implemented (dstFormat %d).", p->dstFormat);
-        return NTC_HIP_ERR_UNSUPPORTED;
-    }
     if (p->srcLeft < 0 || p->srcTop < 0 || p->widthInBlocks < 1 || p->heightInBlocks < 1 || p->dstOffsetX < 0 || p->dstOffsetY < 0
         || p->widthInBlocks > (1 << 20) || p->heightInBlocks > (1 << 20) || p->dstOffsetX > (1 << 20) || p->dstOffsetY > (1 << 20)) {
         set_error("ntc_hip_block_compress: bad extent or destination offset.");

@@ -215,16 +215,16 @@ struct ImageDifferenceParameters
 };
 
 // The fields of MakeBlockCompressionComputePassParameters (include/libntc/ntc.h:1050-1100) that BC1 ..
-// BC5 and BC7 use, plus what a graphics application binds to that pass: the source image and the destination.
+// BC7 use, plus what a graphics application binds to that pass: the source image and the destination.
 struct Point { int x = 0; int y = 0; };
 struct BlockCompressionParameters
 {
     ImageDesc srcImage;                 // device memory
     Rect srcRect;                       // pixels to compress; width and height are rounded up to whole blocks
     Point dstOffsetInBlocks;
-    BlockCompressedFormat dstFormat = BlockCompressedFormat::None;      // BC1 .. BC5, BC7
+    BlockCompressedFormat dstFormat = BlockCompressedFormat::None;      // BC1 .. BC7
     float alphaThreshold = 1.f / 255.f; // BC1: pixels with alpha at or below it may become transparent
-    void* pDstData = nullptr;           // device memory: rows of 8-byte (BC1, BC4) or 16-byte (BC2, BC3, BC5) blocks
+    void* pDstData = nullptr;           // device memory: rows of 8-byte (BC1, BC4) or 16-byte (all others) blocks
     size_t dstDataSize = 0;
     size_t dstRowPitch = 0;             // bytes per row of blocks
     // BC7 with a mode buffer (the reference's modeBufferSource == Custom): device memory holding
@@ -407,8 +407,7 @@ public:
     virtual Status ComputeImageDifference(ImageDifferenceParameters const& params) const = 0;
     // Runs the block-compression pass that IContext::MakeBlockCompressionComputePass describes for a
     // graphics API (include/libntc/ntc.h:1213-1225, src/Context.cpp:630-779, src/shaders/CompressBC1.hlsl ..
-    // CompressBC5.hlsl, CompressBC7.hlsl) on the device, asynchronously.  BC1 .. BC5 and BC7; BC6 returns
-    // Status::Unsupported.
+    // CompressBC7.hlsl) on the device, asynchronously.  All seven formats; BC6 is the unsigned variant.
     virtual Status CompressBlocks(BlockCompressionParameters const& params) const = 0;
     // True when a gfx950 device was initialised (reference: IsCudaAvailable).
     virtual bool IsCudaAvailable() const = 0;

@@ -525,8 +525,20 @@ static int imageDifference()
             bp.pModeBuffer = nullptr;
             CHECK(ntc_hip_free(dModes) == 0);
         }
+        // BC6H of the same image: the zero corner is the one-subset block with zero endpoints; the white blocks are
+        // all the same block in one of the three modes the encoder emits
         bp.dstFormat = BlockCompressedFormat::BC6;
-        CHECK(ctx->CompressBlocks(bp) == Status::Unsupported);
+        CHECK(ctx->CompressBlocks(bp) == Status::Ok);
+        CHECK(ntc_hip_download(blocks.data(), dBlocks, blocks.size() * 8) == 0);
+        {
+            uint64_t const whiteLo = blocks[(blocksY - 1) * blocksX * 2], whiteHi = blocks[(blocksY - 1) * blocksX * 2 + 1];
+            CHECK((whiteLo & 3u) == 1u || (whiteLo & 31u) == 0x0Eu || (whiteLo & 31u) == 0x03u);
+            for (size_t by = 0; by < blocksY; ++by)
+                for (size_t bx = 0; bx < blocksX; ++bx) {
+                    bool const corner = bx < 8 && by < 4;
+                    CHECK(blocks[(by * blocksX + bx) * 2] == (corner ? 0x03u : whiteLo) && blocks[(by * blocksX + bx) * 2 + 1] == (corner ? 0u : whiteHi));
+                }
+        }
         bp.dstFormat = BlockCompressedFormat::None;
         CHECK(ctx->CompressBlocks(bp) == Status::OutOfRange);
         bp.dstFormat = BlockCompressedFormat::BC4; bp.dstDataSize = 8;

@@ -78,6 +78,10 @@ def load_oracle():
         lib.ntc_oracle_resize_planar.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]
         lib.ntc_oracle_block_compress.restype = C.c_int
         lib.ntc_oracle_block_compress.argtypes = [C.c_void_p]
+        lib.ntc_oracle_bc6_log2.restype = C.c_float
+        lib.ntc_oracle_bc6_log2.argtypes = [C.c_float]
+        lib.ntc_oracle_bc6_exp2.restype = C.c_float
+        lib.ntc_oracle_bc6_exp2.argtypes = [C.c_float]
         lib.ntc_oracle_bc7_tables.restype = None
         lib.ntc_oracle_bc7_tables.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
         lib.ntc_oracle_bc1_match_tables.restype = None

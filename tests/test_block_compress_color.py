@@ -303,7 +303,7 @@ def test_gpu_colour_block_compress_three_channel_source_and_arguments(ntc, devic
     d_dst = device.upload(np.zeros(12 * 8 * 16, dtype=np.uint8))
     fill_image(p.src, d_src.ptr, d_src.nbytes, 3, 3 * 48, 48, 32, 1, 3)
     p.widthInBlocks, p.heightInBlocks, p.dst, p.dstBytes, p.dstRowPitch = 12, 8, d_dst.ptr, d_dst.nbytes, 12 * 16
-    for dst_format, status in ((6, ntc.abi.ERR_UNSUPPORTED), (0, ntc.abi.ERR_INVALID_ARG), (8, ntc.abi.ERR_INVALID_ARG)):
+    for dst_format, status in ((0, ntc.abi.ERR_INVALID_ARG), (8, ntc.abi.ERR_INVALID_ARG), (-1, ntc.abi.ERR_INVALID_ARG)):
         p.dstFormat = dst_format
         assert device.lib.ntc_hip_block_compress(p) == status
     p.dstFormat, p.dstBytes = 3, 12 * 8 * 16 - 1
