@@ -2117,7 +2117,8 @@ int ntc_oracle_block_compress(const NtcHipBlockCompress* p)
     if (p->dstFormat < 1 || p->dstFormat > 7) return -1;
     auto fetch = [&](int x, int y, int c) -> float {
         if (x < 0 || y < 0 || x >= p->src.width || y >= p->src.height) return 0.f;
-        return diff_channel(p->src, static_cast<uint8_t const*>(p->src.data) + size_t(y) * p->src.rowPitch + size_t(x) * p->src.pixelStride, c);
+        // "+ 0.f": a stored -0 becomes +0 (minima and maxima of +0 and -0 depend on the operand order otherwise)
+        return diff_channel(p->src, static_cast<uint8_t const*>(p->src.data) + size_t(y) * p->src.rowPitch + size_t(x) * p->src.pixelStride, c) + 0.f;
     };
     size_t const blockBytes = (p->dstFormat == 1 || p->dstFormat == 4) ? 8 : 16;
     for (int by = 0; by < p->heightInBlocks; ++by)

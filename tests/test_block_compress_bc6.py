@@ -202,6 +202,7 @@ def test_gpu_bc6_matches_checker(ntc, device, oracle, fmt):
         image = np.clip(np.rint(image * 4), 0, 255).astype(np.uint8)         # low dynamic range input works too
     else:
         image = image.astype(np.float16 if fmt == 3 else np.float32)
+        image[44:48, 60:64] = np.where(rng.random((4, 4, 3)) < 0.5, -0.0, 0.0)             # signed zeros
         if fmt == 4:
             image[5, 7, 1], image[33, 90, 2], image[40, 3, 0], image[41, 100, 1] = np.nan, np.inf, -3.0, 1e7
     blocks_x, blocks_y = (w + 3) // 4, (h + 3) // 4

@@ -321,6 +321,7 @@ def test_gpu_bc7_matches_checker(ntc, device, oracle, tables, fmt):
     else:
         image = (noisy * 1.2 - 0.1).astype(np.float16 if fmt == 3 else np.float32)
         image[:, : w // 2, 3] = 1.0
+        image[44:48, 60:64, :3] = np.where(rng.random((4, 4, 3)) < 0.5, -0.0, 0.0)     # signed zeros
         if fmt == 4:
             image[5, 7, 1] = np.nan
             image[33, 90, 3] = np.nan

@@ -276,6 +276,7 @@ def test_gpu_colour_block_compress_matches_checker(ntc, device, oracle, fmt, dst
     else:
         wild = noisy * 1.3 - 0.15                                                                        # values outside [0, 1]
         image = wild.astype(np.float16 if fmt == 3 else np.float32)
+        image[44:48, 60:64, :3] = np.where(rng.random((4, 4, 3)) < 0.5, -0.0, 0.0)                          # signed zeros
         if fmt == 4:
             image[5, 7, 1] = np.nan
             image[33, 90, 3] = np.nan
