@@ -341,8 +341,9 @@ bc6_compress_kernel(BlockCompressArgs a)
 #pragma unroll
     for (int t = 0; t < 16; ++t) {
         int const x = a.srcLeft + bx * 4 + (t & 3), y = a.srcTop + by * 4 + (t >> 2);
-        px[t] = V3{ clampf(source_channel(a, x, y, 0), 0.f, kHalfMax), clampf(source_channel(a, x, y, 1), 0.f, kHalfMax),
-                    clampf(source_channel(a, x, y, 2), 0.f, kHalfMax) };
+        float c[4];
+        source_pixel(a, x, y, c);
+        px[t] = V3{ clampf(c[0], 0.f, kHalfMax), clampf(c[1], 0.f, kHalfMax), clampf(c[2], 0.f, kHalfMax) };
     }
     Block best = encode_one_subset(px);
     float bestScore = pattern_score(px, kSecondSubset[0]);

@@ -532,58 +532,103 @@ BC7_INLINE void bc7_encode(Color<4> const (&px)[16], int fixedMode, int fixedPar
     lo = best.lo; hi = best.hi;
 }
 
+BC7_INLINE void load_block(BlockCompressArgs const& a, int bx, int by, Color<4> (&px)[16])
+{
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+        int const x = a.srcLeft + bx * 4 + (t & 3), y = a.srcTop + by * 4 + (t >> 2);
+        source_pixel(a, x, y, px[t].c);
+    }
+}
+BC7_INLINE void store_block(BlockCompressArgs const& a, int bx, int by, uint64_t lo, uint64_t hi)
+{
+    uint64_t* const dst = reinterpret_cast<uint64_t*>(a.dst + size_t(by + a.dstOffsetY) * a.dstRowPitch) + size_t(bx + a.dstOffsetX) * 2;
+    dst[0] = lo; dst[1] = hi;
+}
+
 } // namespace
 
-// 8 x 8 blocks per 64-thread group, registers capped at 256 so that two waves share a SIMD: the full
-// search is a long chain of scalar branches over uniform subset masks, and a second wave fills the
+// Full search.  8 x 8 blocks per 64-thread group, registers capped at 256 so that two waves share a SIMD:
+// the search is a long chain of scalar branches over uniform subset masks, and a second wave fills the
 // issue slots the first one leaves (1.7 times faster than one wave with 263 registers; three waves
 // with 168 registers spill and are slower than one).
-template <bool FIXED>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2)))
 bc7_compress_kernel(BlockCompressArgs a)
 {
     int const bx = blockIdx.x * 8 + (threadIdx.x & 7), by = blockIdx.y * 8 + (threadIdx.x >> 3);
     if (bx >= a.widthInBlocks || by >= a.heightInBlocks) return;
+    Color<4> px[16];
+    load_block(a, bx, by, px);
     uint64_t lo, hi;
-    int mode = -1, partition = 0;
-    bool valid = true;
-    if constexpr (FIXED) {
-        // 9 bits per block of the mode map; 0 = no entry, 0x1BF stands for mode 0 partition 0
-        int64_t const mx = int64_t(bx) + a.modeMapOffsetX, my = int64_t(by) + a.modeMapOffsetY;
-        valid = mx >= 0 && my >= 0 && mx < a.modeMapWidthInBlocks && my < a.modeMapHeightInBlocks;
-        if (valid) {
-            uint64_t const bit = (uint64_t(my) * uint64_t(a.modeMapWidthInBlocks) + uint64_t(mx)) * 9u;
-            uint32_t const* words = a.modeBuffer + (bit >> 5);
-            uint32_t const shift = uint32_t(bit & 31u);
-            uint32_t entry = words[0] >> shift;
-            if (shift > 23u) entry |= words[1] << (32u - shift);
-            entry &= 0x1FFu;
-            valid = entry != 0u;
-            if (entry == 0x1BFu) entry = 0u;
-            mode = int((entry >> 6) & 7u); partition = int(entry & 63u);
+    bc7_encode<false>(px, -1, 0, lo, hi);
+    store_block(a, bx, by, lo, hi);
+}
+
+// With a mode buffer.  A workgroup covers 16 x 16 blocks; its threads first read their blocks' entries,
+// then trade blocks through LDS so that thread i takes the i-th block in order of mode: the waves of the
+// group then run (nearly) one mode each instead of every mode some lane of theirs happens to have
+// (the reference's ReorderThreadsByMode, CompressBC7.hlsl:1445-1509).  Which thread encodes which block
+// depends on the order the LDS counters are hit in; what is written for a block does not.
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
+bc7_compress_modes_kernel(BlockCompressArgs a)
+{
+    __shared__ uint32_t counts[8];
+    __shared__ uint32_t tasks[8][256];
+    if (threadIdx.x < 8) counts[threadIdx.x] = 0;
+    __syncthreads();
+    {
+        int const bx = blockIdx.x * 16 + (threadIdx.x & 15), by = blockIdx.y * 16 + (threadIdx.x >> 4);
+        if (bx < a.widthInBlocks && by < a.heightInBlocks) {
+            // 9 bits per block of the mode map; 0 = no entry, 0x1BF stands for mode 0 partition 0
+            int64_t const mx = int64_t(bx) + a.modeMapOffsetX, my = int64_t(by) + a.modeMapOffsetY;
+            uint32_t entry = 0;
+            if (mx >= 0 && my >= 0 && mx < a.modeMapWidthInBlocks && my < a.modeMapHeightInBlocks) {
+                uint64_t const bit = (uint64_t(my) * uint64_t(a.modeMapWidthInBlocks) + uint64_t(mx)) * 9u;
+                uint32_t const* words = a.modeBuffer + (bit >> 5);
+                uint32_t const shift = uint32_t(bit & 31u);
+                entry = words[0] >> shift;
+                if (shift > 23u) entry |= words[1] << (32u - shift);
+                entry &= 0x1FFu;
+            }
+            if (entry == 0u) {
+                store_block(a, bx, by, 0x0001f00000f80004ull, 0x1f9e00003ff0001full);     // the reference's marker: black, red, green and blue squares
+            } else {
+                if (entry == 0x1BFu) entry = 0u;
+                uint32_t const mode = (entry >> 6) & 7u;
+                uint32_t const slot = atomicAdd(&counts[mode], 1u);
+                tasks[mode][slot] = ((entry & 63u) << 8) | threadIdx.x;
+            }
         }
     }
-    if (valid) {
-        Color<4> px[16];
+    __syncthreads();
+    uint32_t rank = threadIdx.x, task = 0;
+    int mode = -1;
 #pragma unroll
-        for (int t = 0; t < 16; ++t) {
-            int const x = a.srcLeft + bx * 4 + (t & 3), y = a.srcTop + by * 4 + (t >> 2);
-#pragma unroll
-            for (int c = 0; c < 4; ++c) px[t].c[c] = source_channel(a, x, y, c);
+    for (int m = 0; m < 8; ++m) {
+        uint32_t const n = counts[m];
+        if (mode < 0) {
+            if (rank < n) { mode = m; task = tasks[m][rank]; }
+            else rank -= n;
         }
-        bc7_encode<FIXED>(px, mode, partition, lo, hi);
-    } else {
-        lo = 0x0001f00000f80004ull; hi = 0x1f9e00003ff0001full;       // the reference's marker: black, red, green and blue squares
     }
-    uint64_t* const dst = reinterpret_cast<uint64_t*>(a.dst + size_t(by + a.dstOffsetY) * a.dstRowPitch) + size_t(bx + a.dstOffsetX) * 2;
-    dst[0] = lo; dst[1] = hi;
+    if (mode < 0) return;
+    int const bx = blockIdx.x * 16 + int(task & 15u), by = blockIdx.y * 16 + int((task >> 4) & 15u);
+    Color<4> px[16];
+    load_block(a, bx, by, px);
+    uint64_t lo, hi;
+    bc7_encode<true>(px, mode, int(task >> 8), lo, hi);
+    store_block(a, bx, by, lo, hi);
 }
 
 hipError_t launch_bc7_compress(BlockCompressArgs const& a, hipStream_t stream)
 {
-    dim3 const grid((a.widthInBlocks + 7) / 8, (a.heightInBlocks + 7) / 8);
-    if (a.modeBuffer) hipLaunchKernelGGL(bc7_compress_kernel<true>, grid, dim3(64), 0, stream, a);
-    else              hipLaunchKernelGGL(bc7_compress_kernel<false>, grid, dim3(64), 0, stream, a);
+    if (a.modeBuffer) {
+        dim3 const grid((a.widthInBlocks + 15) / 16, (a.heightInBlocks + 15) / 16);
+        hipLaunchKernelGGL(bc7_compress_modes_kernel, grid, dim3(256), 0, stream, a);
+    } else {
+        dim3 const grid((a.widthInBlocks + 7) / 8, (a.heightInBlocks + 7) / 8);
+        hipLaunchKernelGGL(bc7_compress_kernel, grid, dim3(64), 0, stream, a);
+    }
     return hipGetLastError();
 }
 

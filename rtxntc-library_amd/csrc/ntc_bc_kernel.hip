@@ -485,7 +485,9 @@ bc1_compress_kernel(BlockCompressArgs a)
 #pragma unroll
     for (int t = 0; t < 16; ++t) {
         int const x = a.srcLeft + bx * 4 + (t & 3), y = a.srcTop + by * 4 + (t >> 2);
-        px[t] = Rgba{ source_channel(a, x, y, 0), source_channel(a, x, y, 1), source_channel(a, x, y, 2), source_channel(a, x, y, 3) };
+        float c[4];
+        source_pixel(a, x, y, c);
+        px[t] = Rgba{ c[0], c[1], c[2], c[3] };
         if constexpr (FORMAT != 1) { alpha[t] = px[t].a; px[t].a = 1.f; }
     }
     uint64_t const color = bc1_encode(px, FORMAT == 1, a.alphaThreshold);

@@ -134,6 +134,7 @@ struct BlockCompressArgs {
     // BC7: 9-bit (mode, partition) entries of a modeMapWidthInBlocks x modeMapHeightInBlocks map, or null
     uint32_t const* modeBuffer;
     int32_t modeMapWidthInBlocks, modeMapHeightInBlocks, modeMapOffsetX, modeMapOffsetY;
+    int32_t packedRgba8;        // source = four UNORM8 channels, every pixel 4-byte aligned
 };
 // Sets `bytes` bytes at dst to `value` (any alignment).
 hipError_t launch_fill(uint8_t* dst, uint8_t value, uint64_t bytes, hipStream_t stream);

@@ -878,6 +878,8 @@ int ntc_hip_block_compress(const NtcHipBlockCompress* p)
     }
     a.src = image.data; a.pixelStride = image.pixelStride; a.rowPitch = image.rowPitch; a.format = image.format; a.numChannels = image.numChannels;
     a.srcWidth = p->src.width; a.srcHeight = p->src.height;
+    a.packedRgba8 = image.format == NTC_HIP_DEV_FORMAT_UNORM8 && image.numChannels == 4
+        && ((reinterpret_cast<uintptr_t>(image.data) | image.pixelStride | image.rowPitch) & 3u) == 0;
     a.dst = static_cast<uint8_t*>(p->dst); a.dstRowPitch = p->dstRowPitch;
     a.srcLeft = p->srcLeft; a.srcTop = p->srcTop; a.widthInBlocks = p->widthInBlocks; a.heightInBlocks = p->heightInBlocks;
     a.dstOffsetX = p->dstOffsetX; a.dstOffsetY = p->dstOffsetY;

@@ -225,3 +225,23 @@ def test_gpu_block_compress_matches_checker(ntc, device, oracle, fmt, dst_format
     p.dstBytes = d_dst.nbytes
     p.dstRowPitch = pitch - 4
     assert device.lib.ntc_hip_block_compress(p) == ntc.abi.ERR_INVALID_ARG
+
+
+def test_unorm_quotient_shortcut_is_exact():
+    """The kernels turn UNORM8 / UNORM16 texels into floats with q = k * r, q + fma(-q, d, k) * r (r = 1 / d
+    rounded) instead of a division; that is the correctly rounded k / d for every k (exact rationals here)."""
+    from fractions import Fraction
+
+    def rn32(value):
+        f = np.float32(float(value))
+        candidates = [f, np.nextafter(f, np.float32(np.inf)), np.nextafter(f, np.float32(-np.inf))]
+        return min(candidates, key=lambda c: (abs(Fraction(float(c)) - value), int(np.float32(c).view(np.uint32)) & 1))
+    for d in (255, 65535):
+        r = np.float32(1.0) / np.float32(d)
+        ks = range(d + 1) if d == 255 else list(range(0, 65536, 7)) + [65535, 65534, 32768, 32767, 1, 2, 3]
+        for k in ks:
+            q = np.float32(k) * r
+            rem = rn32(Fraction(float(-q)) * d + k)
+            q2 = rn32(Fraction(float(rem)) * Fraction(float(r)) + Fraction(float(q)))
+            assert q2 == np.float32(k) / np.float32(d), (d, k)
+
