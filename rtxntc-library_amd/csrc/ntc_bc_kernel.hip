@@ -67,20 +67,25 @@ __device__ __forceinline__ float bc4_assign(uint32_t const (&values)[16], uint64
     float total = 0.f;
 #pragma unroll
     for (int t = 0; t < 16; ++t) {
-        int best = 0x7fffffff;
-        uint32_t pick = 0;
+        // key = distance * 8 + entry: the smallest key is the nearest entry, the first among equally near ones
+        uint32_t key[8];
 #pragma unroll
-        for (uint32_t k = 0; k < 8; ++k) {
-            int const d = int(values[t]) - int(palette[k]);
-            if (d * d < best) { best = d * d; pick = k; }
-        }
-        total += float(best);
-        block |= uint64_t(pick) << (16 + 3 * t);
+        for (uint32_t k = 0; k < 8; ++k) key[k] = (__sad(int(values[t]), int(palette[k]), 0u) << 3) + k;
+        uint32_t const best = min(min(min(key[0], key[1]), min(key[2], key[3])), min(min(key[4], key[5]), min(key[6], key[7])));
+        uint32_t const distance = best >> 3;
+        total += float(distance * distance);
+        block |= uint64_t(best & 7u) << (16 + 3 * t);
     }
     return total;
 }
 
 __device__ __forceinline__ uint32_t bc4_endpoint(float v) { return uint32_t(rintf(fminf(fmaxf(v, 0.f), 255.f))); }   // a NaN becomes 0
+
+// Weight of endpoint 0 in palette entry k, for the eight-value and the six-value palette (entries 6 and 7
+// of the latter are the constants 0 and 255 and take no part in a fit): the quotients the fit divides
+// out, (8 - k) / 7 and (6 - k) / 5, evaluated once by the compiler.
+__constant__ float kWeight8[8] = { 1.f, 0.f, 6.f / 7.f, 5.f / 7.f, 4.f / 7.f, 3.f / 7.f, 2.f / 7.f, 1.f / 7.f };
+__constant__ float kWeight6[8] = { 1.f, 0.f, 4.f / 5.f, 3.f / 5.f, 2.f / 5.f, 1.f / 5.f, 0.f, 0.f };
 
 // Least-squares endpoints for the block's current assignment.  With `eightValues` every texel takes
 // part and weights are 1, 0, 6/7 ... 1/7; otherwise indices 6 and 7 (the fixed 0 and 255) are left
@@ -91,11 +96,8 @@ __device__ __forceinline__ uint64_t bc4_refit(uint32_t const (&values)[16], uint
 #pragma unroll
     for (int t = 0; t < 16; ++t) {
         uint32_t const k = bc4_index(block, t);
-        float alpha;
-        if (k < 2) alpha = 1.f - float(k);
-        else if (eightValues) alpha = (8.f - float(k)) / 7.f;
-        else if (k < 6) alpha = (6.f - float(k)) / 5.f;
-        else continue;
+        if (!eightValues && k >= 6) continue;
+        float const alpha = eightValues ? kWeight8[k] : kWeight6[k];
         float const beta = 1.f - alpha, x = float(values[t]);
         aa += alpha * alpha; bb += beta * beta; ab += alpha * beta;
         ax += alpha * x; bx += beta * x;
