@@ -278,6 +278,7 @@ def main():
             cpu = {"value": n / t / 1e9, "unit": "Gtexels/s", "cores": cores, "kind": "port",
                    "sample": f"the first {n} queries of the same list, {t:.1f} s"}
 
+    headline = wl == "cfg1" and fmt_name == "fp16" and not args.size
     line = {
         "metric": "decoded Gtexels/s, 4096^2 16-ch set, 64-48-32 int8; % of int8-MFMA/HBM roof",
         "value": gtexels, "unit": "Gtexels/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -288,9 +289,14 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved_gbs / HBM_PEAK_GBS,
                      # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE (profiles/), headline workload only
-                     "traffic": 766.4e6 if (wl == "cfg1" and fmt_name == "fp16" and not args.size) else None,
+                     "traffic": 766.4e6 if headline else None,
                      "kernel_ms": kernel_ms, "bytes_per_texel": bytes_per_texel,
-                     "mfma_achieved_tops": achieved_tops, "mfma_frac": achieved_tops / INT8_PEAK_TOPS},
+                     "mfma_achieved_tops": achieved_tops, "mfma_frac": achieved_tops / INT8_PEAK_TOPS,
+                     # what actually binds the headline kernel: vector-instruction issue.  1263 vector operations per texel
+                     # (rocprofv3 SQ_INSTS_VALU, profiles/) against 64 lanes per CU and clock at 2.4 GHz
+                     "valu_ops_per_texel": 1263 if headline else None,
+                     "valu_ceiling_gtexels": dev.compute_units * 64 * 2.4 / 1263 if headline else None,
+                     "valu_frac": (texels / (kernel_ms * 1e-3) / 1e9) / (dev.compute_units * 64 * 2.4 / 1263) if headline else None},
         "cpu_baseline": cpu,
     }
     print(json.dumps(line))
