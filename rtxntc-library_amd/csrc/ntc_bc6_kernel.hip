@@ -78,8 +78,8 @@ BC6_INLINE V3 operator-(V3 a, V3 b) { return { a.x - b.x, a.y - b.y, a.z - b.z }
 BC6_INLINE V3 operator*(V3 a, float s) { return { a.x * s, a.y * s, a.z * s }; }
 BC6_INLINE V3 operator*(V3 a, V3 b) { return { a.x * b.x, a.y * b.y, a.z * b.z }; }
 BC6_INLINE float dot(V3 a, V3 b) { return a.x * b.x + a.y * b.y + a.z * b.z; }
-BC6_INLINE V3 vmin(V3 a, V3 b) { return { fminf(a.x, b.x), fminf(a.y, b.y), fminf(a.z, b.z) }; }
-BC6_INLINE V3 vmax(V3 a, V3 b) { return { fmaxf(a.x, b.x), fmaxf(a.y, b.y), fmaxf(a.z, b.z) }; }
+BC6_INLINE V3 vmin(V3 a, V3 b) { return { min_f32(a.x, b.x), min_f32(a.y, b.y), min_f32(a.z, b.z) }; }
+BC6_INLINE V3 vmax(V3 a, V3 b) { return { max_f32(a.x, b.x), max_f32(a.y, b.y), max_f32(a.z, b.z) }; }
 BC6_INLINE float clampf(float v, float lo, float hi) { return fminf(fmaxf(v, lo), hi); }
 // A float as the number of its half-precision bit pattern, and back (the latter truncates to an integer first).
 // (a NaN always gives the code 0x7e00, whatever its sign and payload)

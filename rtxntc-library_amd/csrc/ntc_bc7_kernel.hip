@@ -115,7 +115,7 @@ template <int C> BC7_INLINE void min_max(Color<C> const (&px)[16], uint32_t mask
     for (int t = 0; t < 16; ++t)
         if (has_texel(mask, t)) {
 #pragma unroll
-            for (int k = 0; k < C; ++k) { lo.c[k] = fminf(lo.c[k], px[t].c[k]); hi.c[k] = fmaxf(hi.c[k], px[t].c[k]); }
+            for (int k = 0; k < C; ++k) { lo.c[k] = min_f32(lo.c[k], px[t].c[k]); hi.c[k] = max_f32(hi.c[k], px[t].c[k]); }
         }
 }
 

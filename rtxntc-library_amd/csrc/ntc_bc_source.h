@@ -7,6 +7,12 @@
 
 namespace ntc_hip_dev {
 
+// fminf / fmaxf as single instructions.  The compiler brackets the library functions with two
+// canonicalising instructions (it cannot know that its operands are already quiet); v_min_f32 /
+// v_max_f32 themselves return the other operand when one is a NaN, which is all fminf / fmaxf promise.
+__device__ __forceinline__ float min_f32(float a, float b) { float r; asm("v_min_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b)); return r; }
+__device__ __forceinline__ float max_f32(float a, float b) { float r; asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b)); return r; }
+
 // k / d for an integer k in [0, d], d = 255 or 65535, r = 1 / d rounded: one Newton step on k * r gives the
 // correctly rounded quotient for every such k (all 256 + 65536 cases are checked in the tests with exact
 // rational arithmetic) at a third of the instructions of a division.
