@@ -449,6 +449,28 @@ public:
     }
     int GetNumLatentImages() const override { return m_numNeuralLods; }
 
+    // src/TextureSetMetadata.cpp:119-144
+    Status GetLatentTextureFootprint(int latentMipLevel, int arrayLayer, LatentTextureFootprint& outFootprint) const override
+    {
+        if (latentMipLevel < 0 || latentMipLevel >= m_numNeuralLods) {
+            SetErrorMessage("latentMipLevel (%d) must be between 0 and %d", latentMipLevel, m_numNeuralLods - 1);
+            return Status::OutOfRange;
+        }
+        int const arraySize = (m_latentShape.numFeatures + 3) / 4;
+        if (arrayLayer < 0 || arrayLayer >= arraySize) {
+            SetErrorMessage("arrayLayer (%d) must be between 0 and %d", arrayLayer, arraySize);
+            return Status::OutOfRange;
+        }
+        outFootprint = LatentTextureFootprint();
+        size_t const index = size_t(latentMipLevel) * size_t(arraySize) + size_t(arrayLayer);
+        if (index < m_latentFootprints.size()) outFootprint.buffer = m_latentFootprints[index];
+        outFootprint.width = GridDimension(m_desc.width, latentMipLevel, m_latentShape.gridSizeScale);
+        outFootprint.height = GridDimension(m_desc.height, latentMipLevel, m_latentShape.gridSizeScale);
+        outFootprint.rowPitch = size_t(outFootprint.width) * 2u;      // FeatureGridMath::BytesPerLatentPixel
+        ClearErrorMessage();
+        return Status::Ok;
+    }
+
     Status GetFusedMipLevels(int mipLevel, int* pOutFirstFusedMip, int* pOutLastFusedMip) const override
     {
         if (m_numNeuralLods == 0) { SetErrorMessage("This decoder geometry has no shared latent images."); return Status::Unsupported; }
@@ -739,6 +761,7 @@ public:
 
         // Latents: u16 layers, neural LOD after neural LOD (src/FeatureGridHost.cpp:140-161).
         std::vector<uint8_t> latents;
+        std::vector<BufferFootprint> footprints;
         for (int neuralLod = 0; neuralLod < neuralLods; ++neuralLod) {
             file::LatentImage const& image = document.latents[size_t(neuralLod)];
             size_t const layerSize = size_t(image.width) * size_t(image.height) * 2u;
@@ -749,6 +772,11 @@ public:
                     SetErrorMessage("Latent image view %d is stored with GDeflate compression, which this library does not decode.", int(viewIndex));
                     return Status::Unsupported;
                 }
+                BufferFootprint footprint;
+                footprint.rangeInStream = StreamRange{ view.offset + binaryChunkOffset, view.storedSize };
+                footprint.uncompressedSize = view.storedSize;
+                footprint.uncompressedCrc32 = view.crc32.value_or(0);
+                footprints.push_back(footprint);
                 size_t const at = latents.size();
                 latents.resize(at + layerSize);
                 if (!(stream->Seek(binaryChunkOffset + view.offset) && stream->Read(latents.data() + at, layerSize))) {
@@ -761,6 +789,7 @@ public:
         // Same order as the reference: the shape is (re)applied, then the data goes in.
         m_latentShape = LatentShape::Empty();
         if (Status st = SetLatentShape(shape); st != Status::Ok) return st;
+        m_latentFootprints = std::move(footprints);     // file metadata: valid whether or not the uploads below succeed
         if (latents.size() != m_latentBytes || blob.size() != m_weightLayout.bufferSize) { SetErrorMessage("Inconsistent sizes for MLP or latent data"); return Status::InternalError; }
         if (Status st = SetWeightData(blob.data(), blob.size()); st != Status::Ok) return st;
         if (Status st = SetLatentData(latents.data(), latents.size()); st != Status::Ok) return st;
@@ -1144,6 +1173,7 @@ private:
     {
         ReleaseDevice(m_latents); ReleaseDevice(m_weights);
         m_hostWeights.clear();
+        m_latentFootprints.clear();
         m_latentBytes = 0; m_haveLatents = m_haveWeights = false;
         m_numNeuralLods = 0;
         m_state = NetworkState::Empty;
@@ -1164,6 +1194,7 @@ private:
         if (ntc_hip_weight_layout(&m_spec, &m_weightLayout) != 0) { SetErrorMessage("%s", ntc_hip_last_error()); return Status::InternalError; }
         ReleaseDevice(m_latents); ReleaseDevice(m_weights);
         m_hostWeights.clear();
+        m_latentFootprints.clear();
         m_haveLatents = m_haveWeights = false;
         if (m_deviceAvailable) {
             if (int r = ntc_hip_alloc(&m_latents, m_latentBytes)) return AllocationFailure(r, "latent", m_latentBytes);
@@ -1254,6 +1285,7 @@ private:
     int m_numNeuralLods = 0;                       // shared-LOD geometry only
     int m_neuralLodOfMip[NTC_HIP_MAX_MIPS] = {};
     std::vector<uint8_t> m_hostWeights;
+    std::vector<BufferFootprint> m_latentFootprints;    // per (latent image, layer) of the file last loaded; empty otherwise
     ShuffleSource m_shuffle[NTC_HIP_MAX_CHANNELS];
     void ResetShuffle() { for (int ch = 0; ch < NTC_HIP_MAX_CHANNELS; ++ch) m_shuffle[ch] = ShuffleSource::Channel(ch); }
     int m_maskChannelIndex = -1;

@@ -49,6 +49,13 @@ struct BufferFootprint
     uint64_t uncompressedSize = 0;      // equals rangeInStream.size when not compressed
     uint32_t uncompressedCrc32 = 0;     // 0 = none recorded
 };
+struct LatentTextureFootprint
+{
+    BufferFootprint buffer;
+    int width = 0;
+    int height = 0;
+    size_t rowPitch = 0;                // bytes
+};
 
 // include/libntc/ntc.h:43-51
 struct VersionInfo
@@ -315,6 +322,11 @@ public:
     // other decoder presets every colour mip owns its grids and these return zeros / Status::Unsupported.
     virtual LatentTextureDesc GetLatentTextureDesc() const = 0;
     virtual int GetNumLatentImages() const = 0;
+    // Where one layer (four features) of one latent image lies in the file the set was loaded from, and its
+    // size (include/libntc/ntc.h:530-537,577-581, src/TextureSetMetadata.cpp:119-144): for callers that stream
+    // latent layers themselves.  OutOfRange for indices outside the set; the footprint is empty (size 0) when
+    // the set was not loaded from a file.
+    virtual Status GetLatentTextureFootprint(int latentMipLevel, int arrayLayer, LatentTextureFootprint& outFootprint) const = 0;
     // The range of colour mips decoded from the same latent image as mipLevel.
     virtual Status GetFusedMipLevels(int mipLevel, int* pOutFirstFusedMip, int* pOutLastFusedMip) const = 0;
     // The range of colour mips whose high-resolution grid is latent image latentImageIndex.

@@ -688,7 +688,7 @@ static int loss(int argc, char** argv)
     return 0;
 }
 
-static void describe(ITextureSet* set)
+static int describe(ITextureSet* set)
 {
     TextureSetDesc const& d = set->GetDesc();
     std::printf("desc %d %d %d %d\n", d.width, d.height, d.channels, d.mips);
@@ -709,9 +709,28 @@ static void describe(ITextureSet* set)
                 int(fp.compressionType), (unsigned long long)fp.uncompressedSize, size, sum);
         }
     }
+    LatentTextureDesc const lt = set->GetLatentTextureDesc();
+    for (int level = 0; level < set->GetNumLatentImages(); ++level)
+        for (int layer = 0; layer < lt.arraySize; ++layer) {
+            LatentTextureFootprint fp;
+            CHECK(set->GetLatentTextureFootprint(level, layer, fp) == Status::Ok);
+            std::printf("latent %d %d %llu %llu %d %llu %u %d %d %zu\n", level, layer, (unsigned long long)fp.buffer.rangeInStream.offset,
+                (unsigned long long)fp.buffer.rangeInStream.size, int(fp.buffer.compressionType), (unsigned long long)fp.buffer.uncompressedSize,
+                fp.buffer.uncompressedCrc32, fp.width, fp.height, fp.rowPitch);
+        }
+    {
+        LatentTextureFootprint fp;
+        CHECK(set->GetLatentTextureFootprint(-1, 0, fp) == Status::OutOfRange);
+        CHECK(set->GetLatentTextureFootprint(set->GetNumLatentImages(), 0, fp) == Status::OutOfRange);
+        if (set->GetNumLatentImages() > 0) {
+            CHECK(set->GetLatentTextureFootprint(0, -1, fp) == Status::OutOfRange);
+            CHECK(set->GetLatentTextureFootprint(0, lt.arraySize, fp) == Status::OutOfRange);
+        }
+    }
     std::printf("colorspaces");
     for (int c = 0; c < d.channels; ++c) std::printf(" %d", int(set->GetChannelStorageColorSpace(c)));
     std::printf("\nmask 0x%x\n", set->GetValidChannelMask());
+    return 0;
 }
 
 static int load(int argc, char** argv)
@@ -733,7 +752,7 @@ static int load(int argc, char** argv)
         CHECK((status == Status::Ok) == (set != nullptr));
     }
     std::printf("status %d %s\nmessage %s\n", int(status), StatusToString(status), GetLastErrorMessage());
-    if (set) { describe(set); ctx->DestroyTextureSet(set); }
+    if (set) { CHECK(describe(set) == 0); ctx->DestroyTextureSet(set); }
     DestroyContext(ctx);
     return 0;
 }
@@ -750,7 +769,7 @@ static int decodeFile(int argc, char** argv)
     features.stagingBytesPerPixel = 16 * 2;
     ITextureSet* set = nullptr;
     CHECK(ctx->CreateCompressedTextureSetFromMemory(image.data(), image.size(), features, &set) == Status::Ok);
-    describe(set);
+    CHECK(describe(set) == 0);
     CHECK(set->Decompress(nullptr) == Status::Ok);
     TextureSetDesc const desc = set->GetDesc();
     for (int mip = 0; mip < desc.mips; ++mip) {

@@ -98,6 +98,21 @@ def test_writer_files_are_accepted_by_the_reference_front_end_and_by_the_host_la
     assert info["sizes"] == f"{case.latents.nbytes} 9472"
     assert info["textures"] == ["albedo|0|3|UNORM8|7|1|0", 'normal "ts"|3|2|UNORM16|0|0|0', "height|7|1|FLOAT32|0|0|2"]
     assert info["mask"] == "0x9f"
+    # file footprint of every latent layer (include/libntc/ntc.h:577-581): offsets from the start of the file,
+    # in the order the views were written, each one layer of u16 cells
+    text, binary = nw.split_container(data)
+    doc = json.loads(text)
+    chunk_offset = len(data) - len(binary)
+    rows = [ln.split()[1:] for ln in run_exe("load", tmp_path / "case.ntc", 0, width, height, 8, len(case.mips)).splitlines() if ln.startswith("latent ")]
+    expected = []
+    for level, image in enumerate(doc["latents"]):
+        assert len(image["layerViews"]) == (features + 3) // 4
+        for layer, view_index in enumerate(image["layerViews"]):
+            view = doc["views"][view_index]
+            size = image["width"] * image["height"] * 2
+            assert view["storedSize"] == size
+            expected.append([str(v) for v in (level, layer, view["offset"] + chunk_offset, size, 0, size, 0, image["width"], image["height"], image["width"] * 2)])
+    assert rows == expected and len(rows) > 0
 
 
 def malformed_variants(ntc):
