@@ -506,6 +506,28 @@ public:
         return Status::Ok;
     }
 
+    // FillColorMipConstants, GetWeightOffsets, GetPackedColorSpaces (src/TextureSetMetadata.cpp:786-858)
+    void FillInferenceConstants(int firstLatentMipInTexture, NtcTextureSetConstants& constants) const
+    {
+        for (int mip = 0; mip < m_desc.mips; ++mip) {
+            NtcColorMipConstants& colorMip = constants.colorMips[mip];
+            colorMip.neuralMip = m_neuralLodOfMip[mip] - firstLatentMipInTexture;
+            colorMip.positionLod = m_mips[mip].positionLod;
+            colorMip.positionScale = m_mips[mip].positionScale;
+        }
+        for (int layer = 0; layer < NTC_HIP_MLP_LAYERS; ++layer) {
+            constants.networkWeightOffsets[layer] = int(m_weightLayout.weightOffset[layer]);
+            constants.networkBiasOffsets[layer] = int(m_weightLayout.biasOffset[layer]);
+            constants.networkScaleOffsets[layer] = int(m_weightLayout.scaleOffset[layer]);
+        }
+        constants.imageWidth = m_desc.width;
+        constants.imageHeight = m_desc.height;
+        constants.imageMips = m_desc.mips;
+        constants.validChannelMask = GetValidChannelMask();
+        for (int channel = 0; channel < NTC_HIP_MAX_CHANNELS; ++channel)
+            constants.channelColorSpaces |= uint32_t(GetChannelStorageColorSpace(channel)) << (2 * channel);
+    }
+
     bool IsInferenceWeightTypeSupported(InferenceWeightType weightType) const override
     {
         return weightType == InferenceWeightType::GenericInt8 && !m_hostWeights.empty();
@@ -827,7 +849,9 @@ public:
     Status SetWeightData(void const* data, size_t size) override
     {
         Status const st = Upload(data, size, m_weightLayout.bufferSize, m_weights, "weight", m_haveWeights);
-        if (st == Status::Ok) {                              // the copy GetInferenceWeights hands out; a new blob starts un-shuffled
+        // The copy GetInferenceWeights hands out; a new blob starts un-shuffled.  A context without a device keeps
+        // it too (the blob passed every check but the upload), as the reference's metadata-only objects do.
+        if (st == Status::Ok || st == Status::CudaUnavailable) {
             m_hostWeights.assign(static_cast<uint8_t const*>(data), static_cast<uint8_t const*>(data) + size);
             ResetShuffle();
         }
@@ -1414,6 +1438,33 @@ public:
     void CloseMemory(IStream* stream) const override { delete stream; }
 
     // src/Context.cpp:296-352
+    // src/Context.cpp:864-922
+    Status MakeInferenceData(ITextureSet* textureSet, InferenceWeightType weightType, int firstLatentMipInTexture,
+        InferenceData* pOutInferenceData) const override
+    {
+        if (!pOutInferenceData) { SetErrorMessage("pOutInferenceData is NULL"); return Status::InvalidArgument; }
+        TextureSet* const set = dynamic_cast<TextureSet*>(textureSet);
+        if (!set) { SetErrorMessage("textureSetMetadata is NULL or points at a wrong object type"); return Status::InvalidArgument; }
+        switch (weightType) {
+        case InferenceWeightType::GenericInt8: case InferenceWeightType::GenericFP8: case InferenceWeightType::CoopVecFP8: break;
+        default:
+            SetErrorMessage("Unsupported weightType (%s)", InferenceWeightTypeToString(weightType));
+            return Status::Unsupported;
+        }
+        if (!set->IsInferenceWeightTypeSupported(weightType)) {
+            SetErrorMessage("The texture set does not provide %s weights", InferenceWeightTypeToString(weightType));
+            return Status::Unsupported;
+        }
+        if (set->GetNumLatentImages() == 0) {
+            SetErrorMessage("This decoder geometry has no shared latent images.");
+            return Status::Unsupported;
+        }
+        std::memset(pOutInferenceData, 0, sizeof(InferenceData));
+        set->FillInferenceConstants(firstLatentMipInTexture, pOutInferenceData->constants);
+        ClearErrorMessage();
+        return Status::Ok;
+    }
+
     Status CreateCompressedTextureSetFromStream(IStream* inputStream, TextureSetFeatures const& features, ITextureSet** pOutTextureSet) const override
     {
         if (!pOutTextureSet) { SetErrorMessage("pOutTextureSet is NULL."); return Status::InvalidArgument; }

@@ -57,6 +57,32 @@ struct LatentTextureFootprint
     size_t rowPitch = 0;                // bytes
 };
 
+// What a shader (or any other kernel) that decodes single texels of a set needs besides the latents and the
+// weight blob (include/libntc/shaders/InferenceConstants.h:43-85, include/libntc/ntc.h:359-365).
+struct NtcColorMipConstants
+{
+    int neuralMip;          // latent image of the colour mip, counted from firstLatentMipInTexture
+    float positionLod;
+    float positionScale;
+    int pad;
+};
+struct NtcTextureSetConstants
+{
+    NtcColorMipConstants colorMips[16];
+    int networkWeightOffsets[4];
+    int networkBiasOffsets[4];
+    int networkScaleOffsets[4];
+    int imageWidth;
+    int imageHeight;
+    int imageMips;
+    int pad0;
+    unsigned int validChannelMask;
+    unsigned int channelColorSpaces;    // 2 bits per channel
+    int pad1;
+    int pad2;
+};
+struct InferenceData { NtcTextureSetConstants constants; };
+
 // include/libntc/ntc.h:43-51
 struct VersionInfo
 {
@@ -421,6 +447,12 @@ public:
     // graphics API (include/libntc/ntc.h:1213-1225, src/Context.cpp:630-779, src/shaders/CompressBC1.hlsl ..
     // CompressBC7.hlsl) on the device, asynchronously.  All seven formats; BC6 is the unsigned variant.
     virtual Status CompressBlocks(BlockCompressionParameters const& params) const = 0;
+    // Fills the constants for decoding single texels of a set outside this library (include/libntc/ntc.h:1251-1255,
+    // src/Context.cpp:864-922): per colour mip the latent image and the position constants, the offsets of
+    // every layer's weights, scales and biases in the blob GetInferenceWeights returns, the image size, the
+    // valid-channel mask and the packed storage colour spaces.  Sets with shared latent images only.
+    virtual Status MakeInferenceData(ITextureSet* textureSet, InferenceWeightType weightType, int firstLatentMipInTexture,
+        InferenceData* pOutInferenceData) const = 0;
     // True when a gfx950 device was initialised (reference: IsCudaAvailable).
     virtual bool IsCudaAvailable() const = 0;
     virtual ~IContext() = default;

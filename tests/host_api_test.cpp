@@ -158,6 +158,35 @@ static int cpuChecks()
     CHECK(set->SetWeightData(blob.data(), 100) == Status::InvalidArgument);
     CHECK(set->SetWeightData(nullptr, 9472) == Status::InvalidArgument);
     CHECK(set->SetWeightData(blob.data(), blob.size()) == Status::CudaUnavailable);
+    // constants for decoding single texels elsewhere (src/Context.cpp:864-922): the host copy of the blob is kept
+    // without a device, so the offsets (src/WeightLayout.cpp:184-265) and per-mip constants
+    // (src/TextureSet.cpp:450-463) can be had
+    {
+        InferenceData data;
+        std::memset(&data, 0xff, sizeof(data));
+        CHECK(ctx->MakeInferenceData(set, InferenceWeightType::GenericInt8, 0, nullptr) == Status::InvalidArgument);
+        CHECK(ctx->MakeInferenceData(nullptr, InferenceWeightType::GenericInt8, 0, &data) == Status::InvalidArgument);
+        CHECK(ctx->MakeInferenceData(set, InferenceWeightType::Unknown, 0, &data) == Status::Unsupported);
+        CHECK(ctx->MakeInferenceData(set, InferenceWeightType::CoopVecFP8, 0, &data) == Status::Unsupported);
+        CHECK(std::strstr(GetLastErrorMessage(), "does not provide CoopVecFP8 weights") != nullptr);
+        CHECK(ctx->MakeInferenceData(set, InferenceWeightType::GenericInt8, 0, &data) == Status::Ok);
+        NtcTextureSetConstants const& c = data.constants;
+        static int const neural[13] = { 0, 0, 0, 2, 2, 4, 4, 6, 6, 6, 6, 6, 6 };
+        static float const scale[13] = { .25f, .5f, 1.f, .5f, 1.f, .5f, 1.f, .5f, 1.f, 2.f, 4.f, 8.f, 16.f };
+        static float const lod[13] = { -.5f, -.25f, 0.f, -.25f, 0.f, -.25f, 0.f, -.25f, 0.f, .25f, .5f, .75f, 1.f };
+        for (int mip = 0; mip < 16; ++mip) {
+            NtcColorMipConstants const& m = c.colorMips[mip];
+            if (mip < 13) CHECK(m.neuralMip == neural[mip] && m.positionScale == scale[mip] && m.positionLod == lod[mip] && m.pad == 0);
+            else CHECK(m.neuralMip == 0 && m.positionScale == 0.f && m.positionLod == 0.f && m.pad == 0);
+        }
+        static int const weights[4] = { 0, 3072, 6144, 7680 }, scales[4] = { 8192, 8448, 8640, 8768 }, biases[4] = { 8832, 9088, 9280, 9408 };
+        for (int layer = 0; layer < 4; ++layer)
+            CHECK(c.networkWeightOffsets[layer] == weights[layer] && c.networkScaleOffsets[layer] == scales[layer] && c.networkBiasOffsets[layer] == biases[layer]);
+        CHECK(c.imageWidth == 4096 && c.imageHeight == 4096 && c.imageMips == 13 && c.pad0 == 0 && c.pad1 == 0 && c.pad2 == 0);
+        CHECK(c.validChannelMask == 0 && c.channelColorSpaces == 0);        // no textures described yet
+        CHECK(ctx->MakeInferenceData(set, InferenceWeightType::GenericInt8, 2, &data) == Status::Ok);
+        CHECK(c.colorMips[0].neuralMip == -2 && c.colorMips[3].neuralMip == 0 && c.colorMips[12].neuralMip == 4);
+    }
     CHECK(set->SetDecoderPreset(DecoderPreset::Concat2x2_64) == Status::Ok);
     CHECK(set->GetWeightDataSize() == 10496 && set->GetLatentDataSize() == 22369636ull);
     CHECK(set->GetNumLatentImages() == 0 && set->GetFusedMipLevels(0, nullptr, nullptr) == Status::Unsupported);   // per-mip grids
