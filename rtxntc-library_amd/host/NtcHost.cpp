@@ -13,10 +13,12 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <limits>
 #include <new>
 #include <string>
+#include <utility>
 #include <vector>
 
 namespace ntc
@@ -167,6 +169,28 @@ void SetQuantizeError(char const* fmt, ...)
 }
 
 class Context;
+
+// Public objects are constructed in memory from the context's allocator and destroyed through it
+// (src/Context.cpp:201-233,263-293, src/PublicFunctions.cpp:46-60,164-172).
+class DefaultAllocator final : public IAllocator
+{
+public:
+    void* Allocate(size_t size) override { return std::malloc(size); }
+    void Deallocate(void* ptr, size_t) override { std::free(ptr); }
+};
+DefaultAllocator g_defaultAllocator;
+
+template <class T, class... Args> T* MakeObject(IAllocator* allocator, Args&&... args)
+{
+    void* const memory = allocator->Allocate(sizeof(T));
+    return memory ? new (memory) T(std::forward<Args>(args)...) : nullptr;
+}
+template <class T> void DestroyObject(IAllocator* allocator, T* object)      // T: the object's own (final) class
+{
+    if (!object) return;
+    object->~T();
+    allocator->Deallocate(object, sizeof(T));
+}
 
 // src/TextureMetadata.cpp:30-75 (name and channel range only)
 class TextureMetadata final : public ITextureMetadata
@@ -391,7 +415,7 @@ public:
     LatentShape const& GetLatentShape() const override { return m_latentShape; }
     ITextureMetadata* AddTexture() override
     {
-        TextureMetadata* t = new (std::nothrow) TextureMetadata(m_desc);
+        TextureMetadata* t = MakeObject<TextureMetadata>(Allocator(), m_desc);
         if (t) m_textures.push_back(t);
         return t;
     }
@@ -399,11 +423,11 @@ public:
     {
         auto it = std::find(m_textures.begin(), m_textures.end(), texture);
         if (it == m_textures.end()) { SetErrorMessage("The texture does not belong to this texture set."); return Status::OutOfRange; }
-        delete *it;
+        DestroyObject(Allocator(), *it);
         m_textures.erase(it);
         return Status::Ok;
     }
-    void ClearTextureMetadata() override { for (TextureMetadata* t : m_textures) delete t; m_textures.clear(); }
+    void ClearTextureMetadata() override { for (TextureMetadata* t : m_textures) DestroyObject(Allocator(), t); m_textures.clear(); }
     int GetTextureCount() const override { return int(m_textures.size()); }
     ITextureMetadata* GetTexture(int index) override { return (index >= 0 && index < int(m_textures.size())) ? m_textures[size_t(index)] : nullptr; }
 
@@ -1288,6 +1312,8 @@ private:
         return Status::Ok;
     }
 
+    IAllocator* Allocator() const;      // the context's
+
     Context const* m_context;
     TextureSetDesc m_desc;
     TextureSetFeatures m_features;
@@ -1320,7 +1346,8 @@ private:
 class Context final : public IContext
 {
 public:
-    explicit Context(bool deviceAvailable) : m_deviceAvailable(deviceAvailable) {}
+    Context(IAllocator* allocator, bool deviceAvailable) : m_allocator(allocator), m_deviceAvailable(deviceAvailable) {}
+    IAllocator* GetAllocator() const { return m_allocator; }
 
     // src/Context.cpp:235-261 with the descriptor rules of src/TextureSetMetadata.cpp:1161-1178
     Status CreateTextureSet(TextureSetDesc const& desc, TextureSetFeatures const& features, ITextureSet** pOutTextureSet) const override
@@ -1328,16 +1355,16 @@ public:
         if (!pOutTextureSet) { SetErrorMessage("pOutTextureSet is NULL."); return Status::InvalidArgument; }
         *pOutTextureSet = nullptr;
         if (Status st = ValidateTextureSetDesc(desc); st != Status::Ok) return st;
-        TextureSet* set = new (std::nothrow) TextureSet(this, desc, features);
+        TextureSet* set = MakeObject<TextureSet>(m_allocator, this, desc, features);
         if (!set) { SetErrorMessage("Failed to allocate the texture set object."); return Status::OutOfMemory; }
         Status const status = set->Initialize(m_deviceAvailable);
-        if (status != Status::Ok) { delete set; return status; }
+        if (status != Status::Ok) { DestroyObject(m_allocator, set); return status; }
         *pOutTextureSet = set;
         ClearErrorMessage();
         return Status::Ok;
     }
 
-    void DestroyTextureSet(ITextureSet* textureSet) const override { delete textureSet; }
+    void DestroyTextureSet(ITextureSet* textureSet) const override { DestroyObject(m_allocator, static_cast<TextureSet*>(textureSet)); }
     bool IsCudaAvailable() const override { return m_deviceAvailable; }
 
     Status CompressBlocks(BlockCompressionParameters const& params) const override
@@ -1425,17 +1452,17 @@ public:
         if (!pOutStream) { SetErrorMessage("pOutStream is NULL."); return Status::InvalidArgument; }
         FILE* file = std::fopen(fileName, write ? "wb" : "rb");
         if (!file) { SetErrorMessage("Cannot open file '%s': %s.", fileName, std::strerror(errno)); return Status::FileUnavailable; }
-        *pOutStream = new (std::nothrow) FileStream(file);
+        *pOutStream = MakeObject<FileStream>(m_allocator, file);
         if (!*pOutStream) { std::fclose(file); SetErrorMessage("Failed to allocate the stream object."); return Status::OutOfMemory; }
         return Status::Ok;
     }
-    void CloseFile(IStream* stream) const override { delete stream; }
+    void CloseFile(IStream* stream) const override { DestroyObject(m_allocator, static_cast<FileStream*>(stream)); }
     Status OpenMemory(void* pData, size_t size, IStream** pOutStream) const override { return OpenMemoryStream(pData, size, false, pOutStream); }
     Status OpenReadOnlyMemory(void const* pData, size_t size, IStream** pOutStream) const override
     {
         return OpenMemoryStream(const_cast<void*>(pData), size, true, pOutStream);
     }
-    void CloseMemory(IStream* stream) const override { delete stream; }
+    void CloseMemory(IStream* stream) const override { DestroyObject(m_allocator, static_cast<MemoryStream*>(stream)); }
 
     // src/Context.cpp:296-352
     // src/Context.cpp:864-922
@@ -1507,13 +1534,16 @@ private:
         if (!pData) { SetErrorMessage("pData is NULL."); return Status::InvalidArgument; }
         if (size == 0) { SetErrorMessage("size is 0."); return Status::InvalidArgument; }
         if (!pOutStream) { SetErrorMessage("pOutStream is NULL."); return Status::InvalidArgument; }
-        *pOutStream = new (std::nothrow) MemoryStream(static_cast<uint8_t*>(pData), size, readonly);
+        *pOutStream = MakeObject<MemoryStream>(m_allocator, static_cast<uint8_t*>(pData), size, readonly);
         if (!*pOutStream) { SetErrorMessage("Failed to allocate the stream object."); return Status::OutOfMemory; }
         return Status::Ok;
     }
 
+    IAllocator* m_allocator;
     bool m_deviceAvailable;
 };
+
+IAllocator* TextureSet::Allocator() const { return m_context->GetAllocator(); }
 
 extern "C" {
 
@@ -1533,13 +1563,19 @@ Status CreateContext(IContext** pOutContext, ContextParameters const& params)
         if (ntc_hip_init(params.cudaDevice) == 0) deviceAvailable = true;
         else SetErrorMessage("%s", ntc_hip_last_error());
     }
-    Context* context = new (std::nothrow) Context(deviceAvailable);
+    IAllocator* const allocator = params.pAllocator ? params.pAllocator : &g_defaultAllocator;
+    Context* context = MakeObject<Context>(allocator, allocator, deviceAvailable);
     if (!context) { SetErrorMessage("Failed to allocate the context object."); return Status::OutOfMemory; }
     *pOutContext = context;
     return deviceAvailable ? Status::Ok : Status::CudaUnavailable;
 }
 
-void DestroyContext(IContext* context) { delete context; }
+void DestroyContext(IContext* context)
+{
+    if (!context) return;
+    Context* const object = static_cast<Context*>(context);
+    DestroyObject(object->GetAllocator(), object);
+}
 
 char const* GetLastErrorMessage() { return t_message; }
 

@@ -206,9 +206,22 @@ struct DecompressionStats
 };
 
 // include/libntc/ntc.h:1278-1305 (graphics-API fields left out)
+// A custom CPU memory allocator (include/libntc/ntc.h:76-87).
+class IAllocator
+{
+public:
+    virtual void* Allocate(size_t size) = 0;
+    virtual void Deallocate(void* ptr, size_t size) = 0;    // size: what Allocate was asked for
+    virtual ~IAllocator() = default;
+};
+
 struct ContextParameters
 {
     uint32_t interfaceVersion = InterfaceVersion;
+    // Optional (include/libntc/ntc.h:1284-1287): where the context, its texture sets, texture metadata and
+    // stream objects live; null = the C runtime's heap.  Must outlive the context.  Buffers inside those
+    // objects (names, host copies of weights and mode maps) come from the C++ runtime either way.
+    IAllocator* pAllocator = nullptr;
     int cudaDevice = 0;             // index of the HIP device; the name is kept for source compatibility
 };
 

@@ -29,6 +29,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <string>
+#include <utility>
 #include <vector>
 
 using namespace ntc;
@@ -55,8 +56,68 @@ static bool writeFile(std::string const& path, void const* p, size_t n)
     return ok;
 }
 
+// Counts what the library takes from and returns to a caller's allocator.
+struct CountingAllocator final : IAllocator
+{
+    size_t allocations = 0, releases = 0, liveBytes = 0;
+    bool sizesMatch = true;
+    std::vector<std::pair<void*, size_t>> live;
+    void* Allocate(size_t size) override
+    {
+        void* const p = std::malloc(size);
+        if (p) { ++allocations; liveBytes += size; live.emplace_back(p, size); }
+        return p;
+    }
+    void Deallocate(void* ptr, size_t size) override
+    {
+        for (size_t i = 0; i < live.size(); ++i)
+            if (live[i].first == ptr) {
+                if (live[i].second != size) sizesMatch = false;
+                liveBytes -= live[i].second;
+                live.erase(live.begin() + long(i));
+                ++releases;
+                std::free(ptr);
+                return;
+            }
+        sizesMatch = false;     // not ours
+    }
+};
+
+// Public objects come from the allocator given in ContextParameters and go back to it with the size they
+// were allocated with (include/libntc/ntc.h:76-87,1284-1287, src/Context.cpp:201-233,263-293).
+static int allocatorChecks()
+{
+    CountingAllocator allocator;
+    IContext* ctx = nullptr;
+    ContextParameters params; params.cudaDevice = DisableCudaDevice; params.pAllocator = &allocator;
+    CHECK(CreateContext(&ctx, params) == Status::CudaUnavailable && ctx != nullptr);
+    CHECK(allocator.allocations == 1);
+    TextureSetDesc desc; desc.width = 64; desc.height = 64; desc.channels = 4; desc.mips = 1;
+    ITextureSet* set = nullptr;
+    CHECK(ctx->CreateTextureSet(desc, TextureSetFeatures(), &set) == Status::Ok && allocator.allocations == 2);
+    ITextureMetadata* a = set->AddTexture();
+    ITextureMetadata* b = set->AddTexture();
+    CHECK(a && b && allocator.allocations == 4 && allocator.releases == 0);
+    CHECK(set->RemoveTexture(a) == Status::Ok && allocator.releases == 1);
+    unsigned char bytes[16] = {};
+    IStream* stream = nullptr;
+    CHECK(ctx->OpenReadOnlyMemory(bytes, sizeof bytes, &stream) == Status::Ok && allocator.allocations == 5);
+    ctx->CloseMemory(stream);
+    CHECK(allocator.releases == 2);
+    desc.width = 0;                                           // a set that fails validation leaves nothing behind
+    ITextureSet* bad = nullptr;
+    CHECK(ctx->CreateTextureSet(desc, TextureSetFeatures(), &bad) != Status::Ok && bad == nullptr);
+    ctx->DestroyTextureSet(set);                              // takes texture b with it
+    CHECK(allocator.releases == 4 && allocator.live.size() == 1);
+    DestroyContext(ctx);
+    CHECK(allocator.allocations == allocator.releases && allocator.liveBytes == 0 && allocator.live.empty() && allocator.sizesMatch);
+    DestroyContext(nullptr);                                  // allowed (src/PublicFunctions.cpp:164-167)
+    return 0;
+}
+
 static int cpuChecks()
 {
+    CHECK(allocatorChecks() == 0);
     {   // BC7 mode maps kept with a texture (include/libntc/ntc.h:437-453)
         IContext* c = nullptr; ContextParameters cp; cp.cudaDevice = DisableCudaDevice;
         (void)CreateContext(&c, cp);
