@@ -673,8 +673,10 @@ public:
     // LoadMetadataFromStream + LoadFromStreamPostHeader + LoadWeightsFromStream
     // (src/TextureSetMetadata.cpp:434-581,676-784, src/TextureSet.cpp:154-294).  Everything is
     // validated and assembled in host memory first; the device is touched last.
+    // With metadataOnly the latent layers are described (footprints) but neither read nor uploaded, so GDeflate
+    // views are acceptable there, and the weights stay in host memory.
     Status LoadFromStreamPostHeader(file::Document const& document, uint64_t binaryChunkOffset, uint64_t binaryChunkSize,
-        IStream* stream, LatentShape const& shape)
+        IStream* stream, LatentShape const& shape, bool metadataOnly = false)
     {
         ClearTextureMetadata();
         if (shape.IsEmpty()) { SetErrorMessage("The file does not describe a latent shape."); return Status::FileUnrecognized; }
@@ -814,15 +816,17 @@ public:
             for (uint32_t viewIndex : image.layerViews) {
                 file::BufferView const& view = document.views[viewIndex];
                 file::Compression const compression = view.compression.value_or(file::Compression::None);
+                BufferFootprint footprint;
+                footprint.rangeInStream = StreamRange{ view.offset + binaryChunkOffset, view.storedSize };
+                footprint.compressionType = CompressionType(int(compression));
+                footprint.uncompressedSize = view.uncompressedSize.value_or(view.storedSize);
+                footprint.uncompressedCrc32 = view.crc32.value_or(0);
+                footprints.push_back(footprint);
+                if (metadataOnly) continue;
                 if (compression != file::Compression::None) {
                     SetErrorMessage("Latent image view %d is stored with GDeflate compression, which this library does not decode.", int(viewIndex));
                     return Status::Unsupported;
                 }
-                BufferFootprint footprint;
-                footprint.rangeInStream = StreamRange{ view.offset + binaryChunkOffset, view.storedSize };
-                footprint.uncompressedSize = view.storedSize;
-                footprint.uncompressedCrc32 = view.crc32.value_or(0);
-                footprints.push_back(footprint);
                 size_t const at = latents.size();
                 latents.resize(at + layerSize);
                 if (!(stream->Seek(binaryChunkOffset + view.offset) && stream->Read(latents.data() + at, layerSize))) {
@@ -836,7 +840,13 @@ public:
         m_latentShape = LatentShape::Empty();
         if (Status st = SetLatentShape(shape); st != Status::Ok) return st;
         m_latentFootprints = std::move(footprints);     // file metadata: valid whether or not the uploads below succeed
-        if (latents.size() != m_latentBytes || blob.size() != m_weightLayout.bufferSize) { SetErrorMessage("Inconsistent sizes for MLP or latent data"); return Status::InternalError; }
+        if ((!metadataOnly && latents.size() != m_latentBytes) || blob.size() != m_weightLayout.bufferSize) { SetErrorMessage("Inconsistent sizes for MLP or latent data"); return Status::InternalError; }
+        if (metadataOnly) {
+            Status const st = SetWeightData(blob.data(), blob.size());      // no device behind a metadata object: the host copy is what counts
+            if (st != Status::Ok && st != Status::CudaUnavailable) return st;
+            ClearErrorMessage();
+            return Status::Ok;
+        }
         if (Status st = SetWeightData(blob.data(), blob.size()); st != Status::Ok) return st;
         if (Status st = SetLatentData(latents.data(), latents.size()); st != Status::Ok) return st;
         ClearErrorMessage();
@@ -1491,6 +1501,29 @@ public:
         ClearErrorMessage();
         return Status::Ok;
     }
+
+    // src/Context.cpp:263-293: everything a file says about a set, without its latents and without a device.
+    Status CreateTextureSetMetadataFromStream(IStream* inputStream, ITextureSet** pOutMetadata) const override
+    {
+        if (!pOutMetadata) { SetErrorMessage("pOutMetadata is NULL."); return Status::InvalidArgument; }
+        *pOutMetadata = nullptr;
+        if (!inputStream) { SetErrorMessage("inputStream is NULL."); return Status::InvalidArgument; }
+        file::Document document;
+        uint64_t binaryChunkOffset = 0, binaryChunkSize = 0;
+        if (Status st = LoadFileHeadersFromStream(inputStream, document, binaryChunkOffset, binaryChunkSize); st != Status::Ok) return st;
+        TextureSetDesc desc;
+        LatentShape shape;
+        if (Status st = DeserializeTextureSetDesc(document, desc, shape); st != Status::Ok) return st;
+        TextureSet* set = MakeObject<TextureSet>(m_allocator, this, desc, TextureSetFeatures());
+        if (!set) { SetErrorMessage("Failed to allocate the texture set object."); return Status::OutOfMemory; }
+        Status status = set->Initialize(false);
+        if (status == Status::Ok) status = set->LoadFromStreamPostHeader(document, binaryChunkOffset, binaryChunkSize, inputStream, shape, true);
+        if (status != Status::Ok) { DestroyObject(m_allocator, set); return status; }
+        *pOutMetadata = set;
+        ClearErrorMessage();
+        return Status::Ok;
+    }
+    void DestroyTextureSetMetadata(ITextureSet* textureSetMetadata) const override { DestroyTextureSet(textureSetMetadata); }
 
     Status CreateCompressedTextureSetFromStream(IStream* inputStream, TextureSetFeatures const& features, ITextureSet** pOutTextureSet) const override
     {

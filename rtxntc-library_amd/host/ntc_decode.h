@@ -444,6 +444,13 @@ public:
     virtual Status OpenMemory(void* pData, size_t size, IStream** pOutStream) const = 0;
     virtual Status OpenReadOnlyMemory(void const* pData, size_t size, IStream** pOutStream) const = 0;
     virtual void CloseMemory(IStream* stream) const = 0;
+    // Reads what an NTC file says about a set - descriptor, latent shape, textures, colour spaces, the Int8 weights
+    // (GetInferenceWeights, MakeInferenceData), BC7 mode maps and where every latent layer lies in the file
+    // (GetLatentTextureFootprint) - without reading the latents and without a device
+    // (include/libntc/ntc.h:1158-1163, src/Context.cpp:263-293).  Latent layers stored with GDeflate are fine here:
+    // their footprints say so.  Device work on the returned object fails with CudaUnavailable / InvalidState.
+    virtual Status CreateTextureSetMetadataFromStream(IStream* inputStream, ITextureSet** pOutMetadata) const = 0;
+    virtual void DestroyTextureSetMetadata(ITextureSet* textureSetMetadata) const = 0;
     // Creates a texture set with the dimensions found in an NTC file and loads it
     // (include/libntc/ntc.h:1166-1177, src/Context.cpp:296-376).
     virtual Status CreateCompressedTextureSetFromStream(IStream* inputStream, TextureSetFeatures const& features,

@@ -847,6 +847,42 @@ static int load(int argc, char** argv)
     return 0;
 }
 
+// What a file says about its set, read without a device and without the latents.
+static int metadata(int argc, char** argv)
+{
+    if (argc < 3) { std::fprintf(stderr, "usage: metadata <file>\n"); return 2; }
+    IContext* ctx = nullptr;
+    ContextParameters params; params.cudaDevice = DisableCudaDevice;
+    CHECK(CreateContext(&ctx, params) == Status::CudaUnavailable && ctx != nullptr);
+    IStream* stream = nullptr;
+    CHECK(ctx->OpenFile(argv[2], false, &stream) == Status::Ok);
+    ITextureSet* set = nullptr;
+    CHECK(ctx->CreateTextureSetMetadataFromStream(stream, nullptr) == Status::InvalidArgument);
+    CHECK(ctx->CreateTextureSetMetadataFromStream(nullptr, &set) == Status::InvalidArgument);
+    Status const status = ctx->CreateTextureSetMetadataFromStream(stream, &set);
+    ctx->CloseFile(stream);
+    CHECK((status == Status::Ok) == (set != nullptr));
+    std::printf("status %d %s\nmessage %s\n", int(status), StatusToString(status), GetLastErrorMessage());
+    if (set) {
+        CHECK(describe(set) == 0);
+        CHECK(set->Decompress(nullptr) != Status::Ok);                       // nothing to decode with
+        void const* weights = nullptr; size_t weightSize = 0;
+        CHECK(set->GetInferenceWeights(InferenceWeightType::GenericInt8, &weights, &weightSize, nullptr) == Status::Ok);
+        unsigned long long sum = 0;
+        for (size_t b = 0; b < weightSize; ++b) sum = sum * 131 + static_cast<unsigned char const*>(weights)[b];
+        InferenceData data;
+        CHECK(ctx->MakeInferenceData(set, InferenceWeightType::GenericInt8, 0, &data) == Status::Ok);
+        std::printf("weights %zu %llu\ninference 0x%x 0x%x %d", weightSize, sum, data.constants.validChannelMask, data.constants.channelColorSpaces,
+            data.constants.imageMips);
+        for (int mip = 0; mip < data.constants.imageMips; ++mip)
+            std::printf(" %d:%g:%g", data.constants.colorMips[mip].neuralMip, data.constants.colorMips[mip].positionScale, data.constants.colorMips[mip].positionLod);
+        std::printf("\n");
+        ctx->DestroyTextureSetMetadata(set);
+    }
+    DestroyContext(ctx);
+    return 0;
+}
+
 static int decodeFile(int argc, char** argv)
 {
     if (argc < 4) { std::fprintf(stderr, "usage: decodefile <file> <outPrefix>\n"); return 2; }
@@ -888,6 +924,7 @@ static int decodeFile(int argc, char** argv)
 int main(int argc, char** argv)
 {
     if (argc >= 2 && std::strcmp(argv[1], "load") == 0) return load(argc, argv);
+    if (argc >= 2 && std::strcmp(argv[1], "metadata") == 0) return metadata(argc, argv);
     if (argc >= 2 && std::strcmp(argv[1], "decodefile") == 0) return decodeFile(argc, argv);
     if (argc >= 2 && std::strcmp(argv[1], "loss") == 0) return loss(argc, argv);
     if (argc >= 2 && std::strcmp(argv[1], "shuffle") == 0) return shuffle(argc, argv);

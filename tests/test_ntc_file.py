@@ -347,3 +347,54 @@ def test_gpu_narrow_hidden_layers_are_expanded(ntc, oracle, tmp_path):
         planar = np.ascontiguousarray(host.output[mip.outOffset: mip.outOffset + mip.width * mip.height * channels * 2].view(np.uint16))
         got = np.fromfile(f"{prefix}_mip{m}.bin", dtype=np.uint16)
         assert np.array_equal(got, pixels_from_planar(planar, mip.width, mip.height, channels)), f"mip {m}"
+
+
+def test_metadata_only_loading(ntc, tmp_path):
+    """CreateTextureSetMetadataFromStream (include/libntc/ntc.h:1158-1163, src/Context.cpp:263-293): the file's
+    description of the set without its latents and without a device - also for files whose latent layers are
+    stored with GDeflate, which a full load refuses; the footprints then carry the compression type."""
+    width, height, grid_scale, features = 64, 32, 2, 8
+    case = make_case(ntc, width, height, None, grid_scale, features)
+    data = file_of(case, width, height, grid_scale, features, 8, textures=TEXTURES, channel_color_spaces=["sRGB"] * 3 + [None] * 4 + ["HLG"])
+    path = tmp_path / "plain.ntc"
+    path.write_bytes(data)
+
+    def parse(out):
+        lines = out.splitlines()
+        return int(lines[0].split()[1]), lines[1], lines[2:]
+
+    status, message, lines = parse(run_exe("metadata", path))
+    assert status == STATUS["Ok"], message
+    # the same description a full load gives (which fails at the upload here, after everything was parsed)
+    loaded = run_exe("load", path, 0, width, height, 8, len(case.mips)).splitlines()[2:]
+    assert [ln for ln in lines if not ln.startswith(("weights", "inference"))] == loaded
+    weights = np.frombuffer(case.weights, np.uint8)
+    digest = 0
+    for b in weights.tolist():
+        digest = (digest * 131 + b) % (1 << 64)
+    assert f"weights {weights.size} {digest}" in lines
+    inference = [ln for ln in lines if ln.startswith("inference ")][0].split()
+    # TEXTURES claims channels 0-4 and 7; the storage colour spaces of the channels, two bits each
+    spaces = [int(v) for v in [ln for ln in lines if ln.startswith("colorspaces")][0].split()[1:]]
+    assert inference[1] == "0x9f" and int(inference[3]) == len(case.mips)
+    assert int(inference[2], 16) == sum(v << (2 * c) for c, v in enumerate(spaces)) == 0b10_00_00_00_00_01_01_01
+    text, binary = nw.split_container(data)
+    doc = json.loads(text)
+    for token, mip in zip(inference[4:], doc["colorMips"]):
+        neural, scale, lod = token.split(":")
+        assert int(neural) == mip["latentMip"] and float(scale) == mip["positionScale"] and float(lod) == mip["positionLod"]
+
+    # latent layers marked as GDeflate streams: described, not read
+    for view_index in doc["latents"][0]["layerViews"]:
+        view = doc["views"][view_index]
+        view.update(compression="GDeflate", uncompressedSize=view["storedSize"], crc32=12345)
+    packed = tmp_path / "packed.ntc"
+    packed.write_bytes(nw.pack_container(json.dumps(doc), binary))
+    status, message, _ = host_load(tmp_path, packed.read_bytes(), name="packed_full.ntc")
+    assert status == STATUS["Unsupported"], message
+    status, message, lines = parse(run_exe("metadata", packed))
+    assert status == STATUS["Ok"], message
+    rows = [ln.split()[1:] for ln in lines if ln.startswith("latent ")]
+    layers = (features + 3) // 4
+    assert [r[4] for r in rows] == ["1"] * layers + ["0"] * (len(rows) - layers)      # compression type per layer
+    assert [r[6] for r in rows[:layers]] == ["12345"] * layers
