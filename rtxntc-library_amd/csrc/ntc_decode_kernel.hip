@@ -110,8 +110,8 @@ __device__ __forceinline__ uint32_t bilinear4(Taps const& tp, uint32_t s00, uint
         t = __builtin_fmaf(tp.w10, q10, t);
         t = __builtin_fmaf(tp.w01, q01, t);
         t = __builtin_fmaf(tp.w11, q11, t);
-        int const c = int(floorf(t * codeScale));          // 0..255
-        packed |= (uint32_t(c) & 0xffu) << (8 * i);
+        // 0..255, integer-valued after the floor: the conversion is exact and drops the byte into its slot
+        packed = __builtin_amdgcn_cvt_pk_u8_f32(floorf(t * codeScale), uint32_t(i), packed);
     }
     return packed ^ 0x80808080u;                            // -128 on every byte
 }
