@@ -271,10 +271,13 @@ template <int HR_MODE_, int HR_F_, int HR_BITS_, int HR_SLOTS_, int LR_F_, int L
           int IN_, int H0_, int H1_, int H2_, bool FP8_WEIGHTS_ = false>
 struct Variant {
     // e4m3 weights in the three hidden layers: each weight w is the integer 512*w (at most 18 bits
-    // plus sign) split into three 6-bit planes, 512*w = 4096*c2 + 64*c1 + c0, and the layer runs
-    // as three int8 MFMA passes whose int32 results are recombined exactly.
+    // plus sign).  On the int8 matrix instruction it is split into three 6-bit planes,
+    // 512*w = 4096*c2 + 64*c1 + c0, and a layer runs as three passes whose int32 results are recombined
+    // exactly; on the fp16 matrix instruction (layers 1 and 2) into two planes, 512*w = 1024*hi + lo with
+    // 0 <= lo < 1024, whose fp32 sums are exact integers and recombine with one fused multiply-add.
     static constexpr bool FP8_WEIGHTS = FP8_WEIGHTS_;
     static constexpr int PLANES = FP8_WEIGHTS_ ? 3 : 1;
+    static constexpr int F16_PLANES = FP8_WEIGHTS_ ? 2 : 1;
     static constexpr int HR_MODE = HR_MODE_, HR_F = HR_F_, HR_BITS = HR_BITS_, HR_SLOTS = HR_SLOTS_;
     static constexpr int LR_F = LR_F_, LR_SLOTS = LR_SLOTS_, LOD = LOD_;
     static constexpr int IN = IN_, H0 = H0_, H1 = H1_, H2 = H2_, OUT = 16;
@@ -290,27 +293,34 @@ struct Variant {
     // Layers 1..3 can also run on the fp16 matrix instruction (see mlp_forward_f16).  Their A operands
     // then take, per output tile, one 1024-byte block for every pair of input tiles (K = 32) and one
     // 512-byte block for an odd last input tile (K = 16); sizes below are in 16-byte units.
-    static constexpr bool F16_LAYERS = !FP8_WEIGHTS_;
+    // (Layers 1 and 2 of an e4m3 variant hold F16_PLANES such sets of blocks, plane after plane.)
+    static constexpr bool F16_LAYERS = true;
     static constexpr int f16_units(int inTiles) { return (inTiles / 2) * 64 + (inTiles % 2) * 32; }
     static constexpr int F16_L1 = 0;
-    static constexpr int F16_L2 = F16_L1 + T1 * f16_units(T0);
-    static constexpr int F16_L3 = F16_L2 + T2 * f16_units(T1);
+    static constexpr int F16_L2 = F16_L1 + F16_PLANES * T1 * f16_units(T0);
+    static constexpr int F16_L3 = F16_L2 + F16_PLANES * T2 * f16_units(T1);
     static constexpr int F16_END = F16_L3 + T3 * f16_units(T2);
-    static constexpr int LATE_INT8_UNITS = (T1 + T2 + T3) * 64;
-    static constexpr int LATE_UNITS = F16_LAYERS ? (F16_END > LATE_INT8_UNITS ? F16_END : LATE_INT8_UNITS) : 1;
-    // A operands kept in `w`: every layer for the e4m3 variants, layer 0 only otherwise (the later
-    // layers then live in `late`, as int8 or as fp16).
-    static constexpr int W_TILES = F16_LAYERS ? T0 : NTILES;
+    // The same layers as int8 tiles: [plane][tile of layers 1..3][lane], one 16-byte unit each.
+    static constexpr int LATE_TILES = T1 + T2 + T3;
+    static constexpr int LATE_INT8_UNITS = PLANES * LATE_TILES * 64;
+    static constexpr int LATE_UNITS = F16_END > LATE_INT8_UNITS ? F16_END : LATE_INT8_UNITS;
+    // A operands kept in `w`: layer 0 (the later layers live in `late`, as int8 or as fp16).
+    static constexpr int W_TILES = T0;
     static constexpr int LATE_CHANNELS = H1 + H2 + OUT;
     static_assert(POS_BASE + 12 + LOD <= IN, "input vector does not fit");
     static_assert(IN % 16 == 0 && IN <= 64 && H0 <= 64 && H1 <= 64 && H2 <= 64, "layer widths");
     static_assert(HR_INPUTS % 4 == 0 && LR_INPUTS % 4 == 0, "grid blocks are dword aligned");
 };
 
+// Low part of the start value of two-plane fp16 layers ([M-tile][g][r] like `bias`): e4m3 variants only, so
+// that the others keep their LDS footprint (the query kernel's is exactly a quarter of a CU's LDS).
+template <bool ENABLED, int TILES> struct BiasLoT { float biasLo[TILES][4][4]; };
+template <int TILES> struct BiasLoT<false, TILES> {};
+
 template <class V>
-struct alignas(16) LdsT {
+struct alignas(16) LdsT : BiasLoT<V::FP8_WEIGHTS, V::NTILES> {
     uint32_t w[V::PLANES][V::W_TILES][64][4];  // int8 A operands: [plane][M-tile][lane][4 dwords]
-    uint4    late[V::LATE_UNITS];              // A operands of layers 1..3 when V::F16_LAYERS: int8 tiles or fp16 blocks
+    uint4    late[V::LATE_UNITS];              // A operands of layers 1..3: int8 tiles or fp16 blocks
     float    scale[V::NTILES][4][4];           // [M-tile][k-group g][r]  -> channel 16t+4g+r
     int32_t  bias[V::NTILES][4][4];
     uint32_t in[kWaves][kWaveTexels][kInStride];
@@ -337,6 +347,25 @@ __device__ __forceinline__ uint32_t weight_dword(uint32_t const* blob32, int wof
     return (k < in) ? blob32[(woff + row * in + k) >> 2] : 0u;
 }
 
+__device__ __forceinline__ uint32_t halves_of_ints(int a, int b)                   // two integers of at most 11 bits -> two fp16 (exact)
+{
+    v2h const h = { _Float16(a), _Float16(b) };
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+// Four e4m3 bytes -> the three int8 planes of their 512-fold values: 6 bits, 6 bits, signed rest.
+__device__ __forceinline__ void int8_planes(uint32_t v, uint32_t (&planes)[3])
+{
+    planes[0] = planes[1] = planes[2] = 0;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        int32_t const W = e4m3_times_512((v >> (8 * r)) & 0xffu);
+        planes[0] |= uint32_t(W & 63) << (8 * r);
+        planes[1] |= uint32_t((W >> 6) & 63) << (8 * r);
+        planes[2] |= (uint32_t(W >> 12) & 0xffu) << (8 * r);
+    }
+}
+
 __device__ __forceinline__ uint32_t halves_of_bytes(uint32_t v, int firstByte)     // two int8 -> two fp16 (exact)
 {
     v2h const h = { _Float16(int(int8_t(v >> (8 * firstByte)))), _Float16(int(int8_t(v >> (8 * firstByte + 8)))) };
@@ -346,7 +375,8 @@ __device__ __forceinline__ uint32_t halves_of_bytes(uint32_t v, int firstByte)  
 // Copies the int8 blob (src/WeightLayout.cpp:42-49: matrices, then fp32 scales, then int32
 // biases; W[c*IN + k]) into LDS in MFMA operand order.  Returns kStagedF16 when layers 1..3 were
 // staged for the fp16 matrix instruction (see mlp_forward_f16): that needs, for every channel of
-// those layers, |bias - 113*sum(W)| + 240*sum|W| < 2^24; otherwise they are staged as int8 tiles.
+// those layers, |bias - 113*sum(W)| + 240*sum|W| < 2^24 (for e4m3 rows: the same for either plane, and
+// |bias| + 128*sum|512 w| < 2^31); otherwise they are staged as int8 tiles.
 // With kStagedF16, kOutputsBounded says that no output can come near the fp16 overflow threshold
 // (the same bound times the channel's scale stays below 60000), so stores may skip that check.
 constexpr int kStagedF16 = 1, kOutputsBounded = 2;
@@ -374,116 +404,137 @@ __device__ int stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
         }
     }
 
-    // int8 tiles: all layers for the e4m3 variants, layer 0 otherwise
-    {
+    // int8 tiles of layer 0 (three planes for e4m3 weights)
+    for (int e = threadIdx.x; e < V::T0 * 64 * 4; e += blockDim.x) {
+        int const d = e & 3, lane = (e >> 2) & 63, t = e >> 8;
+        int const i = lane & 15, g = lane >> 4;
+        // k-slot (g, 4d+r) = input 16g+4d+r
+        uint32_t const v = weight_dword(blob32, 0, 16 * t + i, V::IN, 16 * g + 4 * d);
+        if constexpr (V::FP8_WEIGHTS) {
+            uint32_t planes[3];
+            int8_planes(v, planes);
+#pragma unroll
+            for (int q = 0; q < V::PLANES; ++q) lds.w[q][t][lane][d] = planes[q];
+        } else {
+            lds.w[0][t][lane][d] = v;
+        }
+    }
+
+    // One thread per channel of layers 1..3: row sums decide whether the fp16 path is exact.
+    bool fits = true, bounded = true;
+    int64_t shifted = 0;
+    bool twoPlanes = false;
+    int slotTile = 0, slotG = 0, slotR = 0;
+    if (threadIdx.x < V::LATE_CHANNELS) {
+        int const c = threadIdx.x;
+        int const l = c < V::H1 ? 1 : (c < V::H1 + V::H2 ? 2 : 3);
+        int const row = c - (l == 1 ? 0 : (l == 2 ? V::H1 : V::H1 + V::H2));
+        int const in = l == 1 ? V::H0 : (l == 2 ? V::H1 : V::H2);
+        int const off = l == 1 ? V::W1_OFF : (l == 2 ? V::W2_OFF : V::W3_OFF);
+        twoPlanes = V::FP8_WEIGHTS && l < 3;
+        int64_t sum = 0, sumAbs = 0, sumAbsHi = 0, sumLo = 0;
+        for (int k = 0; k < in; k += 4) {
+            uint32_t const v = blob32[(off + row * in + k) >> 2];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                uint32_t const byte = (v >> (8 * r)) & 0xffu;
+                int const w = twoPlanes ? e4m3_times_512(byte) : int(int8_t(byte));
+                int const hi = w >> 10;
+                sum += w;
+                sumAbs += w < 0 ? -w : w;
+                sumAbsHi += hi < 0 ? -hi : hi;
+                sumLo += w & 1023;
+            }
+        }
+        int32_t const bias = reinterpret_cast<int32_t const*>(blob + V::BIAS_OFF)[V::H0 + c];
+        shifted = int64_t(bias) - 113 * int64_t(sum);     // activations enter as q + 113 in [-15, 240]
+        int64_t const absBias = bias < 0 ? -int64_t(bias) : int64_t(bias);
+        int64_t const absShifted = shifted < 0 ? -shifted : shifted;
+        if (twoPlanes) {
+            // Exact when the int32 accumulator the result is defined by cannot wrap (inputs in [-128, 127])
+            // and both fp32 partial sums, started at floor(shifted / 1024) and shifted mod 1024, stay integers.
+            int64_t const startHi = shifted >> 10;
+            fits = absBias + 128 * sumAbs < (int64_t(1) << 31)
+                && (startHi < 0 ? -startHi : startHi) + 240 * sumAbsHi < (int64_t(1) << 24)
+                && 1023 + 240 * sumLo < (int64_t(1) << 24);
+        } else {
+            int64_t const bound = absShifted + 240 * sumAbs;
+            fits = bound < (int64_t(1) << 24);
+            if (l == 3) bounded = float(bound) * fabsf(reinterpret_cast<float const*>(blob + V::SCALE_OFF)[V::H0 + c]) < 60000.f;
+        }
+        slotTile = V::T0 + (l == 1 ? 0 : (l == 2 ? V::T1 : V::T1 + V::T2)) + row / 16;
+        slotG = (row >> 2) & 3;
+        slotR = row & 3;
+    }
+    bool const useF16 = __syncthreads_and(fits ? 1 : 0) != 0;     // also orders the bias writes above
+    bool const outputsBounded = __syncthreads_and(bounded ? 1 : 0) != 0;
+    constexpr int base[4] = { 0, V::F16_L1, V::F16_L2, V::F16_L3 };
+    uint32_t* const late32 = reinterpret_cast<uint32_t*>(lds.late);
+    if (useF16) {
+        if (threadIdx.x < V::LATE_CHANNELS) {
+            if constexpr (V::FP8_WEIGHTS) {
+                if (twoPlanes) lds.biasLo[slotTile][slotG][slotR] = float(shifted & 1023);
+            }
+            lds.bias[slotTile][slotG][slotR] = __builtin_bit_cast(int32_t, float(twoPlanes ? (shifted >> 10) : shifted));
+        }
+        // fp16 blocks.  Lane (i, kg) of the block of output tile t and input-tile pair p holds
+        // W[16t + i][16*(2p + e/4) + 4*kg + e%4], e = 0..7: the channels lane (j, kg) of the
+        // previous layer's D registers owns, in register order.
+#pragma unroll
+        for (int l = 1; l < 4; ++l) {
+            int const in = ins[l];
+            int const inTiles = tiles[l - 1], pairs = inTiles / 2, per = V::f16_units(inTiles);
+            int const planeDwords = tiles[l] * per * 4;
+            // one work item = one (output tile, input tile, lane): 4 weights -> 2 dwords (per plane)
+            for (int e = threadIdx.x; e < tiles[l] * inTiles * 64; e += blockDim.x) {
+                int const lane = e & 63, rest = e >> 6;
+                int const ti = rest % inTiles, t = rest / inTiles;
+                int const i = lane & 15, kg = lane >> 4;
+                uint32_t const v = blob32[(woff[l] + (16 * t + i) * in + 16 * ti + 4 * kg) >> 2];
+                int const p = ti >> 1;
+                // dword index inside `late`: paired blocks hold 4 dwords per lane, the tail block 2
+                int const at = (p < pairs) ? ((base[l] + t * per + p * 64 + lane) * 4 + (ti & 1) * 2)
+                                           : ((base[l] + t * per + pairs * 64) * 4 + lane * 2);
+                if (V::FP8_WEIGHTS && l < 3) {
+                    int32_t W[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) W[r] = e4m3_times_512((v >> (8 * r)) & 0xffu);
+                    late32[at]     = halves_of_ints(W[0] >> 10, W[1] >> 10);
+                    late32[at + 1] = halves_of_ints(W[2] >> 10, W[3] >> 10);
+                    late32[at + planeDwords]     = halves_of_ints(W[0] & 1023, W[1] & 1023);
+                    late32[at + planeDwords + 1] = halves_of_ints(W[2] & 1023, W[3] & 1023);
+                } else {
+                    late32[at]     = halves_of_bytes(v, 0);
+                    late32[at + 1] = halves_of_bytes(v, 2);
+                }
+            }
+        }
+    } else {
         int tileBase = 0;
 #pragma unroll
-        for (int l = 0; l < (V::F16_LAYERS ? 1 : 4); ++l) {
+        for (int l = 1; l < 4; ++l) {
             int const in = ins[l];
             for (int e = threadIdx.x; e < tiles[l] * 64 * 4; e += blockDim.x) {
                 int const d = e & 3, lane = (e >> 2) & 63, t = e >> 8;
                 int const i = lane & 15, g = lane >> 4;
-                // layer 0: k-slot (g, 4d+r) = input 16g+4d+r.  layers >= 1: = channel 16d+4g+r.
-                int const k = (l == 0) ? (16 * g + 4 * d) : (16 * d + 4 * g);
-                uint32_t const v = weight_dword(blob32, woff[l], 16 * t + i, in, k);
+                // k-slot (g, 4d+r) = channel 16d+4g+r of the previous layer
+                uint32_t const v = weight_dword(blob32, woff[l], 16 * t + i, in, 16 * d + 4 * g);
+                int const at = ((tileBase + t) * 64 + lane) * 4 + d;
                 if (V::FP8_WEIGHTS && l < 3) {
-                    uint32_t p0 = 0, p1 = 0, p2 = 0;
+                    uint32_t planes[3];
+                    int8_planes(v, planes);
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        int32_t const W = e4m3_times_512((v >> (8 * r)) & 0xffu);
-                        p0 |= uint32_t(W & 63) << (8 * r);
-                        p1 |= uint32_t((W >> 6) & 63) << (8 * r);
-                        p2 |= (uint32_t(W >> 12) & 0xffu) << (8 * r);      // signed top plane
-                    }
-                    lds.w[0][tileBase + t][lane][d] = p0;
-                    lds.w[V::PLANES > 1 ? 1 : 0][tileBase + t][lane][d] = p1;
-                    lds.w[V::PLANES > 2 ? 2 : 0][tileBase + t][lane][d] = p2;
+                    for (int q = 0; q < V::PLANES; ++q) late32[q * V::LATE_TILES * 256 + at] = planes[q];
                 } else {
-                    lds.w[0][tileBase + t][lane][d] = v;
+                    late32[at] = v;
                 }
             }
             tileBase += tiles[l];
         }
     }
-    if constexpr (!V::F16_LAYERS) {
-        return 0;
-    } else {
-        // One thread per channel of layers 1..3: row sums decide whether the fp16 path is exact.
-        bool fits = true, bounded = true;
-        int64_t shifted = 0;
-        int slotTile = 0, slotG = 0, slotR = 0;
-        if (threadIdx.x < V::LATE_CHANNELS) {
-            int const c = threadIdx.x;
-            int const l = c < V::H1 ? 1 : (c < V::H1 + V::H2 ? 2 : 3);
-            int const row = c - (l == 1 ? 0 : (l == 2 ? V::H1 : V::H1 + V::H2));
-            int const in = l == 1 ? V::H0 : (l == 2 ? V::H1 : V::H2);
-            int const off = l == 1 ? V::W1_OFF : (l == 2 ? V::W2_OFF : V::W3_OFF);
-            int32_t sum = 0, sumAbs = 0;
-            for (int k = 0; k < in; k += 4) {
-                uint32_t const v = blob32[(off + row * in + k) >> 2];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    int const w = int(int8_t(v >> (8 * r)));
-                    sum += w;
-                    sumAbs += w < 0 ? -w : w;
-                }
-            }
-            int32_t const bias = reinterpret_cast<int32_t const*>(blob + V::BIAS_OFF)[V::H0 + c];
-            shifted = int64_t(bias) - 113 * int64_t(sum);     // activations enter as q + 113 in [-15, 240]
-            int64_t const bound = (shifted < 0 ? -shifted : shifted) + 240 * int64_t(sumAbs);
-            fits = bound < (int64_t(1) << 24);
-            if (l == 3) bounded = float(bound) * fabsf(reinterpret_cast<float const*>(blob + V::SCALE_OFF)[V::H0 + c]) < 60000.f;
-            slotTile = V::T0 + (l == 1 ? 0 : (l == 2 ? V::T1 : V::T1 + V::T2)) + row / 16;
-            slotG = (row >> 2) & 3;
-            slotR = row & 3;
-        }
-        bool const useF16 = __syncthreads_and(fits ? 1 : 0) != 0;     // also orders the bias writes above
-        bool const outputsBounded = __syncthreads_and(bounded ? 1 : 0) != 0;
-        if (useF16) {
-            if (threadIdx.x < V::LATE_CHANNELS)
-                lds.bias[slotTile][slotG][slotR] = __builtin_bit_cast(int32_t, float(shifted));
-            // fp16 blocks.  Lane (i, kg) of the block of output tile t and input-tile pair p holds
-            // W[16t + i][16*(2p + e/4) + 4*kg + e%4], e = 0..7: the channels lane (j, kg) of the
-            // previous layer's D registers owns, in register order.
-            constexpr int base[4] = { 0, V::F16_L1, V::F16_L2, V::F16_L3 };
-            uint32_t* const late32 = reinterpret_cast<uint32_t*>(lds.late);
-#pragma unroll
-            for (int l = 1; l < 4; ++l) {
-                int const in = ins[l];
-                int const inTiles = tiles[l - 1], pairs = inTiles / 2, per = V::f16_units(inTiles);
-                // one work item = one (output tile, input tile, lane): 4 weights -> 2 dwords
-                for (int e = threadIdx.x; e < tiles[l] * inTiles * 64; e += blockDim.x) {
-                    int const lane = e & 63, rest = e >> 6;
-                    int const ti = rest % inTiles, t = rest / inTiles;
-                    int const i = lane & 15, kg = lane >> 4;
-                    uint32_t const v = blob32[(woff[l] + (16 * t + i) * in + 16 * ti + 4 * kg) >> 2];
-                    int const p = ti >> 1;
-                    // dword index inside `late`: paired blocks hold 4 dwords per lane, the tail block 2
-                    int const at = (p < pairs) ? ((base[l] + t * per + p * 64 + lane) * 4 + (ti & 1) * 2)
-                                               : ((base[l] + t * per + pairs * 64) * 4 + lane * 2);
-                    late32[at]     = halves_of_bytes(v, 0);
-                    late32[at + 1] = halves_of_bytes(v, 2);
-                }
-            }
-        } else {
-            int tileBase = 0;
-#pragma unroll
-            for (int l = 1; l < 4; ++l) {
-                int const in = ins[l];
-                for (int e = threadIdx.x; e < tiles[l] * 64 * 4; e += blockDim.x) {
-                    int const d = e & 3, lane = (e >> 2) & 63, t = e >> 8;
-                    int const i = lane & 15, g = lane >> 4;
-                    reinterpret_cast<uint32_t*>(lds.late)[((tileBase + t) * 64 + lane) * 4 + d] =
-                        weight_dword(blob32, woff[l], 16 * t + i, in, 16 * d + 4 * g);
-                }
-                tileBase += tiles[l];
-            }
-        }
-        return useF16 ? (kStagedF16 | (outputsBounded ? kOutputsBounded : 0)) : 0;
-    }
+    return useF16 ? (kStagedF16 | (outputsBounded ? kOutputsBounded : 0)) : 0;
 }
 
-// Input vector of one texel as 16 dwords (int8 x 64, zero padded).
 template <class V>
 __device__ __forceinline__ void prepare_inputs_general(DevMip const& m, int x, int y, uint32_t (&in)[16])
 {
@@ -933,16 +984,17 @@ __device__ __forceinline__ void mlp_forward(LdsT<V>& lds, int wave, int lane, ui
             for (int d = 0; d < 4; ++d) Y[b][d] = 0;
 #pragma unroll
         for (int t = 0; t < tiles[l]; ++t) {
-            uint4 const wa = (V::F16_LAYERS && l > 0) ? lds.late[(tb - V::T0 + t) * 64 + lane]
-                                                      : *reinterpret_cast<uint4 const*>(&lds.w[0][V::F16_LAYERS ? t : tb + t][lane][0]);
-            v4i const A = v4i{ int(wa.x), int(wa.y), int(wa.z), int(wa.w) };
+            // A operand of plane q: layer 0 from `w`, later layers from the int8 tiles in `late`
+            auto const operand = [&](int q) {
+                uint4 const wq = l > 0 ? lds.late[(q * V::LATE_TILES + tb - V::T0 + t) * 64 + lane]
+                                       : *reinterpret_cast<uint4 const*>(&lds.w[q][t][lane][0]);
+                return v4i{ int(wq.x), int(wq.y), int(wq.z), int(wq.w) };
+            };
+            v4i const A = operand(0);
             v4i const C = *reinterpret_cast<v4i const*>(&lds.bias[tb + t][g][0]);
             v4f const Sc = *reinterpret_cast<v4f const*>(&lds.scale[tb + t][g][0]);
             if constexpr (V::FP8_WEIGHTS) {
-                uint4 const wb = *reinterpret_cast<uint4 const*>(&lds.w[V::PLANES > 1 ? 1 : 0][tb + t][lane][0]);
-                uint4 const wc = *reinterpret_cast<uint4 const*>(&lds.w[V::PLANES > 2 ? 2 : 0][tb + t][lane][0]);
-                v4i const A1 = v4i{ int(wb.x), int(wb.y), int(wb.z), int(wb.w) };
-                v4i const A2 = v4i{ int(wc.x), int(wc.y), int(wc.z), int(wc.w) };
+                v4i const A1 = operand(V::PLANES > 1 ? 1 : 0), A2 = operand(V::PLANES > 2 ? 2 : 0);
                 v4i const Z = v4i{ 0, 0, 0, 0 };
 #pragma unroll
                 for (int b = 0; b < 4; ++b) {
@@ -969,7 +1021,7 @@ __device__ __forceinline__ void mlp_forward(LdsT<V>& lds, int wave, int lane, ui
     }
 
     // output layer
-    uint4 const wa = V::F16_LAYERS ? lds.late[(tb - V::T0) * 64 + lane] : *reinterpret_cast<uint4 const*>(&lds.w[0][V::F16_LAYERS ? 0 : tb][lane][0]);
+    uint4 const wa = lds.late[(tb - V::T0) * 64 + lane];
     v4i const A = v4i{ int(wa.x), int(wa.y), int(wa.z), int(wa.w) };
     v4i const C = *reinterpret_cast<v4i const*>(&lds.bias[tb][g][0]);
     S = *reinterpret_cast<v4f const*>(&lds.scale[tb][g][0]);
@@ -1051,6 +1103,33 @@ __device__ __forceinline__ void f16_hidden_layer(LdsT<V> const& lds, int base, i
     }
 }
 
+// The same for a layer with e4m3 weights held as two fp16 planes (512 w = 1024 hi + lo): both sums are exact
+// integers in fp32, and fma(hi, 1024, lo) rounds their exact combination once - the value a conversion of
+// the int32 accumulator to float gives.
+template <class V, int IN_TILES, int OUT_TILES>
+__device__ __forceinline__ void f16_hidden_layer_two_planes(LdsT<V> const& lds, int base, int tileBase, int lane,
+                                                            uint32_t const (&Hin)[4][4][2], uint32_t (&Hout)[4][4][2])
+{
+    constexpr int PLANE = OUT_TILES * V::f16_units(IN_TILES);
+    int const g = lane >> 4;
+#pragma unroll
+    for (int t = 0; t < OUT_TILES; ++t) {
+        v4f const Chi = *reinterpret_cast<v4f const*>(&lds.bias[tileBase + t][g][0]);
+        v4f const Clo = *reinterpret_cast<v4f const*>(&lds.biasLo[tileBase + t][g][0]);
+        v4f const Sc = *reinterpret_cast<v4f const*>(&lds.scale[tileBase + t][g][0]);
+        v4f hi[4] = { Chi, Chi, Chi, Chi }, lo[4] = { Clo, Clo, Clo, Clo };
+        f16_tile<V, IN_TILES>(lds, base, t, lane, Hin, hi);
+        f16_tile<V, IN_TILES>(lds, base + PLANE, t, lane, Hin, lo);
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            v4f acc;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[r] = __builtin_fmaf(hi[b][r], 1024.f, lo[b][r]);
+            activate4_h(acc, Sc, Hout[b][t]);
+        }
+    }
+}
+
 // The network for the 64 texels of one wave with layers 1..3 on the fp16 matrix instruction.
 // Same interface as mlp_forward, except that D holds the output layer's accumulators as floats
 // (exact integers).
@@ -1077,20 +1156,44 @@ __device__ __forceinline__ void mlp_forward_f16(LdsT<V>& lds, int wave, int lane
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
 
-    // layer 0: int8 inputs, int32 accumulators
+    // layer 0: int8 inputs, int32 accumulators (three planes for e4m3 weights, recombined wrapping like int32)
     uint32_t Ha[4][4][2], Hb[4][4][2];
 #pragma unroll
     for (int t = 0; t < V::T0; ++t) {
-        uint4 const wa = *reinterpret_cast<uint4 const*>(&lds.w[0][t][lane][0]);
-        v4i const A = v4i{ int(wa.x), int(wa.y), int(wa.z), int(wa.w) };
+        auto const operand = [&](int q) {
+            uint4 const wq = *reinterpret_cast<uint4 const*>(&lds.w[q][t][lane][0]);
+            return v4i{ int(wq.x), int(wq.y), int(wq.z), int(wq.w) };
+        };
+        v4i const A = operand(0);
         v4i const C = *reinterpret_cast<v4i const*>(&lds.bias[t][g][0]);
         v4f const Sc = *reinterpret_cast<v4f const*>(&lds.scale[t][g][0]);
+        if constexpr (V::FP8_WEIGHTS) {
+            v4i const A1 = operand(V::PLANES > 1 ? 1 : 0), A2 = operand(V::PLANES > 2 ? 2 : 0);
+            v4i const Z = v4i{ 0, 0, 0, 0 };
 #pragma unroll
-        for (int b = 0; b < 4; ++b)
-            activate4_h(__builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0), Sc, Ha[b][t]);
+            for (int b = 0; b < 4; ++b) {
+                v4i const D0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
+                v4i const D1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A1, X[b], Z, 0, 0, 0);
+                v4i const D2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A2, X[b], Z, 0, 0, 0);
+                v4i Dh;
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    Dh[r] = int((((uint32_t(D2[r]) << 6) + uint32_t(D1[r])) << 6) + uint32_t(D0[r]));
+                activate4_h(Dh, Sc, Ha[b][t]);
+            }
+        } else {
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+                activate4_h(__builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0), Sc, Ha[b][t]);
+        }
     }
-    f16_hidden_layer<V, V::T0, V::T1>(lds, V::F16_L1, V::T0, lane, Ha, Hb);
-    f16_hidden_layer<V, V::T1, V::T2>(lds, V::F16_L2, V::T0 + V::T1, lane, Hb, Ha);
+    if constexpr (V::FP8_WEIGHTS) {
+        f16_hidden_layer_two_planes<V, V::T0, V::T1>(lds, V::F16_L1, V::T0, lane, Ha, Hb);
+        f16_hidden_layer_two_planes<V, V::T1, V::T2>(lds, V::F16_L2, V::T0 + V::T1, lane, Hb, Ha);
+    } else {
+        f16_hidden_layer<V, V::T0, V::T1>(lds, V::F16_L1, V::T0, lane, Ha, Hb);
+        f16_hidden_layer<V, V::T1, V::T2>(lds, V::F16_L2, V::T0 + V::T1, lane, Hb, Ha);
+    }
 
     constexpr int outTile = V::T0 + V::T1 + V::T2;
     v4f const C = *reinterpret_cast<v4f const*>(&lds.bias[outTile][g][0]);
@@ -1101,7 +1204,7 @@ __device__ __forceinline__ void mlp_forward_f16(LdsT<V>& lds, int wave, int lane
 }
 
 // Four workgroups per CU (16 waves, 128 VGPRs each) is what the LDS footprint allows and what hides
-// the latency of the input stage; the e4m3 variants hold three weight planes in LDS and fit two.
+// the latency of the input stage; the e4m3 variants hold several planes of every weight in LDS and fit two.
 template <class V>
 __global__ void __launch_bounds__(256, V::FP8_WEIGHTS ? 2 : 4)
 decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)

@@ -127,8 +127,9 @@ def test_cfg2_batch_of_sets(ntc, device):
 @pytest.mark.parametrize("w,h,mips,fmt", [(256, 256, 1, "planar"), (128, 64, 8, "unorm8"), (90, 70, 4, "fp16px")])
 def test_cfg3_fp8_weights(ntc, device, w, h, mips, fmt):
     """Config 3's shape: wide 64-64-64 decoder whose hidden-layer weights are FP8 e4m3 with a per-channel
-    fp32 scale.  The device evaluates the e4m3 dot products exactly (three 6-bit integer planes on the
-    int8 MFMA), so the comparison is byte equality - inside the 1e-3 / 1 LSB bound with room to spare."""
+    fp32 scale.  The device evaluates the e4m3 dot products exactly (integer planes of 512 w: three on the int8
+    MFMA for layer 0, two on the fp16 MFMA for layers 1 and 2), so the comparison is byte equality - inside the
+    1e-3 / 1 LSB bound with room to spare."""
     f = {"planar": ntc.abi.OUT_FP16_PLANAR_PAIRS, "fp16px": ntc.abi.OUT_FP16_PIXELS, "unorm8": ntc.abi.OUT_UNORM8_PIXELS}[fmt]
     for scales in ((-17.0, -13.0), (-10.0, -4.0)):
         case = cfg_case(ntc, ntc.presets.spec_cfg3(), w, h, mips, 16, f, seed=w + mips, scale_log2_range=scales)
@@ -151,6 +152,35 @@ def test_cfg3_fp8_extreme_weights(ntc, device):
     case = cfg_case(ntc, spec, 64, 64, 1, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=19, weights=blob)
     expected, got = run_both(device, case)
     assert_equal_bytes(expected, got, "cfg3 fp8 extreme")
+
+
+@pytest.mark.parametrize("slack", [-1, 0, 1, 1 << 20])
+def test_cfg3_fp8_fp16_layer_path_boundary(ntc, device, slack):
+    """Layers 1 and 2 of the e4m3 decoder run as two fp16 planes only while the int32 accumulator that defines
+    the result cannot wrap: |bias| + 128 * sum|512 w| < 2^31 for every channel.  One channel per layer is put
+    just inside (slack -1), on and past that limit, with both signs of the bias, so the fp16 planes, the
+    three-plane int8 form and the switch between them all face the checker's wrapping arithmetic."""
+    import np_decoder
+    spec = ntc.presets.spec_cfg3()
+    layout = ntc.synth.weight_layout(spec)
+    for sign in (1, -1):
+        blob = ntc.synth.make_weights(spec, 60 + slack % 5, scale_log2_range=(-30.0, -22.0), bias_sigma=1e-7)
+        bias = blob[layout.biasOffset[0]:layout.bufferSize].view(np.int32)
+        inside = True
+        for layer, row in ((1, 7), (2, 42)):
+            w = blob[layout.weightOffset[layer]: layout.weightOffset[layer] + 64 * 64].reshape(64, 64)
+            row_abs = np.abs(np_decoder.e4m3_times_512(w)).sum(axis=1)
+            magnitude = (1 << 31) + slack - 128 * int(row_abs[row])     # |bias| + 128*sum|512 w| = 2^31 + slack
+            magnitude = min(magnitude, (1 << 31) - 1)                     # (an int32 cannot hold more)
+            assert 0 < magnitude
+            bias[64 * layer + row] = sign * magnitude
+            limits = np.abs(bias[64 * layer: 64 * layer + 64].astype(np.int64)) + 128 * row_abs
+            assert ((limits >= 1 << 31) == (np.arange(64) == row)).all() if magnitude + 128 * int(row_abs[row]) >= 1 << 31 else (limits < 1 << 31).all()
+            inside = inside and bool((limits < 1 << 31).all())
+        assert inside == (slack < 0)
+        case = cfg_case(ntc, spec, 128, 64, 3, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=61, weights=blob)
+        expected, got = run_both(device, case)
+        assert_equal_bytes(expected, got, f"cfg3 fp16 path boundary, slack {slack}, sign {sign}")
 
 
 def test_extreme_weights_saturate_cleanly(ntc, device):
