@@ -146,6 +146,7 @@ hipError_t launch_decode(int variant, DevMip const* mips, int numMips, int total
 hipError_t launch_queries(int variant, DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries,
                           uint16_t* out, int gridSize, hipStream_t stream);
 int resident_workgroups_per_cu(int variant);
+int tiles_per_round(int variant);      // tiles a workgroup of the variant's decode kernel works on at a time
 hipError_t launch_selftest_mfma(int8_t const* a, int8_t const* b, int32_t* d, hipStream_t stream);
 hipError_t launch_selftest_mfma_f16(uint16_t const* a, uint16_t const* b, float const* c, float* d, int depth, hipStream_t stream);
 

@@ -49,9 +49,7 @@ __device__ __forceinline__ uint32_t mul24(uint32_t a, uint32_t b)
 }
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-constexpr int kWaves       = 4;     // waves per workgroup
 constexpr int kWaveTexels  = 64;
-constexpr int kInStride    = 20;    // dwords per texel row in the transpose buffer (16 + pad)
 
 // ---- small device helpers -----------------------------------------------------------
 
@@ -278,6 +276,16 @@ struct Variant {
     static constexpr bool FP8_WEIGHTS = FP8_WEIGHTS_;
     static constexpr int PLANES = FP8_WEIGHTS_ ? 3 : 1;
     static constexpr int F16_PLANES = FP8_WEIGHTS_ ? 2 : 1;
+    // Waves per workgroup: four cover one 64 x 4 tile.  The e4m3 variants keep so many weight planes in LDS that
+    // only two workgroups fit a CU; theirs have eight waves (two tiles at a time), which again puts four waves
+    // on every SIMD to overlap matrix and vector work.
+    static constexpr int WAVES = FP8_WEIGHTS_ ? 8 : 4;
+    static constexpr int THREADS = 64 * WAVES;
+    static constexpr int RESIDENT = FP8_WEIGHTS_ ? 2 : 4;      // workgroups per CU the LDS footprint allows
+    static constexpr int WAVES_PER_SIMD = RESIDENT * WAVES / 4; // what the register budget is set for
+    // Dwords per texel in the transpose buffer in front of the network: 16 + 4 of padding, or 12 without
+    // padding for 48 inputs (rows then still start in distinct banks: 12 j mod 64 differ for j = 0..15).
+    static constexpr int IN_STRIDE = (FP8_WEIGHTS_ && IN_ <= 48) ? 12 : 20;
     static constexpr int HR_MODE = HR_MODE_, HR_F = HR_F_, HR_BITS = HR_BITS_, HR_SLOTS = HR_SLOTS_;
     static constexpr int LR_F = LR_F_, LR_SLOTS = LR_SLOTS_, LOD = LOD_;
     static constexpr int IN = IN_, H0 = H0_, H1 = H1_, H2 = H2_, OUT = 16;
@@ -323,7 +331,7 @@ struct alignas(16) LdsT : BiasLoT<V::FP8_WEIGHTS, V::NTILES> {
     uint4    late[V::LATE_UNITS];              // A operands of layers 1..3: int8 tiles or fp16 blocks
     float    scale[V::NTILES][4][4];           // [M-tile][k-group g][r]  -> channel 16t+4g+r
     int32_t  bias[V::NTILES][4][4];
-    uint32_t in[kWaves][kWaveTexels][kInStride];
+    uint32_t in[V::WAVES][kWaveTexels][V::IN_STRIDE];
     uint32_t lut2[256];               // byte of four 2-bit codes -> four input bytes 85*q - 128
     // Positional encoding for every power-of-two positionScale 2^-k, k = 0..5: the entry for phase p of
     // scale 2^-k sits at index (2^k - 1) + p; dword w = enc(px*2^w) | enc(px*2^w + 1/4) << 16, px = p*2^-k.
@@ -943,12 +951,10 @@ __device__ void build_posenc_tables(LdsT<V>& lds)
     }
 }
 
-// The network for the 64 texels of one wave.  `in` is the lane's own texel (lane = 16*b + j).
-// On return D[b] holds, for lane (j = lane%16, g = lane/16), the int32 accumulators of output
-// channels 4g..4g+3 of texel 16*b + j, and S their scales.
+// Input vectors of the wave's 64 texels (lane = texel 16*b + j holds its own in `in`) -> B operands of
+// layer 0: X[b] = the four input dwords of k-group g = lane/16 of texel 16b + lane%16.
 template <class V>
-__device__ __forceinline__ void mlp_forward(LdsT<V>& lds, int wave, int lane, uint32_t const (&in)[16], uint32_t c143,
-                                            v4i (&D)[4], v4f& S)
+__device__ __forceinline__ void transpose_inputs(LdsT<V>& lds, int wave, int lane, uint32_t const (&in)[16], v4i (&X)[4])
 {
     int const j = lane & 15, g = lane >> 4;
     {
@@ -956,21 +962,34 @@ __device__ __forceinline__ void mlp_forward(LdsT<V>& lds, int wave, int lane, ui
         dst[0] = make_uint4(in[0], in[1], in[2], in[3]);
         dst[1] = make_uint4(in[4], in[5], in[6], in[7]);
         dst[2] = make_uint4(in[8], in[9], in[10], in[11]);
-        dst[3] = make_uint4(in[12], in[13], in[14], in[15]);
+        if constexpr (V::IN_STRIDE >= 16) dst[3] = make_uint4(in[12], in[13], in[14], in[15]);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-
-    // B operands of layer 0: block b = texels 16b..16b+15, column j, k-group g
-    v4i X[4];
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
-        uint4 const t = *reinterpret_cast<uint4 const*>(&lds.in[wave][b * 16 + j][4 * g]);
+        // a row of 12 dwords has no k-group 3: those inputs are the zero padding
+        int const gRead = V::IN_STRIDE >= 16 ? g : min(g, 2);
+        uint4 t = *reinterpret_cast<uint4 const*>(&lds.in[wave][b * 16 + j][4 * gRead]);
+        if (V::IN_STRIDE < 16 && g == 3) t = make_uint4(0u, 0u, 0u, 0u);
         X[b] = v4i{ int(t.x), int(t.y), int(t.z), int(t.w) };
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
+}
+
+// The network for the 64 texels of one wave.  `in` is the lane's own texel (lane = 16*b + j).
+// On return D[b] holds, for lane (j = lane%16, g = lane/16), the int32 accumulators of output
+// channels 4g..4g+3 of texel 16*b + j, and S their scales.
+template <class V>
+__device__ __forceinline__ void mlp_forward(LdsT<V>& lds, int wave, int lane, uint32_t const (&in)[16], uint32_t c143,
+                                            v4i (&D)[4], v4f& S)
+{
+    int const g = lane >> 4;
+    v4i X[4];
+    transpose_inputs<V>(lds, wave, lane, in, X);
+
 
     // hidden layers
     constexpr int tiles[3] = { V::T0, V::T1, V::T2 };
@@ -1136,25 +1155,9 @@ __device__ __forceinline__ void f16_hidden_layer_two_planes(LdsT<V> const& lds, 
 template <class V>
 __device__ __forceinline__ void mlp_forward_f16(LdsT<V>& lds, int wave, int lane, uint32_t const (&in)[16], v4f (&D)[4], v4f& S)
 {
-    int const j = lane & 15, g = lane >> 4;
-    {
-        uint4* dst = reinterpret_cast<uint4*>(&lds.in[wave][lane][0]);
-        dst[0] = make_uint4(in[0], in[1], in[2], in[3]);
-        dst[1] = make_uint4(in[4], in[5], in[6], in[7]);
-        dst[2] = make_uint4(in[8], in[9], in[10], in[11]);
-        dst[3] = make_uint4(in[12], in[13], in[14], in[15]);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    int const g = lane >> 4;
     v4i X[4];
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-        uint4 const t = *reinterpret_cast<uint4 const*>(&lds.in[wave][b * 16 + j][4 * g]);
-        X[b] = v4i{ int(t.x), int(t.y), int(t.z), int(t.w) };
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
+    transpose_inputs<V>(lds, wave, lane, in, X);
 
     // layer 0: int8 inputs, int32 accumulators (three planes for e4m3 weights, recombined wrapping like int32)
     uint32_t Ha[4][4][2], Hb[4][4][2];
@@ -1206,12 +1209,14 @@ __device__ __forceinline__ void mlp_forward_f16(LdsT<V>& lds, int wave, int lane
 // Four workgroups per CU (16 waves, 128 VGPRs each) is what the LDS footprint allows and what hides
 // the latency of the input stage; the e4m3 variants hold several planes of every weight in LDS and fit two.
 template <class V>
-__global__ void __launch_bounds__(256, V::FP8_WEIGHTS ? 2 : 4)
+__global__ void __launch_bounds__(V::THREADS, V::WAVES_PER_SIMD)
 decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
 {
     __shared__ LdsT<V> lds;
+    constexpr int GROUP = V::WAVES / 4;                      // tiles a workgroup works on at a time
     int const lane = threadIdx.x & 63;
     int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int const member = GROUP > 1 ? wave >> 2 : 0;            // which tile of the group this wave works on
     int const j = lane & 15, g = lane >> 4;
 
     // contiguous share of the tile list for this workgroup
@@ -1235,20 +1240,37 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     int staged = 0;                                          // uniform: how layers 1..3 of the staged set run (kStagedF16, ...)
     int entry = 0;
 
-    for (int tile = tileBegin; tile < tileEnd; ++tile) {
-        while (entry + 1 < numMips && mips[entry + 1].tileStart <= tile) ++entry;
-        DevMip const& m = mips[entry];
+    for (int first = tileBegin; first < tileEnd; ) {
+        while (entry + 1 < numMips && mips[entry + 1].tileStart <= first) ++entry;
 
-        if (m.weights != stagedBlob) {                       // uniform across the workgroup
+        if (mips[entry].weights != stagedBlob) {             // uniform across the workgroup
             __syncthreads();
-            staged = stage_weights<V>(lds, m.weights);
-            stagedBlob = m.weights;
+            staged = stage_weights<V>(lds, mips[entry].weights);
+            stagedBlob = mips[entry].weights;
             __syncthreads();                                 // also publishes the tables built above
         }
 
+        // This round's tiles: `first` and the ones after it that use the staged weights, GROUP at most.  Every
+        // thread computes the same count, so the loop (and the barriers above) stay uniform; a wave without a
+        // tile sits the round out.
+        int count = 1, mine = entry;
+        if constexpr (GROUP > 1) {
+            int next = entry;
+            for (int k = 1; k < GROUP && first + k < tileEnd; ++k) {
+                while (next + 1 < numMips && mips[next + 1].tileStart <= first + k) ++next;
+                if (mips[next].weights != stagedBlob) break;
+                ++count;
+                if (k == member) mine = next;
+            }
+        }
+        int const tile = first + member;
+        first += count;
+        if (GROUP > 1 && member >= count) continue;
+        DevMip const& m = mips[mine];
+
         int const local = tile - m.tileStart;
         int const tileY = local / m.tilesX, tileX = local - tileY * m.tilesX;
-        int const x0 = tileX * 64 + wave * 16;
+        int const x0 = tileX * 64 + (GROUP > 1 ? wave & 3 : wave) * 16;
         int const y0 = tileY * 4;
         if (x0 >= m.width) continue;                         // whole wave tile outside the image
 
@@ -1307,7 +1329,7 @@ struct QueryMip {
 static_assert(sizeof(QueryMip) == 96, "QueryMip layout");
 
 template <class V>
-__global__ void __launch_bounds__(256, V::FP8_WEIGHTS ? 2 : 4)
+__global__ void __launch_bounds__(V::THREADS, V::WAVES_PER_SIMD)
 query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __restrict__ queries, uint64_t numQueries,
              uint16_t* __restrict__ out)
 {
@@ -1341,9 +1363,9 @@ query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __res
     bool const useF16 = (stage_weights<V>(lds, mips[0].weights) & kStagedF16) != 0;
     __syncthreads();
 
-    uint64_t const numBlocks = (numQueries + 255) / 256;
+    uint64_t const numBlocks = (numQueries + V::THREADS - 1) / V::THREADS;
     for (uint64_t block = blockIdx.x; block < numBlocks; block += gridDim.x) {
-        uint64_t const q0 = block * 256 + uint64_t(wave) * 64;
+        uint64_t const q0 = block * V::THREADS + uint64_t(wave) * 64;
         if (q0 >= numQueries) continue;
         uint64_t const qi = min(q0 + uint64_t(lane), numQueries - 1);
         DevQuery const query = queries[qi];
@@ -1449,7 +1471,7 @@ using VCfg3   = Variant<0, 16, 4, 16, 16, 16, 2, 48, 64, 64, 64, true>;   // wid
 template <class V>
 static hipError_t launch_variant(DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream)
 {
-    hipLaunchKernelGGL(decode_kernel<V>, dim3(gridSize), dim3(256), 0, stream, mips, numMips, totalTiles);
+    hipLaunchKernelGGL(decode_kernel<V>, dim3(gridSize), dim3(V::THREADS), 0, stream, mips, numMips, totalTiles);
     return hipGetLastError();
 }
 
@@ -1471,7 +1493,7 @@ template <class V>
 static hipError_t launch_query_variant(DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries,
                                        uint16_t* out, int gridSize, hipStream_t stream)
 {
-    hipLaunchKernelGGL(query_kernel<V>, dim3(gridSize), dim3(256), 0, stream, mips, numMips, queries, numQueries, out);
+    hipLaunchKernelGGL(query_kernel<V>, dim3(gridSize), dim3(V::THREADS), 0, stream, mips, numMips, queries, numQueries, out);
     return hipGetLastError();
 }
 
@@ -1518,7 +1540,7 @@ template <class V>
 static int occupancy_variant()
 {
     int blocks = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, decode_kernel<V>, 256, 0) != hipSuccess || blocks < 1) blocks = 2;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, decode_kernel<V>, V::THREADS, 0) != hipSuccess || blocks < 1) blocks = 2;
     return blocks;
 }
 
@@ -1536,6 +1558,8 @@ int resident_workgroups_per_cu(int variant)
     default: return 2;
     }
 }
+
+int tiles_per_round(int variant) { return variant == NTC_HIP_VARIANT_CFG3_FP8 ? VCfg3::WAVES / 4 : 1; }
 
 hipError_t launch_selftest_mfma(int8_t const* a, int8_t const* b, int32_t* d, hipStream_t stream)
 {

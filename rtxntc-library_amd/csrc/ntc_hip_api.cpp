@@ -363,7 +363,9 @@ int grid_size_for(int variant, int totalTiles)
         perCu[variant] = resident_workgroups_per_cu(variant);
     }
     int const resident = g_lib.computeUnits * perCu[variant];
-    return totalTiles < resident ? totalTiles : resident;
+    // a workgroup takes tiles_per_round(variant) tiles at a time: fewer workgroups than that leaves waves idle
+    int64_t const rounds = (int64_t(totalTiles) + tiles_per_round(variant) - 1) / tiles_per_round(variant);
+    return rounds < resident ? int(rounds) : resident;
 }
 
 } // namespace

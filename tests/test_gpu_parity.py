@@ -124,6 +124,24 @@ def test_cfg2_batch_of_sets(ntc, device):
         assert_equal_bytes(hset.output, c.d_output.download(), f"cfg2 set {i}")
 
 
+def test_cfg3_fp8_batch_of_sets(ntc, device):
+    """Several e4m3 sets with their own weights in one launch.  A workgroup of that decoder works on two tiles at
+    a time as long as both use the staged weights; every set has an odd number of tiles (353) and a workgroup's
+    share is four tiles, so shares straddle set boundaries at either parity."""
+    spec = ntc.presets.spec_cfg3()
+    cases = [cfg_case(ntc, spec, 256, 256, 9, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=300 + i, scale_log2_range=ACTIVE)
+             for i in range(5)]
+    assert sum(((m.width + 63) // 64) * ((m.height + 3) // 4) for m in cases[0].mips) == 353
+    hosts = [c.host_set() for c in cases]
+    for hset in hosts:
+        hset.decode(threads=8)
+    dsets = [c.device_set(device) for c in cases]
+    device.decode(dsets)
+    device.synchronize()
+    for i, (c, hset) in enumerate(zip(cases, hosts)):
+        assert_equal_bytes(hset.output, c.d_output.download(), f"cfg3 set {i}")
+
+
 @pytest.mark.parametrize("w,h,mips,fmt", [(256, 256, 1, "planar"), (128, 64, 8, "unorm8"), (90, 70, 4, "fp16px")])
 def test_cfg3_fp8_weights(ntc, device, w, h, mips, fmt):
     """Config 3's shape: wide 64-64-64 decoder whose hidden-layer weights are FP8 e4m3 with a per-channel
