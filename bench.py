@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the texture-set decode path on one MI355X.
 
-Default (the headline, BASELINE config 1): decode a 4096x4096, 16-channel texture set with its
+Default (the headline configuration): decode a 4096x4096, 16-channel texture set with its
 full 13-level mip chain (22 369 621 texels; 2x2-concat 8x2-bit high-res grid + bilinear 16x4-bit
 low-res grid, MLP 64-48-32 int8, fp16 output), bit-exact arithmetic, ONE launch per step.
 
@@ -9,7 +9,7 @@ Prints ONE JSON line.  A step = one full decode of the workload; inputs (latents
 queries) are resident in HBM before the timed region.  `roofline` is for the decode kernel (the
 only kernel of the path), timed with HIP events on the library's own launch stream;
 `cpu_baseline` is the CPU checker on the same workload (or a bounded sample of it) on this
-machine's host cores.  Other --workload values measure the other BASELINE configurations.
+machine's host cores.  Other --workload values measure the other configurations and kernels.
 """
 import argparse
 import ctypes as C

@@ -1,4 +1,4 @@
-"""BASELINE.json's full-size configurations on the GPU: complete comparison with the CPU checker
+"""The benchmark configurations at their full sizes on the GPU: complete comparison with the CPU checker
 where that takes seconds, and size-independent properties (periodicity under periodic latents,
 batch = individual, queries = raster) where the checker would be too slow to cover everything."""
 import ctypes as C

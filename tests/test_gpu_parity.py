@@ -72,7 +72,7 @@ def test_mfma_f16_integer_sums_are_exact(device, depth):
 
 @pytest.mark.parametrize("scale_range", [(-10.0, -4.0), ACTIVE])
 def test_cfg0_plumbing_512_fp16(ntc, device, scale_range):
-    """BASELINE config 0: 512x512, one mip, 8 channels, 64-48-32 int8, fp16 planar output."""
+    """The plumbing configuration: 512x512, one mip, 8 channels, 64-48-32 int8, fp16 planar output."""
     case = cfg_case(ntc, ntc.presets.spec_cfg01(), 512, 512, 1, 8, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=0,
                     scale_log2_range=scale_range)
     expected, got = run_both(device, case)
