@@ -160,6 +160,52 @@ def test_malformed_files_same_status_as_the_reference_front_end(ntc, tmp_path):
             assert ref_status == status, (name, ref_status, ref_message, status, message)
 
 
+def test_random_document_damage_same_status_as_the_reference_front_end(ntc, tmp_path):
+    """Seeded damage to the JSON document (values replaced by extremes or other types, members and elements
+    removed): whenever the reference's front end (LoadFileHeadersFromStream + its document parser, built from
+    the reference's own sources) refuses a file, the host layer refuses it with the same status, and nearly
+    always with the same complaint (the reference prefixes the position in the text)."""
+    lib = ref_file_lib()
+    if lib is None:
+        pytest.skip("the reference's host-only sources are not built on this machine")
+    import random
+    case = make_case(ntc)
+    text, binary = nw.split_container(file_of(case, 64, 32, 2, 8, 8, textures=TEXTURES))
+    values = [0, -1, 1, 2 ** 31 - 1, 2 ** 31, 2 ** 32 - 1, 2 ** 32, 2 ** 63, 10 ** 30, 0.5, 1e308, 65535, 17,
+              "x", "", None, True, [], {}, [1], {"a": 1}]
+
+    def slots(node):
+        if isinstance(node, dict):
+            for key, value in list(node.items()):
+                yield node, key
+                yield from slots(value)
+        elif isinstance(node, list):
+            for index, value in enumerate(node):
+                yield node, index
+                yield from slots(value)
+
+    rnd = random.Random(2024)
+    refused = same_text = 0
+    for i in range(120):
+        doc = json.loads(text)
+        for _ in range(rnd.randint(1, 2)):
+            owner, key = rnd.choice(list(slots(doc)))
+            if rnd.random() < 0.25:
+                del owner[key]
+            else:
+                owner[key] = rnd.choice(values)
+        data = nw.pack_container(json.dumps(doc), binary)
+        ref_status, _, _, ref_message = ref_parse(lib, data)
+        status, message, _ = host_load(tmp_path, data)
+        if ref_status != 0:
+            refused += 1
+            assert status == ref_status, (i, ref_status, ref_message, status, message)
+            same_text += ref_message.endswith(message)
+        else:
+            assert status != 0          # no device here: at best everything validates and the upload fails
+    assert refused >= 60 and same_text >= 0.9 * refused, (refused, same_text)
+
+
 def test_semantic_errors_of_the_metadata_stage(ntc, tmp_path):
     """Rules of LoadMetadataFromStream / ValidateMLP / ValidateBufferView / LoadFromStreamPostHeader
     (src/TextureSetMetadata.cpp:434-581,978-1135, src/TextureSet.cpp:154-196); the reference needs a
