@@ -27,6 +27,11 @@ struct Value
     uint64_t magnitude = 0;
     double real = 0.0;
     std::string text;
+    // Where the reference's streaming reader stands when it rejects this value (it reports that offset and the
+    // text that follows): the first character of a number; just behind a string, a literal, or the opening
+    // bracket of an array or object.  closeAt: just behind the closing bracket, where missing members of an object
+    // (closing bracket) are noticed.
+    size_t at = 0, closeAt = 0;
     std::vector<Value> items;
     std::vector<std::pair<std::string, Value>> members;
 
@@ -94,23 +99,27 @@ private:
     {
         if (depth > kMaxDepth) return Fail("The document is nested too deeply.");
         if (m_p == m_end) return Fail("Invalid value.");
+        bool ok;
         switch (*m_p) {
         case '{': return ParseObject(out, depth);
         case '[': return ParseArray(out, depth);
-        case '"': out.kind = Value::String; return ParseString(out.text);
-        case 't': out.kind = Value::Bool; out.boolean = true; return Literal("true");
-        case 'f': out.kind = Value::Bool; out.boolean = false; return Literal("false");
-        case 'n': out.kind = Value::Null; return Literal("null");
-        default: return ParseNumber(out);
+        case '"': out.kind = Value::String; ok = ParseString(out.text); break;
+        case 't': out.kind = Value::Bool; out.boolean = true; ok = Literal("true"); break;
+        case 'f': out.kind = Value::Bool; out.boolean = false; ok = Literal("false"); break;
+        case 'n': out.kind = Value::Null; ok = Literal("null"); break;
+        default: out.at = size_t(m_p - m_begin); return ParseNumber(out);
         }
+        out.at = size_t(m_p - m_begin);
+        return ok;
     }
 
     bool ParseObject(Value& out, int depth)
     {
         out.kind = Value::Object;
         ++m_p;
+        out.at = size_t(m_p - m_begin);
         SkipSpace();
-        if (m_p != m_end && *m_p == '}') { ++m_p; return true; }
+        if (m_p != m_end && *m_p == '}') { ++m_p; out.closeAt = size_t(m_p - m_begin); return true; }
         for (;;) {
             SkipSpace();
             if (m_p == m_end || *m_p != '"') return Fail("Missing a name for object member.");
@@ -124,7 +133,7 @@ private:
             if (!ParseValue(out.members.back().second, depth + 1)) return false;
             SkipSpace();
             if (m_p != m_end && *m_p == ',') { ++m_p; continue; }
-            if (m_p != m_end && *m_p == '}') { ++m_p; return true; }
+            if (m_p != m_end && *m_p == '}') { ++m_p; out.closeAt = size_t(m_p - m_begin); return true; }
             return Fail("Missing a comma or '}' after an object member.");
         }
     }
@@ -133,15 +142,16 @@ private:
     {
         out.kind = Value::Array;
         ++m_p;
+        out.at = size_t(m_p - m_begin);
         SkipSpace();
-        if (m_p != m_end && *m_p == ']') { ++m_p; return true; }
+        if (m_p != m_end && *m_p == ']') { ++m_p; out.closeAt = size_t(m_p - m_begin); return true; }
         for (;;) {
             SkipSpace();
             out.items.emplace_back();
             if (!ParseValue(out.items.back(), depth + 1)) return false;
             SkipSpace();
             if (m_p != m_end && *m_p == ',') { ++m_p; continue; }
-            if (m_p != m_end && *m_p == ']') { ++m_p; return true; }
+            if (m_p != m_end && *m_p == ']') { ++m_p; out.closeAt = size_t(m_p - m_begin); return true; }
             return Fail("Missing a comma or ']' after an array element.");
         }
     }
@@ -258,6 +268,31 @@ private:
     std::string& m_error;
 };
 
+// A complaint about the value at text offset `at`, to be completed by ParseDocument, which has the text:
+// marker, offset, marker, message.
+constexpr char kLocated = '\x01';
+std::string LocatedMessage(size_t at, char const* message)
+{
+    return std::string(1, kLocated) + std::to_string(at) + kLocated + message;
+}
+
+// "Error at character N (the 28 characters from there on, "..." when more follow): message", the form of the
+// reference's reader (src/JsonSerialization.cpp:1040-1058).
+std::string ExpandLocatedMessage(std::string const& error, char const* json, size_t length)
+{
+    if (error.empty() || error[0] != kLocated) return error;
+    size_t const second = error.find(kLocated, 1);
+    if (second == std::string::npos) return error;
+    size_t at = size_t(std::strtoull(error.c_str() + 1, nullptr, 10));
+    if (at > length) at = length;
+    size_t left = 0;
+    while (at + left < length && json[at + left] != 0) ++left;
+    size_t const n = left < 28 ? left : 28;
+    char buf[512];
+    std::snprintf(buf, sizeof buf, "Error at character %zu (%.*s%s): %s", at, int(n), json + at, left > n ? "..." : "", error.c_str() + second + 1);
+    return buf;
+}
+
 // Typed access to the members of one JSON object of schema type `typeName`.
 class Members
 {
@@ -317,6 +352,19 @@ public:
         out = m_found;
         return true;
     }
+    // Hands the elements of an array of objects to `read`, one after the other in the order of the text, each
+    // checked to be an object first.  Never required; a bare object counts as an array of one, as with the
+    // reference's reader.
+    template <typename Read> bool ForEachObject(char const* name, Read read)
+    {
+        if (!Optional(name)) return true;
+        Value const& field = *m_found;
+        if (field.kind == Value::Object) return read(field);
+        if (field.kind != Value::Array) return WrongType(name, "array", field);
+        for (Value const& item : field.items)
+            if (!ElementMustBeObject(name, item, field) || !read(item)) return false;
+        return true;
+    }
     bool OptionalObject(char const* name, Value const*& out)
     {
         out = nullptr;
@@ -327,25 +375,50 @@ public:
     }
     bool ArrayOfUInt(char const* name, std::vector<uint32_t>& out)
     {
-        Value const* array;
-        if (!Array(name, "uint", array)) return false;
-        if (array) for (Value const& item : array->items)
-            if (!AsUnsigned(name, item, UINT32_MAX, "uint", [&](uint64_t v) { out.push_back(uint32_t(v)); })) return false;
-        return true;
+        if (!Optional(name)) return true;
+        // a bare number counts as an array of one, as with the reference's reader
+        if (m_found->kind == Value::Integer) return AsUnsigned(name, *m_found, UINT32_MAX, "uint", [&](uint64_t v) { out.push_back(uint32_t(v)); });
+        if (m_found->kind != Value::Array) return WrongType(name, "uint", *m_found);
+        return UIntElements(name, *m_found, nullptr, out);
     }
-    bool ElementMustBeObject(char const* name, Value const& item) { return item.kind == Value::Object ? true : WrongType(name, "array", item); }
+    // An element of an array of objects.  The reference's reader takes an array in that place for the start of the
+    // field's own array once more: a scalar inside it is then the wrong thing in an array of objects, and when the
+    // nested array closes, the field's array counts as closed, which its real end then trips over.
+    bool ElementMustBeObject(char const* name, Value const& item, Value const& fieldArray)
+    {
+        if (item.kind == Value::Object) return true;
+        Value const* inner = &item;
+        while (inner->kind == Value::Array && !inner->items.empty() && inner->items.front().kind == Value::Array) inner = &inner->items.front();
+        if (inner->kind != Value::Array) return WrongType(name, "array", item);
+        if (!inner->items.empty() && inner->items.front().kind != Value::Object) return WrongType(name, "array", inner->items.front());
+        m_error = LocatedMessage(fieldArray.closeAt, "End-of-array encountered outside of an array");
+        return false;
+    }
 
 private:
+    // The elements of an array of numbers.  A nested array is taken by the reference's reader for the start of the
+    // field's array once more; when the first such array closes, the field's array counts as closed, the
+    // elements that follow are skipped, and the next closing bracket (the parent's) is one too many.
+    bool UIntElements(char const* name, Value const& array, Value const* parent, std::vector<uint32_t>& out)
+    {
+        for (Value const& item : array.items) {
+            if (item.kind == Value::Array) return UIntElements(name, item, &array, out);
+            if (!AsUnsigned(name, item, UINT32_MAX, "uint", [&](uint64_t v) { out.push_back(uint32_t(v)); })) return false;
+        }
+        if (!parent) return true;
+        m_error = LocatedMessage(parent->closeAt, "End-of-array encountered outside of an array");
+        return false;
+    }
     bool Optional(char const* name) { m_found = m_object.Find(name); return m_found != nullptr; }
     bool Required(char const* name)
     {
         if (Optional(name)) return true;
-        Format("Missing value for required field '%s.%s'", m_type, name);
+        Format(m_object.closeAt, "Missing value for required field '%s.%s'", m_type, name);
         return false;
     }
     bool WrongType(char const* name, char const* expected, Value const& v)
     {
-        Format("Expected %s for '%s.%s', got %s", expected, m_type, name, KindName(v.kind));
+        Format(v.at, "Expected %s for '%s.%s', got %s", expected, m_type, name, KindName(v.kind));
         return false;
     }
     template <typename Store> bool AsUnsigned(char const* name, Value const& v, uint64_t limit, char const* expected, Store store)
@@ -353,8 +426,12 @@ private:
         if (v.kind != Value::Integer) return WrongType(name, expected, v);
         if (v.negative || v.magnitude > limit) {
             char buf[256];
-            std::snprintf(buf, sizeof buf, "Value %s%" PRIu64 " is out of range for %s field '%s.%s'", v.negative ? "-" : "", v.magnitude, expected, m_type, name);
-            m_error = buf;
+            // the reference prints the value through a signed 64-bit integer: 2^63 and above come out negative
+            if (!v.negative && v.magnitude > uint64_t(INT64_MAX))
+                std::snprintf(buf, sizeof buf, "Value %" PRId64 " is out of range for %s field '%s.%s'", int64_t(v.magnitude), expected, m_type, name);
+            else
+                std::snprintf(buf, sizeof buf, "Value %s%" PRIu64 " is out of range for %s field '%s.%s'", v.negative ? "-" : "", v.magnitude, expected, m_type, name);
+            m_error = LocatedMessage(v.at, buf);
             return false;
         }
         store(v.magnitude);
@@ -368,14 +445,14 @@ private:
             if (v.text == candidate) return true;
             ++index;
         }
-        Format("Unknown value '%s' specified for '%s.%s'", v.text.c_str(), m_type, name);
+        Format(v.at, "Unknown value '%s' specified for '%s.%s'", v.text.c_str(), m_type, name);
         return false;
     }
-    void Format(char const* fmt, char const* a, char const* b, char const* c = nullptr, char const* d = nullptr)
+    void Format(size_t at, char const* fmt, char const* a, char const* b, char const* c = nullptr, char const* d = nullptr)
     {
         char buf[320];
         std::snprintf(buf, sizeof buf, fmt, a, b, c, d);
-        m_error = buf;
+        m_error = LocatedMessage(at, buf);
     }
 
     Value const& m_object;
@@ -411,13 +488,8 @@ bool ReadLayer(Value const& v, MlpLayer& out, std::string& error)
 bool ReadMlp(Value const& v, Mlp& out, std::string& error)
 {
     Members m(v, "MLP", error);
-    Value const* layers;
-    if (!m.Array("layers", "array", layers)) return false;
-    if (layers) for (Value const& item : layers->items) {
-        if (!m.ElementMustBeObject("layers", item)) return false;
-        out.layers.emplace_back();
-        if (!ReadLayer(item, out.layers.back(), error)) return false;
-    }
+    if (!m.ForEachObject("layers", [&](Value const& item) { out.layers.emplace_back(); return ReadLayer(item, out.layers.back(), error); }))
+        return false;
     std::optional<int> activation;
     return m.OptionalEnum("activation", activation, { "HGELUClamp" })
         && m.OptionalEnum("weightLayout", out.weightLayout, { "RowMajor", "ColumnMajor" });
@@ -426,23 +498,20 @@ bool ReadMlp(Value const& v, Mlp& out, std::string& error)
 bool ReadTexture(Value const& v, Texture& out, std::string& error)
 {
     Members m(v, "Texture", error);
-    Value const* modeBuffers;
     if (!(m.String("name", out.name) && m.UInt("firstChannel", out.firstChannel) && m.UInt("numChannels", out.numChannels)
         && m.OptionalEnum("channelFormat", out.channelFormat, NTC_FILE_CHANNEL_FORMATS)
         && m.OptionalEnum("rgbColorSpace", out.rgbColorSpace, NTC_FILE_COLOR_SPACES)
         && m.OptionalEnum("alphaColorSpace", out.alphaColorSpace, NTC_FILE_COLOR_SPACES)
-        && m.OptionalEnum("bcFormat", out.bcFormat, NTC_FILE_BC_FORMATS)
-        && m.Array("bcModeBuffers", "array", modeBuffers)))
+        && m.OptionalEnum("bcFormat", out.bcFormat, NTC_FILE_BC_FORMATS)))
         return false;
     // BC7 mode buffers: which view holds the (mode, partition) map of which colour mip
-    if (modeBuffers) for (Value const& item : modeBuffers->items) {
-        if (!m.ElementMustBeObject("bcModeBuffers", item)) return false;
+    return m.ForEachObject("bcModeBuffers", [&](Value const& item) {
         Members b(item, "BCModeBuffer", error);
         Texture::ModeBuffer ref;
         if (!(b.UInt("mipLevel", ref.mipLevel) && b.UInt("view", ref.view))) return false;
         out.bcModeBuffers.push_back(ref);
-    }
-    return true;
+        return true;
+    });
 }
 
 bool ReadColorMip(Value const& v, ColorMip& out, std::string& error)
@@ -455,31 +524,38 @@ bool ReadColorMip(Value const& v, ColorMip& out, std::string& error)
 template <typename T, typename ReadOne>
 bool ReadObjectArray(Members& parent, char const* name, std::vector<T>& out, ReadOne readOne)
 {
-    Value const* array;
-    if (!parent.Array(name, "array", array)) return false;
-    if (array) for (Value const& item : array->items) {
-        if (!parent.ElementMustBeObject(name, item)) return false;
-        out.emplace_back();
-        if (!readOne(item, out.back())) return false;
-    }
-    return true;
+    return parent.ForEachObject(name, [&](Value const& item) { out.emplace_back(); return readOne(item, out.back()); });
 }
 
 } // namespace
 
+namespace
+{
+bool ParseDocumentValues(char const* json, size_t length, Document& out, std::string& error);
+}
+
 bool ParseDocument(char const* json, size_t length, Document& out, std::string& error)
+{
+    if (ParseDocumentValues(json, length, out, error)) return true;
+    error = ExpandLocatedMessage(error, json, length);
+    return false;
+}
+
+namespace
+{
+bool ParseDocumentValues(char const* json, size_t length, Document& out, std::string& error)
 {
     Value root;
     Reader reader(json, length, error);
     if (!reader.ParseRoot(root)) return false;
-    if (root.kind != Value::Object) { error = std::string("Expected object, got ") + KindName(root.kind); return false; }
+    if (root.kind != Value::Object) { error = LocatedMessage(root.at, (std::string("Expected object, got ") + KindName(root.kind)).c_str()); return false; }
 
     Members m(root, "Document", error);
     if (!m.UInt("schemaVersion", out.schemaVersion)) return false;
     if (out.schemaVersion != kSchemaVersion) {      // src/JsonFileFormat.cpp:194-210
         char buf[128];
         std::snprintf(buf, sizeof buf, "Incompatible file schema version %u, expected %u", out.schemaVersion, kSchemaVersion);
-        error = buf;
+        error = LocatedMessage(root.Find("schemaVersion")->at, buf);
         return false;
     }
     if (!(m.UInt("width", out.width) && m.UInt("height", out.height) && m.UInt("numChannels", out.numChannels)
@@ -504,6 +580,7 @@ bool ParseDocument(char const* json, size_t length, Document& out, std::string& 
         && ReadObjectArray(m, "colorMips", out.colorMips, [&](Value const& v, ColorMip& o) { return ReadColorMip(v, o, error); })
         && ReadObjectArray(m, "views", out.views, [&](Value const& v, BufferView& o) { return ReadView(v, o, error); });
 }
+} // namespace
 
 Header DecodeHeader(unsigned char const* b)
 {

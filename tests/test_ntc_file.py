@@ -164,7 +164,9 @@ def test_random_document_damage_same_status_as_the_reference_front_end(ntc, tmp_
     """Seeded damage to the JSON document (values replaced by extremes or other types, members and elements
     removed): whenever the reference's front end (LoadFileHeadersFromStream + its document parser, built from
     the reference's own sources) refuses a file, the host layer refuses it with the same status, and nearly
-    always with the same complaint (the reference prefixes the position in the text)."""
+    always with the same complaint, position and quoted text included (a streaming reader reports the first
+    fault in the order of the text, the host layer the first in the order of its schema: with two faults in one
+    document the two may pick different ones)."""
     lib = ref_file_lib()
     if lib is None:
         pytest.skip("the reference's host-only sources are not built on this machine")
@@ -200,10 +202,10 @@ def test_random_document_damage_same_status_as_the_reference_front_end(ntc, tmp_
         if ref_status != 0:
             refused += 1
             assert status == ref_status, (i, ref_status, ref_message, status, message)
-            same_text += ref_message.endswith(message)
+            same_text += ref_message == message
         else:
             assert status != 0          # no device here: at best everything validates and the upload fails
-    assert refused >= 60 and same_text >= 0.9 * refused, (refused, same_text)
+    assert refused >= 60 and same_text >= 0.93 * refused, (refused, same_text)
 
 
 def test_semantic_errors_of_the_metadata_stage(ntc, tmp_path):
