@@ -299,8 +299,16 @@ class Members
 public:
     Members(Value const& object, char const* typeName, std::string& error) : m_object(object), m_type(typeName), m_error(error) {}
 
-    bool UInt(char const* name, uint32_t& out) { return Required(name) && AsUnsigned(name, *m_found, UINT32_MAX, "uint", [&](uint64_t v) { out = uint32_t(v); }); }
-    bool UInt64(char const* name, uint64_t& out) { return Required(name) && AsUnsigned(name, *m_found, uint64_t(INT64_MAX), "uint64", [&](uint64_t v) { out = v; }); }
+    bool UInt(char const* name, uint32_t& out) { return !Required(name) || AsUnsigned(name, *m_found, UINT32_MAX, "uint", [&](uint64_t v) { out = uint32_t(v); }); }
+    bool UInt64(char const* name, uint64_t& out) { return !Required(name) || AsUnsigned(name, *m_found, UINT64_MAX, "uint64", [&](uint64_t v) { out = v; }); }
+    // To be called when every member has been read: fails if a required one was absent.
+    bool Complete()
+    {
+        if (!m_missing) return true;
+        Format(m_object.closeAt, "Missing value for required field '%s.%s'", m_type, m_missing);
+        return false;
+    }
+    bool Has(char const* name) const { return m_object.Find(name) != nullptr; }
     bool OptionalUInt(char const* name, std::optional<uint32_t>& out)
     {
         if (!Optional(name)) return true;
@@ -309,7 +317,7 @@ public:
     bool OptionalUInt64(char const* name, std::optional<uint64_t>& out)
     {
         if (!Optional(name)) return true;
-        return AsUnsigned(name, *m_found, uint64_t(INT64_MAX), "uint64", [&](uint64_t v) { out = v; });
+        return AsUnsigned(name, *m_found, UINT64_MAX, "uint64", [&](uint64_t v) { out = v; });
     }
     bool OptionalFloat(char const* name, std::optional<float>& out)
     {
@@ -321,7 +329,7 @@ public:
     }
     bool String(char const* name, std::string& out)
     {
-        if (!Required(name)) return false;
+        if (!Required(name)) return true;
         if (m_found->kind != Value::String) return WrongType(name, "string", *m_found);
         out = m_found->text;
         return true;
@@ -329,7 +337,7 @@ public:
     // names[i] is the spelling of enum value i
     template <typename E> bool Enum(char const* name, E& out, std::initializer_list<char const*> names)
     {
-        if (!Required(name)) return false;
+        if (!Required(name)) return true;
         int index;
         if (!AsEnum(name, *m_found, names, index)) return false;
         out = E(index);
@@ -410,10 +418,12 @@ private:
         return false;
     }
     bool Optional(char const* name) { m_found = m_object.Find(name); return m_found != nullptr; }
+    // A required member that is absent is noticed where the object ends (Complete), after the members that are
+    // there have had their say: the order in which a streaming reader meets the faults of a document.
     bool Required(char const* name)
     {
         if (Optional(name)) return true;
-        Format(m_object.closeAt, "Missing value for required field '%s.%s'", m_type, name);
+        if (!m_missing) m_missing = name;
         return false;
     }
     bool WrongType(char const* name, char const* expected, Value const& v)
@@ -424,6 +434,9 @@ private:
     template <typename Store> bool AsUnsigned(char const* name, Value const& v, uint64_t limit, char const* expected, Store store)
     {
         if (v.kind != Value::Integer) return WrongType(name, expected, v);
+        // a 64-bit field takes any integer, a negative one as its two's complement: the reference's reader stores
+        // what it is given there (src/JsonSerialization.cpp:499-527); what such a value means is checked later
+        if (limit == UINT64_MAX) { store(v.negative ? uint64_t(0) - v.magnitude : v.magnitude); return true; }
         if (v.negative || v.magnitude > limit) {
             char buf[256];
             // the reference prints the value through a signed 64-bit integer: 2^63 and above come out negative
@@ -459,6 +472,7 @@ private:
     char const* m_type;
     std::string& m_error;
     Value const* m_found = nullptr;
+    char const* m_missing = nullptr;        // the first required member found absent
 };
 
 // spellings in the order of the enums (src/JsonFileFormat.cpp:25-113)
@@ -472,7 +486,7 @@ bool ReadView(Value const& v, BufferView& out, std::string& error)
     Members m(v, "BufferView", error);
     return m.UInt64("offset", out.offset) && m.UInt64("storedSize", out.storedSize)
         && m.OptionalEnum("compression", out.compression, { "None", "GDeflate" })
-        && m.OptionalUInt64("uncompressedSize", out.uncompressedSize) && m.OptionalUInt("crc32", out.crc32);
+        && m.OptionalUInt64("uncompressedSize", out.uncompressedSize) && m.OptionalUInt("crc32", out.crc32) && m.Complete();
 }
 
 bool ReadLayer(Value const& v, MlpLayer& out, std::string& error)
@@ -482,7 +496,7 @@ bool ReadLayer(Value const& v, MlpLayer& out, std::string& error)
         && m.UInt("weightView", out.weightView) && m.OptionalUInt("scaleView", out.scaleView) && m.UInt("biasView", out.biasView)
         && m.Enum("weightType", out.weightType, NTC_FILE_MLP_TYPES)
         && m.OptionalEnum("scaleType", out.scaleType, NTC_FILE_MLP_TYPES)
-        && m.Enum("biasType", out.biasType, NTC_FILE_MLP_TYPES);
+        && m.Enum("biasType", out.biasType, NTC_FILE_MLP_TYPES) && m.Complete();
 }
 
 bool ReadMlp(Value const& v, Mlp& out, std::string& error)
@@ -492,7 +506,7 @@ bool ReadMlp(Value const& v, Mlp& out, std::string& error)
         return false;
     std::optional<int> activation;
     return m.OptionalEnum("activation", activation, { "HGELUClamp" })
-        && m.OptionalEnum("weightLayout", out.weightLayout, { "RowMajor", "ColumnMajor" });
+        && m.OptionalEnum("weightLayout", out.weightLayout, { "RowMajor", "ColumnMajor" }) && m.Complete();
 }
 
 bool ReadTexture(Value const& v, Texture& out, std::string& error)
@@ -508,17 +522,17 @@ bool ReadTexture(Value const& v, Texture& out, std::string& error)
     return m.ForEachObject("bcModeBuffers", [&](Value const& item) {
         Members b(item, "BCModeBuffer", error);
         Texture::ModeBuffer ref;
-        if (!(b.UInt("mipLevel", ref.mipLevel) && b.UInt("view", ref.view))) return false;
+        if (!(b.UInt("mipLevel", ref.mipLevel) && b.UInt("view", ref.view) && b.Complete())) return false;
         out.bcModeBuffers.push_back(ref);
         return true;
-    });
+    }) && m.Complete();
 }
 
 bool ReadColorMip(Value const& v, ColorMip& out, std::string& error)
 {
     Members m(v, "ColorMip", error);
     return m.OptionalUInt("width", out.width) && m.OptionalUInt("height", out.height) && m.OptionalUInt("latentMip", out.latentMip)
-        && m.OptionalFloat("positionLod", out.positionLod) && m.OptionalFloat("positionScale", out.positionScale);
+        && m.OptionalFloat("positionLod", out.positionLod) && m.OptionalFloat("positionScale", out.positionScale) && m.Complete();
 }
 
 template <typename T, typename ReadOne>
@@ -552,7 +566,7 @@ bool ParseDocumentValues(char const* json, size_t length, Document& out, std::st
 
     Members m(root, "Document", error);
     if (!m.UInt("schemaVersion", out.schemaVersion)) return false;
-    if (out.schemaVersion != kSchemaVersion) {      // src/JsonFileFormat.cpp:194-210
+    if (m.Has("schemaVersion") && out.schemaVersion != kSchemaVersion) {      // src/JsonFileFormat.cpp:194-210
         char buf[128];
         std::snprintf(buf, sizeof buf, "Incompatible file schema version %u, expected %u", out.schemaVersion, kSchemaVersion);
         error = LocatedMessage(root.Find("schemaVersion")->at, buf);
@@ -565,20 +579,21 @@ bool ParseDocumentValues(char const* json, size_t length, Document& out, std::st
     if (!m.OptionalObject("latentShape", latentShape)) return false;
     if (latentShape) {
         Members s(*latentShape, "LatentShape", error);
-        uint32_t features;
-        if (!s.UInt("numFeatures", features)) return false;
+        uint32_t features = 0;
+        if (!(s.UInt("numFeatures", features) && s.Complete())) return false;
         out.latentFeatures = features;
     }
     return ReadObjectArray(m, "mlpVersions", out.mlpVersions, [&](Value const& v, Mlp& o) { return ReadMlp(v, o, error); })
         && ReadObjectArray(m, "textures", out.textures, [&](Value const& v, Texture& o) { return ReadTexture(v, o, error); })
         && ReadObjectArray(m, "channels", out.channelColorSpaces, [&](Value const& v, std::optional<int>& o) {
                Members c(v, "Channel", error);
-               return c.OptionalEnum("colorSpace", o, NTC_FILE_COLOR_SPACES); })
+               return c.OptionalEnum("colorSpace", o, NTC_FILE_COLOR_SPACES) && c.Complete(); })
         && ReadObjectArray(m, "latents", out.latents, [&](Value const& v, LatentImage& o) {
                Members l(v, "LatentImage", error);
-               return l.UInt("width", o.width) && l.UInt("height", o.height) && l.ArrayOfUInt("layerViews", o.layerViews); })
+               return l.UInt("width", o.width) && l.UInt("height", o.height) && l.ArrayOfUInt("layerViews", o.layerViews) && l.Complete(); })
         && ReadObjectArray(m, "colorMips", out.colorMips, [&](Value const& v, ColorMip& o) { return ReadColorMip(v, o, error); })
-        && ReadObjectArray(m, "views", out.views, [&](Value const& v, BufferView& o) { return ReadView(v, o, error); });
+        && ReadObjectArray(m, "views", out.views, [&](Value const& v, BufferView& o) { return ReadView(v, o, error); })
+        && m.Complete();
 }
 } // namespace
 
