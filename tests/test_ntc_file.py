@@ -166,7 +166,7 @@ def test_random_document_damage_same_status_as_the_reference_front_end(ntc, tmp_
     the reference's own sources) refuses a file, the host layer refuses it with the same status, and nearly
     always with the same complaint, position and quoted text included (a streaming reader reports the first
     fault in the order of the text, the host layer the first in the order of its schema: with two faults in one
-    document the two may pick different ones)."""
+    object whose members are out of schema order the two could pick different ones)."""
     lib = ref_file_lib()
     if lib is None:
         pytest.skip("the reference's host-only sources are not built on this machine")
@@ -205,7 +205,7 @@ def test_random_document_damage_same_status_as_the_reference_front_end(ntc, tmp_
             same_text += ref_message == message
         else:
             assert status != 0          # no device here: at best everything validates and the upload fails
-    assert refused >= 60 and same_text >= 0.93 * refused, (refused, same_text)
+    assert refused >= 60 and same_text >= 0.98 * refused, (refused, same_text)
 
 
 def test_semantic_errors_of_the_metadata_stage(ntc, tmp_path):
