@@ -296,8 +296,12 @@ Status LoadFileHeadersFromStream(IStream* stream, file::Document& document, uint
     uint64_t const expected = std::max(header.jsonChunkOffset + header.jsonChunkSize, header.binaryChunkOffset + header.binaryChunkSize);
     bool const wraps = header.jsonChunkOffset + header.jsonChunkSize < header.jsonChunkOffset
                     || header.binaryChunkOffset + header.binaryChunkSize < header.binaryChunkOffset;
-    if (wraps || streamSize < expected) {
+    if (streamSize < expected) {
         SetErrorMessage("File incomplete: expected at least %" PRIu64 " bytes, actual size %" PRIu64 " bytes.", expected, streamSize);
+        return Status::FileUnrecognized;
+    }
+    if (wraps) {        // a sum that wrapped slips through the test above (the reference then allocates a chunk of that size)
+        SetErrorMessage("File header describes a chunk that reaches past the 64-bit offset range.");
         return Status::FileUnrecognized;
     }
     if (!stream->Seek(header.jsonChunkOffset)) return Status::IOError;

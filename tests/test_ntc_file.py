@@ -208,6 +208,22 @@ def test_random_document_damage_same_status_as_the_reference_front_end(ntc, tmp_
     assert refused >= 60 and same_text >= 0.98 * refused, (refused, same_text)
 
 
+def test_header_sums_that_wrap_are_refused(ntc, tmp_path):
+    """Chunk offset + size past 2^64: the reference adds the two without a check, finds the (wrapped) end inside
+    the file and goes on to allocate a chunk of that size, so it is not asked here; the host layer refuses."""
+    import struct
+    case = make_case(ntc)
+    good = bytearray(file_of(case, 64, 32, 2, 8, 8))
+    for field, value in ((16, 2 ** 64 - 40), (32, 2 ** 64 - 1), (8, 2 ** 64 - 8), (24, 2 ** 64 - 64)):
+        data = bytearray(good)
+        struct.pack_into("<Q", data, field, value & (2 ** 64 - 1))
+        if field in (8, 24):                                     # an offset: give it a size that wraps the sum back into the file
+            struct.pack_into("<Q", data, field + 8, (100 - value) & (2 ** 64 - 1))
+        status, message, _ = host_load(tmp_path, bytes(data))
+        assert status == STATUS["FileUnrecognized"], (field, status, message)
+        assert "64-bit offset range" in message or "File incomplete" in message, message
+
+
 def test_semantic_errors_of_the_metadata_stage(ntc, tmp_path):
     """Rules of LoadMetadataFromStream / ValidateMLP / ValidateBufferView / LoadFromStreamPostHeader
     (src/TextureSetMetadata.cpp:434-581,978-1135, src/TextureSet.cpp:154-196); the reference needs a
