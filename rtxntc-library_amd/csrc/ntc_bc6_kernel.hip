@@ -332,7 +332,10 @@ BC6_INLINE void encode_two_subsets(V3 const (&px)[16], int pattern, Block& best)
 
 } // namespace
 
-__global__ void __launch_bounds__(128)
+// Registers capped at 168 so that three waves share a SIMD: the encoder is long chains of dependent divisions
+// and logarithms, and the other waves fill the issue slots one leaves (4096^2: 1.77 ms with one wave and 256
+// registers, 1.05 ms with two, 0.98 ms with three in spite of 175 spilled registers, 1.02 ms with four).
+__global__ void __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(3)))
 bc6_compress_kernel(BlockCompressArgs a)
 {
     int const bx = blockIdx.x * 16 + (threadIdx.x & 15), by = blockIdx.y * 8 + (threadIdx.x >> 4);
