@@ -184,6 +184,21 @@ int ntc_hip_decode(const NtcHipTextureSet* sets, int32_t numSets);
 int ntc_hip_decode_timed(const NtcHipTextureSet* sets, int32_t numSets, int32_t iterations,
                          float* outMillisecondsPerIteration);
 
+/* ntc_hip_decode for callers that cannot allocate device memory: code under HIP graph capture, serving
+ * loops and harnesses that forbid hipMalloc.  No counterpart in the reference.  ntc_hip_decode keeps its
+ * mip table in device memory that it allocates (and grows) on demand and fills through pinned staging
+ * memory; here the table lives in an array built into the library's code object, NTC_HIP_STATIC_TABLE_MIPS
+ * entries (about 34 KB, held by every GPU the library runs on until the process ends), and travels to the
+ * device as kernel arguments.  The call allocates nothing, frees nothing and copies nothing: it launches
+ * one small table-writing kernel per 16 mips and then the decode kernel of ntc_hip_decode, same results.
+ * More than NTC_HIP_STATIC_TABLE_MIPS mips over all sets of one call: NTC_HIP_ERR_INVALID_ARG.
+ * All calls on one GPU share that GPU's array, which keeps the last call's table.  Calls queued on the
+ * library stream run in order and are safe; calls that overlap on one GPU (several processes' threads
+ * are not meant: several threads of one process without the serialisation this library asks for) race.
+ * Asynchronous on the library stream. */
+#define NTC_HIP_STATIC_TABLE_MIPS 256
+int ntc_hip_decode_static(const NtcHipTextureSet* sets, int32_t numSets);
+
 /* Random-access decode: "inference on sample", NtcSampleTextureSet of
  * include/libntc/shaders/Inference.hlsli:282-357, for a list of sample points instead of a
  * shader invocation.  Query i decodes texel (floor(u*W), floor(v*H)) of colour mip `mip`

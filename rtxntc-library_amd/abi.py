@@ -146,6 +146,7 @@ EXPORTS = [
     ("ntc_hip_weight_layout", C.c_int, [C.POINTER(DecoderSpec), C.POINTER(WeightLayout)]),
     ("ntc_hip_grid_bytes", C.c_uint64, [C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     ("ntc_hip_decode", C.c_int, [C.POINTER(TextureSet), C.c_int32]),
+    ("ntc_hip_decode_static", C.c_int, [C.POINTER(TextureSet), C.c_int32]),
     ("ntc_hip_decode_timed", C.c_int, [C.POINTER(TextureSet), C.c_int32, C.c_int32, C.POINTER(C.c_float)]),
     ("ntc_hip_decode_queries", C.c_int, [C.POINTER(TextureSet), C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint64]),
     ("ntc_hip_decode_queries_timed", C.c_int, [C.POINTER(TextureSet), C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint64,

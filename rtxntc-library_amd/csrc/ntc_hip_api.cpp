@@ -4,7 +4,7 @@
 #include "../../include/ntc_hip.h"
 #include "ntc_decode_kernel.h"
 
-#include <hip/hip_runtime_api.h>
+#include <hip/hip_runtime.h>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -34,6 +34,27 @@ int hip_fail(char const* call, hipError_t err)
 }
 #define HIP_TRY(expr) do { hipError_t e_ = (expr); if (e_ != hipSuccess) return hip_fail(#expr, e_); } while (0)
 
+// Mip table of ntc_hip_decode_static: device memory that exists from the moment the library is loaded,
+// so that entry point never allocates.  Each GPU holds its own copy of the array at its own address;
+// on the host the array's NAME is only a stand-in for it, so every use below goes through the address
+// hipGetSymbolAddress returned for the device (Library::staticTable), never through the name.
+constexpr int kStaticTableEntries = NTC_HIP_STATIC_TABLE_MIPS;                      // 16 sets with a full mip chain each
+constexpr int kTableChunkEntries = 16;                         // entries one table-writing launch carries
+static __device__ __align__(256) unsigned char scratch[kStaticTableEntries * sizeof(DevMip)];
+constexpr int kMaxDevices = 64;
+void* g_staticTable[kMaxDevices] = { nullptr };                // per device: address of `scratch` there
+
+// Carries up to kTableChunkEntries table entries to the device as a kernel argument (no host-to-device
+// copy, no staging memory) and stores them with ordinary vector stores.
+struct TableChunk { DevMip entries[kTableChunkEntries]; };
+static_assert(sizeof(TableChunk) <= 3072, "a table chunk must fit the kernel-argument segment");
+static_assert(sizeof(DevMip) % 4 == 0, "table entries are copied as dwords");
+__global__ void __launch_bounds__(256) write_table_kernel(uint32_t* dst, TableChunk chunk, int dwords)
+{
+    uint32_t const* src = reinterpret_cast<uint32_t const*>(&chunk);
+    for (int i = threadIdx.x; i < dwords; i += blockDim.x) dst[i] = src[i];
+}
+
 struct Library {
     bool initialized = false;
     int device = -1;
@@ -42,6 +63,7 @@ struct Library {
     hipStream_t stream = nullptr;
     hipEvent_t evStart = nullptr, evStop = nullptr;
     DevMip* tableDev = nullptr;        // device copy of the mip table
+    DevMip* staticTable = nullptr;     // this device's `scratch` array (ntc_hip_decode_static)
     size_t tableCapacity = 0;          // entries
     std::vector<DevMip> lastTable;     // what tableDev currently holds (or will, in stream order)
     double* lossDev = nullptr;         // per-workgroup partial sums of the loss pass
@@ -396,6 +418,13 @@ int ntc_hip_init(int device)
     g_lib.device = device;
     g_lib.computeUnits = prop.multiProcessorCount;
     std::snprintf(g_lib.name, sizeof(g_lib.name), "%s (%s)", prop.name, prop.gcnArchName);
+    if (device >= kMaxDevices) { set_error("ntc_hip_init: device index %d is beyond the %d this library keeps state for.", device, kMaxDevices); return NTC_HIP_ERR_UNSUPPORTED; }
+    if (!g_staticTable[device]) {       // once per device, with that device current
+        void* address = nullptr;
+        HIP_TRY(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)));
+        g_staticTable[device] = address;
+    }
+    g_lib.staticTable = static_cast<DevMip*>(g_staticTable[device]);
     HIP_TRY(hipStreamCreate(&g_lib.stream));
     HIP_TRY(hipEventCreate(&g_lib.evStart));
     HIP_TRY(hipEventCreate(&g_lib.evStop));
@@ -523,6 +552,34 @@ int ntc_hip_decode(const NtcHipTextureSet* sets, int32_t numSets)
     if (int r = build_table(sets, numSets, table, variant, totalTiles)) return r;
     if (int r = upload_table(table)) return r;
     HIP_TRY(launch_decode(variant, g_lib.tableDev, int(table.size()), totalTiles, grid_size_for(variant, totalTiles), g_lib.stream));
+    clear_error();
+    return 0;
+}
+
+int ntc_hip_decode_static(const NtcHipTextureSet* sets, int32_t numSets)
+{
+    if (int r = require_init()) return r;
+    std::vector<DevMip> table;
+    int variant = NTC_HIP_VARIANT_NONE, totalTiles = 0;
+    if (int r = build_table(sets, numSets, table, variant, totalTiles)) return r;
+    if (table.size() > size_t(kStaticTableEntries)) {
+        set_error("ntc_hip_decode_static: %zu mips in one call; the built-in table holds %d (use ntc_hip_decode).",
+                  table.size(), kStaticTableEntries);
+        return NTC_HIP_ERR_INVALID_ARG;
+    }
+    Library& L = g_lib;
+    // The table travels as kernel arguments, a chunk per launch, into this device's built-in array.
+    // Stream order keeps a decode that still reads the previous table ahead of these stores.
+    for (size_t first = 0; first < table.size(); first += kTableChunkEntries) {
+        size_t const count = table.size() - first < size_t(kTableChunkEntries) ? table.size() - first : size_t(kTableChunkEntries);
+        TableChunk chunk;
+        std::memset(&chunk, 0, sizeof(chunk));
+        std::memcpy(chunk.entries, table.data() + first, count * sizeof(DevMip));
+        write_table_kernel<<<1, 256, 0, L.stream>>>(reinterpret_cast<uint32_t*>(L.staticTable + first), chunk,
+                                                    int(count * sizeof(DevMip) / 4));
+        HIP_TRY(hipGetLastError());
+    }
+    HIP_TRY(launch_decode(variant, L.staticTable, int(table.size()), totalTiles, grid_size_for(variant, totalTiles), L.stream));
     clear_error();
     return 0;
 }

@@ -39,6 +39,11 @@ class Device:
         arr = self.pack_sets(sets)
         abi.check(self.lib.ntc_hip_decode(arr, len(arr)))
 
+    def decode_static(self, sets):
+        """ntc_hip_decode_static: the same decode with the mip table in the library's built-in array."""
+        arr = self.pack_sets(sets)
+        abi.check(self.lib.ntc_hip_decode_static(arr, len(arr)))
+
     def decode_timed(self, sets, iterations):
         arr = self.pack_sets(sets)
         ms = C.c_float(0)
