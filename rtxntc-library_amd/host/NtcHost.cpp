@@ -1,8 +1,14 @@
-// NtcHost.cpp - host side of the decoder behind the interface of ntc_decode.h.
+// NtcHost.cpp - libntc.so: LibNTC's public interface (the unmodified <libntc/ntc.h> of the LibNTC tree,
+// included through ntc_decode.h) implemented over the gfx950 decoder.
 //
 // Counterpart of the parts of reference src/Context.cpp, src/TextureSet.cpp,
 // src/FeatureGridHost.cpp, src/FeatureGridMath.cpp and src/Errors.cpp that the decompression
-// path goes through, src/TextureSetMetadata.cpp for loading NTC files and src/Stream.cpp.  All device work is done by libntc_hip.so through include/ntc_hip.h.
+// path goes through, src/TextureSetMetadata.cpp for loading NTC files and src/Stream.cpp.  The classes
+// here derive from LibNTC's own IContext / ITextureSet (: virtual ITextureSetMetadata) / ITextureMetadata /
+// IStream, so their vtables are the ones an application compiled against that header expects; entry points
+// outside the decompression path (compression, saving files, graphics-API passes, shared textures) have
+// bodies that set the error message and return Status::NotImplemented or Unsupported.
+// All device work is done by libntc_hip.so through include/ntc_hip.h.
 #include "ntc_decode.h"
 #include "NtcFile.h"
 #include "../../include/ntc_hip.h"
@@ -23,6 +29,10 @@
 
 namespace ntc
 {
+using amd::DecoderPreset;
+using amd::ImageDesc;
+using amd::ImageDifferenceParameters;
+using amd::BlockCompressionParameters;
 
 // ---- errors: a thread-local message buffer, set on failure and cleared on success
 // (src/Errors.cpp:21-52) -------------------------------------------------------------------
@@ -50,6 +60,13 @@ Status DeviceFailure(int code)
     case NTC_HIP_ERR_NOT_INITIALIZED: return Status::CudaUnavailable;
     default: return Status::InvalidArgument;
     }
+}
+
+// Entry points of LibNTC's interface that lie outside the decompression path.
+Status NotPartOfThisLibrary(char const* function, char const* what)
+{
+    SetErrorMessage("%s: %s is not part of this build of LibNTC (MI355X decompression path only).", function, what);
+    return Status::NotImplemented;
 }
 
 enum class NetworkState { Empty, Initialized, Complete };
@@ -370,7 +387,7 @@ Status DeserializeTextureSetDesc(file::Document const& document, TextureSetDesc&
     return ValidateLatentShape(shape);
 }
 
-class TextureSet final : public ITextureSet
+class TextureSet final : public ITextureSet, public amd::ITextureSetExtension
 {
 public:
     TextureSet(Context const* context, TextureSetDesc const& desc, TextureSetFeatures const& features)
@@ -384,6 +401,7 @@ public:
         ReleaseDevice(m_staging);
         ReleaseDevice(m_latents);
         ReleaseDevice(m_weights);
+        ReleaseDevice(m_weightsFP8);
     }
 
     // src/TextureSet.cpp:81-152: even channel count, per-mip offsets, texture and staging memory
@@ -434,6 +452,34 @@ public:
     void ClearTextureMetadata() override { for (TextureMetadata* t : m_textures) DestroyObject(Allocator(), t); m_textures.clear(); }
     int GetTextureCount() const override { return int(m_textures.size()); }
     ITextureMetadata* GetTexture(int index) override { return (index >= 0 && index < int(m_textures.size())) ? m_textures[size_t(index)] : nullptr; }
+    ITextureMetadata const* GetTexture(int index) const override { return (index >= 0 && index < int(m_textures.size())) ? m_textures[size_t(index)] : nullptr; }
+
+    // ---- outside the decompression path (include/libntc/ntc.h:863-867,873-894,904-908,914-927) ----
+    uint64_t GetOutputStreamSize() override { (void)NotPartOfThisLibrary("GetOutputStreamSize", "saving texture sets"); return 0; }
+    Status SaveToStream(IStream*, LosslessCompressionStats*) override { return NotPartOfThisLibrary("SaveToStream", "saving texture sets"); }
+    Status SaveToMemory(void*, size_t*, LosslessCompressionStats*) override { return NotPartOfThisLibrary("SaveToMemory", "saving texture sets"); }
+    Status SaveToFile(char const*, LosslessCompressionStats*) override { return NotPartOfThisLibrary("SaveToFile", "saving texture sets"); }
+    Status ConfigureLosslessCompression(LosslessCompressionSettings const&) override { return NotPartOfThisLibrary("ConfigureLosslessCompression", "saving texture sets"); }
+    Status WriteChannelsFromTexture(WriteChannelsFromTextureParameters const&) override { return NotPartOfThisLibrary("WriteChannelsFromTexture", "graphics-API texture sharing"); }
+    Status ReadChannelsIntoTexture(ReadChannelsIntoTextureParameters const&) override { return NotPartOfThisLibrary("ReadChannelsIntoTexture", "graphics-API texture sharing"); }
+    Status BeginCompression(CompressionSettings const&) override { return NotPartOfThisLibrary("BeginCompression", "compression (training)"); }
+    Status RunCompressionSteps(CompressionStats*) override { return NotPartOfThisLibrary("RunCompressionSteps", "compression (training)"); }
+    Status FinalizeCompression() override { return NotPartOfThisLibrary("FinalizeCompression", "compression (training)"); }
+    void AbortCompression() override {}
+    // src/TextureSetMetadata.cpp:607-658: the conversion is for cooperative-vector layouts of a graphics device
+    Status ConvertInferenceWeights(InferenceWeightType weightType, void* commandList, void* srcBuffer, uint64_t, void* dstBuffer, uint64_t) override
+    {
+        if (!commandList) { SetErrorMessage("commandList is NULL"); return Status::InvalidArgument; }
+        if (!srcBuffer) { SetErrorMessage("srcBuffer is NULL"); return Status::InvalidArgument; }
+        if (!dstBuffer) { SetErrorMessage("dstBuffer is NULL"); return Status::InvalidArgument; }
+        if (dstBuffer == srcBuffer) { SetErrorMessage("dstBuffer must not be the same as srcBuffer"); return Status::InvalidArgument; }
+        if (weightType != InferenceWeightType::CoopVecFP8) {
+            SetErrorMessage("Unsupported weightType (%s), must be one of the CoopVec types", InferenceWeightTypeToString(weightType));
+            return Status::InvalidArgument;
+        }
+        SetErrorMessage("The requested conversion operation is not supported by the graphics device or disabled by the context settings.");
+        return Status::Unsupported;
+    }
 
     // src/TextureSetMetadata.cpp:807-832 (no output shuffling here)
     // src/TextureSet.cpp:1899-1907
@@ -535,8 +581,9 @@ public:
     }
 
     // FillColorMipConstants, GetWeightOffsets, GetPackedColorSpaces (src/TextureSetMetadata.cpp:786-858)
-    void FillInferenceConstants(int firstLatentMipInTexture, NtcTextureSetConstants& constants) const
+    void FillInferenceConstants(InferenceWeightType weightType, int firstLatentMipInTexture, NtcTextureSetConstants& constants) const
     {
+        NtcHipWeightLayout const& layout = weightType == InferenceWeightType::GenericInt8 ? m_weightLayout : m_weightLayoutFP8;
         for (int mip = 0; mip < m_desc.mips; ++mip) {
             NtcColorMipConstants& colorMip = constants.colorMips[mip];
             colorMip.neuralMip = m_neuralLodOfMip[mip] - firstLatentMipInTexture;
@@ -544,9 +591,9 @@ public:
             colorMip.positionScale = m_mips[mip].positionScale;
         }
         for (int layer = 0; layer < NTC_HIP_MLP_LAYERS; ++layer) {
-            constants.networkWeightOffsets[layer] = int(m_weightLayout.weightOffset[layer]);
-            constants.networkBiasOffsets[layer] = int(m_weightLayout.biasOffset[layer]);
-            constants.networkScaleOffsets[layer] = int(m_weightLayout.scaleOffset[layer]);
+            constants.networkWeightOffsets[layer] = int(layout.weightOffset[layer]);
+            constants.networkBiasOffsets[layer] = int(layout.biasOffset[layer]);
+            constants.networkScaleOffsets[layer] = int(layout.scaleOffset[layer]);
         }
         constants.imageWidth = m_desc.width;
         constants.imageHeight = m_desc.height;
@@ -556,12 +603,18 @@ public:
             constants.channelColorSpaces |= uint32_t(GetChannelStorageColorSpace(channel)) << (2 * channel);
     }
 
+    // src/TextureSetMetadata.cpp:288-303; no cooperative-vector layout exists without a graphics device
     bool IsInferenceWeightTypeSupported(InferenceWeightType weightType) const override
     {
-        return weightType == InferenceWeightType::GenericInt8 && !m_hostWeights.empty();
+        switch (weightType) {
+        case InferenceWeightType::GenericInt8: return !m_hostWeights.empty();
+        case InferenceWeightType::GenericFP8: return !m_hostWeightsFP8.empty();
+        default: return false;
+        }
     }
     void SetExperimentalKnob(float) override {}
 
+    // src/TextureSetMetadata.cpp:233-243: CoopVecFP8 first (never available here), then GenericInt8
     InferenceWeightType GetBestSupportedWeightType() const override
     {
         return m_hostWeights.empty() ? InferenceWeightType::Unknown : InferenceWeightType::GenericInt8;
@@ -570,12 +623,13 @@ public:
     // src/TextureSetMetadata.cpp:245-286
     Status GetInferenceWeights(InferenceWeightType weightType, void const** pOutData, size_t* pOutSize, size_t* pOutConvertedSize) override
     {
-        if (weightType != InferenceWeightType::GenericInt8 || m_hostWeights.empty()) {
+        if (!IsInferenceWeightTypeSupported(weightType)) {
             SetErrorMessage("No weights available for weightType = %s.", InferenceWeightTypeToString(weightType));
             return Status::Unsupported;
         }
-        if (pOutData) *pOutData = m_hostWeights.data();
-        if (pOutSize) *pOutSize = m_hostWeights.size();
+        std::vector<uint8_t> const& blob = weightType == InferenceWeightType::GenericInt8 ? m_hostWeights : m_hostWeightsFP8;
+        if (pOutData) *pOutData = blob.data();
+        if (pOutSize) *pOutSize = blob.size();
         if (pOutConvertedSize) *pOutConvertedSize = 0;
         ClearErrorMessage();
         return Status::Ok;
@@ -596,13 +650,17 @@ public:
                 return Status::OutOfRange;
             }
         }
-        if (!m_hostWeights.empty()) {
+        // the output layer is int8 with fp32 scale and int32 bias in both blobs (src/TextureSetMetadata.cpp:362-365)
+        for (int version = 0; version < 2; ++version) {
+            std::vector<uint8_t>& blob = version == 0 ? m_hostWeights : m_hostWeightsFP8;
+            NtcHipWeightLayout const& layout = version == 0 ? m_weightLayout : m_weightLayoutFP8;
+            if (blob.empty()) continue;
             constexpr int last = NTC_HIP_MLP_LAYERS - 1, outputs = NTC_HIP_MAX_CHANNELS;
             constexpr float constantUnit = 65536.f;          // constants are stored as bias = round(c * 2^16), scale = 2^-16
             int const inputs = m_spec.hiddenChannels[last - 1];
-            uint8_t* const weights = m_hostWeights.data() + m_weightLayout.weightOffset[last];
-            uint8_t* const scales = m_hostWeights.data() + m_weightLayout.scaleOffset[last];
-            uint8_t* const biases = m_hostWeights.data() + m_weightLayout.biasOffset[last];
+            uint8_t* const weights = blob.data() + layout.weightOffset[last];
+            uint8_t* const scales = blob.data() + layout.scaleOffset[last];
+            uint8_t* const biases = blob.data() + layout.biasOffset[last];
             std::vector<uint8_t> newWeights(size_t(inputs) * outputs, 0);
             float newScales[outputs];
             int32_t newBiases[outputs];
@@ -799,17 +857,23 @@ public:
             return Status::FileUnrecognized;
         }
 
-        // MLP data: the Int8 version, expanded to the layer sizes the decoder is built for.
-        NtcHipWeightLayout layout{};
-        if (ntc_hip_weight_layout(&spec, &layout) != 0) { SetErrorMessage("%s", ntc_hip_last_error()); return Status::InternalError; }
-        std::vector<uint8_t> blob(layout.bufferSize, 0);
-        bool haveInt8 = false;
+        // MLP data: the Int8 and the FP8 version, each expanded to the layer sizes the decoder is built for
+        // (LoadWeightsFromStream, src/TextureSetMetadata.cpp:675-784).
+        NtcHipWeightLayout layout{}, layoutFP8{};
+        NtcHipDecoderSpec specFP8 = spec;
+        specFP8.weightType = NTC_HIP_WEIGHTS_FP8;
+        if (ntc_hip_weight_layout(&spec, &layout) != 0 || ntc_hip_weight_layout(&specFP8, &layoutFP8) != 0) { SetErrorMessage("%s", ntc_hip_last_error()); return Status::InternalError; }
+        std::vector<uint8_t> blob, blobFP8;
         for (file::Mlp const& mlp : document.mlpVersions) {
-            if (mlp.layers.empty() || mlp.layers[0].weightType != file::MlpDataType::Int8) continue;
-            if (Status st = ReadMlpData(document, mlp, spec, layout, binaryChunkOffset, stream, blob); st != Status::Ok) return st;
-            haveInt8 = true;
+            if (mlp.layers.empty()) continue;
+            if (mlp.layers[0].weightType == file::MlpDataType::Int8) {
+                blob.assign(layout.bufferSize, 0);
+                if (Status st = ReadMlpData(document, mlp, spec, layout, binaryChunkOffset, stream, blob); st != Status::Ok) return st;
+            } else if (mlp.layers[0].weightType == file::MlpDataType::FloatE4M3) {
+                blobFP8.assign(layoutFP8.bufferSize, 0);
+                if (Status st = ReadMlpData(document, mlp, specFP8, layoutFP8, binaryChunkOffset, stream, blobFP8); st != Status::Ok) return st;
+            }
         }
-        if (!haveInt8) { SetErrorMessage("The file holds no Int8 version of the MLP; FP8 weights are not decoded by this library."); return Status::Unsupported; }
 
         // Latents: u16 layers, neural LOD after neural LOD (src/FeatureGridHost.cpp:140-161).
         std::vector<uint8_t> latents;
@@ -844,14 +908,23 @@ public:
         m_latentShape = LatentShape::Empty();
         if (Status st = SetLatentShape(shape); st != Status::Ok) return st;
         m_latentFootprints = std::move(footprints);     // file metadata: valid whether or not the uploads below succeed
-        if ((!metadataOnly && latents.size() != m_latentBytes) || blob.size() != m_weightLayout.bufferSize) { SetErrorMessage("Inconsistent sizes for MLP or latent data"); return Status::InternalError; }
+        if ((!metadataOnly && latents.size() != m_latentBytes) || (!blob.empty() && blob.size() != m_weightLayout.bufferSize)
+            || (!blobFP8.empty() && blobFP8.size() != m_weightLayoutFP8.bufferSize)) { SetErrorMessage("Inconsistent sizes for MLP or latent data"); return Status::InternalError; }
         if (metadataOnly) {
-            Status const st = SetWeightData(blob.data(), blob.size());      // no device behind a metadata object: the host copy is what counts
-            if (st != Status::Ok && st != Status::CudaUnavailable) return st;
+            // no device behind a metadata object: the host copies are what counts
+            for (int version = 0; version < 2; ++version) {
+                std::vector<uint8_t> const& data = version == 0 ? blob : blobFP8;
+                if (data.empty()) continue;
+                Status const st = version == 0 ? SetWeightData(data.data(), data.size()) : SetFP8WeightData(data.data(), data.size());
+                if (st != Status::Ok && st != Status::CudaUnavailable) return st;
+            }
             ClearErrorMessage();
             return Status::Ok;
         }
-        if (Status st = SetWeightData(blob.data(), blob.size()); st != Status::Ok) return st;
+        if (!blob.empty())
+            if (Status st = SetWeightData(blob.data(), blob.size()); st != Status::Ok) return st;
+        if (!blobFP8.empty())
+            if (Status st = SetFP8WeightData(blobFP8.data(), blobFP8.size()); st != Status::Ok) return st;
         if (Status st = SetLatentData(latents.data(), latents.size()); st != Status::Ok) return st;
         ClearErrorMessage();
         return Status::Ok;
@@ -882,6 +955,7 @@ public:
 
     uint64_t GetLatentDataSize() const override { return m_state == NetworkState::Empty ? 0 : m_latentBytes; }
     uint64_t GetWeightDataSize() const override { return m_state == NetworkState::Empty ? 0 : m_weightLayout.bufferSize; }
+    uint64_t GetFP8WeightDataSize() const override { return (m_state == NetworkState::Empty || m_preset != DecoderPreset::LibNTC092) ? 0 : m_weightLayoutFP8.bufferSize; }
 
     Status SetLatentData(void const* data, size_t size) override { return Upload(data, size, m_latentBytes, m_latents, "latent", m_haveLatents); }
     Status SetWeightData(void const* data, size_t size) override
@@ -896,10 +970,29 @@ public:
         return st;
     }
 
-    Status Decompress(DecompressionStats* pOutStats, bool /*useInt8Weights*/) override
+    Status SetFP8WeightData(void const* data, size_t size) override
     {
-        if (m_state != NetworkState::Complete) {
-            SetErrorMessage("Invalid network state for Decompress (%s), must be Complete.", NetworkStateToString(m_state));
+        if (m_state != NetworkState::Empty && m_preset != DecoderPreset::LibNTC092) {
+            SetErrorMessage("FP8 weights exist for the LibNTC092 decoder preset only.");
+            return Status::Unsupported;
+        }
+        Status const st = Upload(data, size, m_weightLayoutFP8.bufferSize, m_weightsFP8, "FP8 weight", m_haveWeightsFP8);
+        if (st == Status::Ok || st == Status::CudaUnavailable)
+            m_hostWeightsFP8.assign(static_cast<uint8_t const*>(data), static_cast<uint8_t const*>(data) + size);
+        return st;
+    }
+
+    // useInt8Weights selects the MLP version, as in the reference (src/TextureSet.cpp:1664-1682,1812,1826):
+    // false, the default, decodes with the FP8 version (e4m3 hidden layers), true with the Int8 version.
+    Status Decompress(DecompressionStats* pOutStats, bool useInt8Weights) override
+    {
+        bool const complete = m_haveLatents && (useInt8Weights ? m_haveWeights : m_haveWeightsFP8);
+        if (m_state == NetworkState::Empty || !complete) {
+            if (m_state != NetworkState::Empty && m_haveLatents && (m_haveWeights || m_haveWeightsFP8))
+                SetErrorMessage("The texture set holds no %s version of the MLP weights; call Decompress with useInt8Weights = %s.",
+                    useInt8Weights ? "Int8" : "FP8", useInt8Weights ? "false" : "true");
+            else
+                SetErrorMessage("Invalid network state for Decompress (%s), must be Complete.", NetworkStateToString(m_state));
             return Status::InvalidState;
         }
         if (pOutStats) { *pOutStats = DecompressionStats(); std::fill_n(pOutStats->perChannelLoss, 16, 0.f); std::fill_n(pOutStats->perMipLoss, 16, 0.f); }
@@ -917,11 +1010,13 @@ public:
 
         NtcHipTextureSet set{};
         set.spec = m_spec;
+        if (!useInt8Weights) set.spec.weightType = NTC_HIP_WEIGHTS_FP8;
         set.numMips = m_desc.mips;
         set.numChannels = m_desc.channels;
         set.outputFormat = NTC_HIP_OUT_FP16_PLANAR_PAIRS;
         set.latents = m_latents; set.latentsBytes = m_latentBytes;
-        set.weights = m_weights; set.weightsBytes = m_weightLayout.bufferSize;
+        set.weights = useInt8Weights ? m_weights : m_weightsFP8;
+        set.weightsBytes = useInt8Weights ? m_weightLayout.bufferSize : m_weightLayoutFP8.bufferSize;
         set.output = outPage; set.outputBytes = m_textureBytes;
         for (int mip = 0; mip < m_desc.mips; ++mip) {
             set.mips[mip] = m_mips[mip];
@@ -1213,11 +1308,16 @@ private:
             } else if (!readView(layer.weightView, weights, expectedInputs * expectedOutputs)) {
                 return ReadFailure("weights", l);
             }
-            float* const scales = reinterpret_cast<float*>(blob.data() + layout.scaleOffset[l]);
-            size_t const providedScales = layer.scaleView.has_value() ? layer.outputChannels : 0;
-            if (providedScales && !readView(*layer.scaleView, scales, providedScales * sizeof(float))) return ReadFailure("scales", l);
-            for (size_t i = providedScales; i < expectedOutputs; ++i) scales[i] = 1.0f;
-            if (!readView(layer.biasView, blob.data() + layout.biasOffset[l], size_t(layer.outputChannels) * sizeof(int32_t))) return ReadFailure("biases", l);
+            // e4m3 layers of the FP8 blob carry no scales and fp16 biases (src/WeightLayout.cpp:51-71)
+            bool const e4m3Layer = spec.weightType == NTC_HIP_WEIGHTS_FP8 && l < 3;
+            if (!e4m3Layer) {
+                float* const scales = reinterpret_cast<float*>(blob.data() + layout.scaleOffset[l]);
+                size_t const providedScales = layer.scaleView.has_value() ? layer.outputChannels : 0;
+                if (providedScales && !readView(*layer.scaleView, scales, providedScales * sizeof(float))) return ReadFailure("scales", l);
+                for (size_t i = providedScales; i < expectedOutputs; ++i) scales[i] = 1.0f;
+            }
+            size_t const biasElement = e4m3Layer ? sizeof(uint16_t) : sizeof(int32_t);
+            if (!readView(layer.biasView, blob.data() + layout.biasOffset[l], size_t(layer.outputChannels) * biasElement)) return ReadFailure("biases", l);
         }
         return Status::Ok;
     }
@@ -1233,10 +1333,10 @@ private:
 
     Status ResetShape()
     {
-        ReleaseDevice(m_latents); ReleaseDevice(m_weights);
-        m_hostWeights.clear();
+        ReleaseDevice(m_latents); ReleaseDevice(m_weights); ReleaseDevice(m_weightsFP8);
+        m_hostWeights.clear(); m_hostWeightsFP8.clear();
         m_latentFootprints.clear();
-        m_latentBytes = 0; m_haveLatents = m_haveWeights = false;
+        m_latentBytes = 0; m_haveLatents = m_haveWeights = m_haveWeightsFP8 = false;
         m_numNeuralLods = 0;
         m_state = NetworkState::Empty;
         ClearErrorMessage();
@@ -1254,13 +1354,21 @@ private:
             BuildPerMipGrids();
         }
         if (ntc_hip_weight_layout(&m_spec, &m_weightLayout) != 0) { SetErrorMessage("%s", ntc_hip_last_error()); return Status::InternalError; }
-        ReleaseDevice(m_latents); ReleaseDevice(m_weights);
-        m_hostWeights.clear();
+        m_weightLayoutFP8 = NtcHipWeightLayout{};
+        if (m_preset == DecoderPreset::LibNTC092) {
+            NtcHipDecoderSpec specFP8 = m_spec;
+            specFP8.weightType = NTC_HIP_WEIGHTS_FP8;
+            if (ntc_hip_weight_layout(&specFP8, &m_weightLayoutFP8) != 0) { SetErrorMessage("%s", ntc_hip_last_error()); return Status::InternalError; }
+        }
+        ReleaseDevice(m_latents); ReleaseDevice(m_weights); ReleaseDevice(m_weightsFP8);
+        m_hostWeights.clear(); m_hostWeightsFP8.clear();
         m_latentFootprints.clear();
-        m_haveLatents = m_haveWeights = false;
+        m_haveLatents = m_haveWeights = m_haveWeightsFP8 = false;
         if (m_deviceAvailable) {
             if (int r = ntc_hip_alloc(&m_latents, m_latentBytes)) return AllocationFailure(r, "latent", m_latentBytes);
             if (int r = ntc_hip_alloc(&m_weights, m_weightLayout.bufferSize)) return AllocationFailure(r, "MLP weights", m_weightLayout.bufferSize);
+            if (m_weightLayoutFP8.bufferSize)
+                if (int r = ntc_hip_alloc(&m_weightsFP8, m_weightLayoutFP8.bufferSize)) return AllocationFailure(r, "MLP weights (FP8)", m_weightLayoutFP8.bufferSize);
         }
         m_state = NetworkState::Initialized;
         ClearErrorMessage();
@@ -1321,7 +1429,7 @@ private:
         if (!m_deviceAvailable) { SetErrorMessage("No HIP device is available to this context."); return Status::CudaUnavailable; }
         if (int r = ntc_hip_upload(device, data, size)) return DeviceFailure(r);
         have = true;
-        if (m_haveLatents && m_haveWeights) m_state = NetworkState::Complete;
+        if (m_haveLatents && (m_haveWeights || m_haveWeightsFP8)) m_state = NetworkState::Complete;
         ClearErrorMessage();
         return Status::Ok;
     }
@@ -1335,7 +1443,7 @@ private:
     DecoderPreset m_preset = DecoderPreset::LibNTC092;
     NetworkState m_state = NetworkState::Empty;
     NtcHipDecoderSpec m_spec{};
-    NtcHipWeightLayout m_weightLayout{};
+    NtcHipWeightLayout m_weightLayout{}, m_weightLayoutFP8{};
     NtcHipMipDesc m_mips[NTC_HIP_MAX_MIPS]{};
     uint64_t m_mipOffsets[NTC_HIP_MAX_MIPS + 1]{};
     uint64_t m_textureBytes = 0, m_stagingBytes = 0, m_latentBytes = 0;
@@ -1346,28 +1454,33 @@ private:
     void* m_staging = nullptr;
     void* m_latents = nullptr;
     void* m_weights = nullptr;
+    void* m_weightsFP8 = nullptr;
     int m_numNeuralLods = 0;                       // shared-LOD geometry only
     int m_neuralLodOfMip[NTC_HIP_MAX_MIPS] = {};
-    std::vector<uint8_t> m_hostWeights;
+    std::vector<uint8_t> m_hostWeights, m_hostWeightsFP8;
     std::vector<BufferFootprint> m_latentFootprints;    // per (latent image, layer) of the file last loaded; empty otherwise
     ShuffleSource m_shuffle[NTC_HIP_MAX_CHANNELS];
     void ResetShuffle() { for (int ch = 0; ch < NTC_HIP_MAX_CHANNELS; ++ch) m_shuffle[ch] = ShuffleSource::Channel(ch); }
     int m_maskChannelIndex = -1;
     bool m_discardMaskedOutPixels = false;
-    bool m_deviceAvailable = false, m_haveLatents = false, m_haveWeights = false, m_decompressed = false;
+    bool m_deviceAvailable = false, m_haveLatents = false, m_haveWeights = false, m_haveWeightsFP8 = false, m_decompressed = false;
 };
 
-class Context final : public IContext
+class Context final : public IContext, public amd::IContextExtension
 {
 public:
     Context(IAllocator* allocator, bool deviceAvailable) : m_allocator(allocator), m_deviceAvailable(deviceAvailable) {}
     IAllocator* GetAllocator() const { return m_allocator; }
 
-    // src/Context.cpp:235-261 with the descriptor rules of src/TextureSetMetadata.cpp:1161-1178
+    // src/Context.cpp:177-218 with the descriptor rules of src/TextureSetMetadata.cpp:1161-1178
     Status CreateTextureSet(TextureSetDesc const& desc, TextureSetFeatures const& features, ITextureSet** pOutTextureSet) const override
     {
         if (!pOutTextureSet) { SetErrorMessage("pOutTextureSet is NULL."); return Status::InvalidArgument; }
         *pOutTextureSet = nullptr;
+        if (!m_deviceAvailable && !m_allowSetsWithoutDevice) {
+            SetErrorMessage("Cannot create a TextureSet object when no suitable CUDA device is available.");
+            return Status::CudaUnavailable;
+        }
         if (Status st = ValidateTextureSetDesc(desc); st != Status::Ok) return st;
         TextureSet* set = MakeObject<TextureSet>(m_allocator, this, desc, features);
         if (!set) { SetErrorMessage("Failed to allocate the texture set object."); return Status::OutOfMemory; }
@@ -1378,8 +1491,62 @@ public:
         return Status::Ok;
     }
 
-    void DestroyTextureSet(ITextureSet* textureSet) const override { DestroyObject(m_allocator, static_cast<TextureSet*>(textureSet)); }
-    bool IsCudaAvailable() const override { return m_deviceAvailable; }
+    void DestroyTextureSet(ITextureSet* textureSet) const override { DestroyObject(m_allocator, dynamic_cast<TextureSet*>(textureSet)); }
+    bool IsDeviceAvailable() const override { return m_deviceAvailable; }
+    void AllowTextureSetsWithoutDevice(bool allow) const override { m_allowSetsWithoutDevice = allow; }
+
+    // ---- outside the decompression path ----
+    // src/Context.cpp:380-415: sharing textures with a graphics API
+    Status RegisterSharedTexture(SharedTextureDesc const&, ISharedTexture** pOutTexture) const override
+    {
+        if (!pOutTexture) { SetErrorMessage("pOutTexture is NULL."); return Status::InvalidArgument; }
+        *pOutTexture = nullptr;
+        return NotPartOfThisLibrary("RegisterSharedTexture", "graphics-API texture sharing");
+    }
+    void ReleaseSharedTexture(ISharedTexture*) const override {}
+    // src/Context.cpp:432-451: the search over compression presets
+    Status CreateAdaptiveCompressionSession(IAdaptiveCompressionSession** pOutSession) const override
+    {
+        if (!pOutSession) { SetErrorMessage("pOutSession is NULL"); return Status::InvalidArgument; }
+        *pOutSession = nullptr;
+        return NotPartOfThisLibrary("CreateAdaptiveCompressionSession", "compression (training)");
+    }
+    void DestroyAdaptiveCompressionSession(IAdaptiveCompressionSession*) const override {}
+    // src/Context.cpp:453-464,630-643,781-794: the three passes are described for a graphics API, and a context
+    // without one answers InvalidArgument.  On the device they run through ntc::amd::IContextExtension and
+    // ITextureSet::Decompress.
+    Status MakeDecompressionComputePass(MakeDecompressionComputePassParameters const&, ComputePassDesc* pOutComputePass) const override { return NoGraphicsApi(pOutComputePass); }
+    Status MakeBlockCompressionComputePass(MakeBlockCompressionComputePassParameters const&, ComputePassDesc* pOutComputePass) const override { return NoGraphicsApi(pOutComputePass); }
+    Status MakeImageDifferenceComputePass(MakeImageDifferenceComputePassParameters const&, ComputePassDesc* pOutComputePass) const override { return NoGraphicsApi(pOutComputePass); }
+    bool IsCooperativeVectorSupported() const override { return false; }      // src/Context.cpp:924-930
+    // src/Context.cpp:952-991.  GDeflate needs the reference's external codec, which its tree does not contain.
+    Status DecompressBuffer(CompressionType compressionType, void const* pCompressedData, size_t compressedSize,
+        void* pOutDecompressedData, size_t outputBufferSize, uint32_t /*expectedCrc32*/) const override
+    {
+        switch (compressionType) {
+        case CompressionType::None:
+            if (!pCompressedData) { SetErrorMessage("pCompressedData is NULL."); return Status::InvalidArgument; }
+            if (!pOutDecompressedData) { SetErrorMessage("pOutDecompressedData is NULL."); return Status::InvalidArgument; }
+            if (outputBufferSize < compressedSize) {
+                SetErrorMessage("When compressionType == None, outputBufferSize (%zu) must be no less than compressedSize (%zu).", outputBufferSize, compressedSize);
+                return Status::InvalidArgument;
+            }
+            std::memcpy(pOutDecompressedData, pCompressedData, compressedSize);
+            ClearErrorMessage();
+            return Status::Ok;
+        case CompressionType::GDeflate:
+            SetErrorMessage("GDeflate decompression is not part of this build of LibNTC.");
+            return Status::Unsupported;
+        default:
+            SetErrorMessage("Unknown compressionType (%d).", int(compressionType));
+            return Status::InvalidArgument;
+        }
+    }
+    Status DecompressGDeflateOnVulkanGPU(void*, void const*, size_t, uint64_t, uint64_t) const override
+    {
+        SetErrorMessage("GDeflate decompression on a Vulkan device is not part of this build of LibNTC.");
+        return Status::Unsupported;
+    }
 
     Status CompressBlocks(BlockCompressionParameters const& params) const override
     {
@@ -1480,7 +1647,7 @@ public:
 
     // src/Context.cpp:296-352
     // src/Context.cpp:864-922
-    Status MakeInferenceData(ITextureSet* textureSet, InferenceWeightType weightType, int firstLatentMipInTexture,
+    Status MakeInferenceData(ITextureSetMetadata* textureSet, InferenceWeightType weightType, int firstLatentMipInTexture,
         InferenceData* pOutInferenceData) const override
     {
         if (!pOutInferenceData) { SetErrorMessage("pOutInferenceData is NULL"); return Status::InvalidArgument; }
@@ -1501,13 +1668,13 @@ public:
             return Status::Unsupported;
         }
         std::memset(pOutInferenceData, 0, sizeof(InferenceData));
-        set->FillInferenceConstants(firstLatentMipInTexture, pOutInferenceData->constants);
+        set->FillInferenceConstants(weightType, firstLatentMipInTexture, pOutInferenceData->constants);
         ClearErrorMessage();
         return Status::Ok;
     }
 
     // src/Context.cpp:263-293: everything a file says about a set, without its latents and without a device.
-    Status CreateTextureSetMetadataFromStream(IStream* inputStream, ITextureSet** pOutMetadata) const override
+    Status CreateTextureSetMetadataFromStream(IStream* inputStream, ITextureSetMetadata** pOutMetadata) const override
     {
         if (!pOutMetadata) { SetErrorMessage("pOutMetadata is NULL."); return Status::InvalidArgument; }
         *pOutMetadata = nullptr;
@@ -1527,13 +1694,17 @@ public:
         ClearErrorMessage();
         return Status::Ok;
     }
-    void DestroyTextureSetMetadata(ITextureSet* textureSetMetadata) const override { DestroyTextureSet(textureSetMetadata); }
+    void DestroyTextureSetMetadata(ITextureSetMetadata* textureSetMetadata) const override { DestroyObject(m_allocator, dynamic_cast<TextureSet*>(textureSetMetadata)); }
 
     Status CreateCompressedTextureSetFromStream(IStream* inputStream, TextureSetFeatures const& features, ITextureSet** pOutTextureSet) const override
     {
         if (!pOutTextureSet) { SetErrorMessage("pOutTextureSet is NULL."); return Status::InvalidArgument; }
         *pOutTextureSet = nullptr;
         if (!inputStream) { SetErrorMessage("inputStream is NULL."); return Status::InvalidArgument; }
+        if (!m_deviceAvailable && !m_allowSetsWithoutDevice) {   // src/Context.cpp:311-315
+            SetErrorMessage("Cannot create a TextureSet object when no suitable CUDA device is available.");
+            return Status::CudaUnavailable;
+        }
         file::Document document;
         uint64_t binaryChunkOffset = 0, binaryChunkSize = 0;
         if (Status st = LoadFileHeadersFromStream(inputStream, document, binaryChunkOffset, binaryChunkSize); st != Status::Ok) return st;
@@ -1542,7 +1713,7 @@ public:
         if (Status st = DeserializeTextureSetDesc(document, desc, shape); st != Status::Ok) return st;
         ITextureSet* created = nullptr;
         if (Status st = CreateTextureSet(desc, features, &created); st != Status::Ok) return st;
-        Status const status = static_cast<TextureSet*>(created)->LoadFromStreamPostHeader(document, binaryChunkOffset, binaryChunkSize, inputStream, shape);
+        Status const status = dynamic_cast<TextureSet*>(created)->LoadFromStreamPostHeader(document, binaryChunkOffset, binaryChunkSize, inputStream, shape);
         if (status != Status::Ok) { DestroyTextureSet(created); return status; }
         *pOutTextureSet = created;
         ClearErrorMessage();
@@ -1566,6 +1737,13 @@ public:
     }
 
 private:
+    static Status NoGraphicsApi(ComputePassDesc* pOutComputePass)
+    {
+        if (!pOutComputePass) { SetErrorMessage("pOutComputePass is NULL"); return Status::InvalidArgument; }
+        SetErrorMessage("The context was initialized with graphicsApi == None");
+        return Status::InvalidArgument;
+    }
+
     Status OpenMemoryStream(void* pData, size_t size, bool readonly, IStream** pOutStream) const
     {
         if (!pData) { SetErrorMessage("pData is NULL."); return Status::InvalidArgument; }
@@ -1578,9 +1756,18 @@ private:
 
     IAllocator* m_allocator;
     bool m_deviceAvailable;
+    mutable bool m_allowSetsWithoutDevice = false;
 };
 
 IAllocator* TextureSet::Allocator() const { return m_context->GetAllocator(); }
+
+namespace amd
+{
+extern "C" {
+ITextureSetExtension* GetTextureSetExtension(ITextureSetMetadata* textureSet) { return dynamic_cast<TextureSet*>(textureSet); }
+IContextExtension* GetContextExtension(IContext* context) { return dynamic_cast<Context*>(context); }
+}
+}
 
 extern "C" {
 
@@ -1595,6 +1782,12 @@ Status CreateContext(IContext** pOutContext, ContextParameters const& params)
         return Status::InterfaceMismatch;
     }
     if (!pOutContext) { SetErrorMessage("pOutContext is NULL."); return Status::InvalidArgument; }
+    switch (params.graphicsApi) {                            // src/PublicFunctions.cpp:118-153: built without D3D12 and Vulkan
+    case GraphicsAPI::None: break;
+    case GraphicsAPI::D3D12: SetErrorMessage("This version of LibNTC doesn't support D3D12."); return Status::NotImplemented;
+    case GraphicsAPI::Vulkan: SetErrorMessage("This version of LibNTC doesn't support Vulkan."); return Status::NotImplemented;
+    default: SetErrorMessage("Invalid graphicsApi (%d).", int(params.graphicsApi)); return Status::InvalidArgument;
+    }
     bool deviceAvailable = false;
     if (params.cudaDevice >= 0) {
         if (ntc_hip_init(params.cudaDevice) == 0) deviceAvailable = true;
@@ -1603,6 +1796,8 @@ Status CreateContext(IContext** pOutContext, ContextParameters const& params)
     IAllocator* const allocator = params.pAllocator ? params.pAllocator : &g_defaultAllocator;
     Context* context = MakeObject<Context>(allocator, allocator, deviceAvailable);
     if (!context) { SetErrorMessage("Failed to allocate the context object."); return Status::OutOfMemory; }
+    // for host-side checks by programs that know LibNTC's header only (see ntc::amd::IContextExtension)
+    if (std::getenv("LIBNTC_ALLOW_TEXTURE_SETS_WITHOUT_DEVICE")) context->AllowTextureSetsWithoutDevice(true);
     *pOutContext = context;
     return deviceAvailable ? Status::Ok : Status::CudaUnavailable;
 }
@@ -1618,15 +1813,12 @@ char const* GetLastErrorMessage() { return t_message; }
 
 // Enum names as include/libntc/ntc.h spells them; a value outside the enum is printed as its number
 // into a static buffer, as the reference does (src/PublicFunctions.cpp:177-327).
-namespace
-{
-char const* NameOrNumber(char const* const* names, int count, int value)
+static char const* NameOrNumber(char const* const* names, int count, int value)
 {
     static char number[16];
     if (value >= 0 && value < count) return names[value];
     snprintf(number, sizeof number, "%d", value);
     return number;
-}
 }
 
 char const* StatusToString(Status status)

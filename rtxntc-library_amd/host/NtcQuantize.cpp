@@ -27,6 +27,8 @@ namespace ntc
 {
 void SetQuantizeError(char const* fmt, ...);      // NtcHost.cpp: writes the thread's error message
 
+namespace amd
+{
 namespace
 {
 float RoundHalfAway(float v) { return std::round(v); }      // CUDA round(): half away from zero
@@ -226,4 +228,5 @@ extern "C" Status QuantizeNetworkFP8(FloatLayerDesc const* layers, int numLayers
     return Status::Ok;
 }
 
+} // namespace amd
 } // namespace ntc

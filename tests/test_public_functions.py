@@ -13,7 +13,7 @@ import os
 import numpy as np
 import pytest
 
-HOST_LIB = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "rtxntc-library_amd", "host", "libntc_amd.so")
+HOST_LIB = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "rtxntc-library_amd", "host", "libntc.so")
 
 
 class LatentShape(C.Structure):

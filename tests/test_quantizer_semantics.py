@@ -75,7 +75,7 @@ def test_integer_layer_equals_dequantised_float_layer(oracle, n_in, n_out, input
 import ctypes as C
 import os
 
-HOST_LIB = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "rtxntc-library_amd", "host", "libntc_amd.so")
+HOST_LIB = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "rtxntc-library_amd", "host", "libntc.so")
 
 
 class FloatLayerDesc(C.Structure):
