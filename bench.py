@@ -25,6 +25,32 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0        # MI355X dense int8 MFMA
+# Per-launch hardware counters of the decode kernel (rocprofv3 --pmc runs of this file), keyed by workload.
+COUNTERS_FILE = os.path.join(ROOT, "profiles", "decode_kernel_counters.json")
+
+
+def cpu_threads():
+    """Threads for the CPU baseline: this job's share of the host (OMP_NUM_THREADS where the box sets one
+    below the machine's core count), else every hardware thread."""
+    total = os.cpu_count() or 1
+    try:
+        share = int(os.environ.get("OMP_NUM_THREADS", "0"))
+    except ValueError:
+        share = 0
+    return (min(share, total) if share > 0 else total), total
+
+
+def measured_counters(workload, fmt_name):
+    """Counter figures for this workload from profiles/decode_kernel_counters.json, or None."""
+    try:
+        with open(COUNTERS_FILE) as f:
+            table = json.load(f)
+    except (OSError, ValueError):
+        return None
+    entry = table.get("workloads", {}).get(f"{workload}_{fmt_name}")
+    if entry:
+        entry = dict(entry, source=f"profiles/{os.path.basename(COUNTERS_FILE)} (commit {table.get('commit', '?')})")
+    return entry
 
 
 def macs(widths):
@@ -246,7 +272,7 @@ def main():
     if not args.no_cpu:
         # The CPU checker (scalar C++ restatement, oracle/ntc_oracle.cpp) on this machine's host
         # cores, over the whole workload when that fits the time budget, else over a leading part.
-        cores = min(16, os.cpu_count() or 1)
+        cores, host_cpus = cpu_threads()
         from oracle_lib import load_oracle
         orc = load_oracle()
         host = cases[0].host_set()
@@ -261,12 +287,12 @@ def main():
                 for _ in range(2):
                     total = sum(orc.ntc_oracle_decode(h.desc, cores) for h in hosts)
                     best = total if best is None else min(best, total)
-                cpu = {"value": texels / best / 1e9, "unit": "Gtexels/s", "cores": cores, "kind": "port",
+                cpu = {"value": texels / best / 1e9, "unit": "Gtexels/s", "cores": cores, "host_cpus": host_cpus, "kind": "port",
                        "sample": f"the whole workload ({texels} texels), best of 2, {best:.2f} s"}
             else:
                 rows = int(max(rows, min(mip0.height, args.cpu_seconds / (per_texel * mip0.width))))
                 t = orc.ntc_oracle_decode_rows(host.desc, 0, 0, rows, cores)
-                cpu = {"value": rows * mip0.width / t / 1e9, "unit": "Gtexels/s", "cores": cores, "kind": "port",
+                cpu = {"value": rows * mip0.width / t / 1e9, "unit": "Gtexels/s", "cores": cores, "host_cpus": host_cpus, "kind": "port",
                        "sample": f"rows 0..{rows} of mip 0 of the first set ({rows * mip0.width} texels), {t:.1f} s"}
         else:
             import numpy as np
@@ -275,10 +301,21 @@ def main():
             t0 = time.perf_counter()
             orc.ntc_oracle_decode_queries(host.desc, queries.ctypes.data, n, out.ctypes.data, cores)
             t = time.perf_counter() - t0
-            cpu = {"value": n / t / 1e9, "unit": "Gtexels/s", "cores": cores, "kind": "port",
+            cpu = {"value": n / t / 1e9, "unit": "Gtexels/s", "cores": cores, "host_cpus": host_cpus, "kind": "port",
                    "sample": f"the first {n} queries of the same list, {t:.1f} s"}
 
-    headline = wl == "cfg1" and fmt_name == "fp16" and not args.size
+    # Ceilings of the kernel, lowest first decides `bound`: HBM (algorithmic bytes), int8 MFMA (algorithmic
+    # operations), and vector-instruction issue: a CU issues 64 lane-operations per clock (no packed fp32),
+    # so the ceiling is CUs x 64 x clock / (vector operations per texel, from the SQ_INSTS_VALU counter).
+    counters = None if args.size else measured_counters(wl, fmt_name)
+    rate = texels / (kernel_ms * 1e-3) / 1e9
+    fracs = {"hbm": achieved_gbs / HBM_PEAK_GBS, "mfma": achieved_tops / INT8_PEAK_TOPS}
+    valu = {}
+    if counters and counters.get("valu_ops_per_texel"):
+        ceiling = dev.compute_units * 64 * dev.clock_ghz / counters["valu_ops_per_texel"]
+        fracs["valu"] = rate / ceiling
+        valu = {"valu_ops_per_texel": counters["valu_ops_per_texel"], "valu_clock_ghz": dev.clock_ghz,
+                "valu_ceiling_gtexels": ceiling, "valu_frac": fracs["valu"], "counters_source": counters["source"]}
     line = {
         "metric": "decoded Gtexels/s, 4096^2 16-ch set, 64-48-32 int8; % of int8-MFMA/HBM roof",
         "value": gtexels, "unit": "Gtexels/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -286,17 +323,14 @@ def main():
         "dtype": "int8", "data": "synthetic",
         "config": {"workload": f"{what}, {fmt_name} output, {texels} texels per step",
                    "device": dev.name, "compute_units": dev.compute_units},
-        "roofline": {"bound": "hbm", "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved_gbs / HBM_PEAK_GBS,
-                     # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE (profiles/), headline workload only
-                     "traffic": 766.4e6 if headline else None,
+        # achieved / peak / frac: the HBM roof (algorithmic bytes over the kernel's HIP-event time), the lower of
+        # the two roofs the metric names; `bound` names the ceiling the kernel actually runs closest to.
+        "roofline": {"bound": max(fracs, key=fracs.get), "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": fracs["hbm"],
+                     # HBM bytes per launch from the FETCH_SIZE + WRITE_SIZE counters
+                     "traffic": counters.get("hbm_traffic_bytes") if counters else None,
                      "kernel_ms": kernel_ms, "bytes_per_texel": bytes_per_texel,
-                     "mfma_achieved_tops": achieved_tops, "mfma_frac": achieved_tops / INT8_PEAK_TOPS,
-                     # what actually binds the headline kernel: vector-instruction issue.  1263 vector operations per texel
-                     # (rocprofv3 SQ_INSTS_VALU, profiles/) against 64 lanes per CU and clock at 2.4 GHz
-                     "valu_ops_per_texel": 1263 if headline else None,
-                     "valu_ceiling_gtexels": dev.compute_units * 64 * 2.4 / 1263 if headline else None,
-                     "valu_frac": (texels / (kernel_ms * 1e-3) / 1e9) / (dev.compute_units * 64 * 2.4 / 1263) if headline else None},
+                     "hbm_frac": fracs["hbm"], "mfma_achieved_tops": achieved_tops, "mfma_frac": fracs["mfma"], **valu},
         "cpu_baseline": cpu,
     }
     print(json.dumps(line))

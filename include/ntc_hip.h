@@ -156,6 +156,9 @@ void ntc_hip_shutdown(void);
 const char* ntc_hip_last_error(void);
 /* Name, compute-unit count of the initialised device. */
 int ntc_hip_device_info(char* name, size_t nameSize, int* computeUnits);
+/* Peak engine clock of the initialised device in kHz (hipDeviceProp_t::clockRate), for ceilings that are
+ * quoted per clock. */
+int ntc_hip_device_clock(int* clockRateKHz);
 
 /* ---- memory (DeviceArray<T> of src/CudaArray.h:104-181) --------------------------- */
 int ntc_hip_alloc(void** devPtr, size_t bytes);

@@ -137,6 +137,7 @@ EXPORTS = [
     ("ntc_hip_shutdown", None, []),
     ("ntc_hip_last_error", C.c_char_p, []),
     ("ntc_hip_device_info", C.c_int, [C.c_char_p, C.c_size_t, C.POINTER(C.c_int)]),
+    ("ntc_hip_device_clock", C.c_int, [C.POINTER(C.c_int)]),
     ("ntc_hip_alloc", C.c_int, [C.POINTER(C.c_void_p), C.c_size_t]),
     ("ntc_hip_free", C.c_int, [C.c_void_p]),
     ("ntc_hip_upload", C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),

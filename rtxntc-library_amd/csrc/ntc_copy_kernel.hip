@@ -187,6 +187,18 @@ read_channels_kernel(ReadChannelsArgs a)
             for (int q = 0; q < bytes / 4; ++q) reinterpret_cast<uint32_t*>(out)[q] = words[q];
         }
     }
+    // Destination channels beyond the sixteen a set can hold (a pixel stride of more than 16 components): the
+    // default value 0 in every format and colour space, dithered or not (|noise| < 1/2 step rounds to 0).
+    int const tailBegin = NTC_HIP_DEV_MAX_CHANNELS * BPC, tailEnd = a.dstChannels * BPC;      // bytes; uniform
+    if (tailEnd > tailBegin) {
+        if (((tailEnd - tailBegin) & 3) == 0 && a.vectorBytes >= 4) {
+            for (int b = tailBegin; b < tailEnd; b += 4) *reinterpret_cast<uint32_t*>(px + b) = 0u;
+        } else if constexpr (BPC == 2) {
+            for (int b = tailBegin; b < tailEnd; b += 2) *reinterpret_cast<uint16_t*>(px + b) = uint16_t(0);
+        } else {
+            for (int b = tailBegin; b < tailEnd; ++b) px[b] = uint8_t(0);
+        }
+    }
 }
 
 // ReadImageChannel, src/ImageProcessing.cu:113-139: channel k of a 16-byte piece of the pixel.

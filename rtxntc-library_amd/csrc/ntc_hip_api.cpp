@@ -59,6 +59,7 @@ struct Library {
     bool initialized = false;
     int device = -1;
     int computeUnits = 0;
+    int clockRateKHz = 0;
     char name[256] = "";
     hipStream_t stream = nullptr;
     hipEvent_t evStart = nullptr, evStop = nullptr;
@@ -271,6 +272,13 @@ int build_table(NtcHipTextureSet const* sets, int32_t numSets, std::vector<DevMi
             set_error("ntc_hip_decode: set %d: pixel stride %d is smaller than %d channels.", s, set.outPixelStride, set.numChannels);
             return NTC_HIP_ERR_INVALID_ARG;
         }
+        // the kernel addresses a texel inside its row with 32 bits
+        if (!forQueries && set.outputFormat != NTC_HIP_OUT_FP16_PLANAR_PAIRS)
+            for (int m = 0; m < set.numMips; ++m)
+                if (set.mips[m].width >= 1 && uint64_t(set.mips[m].width - 1) * uint64_t(set.outPixelStride) + uint64_t(set.numChannels * bytesPerChannel) >= (uint64_t(1) << 32)) {
+                    set_error("ntc_hip_decode: set %d mip %d: a row of %d pixels with a stride of %d bytes reaches past 4 GiB.", s, m, set.mips[m].width, set.outPixelStride);
+                    return NTC_HIP_ERR_INVALID_ARG;
+                }
         for (int m = 0; m < set.numMips; ++m) {
             NtcHipMipDesc const& d = set.mips[m];
             if (d.width < 1 || d.height < 1 || d.hrWidth < 1 || d.hrHeight < 1 || d.lrWidth < 1 || d.lrHeight < 1
@@ -417,6 +425,7 @@ int ntc_hip_init(int device)
     }
     g_lib.device = device;
     g_lib.computeUnits = prop.multiProcessorCount;
+    g_lib.clockRateKHz = prop.clockRate;
     std::snprintf(g_lib.name, sizeof(g_lib.name), "%s (%s)", prop.name, prop.gcnArchName);
     if (device >= kMaxDevices) { set_error("ntc_hip_init: device index %d is beyond the %d this library keeps state for.", device, kMaxDevices); return NTC_HIP_ERR_UNSUPPORTED; }
     if (!g_staticTable[device]) {       // once per device, with that device current
@@ -456,6 +465,14 @@ int ntc_hip_device_info(char* name, size_t nameSize, int* computeUnits)
     if (int r = require_init()) return r;
     if (name && nameSize) { std::snprintf(name, nameSize, "%s", g_lib.name); }
     if (computeUnits) *computeUnits = g_lib.computeUnits;
+    return 0;
+}
+
+int ntc_hip_device_clock(int* clockRateKHz)
+{
+    if (int r = require_init()) return r;
+    if (!clockRateKHz) { set_error("ntc_hip_device_clock: null out-pointer."); return NTC_HIP_ERR_INVALID_ARG; }
+    *clockRateKHz = g_lib.clockRateKHz;
     return 0;
 }
 

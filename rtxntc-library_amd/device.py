@@ -17,6 +17,9 @@ class Device:
         abi.check(self.lib.ntc_hip_device_info(name, 256, C.byref(cus)))
         self.name = name.value.decode()
         self.compute_units = cus.value
+        khz = C.c_int(0)
+        abi.check(self.lib.ntc_hip_device_clock(C.byref(khz)))
+        self.clock_ghz = khz.value / 1e6
 
     def alloc(self, nbytes):
         return DeviceBuffer(self, nbytes)

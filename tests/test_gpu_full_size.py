@@ -24,6 +24,29 @@ def test_headline_4096_full_mip_chain_equals_checker(ntc, device):
     assert mm is None, f"{mm[1]} bytes differ, first at {mm[0]}"
 
 
+@pytest.mark.parametrize("fmt,scale_range", [("unorm8", (-10.0, -4.0)), ("unorm8", (-17.0, -12.0)), ("fp16", (-17.0, -12.0))])
+def test_headline_4096_row_bands_equal_checker(ntc, device, oracle, fmt, scale_range):
+    """Config 1 at full size in the other output format and with scales that keep HGELU un-saturated (the
+    distribution of the configuration saturates nearly every activation, so the rounding of the requantiser
+    is exercised here): bands of rows of mip 0 at the top, middle and bottom, and every smaller mip whole."""
+    f = ntc.abi.OUT_UNORM8_PIXELS if fmt == "unorm8" else ntc.abi.OUT_FP16_PLANAR_PAIRS
+    case = cfg_case(ntc, ntc.presets.spec_cfg01(), 4096, 4096, 13, 16, f, seed=12, scale_log2_range=scale_range)
+    dset = case.device_set(device)
+    device.decode([dset])
+    device.synchronize()
+    got = case.d_output.download()
+    host = case.host_set()
+    row_bytes = 4096 * 16 * (1 if fmt == "unorm8" else 2)
+    for y0 in (0, 2044, 4096 - 20):
+        oracle.ntc_oracle_decode_rows(host.desc, 0, y0, y0 + 20, 16)
+        assert np.array_equal(host.output[y0 * row_bytes:(y0 + 20) * row_bytes], got[y0 * row_bytes:(y0 + 20) * row_bytes]), (fmt, y0)
+    for m in range(3, 13):                                      # 512^2 and smaller: quick on the CPU
+        oracle.ntc_oracle_decode_rows(host.desc, m, 0, case.mips[m].height, 16)
+    start = case.mips[3].outOffset
+    assert np.array_equal(host.output[start:], got[start:])
+    assert len(np.unique(got[:20 * row_bytes])) > 50            # a real image: not saturated to a few values
+
+
 def test_headline_4096_periodic_latents_give_periodic_output(ntc, device):
     """Wrap addressing + periodic positional encoding: latents that repeat every P cells must decode
     to an image that repeats every 2P (HR) = 4P' (LR) texels.  No checker involved; unorm8 output."""

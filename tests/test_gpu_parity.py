@@ -287,6 +287,23 @@ def test_offsets_that_would_wrap_are_rejected(ntc, device):
         assert e.value.code == ntc.abi.ERR_INVALID_ARG, field
 
 
+def test_pixel_rows_beyond_4_gib_are_rejected(ntc, device):
+    """A texel's place inside its row is a 32-bit offset in the kernel: a width and pixel stride whose product
+    passes 2^32 must be refused, not wrapped."""
+    case = cfg_case(ntc, ntc.presets.spec_cfg01(), 8192, 4, 1, 8, ntc.abi.OUT_UNORM8_PIXELS, seed=1)
+    dset = case.device_set(device)
+    dset.outPixelStride = 1 << 19                         # 8191 * 2^19 + 8 = 4 GiB - 2^19 + 8: still fine, were the buffer that large
+    dset.mips[0].outRowPitch = 8192 << 19
+    with pytest.raises(ntc.NtcHipError) as e:
+        device.decode([dset])
+    assert e.value.code == ntc.abi.ERR_INVALID_ARG and "output buffer" in e.value.message
+    dset.outPixelStride = 1 << 20                         # 8191 * 2^20 passes 2^32
+    dset.mips[0].outRowPitch = 8192 << 20
+    with pytest.raises(ntc.NtcHipError) as e:
+        device.decode([dset])
+    assert e.value.code == ntc.abi.ERR_INVALID_ARG and "4 GiB" in e.value.message
+
+
 def test_fill_any_alignment(ntc, device):
     """ntc_hip_memset is a kernel: every alignment of start and end, bytes outside untouched."""
     rng = np.random.default_rng(5)

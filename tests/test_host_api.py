@@ -89,7 +89,8 @@ def test_gpu_read_channels_all_formats(ntc, device, oracle, fmt):
     planar = random_planar(rng, w, h, C_)
     d_src = device.upload(planar)
     bpc = {1: 1, 2: 2, 3: 2, 4: 4, 5: 4}[fmt]
-    for first, count, dst_channels in ((0, 16, 16), (5, 3, 4), (15, 1, 1), (2, 7, 7)):
+    # (the last two: a pixel stride of more than 16 components - every one of them is written, src/ImageProcessing.cu:237-240)
+    for first, count, dst_channels in ((0, 16, 16), (5, 3, 4), (15, 1, 1), (2, 7, 7), (0, 16, 21), (3, 2, 64)):
         stride = dst_channels * bpc
         pitch = w * stride + 4 * bpc
         d_dst = device.alloc(h * pitch)
