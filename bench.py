@@ -158,7 +158,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=30)   # the GPU clock takes ~30 launches to settle
-    ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4", "ref092", "read", "write", "loss", "bc1", "bc3", "bc5", "bc6", "bc7", "bc7m"])
+    ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4", "ref092", "ref092fp8", "read", "write", "loss", "bc1", "bc3", "bc5", "bc6", "bc7", "bc7m"])
     ap.add_argument("--size", type=int, default=0, help="override the texture size of the workload")
     ap.add_argument("--format", choices=["fp16", "unorm8"], default=None)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="time budget of the CPU-baseline sample")
@@ -208,6 +208,15 @@ def main():
         cases = [ref_case(ntc, P.spec_ref092(16), size, size, P.full_mip_count(size, size), 2, 16, fmt, seed=5)]
         widths, channels, latent_b = (46, 64, 48, 32, 16), 16, 44738560 / 22369621.0
         what = f"LibNTC 0.9.2 geometry: {size}x{size}, full mip chain, grid scale 2, 16 features, MLP 48(46)-64-48-32-16 int8"
+    elif wl == "ref092fp8":
+        from cases import Case
+        size = args.size or 4096
+        spec = P.spec_ref092_fp8(16)
+        mips, latent_bytes = P.mips_ref092(spec, size, size, P.full_mip_count(size, size), 2)
+        cases = [Case(ntc, spec, mips, latent_bytes, 16, fmt, seed=5, weights=ntc.synth.make_fp8_weights(spec, 6))]
+        widths, channels, latent_b = (46, 64, 48, 32, 16), 16, 44738560 / 22369621.0
+        what = (f"LibNTC 0.9.2 geometry with the FP8 network: {size}x{size}, full mip chain, grid scale 2, 16 features, "
+                "MLP 48(46)-64-48-32-16, e4m3 hidden layers (GenericFP8 blob)")
     else:
         size = args.size or 8192
         cases = [cfg_case(ntc, P.spec_cfg01(), size, size, P.full_mip_count(size, size), 16, fmt, seed=4)]

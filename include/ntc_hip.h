@@ -61,8 +61,12 @@ typedef enum NtcHipGridMode {
 typedef enum NtcHipWeightType {
     NTC_HIP_WEIGHTS_INT8 = 0, /* GenericInt8 blob, src/WeightLayout.cpp:42-49,184-247 */
     /* The reference's GenericFP8 blob (src/WeightLayout.cpp:51-71,249-262): e4m3 matrices and fp16
-     * biases for the hidden layers, int8 + fp32 scale + int32 bias for the output layer.  Only the
-     * layout helper knows it; no decode kernel consumes it. */
+     * biases for the hidden layers, int8 + fp32 scale + int32 bias for the output layer - the FP8
+     * version of the network that ITextureSet::Decompress uses unless asked for Int8 weights
+     * (src/TextureSet.cpp:1812,1826), evaluated as include/libntc/shaders/InferenceCoopVec.hlsli:22-124,
+     * 127-160,235-398 describes: e4m3-rounded fp16 inputs and activations, exact dot products, fp16 bias
+     * and HGELU-clamp activation, int8 output layer.  Decoded by ntc_hip_decode for the LibNTC 0.9.2
+     * geometry (both grids bilinear 4-bit with 4 / 8 / 12 / 16 features, MLP 48-64-48-32-16). */
     NTC_HIP_WEIGHTS_FP8  = 1,
     /* Laid out exactly like NTC_HIP_WEIGHTS_INT8, but the bytes of the three hidden-layer matrices
      * are OCP e4m3 values w.  A hidden layer computes acc = bias_i32 + sum(512*w * in) exactly in
@@ -377,6 +381,12 @@ int ntc_hip_selftest_mfma(const int8_t* a16x64, const int8_t* b64x16, int32_t* d
  * floats, depth 16 or 32.  With integer-valued operands of that size the result must be the
  * exact integer, whatever order the hardware adds in.  No reference counterpart; used by the tests. */
 int ntc_hip_selftest_mfma_f16(const uint16_t* aHalves, const uint16_t* bHalves, const float* c16x16, float* d16x16, int32_t depth);
+
+/* The fp16 primitives of the FP8 network's activation stage applied to `count` halves (at most 2^20):
+ * out[0..count) the HGELU-clamp of each input, out[count..2 count) each input rounded to e4m3 (as a half),
+ * out[2 count..3 count) 80 x - 113 rounded to an integer (as a half; defined for inputs in [-0.1875, 3]).
+ * No reference counterpart; used by the tests. */
+int ntc_hip_selftest_fp8_activation(const uint16_t* halves, int32_t count, uint16_t* out);
 
 #ifdef __cplusplus
 }

@@ -1,5 +1,5 @@
 /*
- * ntc_oracle.cpp - CPU restatement of LibNTC's int8 texture-set decode arithmetic.
+ * ntc_oracle.cpp - CPU restatement of LibNTC's texture-set decode arithmetic (Int8 and FP8 networks).
  *
  * TEST INFRASTRUCTURE ONLY.  This file is the checker the HIP decoder is compared
  * against; nothing in the shipped library links, loads or calls it.  Only tests, the
@@ -86,6 +86,14 @@
  *                            path reproduces the full search's blocks
  *                            (tests/test_block_compress_bc7.py).  Float operation order as for
  *                            BC1: parity with the reference's exact blocks is unpinned.
+ *   FP8 network              parity with the reference's own bits is UNPINNED by construction: its e4m3
+ *   (decode_texel_fp8,       matrix-vector products are left to the graphics driver (cooperative vectors) or run
+ *   layer_e4m3, hgelu_half,  as FP16 WMMA with half accumulation in CUDA.  The deterministic reading implemented
+ *   half_to_e4m3, inputs)    here is pinned by: brute force over the 127 non-negative e4m3 values for every half;
+ *                            numpy's IEEE double -> half conversion; the fp16 activation in numpy float64 with one
+ *                            rounding per operation over every half plus closed forms; exact rational dot products
+ *                            (python integers) for the layer; closed forms of the input vector; an independent
+ *                            numpy restatement end to end (tests/test_fp8_network.py, tests/np_decoder.py).
  *   The exact bits of the reference's FP16-WMMA CUDA kernel (half accumulation order,
  *   --use_fast_math) and of a hardware bilinear sampler are NOT reproduced: parity unpinned
  *   for those two, by construction; the integer contract of Inference.hlsli is what is pinned.
@@ -370,12 +378,118 @@ void layer_fp8_weights(int32_t const* W512 /* 512*w, decoded once per set */, fl
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// The FP8 network: NtcSampleTextureSet_CoopVec_FP8 and what it calls
+// (include/libntc/shaders/InferenceCoopVec.hlsli:22-124,127-160,235-309,312-398), with the weight blob of
+// src/WeightLayout.cpp:51-71 (e4m3 matrices and fp16 biases for the three hidden layers, the int8 output
+// layer).  The shader hands e4m3 matrix-vector products to the driver ("cooperative vectors"): rounding of
+// the inputs to e4m3, accumulation order and precision, fusion inside the fp16 activation are NOT defined
+// by the reference - parity with any particular driver is unpinned by construction.  What is implemented
+// here is one deterministic reading, stated operation by operation:
+//   inputs   latent feature: t = the fp32 bilinear filter of the codes (the same chain as the int8
+//            contract), v = fma(t, 2/15, -1) (the sampler's t/15, then *2 - 1 of hlsli:40), half(v);
+//            positional encoding and lod: half of the fp32 values of Inference.hlsli:89-120; every input
+//            is then rounded to e4m3 (round-to-nearest-even, the grid of src/tin/tin_activation.h:44-81
+//            including its subnormals, saturating at 448), which is how the driver reads an fp16 vector
+//            as FloatE4M3 (hlsli:244,266);
+//   layer    the exact dot product of e4m3 weights and e4m3 inputs is accumulated in three parts by the
+//            bits of |512 w| (bits 14.., 7..13, 0..6: each part's sum is exactly representable in fp32),
+//            r = ((s2 + s1) + s0) + float(bias_fp16) with three fp32 additions, x = half(r);
+//   HGELU    in fp16 as NtcHGELUClamp_Forward_CoopVec writes it: t = sat(fma(x, half(1/3), 1/2)) (one
+//            rounding), y = half(clamp(x, -3, 3) * t) - the lower clamp changes nothing where t > 0 and
+//            keeps -inf * 0 out; a NaN x gives 0;
+//   between  hidden layers: y rounded to e4m3; after the last one: q = rne(80 y - 113), the int8 input of
+//            the output layer (hlsli:143-148,333-334), computed exactly and rounded once;
+//   output   acc = bias_i32 + sum W_i8 q exactly, o = float(acc) * scale (hlsli:333-345).
+// ---------------------------------------------------------------------------------------
+uint16_t double_to_half_rne(double d)                        // one rounding, ties to even, overflow to infinity
+{
+    if (std::isnan(d)) return 0x7e00;
+    uint16_t const sign = std::signbit(d) ? 0x8000 : 0;
+    double const a = std::fabs(d);
+    if (a >= 65520.0) return uint16_t(sign | 0x7c00);
+    if (a == 0.0) return sign;
+    int e;
+    (void)std::frexp(a, &e);                                 // a = m * 2^e, m in [0.5, 1)
+    int const exponent = std::max(e - 1, -14);               // of the half's binade (subnormals share -14)
+    double const quantum = std::ldexp(1.0, exponent - 10);
+    double const q = std::nearbyint(a / quantum);            // exact division, default rounding = nearest-even
+    return uint16_t(sign | float_to_half_rne(float(q * quantum)));       // q * quantum has at most 12 bits: exact
+}
+inline double half_value(uint16_t h) { return double(half_to_float(h)); }
+uint16_t half_fma(uint16_t a, uint16_t b, uint16_t c) { return double_to_half_rne(half_value(a) * half_value(b) + half_value(c)); }   // exact in double
+
+// IEEE half -> the integer 512 * (nearest e4m3 value): round to nearest, ties to even, on the e4m3 grid
+// (3 mantissa bits from 2^-6 up, steps of 2^-9 below), magnitudes from 464 up (and infinities) saturate
+// at 448; NaN gives 0.
+int32_t half_to_e4m3_times_512(uint16_t h)
+{
+    if ((h & 0x7fffu) > 0x7c00u) return 0;
+    double const a = std::fabs(half_value(h));
+    double r;
+    if (a >= 464.0) r = 448.0;                               // 464 = midpoint of 448 and the absent 480: ties go to the even 448... and beyond saturates
+    else {
+        int e;
+        (void)std::frexp(a, &e);
+        int const exponent = a == 0.0 ? -6 : std::max(e - 1, -6);
+        double const quantum = std::ldexp(1.0, exponent - 3);
+        r = std::min(std::nearbyint(a / quantum) * quantum, 448.0);
+    }
+    int32_t const v = int32_t(r * 512.0);
+    return (h & 0x8000u) ? -v : v;
+}
+
+constexpr uint16_t kHalfThird = 0x3555, kHalfOneHalf = 0x3800;     // half(1/3) = 0.33325195, 1/2
+
+// x (fp16 layer output) -> y (fp16): NtcHGELUClamp_Forward_CoopVec, hlsli:150-153
+uint16_t hgelu_half(uint16_t x)
+{
+    if ((x & 0x7fffu) > 0x7c00u) return 0;
+    double t = half_value(half_fma(x, kHalfThird, kHalfOneHalf));      // +-inf stay +-inf, then saturate
+    t = std::min(std::max(t, 0.0), 1.0);
+    double const xc = std::min(std::max(half_value(x), -3.0), 3.0);
+    return double_to_half_rne(xc * t);
+}
+
+struct Fp8Layers {                                           // decoded once per set
+    std::vector<int32_t> w512;                               // 512 * w of the three e4m3 matrices, blob order
+    void prepare(NtcHipTextureSet const& set, NtcHipWeightLayout const& layout)
+    {
+        uint8_t const* blob = static_cast<uint8_t const*>(set.weights);
+        w512.resize(layout.weightOffset[NTC_HIP_MLP_LAYERS - 1]);
+        for (size_t i = 0; i < w512.size(); ++i) w512[i] = e4m3_times_512(blob[i]);
+    }
+};
+
+// One e4m3 layer: inputs a512 = 512 * a, result the fp16 layer output x (before the activation).
+void layer_e4m3(int32_t const* W512, uint16_t const* biasHalf, int in, int out, int32_t const* a512, uint16_t* x)
+{
+    for (int c = 0; c < out; ++c) {
+        int64_t s[3] = { 0, 0, 0 };
+        for (int k = 0; k < in; ++k) {
+            int32_t const w = W512[c * in + k];
+            int64_t const mag = w < 0 ? -int64_t(w) : w, sign = w < 0 ? -1 : 1;
+            s[0] += sign * (mag & 127) * a512[k];
+            s[1] += sign * ((mag >> 7) & 127) * a512[k];
+            s[2] += sign * (mag >> 14) * a512[k];
+        }
+        // each part is an integer below 2^24 in units of 2^-18, 2^-11 and 2^-4: exact in fp32
+        float const f0 = float(s[0]) * 0x1p-18f, f1 = float(s[1]) * 0x1p-11f, f2 = float(s[2]) * 0x1p-4f;
+        float r = f2 + f1;
+        r = r + f0;
+        r = r + half_to_float(biasHalf[c]);
+        x[c] = float_to_half_rne(r);
+    }
+}
+
 struct SetView {
     NtcHipTextureSet const* set;
     NtcHipWeightLayout layout;
     std::vector<int32_t> fp8Weights;       // 512*w of every e4m3 weight, blob order (hidden layers)
+    Fp8Layers fp8;
     void prepare()
     {
+        if (set->spec.weightType == NTC_HIP_WEIGHTS_FP8) fp8.prepare(*set, layout);
         if (set->spec.weightType != NTC_HIP_WEIGHTS_FP8_SCALED) return;
         uint8_t const* blob = static_cast<uint8_t const*>(set->weights);
         fp8Weights.resize(layout.weightOffset[NTC_HIP_MLP_LAYERS - 1]);
@@ -403,7 +517,74 @@ void prepare_inputs(NtcHipTextureSet const& set, NtcHipMipDesc const& mip, int x
 
 inline bool decodable(NtcHipDecoderSpec const& s)
 {
+    if (s.weightType == NTC_HIP_WEIGHTS_FP8)                 // the FP8 network exists for bilinear 4-bit grids (the reference's geometry)
+        return s.hrMode == NTC_HIP_GRID_BILINEAR && s.lrMode == NTC_HIP_GRID_BILINEAR && s.hrBits == 4 && s.lrBits == 4;
     return s.weightType == NTC_HIP_WEIGHTS_INT8 || s.weightType == NTC_HIP_WEIGHTS_FP8_SCALED;
+}
+
+// The input vector of the FP8 network as 512 * (e4m3 value) per input: NtcPrepareNetworkInputsInternal_FP16,
+// InferenceCoopVec.hlsli:77-107, then the e4m3 reading of the vector.
+void prepare_inputs_fp8(NtcHipTextureSet const& set, NtcHipMipDesc const& mip, int x, int y, int32_t* in512, uint16_t* halvesOut)
+{
+    NtcHipDecoderSpec const& s = set.spec;
+    uint16_t h[NTC_HIP_MAX_LAYER_WIDTH] = {};
+    float const u = (float(x) + 0.5f) / float(mip.width);
+    float const v = (float(y) + 0.5f) / float(mip.height);
+    uint8_t const* lat = static_cast<uint8_t const*>(set.latents);
+    Grid const grids[2] = {
+        { reinterpret_cast<uint16_t const*>(lat + mip.hrOffset), mip.hrWidth, mip.hrHeight, s.hrFeatures, s.hrBits },
+        { reinterpret_cast<uint16_t const*>(lat + mip.lrOffset), mip.lrWidth, mip.lrHeight, s.lrFeatures, s.lrBits } };
+    int const base[2] = { 0, s.hrFeatureSlots };
+    for (int g = 0; g < 2; ++g) {
+        Footprint const fp = bilinear_footprint(u, v, grids[g].width, grids[g].height);
+        for (int f = 0; f < grids[g].features; ++f) {
+            float t = fp.w00 * float(grids[g].fetch(fp.x0, fp.y0, f));
+            t = std::fmaf(fp.w10, float(grids[g].fetch(fp.x1, fp.y0, f)), t);
+            t = std::fmaf(fp.w01, float(grids[g].fetch(fp.x0, fp.y1, f)), t);
+            t = std::fmaf(fp.w11, float(grids[g].fetch(fp.x1, fp.y1, f)), t);
+            h[base[g] + f] = float_to_half_rne(std::fmaf(t, 0.13333334f, -1.f));     // hlsli:38-45
+        }
+    }
+    int idx = s.hrFeatureSlots + s.lrFeatureSlots;           // hlsli:51-75
+    float px = float(x) * mip.positionScale, py = float(y) * mip.positionScale;
+    for (int w = 0; w < s.posEncWaves; ++w) {
+        h[idx++] = float_to_half_rne(frac_hlsl(px) * 2.f - 1.f);
+        h[idx++] = float_to_half_rne(frac_hlsl(py) * 2.f - 1.f);
+        h[idx++] = float_to_half_rne(frac_hlsl(px + 0.25f) * 2.f - 1.f);
+        h[idx++] = float_to_half_rne(frac_hlsl(py + 0.25f) * 2.f - 1.f);
+        px *= 2.f; py *= 2.f;
+    }
+    for (int i = 0; i < s.lodInputs; ++i) h[idx++] = float_to_half_rne(mip.positionLod);
+    for (int k = 0; k < s.inputChannels; ++k) in512[k] = half_to_e4m3_times_512(h[k]);
+    if (halvesOut) std::memcpy(halvesOut, h, size_t(s.inputChannels) * 2);
+}
+
+// One texel through the FP8 network: NtcEvaluateMLP_CoopVec_FP8, InferenceCoopVec.hlsli:348-398.
+void decode_texel_fp8(SetView const& sv, NtcHipMipDesc const& mip, int x, int y, float* outputs)
+{
+    NtcHipTextureSet const& set = *sv.set;
+    NtcHipDecoderSpec const& s = set.spec;
+    uint8_t const* blob = static_cast<uint8_t const*>(set.weights);
+    int32_t a512[NTC_HIP_MAX_LAYER_WIDTH];
+    prepare_inputs_fp8(set, mip, x, y, a512, nullptr);
+    uint16_t xh[NTC_HIP_MAX_LAYER_WIDTH];
+    int8_t q[NTC_HIP_MAX_LAYER_WIDTH];
+    constexpr int last = NTC_HIP_MLP_LAYERS - 1;
+    for (int l = 0; l < last; ++l) {
+        int const in = layer_inputs(s, l), out = layer_outputs(s, l);
+        layer_e4m3(sv.fp8.w512.data() + sv.layout.weightOffset[l], reinterpret_cast<uint16_t const*>(blob + sv.layout.biasOffset[l]), in, out, a512, xh);
+        for (int c = 0; c < out; ++c) {
+            uint16_t const yh = hgelu_half(xh[c]);
+            if (l < last - 1) a512[c] = half_to_e4m3_times_512(yh);
+            else q[c] = int8_t(int(std::nearbyint(80.0 * half_value(yh) - 113.0)));    // hlsli:155-158: y*80 + (-113), in [-128, 127]
+        }
+    }
+    float r[NTC_HIP_MAX_LAYER_WIDTH];
+    layer_int8(reinterpret_cast<int8_t const*>(blob + sv.layout.weightOffset[last]),
+               reinterpret_cast<float const*>(blob + sv.layout.scaleOffset[last]),
+               reinterpret_cast<int32_t const*>(blob + sv.layout.biasOffset[last]),
+               layer_inputs(s, last), layer_outputs(s, last), q, r);
+    for (int c = 0; c < s.outputChannels; ++c) outputs[c] = r[c];
 }
 
 // One texel through the int8 network: NtcSampleTextureSet, Inference.hlsli:282-357.
@@ -432,6 +613,14 @@ void decode_texel_int8(SetView const& sv, NtcHipMipDesc const& mip, int x, int y
         for (int c = 0; c < out; ++c) act[c] = int8_t(hgelu_quantize(r[c]));   // NtcPackInt8x4: & 0xff
     }
     for (int c = 0; c < s.outputChannels; ++c) outputs[c] = r[c];
+}
+
+// One texel through the network the set's weight type selects.  inputsOut (optional) receives the int8
+// input vector; the FP8 network has none.
+void decode_texel(SetView const& sv, NtcHipMipDesc const& mip, int x, int y, float* outputs, int8_t* inputsOut)
+{
+    if (sv.set->spec.weightType == NTC_HIP_WEIGHTS_FP8) decode_texel_fp8(sv, mip, x, y, outputs);
+    else decode_texel_int8(sv, mip, x, y, outputs, inputsOut);
 }
 
 // Output addressing.  Planar pairs: GetPixelBaseAddress/GetChannelAddress,
@@ -510,10 +699,27 @@ void ntc_oracle_bilinear_footprint(float u, float v, int gw, int gh, int* xy, fl
 // Inputs (int8, spec.inputChannels of them) and raw fp32 outputs of one texel.
 int ntc_oracle_decode_texel(const NtcHipTextureSet* set, int mip, int x, int y, float* outputs, int8_t* inputs)
 {
-    SetView sv{ set, {}, {} };
+    SetView sv{ set, {}, {}, {} };
     if (!decodable(set->spec) || !weight_layout(set->spec, sv.layout)) return -1;
     sv.prepare();
-    decode_texel_int8(sv, set->mips[mip], x, y, outputs, inputs);
+    decode_texel(sv, set->mips[mip], x, y, outputs, inputs);
+    return 0;
+}
+
+// Pieces of the FP8 network, for the tests that pin them.
+int32_t  ntc_oracle_half_to_e4m3_times_512(uint16_t h) { return half_to_e4m3_times_512(h); }
+uint16_t ntc_oracle_hgelu_half(uint16_t x) { return hgelu_half(x); }
+uint16_t ntc_oracle_double_to_half(double d) { return double_to_half_rne(d); }
+void     ntc_oracle_layer_e4m3(const uint8_t* weightsE4M3, const uint16_t* biasHalf, int in, int out, const int32_t* a512, uint16_t* x)
+{
+    std::vector<int32_t> w512(size_t(in) * size_t(out));
+    for (size_t i = 0; i < w512.size(); ++i) w512[i] = e4m3_times_512(weightsE4M3[i]);
+    layer_e4m3(w512.data(), biasHalf, in, out, a512, x);
+}
+int ntc_oracle_fp8_inputs(const NtcHipTextureSet* set, int mip, int x, int y, uint16_t* halves, int32_t* in512)
+{
+    if (!set || mip < 0 || mip >= set->numMips || set->spec.weightType != NTC_HIP_WEIGHTS_FP8 || !decodable(set->spec)) return -1;
+    prepare_inputs_fp8(*set, set->mips[mip], x, y, in512, halves);
     return 0;
 }
 
@@ -2178,7 +2384,7 @@ int ntc_oracle_block_compress(const NtcHipBlockCompress* p)
 int ntc_oracle_decode_queries(const NtcHipTextureSet* set, const float* uvmip /* 3 words per query: u, v, int32 mip */,
                               uint64_t numQueries, uint16_t* out, int threads)
 {
-    SetView sv{ set, {}, {} };
+    SetView sv{ set, {}, {}, {} };
     if (!decodable(set->spec) || !weight_layout(set->spec, sv.layout)) return -1;
     sv.prepare();
     if (threads < 1) threads = 1;
@@ -2196,7 +2402,7 @@ int ntc_oracle_decode_queries(const NtcHipTextureSet* set, const float* uvmip /*
                 int x = int(std::floor(u * float(mip.width))), y = int(std::floor(v * float(mip.height)));
                 x = std::max(0, std::min(x, mip.width - 1));
                 y = std::max(0, std::min(y, mip.height - 1));
-                decode_texel_int8(sv, mip, x, y, o, nullptr);
+                decode_texel(sv, mip, x, y, o, nullptr);
                 for (int c = 0; c < 16; ++c) out[16 * q + uint64_t(c)] = output_to_half(o[c]);
             }
         }
@@ -2211,7 +2417,7 @@ int ntc_oracle_decode_queries(const NtcHipTextureSet* set, const float* uvmip /*
 // out in bands to `threads` workers.  Returns seconds spent decoding (steady clock), < 0 on error.
 double ntc_oracle_decode(const NtcHipTextureSet* set, int threads)
 {
-    SetView sv{ set, {}, {} };
+    SetView sv{ set, {}, {}, {} };
     if (!decodable(set->spec) || !weight_layout(set->spec, sv.layout)) return -1.0;
     sv.prepare();
     if (threads < 1) threads = 1;
@@ -2228,7 +2434,7 @@ double ntc_oracle_decode(const NtcHipTextureSet* set, int threads)
                 int const y1 = std::min(mip.height, y0 + band);
                 for (int y = y0; y < y1; ++y)
                     for (int x = 0; x < mip.width; ++x) {
-                        decode_texel_int8(sv, mip, x, y, o, nullptr);
+                        decode_texel(sv, mip, x, y, o, nullptr);
                         store_texel(*set, mip, x, y, o);
                     }
             }
@@ -2247,7 +2453,7 @@ double ntc_oracle_decode(const NtcHipTextureSet* set, int threads)
 // Decodes only rows [y0, y1) of mip `mipIndex` (bounded CPU-baseline samples).
 double ntc_oracle_decode_rows(const NtcHipTextureSet* set, int mipIndex, int y0, int y1, int threads)
 {
-    SetView sv{ set, {}, {} };
+    SetView sv{ set, {}, {}, {} };
     if (!decodable(set->spec) || !weight_layout(set->spec, sv.layout)) return -1.0;
     sv.prepare();
     NtcHipMipDesc const& mip = set->mips[mipIndex];
@@ -2261,7 +2467,7 @@ double ntc_oracle_decode_rows(const NtcHipTextureSet* set, int mipIndex, int y0,
             int const y = nextRow.fetch_add(1);
             if (y >= y1) break;
             for (int x = 0; x < mip.width; ++x) {
-                decode_texel_int8(sv, mip, x, y, o, nullptr);
+                decode_texel(sv, mip, x, y, o, nullptr);
                 store_texel(*set, mip, x, y, o);
             }
         }

@@ -164,6 +164,7 @@ EXPORTS = [
                                         C.c_int32, C.c_void_p]),
     ("ntc_hip_selftest_mfma", C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
     ("ntc_hip_selftest_mfma_f16", C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32]),
+    ("ntc_hip_selftest_fp8_activation", C.c_int, [C.c_void_p, C.c_int32, C.c_void_p]),
 ]
 
 _HERE = os.path.dirname(os.path.abspath(__file__))

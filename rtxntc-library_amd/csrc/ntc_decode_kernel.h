@@ -20,8 +20,15 @@ enum {
     NTC_HIP_VARIANT_REF12,
     NTC_HIP_VARIANT_REF8,
     NTC_HIP_VARIANT_REF4,
-    NTC_HIP_VARIANT_CFG3_FP8    // both grids bilinear 16 x 4-bit, (lod,lod), IN 48, 64-64-64, e4m3 hidden-layer weights
+    NTC_HIP_VARIANT_CFG3_FP8,   // both grids bilinear 16 x 4-bit, (lod,lod), IN 48, 64-64-64, e4m3 hidden-layer weights
+    // LibNTC 0.9.2 geometry with the FP8 version of the network (GenericFP8 blob): ntc_decode_fp8_kernel.hip
+    NTC_HIP_VARIANT_REF16_FP8,
+    NTC_HIP_VARIANT_REF12_FP8,
+    NTC_HIP_VARIANT_REF8_FP8,
+    NTC_HIP_VARIANT_REF4_FP8,
+    NTC_HIP_VARIANT_COUNT
 };
+inline bool variant_is_fp8_network(int variant) { return variant >= NTC_HIP_VARIANT_REF16_FP8 && variant <= NTC_HIP_VARIANT_REF4_FP8; }
 
 // One colour mip of one texture set, as the kernel sees it.  Entries are sorted by
 // tileStart; a workgroup tile covers 64 x 4 texels.
@@ -145,6 +152,9 @@ hipError_t launch_bc7_compress(BlockCompressArgs const& args, hipStream_t stream
 hipError_t launch_decode(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream);
 hipError_t launch_queries(int variant, DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries,
                           uint16_t* out, int gridSize, hipStream_t stream);
+hipError_t launch_decode_fp8(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream);
+int resident_fp8_workgroups_per_cu();
+hipError_t launch_selftest_fp8_activation(uint16_t const* in, uint16_t* out, int n, hipStream_t stream);
 int resident_workgroups_per_cu(int variant);
 int tiles_per_round(int variant);      // tiles a workgroup of the variant's decode kernel works on at a time
 hipError_t launch_selftest_mfma(int8_t const* a, int8_t const* b, int32_t* d, hipStream_t stream);

@@ -25,94 +25,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include "ntc_decode_kernel.h"
+#include "ntc_decode_device.h"
 
 namespace ntc_hip_dev {
-
-typedef int   v4i __attribute__((ext_vector_type(4)));
-// Latent grids live in global memory; saying so lets loads use "scalar base + 32-bit lane offset"
-// addressing instead of 64-bit flat addresses built per lane.
-typedef __attribute__((address_space(1))) uint16_t const* GlobalU16Ptr;
-typedef __attribute__((address_space(1))) uint8_t const*  GlobalU8Ptr;
-
-// One u16 at a uniform base plus a 32-bit byte offset per lane (global_load_ushort v, v_off, s[base]).
-__device__ __forceinline__ uint32_t load_u16(GlobalU8Ptr base, uint32_t byteOffset)
-{
-    return *reinterpret_cast<GlobalU16Ptr>(base + byteOffset);
-}
-
-// 24-bit multiply, full rate (the compiler otherwise picks the quarter-rate 32-bit multiply).
-__device__ __forceinline__ uint32_t mul24(uint32_t a, uint32_t b)
-{
-    uint32_t r;
-    asm("v_mul_u32_u24 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-    return r;
-}
-typedef float v4f __attribute__((ext_vector_type(4)));
-
-constexpr int kWaveTexels  = 64;
-
-// ---- small device helpers -----------------------------------------------------------
-
-__device__ __forceinline__ uint32_t spread2(uint32_t byte)     // 4 x 2-bit fields -> 4 bytes
-{
-    uint32_t x = byte & 0xffu;
-    x = (x | (x << 12)) & 0x000f000fu;
-    x = (x | (x << 6))  & 0x03030303u;
-    return x;
-}
-__device__ __forceinline__ uint32_t spread4(uint32_t word)     // 4 x 4-bit fields -> 4 bytes
-{
-    uint32_t x = word & 0xffffu;
-    x = (x | (x << 8)) & 0x00ff00ffu;
-    x = (x | (x << 4)) & 0x0f0f0f0fu;
-    return x;
-}
-
-// Wrap addressing of FeatureGrid::SetupBilinearFilter (src/FeatureGridDevice.h:51-57).
-struct Taps { int x0, y0, x1, y1; float w00, w10, w01, w11; };
-
-__device__ __forceinline__ Taps footprint(float u, float v, int gw, int gh)
-{
-    float const x = u * float(gw) - 0.5f;
-    float const y = v * float(gh) - 0.5f;
-    float const fx = floorf(x), fy = floorf(y);
-    float const dx = x - fx, dy = y - fy;
-    float const dxn = 1.f - dx, dyn = 1.f - dy;
-    Taps t;
-    t.w00 = dxn * dyn; t.w10 = dx * dyn; t.w01 = dxn * dy; t.w11 = dx * dy;
-    // u, v lie in (0, 1), so floor() lands in [-1, g-1] (g itself only through rounding): the
-    // reference's "add g if negative, then mod g" is a conditional add / subtract here.
-    int xb = int(fx), yb = int(fy);
-    if (xb < 0) xb += gw;
-    if (yb < 0) yb += gh;
-    if (xb >= gw) xb -= gw;
-    if (yb >= gh) yb -= gh;
-    t.x0 = xb; t.y0 = yb;
-    t.x1 = (xb + 1 >= gw) ? xb + 1 - gw : xb + 1;
-    t.y1 = (yb + 1 >= gh) ? yb + 1 - gh : yb + 1;
-    return t;
-}
-
-// floor(t * codeScale) - 128 for four features at once, returned as four packed bytes.
-__device__ __forceinline__ uint32_t bilinear4(Taps const& tp, uint32_t s00, uint32_t s10, uint32_t s01, uint32_t s11,
-                                              float codeScale)
-{
-    uint32_t packed = 0;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        float const q00 = float((s00 >> (8 * i)) & 0xffu);
-        float const q10 = float((s10 >> (8 * i)) & 0xffu);
-        float const q01 = float((s01 >> (8 * i)) & 0xffu);
-        float const q11 = float((s11 >> (8 * i)) & 0xffu);
-        float t = tp.w00 * q00;
-        t = __builtin_fmaf(tp.w10, q10, t);
-        t = __builtin_fmaf(tp.w01, q01, t);
-        t = __builtin_fmaf(tp.w11, q11, t);
-        // 0..255, integer-valued after the floor: the conversion is exact and drops the byte into its slot
-        packed = __builtin_amdgcn_cvt_pk_u8_f32(floorf(t * codeScale), uint32_t(i), packed);
-    }
-    return packed ^ 0x80808080u;                            // -128 on every byte
-}
 
 // HGELU-clamp + requantise of four D values of one lane (Inference.hlsli:36-39,123-131,164-179).
 // round-half-even of y*80 is taken from the low mantissa bits of y*80 + 1.5*2^23; the "-113"
@@ -138,93 +53,6 @@ __device__ __forceinline__ uint32_t activate4(v4i acc, v4f scale, uint32_t c143)
     asm("v_add_u32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_0 src1_sel:DWORD"
         : "+v"(packed) : "v"(z[3]), "v"(c143));
     return packed;
-}
-
-typedef _Float16 v2h __attribute__((ext_vector_type(2)));
-typedef _Float16 v4h __attribute__((ext_vector_type(4)));
-typedef _Float16 v8h __attribute__((ext_vector_type(8)));
-typedef float    v2f __attribute__((ext_vector_type(2)));
-
-// Two network outputs -> two fp16 in one dword.  The output is an fp32 product that is THEN
-// rounded to half (round-nearest-even); a half that would be Inf/NaN is stored as zero
-// (IsHalfSpecial, Inference.cu:125-126).  |o| >= 65520 is exactly the set that rounds to
-// Inf.  The empty asm keeps the compiler from folding multiply + convert into
-// v_fma_mixlo_f16, which rounds the exact product once, straight to half.
-// CHECKED = false is for callers that know |a|, |b| stay far below 65520.
-template <bool CHECKED = true>
-__device__ __forceinline__ uint32_t to_half2_bits(float a, float b)
-{
-    asm("" : "+v"(a));
-    asm("" : "+v"(b));
-    if constexpr (CHECKED) {
-        a = (__builtin_fabsf(a) < 65520.f) ? a : 0.f;
-        b = (__builtin_fabsf(b) < 65520.f) ? b : 0.f;
-    }
-    v2h const h = __builtin_convertvector(v2f{a, b}, v2h);
-    return __builtin_bit_cast(uint32_t, h);
-}
-
-// WriteImageChannel UNORM8 (src/ImageProcessing.cu:146-149): u8(clamp(roundf(v * 255), 0, 255)) of
-// the stored half.  v*255 is exact (11-bit x 8-bit significands) and so is v*255 + 1/2 wherever the
-// result matters (below 256), so floor(fma(v, 255, 1/2)) equals roundf(v*255) for v >= 0; negatives
-// end at or below 0.  v_cvt_pk_u8_f32 then converts the integer-valued float with saturation to
-// [0, 255] and drops it into byte `slot` of `packed`.
-__device__ __forceinline__ uint32_t pack_unorm8(_Float16 h, uint32_t slot, uint32_t packed)
-{
-    float const v = floorf(__builtin_fmaf(float(h), 255.f, 0.5f));
-    return __builtin_amdgcn_cvt_pk_u8_f32(v, slot, packed);
-}
-
-typedef __attribute__((address_space(1))) uint8_t* GlobalOutPtr;
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-
-// Stores of one 16-texel block row.  `row` is uniform (start of image row y in the output),
-// `laneOff` the lane's byte offset inside the row, h01/h23 the lane's four channels as halves.
-template <int FORMAT>
-__device__ __forceinline__ void store_channels(GlobalOutPtr row, uint32_t laneOff, uint32_t planarPairStride,
-                                               uint32_t h01, uint32_t h23, int nch)
-{
-    GlobalOutPtr const dst = row + laneOff;
-    if constexpr (FORMAT == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS) {
-        // src/RegressionKernels.h:36-45; whole half2 pairs (Inference.cu:131-134)
-        *reinterpret_cast<__attribute__((address_space(1))) uint32_t*>(dst) = h01;
-        if (nch > 2) *reinterpret_cast<__attribute__((address_space(1))) uint32_t*>(dst + planarPairStride) = h23;
-    } else if constexpr (FORMAT == NTC_HIP_DEV_OUT_FP16_PIXELS) {
-        if (nch == 4 && ((reinterpret_cast<uintptr_t>(dst) & 7u) == 0)) {
-            *reinterpret_cast<__attribute__((address_space(1))) u32x2*>(dst) = u32x2{ h01, h23 };
-        } else {
-            uint32_t const h[4] = { h01 & 0xffffu, h01 >> 16, h23 & 0xffffu, h23 >> 16 };
-            for (int r = 0; r < nch; ++r) reinterpret_cast<__attribute__((address_space(1))) uint16_t*>(dst)[r] = uint16_t(h[r]);
-        }
-    } else {
-        v2h const a = __builtin_bit_cast(v2h, h01), b = __builtin_bit_cast(v2h, h23);
-        uint32_t const u8 = pack_unorm8(b[1], 3, pack_unorm8(b[0], 2, pack_unorm8(a[1], 1, pack_unorm8(a[0], 0, 0u))));
-        if (nch == 4 && ((reinterpret_cast<uintptr_t>(dst) & 3u) == 0)) {
-            *reinterpret_cast<__attribute__((address_space(1))) uint32_t*>(dst) = u8;
-        } else {
-            for (int r = 0; r < nch; ++r) dst[r] = uint8_t(u8 >> (8 * r));
-        }
-    }
-}
-
-template <int FORMAT, bool CHECKED = true, class Acc>
-__device__ __forceinline__ void store_tile(DevMip const& m, Acc const (&D)[4], v4f S, int x, int y0, int chBase)
-{
-    int const nch = min(4, m.numChannels - chBase);
-    if (x >= m.width || nch <= 0) return;
-    uint32_t const C2 = uint32_t((m.numChannels + 1) & ~1);
-    uint32_t const laneOff = (FORMAT == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)
-        ? (uint32_t(chBase) * uint32_t(m.width) + uint32_t(x) * 2u) * 2u
-        : uint32_t(x) * uint32_t(m.outPixelStride) + uint32_t(chBase) * (FORMAT == NTC_HIP_DEV_OUT_FP16_PIXELS ? 2u : 1u);
-    size_t const rowBytes = (FORMAT == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS) ? size_t(m.width) * C2 * 2 : size_t(m.outRowPitch);
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-        int const y = y0 + b;
-        if (y >= m.height) break;                            // uniform
-        uint32_t const h01 = to_half2_bits<CHECKED>(float(D[b][0]) * S[0], float(D[b][1]) * S[1]);
-        uint32_t const h23 = to_half2_bits<CHECKED>(float(D[b][2]) * S[2], float(D[b][3]) * S[3]);
-        store_channels<FORMAT>((GlobalOutPtr)m.out + size_t(y) * rowBytes, laneOff, uint32_t(m.width) * 4u, h01, h23, nch);
-    }
 }
 
 // ---- all-integer input stage (power-of-two mip and grid sizes) --------------------------

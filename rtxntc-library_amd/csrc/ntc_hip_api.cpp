@@ -117,9 +117,10 @@ int pick_variant(NtcHipDecoderSpec const& s)
             && s.hiddenChannels[0] == 64 && s.hiddenChannels[1] == 64 && s.hiddenChannels[2] == 64;
         return wide ? NTC_HIP_VARIANT_CFG3_FP8 : NTC_HIP_VARIANT_NONE;
     }
-    if (s.weightType != NTC_HIP_WEIGHTS_INT8) return NTC_HIP_VARIANT_NONE;
+    if (s.weightType != NTC_HIP_WEIGHTS_INT8 && s.weightType != NTC_HIP_WEIGHTS_FP8) return NTC_HIP_VARIANT_NONE;
+    bool const fp8 = s.weightType == NTC_HIP_WEIGHTS_FP8;    // the FP8 network exists for the LibNTC 0.9.2 geometry only
     bool const concat8x2 = s.hrMode == NTC_HIP_GRID_CONCAT2X2 && s.hrFeatures == 8 && s.hrBits == 2 && s.hrFeatureSlots == 8;
-    if (concat8x2 && s.lodInputs == 0 && s.inputChannels == 64 && s.hiddenChannels[2] == 32) {
+    if (!fp8 && concat8x2 && s.lodInputs == 0 && s.inputChannels == 64 && s.hiddenChannels[2] == 32) {
         if (s.lrFeatures == 16 && s.lrFeatureSlots == 16 && s.hiddenChannels[0] == 64 && s.hiddenChannels[1] == 48)
             return NTC_HIP_VARIANT_CFG01;
         if (s.lrFeatures == 12 && s.lrFeatureSlots == 12 && s.hiddenChannels[0] == 48 && s.hiddenChannels[1] == 48)
@@ -130,10 +131,10 @@ int pick_variant(NtcHipDecoderSpec const& s)
         && s.hiddenChannels[0] == 64 && s.hiddenChannels[1] == 48 && s.hiddenChannels[2] == 32;
     if (ref) {
         switch (s.hrFeatures) {
-        case 16: return NTC_HIP_VARIANT_REF16;
-        case 12: return NTC_HIP_VARIANT_REF12;
-        case 8:  return NTC_HIP_VARIANT_REF8;
-        case 4:  return NTC_HIP_VARIANT_REF4;
+        case 16: return fp8 ? NTC_HIP_VARIANT_REF16_FP8 : NTC_HIP_VARIANT_REF16;
+        case 12: return fp8 ? NTC_HIP_VARIANT_REF12_FP8 : NTC_HIP_VARIANT_REF12;
+        case 8:  return fp8 ? NTC_HIP_VARIANT_REF8_FP8 : NTC_HIP_VARIANT_REF8;
+        case 4:  return fp8 ? NTC_HIP_VARIANT_REF4_FP8 : NTC_HIP_VARIANT_REF4;
         default: break;
         }
     }
@@ -388,14 +389,20 @@ int upload_table(std::vector<DevMip> const& table)
 int grid_size_for(int variant, int totalTiles)
 {
     // Persistent workgroups: as many as stay resident at once, each walking a contiguous share of tiles.
-    static int perCu[16] = { 0 };
+    static int perCu[NTC_HIP_VARIANT_COUNT] = { 0 };
     if (perCu[variant] == 0) {
-        perCu[variant] = resident_workgroups_per_cu(variant);
+        perCu[variant] = variant_is_fp8_network(variant) ? resident_fp8_workgroups_per_cu() : resident_workgroups_per_cu(variant);
     }
     int const resident = g_lib.computeUnits * perCu[variant];
     // a workgroup takes tiles_per_round(variant) tiles at a time: fewer workgroups than that leaves waves idle
     int64_t const rounds = (int64_t(totalTiles) + tiles_per_round(variant) - 1) / tiles_per_round(variant);
     return rounds < resident ? int(rounds) : resident;
+}
+
+hipError_t launch_decode_any(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream)
+{
+    return variant_is_fp8_network(variant) ? launch_decode_fp8(variant, mips, numMips, totalTiles, gridSize, stream)
+                                           : launch_decode(variant, mips, numMips, totalTiles, gridSize, stream);
 }
 
 } // namespace
@@ -568,7 +575,7 @@ int ntc_hip_decode(const NtcHipTextureSet* sets, int32_t numSets)
     int variant = NTC_HIP_VARIANT_NONE, totalTiles = 0;
     if (int r = build_table(sets, numSets, table, variant, totalTiles)) return r;
     if (int r = upload_table(table)) return r;
-    HIP_TRY(launch_decode(variant, g_lib.tableDev, int(table.size()), totalTiles, grid_size_for(variant, totalTiles), g_lib.stream));
+    HIP_TRY(launch_decode_any(variant, g_lib.tableDev, int(table.size()), totalTiles, grid_size_for(variant, totalTiles), g_lib.stream));
     clear_error();
     return 0;
 }
@@ -596,7 +603,7 @@ int ntc_hip_decode_static(const NtcHipTextureSet* sets, int32_t numSets)
                                                     int(count * sizeof(DevMip) / 4));
         HIP_TRY(hipGetLastError());
     }
-    HIP_TRY(launch_decode(variant, L.staticTable, int(table.size()), totalTiles, grid_size_for(variant, totalTiles), L.stream));
+    HIP_TRY(launch_decode_any(variant, L.staticTable, int(table.size()), totalTiles, grid_size_for(variant, totalTiles), L.stream));
     clear_error();
     return 0;
 }
@@ -612,7 +619,7 @@ int ntc_hip_decode_timed(const NtcHipTextureSet* sets, int32_t numSets, int32_t 
     int const grid = grid_size_for(variant, totalTiles);
     HIP_TRY(hipEventRecord(g_lib.evStart, g_lib.stream));
     for (int i = 0; i < iterations; ++i)
-        HIP_TRY(launch_decode(variant, g_lib.tableDev, int(table.size()), totalTiles, grid, g_lib.stream));
+        HIP_TRY(launch_decode_any(variant, g_lib.tableDev, int(table.size()), totalTiles, grid, g_lib.stream));
     HIP_TRY(hipEventRecord(g_lib.evStop, g_lib.stream));
     HIP_TRY(hipEventSynchronize(g_lib.evStop));
     float ms = 0.f;
@@ -634,6 +641,7 @@ static int run_queries(const NtcHipTextureSet* set, const NtcHipQuery* queries, 
     std::vector<DevMip> table;
     int variant = NTC_HIP_VARIANT_NONE, totalTiles = 0;
     if (int r = build_table(set, 1, table, variant, totalTiles, true)) return r;
+    if (variant_is_fp8_network(variant)) { set_error("ntc_hip_decode_queries: the FP8 network is available to ntc_hip_decode only."); return NTC_HIP_ERR_UNSUPPORTED; }
     if (int r = upload_table(table)) return r;
     uint64_t const blocks = (numQueries + 255) / 256;
     uint64_t const resident = uint64_t(g_lib.computeUnits) * uint64_t(grid_size_for(variant, 0x7fffffff) / g_lib.computeUnits);
@@ -996,6 +1004,21 @@ int ntc_hip_selftest_mfma(const int8_t* a16x64, const int8_t* b64x16, int32_t* d
     HIP_TRY(hipStreamSynchronize(g_lib.stream));
     HIP_TRY(hipMemcpy(d16x16, d, 1024, hipMemcpyDeviceToHost));
     (void)hipFree(a); (void)hipFree(b); (void)hipFree(d);
+    return 0;
+}
+
+int ntc_hip_selftest_fp8_activation(const uint16_t* halves, int32_t count, uint16_t* out)
+{
+    if (int r = require_init()) return r;
+    if (!halves || !out || count < 1 || count > (1 << 20)) { set_error("ntc_hip_selftest_fp8_activation: null pointer or count outside 1..2^20."); return NTC_HIP_ERR_INVALID_ARG; }
+    uint16_t* dev = nullptr;
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&dev), size_t(count) * 8));
+    hipError_t e = hipMemcpy(dev, halves, size_t(count) * 2, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = launch_selftest_fp8_activation(dev, dev + count, count, g_lib.stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(g_lib.stream);
+    if (e == hipSuccess) e = hipMemcpy(out, dev + count, size_t(count) * 6, hipMemcpyDeviceToHost);
+    (void)hipFree(dev);
+    HIP_TRY(e);
     return 0;
 }
 

@@ -32,6 +32,13 @@ def spec_ref092(num_features=16):
     return make_spec((num_features, 4, abi.GRID_BILINEAR, 16), (num_features, 4, abi.GRID_BILINEAR, 16), 2, 48, (64, 48, 32))
 
 
+def spec_ref092_fp8(num_features=16):
+    """The same decoder with the FP8 version of the network (GenericFP8 weight blob)."""
+    s = spec_ref092(num_features)
+    s.weightType = abi.WEIGHTS_FP8
+    return s
+
+
 def spec_cfg01():
     return make_spec((8, 2, abi.GRID_CONCAT2X2, 8), (16, 4, abi.GRID_BILINEAR, 16), 0, 64, (64, 48, 32))
 

@@ -169,6 +169,114 @@ def decode_mip(spec, layout, blob, latents_u16, mip):
     return inputs, out.reshape(H, W, 16)
 
 
+# ---- the FP8 network (include/libntc/shaders/InferenceCoopVec.hlsli:22-124,127-160,235-398) -------------------
+
+E4M3_POSITIVE = np.array([(m / 8.0) * 2.0 ** -6 if e == 0 else (1 + m / 8.0) * 2.0 ** (e - 7) for e in range(16) for m in range(8)][:127])
+
+
+def round_to_e4m3(values):
+    """Nearest e4m3 value of each float (brute force over the 127 non-negative values, ties to the even
+    code, everything from 448 up saturates at 448); NaN -> 0."""
+    v = np.asarray(values, dtype=np.float64)
+    a = np.abs(np.nan_to_num(v, nan=0.0, posinf=1e9, neginf=-1e9))
+    hi = np.clip(np.searchsorted(E4M3_POSITIVE, a, side="left"), 1, 126)     # E4M3_POSITIVE[hi-1] <= a <= E4M3_POSITIVE[hi] inside the range
+    lo = hi - 1
+    d_lo, d_hi = a - E4M3_POSITIVE[lo], E4M3_POSITIVE[hi] - a
+    pick_hi = (d_hi < d_lo) | ((d_hi == d_lo) & (hi % 2 == 0))
+    r = np.where(pick_hi, E4M3_POSITIVE[hi], E4M3_POSITIVE[lo])
+    r = np.where(a >= 448.0, 448.0, r)
+    return np.copysign(r, np.where(np.isnan(v), 0.0, v))
+
+
+def hgelu_half(x16):
+    """NtcHGELUClamp_Forward_CoopVec (hlsli:150-153) on float16 arrays, every operation rounded to half once."""
+    x = np.asarray(x16, dtype=np.float16).astype(np.float64)
+    third = np.float64(np.float16(1.0 / 3.0))
+    with np.errstate(over="ignore", invalid="ignore"):
+        t = (x * third + 0.5).astype(np.float16).astype(np.float64)          # exact in float64, one rounding
+        t = np.clip(t, 0.0, 1.0)
+        y = (np.clip(x, -3.0, 3.0) * t).astype(np.float16)
+    return np.where(np.isnan(x), np.float16(0), y)
+
+
+def fp8_inputs(spec, latents_u16, mip):
+    """[H, W, 48] float16: the network's input vector before its e4m3 reading (hlsli:22-107)."""
+    W, H = mip.width, mip.height
+    out = np.zeros((H, W, spec.inputChannels), dtype=np.float16)
+    for base, words, gw, gh, features in ((0, latents_u16[mip.hrOffset // 2:], mip.hrWidth, mip.hrHeight, spec.hrFeatures),
+                                          (spec.hrFeatureSlots, latents_u16[mip.lrOffset // 2:], mip.lrWidth, mip.lrHeight, spec.lrFeatures)):
+        codes = unpack_grid(words, gw, gh, features, 4)
+        x0, x1, dx = footprint(W, W, gw)
+        y0, y1, dy = footprint(H, H, gh)
+        taps = [codes[np.ix_(y0, x0)], codes[np.ix_(y0, x1)], codes[np.ix_(y1, x0)], codes[np.ix_(y1, x1)]]
+        dxn, dyn = F32(1) - dx, F32(1) - dy
+        w = [(dyn[:, None] * dxn[None, :]).astype(F32), (dyn[:, None] * dx[None, :]).astype(F32),
+             (dy[:, None] * dxn[None, :]).astype(F32), (dy[:, None] * dx[None, :]).astype(F32)]
+        for f in range(features):
+            q = [tap[:, :, f].astype(F32) for tap in taps]
+            t = (w[0] * q[0]).astype(F32)
+            for i in (1, 2, 3):
+                t = fma32(w[i], q[i], t).reshape(H, W)
+            out[:, :, base + f] = fma32(t, F32(2.0 / 15.0), F32(-1)).reshape(H, W).astype(np.float16)
+    at = spec.hrFeatureSlots + spec.lrFeatureSlots
+    px = (np.arange(W, dtype=F32) * F32(mip.positionScale)).astype(F32)
+    py = (np.arange(H, dtype=F32) * F32(mip.positionScale)).astype(F32)
+
+    def enc(p):
+        return (((p - np.floor(p)).astype(F32) * F32(2)).astype(F32) - F32(1)).astype(F32).astype(np.float16)
+
+    for _ in range(spec.posEncWaves):
+        out[:, :, at + 0] = enc(px)[None, :]
+        out[:, :, at + 1] = enc(py)[:, None]
+        out[:, :, at + 2] = enc((px + F32(0.25)).astype(F32))[None, :]
+        out[:, :, at + 3] = enc((py + F32(0.25)).astype(F32))[:, None]
+        px, py, at = (px * F32(2)).astype(F32), (py * F32(2)).astype(F32), at + 4
+    out[:, :, at: at + spec.lodInputs] = np.float16(F32(mip.positionLod))
+    return out
+
+
+def layer_e4m3(w_bytes, bias16, a):
+    """Layer outputs (float16) from e4m3 weights [out, in], fp16 biases and e4m3-valued inputs a [n, in]: the
+    exact dot product in three parts by the bits of |512 w|, added in fp32 as ((s2 + s1) + s0) + bias."""
+    w512 = e4m3_times_512(w_bytes)
+    a512 = np.rint(np.asarray(a, dtype=np.float64) * 512.0).astype(np.int64)
+    assert np.array_equal(a512 / 512.0, np.asarray(a, dtype=np.float64))
+    mag, sign = np.abs(w512), np.sign(w512)
+    parts = []
+    for shift, unit in ((0, -18), (7, -11), (14, -4)):
+        plane = sign * ((mag >> shift) & (127 if shift < 14 else 0xFFFF))
+        s_int = a512 @ plane.T
+        assert np.abs(s_int).max(initial=0) < (1 << 24)
+        parts.append(np.ldexp(s_int.astype(np.float64), unit).astype(F32))
+    with np.errstate(over="ignore"):
+        r = ((parts[2] + parts[1]).astype(F32) + parts[0]).astype(F32)
+        r = (r + np.asarray(bias16, dtype=np.float16).astype(F32)[None, :]).astype(F32)
+        return r.astype(np.float16)
+
+
+def decode_mip_fp8(spec, layout, blob, latents_u16, mip):
+    """Outputs float32 [H, W, 16] of one colour mip through the FP8 network (NtcEvaluateMLP_CoopVec_FP8)."""
+    H, W = mip.height, mip.width
+    a = round_to_e4m3(fp8_inputs(spec, latents_u16, mip).reshape(-1, spec.inputChannels).astype(np.float64))
+    q = None
+    for layer in range(3):
+        n_in, n_out = spec.layer_inputs(layer), spec.layer_outputs(layer)
+        w = blob[layout.weightOffset[layer]: layout.weightOffset[layer] + n_in * n_out].reshape(n_out, n_in)
+        bias = blob[layout.biasOffset[layer]: layout.biasOffset[layer] + 2 * n_out].view(np.float16)
+        y = hgelu_half(layer_e4m3(w, bias, a))
+        if layer < 2:
+            a = round_to_e4m3(y.astype(np.float64))
+        else:
+            q = np.rint(80.0 * y.astype(np.float64) - 113.0).astype(np.int64)     # exact in float64, one rounding
+            assert q.min() >= -128 and q.max() <= 127
+    n_in = spec.layer_inputs(3)
+    w = blob[layout.weightOffset[3]: layout.weightOffset[3] + n_in * 16].view(np.int8).reshape(16, n_in).astype(np.int64)
+    scale = blob[layout.scaleOffset[3]: layout.scaleOffset[3] + 64].view(np.float32)
+    bias = blob[layout.biasOffset[3]: layout.biasOffset[3] + 64].view(np.int32).astype(np.int64)
+    acc = (q @ w.T + bias).astype(np.int32)
+    return (acc.astype(F32) * scale[None, :]).astype(F32).reshape(H, W, 16)
+
+
 def to_half_bits(outputs):
     h = np.asarray(outputs, dtype=F32).astype(np.float16)        # IEEE round-to-nearest-even
     bits = h.view(np.uint16).copy()

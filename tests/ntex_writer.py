@@ -69,8 +69,25 @@ def split_int8_blob(blob, widths=LAYER_WIDTHS_092):
     return weights, scales, biases
 
 
+def split_fp8_blob(blob, widths=LAYER_WIDTHS_092):
+    """(weights per layer, output-layer scales, biases per layer) from a GenericFP8 blob (src/WeightLayout.cpp:51-71):
+    all matrices, then the fp16 biases of the three e4m3 layers, then the output layer's fp32 scales and int32 biases."""
+    blob = np.asarray(blob, dtype=np.uint8)
+    at = 0
+    weights, biases = [], []
+    for i, o in widths:
+        weights.append(blob[at: at + i * o]); at += i * o
+    for _, o in widths[:-1]:
+        biases.append(blob[at: at + 2 * o]); at += 2 * o
+    out = widths[-1][1]
+    scales = blob[at: at + 4 * out]; at += 4 * out
+    biases.append(blob[at: at + 4 * out]); at += 4 * out
+    assert at == blob.size
+    return weights, scales, biases
+
+
 def write_ntex(width, height, channels, mips, grid_scale, features, latents, int8_blob, textures=(),
-               fp8_version=True, layer_widths=None, layer_data=None, channel_color_spaces=None,
+               fp8_version=True, fp8_blob=None, layer_widths=None, layer_data=None, channel_color_spaces=None,
                extra_document_fields=None, mutate=None, json_indent=None, mode_buffers=()):
     """Returns the bytes of an NTC file.
 
@@ -99,16 +116,18 @@ def write_ntex(width, height, channels, mips, grid_scale, features, latents, int
     if fp8_version:   # e4m3 hidden layers with fp16 biases and no scales; int8 output layer (src/TextureSet.cpp:561-590)
         rng = np.random.default_rng(7)
         fp8_layers = []
+        # the pieces of a GenericFP8 blob (src/WeightLayout.cpp:51-71) when one is given, else arbitrary bytes
+        pieces = split_fp8_blob(fp8_blob) if fp8_blob is not None else None
         for index, (n_in, n_out) in enumerate(LAYER_WIDTHS_092):
             last = index == 3
-            layer = {"inputChannels": n_in, "outputChannels": n_out,
-                     "weightView": table.add(rng.integers(0, 120, n_in * n_out, dtype=np.uint8))}
+            weights = pieces[0][index] if pieces else rng.integers(0, 120, n_in * n_out, dtype=np.uint8)
+            layer = {"inputChannels": n_in, "outputChannels": n_out, "weightView": table.add(weights)}
             if last:
-                layer.update({"weightType": "Int8", "scaleType": "Float32", "biasType": "Int32",
-                              "scaleView": table.add(np.ones(n_out, np.float32).view(np.uint8))})
+                scales = pieces[1] if pieces else np.ones(n_out, np.float32).view(np.uint8)
+                layer.update({"weightType": "Int8", "scaleType": "Float32", "biasType": "Int32", "scaleView": table.add(scales)})
             else:
                 layer.update({"weightType": "FloatE4M3", "biasType": "Float16"})
-            layer["biasView"] = table.add(np.zeros(n_out, np.int32 if last else np.float16).view(np.uint8))
+            layer["biasView"] = table.add(pieces[2][index] if pieces else np.zeros(n_out, np.int32 if last else np.float16).view(np.uint8))
             fp8_layers.append(layer)
         versions.append({"layers": fp8_layers, "activation": "HGELUClamp", "weightLayout": "RowMajor"})
 

@@ -109,6 +109,27 @@ def test_wide_fp8_4096_rows_equal_checker(ntc, device, oracle):
         assert np.array_equal(host.output[y0 * row_bytes:(y0 + 24) * row_bytes], got[y0 * row_bytes:(y0 + 24) * row_bytes]), y0
 
 
+def test_fp8_network_4096_row_bands_equal_checker(ntc, device, oracle):
+    """The LibNTC 0.9.2 geometry with the FP8 version of the network at 4096^2 with its full mip chain: bands of
+    rows of mip 0 and every mip from 512^2 down against the checker."""
+    spec = ntc.presets.spec_ref092_fp8(16)
+    mips, latent_bytes = ntc.presets.mips_ref092(spec, 4096, 4096, 13, 2)
+    case = Case(ntc, spec, mips, latent_bytes, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=5, weights=ntc.synth.make_fp8_weights(spec, 6))
+    dset = case.device_set(device)
+    device.decode([dset])
+    device.synchronize()
+    got = case.d_output.download()
+    host = case.host_set()
+    row_bytes = 4096 * 16 * 2
+    for y0 in (0, 2046, 4096 - 12):
+        oracle.ntc_oracle_decode_rows(host.desc, 0, y0, y0 + 12, 16)
+        assert np.array_equal(host.output[y0 * row_bytes:(y0 + 12) * row_bytes], got[y0 * row_bytes:(y0 + 12) * row_bytes]), y0
+    for m in range(3, 13):
+        oracle.ntc_oracle_decode_rows(host.desc, m, 0, case.mips[m].height, 16)
+    start = case.mips[3].outOffset
+    assert np.array_equal(host.output[start:], got[start:])
+
+
 def test_random_access_8192_queries(ntc, device, oracle):
     """Config 4 at full size: 2^24 queries into an 8192^2, 14-mip set.  A 2^20 sample goes to the
     checker; repeated queries must repeat their answers; mip 13 (1x1) answers are all one texel."""

@@ -15,6 +15,7 @@ import subprocess
 import numpy as np
 import pytest
 
+from cases import Case
 from test_ntc_file import TEXTURES, file_of, make_case, pixels_from_planar
 
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -86,3 +87,28 @@ def test_gpu_decode_through_the_reference_header_equals_the_checker(ntc, oracle,
         planar = np.ascontiguousarray(host.output[mip.outOffset: mip.outOffset + mip.width * mip.height * channels * 2].view(np.uint16))
         got = np.fromfile(f"{prefix}_mip{m}.bin", dtype=np.uint16)
         assert np.array_equal(got, pixels_from_planar(planar, mip.width, mip.height, channels)), f"mip {m}"
+
+
+@pytest.mark.gpu
+def test_gpu_decode_with_the_default_fp8_weights_equals_the_checker(ntc, oracle, tmp_path):
+    """Decompress(stats) with useInt8Weights left at its default decodes with the file's FP8 version of the network
+    (src/TextureSet.cpp:1664-1682,1812,1826); the checker's FP8 network on the same blob gives the same bytes, and
+    the Int8 version of the same file still decodes to ITS bytes."""
+    width, height, grid_scale, features, channels = 128, 96, 2, 16, 10
+    case = make_case(ntc, width, height, None, grid_scale, features, channels, seed=43)
+    spec_fp8 = ntc.presets.spec_ref092_fp8(features)
+    fp8_blob = ntc.synth.make_fp8_weights(spec_fp8, 44)
+    path = tmp_path / "set.ntc"
+    path.write_bytes(file_of(case, width, height, grid_scale, features, channels, textures=TEXTURES, fp8_blob=fp8_blob))
+    for use_int8, name in ((0, "FP8"), (1, "Int8")):
+        prefix = str(tmp_path / f"out{use_int8}")
+        out = run_dropin("decode", path, prefix, use_int8)
+        assert f"{name} weights" in out
+        checker = case if use_int8 else Case(ntc, spec_fp8, case.mips, case.latents.nbytes, channels, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=0,
+                                               latents=case.latents, weights=fp8_blob)
+        host = checker.host_set()
+        host.decode(threads=8)
+        for m, mip in enumerate(case.mips):
+            planar = np.ascontiguousarray(host.output[mip.outOffset: mip.outOffset + mip.width * mip.height * channels * 2].view(np.uint16))
+            got = np.fromfile(f"{prefix}_mip{m}.bin", dtype=np.uint16)
+            assert np.array_equal(got, pixels_from_planar(planar, mip.width, mip.height, channels)), (name, m)
