@@ -20,10 +20,17 @@
  * A message for the last failure on the calling thread is kept per thread, like
  * the reference's thread-local error buffer (src/Errors.cpp:21-52).
  *
- * Threading: the library holds one device, one stream, one mip table and one set of loss partials per
- * process and takes no locks (nor does the reference: its texture sets share __constant__ state,
- * src/Regression.cu:40-51).  Calls from several threads must be serialised by the caller.  Work is
- * queued on the library's stream in call order; ntc_hip_synchronize waits for it.
+ * Contexts: all device state - the device, a stream, the decode kernels' mip table with its staging
+ * memory, the loss pass's partial sums, timing events - belongs to an NtcHipContext (ntc_hip_create /
+ * ntc_hip_destroy), as the reference scopes its device per context (include/libntc/ntc.h:1289-1290,
+ * src/CudaDeviceGuard.cpp:21-62).  Every entry point exists as ntc_hip_ctx_<name>(context, ...); the
+ * functions without a context argument run on one default context that ntc_hip_init creates.  Contexts
+ * share nothing (except the per-device table of ntc_hip_decode_static, see there); each queues its work
+ * on its own stream in call order, and ntc_hip_ctx_synchronize waits for it.  A call makes its context's
+ * device current and restores the caller's before it returns.
+ * Threading: no locks (nor in the reference: its texture sets share __constant__ state,
+ * src/Regression.cu:40-51).  Calls on ONE context must be serialised by the caller; different contexts may
+ * be used from different threads at the same time.
  */
 #ifndef NTC_HIP_H
 #define NTC_HIP_H
@@ -152,8 +159,17 @@ typedef struct NtcHipTextureSet {
 
 /* ---- library / device ------------------------------------------------------------ */
 
-/* Selects the HIP device and creates the library's stream.  Replaces the reference's
- * cudaSetDevice + cudaInitDevice in CreateContext (src/PublicFunctions.cpp:84-112). */
+/* A context: one device, one stream (opaque). */
+typedef struct NtcHipContext NtcHipContext;
+/* Creates a context on HIP device `device` (which must be a gfx950 device) with a stream of its own.
+ * Replaces the reference's cudaSetDevice + cudaInitDevice in CreateContext (src/PublicFunctions.cpp:84-112). */
+int ntc_hip_create(int device, NtcHipContext** outContext);
+/* Waits for the context's work, then releases its stream and working memory.  Memory from
+ * ntc_hip_ctx_alloc is the caller's to free first. */
+void ntc_hip_destroy(NtcHipContext* context);
+
+/* Creates the default context (the one behind every function below that takes no context) on `device`
+ * and makes that device current; a second call with another device replaces it. */
 int ntc_hip_init(int device);
 void ntc_hip_shutdown(void);
 /* Message of the last failed call on this thread ("" if none). GetLastErrorMessage, include/libntc/ntc.h:1331. */
@@ -199,10 +215,10 @@ int ntc_hip_decode_timed(const NtcHipTextureSet* sets, int32_t numSets, int32_t 
  * device as kernel arguments.  The call allocates nothing, frees nothing and copies nothing: it launches
  * one small table-writing kernel per 16 mips and then the decode kernel of ntc_hip_decode, same results.
  * More than NTC_HIP_STATIC_TABLE_MIPS mips over all sets of one call: NTC_HIP_ERR_INVALID_ARG.
- * All calls on one GPU share that GPU's array, which keeps the last call's table.  Calls queued on the
- * library stream run in order and are safe; calls that overlap on one GPU (several processes' threads
- * are not meant: several threads of one process without the serialisation this library asks for) race.
- * Asynchronous on the library stream. */
+ * All calls on one GPU, from whatever context, share that GPU's array, which keeps the last call's table.
+ * Calls queued on ONE context's stream run in order and are safe; calls that overlap on one GPU - from
+ * two contexts, whose streams are not ordered against each other, or from threads of one process without
+ * the serialisation this library asks for - race on it.  Asynchronous on the context's stream. */
 #define NTC_HIP_STATIC_TABLE_MIPS 256
 int ntc_hip_decode_static(const NtcHipTextureSet* sets, int32_t numSets);
 
@@ -370,6 +386,28 @@ typedef struct NtcHipBlockCompress {
     int32_t     modeMapOffsetX, modeMapOffsetY;
 } NtcHipBlockCompress;
 int ntc_hip_block_compress(const NtcHipBlockCompress* params);
+
+/* ---- every entry point above on a context of the caller's (same arguments, same results) ------------ */
+int ntc_hip_ctx_device_info(NtcHipContext* context, char* name, size_t nameSize, int* computeUnits);
+int ntc_hip_ctx_device_clock(NtcHipContext* context, int* clockRateKHz);
+int ntc_hip_ctx_alloc(NtcHipContext* context, void** devPtr, size_t bytes);
+int ntc_hip_ctx_free(NtcHipContext* context, void* devPtr);
+int ntc_hip_ctx_upload(NtcHipContext* context, void* dst, const void* src, size_t bytes);
+int ntc_hip_ctx_download(NtcHipContext* context, void* dst, const void* src, size_t bytes);
+int ntc_hip_ctx_memset(NtcHipContext* context, void* dst, int value, size_t bytes);
+int ntc_hip_ctx_synchronize(NtcHipContext* context);
+int ntc_hip_ctx_decode(NtcHipContext* context, const NtcHipTextureSet* sets, int32_t numSets);
+int ntc_hip_ctx_decode_static(NtcHipContext* context, const NtcHipTextureSet* sets, int32_t numSets);
+int ntc_hip_ctx_decode_timed(NtcHipContext* context, const NtcHipTextureSet* sets, int32_t numSets, int32_t iterations, float* outMs);
+int ntc_hip_ctx_build_query_latents(NtcHipContext* context, const NtcHipTextureSet* set, void* dst, uint64_t dstBytes);
+int ntc_hip_ctx_decode_queries(NtcHipContext* context, const NtcHipTextureSet* set, const NtcHipQuery* queries, uint64_t numQueries, void* out, uint64_t outBytes);
+int ntc_hip_ctx_decode_queries_timed(NtcHipContext* context, const NtcHipTextureSet* set, const NtcHipQuery* queries, uint64_t numQueries, void* out, uint64_t outBytes, int32_t iterations, float* outMillisecondsPerIteration);
+int ntc_hip_ctx_read_channels(NtcHipContext* context, const NtcHipReadChannels* p);
+int ntc_hip_ctx_write_channels(NtcHipContext* context, const NtcHipWriteChannels* p);
+int ntc_hip_ctx_image_loss(NtcHipContext* context, void* decoded, const void* reference, uint64_t planarBytes, int32_t width, int32_t height, int32_t setChannels, uint32_t validChannelMask, int32_t maskChannelIndex, int32_t discardMaskedOutPixels, float* outMse);
+int ntc_hip_ctx_resize_planar(NtcHipContext* context, const void* src, uint64_t srcBytes, int32_t srcWidth, int32_t srcHeight, void* dst, uint64_t dstBytes, int32_t dstWidth, int32_t dstHeight, int32_t setChannels, const uint8_t* channelColorSpaces);
+int ntc_hip_ctx_image_difference(NtcHipContext* context, const NtcHipImageDifference* p);
+int ntc_hip_ctx_block_compress(NtcHipContext* context, const NtcHipBlockCompress* p);
 
 /* Self-check of the MFMA operand layout the kernels assume: multiplies a 16x64 by a
  * 64x16 int8 matrix on the device (row-major host arrays), writes the 16x16 int32

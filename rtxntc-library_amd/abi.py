@@ -167,6 +167,14 @@ EXPORTS = [
     ("ntc_hip_selftest_fp8_activation", C.c_int, [C.c_void_p, C.c_int32, C.c_void_p]),
 ]
 
+# The context forms: ntc_hip_ctx_<name>(context, same arguments); ntc_hip_create / ntc_hip_destroy.
+_CONTEXT_FORMS = ["device_info", "device_clock", "alloc", "free", "upload", "download", "memset", "synchronize", "decode",
+                  "decode_static", "decode_timed", "build_query_latents", "decode_queries", "decode_queries_timed", "read_channels",
+                  "write_channels", "image_loss", "resize_planar", "image_difference", "block_compress"]
+_BY_NAME = {name: (restype, argtypes) for name, restype, argtypes in EXPORTS}
+EXPORTS += [("ntc_hip_ctx_" + n, _BY_NAME["ntc_hip_" + n][0], [C.c_void_p] + _BY_NAME["ntc_hip_" + n][1]) for n in _CONTEXT_FORMS]
+EXPORTS += [("ntc_hip_create", C.c_int, [C.c_int, C.POINTER(C.c_void_p)]), ("ntc_hip_destroy", None, [C.c_void_p])]
+
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libntc_hip.so")
 _lib = None

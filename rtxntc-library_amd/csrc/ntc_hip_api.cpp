@@ -9,6 +9,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <new>
 #include <vector>
 
 using namespace ntc_hip_dev;
@@ -55,8 +56,13 @@ __global__ void __launch_bounds__(256) write_table_kernel(uint32_t* dst, TableCh
     for (int i = threadIdx.x; i < dwords; i += blockDim.x) dst[i] = src[i];
 }
 
-struct Library {
-    bool initialized = false;
+} // namespace
+
+// One device, one stream and the device-side working memory of the calls made through it: the mip table of
+// the decode kernels with its pinned staging slots, the partial sums of the loss pass, two timing events.
+// Contexts share nothing but the per-device table of ntc_hip_decode_static.
+struct NtcHipContext {
+    bool initialized = false;      // false again once destroyed
     int device = -1;
     int computeUnits = 0;
     int clockRateKHz = 0;
@@ -75,16 +81,30 @@ struct Library {
     Slot slots[kSlots];                // pinned staging for asynchronous table uploads
     int nextSlot = 0;
 };
-Library g_lib;
 
-int require_init()
-{
-    if (!g_lib.initialized) {
-        set_error("ntc_hip_init has not been called (or found no HIP device).");
-        return NTC_HIP_ERR_NOT_INITIALIZED;
+
+namespace {
+using Library = NtcHipContext;
+Library* g_default = nullptr;          // the context behind the functions that take none (ntc_hip_init)
+
+// Makes the context's device current for the duration of a call and restores the caller's afterwards, as the
+// reference's CudaDeviceGuard does around every entry point (src/CudaDeviceGuard.cpp:21-62).
+struct DeviceGuard {
+    int previous = -1;
+    bool changed = false;
+    explicit DeviceGuard(int device)
+    {
+        if (hipGetDevice(&previous) == hipSuccess && previous != device) changed = hipSetDevice(device) == hipSuccess;
     }
-    return 0;
+    ~DeviceGuard() { if (changed) (void)hipSetDevice(previous); }
+};
+
+int not_initialized()
+{
+    set_error("ntc_hip_init has not been called (or found no HIP device), or the context is null or destroyed.");
+    return NTC_HIP_ERR_NOT_INITIALIZED;
 }
+#define CTX_ENTER(ctx) if (!(ctx) || !(ctx)->initialized) return not_initialized(); Library& L = *(ctx); DeviceGuard deviceGuard_(L.device)
 
 // Caller-given strides and offsets enter 64-bit size products: bounded so that none can wrap.
 constexpr uint64_t kMaxRowPitch = uint64_t(1) << 40, kMaxPixelStride = uint64_t(1) << 20;
@@ -354,9 +374,8 @@ int build_table(NtcHipTextureSet const* sets, int32_t numSets, std::vector<DevMi
 // Makes the device table hold `table` (re-uploads only when it changed).  The copy is asynchronous
 // from one of a few pinned staging slots; a slot is reused only after the copy that last read it
 // has completed (its event), so back-to-back launches with different tables never wait on the GPU.
-int upload_table(std::vector<DevMip> const& table)
+int upload_table(Library& L, std::vector<DevMip> const& table)
 {
-    Library& L = g_lib;
     bool const same = L.lastTable.size() == table.size()
         && std::memcmp(L.lastTable.data(), table.data(), table.size() * sizeof(DevMip)) == 0;
     if (same) return 0;
@@ -386,14 +405,14 @@ int upload_table(std::vector<DevMip> const& table)
     return 0;
 }
 
-int grid_size_for(int variant, int totalTiles)
+int grid_size_for(Library const& L, int variant, int totalTiles)
 {
     // Persistent workgroups: as many as stay resident at once, each walking a contiguous share of tiles.
     static int perCu[NTC_HIP_VARIANT_COUNT] = { 0 };
     if (perCu[variant] == 0) {
         perCu[variant] = variant_is_fp8_network(variant) ? resident_fp8_workgroups_per_cu() : resident_workgroups_per_cu(variant);
     }
-    int const resident = g_lib.computeUnits * perCu[variant];
+    int const resident = L.computeUnits * perCu[variant];
     // a workgroup takes tiles_per_round(variant) tiles at a time: fewer workgroups than that leaves waves idle
     int64_t const rounds = (int64_t(totalTiles) + tiles_per_round(variant) - 1) / tiles_per_round(variant);
     return rounds < resident ? int(rounds) : resident;
@@ -409,9 +428,12 @@ hipError_t launch_decode_any(int variant, DevMip const* mips, int numMips, int t
 
 extern "C" {
 
-int ntc_hip_init(int device)
+// Builds a context on `device`: cudaSetDevice + cudaInitDevice of CreateContext (src/PublicFunctions.cpp:84-112).
+static int create_context(int device, NtcHipContext** outContext)
 {
     clear_error();
+    if (!outContext) { set_error("ntc_hip_create: null out-pointer."); return NTC_HIP_ERR_INVALID_ARG; }
+    *outContext = nullptr;
     int count = 0;
     hipError_t err = hipGetDeviceCount(&count);
     if (err != hipSuccess || count == 0) {
@@ -419,121 +441,148 @@ int ntc_hip_init(int device)
         return NTC_HIP_ERR_NO_DEVICE;
     }
     if (device < 0 || device >= count) { set_error("ntc_hip_init: device %d out of range 0..%d.", device, count - 1); return NTC_HIP_ERR_INVALID_ARG; }
-    if (g_lib.initialized) {
-        if (g_lib.device == device) return 0;
-        ntc_hip_shutdown();
-    }
-    HIP_TRY(hipSetDevice(device));
+    if (device >= kMaxDevices) { set_error("ntc_hip_init: device index %d is beyond the %d this library keeps state for.", device, kMaxDevices); return NTC_HIP_ERR_UNSUPPORTED; }
     hipDeviceProp_t prop;
     HIP_TRY(hipGetDeviceProperties(&prop, device));
     if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
         set_error("ntc_hip_init: device %d is %s; this library holds gfx950 code only.", device, prop.gcnArchName);
         return NTC_HIP_ERR_UNSUPPORTED;
     }
-    g_lib.device = device;
-    g_lib.computeUnits = prop.multiProcessorCount;
-    g_lib.clockRateKHz = prop.clockRate;
-    std::snprintf(g_lib.name, sizeof(g_lib.name), "%s (%s)", prop.name, prop.gcnArchName);
-    if (device >= kMaxDevices) { set_error("ntc_hip_init: device index %d is beyond the %d this library keeps state for.", device, kMaxDevices); return NTC_HIP_ERR_UNSUPPORTED; }
+    DeviceGuard guard(device);
     if (!g_staticTable[device]) {       // once per device, with that device current
         void* address = nullptr;
         HIP_TRY(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)));
         g_staticTable[device] = address;
     }
-    g_lib.staticTable = static_cast<DevMip*>(g_staticTable[device]);
-    HIP_TRY(hipStreamCreate(&g_lib.stream));
-    HIP_TRY(hipEventCreate(&g_lib.evStart));
-    HIP_TRY(hipEventCreate(&g_lib.evStop));
-    g_lib.initialized = true;
+    NtcHipContext* L = new (std::nothrow) NtcHipContext();
+    if (!L) { set_error("ntc_hip_create: out of host memory."); return NTC_HIP_ERR_INVALID_ARG; }
+    L->device = device;
+    L->computeUnits = prop.multiProcessorCount;
+    L->clockRateKHz = prop.clockRate;
+    std::snprintf(L->name, sizeof(L->name), "%s (%s)", prop.name, prop.gcnArchName);
+    L->staticTable = static_cast<DevMip*>(g_staticTable[device]);
+    hipError_t e = hipStreamCreate(&L->stream);
+    if (e == hipSuccess) e = hipEventCreate(&L->evStart);
+    if (e == hipSuccess) e = hipEventCreate(&L->evStop);
+    if (e != hipSuccess) {
+        if (L->evStart) (void)hipEventDestroy(L->evStart);
+        if (L->stream) (void)hipStreamDestroy(L->stream);
+        delete L;
+        return hip_fail("hipStreamCreate / hipEventCreate", e);
+    }
+    L->initialized = true;
+    *outContext = L;
     return 0;
+}
+
+static void destroy_context(NtcHipContext* L)
+{
+    if (!L || !L->initialized) return;
+    DeviceGuard guard(L->device);
+    (void)hipStreamSynchronize(L->stream);
+    if (L->tableDev) (void)hipFree(L->tableDev);
+    if (L->lossDev) (void)hipFree(L->lossDev);
+    if (L->lossHost) (void)hipHostFree(L->lossHost);
+    for (Library::Slot& slot : L->slots) {
+        if (slot.host) (void)hipHostFree(slot.host);
+        if (slot.done) (void)hipEventDestroy(slot.done);
+    }
+    (void)hipEventDestroy(L->evStart);
+    (void)hipEventDestroy(L->evStop);
+    (void)hipStreamDestroy(L->stream);
+    L->initialized = false;
+    delete L;
+}
+
+int ntc_hip_create(int device, NtcHipContext** outContext) { return create_context(device, outContext); }
+void ntc_hip_destroy(NtcHipContext* context) { if (context == g_default) g_default = nullptr; destroy_context(context); }
+
+int ntc_hip_init(int device)
+{
+    if (g_default && g_default->initialized) {
+        if (g_default->device == device) { clear_error(); return 0; }
+        ntc_hip_shutdown();
+    }
+    int const rc = create_context(device, &g_default);
+    if (rc == 0) (void)hipSetDevice(device);      // callers of the context-free functions may use HIP themselves afterwards
+    return rc;
 }
 
 void ntc_hip_shutdown(void)
 {
-    if (!g_lib.initialized) return;
-    (void)hipStreamSynchronize(g_lib.stream);
-    if (g_lib.tableDev) (void)hipFree(g_lib.tableDev);
-    if (g_lib.lossDev) (void)hipFree(g_lib.lossDev);
-    if (g_lib.lossHost) (void)hipHostFree(g_lib.lossHost);
-    for (Library::Slot& slot : g_lib.slots) {
-        if (slot.host) (void)hipHostFree(slot.host);
-        if (slot.done) (void)hipEventDestroy(slot.done);
-    }
-    (void)hipEventDestroy(g_lib.evStart);
-    (void)hipEventDestroy(g_lib.evStop);
-    (void)hipStreamDestroy(g_lib.stream);
-    g_lib = Library();
+    destroy_context(g_default);
+    g_default = nullptr;
 }
 
 const char* ntc_hip_last_error(void) { return t_error; }
 
-int ntc_hip_device_info(char* name, size_t nameSize, int* computeUnits)
+int ntc_hip_ctx_device_info(NtcHipContext* ctx, char* name, size_t nameSize, int* computeUnits)
 {
-    if (int r = require_init()) return r;
-    if (name && nameSize) { std::snprintf(name, nameSize, "%s", g_lib.name); }
-    if (computeUnits) *computeUnits = g_lib.computeUnits;
+    CTX_ENTER(ctx);
+    if (name && nameSize) { std::snprintf(name, nameSize, "%s", L.name); }
+    if (computeUnits) *computeUnits = L.computeUnits;
     return 0;
 }
 
-int ntc_hip_device_clock(int* clockRateKHz)
+int ntc_hip_ctx_device_clock(NtcHipContext* ctx, int* clockRateKHz)
 {
-    if (int r = require_init()) return r;
+    CTX_ENTER(ctx);
     if (!clockRateKHz) { set_error("ntc_hip_device_clock: null out-pointer."); return NTC_HIP_ERR_INVALID_ARG; }
-    *clockRateKHz = g_lib.clockRateKHz;
+    *clockRateKHz = L.clockRateKHz;
     return 0;
 }
 
-int ntc_hip_alloc(void** devPtr, size_t bytes)
+int ntc_hip_ctx_alloc(NtcHipContext* ctx, void** devPtr, size_t bytes)
 {
-    if (int r = require_init()) return r;
+    CTX_ENTER(ctx);
     if (!devPtr) { set_error("ntc_hip_alloc: null out-pointer."); return NTC_HIP_ERR_INVALID_ARG; }
     *devPtr = nullptr;
     HIP_TRY(hipMalloc(devPtr, bytes ? bytes : 1));
     return 0;
 }
 
-int ntc_hip_free(void* devPtr)
+int ntc_hip_ctx_free(NtcHipContext* ctx, void* devPtr)
 {
-    if (int r = require_init()) return r;
+    CTX_ENTER(ctx);
     if (!devPtr) return 0;
-    HIP_TRY(hipStreamSynchronize(g_lib.stream));
+    HIP_TRY(hipStreamSynchronize(L.stream));
     HIP_TRY(hipFree(devPtr));
     return 0;
 }
 
-int ntc_hip_upload(void* dst, const void* src, size_t bytes)
+int ntc_hip_ctx_upload(NtcHipContext* ctx, void* dst, const void* src, size_t bytes)
 {
-    if (int r = require_init()) return r;
+    CTX_ENTER(ctx);
     if (bytes == 0) return 0;
     if (!dst || !src) { set_error("ntc_hip_upload: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
-    HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g_lib.stream));
-    HIP_TRY(hipStreamSynchronize(g_lib.stream));
+    HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, L.stream));
+    HIP_TRY(hipStreamSynchronize(L.stream));
     return 0;
 }
 
-int ntc_hip_download(void* dst, const void* src, size_t bytes)
+int ntc_hip_ctx_download(NtcHipContext* ctx, void* dst, const void* src, size_t bytes)
 {
-    if (int r = require_init()) return r;
+    CTX_ENTER(ctx);
     if (bytes == 0) return 0;
     if (!dst || !src) { set_error("ntc_hip_download: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
-    HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g_lib.stream));
-    HIP_TRY(hipStreamSynchronize(g_lib.stream));
+    HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, L.stream));
+    HIP_TRY(hipStreamSynchronize(L.stream));
     return 0;
 }
 
-int ntc_hip_memset(void* dst, int value, size_t bytes)
+int ntc_hip_ctx_memset(NtcHipContext* ctx, void* dst, int value, size_t bytes)
 {
-    if (int r = require_init()) return r;
+    CTX_ENTER(ctx);
     if (bytes == 0) return 0;
     if (!dst) { set_error("ntc_hip_memset: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
-    HIP_TRY(launch_fill(static_cast<uint8_t*>(dst), uint8_t(value), bytes, g_lib.stream));    // a kernel, not hipMemsetAsync
+    HIP_TRY(launch_fill(static_cast<uint8_t*>(dst), uint8_t(value), bytes, L.stream));    // a kernel, not hipMemsetAsync
     return 0;
 }
 
-int ntc_hip_synchronize(void)
+int ntc_hip_ctx_synchronize(NtcHipContext* ctx)
 {
-    if (int r = require_init()) return r;
-    HIP_TRY(hipStreamSynchronize(g_lib.stream));
+    CTX_ENTER(ctx);
+    HIP_TRY(hipStreamSynchronize(L.stream));
     return 0;
 }
 
@@ -568,21 +617,21 @@ uint64_t ntc_hip_grid_bytes(int32_t width, int32_t height, int32_t features, int
     return grid_bytes(width, height, features, bits);
 }
 
-int ntc_hip_decode(const NtcHipTextureSet* sets, int32_t numSets)
+int ntc_hip_ctx_decode(NtcHipContext* ctx, const NtcHipTextureSet* sets, int32_t numSets)
 {
-    if (int r = require_init()) return r;
+    CTX_ENTER(ctx);
     std::vector<DevMip> table;
     int variant = NTC_HIP_VARIANT_NONE, totalTiles = 0;
     if (int r = build_table(sets, numSets, table, variant, totalTiles)) return r;
-    if (int r = upload_table(table)) return r;
-    HIP_TRY(launch_decode_any(variant, g_lib.tableDev, int(table.size()), totalTiles, grid_size_for(variant, totalTiles), g_lib.stream));
+    if (int r = upload_table(L, table)) return r;
+    HIP_TRY(launch_decode_any(variant, L.tableDev, int(table.size()), totalTiles, grid_size_for(L, variant, totalTiles), L.stream));
     clear_error();
     return 0;
 }
 
-int ntc_hip_decode_static(const NtcHipTextureSet* sets, int32_t numSets)
+int ntc_hip_ctx_decode_static(NtcHipContext* ctx, const NtcHipTextureSet* sets, int32_t numSets)
 {
-    if (int r = require_init()) return r;
+    CTX_ENTER(ctx);
     std::vector<DevMip> table;
     int variant = NTC_HIP_VARIANT_NONE, totalTiles = 0;
     if (int r = build_table(sets, numSets, table, variant, totalTiles)) return r;
@@ -591,7 +640,6 @@ int ntc_hip_decode_static(const NtcHipTextureSet* sets, int32_t numSets)
                   table.size(), kStaticTableEntries);
         return NTC_HIP_ERR_INVALID_ARG;
     }
-    Library& L = g_lib;
     // The table travels as kernel arguments, a chunk per launch, into this device's built-in array.
     // Stream order keeps a decode that still reads the previous table ahead of these stores.
     for (size_t first = 0; first < table.size(); first += kTableChunkEntries) {
@@ -603,36 +651,36 @@ int ntc_hip_decode_static(const NtcHipTextureSet* sets, int32_t numSets)
                                                     int(count * sizeof(DevMip) / 4));
         HIP_TRY(hipGetLastError());
     }
-    HIP_TRY(launch_decode_any(variant, L.staticTable, int(table.size()), totalTiles, grid_size_for(variant, totalTiles), L.stream));
+    HIP_TRY(launch_decode_any(variant, L.staticTable, int(table.size()), totalTiles, grid_size_for(L, variant, totalTiles), L.stream));
     clear_error();
     return 0;
 }
 
-int ntc_hip_decode_timed(const NtcHipTextureSet* sets, int32_t numSets, int32_t iterations, float* outMs)
+int ntc_hip_ctx_decode_timed(NtcHipContext* ctx, const NtcHipTextureSet* sets, int32_t numSets, int32_t iterations, float* outMs)
 {
-    if (int r = require_init()) return r;
+    CTX_ENTER(ctx);
     if (iterations < 1 || !outMs) { set_error("ntc_hip_decode_timed: iterations must be >= 1 and the result pointer non-null."); return NTC_HIP_ERR_INVALID_ARG; }
     std::vector<DevMip> table;
     int variant = NTC_HIP_VARIANT_NONE, totalTiles = 0;
     if (int r = build_table(sets, numSets, table, variant, totalTiles)) return r;
-    if (int r = upload_table(table)) return r;
-    int const grid = grid_size_for(variant, totalTiles);
-    HIP_TRY(hipEventRecord(g_lib.evStart, g_lib.stream));
+    if (int r = upload_table(L, table)) return r;
+    int const grid = grid_size_for(L, variant, totalTiles);
+    HIP_TRY(hipEventRecord(L.evStart, L.stream));
     for (int i = 0; i < iterations; ++i)
-        HIP_TRY(launch_decode_any(variant, g_lib.tableDev, int(table.size()), totalTiles, grid, g_lib.stream));
-    HIP_TRY(hipEventRecord(g_lib.evStop, g_lib.stream));
-    HIP_TRY(hipEventSynchronize(g_lib.evStop));
+        HIP_TRY(launch_decode_any(variant, L.tableDev, int(table.size()), totalTiles, grid, L.stream));
+    HIP_TRY(hipEventRecord(L.evStop, L.stream));
+    HIP_TRY(hipEventSynchronize(L.evStop));
     float ms = 0.f;
-    HIP_TRY(hipEventElapsedTime(&ms, g_lib.evStart, g_lib.evStop));
+    HIP_TRY(hipEventElapsedTime(&ms, L.evStart, L.evStop));
     *outMs = ms / float(iterations);
     clear_error();
     return 0;
 }
 
-static int run_queries(const NtcHipTextureSet* set, const NtcHipQuery* queries, uint64_t numQueries, void* out, uint64_t outBytes,
+static int run_queries(NtcHipContext* ctx, const NtcHipTextureSet* set, const NtcHipQuery* queries, uint64_t numQueries, void* out, uint64_t outBytes,
                        int iterations, float* outMs)
 {
-    if (int r = require_init()) return r;
+    CTX_ENTER(ctx);
     if (!set || !queries || !out) { set_error("ntc_hip_decode_queries: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
     if (numQueries == 0) { if (outMs) *outMs = 0.f; return 0; }
     if (numQueries > (uint64_t(1) << 40)) { set_error("ntc_hip_decode_queries: too many queries in one call."); return NTC_HIP_ERR_INVALID_ARG; }
@@ -642,19 +690,19 @@ static int run_queries(const NtcHipTextureSet* set, const NtcHipQuery* queries, 
     int variant = NTC_HIP_VARIANT_NONE, totalTiles = 0;
     if (int r = build_table(set, 1, table, variant, totalTiles, true)) return r;
     if (variant_is_fp8_network(variant)) { set_error("ntc_hip_decode_queries: the FP8 network is available to ntc_hip_decode only."); return NTC_HIP_ERR_UNSUPPORTED; }
-    if (int r = upload_table(table)) return r;
+    if (int r = upload_table(L, table)) return r;
     uint64_t const blocks = (numQueries + 255) / 256;
-    uint64_t const resident = uint64_t(g_lib.computeUnits) * uint64_t(grid_size_for(variant, 0x7fffffff) / g_lib.computeUnits);
+    uint64_t const resident = uint64_t(L.computeUnits) * uint64_t(grid_size_for(L, variant, 0x7fffffff) / L.computeUnits);
     int const grid = int(blocks < resident ? blocks : resident);
-    if (outMs) HIP_TRY(hipEventRecord(g_lib.evStart, g_lib.stream));
+    if (outMs) HIP_TRY(hipEventRecord(L.evStart, L.stream));
     for (int i = 0; i < iterations; ++i)
-        HIP_TRY(launch_queries(variant, g_lib.tableDev, int(table.size()), reinterpret_cast<DevQuery const*>(queries), numQueries,
-                               static_cast<uint16_t*>(out), grid, g_lib.stream));
+        HIP_TRY(launch_queries(variant, L.tableDev, int(table.size()), reinterpret_cast<DevQuery const*>(queries), numQueries,
+                               static_cast<uint16_t*>(out), grid, L.stream));
     if (outMs) {
-        HIP_TRY(hipEventRecord(g_lib.evStop, g_lib.stream));
-        HIP_TRY(hipEventSynchronize(g_lib.evStop));
+        HIP_TRY(hipEventRecord(L.evStop, L.stream));
+        HIP_TRY(hipEventSynchronize(L.evStop));
         float ms = 0.f;
-        HIP_TRY(hipEventElapsedTime(&ms, g_lib.evStart, g_lib.evStop));
+        HIP_TRY(hipEventElapsedTime(&ms, L.evStart, L.evStop));
         *outMs = ms / float(iterations);
     }
     clear_error();
@@ -668,9 +716,9 @@ uint64_t ntc_hip_query_latents_bytes(const NtcHipTextureSet* set)
     return plan.totalBytes;
 }
 
-int ntc_hip_build_query_latents(const NtcHipTextureSet* set, void* dst, uint64_t dstBytes)
+int ntc_hip_ctx_build_query_latents(NtcHipContext* ctx, const NtcHipTextureSet* set, void* dst, uint64_t dstBytes)
 {
-    if (int r = require_init()) return r;
+    CTX_ENTER(ctx);
     if (!set || !dst || !set->latents) { set_error("ntc_hip_build_query_latents: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
     BrickPlan plan;
     if (!plan_bricks(*set, plan)) { set_error("ntc_hip_build_query_latents: malformed texture set."); return NTC_HIP_ERR_INVALID_ARG; }
@@ -688,21 +736,20 @@ int ntc_hip_build_query_latents(const NtcHipTextureSet* set, void* dst, uint64_t
     // (bricks of grids narrower than a brick keep cells that nothing writes and no query reads)
     for (BrickGrid const& g : plan.grids)
         HIP_TRY(launch_build_bricks(reinterpret_cast<uint16_t const*>(static_cast<uint8_t const*>(set->latents) + g.srcOffset),
-                                    static_cast<uint8_t*>(dst) + g.dstOffset, g.width, g.height, g.layers, g_lib.stream));
+                                    static_cast<uint8_t*>(dst) + g.dstOffset, g.width, g.height, g.layers, L.stream));
     clear_error();
     return 0;
 }
 
-int ntc_hip_decode_queries(const NtcHipTextureSet* set, const NtcHipQuery* queries, uint64_t numQueries, void* out, uint64_t outBytes)
+int ntc_hip_ctx_decode_queries(NtcHipContext* ctx, const NtcHipTextureSet* set, const NtcHipQuery* queries, uint64_t numQueries, void* out, uint64_t outBytes)
 {
-    return run_queries(set, queries, numQueries, out, outBytes, 1, nullptr);
+    return run_queries(ctx, set, queries, numQueries, out, outBytes, 1, nullptr);
 }
 
-int ntc_hip_decode_queries_timed(const NtcHipTextureSet* set, const NtcHipQuery* queries, uint64_t numQueries, void* out, uint64_t outBytes,
-                                 int32_t iterations, float* outMillisecondsPerIteration)
+int ntc_hip_ctx_decode_queries_timed(NtcHipContext* ctx, const NtcHipTextureSet* set, const NtcHipQuery* queries, uint64_t numQueries, void* out, uint64_t outBytes, int32_t iterations, float* outMillisecondsPerIteration)
 {
     if (iterations < 1 || !outMillisecondsPerIteration) { set_error("ntc_hip_decode_queries_timed: iterations must be >= 1 and the result pointer non-null."); return NTC_HIP_ERR_INVALID_ARG; }
-    return run_queries(set, queries, numQueries, out, outBytes, iterations, outMillisecondsPerIteration);
+    return run_queries(ctx, set, queries, numQueries, out, outBytes, iterations, outMillisecondsPerIteration);
 }
 
 // Largest power of two up to 16 that divides the base address, the row pitch and the pixel stride:
@@ -713,9 +760,9 @@ static int32_t common_alignment(uintptr_t base, uint64_t rowPitch, uint64_t pixe
     return int32_t(bits & (~bits + 1));
 }
 
-int ntc_hip_read_channels(const NtcHipReadChannels* p)
+int ntc_hip_ctx_read_channels(NtcHipContext* ctx, const NtcHipReadChannels* p)
 {
-    if (int r = require_init()) return r;
+    CTX_ENTER(ctx);
     if (!p || !p->planarPairs || !p->dst) { set_error("ntc_hip_read_channels: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
     int bpc = 0;
     switch (p->format) {
@@ -763,7 +810,7 @@ int ntc_hip_read_channels(const NtcHipReadChannels* p)
         a.srcColorSpaces[i] = p->srcColorSpaces[i];
         a.dstColorSpaces[i] = p->dstColorSpaces[i];
     }
-    HIP_TRY(launch_read_channels(a, g_lib.stream));
+    HIP_TRY(launch_read_channels(a, L.stream));
     clear_error();
     return 0;
 }
@@ -778,9 +825,9 @@ static int bytes_per_component(int format)
     }
 }
 
-int ntc_hip_write_channels(const NtcHipWriteChannels* p)
+int ntc_hip_ctx_write_channels(NtcHipContext* ctx, const NtcHipWriteChannels* p)
 {
-    if (int r = require_init()) return r;
+    CTX_ENTER(ctx);
     if (!p || !p->src || !p->planarPairs) { set_error("ntc_hip_write_channels: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
     int const bpc = bytes_per_component(p->format);
     if (!bpc) { set_error("ntc_hip_write_channels: unknown channel format %d.", p->format); return NTC_HIP_ERR_INVALID_ARG; }
@@ -816,16 +863,14 @@ int ntc_hip_write_channels(const NtcHipWriteChannels* p)
         a.srcColorSpaces[i] = p->srcColorSpaces[i];
         a.dstColorSpaces[i] = p->dstColorSpaces[i];
     }
-    HIP_TRY(launch_write_channels(a, g_lib.stream));
+    HIP_TRY(launch_write_channels(a, L.stream));
     clear_error();
     return 0;
 }
 
-int ntc_hip_image_loss(void* decoded, const void* reference, uint64_t planarBytes, int32_t width, int32_t height,
-                       int32_t setChannels, uint32_t validChannelMask, int32_t maskChannelIndex, int32_t discardMaskedOutPixels,
-                       float* outMse)
+int ntc_hip_ctx_image_loss(NtcHipContext* ctx, void* decoded, const void* reference, uint64_t planarBytes, int32_t width, int32_t height, int32_t setChannels, uint32_t validChannelMask, int32_t maskChannelIndex, int32_t discardMaskedOutPixels, float* outMse)
 {
-    if (int r = require_init()) return r;
+    CTX_ENTER(ctx);
     if (!decoded || !reference || !outMse) { set_error("ntc_hip_image_loss: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
     if (width < 1 || height < 1 || setChannels < 2 || (setChannels & 1) || setChannels > NTC_HIP_MAX_CHANNELS
         || uint64_t(width) * uint64_t(height) * uint64_t(setChannels) * 2u > planarBytes) {
@@ -846,7 +891,6 @@ int ntc_hip_image_loss(void* decoded, const void* reference, uint64_t planarByte
     }
     size_t const blocks = image_loss_blocks(width, height);
     size_t const bytes = (blocks + 1) * NTC_HIP_DEV_MAX_CHANNELS * sizeof(double);    // partial sums, then the 16 totals
-    Library& L = g_lib;
     if (bytes > L.lossBytes) {
         HIP_TRY(hipStreamSynchronize(L.stream));
         if (L.lossDev) { HIP_TRY(hipFree(L.lossDev)); L.lossDev = nullptr; }
@@ -867,11 +911,9 @@ int ntc_hip_image_loss(void* decoded, const void* reference, uint64_t planarByte
     return 0;
 }
 
-int ntc_hip_resize_planar(const void* src, uint64_t srcBytes, int32_t srcWidth, int32_t srcHeight,
-                          void* dst, uint64_t dstBytes, int32_t dstWidth, int32_t dstHeight,
-                          int32_t setChannels, const uint8_t* channelColorSpaces)
+int ntc_hip_ctx_resize_planar(NtcHipContext* ctx, const void* src, uint64_t srcBytes, int32_t srcWidth, int32_t srcHeight, void* dst, uint64_t dstBytes, int32_t dstWidth, int32_t dstHeight, int32_t setChannels, const uint8_t* channelColorSpaces)
 {
-    if (int r = require_init()) return r;
+    CTX_ENTER(ctx);
     if (!src || !dst) { set_error("ntc_hip_resize_planar: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
     if (srcWidth < 1 || srcHeight < 1 || dstWidth < 1 || dstHeight < 1 || setChannels < 2 || (setChannels & 1) || setChannels > NTC_HIP_MAX_CHANNELS) {
         set_error("ntc_hip_resize_planar: bad image shape.");
@@ -887,7 +929,7 @@ int ntc_hip_resize_planar(const void* src, uint64_t srcBytes, int32_t srcWidth, 
         for (int i = 0; i < 16; ++i)
             if (channelColorSpaces[i] > 2) { set_error("ntc_hip_resize_planar: unknown colour space for channel %d.", i); return NTC_HIP_ERR_INVALID_ARG; }
     HIP_TRY(launch_resize_planar(static_cast<uint16_t const*>(src), srcWidth, srcHeight, static_cast<uint16_t*>(dst), dstWidth, dstHeight,
-                                 setChannels, channelColorSpaces, g_lib.stream));
+                                 setChannels, channelColorSpaces, L.stream));
     clear_error();
     return 0;
 }
@@ -915,9 +957,9 @@ static int check_diff_image(NtcHipImage const& im, char const* which, int left, 
     return 0;
 }
 
-int ntc_hip_image_difference(const NtcHipImageDifference* p)
+int ntc_hip_ctx_image_difference(NtcHipContext* ctx, const NtcHipImageDifference* p)
 {
-    if (int r = require_init()) return r;
+    CTX_ENTER(ctx);
     if (!p || !p->output) { set_error("ntc_hip_image_difference: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
     // src/Context.cpp:796-812
     if (p->left < 0 || p->top < 0) { set_error("ntc_hip_image_difference: left (%d) and top (%d) must be non-negative.", p->left, p->top); return NTC_HIP_ERR_INVALID_ARG; }
@@ -935,14 +977,14 @@ int ntc_hip_image_difference(const NtcHipImageDifference* p)
     a.left = p->left; a.top = p->top; a.width = p->width; a.height = p->height;
     a.alphaThreshold = p->alphaThreshold; a.useAlphaThreshold = p->useAlphaThreshold ? 1 : 0; a.useMSLE = p->useMSLE ? 1 : 0;
     a.output = reinterpret_cast<unsigned long long*>(static_cast<uint8_t*>(p->output) + p->outputOffset);
-    HIP_TRY(launch_image_difference(a, g_lib.stream));
+    HIP_TRY(launch_image_difference(a, L.stream));
     clear_error();
     return 0;
 }
 
-int ntc_hip_block_compress(const NtcHipBlockCompress* p)
+int ntc_hip_ctx_block_compress(NtcHipContext* ctx, const NtcHipBlockCompress* p)
 {
-    if (int r = require_init()) return r;
+    CTX_ENTER(ctx);
     if (!p || !p->dst) { set_error("ntc_hip_block_compress: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
     if (p->dstFormat < 1 || p->dstFormat > 7) { set_error("ntc_hip_block_compress: dstFormat (%d) is not a block-compressed format.", p->dstFormat); return NTC_HIP_ERR_INVALID_ARG; }
     if (p->srcLeft < 0 || p->srcTop < 0 || p->widthInBlocks < 1 || p->heightInBlocks < 1 || p->dstOffsetX < 0 || p->dstOffsetY < 0
@@ -985,14 +1027,15 @@ int ntc_hip_block_compress(const NtcHipBlockCompress* p)
         a.modeMapWidthInBlocks = p->modeMapWidthInBlocks; a.modeMapHeightInBlocks = p->modeMapHeightInBlocks;
         a.modeMapOffsetX = p->modeMapOffsetX; a.modeMapOffsetY = p->modeMapOffsetY;
     }
-    HIP_TRY(launch_block_compress(a, p->dstFormat, g_lib.stream));
+    HIP_TRY(launch_block_compress(a, p->dstFormat, L.stream));
     clear_error();
     return 0;
 }
 
 int ntc_hip_selftest_mfma(const int8_t* a16x64, const int8_t* b64x16, int32_t* d16x16)
 {
-    if (int r = require_init()) return r;
+    NtcHipContext* const ctx = g_default;
+    CTX_ENTER(ctx);
     if (!a16x64 || !b64x16 || !d16x16) { set_error("ntc_hip_selftest_mfma: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
     int8_t *a = nullptr, *b = nullptr; int32_t* d = nullptr;
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&a), 1024));
@@ -1000,8 +1043,8 @@ int ntc_hip_selftest_mfma(const int8_t* a16x64, const int8_t* b64x16, int32_t* d
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&d), 1024));
     HIP_TRY(hipMemcpy(a, a16x64, 1024, hipMemcpyHostToDevice));
     HIP_TRY(hipMemcpy(b, b64x16, 1024, hipMemcpyHostToDevice));
-    HIP_TRY(launch_selftest_mfma(a, b, d, g_lib.stream));
-    HIP_TRY(hipStreamSynchronize(g_lib.stream));
+    HIP_TRY(launch_selftest_mfma(a, b, d, L.stream));
+    HIP_TRY(hipStreamSynchronize(L.stream));
     HIP_TRY(hipMemcpy(d16x16, d, 1024, hipMemcpyDeviceToHost));
     (void)hipFree(a); (void)hipFree(b); (void)hipFree(d);
     return 0;
@@ -1009,13 +1052,14 @@ int ntc_hip_selftest_mfma(const int8_t* a16x64, const int8_t* b64x16, int32_t* d
 
 int ntc_hip_selftest_fp8_activation(const uint16_t* halves, int32_t count, uint16_t* out)
 {
-    if (int r = require_init()) return r;
+    NtcHipContext* const ctx = g_default;
+    CTX_ENTER(ctx);
     if (!halves || !out || count < 1 || count > (1 << 20)) { set_error("ntc_hip_selftest_fp8_activation: null pointer or count outside 1..2^20."); return NTC_HIP_ERR_INVALID_ARG; }
     uint16_t* dev = nullptr;
     HIP_TRY(hipMalloc(reinterpret_cast<void**>(&dev), size_t(count) * 8));
     hipError_t e = hipMemcpy(dev, halves, size_t(count) * 2, hipMemcpyHostToDevice);
-    if (e == hipSuccess) e = launch_selftest_fp8_activation(dev, dev + count, count, g_lib.stream);
-    if (e == hipSuccess) e = hipStreamSynchronize(g_lib.stream);
+    if (e == hipSuccess) e = launch_selftest_fp8_activation(dev, dev + count, count, L.stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(L.stream);
     if (e == hipSuccess) e = hipMemcpy(out, dev + count, size_t(count) * 6, hipMemcpyDeviceToHost);
     (void)hipFree(dev);
     HIP_TRY(e);
@@ -1024,7 +1068,8 @@ int ntc_hip_selftest_fp8_activation(const uint16_t* halves, int32_t count, uint1
 
 int ntc_hip_selftest_mfma_f16(const uint16_t* aHalves, const uint16_t* bHalves, const float* c16x16, float* d16x16, int32_t depth)
 {
-    if (int r = require_init()) return r;
+    NtcHipContext* const ctx = g_default;
+    CTX_ENTER(ctx);
     if (!aHalves || !bHalves || !c16x16 || !d16x16) { set_error("ntc_hip_selftest_mfma_f16: null pointer."); return NTC_HIP_ERR_INVALID_ARG; }
     if (depth != 16 && depth != 32) { set_error("ntc_hip_selftest_mfma_f16: depth must be 16 or 32."); return NTC_HIP_ERR_INVALID_ARG; }
     size_t const operandBytes = size_t(16) * size_t(depth) * 2;
@@ -1037,12 +1082,34 @@ int ntc_hip_selftest_mfma_f16(const uint16_t* aHalves, const uint16_t* bHalves, 
     hipError_t e = hipMemcpy(a, aHalves, operandBytes, hipMemcpyHostToDevice);
     if (e == hipSuccess) e = hipMemcpy(b, bHalves, operandBytes, hipMemcpyHostToDevice);
     if (e == hipSuccess) e = hipMemcpy(c, c16x16, 1024, hipMemcpyHostToDevice);
-    if (e == hipSuccess) e = launch_selftest_mfma_f16(a, b, c, d, depth, g_lib.stream);
-    if (e == hipSuccess) e = hipStreamSynchronize(g_lib.stream);
+    if (e == hipSuccess) e = launch_selftest_mfma_f16(a, b, c, d, depth, L.stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(L.stream);
     if (e == hipSuccess) e = hipMemcpy(d16x16, d, 1024, hipMemcpyDeviceToHost);
     (void)hipFree(dev);
     HIP_TRY(e);
     return 0;
 }
+
+// ---- the same entry points on the context ntc_hip_init created
+int ntc_hip_device_info(char* name, size_t nameSize, int* computeUnits) { return ntc_hip_ctx_device_info(g_default, name, nameSize, computeUnits); }
+int ntc_hip_device_clock(int* clockRateKHz) { return ntc_hip_ctx_device_clock(g_default, clockRateKHz); }
+int ntc_hip_alloc(void** devPtr, size_t bytes) { return ntc_hip_ctx_alloc(g_default, devPtr, bytes); }
+int ntc_hip_free(void* devPtr) { return ntc_hip_ctx_free(g_default, devPtr); }
+int ntc_hip_upload(void* dst, const void* src, size_t bytes) { return ntc_hip_ctx_upload(g_default, dst, src, bytes); }
+int ntc_hip_download(void* dst, const void* src, size_t bytes) { return ntc_hip_ctx_download(g_default, dst, src, bytes); }
+int ntc_hip_memset(void* dst, int value, size_t bytes) { return ntc_hip_ctx_memset(g_default, dst, value, bytes); }
+int ntc_hip_synchronize(void) { return ntc_hip_ctx_synchronize(g_default); }
+int ntc_hip_decode(const NtcHipTextureSet* sets, int32_t numSets) { return ntc_hip_ctx_decode(g_default, sets, numSets); }
+int ntc_hip_decode_static(const NtcHipTextureSet* sets, int32_t numSets) { return ntc_hip_ctx_decode_static(g_default, sets, numSets); }
+int ntc_hip_decode_timed(const NtcHipTextureSet* sets, int32_t numSets, int32_t iterations, float* outMs) { return ntc_hip_ctx_decode_timed(g_default, sets, numSets, iterations, outMs); }
+int ntc_hip_build_query_latents(const NtcHipTextureSet* set, void* dst, uint64_t dstBytes) { return ntc_hip_ctx_build_query_latents(g_default, set, dst, dstBytes); }
+int ntc_hip_decode_queries(const NtcHipTextureSet* set, const NtcHipQuery* queries, uint64_t numQueries, void* out, uint64_t outBytes) { return ntc_hip_ctx_decode_queries(g_default, set, queries, numQueries, out, outBytes); }
+int ntc_hip_decode_queries_timed(const NtcHipTextureSet* set, const NtcHipQuery* queries, uint64_t numQueries, void* out, uint64_t outBytes, int32_t iterations, float* outMillisecondsPerIteration) { return ntc_hip_ctx_decode_queries_timed(g_default, set, queries, numQueries, out, outBytes, iterations, outMillisecondsPerIteration); }
+int ntc_hip_read_channels(const NtcHipReadChannels* p) { return ntc_hip_ctx_read_channels(g_default, p); }
+int ntc_hip_write_channels(const NtcHipWriteChannels* p) { return ntc_hip_ctx_write_channels(g_default, p); }
+int ntc_hip_image_loss(void* decoded, const void* reference, uint64_t planarBytes, int32_t width, int32_t height, int32_t setChannels, uint32_t validChannelMask, int32_t maskChannelIndex, int32_t discardMaskedOutPixels, float* outMse) { return ntc_hip_ctx_image_loss(g_default, decoded, reference, planarBytes, width, height, setChannels, validChannelMask, maskChannelIndex, discardMaskedOutPixels, outMse); }
+int ntc_hip_resize_planar(const void* src, uint64_t srcBytes, int32_t srcWidth, int32_t srcHeight, void* dst, uint64_t dstBytes, int32_t dstWidth, int32_t dstHeight, int32_t setChannels, const uint8_t* channelColorSpaces) { return ntc_hip_ctx_resize_planar(g_default, src, srcBytes, srcWidth, srcHeight, dst, dstBytes, dstWidth, dstHeight, setChannels, channelColorSpaces); }
+int ntc_hip_image_difference(const NtcHipImageDifference* p) { return ntc_hip_ctx_image_difference(g_default, p); }
+int ntc_hip_block_compress(const NtcHipBlockCompress* p) { return ntc_hip_ctx_block_compress(g_default, p); }
 
 } // extern "C"

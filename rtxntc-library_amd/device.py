@@ -7,19 +7,38 @@ from . import abi, presets
 
 
 class Device:
-    """ntc_hip_init on construction; raises NtcHipError when there is no gfx950 device."""
+    """The library's default context (ntc_hip_init) or, with own_context=True, a context of its own
+    (ntc_hip_create: its own stream and working memory); raises NtcHipError when there is no gfx950 device."""
 
-    def __init__(self, index=0):
+    def __init__(self, index=0, own_context=False):
         self.lib = abi.load_library()
-        abi.check(self.lib.ntc_hip_init(index))
+        self.ctx = None
+        if own_context:
+            handle = C.c_void_p()
+            abi.check(self.lib.ntc_hip_create(index, C.byref(handle)))
+            self.ctx = handle
+        else:
+            abi.check(self.lib.ntc_hip_init(index))
         name = C.create_string_buffer(256)
         cus = C.c_int(0)
-        abi.check(self.lib.ntc_hip_device_info(name, 256, C.byref(cus)))
+        self.call("device_info", name, 256, C.byref(cus))
         self.name = name.value.decode()
         self.compute_units = cus.value
         khz = C.c_int(0)
-        abi.check(self.lib.ntc_hip_device_clock(C.byref(khz)))
+        self.call("device_clock", C.byref(khz))
         self.clock_ghz = khz.value / 1e6
+
+    def call(self, name, *args):
+        """ntc_hip_<name>(args) on the default context, ntc_hip_ctx_<name>(context, args) on an own one."""
+        if self.ctx is None:
+            abi.check(getattr(self.lib, "ntc_hip_" + name)(*args))
+        else:
+            abi.check(getattr(self.lib, "ntc_hip_ctx_" + name)(self.ctx, *args))
+
+    def close(self):
+        if self.ctx is not None:
+            self.lib.ntc_hip_destroy(self.ctx)
+            self.ctx = None
 
     def alloc(self, nbytes):
         return DeviceBuffer(self, nbytes)
@@ -27,11 +46,11 @@ class Device:
     def upload(self, array):
         array = np.ascontiguousarray(array)
         buf = DeviceBuffer(self, array.nbytes)
-        abi.check(self.lib.ntc_hip_upload(buf.ptr, array.ctypes.data, array.nbytes))
+        self.call("upload", buf.ptr, array.ctypes.data, array.nbytes)
         return buf
 
     def synchronize(self):
-        abi.check(self.lib.ntc_hip_synchronize())
+        self.call("synchronize")
 
     @staticmethod
     def pack_sets(sets):
@@ -40,17 +59,17 @@ class Device:
 
     def decode(self, sets):
         arr = self.pack_sets(sets)
-        abi.check(self.lib.ntc_hip_decode(arr, len(arr)))
+        self.call("decode", arr, len(arr))
 
     def decode_static(self, sets):
         """ntc_hip_decode_static: the same decode with the mip table in the library's built-in array."""
         arr = self.pack_sets(sets)
-        abi.check(self.lib.ntc_hip_decode_static(arr, len(arr)))
+        self.call("decode_static", arr, len(arr))
 
     def decode_timed(self, sets, iterations):
         arr = self.pack_sets(sets)
         ms = C.c_float(0)
-        abi.check(self.lib.ntc_hip_decode_timed(arr, len(arr), iterations, C.byref(ms)))
+        self.call("decode_timed", arr, len(arr), iterations, C.byref(ms))
         return ms.value
 
 
@@ -59,26 +78,26 @@ class DeviceBuffer:
         self.device = device
         self.nbytes = int(nbytes)
         p = C.c_void_p()
-        abi.check(device.lib.ntc_hip_alloc(C.byref(p), self.nbytes))
+        device.call("alloc", C.byref(p), self.nbytes)
         self.ptr = p.value
 
     def download(self, dtype=np.uint8):
         out = np.empty(self.nbytes, dtype=np.uint8)
-        abi.check(self.device.lib.ntc_hip_download(out.ctypes.data, self.ptr, self.nbytes))
+        self.device.call("download", out.ctypes.data, self.ptr, self.nbytes)
         return out.view(dtype)
 
     def download_range(self, offset, nbytes, dtype=np.uint8):
         assert 0 <= offset and offset + nbytes <= self.nbytes
         out = np.empty(int(nbytes), dtype=np.uint8)
-        abi.check(self.device.lib.ntc_hip_download(out.ctypes.data, self.ptr + int(offset), int(nbytes)))
+        self.device.call("download", out.ctypes.data, self.ptr + int(offset), int(nbytes))
         return out.view(dtype)
 
     def fill(self, value):
-        abi.check(self.device.lib.ntc_hip_memset(self.ptr, value, self.nbytes))
+        self.device.call("memset", self.ptr, value, self.nbytes)
 
     def free(self):
         if self.ptr:
-            abi.check(self.device.lib.ntc_hip_free(self.ptr))
+            self.device.call("free", self.ptr)
             self.ptr = None
 
     def __del__(self):

@@ -423,12 +423,12 @@ public:
         int const stagingHeight = m_features.stagingHeight > 0 ? m_features.stagingHeight : m_desc.height;
         m_stagingBytes = uint64_t(stagingWidth) * uint64_t(stagingHeight) * uint64_t(std::max(0, m_features.stagingBytesPerPixel));
         if (m_deviceAvailable) {
-            if (int r = ntc_hip_alloc(&m_textureData, m_textureBytes)) return AllocationFailure(r, "texture data", m_textureBytes);
+            if (int r = ntc_hip_ctx_alloc(Hip(), &m_textureData, m_textureBytes)) return AllocationFailure(r, "texture data", m_textureBytes);
             // A second page keeps the reference image apart from the decoded one (src/TextureSet.cpp:103-124).
             if (m_features.separateRefOutData)
-                if (int r = ntc_hip_alloc(&m_textureDataOut, m_textureBytes)) return AllocationFailure(r, "texture data (output)", m_textureBytes);
+                if (int r = ntc_hip_ctx_alloc(Hip(), &m_textureDataOut, m_textureBytes)) return AllocationFailure(r, "texture data (output)", m_textureBytes);
             if (m_stagingBytes)
-                if (int r = ntc_hip_alloc(&m_staging, m_stagingBytes)) return AllocationFailure(r, "staging", m_stagingBytes);
+                if (int r = ntc_hip_ctx_alloc(Hip(), &m_staging, m_stagingBytes)) return AllocationFailure(r, "staging", m_stagingBytes);
         }
         return Status::Ok;
     }
@@ -1005,7 +1005,7 @@ public:
         bool const lossPass = validMask != 0 && (pOutStats || m_maskChannelIndex >= 0);
         bool const lazyOutPage = lossPass && !m_textureDataOut;
         if (lazyOutPage)
-            if (int r = ntc_hip_alloc(&m_textureDataOut, m_textureBytes)) return AllocationFailure(r, "texture data (output)", m_textureBytes);
+            if (int r = ntc_hip_ctx_alloc(Hip(), &m_textureDataOut, m_textureBytes)) return AllocationFailure(r, "texture data (output)", m_textureBytes);
         void* const outPage = m_textureDataOut ? m_textureDataOut : m_textureData;   // src/TextureSet.cpp:1799-1802
 
         NtcHipTextureSet set{};
@@ -1026,9 +1026,9 @@ public:
         // for, and otherwise returns without waiting (src/TextureSet.cpp:1772-1780,1866-1882).
         if (pOutStats) {
             float ms = 0.f;
-            if (int r = ntc_hip_decode_timed(&set, 1, 1, &ms)) return DeviceFailure(r);
+            if (int r = ntc_hip_ctx_decode_timed(Hip(), &set, 1, 1, &ms)) return DeviceFailure(r);
             pOutStats->gpuTimeMilliseconds = ms;
-        } else if (int r = ntc_hip_decode(&set, 1)) {
+        } else if (int r = ntc_hip_ctx_decode(Hip(), &set, 1)) {
             return DeviceFailure(r);
         }
 
@@ -1042,7 +1042,7 @@ public:
             for (int mip = 0; mip < m_desc.mips; ++mip) {
                 uint64_t const offset = m_mipOffsets[mip] * uint64_t(m_desc.channels) * 2u;
                 float mse[16];
-                if (int r = ntc_hip_image_loss(static_cast<uint8_t*>(outPage) + offset, static_cast<uint8_t const*>(m_textureData) + offset,
+                if (int r = ntc_hip_ctx_image_loss(Hip(), static_cast<uint8_t*>(outPage) + offset, static_cast<uint8_t const*>(m_textureData) + offset,
                                                m_textureBytes - offset, m_mips[mip].width, m_mips[mip].height, m_desc.channels, validMask,
                                                m_maskChannelIndex < 0 ? -1 : m_maskChannelIndex, m_discardMaskedOutPixels ? 1 : 0, mse))
                     return DeviceFailure(r);
@@ -1067,7 +1067,7 @@ public:
         // Without separateRefOutData both pages are one memory in the reference and the decode
         // overwrites the reference image; keep that: the decoded page becomes the only page.
         if (lazyOutPage) {
-            if (int r = ntc_hip_synchronize()) return DeviceFailure(r);
+            if (int r = ntc_hip_ctx_synchronize(Hip())) return DeviceFailure(r);
             std::swap(m_textureData, m_textureDataOut);
             ReleaseDevice(m_textureDataOut);
         }
@@ -1087,7 +1087,7 @@ public:
             return st;
         if (!m_deviceAvailable) { SetErrorMessage("No HIP device is available to this context."); return Status::CudaUnavailable; }
         if (fromHost)
-            if (int r = ntc_hip_upload(m_staging, params.pData, sizeToCopy)) return DeviceFailure(r);
+            if (int r = ntc_hip_ctx_upload(Hip(), m_staging, params.pData, sizeToCopy)) return DeviceFailure(r);
         int const mipWidth = std::max(m_desc.width >> params.mipLevel, 1), mipHeight = std::max(m_desc.height >> params.mipLevel, 1);
         NtcHipWriteChannels wc{};
         wc.src = fromHost ? m_staging : static_cast<void const*>(params.pData);
@@ -1109,7 +1109,7 @@ public:
             wc.dstColorSpaces[channel] = uint8_t(storage);
             m_channelColorSpaces[channel + params.firstChannel] = storage;       // src/TextureSet.cpp:899-902
         }
-        if (int r = ntc_hip_write_channels(&wc)) return DeviceFailure(r);
+        if (int r = ntc_hip_ctx_write_channels(Hip(), &wc)) return DeviceFailure(r);
         ClearErrorMessage();
         return Status::Ok;
     }
@@ -1128,7 +1128,7 @@ public:
 
         // Rows the copy does not fully overwrite must not carry garbage to the client (src/TextureSet.cpp:936-946).
         if (toHost && params.rowPitch > params.pixelStride * size_t(params.width))
-            if (int r = ntc_hip_memset(m_staging, 0, sizeToCopy)) return DeviceFailure(r);
+            if (int r = ntc_hip_ctx_memset(Hip(), m_staging, 0, sizeToCopy)) return DeviceFailure(r);
 
         NtcHipReadChannels rc{};
         // GetTextureDataSlice: the output page when it exists and is asked for (src/TextureSet.cpp:1961-1964)
@@ -1150,9 +1150,9 @@ public:
             rc.srcColorSpaces[channel] = uint8_t(m_channelColorSpaces[channel + params.firstChannel]);
             rc.dstColorSpaces[channel] = uint8_t(wanted);
         }
-        if (int r = ntc_hip_read_channels(&rc)) return DeviceFailure(r);
+        if (int r = ntc_hip_ctx_read_channels(Hip(), &rc)) return DeviceFailure(r);
         if (toHost)
-            if (int r = ntc_hip_download(params.pOutData, m_staging, sizeToCopy)) return DeviceFailure(r);
+            if (int r = ntc_hip_ctx_download(Hip(), params.pOutData, m_staging, sizeToCopy)) return DeviceFailure(r);
         ClearErrorMessage();
         return Status::Ok;
     }
@@ -1167,7 +1167,7 @@ public:
         for (int ch = 0; ch < NTC_HIP_MAX_CHANNELS; ++ch) spaces[ch] = uint8_t(m_channelColorSpaces[ch]);
         for (int mip = 1; mip < m_desc.mips; ++mip) {
             uint64_t const srcOffset = m_mipOffsets[mip - 1] * uint64_t(m_desc.channels) * 2u, dstOffset = m_mipOffsets[mip] * uint64_t(m_desc.channels) * 2u;
-            if (int r = ntc_hip_resize_planar(static_cast<uint8_t const*>(m_textureData) + srcOffset, dstOffset - srcOffset,
+            if (int r = ntc_hip_ctx_resize_planar(Hip(), static_cast<uint8_t const*>(m_textureData) + srcOffset, dstOffset - srcOffset,
                                               std::max(m_desc.width >> (mip - 1), 1), std::max(m_desc.height >> (mip - 1), 1),
                                               static_cast<uint8_t*>(m_textureData) + dstOffset, m_textureBytes - dstOffset,
                                               std::max(m_desc.width >> mip, 1), std::max(m_desc.height >> mip, 1), m_desc.channels, spaces))
@@ -1329,7 +1329,7 @@ private:
         return DeviceFailure(code);
     }
 
-    void ReleaseDevice(void*& p) { if (p) { (void)ntc_hip_free(p); p = nullptr; } }
+    void ReleaseDevice(void*& p) { if (p) { (void)ntc_hip_ctx_free(Hip(), p); p = nullptr; } }
 
     Status ResetShape()
     {
@@ -1365,10 +1365,10 @@ private:
         m_latentFootprints.clear();
         m_haveLatents = m_haveWeights = m_haveWeightsFP8 = false;
         if (m_deviceAvailable) {
-            if (int r = ntc_hip_alloc(&m_latents, m_latentBytes)) return AllocationFailure(r, "latent", m_latentBytes);
-            if (int r = ntc_hip_alloc(&m_weights, m_weightLayout.bufferSize)) return AllocationFailure(r, "MLP weights", m_weightLayout.bufferSize);
+            if (int r = ntc_hip_ctx_alloc(Hip(), &m_latents, m_latentBytes)) return AllocationFailure(r, "latent", m_latentBytes);
+            if (int r = ntc_hip_ctx_alloc(Hip(), &m_weights, m_weightLayout.bufferSize)) return AllocationFailure(r, "MLP weights", m_weightLayout.bufferSize);
             if (m_weightLayoutFP8.bufferSize)
-                if (int r = ntc_hip_alloc(&m_weightsFP8, m_weightLayoutFP8.bufferSize)) return AllocationFailure(r, "MLP weights (FP8)", m_weightLayoutFP8.bufferSize);
+                if (int r = ntc_hip_ctx_alloc(Hip(), &m_weightsFP8, m_weightLayoutFP8.bufferSize)) return AllocationFailure(r, "MLP weights (FP8)", m_weightLayoutFP8.bufferSize);
         }
         m_state = NetworkState::Initialized;
         ClearErrorMessage();
@@ -1427,7 +1427,7 @@ private:
         if (!data) { SetErrorMessage("The %s data pointer is NULL.", what); return Status::InvalidArgument; }
         if (size != expected) { SetErrorMessage("The %s data must be %llu bytes, got %zu.", what, (unsigned long long)expected, size); return Status::InvalidArgument; }
         if (!m_deviceAvailable) { SetErrorMessage("No HIP device is available to this context."); return Status::CudaUnavailable; }
-        if (int r = ntc_hip_upload(device, data, size)) return DeviceFailure(r);
+        if (int r = ntc_hip_ctx_upload(Hip(), device, data, size)) return DeviceFailure(r);
         have = true;
         if (m_haveLatents && (m_haveWeights || m_haveWeightsFP8)) m_state = NetworkState::Complete;
         ClearErrorMessage();
@@ -1435,6 +1435,7 @@ private:
     }
 
     IAllocator* Allocator() const;      // the context's
+    NtcHipContext* Hip() const;         // the context's device context (null without a device)
 
     Context const* m_context;
     TextureSetDesc m_desc;
@@ -1469,8 +1470,11 @@ private:
 class Context final : public IContext, public amd::IContextExtension
 {
 public:
-    Context(IAllocator* allocator, bool deviceAvailable) : m_allocator(allocator), m_deviceAvailable(deviceAvailable) {}
+    // `hip`: this context's device, stream and working memory (null: no device); owned.
+    Context(IAllocator* allocator, NtcHipContext* hip) : m_allocator(allocator), m_hip(hip), m_deviceAvailable(hip != nullptr) {}
+    ~Context() override { ntc_hip_destroy(m_hip); }
     IAllocator* GetAllocator() const { return m_allocator; }
+    NtcHipContext* GetHip() const { return m_hip; }
 
     // src/Context.cpp:177-218 with the descriptor rules of src/TextureSetMetadata.cpp:1161-1178
     Status CreateTextureSet(TextureSetDesc const& desc, TextureSetFeatures const& features, ITextureSet** pOutTextureSet) const override
@@ -1493,6 +1497,13 @@ public:
 
     void DestroyTextureSet(ITextureSet* textureSet) const override { DestroyObject(m_allocator, dynamic_cast<TextureSet*>(textureSet)); }
     bool IsDeviceAvailable() const override { return m_deviceAvailable; }
+    Status Synchronize() const override
+    {
+        if (!m_deviceAvailable) { ClearErrorMessage(); return Status::Ok; }
+        if (int r = ntc_hip_ctx_synchronize(m_hip)) return DeviceFailure(r);
+        ClearErrorMessage();
+        return Status::Ok;
+    }
     void AllowTextureSetsWithoutDevice(bool allow) const override { m_allowSetsWithoutDevice = allow; }
 
     // ---- outside the decompression path ----
@@ -1585,7 +1596,7 @@ public:
         p.modeBuffer = params.pModeBuffer; p.modeBufferBytes = params.modeBufferSize; p.modeBufferByteOffset = params.modeBufferByteOffset;
         p.modeMapWidthInBlocks = params.modeMapWidthInBlocks; p.modeMapHeightInBlocks = params.modeMapHeightInBlocks;
         p.modeMapOffsetX = params.modeMapOffsetInBlocks.x; p.modeMapOffsetY = params.modeMapOffsetInBlocks.y;
-        if (int r = ntc_hip_block_compress(&p)) return DeviceFailure(r);
+        if (int r = ntc_hip_ctx_block_compress(m_hip, &p)) return DeviceFailure(r);
         ClearErrorMessage();
         return Status::Ok;
     }
@@ -1621,7 +1632,7 @@ public:
         p.useMSLE = params.useMSLE ? 1 : 0;
         p.outputOffset = params.outputOffset;
         p.output = params.pOutputBuffer; p.outputBytes = params.outputBufferSize;
-        if (int r = ntc_hip_image_difference(&p)) return DeviceFailure(r);
+        if (int r = ntc_hip_ctx_image_difference(m_hip, &p)) return DeviceFailure(r);
         ClearErrorMessage();
         return Status::Ok;
     }
@@ -1755,11 +1766,13 @@ private:
     }
 
     IAllocator* m_allocator;
+    NtcHipContext* m_hip;
     bool m_deviceAvailable;
     mutable bool m_allowSetsWithoutDevice = false;
 };
 
 IAllocator* TextureSet::Allocator() const { return m_context->GetAllocator(); }
+NtcHipContext* TextureSet::Hip() const { return m_context->GetHip(); }
 
 namespace amd
 {
@@ -1788,14 +1801,16 @@ Status CreateContext(IContext** pOutContext, ContextParameters const& params)
     case GraphicsAPI::Vulkan: SetErrorMessage("This version of LibNTC doesn't support Vulkan."); return Status::NotImplemented;
     default: SetErrorMessage("Invalid graphicsApi (%d).", int(params.graphicsApi)); return Status::InvalidArgument;
     }
-    bool deviceAvailable = false;
-    if (params.cudaDevice >= 0) {
-        if (ntc_hip_init(params.cudaDevice) == 0) deviceAvailable = true;
-        else SetErrorMessage("%s", ntc_hip_last_error());
+    // every context has its own device context: device, stream, working memory (src/PublicFunctions.cpp:84-112)
+    NtcHipContext* hip = nullptr;
+    if (params.cudaDevice >= 0 && ntc_hip_create(params.cudaDevice, &hip) != 0) {
+        SetErrorMessage("%s", ntc_hip_last_error());
+        hip = nullptr;
     }
+    bool const deviceAvailable = hip != nullptr;
     IAllocator* const allocator = params.pAllocator ? params.pAllocator : &g_defaultAllocator;
-    Context* context = MakeObject<Context>(allocator, allocator, deviceAvailable);
-    if (!context) { SetErrorMessage("Failed to allocate the context object."); return Status::OutOfMemory; }
+    Context* context = MakeObject<Context>(allocator, allocator, hip);
+    if (!context) { ntc_hip_destroy(hip); SetErrorMessage("Failed to allocate the context object."); return Status::OutOfMemory; }
     // for host-side checks by programs that know LibNTC's header only (see ntc::amd::IContextExtension)
     if (std::getenv("LIBNTC_ALLOW_TEXTURE_SETS_WITHOUT_DEVICE")) context->AllowTextureSetsWithoutDevice(true);
     *pOutContext = context;

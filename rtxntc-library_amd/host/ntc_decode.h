@@ -117,6 +117,10 @@ public:
     virtual Status CompressBlocks(BlockCompressionParameters const& params) const = 0;
     // True when a gfx950 device was initialised for this context.
     virtual bool IsDeviceAvailable() const = 0;
+    // Every context queues its device work (Decompress without statistics, ReadChannels into device memory, the two
+    // passes above) on a stream of its own and returns.  Synchronize waits for all of it: call it before other
+    // code - another context, the application's own streams - touches the memory that work reads or writes.
+    virtual Status Synchronize() const = 0;
     // IContext::CreateTextureSet and CreateCompressedTextureSetFrom* refuse to work without a device, as the
     // reference's do (src/Context.cpp:187-191,311-315).  After AllowTextureSetsWithoutDevice(true) they create
     // the set regardless: everything that needs no device (shapes, sizes, validation, metadata, file parsing)

@@ -39,6 +39,14 @@ using namespace ntc::amd;
 static ITextureSetExtension* X(ITextureSetMetadata* set) { return GetTextureSetExtension(set); }
 static IContextExtension* X(IContext* context) { return GetContextExtension(context); }
 
+// This program's own device buffers live on the C ABI's default context; a libntc context works on a stream of
+// its own, so its results are waited for before they are fetched.
+static int syncedDownload(IContext* context, void* dst, void const* src, size_t bytes)
+{
+    if (X(context)->Synchronize() != Status::Ok) return -1;
+    return ntc_hip_download(dst, src, bytes);
+}
+
 #define CHECK(cond) do { if (!(cond)) { std::fprintf(stderr, "FAILED %s:%d: %s\n  last error: %s\n", __FILE__, __LINE__, #cond, GetLastErrorMessage()); return 1; } } while (0)
 
 static std::vector<unsigned char> readFile(char const* path)
@@ -350,6 +358,7 @@ static int decode(int argc, char** argv)
     IContext* ctx = nullptr;
     ContextParameters params;
     CHECK(CreateContext(&ctx, params) == Status::Ok);
+    CHECK(ntc_hip_init(params.cudaDevice) == 0);              // the default context of the C ABI, for this program's own device buffers
     CHECK(X(ctx)->IsDeviceAvailable());
     TextureSetDesc desc; desc.width = w; desc.height = h; desc.channels = channels; desc.mips = mips;
     TextureSetFeatures features_;
@@ -391,7 +400,7 @@ static int decode(int argc, char** argv)
             rd.pOutData = static_cast<unsigned char*>(dev);
             CHECK(set->ReadChannels(rd) == Status::Ok);
             std::vector<unsigned char> f16(bytes);
-            CHECK(ntc_hip_download(f16.data(), dev, bytes) == 0);
+            CHECK(syncedDownload(ctx, f16.data(), dev, bytes) == 0);
             CHECK(ntc_hip_free(dev) == 0);
             CHECK(writeFile(prefix + "_mip" + std::to_string(mip) + "_rgba16f.bin", f16.data(), f16.size()));
         }
@@ -446,6 +455,7 @@ static int shuffle(int argc, char** argv)
     IContext* ctx = nullptr;
     ContextParameters params;
     CHECK(CreateContext(&ctx, params) == Status::Ok);
+    CHECK(ntc_hip_init(params.cudaDevice) == 0);              // the default context of the C ABI, for this program's own device buffers
     TextureSetDesc desc; desc.width = w; desc.height = h; desc.channels = channels; desc.mips = 1;
     TextureSetFeatures features_;
     features_.stagingBytesPerPixel = 16 * 2;
@@ -547,6 +557,7 @@ static int imageDifference()
     IContext* ctx = nullptr;
     ContextParameters params;
     CHECK(CreateContext(&ctx, params) == Status::Ok);
+    CHECK(ntc_hip_init(params.cudaDevice) == 0);              // the default context of the C ABI, for this program's own device buffers
     int const w = 192, h = 80;
     std::vector<unsigned char> a(size_t(w) * h * 4, 0), b(size_t(w) * h * 4, 255);
     for (int y = 0; y < 16; ++y) for (int x = 0; x < 32; ++x) std::memcpy(&b[(size_t(y) * w + x) * 4], &a[(size_t(y) * w + x) * 4], 4);   // identical corner
@@ -564,13 +575,13 @@ static int imageDifference()
     CHECK(X(ctx)->ComputeImageDifference(dp) == Status::Ok);
     dp.outputOffset = 32; dp.extent = Rect{ 0, 0, 32, 16 };                                     // identical pixels
     CHECK(X(ctx)->ComputeImageDifference(dp) == Status::Ok);
-    CHECK(ntc_hip_download(result, dOut, sizeof result) == 0);
+    CHECK(syncedDownload(ctx, result, dOut, sizeof result) == 0);
     for (int c = 0; c < 4; ++c) CHECK(DecodeImageDifferenceResult(result[c]) == 1.0 && result[4 + c] == 0);
     // both alphas (0 and 1) below a threshold of 2: colour ignored, alpha still compared
     CHECK(ntc_hip_upload(dOut, zeros, sizeof zeros) == 0);
     dp.outputOffset = 0; dp.extent = Rect{ 64, 16, 128, 64 }; dp.useAlphaThreshold = true; dp.alphaThreshold = 2.f;
     CHECK(X(ctx)->ComputeImageDifference(dp) == Status::Ok);
-    CHECK(ntc_hip_download(result, dOut, sizeof result) == 0);
+    CHECK(syncedDownload(ctx, result, dOut, sizeof result) == 0);
     CHECK(result[0] == 0 && result[1] == 0 && result[2] == 0 && DecodeImageDifferenceResult(result[3]) == 1.0);
     dp.extent.width = 200;                                                                      // leaves the image
     CHECK(X(ctx)->ComputeImageDifference(dp) == Status::InvalidArgument);
@@ -587,7 +598,7 @@ static int imageDifference()
         bp.pDstData = dBlocks; bp.dstDataSize = blocksX * blocksY * 16; bp.dstRowPitch = blocksX * 16;
         CHECK(X(ctx)->CompressBlocks(bp) == Status::Ok);
         std::vector<uint64_t> blocks(blocksX * blocksY * 2);
-        CHECK(ntc_hip_download(blocks.data(), dBlocks, blocks.size() * 8) == 0);
+        CHECK(syncedDownload(ctx, blocks.data(), dBlocks, blocks.size() * 8) == 0);
         for (size_t by = 0; by < blocksY; ++by)
             for (size_t bx = 0; bx < blocksX; ++bx) {
                 bool const corner = bx < 8 && by < 4;
@@ -598,7 +609,7 @@ static int imageDifference()
         // the zero corner (alpha 0) the all-transparent block
         bp.dstFormat = BlockCompressedFormat::BC1; bp.dstRowPitch = blocksX * 8;
         CHECK(X(ctx)->CompressBlocks(bp) == Status::Ok);
-        CHECK(ntc_hip_download(blocks.data(), dBlocks, blocksX * blocksY * 8) == 0);
+        CHECK(syncedDownload(ctx, blocks.data(), dBlocks, blocksX * blocksY * 8) == 0);
         for (size_t by = 0; by < blocksY; ++by)
             for (size_t bx = 0; bx < blocksX; ++bx)
                 CHECK(blocks[by * blocksX + bx] == ((bx < 8 && by < 4) ? 0xFFFFFFFF00000000ull : 0xAAAAAAAAFFFFFFFFull));
@@ -607,18 +618,18 @@ static int imageDifference()
         // Opaque white is exact in BC7; the zero corner has alpha 0.
         bp.dstFormat = BlockCompressedFormat::BC7;
         CHECK(X(ctx)->CompressBlocks(bp) == Status::Ok);
-        CHECK(ntc_hip_download(blocks.data(), dBlocks, blocks.size() * 8) == 0);
+        CHECK(syncedDownload(ctx, blocks.data(), dBlocks, blocks.size() * 8) == 0);
         {
             std::vector<uint8_t> modes(GetBC7ModeBufferSize(int(blocksX), int(blocksY)), 0);
             CHECK(MakeBC7ModeBuffer(int(blocksX), int(blocksY), blocks.data(), blocks.size() * 8, blocksX * 16, modes.data(), modes.size()) == Status::Ok);
             void* dModes = nullptr;
             CHECK(ntc_hip_alloc(&dModes, modes.size()) == 0 && ntc_hip_upload(dModes, modes.data(), modes.size()) == 0);
-            CHECK(ntc_hip_memset(dBlocks, 0, blocksX * blocksY * 16) == 0);
+            CHECK(ntc_hip_memset(dBlocks, 0, blocksX * blocksY * 16) == 0 && ntc_hip_synchronize() == 0);
             bp.pModeBuffer = dModes; bp.modeBufferSize = modes.size();
             bp.modeMapWidthInBlocks = int(blocksX); bp.modeMapHeightInBlocks = int(blocksY);
             CHECK(X(ctx)->CompressBlocks(bp) == Status::Ok);
             std::vector<uint64_t> again(blocks.size());
-            CHECK(ntc_hip_download(again.data(), dBlocks, again.size() * 8) == 0);
+            CHECK(syncedDownload(ctx, again.data(), dBlocks, again.size() * 8) == 0);
             CHECK(again == blocks);
             bp.dstFormat = BlockCompressedFormat::BC3;
             CHECK(X(ctx)->CompressBlocks(bp) == Status::InvalidArgument);
@@ -629,7 +640,7 @@ static int imageDifference()
         // all the same block in one of the three modes the encoder emits
         bp.dstFormat = BlockCompressedFormat::BC6;
         CHECK(X(ctx)->CompressBlocks(bp) == Status::Ok);
-        CHECK(ntc_hip_download(blocks.data(), dBlocks, blocks.size() * 8) == 0);
+        CHECK(syncedDownload(ctx, blocks.data(), dBlocks, blocks.size() * 8) == 0);
         {
             uint64_t const whiteLo = blocks[(blocksY - 1) * blocksX * 2], whiteHi = blocks[(blocksY - 1) * blocksX * 2 + 1];
             CHECK((whiteLo & 3u) == 1u || (whiteLo & 31u) == 0x0Eu || (whiteLo & 31u) == 0x03u);
@@ -662,6 +673,7 @@ static int generateMips(int argc, char** argv)
     IContext* ctx = nullptr;
     ContextParameters params;
     CHECK(CreateContext(&ctx, params) == Status::Ok);
+    CHECK(ntc_hip_init(params.cudaDevice) == 0);              // the default context of the C ABI, for this program's own device buffers
     TextureSetDesc desc; desc.width = w; desc.height = h; desc.channels = channels; desc.mips = mips;
     TextureSetFeatures features_;
     features_.stagingBytesPerPixel = 16 * 4; features_.stagingWidth = 2 * w; features_.stagingHeight = 2 * h;
@@ -710,6 +722,7 @@ static int loss(int argc, char** argv)
     IContext* ctx = nullptr;
     ContextParameters params;
     CHECK(CreateContext(&ctx, params) == Status::Ok);
+    CHECK(ntc_hip_init(params.cudaDevice) == 0);              // the default context of the C ABI, for this program's own device buffers
     TextureSetDesc desc; desc.width = w; desc.height = h; desc.channels = channels; desc.mips = mips;
     TextureSetFeatures features_;
     features_.stagingBytesPerPixel = 16 * 4;
@@ -902,6 +915,7 @@ static int decodeFile(int argc, char** argv)
     IContext* ctx = nullptr;
     ContextParameters params;
     CHECK(CreateContext(&ctx, params) == Status::Ok);
+    CHECK(ntc_hip_init(params.cudaDevice) == 0);              // the default context of the C ABI, for this program's own device buffers
     TextureSetFeatures features;
     features.stagingBytesPerPixel = 16 * 2;
     ITextureSet* set = nullptr;

@@ -298,6 +298,27 @@ static int decode(int argc, char** argv)
         std::fclose(f);
         CHECK(ok);
     }
+    {   // a second context in the same process: its own device context and stream; both decode interleaved, without
+        // statistics (so without waiting), and read back the same pixels
+        ContextWrapper other;
+        CHECK(CreateContext(other.ptr(), params) == Status::Ok);
+        TextureSetWrapper otherSet(other);
+        CHECK(other->CreateCompressedTextureSetFromMemory(image.data(), image.size(), features, otherSet.ptr()) == Status::Ok);
+        for (int round = 0; round < 3; ++round) {
+            CHECK(set->Decompress(nullptr, useInt8Weights) == Status::Ok);
+            CHECK(otherSet->Decompress(nullptr, useInt8Weights) == Status::Ok);
+        }
+        ReadChannelsParameters rp;
+        rp.firstChannel = 0; rp.numChannels = desc.channels; rp.width = desc.width; rp.height = desc.height;
+        rp.pixelStride = size_t(desc.channels) * 2; rp.rowPitch = rp.pixelStride * size_t(rp.width);
+        rp.channelFormat = ChannelFormat::FLOAT16;
+        std::vector<unsigned char> a(rp.rowPitch * size_t(rp.height)), b(a.size());
+        rp.pOutData = a.data();
+        CHECK(set->ReadChannels(rp) == Status::Ok);
+        rp.pOutData = b.data();
+        CHECK(otherSet->ReadChannels(rp) == Status::Ok);
+        CHECK(a == b);
+    }
     std::printf("libntc drop-in decode OK: %d x %d, %d channels, %d mips, %s weights, %.3f ms\n", desc.width, desc.height, desc.channels, desc.mips,
                 useInt8Weights ? "Int8" : "FP8", stats.gpuTimeMilliseconds);
     return 0;
