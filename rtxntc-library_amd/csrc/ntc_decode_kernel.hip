@@ -298,6 +298,8 @@ __device__ int stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
             fits = bound < (int64_t(1) << 24);
             if (l == 3) bounded = float(bound) * fabsf(reinterpret_cast<float const*>(blob + V::SCALE_OFF)[V::H0 + c]) < 60000.f;
         }
+        // the channel's scale gets multiplied by 2^24 (activations enter as (q + 113) * 2^-24): must stay finite
+        fits = fits && fabsf(reinterpret_cast<float const*>(blob + V::SCALE_OFF)[V::H0 + c]) < 0x1p100f;
         slotTile = V::T0 + (l == 1 ? 0 : (l == 2 ? V::T1 : V::T1 + V::T2)) + row / 16;
         slotG = (row >> 2) & 3;
         slotR = row & 3;
@@ -309,9 +311,12 @@ __device__ int stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
     if (useF16) {
         if (threadIdx.x < V::LATE_CHANNELS) {
             if constexpr (V::FP8_WEIGHTS) {
-                if (twoPlanes) lds.biasLo[slotTile][slotG][slotR] = float(shifted & 1023);
+                if (twoPlanes) lds.biasLo[slotTile][slotG][slotR] = float(shifted & 1023) * 0x1p-24f;
             }
-            lds.bias[slotTile][slotG][slotR] = __builtin_bit_cast(int32_t, float(twoPlanes ? (shifted >> 10) : shifted));
+            // sums run over (q + 113) * 2^-24 (see activate4_h): every term, this start value included, is an
+            // integer below 2^24 times 2^-24, exact in fp32; the scale takes the 2^24 back
+            lds.bias[slotTile][slotG][slotR] = __builtin_bit_cast(int32_t, float(twoPlanes ? (shifted >> 10) : shifted) * 0x1p-24f);
+            lds.scale[slotTile][slotG][slotR] = reinterpret_cast<float const*>(blob + V::SCALE_OFF)[V::H0 + threadIdx.x] * 0x1p24f;
         }
         // fp16 blocks.  Lane (i, kg) of the block of output tile t and input-tile pair p holds
         // W[16t + i][16*(2p + e/4) + 4*kg + e%4], e = 0..7: the channels lane (j, kg) of the
@@ -880,16 +885,26 @@ __device__ __forceinline__ void mlp_forward(LdsT<V>& lds, int wave, int lane, ui
 //
 // Same integers, fewer vector operations.  The int8 matrix instruction returns int32, which costs a
 // conversion per activation, and its operands are signed bytes, which forces the "- 113" and the
-// clamp of min(x, 3) into fp32.  Here the previous layer's activations enter as the fp16 numbers
-// u = q + 113 in [-15, 240] and the weights as fp16 integers; products and every partial sum are
-// integers below 2^24 (stage_weights checked that), so the fp32 accumulator of
-// v_mfma_f32_16x16x32_f16 holds exactly acc = bias + sum W*(u - 113) once the accumulator starts at
-// bias - 113*sum(W).  The epilogue is then 6 operations per activation:
-//   v_mul (scale), v_fma clamp, v_mul (x*t), v_mul (80), v_rndne, and half each of
-//   v_cvt_pkrtz_f16_f32 and v_pk_min_f16 (the cap at 240 = the min(x, 3) of the definition: below 3
-//   both agree term by term, from 3 on t = 1 and x*80 >= 240).
+// clamp of min(x, 3) into fp32.  Here the previous layer's activations enter as fp16 numbers
+// proportional to u = q + 113 in [-15, 240] (u * 2^-24, see activate4_h) and the weights as fp16 integers;
+// products and every partial sum are integers below 2^24 (stage_weights checked that) times 2^-24, so the
+// fp32 accumulator of v_mfma_f32_16x16x32_f16 holds exactly 2^-24 * (bias + sum W*(u - 113)) once it starts
+// at 2^-24 * (bias - 113*sum(W)), and the channel's scale times 2^24 gives the same product the definition
+// rounds.  The epilogue is then 5 operations per activation:
+//   v_mul (scale), v_fma clamp, v_mul (x*t), v_mul (80 * 2^-24), and half each of v_cvt_pk_f16_f32 and
+//   v_pk_min_i16 (the cap at 240 = the min(x, 3) of the definition: below 3 both agree term by term, from 3
+//   on t = 1 and x*80 >= 240).
 
-// HGELU-clamp + requantise of four accumulators to the fp16 values q + 113, two dwords.
+// HGELU-clamp + requantise of four accumulators to n = q + 113, two dwords of fp16 SUBNORMALS n * 2^-24.
+// Subnormal halves are spaced 2^-24 apart from zero on, so the round-to-nearest-even conversion of
+// fl32(y * 80) * 2^-24 to half IS rint(fl32(y * 80)) (in sign-magnitude: bit pattern |n|, sign bit for n < 0),
+// and the power of two folds into the multiplier: fl32(y * (80 * 2^-24)) = fl32(y * 80) * 2^-24 exactly.
+// That saves the separate v_rndne_f32.  Anything above 240 * 2^-24, normal halves and +Inf included, has a
+// larger bit pattern as a signed 16-bit integer and negatives a smaller one, so the cap is v_pk_min_i16.
+// The fp16 matrix instruction takes subnormal operands as they are (checked by the unit test of the
+// instruction); the layers that consume these values hold their biases times 2^-24 and their scales times 2^24.
+// The empty asm keeps multiply and conversion apart: fused (v_fma_mixlo_f16) they would round once.
+typedef short v2s __attribute__((ext_vector_type(2)));
 template <class Acc>
 __device__ __forceinline__ void activate4_h(Acc acc, v4f scale, uint32_t (&out)[2])
 {
@@ -900,11 +915,12 @@ __device__ __forceinline__ void activate4_h(Acc acc, v4f scale, uint32_t (&out)[
         float t = __builtin_fmaf(x, 0.333333f, 0.5f);
         t = fminf(fmaxf(t, 0.f), 1.f);
         float const y = x * t;
-        v[r] = __builtin_rintf(y * 80.f);
+        v[r] = y * (80.f * 0x1p-24f);
+        asm("" : "+v"(v[r]));
     }
-    v2h const cap = { _Float16(240.f), _Float16(240.f) };
-    v2h const lo = __builtin_bit_cast(v2h, __builtin_amdgcn_cvt_pkrtz(v[0], v[1]));
-    v2h const hi = __builtin_bit_cast(v2h, __builtin_amdgcn_cvt_pkrtz(v[2], v[3]));
+    v2s const cap = { 240, 240 };
+    v2s const lo = __builtin_bit_cast(v2s, __builtin_convertvector(v2f{ v[0], v[1] }, v2h));
+    v2s const hi = __builtin_bit_cast(v2s, __builtin_convertvector(v2f{ v[2], v[3] }, v2h));
     out[0] = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(lo, cap));
     out[1] = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(hi, cap));
 }

@@ -70,6 +70,41 @@ def test_mfma_f16_integer_sums_are_exact(device, depth):
         assert np.array_equal(d.astype(np.int64), exact), (depth, trial)
 
 
+@pytest.mark.parametrize("depth", [16, 32])
+def test_mfma_f16_takes_subnormal_operands_exactly(device, depth):
+    """The form the decode kernel uses: activations n in [-15, 240] enter as the fp16 SUBNORMALS n * 2^-24
+    (bit pattern |n|, sign bit for negatives) and the accumulator starts at bias * 2^-24.  The instruction must
+    neither flush them nor lose a bit: the result times 2^24 is the integer sum, to the last unit of headroom."""
+    from importlib import import_module
+    abi = import_module("rtxntc-library_amd").abi
+    rng = np.random.default_rng(60 + depth)
+    for trial in range(8):
+        a = rng.integers(-127, 128, size=(16, depth))
+        n = rng.integers(-15, 241, size=(depth, 16))
+        if trial == 1:
+            a[:], n[:] = 127, 240
+        if trial == 2:
+            a[:], n[:] = -127, 240
+        if trial == 5:
+            n[:] = rng.integers(-1, 2, size=n.shape)     # the smallest subnormals and both zeros
+        room = (1 << 24) - 1 - np.abs(a).sum(axis=1, keepdims=True) * 240
+        c = rng.integers(-room, room + 1, size=(16, 16))
+        if trial in (1, 3):
+            c = np.broadcast_to(room, (16, 16)).copy()
+        if trial in (2, 4):
+            c = -np.broadcast_to(room, (16, 16)).copy()
+        exact = a @ n + c
+        ah = a.astype(np.float16)
+        bits = np.abs(n).astype(np.uint16) | np.where(n <= 0, 0x8000, 0).astype(np.uint16)    # zero enters as -0
+        bh = np.ascontiguousarray(bits.view(np.float16))
+        assert np.array_equal(bh.astype(np.float64) * 2.0 ** 24, n)
+        cf = (c.astype(np.float64) * 2.0 ** -24).astype(np.float32)
+        assert np.array_equal(cf.astype(np.float64) * 2.0 ** 24, c)
+        d = np.zeros((16, 16), dtype=np.float32)
+        abi.check(device.lib.ntc_hip_selftest_mfma_f16(ah.ctypes.data, bh.ctypes.data, cf.ctypes.data, d.ctypes.data, depth))
+        assert np.array_equal(d.astype(np.float64) * 2.0 ** 24, exact), (depth, trial)
+
+
 @pytest.mark.parametrize("scale_range", [(-10.0, -4.0), ACTIVE])
 def test_cfg0_plumbing_512_fp16(ntc, device, scale_range):
     """The plumbing configuration: 512x512, one mip, 8 channels, 64-48-32 int8, fp16 planar output."""
