@@ -132,17 +132,27 @@ __device__ __forceinline__ uint32_t pack_unorm8(_Float16 h, uint32_t slot, uint3
 typedef __attribute__((address_space(1))) uint8_t* GlobalOutPtr;
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-// Stores of one 16-texel block row.  `row` is uniform (start of image row y in the output),
-// `laneOff` the lane's byte offset inside the row, h01/h23 the lane's four channels as halves.
+// A uniform 64-bit address, pinned to scalar registers so that stores take the "scalar base + 32-bit lane
+// offset" form instead of a 64-bit address computed per lane.
+__device__ __forceinline__ GlobalOutPtr uniform_pointer(uint64_t address)
+{
+    uint32_t const lo = __builtin_amdgcn_readfirstlane(uint32_t(address));
+    uint32_t const hi = __builtin_amdgcn_readfirstlane(uint32_t(address >> 32));
+    return (GlobalOutPtr)((uint64_t(hi) << 32) | lo);
+}
+
+// Stores of one 16-texel block row.  `row` is uniform (start of image row y in the output), `laneOff` the
+// lane's byte offset inside the row (`laneOff2` that of the second channel pair of planar output), h01/h23 the
+// lane's four channels as halves.
 template <int FORMAT>
-__device__ __forceinline__ void store_channels(GlobalOutPtr row, uint32_t laneOff, uint32_t planarPairStride,
+__device__ __forceinline__ void store_channels(GlobalOutPtr row, uint32_t laneOff, uint32_t laneOff2,
                                                uint32_t h01, uint32_t h23, int nch)
 {
     GlobalOutPtr const dst = row + laneOff;
     if constexpr (FORMAT == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS) {
         // src/RegressionKernels.h:36-45; whole half2 pairs (Inference.cu:131-134)
         *reinterpret_cast<__attribute__((address_space(1))) uint32_t*>(dst) = h01;
-        if (nch > 2) *reinterpret_cast<__attribute__((address_space(1))) uint32_t*>(dst + planarPairStride) = h23;
+        if (nch > 2) *reinterpret_cast<__attribute__((address_space(1))) uint32_t*>(row + laneOff2) = h23;
     } else if constexpr (FORMAT == NTC_HIP_DEV_OUT_FP16_PIXELS) {
         if (nch == 4 && ((reinterpret_cast<uintptr_t>(dst) & 7u) == 0)) {
             *reinterpret_cast<__attribute__((address_space(1))) u32x2*>(dst) = u32x2{ h01, h23 };
@@ -170,6 +180,7 @@ __device__ __forceinline__ void store_tile(DevMip const& m, Acc const (&D)[4], v
     uint32_t const laneOff = (FORMAT == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)
         ? (uint32_t(chBase) * uint32_t(m.width) + uint32_t(x) * 2u) * 2u
         : uint32_t(x) * uint32_t(m.outPixelStride) + uint32_t(chBase) * (FORMAT == NTC_HIP_DEV_OUT_FP16_PIXELS ? 2u : 1u);
+    uint32_t const laneOff2 = laneOff + uint32_t(m.width) * 4u;
     size_t const rowBytes = (FORMAT == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS) ? size_t(m.width) * C2 * 2 : size_t(m.outRowPitch);
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
@@ -177,7 +188,8 @@ __device__ __forceinline__ void store_tile(DevMip const& m, Acc const (&D)[4], v
         if (y >= m.height) break;                            // uniform
         uint32_t const h01 = to_half2_bits<CHECKED>(float(D[b][0]) * S[0], float(D[b][1]) * S[1]);
         uint32_t const h23 = to_half2_bits<CHECKED>(float(D[b][2]) * S[2], float(D[b][3]) * S[3]);
-        store_channels<FORMAT>((GlobalOutPtr)m.out + size_t(y) * rowBytes, laneOff, uint32_t(m.width) * 4u, h01, h23, nch);
+        GlobalOutPtr const row = uniform_pointer(reinterpret_cast<uint64_t>(m.out) + size_t(y) * rowBytes);
+        store_channels<FORMAT>(row, laneOff, laneOff2, h01, h23, nch);
     }
 }
 

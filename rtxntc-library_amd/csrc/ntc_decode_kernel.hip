@@ -75,19 +75,31 @@ __device__ __forceinline__ AxisFoot axis_fast(int x, uint32_t packedAxis, int gr
     return a;
 }
 
-// Four 4-bit features of the four taps, filtered: ((17 * sum w*q) >> n) - 128 per byte.
-// Nibbles are spread into 16-bit lanes, two dwords per tap ((f0,f2) and (f1,f3)); weights
-// are pre-multiplied by 17; no lane can overflow because 17*15*2^n < 65536 (n <= 8).
+// 24-bit multiply-add, full rate: a * b + c.
+__device__ __forceinline__ uint32_t mad24(uint32_t a, uint32_t b, uint32_t c)
+{
+    uint32_t r;
+    asm("v_mad_u32_u24 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+// Four 4-bit features of the four taps, filtered: ((17 * sum w*q) >> n) - 128 per byte; the weights w sum to 2^n
+// (n <= 8).  A cell c = f0 | f1<<4 | f2<<8 | f3<<12 is spread to P = byte0 | byte1<<16 (16-bit lanes holding
+// f0 + 16 f1 and f2 + 16 f3); E = P & 0x000f000f holds the even features alone.  S = sum w*P and T = sum w*E stay
+// below 2^16 per lane (255 * 2^n), so lanes never mix, and (S - T) / 16 is sum w*f for the odd features, exactly.
+// Times 17 (T + 16 T, and D/16 + D for the odd ones) is at most 17 * 15 * 2^8 < 2^16: still inside the lane.
 __device__ __forceinline__ uint32_t bilinear4_int(uint32_t c00, uint32_t c10, uint32_t c01, uint32_t c11,
                                                   uint32_t w00, uint32_t w10, uint32_t w01, uint32_t w11, uint32_t n)
 {
     uint32_t const m = 0x000f000fu;
-    uint32_t const d00 = c00 | (c00 << 8), d10 = c10 | (c10 << 8), d01 = c01 | (c01 << 8), d11 = c11 | (c11 << 8);
-    uint32_t const te = __umul24(w00, d00 & m) + __umul24(w10, d10 & m) + __umul24(w01, d01 & m) + __umul24(w11, d11 & m);
-    uint32_t const to = __umul24(w00, (d00 >> 4) & m) + __umul24(w10, (d10 >> 4) & m)
-                      + __umul24(w01, (d01 >> 4) & m) + __umul24(w11, (d11 >> 4) & m);
-    uint32_t const ve = (te >> n) & 0x00ff00ffu;             // features 0 and 2 in bytes 0 and 2
-    uint32_t const vo = (to >> n) & 0x00ff00ffu;             // features 1 and 3
+    uint32_t const sel = 0x0c010c00u;                        // v_perm_b32: bytes [0, zero, 1, zero] of the cell
+    uint32_t const p00 = __builtin_amdgcn_perm(0u, c00, sel), p10 = __builtin_amdgcn_perm(0u, c10, sel);
+    uint32_t const p01 = __builtin_amdgcn_perm(0u, c01, sel), p11 = __builtin_amdgcn_perm(0u, c11, sel);
+    uint32_t const S = mad24(w11, p11, mad24(w01, p01, mad24(w10, p10, mul24(w00, p00))));
+    uint32_t const T = mad24(w11, p11 & m, mad24(w01, p01 & m, mad24(w10, p10 & m, mul24(w00, p00 & m))));
+    uint32_t const D = S - T;                                // 16 * sum w*f of features 1 and 3
+    uint32_t const ve = (((T << 4) + T) >> n) & 0x00ff00ffu; // features 0 and 2 in bytes 0 and 2
+    uint32_t const vo = ((D + (D >> 4)) >> n) & 0x00ff00ffu; // 17 * (D / 16): features 1 and 3
     return (ve | (vo << 8)) ^ 0x80808080u;
 }
 
@@ -499,7 +511,7 @@ __device__ __forceinline__ void prepare_inputs_fast(Mip const& m, LdsT<V> const&
             }
         } else {
             uint32_t const nx = (m.hrAxisX >> 8) & 0xffu, ny = (m.hrAxisY >> 8) & 0xffu;
-            uint32_t const wx1 = ax.f, wx0 = (1u << nx) - ax.f, wy1 = ay.f * 17u, wy0 = ((1u << ny) - ay.f) * 17u;
+            uint32_t const wx1 = ax.f, wx0 = (1u << nx) - ax.f, wy1 = ay.f, wy0 = (1u << ny) - ay.f;
             uint32_t const w00 = mul24(wx0, wy0), w10 = mul24(wx1, wy0), w01 = mul24(wx0, wy1), w11 = mul24(wx1, wy1);
             constexpr int layers = (V::HR_F + 3) / 4;
 #pragma unroll
@@ -521,7 +533,7 @@ __device__ __forceinline__ void prepare_inputs_fast(Mip const& m, LdsT<V> const&
         uint32_t const r0 = ay.c0 << lgw, r1 = ay.c1 << lgw, c0 = ax.c0 << 1, c1 = ax.c1 << 1;
         uint32_t const a00 = r0 + c0, a10 = r0 + c1, a01 = r1 + c0, a11 = r1 + c1;
         uint32_t const nx = (m.lrAxisX >> 8) & 0xffu, ny = (m.lrAxisY >> 8) & 0xffu;
-        uint32_t const wx1 = ax.f, wx0 = (1u << nx) - ax.f, wy1 = ay.f * 17u, wy0 = ((1u << ny) - ay.f) * 17u;
+        uint32_t const wx1 = ax.f, wx0 = (1u << nx) - ax.f, wy1 = ay.f, wy0 = (1u << ny) - ay.f;
         uint32_t const w00 = mul24(wx0, wy0), w10 = mul24(wx1, wy0), w01 = mul24(wx0, wy1), w11 = mul24(wx1, wy1);
         constexpr int layers = (V::LR_F + 3) / 4;
 #pragma unroll
@@ -620,7 +632,7 @@ __device__ __forceinline__ void prepare_inputs_scattered(Mip const& m, LdsT<V> c
         }
     } else {
         uint32_t const nx = (m.hrAxisX >> 8) & 0xffu, ny = (m.hrAxisY >> 8) & 0xffu;
-        uint32_t const wx1 = hx.f, wx0 = (1u << nx) - hx.f, wy1 = hy.f * 17u, wy0 = ((1u << ny) - hy.f) * 17u;
+        uint32_t const wx1 = hx.f, wx0 = (1u << nx) - hx.f, wy1 = hy.f, wy0 = (1u << ny) - hy.f;
         uint32_t const w00 = mul24(wx0, wy0), w10 = mul24(wx1, wy0), w01 = mul24(wx0, wy1), w11 = mul24(wx1, wy1);
 #pragma unroll
         for (int L = 0; L < HL; ++L) {
@@ -631,7 +643,7 @@ __device__ __forceinline__ void prepare_inputs_scattered(Mip const& m, LdsT<V> c
     }
     {
         uint32_t const nx = (m.lrAxisX >> 8) & 0xffu, ny = (m.lrAxisY >> 8) & 0xffu;
-        uint32_t const wx1 = lx.f, wx0 = (1u << nx) - lx.f, wy1 = ly.f * 17u, wy0 = ((1u << ny) - ly.f) * 17u;
+        uint32_t const wx1 = lx.f, wx0 = (1u << nx) - lx.f, wy1 = ly.f, wy0 = (1u << ny) - ly.f;
         uint32_t const w00 = mul24(wx0, wy0), w10 = mul24(wx1, wy0), w01 = mul24(wx0, wy1), w11 = mul24(wx1, wy1);
 #pragma unroll
         for (int L = 0; L < LL; ++L) {
@@ -722,7 +734,7 @@ __device__ __forceinline__ void prepare_inputs_bricked(Mip const& m, LdsT<V> con
         }
     } else {
         uint32_t const nx = (m.hrAxisX >> 8) & 0xffu, ny = (m.hrAxisY >> 8) & 0xffu;
-        uint32_t const wx1 = hx.f, wx0 = (1u << nx) - hx.f, wy1 = hy.f * 17u, wy0 = ((1u << ny) - hy.f) * 17u;
+        uint32_t const wx1 = hx.f, wx0 = (1u << nx) - hx.f, wy1 = hy.f, wy0 = (1u << ny) - hy.f;
         uint32_t const w00 = mul24(wx0, wy0), w10 = mul24(wx1, wy0), w01 = mul24(wx0, wy1), w11 = mul24(wx1, wy1);
 #pragma unroll
         for (int L = 0; L < HL; ++L) {
@@ -733,7 +745,7 @@ __device__ __forceinline__ void prepare_inputs_bricked(Mip const& m, LdsT<V> con
     }
     {
         uint32_t const nx = (m.lrAxisX >> 8) & 0xffu, ny = (m.lrAxisY >> 8) & 0xffu;
-        uint32_t const wx1 = lx.f, wx0 = (1u << nx) - lx.f, wy1 = ly.f * 17u, wy0 = ((1u << ny) - ly.f) * 17u;
+        uint32_t const wx1 = lx.f, wx0 = (1u << nx) - lx.f, wy1 = ly.f, wy0 = (1u << ny) - ly.f;
         uint32_t const w00 = mul24(wx0, wy0), w10 = mul24(wx1, wy0), w01 = mul24(wx0, wy1), w11 = mul24(wx1, wy1);
 #pragma unroll
         for (int L = 0; L < LL; ++L) {
