@@ -314,16 +314,19 @@ def main():
                    "sample": f"the first {n} queries of the same list, {t:.1f} s"}
 
     # Ceilings of the kernel, lowest first decides `bound`: HBM (algorithmic bytes), int8 MFMA (algorithmic
-    # operations), and vector-instruction issue: a CU issues 64 lane-operations per clock (no packed fp32),
-    # so the ceiling is CUs x 64 x clock / (vector operations per texel, from the SQ_INSTS_VALU counter).
+    # operations), and vector-instruction issue: a CU issues 64 lane-operations per clock (no packed fp32), and a
+    # matrix instruction takes one such issue slot too, so the ceiling is CUs x 64 x clock / (issue slots per texel,
+    # from the SQ_INSTS_VALU and SQ_INSTS_MFMA counters).
     counters = None if args.size else measured_counters(wl, fmt_name)
     rate = texels / (kernel_ms * 1e-3) / 1e9
     fracs = {"hbm": achieved_gbs / HBM_PEAK_GBS, "mfma": achieved_tops / INT8_PEAK_TOPS}
     valu = {}
     if counters and counters.get("valu_ops_per_texel"):
-        ceiling = dev.compute_units * 64 * dev.clock_ghz / counters["valu_ops_per_texel"]
+        mfma_slots = counters.get("SQ_INSTS_MFMA", 0) * 64 / counters["texels_per_launch"]
+        ceiling = dev.compute_units * 64 * dev.clock_ghz / (counters["valu_ops_per_texel"] + mfma_slots)
         fracs["valu"] = rate / ceiling
-        valu = {"valu_ops_per_texel": counters["valu_ops_per_texel"], "valu_clock_ghz": dev.clock_ghz,
+        valu = {"valu_ops_per_texel": counters["valu_ops_per_texel"], "mfma_issue_slots_per_texel": mfma_slots,
+                "valu_clock_ghz": dev.clock_ghz,
                 "valu_ceiling_gtexels": ceiling, "valu_frac": fracs["valu"], "counters_source": counters["source"]}
     line = {
         "metric": "decoded Gtexels/s, 4096^2 16-ch set, 64-48-32 int8; % of int8-MFMA/HBM roof",
