@@ -160,6 +160,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=30)   # the GPU clock takes ~30 launches to settle
     ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4", "ref092", "ref092fp8", "read", "write", "loss", "bc1", "bc3", "bc5", "bc6", "bc7", "bc7m"])
     ap.add_argument("--size", type=int, default=0, help="override the texture size of the workload")
+    ap.add_argument("--settle-ms", type=float, default=60.0,
+                    help="untimed decode steps for this long before the warm-up, so that clocks have ramped (0 = none)")
     ap.add_argument("--format", choices=["fp16", "unorm8"], default=None)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="time budget of the CPU-baseline sample")
     ap.add_argument("--no-cpu", action="store_true")
@@ -262,6 +264,14 @@ def main():
             return ms.value
     ops_per_texel = 2 * macs(widths)
 
+    # An idle GPU runs its first few dozen launches below its sustained clock.  Untimed steps, for `--settle-ms`
+    # of wall time, come before the W warm-up steps so that a short warm-up does not time the ramp.
+    t_settle = time.perf_counter()
+    while (time.perf_counter() - t_settle) * 1e3 < args.settle_ms:
+        for _ in range(4):
+            run()
+        dev.synchronize()
+
     for _ in range(args.warmup):
         run()
     dev.synchronize()
@@ -272,7 +282,7 @@ def main():
     wall = time.perf_counter() - t0
     ms_per_step = wall / args.steps * 1e3
 
-    kernel_ms = run_timed(args.steps)                 # HIP events on the launch stream
+    kernel_ms = run_timed(args.steps)                 # the same K launches again, HIP events on the launch stream
     gtexels = texels / (ms_per_step * 1e-3) / 1e9
     achieved_gbs = texels * bytes_per_texel / (kernel_ms * 1e-3) / 1e9
     achieved_tops = texels * ops_per_texel / (kernel_ms * 1e-3) / 1e12
@@ -334,7 +344,7 @@ def main():
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8", "data": "synthetic",
         "config": {"workload": f"{what}, {fmt_name} output, {texels} texels per step",
-                   "device": dev.name, "compute_units": dev.compute_units},
+                   "device": dev.name, "compute_units": dev.compute_units, "settle_ms": args.settle_ms},
         # achieved / peak / frac: the HBM roof (algorithmic bytes over the kernel's HIP-event time), the lower of
         # the two roofs the metric names; `bound` names the ceiling the kernel actually runs closest to.
         "roofline": {"bound": max(fracs, key=fracs.get), "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -119,14 +119,13 @@ __device__ __forceinline__ uint32_t to_half2_bits(float a, float b)
 }
 
 // WriteImageChannel UNORM8 (src/ImageProcessing.cu:146-149): u8(clamp(roundf(v * 255), 0, 255)) of
-// the stored half.  v*255 is exact (11-bit x 8-bit significands) and so is v*255 + 1/2 wherever the
-// result matters (below 256), so floor(fma(v, 255, 1/2)) equals roundf(v*255) for v >= 0; negatives
-// end at or below 0.  v_cvt_pk_u8_f32 then converts the integer-valued float with saturation to
-// [0, 255] and drops it into byte `slot` of `packed`.
+// the stored half.  v*255 is exact in fp32 (11-bit x 8-bit significands).  v_cvt_pk_u8_f32 rounds to nearest
+// even and saturates to [0, 255]; that equals roundf (half away from zero) here because the only tie inside
+// the range is v = 1/2 (v*255 = k + 1/2 needs 255 | 2k + 1 for a dyadic v): 127.5 -> 128 under both rules.
+// The result drops into byte `slot` of `packed`.
 __device__ __forceinline__ uint32_t pack_unorm8(_Float16 h, uint32_t slot, uint32_t packed)
 {
-    float const v = floorf(__builtin_fmaf(float(h), 255.f, 0.5f));
-    return __builtin_amdgcn_cvt_pk_u8_f32(v, slot, packed);
+    return __builtin_amdgcn_cvt_pk_u8_f32(float(h) * 255.f, slot, packed);
 }
 
 typedef __attribute__((address_space(1))) uint8_t* GlobalOutPtr;

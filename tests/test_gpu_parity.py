@@ -286,6 +286,31 @@ def test_outputs_beyond_the_fp16_range_become_zero(ntc, device):
     assert (halves == 0).mean() > 0.01 and (np.abs(halves.view(np.float16).astype(np.float32)) > 30000).mean() > 0.01
 
 
+@pytest.mark.parametrize("fmt_name", ["OUT_UNORM8_PIXELS", "OUT_FP16_PIXELS"])
+def test_stores_of_chosen_output_values(ntc, device, fmt_name):
+    """Output layer with zero weights: every texel's channel c is bias[c] * 2^-11, so the stores see chosen
+    values - the unorm8 tie 1/2 (-> 128), values next to the half-integers of v * 255, the clamps at 0 and 255,
+    and halves that need rounding.  The checker must agree and the tie must come out as 128."""
+    spec = ntc.presets.spec_cfg01()
+    layout = ntc.synth.weight_layout(spec)
+    blob = ntc.synth.make_weights(spec, 5, scale_log2_range=ACTIVE)
+    last = ntc.abi.MLP_LAYERS - 1
+    n_in, n_out = spec.layer_inputs(last), spec.layer_outputs(last)
+    blob[layout.weightOffset[last]:layout.weightOffset[last] + n_in * n_out] = 0
+    blob[layout.scaleOffset[last]:layout.scaleOffset[last] + 4 * n_out] = np.full(n_out, 2.0 ** -11, dtype=np.float32).view(np.uint8)
+    #          1/2   just below / above   0.5/255 region       1    >1    <0    0   1/255-ish   odd 11-bit patterns
+    biases = [1024, 1023, 1025, 4, 5, 3, 2048, 4096, -512, 0, 8, 9, 2047, 1365, 683, 1]
+    blob[layout.biasOffset[last]:layout.biasOffset[last] + 4 * n_out] = np.array(biases, dtype=np.int32).view(np.uint8)
+    fmt = getattr(ntc.abi, fmt_name)
+    case = cfg_case(ntc, spec, 96, 40, 2, 16, fmt, seed=6, weights=blob)
+    expected, got = run_both(device, case)
+    assert_equal_bytes(expected, got, f"chosen outputs, {fmt_name}")
+    if fmt == ntc.abi.OUT_UNORM8_PIXELS:
+        first = np.asarray(expected).view(np.uint8)[:16].tolist()
+        assert first[0] == 128 and first[6] == 255 and first[7] == 255 and first[8] == 0 and first[9] == 0
+        assert first[1] == 127 and first[2] == 128           # 0.49951 * 255 = 127.38, 0.50049 * 255 = 127.62
+
+
 def test_decode_is_idempotent_and_timed_variant_matches(ntc, device):
     case = cfg_case(ntc, ntc.presets.spec_cfg01(), 320, 200, 4, 16, ntc.abi.OUT_UNORM8_PIXELS, seed=21, scale_log2_range=ACTIVE)
     dset = case.device_set(device)

@@ -239,6 +239,21 @@ def test_unorm8_exhaustive_over_halves(oracle):
     assert oracle.ntc_oracle_half_to_unorm8(int(np.float16(1.0).view(np.uint16))) == 255
 
 
+def test_unorm8_round_half_even_equals_roundf_on_every_half(oracle):
+    """The decode kernel converts with the hardware's saturating round-to-nearest-EVEN conversion of the exact
+    product v * 255; the definition rounds half away from zero.  They agree on every finite half: inside
+    [0, 255] the only tie is v = 1/2 -> 127.5 -> 128 under both rules."""
+    all_bits = np.arange(65536, dtype=np.uint16)
+    finite = all_bits[(all_bits & 0x7C00) != 0x7C00]
+    product = finite.view(np.float16).astype(np.float32) * np.float32(255.0)
+    assert np.array_equal(product.astype(np.float64), finite.view(np.float16).astype(np.float64) * 255.0)   # exact in fp32
+    half_even = np.clip(np.rint(product), 0, 255).astype(np.uint8)
+    want = np.array([oracle.ntc_oracle_half_to_unorm8(int(b)) for b in finite], dtype=np.uint8)
+    assert np.array_equal(half_even, want)
+    ties = product[(product > 0) & (product < 255) & (product - np.floor(product) == 0.5)]
+    assert ties.tolist() == [127.5]
+
+
 # ---------------------------------------------------------------------------------------
 # HGELU-clamp quantiser
 # ---------------------------------------------------------------------------------------
