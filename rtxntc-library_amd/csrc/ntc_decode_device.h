@@ -20,13 +20,36 @@ __device__ __forceinline__ uint32_t load_u16(GlobalU8Ptr base, uint32_t byteOffs
     return *reinterpret_cast<GlobalU16Ptr>(base + byteOffset);
 }
 
-// 24-bit multiply, full rate (the compiler otherwise picks the quarter-rate 32-bit multiply).
+// 24-bit multiply, full rate (a plain 32-bit multiply is quarter rate).  Written with the builtin rather
+// than inline assembly on purpose: the compiler inserts the wait states that matrix instructions in flight
+// need only around instructions it can see, and an assembly statement is opaque to it.
 __device__ __forceinline__ uint32_t mul24(uint32_t a, uint32_t b)
 {
-    uint32_t r;
-    asm("v_mul_u32_u24 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-    return r;
+    return __umul24(a, b);
 }
+// Footprint of one axis of a bilinear tap pair in integers, for power-of-two sizes: with
+// p = u*grid - 1/2 = N / 2^n, N = ((2x+1) << shl) - (1 << sublog) (the packed axis word of DevMip),
+// floor and fraction are a shift and a mask, and the two cells wrap by masking.
+struct AxisFoot { uint32_t c0, c1, f; };
+
+__device__ __forceinline__ AxisFoot axis_fast(int x, uint32_t packedAxis, int gridSize)
+{
+    int const shl = int(packedAxis & 0xffu), n = int((packedAxis >> 8) & 0xffu), sublog = int((packedAxis >> 16) & 0xffu);
+    int const N = ((2 * x + 1) << shl) - (1 << sublog);
+    int const b = N >> n;                                    // arithmetic shift = floor
+    AxisFoot a;
+    a.f = uint32_t(N) & ((1u << n) - 1u);
+    a.c0 = uint32_t(b) & uint32_t(gridSize - 1);             // wrap addressing
+    a.c1 = uint32_t(b + 1) & uint32_t(gridSize - 1);
+    return a;
+}
+
+// 24-bit multiply-add, full rate: a * b + c (v_mad_u32_u24).
+__device__ __forceinline__ uint32_t mad24(uint32_t a, uint32_t b, uint32_t c)
+{
+    return __umul24(a, b) + c;
+}
+
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kWaveTexels  = 64;

@@ -47,26 +47,31 @@ __device__ __forceinline__ uint32_t halves_rne(float a, float b)
     return __builtin_bit_cast(uint32_t, h);
 }
 
-// HGELU-clamp on two fp16 layer outputs (NtcHGELUClamp_Forward_CoopVec, InferenceCoopVec.hlsli:150-153).
-__device__ __forceinline__ uint32_t hgelu_pk(uint32_t x)
+// HGELU-clamp on two fp16 layer outputs (NtcHGELUClamp_Forward_CoopVec, InferenceCoopVec.hlsli:150-153):
+// v_pk_fma_f16 with clamp, v_pk_max_f16, v_pk_min_f16, v_pk_mul_f16.  Written as vector arithmetic, not as
+// inline assembly: these instructions are interleaved with matrix instructions, and the compiler inserts the
+// wait states an in-flight matrix instruction needs (e.g. before one of its source registers is overwritten)
+// only around instructions it can see.
+__device__ __forceinline__ uint32_t hgelu_pk(uint32_t xBits)
 {
-    uint32_t const third = 0x35553555u, half = 0x38003800u, three = 0x42004200u, minusThree = 0xc200c200u;
-    uint32_t t, xc, y;
-    asm("v_pk_fma_f16 %0, %1, %2, %3 clamp" : "=v"(t) : "v"(x), "v"(third), "v"(half));
-    asm("v_pk_max_f16 %0, %1, %2" : "=v"(xc) : "v"(x), "v"(minusThree));
-    asm("v_pk_min_f16 %0, %1, %2" : "=v"(xc) : "v"(xc), "v"(three));
-    asm("v_pk_mul_f16 %0, %1, %2" : "=v"(y) : "v"(xc), "v"(t));
-    return y;
+    v2h const x = __builtin_bit_cast(v2h, xBits);
+    v2h const third = __builtin_bit_cast(v2h, 0x35553555u), half = { _Float16(0.5f), _Float16(0.5f) };
+    v2h const zero = { _Float16(0.f), _Float16(0.f) }, one = { _Float16(1.f), _Float16(1.f) }, three = { _Float16(3.f), _Float16(3.f) };
+    v2h t = __builtin_elementwise_fma(x, third, half);
+    t = __builtin_elementwise_min(__builtin_elementwise_max(t, zero), one);
+    v2h const xc = __builtin_elementwise_min(__builtin_elementwise_max(x, -three), three);
+    return __builtin_bit_cast(uint32_t, xc * t);
 }
 
 // After the last hidden layer: q = rne(80 y - 113) as fp16 integers in [-128, 127] (hlsli:155-158).
-__device__ __forceinline__ uint32_t quantize_int8_pk(uint32_t y)
+__device__ __forceinline__ uint32_t quantize_int8_pk(uint32_t yBits)
 {
-    uint32_t const eighty = 0x55005500u, c1423 = 0x658f658fu, minus1536 = 0xe600e600u;
-    uint32_t z, q;
-    asm("v_pk_fma_f16 %0, %1, %2, %3" : "=v"(z) : "v"(y), "v"(eighty), "v"(c1423));
-    asm("v_pk_add_f16 %0, %1, %2" : "=v"(q) : "v"(z), "v"(minus1536));
-    return q;
+    v2h const y = __builtin_bit_cast(v2h, yBits);
+    v2h const eighty = { _Float16(80.f), _Float16(80.f) }, c1423 = { _Float16(1423.f), _Float16(1423.f) };
+    v2h const minus1536 = { _Float16(-1536.f), _Float16(-1536.f) };
+    v2h z = __builtin_elementwise_fma(y, eighty, c1423);
+    asm("" : "+v"(z));                                       // keeps the two roundings apart
+    return __builtin_bit_cast(uint32_t, z + minus1536);
 }
 
 template <int FEATURES_>
@@ -94,6 +99,10 @@ struct alignas(16) Fp8Lds {
     float outScale[4][4];      // output layer: [g][r]
     int32_t outBias[4][4];
     uint32_t in[4][kWaveTexels][28];
+    // Positional encoding for every power-of-two positionScale 2^-k, k = 0..5: the entry for phase p of scale
+    // 2^-k sits at index (2^k - 1) + p; dwords 0..2 hold enc(px * 2^w), dwords 3..5 enc(px * 2^w + 1/4), w = 0..2,
+    // as e4m3-rounded halves in the low 16 bits (px = p * 2^-k).
+    uint32_t postab[64][8];
 };
 
 // OCP e4m3 byte -> the integer 512 * value (NaN encodings decode as 0).
@@ -132,10 +141,25 @@ __device__ __forceinline__ void stage_plane_halves(uint32_t* dst, uint8_t const*
 // natural order (lane (i, kg) of a block of 32 holds inputs 8kg..8kg+7, of a block of 16 inputs 32+4kg..+3);
 // layers 1..3 take theirs in the order the previous layer's result registers hold them: lane (i, kg) of the
 // block for input tiles (2p, 2p+1) holds inputs 16*(2p + e/4) + 4kg + e%4, e = 0..7.
+// Returns a mask: bit l set when some weight of hidden layer l has a non-zero top plane (|w| >= 32); a layer
+// without one runs on two planes.
 template <class V>
-__device__ void stage_fp8_weights(Fp8Lds& lds, uint8_t const* __restrict__ blob)
+__device__ int stage_fp8_weights(Fp8Lds& lds, uint8_t const* __restrict__ blob)
 {
     int const tid = threadIdx.x;
+    int topMask = 0;
+    {
+        constexpr int first[3] = { 0, V::W1_OFF, V::W2_OFF }, count[3] = { V::W1_OFF, V::W2_OFF - V::W1_OFF, V::W3_OFF - V::W2_OFF };
+#pragma unroll
+        for (int l = 0; l < 3; ++l) {
+            int any = 0;
+            for (int e = tid; e < count[l]; e += V::THREADS) {
+                int32_t const w = fp8_times_512(blob[first[l] + e]);
+                any |= ((w < 0 ? -w : w) >> 14) != 0;
+            }
+            if (__syncthreads_or(any)) topMask |= 1 << l;
+        }
+    }
     // biases of the hidden layers (fp16 in the blob), scale and bias of the output layer
     for (int e = tid; e < 9 * 16; e += V::THREADS) {
         int const r = e & 3, g = (e >> 2) & 3, t = e >> 4;
@@ -185,6 +209,7 @@ __device__ void stage_fp8_weights(Fp8Lds& lds, uint8_t const* __restrict__ blob)
             dst[q >> 1] = __builtin_bit_cast(uint32_t, h);
         }
     }
+    return topMask;
 }
 
 // The 48 inputs of one texel as 24 dwords of e4m3-rounded halves (NtcPrepareNetworkInputsInternal_FP16,
@@ -238,15 +263,94 @@ __device__ __forceinline__ void prepare_inputs_fp8(DevMip const& m, int x, int y
     in[22] = round_e4m3_pk(halves_rne(m.positionLod, m.positionLod));
 }
 
+// The same 24 dwords from integer arithmetic, for mips whose sizes, grid sizes and positionScale are powers of
+// two (DevMip::fast).  There every float operation of prepare_inputs_fp8 is exact up to the fused multiply-add:
+// the filtered feature is t = T / 2^n with the integer T = sum w*q (weights w = products of the axis fractions,
+// summing to 2^n, n <= 8), and fma(t, c, -1) = fma(float(T), c * 2^-n, -1) is the same real number rounded
+// once.  T comes from the packed 16-bit-lane filter of the int8 kernel: a cell c = f0 | f1<<4 | f2<<8 | f3<<12
+// is spread to P = byte0 | byte1<<16, E = P & 0x000f000f holds the even features, S = sum w*P and T = sum w*E
+// stay below 2^16 per lane, and (S - T) / 16 holds the odd features.  The positional encoding of texel x depends
+// only on x mod 2^k for positionScale = 2^-k and comes from a table in LDS.
+template <class V>
+__device__ __forceinline__ void prepare_inputs_fp8_fast(DevMip const& m, Fp8Lds const& lds, int x, int y, uint32_t (&in)[24])
+{
+#pragma unroll
+    for (int i = 0; i < 24; ++i) in[i] = 0;
+    constexpr int layers = (V::F + 3) / 4;
+#pragma unroll
+    for (int grid = 0; grid < 2; ++grid) {
+        uint32_t const axisX = grid == 0 ? m.hrAxisX : m.lrAxisX, axisY = grid == 0 ? m.hrAxisY : m.lrAxisY;
+        int const gw = grid == 0 ? m.hrWidth : m.lrWidth, gh = grid == 0 ? m.hrHeight : m.lrHeight;
+        AxisFoot const ax = axis_fast(x, axisX, gw), ay = axis_fast(y, axisY, gh);
+        GlobalU8Ptr const g = (GlobalU8Ptr)(grid == 0 ? m.hr : m.lr);
+        uint32_t const lgw = ((axisX >> 24) & 0xffu) + 1u;       // log2(bytes per grid row)
+        uint32_t const layerStride = uint32_t(gw) * uint32_t(gh) * 2u;   // bytes
+        uint32_t const r0 = ay.c0 << lgw, r1 = ay.c1 << lgw, c0 = ax.c0 << 1, c1 = ax.c1 << 1;
+        uint32_t const a00 = r0 + c0, a10 = r0 + c1, a01 = r1 + c0, a11 = r1 + c1;   // byte offsets
+        uint32_t const nx = (axisX >> 8) & 0xffu, ny = (axisY >> 8) & 0xffu;
+        uint32_t const wx1 = ax.f, wx0 = (1u << nx) - ax.f, wy1 = ay.f, wy0 = (1u << ny) - ay.f;
+        uint32_t const w00 = mul24(wx0, wy0), w10 = mul24(wx1, wy0), w01 = mul24(wx0, wy1), w11 = mul24(wx1, wy1);
+        float const k = __builtin_ldexpf(0.13333334f, -int(nx + ny));
+        uint32_t const msk = 0x000f000fu, sel = 0x0c010c00u;     // v_perm_b32: bytes [0, zero, 1, zero] of the cell
+#pragma unroll
+        for (int L = 0; L < layers; ++L) {
+            GlobalU8Ptr const gl = g + size_t(L) * layerStride;
+            uint32_t const p00 = __builtin_amdgcn_perm(0u, load_u16(gl, a00), sel), p10 = __builtin_amdgcn_perm(0u, load_u16(gl, a10), sel);
+            uint32_t const p01 = __builtin_amdgcn_perm(0u, load_u16(gl, a01), sel), p11 = __builtin_amdgcn_perm(0u, load_u16(gl, a11), sel);
+            uint32_t const S = mad24(w11, p11, mad24(w01, p01, mad24(w10, p10, mul24(w00, p00))));
+            uint32_t const T = mad24(w11, p11 & msk, mad24(w01, p01 & msk, mad24(w10, p10 & msk, mul24(w00, p00 & msk))));
+            uint32_t const O = (S - T) >> 4;                     // lanes: features 1 and 3; T: features 0 and 2
+            float value[4] = { float(T & 0xffffu), float(O & 0xffffu), float(T >> 16), float(O >> 16) };
+#pragma unroll
+            for (int i = 0; i < 4; ++i) value[i] = (4 * L + i < V::F) ? __builtin_fmaf(value[i], k, -1.f) : 0.f;
+            in[8 * grid + 2 * L]     = round_e4m3_pk(halves_rne(value[0], value[1]));
+            in[8 * grid + 2 * L + 1] = round_e4m3_pk(halves_rne(value[2], value[3]));
+        }
+    }
+    {
+        uint32_t const* const ex = lds.postab[m.posMask + (uint32_t(x) & m.posMask)];
+        uint32_t const* const ey = lds.postab[m.posMask + (uint32_t(y) & m.posMask)];
+        uint4 const x0 = *reinterpret_cast<uint4 const*>(ex), y0 = *reinterpret_cast<uint4 const*>(ey);
+        uint2 const x1 = *reinterpret_cast<uint2 const*>(ex + 4), y1 = *reinterpret_cast<uint2 const*>(ey + 4);
+        in[16] = x0.x | (y0.x << 16);  in[17] = x0.w | (y0.w << 16);     // (e0, e1), (e2, e3) of wave 0
+        in[18] = x0.y | (y0.y << 16);  in[19] = x1.x | (y1.x << 16);
+        in[20] = x0.z | (y0.z << 16);  in[21] = x1.y | (y1.y << 16);
+    }
+    in[22] = round_e4m3_pk(halves_rne(m.positionLod, m.positionLod));
+}
+
+// Fills the positional table: one entry per thread, threads 0..62.
+__device__ void build_fp8_posenc_table(Fp8Lds& lds)
+{
+    int const t = threadIdx.x;
+    if (t < 63) {
+        int const k = 31 - __builtin_clz(uint32_t(t + 1));   // floor(log2(t + 1))
+        int const phase = t + 1 - (1 << k);
+        float p = float(phase) * __builtin_ldexpf(1.f, -k);
+#pragma unroll
+        for (int w = 0; w < 3; ++w) {
+            float const q = p + 0.25f;
+            float const e0 = (p - floorf(p)) * 2.f - 1.f, e2 = (q - floorf(q)) * 2.f - 1.f;
+            uint32_t const pair = round_e4m3_pk(halves_rne(e0, e2));
+            lds.postab[t][w] = pair & 0xffffu;
+            lds.postab[t][3 + w] = pair >> 16;
+            p *= 2.f;
+        }
+        lds.postab[t][6] = lds.postab[t][7] = 0;
+    }
+}
+
 // One hidden layer's epilogue for the four channels a lane holds of one texel: sums of the three planes ->
 // layer output -> activation -> the next layer's inputs (two dwords of halves).
-template <bool LAST_HIDDEN>
+// With TOP_PLANE false the top plane of the layer's weights is all zero: s2 = +0 and (s2 + s1) = s1 exactly
+// (a plane's sum is never -0: its accumulator starts at +0), so the first addition is left out.
+template <bool LAST_HIDDEN, bool TOP_PLANE>
 __device__ __forceinline__ void fp8_epilogue(v4f s2, v4f s1, v4f s0, v4f bias, uint32_t (&out)[2])
 {
     float r[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        float a = s2[i] + s1[i];
+        float a = TOP_PLANE ? s2[i] + s1[i] : s1[i];
         a = a + s0[i];
         r[i] = a + bias[i];
     }
@@ -264,17 +368,111 @@ __device__ __forceinline__ void mfma32(uint4 const& a, uint4 const (&x)[4], v4f 
 #pragma unroll
     for (int b = 0; b < 4; ++b) acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, __builtin_bit_cast(v8h, x[b]), acc[b], 0, 0, 0);
 }
+// The same for a block of 16 inputs.  32-deep and 16-deep instructions are never mixed in one accumulator's
+// chain: in either order that gave wrong sums here with some instruction schedules (the wait between the two
+// was not always there; compiling with padded matrix instructions made the same code correct), while chains of
+// one kind are reliable.  Layers whose input count is not a multiple of 32 therefore split their 32-deep blocks
+// with mfma32_as_two_16: a block's unit holds k-slots 8kg..8kg+7 of lane (i, kg) on both sides, so its first and
+// last four halves are two valid 16-deep operands.  The matrix pipeline takes the same time either way.
 __device__ __forceinline__ void mfma16(uint2 const& a, uint2 const (&x)[4], v4f (&acc)[4])
 {
     v4h const A = __builtin_bit_cast(v4h, a);
 #pragma unroll
     for (int b = 0; b < 4; ++b) acc[b] = __builtin_amdgcn_mfma_f32_16x16x16f16(A, __builtin_bit_cast(v4h, x[b]), acc[b], 0, 0, 0);
 }
+__device__ __forceinline__ void mfma32_as_two_16(uint4 const& a, uint4 const (&x)[4], v4f (&acc)[4])
+{
+    uint2 lo[4], hi[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) { lo[b] = make_uint2(x[b].x, x[b].y); hi[b] = make_uint2(x[b].z, x[b].w); }
+    mfma16(make_uint2(a.x, a.y), lo, acc);
+    mfma16(make_uint2(a.z, a.w), hi, acc);
+}
 
-// The FP8 network for the 64 texels of one wave.  `in` is the lane's own texel.  On return D[b] holds, for
-// lane (j, g), the int32 accumulators of output channels 4g..4g+3 of texel 16b + j, and S their scales.
+// Hidden layers.  PLANES = 3, or 2 when the layer's top plane is all zero (see stage_fp8_weights).
+template <class V, int PLANES>
+__device__ __forceinline__ void fp8_layer0(Fp8Lds const& lds, int lane, uint4 const (&X32)[4], uint2 const (&X16)[4], uint32_t (&H)[4][4][2])
+{
+    int const g = lane >> 4;
+    v4f const zero = { 0.f, 0.f, 0.f, 0.f };
+#pragma unroll
+    for (int t = 0; t < V::T0; ++t) {
+        v4f acc[3][4];
+#pragma unroll
+        for (int p = 0; p < 3; ++p) {
+#pragma unroll
+            for (int b = 0; b < 4; ++b) acc[p][b] = zero;
+            if (p >= PLANES) continue;
+            mfma32_as_two_16(lds.w0[p][t][lane], X32, acc[p]);
+            mfma16(reinterpret_cast<uint2 const*>(&lds.w0[p][t][64])[lane], X16, acc[p]);
+        }
+        v4f const bias = *reinterpret_cast<v4f const*>(&lds.bias[t][g][0]);
+#pragma unroll
+        for (int b = 0; b < 4; ++b) fp8_epilogue<false, PLANES == 3>(acc[2][b], acc[1][b], acc[0][b], bias, H[b][t]);
+    }
+}
+
+template <class V, int PLANES>
+__device__ __forceinline__ void fp8_layer1(Fp8Lds const& lds, int lane, uint32_t const (&Hin)[4][4][2], uint32_t (&H)[4][4][2])
+{
+    int const g = lane >> 4;
+    v4f const zero = { 0.f, 0.f, 0.f, 0.f };
+#pragma unroll
+    for (int t = 0; t < V::T1; ++t) {
+        v4f acc[3][4];
+#pragma unroll
+        for (int p = 0; p < 3; ++p) {
+#pragma unroll
+            for (int b = 0; b < 4; ++b) acc[p][b] = zero;
+            if (p >= PLANES) continue;
+#pragma unroll
+            for (int pair = 0; pair < 2; ++pair) {
+                uint4 x[4];
+#pragma unroll
+                for (int b = 0; b < 4; ++b) x[b] = make_uint4(Hin[b][2 * pair][0], Hin[b][2 * pair][1], Hin[b][2 * pair + 1][0], Hin[b][2 * pair + 1][1]);
+                mfma32(lds.w1[p][t][pair * 64 + lane], x, acc[p]);
+            }
+        }
+        v4f const bias = *reinterpret_cast<v4f const*>(&lds.bias[V::T0 + t][g][0]);
+#pragma unroll
+        for (int b = 0; b < 4; ++b) fp8_epilogue<false, PLANES == 3>(acc[2][b], acc[1][b], acc[0][b], bias, H[b][t]);
+    }
+}
+
+// layer 2: its activations are quantised to the int8 inputs of the output layer
+template <class V, int PLANES>
+__device__ __forceinline__ void fp8_layer2(Fp8Lds const& lds, int lane, uint32_t const (&Hin)[4][4][2], uint32_t (&H)[4][4][2])
+{
+    int const g = lane >> 4;
+    v4f const zero = { 0.f, 0.f, 0.f, 0.f };
+#pragma unroll
+    for (int t = 0; t < V::T2; ++t) {
+        v4f acc[3][4];
+#pragma unroll
+        for (int p = 0; p < 3; ++p) {
+            uint4 x[4];
+            uint2 xt[4];
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                acc[p][b] = zero;
+                x[b] = make_uint4(Hin[b][0][0], Hin[b][0][1], Hin[b][1][0], Hin[b][1][1]);
+                xt[b] = make_uint2(Hin[b][2][0], Hin[b][2][1]);
+            }
+            if (p >= PLANES) continue;
+            mfma32_as_two_16(lds.w2[p][t][lane], x, acc[p]);
+            mfma16(reinterpret_cast<uint2 const*>(&lds.w2[p][t][64])[lane], xt, acc[p]);
+        }
+        v4f const bias = *reinterpret_cast<v4f const*>(&lds.bias[V::T0 + V::T1 + t][g][0]);
+#pragma unroll
+        for (int b = 0; b < 4; ++b) fp8_epilogue<true, PLANES == 3>(acc[2][b], acc[1][b], acc[0][b], bias, H[b][t]);
+    }
+}
+
+// The FP8 network for the 64 texels of one wave.  `in` is the lane's own texel; `topMask` (uniform) says which
+// hidden layers need their top weight plane.  On return D[b] holds, for lane (j, g), the int32 accumulators of
+// output channels 4g..4g+3 of texel 16b + j, and S their scales.
 template <class V>
-__device__ __forceinline__ void mlp_forward_fp8(Fp8Lds& lds, int wave, int lane, uint32_t const (&in)[24], v4i (&D)[4], v4f& S)
+__device__ __forceinline__ void mlp_forward_fp8(Fp8Lds& lds, int wave, int lane, int topMask, uint32_t const (&in)[24], v4i (&D)[4], v4f& S)
 {
     int const j = lane & 15, g = lane >> 4;
     // transpose: lane = texel -> lane (j, kg) holds inputs 8kg..8kg+7 (block of 32) and 32+4kg..+3 (block of 16)
@@ -296,66 +494,13 @@ __device__ __forceinline__ void mlp_forward_fp8(Fp8Lds& lds, int wave, int lane,
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
 
-    v4f const zero = { 0.f, 0.f, 0.f, 0.f };
-    // layer 0: 48 -> 64
     uint32_t Ha[4][4][2], Hb[4][4][2];                       // [texel block][tile of 16 channels][2 dwords = 4 halves]
-#pragma unroll
-    for (int t = 0; t < V::T0; ++t) {
-        v4f acc[3][4];
-#pragma unroll
-        for (int p = 0; p < 3; ++p) {
-#pragma unroll
-            for (int b = 0; b < 4; ++b) acc[p][b] = zero;
-            mfma32(lds.w0[p][t][lane], X32, acc[p]);
-            mfma16(reinterpret_cast<uint2 const*>(&lds.w0[p][t][64])[lane], X16, acc[p]);
-        }
-        v4f const bias = *reinterpret_cast<v4f const*>(&lds.bias[t][g][0]);
-#pragma unroll
-        for (int b = 0; b < 4; ++b) fp8_epilogue<false>(acc[2][b], acc[1][b], acc[0][b], bias, Ha[b][t]);
-    }
-    // layer 1: 64 -> 48
-#pragma unroll
-    for (int t = 0; t < V::T1; ++t) {
-        v4f acc[3][4];
-#pragma unroll
-        for (int p = 0; p < 3; ++p) {
-#pragma unroll
-            for (int b = 0; b < 4; ++b) acc[p][b] = zero;
-#pragma unroll
-            for (int pair = 0; pair < 2; ++pair) {
-                uint4 x[4];
-#pragma unroll
-                for (int b = 0; b < 4; ++b) x[b] = make_uint4(Ha[b][2 * pair][0], Ha[b][2 * pair][1], Ha[b][2 * pair + 1][0], Ha[b][2 * pair + 1][1]);
-                mfma32(lds.w1[p][t][pair * 64 + lane], x, acc[p]);
-            }
-        }
-        v4f const bias = *reinterpret_cast<v4f const*>(&lds.bias[V::T0 + t][g][0]);
-#pragma unroll
-        for (int b = 0; b < 4; ++b) fp8_epilogue<false>(acc[2][b], acc[1][b], acc[0][b], bias, Hb[b][t]);
-    }
-    // layer 2: 48 -> 32, its activations quantised to the int8 inputs of the output layer
-#pragma unroll
-    for (int t = 0; t < V::T2; ++t) {
-        v4f acc[3][4];
-#pragma unroll
-        for (int p = 0; p < 3; ++p) {
-            uint4 x[4];
-            uint2 xt[4];
-#pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                acc[p][b] = zero;
-                x[b] = make_uint4(Hb[b][0][0], Hb[b][0][1], Hb[b][1][0], Hb[b][1][1]);
-                xt[b] = make_uint2(Hb[b][2][0], Hb[b][2][1]);
-            }
-            mfma32(lds.w2[p][t][lane], x, acc[p]);
-            mfma16(reinterpret_cast<uint2 const*>(&lds.w2[p][t][64])[lane], xt, acc[p]);
-        }
-        v4f const bias = *reinterpret_cast<v4f const*>(&lds.bias[V::T0 + V::T1 + t][g][0]);
-#pragma unroll
-        for (int b = 0; b < 4; ++b) fp8_epilogue<true>(acc[2][b], acc[1][b], acc[0][b], bias, Ha[b][t]);
-    }
+    if (topMask & 1) fp8_layer0<V, 3>(lds, lane, X32, X16, Ha); else fp8_layer0<V, 2>(lds, lane, X32, X16, Ha);   // 48 -> 64
+    if (topMask & 2) fp8_layer1<V, 3>(lds, lane, Ha, Hb);      else fp8_layer1<V, 2>(lds, lane, Ha, Hb);           // 64 -> 48
+    if (topMask & 4) fp8_layer2<V, 3>(lds, lane, Hb, Ha);      else fp8_layer2<V, 2>(lds, lane, Hb, Ha);           // 48 -> 32
     // output layer: 32 -> 16, exact: |sum W q| <= 32 * 127 * 128 < 2^24
     {
+        v4f const zero = { 0.f, 0.f, 0.f, 0.f };
         v4f acc[4] = { zero, zero, zero, zero };
         uint4 x[4];
 #pragma unroll
@@ -384,15 +529,18 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     int const tileBegin = blockIdx.x * per;
     int const tileEnd = min(totalTiles, tileBegin + per);
 
+    build_fp8_posenc_table(lds);
+
     uint8_t const* stagedBlob = nullptr;
+    int topMask = 7;                                         // uniform: hidden layers that need their top weight plane
     int entry = 0;
     for (int tile = tileBegin; tile < tileEnd; ++tile) {
         while (entry + 1 < numMips && mips[entry + 1].tileStart <= tile) ++entry;
         if (mips[entry].weights != stagedBlob) {             // uniform across the workgroup
             __syncthreads();
-            stage_fp8_weights<V>(lds, mips[entry].weights);
+            topMask = stage_fp8_weights<V>(lds, mips[entry].weights);
             stagedBlob = mips[entry].weights;
-            __syncthreads();
+            __syncthreads();                                 // also publishes the table built above
         }
         DevMip const& m = mips[entry];
         int const local = tile - m.tileStart;
@@ -402,10 +550,14 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
         if (x0 >= m.width) continue;                         // whole wave tile outside the image
 
         uint32_t in[24];
-        prepare_inputs_fp8<V>(m, min(x0 + j, m.width - 1), min(y0 + g, m.height - 1), in);
+        {
+            int const x = min(x0 + j, m.width - 1), y = min(y0 + g, m.height - 1);
+            if (m.fast) prepare_inputs_fp8_fast<V>(m, lds, x, y, in);
+            else        prepare_inputs_fp8<V>(m, x, y, in);
+        }
         v4i D[4];
         v4f S;
-        mlp_forward_fp8<V>(lds, wave, lane, in, D, S);
+        mlp_forward_fp8<V>(lds, wave, lane, topMask, in, D, S);
         if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)      store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, x0 + j, y0, 4 * g);
         else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)       store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
         else                                                       store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, x0 + j, y0, 4 * g);

@@ -30,29 +30,26 @@
 namespace ntc_hip_dev {
 
 // HGELU-clamp + requantise of four D values of one lane (Inference.hlsli:36-39,123-131,164-179).
-// round-half-even of y*80 is taken from the low mantissa bits of y*80 + 1.5*2^23; the "-113"
-// (= +143 mod 256) and the byte packing are one SDWA integer add per value.
-__device__ __forceinline__ uint32_t activate4(v4i acc, v4f scale, uint32_t c143)
+// round-half-even of y*80 is taken from the low mantissa bits of y*80 + 1.5*2^23; the four low bytes are
+// gathered with byte permutes and the "-113" (= +143 mod 256) is one add on all four bytes at once, with the
+// carries kept inside each byte.  No inline assembly here: the compiler adds the wait states that matrix
+// instructions in flight require only around instructions it can see.
+__device__ __forceinline__ uint32_t activate4(v4i acc, v4f scale)
 {
-    float z[4];
+    uint32_t z[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         float const x = float(acc[r]) * scale[r];
         float t = __builtin_fmaf(x, 0.333333f, 0.5f);
         t = fminf(fmaxf(t, 0.f), 1.f);
         float const y = fminf(x, 3.f) * t;
-        z[r] = y * 80.f + 12582912.f;                        // low byte = rne(y*80) mod 256
+        z[r] = __builtin_bit_cast(uint32_t, y * 80.f + 12582912.f);     // low byte = rne(y*80) mod 256
     }
-    uint32_t packed;
-    asm("v_add_u32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:BYTE_0 src1_sel:DWORD"
-        : "=v"(packed) : "v"(z[0]), "v"(c143));
-    asm("v_add_u32_sdwa %0, %1, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_0 src1_sel:DWORD"
-        : "+v"(packed) : "v"(z[1]), "v"(c143));
-    asm("v_add_u32_sdwa %0, %1, %2 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_0 src1_sel:DWORD"
-        : "+v"(packed) : "v"(z[2]), "v"(c143));
-    asm("v_add_u32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_0 src1_sel:DWORD"
-        : "+v"(packed) : "v"(z[3]), "v"(c143));
-    return packed;
+    uint32_t const lo = __builtin_amdgcn_perm(z[1], z[0], 0x0c0c0400u);  // bytes [z0.0, z1.0, 0, 0]
+    uint32_t const hi = __builtin_amdgcn_perm(z[3], z[2], 0x04000c0cu);  // bytes [0, 0, z2.0, z3.0]
+    uint32_t const p = lo | hi;
+    // p + 0x8f8f8f8f byte by byte: low seven bits added with room for the carry, top bits combined by xor
+    return ((p & 0x7f7f7f7fu) + 0x0f0f0f0fu) ^ (~p & 0x80808080u);
 }
 
 // ---- all-integer input stage (power-of-two mip and grid sizes) --------------------------
@@ -60,28 +57,6 @@ __device__ __forceinline__ uint32_t activate4(v4i acc, v4f scale, uint32_t c143)
 // With W and the grid size powers of two, u*Wg - 1/2 = ((2x+1)*2^e - 1)/2 with e = log2(Wg/W):
 // floor and fraction are shifts and masks, the bilinear weights are small integers, and
 // every float operation of the general path is exact, so both paths give the same bytes.
-
-struct AxisFoot { uint32_t c0, c1, f; };
-
-__device__ __forceinline__ AxisFoot axis_fast(int x, uint32_t packedAxis, int gridSize)
-{
-    int const shl = int(packedAxis & 0xffu), n = int((packedAxis >> 8) & 0xffu), sublog = int((packedAxis >> 16) & 0xffu);
-    int const N = ((2 * x + 1) << shl) - (1 << sublog);
-    int const b = N >> n;                                    // arithmetic shift = floor
-    AxisFoot a;
-    a.f = uint32_t(N) & ((1u << n) - 1u);
-    a.c0 = uint32_t(b) & uint32_t(gridSize - 1);             // wrap addressing
-    a.c1 = uint32_t(b + 1) & uint32_t(gridSize - 1);
-    return a;
-}
-
-// 24-bit multiply-add, full rate: a * b + c.
-__device__ __forceinline__ uint32_t mad24(uint32_t a, uint32_t b, uint32_t c)
-{
-    uint32_t r;
-    asm("v_mad_u32_u24 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-    return r;
-}
 
 // Four 4-bit features of the four taps, filtered: ((17 * sum w*q) >> n) - 128 per byte; the weights w sum to 2^n
 // (n <= 8).  A cell c = f0 | f1<<4 | f2<<8 | f3<<12 is spread to P = byte0 | byte1<<16 (16-bit lanes holding
@@ -828,7 +803,7 @@ __device__ __forceinline__ void transpose_inputs(LdsT<V>& lds, int wave, int lan
 // On return D[b] holds, for lane (j = lane%16, g = lane/16), the int32 accumulators of output
 // channels 4g..4g+3 of texel 16*b + j, and S their scales.
 template <class V>
-__device__ __forceinline__ void mlp_forward(LdsT<V>& lds, int wave, int lane, uint32_t const (&in)[16], uint32_t c143,
+__device__ __forceinline__ void mlp_forward(LdsT<V>& lds, int wave, int lane, uint32_t const (&in)[16],
                                             v4i (&D)[4], v4f& S)
 {
     int const g = lane >> 4;
@@ -869,13 +844,13 @@ __device__ __forceinline__ void mlp_forward(LdsT<V>& lds, int wave, int lane, ui
 #pragma unroll
                     for (int r = 0; r < 4; ++r)                    // 4096*D2 + 64*D1 + D0, wrapping like int32
                         Dh[r] = int((((uint32_t(D2[r]) << 6) + uint32_t(D1[r])) << 6) + uint32_t(D0[r]));
-                    Y[b][t] = activate4(Dh, Sc, c143);
+                    Y[b][t] = activate4(Dh, Sc);
                 }
             } else {
 #pragma unroll
                 for (int b = 0; b < 4; ++b) {
                     v4i const Dh = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
-                    Y[b][t] = activate4(Dh, Sc, c143);
+                    Y[b][t] = activate4(Dh, Sc);
                 }
             }
         }
@@ -943,21 +918,37 @@ __device__ __forceinline__ void f16_tile(LdsT<V> const& lds, int base, int t, in
 {
     constexpr int PAIRS = IN_TILES / 2, PER = V::f16_units(IN_TILES);
     uint4 const* const block = lds.late + base + t * PER;
+    if constexpr (IN_TILES % 2 == 0) {
 #pragma unroll
-    for (int p = 0; p < PAIRS; ++p) {
-        v8h const A = __builtin_bit_cast(v8h, block[p * 64 + lane]);
+        for (int p = 0; p < PAIRS; ++p) {
+            v8h const A = __builtin_bit_cast(v8h, block[p * 64 + lane]);
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            uint4 const h = make_uint4(H[b][2 * p][0], H[b][2 * p][1], H[b][2 * p + 1][0], H[b][2 * p + 1][1]);
-            acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, __builtin_bit_cast(v8h, h), acc[b], 0, 0, 0);
+            for (int b = 0; b < 4; ++b) {
+                uint4 const h = make_uint4(H[b][2 * p][0], H[b][2 * p][1], H[b][2 * p + 1][0], H[b][2 * p + 1][1]);
+                acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, __builtin_bit_cast(v8h, h), acc[b], 0, 0, 0);
+            }
         }
-    }
-    if constexpr (IN_TILES % 2 == 1) {
-        v4h const A = __builtin_bit_cast(v4h, reinterpret_cast<uint2 const*>(block + PAIRS * 64)[lane]);
+    } else {
+        // An odd number of input tiles: every tile takes the 16-deep instruction (a pair's block holds tile 2p in
+        // its first four halves per lane and tile 2p+1 in the last four).  32-deep and 16-deep instructions are
+        // never mixed in one accumulator's chain: in either order that gave wrong sums with some instruction
+        // schedules (the wait between the two was not always there), while chains of one kind are reliable; the
+        // matrix pipeline takes the same time either way.
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            uint2 const h = make_uint2(H[b][IN_TILES - 1][0], H[b][IN_TILES - 1][1]);
-            acc[b] = __builtin_amdgcn_mfma_f32_16x16x16f16(A, __builtin_bit_cast(v4h, h), acc[b], 0, 0, 0);
+        for (int ti = 0; ti < IN_TILES; ++ti) {
+            uint2 a;
+            if (ti < 2 * PAIRS) {
+                uint4 const unit = block[(ti >> 1) * 64 + lane];
+                a = (ti & 1) ? make_uint2(unit.z, unit.w) : make_uint2(unit.x, unit.y);
+            } else {
+                a = reinterpret_cast<uint2 const*>(block + PAIRS * 64)[lane];
+            }
+            v4h const A = __builtin_bit_cast(v4h, a);
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                uint2 const h = make_uint2(H[b][ti][0], H[b][ti][1]);
+                acc[b] = __builtin_amdgcn_mfma_f32_16x16x16f16(A, __builtin_bit_cast(v4h, h), acc[b], 0, 0, 0);
+            }
         }
     }
 }
@@ -1087,9 +1078,6 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
         lds.lut2[threadIdx.x & 0xffu] = (x * 85u) ^ 0x80808080u;
     }
 
-    uint32_t c143 = 143u;
-    asm volatile("" : "+v"(c143));                           // stays in a VGPR: SDWA operands cannot be literals
-
     build_posenc_tables<V>(lds);
 
     uint8_t const* stagedBlob = nullptr;
@@ -1154,7 +1142,7 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
         } else {
             v4i D[4];
             v4f S;
-            mlp_forward<V>(lds, wave, lane, in, c143, D, S);
+            mlp_forward<V>(lds, wave, lane, in, D, S);
             if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)      store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, x0 + j, y0, 4 * g);
             else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)       store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
             else                                                       store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
@@ -1206,8 +1194,6 @@ query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __res
     int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int const j = lane & 15, g = lane >> 4;
 
-    uint32_t c143 = 143u;
-    asm volatile("" : "+v"(c143));
 
     {   // 2-bit code bytes -> input bytes (see decode_kernel)
         uint32_t x = threadIdx.x & 0xffu;
@@ -1246,7 +1232,7 @@ query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __res
             mlp_forward_f16<V>(lds, wave, lane, in, F, S);
         } else {
             v4i D[4];
-            mlp_forward<V>(lds, wave, lane, in, c143, D, S);
+            mlp_forward<V>(lds, wave, lane, in, D, S);
 #pragma unroll
             for (int b = 0; b < 4; ++b) F[b] = v4f{ float(D[b][0]), float(D[b][1]), float(D[b][2]), float(D[b][3]) };
         }

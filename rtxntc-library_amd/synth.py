@@ -39,7 +39,8 @@ def e4m3_encode(values):
 
 def make_fp8_weights(spec, seed, weight_sigma=0.35, bias_sigma=0.3, out_scale_log2_range=(-14.0, -11.0)):
     """The GenericFP8 blob (reference src/WeightLayout.cpp:51-71) for `spec` (weightType FP8): e4m3 hidden-layer
-    weights ~ N(0, weight_sigma / sqrt(fan-in) * 4), fp16 biases ~ N(0, bias_sigma), and an int8 output layer."""
+    weights ~ N(0, weight_sigma / sqrt(fan-in) * 4) (weight_sigma: one value, or one per hidden layer), fp16
+    biases ~ N(0, bias_sigma), and an int8 output layer."""
     assert spec.weightType == abi.WEIGHTS_FP8
     layout = weight_layout(spec)
     rng = np.random.default_rng(seed)
@@ -49,7 +50,8 @@ def make_fp8_weights(spec, seed, weight_sigma=0.35, bias_sigma=0.3, out_scale_lo
         n_in, n_out = spec.layer_inputs(layer), spec.layer_outputs(layer)
         at = layout.weightOffset[layer]
         if layer < last:
-            w = rng.normal(0.0, weight_sigma * 4.0 / np.sqrt(n_in), size=(n_out, n_in))
+            sigma = weight_sigma[layer] if isinstance(weight_sigma, (tuple, list)) else weight_sigma
+            w = rng.normal(0.0, sigma * 4.0 / np.sqrt(n_in), size=(n_out, n_in))
             blob[at:at + n_in * n_out] = e4m3_encode(w).reshape(-1)
             bias = rng.normal(0.0, bias_sigma, size=n_out).astype(np.float16)
             blob[layout.biasOffset[layer]:layout.biasOffset[layer] + 2 * n_out] = bias.view(np.uint8)

@@ -233,6 +233,42 @@ def test_gpu_fp8_decode_with_extreme_weights(ntc, device):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("sigmas", [(300.0, 0.35, 0.35), (0.35, 300.0, 0.35), (0.35, 0.35, 300.0), (40.0, 0.35, 40.0)])
+def test_gpu_fp8_decode_with_large_weights_in_some_layers(ntc, device, sigmas):
+    """A hidden layer whose weights all stay below 32 runs without its top weight plane; layers are decided one
+    by one.  Power-of-two sizes, so the integer input stage runs as well."""
+    case = fp8_case(ntc, 16, 128, 64, 8, 2, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=31, weight_sigma=sigmas, bias_sigma=1.0)
+    expected, got = run_both(device, case)
+    assert first_mismatch(expected, got) is None, sigmas
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("features,grid_scale,w,h", [(16, 1, 256, 64), (16, 2, 64, 256), (12, 4, 512, 128), (8, 2, 128, 128), (4, 4, 256, 256)])
+def test_gpu_fp8_integer_input_stage_equals_checker(ntc, device, features, grid_scale, w, h):
+    """Power-of-two mips, grids and position scales take the all-integer input stage (and the positional table);
+    every mip down to 1 x 1, where footprints wrap around grids one or two cells wide."""
+    case = fp8_case(ntc, features, w, h, ntc.presets.full_mip_count(w, h), grid_scale, 16, ntc.abi.OUT_FP16_PIXELS, seed=7 * features + grid_scale)
+    expected, got = run_both(device, case)
+    mm = first_mismatch(expected, got)
+    assert mm is None, f"{mm[1]} of {expected.size} bytes differ, first at {mm[0]}"
+
+
+@pytest.mark.gpu
+def test_gpu_fp8_batch_mixes_sets_with_and_without_top_planes(ntc, device):
+    """One launch over sets whose weights need three planes, two planes, three again: the plane choice follows the
+    staged set."""
+    sigmas = [300.0, 0.35, (0.35, 300.0, 0.35), 0.35]
+    cases = [fp8_case(ntc, 8, 64, 32, 6, 2, 8, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=90 + i, weight_sigma=s) for i, s in enumerate(sigmas)]
+    hosts = [c.host_set() for c in cases]
+    for hset in hosts:
+        hset.decode(threads=8)
+    device.decode([c.device_set(device) for c in cases])
+    device.synchronize()
+    for i, (c, hset) in enumerate(zip(cases, hosts)):
+        assert first_mismatch(hset.output, c.d_output.download()) is None, i
+
+
+@pytest.mark.gpu
 def test_gpu_fp8_batch_of_sets_and_static_table(ntc, device):
     cases = [fp8_case(ntc, 8, 64, 64, 7, 2, 8, ntc.abi.OUT_UNORM8_PIXELS, seed=80 + i) for i in range(3)]
     hosts = [c.host_set() for c in cases]
