@@ -20,12 +20,16 @@ __device__ __forceinline__ uint32_t load_u16(GlobalU8Ptr base, uint32_t byteOffs
     return *reinterpret_cast<GlobalU16Ptr>(base + byteOffset);
 }
 
-// 24-bit multiply, full rate (a plain 32-bit multiply is quarter rate).  Written with the builtin rather
-// than inline assembly on purpose: the compiler inserts the wait states that matrix instructions in flight
-// need only around instructions it can see, and an assembly statement is opaque to it.
+// 24-bit multiply, full rate.  Inline assembly because the compiler turns the builtin back into the
+// quarter-rate 32-bit multiply in places.  Only for the input stages: the compiler inserts the wait states that
+// matrix instructions in flight need around instructions it can see, and an assembly statement is opaque to it.
+// The input stage of a tile runs when none is in flight - after the previous tile's results were read for
+// its stores and before this tile's first matrix instruction, in a basic block of its own.
 __device__ __forceinline__ uint32_t mul24(uint32_t a, uint32_t b)
 {
-    return __umul24(a, b);
+    uint32_t r;
+    asm("v_mul_u32_u24 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
 }
 // Footprint of one axis of a bilinear tap pair in integers, for power-of-two sizes: with
 // p = u*grid - 1/2 = N / 2^n, N = ((2x+1) << shl) - (1 << sublog) (the packed axis word of DevMip),
@@ -44,10 +48,12 @@ __device__ __forceinline__ AxisFoot axis_fast(int x, uint32_t packedAxis, int gr
     return a;
 }
 
-// 24-bit multiply-add, full rate: a * b + c (v_mad_u32_u24).
+// 24-bit multiply-add, full rate: a * b + c.  Input stages only, like mul24.
 __device__ __forceinline__ uint32_t mad24(uint32_t a, uint32_t b, uint32_t c)
 {
-    return __umul24(a, b) + c;
+    uint32_t r;
+    asm("v_mad_u32_u24 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
 }
 
 typedef float v4f __attribute__((ext_vector_type(4)));
