@@ -29,10 +29,12 @@ namespace ntc_hip_dev {
 
 typedef short v2s __attribute__((ext_vector_type(2)));
 
-// Two halves -> the nearest e4m3 values (as halves): v_cvt_scalef32_pk_fp8_f16 and back, scale 1.
+// Two halves -> the nearest e4m3 values (as halves): v_cvt_scalef32_pk_fp8_f16 and back, scale 1.  The first
+// instruction writes the two bytes into one half of its destination and keeps the other half; that other half
+// is never read here, so the destination starts as the source itself and needs no clearing.
 __device__ __forceinline__ uint32_t round_e4m3_pk(uint32_t halves)
 {
-    v2s const bytes = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(v2s{ 0, 0 }, __builtin_bit_cast(v2h, halves), 1.0f, false);
+    v2s const bytes = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(__builtin_bit_cast(v2s, halves), __builtin_bit_cast(v2h, halves), 1.0f, false);
     v2h const back = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(__builtin_bit_cast(uint32_t, bytes), 1.0f, false);
     return __builtin_bit_cast(uint32_t, back);
 }
@@ -52,6 +54,10 @@ __device__ __forceinline__ uint32_t halves_rne(float a, float b)
 // inline assembly: these instructions are interleaved with matrix instructions, and the compiler inserts the
 // wait states an in-flight matrix instruction needs (e.g. before one of its source registers is overwritten)
 // only around instructions it can see.
+// LOWER_CLAMP false leaves out max(x, -3).  For finite x < -3 that changes nothing: t is +0 from x = -1.5 down,
+// and x * (+0) = -3 * (+0) = -0.  It differs for x = -Inf or NaN only (-Inf * 0 is NaN, -3 * 0 is not), so it is
+// for layers whose outputs are known to be finite.
+template <bool LOWER_CLAMP = true>
 __device__ __forceinline__ uint32_t hgelu_pk(uint32_t xBits)
 {
     v2h const x = __builtin_bit_cast(v2h, xBits);
@@ -59,7 +65,7 @@ __device__ __forceinline__ uint32_t hgelu_pk(uint32_t xBits)
     v2h const zero = { _Float16(0.f), _Float16(0.f) }, one = { _Float16(1.f), _Float16(1.f) }, three = { _Float16(3.f), _Float16(3.f) };
     v2h t = __builtin_elementwise_fma(x, third, half);
     t = __builtin_elementwise_min(__builtin_elementwise_max(t, zero), one);
-    v2h const xc = __builtin_elementwise_min(__builtin_elementwise_max(x, -three), three);
+    v2h const xc = __builtin_elementwise_min(LOWER_CLAMP ? __builtin_elementwise_max(x, -three) : x, three);
     return __builtin_bit_cast(uint32_t, xc * t);
 }
 
@@ -141,8 +147,10 @@ __device__ __forceinline__ void stage_plane_halves(uint32_t* dst, uint8_t const*
 // natural order (lane (i, kg) of a block of 32 holds inputs 8kg..8kg+7, of a block of 16 inputs 32+4kg..+3);
 // layers 1..3 take theirs in the order the previous layer's result registers hold them: lane (i, kg) of the
 // block for input tiles (2p, 2p+1) holds inputs 16*(2p + e/4) + 4kg + e%4, e = 0..7.
-// Returns a mask: bit l set when some weight of hidden layer l has a non-zero top plane (|w| >= 32); a layer
-// without one runs on two planes.
+// Returns a mask: bit l set when hidden layer l needs the general evaluation (three planes, both clamps of the
+// activation), i.e. when some weight of it has a non-zero top plane (|w| >= 32) or some bias is not a finite
+// half of magnitude <= 57344.  The other layers (every layer of a trained network) are "tame": two planes, and
+// since |sum| <= 64 * 31.75 * 3 = 6096 their outputs stay below 63440 + rounding < 65520, finite as halves.
 template <class V>
 __device__ int stage_fp8_weights(Fp8Lds& lds, uint8_t const* __restrict__ blob)
 {
@@ -157,6 +165,8 @@ __device__ int stage_fp8_weights(Fp8Lds& lds, uint8_t const* __restrict__ blob)
                 int32_t const w = fp8_times_512(blob[first[l] + e]);
                 any |= ((w < 0 ? -w : w) >> 14) != 0;
             }
+            constexpr int firstBias[3] = { 0, V::H0, V::H0 + V::H1 }, biases[3] = { V::H0, V::H1, V::H2 };
+            if (tid < biases[l]) any |= (reinterpret_cast<uint16_t const*>(blob + V::BIAS_OFF)[firstBias[l] + tid] & 0x7fffu) > 0x7b00u;
             if (__syncthreads_or(any)) topMask |= 1 << l;
         }
     }
@@ -271,12 +281,20 @@ __device__ __forceinline__ void prepare_inputs_fp8(DevMip const& m, int x, int y
 // is spread to P = byte0 | byte1<<16, E = P & 0x000f000f holds the even features, S = sum w*P and T = sum w*E
 // stay below 2^16 per lane, and (S - T) / 16 holds the odd features.  The positional encoding of texel x depends
 // only on x mod 2^k for positionScale = 2^-k and comes from a table in LDS.
+//
+// The stage comes in two halves so that a tile's latent loads can be in flight while the previous tile runs
+// through the network: fetch_latents_fast issues the loads (four taps of every stored layer of both grids) and
+// keeps the four axis fractions, finish_inputs_fast does the arithmetic.
 template <class V>
-__device__ __forceinline__ void prepare_inputs_fp8_fast(DevMip const& m, Fp8Lds const& lds, int x, int y, uint32_t (&in)[24])
+struct Fp8Fetch {
+    static constexpr int LAYERS = (V::F + 3) / 4;
+    uint32_t cell[2][LAYERS][4];                             // [grid][layer][tap 00, 10, 01, 11]
+    uint32_t fx[2], fy[2];                                   // axis fractions of the footprint, per grid
+};
+
+template <class V>
+__device__ __forceinline__ void fetch_latents_fast(DevMip const& m, int x, int y, Fp8Fetch<V>& f)
 {
-#pragma unroll
-    for (int i = 0; i < 24; ++i) in[i] = 0;
-    constexpr int layers = (V::F + 3) / 4;
 #pragma unroll
     for (int grid = 0; grid < 2; ++grid) {
         uint32_t const axisX = grid == 0 ? m.hrAxisX : m.lrAxisX, axisY = grid == 0 ? m.hrAxisY : m.lrAxisY;
@@ -287,16 +305,33 @@ __device__ __forceinline__ void prepare_inputs_fp8_fast(DevMip const& m, Fp8Lds 
         uint32_t const layerStride = uint32_t(gw) * uint32_t(gh) * 2u;   // bytes
         uint32_t const r0 = ay.c0 << lgw, r1 = ay.c1 << lgw, c0 = ax.c0 << 1, c1 = ax.c1 << 1;
         uint32_t const a00 = r0 + c0, a10 = r0 + c1, a01 = r1 + c0, a11 = r1 + c1;   // byte offsets
+        f.fx[grid] = ax.f; f.fy[grid] = ay.f;
+#pragma unroll
+        for (int L = 0; L < Fp8Fetch<V>::LAYERS; ++L) {
+            GlobalU8Ptr const gl = g + size_t(L) * layerStride;
+            f.cell[grid][L][0] = load_u16(gl, a00); f.cell[grid][L][1] = load_u16(gl, a10);
+            f.cell[grid][L][2] = load_u16(gl, a01); f.cell[grid][L][3] = load_u16(gl, a11);
+        }
+    }
+}
+
+template <class V>
+__device__ __forceinline__ void finish_inputs_fast(DevMip const& m, Fp8Lds const& lds, int x, int y, Fp8Fetch<V> const& f, uint32_t (&in)[24])
+{
+#pragma unroll
+    for (int i = 0; i < 24; ++i) in[i] = 0;
+#pragma unroll
+    for (int grid = 0; grid < 2; ++grid) {
+        uint32_t const axisX = grid == 0 ? m.hrAxisX : m.lrAxisX, axisY = grid == 0 ? m.hrAxisY : m.lrAxisY;
         uint32_t const nx = (axisX >> 8) & 0xffu, ny = (axisY >> 8) & 0xffu;
-        uint32_t const wx1 = ax.f, wx0 = (1u << nx) - ax.f, wy1 = ay.f, wy0 = (1u << ny) - ay.f;
+        uint32_t const wx1 = f.fx[grid], wx0 = (1u << nx) - wx1, wy1 = f.fy[grid], wy0 = (1u << ny) - wy1;
         uint32_t const w00 = mul24(wx0, wy0), w10 = mul24(wx1, wy0), w01 = mul24(wx0, wy1), w11 = mul24(wx1, wy1);
         float const k = __builtin_ldexpf(0.13333334f, -int(nx + ny));
         uint32_t const msk = 0x000f000fu, sel = 0x0c010c00u;     // v_perm_b32: bytes [0, zero, 1, zero] of the cell
 #pragma unroll
-        for (int L = 0; L < layers; ++L) {
-            GlobalU8Ptr const gl = g + size_t(L) * layerStride;
-            uint32_t const p00 = __builtin_amdgcn_perm(0u, load_u16(gl, a00), sel), p10 = __builtin_amdgcn_perm(0u, load_u16(gl, a10), sel);
-            uint32_t const p01 = __builtin_amdgcn_perm(0u, load_u16(gl, a01), sel), p11 = __builtin_amdgcn_perm(0u, load_u16(gl, a11), sel);
+        for (int L = 0; L < Fp8Fetch<V>::LAYERS; ++L) {
+            uint32_t const p00 = __builtin_amdgcn_perm(0u, f.cell[grid][L][0], sel), p10 = __builtin_amdgcn_perm(0u, f.cell[grid][L][1], sel);
+            uint32_t const p01 = __builtin_amdgcn_perm(0u, f.cell[grid][L][2], sel), p11 = __builtin_amdgcn_perm(0u, f.cell[grid][L][3], sel);
             uint32_t const S = mad24(w11, p11, mad24(w01, p01, mad24(w10, p10, mul24(w00, p00))));
             uint32_t const T = mad24(w11, p11 & msk, mad24(w01, p01 & msk, mad24(w10, p10 & msk, mul24(w00, p00 & msk))));
             uint32_t const O = (S - T) >> 4;                     // lanes: features 1 and 3; T: features 0 and 2
@@ -342,8 +377,9 @@ __device__ void build_fp8_posenc_table(Fp8Lds& lds)
 
 // One hidden layer's epilogue for the four channels a lane holds of one texel: sums of the three planes ->
 // layer output -> activation -> the next layer's inputs (two dwords of halves).
-// With TOP_PLANE false the top plane of the layer's weights is all zero: s2 = +0 and (s2 + s1) = s1 exactly
-// (a plane's sum is never -0: its accumulator starts at +0), so the first addition is left out.
+// With TOP_PLANE false the layer is tame (see stage_fp8_weights): the top plane of its weights is all zero,
+// s2 = +0 and (s2 + s1) = s1 exactly (a plane's sum is never -0: its accumulator starts at +0), so the first
+// addition is left out; and its outputs are finite, so the activation's lower clamp is left out too.
 template <bool LAST_HIDDEN, bool TOP_PLANE>
 __device__ __forceinline__ void fp8_epilogue(v4f s2, v4f s1, v4f s0, v4f bias, uint32_t (&out)[2])
 {
@@ -356,7 +392,7 @@ __device__ __forceinline__ void fp8_epilogue(v4f s2, v4f s1, v4f s0, v4f bias, u
     }
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-        uint32_t const y = hgelu_pk(halves_rne(r[2 * h], r[2 * h + 1]));
+        uint32_t const y = hgelu_pk<TOP_PLANE>(halves_rne(r[2 * h], r[2 * h + 1]));
         out[h] = LAST_HIDDEN ? quantize_int8_pk(y) : round_e4m3_pk(y);
     }
 }
@@ -389,7 +425,7 @@ __device__ __forceinline__ void mfma32_as_two_16(uint4 const& a, uint4 const (&x
     mfma16(make_uint2(a.z, a.w), hi, acc);
 }
 
-// Hidden layers.  PLANES = 3, or 2 when the layer's top plane is all zero (see stage_fp8_weights).
+// Hidden layers.  PLANES = 3, or 2 for a tame layer (see stage_fp8_weights).
 template <class V, int PLANES>
 __device__ __forceinline__ void fp8_layer0(Fp8Lds const& lds, int lane, uint4 const (&X32)[4], uint2 const (&X16)[4], uint32_t (&H)[4][4][2])
 {
@@ -469,7 +505,7 @@ __device__ __forceinline__ void fp8_layer2(Fp8Lds const& lds, int lane, uint32_t
 }
 
 // The FP8 network for the 64 texels of one wave.  `in` is the lane's own texel; `topMask` (uniform) says which
-// hidden layers need their top weight plane.  On return D[b] holds, for lane (j, g), the int32 accumulators of
+// hidden layers need the general evaluation.  On return D[b] holds, for lane (j, g), the int32 accumulators of
 // output channels 4g..4g+3 of texel 16b + j, and S their scales.
 template <class V>
 __device__ __forceinline__ void mlp_forward_fp8(Fp8Lds& lds, int wave, int lane, int topMask, uint32_t const (&in)[24], v4i (&D)[4], v4f& S)
@@ -515,7 +551,26 @@ __device__ __forceinline__ void mlp_forward_fp8(Fp8Lds& lds, int wave, int lane,
     }
 }
 
-// 76.5 KB of LDS: two workgroups per CU.
+// Where a wave stands in the image for one workgroup tile: the mip's table entry, the wave tile's corner and
+// whether any of it lies inside the image.  All uniform across the wave.
+struct WaveTile { int entry, x0, y0; bool work; };
+
+__device__ __forceinline__ WaveTile locate_tile(DevMip const* __restrict__ mips, int numMips, int tile, int entry, int wave)
+{
+    while (entry + 1 < numMips && mips[entry + 1].tileStart <= tile) ++entry;
+    DevMip const& m = mips[entry];
+    int const local = tile - m.tileStart;
+    int const tileY = local / m.tilesX, tileX = local - tileY * m.tilesX;
+    WaveTile t;
+    t.entry = entry; t.x0 = tileX * 64 + wave * 16; t.y0 = tileY * 4;
+    t.work = t.x0 < m.width;
+    return t;
+}
+
+// 77 KB of LDS: two workgroups per CU, two waves per SIMD, up to 256 registers per lane.  With so few waves
+// nothing else covers a tile's latent loads, so the loop is staggered: the loads of tile i+1 are issued before
+// tile i goes through the network and turned into tile i+1's input vector right after it, before tile i's
+// stores - at which point they have long arrived, and no store is ever waited for.
 template <class V>
 __global__ void __launch_bounds__(V::THREADS, 2)
 decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
@@ -528,39 +583,60 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     int const per = (totalTiles + gridDim.x - 1) / gridDim.x;
     int const tileBegin = blockIdx.x * per;
     int const tileEnd = min(totalTiles, tileBegin + per);
+    if (tileBegin >= tileEnd) return;                        // uniform across the workgroup
 
     build_fp8_posenc_table(lds);
+    __syncthreads();
 
     uint8_t const* stagedBlob = nullptr;
-    int topMask = 7;                                         // uniform: hidden layers that need their top weight plane
-    int entry = 0;
-    for (int tile = tileBegin; tile < tileEnd; ++tile) {
-        while (entry + 1 < numMips && mips[entry + 1].tileStart <= tile) ++entry;
-        if (mips[entry].weights != stagedBlob) {             // uniform across the workgroup
-            __syncthreads();
-            topMask = stage_fp8_weights<V>(lds, mips[entry].weights);
-            stagedBlob = mips[entry].weights;
-            __syncthreads();                                 // also publishes the table built above
-        }
-        DevMip const& m = mips[entry];
-        int const local = tile - m.tileStart;
-        int const tileY = local / m.tilesX, tileX = local - tileY * m.tilesX;
-        int const x0 = tileX * 64 + wave * 16;
-        int const y0 = tileY * 4;
-        if (x0 >= m.width) continue;                         // whole wave tile outside the image
+    int topMask = 7;                                         // uniform: hidden layers that need the general evaluation
+    uint32_t in[24];
+    Fp8Fetch<V> fetch;
 
-        uint32_t in[24];
-        {
-            int const x = min(x0 + j, m.width - 1), y = min(y0 + g, m.height - 1);
-            if (m.fast) prepare_inputs_fp8_fast<V>(m, lds, x, y, in);
-            else        prepare_inputs_fp8<V>(m, x, y, in);
+    // Input vector of the lane's texel of a wave tile; `fetched` says that fetch_latents_fast ran for it.
+    auto inputs_of = [&](WaveTile const& t, bool fetched) {
+        DevMip const& m = mips[t.entry];
+        int const x = min(t.x0 + j, m.width - 1), y = min(t.y0 + g, m.height - 1);
+        if (fetched) finish_inputs_fast<V>(m, lds, x, y, fetch, in);
+        else         prepare_inputs_fp8<V>(m, x, y, in);
+    };
+    auto fetch_of = [&](WaveTile const& t) -> bool {
+        DevMip const& m = mips[t.entry];
+        if (!t.work || !m.fast) return false;
+        fetch_latents_fast<V>(m, min(t.x0 + j, m.width - 1), min(t.y0 + g, m.height - 1), fetch);
+        return true;
+    };
+
+    WaveTile cur = locate_tile(mips, numMips, tileBegin, 0, wave);
+    {
+        bool const fetched = fetch_of(cur);
+        if (cur.work) inputs_of(cur, fetched);
+    }
+    for (int tile = tileBegin; tile < tileEnd; ++tile) {
+        DevMip const& m = mips[cur.entry];
+        if (m.weights != stagedBlob) {                       // uniform across the workgroup
+            __syncthreads();
+            topMask = stage_fp8_weights<V>(lds, m.weights);
+            stagedBlob = m.weights;
+            __syncthreads();
+        }
+        bool const more = tile + 1 < tileEnd;
+        WaveTile next = cur;
+        bool fetched = false;
+        if (more) {
+            next = locate_tile(mips, numMips, tile + 1, cur.entry, wave);
+            fetched = fetch_of(next);
         }
         v4i D[4];
         v4f S;
-        mlp_forward_fp8<V>(lds, wave, lane, topMask, in, D, S);
-        if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)      store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, x0 + j, y0, 4 * g);
-        else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)       store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
-        else                                                       store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
+        if (cur.work) mlp_forward_fp8<V>(lds, wave, lane, topMask, in, D, S);
+        if (more && next.work) inputs_of(next, fetched);
+        if (cur.work) {
+            if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)      store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, cur.x0 + j, cur.y0, 4 * g);
+            else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)       store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, cur.x0 + j, cur.y0, 4 * g);
+            else                                                       store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, cur.x0 + j, cur.y0, 4 * g);
+        }
+        cur = next;
     }
 }
 

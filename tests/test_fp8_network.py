@@ -243,6 +243,24 @@ def test_gpu_fp8_decode_with_large_weights_in_some_layers(ntc, device, sigmas):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("layer", [0, 1, 2])
+def test_gpu_fp8_decode_with_biases_at_and_beyond_the_finite_range(ntc, device, layer):
+    """A hidden layer with small weights and biases of at most 57344 in magnitude cannot leave the finite halves
+    and runs without the activation's lower clamp; one bias beyond that (the next half, an infinity, a NaN) sends
+    the layer through the general evaluation.  Both sides of the limit, in every hidden layer."""
+    spec = ntc.presets.spec_ref092_fp8(16)
+    layout = ntc.synth.weight_layout(spec)
+    for trial, specials in enumerate([(0x7B00, 0xFB00, 0x7AFF), (0x7B01,), (0xFB01,), (0x7C00, 0xFC00), (0x7E00, 0xFB00), (0xFBFF, 0x7BFF)]):
+        case = fp8_case(ntc, 16, 64, 32, 3, 2, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=200 + 10 * layer + trial, bias_sigma=0.5)
+        bias = case.weights[layout.biasOffset[layer]:layout.biasOffset[layer] + 2 * spec.layer_outputs(layer)].view(np.uint16)
+        for i, bits in enumerate(specials):
+            bias[5 + 7 * i] = bits
+        expected, got = run_both(device, case)
+        assert first_mismatch(expected, got) is None, (layer, specials)
+        assert len(np.unique(got.view(np.uint16))) > 500
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("features,grid_scale,w,h", [(16, 1, 256, 64), (16, 2, 64, 256), (12, 4, 512, 128), (8, 2, 128, 128), (4, 4, 256, 256)])
 def test_gpu_fp8_integer_input_stage_equals_checker(ntc, device, features, grid_scale, w, h):
     """Power-of-two mips, grids and position scales take the all-integer input stage (and the positional table);
