@@ -109,7 +109,12 @@ struct alignas(16) Fp8Lds {
     // 2^-k sits at index (2^k - 1) + p; dwords 0..2 hold enc(px * 2^w), dwords 3..5 enc(px * 2^w + 1/4), w = 0..2,
     // as e4m3-rounded halves in the low 16 bits (px = p * 2^-k).
     uint32_t postab[64][8];
+    // Filtered feature -> network input, for the integer input stage: entry kFeatureLutBase(n) + T holds the
+    // e4m3-rounded half of fma(float(T), (2/15) * 2^-n, -1) for T = 0 .. 15 * 2^n, n = 0, 2, 4, 6 (what square
+    // power-of-two geometry produces; other n take the arithmetic).
+    uint16_t featureLut[1280];
 };
+__host__ __device__ constexpr int kFeatureLutBase(int n) { return n == 0 ? 0 : (n == 2 ? 16 : (n == 4 ? 77 : 318)); }   // 16 + 61 + 241 + 961 = 1279 entries
 
 // OCP e4m3 byte -> the integer 512 * value (NaN encodings decode as 0).
 __device__ __forceinline__ int32_t fp8_times_512(uint32_t byte)
@@ -325,9 +330,31 @@ __device__ __forceinline__ void finish_inputs_fast(DevMip const& m, Fp8Lds const
         uint32_t const axisX = grid == 0 ? m.hrAxisX : m.lrAxisX, axisY = grid == 0 ? m.hrAxisY : m.lrAxisY;
         uint32_t const nx = (axisX >> 8) & 0xffu, ny = (axisY >> 8) & 0xffu;
         uint32_t const wx1 = f.fx[grid], wx0 = (1u << nx) - wx1, wy1 = f.fy[grid], wy0 = (1u << ny) - wy1;
+        uint32_t const msk = 0x000f000fu, sel = 0x0c010c00u;     // v_perm_b32: bytes [0, zero, 1, zero] of the cell
+        uint32_t const n = nx + ny;
+        if (V::F % 4 == 0 && n <= 6u && !(n & 1u)) {             // uniform
+            // Table form: with doubled weights and start values 2*base resp. 17 * 2*base the 16-bit lanes of T and
+            // O come out as byte offsets into the table (S stays below 2^16: 2 * 255 * 64 + 34 * 318).
+            uint32_t const w00 = mul24(2u * wx0, wy0), w10 = mul24(2u * wx1, wy0), w01 = mul24(2u * wx0, wy1), w11 = mul24(2u * wx1, wy1);
+            uint32_t const base = uint32_t(n == 0u ? kFeatureLutBase(0) : (n == 2u ? kFeatureLutBase(2) : (n == 4u ? kFeatureLutBase(4) : kFeatureLutBase(6))));
+            uint32_t const t0 = (2u * base) * 0x00010001u, s0 = 17u * t0;
+            uint8_t const* const lut = reinterpret_cast<uint8_t const*>(lds.featureLut);
+#pragma unroll
+            for (int L = 0; L < Fp8Fetch<V>::LAYERS; ++L) {
+                uint32_t const p00 = __builtin_amdgcn_perm(0u, f.cell[grid][L][0], sel), p10 = __builtin_amdgcn_perm(0u, f.cell[grid][L][1], sel);
+                uint32_t const p01 = __builtin_amdgcn_perm(0u, f.cell[grid][L][2], sel), p11 = __builtin_amdgcn_perm(0u, f.cell[grid][L][3], sel);
+                uint32_t const S = mad24(w11, p11, mad24(w01, p01, mad24(w10, p10, mad24(w00, p00, s0))));
+                uint32_t const T = mad24(w11, p11 & msk, mad24(w01, p01 & msk, mad24(w10, p10 & msk, mad24(w00, p00 & msk, t0))));
+                uint32_t const O = (S - T) >> 4;
+                v2s const a = { short(*reinterpret_cast<uint16_t const*>(lut + (T & 0xffffu))), short(*reinterpret_cast<uint16_t const*>(lut + (O & 0xffffu))) };
+                v2s const b = { short(*reinterpret_cast<uint16_t const*>(lut + (T >> 16))), short(*reinterpret_cast<uint16_t const*>(lut + (O >> 16))) };
+                in[8 * grid + 2 * L]     = __builtin_bit_cast(uint32_t, a);
+                in[8 * grid + 2 * L + 1] = __builtin_bit_cast(uint32_t, b);
+            }
+            continue;
+        }
         uint32_t const w00 = mul24(wx0, wy0), w10 = mul24(wx1, wy0), w01 = mul24(wx0, wy1), w11 = mul24(wx1, wy1);
         float const k = __builtin_ldexpf(0.13333334f, -int(nx + ny));
-        uint32_t const msk = 0x000f000fu, sel = 0x0c010c00u;     // v_perm_b32: bytes [0, zero, 1, zero] of the cell
 #pragma unroll
         for (int L = 0; L < Fp8Fetch<V>::LAYERS; ++L) {
             uint32_t const p00 = __builtin_amdgcn_perm(0u, f.cell[grid][L][0], sel), p10 = __builtin_amdgcn_perm(0u, f.cell[grid][L][1], sel);
@@ -372,6 +399,17 @@ __device__ void build_fp8_posenc_table(Fp8Lds& lds)
             p *= 2.f;
         }
         lds.postab[t][6] = lds.postab[t][7] = 0;
+    }
+}
+
+// Fills the feature table with the same operations the arithmetic path applies per lane.
+__device__ void build_fp8_feature_lut(Fp8Lds& lds)
+{
+    for (int e = threadIdx.x; e < 1279; e += blockDim.x) {
+        int const n = e < 16 ? 0 : (e < 77 ? 2 : (e < 318 ? 4 : 6));
+        int const T = e - kFeatureLutBase(n);
+        float const v = __builtin_fmaf(float(T), __builtin_ldexpf(0.13333334f, -n), -1.f);
+        lds.featureLut[e] = uint16_t(round_e4m3_pk(halves_rne(v, v)));
     }
 }
 
@@ -586,6 +624,7 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     if (tileBegin >= tileEnd) return;                        // uniform across the workgroup
 
     build_fp8_posenc_table(lds);
+    build_fp8_feature_lut(lds);
     __syncthreads();
 
     uint8_t const* stagedBlob = nullptr;
@@ -598,11 +637,17 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
         DevMip const& m = mips[t.entry];
         int const x = min(t.x0 + j, m.width - 1), y = min(t.y0 + g, m.height - 1);
         if (fetched) finish_inputs_fast<V>(m, lds, x, y, fetch, in);
+#ifdef NTC_EXP_NOPREFETCH
+        else if (m.fast) { fetch_latents_fast<V>(m, x, y, fetch); finish_inputs_fast<V>(m, lds, x, y, fetch, in); }
+#endif
         else         prepare_inputs_fp8<V>(m, x, y, in);
     };
     auto fetch_of = [&](WaveTile const& t) -> bool {
         DevMip const& m = mips[t.entry];
         if (!t.work || !m.fast) return false;
+#ifdef NTC_EXP_NOPREFETCH
+        return false;
+#endif
         fetch_latents_fast<V>(m, min(t.x0 + j, m.width - 1), min(t.y0 + g, m.height - 1), fetch);
         return true;
     };
