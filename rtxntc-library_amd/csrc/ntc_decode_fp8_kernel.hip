@@ -591,7 +591,7 @@ __device__ __forceinline__ void mlp_forward_fp8(Fp8Lds& lds, int wave, int lane,
 
 // Where a wave stands in the image for one workgroup tile: the mip's table entry, the wave tile's corner and
 // whether any of it lies inside the image.  All uniform across the wave.
-struct WaveTile { int entry, x0, y0; bool work; };
+struct WaveTile { int entry, x0, y0, work; };             // (four ints: a bool would leave padding bytes that copies carry through memory)
 
 __device__ __forceinline__ WaveTile locate_tile(DevMip const* __restrict__ mips, int numMips, int tile, int entry, int wave)
 {
@@ -601,7 +601,7 @@ __device__ __forceinline__ WaveTile locate_tile(DevMip const* __restrict__ mips,
     int const tileY = local / m.tilesX, tileX = local - tileY * m.tilesX;
     WaveTile t;
     t.entry = entry; t.x0 = tileX * 64 + wave * 16; t.y0 = tileY * 4;
-    t.work = t.x0 < m.width;
+    t.work = t.x0 < m.width ? 1 : 0;
     return t;
 }
 
