@@ -49,7 +49,8 @@ def measured_counters(workload, fmt_name):
         return None
     entry = table.get("workloads", {}).get(f"{workload}_{fmt_name}")
     if entry:
-        entry = dict(entry, source=f"profiles/{os.path.basename(COUNTERS_FILE)} (commit {table.get('commit', '?')})")
+        entry = dict(entry, source=f"profiles/{os.path.basename(COUNTERS_FILE)} (commit {table.get('commit', '?')})",
+                     issue_rates_ns=table.get("issue_rates_ns"))
     return entry
 
 
@@ -324,19 +325,26 @@ def main():
                    "sample": f"the first {n} queries of the same list, {t:.1f} s"}
 
     # Ceilings of the kernel, lowest first decides `bound`: HBM (algorithmic bytes), int8 MFMA (algorithmic
-    # operations), and vector-instruction issue: a CU issues 64 lane-operations per clock (no packed fp32), and a
-    # matrix instruction takes one such issue slot too, so the ceiling is CUs x 64 x clock / (issue slots per texel,
-    # from the SQ_INSTS_VALU and SQ_INSTS_MFMA counters).
+    # operations), and instruction issue.  The issue ceiling is what the kernel's own instruction stream would take
+    # if every instruction issued at the rate it reaches in isolation (profiles/valu_issue_rates_mi355x.md: plain
+    # fp32 / 32-bit integer instructions, the slower conversions / packed 16-bit / three-operand integer ones, and
+    # matrix instructions, which plain fp32 instructions do not overlap with): per 64-texel wave tile and SIMD,
+    #   SQ_INSTS_VALU x (share of plain ones x their ns + the rest x theirs) + SQ_INSTS_MFMA x their ns,
+    # with the instruction counts from the counters and the share from the kernel's assembly.
     counters = None if args.size else measured_counters(wl, fmt_name)
     rate = texels / (kernel_ms * 1e-3) / 1e9
     fracs = {"hbm": achieved_gbs / HBM_PEAK_GBS, "mfma": achieved_tops / INT8_PEAK_TOPS}
     valu = {}
-    if counters and counters.get("valu_ops_per_texel"):
-        mfma_slots = counters.get("SQ_INSTS_MFMA", 0) * 64 / counters["texels_per_launch"]
-        ceiling = dev.compute_units * 64 * dev.clock_ghz / (counters["valu_ops_per_texel"] + mfma_slots)
+    if counters and counters.get("valu_ops_per_texel") and counters.get("issue_rates_ns"):
+        rates = counters["issue_rates_ns"]
+        mfma_per_tile = counters.get("SQ_INSTS_MFMA", 0) * 64 / counters["texels_per_launch"]
+        share = counters["valu_plain_share"]
+        tile_ns = counters["valu_ops_per_texel"] * (share * rates["plain"] + (1.0 - share) * rates["other"]) + mfma_per_tile * rates["matrix"]
+        ceiling = dev.compute_units * 4 * 64 / tile_ns                 # Gtexels/s: four SIMDs a CU, 64 texels a wave tile
         fracs["valu"] = rate / ceiling
-        valu = {"valu_ops_per_texel": counters["valu_ops_per_texel"], "mfma_issue_slots_per_texel": mfma_slots,
-                "valu_clock_ghz": dev.clock_ghz,
+        valu = {"valu_ops_per_texel": counters["valu_ops_per_texel"], "mfma_per_wave_tile": mfma_per_tile,
+                "valu_plain_share": share, "issue_rates_ns": rates,
+                "issue_ns_per_wave_tile_model": tile_ns, "issue_ns_per_wave_tile_measured": dev.compute_units * 4 * 64 / rate,
                 "valu_ceiling_gtexels": ceiling, "valu_frac": fracs["valu"], "counters_source": counters["source"]}
     line = {
         "metric": "decoded Gtexels/s, 4096^2 16-ch set, 64-48-32 int8; % of int8-MFMA/HBM roof",

@@ -202,7 +202,11 @@ __device__ __forceinline__ uint32_t halves_of_bytes(uint32_t v, int firstByte)  
 // |bias| + 128*sum|512 w| < 2^31); otherwise they are staged as int8 tiles.
 // With kStagedF16, kOutputsBounded says that no output can come near the fp16 overflow threshold
 // (the same bound times the channel's scale stays below 60000), so stores may skip that check.
-constexpr int kStagedF16 = 1, kOutputsBounded = 2;
+// kL0Magic (with kStagedF16, variants without e4m3 weights): layer 0's accumulators start at bias + 0x4B400000,
+// so that the int32 result, read as a float, is 1.5 * 2^23 + acc and one fp32 subtraction replaces the conversion
+// (needs |acc| < 2^22: |bias| <= 3 100 000 for every channel, the inputs add at most 64 * 128 * 127).
+constexpr int kStagedF16 = 1, kOutputsBounded = 2, kL0Magic = 4;
+constexpr int32_t kMagicBits = 0x4B400000;                   // 12582912.0f = 1.5 * 2^23
 template <class V>
 __device__ int stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
 {
@@ -293,6 +297,19 @@ __device__ int stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
     }
     bool const useF16 = __syncthreads_and(fits ? 1 : 0) != 0;     // also orders the bias writes above
     bool const outputsBounded = __syncthreads_and(bounded ? 1 : 0) != 0;
+    bool l0Magic = false;
+    if constexpr (!V::FP8_WEIGHTS) {
+        bool small = true;
+        if (threadIdx.x < V::H0) {
+            int32_t const b = reinterpret_cast<int32_t const*>(blob + V::BIAS_OFF)[threadIdx.x];
+            small = b >= -3100000 && b <= 3100000;
+        }
+        l0Magic = (__syncthreads_and(small ? 1 : 0) != 0) && useF16;
+        if (l0Magic && threadIdx.x < V::H0) {
+            int const c = threadIdx.x;
+            lds.bias[c >> 4][(c >> 2) & 3][c & 3] += kMagicBits;
+        }
+    }
     constexpr int base[4] = { 0, V::F16_L1, V::F16_L2, V::F16_L3 };
     uint32_t* const late32 = reinterpret_cast<uint32_t*>(lds.late);
     if (useF16) {
@@ -360,7 +377,7 @@ __device__ int stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
             tileBase += tiles[l];
         }
     }
-    return useF16 ? (kStagedF16 | (outputsBounded ? kOutputsBounded : 0)) : 0;
+    return useF16 ? (kStagedF16 | (outputsBounded ? kOutputsBounded : 0) | (l0Magic ? kL0Magic : 0)) : 0;
 }
 
 template <class V>
@@ -1000,7 +1017,7 @@ __device__ __forceinline__ void f16_hidden_layer_two_planes(LdsT<V> const& lds, 
 // Same interface as mlp_forward, except that D holds the output layer's accumulators as floats
 // (exact integers).
 template <class V>
-__device__ __forceinline__ void mlp_forward_f16(LdsT<V>& lds, int wave, int lane, uint32_t const (&in)[16], v4f (&D)[4], v4f& S)
+__device__ __forceinline__ void mlp_forward_f16(LdsT<V>& lds, int wave, int lane, bool l0Magic, uint32_t const (&in)[16], v4f (&D)[4], v4f& S)
 {
     int const g = lane >> 4;
     v4i X[4];
@@ -1008,6 +1025,27 @@ __device__ __forceinline__ void mlp_forward_f16(LdsT<V>& lds, int wave, int lane
 
     // layer 0: int8 inputs, int32 accumulators (three planes for e4m3 weights, recombined wrapping like int32)
     uint32_t Ha[4][4][2], Hb[4][4][2];
+    if (!V::FP8_WEIGHTS && l0Magic) {                        // uniform
+        // the accumulator started at bias + 0x4B400000: its bits are the float 1.5 * 2^23 + acc, exactly
+#pragma unroll
+        for (int t = 0; t < V::T0; ++t) {
+            uint4 const wq = *reinterpret_cast<uint4 const*>(&lds.w[0][t][lane][0]);
+            v4i const A = v4i{ int(wq.x), int(wq.y), int(wq.z), int(wq.w) };
+            v4i const C = *reinterpret_cast<v4i const*>(&lds.bias[t][g][0]);
+            v4f const Sc = *reinterpret_cast<v4f const*>(&lds.scale[t][g][0]);
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                v4i const Dh = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
+                v4f acc;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    int32_t const bits = Dh[r];                  // (a copy: bit_cast of a vector element expression reads element 0)
+                    acc[r] = __builtin_bit_cast(float, bits) - 12582912.f;
+                }
+                activate4_h(acc, Sc, Ha[b][t]);
+            }
+        }
+    } else {
 #pragma unroll
     for (int t = 0; t < V::T0; ++t) {
         auto const operand = [&](int q) {
@@ -1036,6 +1074,7 @@ __device__ __forceinline__ void mlp_forward_f16(LdsT<V>& lds, int wave, int lane
             for (int b = 0; b < 4; ++b)
                 activate4_h(__builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0), Sc, Ha[b][t]);
         }
+    }
     }
     if constexpr (V::FP8_WEIGHTS) {
         f16_hidden_layer_two_planes<V, V::T0, V::T1>(lds, V::F16_L1, V::T0, lane, Ha, Hb);
@@ -1129,7 +1168,7 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
         if (V::F16_LAYERS && (staged & kStagedF16)) {
             v4f D[4];
             v4f S;
-            mlp_forward_f16<V>(lds, wave, lane, in, D, S);
+            mlp_forward_f16<V>(lds, wave, lane, (staged & kL0Magic) != 0, in, D, S);
             if (staged & kOutputsBounded) {
                 if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)  store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS, false>(m, D, S, x0 + j, y0, 4 * g);
                 else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)   store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS, false>(m, D, S, x0 + j, y0, 4 * g);
@@ -1202,7 +1241,8 @@ query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __res
         lds.lut2[threadIdx.x & 0xffu] = (x * 85u) ^ 0x80808080u;
     }
     build_posenc_tables<V>(lds);
-    bool const useF16 = (stage_weights<V>(lds, mips[0].weights) & kStagedF16) != 0;
+    int const staged = stage_weights<V>(lds, mips[0].weights);
+    bool const useF16 = (staged & kStagedF16) != 0;
     __syncthreads();
 
     uint64_t const numBlocks = (numQueries + V::THREADS - 1) / V::THREADS;
@@ -1229,7 +1269,7 @@ query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __res
         v4f F[4];
         v4f S;
         if (V::F16_LAYERS && useF16) {
-            mlp_forward_f16<V>(lds, wave, lane, in, F, S);
+            mlp_forward_f16<V>(lds, wave, lane, (staged & kL0Magic) != 0, in, F, S);
         } else {
             v4i D[4];
             mlp_forward<V>(lds, wave, lane, in, D, S);

@@ -273,6 +273,23 @@ def test_fp16_layer_path_boundary(ntc, device, slack):
         assert_equal_bytes(expected, got, f"fp16 path boundary, slack {slack}, sign {sign}")
 
 
+@pytest.mark.parametrize("spec_name", ["spec_cfg01", "spec_cfg2"])
+def test_layer0_conversion_shortcut_boundary(ntc, device, spec_name):
+    """Layer 0's int32 accumulators are read as floats through a magic-number start value while every bias of the
+    layer is at most 3 100 000 in magnitude (|acc| < 2^22); one bias at the limit and one just past it, with both
+    signs, send a set through either form of the layer."""
+    spec = getattr(ntc.presets, spec_name)()
+    layout = ntc.synth.weight_layout(spec)
+    for value in (3100000, 3100001, -3100000, -3100001):
+        blob = ntc.synth.make_weights(spec, 90 + abs(value) % 5, scale_log2_range=(-22.0, -21.0))
+        bias = blob[layout.biasOffset[0]:layout.bufferSize].view(np.int32)
+        bias[7] = value
+        bias[40] = -value // 2
+        case = cfg_case(ntc, spec, 128, 64, 3, 12, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=91, weights=blob)
+        expected, got = run_both(device, case)
+        assert_equal_bytes(expected, got, f"layer-0 conversion shortcut, bias {value}")
+
+
 def test_outputs_beyond_the_fp16_range_become_zero(ntc, device):
     """Large output scales: network outputs pass 65520 in magnitude, which the contract stores as 0
     (Inference.cu:125-126).  The weights still qualify for the fp16 form of layers 1..3, but not for
