@@ -464,53 +464,84 @@ __device__ __forceinline__ void mfma32_as_two_16(uint4 const& a, uint4 const (&x
 }
 
 // Hidden layers.  PLANES = 3, or 2 for a tame layer (see stage_fp8_weights).
-template <class V, int PLANES>
-__device__ __forceinline__ void fp8_layer0(Fp8Lds const& lds, int lane, uint4 const (&X32)[4], uint2 const (&X16)[4], uint32_t (&H)[4][4][2])
+//
+// With two waves on a SIMD little else covers the LDS latency of a tile's weight operands, so a layer loads the
+// operands of output tile t + 1 before it works on tile t (two sets of registers, alternating), and a scheduling
+// barrier that only LDS reads may not cross keeps the compiler from moving those loads back down to their uses.
+template <int NK32, bool HAS16>
+struct TileOperands { uint4 a32[3][NK32]; uint2 a16[3]; v4f bias; };
+
+// One hidden layer: TILES output tiles of 16 channels; its inputs as NK32 blocks of 32 (B32[kb][b]) and, with
+// HAS16, one block of 16 (B16[b]); load(t, operands) reads tile t's weight operands and bias.  A layer with a
+// block of 16 runs on 16-deep instructions only (see mfma16).
+template <int PLANES, int TILES, int NK32, bool HAS16, bool LAST_HIDDEN, class Load>
+__device__ __forceinline__ void fp8_hidden_layer(Load&& load, uint4 const (&B32)[NK32][4], uint2 const (&B16)[4], uint32_t (&H)[4][4][2])
 {
-    int const g = lane >> 4;
     v4f const zero = { 0.f, 0.f, 0.f, 0.f };
+    TileOperands<NK32, HAS16> ops[2];
+    load(0, ops[0]);
 #pragma unroll
-    for (int t = 0; t < V::T0; ++t) {
+    for (int t = 0; t < TILES; ++t) {
+        if (t + 1 < TILES) {
+            load(t + 1, ops[(t + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0x67f);           // everything but LDS instructions may cross
+        }
+        TileOperands<NK32, HAS16> const& o = ops[t & 1];
         v4f acc[3][4];
 #pragma unroll
         for (int p = 0; p < 3; ++p) {
 #pragma unroll
             for (int b = 0; b < 4; ++b) acc[p][b] = zero;
             if (p >= PLANES) continue;
-            mfma32_as_two_16(lds.w0[p][t][lane], X32, acc[p]);
-            mfma16(reinterpret_cast<uint2 const*>(&lds.w0[p][t][64])[lane], X16, acc[p]);
-        }
-        v4f const bias = *reinterpret_cast<v4f const*>(&lds.bias[t][g][0]);
 #pragma unroll
-        for (int b = 0; b < 4; ++b) fp8_epilogue<false, PLANES == 3>(acc[2][b], acc[1][b], acc[0][b], bias, H[b][t]);
+            for (int kb = 0; kb < NK32; ++kb) {
+                if (HAS16) mfma32_as_two_16(o.a32[p][kb], B32[kb], acc[p]);
+                else       mfma32(o.a32[p][kb], B32[kb], acc[p]);
+            }
+            if (HAS16) mfma16(o.a16[p], B16, acc[p]);
+        }
+#pragma unroll
+        for (int b = 0; b < 4; ++b) fp8_epilogue<LAST_HIDDEN, PLANES == 3>(acc[2][b], acc[1][b], acc[0][b], o.bias, H[b][t]);
     }
+}
+
+template <class V, int PLANES>
+__device__ __forceinline__ void fp8_layer0(Fp8Lds const& lds, int lane, uint4 const (&X32)[4], uint2 const (&X16)[4], uint32_t (&H)[4][4][2])
+{
+    int const g = lane >> 4;
+    uint4 B32[1][4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) B32[0][b] = X32[b];
+    fp8_hidden_layer<PLANES, V::T0, 1, true, false>([&](int t, TileOperands<1, true>& o) {
+#pragma unroll
+        for (int p = 0; p < PLANES; ++p) {
+            o.a32[p][0] = lds.w0[p][t][lane];
+            o.a16[p] = reinterpret_cast<uint2 const*>(&lds.w0[p][t][64])[lane];
+        }
+        o.bias = *reinterpret_cast<v4f const*>(&lds.bias[t][g][0]);
+    }, B32, X16, H);
 }
 
 template <class V, int PLANES>
 __device__ __forceinline__ void fp8_layer1(Fp8Lds const& lds, int lane, uint32_t const (&Hin)[4][4][2], uint32_t (&H)[4][4][2])
 {
     int const g = lane >> 4;
-    v4f const zero = { 0.f, 0.f, 0.f, 0.f };
+    uint4 B32[2][4];
+    uint2 B16[4];
 #pragma unroll
-    for (int t = 0; t < V::T1; ++t) {
-        v4f acc[3][4];
-#pragma unroll
-        for (int p = 0; p < 3; ++p) {
-#pragma unroll
-            for (int b = 0; b < 4; ++b) acc[p][b] = zero;
-            if (p >= PLANES) continue;
-#pragma unroll
-            for (int pair = 0; pair < 2; ++pair) {
-                uint4 x[4];
-#pragma unroll
-                for (int b = 0; b < 4; ++b) x[b] = make_uint4(Hin[b][2 * pair][0], Hin[b][2 * pair][1], Hin[b][2 * pair + 1][0], Hin[b][2 * pair + 1][1]);
-                mfma32(lds.w1[p][t][pair * 64 + lane], x, acc[p]);
-            }
-        }
-        v4f const bias = *reinterpret_cast<v4f const*>(&lds.bias[V::T0 + t][g][0]);
-#pragma unroll
-        for (int b = 0; b < 4; ++b) fp8_epilogue<false, PLANES == 3>(acc[2][b], acc[1][b], acc[0][b], bias, H[b][t]);
+    for (int b = 0; b < 4; ++b) {
+        B32[0][b] = make_uint4(Hin[b][0][0], Hin[b][0][1], Hin[b][1][0], Hin[b][1][1]);
+        B32[1][b] = make_uint4(Hin[b][2][0], Hin[b][2][1], Hin[b][3][0], Hin[b][3][1]);
+        B16[b] = make_uint2(0u, 0u);
     }
+    fp8_hidden_layer<PLANES, V::T1, 2, false, false>([&](int t, TileOperands<2, false>& o) {
+#pragma unroll
+        for (int p = 0; p < PLANES; ++p) {
+            o.a32[p][0] = lds.w1[p][t][lane];
+            o.a32[p][1] = lds.w1[p][t][64 + lane];
+        }
+        o.bias = *reinterpret_cast<v4f const*>(&lds.bias[V::T0 + t][g][0]);
+    }, B32, B16, H);
 }
 
 // layer 2: its activations are quantised to the int8 inputs of the output layer
@@ -518,28 +549,21 @@ template <class V, int PLANES>
 __device__ __forceinline__ void fp8_layer2(Fp8Lds const& lds, int lane, uint32_t const (&Hin)[4][4][2], uint32_t (&H)[4][4][2])
 {
     int const g = lane >> 4;
-    v4f const zero = { 0.f, 0.f, 0.f, 0.f };
+    uint4 B32[1][4];
+    uint2 B16[4];
 #pragma unroll
-    for (int t = 0; t < V::T2; ++t) {
-        v4f acc[3][4];
-#pragma unroll
-        for (int p = 0; p < 3; ++p) {
-            uint4 x[4];
-            uint2 xt[4];
-#pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                acc[p][b] = zero;
-                x[b] = make_uint4(Hin[b][0][0], Hin[b][0][1], Hin[b][1][0], Hin[b][1][1]);
-                xt[b] = make_uint2(Hin[b][2][0], Hin[b][2][1]);
-            }
-            if (p >= PLANES) continue;
-            mfma32_as_two_16(lds.w2[p][t][lane], x, acc[p]);
-            mfma16(reinterpret_cast<uint2 const*>(&lds.w2[p][t][64])[lane], xt, acc[p]);
-        }
-        v4f const bias = *reinterpret_cast<v4f const*>(&lds.bias[V::T0 + V::T1 + t][g][0]);
-#pragma unroll
-        for (int b = 0; b < 4; ++b) fp8_epilogue<true, PLANES == 3>(acc[2][b], acc[1][b], acc[0][b], bias, H[b][t]);
+    for (int b = 0; b < 4; ++b) {
+        B32[0][b] = make_uint4(Hin[b][0][0], Hin[b][0][1], Hin[b][1][0], Hin[b][1][1]);
+        B16[b] = make_uint2(Hin[b][2][0], Hin[b][2][1]);
     }
+    fp8_hidden_layer<PLANES, V::T2, 1, true, true>([&](int t, TileOperands<1, true>& o) {
+#pragma unroll
+        for (int p = 0; p < PLANES; ++p) {
+            o.a32[p][0] = lds.w2[p][t][lane];
+            o.a16[p] = reinterpret_cast<uint2 const*>(&lds.w2[p][t][64])[lane];
+        }
+        o.bias = *reinterpret_cast<v4f const*>(&lds.bias[V::T0 + V::T1 + t][g][0]);
+    }, B32, B16, H);
 }
 
 // The FP8 network for the 64 texels of one wave.  `in` is the lane's own texel; `topMask` (uniform) says which
