@@ -90,7 +90,9 @@ struct Fp8Variant {
     static constexpr int WEIGHT_BYTES = W3_OFF + H2 * OUT;
     // src/WeightLayout.cpp:249-262: fp16 biases of the three e4m3 layers, then scale and bias of the output layer
     static constexpr int BIAS_OFF = WEIGHT_BYTES, SCALE3_OFF = BIAS_OFF + 2 * (H0 + H1 + H2), BIAS3_OFF = SCALE3_OFF + 4 * OUT;
-    static constexpr int WAVES = 4, THREADS = 256;
+    // Twelve waves share one copy of the weight planes: one workgroup per CU, three waves per SIMD, working on
+    // GROUP tiles at a time.
+    static constexpr int WAVES = 12, THREADS = 64 * WAVES, GROUP = WAVES / 4;
     static constexpr int IN_STRIDE = 28;                     // dwords per texel in the transpose buffer: 24 + 4 of padding
 };
 
@@ -104,7 +106,7 @@ struct alignas(16) Fp8Lds {
     float bias[9][4][4];       // hidden layers: [output tile of layers 0..2][g][r] -> channel 16t+4g+r
     float outScale[4][4];      // output layer: [g][r]
     int32_t outBias[4][4];
-    uint32_t in[4][kWaveTexels][28];
+    uint32_t in[12][kWaveTexels][28];
     // Positional encoding for every power-of-two positionScale 2^-k, k = 0..5: the entry for phase p of scale
     // 2^-k sits at index (2^k - 1) + p; dwords 0..2 hold enc(px * 2^w), dwords 3..5 enc(px * 2^w + 1/4), w = 0..2,
     // as e4m3-rounded halves in the low 16 bits (px = p * 2^-k).
@@ -447,7 +449,9 @@ __device__ __forceinline__ void mfma32(uint4 const& a, uint4 const (&x)[4], v4f 
 // was not always there; compiling with padded matrix instructions made the same code correct), while chains of
 // one kind are reliable.  Layers whose input count is not a multiple of 32 therefore split their 32-deep blocks
 // with mfma32_as_two_16: a block's unit holds k-slots 8kg..8kg+7 of lane (i, kg) on both sides, so its first and
-// last four halves are two valid 16-deep operands.  The matrix pipeline takes the same time either way.
+// last four halves are two valid 16-deep operands.  (The other way round - the block of 16 padded with zero
+// weights to a 32-deep instruction, 148 instead of 196 matrix instructions per wave tile - measured 1.5 % slower:
+// two 16-deep instructions cost this kernel no more than one 32-deep one.)
 __device__ __forceinline__ void mfma16(uint2 const& a, uint2 const (&x)[4], v4f (&acc)[4])
 {
     v4h const A = __builtin_bit_cast(v4h, a);
@@ -464,12 +468,8 @@ __device__ __forceinline__ void mfma32_as_two_16(uint4 const& a, uint4 const (&x
 }
 
 // Hidden layers.  PLANES = 3, or 2 for a tame layer (see stage_fp8_weights).
-//
-// With two waves on a SIMD little else covers the LDS latency of a tile's weight operands, so a layer loads the
-// operands of output tile t + 1 before it works on tile t (two sets of registers, alternating), and a scheduling
-// barrier that only LDS reads may not cross keeps the compiler from moving those loads back down to their uses.
 template <int NK32, bool HAS16>
-struct TileOperands { uint4 a32[3][NK32]; uint2 a16[3]; v4f bias; };
+struct TileOperands { uint4 a32[3][NK32]; uint2 a16[3]; v4f bias; };     // one output tile's weight operands and bias
 
 // One hidden layer: TILES output tiles of 16 channels; its inputs as NK32 blocks of 32 (B32[kb][b]) and, with
 // HAS16, one block of 16 (B16[b]); load(t, operands) reads tile t's weight operands and bias.  A layer with a
@@ -478,15 +478,10 @@ template <int PLANES, int TILES, int NK32, bool HAS16, bool LAST_HIDDEN, class L
 __device__ __forceinline__ void fp8_hidden_layer(Load&& load, uint4 const (&B32)[NK32][4], uint2 const (&B16)[4], uint32_t (&H)[4][4][2])
 {
     v4f const zero = { 0.f, 0.f, 0.f, 0.f };
-    TileOperands<NK32, HAS16> ops[2];
-    load(0, ops[0]);
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
-        if (t + 1 < TILES) {
-            load(t + 1, ops[(t + 1) & 1]);
-            __builtin_amdgcn_sched_barrier(0x67f);           // everything but LDS instructions may cross
-        }
-        TileOperands<NK32, HAS16> const& o = ops[t & 1];
+        TileOperands<NK32, HAS16> o;
+        load(t, o);
         v4f acc[3][4];
 #pragma unroll
         for (int p = 0; p < 3; ++p) {
@@ -617,24 +612,49 @@ __device__ __forceinline__ void mlp_forward_fp8(Fp8Lds& lds, int wave, int lane,
 // whether any of it lies inside the image.  All uniform across the wave.
 struct WaveTile { int entry, x0, y0, work; };             // (four ints: a bool would leave padding bytes that copies carry through memory)
 
-__device__ __forceinline__ WaveTile locate_tile(DevMip const* __restrict__ mips, int numMips, int tile, int entry, int wave)
+// One round of a workgroup: tiles first .. first + count - 1 share one weight blob (count <= GROUP), member k of
+// the workgroup (waves 4k .. 4k+3) works on tile first + k.  All uniform across the workgroup except `mine`,
+// which is uniform across the wave.
+struct Round { int first, count, entry, lastEntry; WaveTile mine; };
+
+template <class V>
+__device__ __forceinline__ Round plan_round(DevMip const* __restrict__ mips, int numMips, int first, int entry, int tileEnd, int wave)
 {
-    while (entry + 1 < numMips && mips[entry + 1].tileStart <= tile) ++entry;
-    DevMip const& m = mips[entry];
-    int const local = tile - m.tileStart;
-    int const tileY = local / m.tilesX, tileX = local - tileY * m.tilesX;
-    WaveTile t;
-    t.entry = entry; t.x0 = tileX * 64 + wave * 16; t.y0 = tileY * 4;
-    t.work = t.x0 < m.width ? 1 : 0;
-    return t;
+    while (entry + 1 < numMips && mips[entry + 1].tileStart <= first) ++entry;
+    Round r;
+    r.first = first; r.count = 1; r.entry = entry; r.lastEntry = entry;
+    int const member = V::GROUP > 1 ? wave >> 2 : 0;
+    int mine = entry;
+    if constexpr (V::GROUP > 1) {
+        uint8_t const* const blob = mips[entry].weights;
+        int next = entry;
+        for (int k = 1; k < V::GROUP && first + k < tileEnd; ++k) {
+            while (next + 1 < numMips && mips[next + 1].tileStart <= first + k) ++next;
+            if (mips[next].weights != blob) break;
+            ++r.count;
+            r.lastEntry = next;
+            if (k == member) mine = next;
+        }
+    }
+    if (member < r.count) {
+        DevMip const& m = mips[mine];
+        int const local = first + member - m.tileStart;
+        int const tileY = local / m.tilesX, tileX = local - tileY * m.tilesX;
+        r.mine.entry = mine; r.mine.x0 = tileX * 64 + (wave & 3) * 16; r.mine.y0 = tileY * 4;
+        r.mine.work = r.mine.x0 < m.width ? 1 : 0;
+    } else {
+        r.mine.entry = entry; r.mine.x0 = 0; r.mine.y0 = 0; r.mine.work = 0;
+    }
+    return r;
 }
 
-// 77 KB of LDS: two workgroups per CU, two waves per SIMD, up to 256 registers per lane.  With so few waves
-// nothing else covers a tile's latent loads, so the loop is staggered: the loads of tile i+1 are issued before
-// tile i goes through the network and turned into tile i+1's input vector right after it, before tile i's
-// stores - at which point they have long arrived, and no store is ever waited for.
+// 135 KB of LDS - three planes of every hidden layer's weights, shared by the twelve waves of the one workgroup
+// a CU holds, and a transposition buffer per wave: three waves per SIMD, 168 registers per lane.  With so few
+// waves little else covers a tile's latent loads, so the loop is staggered: the loads of a wave's next tile are
+// issued before its current tile goes through the network and turned into the next input vector right after
+// it, before the current tile's stores - at which point they have long arrived, and no store is ever waited for.
 template <class V>
-__global__ void __launch_bounds__(V::THREADS, 2)
+__global__ void __launch_bounds__(V::THREADS, 1)
 decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
 {
     __shared__ Fp8Lds lds;
@@ -653,59 +673,40 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
 
     uint8_t const* stagedBlob = nullptr;
     int topMask = 7;                                         // uniform: hidden layers that need the general evaluation
-    uint32_t in[24];
-    Fp8Fetch<V> fetch;
 
-    // Input vector of the lane's texel of a wave tile; `fetched` says that fetch_latents_fast ran for it.
-    auto inputs_of = [&](WaveTile const& t, bool fetched) {
-        DevMip const& m = mips[t.entry];
-        int const x = min(t.x0 + j, m.width - 1), y = min(t.y0 + g, m.height - 1);
-        if (fetched) finish_inputs_fast<V>(m, lds, x, y, fetch, in);
-#ifdef NTC_EXP_NOPREFETCH
-        else if (m.fast) { fetch_latents_fast<V>(m, x, y, fetch); finish_inputs_fast<V>(m, lds, x, y, fetch, in); }
-#endif
-        else         prepare_inputs_fp8<V>(m, x, y, in);
-    };
-    auto fetch_of = [&](WaveTile const& t) -> bool {
-        DevMip const& m = mips[t.entry];
-        if (!t.work || !m.fast) return false;
-#ifdef NTC_EXP_NOPREFETCH
-        return false;
-#endif
-        fetch_latents_fast<V>(m, min(t.x0 + j, m.width - 1), min(t.y0 + g, m.height - 1), fetch);
-        return true;
-    };
-
-    WaveTile cur = locate_tile(mips, numMips, tileBegin, 0, wave);
-    {
-        bool const fetched = fetch_of(cur);
-        if (cur.work) inputs_of(cur, fetched);
-    }
-    for (int tile = tileBegin; tile < tileEnd; ++tile) {
-        DevMip const& m = mips[cur.entry];
-        if (m.weights != stagedBlob) {                       // uniform across the workgroup
+    int entry = 0;
+    for (int first = tileBegin; first < tileEnd; ) {         // every wave of the workgroup walks the same rounds
+        Round const round = plan_round<V>(mips, numMips, first, entry, tileEnd, wave);
+        first += round.count;
+        entry = round.lastEntry;
+        uint8_t const* const blob = mips[round.entry].weights;
+        if (blob != stagedBlob) {                            // uniform across the workgroup
             __syncthreads();
-            topMask = stage_fp8_weights<V>(lds, m.weights);
-            stagedBlob = m.weights;
+            topMask = stage_fp8_weights<V>(lds, blob);
+            stagedBlob = blob;
             __syncthreads();
         }
-        bool const more = tile + 1 < tileEnd;
-        WaveTile next = cur;
-        bool fetched = false;
-        if (more) {
-            next = locate_tile(mips, numMips, tile + 1, cur.entry, wave);
-            fetched = fetch_of(next);
+        WaveTile const& t = round.mine;
+        if (!t.work) continue;
+        DevMip const& m = mips[t.entry];
+
+        uint32_t in[24];
+        {
+            int const x = min(t.x0 + j, m.width - 1), y = min(t.y0 + g, m.height - 1);
+            if (m.fast) {
+                Fp8Fetch<V> fetch;
+                fetch_latents_fast<V>(m, x, y, fetch);
+                finish_inputs_fast<V>(m, lds, x, y, fetch, in);
+            } else {
+                prepare_inputs_fp8<V>(m, x, y, in);
+            }
         }
         v4i D[4];
         v4f S;
-        if (cur.work) mlp_forward_fp8<V>(lds, wave, lane, topMask, in, D, S);
-        if (more && next.work) inputs_of(next, fetched);
-        if (cur.work) {
-            if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)      store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, cur.x0 + j, cur.y0, 4 * g);
-            else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)       store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, cur.x0 + j, cur.y0, 4 * g);
-            else                                                       store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, cur.x0 + j, cur.y0, 4 * g);
-        }
-        cur = next;
+        mlp_forward_fp8<V>(lds, wave, lane, topMask, in, D, S);
+        if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)      store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, t.x0 + j, t.y0, 4 * g);
+        else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)       store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, t.x0 + j, t.y0, 4 * g);
+        else                                                       store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, t.x0 + j, t.y0, 4 * g);
     }
 }
 
@@ -747,9 +748,11 @@ hipError_t launch_decode_fp8(int variant, DevMip const* mips, int numMips, int t
 int resident_fp8_workgroups_per_cu()
 {
     int blocks = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, decode_fp8_kernel<VFp8_16>, VFp8_16::THREADS, 0) != hipSuccess || blocks < 1) blocks = 2;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, decode_fp8_kernel<VFp8_16>, VFp8_16::THREADS, 0) != hipSuccess || blocks < 1) blocks = 1;
     return blocks;
 }
+
+int fp8_tiles_per_round() { return VFp8_16::GROUP; }
 
 hipError_t launch_selftest_fp8_activation(uint16_t const* in, uint16_t* out, int n, hipStream_t stream)
 {

@@ -949,8 +949,8 @@ __device__ __forceinline__ void f16_tile(LdsT<V> const& lds, int base, int t, in
         // An odd number of input tiles: every tile takes the 16-deep instruction (a pair's block holds tile 2p in
         // its first four halves per lane and tile 2p+1 in the last four).  32-deep and 16-deep instructions are
         // never mixed in one accumulator's chain: in either order that gave wrong sums with some instruction
-        // schedules (the wait between the two was not always there), while chains of one kind are reliable; the
-        // matrix pipeline takes the same time either way.
+        // schedules (the wait between the two was not always there), while chains of one kind are reliable; two
+        // 16-deep instructions cost no more than one 32-deep one.
 #pragma unroll
         for (int ti = 0; ti < IN_TILES; ++ti) {
             uint2 a;

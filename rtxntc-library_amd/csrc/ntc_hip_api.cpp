@@ -414,7 +414,8 @@ int grid_size_for(Library const& L, int variant, int totalTiles)
     }
     int const resident = L.computeUnits * perCu[variant];
     // a workgroup takes tiles_per_round(variant) tiles at a time: fewer workgroups than that leaves waves idle
-    int64_t const rounds = (int64_t(totalTiles) + tiles_per_round(variant) - 1) / tiles_per_round(variant);
+    int const group = variant_is_fp8_network(variant) ? fp8_tiles_per_round() : tiles_per_round(variant);
+    int64_t const rounds = (int64_t(totalTiles) + group - 1) / group;
     return rounds < resident ? int(rounds) : resident;
 }
 

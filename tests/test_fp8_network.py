@@ -287,6 +287,24 @@ def test_gpu_fp8_batch_mixes_sets_with_and_without_top_planes(ntc, device):
 
 
 @pytest.mark.gpu
+def test_gpu_fp8_batch_with_set_boundaries_inside_the_rounds_of_a_workgroup(ntc, device):
+    """More tiles than resident workgroups take three at a time: every workgroup walks a share of several tiles in
+    rounds of up to three that stop at the next set (other weights), so sets begin in the middle of a share, at
+    every position of a round.  Sizes chosen so that the sets' tile counts are not multiples of three."""
+    sizes = [(256, 256), (320, 192), (256, 128), (192, 320), (256, 256), (64, 448)]
+    cases = [fp8_case(ntc, 16, w, h, ntc.presets.full_mip_count(w, h), 2, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=300 + i,
+                      weight_sigma=(0.35 if i % 2 else (0.35, 40.0, 0.35))) for i, (w, h) in enumerate(sizes)]
+    hosts = [c.host_set() for c in cases]
+    for hset in hosts:
+        hset.decode(threads=8)
+    device.decode([c.device_set(device) for c in cases])
+    device.synchronize()
+    for i, (c, hset) in enumerate(zip(cases, hosts)):
+        mm = first_mismatch(hset.output, c.d_output.download())
+        assert mm is None, (i, mm)
+
+
+@pytest.mark.gpu
 def test_gpu_fp8_batch_of_sets_and_static_table(ntc, device):
     cases = [fp8_case(ntc, 8, 64, 64, 7, 2, 8, ntc.abi.OUT_UNORM8_PIXELS, seed=80 + i) for i in range(3)]
     hosts = [c.host_set() for c in cases]
