@@ -159,7 +159,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=30)   # the GPU clock takes ~30 launches to settle
-    ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4", "ref092", "ref092fp8", "read", "write", "loss", "bc1", "bc3", "bc5", "bc6", "bc7", "bc7m"])
+    ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg2", "cfg3", "cfg4", "cfg4fp8", "ref092", "ref092fp8", "read", "write", "loss", "bc1", "bc3", "bc5", "bc6", "bc7", "bc7m"])
     ap.add_argument("--size", type=int, default=0, help="override the texture size of the workload")
     ap.add_argument("--settle-ms", type=float, default=60.0,
                     help="untimed decode steps for this long before the warm-up, so that clocks have ramped (0 = none)")
@@ -222,8 +222,15 @@ def main():
                 "MLP 48(46)-64-48-32-16, e4m3 hidden layers (GenericFP8 blob)")
     else:
         size = args.size or 8192
-        cases = [cfg_case(ntc, P.spec_cfg01(), size, size, P.full_mip_count(size, size), 16, fmt, seed=4)]
-        widths, channels, latent_b = (64, 64, 48, 32, 16), 16, 0.0
+        if wl == "cfg4fp8":
+            from cases import Case
+            spec = P.spec_ref092_fp8(16)
+            mips, latent_bytes = P.mips_ref092(spec, size, size, P.full_mip_count(size, size), 2)
+            cases = [Case(ntc, spec, mips, latent_bytes, 16, fmt, seed=4, weights=ntc.synth.make_fp8_weights(spec, 6))]
+            widths, channels, latent_b = (46, 64, 48, 32, 16), 16, 0.0
+        else:
+            cases = [cfg_case(ntc, P.spec_cfg01(), size, size, P.full_mip_count(size, size), 16, fmt, seed=4)]
+            widths, channels, latent_b = (64, 64, 48, 32, 16), 16, 0.0
         import numpy as np
         n = 1 << 24
         rng = np.random.default_rng(4)
@@ -231,6 +238,8 @@ def main():
         queries["u"], queries["v"] = rng.random(n, dtype=np.float32), rng.random(n, dtype=np.float32)
         queries["mip"] = rng.integers(0, len(cases[0].mips), n)
         what = f"cfg4 random access: {size}x{size} set, {len(cases[0].mips)} mips, 2^24 (u,v,mip) queries, 16 x fp16 per query"
+        if wl == "cfg4fp8":
+            what = "FP8 network of the LibNTC 0.9.2 geometry (grid scale 2, 16 features in both grids), " + what
         fmt_name = "fp16"
 
     dsets = [c.device_set(dev) for c in cases]
@@ -243,7 +252,7 @@ def main():
         run_timed = lambda k: dev.decode_timed(sets, k)
     else:
         texels = queries.size
-        bytes_per_texel = 32 + 12 + 40                # output + the query + 4 HR cells x 2 B + 4 LR cells x 8 B
+        bytes_per_texel = 32 + 12 + (64 if wl == "cfg4fp8" else 40)   # output + the query + 4 HR cells (2 B; 8 B in the 0.9.2 geometry) + 4 LR cells x 8 B
         d_q = dev.upload(queries.view("u1"))
         d_out = dev.alloc(queries.size * 32)
         if not args.file_order_latents:

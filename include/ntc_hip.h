@@ -72,8 +72,9 @@ typedef enum NtcHipWeightType {
      * version of the network that ITextureSet::Decompress uses unless asked for Int8 weights
      * (src/TextureSet.cpp:1812,1826), evaluated as include/libntc/shaders/InferenceCoopVec.hlsli:22-124,
      * 127-160,235-398 describes: e4m3-rounded fp16 inputs and activations, exact dot products, fp16 bias
-     * and HGELU-clamp activation, int8 output layer.  Decoded by ntc_hip_decode for the LibNTC 0.9.2
-     * geometry (both grids bilinear 4-bit with 4 / 8 / 12 / 16 features, MLP 48-64-48-32-16). */
+     * and HGELU-clamp activation, int8 output layer.  Decoded by ntc_hip_decode and
+     * ntc_hip_decode_queries for the LibNTC 0.9.2 geometry (both grids bilinear 4-bit with 4 / 8 / 12 / 16
+     * features, MLP 48-64-48-32-16). */
     NTC_HIP_WEIGHTS_FP8  = 1,
     /* Laid out exactly like NTC_HIP_WEIGHTS_INT8, but the bytes of the three hidden-layer matrices
      * are OCP e4m3 values w.  A hidden layer computes acc = bias_i32 + sum(512*w * in) exactly in

@@ -221,4 +221,60 @@ __device__ __forceinline__ void store_tile(DevMip const& m, Acc const (&D)[4], v
     }
 }
 
+// ---- random-access decode: pieces shared by the query kernels ----------------------------------
+
+// Two adjacent u16 cells as one 32-bit load (2-byte aligned).
+typedef uint32_t __attribute__((aligned(2))) u32_align2;
+typedef __attribute__((address_space(1))) u32_align2 const* GlobalU32A2Ptr;
+
+// The query-ordered copy of a grid: bricks of T x T cells (T = 4, or 8 for a one-layer grid),
+// [brick row][brick column][cell row][cell column][layer], so that all layers of a cell are one load of 2, 4,
+// 6 or 8 bytes and a 2 x 2 footprint usually lies in one or two cache lines.
+typedef __attribute__((address_space(1))) u32x2 const* GlobalU32x2Ptr;
+
+template <int LAYERS>
+__device__ __forceinline__ uint32_t brick_offset(uint32_t cx, uint32_t cy, uint32_t log2GridWidth)
+{
+    constexpr uint32_t T = brick_side_log2(LAYERS), MASK = (1u << T) - 1u;
+    uint32_t const lgBricksX = log2GridWidth > T ? log2GridWidth - T : 0u;
+    uint32_t const brick = ((cy >> T) << lgBricksX) + (cx >> T);
+    uint32_t const cell = ((cy & MASK) << T) + (cx & MASK);
+    return brick * uint32_t(brick_bytes(LAYERS)) + cell * uint32_t(2 * LAYERS);     // below 2^32: a grid holds less than 2^31 bytes
+}
+
+// All layers of one cell: layer L in the low or high half of out[L / 2].
+template <int LAYERS>
+__device__ __forceinline__ void load_brick_cell(GlobalU8Ptr base, uint32_t off, uint32_t (&out)[2])
+{
+    out[0] = 0; out[1] = 0;
+    if constexpr (LAYERS == 1) {
+        out[0] = load_u16(base, off);
+    } else if constexpr (LAYERS == 2) {
+        out[0] = *reinterpret_cast<GlobalU32A2Ptr>(base + off);
+    } else if constexpr (LAYERS == 3) {
+        out[0] = *reinterpret_cast<GlobalU32A2Ptr>(base + off);
+        out[1] = load_u16(base, off + 4u);
+    } else {
+        u32x2 const v = *reinterpret_cast<GlobalU32x2Ptr>(base + off);
+        out[0] = v[0]; out[1] = v[1];
+    }
+}
+
+// What a query needs of its mip, kept in LDS: every lane of a wave may address another mip, and
+// fetching these fields per lane from the table in global memory put a long dependent load in
+// front of the latent gathers.
+struct QueryMip {
+    uint16_t const* hr;
+    uint16_t const* lr;
+    uint32_t hrAxisX, hrAxisY, lrAxisX, lrAxisY;
+    int32_t hrWidth, hrHeight, lrWidth, lrHeight;
+    int32_t width, height;
+    uint32_t posMask, fast;
+    float positionLod;
+    uint32_t pad[3];
+    uint8_t const* hrBricks;
+    uint8_t const* lrBricks;
+};
+static_assert(sizeof(QueryMip) == 96, "QueryMip layout");
+
 } // namespace ntc_hip_dev

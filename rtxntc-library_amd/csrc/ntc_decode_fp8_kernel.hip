@@ -299,8 +299,8 @@ struct Fp8Fetch {
     uint32_t fx[2], fy[2];                                   // axis fractions of the footprint, per grid
 };
 
-template <class V>
-__device__ __forceinline__ void fetch_latents_fast(DevMip const& m, int x, int y, Fp8Fetch<V>& f)
+template <class V, class Mip>
+__device__ __forceinline__ void fetch_latents_fast(Mip const& m, int x, int y, Fp8Fetch<V>& f)
 {
 #pragma unroll
     for (int grid = 0; grid < 2; ++grid) {
@@ -322,8 +322,35 @@ __device__ __forceinline__ void fetch_latents_fast(DevMip const& m, int x, int y
     }
 }
 
-template <class V>
-__device__ __forceinline__ void finish_inputs_fast(DevMip const& m, Fp8Lds const& lds, int x, int y, Fp8Fetch<V> const& f, uint32_t (&in)[24])
+// The same cells from the query-ordered copy of the grids (bricks with all layers of a cell together): four
+// loads per grid instead of four per layer.
+template <class V, class Mip>
+__device__ __forceinline__ void fetch_latents_bricked(Mip const& m, int x, int y, Fp8Fetch<V>& f)
+{
+    constexpr int LAYERS = Fp8Fetch<V>::LAYERS;
+#pragma unroll
+    for (int grid = 0; grid < 2; ++grid) {
+        uint32_t const axisX = grid == 0 ? m.hrAxisX : m.lrAxisX, axisY = grid == 0 ? m.hrAxisY : m.lrAxisY;
+        int const gw = grid == 0 ? m.hrWidth : m.lrWidth, gh = grid == 0 ? m.hrHeight : m.lrHeight;
+        AxisFoot const ax = axis_fast(x, axisX, gw), ay = axis_fast(y, axisY, gh);
+        GlobalU8Ptr const g = (GlobalU8Ptr)(grid == 0 ? m.hrBricks : m.lrBricks);
+        uint32_t const lg = (axisX >> 24) & 0xffu;                // log2(grid width)
+        f.fx[grid] = ax.f; f.fy[grid] = ay.f;
+        uint32_t cell[4][2];                                      // taps 00, 10, 01, 11
+        load_brick_cell<LAYERS>(g, brick_offset<LAYERS>(ax.c0, ay.c0, lg), cell[0]);
+        load_brick_cell<LAYERS>(g, brick_offset<LAYERS>(ax.c1, ay.c0, lg), cell[1]);
+        load_brick_cell<LAYERS>(g, brick_offset<LAYERS>(ax.c0, ay.c1, lg), cell[2]);
+        load_brick_cell<LAYERS>(g, brick_offset<LAYERS>(ax.c1, ay.c1, lg), cell[3]);
+#pragma unroll
+        for (int L = 0; L < LAYERS; ++L)
+#pragma unroll
+            for (int tap = 0; tap < 4; ++tap)
+                f.cell[grid][L][tap] = (L & 1) ? cell[tap][L >> 1] >> 16 : cell[tap][L >> 1] & 0xffffu;
+    }
+}
+
+template <class V, class Mip>
+__device__ __forceinline__ void finish_inputs_fast(Mip const& m, Fp8Lds const& lds, int x, int y, Fp8Fetch<V> const& f, uint32_t (&in)[24])
 {
 #pragma unroll
     for (int i = 0; i < 24; ++i) in[i] = 0;
@@ -334,7 +361,7 @@ __device__ __forceinline__ void finish_inputs_fast(DevMip const& m, Fp8Lds const
         uint32_t const wx1 = f.fx[grid], wx0 = (1u << nx) - wx1, wy1 = f.fy[grid], wy0 = (1u << ny) - wy1;
         uint32_t const msk = 0x000f000fu, sel = 0x0c010c00u;     // v_perm_b32: bytes [0, zero, 1, zero] of the cell
         uint32_t const n = nx + ny;
-        if (V::F % 4 == 0 && n <= 6u && !(n & 1u)) {             // uniform
+        if (V::F % 4 == 0 && n <= 6u && !(n & 1u)) {             // (uniform in the raster kernel, per lane for queries)
             // Table form: with doubled weights and start values 2*base resp. 17 * 2*base the 16-bit lanes of T and
             // O come out as byte offsets into the table (S stays below 2^16: 2 * 255 * 64 + 34 * 318).
             uint32_t const w00 = mul24(2u * wx0, wy0), w10 = mul24(2u * wx1, wy0), w01 = mul24(2u * wx0, wy1), w11 = mul24(2u * wx1, wy1);
@@ -710,6 +737,75 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     }
 }
 
+// Random-access decode with the FP8 network (NtcSampleTextureSet_CoopVec_FP8, InferenceCoopVec.hlsli:400-440,
+// for a list of sample points): query_kernel of ntc_decode_kernel.hip with this file's input stage and network.  Lane = query in the input stage (each lane with its own mip, kept in LDS); one set, hence one
+// weight blob, per launch.  A query whose mip is out of range writes zeros.
+template <class V>
+__global__ void __launch_bounds__(V::THREADS, 1)
+query_fp8_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __restrict__ queries, uint64_t numQueries,
+                 uint16_t* __restrict__ out)
+{
+    __shared__ Fp8Lds lds;
+    __shared__ QueryMip qmips[16];
+    if (threadIdx.x < 16) {
+        DevMip const& d = mips[min(int(threadIdx.x), numMips - 1)];
+        QueryMip& q = qmips[threadIdx.x];
+        q.hr = d.hr; q.lr = d.lr;
+        q.hrAxisX = d.hrAxisX; q.hrAxisY = d.hrAxisY; q.lrAxisX = d.lrAxisX; q.lrAxisY = d.lrAxisY;
+        q.hrWidth = d.hrWidth; q.hrHeight = d.hrHeight; q.lrWidth = d.lrWidth; q.lrHeight = d.lrHeight;
+        q.width = d.width; q.height = d.height;
+        q.posMask = d.posMask; q.fast = d.fast; q.positionLod = d.positionLod;
+        q.hrBricks = d.hrBricks; q.lrBricks = d.lrBricks;
+    }
+    bool const bricked = mips[0].hrBricks != nullptr;          // a set has the query-ordered copy for all of its mips or for none
+    int const lane = threadIdx.x & 63;
+    int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int const j = lane & 15, g = lane >> 4;
+
+    build_fp8_posenc_table(lds);
+    build_fp8_feature_lut(lds);
+    int const topMask = stage_fp8_weights<V>(lds, mips[0].weights);
+    __syncthreads();
+
+    uint64_t const numBlocks = (numQueries + V::THREADS - 1) / V::THREADS;
+    for (uint64_t block = blockIdx.x; block < numBlocks; block += gridDim.x) {
+        uint64_t const q0 = block * V::THREADS + uint64_t(wave) * 64;
+        if (q0 >= numQueries) continue;
+        uint64_t const qi = min(q0 + uint64_t(lane), numQueries - 1);
+        DevQuery const query = queries[qi];
+        bool const validMip = query.mip >= 0 && query.mip < numMips;
+        QueryMip const& m = qmips[validMip ? query.mip : 0];
+        int x = int(floorf(query.u * float(m.width)));
+        int y = int(floorf(query.v * float(m.height)));
+        x = max(0, min(x, m.width - 1));
+        y = max(0, min(y, m.height - 1));
+        uint32_t in[24];
+        if (__all(m.fast != 0)) {                                // every lane's mip is power-of-two sized
+            Fp8Fetch<V> fetch;
+            if (bricked) fetch_latents_bricked<V>(m, x, y, fetch);
+            else         fetch_latents_fast<V>(m, x, y, fetch);
+            finish_inputs_fast<V>(m, lds, x, y, fetch, in);
+        } else {
+            prepare_inputs_fp8<V>(mips[validMip ? query.mip : 0], x, y, in);
+        }
+        v4i D[4];
+        v4f S;
+        mlp_forward_fp8<V>(lds, wave, lane, topMask, in, D, S);
+
+        // lane (j, g) holds channels 4g..4g+3 of query q0 + 16b + j; validity travels by shuffle
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            uint64_t const q = q0 + uint64_t(16 * b + j);
+            int const ok = __shfl(validMip ? 1 : 0, 16 * b + j, 64);
+            if (q >= numQueries) continue;
+            uint32_t h01 = to_half2_bits(float(D[b][0]) * S[0], float(D[b][1]) * S[1]);
+            uint32_t h23 = to_half2_bits(float(D[b][2]) * S[2], float(D[b][3]) * S[3]);
+            if (!ok) { h01 = 0; h23 = 0; }
+            *reinterpret_cast<u32x2*>(out + q * 16 + 4 * g) = u32x2{ h01, h23 };
+        }
+    }
+}
+
 // The two fp16 primitives of the activation stage applied to a list of halves (for the tests): out[0..n) the
 // HGELU-clamp result, out[n..2n) the input rounded to e4m3, out[2n..3n) the int8 quantisation of the input.
 __global__ void selftest_fp8_activation_kernel(uint16_t const* __restrict__ in, uint16_t* __restrict__ out, int n)
@@ -744,6 +840,27 @@ hipError_t launch_decode_fp8(int variant, DevMip const* mips, int numMips, int t
     default: return hipErrorInvalidValue;
     }
 }
+
+template <class V>
+static hipError_t launch_fp8_query_variant(DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries, uint16_t* out, int gridSize, hipStream_t stream)
+{
+    hipLaunchKernelGGL(query_fp8_kernel<V>, dim3(gridSize), dim3(V::THREADS), 0, stream, mips, numMips, queries, numQueries, out);
+    return hipGetLastError();
+}
+
+hipError_t launch_queries_fp8(int variant, DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries,
+                              uint16_t* out, int gridSize, hipStream_t stream)
+{
+    switch (variant) {
+    case NTC_HIP_VARIANT_REF16_FP8: return launch_fp8_query_variant<VFp8_16>(mips, numMips, queries, numQueries, out, gridSize, stream);
+    case NTC_HIP_VARIANT_REF12_FP8: return launch_fp8_query_variant<VFp8_12>(mips, numMips, queries, numQueries, out, gridSize, stream);
+    case NTC_HIP_VARIANT_REF8_FP8:  return launch_fp8_query_variant<VFp8_8>(mips, numMips, queries, numQueries, out, gridSize, stream);
+    case NTC_HIP_VARIANT_REF4_FP8:  return launch_fp8_query_variant<VFp8_4>(mips, numMips, queries, numQueries, out, gridSize, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+int fp8_threads_per_workgroup() { return VFp8_16::THREADS; }
 
 int resident_fp8_workgroups_per_cu()
 {

@@ -155,6 +155,9 @@ hipError_t launch_queries(int variant, DevMip const* mips, int numMips, DevQuery
 hipError_t launch_decode_fp8(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream);
 int resident_fp8_workgroups_per_cu();
 int fp8_tiles_per_round();               // tiles a workgroup of decode_fp8_kernel works on at a time
+int fp8_threads_per_workgroup();
+hipError_t launch_queries_fp8(int variant, DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries,
+                              uint16_t* out, int gridSize, hipStream_t stream);
 hipError_t launch_selftest_fp8_activation(uint16_t const* in, uint16_t* out, int n, hipStream_t stream);
 int resident_workgroups_per_cu(int variant);
 int tiles_per_round(int variant);      // tiles a workgroup of the variant's decode kernel works on at a time

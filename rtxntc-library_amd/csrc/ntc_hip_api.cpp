@@ -690,15 +690,16 @@ static int run_queries(NtcHipContext* ctx, const NtcHipTextureSet* set, const Nt
     std::vector<DevMip> table;
     int variant = NTC_HIP_VARIANT_NONE, totalTiles = 0;
     if (int r = build_table(set, 1, table, variant, totalTiles, true)) return r;
-    if (variant_is_fp8_network(variant)) { set_error("ntc_hip_decode_queries: the FP8 network is available to ntc_hip_decode only."); return NTC_HIP_ERR_UNSUPPORTED; }
+    bool const fp8 = variant_is_fp8_network(variant);
     if (int r = upload_table(L, table)) return r;
-    uint64_t const blocks = (numQueries + 255) / 256;
+    uint64_t const perBlock = fp8 ? uint64_t(fp8_threads_per_workgroup()) : 256u;
+    uint64_t const blocks = (numQueries + perBlock - 1) / perBlock;
     uint64_t const resident = uint64_t(L.computeUnits) * uint64_t(grid_size_for(L, variant, 0x7fffffff) / L.computeUnits);
     int const grid = int(blocks < resident ? blocks : resident);
     if (outMs) HIP_TRY(hipEventRecord(L.evStart, L.stream));
     for (int i = 0; i < iterations; ++i)
-        HIP_TRY(launch_queries(variant, L.tableDev, int(table.size()), reinterpret_cast<DevQuery const*>(queries), numQueries,
-                               static_cast<uint16_t*>(out), grid, L.stream));
+        HIP_TRY((fp8 ? launch_queries_fp8 : launch_queries)(variant, L.tableDev, int(table.size()), reinterpret_cast<DevQuery const*>(queries), numQueries,
+                                                           static_cast<uint16_t*>(out), grid, L.stream));
     if (outMs) {
         HIP_TRY(hipEventRecord(L.evStop, L.stream));
         HIP_TRY(hipEventSynchronize(L.evStop));

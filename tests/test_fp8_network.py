@@ -323,7 +323,7 @@ def test_gpu_fp8_batch_of_sets_and_static_table(ntc, device):
 
 
 @pytest.mark.gpu
-def test_gpu_fp8_network_is_not_offered_for_other_geometries_or_queries(ntc, device):
+def test_gpu_fp8_network_is_not_offered_for_other_geometries(ntc, device):
     spec = ntc.presets.spec_cfg01()
     spec.weightType = ntc.abi.WEIGHTS_FP8
     case = Case(ntc, spec, *ntc.presets.mips_private_grids(spec, 64, 64, 1), 8, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=1,
@@ -331,9 +331,75 @@ def test_gpu_fp8_network_is_not_offered_for_other_geometries_or_queries(ntc, dev
     with pytest.raises(ntc.NtcHipError) as e:
         device.decode([case.device_set(device)])
     assert e.value.code == ntc.abi.ERR_UNSUPPORTED
-    good = fp8_case(ntc, 16, 64, 64, 1, 2, 8, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=2)
-    dset = good.device_set(device)
     q = device.upload(np.zeros(3 * 4, dtype=np.float32))
     out = device.alloc(4 * 32)
-    rc = device.lib.ntc_hip_decode_queries(dset, q.ptr, 4, out.ptr, out.nbytes)
-    assert rc == ntc.abi.ERR_UNSUPPORTED
+    assert device.lib.ntc_hip_decode_queries(case.device_set(device), q.ptr, 4, out.ptr, out.nbytes) == ntc.abi.ERR_UNSUPPORTED
+
+
+def fp8_queries(rng, n, num_mips):
+    q = np.zeros(n, dtype=[("u", np.float32), ("v", np.float32), ("mip", np.int32)])
+    q["u"] = rng.random(n, dtype=np.float32)
+    q["v"] = rng.random(n, dtype=np.float32)
+    q["mip"] = rng.integers(0, num_mips, n)
+    if n >= 12:
+        q["u"][:6] = [0.0, np.nextafter(np.float32(1), np.float32(0)), 1.0, 1.5, -0.25, 0.5]
+        q["v"][:6] = [0.0, np.nextafter(np.float32(1), np.float32(0)), 2.0, -3.0, 0.999, 0.5]
+        q["mip"][6:9] = [-1, num_mips, 99]                 # outside the set: zeros
+        q["mip"][9:12] = [num_mips - 1, 0, 0]
+    return q
+
+
+def test_checker_fp8_queries_are_its_raster_decode_at_the_texels_hit(ntc, oracle):
+    case = fp8_case(ntc, 16, 48, 40, 6, 2, 16, ntc.abi.OUT_FP16_PIXELS, seed=77)
+    host = case.host_set()
+    host.decode(threads=8)
+    n = 400
+    q = fp8_queries(np.random.default_rng(5), n, len(case.mips))
+    got = np.zeros((n, 16), dtype=np.uint16)
+    assert oracle.ntc_oracle_decode_queries(host.desc, q.ctypes.data, n, got.ctypes.data, 4) == 0
+    raster = host.output.view(np.uint16)
+    for i in range(n):
+        m = int(q["mip"][i])
+        if m < 0 or m >= len(case.mips):
+            assert not got[i].any()
+            continue
+        d = case.mips[m]
+        x = int(np.clip(np.floor(np.float32(q["u"][i]) * np.float32(d.width)), 0, d.width - 1))
+        y = int(np.clip(np.floor(np.float32(q["v"][i]) * np.float32(d.height)), 0, d.height - 1))
+        start = (d.outOffset + y * d.outRowPitch + x * case.pixel_stride) // 2
+        assert np.array_equal(got[i], raster[start:start + 16]), (i, m, x, y)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("features,size,grid_scale,n,sigma", [(16, 512, 2, 6000, 0.35), (12, 256, 4, 3001, 0.35), (8, 512, 1, 777, 0.35), (4, 256, 2, 1, 0.35),
+                                                         (16, 320, 3, 4000, 0.35), (8, 200, 2, 2049, 0.35), (16, 256, 2, 5000, (0.35, 40.0, 300.0))])
+def test_gpu_fp8_queries_match_checker(ntc, device, oracle, features, size, grid_scale, n, sigma):
+    """Random-access decode with the FP8 network: sample points over every mip of a set (edges, mips outside the
+    set), from the file-ordered grids and from the query-ordered copy, against the checker's decode of the texels
+    they hit.  Sizes that are not powers of two take the float input stage; one case has layers with large weights
+    (three weight planes)."""
+    A = ntc.abi
+    case = fp8_case(ntc, features, size, size, ntc.presets.full_mip_count(size, size), grid_scale, 16, A.OUT_FP16_PLANAR_PAIRS,
+                    seed=400 + features + n, weight_sigma=sigma)
+    host = case.host_set()
+    q = fp8_queries(np.random.default_rng(n + features), n, len(case.mips))
+    want = np.zeros((n, 16), dtype=np.uint16)
+    assert oracle.ntc_oracle_decode_queries(host.desc, q.ctypes.data, n, want.ctypes.data, 8) == 0
+    assert len(np.unique(want)) > min(n, 300)
+    dset = case.device_set(device)
+    d_q = device.upload(q.view(np.uint8))
+    d_out = device.alloc(n * 32)
+    need = device.lib.ntc_hip_query_latents_bytes(dset)
+    d_bricks = device.alloc(need)
+    A.check(device.lib.ntc_hip_build_query_latents(dset, d_bricks.ptr, d_bricks.nbytes))
+    for use_bricks in (False, True):
+        dset.queryLatents, dset.queryLatentsBytes = (d_bricks.ptr, d_bricks.nbytes) if use_bricks else (None, 0)
+        d_out.fill(0xCD)
+        A.check(device.lib.ntc_hip_decode_queries(dset, d_q.ptr, n, d_out.ptr, d_out.nbytes))
+        device.synchronize()
+        got = d_out.download(np.uint16).reshape(n, 16)
+        bad = np.nonzero((got != want).any(axis=1))[0]
+        assert bad.size == 0, f"bricks={use_bricks}: {bad.size} of {n} queries differ, first {bad[0]}: {q[bad[0]]} gpu {got[bad[0]]} checker {want[bad[0]]}"
+    ms = C.c_float()
+    A.check(device.lib.ntc_hip_decode_queries_timed(dset, d_q.ptr, n, d_out.ptr, d_out.nbytes, 2, C.byref(ms)))
+    assert ms.value > 0 and np.array_equal(d_out.download(np.uint16).reshape(n, 16), want)
