@@ -635,51 +635,14 @@ __device__ __forceinline__ void mlp_forward_fp8(Fp8Lds& lds, int wave, int lane,
     }
 }
 
-// Where a wave stands in the image for one workgroup tile: the mip's table entry, the wave tile's corner and
-// whether any of it lies inside the image.  All uniform across the wave.
-struct WaveTile { int entry, x0, y0, work; };             // (four ints: a bool would leave padding bytes that copies carry through memory)
-
-// One round of a workgroup: tiles first .. first + count - 1 share one weight blob (count <= GROUP), member k of
-// the workgroup (waves 4k .. 4k+3) works on tile first + k.  All uniform across the workgroup except `mine`,
-// which is uniform across the wave.
-struct Round { int first, count, entry, lastEntry; WaveTile mine; };
-
-template <class V>
-__device__ __forceinline__ Round plan_round(DevMip const* __restrict__ mips, int numMips, int first, int entry, int tileEnd, int wave)
-{
-    while (entry + 1 < numMips && mips[entry + 1].tileStart <= first) ++entry;
-    Round r;
-    r.first = first; r.count = 1; r.entry = entry; r.lastEntry = entry;
-    int const member = V::GROUP > 1 ? wave >> 2 : 0;
-    int mine = entry;
-    if constexpr (V::GROUP > 1) {
-        uint8_t const* const blob = mips[entry].weights;
-        int next = entry;
-        for (int k = 1; k < V::GROUP && first + k < tileEnd; ++k) {
-            while (next + 1 < numMips && mips[next + 1].tileStart <= first + k) ++next;
-            if (mips[next].weights != blob) break;
-            ++r.count;
-            r.lastEntry = next;
-            if (k == member) mine = next;
-        }
-    }
-    if (member < r.count) {
-        DevMip const& m = mips[mine];
-        int const local = first + member - m.tileStart;
-        int const tileY = local / m.tilesX, tileX = local - tileY * m.tilesX;
-        r.mine.entry = mine; r.mine.x0 = tileX * 64 + (wave & 3) * 16; r.mine.y0 = tileY * 4;
-        r.mine.work = r.mine.x0 < m.width ? 1 : 0;
-    } else {
-        r.mine.entry = entry; r.mine.x0 = 0; r.mine.y0 = 0; r.mine.work = 0;
-    }
-    return r;
-}
-
 // 135 KB of LDS - three planes of every hidden layer's weights, shared by the twelve waves of the one workgroup
-// a CU holds, and a transposition buffer per wave: three waves per SIMD, 168 registers per lane.  With so few
-// waves little else covers a tile's latent loads, so the loop is staggered: the loads of a wave's next tile are
-// issued before its current tile goes through the network and turned into the next input vector right after
-// it, before the current tile's stores - at which point they have long arrived, and no store is ever waited for.
+// a CU holds, and a transposition buffer per wave: three waves per SIMD, 168 registers per lane.
+//
+// A workgroup owns a contiguous share of the tile list.  It walks that share in segments of tiles that use the
+// same weight blob (one segment, unless sets of a batch meet inside the share), and inside a segment each of its
+// GROUP wave quartets walks a contiguous part, so that a quartet's consecutive tiles are neighbours in the image
+// and find the cache lines they share with the previous tile still in place.  (Quartets taking every third tile
+// of a common sequence drift apart in time, and the latent reads from memory doubled.)
 template <class V>
 __global__ void __launch_bounds__(V::THREADS, 1)
 decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
@@ -687,6 +650,7 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     __shared__ Fp8Lds lds;
     int const lane = threadIdx.x & 63;
     int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int const member = wave >> 2;                            // which quartet of the workgroup
     int const j = lane & 15, g = lane >> 4;
 
     int const per = (totalTiles + gridDim.x - 1) / gridDim.x;
@@ -698,42 +662,48 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     build_fp8_feature_lut(lds);
     __syncthreads();
 
-    uint8_t const* stagedBlob = nullptr;
     int topMask = 7;                                         // uniform: hidden layers that need the general evaluation
-
     int entry = 0;
-    for (int first = tileBegin; first < tileEnd; ) {         // every wave of the workgroup walks the same rounds
-        Round const round = plan_round<V>(mips, numMips, first, entry, tileEnd, wave);
-        first += round.count;
-        entry = round.lastEntry;
-        uint8_t const* const blob = mips[round.entry].weights;
-        if (blob != stagedBlob) {                            // uniform across the workgroup
-            __syncthreads();
-            topMask = stage_fp8_weights<V>(lds, blob);
-            stagedBlob = blob;
-            __syncthreads();
-        }
-        WaveTile const& t = round.mine;
-        if (!t.work) continue;
-        DevMip const& m = mips[t.entry];
+    for (int segBegin = tileBegin; segBegin < tileEnd; ) {   // uniform across the workgroup
+        while (entry + 1 < numMips && mips[entry + 1].tileStart <= segBegin) ++entry;
+        uint8_t const* const blob = mips[entry].weights;
+        int segEnd = tileEnd;
+        for (int k = entry + 1; k < numMips && mips[k].tileStart < tileEnd; ++k)
+            if (mips[k].weights != blob) { segEnd = mips[k].tileStart; break; }
+        if (segBegin != tileBegin) __syncthreads();          // every wave has left the previous segment's weights
+        topMask = stage_fp8_weights<V>(lds, blob);
+        __syncthreads();
 
-        uint32_t in[24];
-        {
-            int const x = min(t.x0 + j, m.width - 1), y = min(t.y0 + g, m.height - 1);
-            if (m.fast) {
-                Fp8Fetch<V> fetch;
-                fetch_latents_fast<V>(m, x, y, fetch);
-                finish_inputs_fast<V>(m, lds, x, y, fetch, in);
-            } else {
-                prepare_inputs_fp8<V>(m, x, y, in);
+        int const part = (segEnd - segBegin + V::GROUP - 1) / V::GROUP;
+        int const myBegin = segBegin + member * part, myEnd = min(segEnd, myBegin + part);
+        int mine = entry;
+        for (int tile = myBegin; tile < myEnd; ++tile) {     // uniform across the wave
+            while (mine + 1 < numMips && mips[mine + 1].tileStart <= tile) ++mine;
+            DevMip const& m = mips[mine];
+            int const local = tile - m.tileStart;
+            int const tileY = local / m.tilesX, tileX = local - tileY * m.tilesX;
+            int const x0 = tileX * 64 + (wave & 3) * 16, y0 = tileY * 4;
+            if (x0 >= m.width) continue;                     // whole wave tile outside the image
+
+            uint32_t in[24];
+            {
+                int const x = min(x0 + j, m.width - 1), y = min(y0 + g, m.height - 1);
+                if (m.fast) {
+                    Fp8Fetch<V> fetch;
+                    fetch_latents_fast<V>(m, x, y, fetch);
+                    finish_inputs_fast<V>(m, lds, x, y, fetch, in);
+                } else {
+                    prepare_inputs_fp8<V>(m, x, y, in);
+                }
             }
+            v4i D[4];
+            v4f S;
+            mlp_forward_fp8<V>(lds, wave, lane, topMask, in, D, S);
+            if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)      store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, x0 + j, y0, 4 * g);
+            else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)       store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
+            else                                                       store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
         }
-        v4i D[4];
-        v4f S;
-        mlp_forward_fp8<V>(lds, wave, lane, topMask, in, D, S);
-        if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)      store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, t.x0 + j, t.y0, 4 * g);
-        else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)       store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, t.x0 + j, t.y0, 4 * g);
-        else                                                       store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, t.x0 + j, t.y0, 4 * g);
+        segBegin = segEnd;
     }
 }
 

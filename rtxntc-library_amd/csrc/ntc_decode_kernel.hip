@@ -1091,39 +1091,13 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     int staged = 0;                                          // uniform: how layers 1..3 of the staged set run (kStagedF16, ...)
     int entry = 0;
 
-    for (int first = tileBegin; first < tileEnd; ) {
-        while (entry + 1 < numMips && mips[entry + 1].tileStart <= first) ++entry;
-
-        if (mips[entry].weights != stagedBlob) {             // uniform across the workgroup
-            __syncthreads();
-            staged = stage_weights<V>(lds, mips[entry].weights);
-            stagedBlob = mips[entry].weights;
-            __syncthreads();                                 // also publishes the tables built above
-        }
-
-        // This round's tiles: `first` and the ones after it that use the staged weights, GROUP at most.  Every
-        // thread computes the same count, so the loop (and the barriers above) stay uniform; a wave without a
-        // tile sits the round out.
-        int count = 1, mine = entry;
-        if constexpr (GROUP > 1) {
-            int next = entry;
-            for (int k = 1; k < GROUP && first + k < tileEnd; ++k) {
-                while (next + 1 < numMips && mips[next + 1].tileStart <= first + k) ++next;
-                if (mips[next].weights != stagedBlob) break;
-                ++count;
-                if (k == member) mine = next;
-            }
-        }
-        int const tile = first + member;
-        first += count;
-        if (GROUP > 1 && member >= count) continue;
-        DevMip const& m = mips[mine];
-
+    // One wave tile: the 16 x 4 texels of this wave in tile `tile` of mip m.
+    auto decode_wave_tile = [&](DevMip const& m, int tile) __attribute__((always_inline)) {
         int const local = tile - m.tileStart;
         int const tileY = local / m.tilesX, tileX = local - tileY * m.tilesX;
         int const x0 = tileX * 64 + (GROUP > 1 ? wave & 3 : wave) * 16;
         int const y0 = tileY * 4;
-        if (x0 >= m.width) continue;                         // whole wave tile outside the image
+        if (x0 >= m.width) return;                           // whole wave tile outside the image
 
         // ---- 1. input stage: lane = texel (tx = lane%16, ty = lane/16)
         uint32_t in[16];
@@ -1153,6 +1127,46 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
             if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)      store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, x0 + j, y0, 4 * g);
             else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)       store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
             else                                                       store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
+        }
+    };
+
+    if constexpr (GROUP == 1) {
+        for (int tile = tileBegin; tile < tileEnd; ++tile) {
+            while (entry + 1 < numMips && mips[entry + 1].tileStart <= tile) ++entry;
+            if (mips[entry].weights != stagedBlob) {         // uniform across the workgroup
+                __syncthreads();
+                staged = stage_weights<V>(lds, mips[entry].weights);
+                stagedBlob = mips[entry].weights;
+                __syncthreads();                             // also publishes the tables built above
+            }
+            decode_wave_tile(mips[entry], tile);
+        }
+    } else {
+        // Several wave quartets share the staged weights.  The workgroup walks its share in segments of tiles that
+        // use one weight blob (a single segment, unless sets of a batch meet inside the share), and inside a
+        // segment every quartet walks a contiguous part: its consecutive tiles are neighbours in the image and
+        // find the cache lines they share still in place.  (Quartets that took alternate tiles of one sequence
+        // drifted apart in time, and latent reads from memory doubled.)
+        for (int segBegin = tileBegin; segBegin < tileEnd; ) {
+            while (entry + 1 < numMips && mips[entry + 1].tileStart <= segBegin) ++entry;
+            uint8_t const* const blob = mips[entry].weights;
+            int segEnd = tileEnd;
+            for (int k = entry + 1; k < numMips && mips[k].tileStart < tileEnd; ++k)
+                if (mips[k].weights != blob) { segEnd = mips[k].tileStart; break; }
+            if (blob != stagedBlob) {                        // uniform across the workgroup
+                __syncthreads();                             // every wave has left the previous segment's weights
+                staged = stage_weights<V>(lds, blob);
+                stagedBlob = blob;
+                __syncthreads();                             // also publishes the tables built above
+            }
+            int const part = (segEnd - segBegin + GROUP - 1) / GROUP;
+            int const myBegin = segBegin + member * part, myEnd = min(segEnd, myBegin + part);
+            int mine = entry;
+            for (int tile = myBegin; tile < myEnd; ++tile) {
+                while (mine + 1 < numMips && mips[mine + 1].tileStart <= tile) ++mine;
+                decode_wave_tile(mips[mine], tile);
+            }
+            segBegin = segEnd;
         }
     }
 }
