@@ -159,6 +159,23 @@ def test_cfg2_batch_of_sets(ntc, device):
         assert_equal_bytes(hset.output, c.d_output.download(), f"cfg2 set {i}")
 
 
+def test_cfg3_batch_with_set_boundaries_inside_a_workgroups_share(ntc, device):
+    """More tiles than resident workgroups can take a few at a time: every workgroup owns a share of ten tiles, its
+    two wave quartets walk one half each of the part that uses one set's weights, and sets begin in the middle of
+    shares.  Tile counts per set that are odd and even."""
+    sizes = [(512, 384), (320, 200), (448, 512), (64, 700), (512, 512), (384, 320)]
+    spec = ntc.presets.spec_cfg3()
+    cases = [cfg_case(ntc, spec, w, h, ntc.presets.full_mip_count(w, h), 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=500 + i,
+                      scale_log2_range=(-17.0, -13.0)) for i, (w, h) in enumerate(sizes)]
+    hosts = [c.host_set() for c in cases]
+    for hset in hosts:
+        hset.decode(threads=8)
+    device.decode([c.device_set(device) for c in cases])
+    device.synchronize()
+    for i, (c, hset) in enumerate(zip(cases, hosts)):
+        assert_equal_bytes(hset.output, c.d_output.download(), f"cfg3 batch, set {i}")
+
+
 def test_cfg3_fp8_batch_of_sets(ntc, device):
     """Several e4m3 sets with their own weights in one launch.  A workgroup of that decoder works on two tiles at
     a time as long as both use the staged weights; every set has an odd number of tiles (353) and a workgroup's
