@@ -505,10 +505,18 @@ template <int PLANES, int TILES, int NK32, bool HAS16, bool LAST_HIDDEN, class L
 __device__ __forceinline__ void fp8_hidden_layer(Load&& load, uint4 const (&B32)[NK32][4], uint2 const (&B16)[4], uint32_t (&H)[4][4][2])
 {
     v4f const zero = { 0.f, 0.f, 0.f, 0.f };
+    // The operands of output tile t + 1 are loaded before the work on tile t (two sets of registers, alternating);
+    // a scheduling barrier that only LDS reads may not cross keeps the compiler from moving those loads back down
+    // to their uses.
+    TileOperands<NK32, HAS16> ops[2];
+    load(0, ops[0]);
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
-        TileOperands<NK32, HAS16> o;
-        load(t, o);
+        if (t + 1 < TILES) {
+            load(t + 1, ops[(t + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0x67f);           // everything but LDS instructions may cross
+        }
+        TileOperands<NK32, HAS16> const& o = ops[t & 1];
         v4f acc[3][4];
 #pragma unroll
         for (int p = 0; p < 3; ++p) {
