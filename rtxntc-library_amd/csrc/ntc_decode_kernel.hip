@@ -477,62 +477,72 @@ __device__ __forceinline__ void prepare_inputs_general(DevMip const& m, int x, i
     }
 }
 
-// Input vector of one texel from integer arithmetic only (see axis_fast above).
+// Input vector of one texel from integer arithmetic only (see axis_fast above).  All gathers of both grids are
+// issued before any of them is waited for (the scheduling barrier keeps the compiler from sinking the last of them
+// below the first wait): one memory round trip per tile, not two.
 template <class V, class Mip = DevMip>
 __device__ __forceinline__ void prepare_inputs_fast(Mip const& m, LdsT<V> const& lds, int x, int y, uint32_t (&in)[16])
 {
+    constexpr int HL = V::HR_MODE == 1 ? 1 : (V::HR_F + 3) / 4, LL = (V::LR_F + 3) / 4;
 #pragma unroll
     for (int i = 0; i < 16; ++i) in[i] = 0;
 
-    // ---- high-res grid
+    AxisFoot const hx = axis_fast(x, m.hrAxisX, m.hrWidth), hy = axis_fast(y, m.hrAxisY, m.hrHeight);
+    AxisFoot const lx = axis_fast(x, m.lrAxisX, m.lrWidth), ly = axis_fast(y, m.lrAxisY, m.lrHeight);
+    uint32_t hv[HL][4], lv[LL][4];                           // [layer][tap 00, 10, 01, 11]
     {
-        AxisFoot const ax = axis_fast(x, m.hrAxisX, m.hrWidth), ay = axis_fast(y, m.hrAxisY, m.hrHeight);
         GlobalU8Ptr const g = (GlobalU8Ptr)m.hr;
         uint32_t const lgw = ((m.hrAxisX >> 24) & 0xffu) + 1u;   // log2(bytes per grid row)
         uint32_t const layerStride = uint32_t(m.hrWidth) * uint32_t(m.hrHeight) * 2u;   // bytes
-        uint32_t const r0 = ay.c0 << lgw, r1 = ay.c1 << lgw, c0 = ax.c0 << 1, c1 = ax.c1 << 1;
+        uint32_t const r0 = hy.c0 << lgw, r1 = hy.c1 << lgw, c0 = hx.c0 << 1, c1 = hx.c1 << 1;
         uint32_t const a00 = r0 + c0, a10 = r0 + c1, a01 = r1 + c0, a11 = r1 + c1;   // byte offsets
-        if constexpr (V::HR_MODE == 1) {
-            static_assert(V::HR_MODE != 1 || (V::HR_BITS == 2 && V::HR_F == 8 && V::HR_SLOTS == 8), "concat grids: 8 x 2-bit");
-            uint32_t const addr[4] = { a00, a10, a01, a11 };
 #pragma unroll
-            for (int tap = 0; tap < 4; ++tap) {
-                uint32_t const w = load_u16(g, addr[tap]);
-                in[2 * tap]     = lds.lut2[w & 0xffu];
-                in[2 * tap + 1] = lds.lut2[w >> 8];
-            }
-        } else {
-            uint32_t const nx = (m.hrAxisX >> 8) & 0xffu, ny = (m.hrAxisY >> 8) & 0xffu;
-            uint32_t const wx1 = ax.f, wx0 = (1u << nx) - ax.f, wy1 = ay.f, wy0 = (1u << ny) - ay.f;
-            uint32_t const w00 = mul24(wx0, wy0), w10 = mul24(wx1, wy0), w01 = mul24(wx0, wy1), w11 = mul24(wx1, wy1);
-            constexpr int layers = (V::HR_F + 3) / 4;
+        for (int L = 0; L < HL; ++L) {
+            GlobalU8Ptr const gl = g + size_t(L) * layerStride;
+            hv[L][0] = load_u16(gl, a00); hv[L][1] = load_u16(gl, a10); hv[L][2] = load_u16(gl, a01); hv[L][3] = load_u16(gl, a11);
+        }
+    }
+    {
+        GlobalU8Ptr const g = (GlobalU8Ptr)m.lr;
+        uint32_t const lgw = ((m.lrAxisX >> 24) & 0xffu) + 1u;
+        uint32_t const layerStride = uint32_t(m.lrWidth) * uint32_t(m.lrHeight) * 2u;
+        uint32_t const r0 = ly.c0 << lgw, r1 = ly.c1 << lgw, c0 = lx.c0 << 1, c1 = lx.c1 << 1;
+        uint32_t const a00 = r0 + c0, a10 = r0 + c1, a01 = r1 + c0, a11 = r1 + c1;
 #pragma unroll
-            for (int L = 0; L < layers; ++L) {
-                GlobalU8Ptr const gl = g + size_t(L) * layerStride;
-                uint32_t b = bilinear4_int(load_u16(gl, a00), load_u16(gl, a10), load_u16(gl, a01), load_u16(gl, a11),
-                                           w00, w10, w01, w11, nx + ny);
-                if (4 * L + 4 > V::HR_F) b &= (1u << (8 * (V::HR_F - 4 * L))) - 1u;
-                in[L] = b;
-            }
+        for (int L = 0; L < LL; ++L) {
+            GlobalU8Ptr const gl = g + size_t(L) * layerStride;
+            lv[L][0] = load_u16(gl, a00); lv[L][1] = load_u16(gl, a10); lv[L][2] = load_u16(gl, a01); lv[L][3] = load_u16(gl, a11);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- high-res grid
+    if constexpr (V::HR_MODE == 1) {
+        static_assert(V::HR_MODE != 1 || (V::HR_BITS == 2 && V::HR_F == 8 && V::HR_SLOTS == 8), "concat grids: 8 x 2-bit");
+#pragma unroll
+        for (int tap = 0; tap < 4; ++tap) {
+            in[2 * tap]     = lds.lut2[hv[0][tap] & 0xffu];
+            in[2 * tap + 1] = lds.lut2[hv[0][tap] >> 8];
+        }
+    } else {
+        uint32_t const nx = (m.hrAxisX >> 8) & 0xffu, ny = (m.hrAxisY >> 8) & 0xffu;
+        uint32_t const wx1 = hx.f, wx0 = (1u << nx) - hx.f, wy1 = hy.f, wy0 = (1u << ny) - hy.f;
+        uint32_t const w00 = mul24(wx0, wy0), w10 = mul24(wx1, wy0), w01 = mul24(wx0, wy1), w11 = mul24(wx1, wy1);
+#pragma unroll
+        for (int L = 0; L < HL; ++L) {
+            uint32_t b = bilinear4_int(hv[L][0], hv[L][1], hv[L][2], hv[L][3], w00, w10, w01, w11, nx + ny);
+            if (4 * L + 4 > V::HR_F) b &= (1u << (8 * (V::HR_F - 4 * L))) - 1u;
+            in[L] = b;
         }
     }
     // ---- low-res grid: bilinear, 4-bit
     {
-        AxisFoot const ax = axis_fast(x, m.lrAxisX, m.lrWidth), ay = axis_fast(y, m.lrAxisY, m.lrHeight);
-        GlobalU8Ptr const g = (GlobalU8Ptr)m.lr;
-        uint32_t const lgw = ((m.lrAxisX >> 24) & 0xffu) + 1u;
-        uint32_t const layerStride = uint32_t(m.lrWidth) * uint32_t(m.lrHeight) * 2u;
-        uint32_t const r0 = ay.c0 << lgw, r1 = ay.c1 << lgw, c0 = ax.c0 << 1, c1 = ax.c1 << 1;
-        uint32_t const a00 = r0 + c0, a10 = r0 + c1, a01 = r1 + c0, a11 = r1 + c1;
         uint32_t const nx = (m.lrAxisX >> 8) & 0xffu, ny = (m.lrAxisY >> 8) & 0xffu;
-        uint32_t const wx1 = ax.f, wx0 = (1u << nx) - ax.f, wy1 = ay.f, wy0 = (1u << ny) - ay.f;
+        uint32_t const wx1 = lx.f, wx0 = (1u << nx) - lx.f, wy1 = ly.f, wy0 = (1u << ny) - ly.f;
         uint32_t const w00 = mul24(wx0, wy0), w10 = mul24(wx1, wy0), w01 = mul24(wx0, wy1), w11 = mul24(wx1, wy1);
-        constexpr int layers = (V::LR_F + 3) / 4;
 #pragma unroll
-        for (int L = 0; L < layers; ++L) {
-            GlobalU8Ptr const gl = g + size_t(L) * layerStride;
-            uint32_t b = bilinear4_int(load_u16(gl, a00), load_u16(gl, a10), load_u16(gl, a01), load_u16(gl, a11),
-                                       w00, w10, w01, w11, nx + ny);
+        for (int L = 0; L < LL; ++L) {
+            uint32_t b = bilinear4_int(lv[L][0], lv[L][1], lv[L][2], lv[L][3], w00, w10, w01, w11, nx + ny);
             if (4 * L + 4 > V::LR_F) b &= (1u << (8 * (V::LR_F - 4 * L))) - 1u;
             in[V::HR_INPUTS / 4 + L] = b;
         }
