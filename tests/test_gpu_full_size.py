@@ -157,6 +157,44 @@ def test_random_access_8192_queries(ntc, device, oracle):
     assert np.array_equal(got[:sample], want)
 
 
+def test_fp8_network_random_access_8192_queries(ntc, device, oracle):
+    """The same 2^24 sample points into an 8192^2, 14-mip set of the LibNTC 0.9.2 geometry, decoded with the FP8
+    network from the query-ordered copy of the latents: a 2^20 sample against the checker, repeated queries repeat
+    their answers, the 1 x 1 mip answers with one texel, and the file-ordered grids give the same bits."""
+    spec = ntc.presets.spec_ref092_fp8(16)
+    mips, latent_bytes = ntc.presets.mips_ref092(spec, 8192, 8192, 14, 2)
+    case = Case(ntc, spec, mips, latent_bytes, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=4, weights=ntc.synth.make_fp8_weights(spec, 6))
+    n = 1 << 24
+    rng = np.random.default_rng(4)
+    q = np.zeros(n, dtype=[("u", np.float32), ("v", np.float32), ("mip", np.int32)])
+    q["u"], q["v"] = rng.random(n, dtype=np.float32), rng.random(n, dtype=np.float32)
+    q["mip"] = rng.integers(0, 14, n)
+    q[n // 2:] = q[: n // 2]                                    # second half repeats the first
+    d_lat, d_w = device.upload(case.latents), device.upload(case.weights)
+    dset = ntc.make_texture_set(case.spec, case.mips, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, d_lat.ptr, d_lat.nbytes,
+                                d_w.ptr, d_w.nbytes, None, 0)
+    d_q, d_out = device.upload(q.view(np.uint8)), device.alloc(n * 32)
+    ntc.abi.check(device.lib.ntc_hip_decode_queries(dset, d_q.ptr, n, d_out.ptr, d_out.nbytes))
+    device.synchronize()
+    from_file_order = d_out.download(np.uint16).reshape(n, 16)
+    d_bricks = device.alloc(device.lib.ntc_hip_query_latents_bytes(dset))
+    ntc.abi.check(device.lib.ntc_hip_build_query_latents(dset, d_bricks.ptr, d_bricks.nbytes))
+    dset.queryLatents, dset.queryLatentsBytes = d_bricks.ptr, d_bricks.nbytes
+    d_out.fill(0xCD)
+    ntc.abi.check(device.lib.ntc_hip_decode_queries(dset, d_q.ptr, n, d_out.ptr, d_out.nbytes))
+    device.synchronize()
+    got = d_out.download(np.uint16).reshape(n, 16)
+    assert np.array_equal(got, from_file_order)
+    assert np.array_equal(got[: n // 2], got[n // 2:])
+    last = got[q["mip"] == 13]
+    assert np.array_equal(last, np.broadcast_to(last[0], last.shape))
+    host = case.host_set()
+    sample = 1 << 20
+    want = np.zeros((sample, 16), dtype=np.uint16)
+    assert oracle.ntc_oracle_decode_queries(host.desc, q.ctypes.data, sample, want.ctypes.data, 16) == 0
+    assert np.array_equal(got[:sample], want)
+
+
 def test_single_mip_beyond_4_gib(ntc, device, oracle):
     """16384 x 16384, 10 channels, one mip: a 5.4 GB planar image, so byte offsets inside one mip pass
     2^32 (at row 13107).  Bands of rows at the top, across that row and at the bottom against the checker."""
