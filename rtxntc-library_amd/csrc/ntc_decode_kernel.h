@@ -161,6 +161,7 @@ hipError_t launch_queries_fp8(int variant, DevMip const* mips, int numMips, DevQ
 hipError_t launch_selftest_fp8_activation(uint16_t const* in, uint16_t* out, int n, hipStream_t stream);
 int resident_workgroups_per_cu(int variant);
 int tiles_per_round(int variant);      // tiles a workgroup of the variant's decode kernel works on at a time
+int threads_per_workgroup(int variant);
 hipError_t launch_selftest_mfma(int8_t const* a, int8_t const* b, int32_t* d, hipStream_t stream);
 hipError_t launch_selftest_mfma_f16(uint16_t const* a, uint16_t const* b, float const* c, float* d, int depth, hipStream_t stream);
 

@@ -91,12 +91,18 @@ struct Variant {
     static constexpr bool FP8_WEIGHTS = FP8_WEIGHTS_;
     static constexpr int PLANES = FP8_WEIGHTS_ ? 3 : 1;
     static constexpr int F16_PLANES = FP8_WEIGHTS_ ? 2 : 1;
-    // Waves per workgroup: four cover one 64 x 4 tile.  The e4m3 variants keep so many weight planes in LDS that
-    // only two workgroups fit a CU; theirs have eight waves (two tiles at a time), which again puts four waves
-    // on every SIMD to overlap matrix and vector work.
-    static constexpr int WAVES = FP8_WEIGHTS_ ? 8 : 4;
+    // Waves per workgroup: four (a quartet) cover one 64 x 4 tile.  A workgroup has two quartets around one copy
+    // of the weights, two workgroups fit a CU (the e4m3 variants keep so many weight planes in LDS that no more
+    // would fit anyway): four waves on every SIMD to overlap matrix and vector work.
+    static constexpr int WAVES = 8;
     static constexpr int THREADS = 64 * WAVES;
-    static constexpr int RESIDENT = FP8_WEIGHTS_ ? 2 : 4;      // workgroups per CU the LDS footprint allows
+    static constexpr int RESIDENT = 2;                         // workgroups per CU
+    // How a workgroup's share of tiles is divided: every wave walks a contiguous run of wave tiles of its own, or
+    // every quartet a contiguous run of tiles.  Either way a wave's next tile is a neighbour of its last one and
+    // finds the cache lines they share in place; which of the two is faster depends on the input stage (measured:
+    // waves for the geometries whose high-resolution grid is taken as 2 x 2 cells, quartets where both grids are
+    // filtered and a tile's 32 gathers per lane overlap between the waves of a quartet).
+    static constexpr bool PER_WAVE = !FP8_WEIGHTS_ && HR_MODE_ == 1;
     static constexpr int WAVES_PER_SIMD = RESIDENT * WAVES / 4; // what the register budget is set for
     // Dwords per texel in the transpose buffer in front of the network: 16 + 4 of padding, or 12 without
     // padding for 48 inputs (rows then still start in distinct banks: 12 j mod 64 differ for j = 0..15).
@@ -1070,17 +1076,16 @@ __device__ __forceinline__ void mlp_forward_f16(LdsT<V>& lds, int wave, int lane
     f16_tile<V, V::T2>(lds, V::F16_L3, 0, lane, Ha, D);
 }
 
-// Four workgroups per CU (16 waves, 128 VGPRs each) is what the LDS footprint allows and what hides
-// the latency of the input stage; the e4m3 variants hold several planes of every weight in LDS and fit two.
+// Two workgroups of eight waves per CU: sixteen waves, 128 VGPRs each, four to a SIMD.
 template <class V>
 __global__ void __launch_bounds__(V::THREADS, V::WAVES_PER_SIMD)
 decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
 {
     __shared__ LdsT<V> lds;
-    constexpr int GROUP = V::WAVES / 4;                      // tiles a workgroup works on at a time
+    constexpr int GROUP = V::WAVES / 4;                      // quartets of a workgroup
     int const lane = threadIdx.x & 63;
     int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    int const member = GROUP > 1 ? wave >> 2 : 0;            // which tile of the group this wave works on
+    int const member = wave >> 2;                            // which quartet this wave belongs to
     int const j = lane & 15, g = lane >> 4;
 
     // contiguous share of the tile list for this workgroup
@@ -1102,10 +1107,10 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     int entry = 0;
 
     // One wave tile: the 16 x 4 texels of this wave in tile `tile` of mip m.
-    auto decode_wave_tile = [&](DevMip const& m, int tile) __attribute__((always_inline)) {
+    auto decode_wave_tile = [&](DevMip const& m, int tile, int sub) __attribute__((always_inline)) {
         int const local = tile - m.tileStart;
         int const tileY = local / m.tilesX, tileX = local - tileY * m.tilesX;
-        int const x0 = tileX * 64 + (GROUP > 1 ? wave & 3 : wave) * 16;
+        int const x0 = tileX * 64 + sub * 16;
         int const y0 = tileY * 4;
         if (x0 >= m.width) return;                           // whole wave tile outside the image
 
@@ -1140,44 +1145,38 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
         }
     };
 
-    if constexpr (GROUP == 1) {
-        for (int tile = tileBegin; tile < tileEnd; ++tile) {
-            while (entry + 1 < numMips && mips[entry + 1].tileStart <= tile) ++entry;
-            if (mips[entry].weights != stagedBlob) {         // uniform across the workgroup
-                __syncthreads();
-                staged = stage_weights<V>(lds, mips[entry].weights);
-                stagedBlob = mips[entry].weights;
-                __syncthreads();                             // also publishes the tables built above
-            }
-            decode_wave_tile(mips[entry], tile);
+    // The workgroup walks its share in segments of tiles that use one weight blob (a single segment, unless sets of
+    // a batch meet inside the share); inside a segment its waves or quartets walk contiguous parts.  (Quartets that
+    // took alternate tiles of one sequence drifted apart in time, and latent reads from memory doubled.)
+    for (int segBegin = tileBegin; segBegin < tileEnd; ) {
+        while (entry + 1 < numMips && mips[entry + 1].tileStart <= segBegin) ++entry;
+        uint8_t const* const blob = mips[entry].weights;
+        int segEnd = tileEnd;
+        for (int k = entry + 1; k < numMips && mips[k].tileStart < tileEnd; ++k)
+            if (mips[k].weights != blob) { segEnd = mips[k].tileStart; break; }
+        if (blob != stagedBlob) {                            // uniform across the workgroup
+            __syncthreads();                                 // every wave has left the previous segment's weights
+            staged = stage_weights<V>(lds, blob);
+            stagedBlob = blob;
+            __syncthreads();                                 // also publishes the tables built above
         }
-    } else {
-        // Several wave quartets share the staged weights.  The workgroup walks its share in segments of tiles that
-        // use one weight blob (a single segment, unless sets of a batch meet inside the share), and inside a
-        // segment every quartet walks a contiguous part: its consecutive tiles are neighbours in the image and
-        // find the cache lines they share still in place.  (Quartets that took alternate tiles of one sequence
-        // drifted apart in time, and latent reads from memory doubled.)
-        for (int segBegin = tileBegin; segBegin < tileEnd; ) {
-            while (entry + 1 < numMips && mips[entry + 1].tileStart <= segBegin) ++entry;
-            uint8_t const* const blob = mips[entry].weights;
-            int segEnd = tileEnd;
-            for (int k = entry + 1; k < numMips && mips[k].tileStart < tileEnd; ++k)
-                if (mips[k].weights != blob) { segEnd = mips[k].tileStart; break; }
-            if (blob != stagedBlob) {                        // uniform across the workgroup
-                __syncthreads();                             // every wave has left the previous segment's weights
-                staged = stage_weights<V>(lds, blob);
-                stagedBlob = blob;
-                __syncthreads();                             // also publishes the tables built above
+        int mine = entry;
+        if constexpr (V::PER_WAVE) {
+            int const part = (4 * (segEnd - segBegin) + V::WAVES - 1) / V::WAVES;          // wave tiles: four to a tile
+            int const myBegin = 4 * segBegin + wave * part, myEnd = min(4 * segEnd, myBegin + part);
+            for (int wt = myBegin; wt < myEnd; ++wt) {
+                while (mine + 1 < numMips && mips[mine + 1].tileStart <= (wt >> 2)) ++mine;
+                decode_wave_tile(mips[mine], wt >> 2, wt & 3);
             }
+        } else {
             int const part = (segEnd - segBegin + GROUP - 1) / GROUP;
             int const myBegin = segBegin + member * part, myEnd = min(segEnd, myBegin + part);
-            int mine = entry;
             for (int tile = myBegin; tile < myEnd; ++tile) {
                 while (mine + 1 < numMips && mips[mine + 1].tileStart <= tile) ++mine;
-                decode_wave_tile(mips[mine], tile);
+                decode_wave_tile(mips[mine], tile, wave & 3);
             }
-            segBegin = segEnd;
         }
+        segBegin = segEnd;
     }
 }
 
@@ -1416,7 +1415,8 @@ int resident_workgroups_per_cu(int variant)
     }
 }
 
-int tiles_per_round(int variant) { return variant == NTC_HIP_VARIANT_CFG3_FP8 ? VCfg3::WAVES / 4 : 1; }
+int tiles_per_round(int) { return VCfg01::WAVES / 4; }
+int threads_per_workgroup(int) { return VCfg01::THREADS; }
 
 hipError_t launch_selftest_mfma(int8_t const* a, int8_t const* b, int32_t* d, hipStream_t stream)
 {

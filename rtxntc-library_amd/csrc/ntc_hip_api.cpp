@@ -692,7 +692,7 @@ static int run_queries(NtcHipContext* ctx, const NtcHipTextureSet* set, const Nt
     if (int r = build_table(set, 1, table, variant, totalTiles, true)) return r;
     bool const fp8 = variant_is_fp8_network(variant);
     if (int r = upload_table(L, table)) return r;
-    uint64_t const perBlock = fp8 ? uint64_t(fp8_threads_per_workgroup()) : 256u;
+    uint64_t const perBlock = uint64_t(fp8 ? fp8_threads_per_workgroup() : threads_per_workgroup(variant));
     uint64_t const blocks = (numQueries + perBlock - 1) / perBlock;
     uint64_t const resident = uint64_t(L.computeUnits) * uint64_t(grid_size_for(L, variant, 0x7fffffff) / L.computeUnits);
     int const grid = int(blocks < resident ? blocks : resident);
