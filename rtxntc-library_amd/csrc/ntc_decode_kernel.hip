@@ -97,12 +97,6 @@ struct Variant {
     static constexpr int WAVES = 8;
     static constexpr int THREADS = 64 * WAVES;
     static constexpr int RESIDENT = 2;                         // workgroups per CU
-    // How a workgroup's share of tiles is divided: every wave walks a contiguous run of wave tiles of its own, or
-    // every quartet a contiguous run of tiles.  Either way a wave's next tile is a neighbour of its last one and
-    // finds the cache lines they share in place; which of the two is faster depends on the input stage (measured:
-    // waves for the geometries whose high-resolution grid is taken as 2 x 2 cells, quartets where both grids are
-    // filtered and a tile's 32 gathers per lane overlap between the waves of a quartet).
-    static constexpr bool PER_WAVE = !FP8_WEIGHTS_ && HR_MODE_ == 1;
     static constexpr int WAVES_PER_SIMD = RESIDENT * WAVES / 4; // what the register budget is set for
     // Dwords per texel in the transpose buffer in front of the network: 16 + 4 of padding, or 12 without
     // padding for 48 inputs (rows then still start in distinct banks: 12 j mod 64 differ for j = 0..15).
@@ -1146,8 +1140,11 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     };
 
     // The workgroup walks its share in segments of tiles that use one weight blob (a single segment, unless sets of
-    // a batch meet inside the share); inside a segment its waves or quartets walk contiguous parts.  (Quartets that
-    // took alternate tiles of one sequence drifted apart in time, and latent reads from memory doubled.)
+    // a batch meet inside the share); inside a segment each quartet walks a contiguous part, so that its next tile
+    // is a neighbour of its last one and finds the cache lines they share in place, and the four waves of a quartet
+    // write whole lines together.  (Quartets that took alternate tiles of one sequence drifted apart in time, and
+    // latent reads from memory doubled; waves that each walked wave tiles of their own wrote 12 % more bytes to
+    // memory, half lines at a time.)
     for (int segBegin = tileBegin; segBegin < tileEnd; ) {
         while (entry + 1 < numMips && mips[entry + 1].tileStart <= segBegin) ++entry;
         uint8_t const* const blob = mips[entry].weights;
@@ -1160,21 +1157,12 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
             stagedBlob = blob;
             __syncthreads();                                 // also publishes the tables built above
         }
+        int const part = (segEnd - segBegin + GROUP - 1) / GROUP;
+        int const myBegin = segBegin + member * part, myEnd = min(segEnd, myBegin + part);
         int mine = entry;
-        if constexpr (V::PER_WAVE) {
-            int const part = (4 * (segEnd - segBegin) + V::WAVES - 1) / V::WAVES;          // wave tiles: four to a tile
-            int const myBegin = 4 * segBegin + wave * part, myEnd = min(4 * segEnd, myBegin + part);
-            for (int wt = myBegin; wt < myEnd; ++wt) {
-                while (mine + 1 < numMips && mips[mine + 1].tileStart <= (wt >> 2)) ++mine;
-                decode_wave_tile(mips[mine], wt >> 2, wt & 3);
-            }
-        } else {
-            int const part = (segEnd - segBegin + GROUP - 1) / GROUP;
-            int const myBegin = segBegin + member * part, myEnd = min(segEnd, myBegin + part);
-            for (int tile = myBegin; tile < myEnd; ++tile) {
-                while (mine + 1 < numMips && mips[mine + 1].tileStart <= tile) ++mine;
-                decode_wave_tile(mips[mine], tile, wave & 3);
-            }
+        for (int tile = myBegin; tile < myEnd; ++tile) {
+            while (mine + 1 < numMips && mips[mine + 1].tileStart <= tile) ++mine;
+            decode_wave_tile(mips[mine], tile, wave & 3);
         }
         segBegin = segEnd;
     }
