@@ -671,6 +671,30 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     __syncthreads();
 
     int topMask = 7;                                         // uniform: hidden layers that need the general evaluation
+
+    // One wave tile: the 16 x 4 texels of this wave in tile (tileX, tileY) of mip m.
+    auto decode_wave_tile = [&](DevMip const& m, int tileX, int tileY) __attribute__((always_inline)) {
+        int const x0 = tileX * 64 + (wave & 3) * 16, y0 = tileY * 4;
+        if (x0 >= m.width) return;                           // whole wave tile outside the image
+        uint32_t in[24];
+        {
+            int const x = min(x0 + j, m.width - 1), y = min(y0 + g, m.height - 1);
+            if (m.fast) {
+                Fp8Fetch<V> fetch;
+                fetch_latents_fast<V>(m, x, y, fetch);
+                finish_inputs_fast<V>(m, lds, x, y, fetch, in);
+            } else {
+                prepare_inputs_fp8<V>(m, x, y, in);
+            }
+        }
+        v4i D[4];
+        v4f S;
+        mlp_forward_fp8<V>(lds, wave, lane, topMask, in, D, S);
+        if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)      store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, x0 + j, y0, 4 * g);
+        else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)       store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
+        else                                                       store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
+    };
+
     int entry = 0;
     for (int segBegin = tileBegin; segBegin < tileEnd; ) {   // uniform across the workgroup
         while (entry + 1 < numMips && mips[entry + 1].tileStart <= segBegin) ++entry;
@@ -684,32 +708,19 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
 
         int const part = (segEnd - segBegin + V::GROUP - 1) / V::GROUP;
         int const myBegin = segBegin + member * part, myEnd = min(segEnd, myBegin + part);
+        // The quartet steps through its tiles mip by mip, keeping the tile's place in the mip in registers: no
+        // look-up in the table (a vector load and a wait for every outstanding store, per tile) and no division.
         int mine = entry;
-        for (int tile = myBegin; tile < myEnd; ++tile) {     // uniform across the wave
+        for (int tile = myBegin; tile < myEnd; ) {           // one run of tiles per mip
             while (mine + 1 < numMips && mips[mine + 1].tileStart <= tile) ++mine;
             DevMip const& m = mips[mine];
-            int const local = tile - m.tileStart;
-            int const tileY = local / m.tilesX, tileX = local - tileY * m.tilesX;
-            int const x0 = tileX * 64 + (wave & 3) * 16, y0 = tileY * 4;
-            if (x0 >= m.width) continue;                     // whole wave tile outside the image
-
-            uint32_t in[24];
-            {
-                int const x = min(x0 + j, m.width - 1), y = min(y0 + g, m.height - 1);
-                if (m.fast) {
-                    Fp8Fetch<V> fetch;
-                    fetch_latents_fast<V>(m, x, y, fetch);
-                    finish_inputs_fast<V>(m, lds, x, y, fetch, in);
-                } else {
-                    prepare_inputs_fp8<V>(m, x, y, in);
-                }
+            int const runEnd = min(myEnd, mine + 1 < numMips ? mips[mine + 1].tileStart : 0x7fffffff);
+            int const tilesX = m.tilesX, local = tile - m.tileStart;
+            int tileY = local / tilesX, tileX = local - tileY * tilesX;
+            for (; tile < runEnd; ++tile) {
+                decode_wave_tile(m, tileX, tileY);
+                if (++tileX == tilesX) { tileX = 0; ++tileY; }
             }
-            v4i D[4];
-            v4f S;
-            mlp_forward_fp8<V>(lds, wave, lane, topMask, in, D, S);
-            if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)      store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, x0 + j, y0, 4 * g);
-            else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)       store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
-            else                                                       store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
         }
         segBegin = segEnd;
     }

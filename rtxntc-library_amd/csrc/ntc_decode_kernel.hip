@@ -1100,10 +1100,8 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     int staged = 0;                                          // uniform: how layers 1..3 of the staged set run (kStagedF16, ...)
     int entry = 0;
 
-    // One wave tile: the 16 x 4 texels of this wave in tile `tile` of mip m.
-    auto decode_wave_tile = [&](DevMip const& m, int tile, int sub) __attribute__((always_inline)) {
-        int const local = tile - m.tileStart;
-        int const tileY = local / m.tilesX, tileX = local - tileY * m.tilesX;
+    // One wave tile: the 16 x 4 texels of this wave in tile (tileX, tileY) of mip m.
+    auto decode_wave_tile = [&](DevMip const& m, int tileX, int tileY, int sub) __attribute__((always_inline)) {
         int const x0 = tileX * 64 + sub * 16;
         int const y0 = tileY * 4;
         if (x0 >= m.width) return;                           // whole wave tile outside the image
@@ -1159,10 +1157,24 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
         }
         int const part = (segEnd - segBegin + GROUP - 1) / GROUP;
         int const myBegin = segBegin + member * part, myEnd = min(segEnd, myBegin + part);
-        int mine = entry;
-        for (int tile = myBegin; tile < myEnd; ++tile) {
+        // The quartet steps through its tiles mip by mip, keeping the tile's place in the mip in registers: no
+        // look-up in the table (a vector load and a wait for every outstanding store, per tile) and no division.
+        int mine = entry, nextStart = 0, tilesX = 1, tileX = 0, tileY = 0;
+        auto enter_mip_of = [&](int tile) {
             while (mine + 1 < numMips && mips[mine + 1].tileStart <= tile) ++mine;
-            decode_wave_tile(mips[mine], tile, wave & 3);
+            nextStart = mine + 1 < numMips ? mips[mine + 1].tileStart : 0x7fffffff;
+            tilesX = mips[mine].tilesX;
+            int const local = tile - mips[mine].tileStart;
+            tileY = local / tilesX; tileX = local - tileY * tilesX;
+        };
+        for (int tile = myBegin; tile < myEnd; ) {           // one run of tiles per mip: the mip's fields stay in registers
+            enter_mip_of(tile);
+            DevMip const& m = mips[mine];
+            int const runEnd = min(myEnd, nextStart);
+            for (; tile < runEnd; ++tile) {
+                decode_wave_tile(m, tileX, tileY, wave & 3);
+                if (++tileX == tilesX) { tileX = 0; ++tileY; }
+            }
         }
         segBegin = segEnd;
     }
