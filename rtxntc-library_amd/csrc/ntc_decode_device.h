@@ -199,8 +199,21 @@ __device__ __forceinline__ void store_channels(GlobalOutPtr row, uint32_t laneOf
     }
 }
 
-template <int FORMAT, bool CHECKED = true, class Acc>
-__device__ __forceinline__ void store_tile(DevMip const& m, Acc const (&D)[4], v4f S, int x, int y0, int chBase)
+// What the tile loop and the stores need of a mip for every tile, held by value (in scalar registers) for a run
+// of tiles of one mip; the input stages read the rest through `full`.
+struct RunMip {
+    DevMip const& full;
+    uint8_t* out;
+    uint64_t outRowPitch;
+    int32_t width, height, numChannels, outPixelStride, outFormat;
+    uint32_t fast;
+    __device__ __forceinline__ explicit RunMip(DevMip const& m)
+        : full(m), out(m.out), outRowPitch(m.outRowPitch), width(m.width), height(m.height), numChannels(m.numChannels),
+          outPixelStride(m.outPixelStride), outFormat(m.outFormat), fast(m.fast) {}
+};
+
+template <int FORMAT, bool CHECKED = true, class Acc, class Mip>
+__device__ __forceinline__ void store_tile(Mip const& m, Acc const (&D)[4], v4f S, int x, int y0, int chBase)
 {
     int const nch = min(4, m.numChannels - chBase);
     if (x >= m.width || nch <= 0) return;

@@ -673,7 +673,7 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     int topMask = 7;                                         // uniform: hidden layers that need the general evaluation
 
     // One wave tile: the 16 x 4 texels of this wave in tile (tileX, tileY) of mip m.
-    auto decode_wave_tile = [&](DevMip const& m, int tileX, int tileY) __attribute__((always_inline)) {
+    auto decode_wave_tile = [&](RunMip const& m, int tileX, int tileY) __attribute__((always_inline)) {
         int const x0 = tileX * 64 + (wave & 3) * 16, y0 = tileY * 4;
         if (x0 >= m.width) return;                           // whole wave tile outside the image
         uint32_t in[24];
@@ -681,10 +681,10 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
             int const x = min(x0 + j, m.width - 1), y = min(y0 + g, m.height - 1);
             if (m.fast) {
                 Fp8Fetch<V> fetch;
-                fetch_latents_fast<V>(m, x, y, fetch);
-                finish_inputs_fast<V>(m, lds, x, y, fetch, in);
+                fetch_latents_fast<V>(m.full, x, y, fetch);
+                finish_inputs_fast<V>(m.full, lds, x, y, fetch, in);
             } else {
-                prepare_inputs_fp8<V>(m, x, y, in);
+                prepare_inputs_fp8<V>(m.full, x, y, in);
             }
         }
         v4i D[4];
@@ -713,9 +713,9 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
         int mine = entry;
         for (int tile = myBegin; tile < myEnd; ) {           // one run of tiles per mip
             while (mine + 1 < numMips && mips[mine + 1].tileStart <= tile) ++mine;
-            DevMip const& m = mips[mine];
+            RunMip const m(mips[mine]);
             int const runEnd = min(myEnd, mine + 1 < numMips ? mips[mine + 1].tileStart : 0x7fffffff);
-            int const tilesX = m.tilesX, local = tile - m.tileStart;
+            int const tilesX = m.full.tilesX, local = tile - m.full.tileStart;
             int tileY = local / tilesX, tileX = local - tileY * tilesX;
             for (; tile < runEnd; ++tile) {
                 decode_wave_tile(m, tileX, tileY);

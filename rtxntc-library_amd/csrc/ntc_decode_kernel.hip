@@ -1101,7 +1101,7 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     int entry = 0;
 
     // One wave tile: the 16 x 4 texels of this wave in tile (tileX, tileY) of mip m.
-    auto decode_wave_tile = [&](DevMip const& m, int tileX, int tileY, int sub) __attribute__((always_inline)) {
+    auto decode_wave_tile = [&](RunMip const& m, int tileX, int tileY, int sub) __attribute__((always_inline)) {
         int const x0 = tileX * 64 + sub * 16;
         int const y0 = tileY * 4;
         if (x0 >= m.width) return;                           // whole wave tile outside the image
@@ -1110,8 +1110,8 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
         uint32_t in[16];
         {
             int const x = min(x0 + j, m.width - 1), y = min(y0 + g, m.height - 1);
-            if (m.fast) prepare_inputs_fast<V>(m, lds, x, y, in);
-            else        prepare_inputs_general<V>(m, x, y, in);
+            if (m.fast) prepare_inputs_fast<V>(m.full, lds, x, y, in);
+            else        prepare_inputs_general<V>(m.full, x, y, in);
         }
         // ---- 2.-4. transpose, hidden layers, output layer
         if (V::F16_LAYERS && (staged & kStagedF16)) {
@@ -1169,7 +1169,7 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
         };
         for (int tile = myBegin; tile < myEnd; ) {           // one run of tiles per mip: the mip's fields stay in registers
             enter_mip_of(tile);
-            DevMip const& m = mips[mine];
+            RunMip const m(mips[mine]);
             int const runEnd = min(myEnd, nextStart);
             for (; tile < runEnd; ++tile) {
                 decode_wave_tile(m, tileX, tileY, wave & 3);
