@@ -345,6 +345,27 @@ def test_stores_of_chosen_output_values(ntc, device, fmt_name):
         assert first[1] == 127 and first[2] == 128           # 0.49951 * 255 = 127.38, 0.50049 * 255 = 127.62
 
 
+@pytest.mark.parametrize("fmt_name,shift,row_pad,stride", [
+    ("OUT_FP16_PIXELS", 2, 0, 32), ("OUT_FP16_PIXELS", 0, 2, 32), ("OUT_FP16_PIXELS", 0, 0, 34), ("OUT_FP16_PIXELS", 4, 4, 36),
+    ("OUT_FP16_PIXELS", 8, 8, 40),
+    ("OUT_UNORM8_PIXELS", 1, 0, 16), ("OUT_UNORM8_PIXELS", 0, 3, 16), ("OUT_UNORM8_PIXELS", 0, 0, 17), ("OUT_UNORM8_PIXELS", 2, 2, 18),
+    ("OUT_UNORM8_PIXELS", 4, 4, 20)])
+def test_pixel_layouts_with_and_without_vector_stores(ntc, device, fmt_name, shift, row_pad, stride):
+    """A lane's four channels go out as one store only where the mip's start, row pitch and pixel stride are all
+    multiples of the group's size (8 bytes of fp16, 4 of unorm8); any other layout takes the channel-by-channel
+    stores.  Starts, pitches and strides off those multiples, one at a time and together, and a padded layout on
+    them; every byte of the buffer - the gaps keep their fill pattern - against the checker."""
+    fmt = getattr(ntc.abi, fmt_name)
+    case = cfg_case(ntc, ntc.presets.spec_cfg01(), 96, 40, 3, 16, fmt, seed=77, scale_log2_range=ACTIVE, pixel_stride=stride)
+    cursor = shift
+    for d in case.mips:                                    # re-place the mips: shifted starts, padded rows
+        d.outOffset, d.outRowPitch = cursor, d.width * stride + row_pad
+        cursor = ((cursor + d.height * d.outRowPitch + 15) & ~15) + shift
+    case.output_bytes = cursor + 16
+    expected, got = run_both(device, case)
+    assert_equal_bytes(expected, got, f"{fmt_name} start {shift} pad {row_pad} stride {stride}")
+
+
 def test_decode_is_idempotent_and_timed_variant_matches(ntc, device):
     case = cfg_case(ntc, ntc.presets.spec_cfg01(), 320, 200, 4, 16, ntc.abi.OUT_UNORM8_PIXELS, seed=21, scale_log2_range=ACTIVE)
     dset = case.device_set(device)
