@@ -129,8 +129,9 @@ __device__ __forceinline__ int32_t fp8_times_512(uint32_t byte)
 
 // Plane p of an e4m3 weight as an fp16 value: bits [7p, 7p+7) (the top plane: the rest) of |512 w|, with w's
 // sign, in units of 2^(7p - 9).
-__device__ __forceinline__ _Float16 plane_value(int32_t w512, int plane)
+__device__ __forceinline__ _Float16 plane_value(int32_t w512, int plane, bool whole = false)
 {
+    if (whole) return _Float16(float(w512) * 0x1p-9f);       // the weight itself: every e4m3 value is a half
     int32_t const mag = w512 < 0 ? -w512 : w512;
     int32_t const bits = plane == 2 ? mag >> 14 : (mag >> (7 * plane)) & 127;
     float const unit = plane == 0 ? 0x1p-9f : (plane == 1 ? 0x1p-2f : 0x1p5f);
@@ -140,11 +141,12 @@ __device__ __forceinline__ _Float16 plane_value(int32_t w512, int plane)
 
 // Stores the 8 (or 4) halves of one lane of an A block: weights W[row][k[e]] of one plane.
 template <class V>
-__device__ __forceinline__ void stage_plane_halves(uint32_t* dst, uint8_t const* __restrict__ matrix, int in, int row, int const* k, int count, int plane)
+__device__ __forceinline__ void stage_plane_halves(uint32_t* dst, uint8_t const* __restrict__ matrix, int in, int row, int const* k, int count, int plane,
+                                                   bool whole)
 {
     for (int e = 0; e < count; e += 2) {
-        _Float16 const a = plane_value(fp8_times_512(matrix[row * in + k[e]]), plane);
-        _Float16 const b = plane_value(fp8_times_512(matrix[row * in + k[e + 1]]), plane);
+        _Float16 const a = plane_value(fp8_times_512(matrix[row * in + k[e]]), plane, whole);
+        _Float16 const b = plane_value(fp8_times_512(matrix[row * in + k[e + 1]]), plane, whole);
         v2h const h = { a, b };
         dst[e >> 1] = __builtin_bit_cast(uint32_t, h);
     }
@@ -154,15 +156,25 @@ __device__ __forceinline__ void stage_plane_halves(uint32_t* dst, uint8_t const*
 // natural order (lane (i, kg) of a block of 32 holds inputs 8kg..8kg+7, of a block of 16 inputs 32+4kg..+3);
 // layers 1..3 take theirs in the order the previous layer's result registers hold them: lane (i, kg) of the
 // block for input tiles (2p, 2p+1) holds inputs 16*(2p + e/4) + 4kg + e%4, e = 0..7.
-// Returns a mask: bit l set when hidden layer l needs the general evaluation (three planes, both clamps of the
-// activation), i.e. when some weight of it has a non-zero top plane (|w| >= 32) or some bias is not a finite
-// half of magnitude <= 57344.  The other layers (every layer of a trained network) are "tame": two planes, and
-// since |sum| <= 64 * 31.75 * 3 = 6096 their outputs stay below 63440 + rounding < 65520, finite as halves.
+// Returns the layers' modes.  Bit l is set when hidden layer l needs the general evaluation (three planes, both
+// clamps of the activation), i.e. when some weight of it has a non-zero top plane (|w| >= 32) or some bias is not
+// a finite half of magnitude <= 57344.  The other layers (every layer of a trained network) are "tame": two
+// planes, and since |sum| <= 64 * 31.75 * 3 = 6096 their outputs stay below 63440 + rounding < 65520, finite as
+// halves.  Bit 4 + l is set when a tame layer needs ONE plane only, the weights themselves (stored in plane 0's
+// place): when for every output channel  sum_k |512 w_k| * 1536 < 2^24.  Inputs are at most 3 in magnitude
+// (1536 units of 2^-9), every product is a multiple of 2^-18, so every partial sum of a channel's dot product, in
+// any order, is then a multiple of 2^-18 below 2^24 of them: exact in fp32.  The sums of the planes are such
+// partial sums and so are (s2 + s1) and ((s2 + s1) + s0): the three-part evaluation the contract prescribes
+// performs no rounding before the bias is added, and one matrix-instruction chain over the whole weights gives
+// the same bits with half the matrix instructions and one addition less per activation.
+constexpr int32_t kOnePlaneLimit = ((1 << 24) - 1) / 1536;   // largest sum_k |512 w_k| with sum * 1536 < 2^24: 10922
+constexpr int kOnePlaneShift = 4;
+
 template <class V>
 __device__ int stage_fp8_weights(Fp8Lds& lds, uint8_t const* __restrict__ blob)
 {
     int const tid = threadIdx.x;
-    int topMask = 0;
+    int topMask = 0, oneMask = 0;
     {
         constexpr int first[3] = { 0, V::W1_OFF, V::W2_OFF }, count[3] = { V::W1_OFF, V::W2_OFF - V::W1_OFF, V::W3_OFF - V::W2_OFF };
 #pragma unroll
@@ -175,6 +187,17 @@ __device__ int stage_fp8_weights(Fp8Lds& lds, uint8_t const* __restrict__ blob)
             constexpr int firstBias[3] = { 0, V::H0, V::H0 + V::H1 }, biases[3] = { V::H0, V::H1, V::H2 };
             if (tid < biases[l]) any |= (reinterpret_cast<uint16_t const*>(blob + V::BIAS_OFF)[firstBias[l] + tid] & 0x7fffu) > 0x7b00u;
             if (__syncthreads_or(any)) topMask |= 1 << l;
+            constexpr int rows[3] = { V::H0, V::H1, V::H2 }, ins[3] = { V::IN, V::H0, V::H1 };
+            int over = 0;
+            if (tid < rows[l]) {
+                int32_t sum = 0;
+                for (int k = 0; k < ins[l]; ++k) {
+                    int32_t const w = fp8_times_512(blob[first[l] + tid * ins[l] + k]);
+                    sum += w < 0 ? -w : w;
+                }
+                over = sum > kOnePlaneLimit;
+            }
+            if (!__syncthreads_or(over) && !(topMask & (1 << l))) oneMask |= 1 << l;
         }
     }
     // biases of the hidden layers (fp16 in the blob), scale and bias of the output layer
@@ -194,8 +217,9 @@ __device__ int stage_fp8_weights(Fp8Lds& lds, uint8_t const* __restrict__ blob)
         int k32[8], k16[4];
         for (int q = 0; q < 8; ++q) k32[q] = 8 * kg + q;
         for (int q = 0; q < 4; ++q) k16[q] = 32 + 4 * kg + q;
-        stage_plane_halves<V>(reinterpret_cast<uint32_t*>(&lds.w0[p][t][lane]), blob, V::IN, 16 * t + i, k32, 8, p);
-        stage_plane_halves<V>(reinterpret_cast<uint32_t*>(&lds.w0[p][t][64]) + 2 * lane, blob, V::IN, 16 * t + i, k16, 4, p);
+        bool const whole = p == 0 && (oneMask & 1);
+        stage_plane_halves<V>(reinterpret_cast<uint32_t*>(&lds.w0[p][t][lane]), blob, V::IN, 16 * t + i, k32, 8, p, whole);
+        stage_plane_halves<V>(reinterpret_cast<uint32_t*>(&lds.w0[p][t][64]) + 2 * lane, blob, V::IN, 16 * t + i, k16, 4, p, whole);
     }
     // layer 1: 64 inputs = two blocks of 32
     for (int e = tid; e < 3 * V::T1 * 2 * 64; e += V::THREADS) {
@@ -203,7 +227,7 @@ __device__ int stage_fp8_weights(Fp8Lds& lds, uint8_t const* __restrict__ blob)
         int const i = lane & 15, kg = lane >> 4;
         int k[8];
         for (int q = 0; q < 8; ++q) k[q] = 16 * (2 * pair + q / 4) + 4 * kg + q % 4;
-        stage_plane_halves<V>(reinterpret_cast<uint32_t*>(&lds.w1[p][t][pair * 64 + lane]), blob + V::W1_OFF, V::H0, 16 * t + i, k, 8, p);
+        stage_plane_halves<V>(reinterpret_cast<uint32_t*>(&lds.w1[p][t][pair * 64 + lane]), blob + V::W1_OFF, V::H0, 16 * t + i, k, 8, p, p == 0 && (oneMask & 2));
     }
     // layer 2: 48 inputs = one block of 32 and one of 16
     for (int e = tid; e < 3 * V::T2 * 64; e += V::THREADS) {
@@ -212,8 +236,9 @@ __device__ int stage_fp8_weights(Fp8Lds& lds, uint8_t const* __restrict__ blob)
         int k32[8], k16[4];
         for (int q = 0; q < 8; ++q) k32[q] = 16 * (q / 4) + 4 * kg + q % 4;
         for (int q = 0; q < 4; ++q) k16[q] = 32 + 4 * kg + q;
-        stage_plane_halves<V>(reinterpret_cast<uint32_t*>(&lds.w2[p][t][lane]), blob + V::W2_OFF, V::H1, 16 * t + i, k32, 8, p);
-        stage_plane_halves<V>(reinterpret_cast<uint32_t*>(&lds.w2[p][t][64]) + 2 * lane, blob + V::W2_OFF, V::H1, 16 * t + i, k16, 4, p);
+        bool const whole = p == 0 && (oneMask & 4);
+        stage_plane_halves<V>(reinterpret_cast<uint32_t*>(&lds.w2[p][t][lane]), blob + V::W2_OFF, V::H1, 16 * t + i, k32, 8, p, whole);
+        stage_plane_halves<V>(reinterpret_cast<uint32_t*>(&lds.w2[p][t][64]) + 2 * lane, blob + V::W2_OFF, V::H1, 16 * t + i, k16, 4, p, whole);
     }
     // output layer: int8 weights as halves, 32 inputs = one block
     if (tid < 64) {
@@ -226,7 +251,7 @@ __device__ int stage_fp8_weights(Fp8Lds& lds, uint8_t const* __restrict__ blob)
             dst[q >> 1] = __builtin_bit_cast(uint32_t, h);
         }
     }
-    return topMask;
+    return topMask | (oneMask << kOnePlaneShift);
 }
 
 // The 48 inputs of one texel as 24 dwords of e4m3-rounded halves (NtcPrepareNetworkInputsInternal_FP16,
@@ -444,22 +469,24 @@ __device__ void build_fp8_feature_lut(Fp8Lds& lds)
 
 // One hidden layer's epilogue for the four channels a lane holds of one texel: sums of the three planes ->
 // layer output -> activation -> the next layer's inputs (two dwords of halves).
-// With TOP_PLANE false the layer is tame (see stage_fp8_weights): the top plane of its weights is all zero,
+// With PLANES < 3 the layer is tame (see stage_fp8_weights): the top plane of its weights is all zero,
 // s2 = +0 and (s2 + s1) = s1 exactly (a plane's sum is never -0: its accumulator starts at +0), so the first
-// addition is left out; and its outputs are finite, so the activation's lower clamp is left out too.
-template <bool LAST_HIDDEN, bool TOP_PLANE>
+// addition is left out; and its outputs are finite, so the activation's lower clamp is left out too.  With
+// PLANES == 1, s0 is the sum over the whole weights, which is what ((s2 + s1) + s0) comes to there without rounding.
+template <bool LAST_HIDDEN, int PLANES>
 __device__ __forceinline__ void fp8_epilogue(v4f s2, v4f s1, v4f s0, v4f bias, uint32_t (&out)[2])
 {
     float r[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        float a = TOP_PLANE ? s2[i] + s1[i] : s1[i];
-        a = a + s0[i];
+        float a = s0[i];
+        if (PLANES == 3)      a = (s2[i] + s1[i]) + s0[i];
+        else if (PLANES == 2) a = s1[i] + s0[i];
         r[i] = a + bias[i];
     }
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-        uint32_t const y = hgelu_pk<TOP_PLANE>(halves_rne(r[2 * h], r[2 * h + 1]));
+        uint32_t const y = hgelu_pk<PLANES == 3>(halves_rne(r[2 * h], r[2 * h + 1]));
         out[h] = LAST_HIDDEN ? quantize_int8_pk(y) : round_e4m3_pk(y);
     }
 }
@@ -494,7 +521,7 @@ __device__ __forceinline__ void mfma32_as_two_16(uint4 const& a, uint4 const (&x
     mfma16(make_uint2(a.z, a.w), hi, acc);
 }
 
-// Hidden layers.  PLANES = 3, or 2 for a tame layer (see stage_fp8_weights).
+// Hidden layers.  PLANES = 3, 2 for a tame layer, 1 where the whole weights sum exactly (see stage_fp8_weights).
 template <int NK32, bool HAS16>
 struct TileOperands { uint4 a32[3][NK32]; uint2 a16[3]; v4f bias; };     // one output tile's weight operands and bias
 
@@ -531,7 +558,7 @@ __device__ __forceinline__ void fp8_hidden_layer(Load&& load, uint4 const (&B32)
             if (HAS16) mfma16(o.a16[p], B16, acc[p]);
         }
 #pragma unroll
-        for (int b = 0; b < 4; ++b) fp8_epilogue<LAST_HIDDEN, PLANES == 3>(acc[2][b], acc[1][b], acc[0][b], o.bias, H[b][t]);
+        for (int b = 0; b < 4; ++b) fp8_epilogue<LAST_HIDDEN, PLANES>(acc[2][b], acc[1][b], acc[0][b], o.bias, H[b][t]);
     }
 }
 
@@ -596,11 +623,11 @@ __device__ __forceinline__ void fp8_layer2(Fp8Lds const& lds, int lane, uint32_t
     }, B32, B16, H);
 }
 
-// The FP8 network for the 64 texels of one wave.  `in` is the lane's own texel; `topMask` (uniform) says which
-// hidden layers need the general evaluation.  On return D[b] holds, for lane (j, g), the int32 accumulators of
+// The FP8 network for the 64 texels of one wave.  `in` is the lane's own texel; `modes` (uniform) holds the hidden
+// layers' modes as stage_fp8_weights returns them.  On return D[b] holds, for lane (j, g), the int32 accumulators of
 // output channels 4g..4g+3 of texel 16b + j, and S their scales.
 template <class V>
-__device__ __forceinline__ void mlp_forward_fp8(Fp8Lds& lds, int wave, int lane, int topMask, uint32_t const (&in)[24], v4i (&D)[4], v4f& S)
+__device__ __forceinline__ void mlp_forward_fp8(Fp8Lds& lds, int wave, int lane, int modes, uint32_t const (&in)[24], v4i (&D)[4], v4f& S)
 {
     int const j = lane & 15, g = lane >> 4;
     // transpose: lane = texel -> lane (j, kg) holds inputs 8kg..8kg+7 (block of 32) and 32+4kg..+3 (block of 16)
@@ -623,9 +650,16 @@ __device__ __forceinline__ void mlp_forward_fp8(Fp8Lds& lds, int wave, int lane,
     __builtin_amdgcn_wave_barrier();
 
     uint32_t Ha[4][4][2], Hb[4][4][2];                       // [texel block][tile of 16 channels][2 dwords = 4 halves]
-    if (topMask & 1) fp8_layer0<V, 3>(lds, lane, X32, X16, Ha); else fp8_layer0<V, 2>(lds, lane, X32, X16, Ha);   // 48 -> 64
-    if (topMask & 2) fp8_layer1<V, 3>(lds, lane, Ha, Hb);      else fp8_layer1<V, 2>(lds, lane, Ha, Hb);           // 64 -> 48
-    if (topMask & 4) fp8_layer2<V, 3>(lds, lane, Hb, Ha);      else fp8_layer2<V, 2>(lds, lane, Hb, Ha);           // 48 -> 32
+    int const one = modes >> kOnePlaneShift;
+    if (one & 1)          fp8_layer0<V, 1>(lds, lane, X32, X16, Ha);                                               // 48 -> 64
+    else if (modes & 1) fp8_layer0<V, 3>(lds, lane, X32, X16, Ha);
+    else                  fp8_layer0<V, 2>(lds, lane, X32, X16, Ha);
+    if (one & 2)          fp8_layer1<V, 1>(lds, lane, Ha, Hb);                                                     // 64 -> 48
+    else if (modes & 2) fp8_layer1<V, 3>(lds, lane, Ha, Hb);
+    else                  fp8_layer1<V, 2>(lds, lane, Ha, Hb);
+    if (one & 4)          fp8_layer2<V, 1>(lds, lane, Hb, Ha);                                                     // 48 -> 32
+    else if (modes & 4) fp8_layer2<V, 3>(lds, lane, Hb, Ha);
+    else                  fp8_layer2<V, 2>(lds, lane, Hb, Ha);
     // output layer: 32 -> 16, exact: |sum W q| <= 32 * 127 * 128 < 2^24
     {
         v4f const zero = { 0.f, 0.f, 0.f, 0.f };
@@ -670,7 +704,7 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     build_fp8_feature_lut(lds);
     __syncthreads();
 
-    int topMask = 7;                                         // uniform: hidden layers that need the general evaluation
+    int modes = 7;                                           // uniform: the hidden layers' modes (stage_fp8_weights)
 
     // One wave tile: the 16 x 4 texels of this wave in tile (tileX, tileY) of mip m.
     auto decode_wave_tile = [&](RunMip const& m, int tileX, int tileY) __attribute__((always_inline)) {
@@ -689,7 +723,7 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
         }
         v4i D[4];
         v4f S;
-        mlp_forward_fp8<V>(lds, wave, lane, topMask, in, D, S);
+        mlp_forward_fp8<V>(lds, wave, lane, modes, in, D, S);
         if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)      store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, x0 + j, y0, 4 * g);
         else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)       store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
         else                                                       store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
@@ -703,7 +737,7 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
         for (int k = entry + 1; k < numMips && mips[k].tileStart < tileEnd; ++k)
             if (mips[k].weights != blob) { segEnd = mips[k].tileStart; break; }
         if (segBegin != tileBegin) __syncthreads();          // every wave has left the previous segment's weights
-        topMask = stage_fp8_weights<V>(lds, blob);
+        modes = stage_fp8_weights<V>(lds, blob);
         __syncthreads();
 
         int const part = (segEnd - segBegin + V::GROUP - 1) / V::GROUP;
@@ -753,7 +787,7 @@ query_fp8_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* _
 
     build_fp8_posenc_table(lds);
     build_fp8_feature_lut(lds);
-    int const topMask = stage_fp8_weights<V>(lds, mips[0].weights);
+    int const modes = stage_fp8_weights<V>(lds, mips[0].weights);
     __syncthreads();
 
     uint64_t const numBlocks = (numQueries + V::THREADS - 1) / V::THREADS;
@@ -779,7 +813,7 @@ query_fp8_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* _
         }
         v4i D[4];
         v4f S;
-        mlp_forward_fp8<V>(lds, wave, lane, topMask, in, D, S);
+        mlp_forward_fp8<V>(lds, wave, lane, modes, in, D, S);
 
         // lane (j, g) holds channels 4g..4g+3 of query q0 + 16b + j; validity travels by shuffle
 #pragma unroll

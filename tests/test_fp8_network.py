@@ -195,6 +195,48 @@ def test_gpu_matrix_instruction_is_exact_on_weight_planes(ntc, device, depth):
             assert np.array_equal(d.astype(np.float64), a @ b), (plane, trial)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("depth", [16, 32])
+def test_gpu_matrix_instruction_is_exact_on_whole_weights_within_the_one_plane_limit(ntc, device, depth):
+    """What lets a layer run on one plane, the e4m3 weights themselves: while sum |512 w| * 1536 stays below 2^24
+    for a channel, every partial sum of its products with inputs of at most 3 is a multiple of 2^-18 that fp32
+    holds exactly, although the products span 2^-18 .. 2^6.  Operands of that kind - one large weight among tiny
+    ones, alternating signs, inputs at the two ends of their range - and an accumulator input that uses up the
+    rest of the limit, as the second and third instruction of a chain see it."""
+    rng = np.random.default_rng(140 + depth)
+    grid = np.unique(np.abs(nd.round_to_e4m3(np.concatenate([np.arange(8) * 2.0 ** -9] + [np.arange(8, 16) * 2.0 ** (e - 10) for e in range(1, 16)]))))
+    limit = ((1 << 24) - 1) // 1536                                          # of sum |512 w|
+    assert limit == 10922 and len(grid) == 127
+    for trial in range(60):
+        kind = trial % 4
+        if kind == 0:
+            a = rng.choice(grid[grid < 1.0], (16, depth)) * rng.choice([-1, 1], (16, depth))
+        elif kind == 1:                                                      # one large weight per channel, the rest tiny
+            a = rng.choice(grid[grid < 2.0 ** -6], (16, depth)) * rng.choice([-1, 1], (16, depth))
+            a[np.arange(16), rng.integers(0, depth, 16)] = rng.choice(grid[(grid >= 4) & (grid <= 8)], 16)
+        elif kind == 2:                                                      # alternating signs: large sums cancel
+            a = rng.choice(grid[grid < 0.6], (16, depth)) * np.where(np.arange(depth) % 2 == 0, 1, -1)
+        else:
+            a = rng.choice(grid[grid < 1.3], (16, depth)) * rng.choice([-1, 1], (16, depth))
+        for r in range(16):                                                  # this instruction takes at most half of the limit
+            while np.abs(a[r] * 512).sum() > limit // 2:
+                a[r, rng.integers(0, depth)] = 0
+        b = nd.round_to_e4m3(rng.uniform(-3.0, 3.0, (depth, 16)))
+        if trial % 3 == 0:
+            b = np.where(rng.random((depth, 16)) < 0.5, 2.0 ** -9, 3.0) * rng.choice([-1, 1], (depth, 16))
+        room = (limit - limit // 2) * 1536                                   # the accumulator input: the rest of it
+        c = rng.integers(-room, room + 1, (16, 16)).astype(np.float64) * 2.0 ** -18
+        if trial == 1:
+            a[:], b[:], c[:] = 0, 3.0, room * 2.0 ** -18                     # everything at the limit, one sign
+            a[:, :6] = [8.0, 2.0, 0.5, 0.125, 0.03125, 5.0 / 512]            # 512 w = 4096 + 1024 + 256 + 64 + 16 + 5 = 5461 = limit // 2
+        ah, bh, cf = a.astype(np.float16), b.astype(np.float16), c.astype(np.float32)
+        assert np.array_equal(ah.astype(np.float64), a) and np.array_equal(bh.astype(np.float64), b) and np.array_equal(cf.astype(np.float64), c)
+        assert (np.abs(a * 512).sum(axis=1) <= limit // 2).all()
+        d = np.zeros((16, 16), dtype=np.float32)
+        ntc.abi.check(device.lib.ntc_hip_selftest_mfma_f16(ah.ctypes.data, bh.ctypes.data, cf.ctypes.data, d.ctypes.data, depth))
+        assert np.array_equal(d.astype(np.float64), a @ b + c), trial
+
+
 def run_both(device, case):
     host = case.host_set()
     host.decode(threads=8)
@@ -240,6 +282,48 @@ def test_gpu_fp8_decode_with_large_weights_in_some_layers(ntc, device, sigmas):
     case = fp8_case(ntc, 16, 128, 64, 8, 2, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=31, weight_sigma=sigmas, bias_sigma=1.0)
     expected, got = run_both(device, case)
     assert first_mismatch(expected, got) is None, sigmas
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("sigmas", [(1.5, 1.5, 1.5), (0.35, 1.5, 300.0), (1.5, 300.0, 0.35), (300.0, 0.35, 1.5), (0.1, 0.1, 0.1)])
+def test_gpu_fp8_decode_with_one_two_and_three_planes_in_some_layers(ntc, device, sigmas):
+    """How many weight planes a hidden layer's matrix instructions go through is decided layer by layer from its
+    weights: one where sum |w| of every channel is small enough for the whole dot product to be exact in fp32
+    (sigma 0.35 and below here), two while all weights stay below 32 (sigma 1.5: sums of 30 and more), else three.
+    The bytes must not depend on it."""
+    case = fp8_case(ntc, 16, 128, 64, 8, 2, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=47, weight_sigma=sigmas, bias_sigma=1.0)
+    spec = ntc.presets.spec_ref092_fp8(16)
+    layout = ntc.synth.weight_layout(spec)
+    for layer, sigma in enumerate(sigmas):                                   # the networks are what the test says they are
+        n_in, n_out = spec.layer_inputs(layer), spec.layer_outputs(layer)
+        w512 = np.abs(nd.e4m3_times_512(case.weights[layout.weightOffset[layer]:layout.weightOffset[layer] + n_in * n_out])).reshape(n_out, n_in)
+        planes = 3 if w512.max() >= 32 * 512 else (2 if w512.sum(axis=1).max() > 10922 else 1)
+        assert planes == {300.0: 3, 1.5: 2, 0.35: 1, 0.1: 1}[sigma], (layer, sigma, planes)
+    expected, got = run_both(device, case)
+    assert first_mismatch(expected, got) is None, sigmas
+    assert len(np.unique(got.view(np.uint16))) > 500
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("layer", [0, 1, 2])
+def test_gpu_fp8_decode_at_the_one_plane_limit(ntc, device, layer):
+    """One channel of one hidden layer with sum |512 w| = 10922 (the largest sum whose products with inputs of 3
+    stay below 2^24 units of 2^-18: one plane) and with 10923 (two planes), the large weights on the channel's
+    first inputs; both sides of the limit give the checker's bytes."""
+    spec = ntc.presets.spec_ref092_fp8(16)
+    layout = ntc.synth.weight_layout(spec)
+    n_in, n_out = spec.layer_inputs(layer), spec.layer_outputs(layer)
+    for last in (10, 11):                                                    # 7168 + 3584 + 160 + 10 = 10922
+        case = fp8_case(ntc, 16, 64, 64, 4, 2, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=300 + layer, weight_sigma=0.1, bias_sigma=0.5)
+        w = case.weights[layout.weightOffset[layer]:layout.weightOffset[layer] + n_in * n_out].reshape(n_out, n_in)
+        row = np.zeros(n_in)
+        row[:4] = np.array([7168, -3584, 160, last]) / 512.0
+        w[9] = ntc.synth.e4m3_encode(row)
+        assert np.abs(nd.e4m3_times_512(w[9])).sum() == 10912 + last
+        assert np.abs(nd.e4m3_times_512(w.reshape(-1))).reshape(n_out, n_in).sum(axis=1).max() == 10912 + last
+        expected, got = run_both(device, case)
+        assert first_mismatch(expected, got) is None, (layer, last)
+        assert len(np.unique(got.view(np.uint16))) > 500
 
 
 @pytest.mark.gpu
