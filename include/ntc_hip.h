@@ -130,7 +130,7 @@ typedef struct NtcHipMipDesc {
     int32_t  hrWidth, hrHeight;      /* highResLatentWidth / Height                     */
     int32_t  lrWidth, lrHeight;      /* lowResLatentWidth / Height                      */
     float    positionScale;          /* src/TextureSet.cpp:460                          */
-    float    positionLod;            /* src/TextureSet.cpp:461                          */
+    float    positionLod;            /* src/TextureSet.cpp:461; FP8 network: |lod| <= 3 */
     uint64_t hrOffset;               /* byte offset of the grid's first u16 layer in `latents` */
     uint64_t lrOffset;
     uint64_t outOffset;              /* byte offset of this mip in `output`             */

@@ -308,6 +308,12 @@ int build_table(NtcHipTextureSet const* sets, int32_t numSets, std::vector<DevMi
                 return NTC_HIP_ERR_INVALID_ARG;
             }
             if ((d.hrOffset & 1u) || (d.lrOffset & 1u)) { set_error("ntc_hip_decode: set %d mip %d: latent offsets must be even.", s, m); return NTC_HIP_ERR_INVALID_ARG; }
+            // The FP8 network's exact sums are proven for inputs of at most 3 in magnitude; features and positional
+            // encoding lie in [-1, 1], the level-of-detail input is the caller's (the reference's own: [-1, 1]).
+            if (set.spec.weightType == NTC_HIP_WEIGHTS_FP8 && !(std::fabs(d.positionLod) <= 3.f)) {
+                set_error("ntc_hip_decode: set %d mip %d: positionLod %g is outside [-3, 3] (FP8 network).", s, m, double(d.positionLod));
+                return NTC_HIP_ERR_INVALID_ARG;
+            }
             if (forQueries) {
                 // no per-mip output
             } else if (set.outputFormat == NTC_HIP_OUT_FP16_PLANAR_PAIRS) {

@@ -327,6 +327,33 @@ def test_gpu_fp8_decode_at_the_one_plane_limit(ntc, device, layer):
 
 
 @pytest.mark.gpu
+def test_gpu_fp8_level_of_detail_input_up_to_three(ntc, device):
+    """The exactness of the layer sums is proven for inputs of at most 3 in magnitude.  Features and positional
+    encoding lie in [-1, 1]; the level-of-detail input comes from the caller's descriptor: +-3 decodes to the
+    checker's bytes (layer 0 on one plane, its largest channel sum just inside the limit), anything beyond - and
+    a NaN - is refused."""
+    spec = ntc.presets.spec_ref092_fp8(16)
+    layout = ntc.synth.weight_layout(spec)
+    for lod in (3.0, -3.0, 2.75):
+        case = fp8_case(ntc, 16, 64, 64, 3, 2, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=71, weight_sigma=0.1, bias_sigma=0.5)
+        w = case.weights[layout.weightOffset[0]:layout.weightOffset[0] + 48 * 64].reshape(64, 48)
+        row = np.zeros(48)
+        row[44:46] = np.array([7168, 3584]) / 512.0                          # the two level-of-detail inputs
+        row[:2] = np.array([160, 10]) / 512.0                                # sum |512 w| = 10922
+        w[3] = ntc.synth.e4m3_encode(row)
+        for d in case.mips:
+            d.positionLod = lod
+        expected, got = run_both(device, case)
+        assert first_mismatch(expected, got) is None, lod
+    for lod in (3.0001, -4.0, float("nan"), float("inf")):
+        case = fp8_case(ntc, 16, 64, 64, 3, 2, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=71)
+        case.mips[1].positionLod = lod
+        with pytest.raises(ntc.NtcHipError) as e:
+            device.decode([case.device_set(device)])
+        assert e.value.code == ntc.abi.ERR_INVALID_ARG and "positionLod" in e.value.message, lod
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("layer", [0, 1, 2])
 def test_gpu_fp8_decode_with_biases_at_and_beyond_the_finite_range(ntc, device, layer):
     """A hidden layer with small weights and biases of at most 57344 in magnitude cannot leave the finite halves
