@@ -166,6 +166,9 @@ def main():
     ap.add_argument("--format", choices=["fp16", "unorm8"], default=None)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="time budget of the CPU-baseline sample")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--fp8-weight-sigma", type=float, default=0.35,
+                    help="FP8-network workloads: spread of the hidden-layer weights (synth.make_fp8_weights); 0.35 lets every "
+                         "layer run on one weight plane, 1.5 needs two, 300 three")
     ap.add_argument("--file-order-latents", action="store_true",
                     help="cfg4: gather from the grids as the file stores them instead of the query-ordered copy")
     args = ap.parse_args()
@@ -216,7 +219,7 @@ def main():
         size = args.size or 4096
         spec = P.spec_ref092_fp8(16)
         mips, latent_bytes = P.mips_ref092(spec, size, size, P.full_mip_count(size, size), 2)
-        cases = [Case(ntc, spec, mips, latent_bytes, 16, fmt, seed=5, weights=ntc.synth.make_fp8_weights(spec, 6))]
+        cases = [Case(ntc, spec, mips, latent_bytes, 16, fmt, seed=5, weights=ntc.synth.make_fp8_weights(spec, 6, weight_sigma=args.fp8_weight_sigma))]
         widths, channels, latent_b = (46, 64, 48, 32, 16), 16, 44738560 / 22369621.0
         what = (f"LibNTC 0.9.2 geometry with the FP8 network: {size}x{size}, full mip chain, grid scale 2, 16 features, "
                 "MLP 48(46)-64-48-32-16, e4m3 hidden layers (GenericFP8 blob)")
@@ -226,7 +229,7 @@ def main():
             from cases import Case
             spec = P.spec_ref092_fp8(16)
             mips, latent_bytes = P.mips_ref092(spec, size, size, P.full_mip_count(size, size), 2)
-            cases = [Case(ntc, spec, mips, latent_bytes, 16, fmt, seed=4, weights=ntc.synth.make_fp8_weights(spec, 6))]
+            cases = [Case(ntc, spec, mips, latent_bytes, 16, fmt, seed=4, weights=ntc.synth.make_fp8_weights(spec, 6, weight_sigma=args.fp8_weight_sigma))]
             widths, channels, latent_b = (46, 64, 48, 32, 16), 16, 0.0
         else:
             cases = [cfg_case(ntc, P.spec_cfg01(), size, size, P.full_mip_count(size, size), 16, fmt, seed=4)]

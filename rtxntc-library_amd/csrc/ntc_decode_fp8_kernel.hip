@@ -80,8 +80,15 @@ __device__ __forceinline__ uint32_t quantize_int8_pk(uint32_t yBits)
     return __builtin_bit_cast(uint32_t, z + minus1536);
 }
 
-template <int FEATURES_>
+// ONE_: the instantiation for texture sets all of whose hidden layers run on one weight plane (see
+// classify_fp8_weights): it holds one plane in LDS instead of three, which leaves room for the transposition
+// buffers of sixteen waves, and its network has one form per layer, which fits the 128 registers four waves per
+// SIMD leave a lane (108 used; the general form needs 150).  The two instantiations are launched one after the
+// other; each decodes the sets that are its own.
+template <int FEATURES_, bool ONE_ = false>
 struct Fp8Variant {
+    static constexpr bool ONE = ONE_;
+    static constexpr int HELD = ONE_ ? 1 : 3;                // weight planes kept in LDS
     static constexpr int F = FEATURES_;                      // features stored per cell of either grid (slots: 16)
     static constexpr int IN = 48, H0 = 64, H1 = 48, H2 = 32, OUT = 16;      // InferenceConstants.h:28-40
     static constexpr int T0 = H0 / 16, T1 = H1 / 16, T2 = H2 / 16;
@@ -90,23 +97,24 @@ struct Fp8Variant {
     static constexpr int WEIGHT_BYTES = W3_OFF + H2 * OUT;
     // src/WeightLayout.cpp:249-262: fp16 biases of the three e4m3 layers, then scale and bias of the output layer
     static constexpr int BIAS_OFF = WEIGHT_BYTES, SCALE3_OFF = BIAS_OFF + 2 * (H0 + H1 + H2), BIAS3_OFF = SCALE3_OFF + 4 * OUT;
-    // Twelve waves share one copy of the weight planes: one workgroup per CU, three waves per SIMD, working on
-    // GROUP tiles at a time.
-    static constexpr int WAVES = 12, THREADS = 64 * WAVES, GROUP = WAVES / 4;
+    // Twelve waves (sixteen with one plane) share one copy of the weight planes: one workgroup per CU, three (four)
+    // waves per SIMD, working on GROUP tiles at a time.
+    static constexpr int WAVES = ONE_ ? 16 : 12, THREADS = 64 * WAVES, GROUP = WAVES / 4;
     static constexpr int IN_STRIDE = 28;                     // dwords per texel in the transpose buffer: 24 + 4 of padding
 };
 
 // A operands in LDS, in 16-byte units.  A block for 32 inputs holds one unit per lane (8 halves), a block for
 // 16 inputs half a unit per lane (4 halves, 32 units).
-struct alignas(16) Fp8Lds {
-    uint4 w0[3][4][96];        // layer 0, inputs in their natural order: [plane][output tile][K32 block | K16 block]
-    uint4 w1[3][3][128];       // layer 1: two blocks of 32 (input-tile pairs 0-1, 2-3)
-    uint4 w2[3][2][96];        // layer 2: input-tile pair 0-1, then input tile 2
+template <int HELD, int WAVES>
+struct alignas(16) Fp8LdsT {
+    uint4 w0[HELD][4][96];     // layer 0, inputs in their natural order: [plane][output tile][K32 block | K16 block]
+    uint4 w1[HELD][3][128];    // layer 1: two blocks of 32 (input-tile pairs 0-1, 2-3)
+    uint4 w2[HELD][2][96];     // layer 2: input-tile pair 0-1, then input tile 2
     uint4 w3[64];              // output layer (int8 weights as halves): input-tile pair 0-1
     float bias[9][4][4];       // hidden layers: [output tile of layers 0..2][g][r] -> channel 16t+4g+r
     float outScale[4][4];      // output layer: [g][r]
     int32_t outBias[4][4];
-    uint32_t in[12][kWaveTexels][28];
+    uint32_t in[WAVES][kWaveTexels][28];
     // Positional encoding for every power-of-two positionScale 2^-k, k = 0..5: the entry for phase p of scale
     // 2^-k sits at index (2^k - 1) + p; dwords 0..2 hold enc(px * 2^w), dwords 3..5 enc(px * 2^w + 1/4), w = 0..2,
     // as e4m3-rounded halves in the low 16 bits (px = p * 2^-k).
@@ -115,7 +123,11 @@ struct alignas(16) Fp8Lds {
     // e4m3-rounded half of fma(float(T), (2/15) * 2^-n, -1) for T = 0 .. 15 * 2^n, n = 0, 2, 4, 6 (what square
     // power-of-two geometry produces; other n take the arithmetic).
     uint16_t featureLut[1280];
+    // classify_fp8_weights: sum |512 w| of every output channel of the three hidden layers, and the flags it gathers
+    int32_t channelSum[3][64];
+    uint32_t classFlags;
 };
+template <class V> using Fp8Lds = Fp8LdsT<V::HELD, V::WAVES>;
 __host__ __device__ constexpr int kFeatureLutBase(int n) { return n == 0 ? 0 : (n == 2 ? 16 : (n == 4 ? 77 : 318)); }   // 16 + 61 + 241 + 961 = 1279 entries
 
 // OCP e4m3 byte -> the integer 512 * value (NaN encodings decode as 0).
@@ -156,7 +168,7 @@ __device__ __forceinline__ void stage_plane_halves(uint32_t* dst, uint8_t const*
 // natural order (lane (i, kg) of a block of 32 holds inputs 8kg..8kg+7, of a block of 16 inputs 32+4kg..+3);
 // layers 1..3 take theirs in the order the previous layer's result registers hold them: lane (i, kg) of the
 // block for input tiles (2p, 2p+1) holds inputs 16*(2p + e/4) + 4kg + e%4, e = 0..7.
-// Returns the layers' modes.  Bit l is set when hidden layer l needs the general evaluation (three planes, both
+// stage_fp8_weights takes the layers' modes from classify_fp8_weights, which reads the blob only.  Bit l is set when hidden layer l needs the general evaluation (three planes, both
 // clamps of the activation), i.e. when some weight of it has a non-zero top plane (|w| >= 32) or some bias is not
 // a finite half of magnitude <= 57344.  The other layers (every layer of a trained network) are "tame": two
 // planes, and since |sum| <= 64 * 31.75 * 3 = 6096 their outputs stay below 63440 + rounding < 65520, finite as
@@ -170,36 +182,58 @@ __device__ __forceinline__ void stage_plane_halves(uint32_t* dst, uint8_t const*
 constexpr int32_t kOnePlaneLimit = ((1 << 24) - 1) / 1536;   // largest sum_k |512 w_k| with sum * 1536 < 2^24: 10922
 constexpr int kOnePlaneShift = 4;
 
+constexpr int kAllOnePlane = 7 << kOnePlaneShift;         // every hidden layer runs on one plane
+
+// Reads the blob a dword per thread (the api requires 4-byte alignment; rows of 48 or 64 bytes: a dword never
+// straddles two channels) and gathers sums and flags in LDS: every workgroup of both instantiations does this for
+// every set it meets, and the workgroups of the one that passes over the set do nothing else.
 template <class V>
-__device__ int stage_fp8_weights(Fp8Lds& lds, uint8_t const* __restrict__ blob)
+__device__ int classify_fp8_weights(Fp8Lds<V>& lds, uint8_t const* __restrict__ blob)
 {
     int const tid = threadIdx.x;
-    int topMask = 0, oneMask = 0;
-    {
-        constexpr int first[3] = { 0, V::W1_OFF, V::W2_OFF }, count[3] = { V::W1_OFF, V::W2_OFF - V::W1_OFF, V::W3_OFF - V::W2_OFF };
+    constexpr int rows[3] = { V::H0, V::H1, V::H2 }, ins[3] = { V::IN, V::H0, V::H1 };
+    constexpr int dwords[3] = { V::W1_OFF / 4, (V::W2_OFF - V::W1_OFF) / 4, (V::W3_OFF - V::W2_OFF) / 4 };
+    static_assert(V::IN % 4 == 0 && V::H0 % 4 == 0 && V::H1 % 4 == 0 && V::H0 <= 64, "a dword of weights belongs to one channel");
+    if (tid == 0) lds.classFlags = 0;
+    if (tid < 192) (&lds.channelSum[0][0])[tid] = 0;
+    __syncthreads();                                         // also: every wave has left the previous set's tiles
+    for (int e = tid; e < dwords[0] + dwords[1] + dwords[2]; e += V::THREADS) {
+        int const l = e < dwords[0] ? 0 : (e < dwords[0] + dwords[1] ? 1 : 2);
+        int const d = e - (l == 0 ? 0 : (l == 1 ? dwords[0] : dwords[0] + dwords[1]));
+        uint32_t const four = reinterpret_cast<uint32_t const*>(blob)[e];      // the three matrices follow each other
+        int32_t sum = 0, top = 0;
 #pragma unroll
-        for (int l = 0; l < 3; ++l) {
-            int any = 0;
-            for (int e = tid; e < count[l]; e += V::THREADS) {
-                int32_t const w = fp8_times_512(blob[first[l] + e]);
-                any |= ((w < 0 ? -w : w) >> 14) != 0;
-            }
-            constexpr int firstBias[3] = { 0, V::H0, V::H0 + V::H1 }, biases[3] = { V::H0, V::H1, V::H2 };
-            if (tid < biases[l]) any |= (reinterpret_cast<uint16_t const*>(blob + V::BIAS_OFF)[firstBias[l] + tid] & 0x7fffu) > 0x7b00u;
-            if (__syncthreads_or(any)) topMask |= 1 << l;
-            constexpr int rows[3] = { V::H0, V::H1, V::H2 }, ins[3] = { V::IN, V::H0, V::H1 };
-            int over = 0;
-            if (tid < rows[l]) {
-                int32_t sum = 0;
-                for (int k = 0; k < ins[l]; ++k) {
-                    int32_t const w = fp8_times_512(blob[first[l] + tid * ins[l] + k]);
-                    sum += w < 0 ? -w : w;
-                }
-                over = sum > kOnePlaneLimit;
-            }
-            if (!__syncthreads_or(over) && !(topMask & (1 << l))) oneMask |= 1 << l;
+        for (int q = 0; q < 4; ++q) {
+            int32_t const w = fp8_times_512((four >> (8 * q)) & 0xffu);
+            int32_t const mag = w < 0 ? -w : w;
+            sum += mag;
+            top |= mag >> 14;
         }
+        atomicAdd(&lds.channelSum[l][(4 * d) / ins[l]], sum);
+        if (top) atomicOr(&lds.classFlags, 1u << l);
     }
+    if (tid < V::H0 + V::H1 + V::H2) {                       // a bias that is not a finite half of at most 57344
+        int const l = tid < V::H0 ? 0 : (tid < V::H0 + V::H1 ? 1 : 2);
+        if ((reinterpret_cast<uint16_t const*>(blob + V::BIAS_OFF)[tid] & 0x7fffu) > 0x7b00u) atomicOr(&lds.classFlags, 1u << l);
+    }
+    __syncthreads();
+    if (tid < 192) {
+        int const l = tid >> 6, r = tid & 63;
+        if (r < rows[l] && lds.channelSum[l][r] > kOnePlaneLimit) atomicOr(&lds.classFlags, 16u << l);
+    }
+    __syncthreads();
+    uint32_t const flags = lds.classFlags;
+    __syncthreads();                                         // read by all before the next call clears it
+    int const topMask = int(flags & 7u);
+    int const oneMask = int(~(flags >> 4) & ~flags & 7u);
+    return topMask | (oneMask << kOnePlaneShift);
+}
+
+template <class V>
+__device__ void stage_fp8_weights(Fp8Lds<V>& lds, uint8_t const* __restrict__ blob, int modes)
+{
+    int const tid = threadIdx.x;
+    int const oneMask = modes >> kOnePlaneShift;
     // biases of the hidden layers (fp16 in the blob), scale and bias of the output layer
     for (int e = tid; e < 9 * 16; e += V::THREADS) {
         int const r = e & 3, g = (e >> 2) & 3, t = e >> 4;
@@ -211,7 +245,7 @@ __device__ int stage_fp8_weights(Fp8Lds& lds, uint8_t const* __restrict__ blob)
         lds.outBias[tid >> 2][tid & 3] = reinterpret_cast<int32_t const*>(blob + V::BIAS3_OFF)[tid];
     }
     // layer 0: (plane, tile, lane) -> one K32 unit and half a K16 unit
-    for (int e = tid; e < 3 * V::T0 * 64; e += V::THREADS) {
+    for (int e = tid; e < V::HELD * V::T0 * 64; e += V::THREADS) {
         int const lane = e & 63, t = (e >> 6) % V::T0, p = e / (64 * V::T0);
         int const i = lane & 15, kg = lane >> 4;
         int k32[8], k16[4];
@@ -222,7 +256,7 @@ __device__ int stage_fp8_weights(Fp8Lds& lds, uint8_t const* __restrict__ blob)
         stage_plane_halves<V>(reinterpret_cast<uint32_t*>(&lds.w0[p][t][64]) + 2 * lane, blob, V::IN, 16 * t + i, k16, 4, p, whole);
     }
     // layer 1: 64 inputs = two blocks of 32
-    for (int e = tid; e < 3 * V::T1 * 2 * 64; e += V::THREADS) {
+    for (int e = tid; e < V::HELD * V::T1 * 2 * 64; e += V::THREADS) {
         int const lane = e & 63, pair = (e >> 6) & 1, t = (e >> 7) % V::T1, p = e / (128 * V::T1);
         int const i = lane & 15, kg = lane >> 4;
         int k[8];
@@ -230,7 +264,7 @@ __device__ int stage_fp8_weights(Fp8Lds& lds, uint8_t const* __restrict__ blob)
         stage_plane_halves<V>(reinterpret_cast<uint32_t*>(&lds.w1[p][t][pair * 64 + lane]), blob + V::W1_OFF, V::H0, 16 * t + i, k, 8, p, p == 0 && (oneMask & 2));
     }
     // layer 2: 48 inputs = one block of 32 and one of 16
-    for (int e = tid; e < 3 * V::T2 * 64; e += V::THREADS) {
+    for (int e = tid; e < V::HELD * V::T2 * 64; e += V::THREADS) {
         int const lane = e & 63, t = (e >> 6) % V::T2, p = e / (64 * V::T2);
         int const i = lane & 15, kg = lane >> 4;
         int k32[8], k16[4];
@@ -251,7 +285,6 @@ __device__ int stage_fp8_weights(Fp8Lds& lds, uint8_t const* __restrict__ blob)
             dst[q >> 1] = __builtin_bit_cast(uint32_t, h);
         }
     }
-    return topMask | (oneMask << kOnePlaneShift);
 }
 
 // The 48 inputs of one texel as 24 dwords of e4m3-rounded halves (NtcPrepareNetworkInputsInternal_FP16,
@@ -375,7 +408,7 @@ __device__ __forceinline__ void fetch_latents_bricked(Mip const& m, int x, int y
 }
 
 template <class V, class Mip>
-__device__ __forceinline__ void finish_inputs_fast(Mip const& m, Fp8Lds const& lds, int x, int y, Fp8Fetch<V> const& f, uint32_t (&in)[24])
+__device__ __forceinline__ void finish_inputs_fast(Mip const& m, Fp8Lds<V> const& lds, int x, int y, Fp8Fetch<V> const& f, uint32_t (&in)[24])
 {
 #pragma unroll
     for (int i = 0; i < 24; ++i) in[i] = 0;
@@ -436,7 +469,8 @@ __device__ __forceinline__ void finish_inputs_fast(Mip const& m, Fp8Lds const& l
 }
 
 // Fills the positional table: one entry per thread, threads 0..62.
-__device__ void build_fp8_posenc_table(Fp8Lds& lds)
+template <class Lds>
+__device__ void build_fp8_posenc_table(Lds& lds)
 {
     int const t = threadIdx.x;
     if (t < 63) {
@@ -457,7 +491,8 @@ __device__ void build_fp8_posenc_table(Fp8Lds& lds)
 }
 
 // Fills the feature table with the same operations the arithmetic path applies per lane.
-__device__ void build_fp8_feature_lut(Fp8Lds& lds)
+template <class Lds>
+__device__ void build_fp8_feature_lut(Lds& lds)
 {
     for (int e = threadIdx.x; e < 1279; e += blockDim.x) {
         int const n = e < 16 ? 0 : (e < 77 ? 2 : (e < 318 ? 4 : 6));
@@ -563,7 +598,7 @@ __device__ __forceinline__ void fp8_hidden_layer(Load&& load, uint4 const (&B32)
 }
 
 template <class V, int PLANES>
-__device__ __forceinline__ void fp8_layer0(Fp8Lds const& lds, int lane, uint4 const (&X32)[4], uint2 const (&X16)[4], uint32_t (&H)[4][4][2])
+__device__ __forceinline__ void fp8_layer0(Fp8Lds<V> const& lds, int lane, uint4 const (&X32)[4], uint2 const (&X16)[4], uint32_t (&H)[4][4][2])
 {
     int const g = lane >> 4;
     uint4 B32[1][4];
@@ -580,7 +615,7 @@ __device__ __forceinline__ void fp8_layer0(Fp8Lds const& lds, int lane, uint4 co
 }
 
 template <class V, int PLANES>
-__device__ __forceinline__ void fp8_layer1(Fp8Lds const& lds, int lane, uint32_t const (&Hin)[4][4][2], uint32_t (&H)[4][4][2])
+__device__ __forceinline__ void fp8_layer1(Fp8Lds<V> const& lds, int lane, uint32_t const (&Hin)[4][4][2], uint32_t (&H)[4][4][2])
 {
     int const g = lane >> 4;
     uint4 B32[2][4];
@@ -603,7 +638,7 @@ __device__ __forceinline__ void fp8_layer1(Fp8Lds const& lds, int lane, uint32_t
 
 // layer 2: its activations are quantised to the int8 inputs of the output layer
 template <class V, int PLANES>
-__device__ __forceinline__ void fp8_layer2(Fp8Lds const& lds, int lane, uint32_t const (&Hin)[4][4][2], uint32_t (&H)[4][4][2])
+__device__ __forceinline__ void fp8_layer2(Fp8Lds<V> const& lds, int lane, uint32_t const (&Hin)[4][4][2], uint32_t (&H)[4][4][2])
 {
     int const g = lane >> 4;
     uint4 B32[1][4];
@@ -627,7 +662,7 @@ __device__ __forceinline__ void fp8_layer2(Fp8Lds const& lds, int lane, uint32_t
 // layers' modes as stage_fp8_weights returns them.  On return D[b] holds, for lane (j, g), the int32 accumulators of
 // output channels 4g..4g+3 of texel 16b + j, and S their scales.
 template <class V>
-__device__ __forceinline__ void mlp_forward_fp8(Fp8Lds& lds, int wave, int lane, int modes, uint32_t const (&in)[24], v4i (&D)[4], v4f& S)
+__device__ __forceinline__ void mlp_forward_fp8(Fp8Lds<V>& lds, int wave, int lane, int modes, uint32_t const (&in)[24], v4i (&D)[4], v4f& S)
 {
     int const j = lane & 15, g = lane >> 4;
     // transpose: lane = texel -> lane (j, kg) holds inputs 8kg..8kg+7 (block of 32) and 32+4kg..+3 (block of 16)
@@ -650,16 +685,22 @@ __device__ __forceinline__ void mlp_forward_fp8(Fp8Lds& lds, int wave, int lane,
     __builtin_amdgcn_wave_barrier();
 
     uint32_t Ha[4][4][2], Hb[4][4][2];                       // [texel block][tile of 16 channels][2 dwords = 4 halves]
-    int const one = modes >> kOnePlaneShift;
-    if (one & 1)          fp8_layer0<V, 1>(lds, lane, X32, X16, Ha);                                               // 48 -> 64
-    else if (modes & 1) fp8_layer0<V, 3>(lds, lane, X32, X16, Ha);
-    else                  fp8_layer0<V, 2>(lds, lane, X32, X16, Ha);
-    if (one & 2)          fp8_layer1<V, 1>(lds, lane, Ha, Hb);                                                     // 64 -> 48
-    else if (modes & 2) fp8_layer1<V, 3>(lds, lane, Ha, Hb);
-    else                  fp8_layer1<V, 2>(lds, lane, Ha, Hb);
-    if (one & 4)          fp8_layer2<V, 1>(lds, lane, Hb, Ha);                                                     // 48 -> 32
-    else if (modes & 4) fp8_layer2<V, 3>(lds, lane, Hb, Ha);
-    else                  fp8_layer2<V, 2>(lds, lane, Hb, Ha);
+    if constexpr (V::ONE) {
+        fp8_layer0<V, 1>(lds, lane, X32, X16, Ha);                                                                 // 48 -> 64
+        fp8_layer1<V, 1>(lds, lane, Ha, Hb);                                                                       // 64 -> 48
+        fp8_layer2<V, 1>(lds, lane, Hb, Ha);                                                                       // 48 -> 32
+    } else {
+        int const one = modes >> kOnePlaneShift;
+        if (one & 1)        fp8_layer0<V, 1>(lds, lane, X32, X16, Ha);
+        else if (modes & 1) fp8_layer0<V, 3>(lds, lane, X32, X16, Ha);
+        else                fp8_layer0<V, 2>(lds, lane, X32, X16, Ha);
+        if (one & 2)        fp8_layer1<V, 1>(lds, lane, Ha, Hb);
+        else if (modes & 2) fp8_layer1<V, 3>(lds, lane, Ha, Hb);
+        else                fp8_layer1<V, 2>(lds, lane, Ha, Hb);
+        if (one & 4)        fp8_layer2<V, 1>(lds, lane, Hb, Ha);
+        else if (modes & 4) fp8_layer2<V, 3>(lds, lane, Hb, Ha);
+        else                fp8_layer2<V, 2>(lds, lane, Hb, Ha);
+    }
     // output layer: 32 -> 16, exact: |sum W q| <= 32 * 127 * 128 < 2^24
     {
         v4f const zero = { 0.f, 0.f, 0.f, 0.f };
@@ -678,7 +719,9 @@ __device__ __forceinline__ void mlp_forward_fp8(Fp8Lds& lds, int wave, int lane,
 }
 
 // 135 KB of LDS - three planes of every hidden layer's weights, shared by the twelve waves of the one workgroup
-// a CU holds, and a transposition buffer per wave: three waves per SIMD, 168 registers per lane.
+// a CU holds, and a transposition buffer per wave: three waves per SIMD, 168 registers per lane; the one-plane
+// instantiation: one plane, sixteen waves, four per SIMD, 128 registers.  Each of the two decodes the segments
+// whose set is its own (all hidden layers on one plane, or not) and passes over the others.
 //
 // A workgroup owns a contiguous share of the tile list.  It walks that share in segments of tiles that use the
 // same weight blob (one segment, unless sets of a batch meet inside the share), and inside a segment each of its
@@ -689,7 +732,7 @@ template <class V>
 __global__ void __launch_bounds__(V::THREADS, 1)
 decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
 {
-    __shared__ Fp8Lds lds;
+    __shared__ Fp8Lds<V> lds;
     int const lane = threadIdx.x & 63;
     int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int const member = wave >> 2;                            // which quartet of the workgroup
@@ -702,7 +745,6 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
 
     build_fp8_posenc_table(lds);
     build_fp8_feature_lut(lds);
-    __syncthreads();
 
     int modes = 7;                                           // uniform: the hidden layers' modes (stage_fp8_weights)
 
@@ -736,9 +778,11 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
         int segEnd = tileEnd;
         for (int k = entry + 1; k < numMips && mips[k].tileStart < tileEnd; ++k)
             if (mips[k].weights != blob) { segEnd = mips[k].tileStart; break; }
-        if (segBegin != tileBegin) __syncthreads();          // every wave has left the previous segment's weights
-        modes = stage_fp8_weights<V>(lds, blob);
-        __syncthreads();
+        modes = classify_fp8_weights<V>(lds, blob);
+        if (((modes & kAllOnePlane) == kAllOnePlane) != V::ONE) { segBegin = segEnd; continue; }   // the other instantiation's segment
+        __syncthreads();                                     // every wave has left the previous segment's weights
+        stage_fp8_weights<V>(lds, blob, modes);
+        __syncthreads();                                     // also publishes the tables built above
 
         int const part = (segEnd - segBegin + V::GROUP - 1) / V::GROUP;
         int const myBegin = segBegin + member * part, myEnd = min(segEnd, myBegin + part);
@@ -768,7 +812,7 @@ __global__ void __launch_bounds__(V::THREADS, 1)
 query_fp8_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __restrict__ queries, uint64_t numQueries,
                  uint16_t* __restrict__ out)
 {
-    __shared__ Fp8Lds lds;
+    __shared__ Fp8Lds<V> lds;
     __shared__ QueryMip qmips[16];
     if (threadIdx.x < 16) {
         DevMip const& d = mips[min(int(threadIdx.x), numMips - 1)];
@@ -785,9 +829,11 @@ query_fp8_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* _
     int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int const j = lane & 15, g = lane >> 4;
 
+    int const modes = classify_fp8_weights<V>(lds, mips[0].weights);
+    if (((modes & kAllOnePlane) == kAllOnePlane) != V::ONE) return;      // the other instantiation's set (uniform over the grid)
     build_fp8_posenc_table(lds);
     build_fp8_feature_lut(lds);
-    int const modes = stage_fp8_weights<V>(lds, mips[0].weights);
+    stage_fp8_weights<V>(lds, mips[0].weights, modes);
     __syncthreads();
 
     uint64_t const numBlocks = (numQueries + V::THREADS - 1) / V::THREADS;
@@ -842,32 +888,41 @@ __global__ void selftest_fp8_activation_kernel(uint16_t const* __restrict__ in, 
 }
 
 using VFp8_16 = Fp8Variant<16>;
-using VFp8_12 = Fp8Variant<12>;
-using VFp8_8  = Fp8Variant<8>;
-using VFp8_4  = Fp8Variant<4>;
 
-template <class V>
+// Both instantiations, the one-plane one first; a set is decoded by the one it belongs to (decided on the device
+// from its weights), the other passes over it after reading the weights once per workgroup.
+template <int FEATURES>
 static hipError_t launch_fp8_variant(DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream)
 {
-    hipLaunchKernelGGL(decode_fp8_kernel<V>, dim3(gridSize), dim3(V::THREADS), 0, stream, mips, numMips, totalTiles);
+    using One = Fp8Variant<FEATURES, true>;
+    using Any = Fp8Variant<FEATURES, false>;
+    hipLaunchKernelGGL(decode_fp8_kernel<One>, dim3(gridSize), dim3(One::THREADS), 0, stream, mips, numMips, totalTiles);
+    hipError_t const e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(decode_fp8_kernel<Any>, dim3(gridSize), dim3(Any::THREADS), 0, stream, mips, numMips, totalTiles);
     return hipGetLastError();
 }
 
 hipError_t launch_decode_fp8(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream)
 {
     switch (variant) {
-    case NTC_HIP_VARIANT_REF16_FP8: return launch_fp8_variant<VFp8_16>(mips, numMips, totalTiles, gridSize, stream);
-    case NTC_HIP_VARIANT_REF12_FP8: return launch_fp8_variant<VFp8_12>(mips, numMips, totalTiles, gridSize, stream);
-    case NTC_HIP_VARIANT_REF8_FP8:  return launch_fp8_variant<VFp8_8>(mips, numMips, totalTiles, gridSize, stream);
-    case NTC_HIP_VARIANT_REF4_FP8:  return launch_fp8_variant<VFp8_4>(mips, numMips, totalTiles, gridSize, stream);
+    case NTC_HIP_VARIANT_REF16_FP8: return launch_fp8_variant<16>(mips, numMips, totalTiles, gridSize, stream);
+    case NTC_HIP_VARIANT_REF12_FP8: return launch_fp8_variant<12>(mips, numMips, totalTiles, gridSize, stream);
+    case NTC_HIP_VARIANT_REF8_FP8:  return launch_fp8_variant<8>(mips, numMips, totalTiles, gridSize, stream);
+    case NTC_HIP_VARIANT_REF4_FP8:  return launch_fp8_variant<4>(mips, numMips, totalTiles, gridSize, stream);
     default: return hipErrorInvalidValue;
     }
 }
 
-template <class V>
+template <int FEATURES>
 static hipError_t launch_fp8_query_variant(DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries, uint16_t* out, int gridSize, hipStream_t stream)
 {
-    hipLaunchKernelGGL(query_fp8_kernel<V>, dim3(gridSize), dim3(V::THREADS), 0, stream, mips, numMips, queries, numQueries, out);
+    using One = Fp8Variant<FEATURES, true>;
+    using Any = Fp8Variant<FEATURES, false>;
+    hipLaunchKernelGGL(query_fp8_kernel<One>, dim3(gridSize), dim3(One::THREADS), 0, stream, mips, numMips, queries, numQueries, out);
+    hipError_t const e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(query_fp8_kernel<Any>, dim3(gridSize), dim3(Any::THREADS), 0, stream, mips, numMips, queries, numQueries, out);
     return hipGetLastError();
 }
 
@@ -875,10 +930,10 @@ hipError_t launch_queries_fp8(int variant, DevMip const* mips, int numMips, DevQ
                               uint16_t* out, int gridSize, hipStream_t stream)
 {
     switch (variant) {
-    case NTC_HIP_VARIANT_REF16_FP8: return launch_fp8_query_variant<VFp8_16>(mips, numMips, queries, numQueries, out, gridSize, stream);
-    case NTC_HIP_VARIANT_REF12_FP8: return launch_fp8_query_variant<VFp8_12>(mips, numMips, queries, numQueries, out, gridSize, stream);
-    case NTC_HIP_VARIANT_REF8_FP8:  return launch_fp8_query_variant<VFp8_8>(mips, numMips, queries, numQueries, out, gridSize, stream);
-    case NTC_HIP_VARIANT_REF4_FP8:  return launch_fp8_query_variant<VFp8_4>(mips, numMips, queries, numQueries, out, gridSize, stream);
+    case NTC_HIP_VARIANT_REF16_FP8: return launch_fp8_query_variant<16>(mips, numMips, queries, numQueries, out, gridSize, stream);
+    case NTC_HIP_VARIANT_REF12_FP8: return launch_fp8_query_variant<12>(mips, numMips, queries, numQueries, out, gridSize, stream);
+    case NTC_HIP_VARIANT_REF8_FP8:  return launch_fp8_query_variant<8>(mips, numMips, queries, numQueries, out, gridSize, stream);
+    case NTC_HIP_VARIANT_REF4_FP8:  return launch_fp8_query_variant<4>(mips, numMips, queries, numQueries, out, gridSize, stream);
     default: return hipErrorInvalidValue;
     }
 }
