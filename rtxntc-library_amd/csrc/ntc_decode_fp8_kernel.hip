@@ -773,11 +773,9 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
 
     int entry = 0;
     for (int segBegin = tileBegin; segBegin < tileEnd; ) {   // uniform across the workgroup
-        while (entry + 1 < numMips && mips[entry + 1].tileStart <= segBegin) ++entry;
+        entry = table_entry_of(mips, numMips, entry, segBegin);
         uint8_t const* const blob = mips[entry].weights;
-        int segEnd = tileEnd;
-        for (int k = entry + 1; k < numMips && mips[k].tileStart < tileEnd; ++k)
-            if (mips[k].weights != blob) { segEnd = mips[k].tileStart; break; }
+        int const segEnd = segment_end(mips, numMips, entry, tileEnd, blob);
         modes = classify_fp8_weights<V>(lds, blob);
         if (((modes & kAllOnePlane) == kAllOnePlane) != V::ONE) { segBegin = segEnd; continue; }   // the other instantiation's segment
         __syncthreads();                                     // every wave has left the previous segment's weights
