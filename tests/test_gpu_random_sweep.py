@@ -49,7 +49,7 @@ def test_random_sets_and_queries_equal_checker(ntc, device, oracle, seed):
             else:
                 spec = P.spec_ref092_fp8(features)
                 mip_list, latent_bytes = P.mips_ref092(spec, w, h, mips, grid_scale)
-                sigma = rnd.choice([0.35, 0.35, 0.35, (0.35, 40.0, 0.35), 300.0])
+                sigma = rnd.choice([0.35, 0.35, 0.1, 1.5, (0.35, 1.5, 0.35), (1.5, 0.35, 300.0), (0.35, 40.0, 0.35), 300.0])   # one, two, three weight planes per layer
                 c = Case(ntc, spec, mip_list, latent_bytes, rnd.randint(1, 16), fmt, s, weights=ntc.synth.make_fp8_weights(spec, s + 1, weight_sigma=sigma))
             cases.append(c)
             described.append((w, h, mips, c.num_channels))
