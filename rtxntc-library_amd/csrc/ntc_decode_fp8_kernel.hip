@@ -183,6 +183,11 @@ constexpr int32_t kOnePlaneLimit = ((1 << 24) - 1) / 1536;   // largest sum_k |5
 constexpr int kOnePlaneShift = 4;
 
 constexpr int kAllOnePlane = 7 << kOnePlaneShift;         // every hidden layer runs on one plane
+// Bit 8: no output can come near the fp16 overflow threshold, so stores may skip that check.  The output layer's
+// int32 accumulator is at most 32 * 127 * 128 = 520192 in magnitude before the bias; bounded means
+// (|bias| + 520192) * |scale| < 60000 for every channel (no wrap of the int32 sum either: that is far below 2^31
+// unless the scale is tiny, and then |bias| itself must be checked).
+constexpr int kFp8OutputsBounded = 1 << 8;
 
 // Reads the blob a dword per thread (the api requires 4-byte alignment; rows of 48 or 64 bytes: a dword never
 // straddles two channels) and gathers sums and flags in LDS: every workgroup of both instantiations does this for
@@ -212,6 +217,11 @@ __device__ int classify_fp8_weights(Fp8Lds<V>& lds, uint8_t const* __restrict__ 
         atomicAdd(&lds.channelSum[l][(4 * d) / ins[l]], sum);
         if (top) atomicOr(&lds.classFlags, 1u << l);
     }
+    if (tid < V::OUT) {
+        float const bias = fabsf(float(reinterpret_cast<int32_t const*>(blob + V::BIAS3_OFF)[tid]));
+        float const scale = fabsf(reinterpret_cast<float const*>(blob + V::SCALE3_OFF)[tid]);
+        if (!((bias + 520192.f) * scale < 60000.f) || !(bias < 2.0e9f)) atomicOr(&lds.classFlags, 1u << 8);
+    }
     if (tid < V::H0 + V::H1 + V::H2) {                       // a bias that is not a finite half of at most 57344
         int const l = tid < V::H0 ? 0 : (tid < V::H0 + V::H1 ? 1 : 2);
         if ((reinterpret_cast<uint16_t const*>(blob + V::BIAS_OFF)[tid] & 0x7fffu) > 0x7b00u) atomicOr(&lds.classFlags, 1u << l);
@@ -226,7 +236,7 @@ __device__ int classify_fp8_weights(Fp8Lds<V>& lds, uint8_t const* __restrict__ 
     __syncthreads();                                         // read by all before the next call clears it
     int const topMask = int(flags & 7u);
     int const oneMask = int(~(flags >> 4) & ~flags & 7u);
-    return topMask | (oneMask << kOnePlaneShift);
+    return topMask | (oneMask << kOnePlaneShift) | ((flags & (1u << 8)) ? 0 : kFp8OutputsBounded);
 }
 
 template <class V>
@@ -766,7 +776,12 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
         v4i D[4];
         v4f S;
         mlp_forward_fp8<V>(lds, wave, lane, modes, in, D, S);
-        if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)      store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, x0 + j, y0, 4 * g);
+        if (V::ONE && (modes & kFp8OutputsBounded)) {        // (the general instantiation keeps to the checked stores)
+            if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)  store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS, false>(m, D, S, x0 + j, y0, 4 * g);
+            else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)   store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS, false>(m, D, S, x0 + j, y0, 4 * g);
+            else                                                   store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS, false>(m, D, S, x0 + j, y0, 4 * g);
+        }
+        else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS) store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, x0 + j, y0, 4 * g);
         else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)       store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
         else                                                       store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
     };

@@ -327,6 +327,28 @@ def test_gpu_fp8_decode_at_the_one_plane_limit(ntc, device, layer):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("scale", [0.107, 0.1072, 0.5, 40.0])
+def test_gpu_fp8_outputs_near_and_beyond_the_fp16_range(ntc, device, scale):
+    """An output whose half would be an infinity is stored as zero (IsHalfSpecial).  The stores skip that check
+    when (|bias| + 32 * 127 * 128) * |scale| < 60000 holds for every channel of the output layer: with biases of
+    +-40000 that is scale < 0.10711.  Either side of it, and scales with which outputs do overflow (zeros must
+    appear, as in the checker)."""
+    spec = ntc.presets.spec_ref092_fp8(16)
+    layout = ntc.synth.weight_layout(spec)
+    last = ntc.abi.MLP_LAYERS - 1
+    case = fp8_case(ntc, 16, 128, 64, 4, 2, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=401, bias_sigma=0.5)
+    case.weights[layout.scaleOffset[last]:layout.scaleOffset[last] + 64] = np.full(16, scale, dtype=np.float32).view(np.uint8)
+    bias = np.where(np.arange(16) % 2 == 0, 40000, -40000).astype(np.int32)
+    case.weights[layout.biasOffset[last]:layout.biasOffset[last] + 64] = bias.view(np.uint8)
+    expected, got = run_both(device, case)
+    assert first_mismatch(expected, got) is None, scale
+    halves = got.view(np.uint16)
+    assert not np.any((halves & 0x7fff) >= 0x7c00)                           # no infinity, no NaN is ever stored
+    if scale >= 40.0:
+        assert np.count_nonzero(halves == 0) > 1000                          # overflowing outputs became zeros
+
+
+@pytest.mark.gpu
 def test_gpu_fp8_level_of_detail_input_up_to_three(ntc, device):
     """The exactness of the layer sums is proven for inputs of at most 3 in magnitude.  Features and positional
     encoding lie in [-1, 1]; the level-of-detail input comes from the caller's descriptor: +-3 decodes to the
