@@ -24,6 +24,7 @@
 // launch, a workgroup tile of 64 x 4 texels = four wave tiles of 16 x 4; lane = texel in the input stage,
 // lane (j = lane%16, g = lane/16) = channels 16t+4g..+3 of texel j in the matrix stages.
 #include "ntc_decode_device.h"
+#include <type_traits>
 
 namespace ntc_hip_dev {
 
@@ -875,16 +876,21 @@ query_fp8_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* _
         mlp_forward_fp8<V>(lds, wave, lane, modes, in, D, S);
 
         // lane (j, g) holds channels 4g..4g+3 of query q0 + 16b + j; validity travels by shuffle
+        auto store_outputs = [&](auto checked) __attribute__((always_inline)) {
+            constexpr bool CHECKED = decltype(checked)::value;
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            uint64_t const q = q0 + uint64_t(16 * b + j);
-            int const ok = __shfl(validMip ? 1 : 0, 16 * b + j, 64);
-            if (q >= numQueries) continue;
-            uint32_t h01 = to_half2_bits(float(D[b][0]) * S[0], float(D[b][1]) * S[1]);
-            uint32_t h23 = to_half2_bits(float(D[b][2]) * S[2], float(D[b][3]) * S[3]);
-            if (!ok) { h01 = 0; h23 = 0; }
-            *reinterpret_cast<u32x2*>(out + q * 16 + 4 * g) = u32x2{ h01, h23 };
-        }
+            for (int b = 0; b < 4; ++b) {
+                uint64_t const q = q0 + uint64_t(16 * b + j);
+                int const ok = __shfl(validMip ? 1 : 0, 16 * b + j, 64);
+                if (q >= numQueries) continue;
+                uint32_t h01 = to_half2_bits<CHECKED>(float(D[b][0]) * S[0], float(D[b][1]) * S[1]);
+                uint32_t h23 = to_half2_bits<CHECKED>(float(D[b][2]) * S[2], float(D[b][3]) * S[3]);
+                if (!ok) { h01 = 0; h23 = 0; }
+                *reinterpret_cast<u32x2*>(out + q * 16 + 4 * g) = u32x2{ h01, h23 };
+            }
+        };
+        if (V::ONE && (modes & kFp8OutputsBounded)) store_outputs(std::false_type{});      // see decode_fp8_kernel
+        else                                        store_outputs(std::true_type{});
     }
 }
 
