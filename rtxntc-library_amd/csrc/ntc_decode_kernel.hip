@@ -26,6 +26,7 @@
 #include <stdint.h>
 #include "ntc_decode_kernel.h"
 #include "ntc_decode_device.h"
+#include <type_traits>
 
 namespace ntc_hip_dev {
 
@@ -1252,16 +1253,21 @@ query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __res
         }
 
         // lane (j, g) holds channels 4g..4g+3 of query q0 + 16b + j; validity travels by shuffle
+        auto store_outputs = [&](auto checked) __attribute__((always_inline)) {
+            constexpr bool CHECKED = decltype(checked)::value;
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            uint64_t const q = q0 + uint64_t(16 * b + j);
-            int const ok = __shfl(validMip ? 1 : 0, 16 * b + j, 64);
-            if (q >= numQueries) continue;
-            uint32_t h01 = to_half2_bits(F[b][0] * S[0], F[b][1] * S[1]);
-            uint32_t h23 = to_half2_bits(F[b][2] * S[2], F[b][3] * S[3]);
-            if (!ok) { h01 = 0; h23 = 0; }
-            *reinterpret_cast<u32x2*>(out + q * 16 + 4 * g) = u32x2{ h01, h23 };
-        }
+            for (int b = 0; b < 4; ++b) {
+                uint64_t const q = q0 + uint64_t(16 * b + j);
+                int const ok = __shfl(validMip ? 1 : 0, 16 * b + j, 64);
+                if (q >= numQueries) continue;
+                uint32_t h01 = to_half2_bits<CHECKED>(F[b][0] * S[0], F[b][1] * S[1]);
+                uint32_t h23 = to_half2_bits<CHECKED>(F[b][2] * S[2], F[b][3] * S[3]);
+                if (!ok) { h01 = 0; h23 = 0; }
+                *reinterpret_cast<u32x2*>(out + q * 16 + 4 * g) = u32x2{ h01, h23 };
+            }
+        };
+        if (useF16 && (staged & kOutputsBounded)) store_outputs(std::false_type{});        // as in decode_kernel
+        else                                      store_outputs(std::true_type{});
     }
 }
 
