@@ -581,11 +581,16 @@ __device__ __forceinline__ void fp8_hidden_layer(Load&& load, uint4 const (&B32)
     // The operands of output tile t + 1 are loaded before the work on tile t (two sets of registers, alternating);
     // a scheduling barrier that only LDS reads may not cross keeps the compiler from moving those loads back down
     // to their uses.
+    // (Not with three planes - a layer with a weight of 32 or more: that form's registers would set the kernel's
+    // budget, and the kernel would spill in its prologue what every workgroup, also one that only passes over
+    // sets, has to write out.)
+    constexpr bool AHEAD = PLANES < 3;
     TileOperands<NK32, HAS16> ops[2];
-    load(0, ops[0]);
+    if (AHEAD) load(0, ops[0]);
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
-        if (t + 1 < TILES) {
+        if (!AHEAD) load(t, ops[t & 1]);
+        if (AHEAD && t + 1 < TILES) {
             load(t + 1, ops[(t + 1) & 1]);
             __builtin_amdgcn_sched_barrier(0x67f);           // everything but LDS instructions may cross
         }
