@@ -257,25 +257,63 @@ __device__ __forceinline__ int segment_end(DevMip const* __restrict__ mips, int 
     return tileEnd;
 }
 
+// What a lane's stores of one wave tile share: channel count, byte offsets inside an output row, row size.
+template <int FORMAT, class Mip>
+struct StorePlace {
+    int nch;
+    uint32_t laneOff, laneOff2;
+    size_t rowBytes;
+    __device__ __forceinline__ StorePlace(Mip const& m, int x, int chBase)
+    {
+        nch = (x < m.width) ? min(4, m.numChannels - chBase) : 0;
+        uint32_t const C2 = uint32_t((m.numChannels + 1) & ~1);
+        laneOff = (FORMAT == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)
+            ? (uint32_t(chBase) * uint32_t(m.width) + uint32_t(x) * 2u) * 2u
+            : uint32_t(x) * uint32_t(m.outPixelStride) + uint32_t(chBase) * (FORMAT == NTC_HIP_DEV_OUT_FP16_PIXELS ? 2u : 1u);
+        laneOff2 = laneOff + uint32_t(m.width) * 4u;
+        rowBytes = (FORMAT == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS) ? size_t(m.width) * C2 * 2 : size_t(m.outRowPitch);
+    }
+};
+
+// The lane's four channels of one texel of image row y (uniform, inside the image): outputs = accumulators times
+// scales, rounded to half.
+template <int FORMAT, bool CHECKED, class AccV, class Mip>
+__device__ __forceinline__ void store_row(Mip const& m, StorePlace<FORMAT, Mip> const& at, AccV D, v4f S, int y)
+{
+    uint32_t const h01 = to_half2_bits<CHECKED>(float(D[0]) * S[0], float(D[1]) * S[1]);
+    uint32_t const h23 = to_half2_bits<CHECKED>(float(D[2]) * S[2], float(D[3]) * S[3]);
+    GlobalOutPtr const row = uniform_pointer(reinterpret_cast<uint64_t>(m.out) + size_t(y) * at.rowBytes);
+    store_channels<FORMAT>(row, at.laneOff, at.laneOff2, h01, h23, at.nch, m.vectorStores);
+}
+
 template <int FORMAT, bool CHECKED = true, class Acc, class Mip>
 __device__ __forceinline__ void store_tile(Mip const& m, Acc const (&D)[4], v4f S, int x, int y0, int chBase)
 {
-    int const nch = min(4, m.numChannels - chBase);
-    if (x >= m.width || nch <= 0) return;
-    uint32_t const C2 = uint32_t((m.numChannels + 1) & ~1);
-    uint32_t const laneOff = (FORMAT == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)
-        ? (uint32_t(chBase) * uint32_t(m.width) + uint32_t(x) * 2u) * 2u
-        : uint32_t(x) * uint32_t(m.outPixelStride) + uint32_t(chBase) * (FORMAT == NTC_HIP_DEV_OUT_FP16_PIXELS ? 2u : 1u);
-    uint32_t const laneOff2 = laneOff + uint32_t(m.width) * 4u;
-    size_t const rowBytes = (FORMAT == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS) ? size_t(m.width) * C2 * 2 : size_t(m.outRowPitch);
+    StorePlace<FORMAT, Mip> const at(m, x, chBase);
+    if (at.nch <= 0) return;
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
         int const y = y0 + b;
         if (y >= m.height) break;                            // uniform
-        uint32_t const h01 = to_half2_bits<CHECKED>(float(D[b][0]) * S[0], float(D[b][1]) * S[1]);
-        uint32_t const h23 = to_half2_bits<CHECKED>(float(D[b][2]) * S[2], float(D[b][3]) * S[3]);
-        GlobalOutPtr const row = uniform_pointer(reinterpret_cast<uint64_t>(m.out) + size_t(y) * rowBytes);
-        store_channels<FORMAT>(row, laneOff, laneOff2, h01, h23, nch, m.vectorStores);
+        store_row<FORMAT, CHECKED>(m, at, D[b], S, y);
+    }
+}
+
+// One row of a wave tile in the mip's own format (checked conversion): the stores of the int8-only network path,
+// which produces the wave's four rows one after the other.
+template <class AccV, class Mip>
+__device__ __forceinline__ void store_row_any_format(Mip const& m, AccV D, v4f S, int x, int y, int chBase)
+{
+    if (y >= m.height) return;
+    if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS) {
+        StorePlace<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS, Mip> const at(m, x, chBase);
+        if (at.nch > 0) store_row<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS, true>(m, at, D, S, y);
+    } else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS) {
+        StorePlace<NTC_HIP_DEV_OUT_FP16_PIXELS, Mip> const at(m, x, chBase);
+        if (at.nch > 0) store_row<NTC_HIP_DEV_OUT_FP16_PIXELS, true>(m, at, D, S, y);
+    } else {
+        StorePlace<NTC_HIP_DEV_OUT_UNORM8_PIXELS, Mip> const at(m, x, chBase);
+        if (at.nch > 0) store_row<NTC_HIP_DEV_OUT_UNORM8_PIXELS, true>(m, at, D, S, y);
     }
 }
 

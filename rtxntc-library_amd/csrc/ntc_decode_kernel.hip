@@ -770,53 +770,54 @@ __device__ void build_posenc_tables(LdsT<V>& lds)
 // Input vectors of the wave's 64 texels (lane = texel 16*b + j holds its own in `in`) -> B operands of
 // layer 0: X[b] = the four input dwords of k-group g = lane/16 of texel 16b + lane%16.
 template <class V>
-__device__ __forceinline__ void transpose_inputs(LdsT<V>& lds, int wave, int lane, uint32_t const (&in)[16], v4i (&X)[4])
+__device__ __forceinline__ void write_inputs(LdsT<V>& lds, int wave, int lane, uint32_t const (&in)[16])
 {
-    int const j = lane & 15, g = lane >> 4;
-    {
-        uint4* dst = reinterpret_cast<uint4*>(&lds.in[wave][lane][0]);
-        dst[0] = make_uint4(in[0], in[1], in[2], in[3]);
-        dst[1] = make_uint4(in[4], in[5], in[6], in[7]);
-        dst[2] = make_uint4(in[8], in[9], in[10], in[11]);
-        if constexpr (V::IN_STRIDE >= 16) dst[3] = make_uint4(in[12], in[13], in[14], in[15]);
-    }
+    uint4* dst = reinterpret_cast<uint4*>(&lds.in[wave][lane][0]);
+    dst[0] = make_uint4(in[0], in[1], in[2], in[3]);
+    dst[1] = make_uint4(in[4], in[5], in[6], in[7]);
+    dst[2] = make_uint4(in[8], in[9], in[10], in[11]);
+    if constexpr (V::IN_STRIDE >= 16) dst[3] = make_uint4(in[12], in[13], in[14], in[15]);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <class V>
+__device__ __forceinline__ v4i read_input_block(LdsT<V> const& lds, int wave, int lane, int b)
+{
+    int const j = lane & 15, g = lane >> 4;
+    // a row of 12 dwords has no k-group 3: those inputs are the zero padding
+    int const gRead = V::IN_STRIDE >= 16 ? g : min(g, 2);
+    uint4 t = *reinterpret_cast<uint4 const*>(&lds.in[wave][b * 16 + j][4 * gRead]);
+    if (V::IN_STRIDE < 16 && g == 3) t = make_uint4(0u, 0u, 0u, 0u);
+    return v4i{ int(t.x), int(t.y), int(t.z), int(t.w) };
+}
+
+template <class V>
+__device__ __forceinline__ void transpose_inputs(LdsT<V>& lds, int wave, int lane, uint32_t const (&in)[16], v4i (&X)[4])
+{
+    write_inputs<V>(lds, wave, lane, in);
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {
-        // a row of 12 dwords has no k-group 3: those inputs are the zero padding
-        int const gRead = V::IN_STRIDE >= 16 ? g : min(g, 2);
-        uint4 t = *reinterpret_cast<uint4 const*>(&lds.in[wave][b * 16 + j][4 * gRead]);
-        if (V::IN_STRIDE < 16 && g == 3) t = make_uint4(0u, 0u, 0u, 0u);
-        X[b] = v4i{ int(t.x), int(t.y), int(t.z), int(t.w) };
-    }
+    for (int b = 0; b < 4; ++b) X[b] = read_input_block<V>(lds, wave, lane, b);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
 }
 
-// The network for the 64 texels of one wave.  `in` is the lane's own texel (lane = 16*b + j).
-// On return D[b] holds, for lane (j = lane%16, g = lane/16), the int32 accumulators of output
-// channels 4g..4g+3 of texel 16*b + j, and S their scales.
+// The network with every layer on the int8 matrix instruction, for ONE 16-texel block of the wave (X = its B
+// operand of layer 0).  This is the path of weights whose sums do not fit the fp16 form (see stage_weights): rare, so
+// the wave's four blocks go through it one after the other in a loop that is not unrolled - a quarter of the code and
+// of the registers of the unrolled form, which had cost the fp16 path of the widest variant its registers.
+// On return D holds, for lane (j = lane%16, g = lane/16), the int32 accumulators of output channels 4g..4g+3 of
+// texel j of the block, and S their scales.
 template <class V>
-__device__ __forceinline__ void mlp_forward(LdsT<V>& lds, int wave, int lane, uint32_t const (&in)[16],
-                                            v4i (&D)[4], v4f& S)
+__device__ __forceinline__ void mlp_forward_block(LdsT<V> const& lds, int lane, v4i X, v4i& D, v4f& S)
 {
     int const g = lane >> 4;
-    v4i X[4];
-    transpose_inputs<V>(lds, wave, lane, in, X);
-
-
-    // hidden layers
     constexpr int tiles[3] = { V::T0, V::T1, V::T2 };
     int tb = 0;
 #pragma unroll
     for (int l = 0; l < 3; ++l) {
-        uint32_t Y[4][4];
-#pragma unroll
-        for (int b = 0; b < 4; ++b)
-#pragma unroll
-            for (int d = 0; d < 4; ++d) Y[b][d] = 0;
+        uint32_t Y[4] = { 0, 0, 0, 0 };
 #pragma unroll
         for (int t = 0; t < tiles[l]; ++t) {
             // A operand of plane q: layer 0 from `w`, later layers from the int8 tiles in `late`
@@ -825,33 +826,20 @@ __device__ __forceinline__ void mlp_forward(LdsT<V>& lds, int wave, int lane, ui
                                        : *reinterpret_cast<uint4 const*>(&lds.w[q][t][lane][0]);
                 return v4i{ int(wq.x), int(wq.y), int(wq.z), int(wq.w) };
             };
-            v4i const A = operand(0);
             v4i const C = *reinterpret_cast<v4i const*>(&lds.bias[tb + t][g][0]);
             v4f const Sc = *reinterpret_cast<v4f const*>(&lds.scale[tb + t][g][0]);
+            v4i Dh = __builtin_amdgcn_mfma_i32_16x16x64_i8(operand(0), X, C, 0, 0, 0);
             if constexpr (V::FP8_WEIGHTS) {
-                v4i const A1 = operand(V::PLANES > 1 ? 1 : 0), A2 = operand(V::PLANES > 2 ? 2 : 0);
                 v4i const Z = v4i{ 0, 0, 0, 0 };
+                v4i const D1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(operand(1), X, Z, 0, 0, 0);
+                v4i const D2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(operand(2), X, Z, 0, 0, 0);
 #pragma unroll
-                for (int b = 0; b < 4; ++b) {
-                    v4i const D0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
-                    v4i const D1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A1, X[b], Z, 0, 0, 0);
-                    v4i const D2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A2, X[b], Z, 0, 0, 0);
-                    v4i Dh;
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)                    // 4096*D2 + 64*D1 + D0, wrapping like int32
-                        Dh[r] = int((((uint32_t(D2[r]) << 6) + uint32_t(D1[r])) << 6) + uint32_t(D0[r]));
-                    Y[b][t] = activate4(Dh, Sc);
-                }
-            } else {
-#pragma unroll
-                for (int b = 0; b < 4; ++b) {
-                    v4i const Dh = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
-                    Y[b][t] = activate4(Dh, Sc);
-                }
+                for (int r = 0; r < 4; ++r)                    // 4096*D2 + 64*D1 + D0, wrapping like int32
+                    Dh[r] = int((((uint32_t(D2[r]) << 6) + uint32_t(D1[r])) << 6) + uint32_t(Dh[r]));
             }
+            Y[t] = activate4(Dh, Sc);
         }
-#pragma unroll
-        for (int b = 0; b < 4; ++b) X[b] = v4i{ int(Y[b][0]), int(Y[b][1]), int(Y[b][2]), int(Y[b][3]) };
+        X = v4i{ int(Y[0]), int(Y[1]), int(Y[2]), int(Y[3]) };
         tb += tiles[l];
     }
 
@@ -860,8 +848,7 @@ __device__ __forceinline__ void mlp_forward(LdsT<V>& lds, int wave, int lane, ui
     v4i const A = v4i{ int(wa.x), int(wa.y), int(wa.z), int(wa.w) };
     v4i const C = *reinterpret_cast<v4i const*>(&lds.bias[tb][g][0]);
     S = *reinterpret_cast<v4f const*>(&lds.scale[tb][g][0]);
-#pragma unroll
-    for (int b = 0; b < 4; ++b) D[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
+    D = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X, C, 0, 0, 0);
 }
 
 // ---- layers 1..3 on the fp16 matrix instruction --------------------------------------------
@@ -1129,12 +1116,19 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
                 else                                                   store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
             }
         } else {
-            v4i D[4];
-            v4f S;
-            mlp_forward<V>(lds, wave, lane, in, D, S);
-            if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)      store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, x0 + j, y0, 4 * g);
-            else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)       store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
-            else                                                       store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
+            // every layer on the int8 matrix instruction: one 16-texel block (= one image row of the tile) at a time
+            write_inputs<V>(lds, wave, lane, in);
+#pragma unroll 1
+            for (int b = 0; b < 4; ++b) {
+                v4i D;
+                v4f S;
+                int laneB = lane;
+                asm volatile("" : "+v"(laneB));                  // keeps the weight reads inside the loop (hoisted, they take every register)
+                mlp_forward_block<V>(lds, laneB, read_input_block<V>(lds, wave, lane, b), D, S);
+                store_row_any_format(m, D, S, x0 + j, y0 + b, 4 * g);
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
         }
     };
 
@@ -1239,35 +1233,45 @@ query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __res
         }
         else                    prepare_inputs_general<V>(mips[validMip ? query.mip : 0], x, y, in);
 
-        // output-layer accumulators as floats: exact either way (|acc| < 2^24 on the fp16 path; the
-        // int32 -> float conversion is the definition's on the int8 path)
-        v4f F[4];
-        v4f S;
-        if (V::F16_LAYERS && useF16) {
-            mlp_forward_f16<V>(lds, wave, lane, (staged & kL0Magic) != 0, in, F, S);
-        } else {
-            v4i D[4];
-            mlp_forward<V>(lds, wave, lane, in, D, S);
-#pragma unroll
-            for (int b = 0; b < 4; ++b) F[b] = v4f{ float(D[b][0]), float(D[b][1]), float(D[b][2]), float(D[b][3]) };
-        }
-
         // lane (j, g) holds channels 4g..4g+3 of query q0 + 16b + j; validity travels by shuffle
-        auto store_outputs = [&](auto checked) __attribute__((always_inline)) {
+        auto store_outputs = [&](auto checked, int b, v4f Fb, v4f S) __attribute__((always_inline)) {
             constexpr bool CHECKED = decltype(checked)::value;
-#pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                uint64_t const q = q0 + uint64_t(16 * b + j);
-                int const ok = __shfl(validMip ? 1 : 0, 16 * b + j, 64);
-                if (q >= numQueries) continue;
-                uint32_t h01 = to_half2_bits<CHECKED>(F[b][0] * S[0], F[b][1] * S[1]);
-                uint32_t h23 = to_half2_bits<CHECKED>(F[b][2] * S[2], F[b][3] * S[3]);
-                if (!ok) { h01 = 0; h23 = 0; }
-                *reinterpret_cast<u32x2*>(out + q * 16 + 4 * g) = u32x2{ h01, h23 };
-            }
+            uint64_t const q = q0 + uint64_t(16 * b + j);
+            int const ok = __shfl(validMip ? 1 : 0, 16 * b + j, 64);
+            if (q >= numQueries) return;
+            uint32_t h01 = to_half2_bits<CHECKED>(Fb[0] * S[0], Fb[1] * S[1]);
+            uint32_t h23 = to_half2_bits<CHECKED>(Fb[2] * S[2], Fb[3] * S[3]);
+            if (!ok) { h01 = 0; h23 = 0; }
+            *reinterpret_cast<u32x2*>(out + q * 16 + 4 * g) = u32x2{ h01, h23 };
         };
-        if (useF16 && (staged & kOutputsBounded)) store_outputs(std::false_type{});        // as in decode_kernel
-        else                                      store_outputs(std::true_type{});
+        if (V::F16_LAYERS && useF16) {
+            // output-layer accumulators as floats: exact integers below 2^24
+            v4f F[4];
+            v4f S;
+            mlp_forward_f16<V>(lds, wave, lane, (staged & kL0Magic) != 0, in, F, S);
+            if (staged & kOutputsBounded) {                                                  // as in decode_kernel
+#pragma unroll
+                for (int b = 0; b < 4; ++b) store_outputs(std::false_type{}, b, F[b], S);
+            } else {
+#pragma unroll
+                for (int b = 0; b < 4; ++b) store_outputs(std::true_type{}, b, F[b], S);
+            }
+        } else {
+            // every layer on the int8 matrix instruction, one 16-query block at a time; the int32 -> float
+            // conversion of the accumulators is the definition's
+            write_inputs<V>(lds, wave, lane, in);
+#pragma unroll 1
+            for (int b = 0; b < 4; ++b) {
+                v4i D;
+                v4f S;
+                int laneB = lane;
+                asm volatile("" : "+v"(laneB));                  // keeps the weight reads inside the loop
+                mlp_forward_block<V>(lds, laneB, read_input_block<V>(lds, wave, lane, b), D, S);
+                store_outputs(std::true_type{}, b, v4f{ float(D[0]), float(D[1]), float(D[2]), float(D[3]) }, S);
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        }
     }
 }
 
