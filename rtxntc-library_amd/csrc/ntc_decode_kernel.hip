@@ -318,7 +318,7 @@ __device__ int stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
             if constexpr (V::FP8_WEIGHTS) {
                 if (twoPlanes) lds.biasLo[slotTile][slotG][slotR] = float(shifted & 1023) * 0x1p-24f;
             }
-            // sums run over (q + 113) * 2^-24 (see activate4_h): every term, this start value included, is an
+            // sums run over (q + 113) * 2^-24 (see activate_scale4): every term, this start value included, is an
             // integer below 2^24 times 2^-24, exact in fp32; the scale takes the 2^24 back
             lds.bias[slotTile][slotG][slotR] = __builtin_bit_cast(int32_t, float(twoPlanes ? (shifted >> 10) : shifted) * 0x1p-24f);
             lds.scale[slotTile][slotG][slotR] = reinterpret_cast<float const*>(blob + V::SCALE_OFF)[V::H0 + threadIdx.x] * 0x1p24f;
@@ -856,7 +856,7 @@ __device__ __forceinline__ void mlp_forward_block(LdsT<V> const& lds, int lane, 
 // Same integers, fewer vector operations.  The int8 matrix instruction returns int32, which costs a
 // conversion per activation, and its operands are signed bytes, which forces the "- 113" and the
 // clamp of min(x, 3) into fp32.  Here the previous layer's activations enter as fp16 numbers
-// proportional to u = q + 113 in [-15, 240] (u * 2^-24, see activate4_h) and the weights as fp16 integers;
+// proportional to u = q + 113 in [-15, 240] (u * 2^-24, see activate_scale4) and the weights as fp16 integers;
 // products and every partial sum are integers below 2^24 (stage_weights checked that) times 2^-24, so the
 // fp32 accumulator of v_mfma_f32_16x16x32_f16 holds exactly 2^-24 * (bias + sum W*(u - 113)) once it starts
 // at 2^-24 * (bias - 113*sum(W)), and the channel's scale times 2^24 gives the same product the definition
@@ -874,11 +874,16 @@ __device__ __forceinline__ void mlp_forward_block(LdsT<V> const& lds, int lane, 
 // The fp16 matrix instruction takes subnormal operands as they are (checked by the unit test of the
 // instruction); the layers that consume these values hold their biases times 2^-24 and their scales times 2^24.
 // The empty asm keeps multiply and conversion apart: fused (v_fma_mixlo_f16) they would round once.
+//
+// In two parts, because the SIMD treats them differently.  The fp32 part (activate_scale4: four multiplies / fused
+// multiply-adds per value) is made of instructions that issue two at a time, one from each of two waves; the packed
+// conversion and minimum (activate_pack4) issue alone, and so does everything while a matrix instruction executes.
+// The layers below therefore hold a tile's conversions back until the NEXT tile's matrix instructions are in flight
+// and put them between those (slots that would be single anyway), and run a tile's fp32 part as a stretch of its own.
 typedef short v2s __attribute__((ext_vector_type(2)));
 template <class Acc>
-__device__ __forceinline__ void activate4_h(Acc acc, v4f scale, uint32_t (&out)[2])
+__device__ __forceinline__ void activate_scale4(Acc acc, v4f scale, float (&v)[4])
 {
-    float v[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         float const x = float(acc[r]) * scale[r];
@@ -888,11 +893,48 @@ __device__ __forceinline__ void activate4_h(Acc acc, v4f scale, uint32_t (&out)[
         v[r] = y * (80.f * 0x1p-24f);
         asm("" : "+v"(v[r]));
     }
+}
+
+__device__ __forceinline__ void activate_pack4(float const (&v)[4], uint32_t (&out)[2])
+{
     v2s const cap = { 240, 240 };
     v2s const lo = __builtin_bit_cast(v2s, __builtin_convertvector(v2f{ v[0], v[1] }, v2h));
     v2s const hi = __builtin_bit_cast(v2s, __builtin_convertvector(v2f{ v[2], v[3] }, v2h));
     out[0] = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(lo, cap));
     out[1] = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(hi, cap));
+}
+
+// A section boundary for the instruction scheduler: vector and matrix instructions stay on their side, scalar and LDS
+// instructions may cross (so that operand reads still go out ahead of their use).
+__device__ __forceinline__ void section_end() { __builtin_amdgcn_sched_barrier(0x4 | 0x80 | 0x100 | 0x200); }
+
+// Inside a section: `groups` times { `matrix` matrix instructions, then `vector` vector instructions }.
+template <int GROUPS, int MATRIX, int VECTOR>
+__device__ __forceinline__ void interleave()
+{
+#pragma unroll
+    for (int i = 0; i < GROUPS; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x8, MATRIX, 0);
+        __builtin_amdgcn_sched_group_barrier(0x2, VECTOR, 0);
+    }
+}
+
+// The scaled outputs of one output tile whose conversion is pending, [block b][r].
+struct PendingTile {
+    float z[4][4];
+    __device__ __forceinline__ void convert_into(uint32_t (&H)[4][4][2], int tile) const
+    {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) activate_pack4(z[b], H[b][tile]);
+    }
+};
+
+// A use of tile `tile` of H at this place (the end of the section that converted it): without one the compiler sinks
+// the conversions to their first real use, the next layer.
+__device__ __forceinline__ void keep_here(uint32_t (&H)[4][4][2], int tile)
+{
+#pragma unroll
+    for (int b = 0; b < 4; ++b) asm volatile("" : "+v"(H[b][tile][0]), "+v"(H[b][tile][1]));
 }
 
 // acc[b] += W(tile t of the layer at `base`) * H[b], for the four 16-texel blocks of the wave.
@@ -936,82 +978,59 @@ __device__ __forceinline__ void f16_tile(LdsT<V> const& lds, int base, int t, in
     }
 }
 
-template <class V, int IN_TILES, int OUT_TILES>
+// One hidden layer on the fp16 matrix instruction (e4m3 variants: weights as two fp16 planes, 512 w = 1024 hi + lo;
+// both sums are exact integers in fp32, and fma(hi, 1024, lo) rounds their exact combination once - the value a
+// conversion of the int32 accumulator to float gives).  On entry `pending` holds the scaled outputs of the LAST tile of
+// Hin, not yet converted; on return those of this layer's last tile.  Per output tile: section A = the tile's matrix
+// instructions with the pending conversions between them, section B = the fp32 part of the tile.  In the first tile
+// the pending tile is an input: its conversions come first in program order, and the matrix instructions that read
+// it are the last ones.
+template <class V, int IN_TILES, int OUT_TILES, bool TWO_PLANES>
 __device__ __forceinline__ void f16_hidden_layer(LdsT<V> const& lds, int base, int tileBase, int lane,
-                                                 uint32_t const (&Hin)[4][4][2], uint32_t (&Hout)[4][4][2])
-{
-    int const g = lane >> 4;
-#pragma unroll
-    for (int t = 0; t < OUT_TILES; ++t) {
-        v4f const C = *reinterpret_cast<v4f const*>(&lds.bias[tileBase + t][g][0]);       // float(bias - 113*sum W)
-        v4f const Sc = *reinterpret_cast<v4f const*>(&lds.scale[tileBase + t][g][0]);
-        v4f acc[4] = { C, C, C, C };
-        f16_tile<V, IN_TILES>(lds, base, t, lane, Hin, acc);
-#pragma unroll
-        for (int b = 0; b < 4; ++b) activate4_h(acc[b], Sc, Hout[b][t]);
-    }
-}
-
-// The same for a layer with e4m3 weights held as two fp16 planes (512 w = 1024 hi + lo): both sums are exact
-// integers in fp32, and fma(hi, 1024, lo) rounds their exact combination once - the value a conversion of
-// the int32 accumulator to float gives.
-template <class V, int IN_TILES, int OUT_TILES>
-__device__ __forceinline__ void f16_hidden_layer_two_planes(LdsT<V> const& lds, int base, int tileBase, int lane,
-                                                            uint32_t const (&Hin)[4][4][2], uint32_t (&Hout)[4][4][2])
+                                                 uint32_t (&Hin)[4][4][2], uint32_t (&Hout)[4][4][2], PendingTile& pending)
 {
     constexpr int PLANE = OUT_TILES * V::f16_units(IN_TILES);
+    constexpr int MATRIX = (TWO_PLANES ? 2 : 1) * 4 * ((IN_TILES % 2 == 0) ? IN_TILES / 2 : IN_TILES);   // matrix instructions per tile
     int const g = lane >> 4;
 #pragma unroll
     for (int t = 0; t < OUT_TILES; ++t) {
-        v4f const Chi = *reinterpret_cast<v4f const*>(&lds.bias[tileBase + t][g][0]);
-        v4f const Clo = *reinterpret_cast<v4f const*>(&lds.biasLo[tileBase + t][g][0]);
+        v4f const C = *reinterpret_cast<v4f const*>(&lds.bias[tileBase + t][g][0]);
         v4f const Sc = *reinterpret_cast<v4f const*>(&lds.scale[tileBase + t][g][0]);
-        v4f hi[4] = { Chi, Chi, Chi, Chi }, lo[4] = { Clo, Clo, Clo, Clo };
-        f16_tile<V, IN_TILES>(lds, base, t, lane, Hin, hi);
-        f16_tile<V, IN_TILES>(lds, base + PLANE, t, lane, Hin, lo);
+        if (t == 0) pending.convert_into(Hin, IN_TILES - 1);
+        else        pending.convert_into(Hout, t - 1);
+        v4f acc[4] = { C, C, C, C };
+        f16_tile<V, IN_TILES>(lds, base, t, lane, Hin, acc);
+        if constexpr (TWO_PLANES) {
+            if constexpr (V::FP8_WEIGHTS) {                  // (biasLo exists in those variants only)
+                v4f const Clo = *reinterpret_cast<v4f const*>(&lds.biasLo[tileBase + t][g][0]);
+                v4f lo[4] = { Clo, Clo, Clo, Clo };
+                f16_tile<V, IN_TILES>(lds, base + PLANE, t, lane, Hin, lo);
+                interleave<8, MATRIX / 8, 2>();
+                if (t > 0) keep_here(Hout, t - 1);
+                section_end();
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            v4f acc;
+                for (int b = 0; b < 4; ++b)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) acc[r] = __builtin_fmaf(hi[b][r], 1024.f, lo[b][r]);
-            activate4_h(acc, Sc, Hout[b][t]);
+                    for (int r = 0; r < 4; ++r) acc[b][r] = __builtin_fmaf(acc[b][r], 1024.f, lo[b][r]);
+            }
+        } else {
+            interleave<8, (MATRIX >= 8 ? MATRIX / 8 : 1), 2>();
+            if (t > 0) keep_here(Hout, t - 1);
+            section_end();
         }
+#pragma unroll
+        for (int b = 0; b < 4; ++b) activate_scale4(acc[b], Sc, pending.z[b]);
+        section_end();
     }
 }
 
-// The network for the 64 texels of one wave with layers 1..3 on the fp16 matrix instruction.
-// Same interface as mlp_forward, except that D holds the output layer's accumulators as floats
-// (exact integers).
-template <class V>
-__device__ __forceinline__ void mlp_forward_f16(LdsT<V>& lds, int wave, int lane, bool l0Magic, uint32_t const (&in)[16], v4f (&D)[4], v4f& S)
+// Layer 0: int8 inputs, int32 accumulators.  MAGIC (variants without e4m3 weights, decided at staging): the
+// accumulators started at bias + 0x4B400000, so their bits are the float 1.5 * 2^23 + acc, exactly, and a subtraction
+// replaces the conversion.  e4m3 variants: three planes, recombined wrapping like int32.  Same sections as above.
+template <class V, bool MAGIC>
+__device__ __forceinline__ void first_layer(LdsT<V> const& lds, int lane, v4i const (&X)[4], uint32_t (&Hout)[4][4][2], PendingTile& pending)
 {
     int const g = lane >> 4;
-    v4i X[4];
-    transpose_inputs<V>(lds, wave, lane, in, X);
-
-    // layer 0: int8 inputs, int32 accumulators (three planes for e4m3 weights, recombined wrapping like int32)
-    uint32_t Ha[4][4][2], Hb[4][4][2];
-    if (!V::FP8_WEIGHTS && l0Magic) {                        // uniform
-        // the accumulator started at bias + 0x4B400000: its bits are the float 1.5 * 2^23 + acc, exactly
-#pragma unroll
-        for (int t = 0; t < V::T0; ++t) {
-            uint4 const wq = *reinterpret_cast<uint4 const*>(&lds.w[0][t][lane][0]);
-            v4i const A = v4i{ int(wq.x), int(wq.y), int(wq.z), int(wq.w) };
-            v4i const C = *reinterpret_cast<v4i const*>(&lds.bias[t][g][0]);
-            v4f const Sc = *reinterpret_cast<v4f const*>(&lds.scale[t][g][0]);
-#pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                v4i const Dh = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
-                v4f acc;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    int32_t const bits = Dh[r];                  // (a copy: bit_cast of a vector element expression reads element 0)
-                    acc[r] = __builtin_bit_cast(float, bits) - 12582912.f;
-                }
-                activate4_h(acc, Sc, Ha[b][t]);
-            }
-        }
-    } else {
 #pragma unroll
     for (int t = 0; t < V::T0; ++t) {
         auto const operand = [&](int q) {
@@ -1021,38 +1040,75 @@ __device__ __forceinline__ void mlp_forward_f16(LdsT<V>& lds, int wave, int lane
         v4i const A = operand(0);
         v4i const C = *reinterpret_cast<v4i const*>(&lds.bias[t][g][0]);
         v4f const Sc = *reinterpret_cast<v4f const*>(&lds.scale[t][g][0]);
+        if (t > 0) pending.convert_into(Hout, t - 1);
+        v4i Dh[4];
         if constexpr (V::FP8_WEIGHTS) {
             v4i const A1 = operand(V::PLANES > 1 ? 1 : 0), A2 = operand(V::PLANES > 2 ? 2 : 0);
             v4i const Z = v4i{ 0, 0, 0, 0 };
+            v4i D1[4], D2[4];
 #pragma unroll
             for (int b = 0; b < 4; ++b) {
-                v4i const D0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
-                v4i const D1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A1, X[b], Z, 0, 0, 0);
-                v4i const D2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(A2, X[b], Z, 0, 0, 0);
-                v4i Dh;
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    Dh[r] = int((((uint32_t(D2[r]) << 6) + uint32_t(D1[r])) << 6) + uint32_t(D0[r]));
-                activate4_h(Dh, Sc, Ha[b][t]);
+                Dh[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
+                D1[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A1, X[b], Z, 0, 0, 0);
+                D2[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A2, X[b], Z, 0, 0, 0);
             }
-        } else {
+            if (t > 0) { interleave<4, 3, 4>(); keep_here(Hout, t - 1); }
+            section_end();
 #pragma unroll
             for (int b = 0; b < 4; ++b)
-                activate4_h(__builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0), Sc, Ha[b][t]);
+#pragma unroll
+                for (int r = 0; r < 4; ++r)                    // 4096*D2 + 64*D1 + D0, wrapping like int32
+                    Dh[b][r] = int((((uint32_t(D2[b][r]) << 6) + uint32_t(D1[b][r])) << 6) + uint32_t(Dh[b][r]));
+        } else {
+#pragma unroll
+            for (int b = 0; b < 4; ++b) Dh[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
+            if (t > 0) { interleave<4, 1, 4>(); keep_here(Hout, t - 1); }
+            section_end();
         }
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            if constexpr (MAGIC) {
+                v4f acc;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    int32_t const bits = Dh[b][r];               // (a copy: bit_cast of a vector element expression reads element 0)
+                    acc[r] = __builtin_bit_cast(float, bits) - 12582912.f;
+                }
+                activate_scale4(acc, Sc, pending.z[b]);
+            } else {
+                activate_scale4(Dh[b], Sc, pending.z[b]);
+            }
+        }
+        section_end();
     }
-    }
+}
+
+// The network for the 64 texels of one wave with layers 1..3 on the fp16 matrix instruction.  `in` is the lane's own
+// texel (lane = 16*b + j).  On return D[b] holds, for lane (j = lane%16, g = lane/16), the accumulators of output
+// channels 4g..4g+3 of texel 16*b + j as floats (exact integers), and S their scales.
+template <class V>
+__device__ __forceinline__ void mlp_forward_f16(LdsT<V>& lds, int wave, int lane, bool l0Magic, uint32_t const (&in)[16], v4f (&D)[4], v4f& S)
+{
+    int const g = lane >> 4;
+    v4i X[4];
+    transpose_inputs<V>(lds, wave, lane, in, X);
+    section_end();
+
+    uint32_t Ha[4][4][2], Hb[4][4][2];
+    PendingTile pending;
     if constexpr (V::FP8_WEIGHTS) {
-        f16_hidden_layer_two_planes<V, V::T0, V::T1>(lds, V::F16_L1, V::T0, lane, Ha, Hb);
-        f16_hidden_layer_two_planes<V, V::T1, V::T2>(lds, V::F16_L2, V::T0 + V::T1, lane, Hb, Ha);
+        first_layer<V, false>(lds, lane, X, Ha, pending);
     } else {
-        f16_hidden_layer<V, V::T0, V::T1>(lds, V::F16_L1, V::T0, lane, Ha, Hb);
-        f16_hidden_layer<V, V::T1, V::T2>(lds, V::F16_L2, V::T0 + V::T1, lane, Hb, Ha);
+        if (l0Magic) first_layer<V, true>(lds, lane, X, Ha, pending);      // uniform
+        else         first_layer<V, false>(lds, lane, X, Ha, pending);
     }
+    f16_hidden_layer<V, V::T0, V::T1, V::FP8_WEIGHTS>(lds, V::F16_L1, V::T0, lane, Ha, Hb, pending);
+    f16_hidden_layer<V, V::T1, V::T2, V::FP8_WEIGHTS>(lds, V::F16_L2, V::T0 + V::T1, lane, Hb, Ha, pending);
 
     constexpr int outTile = V::T0 + V::T1 + V::T2;
     v4f const C = *reinterpret_cast<v4f const*>(&lds.bias[outTile][g][0]);
     S = *reinterpret_cast<v4f const*>(&lds.scale[outTile][g][0]);
+    pending.convert_into(Ha, V::T2 - 1);
 #pragma unroll
     for (int b = 0; b < 4; ++b) D[b] = C;
     f16_tile<V, V::T2>(lds, V::F16_L3, 0, lane, Ha, D);
