@@ -299,6 +299,62 @@ __device__ __forceinline__ void store_tile(Mip const& m, Acc const (&D)[4], v4f 
     }
 }
 
+// The stores of a wave tile at an image edge, of a mip with fewer than sixteen channels or of a pixel format that
+// needs channel-by-channel stores: the general form above, in the mip's format, with the checked conversion (it
+// equals the unchecked one wherever that is allowed).  Not inlined: tiles like these are few, and inlined next to
+// the fast form the six instantiations cost the kernels registers.
+template <class Acc>
+__device__ __attribute__((noinline)) void store_tile_general(DevMip const* mip, Acc D0, Acc D1, Acc D2, Acc D3, v4f S, int x, int y0, int chBase)
+{
+    RunMip const m(*mip);
+    Acc const D[4] = { D0, D1, D2, D3 };
+    if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)  store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS, true>(m, D, S, x, y0, chBase);
+    else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)   store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS, true>(m, D, S, x, y0, chBase);
+    else                                                   store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS, true>(m, D, S, x, y0, chBase);
+}
+
+// The stores of a wave tile that lies inside the image of a mip whose channel count is a multiple of four (the common
+// case): no bounds to test, every lane stores its four channels of all four rows, and the row addresses are one uniform
+// base plus multiples of the row size - a handful of scalar additions instead of a 64-bit product, a test and a
+// branch per row.  x0, y0: first texel of the wave tile; lane = (j, g) holds channels 4g..4g+3 of texel column j.
+template <int FORMAT, bool CHECKED, class Acc, class Mip>
+__device__ __forceinline__ void store_tile_inside(Mip const& m, Acc const (&D)[4], v4f S, int x0, int y0, int j, int g)
+{
+    typedef __attribute__((address_space(1))) uint32_t* DwordPtr;
+    size_t rowBytes;
+    uint32_t laneOff;
+    GlobalOutPtr tile;
+    if (4 * g >= m.numChannels) return;                                          // lanes of channel groups the mip does not have
+    if constexpr (FORMAT == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS) {
+        rowBytes = size_t(m.width) * size_t(m.numChannels) * 2;                  // fp16, a multiple of four channels
+        laneOff = uint32_t(g) * (uint32_t(m.width) * 8u) + uint32_t(j) * 4u;     // (4g * width + 2j) halves
+        tile = (GlobalOutPtr)m.out + (size_t(y0) * rowBytes + size_t(x0) * 4);
+    } else {
+        rowBytes = size_t(m.outRowPitch);
+        laneOff = uint32_t(j) * uint32_t(m.outPixelStride) + uint32_t(g) * (FORMAT == NTC_HIP_DEV_OUT_FP16_PIXELS ? 8u : 4u);
+        tile = (GlobalOutPtr)m.out + (size_t(y0) * rowBytes + size_t(x0) * size_t(m.outPixelStride));
+    }
+    uint32_t laneOff2 = laneOff + uint32_t(m.width) * 4u;                        // planar: the lane's second channel pair
+    // The offsets stay 32-bit values of this tile (hoisted out of the tile loop they become 64-bit lane addresses, and
+    // the stores lose their "scalar base + 32-bit lane offset" form).
+    asm volatile("" : "+v"(laneOff), "+v"(laneOff2));
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        uint32_t const h01 = to_half2_bits<CHECKED>(float(D[b][0]) * S[0], float(D[b][1]) * S[1]);
+        uint32_t const h23 = to_half2_bits<CHECKED>(float(D[b][2]) * S[2], float(D[b][3]) * S[3]);
+        GlobalOutPtr const row = tile + size_t(b) * rowBytes;
+        if constexpr (FORMAT == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS) {
+            *reinterpret_cast<DwordPtr>(row + laneOff) = h01;
+            *reinterpret_cast<DwordPtr>(row + laneOff2) = h23;
+        } else if constexpr (FORMAT == NTC_HIP_DEV_OUT_FP16_PIXELS) {
+            *reinterpret_cast<__attribute__((address_space(1))) u32x2*>(row + laneOff) = u32x2{ h01, h23 };
+        } else {
+            v2h const a = __builtin_bit_cast(v2h, h01), c = __builtin_bit_cast(v2h, h23);
+            *reinterpret_cast<DwordPtr>(row + laneOff) = pack_unorm8(c[1], 3, pack_unorm8(c[0], 2, pack_unorm8(a[1], 1, pack_unorm8(a[0], 0, 0u))));
+        }
+    }
+}
+
 // One row of a wave tile in the mip's own format (checked conversion): the stores of the int8-only network path,
 // which produces the wave's four rows one after the other.
 template <class AccV, class Mip>

@@ -196,6 +196,12 @@ __device__ __forceinline__ uint32_t halves_of_bytes(uint32_t v, int firstByte)  
     return __builtin_bit_cast(uint32_t, h);
 }
 
+// The lane's number in its wave from the execution mask: no register has to keep the thread id alive for it.
+__device__ __forceinline__ int lane_id()
+{
+    return int(__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)));
+}
+
 // Copies the int8 blob (src/WeightLayout.cpp:42-49: matrices, then fp32 scales, then int32
 // biases; W[c*IN + k]) into LDS in MFMA operand order.  Returns kStagedF16 when layers 1..3 were
 // staged for the fp16 matrix instruction (see mlp_forward_f16): that needs, for every channel of
@@ -209,7 +215,7 @@ __device__ __forceinline__ uint32_t halves_of_bytes(uint32_t v, int firstByte)  
 constexpr int kStagedF16 = 1, kOutputsBounded = 2, kL0Magic = 4;
 constexpr int32_t kMagicBits = 0x4B400000;                   // 12582912.0f = 1.5 * 2^23
 template <class V>
-__device__ int stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
+__device__ __attribute__((noinline)) int stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob, int const tid)
 {
     constexpr int ins[4]   = { V::IN, V::H0, V::H1, V::H2 };
     constexpr int tiles[4] = { V::T0, V::T1, V::T2, V::T3 };
@@ -221,7 +227,7 @@ __device__ int stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
         int tileBase = 0, chanBase = 0;
 #pragma unroll
         for (int l = 0; l < 4; ++l) {
-            for (int e = threadIdx.x; e < tiles[l] * 16; e += blockDim.x) {
+            for (int e = tid; e < tiles[l] * 16; e += V::THREADS) {
                 int const r = e & 3, g = (e >> 2) & 3, t = e >> 4;
                 int const c = chanBase + 16 * t + 4 * g + r;
                 lds.scale[tileBase + t][g][r] = reinterpret_cast<float const*>(blob + V::SCALE_OFF)[c];
@@ -233,7 +239,7 @@ __device__ int stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
     }
 
     // int8 tiles of layer 0 (three planes for e4m3 weights)
-    for (int e = threadIdx.x; e < V::T0 * 64 * 4; e += blockDim.x) {
+    for (int e = tid; e < V::T0 * 64 * 4; e += V::THREADS) {
         int const d = e & 3, lane = (e >> 2) & 63, t = e >> 8;
         int const i = lane & 15, g = lane >> 4;
         // k-slot (g, 4d+r) = input 16g+4d+r
@@ -253,8 +259,8 @@ __device__ int stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
     int64_t shifted = 0;
     bool twoPlanes = false;
     int slotTile = 0, slotG = 0, slotR = 0;
-    if (threadIdx.x < V::LATE_CHANNELS) {
-        int const c = threadIdx.x;
+    if (tid < V::LATE_CHANNELS) {
+        int const c = tid;
         int const l = c < V::H1 ? 1 : (c < V::H1 + V::H2 ? 2 : 3);
         int const row = c - (l == 1 ? 0 : (l == 2 ? V::H1 : V::H1 + V::H2));
         int const in = l == 1 ? V::H0 : (l == 2 ? V::H1 : V::H2);
@@ -296,32 +302,47 @@ __device__ int stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
         slotG = (row >> 2) & 3;
         slotR = row & 3;
     }
-    bool const useF16 = __syncthreads_and(fits ? 1 : 0) != 0;     // also orders the bias writes above
-    bool const outputsBounded = __syncthreads_and(bounded ? 1 : 0) != 0;
-    bool l0Magic = false;
+    bool small = true;
     if constexpr (!V::FP8_WEIGHTS) {
-        bool small = true;
-        if (threadIdx.x < V::H0) {
-            int32_t const b = reinterpret_cast<int32_t const*>(blob + V::BIAS_OFF)[threadIdx.x];
+        if (tid < V::H0) {
+            int32_t const b = reinterpret_cast<int32_t const*>(blob + V::BIAS_OFF)[tid];
             small = b >= -3100000 && b <= 3100000;
         }
-        l0Magic = (__syncthreads_and(small ? 1 : 0) != 0) && useF16;
-        if (l0Magic && threadIdx.x < V::H0) {
-            int const c = threadIdx.x;
+    }
+    // The three conditions, each over every thread of the workgroup: a ballot per wave, one LDS atomic per wave on a
+    // word of the (idle) transposition buffer.  The barriers also order the bias writes above.  (The runtime's
+    // workgroup reduction would do, but as a library call it needs the caller's thread ids kept in a vector register
+    // for the whole kernel.)
+    uint32_t* const flags = &lds.in[0][0][0];
+    if (tid == 0) *flags = 7u;
+    __syncthreads();
+    {
+        uint32_t const mine = (__all(fits ? 1 : 0) ? 1u : 0u) | (__all(bounded ? 1 : 0) ? 2u : 0u) | (__all(small ? 1 : 0) ? 4u : 0u);
+        if ((tid & 63) == 0) atomicAnd(flags, mine);
+    }
+    __syncthreads();
+    uint32_t const all = __builtin_amdgcn_readfirstlane(*flags);
+    __syncthreads();                                         // every wave has read the word before the buffer is used again
+    bool const useF16 = (all & 1u) != 0, outputsBounded = (all & 2u) != 0;
+    bool l0Magic = false;
+    if constexpr (!V::FP8_WEIGHTS) {
+        l0Magic = (all & 4u) != 0 && useF16;
+        if (l0Magic && tid < V::H0) {
+            int const c = tid;
             lds.bias[c >> 4][(c >> 2) & 3][c & 3] += kMagicBits;
         }
     }
     constexpr int base[4] = { 0, V::F16_L1, V::F16_L2, V::F16_L3 };
     uint32_t* const late32 = reinterpret_cast<uint32_t*>(lds.late);
     if (useF16) {
-        if (threadIdx.x < V::LATE_CHANNELS) {
+        if (tid < V::LATE_CHANNELS) {
             if constexpr (V::FP8_WEIGHTS) {
                 if (twoPlanes) lds.biasLo[slotTile][slotG][slotR] = float(shifted & 1023) * 0x1p-24f;
             }
             // sums run over (q + 113) * 2^-24 (see activate_scale4): every term, this start value included, is an
             // integer below 2^24 times 2^-24, exact in fp32; the scale takes the 2^24 back
             lds.bias[slotTile][slotG][slotR] = __builtin_bit_cast(int32_t, float(twoPlanes ? (shifted >> 10) : shifted) * 0x1p-24f);
-            lds.scale[slotTile][slotG][slotR] = reinterpret_cast<float const*>(blob + V::SCALE_OFF)[V::H0 + threadIdx.x] * 0x1p24f;
+            lds.scale[slotTile][slotG][slotR] = reinterpret_cast<float const*>(blob + V::SCALE_OFF)[V::H0 + tid] * 0x1p24f;
         }
         // fp16 blocks.  Lane (i, kg) of the block of output tile t and input-tile pair p holds
         // W[16t + i][16*(2p + e/4) + 4*kg + e%4], e = 0..7: the channels lane (j, kg) of the
@@ -332,7 +353,7 @@ __device__ int stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
             int const inTiles = tiles[l - 1], pairs = inTiles / 2, per = V::f16_units(inTiles);
             int const planeDwords = tiles[l] * per * 4;
             // one work item = one (output tile, input tile, lane): 4 weights -> 2 dwords (per plane)
-            for (int e = threadIdx.x; e < tiles[l] * inTiles * 64; e += blockDim.x) {
+            for (int e = tid; e < tiles[l] * inTiles * 64; e += V::THREADS) {
                 int const lane = e & 63, rest = e >> 6;
                 int const ti = rest % inTiles, t = rest / inTiles;
                 int const i = lane & 15, kg = lane >> 4;
@@ -360,7 +381,7 @@ __device__ int stage_weights(LdsT<V>& lds, uint8_t const* __restrict__ blob)
 #pragma unroll
         for (int l = 1; l < 4; ++l) {
             int const in = ins[l];
-            for (int e = threadIdx.x; e < tiles[l] * 64 * 4; e += blockDim.x) {
+            for (int e = tid; e < tiles[l] * 64 * 4; e += V::THREADS) {
                 int const d = e & 3, lane = (e >> 2) & 63, t = e >> 8;
                 int const i = lane & 15, g = lane >> 4;
                 // k-slot (g, 4d+r) = channel 16d+4g+r of the previous layer
@@ -922,24 +943,26 @@ __device__ __forceinline__ void interleave()
 // The scaled outputs of one output tile whose conversion is pending, [block b][r].
 struct PendingTile {
     float z[4][4];
+    template <int FIRST = 0, int COUNT = 4>
     __device__ __forceinline__ void convert_into(uint32_t (&H)[4][4][2], int tile) const
     {
 #pragma unroll
-        for (int b = 0; b < 4; ++b) activate_pack4(z[b], H[b][tile]);
+        for (int b = FIRST; b < FIRST + COUNT; ++b) activate_pack4(z[b], H[b][tile]);
     }
 };
 
-// A use of tile `tile` of H at this place (the end of the section that converted it): without one the compiler sinks
-// the conversions to their first real use, the next layer.
+// A use of tile `tile` of H (blocks FIRST .. FIRST + COUNT - 1) at this place, the end of the section that converted
+// it: without one the compiler sinks the conversions to their first real use, the next layer.
+template <int FIRST = 0, int COUNT = 4>
 __device__ __forceinline__ void keep_here(uint32_t (&H)[4][4][2], int tile)
 {
 #pragma unroll
-    for (int b = 0; b < 4; ++b) asm volatile("" : "+v"(H[b][tile][0]), "+v"(H[b][tile][1]));
+    for (int b = FIRST; b < FIRST + COUNT; ++b) asm volatile("" : "+v"(H[b][tile][0]), "+v"(H[b][tile][1]));
 }
 
-// acc[b] += W(tile t of the layer at `base`) * H[b], for the four 16-texel blocks of the wave.
-template <class V, int IN_TILES>
-__device__ __forceinline__ void f16_tile(LdsT<V> const& lds, int base, int t, int lane, uint32_t const (&H)[4][4][2], v4f (&acc)[4])
+// acc[b - FIRST] += W(tile t of the layer at `base`) * H[b] for the 16-texel blocks b = FIRST .. FIRST + COUNT - 1 of the wave.
+template <class V, int IN_TILES, int FIRST = 0, int COUNT = 4>
+__device__ __forceinline__ void f16_tile(LdsT<V> const& lds, int base, int t, int lane, uint32_t const (&H)[4][4][2], v4f (&acc)[COUNT])
 {
     constexpr int PAIRS = IN_TILES / 2, PER = V::f16_units(IN_TILES);
     uint4 const* const block = lds.late + base + t * PER;
@@ -948,9 +971,9 @@ __device__ __forceinline__ void f16_tile(LdsT<V> const& lds, int base, int t, in
         for (int p = 0; p < PAIRS; ++p) {
             v8h const A = __builtin_bit_cast(v8h, block[p * 64 + lane]);
 #pragma unroll
-            for (int b = 0; b < 4; ++b) {
+            for (int b = FIRST; b < FIRST + COUNT; ++b) {
                 uint4 const h = make_uint4(H[b][2 * p][0], H[b][2 * p][1], H[b][2 * p + 1][0], H[b][2 * p + 1][1]);
-                acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, __builtin_bit_cast(v8h, h), acc[b], 0, 0, 0);
+                acc[b - FIRST] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, __builtin_bit_cast(v8h, h), acc[b - FIRST], 0, 0, 0);
             }
         }
     } else {
@@ -970,9 +993,9 @@ __device__ __forceinline__ void f16_tile(LdsT<V> const& lds, int base, int t, in
             }
             v4h const A = __builtin_bit_cast(v4h, a);
 #pragma unroll
-            for (int b = 0; b < 4; ++b) {
+            for (int b = FIRST; b < FIRST + COUNT; ++b) {
                 uint2 const h = make_uint2(H[b][ti][0], H[b][ti][1]);
-                acc[b] = __builtin_amdgcn_mfma_f32_16x16x16f16(A, __builtin_bit_cast(v4h, h), acc[b], 0, 0, 0);
+                acc[b - FIRST] = __builtin_amdgcn_mfma_f32_16x16x16f16(A, __builtin_bit_cast(v4h, h), acc[b - FIRST], 0, 0, 0);
             }
         }
     }
@@ -996,31 +1019,41 @@ __device__ __forceinline__ void f16_hidden_layer(LdsT<V> const& lds, int base, i
     for (int t = 0; t < OUT_TILES; ++t) {
         v4f const C = *reinterpret_cast<v4f const*>(&lds.bias[tileBase + t][g][0]);
         v4f const Sc = *reinterpret_cast<v4f const*>(&lds.scale[tileBase + t][g][0]);
-        if (t == 0) pending.convert_into(Hin, IN_TILES - 1);
-        else        pending.convert_into(Hout, t - 1);
-        v4f acc[4] = { C, C, C, C };
-        f16_tile<V, IN_TILES>(lds, base, t, lane, Hin, acc);
         if constexpr (TWO_PLANES) {
+            // The upper plane's matrix instructions carry the pending conversions; the lower plane's follow in a section
+            // of their own, so that its accumulators take the registers the converted values have left.
             if constexpr (V::FP8_WEIGHTS) {                  // (biasLo exists in those variants only)
                 v4f const Clo = *reinterpret_cast<v4f const*>(&lds.biasLo[tileBase + t][g][0]);
-                v4f lo[4] = { Clo, Clo, Clo, Clo };
-                f16_tile<V, IN_TILES>(lds, base + PLANE, t, lane, Hin, lo);
-                interleave<8, MATRIX / 8, 2>();
+                if (t == 0) pending.convert_into(Hin, IN_TILES - 1);
+                else        pending.convert_into(Hout, t - 1);
+                v4f acc[4] = { C, C, C, C };
+                f16_tile<V, IN_TILES>(lds, base, t, lane, Hin, acc);
+                interleave<8, MATRIX / 16, 2>();
                 if (t > 0) keep_here(Hout, t - 1);
                 section_end();
+                v4f lo[4] = { Clo, Clo, Clo, Clo };
+                f16_tile<V, IN_TILES>(lds, base + PLANE, t, lane, Hin, lo);
+                section_end();
 #pragma unroll
-                for (int b = 0; b < 4; ++b)
+                for (int b = 0; b < 4; ++b) {
 #pragma unroll
                     for (int r = 0; r < 4; ++r) acc[b][r] = __builtin_fmaf(acc[b][r], 1024.f, lo[b][r]);
+                    activate_scale4(acc[b], Sc, pending.z[b]);
+                }
+                section_end();
             }
         } else {
+            if (t == 0) pending.convert_into(Hin, IN_TILES - 1);
+            else        pending.convert_into(Hout, t - 1);
+            v4f acc[4] = { C, C, C, C };
+            f16_tile<V, IN_TILES>(lds, base, t, lane, Hin, acc);
             interleave<8, (MATRIX >= 8 ? MATRIX / 8 : 1), 2>();
             if (t > 0) keep_here(Hout, t - 1);
             section_end();
-        }
 #pragma unroll
-        for (int b = 0; b < 4; ++b) activate_scale4(acc[b], Sc, pending.z[b]);
-        section_end();
+            for (int b = 0; b < 4; ++b) activate_scale4(acc[b], Sc, pending.z[b]);
+            section_end();
+        }
     }
 }
 
@@ -1040,31 +1073,42 @@ __device__ __forceinline__ void first_layer(LdsT<V> const& lds, int lane, v4i co
         v4i const A = operand(0);
         v4i const C = *reinterpret_cast<v4i const*>(&lds.bias[t][g][0]);
         v4f const Sc = *reinterpret_cast<v4f const*>(&lds.scale[t][g][0]);
-        if (t > 0) pending.convert_into(Hout, t - 1);
-        v4i Dh[4];
         if constexpr (V::FP8_WEIGHTS) {
+            // three planes: two blocks at a time, so that twenty-four accumulator registers are live, not forty-eight
             v4i const A1 = operand(V::PLANES > 1 ? 1 : 0), A2 = operand(V::PLANES > 2 ? 2 : 0);
             v4i const Z = v4i{ 0, 0, 0, 0 };
-            v4i D1[4], D2[4];
+            auto const half = [&](auto first) __attribute__((always_inline)) {
+                constexpr int FIRST = decltype(first)::value;
+                if (t > 0) pending.template convert_into<FIRST, 2>(Hout, t - 1);
+                v4i D0[2], D1[2], D2[2];
 #pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                Dh[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
-                D1[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A1, X[b], Z, 0, 0, 0);
-                D2[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A2, X[b], Z, 0, 0, 0);
-            }
-            if (t > 0) { interleave<4, 3, 4>(); keep_here(Hout, t - 1); }
-            section_end();
+                for (int k = 0; k < 2; ++k) {
+                    D0[k] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[FIRST + k], C, 0, 0, 0);
+                    D1[k] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A1, X[FIRST + k], Z, 0, 0, 0);
+                    D2[k] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A2, X[FIRST + k], Z, 0, 0, 0);
+                }
+                if (t > 0) { interleave<2, 3, 4>(); keep_here<FIRST, 2>(Hout, t - 1); }
+                section_end();
 #pragma unroll
-            for (int b = 0; b < 4; ++b)
+                for (int k = 0; k < 2; ++k) {
+                    v4i Dh;
 #pragma unroll
-                for (int r = 0; r < 4; ++r)                    // 4096*D2 + 64*D1 + D0, wrapping like int32
-                    Dh[b][r] = int((((uint32_t(D2[b][r]) << 6) + uint32_t(D1[b][r])) << 6) + uint32_t(Dh[b][r]));
-        } else {
-#pragma unroll
-            for (int b = 0; b < 4; ++b) Dh[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
-            if (t > 0) { interleave<4, 1, 4>(); keep_here(Hout, t - 1); }
-            section_end();
+                    for (int r = 0; r < 4; ++r)                // 4096*D2 + 64*D1 + D0, wrapping like int32
+                        Dh[r] = int((((uint32_t(D2[k][r]) << 6) + uint32_t(D1[k][r])) << 6) + uint32_t(D0[k][r]));
+                    activate_scale4(Dh, Sc, pending.z[FIRST + k]);
+                }
+                section_end();
+            };
+            half(std::integral_constant<int, 0>{});
+            half(std::integral_constant<int, 2>{});
+            continue;
         }
+        if (t > 0) pending.convert_into(Hout, t - 1);
+        v4i Dh[4];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) Dh[b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A, X[b], C, 0, 0, 0);
+        if (t > 0) { interleave<4, 1, 4>(); keep_here(Hout, t - 1); }
+        section_end();
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
             if constexpr (MAGIC) {
@@ -1162,14 +1206,20 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
             v4f D[4];
             v4f S;
             mlp_forward_f16<V>(lds, wave, lane, (staged & kL0Magic) != 0, in, D, S);
-            if (staged & kOutputsBounded) {
-                if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)  store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS, false>(m, D, S, x0 + j, y0, 4 * g);
-                else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)   store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS, false>(m, D, S, x0 + j, y0, 4 * g);
-                else                                                   store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS, false>(m, D, S, x0 + j, y0, 4 * g);
+            // a wave tile inside the image, channels in whole groups of four (pixel formats: vector stores possible),
+            // takes the stores without tests
+            bool const inside = x0 + 16 <= m.width && y0 + 4 <= m.height && (m.numChannels & 3) == 0
+                             && (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS || m.vectorStores);
+            if (!inside) {
+                store_tile_general(&m.full, D[0], D[1], D[2], D[3], S, x0 + j, y0, 4 * g);
+            } else if (staged & kOutputsBounded) {
+                if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)  store_tile_inside<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS, false>(m, D, S, x0, y0, j, g);
+                else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)   store_tile_inside<NTC_HIP_DEV_OUT_FP16_PIXELS, false>(m, D, S, x0, y0, j, g);
+                else                                                   store_tile_inside<NTC_HIP_DEV_OUT_UNORM8_PIXELS, false>(m, D, S, x0, y0, j, g);
             } else {
-                if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)  store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, x0 + j, y0, 4 * g);
-                else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)   store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
-                else                                                   store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
+                if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)  store_tile_inside<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS, true>(m, D, S, x0, y0, j, g);
+                else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)   store_tile_inside<NTC_HIP_DEV_OUT_FP16_PIXELS, true>(m, D, S, x0, y0, j, g);
+                else                                                   store_tile_inside<NTC_HIP_DEV_OUT_UNORM8_PIXELS, true>(m, D, S, x0, y0, j, g);
             }
         } else {
             // every layer on the int8 matrix instruction: one 16-texel block (= one image row of the tile) at a time
@@ -1202,7 +1252,7 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
             if (mips[k].weights != blob) { segEnd = mips[k].tileStart; break; }
         if (blob != stagedBlob) {                            // uniform across the workgroup
             __syncthreads();                                 // every wave has left the previous segment's weights
-            staged = stage_weights<V>(lds, blob);
+            staged = __builtin_amdgcn_readfirstlane(stage_weights<V>(lds, blob, wave * 64 + lane_id()));
             stagedBlob = blob;
             __syncthreads();                                 // also publishes the tables built above
         }
@@ -1266,7 +1316,7 @@ query_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __res
         lds.lut2[threadIdx.x & 0xffu] = (x * 85u) ^ 0x80808080u;
     }
     build_posenc_tables<V>(lds);
-    int const staged = stage_weights<V>(lds, mips[0].weights);
+    int const staged = __builtin_amdgcn_readfirstlane(stage_weights<V>(lds, mips[0].weights, wave * 64 + lane_id()));
     bool const useF16 = (staged & kStagedF16) != 0;
     __syncthreads();
 
