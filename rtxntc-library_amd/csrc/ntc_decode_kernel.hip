@@ -1170,9 +1170,14 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     int const member = wave >> 2;                            // which quartet this wave belongs to
     int const j = lane & 15, g = lane >> 4;
 
-    // contiguous share of the tile list for this workgroup
+    // Contiguous share of the tile list for this workgroup.  Workgroups are dealt to the eight dies (XCDs) of the
+    // device in turn, and each die has a cache of its own: the shares are numbered so that a die's workgroups hold
+    // neighbouring shares - one eighth of the list per die - and the grid rows that vertically adjacent shares both
+    // read come from memory once per die, not once per share.
     int const per = (totalTiles + gridDim.x - 1) / gridDim.x;
-    int const tileBegin = blockIdx.x * per;
+    constexpr int kDies = 8;
+    int const share = (gridDim.x % kDies == 0) ? int(blockIdx.x % kDies) * int(gridDim.x / kDies) + int(blockIdx.x / kDies) : int(blockIdx.x);
+    int const tileBegin = share * per;
     int const tileEnd = min(totalTiles, tileBegin + per);
 
     {   // 2-bit code bytes -> input bytes: code q maps to 85*q - 128 (255/3 = 85)
