@@ -214,3 +214,44 @@ def test_single_mip_beyond_4_gib(ntc, device, oracle):
     # nothing was written outside the image: the byte after the last row of a slightly larger buffer is not there to check,
     # so check the other end of the same property: the first and last texel differ from the fill pattern
     assert not np.all(case.d_output.download_range(0, 64) == 0xCD) and not np.all(case.d_output.download_range(case.output_bytes - 64, 64) == 0xCD)
+
+
+def test_batch_of_eight_2048_sets_row_bands_equal_checker(ntc, device, oracle):
+    """Config 2 at full size, the two largest mips: bands of rows of mips 0 and 1 of the first and the last set of the
+    batch (top, middle - where the shares of two workgroups meet - and bottom) against the checker, unorm8."""
+    spec = ntc.presets.spec_cfg2()
+    cases = [cfg_case(ntc, spec, 2048, 2048, 12, 12, ntc.abi.OUT_UNORM8_PIXELS, seed=200 + i) for i in range(8)]
+    device.decode([c.device_set(device) for c in cases])
+    device.synchronize()
+    for i in (0, 7):
+        got = cases[i].d_output.download()
+        host = cases[i].host_set()
+        for m in (0, 1):
+            mip = cases[i].mips[m]
+            row_bytes = mip.width * 12
+            for y0 in (0, mip.height // 2 - 10, mip.height - 20):
+                oracle.ntc_oracle_decode_rows(host.desc, m, y0, y0 + 20, 16)
+                a, b = mip.outOffset + y0 * row_bytes, mip.outOffset + (y0 + 20) * row_bytes
+                assert np.array_equal(host.output[a:b], got[a:b]), (i, m, y0)
+
+
+def test_fp8_network_4096_unorm8_row_bands_equal_checker(ntc, device, oracle):
+    """The FP8 network's 4096^2 set decoded to unorm8 pixels: bands of rows of mip 0 and every mip from 512^2 down
+    against the checker."""
+    spec = ntc.presets.spec_ref092_fp8(16)
+    mips, latent_bytes = ntc.presets.mips_ref092(spec, 4096, 4096, 13, 2)
+    case = Case(ntc, spec, mips, latent_bytes, 16, ntc.abi.OUT_UNORM8_PIXELS, seed=5, weights=ntc.synth.make_fp8_weights(spec, 6))
+    dset = case.device_set(device)
+    device.decode([dset])
+    device.synchronize()
+    got = case.d_output.download()
+    host = case.host_set()
+    row_bytes = 4096 * 16
+    for y0 in (0, 2046, 4096 - 12):
+        oracle.ntc_oracle_decode_rows(host.desc, 0, y0, y0 + 12, 16)
+        assert np.array_equal(host.output[y0 * row_bytes:(y0 + 12) * row_bytes], got[y0 * row_bytes:(y0 + 12) * row_bytes]), y0
+    for m in range(3, 13):
+        oracle.ntc_oracle_decode_rows(host.desc, m, 0, case.mips[m].height, 16)
+    start = case.mips[3].outOffset
+    assert np.array_equal(host.output[start:], got[start:])
+    assert len(np.unique(got[:12 * row_bytes])) > 50
