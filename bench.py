@@ -40,8 +40,22 @@ def cpu_threads():
     return (min(share, total) if share > 0 else total), total
 
 
+KERNEL_SOURCES = ("rtxntc-library_amd/csrc/ntc_decode_kernel.hip", "rtxntc-library_amd/csrc/ntc_decode_device.h")
+
+
+def kernel_source_digest():
+    """sha256 over the sources of the decode kernel: the counters file records the one it was measured on."""
+    import hashlib
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
 def measured_counters(workload, fmt_name):
-    """Counter figures for this workload from profiles/decode_kernel_counters.json, or None."""
+    """Counter figures for this workload from profiles/decode_kernel_counters.json, or None.  `stale` is set when the
+    kernel's sources are not the ones the counters were taken on."""
     try:
         with open(COUNTERS_FILE) as f:
             table = json.load(f)
@@ -49,8 +63,11 @@ def measured_counters(workload, fmt_name):
         return None
     entry = table.get("workloads", {}).get(f"{workload}_{fmt_name}")
     if entry:
-        entry = dict(entry, source=f"profiles/{os.path.basename(COUNTERS_FILE)} (commit {table.get('commit', '?')})",
-                     issue_rates_ns=table.get("issue_rates_ns"))
+        try:
+            stale = table.get("kernel_source_sha256") != kernel_source_digest()
+        except OSError:
+            stale = True
+        entry = dict(entry, source=f"profiles/{os.path.basename(COUNTERS_FILE)}", stale=stale)
     return entry
 
 
@@ -221,8 +238,9 @@ def main():
         mips, latent_bytes = P.mips_ref092(spec, size, size, P.full_mip_count(size, size), 2)
         cases = [Case(ntc, spec, mips, latent_bytes, 16, fmt, seed=5, weights=ntc.synth.make_fp8_weights(spec, 6, weight_sigma=args.fp8_weight_sigma))]
         widths, channels, latent_b = (46, 64, 48, 32, 16), 16, 44738560 / 22369621.0
+        planes = "one weight plane per hidden layer" if args.fp8_weight_sigma <= 0.5 else ("two weight planes per hidden layer" if args.fp8_weight_sigma <= 20 else "three weight planes per hidden layer")
         what = (f"LibNTC 0.9.2 geometry with the FP8 network: {size}x{size}, full mip chain, grid scale 2, 16 features, "
-                "MLP 48(46)-64-48-32-16, e4m3 hidden layers (GenericFP8 blob)")
+                f"MLP 48(46)-64-48-32-16, e4m3 hidden layers (GenericFP8 blob), weights drawn with sigma {args.fp8_weight_sigma:g}: {planes}")
     else:
         size = args.size or 8192
         if wl == "cfg4fp8":
@@ -296,6 +314,8 @@ def main():
     ms_per_step = wall / args.steps * 1e3
 
     kernel_ms = run_timed(args.steps)                 # the same K launches again, HIP events on the launch stream
+    singles = sorted(run_timed(1) for _ in range(min(args.steps, 100)))     # launches timed one at a time: median and minimum
+    median_ms, min_ms = singles[len(singles) // 2], singles[0]
     gtexels = texels / (ms_per_step * 1e-3) / 1e9
     achieved_gbs = texels * bytes_per_texel / (kernel_ms * 1e-3) / 1e9
     achieved_tops = texels * ops_per_texel / (kernel_ms * 1e-3) / 1e12
@@ -336,43 +356,34 @@ def main():
             cpu = {"value": n / t / 1e9, "unit": "Gtexels/s", "cores": cores, "host_cpus": host_cpus, "kind": "port",
                    "sample": f"the first {n} queries of the same list, {t:.1f} s"}
 
-    # Ceilings of the kernel, lowest first decides `bound`: HBM (algorithmic bytes), int8 MFMA (algorithmic
-    # operations), and instruction issue.  The issue ceiling is what the kernel's own instruction stream would take
-    # if every instruction issued at the rate it reaches in isolation (profiles/valu_issue_rates_mi355x.md: plain
-    # fp32 / 32-bit integer instructions, the slower conversions / packed 16-bit / three-operand integer ones, and
-    # matrix instructions, which plain fp32 instructions do not overlap with): per 64-texel wave tile and SIMD,
-    #   SQ_INSTS_VALU x (share of plain ones x their ns + the rest x theirs) + SQ_INSTS_MFMA x their ns,
-    # with the instruction counts from the counters and the share from the kernel's assembly.
+    # Two roofs, both from algorithmic work over the kernel's HIP-event time: HBM (output bytes + latent bits) and dense
+    # int8 MFMA (operations of the un-padded network).  `bound` names the lower roof, the one that binds; `frac` is the
+    # fraction of it.  Instruction counts per texel come from the counters file when it matches the kernel's sources.
     counters = None if args.size else measured_counters(wl, fmt_name)
-    rate = texels / (kernel_ms * 1e-3) / 1e9
     fracs = {"hbm": achieved_gbs / HBM_PEAK_GBS, "mfma": achieved_tops / INT8_PEAK_TOPS}
-    valu = {}
-    if counters and counters.get("valu_ops_per_texel") and counters.get("issue_rates_ns"):
-        rates = counters["issue_rates_ns"]
-        mfma_per_tile = counters.get("SQ_INSTS_MFMA", 0) * 64 / counters["texels_per_launch"]
-        share = counters["valu_plain_share"]
-        tile_ns = counters["valu_ops_per_texel"] * (share * rates["plain"] + (1.0 - share) * rates["other"]) + mfma_per_tile * rates["matrix"]
-        ceiling = dev.compute_units * 4 * 64 / tile_ns                 # Gtexels/s: four SIMDs a CU, 64 texels a wave tile
-        fracs["valu"] = rate / ceiling
-        valu = {"valu_ops_per_texel": counters["valu_ops_per_texel"], "mfma_per_wave_tile": mfma_per_tile,
-                "valu_plain_share": share, "issue_rates_ns": rates,
-                "issue_ns_per_wave_tile_model": tile_ns, "issue_ns_per_wave_tile_measured": dev.compute_units * 4 * 64 / rate,
-                "valu_ceiling_gtexels": ceiling, "valu_frac": fracs["valu"], "counters_source": counters["source"]}
+    roofs = {"hbm": HBM_PEAK_GBS * 1e9 / bytes_per_texel / 1e9, "mfma": INT8_PEAK_TOPS * 1e12 / ops_per_texel / 1e9}   # Gtexels/s
+    bound = min(roofs, key=roofs.get)
+    issue = {}
+    if counters and not counters["stale"]:
+        issue = {k: counters[k] for k in ("valu_ops_per_texel", "mfma_per_wave_tile", "slow_valu_per_wave_tile",
+                                          "SQ_ACTIVE_INST_VALU2_per_VALU", "summary") if k in counters}
     line = {
         "metric": "decoded Gtexels/s, 4096^2 16-ch set, 64-48-32 int8; % of int8-MFMA/HBM roof",
         "value": gtexels, "unit": "Gtexels/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": ms_per_step, "ms_per_step_median": median_ms, "ms_per_step_min": min_ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8", "data": "synthetic",
         "config": {"workload": f"{what}, {fmt_name} output, {texels} texels per step",
                    "device": dev.name, "compute_units": dev.compute_units, "settle_ms": args.settle_ms},
-        # achieved / peak / frac: the HBM roof (algorithmic bytes over the kernel's HIP-event time), the lower of
-        # the two roofs the metric names; `bound` names the ceiling the kernel actually runs closest to.
-        "roofline": {"bound": max(fracs, key=fracs.get), "achieved": achieved_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": fracs["hbm"],
-                     # HBM bytes per launch from the FETCH_SIZE + WRITE_SIZE counters
-                     "traffic": counters.get("hbm_traffic_bytes") if counters else None,
-                     "kernel_ms": kernel_ms, "bytes_per_texel": bytes_per_texel,
-                     "hbm_frac": fracs["hbm"], "mfma_achieved_tops": achieved_tops, "mfma_frac": fracs["mfma"], **valu},
+        "roofline": {"bound": bound, "achieved": achieved_gbs if bound == "hbm" else achieved_tops, "peak": HBM_PEAK_GBS if bound == "hbm" else INT8_PEAK_TOPS,
+                     "unit": "GB/s" if bound == "hbm" else "TOP/s", "frac": fracs[bound],
+                     # HBM bytes per launch from the FETCH_SIZE + WRITE_SIZE counters (null when the kernel's sources
+                     # have changed since they were taken)
+                     "traffic": counters.get("hbm_traffic_bytes") if counters and not counters["stale"] else None,
+                     "counters_stale": bool(counters and counters["stale"]),
+                     "kernel_ms": kernel_ms, "bytes_per_texel": bytes_per_texel, "roof_gtexels": roofs,
+                     "hbm_achieved_gbs": achieved_gbs, "hbm_frac": fracs["hbm"],
+                     "mfma_achieved_tops": achieved_tops, "mfma_frac": fracs["mfma"], **issue},
         "cpu_baseline": cpu,
     }
     print(json.dumps(line))
