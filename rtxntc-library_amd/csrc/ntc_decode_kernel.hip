@@ -220,7 +220,21 @@ __device__ __attribute__((noinline)) int stage_weights(LdsT<V>& lds, uint8_t con
     constexpr int ins[4]   = { V::IN, V::H0, V::H1, V::H2 };
     constexpr int tiles[4] = { V::T0, V::T1, V::T2, V::T3 };
     constexpr int woff[4]  = { 0, V::W1_OFF, V::W2_OFF, V::W3_OFF };
-    uint32_t const* blob32 = reinterpret_cast<uint32_t const*>(blob);
+    // The blob first goes into LDS as it is (the transposition buffers are idle now), in one pass of coalesced loads:
+    // everything below - the row sums above all, one thread per channel walking its row - then reads LDS instead of
+    // following a chain of loads from memory.
+    constexpr int kBlobDwords = (V::BIAS_OFF + 4 * V::TOTAL_OUT) / 4;
+    static_assert(sizeof(lds.in) >= size_t(kBlobDwords + 4) * 4, "the blob fits the transposition buffers");
+    uint32_t* const flags = &lds.in[0][0][0];                  // one word for the workgroup's flags, then the blob
+    uint32_t* const raw32 = flags + 4;
+    {
+        uint32_t const* const src = reinterpret_cast<uint32_t const*>(blob);
+        for (int e = tid; e < kBlobDwords; e += V::THREADS) raw32[e] = src[e];
+        if (tid == 0) *flags = 7u;
+    }
+    __syncthreads();
+    uint32_t const* const blob32 = raw32;
+    uint8_t const* const blobBytes = reinterpret_cast<uint8_t const*>(raw32);
 
     // scales and biases of every layer, in D-register order
     {
@@ -230,8 +244,8 @@ __device__ __attribute__((noinline)) int stage_weights(LdsT<V>& lds, uint8_t con
             for (int e = tid; e < tiles[l] * 16; e += V::THREADS) {
                 int const r = e & 3, g = (e >> 2) & 3, t = e >> 4;
                 int const c = chanBase + 16 * t + 4 * g + r;
-                lds.scale[tileBase + t][g][r] = reinterpret_cast<float const*>(blob + V::SCALE_OFF)[c];
-                lds.bias[tileBase + t][g][r]  = reinterpret_cast<int32_t const*>(blob + V::BIAS_OFF)[c];
+                lds.scale[tileBase + t][g][r] = reinterpret_cast<float const*>(blobBytes + V::SCALE_OFF)[c];
+                lds.bias[tileBase + t][g][r]  = reinterpret_cast<int32_t const*>(blobBytes + V::BIAS_OFF)[c];
             }
             tileBase += tiles[l];
             chanBase += tiles[l] * 16;
@@ -280,7 +294,7 @@ __device__ __attribute__((noinline)) int stage_weights(LdsT<V>& lds, uint8_t con
                 sumLo += w & 1023;
             }
         }
-        int32_t const bias = reinterpret_cast<int32_t const*>(blob + V::BIAS_OFF)[V::H0 + c];
+        int32_t const bias = reinterpret_cast<int32_t const*>(blobBytes + V::BIAS_OFF)[V::H0 + c];
         shifted = int64_t(bias) - 113 * int64_t(sum);     // activations enter as q + 113 in [-15, 240]
         int64_t const absBias = bias < 0 ? -int64_t(bias) : int64_t(bias);
         int64_t const absShifted = shifted < 0 ? -shifted : shifted;
@@ -294,10 +308,10 @@ __device__ __attribute__((noinline)) int stage_weights(LdsT<V>& lds, uint8_t con
         } else {
             int64_t const bound = absShifted + 240 * sumAbs;
             fits = bound < (int64_t(1) << 24);
-            if (l == 3) bounded = float(bound) * fabsf(reinterpret_cast<float const*>(blob + V::SCALE_OFF)[V::H0 + c]) < 60000.f;
+            if (l == 3) bounded = float(bound) * fabsf(reinterpret_cast<float const*>(blobBytes + V::SCALE_OFF)[V::H0 + c]) < 60000.f;
         }
         // the channel's scale gets multiplied by 2^24 (activations enter as (q + 113) * 2^-24): must stay finite
-        fits = fits && fabsf(reinterpret_cast<float const*>(blob + V::SCALE_OFF)[V::H0 + c]) < 0x1p100f;
+        fits = fits && fabsf(reinterpret_cast<float const*>(blobBytes + V::SCALE_OFF)[V::H0 + c]) < 0x1p100f;
         slotTile = V::T0 + (l == 1 ? 0 : (l == 2 ? V::T1 : V::T1 + V::T2)) + row / 16;
         slotG = (row >> 2) & 3;
         slotR = row & 3;
@@ -305,7 +319,7 @@ __device__ __attribute__((noinline)) int stage_weights(LdsT<V>& lds, uint8_t con
     bool small = true;
     if constexpr (!V::FP8_WEIGHTS) {
         if (tid < V::H0) {
-            int32_t const b = reinterpret_cast<int32_t const*>(blob + V::BIAS_OFF)[tid];
+            int32_t const b = reinterpret_cast<int32_t const*>(blobBytes + V::BIAS_OFF)[tid];
             small = b >= -3100000 && b <= 3100000;
         }
     }
@@ -313,9 +327,6 @@ __device__ __attribute__((noinline)) int stage_weights(LdsT<V>& lds, uint8_t con
     // word of the (idle) transposition buffer.  The barriers also order the bias writes above.  (The runtime's
     // workgroup reduction would do, but as a library call it needs the caller's thread ids kept in a vector register
     // for the whole kernel.)
-    uint32_t* const flags = &lds.in[0][0][0];
-    if (tid == 0) *flags = 7u;
-    __syncthreads();
     {
         uint32_t const mine = (__all(fits ? 1 : 0) ? 1u : 0u) | (__all(bounded ? 1 : 0) ? 2u : 0u) | (__all(small ? 1 : 0) ? 4u : 0u);
         if ((tid & 63) == 0) atomicAnd(flags, mine);
@@ -342,7 +353,7 @@ __device__ __attribute__((noinline)) int stage_weights(LdsT<V>& lds, uint8_t con
             // sums run over (q + 113) * 2^-24 (see activate_scale4): every term, this start value included, is an
             // integer below 2^24 times 2^-24, exact in fp32; the scale takes the 2^24 back
             lds.bias[slotTile][slotG][slotR] = __builtin_bit_cast(int32_t, float(twoPlanes ? (shifted >> 10) : shifted) * 0x1p-24f);
-            lds.scale[slotTile][slotG][slotR] = reinterpret_cast<float const*>(blob + V::SCALE_OFF)[V::H0 + tid] * 0x1p24f;
+            lds.scale[slotTile][slotG][slotR] = reinterpret_cast<float const*>(blobBytes + V::SCALE_OFF)[V::H0 + tid] * 0x1p24f;
         }
         // fp16 blocks.  Lane (i, kg) of the block of output tile t and input-tile pair p holds
         // W[16t + i][16*(2p + e/4) + 4*kg + e%4], e = 0..7: the channels lane (j, kg) of the
