@@ -9,6 +9,9 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <algorithm>
+#include <atomic>
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -80,6 +83,7 @@ struct NtcHipContext {
     struct Slot { DevMip* host = nullptr; size_t capacity = 0; hipEvent_t done = nullptr; bool inFlight = false; };
     Slot slots[kSlots];                // pinned staging for asynchronous table uploads
     int nextSlot = 0;
+    DevMip staticBuild[NTC_HIP_STATIC_TABLE_MIPS];   // where ntc_hip_decode_static assembles its table (it allocates nothing)
 };
 
 
@@ -104,7 +108,17 @@ int not_initialized()
     set_error("ntc_hip_init has not been called (or found no HIP device), or the context is null or destroyed.");
     return NTC_HIP_ERR_NOT_INITIALIZED;
 }
-#define CTX_ENTER(ctx) if (!(ctx) || !(ctx)->initialized) return not_initialized(); Library& L = *(ctx); DeviceGuard deviceGuard_(L.device)
+// The contexts that exist.  A handle is looked up here before it is dereferenced, so that a destroyed (freed) context
+// is recognised by its address alone.
+std::mutex g_liveMutex;
+std::vector<NtcHipContext*> g_live;
+bool is_live(NtcHipContext* ctx)
+{
+    if (!ctx) return false;
+    std::lock_guard<std::mutex> lock(g_liveMutex);
+    return std::find(g_live.begin(), g_live.end(), ctx) != g_live.end();
+}
+#define CTX_ENTER(ctx) if (!is_live(ctx)) return not_initialized(); Library& L = *(ctx); DeviceGuard deviceGuard_(L.device)
 
 // Caller-given strides and offsets enter 64-bit size products: bounded so that none can wrap.
 constexpr uint64_t kMaxRowPitch = uint64_t(1) << 40, kMaxPixelStride = uint64_t(1) << 20;
@@ -253,9 +267,35 @@ bool plan_bricks(NtcHipTextureSet const& set, BrickPlan& plan)
 }
 
 // Validates the sets, builds the mip table (sorted by tileStart) and picks the kernel.
+// Where build_table puts its entries: a vector, or (ntc_hip_decode_static, which may not allocate) a fixed array.
+struct TableSink {
+    std::vector<DevMip>* vector = nullptr;
+    DevMip* fixed = nullptr;
+    size_t capacity = 0, count = 0;
+    void clear() { count = 0; if (vector) vector->clear(); }
+    void push_back(DevMip const& e)
+    {
+        if (vector) vector->push_back(e);
+        else if (count < capacity) fixed[count] = e;
+        ++count;                                              // beyond the capacity entries are counted, not stored
+    }
+};
+
+int build_table(NtcHipTextureSet const* sets, int32_t numSets, TableSink table, size_t& entries, int& variant, int& totalTiles,
+                bool forQueries = false);
 int build_table(NtcHipTextureSet const* sets, int32_t numSets, std::vector<DevMip>& table, int& variant, int& totalTiles,
                 bool forQueries = false)
 {
+    TableSink sink;
+    sink.vector = &table;
+    size_t entries = 0;
+    return build_table(sets, numSets, sink, entries, variant, totalTiles, forQueries);
+}
+
+int build_table(NtcHipTextureSet const* sets, int32_t numSets, TableSink table, size_t& entries, int& variant, int& totalTiles,
+                bool forQueries)
+{
+    entries = 0;
     if (!sets || numSets < 1) { set_error("ntc_hip_decode: no texture sets given."); return NTC_HIP_ERR_INVALID_ARG; }
     table.clear();
     totalTiles = 0;
@@ -364,6 +404,7 @@ int build_table(NtcHipTextureSet const* sets, int32_t numSets, std::vector<DevMi
             table.push_back(e);
         }
     }
+    entries = table.count;
     variant = pick_variant(sets[0].spec);
     if (variant == NTC_HIP_VARIANT_NONE) {
         set_error("ntc_hip_decode: no compiled kernel covers this decoder spec "
@@ -414,11 +455,13 @@ int upload_table(Library& L, std::vector<DevMip> const& table)
 int grid_size_for(Library const& L, int variant, int totalTiles)
 {
     // Persistent workgroups: as many as stay resident at once, each walking a contiguous share of tiles.
-    static int perCu[NTC_HIP_VARIANT_COUNT] = { 0 };
-    if (perCu[variant] == 0) {
-        perCu[variant] = variant_is_fp8_network(variant) ? resident_fp8_workgroups_per_cu() : resident_workgroups_per_cu(variant);
+    static std::atomic<int> perCu[NTC_HIP_VARIANT_COUNT];      // zero-initialised; every thread computes the same value
+    int workgroups = perCu[variant].load(std::memory_order_relaxed);
+    if (workgroups == 0) {
+        workgroups = variant_is_fp8_network(variant) ? resident_fp8_workgroups_per_cu() : resident_workgroups_per_cu(variant);
+        perCu[variant].store(workgroups, std::memory_order_relaxed);
     }
-    int const resident = L.computeUnits * perCu[variant];
+    int const resident = L.computeUnits * workgroups;
     // a workgroup takes tiles_per_round(variant) tiles at a time: fewer workgroups than that leaves waves idle
     int const group = variant_is_fp8_network(variant) ? fp8_tiles_per_round() : tiles_per_round(variant);
     int64_t const rounds = (int64_t(totalTiles) + group - 1) / group;
@@ -456,10 +499,13 @@ static int create_context(int device, NtcHipContext** outContext)
         return NTC_HIP_ERR_UNSUPPORTED;
     }
     DeviceGuard guard(device);
-    if (!g_staticTable[device]) {       // once per device, with that device current
-        void* address = nullptr;
-        HIP_TRY(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)));
-        g_staticTable[device] = address;
+    {                                   // once per device, with that device current
+        std::lock_guard<std::mutex> lock(g_liveMutex);
+        if (!g_staticTable[device]) {
+            void* address = nullptr;
+            HIP_TRY(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)));
+            g_staticTable[device] = address;
+        }
     }
     NtcHipContext* L = new (std::nothrow) NtcHipContext();
     if (!L) { set_error("ntc_hip_create: out of host memory."); return NTC_HIP_ERR_INVALID_ARG; }
@@ -478,13 +524,22 @@ static int create_context(int device, NtcHipContext** outContext)
         return hip_fail("hipStreamCreate / hipEventCreate", e);
     }
     L->initialized = true;
+    {
+        std::lock_guard<std::mutex> lock(g_liveMutex);
+        g_live.push_back(L);
+    }
     *outContext = L;
     return 0;
 }
 
 static void destroy_context(NtcHipContext* L)
 {
-    if (!L || !L->initialized) return;
+    {                                   // a handle that is not (or no longer) a context's is ignored, never dereferenced
+        std::lock_guard<std::mutex> lock(g_liveMutex);
+        auto const at = std::find(g_live.begin(), g_live.end(), L);
+        if (!L || at == g_live.end()) return;
+        g_live.erase(at);
+    }
     DeviceGuard guard(L->device);
     (void)hipStreamSynchronize(L->stream);
     if (L->tableDev) (void)hipFree(L->tableDev);
@@ -506,7 +561,7 @@ void ntc_hip_destroy(NtcHipContext* context) { if (context == g_default) g_defau
 
 int ntc_hip_init(int device)
 {
-    if (g_default && g_default->initialized) {
+    if (is_live(g_default)) {
         if (g_default->device == device) { clear_error(); return 0; }
         ntc_hip_shutdown();
     }
@@ -639,26 +694,31 @@ int ntc_hip_ctx_decode(NtcHipContext* ctx, const NtcHipTextureSet* sets, int32_t
 int ntc_hip_ctx_decode_static(NtcHipContext* ctx, const NtcHipTextureSet* sets, int32_t numSets)
 {
     CTX_ENTER(ctx);
-    std::vector<DevMip> table;
+    // No allocation on either side: the table is assembled in the context's own array (not in a vector) and
+    // travels to the device as kernel arguments.
+    TableSink sink;
+    sink.fixed = L.staticBuild;
+    sink.capacity = size_t(kStaticTableEntries);
+    size_t entries = 0;
     int variant = NTC_HIP_VARIANT_NONE, totalTiles = 0;
-    if (int r = build_table(sets, numSets, table, variant, totalTiles)) return r;
-    if (table.size() > size_t(kStaticTableEntries)) {
+    if (int r = build_table(sets, numSets, sink, entries, variant, totalTiles)) return r;
+    if (entries > size_t(kStaticTableEntries)) {
         set_error("ntc_hip_decode_static: %zu mips in one call; the built-in table holds %d (use ntc_hip_decode).",
-                  table.size(), kStaticTableEntries);
+                  entries, kStaticTableEntries);
         return NTC_HIP_ERR_INVALID_ARG;
     }
-    // The table travels as kernel arguments, a chunk per launch, into this device's built-in array.
-    // Stream order keeps a decode that still reads the previous table ahead of these stores.
-    for (size_t first = 0; first < table.size(); first += kTableChunkEntries) {
-        size_t const count = table.size() - first < size_t(kTableChunkEntries) ? table.size() - first : size_t(kTableChunkEntries);
+    // A chunk per launch, into this device's built-in array.  Stream order keeps a decode that still reads the
+    // previous table ahead of these stores.
+    for (size_t first = 0; first < entries; first += kTableChunkEntries) {
+        size_t const count = entries - first < size_t(kTableChunkEntries) ? entries - first : size_t(kTableChunkEntries);
         TableChunk chunk;
         std::memset(&chunk, 0, sizeof(chunk));
-        std::memcpy(chunk.entries, table.data() + first, count * sizeof(DevMip));
+        std::memcpy(chunk.entries, L.staticBuild + first, count * sizeof(DevMip));
         write_table_kernel<<<1, 256, 0, L.stream>>>(reinterpret_cast<uint32_t*>(L.staticTable + first), chunk,
                                                     int(count * sizeof(DevMip) / 4));
         HIP_TRY(hipGetLastError());
     }
-    HIP_TRY(launch_decode_any(variant, L.staticTable, int(table.size()), totalTiles, grid_size_for(L, variant, totalTiles), L.stream));
+    HIP_TRY(launch_decode_any(variant, L.staticTable, int(entries), totalTiles, grid_size_for(L, variant, totalTiles), L.stream));
     clear_error();
     return 0;
 }

@@ -306,6 +306,27 @@ def test_gpu_fp8_decode_with_one_two_and_three_planes_in_some_layers(ntc, device
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("layer", [0, 1, 2])
+@pytest.mark.parametrize("planes", [1, 2, 3])
+def test_gpu_fp8_every_form_of_every_layer(ntc, device, layer, planes):
+    """Every (hidden layer, number of weight planes) form of the network on its own: the layer under test runs on
+    `planes` planes, the two others on one.  planes = 1 is the instantiation for one-plane sets; 2 and 3 take the
+    general one, where the layer's form differs from its neighbours'.  Each form has its own chain of matrix
+    instructions (16-deep or 32-deep, one chain per plane): a wrong sum in any of them shows here."""
+    sigma = {1: 0.35, 2: 1.5, 3: 300.0}[planes]
+    sigmas = tuple(sigma if l == layer else 0.35 for l in range(3))
+    case = fp8_case(ntc, 16, 128, 64, 8, 2, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=90 + 3 * layer + planes, weight_sigma=sigmas, bias_sigma=1.0)
+    spec = ntc.presets.spec_ref092_fp8(16)
+    layout = ntc.synth.weight_layout(spec)
+    n_in, n_out = spec.layer_inputs(layer), spec.layer_outputs(layer)
+    w512 = np.abs(nd.e4m3_times_512(case.weights[layout.weightOffset[layer]:layout.weightOffset[layer] + n_in * n_out])).reshape(n_out, n_in)
+    assert planes == (3 if w512.max() >= 32 * 512 else (2 if w512.sum(axis=1).max() > 10922 else 1))
+    expected, got = run_both(device, case)
+    assert first_mismatch(expected, got) is None, (layer, planes)
+    assert len(np.unique(got.view(np.uint16))) > 500
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("layer", [0, 1, 2])
 def test_gpu_fp8_decode_at_the_one_plane_limit(ntc, device, layer):
     """One channel of one hidden layer with sum |512 w| = 10922 (the largest sum whose products with inputs of 3
     stay below 2^24 units of 2^-18: one plane) and with 10923 (two planes), the large weights on the channel's

@@ -53,28 +53,71 @@ def test_assembly_multiplies_stay_out_of_blocks_with_matrix_instructions(assembl
 
 
 def test_no_accumulator_chain_mixes_16_deep_and_32_deep_matrix_instructions(assembly):
-    """Within a block, a matrix instruction whose accumulator input is the result of an earlier one must have
-    the same depth (16x16x16 onto 16x16x16, 16x16x32 onto 16x16x32)."""
+    """A matrix instruction whose accumulator input is the result of an earlier one must have the same depth
+    (16x16x16 onto 16x16x16, 16x16x32 onto 16x16x32).  For every vector register the set of instructions that may have
+    written it last is followed through each function's control flow: a label starts from the union of what falls
+    into it and of what every branch to it carries (iterated until nothing changes, so loops are covered).  An
+    accumulator input that may reach its instruction unwritten - its producer would be unknown - fails the test too."""
     def registers(operand):
-        m = re.match(r"v\[(\d+):(\d+)\]", operand.strip())
-        return (int(m.group(1)), int(m.group(2))) if m else None
-    checked = 0
-    for function, label, instructions in assembly:
-        producer = {}                                         # register range -> mnemonic of the matrix instruction that wrote it
-        for name, operands in instructions:
-            ops = [o.strip() for o in operands.split(",")]
-            if name.startswith("v_mfma_f32_16x16x") and name.endswith("_f16"):
-                dst, src_c = registers(ops[0]), registers(ops[3]) if len(ops) > 3 else None
-                if src_c in producer:
-                    assert producer[src_c] == name, (function, label, producer[src_c], name)
-                    checked += 1
-                producer = {r: n for r, n in producer.items() if dst is None or r[1] < dst[0] or r[0] > dst[1]}
-                if dst:
-                    producer[dst] = name
-            elif ops and registers(ops[0]):                  # any other write to a register range ends the chain
-                dst = registers(ops[0])
-                producer = {r: n for r, n in producer.items() if r[1] < dst[0] or r[0] > dst[1]}
-            elif ops and re.match(r"v\d+$", ops[0]):
-                reg = int(ops[0][1:])
-                producer = {r: n for r, n in producer.items() if not (r[0] <= reg <= r[1])}
-    assert checked > 100
+        operand = operand.strip()
+        m = re.match(r"v\[(\d+):(\d+)\]", operand)
+        if m:
+            return range(int(m.group(1)), int(m.group(2)) + 1)
+        m = re.match(r"v(\d+)$", operand)
+        return range(int(m.group(1)), int(m.group(1)) + 1) if m else None
+
+    def is_f16_matrix(name):
+        return isinstance(name, str) and name.startswith("v_mfma_f32_16x16x") and name.endswith("_f16")
+
+    def merge(a, b):
+        """Union of two states (register -> set of possible last writers; None = possibly unwritten)."""
+        if a is None:
+            return {r: set(w) for r, w in b.items()}
+        out = {}
+        for reg in set(a) | set(b):
+            out[reg] = set(a.get(reg, {None})) | set(b.get(reg, {None}))
+        return out
+
+    functions = {}
+    for fn, label, instructions in assembly:
+        functions.setdefault(fn, []).append((label, instructions))
+    checked = across_branches = 0
+    for fn, blocks in functions.items():
+        carried = {}                                          # label -> state carried by the branches that target it
+        for sweep in range(8):
+            before = {k: {r: frozenset(w) for r, w in v.items()} for k, v in carried.items()}
+            state, final = {}, sweep > 0
+            for label, instructions in blocks:
+                if label in carried:
+                    state = merge(state, carried[label]) if state is not None else merge(None, carried[label])
+                elif state is None:
+                    state = {}                                # unreachable in layout order and not (yet) a branch target
+                for name, operands in instructions:
+                    ops = [o.strip() for o in operands.split(",")]
+                    if name.startswith(("s_cbranch", "s_branch")) and ops and ops[0].startswith(".LBB"):
+                        carried[ops[0]] = merge(carried.get(ops[0]), state)
+                        if name == "s_branch":
+                            state = None                      # nothing falls through
+                        continue
+                    if name in ("s_endpgm", "s_setpc_b64"):
+                        state = None
+                        continue
+                    if state is None:
+                        state = {}
+                    if final and is_f16_matrix(name) and len(ops) > 3 and registers(ops[3]) is not None:    # (a literal 0 starts a chain)
+                        for reg in registers(ops[3]):
+                            writers = state.get(reg, {None})
+                            assert None not in writers, (fn, label, "accumulator input with a possibly unknown producer", name, operands)
+                            for w in writers:
+                                if is_f16_matrix(w):
+                                    assert w == name, (fn, label, w, name)
+                                    checked += 1
+                            across_branches += len(writers) > 1
+                    if ops and name.startswith(("v_", "ds_read", "global_load", "buffer_load", "scratch_load")) and registers(ops[0]) is not None:
+                        for reg in registers(ops[0]):
+                            state[reg] = {name}
+            if sweep > 0 and before == {k: {r: frozenset(w) for r, w in v.items()} for k, v in carried.items()}:
+                break
+        else:
+            raise AssertionError((fn, "the register states did not settle"))
+    assert checked > 400                                      # four registers per chained instruction

@@ -61,3 +61,26 @@ def test_static_table_decode_rejects_more_mips_than_the_table_holds(ntc, device)
     assert err.value.code == ntc.abi.ERR_INVALID_ARG and "built-in table" in err.value.message
     device.decode_static([dset] * 36)                        # 252 mips fit (the sets overlap; only the limit is tested)
     device.synchronize()
+
+
+def test_static_table_decode_leaves_device_memory_as_it_is(ntc, device):
+    """hipMemGetInfo before and after: ntc_hip_decode_static takes no device memory (and gives none back).  The first
+    call of any kernel may make the runtime load code or set up its queue, so one call comes before the measurement."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+    spec = ntc.presets.spec_cfg01()
+    case = cfg_case(ntc, spec, 512, 512, 10, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=23, scale_log2_range=ACTIVE)
+    dset = case.device_set(device)
+    device.decode_static([dset])
+    device.synchronize()
+
+    def free_bytes():
+        free, total = C.c_size_t(0), C.c_size_t(0)
+        assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+        return free.value
+
+    before = free_bytes()
+    for _ in range(3):
+        device.decode_static([dset])
+    device.synchronize()
+    assert free_bytes() == before
