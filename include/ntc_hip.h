@@ -225,8 +225,9 @@ int ntc_hip_decode_timed(const NtcHipTextureSet* sets, int32_t numSets, int32_t 
  * loops and harnesses that forbid hipMalloc.  No counterpart in the reference.  ntc_hip_decode keeps its
  * mip table in device memory that it allocates (and grows) on demand and fills through pinned staging
  * memory; here the table lives in an array built into the library's code object, NTC_HIP_STATIC_TABLE_MIPS
- * entries (about 34 KB, held by every GPU the library runs on until the process ends), and travels to the
- * device as kernel arguments.  The call allocates nothing on the device or the host (the table is assembled
+ * entries and one more 256-byte line (about 34 KB, held by every GPU the library runs on until the process
+ * ends), and travels to the device as kernel arguments; the extra line holds the word through which the first of
+ * the FP8 network's two launches tells the second whether a set is left for it.  The call allocates nothing on the device or the host (the table is assembled
  * in an array inside the context), frees nothing and copies nothing: it launches
  * one small table-writing kernel per 16 mips and then the decode kernel of ntc_hip_decode, same results.
  * More than NTC_HIP_STATIC_TABLE_MIPS mips over all sets of one call: NTC_HIP_ERR_INVALID_ARG.

@@ -746,8 +746,9 @@ __device__ __forceinline__ void mlp_forward_fp8(Fp8Lds<V>& lds, int wave, int la
 // of a common sequence drift apart in time, and the latent reads from memory doubled.)
 template <class V>
 __global__ void __launch_bounds__(V::THREADS, 1)
-decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
+decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles, Fp8Handoff handoff)
 {
+    if (!V::ONE && *handoff.word != handoff.serial) return;  // the one-plane launch before this one met only its own sets
     __shared__ Fp8Lds<V> lds;
     int const lane = threadIdx.x & 63;
     int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -798,7 +799,11 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
         uint8_t const* const blob = mips[entry].weights;
         int const segEnd = segment_end(mips, numMips, entry, tileEnd, blob);
         modes = classify_fp8_weights<V>(lds, blob);
-        if (((modes & kAllOnePlane) == kAllOnePlane) != V::ONE) { segBegin = segEnd; continue; }   // the other instantiation's segment
+        if (((modes & kAllOnePlane) == kAllOnePlane) != V::ONE) { // the other instantiation's segment
+            if (V::ONE && threadIdx.x == 0) *handoff.word = handoff.serial;
+            segBegin = segEnd;
+            continue;
+        }
         __syncthreads();                                     // every wave has left the previous segment's weights
         stage_fp8_weights<V>(lds, blob, modes);
         __syncthreads();                                     // also publishes the tables built above
@@ -829,8 +834,9 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
 template <class V>
 __global__ void __launch_bounds__(V::THREADS, 1)
 query_fp8_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* __restrict__ queries, uint64_t numQueries,
-                 uint16_t* __restrict__ out)
+                 uint16_t* __restrict__ out, Fp8Handoff handoff)
 {
+    if (!V::ONE && *handoff.word != handoff.serial) return;  // the set went to the one-plane launch before this one
     __shared__ Fp8Lds<V> lds;
     __shared__ QueryMip qmips[16];
     if (threadIdx.x < 16) {
@@ -849,7 +855,10 @@ query_fp8_kernel(DevMip const* __restrict__ mips, int numMips, DevQuery const* _
     int const j = lane & 15, g = lane >> 4;
 
     int const modes = classify_fp8_weights<V>(lds, mips[0].weights);
-    if (((modes & kAllOnePlane) == kAllOnePlane) != V::ONE) return;      // the other instantiation's set (uniform over the grid)
+    if (((modes & kAllOnePlane) == kAllOnePlane) != V::ONE) {            // the other instantiation's set (uniform over the grid)
+        if (V::ONE && threadIdx.x == 0) *handoff.word = handoff.serial;
+        return;
+    }
     build_fp8_posenc_table(lds);
     build_fp8_feature_lut(lds);
     stage_fp8_weights<V>(lds, mips[0].weights, modes);
@@ -914,50 +923,53 @@ __global__ void selftest_fp8_activation_kernel(uint16_t const* __restrict__ in, 
 using VFp8_16 = Fp8Variant<16>;
 
 // Both instantiations, the one-plane one first; a set is decoded by the one it belongs to (decided on the device
-// from its weights), the other passes over it after reading the weights once per workgroup.
+// from its weights).  A workgroup of the first launch that meets a set of the other kind writes the launch pair's
+// serial number into the caller's hand-off word; the workgroups of the second launch leave at once unless they
+// find that number there (nothing ever clears the word: a stale match only costs the second launch its look at
+// the weights, after which it passes over the sets that are not its own as before).
 template <int FEATURES>
-static hipError_t launch_fp8_variant(DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream)
+static hipError_t launch_fp8_variant(DevMip const* mips, int numMips, int totalTiles, int gridSize, Fp8Handoff handoff, hipStream_t stream)
 {
     using One = Fp8Variant<FEATURES, true>;
     using Any = Fp8Variant<FEATURES, false>;
-    hipLaunchKernelGGL(decode_fp8_kernel<One>, dim3(gridSize), dim3(One::THREADS), 0, stream, mips, numMips, totalTiles);
+    hipLaunchKernelGGL(decode_fp8_kernel<One>, dim3(gridSize), dim3(One::THREADS), 0, stream, mips, numMips, totalTiles, handoff);
     hipError_t const e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(decode_fp8_kernel<Any>, dim3(gridSize), dim3(Any::THREADS), 0, stream, mips, numMips, totalTiles);
+    hipLaunchKernelGGL(decode_fp8_kernel<Any>, dim3(gridSize), dim3(Any::THREADS), 0, stream, mips, numMips, totalTiles, handoff);
     return hipGetLastError();
 }
 
-hipError_t launch_decode_fp8(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream)
+hipError_t launch_decode_fp8(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, Fp8Handoff handoff, hipStream_t stream)
 {
     switch (variant) {
-    case NTC_HIP_VARIANT_REF16_FP8: return launch_fp8_variant<16>(mips, numMips, totalTiles, gridSize, stream);
-    case NTC_HIP_VARIANT_REF12_FP8: return launch_fp8_variant<12>(mips, numMips, totalTiles, gridSize, stream);
-    case NTC_HIP_VARIANT_REF8_FP8:  return launch_fp8_variant<8>(mips, numMips, totalTiles, gridSize, stream);
-    case NTC_HIP_VARIANT_REF4_FP8:  return launch_fp8_variant<4>(mips, numMips, totalTiles, gridSize, stream);
+    case NTC_HIP_VARIANT_REF16_FP8: return launch_fp8_variant<16>(mips, numMips, totalTiles, gridSize, handoff, stream);
+    case NTC_HIP_VARIANT_REF12_FP8: return launch_fp8_variant<12>(mips, numMips, totalTiles, gridSize, handoff, stream);
+    case NTC_HIP_VARIANT_REF8_FP8:  return launch_fp8_variant<8>(mips, numMips, totalTiles, gridSize, handoff, stream);
+    case NTC_HIP_VARIANT_REF4_FP8:  return launch_fp8_variant<4>(mips, numMips, totalTiles, gridSize, handoff, stream);
     default: return hipErrorInvalidValue;
     }
 }
 
 template <int FEATURES>
-static hipError_t launch_fp8_query_variant(DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries, uint16_t* out, int gridSize, hipStream_t stream)
+static hipError_t launch_fp8_query_variant(DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries, uint16_t* out, int gridSize, Fp8Handoff handoff, hipStream_t stream)
 {
     using One = Fp8Variant<FEATURES, true>;
     using Any = Fp8Variant<FEATURES, false>;
-    hipLaunchKernelGGL(query_fp8_kernel<One>, dim3(gridSize), dim3(One::THREADS), 0, stream, mips, numMips, queries, numQueries, out);
+    hipLaunchKernelGGL(query_fp8_kernel<One>, dim3(gridSize), dim3(One::THREADS), 0, stream, mips, numMips, queries, numQueries, out, handoff);
     hipError_t const e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(query_fp8_kernel<Any>, dim3(gridSize), dim3(Any::THREADS), 0, stream, mips, numMips, queries, numQueries, out);
+    hipLaunchKernelGGL(query_fp8_kernel<Any>, dim3(gridSize), dim3(Any::THREADS), 0, stream, mips, numMips, queries, numQueries, out, handoff);
     return hipGetLastError();
 }
 
 hipError_t launch_queries_fp8(int variant, DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries,
-                              uint16_t* out, int gridSize, hipStream_t stream)
+                              uint16_t* out, int gridSize, Fp8Handoff handoff, hipStream_t stream)
 {
     switch (variant) {
-    case NTC_HIP_VARIANT_REF16_FP8: return launch_fp8_query_variant<16>(mips, numMips, queries, numQueries, out, gridSize, stream);
-    case NTC_HIP_VARIANT_REF12_FP8: return launch_fp8_query_variant<12>(mips, numMips, queries, numQueries, out, gridSize, stream);
-    case NTC_HIP_VARIANT_REF8_FP8:  return launch_fp8_query_variant<8>(mips, numMips, queries, numQueries, out, gridSize, stream);
-    case NTC_HIP_VARIANT_REF4_FP8:  return launch_fp8_query_variant<4>(mips, numMips, queries, numQueries, out, gridSize, stream);
+    case NTC_HIP_VARIANT_REF16_FP8: return launch_fp8_query_variant<16>(mips, numMips, queries, numQueries, out, gridSize, handoff, stream);
+    case NTC_HIP_VARIANT_REF12_FP8: return launch_fp8_query_variant<12>(mips, numMips, queries, numQueries, out, gridSize, handoff, stream);
+    case NTC_HIP_VARIANT_REF8_FP8:  return launch_fp8_query_variant<8>(mips, numMips, queries, numQueries, out, gridSize, handoff, stream);
+    case NTC_HIP_VARIANT_REF4_FP8:  return launch_fp8_query_variant<4>(mips, numMips, queries, numQueries, out, gridSize, handoff, stream);
     default: return hipErrorInvalidValue;
     }
 }

@@ -152,12 +152,16 @@ hipError_t launch_bc7_compress(BlockCompressArgs const& args, hipStream_t stream
 hipError_t launch_decode(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream);
 hipError_t launch_queries(int variant, DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries,
                           uint16_t* out, int gridSize, hipStream_t stream);
-hipError_t launch_decode_fp8(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream);
+// The FP8 network is launched twice (weights of one plane per layer, then any weights); `word` is a dword of device
+// memory through which the first launch tells the second whether any set is left for it, `serial` a number the
+// caller changes with every pair of launches that shares the word.
+struct Fp8Handoff { uint32_t* word; uint32_t serial; };
+hipError_t launch_decode_fp8(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, Fp8Handoff handoff, hipStream_t stream);
 int resident_fp8_workgroups_per_cu();
 int fp8_tiles_per_round();               // tiles a workgroup of decode_fp8_kernel works on at a time
 int fp8_threads_per_workgroup();
 hipError_t launch_queries_fp8(int variant, DevMip const* mips, int numMips, DevQuery const* queries, uint64_t numQueries,
-                              uint16_t* out, int gridSize, hipStream_t stream);
+                              uint16_t* out, int gridSize, Fp8Handoff handoff, hipStream_t stream);
 hipError_t launch_selftest_fp8_activation(uint16_t const* in, uint16_t* out, int n, hipStream_t stream);
 int resident_workgroups_per_cu(int variant);
 int tiles_per_round(int variant);      // tiles a workgroup of the variant's decode kernel works on at a time

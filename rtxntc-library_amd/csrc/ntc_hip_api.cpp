@@ -44,7 +44,8 @@ int hip_fail(char const* call, hipError_t err)
 // hipGetSymbolAddress returned for the device (Library::staticTable), never through the name.
 constexpr int kStaticTableEntries = NTC_HIP_STATIC_TABLE_MIPS;                      // 16 sets with a full mip chain each
 constexpr int kTableChunkEntries = 16;                         // entries one table-writing launch carries
-static __device__ __align__(256) unsigned char scratch[kStaticTableEntries * sizeof(DevMip)];
+constexpr size_t kStaticTableBytes = (kStaticTableEntries * sizeof(DevMip) + 255) / 256 * 256;
+static __device__ __align__(256) unsigned char scratch[kStaticTableBytes + 256];   // the table, then the FP8 hand-off word
 constexpr int kMaxDevices = 64;
 void* g_staticTable[kMaxDevices] = { nullptr };                // per device: address of `scratch` there
 
@@ -74,6 +75,8 @@ struct NtcHipContext {
     hipEvent_t evStart = nullptr, evStop = nullptr;
     DevMip* tableDev = nullptr;        // device copy of the mip table
     DevMip* staticTable = nullptr;     // this device's `scratch` array (ntc_hip_decode_static)
+    uint32_t* handoffDev = nullptr;    // the dword between the two launches of the FP8 network (launch_decode_fp8)
+    uint32_t handoffSerial = 0;        // changes with every pair of such launches
     size_t tableCapacity = 0;          // entries
     std::vector<DevMip> lastTable;     // what tableDev currently holds (or will, in stream order)
     double* lossDev = nullptr;         // per-workgroup partial sums of the loss pass
@@ -468,10 +471,19 @@ int grid_size_for(Library const& L, int variant, int totalTiles)
     return rounds < resident ? int(rounds) : resident;
 }
 
-hipError_t launch_decode_any(int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize, hipStream_t stream)
+// The hand-off word of a launch pair of the FP8 network over table `mips`: the context's own, or the one behind
+// the per-device table when that is the table (then nothing of the context's device memory is used).
+Fp8Handoff next_handoff(Library& L, DevMip const* mips)
 {
-    return variant_is_fp8_network(variant) ? launch_decode_fp8(variant, mips, numMips, totalTiles, gridSize, stream)
-                                           : launch_decode(variant, mips, numMips, totalTiles, gridSize, stream);
+    uint32_t* const word = mips == L.staticTable
+        ? reinterpret_cast<uint32_t*>(reinterpret_cast<unsigned char*>(L.staticTable) + kStaticTableBytes) : L.handoffDev;
+    return Fp8Handoff{ word, ++L.handoffSerial };
+}
+
+hipError_t launch_decode_any(Library& L, int variant, DevMip const* mips, int numMips, int totalTiles, int gridSize)
+{
+    return variant_is_fp8_network(variant) ? launch_decode_fp8(variant, mips, numMips, totalTiles, gridSize, next_handoff(L, mips), L.stream)
+                                           : launch_decode(variant, mips, numMips, totalTiles, gridSize, L.stream);
 }
 
 } // namespace
@@ -517,11 +529,13 @@ static int create_context(int device, NtcHipContext** outContext)
     hipError_t e = hipStreamCreate(&L->stream);
     if (e == hipSuccess) e = hipEventCreate(&L->evStart);
     if (e == hipSuccess) e = hipEventCreate(&L->evStop);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&L->handoffDev), 256);
     if (e != hipSuccess) {
+        if (L->evStop) (void)hipEventDestroy(L->evStop);
         if (L->evStart) (void)hipEventDestroy(L->evStart);
         if (L->stream) (void)hipStreamDestroy(L->stream);
         delete L;
-        return hip_fail("hipStreamCreate / hipEventCreate", e);
+        return hip_fail("hipStreamCreate / hipEventCreate / hipMalloc", e);
     }
     L->initialized = true;
     {
@@ -543,6 +557,7 @@ static void destroy_context(NtcHipContext* L)
     DeviceGuard guard(L->device);
     (void)hipStreamSynchronize(L->stream);
     if (L->tableDev) (void)hipFree(L->tableDev);
+    if (L->handoffDev) (void)hipFree(L->handoffDev);
     if (L->lossDev) (void)hipFree(L->lossDev);
     if (L->lossHost) (void)hipHostFree(L->lossHost);
     for (Library::Slot& slot : L->slots) {
@@ -686,7 +701,7 @@ int ntc_hip_ctx_decode(NtcHipContext* ctx, const NtcHipTextureSet* sets, int32_t
     int variant = NTC_HIP_VARIANT_NONE, totalTiles = 0;
     if (int r = build_table(sets, numSets, table, variant, totalTiles)) return r;
     if (int r = upload_table(L, table)) return r;
-    HIP_TRY(launch_decode_any(variant, L.tableDev, int(table.size()), totalTiles, grid_size_for(L, variant, totalTiles), L.stream));
+    HIP_TRY(launch_decode_any(L, variant, L.tableDev, int(table.size()), totalTiles, grid_size_for(L, variant, totalTiles)));
     clear_error();
     return 0;
 }
@@ -718,7 +733,7 @@ int ntc_hip_ctx_decode_static(NtcHipContext* ctx, const NtcHipTextureSet* sets, 
                                                     int(count * sizeof(DevMip) / 4));
         HIP_TRY(hipGetLastError());
     }
-    HIP_TRY(launch_decode_any(variant, L.staticTable, int(entries), totalTiles, grid_size_for(L, variant, totalTiles), L.stream));
+    HIP_TRY(launch_decode_any(L, variant, L.staticTable, int(entries), totalTiles, grid_size_for(L, variant, totalTiles)));
     clear_error();
     return 0;
 }
@@ -734,7 +749,7 @@ int ntc_hip_ctx_decode_timed(NtcHipContext* ctx, const NtcHipTextureSet* sets, i
     int const grid = grid_size_for(L, variant, totalTiles);
     HIP_TRY(hipEventRecord(L.evStart, L.stream));
     for (int i = 0; i < iterations; ++i)
-        HIP_TRY(launch_decode_any(variant, L.tableDev, int(table.size()), totalTiles, grid, L.stream));
+        HIP_TRY(launch_decode_any(L, variant, L.tableDev, int(table.size()), totalTiles, grid));
     HIP_TRY(hipEventRecord(L.evStop, L.stream));
     HIP_TRY(hipEventSynchronize(L.evStop));
     float ms = 0.f;
@@ -764,8 +779,10 @@ static int run_queries(NtcHipContext* ctx, const NtcHipTextureSet* set, const Nt
     int const grid = int(blocks < resident ? blocks : resident);
     if (outMs) HIP_TRY(hipEventRecord(L.evStart, L.stream));
     for (int i = 0; i < iterations; ++i)
-        HIP_TRY((fp8 ? launch_queries_fp8 : launch_queries)(variant, L.tableDev, int(table.size()), reinterpret_cast<DevQuery const*>(queries), numQueries,
-                                                           static_cast<uint16_t*>(out), grid, L.stream));
+        HIP_TRY(fp8 ? launch_queries_fp8(variant, L.tableDev, int(table.size()), reinterpret_cast<DevQuery const*>(queries), numQueries,
+                                         static_cast<uint16_t*>(out), grid, next_handoff(L, L.tableDev), L.stream)
+                    : launch_queries(variant, L.tableDev, int(table.size()), reinterpret_cast<DevQuery const*>(queries), numQueries,
+                                     static_cast<uint16_t*>(out), grid, L.stream));
     if (outMs) {
         HIP_TRY(hipEventRecord(L.evStop, L.stream));
         HIP_TRY(hipEventSynchronize(L.evStop));

@@ -557,3 +557,23 @@ def test_gpu_fp8_queries_match_checker(ntc, device, oracle, features, size, grid
     ms = C.c_float()
     A.check(device.lib.ntc_hip_decode_queries_timed(dset, d_q.ptr, n, d_out.ptr, d_out.nbytes, 2, C.byref(ms)))
     assert ms.value > 0 and np.array_equal(d_out.download(np.uint16).reshape(n, 16), want)
+
+
+@pytest.mark.gpu
+def test_gpu_fp8_launch_pairs_of_one_context_do_not_inherit_each_others_hand_off(ntc, device):
+    """The network's two launches talk through one dword of the context (and another behind the per-device table):
+    the second leaves at once unless the first met a set that is not its own.  Sets of either kind decoded in turn
+    through one context, by both entry points, with the output cleared before each decode: a launch that believed
+    the previous pair's word would leave its set undecoded."""
+    kinds = [0.35, 1.5, 0.35, 0.35, 300.0, 1.5, 0.35]
+    cases = [fp8_case(ntc, 16, 96, 40, 3, 2, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=400 + i, weight_sigma=s) for i, s in enumerate(kinds)]
+    hosts = [c.host_set() for c in cases]
+    for hset in hosts:
+        hset.decode(threads=8)
+    dsets = [c.device_set(device) for c in cases]
+    for static in (False, True, False):
+        for i, (c, hset) in enumerate(zip(cases, hosts)):
+            c.d_output.fill(0xCD)
+            (device.decode_static if static else device.decode)([dsets[i]])
+            device.synchronize()
+            assert first_mismatch(hset.output, c.d_output.download()) is None, (static, i)
