@@ -268,20 +268,29 @@ __device__ __attribute__((noinline)) int stage_weights(LdsT<V>& lds, uint8_t con
         }
     }
 
-    // One thread per channel of layers 1..3: row sums decide whether the fp16 path is exact.
+    // Four threads per channel of layers 1..3 (two or one where the workgroup has not that many), a part of the row
+    // each: row sums decide whether the fp16 path is exact.  (The sums fit 32 bits: at most 64 weights of at most
+    // 448 * 512 in magnitude.)  After the exchange all of them hold the totals; the first writes the channel's
+    // constants further down.
     bool fits = true, bounded = true;
     int64_t shifted = 0;
     bool twoPlanes = false;
     int slotTile = 0, slotG = 0, slotR = 0;
-    if (tid < V::LATE_CHANNELS) {
-        int const c = tid;
+    constexpr int kSplit = 4 * V::LATE_CHANNELS <= V::THREADS ? 4 : (2 * V::LATE_CHANNELS <= V::THREADS ? 2 : 1);
+    static_assert(V::LATE_CHANNELS <= V::THREADS, "a thread per channel at least");
+    bool const rowThread = tid < kSplit * V::LATE_CHANNELS;
+    bool const rowWriter = rowThread && tid % kSplit == 0;
+    int const c = tid / kSplit;                              // the thread's channel among those of layers 1..3
+    if (rowThread) {
+        int const part = tid % kSplit;
         int const l = c < V::H1 ? 1 : (c < V::H1 + V::H2 ? 2 : 3);
         int const row = c - (l == 1 ? 0 : (l == 2 ? V::H1 : V::H1 + V::H2));
         int const in = l == 1 ? V::H0 : (l == 2 ? V::H1 : V::H2);
         int const off = l == 1 ? V::W1_OFF : (l == 2 ? V::W2_OFF : V::W3_OFF);
         twoPlanes = V::FP8_WEIGHTS && l < 3;
-        int64_t sum = 0, sumAbs = 0, sumAbsHi = 0, sumLo = 0;
-        for (int k = 0; k < in; k += 4) {
+        static_assert(V::H0 % 16 == 0 && V::H1 % 16 == 0 && V::H2 % 16 == 0, "a part of a row is whole dwords");
+        int32_t sum = 0, sumAbs = 0, sumAbsHi = 0, sumLo = 0;
+        for (int k = part * (in / kSplit); k < (part + 1) * (in / kSplit); k += 4) {
             uint32_t const v = blob32[(off + row * in + k) >> 2];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
@@ -294,6 +303,15 @@ __device__ __attribute__((noinline)) int stage_weights(LdsT<V>& lds, uint8_t con
                 sumLo += w & 1023;
             }
         }
+#pragma unroll
+        for (int step = 1; step < kSplit; step *= 2) {        // the parts sit in neighbouring lanes of one wave
+            sum += __shfl_xor(sum, step, 64);
+            sumAbs += __shfl_xor(sumAbs, step, 64);
+            if constexpr (V::FP8_WEIGHTS) {
+                sumAbsHi += __shfl_xor(sumAbsHi, step, 64);
+                sumLo += __shfl_xor(sumLo, step, 64);
+            }
+        }
         int32_t const bias = reinterpret_cast<int32_t const*>(blobBytes + V::BIAS_OFF)[V::H0 + c];
         shifted = int64_t(bias) - 113 * int64_t(sum);     // activations enter as q + 113 in [-15, 240]
         int64_t const absBias = bias < 0 ? -int64_t(bias) : int64_t(bias);
@@ -302,11 +320,11 @@ __device__ __attribute__((noinline)) int stage_weights(LdsT<V>& lds, uint8_t con
             // Exact when the int32 accumulator the result is defined by cannot wrap (inputs in [-128, 127])
             // and both fp32 partial sums, started at floor(shifted / 1024) and shifted mod 1024, stay integers.
             int64_t const startHi = shifted >> 10;
-            fits = absBias + 128 * sumAbs < (int64_t(1) << 31)
-                && (startHi < 0 ? -startHi : startHi) + 240 * sumAbsHi < (int64_t(1) << 24)
-                && 1023 + 240 * sumLo < (int64_t(1) << 24);
+            fits = absBias + 128 * int64_t(sumAbs) < (int64_t(1) << 31)
+                && (startHi < 0 ? -startHi : startHi) + 240 * int64_t(sumAbsHi) < (int64_t(1) << 24)
+                && 1023 + 240 * int64_t(sumLo) < (int64_t(1) << 24);
         } else {
-            int64_t const bound = absShifted + 240 * sumAbs;
+            int64_t const bound = absShifted + 240 * int64_t(sumAbs);
             fits = bound < (int64_t(1) << 24);
             if (l == 3) bounded = float(bound) * fabsf(reinterpret_cast<float const*>(blobBytes + V::SCALE_OFF)[V::H0 + c]) < 60000.f;
         }
@@ -346,14 +364,14 @@ __device__ __attribute__((noinline)) int stage_weights(LdsT<V>& lds, uint8_t con
     constexpr int base[4] = { 0, V::F16_L1, V::F16_L2, V::F16_L3 };
     uint32_t* const late32 = reinterpret_cast<uint32_t*>(lds.late);
     if (useF16) {
-        if (tid < V::LATE_CHANNELS) {
+        if (rowWriter) {
             if constexpr (V::FP8_WEIGHTS) {
                 if (twoPlanes) lds.biasLo[slotTile][slotG][slotR] = float(shifted & 1023) * 0x1p-24f;
             }
             // sums run over (q + 113) * 2^-24 (see activate_scale4): every term, this start value included, is an
             // integer below 2^24 times 2^-24, exact in fp32; the scale takes the 2^24 back
             lds.bias[slotTile][slotG][slotR] = __builtin_bit_cast(int32_t, float(twoPlanes ? (shifted >> 10) : shifted) * 0x1p-24f);
-            lds.scale[slotTile][slotG][slotR] = reinterpret_cast<float const*>(blobBytes + V::SCALE_OFF)[V::H0 + tid] * 0x1p24f;
+            lds.scale[slotTile][slotG][slotR] = reinterpret_cast<float const*>(blobBytes + V::SCALE_OFF)[V::H0 + c] * 0x1p24f;
         }
         // fp16 blocks.  Lane (i, kg) of the block of output tile t and input-tile pair p holds
         // W[16t + i][16*(2p + e/4) + 4*kg + e%4], e = 0..7: the channels lane (j, kg) of the
