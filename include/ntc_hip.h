@@ -221,6 +221,14 @@ int ntc_hip_decode(const NtcHipTextureSet* sets, int32_t numSets);
 int ntc_hip_decode_timed(const NtcHipTextureSet* sets, int32_t numSets, int32_t iterations,
                          float* outMillisecondsPerIteration);
 
+/* Device time of a sequence of calls: ntc_hip_timer_begin records a HIP event on the context's stream, ntc_hip_timer_end
+ * records a second one behind everything queued since, waits for it and returns the milliseconds between the two.
+ * This is how the reference times its own decompression (cudaEventRecord around the per-mip loop,
+ * src/TextureSet.cpp:1772-1779,1866-1882); ntc_hip_decode_timed is the special case of one decode repeated.
+ * One span at a time per context; _end without _begin: NTC_HIP_ERR_INVALID_ARG.  _end is synchronous. */
+int ntc_hip_timer_begin(void);
+int ntc_hip_timer_end(float* outMilliseconds);
+
 /* ntc_hip_decode for callers that cannot allocate device memory: code under HIP graph capture, serving
  * loops and harnesses that forbid hipMalloc.  No counterpart in the reference.  ntc_hip_decode keeps its
  * mip table in device memory that it allocates (and grows) on demand and fills through pinned staging
@@ -414,6 +422,8 @@ int ntc_hip_ctx_memset(NtcHipContext* context, void* dst, int value, size_t byte
 int ntc_hip_ctx_synchronize(NtcHipContext* context);
 int ntc_hip_ctx_decode(NtcHipContext* context, const NtcHipTextureSet* sets, int32_t numSets);
 int ntc_hip_ctx_decode_static(NtcHipContext* context, const NtcHipTextureSet* sets, int32_t numSets);
+int ntc_hip_ctx_timer_begin(NtcHipContext* context);
+int ntc_hip_ctx_timer_end(NtcHipContext* context, float* outMilliseconds);
 int ntc_hip_ctx_decode_timed(NtcHipContext* context, const NtcHipTextureSet* sets, int32_t numSets, int32_t iterations, float* outMs);
 int ntc_hip_ctx_build_query_latents(NtcHipContext* context, const NtcHipTextureSet* set, void* dst, uint64_t dstBytes);
 int ntc_hip_ctx_decode_queries(NtcHipContext* context, const NtcHipTextureSet* set, const NtcHipQuery* queries, uint64_t numQueries, void* out, uint64_t outBytes);

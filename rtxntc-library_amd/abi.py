@@ -149,6 +149,8 @@ EXPORTS = [
     ("ntc_hip_decode", C.c_int, [C.POINTER(TextureSet), C.c_int32]),
     ("ntc_hip_decode_static", C.c_int, [C.POINTER(TextureSet), C.c_int32]),
     ("ntc_hip_decode_timed", C.c_int, [C.POINTER(TextureSet), C.c_int32, C.c_int32, C.POINTER(C.c_float)]),
+    ("ntc_hip_timer_begin", C.c_int, []),
+    ("ntc_hip_timer_end", C.c_int, [C.POINTER(C.c_float)]),
     ("ntc_hip_decode_queries", C.c_int, [C.POINTER(TextureSet), C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint64]),
     ("ntc_hip_decode_queries_timed", C.c_int, [C.POINTER(TextureSet), C.c_void_p, C.c_uint64, C.c_void_p, C.c_uint64,
                                                C.c_int32, C.POINTER(C.c_float)]),
@@ -169,7 +171,7 @@ EXPORTS = [
 
 # The context forms: ntc_hip_ctx_<name>(context, same arguments); ntc_hip_create / ntc_hip_destroy.
 _CONTEXT_FORMS = ["device_info", "device_clock", "alloc", "free", "upload", "download", "memset", "synchronize", "decode",
-                  "decode_static", "decode_timed", "build_query_latents", "decode_queries", "decode_queries_timed", "read_channels",
+                  "decode_static", "decode_timed", "timer_begin", "timer_end", "build_query_latents", "decode_queries", "decode_queries_timed", "read_channels",
                   "write_channels", "image_loss", "resize_planar", "image_difference", "block_compress"]
 _BY_NAME = {name: (restype, argtypes) for name, restype, argtypes in EXPORTS}
 EXPORTS += [("ntc_hip_ctx_" + n, _BY_NAME["ntc_hip_" + n][0], [C.c_void_p] + _BY_NAME["ntc_hip_" + n][1]) for n in _CONTEXT_FORMS]

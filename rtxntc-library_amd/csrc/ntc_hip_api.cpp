@@ -73,6 +73,8 @@ struct NtcHipContext {
     char name[256] = "";
     hipStream_t stream = nullptr;
     hipEvent_t evStart = nullptr, evStop = nullptr;
+    hipEvent_t evSpanStart = nullptr, evSpanStop = nullptr;    // ntc_hip_timer_begin / _end
+    bool spanOpen = false;
     DevMip* tableDev = nullptr;        // device copy of the mip table
     DevMip* staticTable = nullptr;     // this device's `scratch` array (ntc_hip_decode_static)
     uint32_t* handoffDev = nullptr;    // the dword between the two launches of the FP8 network (launch_decode_fp8)
@@ -529,8 +531,12 @@ static int create_context(int device, NtcHipContext** outContext)
     hipError_t e = hipStreamCreate(&L->stream);
     if (e == hipSuccess) e = hipEventCreate(&L->evStart);
     if (e == hipSuccess) e = hipEventCreate(&L->evStop);
+    if (e == hipSuccess) e = hipEventCreate(&L->evSpanStart);
+    if (e == hipSuccess) e = hipEventCreate(&L->evSpanStop);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&L->handoffDev), 256);
     if (e != hipSuccess) {
+        if (L->evSpanStop) (void)hipEventDestroy(L->evSpanStop);
+        if (L->evSpanStart) (void)hipEventDestroy(L->evSpanStart);
         if (L->evStop) (void)hipEventDestroy(L->evStop);
         if (L->evStart) (void)hipEventDestroy(L->evStart);
         if (L->stream) (void)hipStreamDestroy(L->stream);
@@ -566,6 +572,8 @@ static void destroy_context(NtcHipContext* L)
     }
     (void)hipEventDestroy(L->evStart);
     (void)hipEventDestroy(L->evStop);
+    (void)hipEventDestroy(L->evSpanStart);
+    (void)hipEventDestroy(L->evSpanStop);
     (void)hipStreamDestroy(L->stream);
     L->initialized = false;
     delete L;
@@ -755,6 +763,28 @@ int ntc_hip_ctx_decode_timed(NtcHipContext* ctx, const NtcHipTextureSet* sets, i
     float ms = 0.f;
     HIP_TRY(hipEventElapsedTime(&ms, L.evStart, L.evStop));
     *outMs = ms / float(iterations);
+    clear_error();
+    return 0;
+}
+
+int ntc_hip_ctx_timer_begin(NtcHipContext* ctx)
+{
+    CTX_ENTER(ctx);
+    HIP_TRY(hipEventRecord(L.evSpanStart, L.stream));
+    L.spanOpen = true;
+    clear_error();
+    return 0;
+}
+
+int ntc_hip_ctx_timer_end(NtcHipContext* ctx, float* outMilliseconds)
+{
+    CTX_ENTER(ctx);
+    if (!outMilliseconds) { set_error("ntc_hip_timer_end: the result pointer is null."); return NTC_HIP_ERR_INVALID_ARG; }
+    if (!L.spanOpen) { set_error("ntc_hip_timer_end: no ntc_hip_timer_begin before it on this context."); return NTC_HIP_ERR_INVALID_ARG; }
+    L.spanOpen = false;
+    HIP_TRY(hipEventRecord(L.evSpanStop, L.stream));
+    HIP_TRY(hipEventSynchronize(L.evSpanStop));
+    HIP_TRY(hipEventElapsedTime(outMilliseconds, L.evSpanStart, L.evSpanStop));
     clear_error();
     return 0;
 }
@@ -1186,6 +1216,8 @@ int ntc_hip_memset(void* dst, int value, size_t bytes) { return ntc_hip_ctx_mems
 int ntc_hip_synchronize(void) { return ntc_hip_ctx_synchronize(g_default); }
 int ntc_hip_decode(const NtcHipTextureSet* sets, int32_t numSets) { return ntc_hip_ctx_decode(g_default, sets, numSets); }
 int ntc_hip_decode_static(const NtcHipTextureSet* sets, int32_t numSets) { return ntc_hip_ctx_decode_static(g_default, sets, numSets); }
+int ntc_hip_timer_begin(void) { return ntc_hip_ctx_timer_begin(g_default); }
+int ntc_hip_timer_end(float* outMilliseconds) { return ntc_hip_ctx_timer_end(g_default, outMilliseconds); }
 int ntc_hip_decode_timed(const NtcHipTextureSet* sets, int32_t numSets, int32_t iterations, float* outMs) { return ntc_hip_ctx_decode_timed(g_default, sets, numSets, iterations, outMs); }
 int ntc_hip_build_query_latents(const NtcHipTextureSet* set, void* dst, uint64_t dstBytes) { return ntc_hip_ctx_build_query_latents(g_default, set, dst, dstBytes); }
 int ntc_hip_decode_queries(const NtcHipTextureSet* set, const NtcHipQuery* queries, uint64_t numQueries, void* out, uint64_t outBytes) { return ntc_hip_ctx_decode_queries(g_default, set, queries, numQueries, out, outBytes); }

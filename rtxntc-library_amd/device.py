@@ -73,6 +73,17 @@ class Device:
         return ms.value
 
 
+    def timer_begin(self):
+        """ntc_hip_timer_begin: a HIP event on the context's stream in front of what is queued next."""
+        self.call("timer_begin")
+
+    def timer_end(self):
+        """ntc_hip_timer_end: milliseconds of device time since timer_begin (waits for the queued work)."""
+        ms = C.c_float(0)
+        self.call("timer_end", C.byref(ms))
+        return ms.value
+
+
 class DeviceBuffer:
     def __init__(self, device, nbytes):
         self.device = device

@@ -56,6 +56,8 @@ def test_compute_entry_points_refuse_without_device(ntc):
     assert lib.ntc_hip_decode(sets, 1) == ntc.abi.ERR_NOT_INITIALIZED
     ms = C.c_float()
     assert lib.ntc_hip_decode_timed(sets, 1, 1, C.byref(ms)) == ntc.abi.ERR_NOT_INITIALIZED
+    assert lib.ntc_hip_timer_begin() == ntc.abi.ERR_NOT_INITIALIZED
+    assert lib.ntc_hip_timer_end(C.byref(ms)) == ntc.abi.ERR_NOT_INITIALIZED
     p = C.c_void_p()
     assert lib.ntc_hip_alloc(C.byref(p), 16) == ntc.abi.ERR_NOT_INITIALIZED
     with pytest.raises(ntc.NtcHipError):

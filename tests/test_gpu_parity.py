@@ -377,6 +377,28 @@ def test_decode_is_idempotent_and_timed_variant_matches(ntc, device):
     assert np.array_equal(first, case.d_output.download())
 
 
+def test_timer_spans_the_calls_between_its_two_ends(ntc, device):
+    """ntc_hip_timer_begin / _end: device time of whatever was queued between them.  A span around five decodes is
+    at least as long as five decodes timed back to back by ntc_hip_decode_timed (it also holds the table uploads
+    between them) and of the same order; an end without a begin is an error, and so is a second end."""
+    case = cfg_case(ntc, ntc.presets.spec_cfg01(), 1024, 1024, 5, 16, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=22)
+    dsets = device.pack_sets([case.device_set(device)])
+    for _ in range(20):
+        device.decode(dsets)
+    device.synchronize()
+    each = min(device.decode_timed(dsets, 5) for _ in range(3))
+    device.timer_begin()
+    for _ in range(5):
+        device.decode(dsets)
+    span = device.timer_end()
+    assert 0.8 * 5 * each < span < 5 * each * 3 + 1.0, (each, span)
+    with pytest.raises(ntc.NtcHipError) as e:
+        device.timer_end()
+    assert e.value.code == ntc.abi.ERR_INVALID_ARG and "timer_begin" in e.value.message
+    device.timer_begin()
+    assert device.timer_end() >= 0.0                         # an empty span
+
+
 def test_argument_errors_are_reported(ntc, device):
     case = cfg_case(ntc, ntc.presets.spec_cfg01(), 64, 64, 1, 8, ntc.abi.OUT_FP16_PLANAR_PAIRS, seed=1)
     dset = case.device_set(device)
