@@ -567,6 +567,15 @@ __device__ __forceinline__ void mfma32_as_two_16(uint4 const& a, uint4 const (&x
     mfma16(make_uint2(a.z, a.w), hi, acc);
 }
 
+// The wave's priority with the SIMD's arbiter, per part of a tile.  This network's activation stage is packed fp16
+// arithmetic and conversions - instructions that take an issue slot alone - and it is what the SIMD's time goes to;
+// the wave that has reached it goes first, matrix instructions (which then run in the shadow of other waves'
+// activation stages) and the input stage and stores last: one-plane sets -6.3 %, two-plane sets -8.2 %.  Any setting
+// with the activation stage above the rest measures the same; with the matrix instructions on top instead (what the
+// Int8 network's kernel wants, whose fp32 requantiser pairs up between waves) nothing is gained, and with the input
+// stage as high as the activation stage nothing either.
+constexpr int kPrioMatrix = 0, kPrioEpilogue = 2, kPrioOther = 1;
+
 // Hidden layers.  PLANES = 3, 2 for a tame layer, 1 where the whole weights sum exactly (see stage_fp8_weights).
 template <int NK32, bool HAS16>
 struct TileOperands { uint4 a32[3][NK32]; uint2 a16[3]; v4f bias; };     // one output tile's weight operands and bias
@@ -595,6 +604,7 @@ __device__ __forceinline__ void fp8_hidden_layer(Load&& load, uint4 const (&B32)
             __builtin_amdgcn_sched_barrier(0x67f);           // everything but LDS instructions may cross
         }
         TileOperands<NK32, HAS16> const& o = ops[t & 1];
+        __builtin_amdgcn_s_setprio(kPrioMatrix);
         v4f acc[3][4];
 #pragma unroll
         for (int p = 0; p < 3; ++p) {
@@ -608,6 +618,7 @@ __device__ __forceinline__ void fp8_hidden_layer(Load&& load, uint4 const (&B32)
             }
             if (HAS16) mfma16(o.a16[p], B16, acc[p]);
         }
+        __builtin_amdgcn_s_setprio(kPrioEpilogue);
 #pragma unroll
         for (int b = 0; b < 4; ++b) fp8_epilogue<LAST_HIDDEN, PLANES>(acc[2][b], acc[1][b], acc[0][b], o.bias, H[b][t]);
     }
@@ -724,7 +735,9 @@ __device__ __forceinline__ void mlp_forward_fp8(Fp8Lds<V>& lds, int wave, int la
         uint4 x[4];
 #pragma unroll
         for (int b = 0; b < 4; ++b) x[b] = make_uint4(Ha[b][0][0], Ha[b][0][1], Ha[b][1][0], Ha[b][1][1]);
+        __builtin_amdgcn_s_setprio(kPrioMatrix);
         mfma32(lds.w3[lane], x, acc);
+        __builtin_amdgcn_s_setprio(kPrioOther);
         v4i const bias = *reinterpret_cast<v4i const*>(&lds.outBias[g][0]);
         S = *reinterpret_cast<v4f const*>(&lds.outScale[g][0]);
 #pragma unroll
