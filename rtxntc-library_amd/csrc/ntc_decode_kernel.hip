@@ -1006,37 +1006,28 @@ __device__ __forceinline__ void f16_tile(LdsT<V> const& lds, int base, int t, in
 {
     constexpr int PAIRS = IN_TILES / 2, PER = V::f16_units(IN_TILES);
     uint4 const* const block = lds.late + base + t * PER;
-    if constexpr (IN_TILES % 2 == 0) {
 #pragma unroll
-        for (int p = 0; p < PAIRS; ++p) {
-            v8h const A = __builtin_bit_cast(v8h, block[p * 64 + lane]);
+    for (int p = 0; p < PAIRS; ++p) {
+        v8h const A = __builtin_bit_cast(v8h, block[p * 64 + lane]);
 #pragma unroll
-            for (int b = FIRST; b < FIRST + COUNT; ++b) {
-                uint4 const h = make_uint4(H[b][2 * p][0], H[b][2 * p][1], H[b][2 * p + 1][0], H[b][2 * p + 1][1]);
-                acc[b - FIRST] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, __builtin_bit_cast(v8h, h), acc[b - FIRST], 0, 0, 0);
-            }
+        for (int b = FIRST; b < FIRST + COUNT; ++b) {
+            uint4 const h = make_uint4(H[b][2 * p][0], H[b][2 * p][1], H[b][2 * p + 1][0], H[b][2 * p + 1][1]);
+            acc[b - FIRST] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, __builtin_bit_cast(v8h, h), acc[b - FIRST], 0, 0, 0);
         }
-    } else {
-        // An odd number of input tiles: every tile takes the 16-deep instruction (a pair's block holds tile 2p in
-        // its first four halves per lane and tile 2p+1 in the last four).  32-deep and 16-deep instructions are
-        // never mixed in one accumulator's chain: in either order that gave wrong sums with some instruction
-        // schedules (the wait between the two was not always there), while chains of one kind are reliable; two
-        // 16-deep instructions cost no more than one 32-deep one.
+    }
+    if constexpr (IN_TILES % 2 != 0) {
+        // An odd number of input tiles: the last one goes through the same 32-deep instruction with zeros in the
+        // upper half of both operands (its block in LDS holds four halves per lane).  32-deep and 16-deep instructions
+        // are never mixed in one accumulator's chain: in either order that gave wrong sums with some instruction
+        // schedules (the wait between the two was not always there), while chains of one kind are reliable.  (The
+        // whole layer on 16-deep instructions - three per output tile and texel block instead of two - was 0.5 to
+        // 0.9 % slower: every matrix instruction in flight keeps the SIMD from issuing two vector instructions a slot.)
+        uint2 const a = reinterpret_cast<uint2 const*>(block + PAIRS * 64)[lane];
+        v8h const A = __builtin_bit_cast(v8h, make_uint4(a.x, a.y, 0u, 0u));
 #pragma unroll
-        for (int ti = 0; ti < IN_TILES; ++ti) {
-            uint2 a;
-            if (ti < 2 * PAIRS) {
-                uint4 const unit = block[(ti >> 1) * 64 + lane];
-                a = (ti & 1) ? make_uint2(unit.z, unit.w) : make_uint2(unit.x, unit.y);
-            } else {
-                a = reinterpret_cast<uint2 const*>(block + PAIRS * 64)[lane];
-            }
-            v4h const A = __builtin_bit_cast(v4h, a);
-#pragma unroll
-            for (int b = FIRST; b < FIRST + COUNT; ++b) {
-                uint2 const h = make_uint2(H[b][ti][0], H[b][ti][1]);
-                acc[b - FIRST] = __builtin_amdgcn_mfma_f32_16x16x16f16(A, __builtin_bit_cast(v4h, h), acc[b - FIRST], 0, 0, 0);
-            }
+        for (int b = FIRST; b < FIRST + COUNT; ++b) {
+            uint4 const h = make_uint4(H[b][2 * PAIRS][0], H[b][2 * PAIRS][1], 0u, 0u);
+            acc[b - FIRST] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, __builtin_bit_cast(v8h, h), acc[b - FIRST], 0, 0, 0);
         }
     }
 }
@@ -1053,7 +1044,7 @@ __device__ __forceinline__ void f16_hidden_layer(LdsT<V> const& lds, int base, i
                                                  uint32_t (&Hin)[4][4][2], uint32_t (&Hout)[4][4][2], PendingTile& pending)
 {
     constexpr int PLANE = OUT_TILES * V::f16_units(IN_TILES);
-    constexpr int MATRIX = (TWO_PLANES ? 2 : 1) * 4 * ((IN_TILES % 2 == 0) ? IN_TILES / 2 : IN_TILES);   // matrix instructions per tile
+    constexpr int MATRIX = (TWO_PLANES ? 2 : 1) * 4 * ((IN_TILES + 1) / 2);   // matrix instructions per tile
     int const g = lane >> 4;
 #pragma unroll
     for (int t = 0; t < OUT_TILES; ++t) {
