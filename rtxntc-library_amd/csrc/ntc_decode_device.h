@@ -286,16 +286,17 @@ __device__ __forceinline__ void store_row(Mip const& m, StorePlace<FORMAT, Mip> 
     store_channels<FORMAT>(row, at.laneOff, at.laneOff2, h01, h23, at.nch, m.vectorStores);
 }
 
+// The stores of one wave tile: D[b] holds the lane's four channels of the texel in column `x` of block b, where block
+// b of 16 texels begins 16 * (b & 1) texels further right, in row y0 + (b >> 1).
 template <int FORMAT, bool CHECKED = true, class Acc, class Mip>
 __device__ __forceinline__ void store_tile(Mip const& m, Acc const (&D)[4], v4f S, int x, int y0, int chBase)
 {
-    StorePlace<FORMAT, Mip> const at(m, x, chBase);
-    if (at.nch <= 0) return;
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
-        int const y = y0 + b;
+        int const y = y0 + (b >> 1);
         if (y >= m.height) break;                            // uniform
-        store_row<FORMAT, CHECKED>(m, at, D[b], S, y);
+        StorePlace<FORMAT, Mip> const at(m, x + 16 * (b & 1), chBase);
+        if (at.nch > 0) store_row<FORMAT, CHECKED>(m, at, D[b], S, y);
     }
 }
 
@@ -314,7 +315,8 @@ __device__ __attribute__((noinline)) void store_tile_general(DevMip const* mip, 
 }
 
 // The stores of a wave tile that lies inside the image of a mip whose channel count is a multiple of four (the common
-// case): no bounds to test, every lane stores its four channels of all four rows, and the row addresses are one uniform
+// case): no bounds to test, every lane stores its four channels of all four blocks (block b: 16 texels from
+// x0 + 16 * (b & 1) in row y0 + (b >> 1)), and the row addresses are one uniform
 // base plus multiples of the row size - a handful of scalar additions instead of a 64-bit product, a test and a
 // branch per row.  x0, y0: first texel of the wave tile; lane = (j, g) holds channels 4g..4g+3 of texel column j.
 template <int FORMAT, bool CHECKED, class Acc, class Mip>
@@ -342,7 +344,8 @@ __device__ __forceinline__ void store_tile_inside(Mip const& m, Acc const (&D)[4
     for (int b = 0; b < 4; ++b) {
         uint32_t const h01 = to_half2_bits<CHECKED>(float(D[b][0]) * S[0], float(D[b][1]) * S[1]);
         uint32_t const h23 = to_half2_bits<CHECKED>(float(D[b][2]) * S[2], float(D[b][3]) * S[3]);
-        GlobalOutPtr const row = tile + size_t(b) * rowBytes;
+        GlobalOutPtr const row = tile + size_t(b >> 1) * rowBytes
+                               + ((b & 1) ? size_t(16) * (FORMAT == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS ? size_t(4) : size_t(m.outPixelStride)) : size_t(0));
         if constexpr (FORMAT == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS) {
             *reinterpret_cast<DwordPtr>(row + laneOff) = h01;
             *reinterpret_cast<DwordPtr>(row + laneOff2) = h23;
@@ -356,7 +359,7 @@ __device__ __forceinline__ void store_tile_inside(Mip const& m, Acc const (&D)[4
 }
 
 // One row of a wave tile in the mip's own format (checked conversion): the stores of the int8-only network path,
-// which produces the wave's four rows one after the other.
+// which produces the wave's four blocks of 16 texels one after the other.
 template <class AccV, class Mip>
 __device__ __forceinline__ void store_row_any_format(Mip const& m, AccV D, v4f S, int x, int y, int chBase)
 {

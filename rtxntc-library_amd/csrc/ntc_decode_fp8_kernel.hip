@@ -21,7 +21,7 @@
 // the int8 input of the output layer, which is acc = bias + sum W q in exact fp32 / int32, o = float(acc) * scale.
 //
 // Work distribution, tiles and stores are those of decode_kernel (ntc_decode_kernel.hip): one persistent
-// launch, a workgroup tile of 64 x 4 texels = four wave tiles of 16 x 4; lane = texel in the input stage,
+// launch, a workgroup tile of 64 x 4 texels = four wave tiles of 32 x 2 (see decode_kernel); lane = texel in the input stage,
 // lane (j = lane%16, g = lane/16) = channels 16t+4g..+3 of texel j in the matrix stages.
 #include "ntc_decode_device.h"
 #include <type_traits>
@@ -778,13 +778,14 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles, 
 
     int modes = 7;                                           // uniform: the hidden layers' modes (stage_fp8_weights)
 
-    // One wave tile: the 16 x 4 texels of this wave in tile (tileX, tileY) of mip m.
+    // One wave tile: the 32 x 2 texels of this wave in tile (tileX, tileY) of mip m; block b of 16 texels begins at
+    // (x0 + 16 * (b & 1), y0 + (b >> 1)), so that a wave's stores fill whole 128-byte lines of a row (store_tile).
     auto decode_wave_tile = [&](RunMip const& m, int tileX, int tileY) __attribute__((always_inline)) {
-        int const x0 = tileX * 64 + (wave & 3) * 16, y0 = tileY * 4;
-        if (x0 >= m.width) return;                           // whole wave tile outside the image
+        int const x0 = tileX * 64 + (wave & 1) * 32, y0 = tileY * 4 + ((wave >> 1) & 1) * 2;
+        if (x0 >= m.width || y0 >= m.height) return;         // whole wave tile outside the image
         uint32_t in[24];
         {
-            int const x = min(x0 + j, m.width - 1), y = min(y0 + g, m.height - 1);
+            int const x = min(x0 + j + 16 * (g & 1), m.width - 1), y = min(y0 + (g >> 1), m.height - 1);
             if (m.fast) {
                 Fp8Fetch<V> fetch;
                 fetch_latents_fast<V>(m.full, x, y, fetch);

@@ -1,7 +1,8 @@
 // ntc_decode_kernel.hip - texture-set decode for gfx950 (MI355X), int8 network.
 //
 // One persistent launch decodes every colour mip of every texture set handed to it.
-// Work unit: a workgroup tile of 64x4 texels = four wave64 tiles of 16x4 texels.
+// Work unit: a workgroup tile of 64x4 texels = four wave64 tiles of 32x2 texels (four blocks of 16 texels: two side
+// by side in each of two rows, so that a wave writes whole 128-byte lines of a row).
 //
 // Per wave tile:
 //   1. input stage, one texel per lane: latent fetch (2x2 concat or bilinear, wrap
@@ -1235,17 +1236,20 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
     int staged = 0;                                          // uniform: how layers 1..3 of the staged set run (kStagedF16, ...)
     int entry = 0;
 
-    // One wave tile: the 16 x 4 texels of this wave in tile (tileX, tileY) of mip m.
+    // One wave tile: the 32 x 2 texels of this wave in tile (tileX, tileY) of mip m: block b of 16 texels begins at
+    // (x0 + 16 * (b & 1), y0 + (b >> 1)).  (With 16 x 4 texels per wave the two 64-byte halves of an output line came
+    // from two waves, at different times, and the L2 wrote 5 - 10 % of the halves back twice; so each line now comes
+    // from one wave's consecutive stores and the write traffic is exactly the output's size.)
     auto decode_wave_tile = [&](RunMip const& m, int tileX, int tileY, int sub) __attribute__((always_inline)) {
-        int const x0 = tileX * 64 + sub * 16;
-        int const y0 = tileY * 4;
-        if (x0 >= m.width) return;                           // whole wave tile outside the image
+        int const x0 = tileX * 64 + (sub & 1) * 32;
+        int const y0 = tileY * 4 + (sub >> 1) * 2;
+        if (x0 >= m.width || y0 >= m.height) return;         // whole wave tile outside the image
 
-        // ---- 1. input stage: lane = texel (tx = lane%16, ty = lane/16)
+        // ---- 1. input stage: lane = texel (block g = lane/16, column j = lane%16 of the block)
         wave_priority<kPrioOther>();
         uint32_t in[16];
         {
-            int const x = min(x0 + j, m.width - 1), y = min(y0 + g, m.height - 1);
+            int const x = min(x0 + j + 16 * (g & 1), m.width - 1), y = min(y0 + (g >> 1), m.height - 1);
             if (m.fast) prepare_inputs_fast<V>(m.full, lds, x, y, in);
             else        prepare_inputs_general<V>(m.full, x, y, in);
         }
@@ -1256,7 +1260,7 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
             mlp_forward_f16<V>(lds, wave, lane, (staged & kL0Magic) != 0, in, D, S);
             // a wave tile inside the image, channels in whole groups of four (pixel formats: vector stores possible),
             // takes the stores without tests
-            bool const inside = x0 + 16 <= m.width && y0 + 4 <= m.height && (m.numChannels & 3) == 0
+            bool const inside = x0 + 32 <= m.width && y0 + 2 <= m.height && (m.numChannels & 3) == 0
                              && (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS || m.vectorStores);
             if (!inside) {
                 store_tile_general(&m.full, D[0], D[1], D[2], D[3], S, x0 + j, y0, 4 * g);
@@ -1270,7 +1274,7 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
                 else                                                   store_tile_inside<NTC_HIP_DEV_OUT_UNORM8_PIXELS, true>(m, D, S, x0, y0, j, g);
             }
         } else {
-            // every layer on the int8 matrix instruction: one 16-texel block (= one image row of the tile) at a time
+            // every layer on the int8 matrix instruction: one 16-texel block at a time
             write_inputs<V>(lds, wave, lane, in);
 #pragma unroll 1
             for (int b = 0; b < 4; ++b) {
@@ -1279,7 +1283,7 @@ decode_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles)
                 int laneB = lane;
                 asm volatile("" : "+v"(laneB));                  // keeps the weight reads inside the loop (hoisted, they take every register)
                 mlp_forward_block<V>(lds, laneB, read_input_block<V>(lds, wave, lane, b), D, S);
-                store_row_any_format(m, D, S, x0 + j, y0 + b, 4 * g);
+                store_row_any_format(m, D, S, x0 + j + 16 * (b & 1), y0 + (b >> 1), 4 * g);
             }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
