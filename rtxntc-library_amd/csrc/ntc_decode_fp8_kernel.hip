@@ -797,14 +797,22 @@ decode_fp8_kernel(DevMip const* __restrict__ mips, int numMips, int totalTiles, 
         v4i D[4];
         v4f S;
         mlp_forward_fp8<V>(lds, wave, lane, modes, in, D, S);
-        if (V::ONE && (modes & kFp8OutputsBounded)) {        // (the general instantiation keeps to the checked stores)
-            if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)  store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS, false>(m, D, S, x0 + j, y0, 4 * g);
-            else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)   store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS, false>(m, D, S, x0 + j, y0, 4 * g);
-            else                                                   store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS, false>(m, D, S, x0 + j, y0, 4 * g);
+        // a wave tile inside the image, channels in whole groups of four (pixel formats: vector stores possible), takes
+        // the stores without tests; the one-plane instantiation also without the fp16-overflow check where no output
+        // can come near it (the general instantiation keeps to the checked conversion)
+        bool const inside = x0 + 32 <= m.width && y0 + 2 <= m.height && (m.numChannels & 3) == 0
+                         && (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS || m.vectorStores);
+        if (!inside) {
+            store_tile_general(&m.full, D[0], D[1], D[2], D[3], S, x0 + j, y0, 4 * g);
+        } else if (V::ONE && (modes & kFp8OutputsBounded)) {
+            if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)  store_tile_inside<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS, false>(m, D, S, x0, y0, j, g);
+            else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)   store_tile_inside<NTC_HIP_DEV_OUT_FP16_PIXELS, false>(m, D, S, x0, y0, j, g);
+            else                                                   store_tile_inside<NTC_HIP_DEV_OUT_UNORM8_PIXELS, false>(m, D, S, x0, y0, j, g);
+        } else {
+            if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS)  store_tile_inside<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS, true>(m, D, S, x0, y0, j, g);
+            else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)   store_tile_inside<NTC_HIP_DEV_OUT_FP16_PIXELS, true>(m, D, S, x0, y0, j, g);
+            else                                                   store_tile_inside<NTC_HIP_DEV_OUT_UNORM8_PIXELS, true>(m, D, S, x0, y0, j, g);
         }
-        else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS) store_tile<NTC_HIP_DEV_OUT_FP16_PLANAR_PAIRS>(m, D, S, x0 + j, y0, 4 * g);
-        else if (m.outFormat == NTC_HIP_DEV_OUT_FP16_PIXELS)       store_tile<NTC_HIP_DEV_OUT_FP16_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
-        else                                                       store_tile<NTC_HIP_DEV_OUT_UNORM8_PIXELS>(m, D, S, x0 + j, y0, 4 * g);
     };
 
     int entry = 0;
