@@ -526,7 +526,8 @@ static int create_context(int device, NtcHipContext** outContext)
     L->device = device;
     L->computeUnits = prop.multiProcessorCount;
     L->clockRateKHz = prop.clockRate;
-    std::snprintf(L->name, sizeof(L->name), "%s (%s)", prop.name, prop.gcnArchName);
+    // (some driver stacks report no marketing name)
+    std::snprintf(L->name, sizeof(L->name), "%s (%s)", prop.name[0] ? prop.name : "AMD GPU", prop.gcnArchName);
     L->staticTable = static_cast<DevMip*>(g_staticTable[device]);
     hipError_t e = hipStreamCreate(&L->stream);
     if (e == hipSuccess) e = hipEventCreate(&L->evStart);
